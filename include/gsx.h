@@ -1,0 +1,228 @@
+/* gsx.h - C ABI of libgsx.so: hand-written gfx950 (MI355X) kernels for the 3D-Gaussian-splatting
+ * training step that sits behind LichtFeld-Studio's gsplat/Ops.h.
+ *
+ * Conventions
+ *  - Every pointer is a DEVICE pointer unless its name ends in _host.  Tensors are contiguous, fp32
+ *    unless stated, laid out exactly as the reference's at::Tensor arguments (row-major).
+ *  - `stream` is a hipStream_t passed as void* (NULL = the null stream).  No entry point allocates,
+ *    frees or synchronises, except gsx_intersect_tile_count (returns a value to the host) and the
+ *    functions documented as "convenience" which say so.
+ *  - Scratch memory comes from the caller: <op>_workspace_bytes() says how much, and the same
+ *    (workspace, workspace_bytes) pair is handed to the op.  Workspaces need 256-byte alignment.
+ *  - Return value: GSX_OK or a negative gsx_status.  gsx_last_error() gives a thread-local message.
+ *  - Optional pointers may be NULL where the comment says "nullable".
+ *  - Only C = 1 camera, the perfect-pinhole model and a global shutter are implemented (what
+ *    LichtFeld's trainer uses: rasterizer.cpp:33-35, rasterizer_autograd.cpp:59-60); other values
+ *    return GSX_ERR_UNSUPPORTED.
+ *
+ * All file:line citations are relative to the LichtFeld-Studio tree.
+ */
+#ifndef GSX_H
+#define GSX_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(GSX_BUILD)
+#define GSX_API __attribute__((visibility("default")))
+#else
+#define GSX_API
+#endif
+
+typedef enum gsx_status {
+    GSX_OK = 0,
+    GSX_ERR_INVALID_ARGUMENT = -1, /* null pointer, bad size, bad enum */
+    GSX_ERR_UNSUPPORTED = -2,      /* C > 1, non-pinhole camera, rolling shutter, CDIM not built */
+    GSX_ERR_WORKSPACE = -3,        /* workspace too small or misaligned */
+    GSX_ERR_HIP = -4,              /* a HIP runtime call failed (message has the HIP error) */
+    GSX_ERR_OVERFLOW = -5          /* n_isects does not fit the int32 index space */
+} gsx_status;
+
+/* gsplat/Common.h:46-51 */
+typedef enum gsx_camera_model { GSX_PINHOLE = 0, GSX_ORTHO = 1, GSX_FISHEYE = 2, GSX_EQUIRECTANGULAR = 3 } gsx_camera_model;
+/* gsplat/Cameras.h:16-22 */
+typedef enum gsx_shutter_type {
+    GSX_ROLLING_TOP_TO_BOTTOM = 0,
+    GSX_ROLLING_LEFT_TO_RIGHT = 1,
+    GSX_ROLLING_BOTTOM_TO_TOP = 2,
+    GSX_ROLLING_RIGHT_TO_LEFT = 3,
+    GSX_GLOBAL = 4
+} gsx_shutter_type;
+/* gsplat/Cameras.h:27-44 UnscentedTransformParameters (same defaults when zero-initialised via gsx_ut_defaults) */
+typedef struct gsx_ut_params {
+    float alpha, beta, kappa, in_image_margin_factor;
+    int32_t require_all_sigma_points_valid;
+} gsx_ut_params;
+
+GSX_API int gsx_version(void);
+GSX_API const char* gsx_last_error(void);
+GSX_API const char* gsx_status_string(int status);
+GSX_API gsx_ut_params gsx_ut_defaults(void);
+/* Test hook (no counterpart in the reference): evaluates one of the shared fp32 math primitives element-wise on the
+ * device so that a test can compare it bit for bit with a host build.  which: 0 exp, 1 log, 2 rsqrt, 3 sin, 4 acos,
+ * 5 sigmoid, 6 saturating float->u32, 7 pow(x, x2), 8 x / x2, 9 sqrt, 10 fma(x, x2, x). */
+GSX_API int gsx_debug_math(int which, uint32_t n, const float* x, const float* x2, float* y, void* stream);
+
+/* ---- a1: gsplat::projection_ut_3dgs_fused (Ops.h:69-98; kernel ProjectionUT3DGSFused.cu:17-210) ----
+ * means [N,3] quats [N,4] (wxyz) scales [N,3] opacities [N] nullable, viewmats0 [C,4,4], Ks [C,3,3]
+ * -> radii i32 [C,N,2], means2d [C,N,2], depths [C,N], conics [C,N,3], compensations [C,N] nullable.
+ * Rows of culled Gaussians (radii 0) are left untouched in means2d/depths/conics/compensations. */
+GSX_API int gsx_projection_ut_3dgs_fused(
+    uint32_t C, uint32_t N, const float* means, const float* quats, const float* scales, const float* opacities,
+    const float* viewmats0, const float* viewmats1 /*must be NULL*/, const float* Ks, uint32_t image_width,
+    uint32_t image_height, float eps2d, float near_plane, float far_plane, float radius_clip, int camera_model,
+    gsx_ut_params ut, int rs_type, const float* radial_coeffs, const float* tangential_coeffs,
+    const float* thin_prism_coeffs, int32_t* radii, float* means2d, float* depths, float* conics,
+    float* compensations, void* stream);
+
+/* ---- a3: gsplat::spherical_harmonics_fwd / _bwd (Ops.h:12-25; SphericalHarmonicsCUDA.cu:373-529) ----
+ * dirs [N,3], coeffs [N,K,3], masks u8/bool [N] nullable -> colors [N,3] (masked rows untouched).
+ * bwd: v_coeffs [N,K,3] is fully written (zero for masked rows and unused bands); v_dirs [N,3] nullable
+ * (degree <= 3 when requested). */
+GSX_API int gsx_spherical_harmonics_fwd(uint32_t N, uint32_t K, uint32_t degrees_to_use, const float* dirs,
+                                        const float* coeffs, const uint8_t* masks, float* colors, void* stream);
+GSX_API int gsx_spherical_harmonics_bwd(uint32_t N, uint32_t K, uint32_t degrees_to_use, const float* dirs,
+                                        const float* coeffs, const uint8_t* masks, const float* v_colors,
+                                        float* v_coeffs, float* v_dirs, void* stream);
+
+/* ---- a4: gsplat::intersect_tile (Ops.h:28-38; Intersect.cpp:15-122; IntersectTile.cu:23-114) ----
+ * Two calls, as the reference's two passes: count (+ inclusive scan; blocks until the total is on the
+ * host, like Intersect.cpp:76) then emit.  cum_tiles_per_gauss is i64 [C*N]. */
+GSX_API size_t gsx_intersect_tile_count_workspace_bytes(uint32_t C, uint32_t N);
+GSX_API int gsx_intersect_tile_count(uint32_t C, uint32_t N, const float* means2d, const int32_t* radii,
+                                     uint32_t tile_size, uint32_t tile_width, uint32_t tile_height,
+                                     int32_t* tiles_per_gauss, int64_t* cum_tiles_per_gauss, void* workspace,
+                                     size_t workspace_bytes, int64_t* n_isects_host, void* stream);
+GSX_API int gsx_intersect_tile_emit(uint32_t C, uint32_t N, const float* means2d, const int32_t* radii,
+                                    const float* depths, const int64_t* cum_tiles_per_gauss, uint32_t tile_size,
+                                    uint32_t tile_width, uint32_t tile_height, int64_t* isect_ids,
+                                    int32_t* flatten_ids, void* stream);
+/* Intersect.cpp:46-47: floor(log2(n)) + 1 */
+GSX_API uint32_t gsx_n_bits(uint32_t n);
+
+/* ---- a5: gsplat::radix_sort_double_buffer (Intersect.h:39-46; IntersectTile.cu:290-328) ----
+ * Stable ascending LSD radix sort of (i64 key, i32 value) pairs on key bits [0, end_bit).
+ * Buffers 0 (keys0/vals0, the input) and 1 (keys1/vals1) are ping-ponged; *selector_host (host int)
+ * says which pair holds the result (like cub::DoubleBuffer::selector). */
+GSX_API size_t gsx_radix_sort_pairs_workspace_bytes(int64_t n);
+GSX_API int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, int64_t* keys1, int32_t* vals1,
+                                 uint32_t end_bit, void* workspace, size_t workspace_bytes, int* selector_host,
+                                 void* stream);
+
+/* ---- a6: gsplat::intersect_offset (Ops.h:39-43; IntersectTile.cu:206-286) -> offsets i32 [C,Th,Tw] ---- */
+GSX_API int gsx_intersect_offset(int64_t n_isects, const int64_t* isect_ids, uint32_t C, uint32_t tile_width,
+                                 uint32_t tile_height, int32_t* offsets, void* stream);
+
+/* ---- a7: gsplat::rasterize_to_pixels_from_world_3dgs_fwd (Ops.h:100-129; ...3DGSFwd.cu:19-285) ----
+ * colors [C,N,channels] (channels in {1,3,4}), opacities [C,N], backgrounds [C,channels] nullable,
+ * masks u8 [C,Th,Tw] nullable, tile_offsets i32 [C,Th,Tw], flatten_ids i32 [n_isects]
+ * -> render_colors [C,H,W,channels], render_alphas [C,H,W,1], last_ids i32 [C,H,W]. tile_size must be 16. */
+GSX_API int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
+    uint32_t C, uint32_t N, int64_t n_isects, const float* means, const float* quats, const float* scales,
+    const float* colors, uint32_t channels, const float* opacities, const float* backgrounds, const uint8_t* masks,
+    uint32_t image_width, uint32_t image_height, uint32_t tile_size, const float* viewmats0,
+    const float* viewmats1 /*must be NULL*/, const float* Ks, int camera_model, gsx_ut_params ut, int rs_type,
+    const float* radial_coeffs, const float* tangential_coeffs, const float* thin_prism_coeffs,
+    const int32_t* tile_offsets, const int32_t* flatten_ids, float* render_colors, float* render_alphas,
+    int32_t* last_ids, void* stream);
+
+/* ---- a8: gsplat::rasterize_to_pixels_from_world_3dgs_bwd (Ops.h:131-166; ...3DGSBwd.cu:16-379) ----
+ * channels must be 3.  The five gradient outputs are fully WRITTEN (no zero-fill needed; the reference
+ * zero-fills and accumulates, Rasterization.cpp:190-194): v_means [N,3], v_quats [N,4], v_scales [N,3],
+ * v_colors [C,N,3], v_opacities [C,N].  The workspace holds 16 floats per Gaussian. */
+GSX_API size_t gsx_rasterize_bwd_workspace_bytes(uint32_t N);
+GSX_API int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
+    uint32_t C, uint32_t N, int64_t n_isects, const float* means, const float* quats, const float* scales,
+    const float* colors, const float* opacities, const float* backgrounds, const uint8_t* masks,
+    uint32_t image_width, uint32_t image_height, uint32_t tile_size, const float* viewmats0,
+    const float* viewmats1 /*must be NULL*/, const float* Ks, int camera_model, gsx_ut_params ut, int rs_type,
+    const float* radial_coeffs, const float* tangential_coeffs, const float* thin_prism_coeffs,
+    const int32_t* tile_offsets, const int32_t* flatten_ids, const float* render_alphas, const int32_t* last_ids,
+    const float* v_render_colors, const float* v_render_alphas, float* v_means, float* v_quats, float* v_scales,
+    float* v_colors, float* v_opacities, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- g1 glue of a9 (Rasterization.cpp:356-378 and :608-624), fused into one pass each ----
+ * fwd: colors [N,3] = max(SH(means - campos(viewmat)) + 0.5, 0) where radii > 0, else 0.
+ * bwd: v_sh_coeffs [N,K,3] fully written from v_colors with the clamp mask applied. */
+GSX_API int gsx_sh_colors_from_world(uint32_t N, uint32_t K, uint32_t sh_degree, const float* means,
+                                     const float* sh_coeffs, const int32_t* radii, const float* viewmat,
+                                     float* colors, void* stream);
+GSX_API int gsx_sh_colors_from_world_bwd(uint32_t N, uint32_t K, uint32_t sh_degree, const float* means,
+                                         const int32_t* radii, const float* viewmat, const float* colors,
+                                         const float* v_colors, float* v_sh_coeffs, void* stream);
+
+/* ---- a10: fusedssim / fusedssim_backward (include/kernels/ssim.cuh:11-28; src/training/kernels/ssim.cu) ----
+ * img1, img2 [B,CH,H,W].  dm_* nullable together (train == false). */
+GSX_API int gsx_fusedssim(int B, int CH, int H, int W, float C1, float C2, const float* img1, const float* img2,
+                          float* ssim_map, float* dm_dmu1, float* dm_dsigma1_sq, float* dm_dsigma12, void* stream);
+GSX_API int gsx_fusedssim_backward(int B, int CH, int H, int W, float C1, float C2, const float* img1,
+                                   const float* img2, const float* dL_dmap, const float* dm_dmu1,
+                                   const float* dm_dsigma1_sq, const float* dm_dsigma12, float* dL_dimg1,
+                                   void* stream);
+
+/* ---- a11: adam_step (fastgs/optimizer/include/adam_kernels.cuh:13-36; src/adam_api.cu:8-33) ----
+ * gsx_adam_step_multi runs up to GSX_ADAM_MAX_TENSORS parameter groups in ONE launch (the reference
+ * launches once per group, fused_adam.cpp:29-94); entries with n == 0 or grad == NULL are skipped. */
+GSX_API int gsx_adam_step(float* param, float* exp_avg, float* exp_avg_sq, const float* grad, int64_t n, float lr,
+                          float beta1, float beta2, float eps, float bias_correction1_rcp,
+                          float bias_correction2_sqrt_rcp, void* stream);
+#define GSX_ADAM_MAX_TENSORS 8
+typedef struct gsx_adam_group {
+    float* param;
+    float* exp_avg;
+    float* exp_avg_sq;
+    const float* grad;
+    int64_t n;
+    float lr, beta1, beta2, eps, bias_correction1_rcp, bias_correction2_sqrt_rcp;
+} gsx_adam_group;
+GSX_API int gsx_adam_step_multi(const gsx_adam_group* groups_host, int n_groups, void* stream);
+
+/* ---- a12: gsplat::relocation (Ops.h:52-57; RelocationCUDA.cu:11-43) ---- */
+GSX_API int gsx_relocation(int M, const float* opacities, const float* scales, const int32_t* ratios,
+                           const float* binoms, int n_max, float* new_opacities, float* new_scales, void* stream);
+/* ---- a13: gsplat::add_noise (Ops.h:59-65; RelocationCUDA.cu:112-144); means updated in place ---- */
+GSX_API int gsx_add_noise(int N, const float* raw_opacities, const float* raw_scales, const float* raw_quats,
+                          const float* noise, float* means, float current_lr, void* stream);
+/* ---- a14: gsplat::quats_to_rotmats (Ops.h:46-48; QuatToRotmatCUDA.cu:14-39) -> [N,3,3] row-major ---- */
+GSX_API int gsx_quats_to_rotmats(int N, const float* quats, float* rotmats, void* stream);
+
+/* ---- a15: step-driver passes that LichtFeld runs as ATen ops around the boundary, one kernel each ----
+ * activations (src/core/splat_data.cpp:271-286): opacity = sigmoid(raw) [N], scales = exp(raw) [N,3],
+ * quats = raw / max(|raw|, 1e-12) [N,4].  Their VJPs (what autograd applies after Ops.h's backward):
+ * v_opacity_raw = v_o * o (1 - o), v_scaling_raw = v_s * s, v_rotation_raw = normalize VJP. */
+GSX_API int gsx_activate_params(uint32_t N, const float* opacity_raw, const float* scaling_raw,
+                                const float* rotation_raw, float* opacities, float* scales, float* quats,
+                                void* stream);
+GSX_API int gsx_activate_params_bwd(uint32_t N, const float* opacity_raw, const float* scaling_raw,
+                                    const float* rotation_raw, const float* v_opacities, const float* v_scales,
+                                    const float* v_quats, float* v_opacity_raw, float* v_scaling_raw,
+                                    float* v_rotation_raw, void* stream);
+/* image = clamp(render HWC -> CHW, 0, 1) (rasterizer.cpp:205) and the per-pixel part of the photometric
+ * loss of trainer.cpp:126-129: partial sums of |image - gt| into l1_partials [gsx_image_loss_blocks()]. */
+GSX_API uint32_t gsx_image_loss_blocks(uint32_t H, uint32_t W);
+GSX_API int gsx_image_from_render(uint32_t H, uint32_t W, const float* render_hwc, const float* gt_chw,
+                                  float* image_chw, float* l1_partials, void* stream);
+/* mean of the SSIM map over the "valid" crop [5:H-5, 5:W-5] (fused_ssim.cuh:59-67,117-122) as partial sums */
+GSX_API int gsx_ssim_valid_partials(uint32_t CH, uint32_t H, uint32_t W, const float* ssim_map, float* partials,
+                                    void* stream);
+/* loss = (1-lambda) * mean|img-gt| + lambda * (1 - mean_valid(ssim)); one block; writes loss_out[0..2] =
+ * (loss, l1, ssim) on the device */
+GSX_API int gsx_photometric_loss_finish(uint32_t CH, uint32_t H, uint32_t W, float lambda_dssim,
+                                        const float* l1_partials, const float* ssim_partials, uint32_t n_partials,
+                                        float* loss_out, void* stream);
+/* v_render [H,W,3] = d loss / d render: L1 sign term + lambda * SSIM term (dL_dimg_ssim is
+ * gsx_fusedssim_backward's output for dL_dmap = -lambda / count on the valid crop, 0 elsewhere), passed through
+ * the clamp VJP (zero where render < 0 or > 1) and the CHW -> HWC permute. */
+GSX_API int gsx_ssim_valid_grad_map(uint32_t CH, uint32_t H, uint32_t W, float scale, float* dL_dmap, void* stream);
+GSX_API int gsx_render_grad_from_loss(uint32_t H, uint32_t W, float lambda_dssim, const float* render_hwc,
+                                      const float* image_chw, const float* gt_chw, const float* dL_dimg_ssim,
+                                      float* v_render_hwc, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GSX_H */

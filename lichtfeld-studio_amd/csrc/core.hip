@@ -1,0 +1,104 @@
+// core.hip - error reporting, version, argument checks shared by the entry points.
+#include <stdarg.h>
+
+#include "gsx_common.h"
+
+namespace gsx {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+// Only what LichtFeld's trainer exercises is built: one camera per call (the reference's rasterizer indexes
+// per-Gaussian arrays with the flattened [C*N] id, RasterizeToPixelsFromWorld3DGSFwd.cu:203-210, so C > 1 is
+// not usable there either), perfect pinhole, global shutter.
+int check_camera_args(uint32_t C, const float* viewmats1, int camera_model, int rs_type, const float* radial,
+                      const float* tangential, const float* thin_prism) {
+    GSX_REQUIRE(C == 1, GSX_ERR_UNSUPPORTED, "C = %u cameras: only C == 1 is supported", C);
+    GSX_REQUIRE(camera_model == GSX_PINHOLE, GSX_ERR_UNSUPPORTED, "camera model %d: only PINHOLE is supported",
+                camera_model);
+    GSX_REQUIRE(radial == nullptr && tangential == nullptr && thin_prism == nullptr, GSX_ERR_UNSUPPORTED,
+                "distortion coefficients: only the perfect pinhole model is supported");
+    GSX_REQUIRE(rs_type == GSX_GLOBAL && viewmats1 == nullptr, GSX_ERR_UNSUPPORTED,
+                "rolling shutter (rs_type %d / viewmats1): only a global shutter is supported", rs_type);
+    return GSX_OK;
+}
+
+// probe of the shared math primitives on the device (lets a test compare them bit for bit with a host build)
+__global__ void __launch_bounds__(256) math_unary_kernel(int which, uint32_t n, const float* __restrict__ x,
+                                                          const float* __restrict__ x2, float* __restrict__ y) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= n)
+        return;
+    const float a = x[i];
+    float r = 0.f;
+    switch (which) {
+    case 0: r = gsx::exp(a); break;
+    case 1: r = gsx::log(a); break;
+    case 2: r = gsx::rsqrt(a); break;
+    case 3: r = gsx::sin(a); break;
+    case 4: r = gsx::acos(a); break;
+    case 5: r = gsx::sigmoid(a); break;
+    case 6: r = (float)gsx::sat_u32(a); break;
+    case 7: r = gsx::pow(a, x2[i]); break;
+    case 8: r = a / x2[i]; break;
+    case 9: r = gsx::sqrt(a); break;
+    case 10: r = gsx::fma(a, x2[i], a); break;
+    default: break;
+    }
+    y[i] = r;
+}
+
+} // namespace gsx
+
+extern "C" int gsx_debug_math(int which, uint32_t n, const float* x, const float* x2, float* y, void* stream) {
+    if (n == 0)
+        return GSX_OK;
+    GSX_REQUIRE(x && y, GSX_ERR_INVALID_ARGUMENT, "debug_math: null tensor");
+    GSX_REQUIRE(which < 7 || x2 != nullptr, GSX_ERR_INVALID_ARGUMENT, "debug_math: second operand is null");
+    hipLaunchKernelGGL(gsx::math_unary_kernel, dim3(gsx::cdiv(n, 256)), dim3(256), 0, (hipStream_t)stream, which, n, x,
+                       x2, y);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+extern "C" int gsx_version(void) { return 100; }
+
+extern "C" const char* gsx_last_error(void) { return gsx::g_err; }
+
+extern "C" const char* gsx_status_string(int status) {
+    switch (status) {
+    case GSX_OK: return "ok";
+    case GSX_ERR_INVALID_ARGUMENT: return "invalid argument";
+    case GSX_ERR_UNSUPPORTED: return "unsupported configuration";
+    case GSX_ERR_WORKSPACE: return "workspace too small or misaligned";
+    case GSX_ERR_HIP: return "HIP runtime error";
+    case GSX_ERR_OVERFLOW: return "intersection count overflows int32";
+    default: return "unknown status";
+    }
+}
+
+extern "C" gsx_ut_params gsx_ut_defaults(void) {
+    gsx_ut_params p;
+    p.alpha = 0.1f;
+    p.beta = 2.f;
+    p.kappa = 0.f;
+    p.in_image_margin_factor = 0.1f;
+    p.require_all_sigma_points_valid = 1;
+    return p;
+}
+
+extern "C" uint32_t gsx_n_bits(uint32_t n) {
+    // (uint32_t)floor(log2(n)) + 1 for n >= 1 (gsplat/Intersect.cpp:46-47)
+    uint32_t b = 0;
+    while (n) {
+        ++b;
+        n >>= 1;
+    }
+    return b;
+}

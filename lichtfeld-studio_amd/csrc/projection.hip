@@ -1,0 +1,671 @@
+// projection.hip - per-Gaussian streaming kernels: unscented-transform projection, spherical harmonics
+// forward/backward, quaternion -> rotation matrix, parameter activations.
+//
+// All of these touch each Gaussian once and are bound by HBM bandwidth; one lane owns one Gaussian and
+// rows are read with whole-row vector loads.
+#include "gsx_common.h"
+
+namespace gsx {
+
+static constexpr float kAlphaThreshold = 1.f / 255.f; // gsplat/Common.h:54
+
+// ---------------------------------------------------------------------------------------------
+// Unscented-transform projection of one Gaussian (gsplat/ProjectionUT3DGSFused.cu:47-210,
+// gsplat/Cameras.cuh:1064-1186, 416-455).  Returns false when the Gaussian is culled.
+// ---------------------------------------------------------------------------------------------
+struct ProjOut {
+    float rx, ry;     // radii (already ceil'ed)
+    float mx, my;     // mean2d
+    float depth;      // camera z of the mean under the centre-of-shutter pose
+    float c0, c1, c2; // conic
+    float compensation;
+};
+
+struct ProjCfg {
+    uint32_t W, H;
+    float eps2d, near_plane, far_plane, radius_clip;
+    float ut_alpha, ut_beta, ut_kappa, ut_margin;
+    int ut_require_all;
+    float fx, fy, cx, cy;
+};
+
+__device__ __forceinline__ bool pinhole_project(vec3 cam, const ProjCfg& cfg, vec2* out) {
+    out->x = 0.f;
+    out->y = 0.f;
+    if (cam.z <= 0.f)
+        return false;
+    out->x = (cam.x / cam.z) * cfg.fx + cfg.cx;
+    out->y = (cam.y / cam.z) * cfg.fy + cfg.cy;
+    const float mx = (float)cfg.W * cfg.ut_margin;
+    const float my = (float)cfg.H * cfg.ut_margin;
+    bool valid = true;
+    valid &= (-mx) <= out->x && out->x < ((float)cfg.W + mx);
+    valid &= (-my) <= out->y && out->y < ((float)cfg.H + my);
+    return valid;
+}
+
+__device__ __forceinline__ bool project_ut(const ProjCfg& cfg, const CamPose& cp, vec3 mean, quat q_in, vec3 scl,
+                                           bool has_opacity, float opacity_in, ProjOut* o) {
+    const quat q = quat_normalize(q_in);
+    quat qc;
+    vec3 tc;
+    shutter_pose(cp, 0.5f, &qc, &tc);
+    const vec3 mean_c = add(quat_rotate(qc, mean), tc);
+    if (mean_c.z < cfg.near_plane || mean_c.z > cfg.far_plane)
+        return false;
+
+    const float D = 3.0f;
+    const float lambda = cfg.ut_alpha * cfg.ut_alpha * (D + cfg.ut_kappa) - D;
+    const mat3 Rg = mat3_cast(q);
+    const float sq = gsx::sqrt(D + lambda);
+    const float w0m = lambda / (D + lambda);
+    const float w0c = lambda / (D + lambda) + (1.f - cfg.ut_alpha * cfg.ut_alpha + cfg.ut_beta);
+    const float wi = 1.f / (2.f * (D + lambda));
+    const float sc[3] = {scl.x, scl.y, scl.z};
+
+    vec2 ip[7];
+    vec2 m2 = {0.f, 0.f};
+    bool valid = cfg.ut_require_all != 0;
+#pragma unroll
+    for (int i = 0; i < 7; ++i) {
+        vec3 p;
+        if (i == 0) {
+            p = mean;
+        } else {
+            const int a = (i - 1) % 3;
+            const float s = sq * sc[a];
+            const vec3 delta = mk3(s * Rg.m[0][a], s * Rg.m[1][a], s * Rg.m[2][a]);
+            p = (i <= 3) ? add(mean, delta) : sub(mean, delta);
+        }
+        const vec3 pc = add(quat_rotate(cp.q_start, p), cp.t_start);
+        vec2 uv;
+        const bool pv = pinhole_project(pc, cfg, &uv);
+        if (cfg.ut_require_all) {
+            valid &= pv;
+            if (!pv)
+                return false;
+        } else {
+            valid |= pv;
+        }
+        ip[i] = uv;
+        const float w = (i == 0) ? w0m : wi;
+        m2.x += w * uv.x;
+        m2.y += w * uv.y;
+    }
+    if (!valid)
+        return false;
+    float c00 = 0.f, c01 = 0.f, c11 = 0.f;
+#pragma unroll
+    for (int i = 0; i < 7; ++i) {
+        const float w = (i == 0) ? w0c : wi;
+        const float dx = ip[i].x - m2.x, dy = ip[i].y - m2.y;
+        c00 += w * (dx * dx);
+        c01 += w * (dx * dy);
+        c11 += w * (dy * dy);
+    }
+    // add_blur (gsplat/Utils.cuh:171-179)
+    const float det_orig = c00 * c11 - c01 * c01;
+    c00 += cfg.eps2d;
+    c11 += cfg.eps2d;
+    const float det = c00 * c11 - c01 * c01;
+    const float compensation = gsx::sqrt(gsx::fmax(0.f, det_orig / det));
+    if (det <= 0.f)
+        return false;
+    const float ood = 1.0f / det;
+
+    float extend = 3.33f;
+    if (has_opacity) {
+        const float opacity = opacity_in * compensation;
+        if (opacity < kAlphaThreshold)
+            return false;
+        extend = gsx::fmin(extend, gsx::sqrt(2.0f * gsx::log(opacity / kAlphaThreshold)));
+    }
+    const float b = 0.5f * (c00 + c11);
+    const float tmp = gsx::sqrt(gsx::fmax(0.01f, b * b - det));
+    const float v1 = b + tmp;
+    const float r1 = extend * gsx::sqrt(v1);
+    const float radius_x = gsx::ceil(gsx::fmin(extend * gsx::sqrt(c00), r1));
+    const float radius_y = gsx::ceil(gsx::fmin(extend * gsx::sqrt(c11), r1));
+    if (radius_x <= cfg.radius_clip && radius_y <= cfg.radius_clip)
+        return false;
+    if (m2.x + radius_x <= 0 || m2.x - radius_x >= (float)cfg.W || m2.y + radius_y <= 0 ||
+        m2.y - radius_y >= (float)cfg.H)
+        return false;
+    o->rx = radius_x;
+    o->ry = radius_y;
+    o->mx = m2.x;
+    o->my = m2.y;
+    o->depth = mean_c.z;
+    o->c0 = c11 * ood;
+    o->c1 = -c01 * ood;
+    o->c2 = c00 * ood;
+    o->compensation = compensation;
+    return true;
+}
+
+__global__ void __launch_bounds__(256) projection_ut_kernel(
+    uint32_t C, uint32_t N, const float* __restrict__ means, const float* __restrict__ quats,
+    const float* __restrict__ scales, const float* __restrict__ opacities, const float* __restrict__ viewmats0,
+    const float* __restrict__ Ks, ProjCfg cfg, int32_t* __restrict__ radii, float* __restrict__ means2d,
+    float* __restrict__ depths, float* __restrict__ conics, float* __restrict__ compensations) {
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= C * N)
+        return;
+    const uint32_t cid = idx / N, gid = idx % N;
+    cfg.fx = Ks[cid * 9 + 0];
+    cfg.fy = Ks[cid * 9 + 4];
+    cfg.cx = Ks[cid * 9 + 2];
+    cfg.cy = Ks[cid * 9 + 5];
+    const CamPose cp = load_cam_pose(viewmats0 + cid * 16);
+    ProjOut o;
+    const bool ok = project_ut(cfg, cp, ld3(means, gid), ld4q(quats, gid), ld3(scales, gid), opacities != nullptr,
+                               opacities != nullptr ? opacities[gid] : 0.f, &o);
+    int2* r2 = reinterpret_cast<int2*>(radii);
+    if (!ok) {
+        r2[idx] = make_int2(0, 0);
+        return;
+    }
+    r2[idx] = make_int2((int32_t)o.rx, (int32_t)o.ry);
+    reinterpret_cast<float2*>(means2d)[idx] = make_float2(o.mx, o.my);
+    depths[idx] = o.depth;
+    conics[idx * 3 + 0] = o.c0;
+    conics[idx * 3 + 1] = o.c1;
+    conics[idx * 3 + 2] = o.c2;
+    if (compensations != nullptr)
+        compensations[idx] = o.compensation;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Spherical harmonics (gsplat/SphericalHarmonicsCUDA.cu:20-110): basis values and the colour of one
+// channel in the reference's summation order.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ int sh_basis(uint32_t degree, vec3 dir, float* B) {
+    B[0] = 0.2820947917738781f;
+    if (degree < 1)
+        return 1;
+    const float inorm = gsx::rsqrt(dir.x * dir.x + dir.y * dir.y + dir.z * dir.z);
+    const float x = dir.x * inorm, y = dir.y * inorm, z = dir.z * inorm;
+    B[1] = -0.48860251190292f * y;
+    B[2] = 0.48860251190292f * z;
+    B[3] = -0.48860251190292f * x;
+    if (degree < 2)
+        return 4;
+    const float z2 = z * z;
+    const float fTmp0B = -1.092548430592079f * z;
+    const float fC1 = x * x - y * y;
+    const float fS1 = 2.f * x * y;
+    B[6] = (0.9461746957575601f * z2 - 0.3153915652525201f);
+    B[7] = fTmp0B * x;
+    B[5] = fTmp0B * y;
+    B[8] = 0.5462742152960395f * fC1;
+    B[4] = 0.5462742152960395f * fS1;
+    if (degree < 3)
+        return 9;
+    const float fTmp0C = -2.285228997322329f * z2 + 0.4570457994644658f;
+    const float fTmp1B = 1.445305721320277f * z;
+    const float fC2 = x * fC1 - y * fS1;
+    const float fS2 = x * fS1 + y * fC1;
+    B[12] = z * (1.865881662950577f * z2 - 1.119528997770346f);
+    B[13] = fTmp0C * x;
+    B[11] = fTmp0C * y;
+    B[14] = fTmp1B * fC1;
+    B[10] = fTmp1B * fS1;
+    B[15] = -0.5900435899266435f * fC2;
+    B[9] = -0.5900435899266435f * fS2;
+    if (degree < 4)
+        return 16;
+    const float fTmp0D = z * (-4.683325804901025f * z2 + 2.007139630671868f);
+    const float fTmp1C = 3.31161143515146f * z2 - 0.47308734787878f;
+    const float fTmp2B = -1.770130769779931f * z;
+    const float fC3 = x * fC2 - y * fS2;
+    const float fS3 = x * fS2 + y * fC2;
+    B[20] = (1.984313483298443f * z * B[12] - 1.006230589874905f * B[6]);
+    B[21] = fTmp0D * x;
+    B[19] = fTmp0D * y;
+    B[22] = fTmp1C * fC1;
+    B[18] = fTmp1C * fS1;
+    B[23] = fTmp2B * fC2;
+    B[17] = fTmp2B * fS2;
+    B[24] = 0.6258357354491763f * fC3;
+    B[16] = 0.6258357354491763f * fS3;
+    return 25;
+}
+
+// co: the Gaussian's coefficients, element (k, c) at co[k * 3 + c]
+__device__ __forceinline__ float sh_color_channel(uint32_t degree, vec3 dir, const float* B,
+                                                  const float* __restrict__ co, uint32_t c) {
+    float result = 0.2820947917738781f * co[c];
+    if (degree >= 1) {
+        // same value as B[1..3] folded: 0.4886 * (-y k1 + z k2 - x k3), in the reference's order
+        const float inorm = gsx::rsqrt(dir.x * dir.x + dir.y * dir.y + dir.z * dir.z);
+        const float x = dir.x * inorm, y = dir.y * inorm, z = dir.z * inorm;
+        result += 0.48860251190292f * (-y * co[1 * 3 + c] + z * co[2 * 3 + c] - x * co[3 * 3 + c]);
+        if (degree >= 2) {
+            result += B[4] * co[4 * 3 + c] + B[5] * co[5 * 3 + c] + B[6] * co[6 * 3 + c] + B[7] * co[7 * 3 + c] +
+                      B[8] * co[8 * 3 + c];
+            if (degree >= 3) {
+                result += B[9] * co[9 * 3 + c] + B[10] * co[10 * 3 + c] + B[11] * co[11 * 3 + c] +
+                          B[12] * co[12 * 3 + c] + B[13] * co[13 * 3 + c] + B[14] * co[14 * 3 + c] +
+                          B[15] * co[15 * 3 + c];
+                if (degree >= 4) {
+                    result += B[16] * co[16 * 3 + c] + B[17] * co[17 * 3 + c] + B[18] * co[18 * 3 + c] +
+                              B[19] * co[19 * 3 + c] + B[20] * co[20 * 3 + c] + B[21] * co[21 * 3 + c] +
+                              B[22] * co[22 * 3 + c] + B[23] * co[23 * 3 + c] + B[24] * co[24 * 3 + c];
+                }
+            }
+        }
+    }
+    return result;
+}
+
+// One lane per element, all three channels (the reference uses one thread per (element, channel),
+// SphericalHarmonicsCUDA.cu:373-399); a lane's coefficient row is 12*K contiguous bytes.
+__global__ void __launch_bounds__(256) sh_fwd_kernel(uint32_t N, uint32_t K, uint32_t degree,
+                                                      const float* __restrict__ dirs,
+                                                      const float* __restrict__ coeffs,
+                                                      const uint8_t* __restrict__ masks,
+                                                      float* __restrict__ colors) {
+    const uint32_t e = blockIdx.x * 256u + threadIdx.x;
+    if (e >= N)
+        return;
+    if (masks != nullptr && !masks[e])
+        return;
+    const vec3 dir = ld3(dirs, e);
+    float B[25];
+    sh_basis(degree, dir, B);
+    const float* co = coeffs + (size_t)e * K * 3;
+#pragma unroll
+    for (uint32_t c = 0; c < 3; ++c)
+        colors[e * 3 + c] = sh_color_channel(degree, dir, B, co, c);
+}
+
+// VJP wrt the coefficients (SphericalHarmonicsCUDA.cu:112-371 with v_dir == nullptr): every entry of the
+// element's [K,3] row is written (zero for masked elements and bands above `degree`), so the caller needs no
+// memset.
+__global__ void __launch_bounds__(256) sh_bwd_kernel(uint32_t N, uint32_t K, uint32_t degree,
+                                                      const float* __restrict__ dirs,
+                                                      const uint8_t* __restrict__ masks,
+                                                      const float* __restrict__ v_colors,
+                                                      float* __restrict__ v_coeffs) {
+    const uint32_t e = blockIdx.x * 256u + threadIdx.x;
+    if (e >= N)
+        return;
+    float* out = v_coeffs + (size_t)e * K * 3;
+    const bool live = masks == nullptr || masks[e];
+    float B[25];
+    int nb = 0;
+    float v[3] = {0.f, 0.f, 0.f};
+    if (live) {
+        nb = sh_basis(degree, ld3(dirs, e), B);
+#pragma unroll
+        for (int c = 0; c < 3; ++c)
+            v[c] = v_colors[e * 3 + c];
+    }
+    for (uint32_t k = 0; k < K; ++k) {
+        const float b = ((int)k < nb) ? B[k < 25 ? k : 24] : 0.f;
+        out[k * 3 + 0] = b * v[0];
+        out[k * 3 + 1] = b * v[1];
+        out[k * 3 + 2] = b * v[2];
+    }
+}
+
+// direction gradient (degree <= 3), accumulated over the three channels
+// (sh_coeffs_to_color_fast_vjp with v_dir != nullptr; the reference adds the channels with atomics, :474-478)
+__global__ void __launch_bounds__(256) sh_bwd_dirs_kernel(uint32_t N, uint32_t K, uint32_t degree,
+                                                           const float* __restrict__ dirs,
+                                                           const float* __restrict__ coeffs,
+                                                           const uint8_t* __restrict__ masks,
+                                                           const float* __restrict__ v_colors,
+                                                           float* __restrict__ v_dirs) {
+    const uint32_t e = blockIdx.x * 256u + threadIdx.x;
+    if (e >= N)
+        return;
+    if (masks != nullptr && !masks[e])
+        return;
+    const vec3 dir = ld3(dirs, e);
+    float vx = 0.f, vy = 0.f, vz = 0.f;
+    if (degree >= 1) {
+        const float inorm = gsx::rsqrt(dir.x * dir.x + dir.y * dir.y + dir.z * dir.z);
+        const float x = dir.x * inorm, y = dir.y * inorm, z = dir.z * inorm;
+        const float* co = coeffs + (size_t)e * K * 3;
+        for (uint32_t c = 0; c < 3; ++c) {
+            const float v = v_colors[e * 3 + c];
+            float v_x = 0.f, v_y = 0.f, v_z = 0.f;
+            v_x += -0.48860251190292f * co[3 * 3 + c] * v;
+            v_y += -0.48860251190292f * co[1 * 3 + c] * v;
+            v_z += 0.48860251190292f * co[2 * 3 + c] * v;
+            float fC1 = 0, fS1 = 0, fC1_x = 0, fC1_y = 0, fS1_x = 0, fS1_y = 0;
+            const float z2 = z * z;
+            if (degree >= 2) {
+                const float fTmp0B = -1.092548430592079f * z;
+                fC1 = x * x - y * y;
+                fS1 = 2.f * x * y;
+                const float fTmp0B_z = -1.092548430592079f;
+                fC1_x = 2.f * x;
+                fC1_y = -2.f * y;
+                fS1_x = 2.f * y;
+                fS1_y = 2.f * x;
+                const float pSH6_z = 2.f * 0.9461746957575601f * z;
+                const float pSH7_x = fTmp0B, pSH7_z = fTmp0B_z * x;
+                const float pSH5_y = fTmp0B, pSH5_z = fTmp0B_z * y;
+                const float pSH8_x = 0.5462742152960395f * fC1_x, pSH8_y = 0.5462742152960395f * fC1_y;
+                const float pSH4_x = 0.5462742152960395f * fS1_x, pSH4_y = 0.5462742152960395f * fS1_y;
+                v_x += v * (pSH4_x * co[4 * 3 + c] + pSH8_x * co[8 * 3 + c] + pSH7_x * co[7 * 3 + c]);
+                v_y += v * (pSH4_y * co[4 * 3 + c] + pSH8_y * co[8 * 3 + c] + pSH5_y * co[5 * 3 + c]);
+                v_z += v * (pSH6_z * co[6 * 3 + c] + pSH7_z * co[7 * 3 + c] + pSH5_z * co[5 * 3 + c]);
+            }
+            if (degree >= 3) {
+                const float fTmp0C = -2.285228997322329f * z2 + 0.4570457994644658f;
+                const float fTmp1B = 1.445305721320277f * z;
+                const float fTmp0C_z = -2.285228997322329f * 2.f * z;
+                const float fTmp1B_z = 1.445305721320277f;
+                const float fC2_x = fC1 + x * fC1_x - y * fS1_x;
+                const float fC2_y = x * fC1_y - fS1 - y * fS1_y;
+                const float fS2_x = fS1 + x * fS1_x + y * fC1_x;
+                const float fS2_y = x * fS1_y + fC1 + y * fC1_y;
+                const float pSH12_z = 3.f * 1.865881662950577f * z2 - 1.119528997770346f;
+                const float pSH13_x = fTmp0C, pSH13_z = fTmp0C_z * x;
+                const float pSH11_y = fTmp0C, pSH11_z = fTmp0C_z * y;
+                const float pSH14_x = fTmp1B * fC1_x, pSH14_y = fTmp1B * fC1_y, pSH14_z = fTmp1B_z * fC1;
+                const float pSH10_x = fTmp1B * fS1_x, pSH10_y = fTmp1B * fS1_y, pSH10_z = fTmp1B_z * fS1;
+                const float pSH15_x = -0.5900435899266435f * fC2_x, pSH15_y = -0.5900435899266435f * fC2_y;
+                const float pSH9_x = -0.5900435899266435f * fS2_x, pSH9_y = -0.5900435899266435f * fS2_y;
+                v_x += v * (pSH9_x * co[9 * 3 + c] + pSH15_x * co[15 * 3 + c] + pSH10_x * co[10 * 3 + c] +
+                            pSH14_x * co[14 * 3 + c] + pSH13_x * co[13 * 3 + c]);
+                v_y += v * (pSH9_y * co[9 * 3 + c] + pSH15_y * co[15 * 3 + c] + pSH10_y * co[10 * 3 + c] +
+                            pSH14_y * co[14 * 3 + c] + pSH11_y * co[11 * 3 + c]);
+                v_z += v * (pSH12_z * co[12 * 3 + c] + pSH13_z * co[13 * 3 + c] + pSH11_z * co[11 * 3 + c] +
+                            pSH14_z * co[14 * 3 + c] + pSH10_z * co[10 * 3 + c]);
+            }
+            const float d = v_x * x + v_y * y + v_z * z;
+            vx += (v_x - d * x) * inorm;
+            vy += (v_y - d * y) * inorm;
+            vz += (v_z - d * z) * inorm;
+        }
+    }
+    v_dirs[e * 3 + 0] = vx;
+    v_dirs[e * 3 + 1] = vy;
+    v_dirs[e * 3 + 2] = vz;
+}
+
+__global__ void __launch_bounds__(256) quats_to_rotmats_kernel(uint32_t N, const float* __restrict__ quats,
+                                                                float* __restrict__ rotmats) {
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= N)
+        return;
+    const mat3 R = quat_to_rotmat(ld4q(quats, idx));
+#pragma unroll
+    for (int i = 0; i < 3; ++i)
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+            rotmats[(size_t)idx * 9 + i * 3 + j] = R.m[i][j];
+}
+
+// SplatData getters (src/core/splat_data.cpp:271-286) in one pass
+__global__ void __launch_bounds__(256) activate_params_kernel(uint32_t N, const float* __restrict__ opacity_raw,
+                                                               const float* __restrict__ scaling_raw,
+                                                               const float* __restrict__ rotation_raw,
+                                                               float* __restrict__ opacities,
+                                                               float* __restrict__ scales, float* __restrict__ quats) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= N)
+        return;
+    opacities[i] = gsx::sigmoid(opacity_raw[i]);
+    const vec3 s = ld3(scaling_raw, i);
+    scales[3 * i + 0] = gsx::exp(s.x);
+    scales[3 * i + 1] = gsx::exp(s.y);
+    scales[3 * i + 2] = gsx::exp(s.z);
+    const quat q = ld4q(rotation_raw, i);
+    // torch::nn::functional::normalize: x / max(||x||_2, eps), eps = 1e-12
+    const float nrm = gsx::fmax(gsx::sqrt(qdot(q, q)), 1e-12f);
+    reinterpret_cast<float4*>(quats)[i] = make_float4(q.w / nrm, q.x / nrm, q.y / nrm, q.z / nrm);
+}
+
+// VJPs of the three activations (what autograd applies to the gradients Ops.h's backward returns)
+__global__ void __launch_bounds__(256) activate_params_bwd_kernel(
+    uint32_t N, const float* __restrict__ opacity_raw, const float* __restrict__ scaling_raw,
+    const float* __restrict__ rotation_raw, const float* __restrict__ v_opacities, const float* __restrict__ v_scales,
+    const float* __restrict__ v_quats, float* __restrict__ v_opacity_raw, float* __restrict__ v_scaling_raw,
+    float* __restrict__ v_rotation_raw) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= N)
+        return;
+    const float o = gsx::sigmoid(opacity_raw[i]);
+    v_opacity_raw[i] = v_opacities[i] * (o * (1.0f - o));
+    const vec3 s = ld3(scaling_raw, i);
+    v_scaling_raw[3 * i + 0] = v_scales[3 * i + 0] * gsx::exp(s.x);
+    v_scaling_raw[3 * i + 1] = v_scales[3 * i + 1] * gsx::exp(s.y);
+    v_scaling_raw[3 * i + 2] = v_scales[3 * i + 2] * gsx::exp(s.z);
+    const quat q = ld4q(rotation_raw, i);
+    const quat g = ld4q(v_quats, i);
+    const float len = gsx::sqrt(qdot(q, q));
+    float4 out;
+    if (len > 1e-12f) {
+        // y = x / len : v_x = (g - y (y . g)) / len
+        const float inv = 1.0f / len;
+        const float yw = q.w * inv, yx = q.x * inv, yy = q.y * inv, yz = q.z * inv;
+        const float d = g.w * yw + g.x * yx + g.y * yy + g.z * yz;
+        out = make_float4((g.w - yw * d) * inv, (g.x - yx * d) * inv, (g.y - yy * d) * inv, (g.z - yz * d) * inv);
+    } else {
+        out = make_float4(g.w * 1e12f, g.x * 1e12f, g.y * 1e12f, g.z * 1e12f);
+    }
+    reinterpret_cast<float4*>(v_rotation_raw)[i] = out;
+}
+
+// campos = translation column of inverse([R|t]) = -R^T t (Rasterization.cpp:358-359 uses at::inverse; for the
+// rigid matrices LichtFeld passes the two agree).  Evaluated per lane from the uniform matrix: the matrix
+// lives in device memory and a host copy would cost a synchronisation.
+__device__ __forceinline__ vec3 campos_from_viewmat(const float* __restrict__ vm) {
+    mat3 R;
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int c = 0; c < 3; ++c)
+            R.m[r][c] = vm[r * 4 + c];
+    return neg(mul_t(R, mk3(vm[3], vm[7], vm[11])));
+}
+
+// glue of the fused entry point (Rasterization.cpp:356-378): dirs, radii mask, SH, +0.5, clamp in one pass
+__global__ void __launch_bounds__(256) sh_world_fwd_kernel(uint32_t N, uint32_t K, uint32_t degree,
+                                                            const float* __restrict__ means,
+                                                            const float* __restrict__ coeffs,
+                                                            const int32_t* __restrict__ radii,
+                                                            const float* __restrict__ viewmat,
+                                                            float* __restrict__ colors) {
+    const uint32_t e = blockIdx.x * 256u + threadIdx.x;
+    if (e >= N)
+        return;
+    if (!(radii[e * 2] > 0 && radii[e * 2 + 1] > 0)) {
+        colors[e * 3 + 0] = 0.f;
+        colors[e * 3 + 1] = 0.f;
+        colors[e * 3 + 2] = 0.f;
+        return;
+    }
+    const vec3 dir = sub(ld3(means, e), campos_from_viewmat(viewmat));
+    float B[25];
+    sh_basis(degree, dir, B);
+    const float* co = coeffs + (size_t)e * K * 3;
+#pragma unroll
+    for (uint32_t c = 0; c < 3; ++c)
+        colors[e * 3 + c] = gsx::fmax(sh_color_channel(degree, dir, B, co, c) + 0.5f, 0.0f);
+}
+
+__global__ void __launch_bounds__(256) sh_world_bwd_kernel(uint32_t N, uint32_t K, uint32_t degree,
+                                                            const float* __restrict__ means,
+                                                            const int32_t* __restrict__ radii,
+                                                            const float* __restrict__ viewmat,
+                                                            const float* __restrict__ colors,
+                                                            const float* __restrict__ v_colors,
+                                                            float* __restrict__ v_coeffs) {
+    const uint32_t e = blockIdx.x * 256u + threadIdx.x;
+    if (e >= N)
+        return;
+    float* out = v_coeffs + (size_t)e * K * 3;
+    const bool live = radii[e * 2] > 0 && radii[e * 2 + 1] > 0;
+    float B[25];
+    int nb = 0;
+    float v[3] = {0.f, 0.f, 0.f};
+    if (live) {
+        const vec3 dir = sub(ld3(means, e), campos_from_viewmat(viewmat));
+        nb = sh_basis(degree, dir, B);
+#pragma unroll
+        for (int c = 0; c < 3; ++c)
+            v[c] = colors[e * 3 + c] <= 0.0f ? 0.f : v_colors[e * 3 + c];
+    }
+    for (uint32_t k = 0; k < K; ++k) {
+        const float b = ((int)k < nb) ? B[k < 25 ? k : 24] : 0.f;
+        out[k * 3 + 0] = b * v[0];
+        out[k * 3 + 1] = b * v[1];
+        out[k * 3 + 2] = b * v[2];
+    }
+}
+} // namespace gsx
+
+using namespace gsx;
+
+// =============================================================================================
+// C ABI
+// =============================================================================================
+
+extern "C" int gsx_projection_ut_3dgs_fused(
+    uint32_t C, uint32_t N, const float* means, const float* quats, const float* scales, const float* opacities,
+    const float* viewmats0, const float* viewmats1, const float* Ks, uint32_t image_width, uint32_t image_height,
+    float eps2d, float near_plane, float far_plane, float radius_clip, int camera_model, gsx_ut_params ut,
+    int rs_type, const float* radial_coeffs, const float* tangential_coeffs, const float* thin_prism_coeffs,
+    int32_t* radii, float* means2d, float* depths, float* conics, float* compensations, void* stream) {
+    if ((uint64_t)C * N == 0)
+        return GSX_OK; // ProjectionUT3DGSFused.cu:249-252
+    GSX_REQUIRE(means && quats && scales && viewmats0 && Ks && radii && means2d && depths && conics,
+                GSX_ERR_INVALID_ARGUMENT, "projection_ut_3dgs_fused: null tensor");
+    GSX_REQUIRE((uint64_t)C * N < (1ull << 31), GSX_ERR_INVALID_ARGUMENT, "projection_ut_3dgs_fused: C*N >= 2^31");
+    const int rc = check_camera_args(C, viewmats1, camera_model, rs_type, radial_coeffs, tangential_coeffs,
+                                     thin_prism_coeffs);
+    if (rc != GSX_OK)
+        return rc;
+    ProjCfg cfg;
+    cfg.W = image_width;
+    cfg.H = image_height;
+    cfg.eps2d = eps2d;
+    cfg.near_plane = near_plane;
+    cfg.far_plane = far_plane;
+    cfg.radius_clip = radius_clip;
+    cfg.ut_alpha = ut.alpha;
+    cfg.ut_beta = ut.beta;
+    cfg.ut_kappa = ut.kappa;
+    cfg.ut_margin = ut.in_image_margin_factor;
+    cfg.ut_require_all = ut.require_all_sigma_points_valid;
+    cfg.fx = cfg.fy = cfg.cx = cfg.cy = 0.f;
+    hipLaunchKernelGGL(projection_ut_kernel, dim3(cdiv((uint64_t)C * N, 256)), dim3(256), 0, (hipStream_t)stream, C,
+                       N, means, quats, scales, opacities, viewmats0, Ks, cfg, radii, means2d, depths, conics,
+                       compensations);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+extern "C" int gsx_spherical_harmonics_fwd(uint32_t N, uint32_t K, uint32_t degrees_to_use, const float* dirs,
+                                           const float* coeffs, const uint8_t* masks, float* colors, void* stream) {
+    if (N == 0)
+        return GSX_OK;
+    GSX_REQUIRE(dirs && coeffs && colors, GSX_ERR_INVALID_ARGUMENT, "spherical_harmonics_fwd: null tensor");
+    GSX_REQUIRE(degrees_to_use <= 4 && K >= (degrees_to_use + 1) * (degrees_to_use + 1), GSX_ERR_INVALID_ARGUMENT,
+                "spherical_harmonics_fwd: degree %u needs K >= %u (got %u)", degrees_to_use,
+                (degrees_to_use + 1) * (degrees_to_use + 1), K);
+    hipLaunchKernelGGL(sh_fwd_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, K, degrees_to_use,
+                       dirs, coeffs, masks, colors);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+extern "C" int gsx_spherical_harmonics_bwd(uint32_t N, uint32_t K, uint32_t degrees_to_use, const float* dirs,
+                                           const float* coeffs, const uint8_t* masks, const float* v_colors,
+                                           float* v_coeffs, float* v_dirs, void* stream) {
+    if (N == 0)
+        return GSX_OK;
+    GSX_REQUIRE(dirs && coeffs && v_colors && v_coeffs, GSX_ERR_INVALID_ARGUMENT,
+                "spherical_harmonics_bwd: null tensor");
+    GSX_REQUIRE(degrees_to_use <= 4 && K >= (degrees_to_use + 1) * (degrees_to_use + 1), GSX_ERR_INVALID_ARGUMENT,
+                "spherical_harmonics_bwd: degree %u needs K >= %u (got %u)", degrees_to_use,
+                (degrees_to_use + 1) * (degrees_to_use + 1), K);
+    GSX_REQUIRE(v_dirs == nullptr || degrees_to_use <= 3, GSX_ERR_UNSUPPORTED,
+                "spherical_harmonics_bwd: v_dirs is implemented for degree <= 3");
+    hipLaunchKernelGGL(sh_bwd_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, K, degrees_to_use,
+                       dirs, masks, v_colors, v_coeffs);
+    GSX_LAUNCH_CHECK();
+    if (v_dirs != nullptr) {
+        hipLaunchKernelGGL(sh_bwd_dirs_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, K,
+                           degrees_to_use, dirs, coeffs, masks, v_colors, v_dirs);
+        GSX_LAUNCH_CHECK();
+    }
+    return GSX_OK;
+}
+
+extern "C" int gsx_sh_colors_from_world(uint32_t N, uint32_t K, uint32_t sh_degree, const float* means,
+                                        const float* sh_coeffs, const int32_t* radii, const float* viewmat,
+                                        float* colors, void* stream) {
+    if (N == 0)
+        return GSX_OK;
+    GSX_REQUIRE(means && sh_coeffs && radii && viewmat && colors, GSX_ERR_INVALID_ARGUMENT,
+                "sh_colors_from_world: null tensor");
+    GSX_REQUIRE(sh_degree <= 4 && K >= (sh_degree + 1) * (sh_degree + 1), GSX_ERR_INVALID_ARGUMENT,
+                "sh_colors_from_world: degree %u needs K >= %u (got %u)", sh_degree, (sh_degree + 1) * (sh_degree + 1),
+                K);
+    hipLaunchKernelGGL(sh_world_fwd_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, K, sh_degree,
+                       means, sh_coeffs, radii, viewmat, colors);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+extern "C" int gsx_sh_colors_from_world_bwd(uint32_t N, uint32_t K, uint32_t sh_degree, const float* means,
+                                            const int32_t* radii, const float* viewmat, const float* colors,
+                                            const float* v_colors, float* v_sh_coeffs, void* stream) {
+    if (N == 0)
+        return GSX_OK;
+    GSX_REQUIRE(means && radii && viewmat && colors && v_colors && v_sh_coeffs, GSX_ERR_INVALID_ARGUMENT,
+                "sh_colors_from_world_bwd: null tensor");
+    GSX_REQUIRE(sh_degree <= 4 && K >= (sh_degree + 1) * (sh_degree + 1), GSX_ERR_INVALID_ARGUMENT,
+                "sh_colors_from_world_bwd: degree %u needs K >= %u (got %u)", sh_degree,
+                (sh_degree + 1) * (sh_degree + 1), K);
+    hipLaunchKernelGGL(sh_world_bwd_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, K, sh_degree,
+                       means, radii, viewmat, colors, v_colors, v_sh_coeffs);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+extern "C" int gsx_quats_to_rotmats(int N, const float* quats, float* rotmats, void* stream) {
+    if (N <= 0)
+        return GSX_OK;
+    GSX_REQUIRE(quats && rotmats, GSX_ERR_INVALID_ARGUMENT, "quats_to_rotmats: null tensor");
+    hipLaunchKernelGGL(quats_to_rotmats_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, (uint32_t)N,
+                       quats, rotmats);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+extern "C" int gsx_activate_params(uint32_t N, const float* opacity_raw, const float* scaling_raw,
+                                   const float* rotation_raw, float* opacities, float* scales, float* quats,
+                                   void* stream) {
+    if (N == 0)
+        return GSX_OK;
+    GSX_REQUIRE(opacity_raw && scaling_raw && rotation_raw && opacities && scales && quats, GSX_ERR_INVALID_ARGUMENT,
+                "activate_params: null tensor");
+    hipLaunchKernelGGL(activate_params_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, opacity_raw,
+                       scaling_raw, rotation_raw, opacities, scales, quats);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+extern "C" int gsx_activate_params_bwd(uint32_t N, const float* opacity_raw, const float* scaling_raw,
+                                       const float* rotation_raw, const float* v_opacities, const float* v_scales,
+                                       const float* v_quats, float* v_opacity_raw, float* v_scaling_raw,
+                                       float* v_rotation_raw, void* stream) {
+    if (N == 0)
+        return GSX_OK;
+    GSX_REQUIRE(opacity_raw && scaling_raw && rotation_raw && v_opacities && v_scales && v_quats && v_opacity_raw &&
+                    v_scaling_raw && v_rotation_raw,
+                GSX_ERR_INVALID_ARGUMENT, "activate_params_bwd: null tensor");
+    hipLaunchKernelGGL(activate_params_bwd_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N,
+                       opacity_raw, scaling_raw, rotation_raw, v_opacities, v_scales, v_quats, v_opacity_raw,
+                       v_scaling_raw, v_rotation_raw);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}

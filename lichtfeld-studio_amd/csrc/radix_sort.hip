@@ -1,0 +1,251 @@
+// radix_sort.hip - stable LSD radix sort of (int64 key, int32 value) pairs on key bits [0, end_bit)
+// (gsplat/IntersectTile.cu:290-328 calls cub::DeviceRadixSort::SortPairs with a DoubleBuffer).
+//
+// 8-bit digits.  Per pass: block histograms -> exclusive scan of the digit-major histogram table ->
+// stable scatter.  A block owns 4096 consecutive pairs; inside the block each 64-lane wave owns 1024
+// consecutive pairs and ranks them 64 at a time with wave-wide match masks built from ballots, so the
+// order (wave, round, lane) equals the input order and the sort is stable.
+#include "gsx_common.h"
+
+namespace gsx {
+
+static constexpr uint32_t kRadixBits = 8;
+static constexpr uint32_t kRadix = 1u << kRadixBits;
+static constexpr uint32_t kSortItems = 16;
+static constexpr uint32_t kSortTile = 256 * kSortItems; // pairs per block
+static constexpr uint32_t kWaveTile = 64 * kSortItems;  // pairs per wave
+
+__device__ __forceinline__ uint32_t digit_of(int64_t key, uint32_t shift, uint32_t mask) {
+    return (uint32_t)((uint64_t)key >> shift) & mask;
+}
+
+__global__ void __launch_bounds__(256) radix_hist_kernel(uint32_t n, const int64_t* __restrict__ keys,
+                                                          uint32_t shift, uint32_t mask, uint32_t nblocks,
+                                                          uint32_t* __restrict__ hist /*[kRadix][nblocks]*/) {
+    __shared__ uint32_t lh[kRadix];
+    lh[threadIdx.x] = 0;
+    __syncthreads();
+    const uint32_t base = blockIdx.x * kSortTile;
+#pragma unroll
+    for (uint32_t i = 0; i < kSortItems; ++i) {
+        const uint32_t idx = base + i * 256u + threadIdx.x;
+        if (idx < n)
+            atomicAdd(&lh[digit_of(keys[idx], shift, mask)], 1u);
+    }
+    __syncthreads();
+    hist[threadIdx.x * nblocks + blockIdx.x] = lh[threadIdx.x];
+}
+
+// ---- exclusive scan of a uint32 array (three passes) ---------------------------------------------
+static constexpr uint32_t kScanItems = 8;
+static constexpr uint32_t kScanTile = 256 * kScanItems;
+
+__device__ __forceinline__ uint32_t block_exclusive_scan_u32(uint32_t v, uint32_t* lds, uint32_t* total) {
+    const uint32_t t = threadIdx.x;
+    lds[t] = v;
+    __syncthreads();
+#pragma unroll
+    for (uint32_t off = 1; off < 256; off <<= 1) {
+        const uint32_t add = (t >= off) ? lds[t - off] : 0;
+        __syncthreads();
+        lds[t] += add;
+        __syncthreads();
+    }
+    const uint32_t incl = lds[t];
+    *total = lds[255];
+    __syncthreads();
+    return incl - v;
+}
+
+__global__ void __launch_bounds__(256) scan_u32_sums_kernel(uint32_t n, const uint32_t* __restrict__ in,
+                                                             uint32_t* __restrict__ sums) {
+    __shared__ uint32_t lds[256];
+    const uint32_t base = blockIdx.x * kScanTile + threadIdx.x * kScanItems;
+    uint32_t s = 0;
+#pragma unroll
+    for (uint32_t i = 0; i < kScanItems; ++i)
+        if (base + i < n)
+            s += in[base + i];
+    uint32_t total;
+    block_exclusive_scan_u32(s, lds, &total);
+    if (threadIdx.x == 0)
+        sums[blockIdx.x] = total;
+}
+
+__global__ void __launch_bounds__(256) scan_u32_offsets_kernel(uint32_t nb, uint32_t* __restrict__ sums) {
+    __shared__ uint32_t lds[256];
+    uint32_t carry = 0;
+    for (uint32_t start = 0; start < nb; start += 256) {
+        const uint32_t i = start + threadIdx.x;
+        const uint32_t v = i < nb ? sums[i] : 0;
+        uint32_t total;
+        const uint32_t ex = block_exclusive_scan_u32(v, lds, &total);
+        if (i < nb)
+            sums[i] = carry + ex;
+        carry += total;
+    }
+}
+
+__global__ void __launch_bounds__(256) scan_u32_apply_kernel(uint32_t n, uint32_t* __restrict__ data,
+                                                              const uint32_t* __restrict__ offsets) {
+    __shared__ uint32_t lds[256];
+    const uint32_t base = blockIdx.x * kScanTile + threadIdx.x * kScanItems;
+    uint32_t v[kScanItems];
+    uint32_t s = 0;
+#pragma unroll
+    for (uint32_t i = 0; i < kScanItems; ++i) {
+        v[i] = (base + i < n) ? data[base + i] : 0;
+        s += v[i];
+    }
+    uint32_t total;
+    uint32_t run = block_exclusive_scan_u32(s, lds, &total) + offsets[blockIdx.x];
+#pragma unroll
+    for (uint32_t i = 0; i < kScanItems; ++i) {
+        if (base + i < n)
+            data[base + i] = run;
+        run += v[i];
+    }
+}
+
+// ---- stable scatter -------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const int64_t* __restrict__ keys_in,
+                                                             const int32_t* __restrict__ vals_in,
+                                                             int64_t* __restrict__ keys_out,
+                                                             int32_t* __restrict__ vals_out, uint32_t shift,
+                                                             uint32_t mask, uint32_t nblocks,
+                                                             const uint32_t* __restrict__ hist_scanned) {
+    __shared__ uint32_t wave_count[4][kRadix];
+    const uint32_t t = threadIdx.x;
+    const uint32_t w = t >> 6, lane = t & 63u;
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i)
+        wave_count[i][t] = 0;
+    __syncthreads();
+
+    const uint32_t wave_base = blockIdx.x * kSortTile + w * kWaveTile;
+    const uint64_t lt_mask = (1ull << lane) - 1ull;
+    int64_t key[kSortItems];
+    int32_t val[kSortItems];
+    uint32_t rank[kSortItems]; // rank among the wave's pairs with the same digit
+#pragma unroll
+    for (uint32_t r = 0; r < kSortItems; ++r) {
+        const uint32_t idx = wave_base + r * 64u + lane;
+        const bool valid = idx < n;
+        key[r] = valid ? keys_in[idx] : 0;
+        val[r] = valid ? vals_in[idx] : 0;
+    }
+#pragma unroll
+    for (uint32_t r = 0; r < kSortItems; ++r) {
+        const uint32_t idx = wave_base + r * 64u + lane;
+        const bool valid = idx < n;
+        const uint32_t d = digit_of(key[r], shift, mask);
+        uint64_t peers = __ballot(valid);
+#pragma unroll
+        for (uint32_t b = 0; b < kRadixBits; ++b) {
+            const bool bit = (d >> b) & 1u;
+            const uint64_t m = __ballot(bit);
+            peers &= bit ? m : ~m;
+        }
+        uint32_t pre = 0;
+        if (valid)
+            pre = wave_count[w][d];
+        __builtin_amdgcn_wave_barrier();
+        rank[r] = pre + (uint32_t)__popcll(peers & lt_mask);
+        if (valid && (peers & lt_mask) == 0)
+            wave_count[w][d] = pre + (uint32_t)__popcll(peers);
+        __builtin_amdgcn_wave_barrier();
+    }
+    __syncthreads();
+    // digit t: global base of this block + counts of the lower waves
+    {
+        const uint32_t c0 = wave_count[0][t], c1 = wave_count[1][t], c2 = wave_count[2][t];
+        const uint32_t g = hist_scanned[t * nblocks + blockIdx.x];
+        __syncthreads();
+        wave_count[0][t] = g;
+        wave_count[1][t] = g + c0;
+        wave_count[2][t] = g + c0 + c1;
+        wave_count[3][t] = g + c0 + c1 + c2;
+    }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t r = 0; r < kSortItems; ++r) {
+        const uint32_t idx = wave_base + r * 64u + lane;
+        if (idx < n) {
+            const uint32_t pos = wave_count[w][digit_of(key[r], shift, mask)] + rank[r];
+            keys_out[pos] = key[r];
+            vals_out[pos] = val[r];
+        }
+    }
+}
+
+} // namespace gsx
+
+using namespace gsx;
+
+namespace {
+struct SortLayout {
+    uint32_t nblocks;
+    uint32_t hist_len;
+    uint32_t scan_blocks;
+    size_t hist_off, sums_off, total;
+};
+SortLayout sort_layout(int64_t n) {
+    SortLayout L;
+    L.nblocks = cdiv((uint64_t)n, kSortTile);
+    L.hist_len = L.nblocks * kRadix;
+    L.scan_blocks = cdiv(L.hist_len, kScanTile);
+    L.hist_off = 0;
+    L.sums_off = align_up((size_t)L.hist_len * 4, 256);
+    L.total = L.sums_off + align_up((size_t)L.scan_blocks * 4, 256);
+    return L;
+}
+} // namespace
+
+extern "C" size_t gsx_radix_sort_pairs_workspace_bytes(int64_t n) {
+    if (n <= 0)
+        return 256;
+    return sort_layout(n).total;
+}
+
+extern "C" int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, int64_t* keys1, int32_t* vals1,
+                                    uint32_t end_bit, void* workspace, size_t workspace_bytes, int* selector_host,
+                                    void* stream) {
+    if (selector_host)
+        *selector_host = 0;
+    if (n <= 0)
+        return GSX_OK; // IntersectTile.cu:298-300
+    GSX_REQUIRE(n < (1ll << 31), GSX_ERR_OVERFLOW, "radix_sort_pairs: n = %lld does not fit int32", (long long)n);
+    GSX_REQUIRE(keys0 && vals0 && keys1 && vals1, GSX_ERR_INVALID_ARGUMENT, "radix_sort_pairs: null buffer");
+    GSX_REQUIRE(end_bit >= 1 && end_bit <= 64, GSX_ERR_INVALID_ARGUMENT, "radix_sort_pairs: end_bit %u", end_bit);
+    const SortLayout L = sort_layout(n);
+    GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 && workspace_bytes >= L.total,
+                GSX_ERR_WORKSPACE, "radix_sort_pairs: workspace needs %zu bytes, 256-byte aligned", L.total);
+    uint32_t* hist = (uint32_t*)((char*)workspace + L.hist_off);
+    uint32_t* sums = (uint32_t*)((char*)workspace + L.sums_off);
+    hipStream_t s = (hipStream_t)stream;
+    int sel = 0;
+    for (uint32_t shift = 0; shift < end_bit; shift += kRadixBits) {
+        const uint32_t bits = (end_bit - shift) < kRadixBits ? (end_bit - shift) : kRadixBits;
+        const uint32_t mask = (1u << bits) - 1u;
+        const int64_t* kin = sel ? keys1 : keys0;
+        const int32_t* vin = sel ? vals1 : vals0;
+        int64_t* kout = sel ? keys0 : keys1;
+        int32_t* vout = sel ? vals0 : vals1;
+        hipLaunchKernelGGL(radix_hist_kernel, dim3(L.nblocks), dim3(256), 0, s, (uint32_t)n, kin, shift, mask,
+                           L.nblocks, hist);
+        GSX_LAUNCH_CHECK();
+        hipLaunchKernelGGL(scan_u32_sums_kernel, dim3(L.scan_blocks), dim3(256), 0, s, L.hist_len, hist, sums);
+        GSX_LAUNCH_CHECK();
+        hipLaunchKernelGGL(scan_u32_offsets_kernel, dim3(1), dim3(256), 0, s, L.scan_blocks, sums);
+        GSX_LAUNCH_CHECK();
+        hipLaunchKernelGGL(scan_u32_apply_kernel, dim3(L.scan_blocks), dim3(256), 0, s, L.hist_len, hist, sums);
+        GSX_LAUNCH_CHECK();
+        hipLaunchKernelGGL(radix_scatter_kernel, dim3(L.nblocks), dim3(256), 0, s, (uint32_t)n, kin, vin, kout, vout,
+                           shift, mask, L.nblocks, hist);
+        GSX_LAUNCH_CHECK();
+        sel ^= 1;
+    }
+    if (selector_host)
+        *selector_host = sel;
+    return GSX_OK;
+}

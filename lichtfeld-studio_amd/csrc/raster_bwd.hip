@@ -1,0 +1,368 @@
+// raster_bwd.hip - per-tile backward rasterizer "from world"
+// (gsplat/RasterizeToPixelsFromWorld3DGSBwd.cu:16-379, VJP helpers gsplat/Utils.cuh:104-158,186-194).
+//
+// Same tiling as the forward pass (one 256-lane workgroup per 16x16 tile, one lane per pixel, Gaussians staged
+// through LDS 256 at a time, walked back to front).  Two things are organised differently from the reference:
+//
+//  1. What is summed per Gaussian.  The reference pushes every (pixel, Gaussian) pair through the whole chain
+//     down to (v_mean, v_quat, v_scale) and reduces those 10 numbers.  That chain is linear in v_M = d L / d M
+//     (M = diag(1/s) R^T), and v_M = v_grd (x) ray_d + v_gro (x) (ray_o - mean) where ray_o is one constant per
+//     camera.  So the per-pair work stops at v_gro (3) and v_grd (x) ray_d (9); those are summed per Gaussian
+//     (with colour 3 and opacity 1: 16 floats) and a per-Gaussian epilogue applies the linear map once.
+//  2. How it is summed.  A 64-lane wave reduces its 16 partials with a halving butterfly (the array is split in
+//     two at each of the first four steps, so 8+4+2+1+1+1 = 17 exchanges instead of 16*6), after which 16 lanes
+//     hold one total each and add it to the workgroup's LDS accumulators; the workgroup flushes one 64-byte row
+//     per Gaussian to global memory with a single coalesced atomic-add instruction per four Gaussians.
+//
+// Sums are formed in a different order than the reference's warp reduce + atomics (whose order is itself
+// unspecified), so results agree to rounding, not bitwise.
+#include "gsx_common.h"
+
+namespace gsx {
+
+static constexpr uint32_t kTile = 16;
+static constexpr uint32_t kBatch = 256;
+static constexpr uint32_t kAcc = 16; // floats accumulated per Gaussian: rgb 3, v_gro 3, v_grd(x)ray_d 9, opacity 1
+
+__global__ void __launch_bounds__(256) fill_f32_kernel(size_t n, float v, float* __restrict__ out) {
+    const size_t i = (size_t)blockIdx.x * 256u + threadIdx.x;
+    if (i < n)
+        out[i] = v;
+}
+
+// sum of 16 values over the 64 lanes of a wave; on return lane L holds, in v[0], the wave total of component
+// ((L>>5)&1)*8 + ((L>>4)&1)*4 + ((L>>3)&1)*2 + ((L>>2)&1)
+__device__ __forceinline__ float wave_reduce16(float (&v)[16], uint32_t lane) {
+#pragma unroll
+    for (uint32_t step = 0; step < 4; ++step) {
+        const uint32_t m = 32u >> step;
+        const uint32_t half = 8u >> step;
+        const bool upper = (lane & m) != 0;
+#pragma unroll
+        for (uint32_t i = 0; i < half; ++i) {
+            const float send = upper ? v[i] : v[i + half];
+            const float keep = upper ? v[i + half] : v[i];
+            v[i] = keep + __shfl_xor(send, (int)m, 64);
+        }
+    }
+    v[0] += __shfl_xor(v[0], 2, 64);
+    v[0] += __shfl_xor(v[0], 1, 64);
+    return v[0];
+}
+
+__global__ void __launch_bounds__(256) rasterize_bwd_kernel(
+    uint32_t n_isects, const float* __restrict__ means, const float* __restrict__ quats,
+    const float* __restrict__ scales, const float* __restrict__ colors, const float* __restrict__ opacities,
+    const float* __restrict__ backgrounds, const uint8_t* __restrict__ masks, uint32_t image_width,
+    uint32_t image_height, uint32_t tile_width, uint32_t tile_height, const float* __restrict__ viewmat,
+    const float* __restrict__ Kmat, const int32_t* __restrict__ tile_offsets,
+    const int32_t* __restrict__ flatten_ids, const float* __restrict__ render_alphas,
+    const int32_t* __restrict__ last_ids, const float* __restrict__ v_render_colors,
+    const float* __restrict__ v_render_alphas, float* __restrict__ gacc /*[N,16]*/) {
+    __shared__ float4 stage[kBatch * 4];
+    __shared__ int32_t id_batch[kBatch];
+    __shared__ float acc[kBatch * kAcc];
+    __shared__ int32_t block_max;
+
+    const uint32_t tile_id = blockIdx.x;
+    if (masks != nullptr && !masks[tile_id]) // :83-87
+        return;
+    const uint32_t ty = tile_id / tile_width, tx = tile_id % tile_width;
+    const uint32_t tr = threadIdx.x;
+    const uint32_t lane = tr & 63u;
+    const uint32_t i = ty * kTile + (tr >> 4);
+    const uint32_t j = tx * kTile + (tr & 15u);
+    const bool inside = (i < image_height && j < image_width);
+    const uint32_t pix_id = min(i * image_width + j, image_width * image_height - 1); // :92-93
+
+    const CamPose cp = load_cam_pose(viewmat);
+    vec3 ray_o, ray_d;
+    pixel_world_ray(cp, (float)j + 0.5f, (float)i + 0.5f, Kmat[0], Kmat[4], Kmat[2], Kmat[5], &ray_o, &ray_d);
+
+    const int32_t range_start = tile_offsets[tile_id];
+    int32_t range_end = (tile_id == tile_width * tile_height - 1) ? (int32_t)n_isects : tile_offsets[tile_id + 1];
+
+    const float T_final = 1.0f - render_alphas[pix_id];
+    float T = T_final;
+    float buffer[3] = {0.f, 0.f, 0.f};
+    const int32_t bin_final = inside ? last_ids[pix_id] : 0;
+    float v_render_c[3];
+#pragma unroll
+    for (uint32_t k = 0; k < 3; ++k)
+        v_render_c[k] = v_render_colors[(size_t)pix_id * 3 + k];
+    const float v_render_a = v_render_alphas[pix_id];
+    float bg_dot = 0.f;
+    if (backgrounds != nullptr) {
+#pragma unroll
+        for (uint32_t k = 0; k < 3; ++k)
+            bg_dot += backgrounds[k] * v_render_c[k];
+    }
+
+    // last contributing list entry over the wave (:201-203) and over the workgroup: entries behind the
+    // workgroup's maximum are needed by no pixel, so the walk starts there
+    int32_t wave_bin_final = bin_final;
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1)
+        wave_bin_final = max(wave_bin_final, __shfl_xor(wave_bin_final, m, 64));
+    if (tr == 0)
+        block_max = 0;
+    __syncthreads();
+    if (lane == 0)
+        atomicMax(&block_max, wave_bin_final);
+#pragma unroll
+    for (uint32_t k = 0; k < kAcc; ++k)
+        acc[tr * kAcc + k] = 0.f;
+    __syncthreads();
+    range_end = min(range_end, block_max + 1);
+    if (range_end <= range_start)
+        return;
+    const uint32_t num_batches = (uint32_t)(range_end - range_start + (int32_t)kBatch - 1) / kBatch;
+
+    for (uint32_t b = 0; b < num_batches; ++b) {
+        // back to front: entry 0 of the batch is the farthest Gaussian (:211-216)
+        const int32_t batch_end = range_end - 1 - (int32_t)(kBatch * b);
+        const int32_t batch_size = min((int32_t)kBatch, batch_end + 1 - range_start);
+        const int32_t idx = batch_end - (int32_t)tr;
+        if (idx >= range_start) {
+            const int32_t g = flatten_ids[idx];
+            id_batch[tr] = g;
+            const vec3 xyz = ld3(means, g);
+            const float opac = opacities[g];
+            const mat3 R = quat_to_rotmat(ld4q(quats, g));
+            const vec3 s = ld3(scales, g);
+            const float is0 = 1.0f / s.x, is1 = 1.0f / s.y, is2 = 1.0f / s.z;
+            stage[tr * 4 + 0] = make_float4(xyz.x, xyz.y, xyz.z, opac);
+            stage[tr * 4 + 1] = make_float4(is0 * R.m[0][0], is0 * R.m[1][0], is0 * R.m[2][0], is1 * R.m[0][1]);
+            stage[tr * 4 + 2] = make_float4(is1 * R.m[1][1], is1 * R.m[2][1], is2 * R.m[0][2], is2 * R.m[1][2]);
+            stage[tr * 4 + 3] =
+                make_float4(is2 * R.m[2][2], colors[(size_t)g * 3], colors[(size_t)g * 3 + 1], colors[(size_t)g * 3 + 2]);
+        }
+        __syncthreads();
+
+        for (int32_t t = max(0, batch_end - wave_bin_final); t < batch_size; ++t) {
+            bool valid = inside && (batch_end - t <= bin_final);
+            const float4 a = stage[t * 4 + 0];
+            const float4 m0 = stage[t * 4 + 1];
+            const float4 m1 = stage[t * 4 + 2];
+            const float4 m2 = stage[t * 4 + 3];
+            const vec3 o = mk3(ray_o.x - a.x, ray_o.y - a.y, ray_o.z - a.z);
+            const vec3 gro = mk3(fma(m0.z, o.z, fma(m0.y, o.y, m0.x * o.x)), fma(m1.y, o.z, fma(m1.x, o.y, m0.w * o.x)),
+                                 fma(m2.x, o.z, fma(m1.w, o.y, m1.z * o.x)));
+            const vec3 grd = mk3(fma(m0.z, ray_d.z, fma(m0.y, ray_d.y, m0.x * ray_d.x)),
+                                 fma(m1.y, ray_d.z, fma(m1.x, ray_d.y, m0.w * ray_d.x)),
+                                 fma(m2.x, ray_d.z, fma(m1.w, ray_d.y, m1.z * ray_d.x)));
+            const vec3 grd_n = safe_normalize(grd);
+            const vec3 gcrod = cross(grd_n, gro);
+            const float grayDist = dot(gcrod, gcrod);
+            const float power = -0.5f * grayDist;
+            const float vis = gsx::exp(power);
+            const float alpha = gsx::fmin(0.999f, a.w * vis);
+            if (power > 0.f || alpha < 1.f / 255.f)
+                valid = false;
+            if (__builtin_amdgcn_ballot_w64(valid) == 0)
+                continue; // no lane of this wave sees the Gaussian (:286-289)
+
+            float v[kAcc];
+#pragma unroll
+            for (uint32_t k = 0; k < kAcc; ++k)
+                v[k] = 0.f;
+            if (valid) {
+                const float ra = 1.0f / (1.0f - alpha);
+                T *= ra;
+                const float fac = alpha * T;
+                v[0] = fac * v_render_c[0];
+                v[1] = fac * v_render_c[1];
+                v[2] = fac * v_render_c[2];
+                float v_alpha = 0.f;
+                v_alpha += (m2.y * T - buffer[0] * ra) * v_render_c[0];
+                v_alpha += (m2.z * T - buffer[1] * ra) * v_render_c[1];
+                v_alpha += (m2.w * T - buffer[2] * ra) * v_render_c[2];
+                v_alpha += T_final * ra * v_render_a;
+                if (backgrounds != nullptr)
+                    v_alpha += -T_final * ra * bg_dot;
+                if (a.w * vis <= 0.999f) {
+                    const float v_vis = a.w * v_alpha;
+                    const float v_gradDist = -0.5f * vis * v_vis;
+                    const vec3 v_gcrod = scale(gcrod, 2.0f * v_gradDist);
+                    const vec3 v_grd_n = neg(cross(v_gcrod, gro));
+                    const vec3 v_gro = cross(v_gcrod, grd_n);
+                    const vec3 v_grd = safe_normalize_bw(grd, v_grd_n);
+                    v[3] = v_gro.x;
+                    v[4] = v_gro.y;
+                    v[5] = v_gro.z;
+                    v[6] = v_grd.x * ray_d.x;
+                    v[7] = v_grd.x * ray_d.y;
+                    v[8] = v_grd.x * ray_d.z;
+                    v[9] = v_grd.y * ray_d.x;
+                    v[10] = v_grd.y * ray_d.y;
+                    v[11] = v_grd.y * ray_d.z;
+                    v[12] = v_grd.z * ray_d.x;
+                    v[13] = v_grd.z * ray_d.y;
+                    v[14] = v_grd.z * ray_d.z;
+                    v[15] = vis * v_alpha;
+                }
+                buffer[0] += m2.y * fac;
+                buffer[1] += m2.z * fac;
+                buffer[2] += m2.w * fac;
+            }
+            const float total = wave_reduce16(v, lane);
+            if ((lane & 3u) == 0) {
+                const uint32_t comp = ((lane >> 5) & 1u) * 8u + ((lane >> 4) & 1u) * 4u + ((lane >> 3) & 1u) * 2u +
+                                      ((lane >> 2) & 1u);
+                atomicAdd(&acc[(uint32_t)t * kAcc + comp], total); // LDS: ds_add_f32
+            }
+        }
+        __syncthreads();
+        // flush: 16 lanes per Gaussian, one 64-byte row each
+#pragma unroll 4
+        for (uint32_t s = 0; s < kBatch / 16; ++s) {
+            const uint32_t gi = s * 16u + (tr >> 4);
+            const uint32_t k = tr & 15u;
+            if ((int32_t)gi < batch_size) {
+                const float val = acc[gi * kAcc + k];
+                acc[gi * kAcc + k] = 0.f;
+                if (val != 0.f)
+                    unsafeAtomicAdd(&gacc[(size_t)id_batch[gi] * kAcc + k], val);
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// Per-Gaussian epilogue: the linear map from the accumulated (v_gro, v_grd (x) ray_d) to
+// (v_mean, v_quat, v_scale) - quat_scale_to_preci_half_vjp / quat_to_rotmat_vjp of Utils.cuh:104-158.
+__global__ void __launch_bounds__(256) rasterize_bwd_epilogue_kernel(
+    uint32_t N, const float* __restrict__ means, const float* __restrict__ quats, const float* __restrict__ scales,
+    const float* __restrict__ viewmat, const float* __restrict__ gacc, float* __restrict__ v_means,
+    float* __restrict__ v_quats, float* __restrict__ v_scales, float* __restrict__ v_colors,
+    float* __restrict__ v_opacities) {
+    const uint32_t g = blockIdx.x * 256u + threadIdx.x;
+    if (g >= N)
+        return;
+    const float4* row = reinterpret_cast<const float4*>(gacc + (size_t)g * kAcc);
+    const float4 r0 = row[0], r1 = row[1], r2 = row[2], r3 = row[3];
+    // r0 = rgb.xyz, vo.x ; r1 = vo.y, vo.z, G00, G01 ; r2 = G02, G10, G11, G12 ; r3 = G20, G21, G22, v_opacity
+    v_colors[(size_t)g * 3 + 0] = r0.x;
+    v_colors[(size_t)g * 3 + 1] = r0.y;
+    v_colors[(size_t)g * 3 + 2] = r0.z;
+    v_opacities[g] = r3.w;
+    const bool any_geo = (r0.w != 0.f) | (r1.x != 0.f) | (r1.y != 0.f) | (r1.z != 0.f) | (r1.w != 0.f) |
+                         (r2.x != 0.f) | (r2.y != 0.f) | (r2.z != 0.f) | (r2.w != 0.f) | (r3.x != 0.f) |
+                         (r3.y != 0.f) | (r3.z != 0.f);
+    float vm[3] = {0.f, 0.f, 0.f}, vq[4] = {0.f, 0.f, 0.f, 0.f}, vs[3] = {0.f, 0.f, 0.f};
+    if (any_geo) {
+        const CamPose cp = load_cam_pose(viewmat);
+        quat qp;
+        vec3 tp;
+        shutter_pose(cp, 0.f, &qp, &tp);
+        const mat3 R_inv = mat3_cast(quat_inverse(qp));
+        const vec3 ray_o = neg(mul(R_inv, tp));
+        const vec3 om = sub(ray_o, ld3(means, g));
+        const quat q = ld4q(quats, g);
+        const mat3 R = quat_to_rotmat(q);
+        const vec3 s = ld3(scales, g);
+        const float is[3] = {1.0f / s.x, 1.0f / s.y, 1.0f / s.z};
+        mat3 Mt;
+#pragma unroll
+        for (int a = 0; a < 3; ++a)
+#pragma unroll
+            for (int b = 0; b < 3; ++b)
+                Mt.m[a][b] = is[a] * R.m[b][a];
+        const vec3 Vo = mk3(r0.w, r1.x, r1.y);
+        const float G[3][3] = {{r1.z, r1.w, r2.x}, {r2.y, r2.z, r2.w}, {r3.x, r3.y, r3.z}};
+        const float vo[3] = {Vo.x, Vo.y, Vo.z};
+        const float omv[3] = {om.x, om.y, om.z};
+        float v_Mt[3][3];
+#pragma unroll
+        for (int a = 0; a < 3; ++a)
+#pragma unroll
+            for (int b = 0; b < 3; ++b)
+                v_Mt[a][b] = fma(vo[a], omv[b], G[a][b]);
+        const vec3 v_o = mul_t(Mt, Vo);
+        vm[0] = -v_o.x;
+        vm[1] = -v_o.y;
+        vm[2] = -v_o.z;
+        float vr[3][3]; // v_R(k,j) = v_M(k,j) / s_j, v_M = v_Mt^T
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+#pragma unroll
+            for (int jj = 0; jj < 3; ++jj)
+                vr[k][jj] = v_Mt[jj][k] * is[jj];
+        const float inv_norm = gsx::rsqrt(fma(q.w, q.w, fma(q.z, q.z, fma(q.y, q.y, q.x * q.x))));
+        const float x = q.x * inv_norm, y = q.y * inv_norm, z = q.z * inv_norm, w = q.w * inv_norm;
+        const float vq_w = 2.f * (x * (vr[2][1] - vr[1][2]) + y * (vr[0][2] - vr[2][0]) + z * (vr[1][0] - vr[0][1]));
+        const float vq_x = 2.f * (-2.f * x * (vr[1][1] + vr[2][2]) + y * (vr[1][0] + vr[0][1]) +
+                                  z * (vr[2][0] + vr[0][2]) + w * (vr[2][1] - vr[1][2]));
+        const float vq_y = 2.f * (x * (vr[1][0] + vr[0][1]) - 2.f * y * (vr[0][0] + vr[2][2]) +
+                                  z * (vr[2][1] + vr[1][2]) + w * (vr[0][2] - vr[2][0]));
+        const float vq_z = 2.f * (x * (vr[2][0] + vr[0][2]) + y * (vr[2][1] + vr[1][2]) -
+                                  2.f * z * (vr[0][0] + vr[1][1]) + w * (vr[1][0] - vr[0][1]));
+        const float d = vq_w * w + vq_x * x + vq_y * y + vq_z * z;
+        vq[0] = (vq_w - d * w) * inv_norm;
+        vq[1] = (vq_x - d * x) * inv_norm;
+        vq[2] = (vq_y - d * y) * inv_norm;
+        vq[3] = (vq_z - d * z) * inv_norm;
+#pragma unroll
+        for (int jj = 0; jj < 3; ++jj)
+            vs[jj] = -is[jj] * is[jj] *
+                     (R.m[0][jj] * v_Mt[jj][0] + R.m[1][jj] * v_Mt[jj][1] + R.m[2][jj] * v_Mt[jj][2]);
+    }
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        v_means[(size_t)g * 3 + k] = vm[k];
+        v_scales[(size_t)g * 3 + k] = vs[k];
+    }
+    reinterpret_cast<float4*>(v_quats)[g] = make_float4(vq[0], vq[1], vq[2], vq[3]);
+}
+
+} // namespace gsx
+
+using namespace gsx;
+
+extern "C" size_t gsx_rasterize_bwd_workspace_bytes(uint32_t N) { return align_up((size_t)N * kAcc * 4, 256) + 256; }
+
+extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
+    uint32_t C, uint32_t N, int64_t n_isects, const float* means, const float* quats, const float* scales,
+    const float* colors, const float* opacities, const float* backgrounds, const uint8_t* masks,
+    uint32_t image_width, uint32_t image_height, uint32_t tile_size, const float* viewmats0, const float* viewmats1,
+    const float* Ks, int camera_model, gsx_ut_params ut, int rs_type, const float* radial_coeffs,
+    const float* tangential_coeffs, const float* thin_prism_coeffs, const int32_t* tile_offsets,
+    const int32_t* flatten_ids, const float* render_alphas, const int32_t* last_ids, const float* v_render_colors,
+    const float* v_render_alphas, float* v_means, float* v_quats, float* v_scales, float* v_colors,
+    float* v_opacities, void* workspace, size_t workspace_bytes, void* stream) {
+    (void)ut;
+    const int rc = check_camera_args(C, viewmats1, camera_model, rs_type, radial_coeffs, tangential_coeffs,
+                                     thin_prism_coeffs);
+    if (rc != GSX_OK)
+        return rc;
+    if (N == 0)
+        return GSX_OK;
+    GSX_REQUIRE(tile_size == kTile, GSX_ERR_UNSUPPORTED, "rasterize bwd: tile_size %u (only 16 is built)", tile_size);
+    GSX_REQUIRE(n_isects >= 0 && n_isects < (1ll << 31), GSX_ERR_OVERFLOW, "rasterize bwd: n_isects out of range");
+    GSX_REQUIRE(means && quats && scales && colors && opacities && viewmats0 && Ks && tile_offsets && render_alphas &&
+                    last_ids && v_render_colors && v_render_alphas && v_means && v_quats && v_scales && v_colors &&
+                    v_opacities,
+                GSX_ERR_INVALID_ARGUMENT, "rasterize bwd: null tensor");
+    GSX_REQUIRE(n_isects == 0 || flatten_ids, GSX_ERR_INVALID_ARGUMENT, "rasterize bwd: flatten_ids is null");
+    GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 &&
+                    workspace_bytes >= gsx_rasterize_bwd_workspace_bytes(N),
+                GSX_ERR_WORKSPACE, "rasterize bwd: workspace needs %zu bytes, 256-byte aligned",
+                gsx_rasterize_bwd_workspace_bytes(N));
+    float* gacc = (float*)workspace;
+    hipStream_t s = (hipStream_t)stream;
+    const size_t n_acc = (size_t)N * kAcc;
+    hipLaunchKernelGGL(fill_f32_kernel, dim3(cdiv(n_acc, 256)), dim3(256), 0, s, n_acc, 0.f, gacc);
+    GSX_LAUNCH_CHECK();
+    if (n_isects > 0 && image_width > 0 && image_height > 0) { // ...Bwd.cu:440-443
+        const uint32_t tw = cdiv(image_width, kTile), th = cdiv(image_height, kTile);
+        hipLaunchKernelGGL(rasterize_bwd_kernel, dim3(tw * th), dim3(256), 0, s, (uint32_t)n_isects, means, quats,
+                           scales, colors, opacities, backgrounds, masks, image_width, image_height, tw, th, viewmats0,
+                           Ks, tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors, v_render_alphas,
+                           gacc);
+        GSX_LAUNCH_CHECK();
+    }
+    hipLaunchKernelGGL(rasterize_bwd_epilogue_kernel, dim3(cdiv(N, 256)), dim3(256), 0, s, N, means, quats, scales,
+                       viewmats0, gacc, v_means, v_quats, v_scales, v_colors, v_opacities);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}

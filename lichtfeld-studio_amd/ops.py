@@ -1,0 +1,415 @@
+"""Host-side mirror of the reference's operator interface (gsplat/Ops.h:9-272, include/kernels/ssim.cuh,
+fastgs/optimizer adam_step) over torch tensors: same function names, argument order and meaning, same error
+behaviour (non-device or non-contiguous tensors raise, zero-size inputs return without launching), outputs
+freshly allocated like the reference's at::empty / at::zeros.  Every function calls the C ABI of libgsx.so on
+torch's current stream; torch is only used for device memory and streams.
+"""
+import ctypes
+
+import torch
+
+from . import _lib as L
+from ._lib import UTParams, c_f, c_i, c_i64, c_p, c_sz, c_u32, check, lib
+
+CameraModelType = type("CameraModelType", (), dict(PINHOLE=0, ORTHO=1, FISHEYE=2, EQUIRECTANGULAR=3))
+ShutterType = type("ShutterType", (), dict(ROLLING_TOP_TO_BOTTOM=0, ROLLING_LEFT_TO_RIGHT=1, ROLLING_BOTTOM_TO_TOP=2,
+                                           ROLLING_RIGHT_TO_LEFT=3, GLOBAL=4))
+UnscentedTransformParameters = UTParams
+ALPHA_THRESHOLD = 1.0 / 255.0
+
+
+def _check_input(x, name):
+    """CHECK_INPUT of gsplat/Common.h:12-17"""
+    if not isinstance(x, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if not x.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not x.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+
+
+def _ptr(x):
+    return c_p(None) if x is None else c_p(x.data_ptr())
+
+
+def _stream(dev):
+    return c_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+def _workspace(nbytes, dev):
+    return torch.empty((max(int(nbytes), 256),), dtype=torch.uint8, device=dev)
+
+
+def _f32(x, name):
+    _check_input(x, name)
+    if x.dtype != torch.float32:
+        raise RuntimeError(f"{name} must be float32")
+    return x
+
+
+# ------------------------------------------------------------------------------------------------
+def spherical_harmonics_fwd(degrees_to_use, dirs, coeffs, masks=None):
+    """Ops.h:12-17"""
+    _f32(dirs, "dirs"), _f32(coeffs, "coeffs")
+    if masks is not None:
+        _check_input(masks, "masks")
+    if coeffs.size(-1) != 3:
+        raise RuntimeError("coeffs must have last dimension 3")  # SphericalHarmonics.cpp:27
+    if dirs.size(-1) != 3:
+        raise RuntimeError("dirs must have last dimension 3")
+    K = coeffs.size(-2)
+    N = dirs.numel() // 3
+    colors = torch.empty_like(dirs)
+    m8 = None if masks is None else masks.view(torch.uint8) if masks.dtype == torch.bool else masks
+    with torch.cuda.device(dirs.device):
+        check(lib().gsx_spherical_harmonics_fwd(c_u32(N), c_u32(K), c_u32(degrees_to_use), _ptr(dirs), _ptr(coeffs),
+                                                _ptr(m8), _ptr(colors), _stream(dirs.device)))
+    return colors
+
+
+def spherical_harmonics_bwd(K, degrees_to_use, dirs, coeffs, masks, v_colors, compute_v_dirs):
+    """Ops.h:18-25 -> (v_coeffs, v_dirs or None)"""
+    _f32(dirs, "dirs"), _f32(coeffs, "coeffs"), _f32(v_colors, "v_colors")
+    if masks is not None:
+        _check_input(masks, "masks")
+    if v_colors.size(-1) != 3 or coeffs.size(-1) != 3 or dirs.size(-1) != 3:
+        raise RuntimeError("last dimension must be 3")
+    N = dirs.numel() // 3
+    v_coeffs = torch.empty_like(coeffs)
+    v_dirs = torch.empty_like(dirs) if compute_v_dirs else None
+    m8 = None if masks is None else masks.view(torch.uint8) if masks.dtype == torch.bool else masks
+    with torch.cuda.device(dirs.device):
+        check(lib().gsx_spherical_harmonics_bwd(c_u32(N), c_u32(K), c_u32(degrees_to_use), _ptr(dirs), _ptr(coeffs),
+                                                _ptr(m8), _ptr(v_colors), _ptr(v_coeffs), _ptr(v_dirs),
+                                                _stream(dirs.device)))
+    return v_coeffs, v_dirs
+
+
+def intersect_tile(means2d, radii, depths, camera_ids, gaussian_ids, C, tile_size, tile_width, tile_height,
+                   sort=True):
+    """Ops.h:28-38 -> (tiles_per_gauss [C,N] i32, isect_ids [I] i64, flatten_ids [I] i32)"""
+    _f32(means2d, "means2d"), _check_input(radii, "radii"), _f32(depths, "depths")
+    if means2d.dim() == 2:
+        if camera_ids is None or gaussian_ids is None:  # Intersect.cpp:34-36
+            raise RuntimeError("When packed is set, camera_ids and gaussian_ids must be provided.")
+        raise NotImplementedError("packed intersect_tile is not built (LichtFeld never uses it: rasterizer.cpp:25)")
+    if radii.dtype != torch.int32:
+        raise RuntimeError("radii must be int32")
+    dev = means2d.device
+    N = means2d.size(1)
+    tiles_per_gauss = torch.empty_like(depths, dtype=torch.int32)
+    n_isects = c_i64(0)
+    with torch.cuda.device(dev):
+        cum = torch.empty((C * N,), dtype=torch.int64, device=dev)
+        ws_bytes = lib().gsx_intersect_tile_count_workspace_bytes(c_u32(C), c_u32(N))
+        ws = _workspace(ws_bytes, dev)
+        check(lib().gsx_intersect_tile_count(c_u32(C), c_u32(N), _ptr(means2d), _ptr(radii), c_u32(tile_size),
+                                             c_u32(tile_width), c_u32(tile_height), _ptr(tiles_per_gauss), _ptr(cum),
+                                             _ptr(ws), c_sz(ws.numel()), ctypes.byref(n_isects), _stream(dev)))
+        n = n_isects.value
+        isect_ids = torch.empty((n,), dtype=torch.int64, device=dev)
+        flatten_ids = torch.empty((n,), dtype=torch.int32, device=dev)
+        if n:
+            check(lib().gsx_intersect_tile_emit(c_u32(C), c_u32(N), _ptr(means2d), _ptr(radii), _ptr(depths),
+                                                _ptr(cum), c_u32(tile_size), c_u32(tile_width), c_u32(tile_height),
+                                                _ptr(isect_ids), _ptr(flatten_ids), _stream(dev)))
+        if n and sort:
+            tile_n_bits = lib().gsx_n_bits(c_u32(tile_width * tile_height))
+            cam_n_bits = lib().gsx_n_bits(c_u32(C))
+            isect_ids, flatten_ids = radix_sort_double_buffer(n, tile_n_bits, cam_n_bits, isect_ids, flatten_ids)
+    return tiles_per_gauss, isect_ids, flatten_ids
+
+
+def radix_sort_double_buffer(n_isects, tile_n_bits, cam_n_bits, isect_ids, flatten_ids):
+    """Intersect.h:39-46.  Returns the sorted (isect_ids, flatten_ids); like the reference's DoubleBuffer the
+    result may live in either the input tensors or the internally allocated pair."""
+    _check_input(isect_ids, "isect_ids"), _check_input(flatten_ids, "flatten_ids")
+    if n_isects <= 0:
+        return isect_ids, flatten_ids
+    dev = isect_ids.device
+    with torch.cuda.device(dev):
+        k1, v1 = torch.empty_like(isect_ids), torch.empty_like(flatten_ids)
+        ws = _workspace(lib().gsx_radix_sort_pairs_workspace_bytes(c_i64(n_isects)), dev)
+        sel = c_i(0)
+        check(lib().gsx_radix_sort_pairs(c_i64(n_isects), _ptr(isect_ids), _ptr(flatten_ids), _ptr(k1), _ptr(v1),
+                                         c_u32(32 + tile_n_bits + cam_n_bits), _ptr(ws), c_sz(ws.numel()),
+                                         ctypes.byref(sel), _stream(dev)))
+    return (k1, v1) if sel.value else (isect_ids, flatten_ids)
+
+
+def intersect_offset(isect_ids, C, tile_width, tile_height):
+    """Ops.h:39-43 -> offsets [C, tile_height, tile_width] i32"""
+    _check_input(isect_ids, "isect_ids")
+    dev = isect_ids.device
+    offsets = torch.empty((C, tile_height, tile_width), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        check(lib().gsx_intersect_offset(c_i64(isect_ids.numel()), _ptr(isect_ids), c_u32(C), c_u32(tile_width),
+                                         c_u32(tile_height), _ptr(offsets), _stream(dev)))
+    return offsets
+
+
+def quats_to_rotmats(quats):
+    """Ops.h:46-48"""
+    _f32(quats, "quats")
+    N = quats.size(0)
+    out = torch.empty((N, 3, 3), dtype=quats.dtype, device=quats.device)
+    with torch.cuda.device(quats.device):
+        check(lib().gsx_quats_to_rotmats(c_i(N), _ptr(quats), _ptr(out), _stream(quats.device)))
+    return out
+
+
+def relocation(opacities, scales, ratios, binoms, n_max):
+    """Ops.h:52-57 -> (new_opacities, new_scales)"""
+    _f32(opacities, "opacities"), _f32(scales, "scales"), _check_input(ratios, "ratios"), _f32(binoms, "binoms")
+    if ratios.dtype != torch.int32:
+        raise RuntimeError("ratios must be int32")
+    new_opacities, new_scales = torch.empty_like(opacities), torch.empty_like(scales)
+    with torch.cuda.device(opacities.device):
+        check(lib().gsx_relocation(c_i(opacities.size(0)), _ptr(opacities), _ptr(scales), _ptr(ratios), _ptr(binoms),
+                                   c_i(n_max), _ptr(new_opacities), _ptr(new_scales), _stream(opacities.device)))
+    return new_opacities, new_scales
+
+
+def add_noise(raw_opacities, raw_scales, raw_quats, noise, means, current_lr):
+    """Ops.h:59-65; means is modified in place"""
+    for t, n in ((raw_opacities, "raw_opacities"), (raw_scales, "raw_scales"), (raw_quats, "raw_quats"),
+                 (noise, "noise"), (means, "means")):
+        _f32(t, n)
+    with torch.cuda.device(means.device):
+        check(lib().gsx_add_noise(c_i(means.size(0)), _ptr(raw_opacities), _ptr(raw_scales), _ptr(raw_quats),
+                                  _ptr(noise), _ptr(means), c_f(current_lr), _stream(means.device)))
+
+
+def projection_ut_3dgs_fused(means, quats, scales, opacities, viewmats0, viewmats1, Ks, image_width, image_height,
+                             eps2d, near_plane, far_plane, radius_clip, calc_compensations, camera_model, ut_params,
+                             rs_type, radial_coeffs=None, tangential_coeffs=None, thin_prism_coeffs=None):
+    """Ops.h:69-98 -> (radii [C,N,2] i32, means2d [C,N,2], depths [C,N], conics [C,N,3], compensations [C,N] or
+    None).  Rows of culled Gaussians hold unspecified values except radii == 0 (Projection.cpp:70-73 at::empty)."""
+    _f32(means, "means"), _f32(quats, "quats"), _f32(scales, "scales")
+    if opacities is not None:
+        _f32(opacities, "opacities")
+    _f32(viewmats0, "viewmats0"), _f32(Ks, "Ks")
+    for t, n in ((viewmats1, "viewmats1"), (radial_coeffs, "radial_coeffs"), (tangential_coeffs, "tangential_coeffs"),
+                 (thin_prism_coeffs, "thin_prism_coeffs")):
+        if t is not None:
+            _f32(t, n)
+    dev = means.device
+    N, C = means.size(0), viewmats0.size(0)
+    radii = torch.empty((C, N, 2), dtype=torch.int32, device=dev)
+    means2d = torch.empty((C, N, 2), dtype=torch.float32, device=dev)
+    depths = torch.empty((C, N), dtype=torch.float32, device=dev)
+    conics = torch.empty((C, N, 3), dtype=torch.float32, device=dev)
+    comp = torch.zeros((C, N), dtype=torch.float32, device=dev) if calc_compensations else None
+    with torch.cuda.device(dev):
+        check(lib().gsx_projection_ut_3dgs_fused(
+            c_u32(C), c_u32(N), _ptr(means), _ptr(quats), _ptr(scales), _ptr(opacities), _ptr(viewmats0),
+            _ptr(viewmats1), _ptr(Ks), c_u32(image_width), c_u32(image_height), c_f(eps2d), c_f(near_plane),
+            c_f(far_plane), c_f(radius_clip), c_i(camera_model), ut_params, c_i(rs_type), _ptr(radial_coeffs),
+            _ptr(tangential_coeffs), _ptr(thin_prism_coeffs), _ptr(radii), _ptr(means2d), _ptr(depths), _ptr(conics),
+            _ptr(comp), _stream(dev)))
+    return radii, means2d, depths, conics, comp
+
+
+def rasterize_to_pixels_from_world_3dgs_fwd(means, quats, scales, colors, opacities, backgrounds, masks, image_width,
+                                            image_height, tile_size, viewmats0, viewmats1, Ks, camera_model,
+                                            ut_params, rs_type, radial_coeffs, tangential_coeffs, thin_prism_coeffs,
+                                            tile_offsets, flatten_ids):
+    """Ops.h:100-129 -> (renders [C,H,W,channels], alphas [C,H,W,1], last_ids [C,H,W] i32)"""
+    for t, n in ((means, "means"), (quats, "quats"), (scales, "scales"), (colors, "colors"),
+                 (opacities, "opacities"), (viewmats0, "viewmats0"), (Ks, "Ks")):
+        _f32(t, n)
+    _check_input(tile_offsets, "tile_offsets"), _check_input(flatten_ids, "flatten_ids")
+    if backgrounds is not None and backgrounds.numel() == 0:
+        backgrounds = None
+    if backgrounds is not None:
+        _f32(backgrounds, "backgrounds")
+    if masks is not None:
+        _check_input(masks, "masks")
+    dev = means.device
+    C, N = tile_offsets.size(0), means.size(0)
+    channels = colors.size(-1)
+    renders = torch.empty((C, image_height, image_width, channels), dtype=torch.float32, device=dev)
+    alphas = torch.empty((C, image_height, image_width, 1), dtype=torch.float32, device=dev)
+    last_ids = torch.empty((C, image_height, image_width), dtype=torch.int32, device=dev)
+    m8 = None if masks is None else masks.view(torch.uint8) if masks.dtype == torch.bool else masks
+    with torch.cuda.device(dev):
+        check(lib().gsx_rasterize_to_pixels_from_world_3dgs_fwd(
+            c_u32(C), c_u32(N), c_i64(flatten_ids.numel()), _ptr(means), _ptr(quats), _ptr(scales), _ptr(colors),
+            c_u32(channels), _ptr(opacities), _ptr(backgrounds), _ptr(m8), c_u32(image_width), c_u32(image_height),
+            c_u32(tile_size), _ptr(viewmats0), _ptr(viewmats1), _ptr(Ks), c_i(camera_model), ut_params, c_i(rs_type),
+            _ptr(radial_coeffs), _ptr(tangential_coeffs), _ptr(thin_prism_coeffs), _ptr(tile_offsets),
+            _ptr(flatten_ids), _ptr(renders), _ptr(alphas), _ptr(last_ids), _stream(dev)))
+    return renders, alphas, last_ids
+
+
+def rasterize_to_pixels_from_world_3dgs_bwd(means, quats, scales, colors, opacities, backgrounds, masks, image_width,
+                                            image_height, tile_size, viewmats0, viewmats1, Ks, camera_model,
+                                            ut_params, rs_type, radial_coeffs, tangential_coeffs, thin_prism_coeffs,
+                                            tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors,
+                                            v_render_alphas):
+    """Ops.h:131-166 -> (v_means [N,3], v_quats [N,4], v_scales [N,3], v_colors [C,N,3], v_opacities [C,N])"""
+    for t, n in ((means, "means"), (quats, "quats"), (scales, "scales"), (colors, "colors"),
+                 (opacities, "opacities"), (viewmats0, "viewmats0"), (Ks, "Ks"), (render_alphas, "render_alphas"),
+                 (v_render_colors, "v_render_colors"), (v_render_alphas, "v_render_alphas")):
+        _f32(t, n)
+    _check_input(tile_offsets, "tile_offsets"), _check_input(flatten_ids, "flatten_ids")
+    _check_input(last_ids, "last_ids")
+    if colors.size(-1) != 3:
+        raise RuntimeError("Unsupported number of channels: only 3 is built for the backward pass")
+    if backgrounds is not None and backgrounds.numel() == 0:
+        backgrounds = None
+    dev = means.device
+    C, N = tile_offsets.size(0), means.size(0)
+    v_means, v_quats, v_scales = torch.empty_like(means), torch.empty_like(quats), torch.empty_like(scales)
+    v_colors, v_opacities = torch.empty_like(colors), torch.empty_like(opacities)
+    m8 = None if masks is None else masks.view(torch.uint8) if masks.dtype == torch.bool else masks
+    with torch.cuda.device(dev):
+        ws = _workspace(lib().gsx_rasterize_bwd_workspace_bytes(c_u32(N)), dev)
+        check(lib().gsx_rasterize_to_pixels_from_world_3dgs_bwd(
+            c_u32(C), c_u32(N), c_i64(flatten_ids.numel()), _ptr(means), _ptr(quats), _ptr(scales), _ptr(colors),
+            _ptr(opacities), _ptr(backgrounds), _ptr(m8), c_u32(image_width), c_u32(image_height), c_u32(tile_size),
+            _ptr(viewmats0), _ptr(viewmats1), _ptr(Ks), c_i(camera_model), ut_params, c_i(rs_type),
+            _ptr(radial_coeffs), _ptr(tangential_coeffs), _ptr(thin_prism_coeffs), _ptr(tile_offsets),
+            _ptr(flatten_ids), _ptr(render_alphas), _ptr(last_ids), _ptr(v_render_colors), _ptr(v_render_alphas),
+            _ptr(v_means), _ptr(v_quats), _ptr(v_scales), _ptr(v_colors), _ptr(v_opacities), _ptr(ws),
+            c_sz(ws.numel()), _stream(dev)))
+    return v_means, v_quats, v_scales, v_colors, v_opacities
+
+
+def rasterize_from_world_with_sh_fwd(means, quats, scales, opacities, sh_coeffs, sh_degree, backgrounds, masks,
+                                     image_width, image_height, tile_size, viewmats0, viewmats1, Ks, camera_model,
+                                     eps2d, near_plane, far_plane, radius_clip, scaling_modifier, calc_compensations,
+                                     render_mode, ut_params, rs_type, radial_coeffs=None, tangential_coeffs=None,
+                                     thin_prism_coeffs=None, return_isect_ids=False):
+    """Ops.h:174-220 (Rasterization.cpp:279-467).  -> (render_colors, render_alphas, radii, means2d, depths, colors,
+    tile_offsets, flatten_ids, last_ids, compensations).  render_mode 0 (RGB) is built."""
+    for t, n in ((means, "means"), (quats, "quats"), (scales, "scales"), (opacities, "opacities"),
+                 (sh_coeffs, "sh_coeffs"), (viewmats0, "viewmats0"), (Ks, "Ks")):
+        _f32(t, n)
+    if render_mode != 0:
+        raise NotImplementedError("render_mode %d: only RGB (0) is built" % render_mode)
+    dev = means.device
+    N, C = means.size(0), viewmats0.size(0)
+    opacities = opacities.reshape(-1)
+    scaled_scales = scales if scaling_modifier == 1.0 else scales * scaling_modifier  # Rasterization.cpp:327
+    radii, means2d, depths, conics, comp = projection_ut_3dgs_fused(
+        means, quats, scaled_scales, opacities, viewmats0, viewmats1, Ks, image_width, image_height, eps2d,
+        near_plane, far_plane, radius_clip, calc_compensations, camera_model, ut_params, rs_type, radial_coeffs,
+        tangential_coeffs, thin_prism_coeffs)
+    K = sh_coeffs.size(1)
+    colors = torch.empty((C, N, 3), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        check(lib().gsx_sh_colors_from_world(c_u32(N), c_u32(K), c_u32(sh_degree), _ptr(means), _ptr(sh_coeffs),
+                                             _ptr(radii), _ptr(viewmats0), _ptr(colors), _stream(dev)))
+    final_opacities = opacities.unsqueeze(0)
+    if calc_compensations and comp is not None:
+        final_opacities = (final_opacities * comp).contiguous()
+    tile_width = (image_width + tile_size - 1) // tile_size
+    tile_height = (image_height + tile_size - 1) // tile_size
+    _, isect_ids, flatten_ids = intersect_tile(means2d, radii, depths, None, None, C, tile_size, tile_width,
+                                               tile_height, True)
+    offsets = intersect_offset(isect_ids, C, tile_width, tile_height)
+    renders, alphas, last_ids = rasterize_to_pixels_from_world_3dgs_fwd(
+        means, quats, scaled_scales, colors, final_opacities, backgrounds, masks, image_width, image_height,
+        tile_size, viewmats0, viewmats1, Ks, camera_model, ut_params, rs_type, radial_coeffs, tangential_coeffs,
+        thin_prism_coeffs, offsets, flatten_ids)
+    out = (renders, alphas, radii, means2d, depths, colors, offsets, flatten_ids, last_ids, comp)
+    return out + (isect_ids,) if return_isect_ids else out
+
+
+def rasterize_from_world_with_sh_bwd(means, quats, scales, opacities, sh_coeffs, sh_degree, backgrounds, masks,
+                                     image_width, image_height, tile_size, viewmats0, viewmats1, Ks, camera_model,
+                                     eps2d, near_plane, far_plane, radius_clip, scaling_modifier, calc_compensations,
+                                     render_mode, ut_params, rs_type, radial_coeffs, tangential_coeffs,
+                                     thin_prism_coeffs, render_alphas, last_ids, tile_offsets, flatten_ids, colors,
+                                     radii, means2d, depths, compensations, v_render_colors, v_render_alphas):
+    """Ops.h:222-270 (Rasterization.cpp:469-642) -> (v_means, v_quats, v_scales, v_opacities [C,N], v_sh_coeffs)"""
+    for t, n in ((means, "means"), (quats, "quats"), (scales, "scales"), (opacities, "opacities"),
+                 (sh_coeffs, "sh_coeffs"), (v_render_colors, "v_render_colors"),
+                 (v_render_alphas, "v_render_alphas")):
+        _f32(t, n)
+    if render_mode != 0:
+        raise NotImplementedError("render_mode %d: only RGB (0) is built" % render_mode)
+    dev = means.device
+    N = means.size(0)
+    final_opacities = opacities.reshape(1, -1)
+    if calc_compensations and compensations is not None and compensations.numel() > 0:
+        final_opacities = (final_opacities * compensations).contiguous()
+    scaled_scales = scales if scaling_modifier == 1.0 else scales * scaling_modifier
+    v_means, v_quats, v_scales, v_colors, v_opacities = rasterize_to_pixels_from_world_3dgs_bwd(
+        means, quats, scaled_scales, colors, final_opacities, backgrounds, masks, image_width, image_height,
+        tile_size, viewmats0, viewmats1, Ks, camera_model, ut_params, rs_type, radial_coeffs, tangential_coeffs,
+        thin_prism_coeffs, tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors, v_render_alphas)
+    K = sh_coeffs.size(1)
+    v_sh = torch.empty_like(sh_coeffs)
+    with torch.cuda.device(dev):
+        check(lib().gsx_sh_colors_from_world_bwd(c_u32(N), c_u32(K), c_u32(sh_degree), _ptr(means), _ptr(radii),
+                                                 _ptr(viewmats0), _ptr(colors), _ptr(v_colors), _ptr(v_sh),
+                                                 _stream(dev)))
+    if scaling_modifier != 1.0:
+        v_scales = v_scales * scaling_modifier  # Rasterization.cpp:633
+    return v_means, v_quats, v_scales, v_opacities, v_sh
+
+
+# ------------------------------------------------------------------------------------------------
+def fusedssim(C1, C2, img1, img2, train):
+    """include/kernels/ssim.cuh:11-19 -> (ssim_map, dm_dmu1, dm_dsigma1_sq, dm_dsigma12)"""
+    _f32(img1, "img1"), _f32(img2, "img2")
+    B, CH, H, W = img1.shape
+    ssim_map = torch.empty_like(img1)
+    if train:
+        d1, d2, d3 = torch.empty_like(img1), torch.empty_like(img1), torch.empty_like(img1)
+    else:
+        d1 = d2 = d3 = None
+    with torch.cuda.device(img1.device):
+        check(lib().gsx_fusedssim(c_i(B), c_i(CH), c_i(H), c_i(W), c_f(C1), c_f(C2), _ptr(img1), _ptr(img2),
+                                  _ptr(ssim_map), _ptr(d1), _ptr(d2), _ptr(d3), _stream(img1.device)))
+    empty = torch.empty((0,), dtype=img1.dtype, device=img1.device)
+    return ssim_map, (d1 if train else empty), (d2 if train else empty), (d3 if train else empty)
+
+
+def fusedssim_backward(C1, C2, img1, img2, dL_dmap, dm_dmu1, dm_dsigma1_sq, dm_dsigma12):
+    """include/kernels/ssim.cuh:21-28 -> dL_dimg1"""
+    for t, n in ((img1, "img1"), (img2, "img2"), (dL_dmap, "dL_dmap"), (dm_dmu1, "dm_dmu1"),
+                 (dm_dsigma1_sq, "dm_dsigma1_sq"), (dm_dsigma12, "dm_dsigma12")):
+        _f32(t, n)
+    B, CH, H, W = img1.shape
+    out = torch.empty_like(img1)
+    with torch.cuda.device(img1.device):
+        check(lib().gsx_fusedssim_backward(c_i(B), c_i(CH), c_i(H), c_i(W), c_f(C1), c_f(C2), _ptr(img1), _ptr(img2),
+                                           _ptr(dL_dmap), _ptr(dm_dmu1), _ptr(dm_dsigma1_sq), _ptr(dm_dsigma12),
+                                           _ptr(out), _stream(img1.device)))
+    return out
+
+
+def adam_step(param, exp_avg, exp_avg_sq, param_grad, lr, beta1, beta2, eps, bias_correction1_rcp,
+              bias_correction2_sqrt_rcp):
+    """fast_gs::optimizer::adam_step_wrapper (fastgs/optimizer/src/adam_api.cu:8-33); in place"""
+    for t, n in ((param, "param"), (exp_avg, "exp_avg"), (exp_avg_sq, "exp_avg_sq"), (param_grad, "param_grad")):
+        _f32(t, n)
+    with torch.cuda.device(param.device):
+        check(lib().gsx_adam_step(_ptr(param), _ptr(exp_avg), _ptr(exp_avg_sq), _ptr(param_grad),
+                                  c_i64(param.numel()), c_f(lr), c_f(beta1), c_f(beta2), c_f(eps),
+                                  c_f(bias_correction1_rcp), c_f(bias_correction2_sqrt_rcp), _stream(param.device)))
+
+
+def adam_step_multi(groups):
+    """All parameter groups of one optimiser step in a single launch.  groups: list of dicts with the keyword
+    arguments of adam_step (tensors may be None / grad None to skip)."""
+    if not groups:
+        return
+    arr = (L.AdamGroup * len(groups))()
+    dev = None
+    for i, g in enumerate(groups):
+        p = g["param"]
+        dev = p.device
+        for n in ("param", "exp_avg", "exp_avg_sq"):
+            _f32(g[n], n)
+        grad = g.get("param_grad")
+        if grad is not None:
+            _f32(grad, "param_grad")
+        arr[i] = L.AdamGroup(p.data_ptr(), g["exp_avg"].data_ptr(), g["exp_avg_sq"].data_ptr(),
+                             None if grad is None else grad.data_ptr(), p.numel(), g["lr"], g["beta1"], g["beta2"],
+                             g["eps"], g["bias_correction1_rcp"], g["bias_correction2_sqrt_rcp"])
+    with torch.cuda.device(dev):
+        check(lib().gsx_adam_step_multi(arr, c_i(len(groups)), _stream(dev)))

@@ -1,0 +1,34 @@
+"""Build the CPU checker (oracle/gsx_oracle.cpp) into oracle/libgsx_oracle.so.
+
+Test infrastructure only: nothing in the shipped package imports this.
+
+The reference itself cannot be built here (CUDA 12.8 + glm + LibTorch, gsplat/CMakeLists.txt), so
+there is no oracle/_ref build; the checker is the restatement in gsx_oracle.cpp.
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+SRC = os.path.join(HERE, "gsx_oracle.cpp")
+OUT = os.path.join(HERE, "libgsx_oracle.so")
+MATH_INC = os.path.join(ROOT, "lichtfeld-studio_amd", "csrc")
+
+# x86-64-v3 = AVX2 + FMA: gsx::fma must be the hardware instruction, and the binary has to run on
+# the GPU box's host CPU as well as here, so no -march=native.
+FLAGS = ["-O2", "-march=x86-64-v3", "-ffp-contract=off", "-fno-fast-math", "-fopenmp", "-shared", "-fPIC",
+         "-fvisibility=hidden", "-std=c++17", "-Wall", "-Wno-unknown-pragmas"]
+
+
+def build(force=True):
+    if not force and os.path.exists(OUT) and os.path.getmtime(OUT) >= max(
+            os.path.getmtime(SRC), os.path.getmtime(os.path.join(MATH_INC, "gsx_math.h"))):
+        return OUT
+    cmd = ["g++", *FLAGS, "-I", MATH_INC, SRC, "-o", OUT]
+    subprocess.run(cmd, check=True)
+    return OUT
+
+
+if __name__ == "__main__":
+    print(build(force="--if-stale" not in sys.argv))

@@ -1,0 +1,420 @@
+"""GPU parity: every kernel of libgsx.so, called through the C ABI, against the CPU checker on the same seeded
+inputs.  Bars: integer / index / key outputs and everything that feeds them bit-exact; forward image <= 1e-5
+absolute (it is bit-exact by construction, asserted as such); gradients and Adam state <= 1e-3 relative;
+SSIM <= 1e-5.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+def T(a, dev):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def N(t):
+    return t.detach().cpu().numpy()
+
+
+def small_scene(gsx, n=3000, seed=11, W=200, H=136, f=190.0, sh_degree=3):
+    sc = gsx.scenes.cluster_scene(n, seed, "small", sh_degree=sh_degree, logscale_mu=-3.3, logscale_sigma=0.6)
+    cam = gsx.scenes.orbit_camera(0.4, 4.0, W, H, f)
+    return sc, cam
+
+
+def rel_err(a, b, floor):
+    return np.abs(a - b) / (np.abs(b) + floor)
+
+
+# ---------------------------------------------------------------------------------------------
+# shared math primitives: device == host, bit for bit
+# ---------------------------------------------------------------------------------------------
+def test_math_primitives_bit_exact(gsx, orc, cuda):
+    import ctypes
+    L = gsx._lib
+    rng = np.random.default_rng(0)
+    n = 200_000
+    cases = {
+        0: (rng.uniform(-100, 95, n), None, "exp"),
+        1: (np.exp(rng.uniform(-80, 80, n)), None, "log"),
+        2: (np.exp(rng.uniform(-60, 60, n)), None, "rsqrt"),
+        3: (rng.uniform(-np.pi, np.pi, n), None, "sin"),
+        4: (rng.uniform(-1, 1, n), None, "acos"),
+        5: (rng.uniform(-30, 30, n), None, "sigmoid"),
+        6: (rng.uniform(-1e3, 1e5, n), None, "sat_u32"),
+        7: (rng.uniform(1e-6, 1.0, n), rng.uniform(0.01, 52, n), "pow"),
+        8: (rng.normal(0, 100, n), np.exp(rng.uniform(-30, 30, n)), "div"),
+        9: (np.exp(rng.uniform(-80, 80, n)), np.ones(n), "sqrt"),
+        10: (rng.normal(0, 1, n), rng.normal(0, 1, n), "fma"),
+    }
+    for which, (x, x2, name) in cases.items():
+        x = x.astype(np.float32)
+        xd = T(x, cuda)
+        x2d = None if x2 is None else T(x2.astype(np.float32), cuda)
+        y = torch.empty_like(xd)
+        L.check(L.lib().gsx_debug_math(ctypes.c_int(which), ctypes.c_uint32(n), ctypes.c_void_p(xd.data_ptr()),
+                                       ctypes.c_void_p(None if x2d is None else x2d.data_ptr()),
+                                       ctypes.c_void_p(y.data_ptr()), ctypes.c_void_p(None)))
+        torch.cuda.synchronize()
+        ref = orc.math_unary(name, x) if which < 7 else orc.math_binary(name, x, x2.astype(np.float32))
+        got = N(y)
+        assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), \
+            f"{name}: {np.sum(got.view(np.uint32) != ref.view(np.uint32))} of {n} differ"
+
+
+# ---------------------------------------------------------------------------------------------
+# projection / SH / intersect / sort / offsets: bit-exact
+# ---------------------------------------------------------------------------------------------
+def test_projection_bit_exact(gsx, orc, cuda):
+    ops = gsx.ops
+    sc, cam = small_scene(gsx, 20000)
+    means, quats, scales, op, shs = gsx.scenes.activate(sc)
+    for use_op, calc_comp in ((True, False), (False, False), (True, True)):
+        ref = orc.projection_ut_3dgs_fused(means, quats, scales, op if use_op else None, cam.viewmat[None],
+                                           cam.K[None], cam.width, cam.height, calc_compensations=calc_comp)
+        got = ops.projection_ut_3dgs_fused(T(means, cuda), T(quats, cuda), T(scales, cuda),
+                                           T(op, cuda) if use_op else None, T(cam.viewmat[None], cuda), None,
+                                           T(cam.K[None], cuda), cam.width, cam.height, 0.3, 0.01, 1e4, 0.0,
+                                           calc_comp, 0, ops.UnscentedTransformParameters(), 4)
+        radii = N(got[0])
+        assert np.array_equal(radii, ref[0])
+        vis = (radii[0, :, 0] > 0)
+        assert vis.sum() > 1000
+        for k, name in ((1, "means2d"), (2, "depths"), (3, "conics")):
+            a, b = N(got[k])[0][vis], ref[k][0][vis]
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), name
+        if calc_comp:
+            assert np.array_equal(N(got[4])[0][vis].view(np.uint32), ref[4][0][vis].view(np.uint32))
+
+
+def test_projection_unsupported_and_errors(gsx, cuda):
+    ops = gsx.ops
+    sc, cam = small_scene(gsx, 100)
+    means, quats, scales, op, shs = gsx.scenes.activate(sc)
+    args = [T(means, cuda), T(quats, cuda), T(scales, cuda), T(op, cuda), T(cam.viewmat[None], cuda), None,
+            T(cam.K[None], cuda), cam.width, cam.height, 0.3, 0.01, 1e4, 0.0, False]
+    with pytest.raises(gsx._lib.GsxError):  # fisheye model is not built
+        ops.projection_ut_3dgs_fused(*args, 2, ops.UnscentedTransformParameters(), 4)
+    with pytest.raises(gsx._lib.GsxError):  # rolling shutter is not built
+        ops.projection_ut_3dgs_fused(*args, 0, ops.UnscentedTransformParameters(), 0)
+    with pytest.raises(RuntimeError):  # CHECK_INPUT: CPU tensor
+        ops.projection_ut_3dgs_fused(torch.from_numpy(means), *args[1:], 0, ops.UnscentedTransformParameters(), 4)
+    with pytest.raises(RuntimeError):  # CHECK_INPUT: non-contiguous
+        ops.projection_ut_3dgs_fused(T(np.zeros((100, 6), np.float32), cuda)[:, ::2], *args[1:], 0,
+                                     ops.UnscentedTransformParameters(), 4)
+    # N == 0: no launch, empty outputs
+    e = lambda *s: torch.empty(s, dtype=torch.float32, device=cuda)
+    out = ops.projection_ut_3dgs_fused(e(0, 3), e(0, 4), e(0, 3), e(0), *args[4:], 0,
+                                       ops.UnscentedTransformParameters(), 4)
+    assert out[0].shape == (1, 0, 2)
+
+
+@pytest.mark.parametrize("degree", [0, 1, 2, 3, 4])
+def test_spherical_harmonics(gsx, orc, cuda, degree):
+    ops = gsx.ops
+    rng = np.random.default_rng(degree)
+    n, K = 5000, 25
+    dirs = rng.normal(0, 1, (n, 3)).astype(np.float32) * rng.uniform(0.1, 5, (n, 1)).astype(np.float32)
+    coeffs = rng.normal(0, 0.5, (n, K, 3)).astype(np.float32)
+    masks = rng.uniform(0, 1, n) < 0.8
+    v_colors = rng.normal(0, 1, (n, 3)).astype(np.float32)
+    ref = orc.spherical_harmonics_fwd(degree, dirs, coeffs, masks)
+    got = N(ops.spherical_harmonics_fwd(degree, T(dirs, cuda), T(coeffs, cuda), T(masks, cuda)))
+    assert np.array_equal(got[masks].view(np.uint32), ref[masks].view(np.uint32))
+    ref_vc, ref_vd = orc.spherical_harmonics_bwd(K, degree, dirs, coeffs, masks, v_colors, degree <= 3)
+    vc, vd = ops.spherical_harmonics_bwd(K, degree, T(dirs, cuda), T(coeffs, cuda), T(masks, cuda), T(v_colors, cuda),
+                                         degree <= 3)
+    assert np.array_equal(N(vc).view(np.uint32), ref_vc.view(np.uint32))
+    if degree <= 3:
+        np.testing.assert_allclose(N(vd)[masks], ref_vd[masks], rtol=1e-5, atol=1e-6)
+    # no mask
+    got = N(ops.spherical_harmonics_fwd(degree, T(dirs, cuda), T(coeffs, cuda), None))
+    assert np.array_equal(got.view(np.uint32), orc.spherical_harmonics_fwd(degree, dirs, coeffs, None).view(np.uint32))
+
+
+def _projected(gsx, orc, n, **kw):
+    sc, cam = small_scene(gsx, n, **kw)
+    means, quats, scales, op, shs = gsx.scenes.activate(sc)
+    radii, means2d, depths, conics, _ = orc.projection_ut_3dgs_fused(means, quats, scales, op, cam.viewmat[None],
+                                                                      cam.K[None], cam.width, cam.height)
+    return sc, cam, (means, quats, scales, op, shs), (radii, means2d, depths, conics)
+
+
+def test_intersect_sort_offsets_bit_exact(gsx, orc, cuda):
+    ops = gsx.ops
+    sc, cam, _, (radii, means2d, depths, conics) = _projected(gsx, orc, 30000)
+    tw, th = (cam.width + 15) // 16, (cam.height + 15) // 16
+    for sort in (False, True):
+        ref_tpg, ref_ids, ref_flat = orc.intersect_tile(means2d, radii, depths, 1, 16, tw, th, sort)
+        tpg, ids, flat = ops.intersect_tile(T(means2d, cuda), T(radii, cuda), T(depths, cuda), None, None, 1, 16, tw,
+                                            th, sort)
+        assert np.array_equal(N(tpg), ref_tpg)
+        assert ref_ids.shape[0] > 50000
+        assert np.array_equal(N(ids), ref_ids), f"keys differ (sort={sort})"
+        assert np.array_equal(N(flat), ref_flat), f"values differ (sort={sort})"
+    ref_off = orc.intersect_offset(ref_ids, 1, tw, th)
+    off = ops.intersect_offset(ids, 1, tw, th)
+    assert np.array_equal(N(off), ref_off)
+    # no intersections at all
+    off0 = ops.intersect_offset(torch.empty((0,), dtype=torch.int64, device=cuda), 1, tw, th)
+    assert int(off0.abs().sum()) == 0
+    radii0 = np.zeros_like(radii)
+    tpg, ids, flat = ops.intersect_tile(T(means2d, cuda), T(radii0, cuda), T(depths, cuda), None, None, 1, 16, tw, th)
+    assert ids.numel() == 0 and flat.numel() == 0 and int(tpg.sum()) == 0
+
+
+@pytest.mark.parametrize("n", [1, 63, 64, 65, 4095, 4096, 4097, 100_003, 3_000_000])
+def test_radix_sort_stable(gsx, orc, cuda, n):
+    ops = gsx.ops
+    rng = np.random.default_rng(n)
+    tile_bits, cam_bits = 12, 1
+    # few distinct depths and tiles: many exact ties, so stability is exercised
+    depth = rng.integers(0, 1 << 32, max(2, n // 50), dtype=np.uint64)[rng.integers(0, max(2, n // 50), n)]
+    tile = rng.integers(0, 4056, n).astype(np.uint64)
+    keys = ((tile << np.uint64(32)) | depth).astype(np.int64)
+    vals = rng.permutation(n).astype(np.int32)
+    ref_k, ref_v = orc.radix_sort_pairs(keys, vals, 32 + tile_bits + cam_bits)
+    k, v = ops.radix_sort_double_buffer(n, tile_bits, cam_bits, T(keys, cuda), T(vals, cuda))
+    assert np.array_equal(N(k), ref_k)
+    assert np.array_equal(N(v), ref_v)
+
+
+def test_radix_sort_bit_range(gsx, orc, cuda):
+    """only bits [0, end_bit) take part: keys that differ above end_bit keep their input order"""
+    import ctypes
+    L = gsx._lib
+    rng = np.random.default_rng(5)
+    n = 50_000
+    keys = rng.integers(0, 1 << 62, n, dtype=np.int64)
+    vals = np.arange(n, dtype=np.int32)
+    for end_bit in (1, 8, 13, 45, 64):
+        ref_k, ref_v = orc.radix_sort_pairs(keys, vals, end_bit)
+        k0, v0 = T(keys, cuda), T(vals, cuda)
+        k1, v1 = torch.empty_like(k0), torch.empty_like(v0)
+        ws = torch.empty((L.lib().gsx_radix_sort_pairs_workspace_bytes(ctypes.c_int64(n)),), dtype=torch.uint8,
+                         device=cuda)
+        sel = ctypes.c_int(0)
+        L.check(L.lib().gsx_radix_sort_pairs(ctypes.c_int64(n), ctypes.c_void_p(k0.data_ptr()),
+                                             ctypes.c_void_p(v0.data_ptr()), ctypes.c_void_p(k1.data_ptr()),
+                                             ctypes.c_void_p(v1.data_ptr()), ctypes.c_uint32(end_bit),
+                                             ctypes.c_void_p(ws.data_ptr()), ctypes.c_size_t(ws.numel()),
+                                             ctypes.byref(sel), ctypes.c_void_p(None)))
+        torch.cuda.synchronize()
+        k, v = (k1, v1) if sel.value else (k0, v0)
+        assert np.array_equal(N(k), ref_k) and np.array_equal(N(v), ref_v), end_bit
+
+
+# ---------------------------------------------------------------------------------------------
+# rasterizer
+# ---------------------------------------------------------------------------------------------
+def _fused_inputs(gsx, cuda, n, sh_degree=3, **kw):
+    sc, cam = small_scene(gsx, n, sh_degree=sh_degree, **kw)
+    means, quats, scales, op, shs = gsx.scenes.activate(sc)
+    host = dict(means=means, quats=quats, scales=scales, op=op, shs=shs, vm=cam.viewmat[None], K=cam.K[None],
+                bg=np.array([[0.1, 0.2, 0.3]], np.float32))
+    dev = {k: T(v, cuda) for k, v in host.items()}
+    return sc, cam, host, dev
+
+
+@pytest.mark.parametrize("n,bg", [(4000, True), (4000, False), (60000, True)])
+def test_fused_forward_bit_exact(gsx, orc, cuda, n, bg):
+    ops = gsx.ops
+    sc, cam, h, d = _fused_inputs(gsx, cuda, n)
+    ref = orc.rasterize_from_world_with_sh_fwd(h["means"], h["quats"], h["scales"], h["op"], h["shs"], 3,
+                                               h["bg"] if bg else None, cam.width, cam.height, 16, h["vm"], h["K"])
+    got = ops.rasterize_from_world_with_sh_fwd(d["means"], d["quats"], d["scales"], d["op"], d["shs"], 3,
+                                               d["bg"] if bg else None, None, cam.width, cam.height, 16, d["vm"], None,
+                                               d["K"], 0, 0.3, 0.01, 1e4, 0.0, 1.0, False, 0,
+                                               ops.UnscentedTransformParameters(), 4, return_isect_ids=True)
+    renders, alphas, radii, means2d, depths, colors, offsets, flat, last_ids, comp, ids = got
+    r_renders, r_alphas, r_radii, r_means2d, r_depths, r_colors, r_offsets, r_flat, r_last, r_comp, r_ids = ref
+    assert np.array_equal(N(radii), r_radii)
+    assert np.array_equal(N(ids), r_ids), "sorted tile keys"
+    assert np.array_equal(N(flat), r_flat), "sort order"
+    assert np.array_equal(N(offsets), r_offsets), "per-tile ranges"
+    vis = r_radii[0, :, 0] > 0
+    assert np.array_equal(N(colors)[0][vis].view(np.uint32), r_colors[0][vis].view(np.uint32))
+    assert np.array_equal(N(last_ids), r_last)
+    assert float(np.abs(N(renders) - r_renders).max()) <= 1e-5
+    assert float(np.abs(N(alphas) - r_alphas).max()) <= 1e-5
+    assert np.array_equal(N(renders).view(np.uint32), r_renders.view(np.uint32)), "image is expected bit-exact"
+    assert np.array_equal(N(alphas).view(np.uint32), r_alphas.view(np.uint32))
+    assert r_alphas.mean() > 0.05  # the scene actually covers the image
+
+
+def test_fused_backward(gsx, orc, cuda):
+    ops = gsx.ops
+    sc, cam, h, d = _fused_inputs(gsx, cuda, 20000)
+    ut = ops.UnscentedTransformParameters()
+    fwd = ops.rasterize_from_world_with_sh_fwd(d["means"], d["quats"], d["scales"], d["op"], d["shs"], 3, d["bg"],
+                                               None, cam.width, cam.height, 16, d["vm"], None, d["K"], 0, 0.3, 0.01,
+                                               1e4, 0.0, 1.0, False, 0, ut, 4)
+    renders, alphas, radii, means2d, depths, colors, offsets, flat, last_ids, comp = fwd
+    rng = np.random.default_rng(3)
+    v_r = rng.normal(0, 1, tuple(renders.shape)).astype(np.float32)
+    v_a = rng.normal(0, 1, tuple(alphas.shape)).astype(np.float32)
+    got = ops.rasterize_from_world_with_sh_bwd(d["means"], d["quats"], d["scales"], d["op"], d["shs"], 3, d["bg"],
+                                               None, cam.width, cam.height, 16, d["vm"], None, d["K"], 0, 0.3, 0.01,
+                                               1e4, 0.0, 1.0, False, 0, ut, 4, None, None, None, alphas, last_ids,
+                                               offsets, flat, colors, radii, means2d, depths, comp, T(v_r, cuda),
+                                               T(v_a, cuda))
+    ref = orc.rasterize_from_world_with_sh_bwd(h["means"], h["quats"], h["scales"], h["op"], h["shs"], 3, h["bg"],
+                                               cam.width, cam.height, 16, h["vm"], h["K"], 1.0, False, N(alphas),
+                                               N(last_ids), N(offsets), N(flat), N(colors), N(radii), None, v_r, v_a)
+    names = ["v_means", "v_quats", "v_scales", "v_opacities", "v_sh_coeffs"]
+    for name, a, b in zip(names, got, ref):
+        a, b = N(a).reshape(b.shape), b
+        assert np.isfinite(a).all(), name
+        scale = np.abs(b).max()
+        assert scale > 0, name
+        # relative to the element where it is large, to the tensor's scale where it is small (sums of
+        # cancelling terms): 1e-3 relative in both senses
+        err = np.abs(a - b) / (np.abs(b) + 1e-3 * scale)
+        assert err.max() < 1e-3, f"{name}: max rel err {err.max():.3e} at {np.argmax(err)} (scale {scale:.3e})"
+
+
+def test_raster_masks_and_channels(gsx, orc, cuda):
+    ops = gsx.ops
+    sc, cam, h, d = _fused_inputs(gsx, cuda, 4000)
+    ut = ops.UnscentedTransformParameters()
+    radii, means2d, depths, conics, _ = orc.projection_ut_3dgs_fused(h["means"], h["quats"], h["scales"], h["op"],
+                                                                      h["vm"], h["K"], cam.width, cam.height)
+    tw, th = (cam.width + 15) // 16, (cam.height + 15) // 16
+    _, ids, flat = orc.intersect_tile(means2d, radii, depths, 1, 16, tw, th)
+    off = orc.intersect_offset(ids, 1, tw, th)
+    rng = np.random.default_rng(9)
+    masks = rng.uniform(0, 1, (1, th, tw)) < 0.7
+    for cdim in (1, 3, 4):
+        colors = rng.uniform(0, 1, (1, h["means"].shape[0], cdim)).astype(np.float32)
+        bg = rng.uniform(0, 1, (1, cdim)).astype(np.float32)
+        ref = orc.rasterize_to_pixels_from_world_3dgs_fwd(h["means"], h["quats"], h["scales"], colors,
+                                                          h["op"][None], bg, masks, cam.width, cam.height, 16,
+                                                          h["vm"], h["K"], off, flat)
+        got = ops.rasterize_to_pixels_from_world_3dgs_fwd(d["means"], d["quats"], d["scales"], T(colors, cuda),
+                                                          T(h["op"][None], cuda), T(bg, cuda), T(masks, cuda),
+                                                          cam.width, cam.height, 16, d["vm"], None, d["K"], 0, ut, 4,
+                                                          None, None, None, T(off, cuda), T(flat, cuda))
+        pm = np.repeat(np.repeat(masks[0], 16, 0), 16, 1)[:cam.height, :cam.width]
+        assert np.array_equal(N(got[0]).view(np.uint32), ref[0].view(np.uint32)), cdim
+        assert np.array_equal(N(got[1])[0, pm].view(np.uint32), ref[1][0, pm].view(np.uint32))
+        assert np.array_equal(N(got[2])[0, pm], ref[2][0, pm])
+    with pytest.raises(gsx._lib.GsxError):  # channel count that is not built
+        ops.rasterize_to_pixels_from_world_3dgs_fwd(d["means"], d["quats"], d["scales"],
+                                                    torch.zeros((1, 4000, 5), device=cuda), T(h["op"][None], cuda),
+                                                    None, None, cam.width, cam.height, 16, d["vm"], None, d["K"], 0,
+                                                    ut, 4, None, None, None, T(off, cuda), T(flat, cuda))
+
+
+# ---------------------------------------------------------------------------------------------
+# SSIM / Adam / relocation / noise / quats
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", [(1, 3, 64, 80), (2, 3, 37, 53), (1, 1, 9, 9), (1, 3, 16, 16)])
+def test_fused_ssim(gsx, orc, cuda, shape):
+    ops = gsx.ops
+    rng = np.random.default_rng(shape[2])
+    img1 = rng.uniform(0, 1, shape).astype(np.float32)
+    img2 = np.clip(img1 + rng.normal(0, 0.1, shape), 0, 1).astype(np.float32)
+    C1, C2 = 0.01 ** 2, 0.03 ** 2
+    ref = orc.fusedssim(C1, C2, img1, img2, True)
+    got = ops.fusedssim(C1, C2, T(img1, cuda), T(img2, cuda), True)
+    for a, b in zip(got, ref):
+        np.testing.assert_allclose(N(a), b, rtol=0, atol=1e-5 * max(1.0, np.abs(b).max()))
+    assert abs(float(N(got[0]).mean()) - float(ref[0].mean())) < 1e-5
+    dL = rng.normal(0, 1, shape).astype(np.float32)
+    ref_b = orc.fusedssim_backward(C1, C2, img1, img2, dL, ref[1], ref[2], ref[3])
+    got_b = ops.fusedssim_backward(C1, C2, T(img1, cuda), T(img2, cuda), T(dL, cuda), got[1], got[2], got[3])
+    np.testing.assert_allclose(N(got_b), ref_b, rtol=1e-4, atol=1e-5 * np.abs(ref_b).max())
+    # train == False: no derivative maps
+    m, e1, e2, e3 = ops.fusedssim(C1, C2, T(img1, cuda), T(img2, cuda), False)
+    assert e1.numel() == 0 and np.array_equal(N(m), N(got[0]))
+
+
+@pytest.mark.parametrize("n", [1, 3, 1023, 1024, 1025, 300_001])
+def test_adam_step(gsx, orc, cuda, n):
+    ops = gsx.ops
+    rng = np.random.default_rng(n)
+    p = rng.normal(0, 1, n).astype(np.float32)
+    m = rng.normal(0, 0.1, n).astype(np.float32)
+    v = rng.uniform(0, 0.01, n).astype(np.float32)
+    g = rng.normal(0, 1, n).astype(np.float32)
+    g[::7] = 0
+    step = 3
+    bc1 = 1.0 / (1.0 - 0.9 ** step)
+    bc2 = 1.0 / np.sqrt(1.0 - 0.999 ** step)
+    pd, md, vd = T(p, cuda), T(m, cuda), T(v, cuda)
+    ops.adam_step(pd, md, vd, T(g, cuda), 1.6e-4, 0.9, 0.999, 1e-15, bc1, bc2)
+    orc.adam_step(p, m, v, g, 1.6e-4, 0.9, 0.999, 1e-15, bc1, bc2)
+    for a, b in ((pd, p), (md, m), (vd, v)):
+        assert np.array_equal(N(a).view(np.uint32), b.view(np.uint32))
+
+
+def test_adam_multi_matches_single(gsx, orc, cuda):
+    ops = gsx.ops
+    rng = np.random.default_rng(1)
+    sizes = [3000, 3, 45 * 1000 + 1, 0, 4000, 1000]
+    lrs = [1.6e-4, 2.5e-3, 2.5e-3 / 20, 5e-3, 1e-3, 5e-2]
+    groups, refs = [], []
+    for n, lr in zip(sizes, lrs):
+        p, m = rng.normal(0, 1, n).astype(np.float32), rng.normal(0, 0.1, n).astype(np.float32)
+        v, g = rng.uniform(0, 0.01, n).astype(np.float32), rng.normal(0, 1, n).astype(np.float32)
+        groups.append(dict(param=T(p, cuda), exp_avg=T(m, cuda), exp_avg_sq=T(v, cuda), param_grad=T(g, cuda), lr=lr,
+                           beta1=0.9, beta2=0.999, eps=1e-15, bias_correction1_rcp=10.0,
+                           bias_correction2_sqrt_rcp=31.6))
+        if n:
+            orc.adam_step(p, m, v, g, lr, 0.9, 0.999, 1e-15, 10.0, 31.6)
+        refs.append((p, m, v))
+    groups[4]["param_grad"] = None  # a group without gradient is skipped
+    untouched = N(groups[4]["param"]).copy()
+    ops.adam_step_multi(groups)
+    for i, (grp, (p, m, v)) in enumerate(zip(groups, refs)):
+        if i == 4:
+            assert np.array_equal(N(grp["param"]), untouched)
+            continue
+        assert np.array_equal(N(grp["param"]).view(np.uint32), p.view(np.uint32)), i
+        assert np.array_equal(N(grp["exp_avg"]).view(np.uint32), m.view(np.uint32))
+        assert np.array_equal(N(grp["exp_avg_sq"]).view(np.uint32), v.view(np.uint32))
+
+
+def binoms(n_max=51):
+    b = np.zeros((n_max, n_max), np.float32)
+    for n in range(n_max):
+        for k in range(n + 1):
+            x = np.float32(1.0)
+            for i in range(k):
+                x = np.float32(x * (np.float32(n - i) / np.float32(i + 1)))
+            b[n, k] = x
+    return b
+
+
+def test_relocation(gsx, orc, cuda):
+    ops = gsx.ops
+    rng = np.random.default_rng(2)
+    M = 20000
+    op = rng.uniform(0.005, 0.999, M).astype(np.float32)
+    sc = np.exp(rng.normal(-4, 1, (M, 3))).astype(np.float32)
+    ratios = rng.integers(1, 52, M).astype(np.int32)
+    b = binoms()
+    ref_o, ref_s = orc.relocation(op, sc, ratios, b, 51)
+    o, s = ops.relocation(T(op, cuda), T(sc, cuda), T(ratios, cuda), T(b, cuda), 51)
+    assert np.array_equal(N(o).view(np.uint32), ref_o.view(np.uint32))
+    assert np.array_equal(N(s).view(np.uint32), ref_s.view(np.uint32))
+
+
+def test_add_noise_and_quats(gsx, orc, cuda):
+    ops = gsx.ops
+    rng = np.random.default_rng(4)
+    n = 50000
+    ro = rng.normal(0, 2, n).astype(np.float32)
+    rs = rng.normal(-4, 1, (n, 3)).astype(np.float32)
+    rq = rng.normal(0, 1, (n, 4)).astype(np.float32)
+    noise = rng.normal(0, 1, (n, 3)).astype(np.float32)
+    means = rng.normal(0, 1, (n, 3)).astype(np.float32)
+    md = T(means, cuda)
+    ops.add_noise(T(ro, cuda), T(rs, cuda), T(rq, cuda), T(noise, cuda), md, 80.0)
+    orc.add_noise(ro, rs, rq, noise, means, 80.0)
+    assert np.array_equal(N(md).view(np.uint32), means.view(np.uint32))
+    R = ops.quats_to_rotmats(T(rq, cuda))
+    assert np.array_equal(N(R).view(np.uint32), orc.quats_to_rotmats(rq).view(np.uint32))
