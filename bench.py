@@ -1,0 +1,224 @@
+#!/usr/bin/env python3
+"""bench.py - throughput of the full 3D-Gaussian-splatting training step (fwd + loss + bwd + Adam) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps 20] [--warmup 5] [--config 3] [--no-cpu-baseline]
+
+Workload (BASELINE.json configs[2], the one the metric is quoted on): 1M SH-degree-3 Gaussians drawn from the
+32-cluster mixture, one 1237x822 pinhole camera on a radius-4 orbit, L = 0.8 L1 + 0.2 (1 - SSIM) against the render
+of an independently seeded 1M-Gaussian target scene, fused Adam over all parameter tensors.  Inputs are synthetic
+and already resident in HBM when the timed region starts.
+
+Prints ONE JSON line: it/s over exactly --steps steps, the dominant kernel's roofline figures measured with HIP
+events inside the timed region, per-kernel times / rates from a separate instrumented pass, and the CPU checker
+timed on the host cores on the same workload (a reported baseline, not a target).
+"""
+import argparse
+import ctypes
+import importlib.util
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+PKG_DIR = os.path.join(ROOT, "lichtfeld-studio_amd")
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# published MI355X peaks
+PEAK_HBM_GBS = 8000.0
+PEAK_FP32_TFLOPS = 157.3
+
+# algorithmic cost model: bytes per Gaussian / pixel / element, flops per (pixel, Gaussian) pair
+FLOPS_PAIR_FWD = 62.0          # evaluate one pair: 2 mat-vec, normalise, cross, dot, alpha/T update
+FLOPS_PAIR_FWD_COMPOSITE = 6.0  # colour FMAs of a composited pair
+FLOPS_PAIR_BWD_EVAL = 62.0     # recompute
+FLOPS_PAIR_BWD_VJP = 180.0     # VJP chain of a valid pair
+
+
+def load_package():
+    name = "lichtfeld_studio_amd"
+    if name in sys.modules:
+        return sys.modules[name]
+    spec = importlib.util.spec_from_file_location(name, os.path.join(PKG_DIR, "__init__.py"),
+                                                  submodule_search_locations=[PKG_DIR])
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules[name] = mod
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def algorithmic_bytes(N, K, H, W, n_isects, sort_bits):
+    """HBM bytes one launch of each streaming stage has to move (reads + writes), per the cost model."""
+    P = H * W
+    passes = (sort_bits + 7) // 8
+    return {
+        "activate_params": N * (32 + 32),
+        "projection_ut_3dgs_fused": N * (44 + 32),
+        "sh_colors_from_world": N * (12 + 12 * K + 8 + 12),
+        "intersect_tile_count": N * (16 + 4 + 4 + 8 + 4),
+        "intersect_tile_emit": N * (16 + 4 + 8) + n_isects * 12,
+        "radix_sort_pairs": n_isects * (8 + 24) * passes,
+        "intersect_offset": n_isects * 8 + (P // 256) * 4,
+        "image_from_render": P * (12 + 12 + 12),
+        "fusedssim": P * (24 + 12 + 36),
+        "fusedssim_backward": P * (72 + 12),
+        "render_grad_from_loss": P * (12 + 12 + 12 + 12 + 12),
+        "rasterize_bwd_clear": N * 64,
+        "rasterize_bwd_finish": N * (64 + 40 + 56),
+        "sh_colors_from_world_bwd": N * (12 + 8 + 12 + 12 + 12 * K),
+        "activate_params_bwd": N * (32 + 32 + 32),
+        "adam_step_multi": N * (11 + 3 * K) * 28,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", type=int, default=3, help="BASELINE configuration (3 = the metric's)")
+    ap.add_argument("--n", type=int, default=None, help="override the number of Gaussians (parity / debugging)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-threads", type=int, default=0, help="threads for the CPU baseline (0 = all)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (the path has no multi-GPU part); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    gsx = load_package()
+    gsx._lib.lib()  # fail loudly without the HIP library
+    from lichtfeld_studio_amd.trainer import TrainStep
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+
+    t0 = time.time()
+    sc = gsx.scenes.config(args.config, args.n)
+    cam = sc.cameras[0]
+    W, H = cam.width, cam.height
+    viewmat = torch.from_numpy(cam.viewmat[None].copy()).to(dev)
+    Kmat = torch.from_numpy(cam.K[None].copy()).to(dev)
+    # target: render of the independently seeded target scene by the same forward, clamped, CHW
+    if hasattr(sc, "target_scene"):
+        tgt = TrainStep(sc.target_scene, dev)
+        tgt.forward(viewmat, Kmat, W, H)
+        gt = tgt.render[0].clamp(0, 1).permute(2, 0, 1).contiguous()[None].clone()
+        del tgt
+        torch.cuda.empty_cache()
+    else:
+        gt = torch.from_numpy(sc.target[None].copy()).to(dev)
+    use_ssim = args.config != 1  # configuration 1 is L1 only
+    ts = TrainStep(sc, dev, use_ssim=use_ssim)
+    setup_s = time.time() - t0
+
+    dominant = "rasterize_bwd_accumulate"
+    for _ in range(args.warmup):
+        ts.step(viewmat, Kmat, W, H, gt)
+    torch.cuda.synchronize()
+    ts.start_timing([dominant, "rasterize_to_pixels_from_world_3dgs_fwd"])
+    t1 = time.perf_counter()
+    for _ in range(args.steps):
+        ts.step(viewmat, Kmat, W, H, gt)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t1
+    in_loop = ts.stop_timing()
+    ms_per_step = 1e3 * elapsed / args.steps
+    loss = [float(x) for x in ts.loss_out.cpu()]
+
+    # pair counts of the last forward (for flop rates)
+    stats = torch.zeros(3, dtype=torch.int64, device=dev)
+    L = gsx._lib
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    L.check(L.lib().gsx_rasterize_pair_stats(
+        ctypes.c_uint32(ts.N), ctypes.c_int64(ts.n_isects), p(ts.params["means"]), p(ts.act["quats"]),
+        p(ts.act["scales"]), p(ts.act["opacities"]), ctypes.c_uint32(W), ctypes.c_uint32(H), p(viewmat), p(Kmat),
+        p(ts.offsets), p(ts.flatten_ids), p(stats), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    pairs_fwd, pairs_comp, pairs_bwd = [int(x) for x in stats.cpu()]
+
+    # instrumented pass: every stage bracketed by events (not part of the timed region)
+    ts.start_timing(None)
+    n_prof = 5
+    for _ in range(n_prof):
+        ts.step(viewmat, Kmat, W, H, gt)
+    stage_ms = {k: float(np.mean(v)) for k, v in ts.stop_timing().items()}
+
+    tile_bits = int(L.lib().gsx_n_bits(ctypes.c_uint32(ts.tw * ts.th)))
+    abytes = algorithmic_bytes(ts.N, ts.K, H, W, ts.n_isects, 32 + tile_bits + 1)
+    kernels = {}
+    for k, ms in stage_ms.items():
+        e = {"ms": round(ms, 4)}
+        if k in abytes and ms > 0:
+            gbs = abytes[k] / (ms * 1e-3) / 1e9
+            e.update(bound="hbm", alg_bytes=int(abytes[k]), GBps=round(gbs, 1), frac=round(gbs / PEAK_HBM_GBS, 4))
+        kernels[k] = e
+    flops_fwd = FLOPS_PAIR_FWD * pairs_fwd + FLOPS_PAIR_FWD_COMPOSITE * pairs_comp
+    flops_bwd = FLOPS_PAIR_BWD_EVAL * pairs_bwd + FLOPS_PAIR_BWD_VJP * pairs_comp
+    for k, fl in (("rasterize_to_pixels_from_world_3dgs_fwd", flops_fwd), (dominant, flops_bwd)):
+        ms = float(np.mean(in_loop[k])) if k in in_loop else stage_ms.get(k, 0.0)
+        if ms > 0:
+            tf = fl / (ms * 1e-3) / 1e12
+            kernels.setdefault(k, {}).update(ms=round(ms, 4), bound="fp32_valu", alg_flops=int(fl),
+                                             TFLOPs=round(tf, 2), frac=round(tf / PEAK_FP32_TFLOPS, 4))
+    dom_ms = float(np.mean(in_loop[dominant]))
+    dom_tf = flops_bwd / (dom_ms * 1e-3) / 1e12
+    roofline = {
+        "kernel": "rasterize_bwd_kernel", "bound": "fp32_valu", "achieved": round(dom_tf, 3),
+        "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s", "frac": round(dom_tf / PEAK_FP32_TFLOPS, 4), "traffic": None,
+        "avg_launch_ms": round(dom_ms, 4), "launches": len(in_loop[dominant]),
+        "note": "no MFMA and not HBM-bound: per-pair fp32 vector ALU work; algorithmic flops = 62 x pairs "
+                "evaluated + 180 x pairs composited",
+    }
+
+    cpu_baseline = None
+    if not args.no_cpu_baseline:
+        cpu_baseline = run_cpu_baseline(gsx, sc, cam, gt.cpu().numpy()[0], use_ssim, args.cpu_threads)
+
+    out = {
+        "metric": "train it/s (fwd+bwd+Adam) at 1M SH3 Gaussians 1237x822; raster fwd/bwd ms",
+        "value": round(args.steps / elapsed, 3), "unit": "it/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"BASELINE configs[{args.config - 1}]: {ts.N} Gaussians SH degree {ts.sh_degree}, "
+                               f"{W}x{H}, fwd + " + ("0.8 L1 + 0.2 (1-SSIM)" if use_ssim else "L1") +
+                               " + bwd + fused Adam", "n_gaussians": ts.N, "image": [W, H], "n_isects": ts.n_isects,
+                   "tiles": ts.tw * ts.th, "pairs_fwd": pairs_fwd, "pairs_composited": pairs_comp,
+                   "pairs_bwd": pairs_bwd, "loss": loss, "setup_s": round(setup_s, 1)},
+        "raster_fwd_ms": kernels.get("rasterize_to_pixels_from_world_3dgs_fwd", {}).get("ms"),
+        "raster_bwd_ms": round(dom_ms, 4),
+        "roofline": roofline, "cpu_baseline": cpu_baseline, "kernels": kernels,
+    }
+    print(json.dumps(out))
+
+
+def run_cpu_baseline(gsx, sc, cam, gt_chw, use_ssim, threads):
+    """The CPU checker (a port of the reference kernels; the reference itself has no CPU path) on the host cores:
+    one full step - forward, loss, backward, Adam - of the same workload."""
+    import numpy as np
+    from oracle import oracle as orc
+    from oracle.step import OracleTrainStep
+    if threads > 0:
+        orc.set_num_threads(threads)
+    cores = orc.num_threads()
+    st = OracleTrainStep(sc, lambda_dssim=0.2 if use_ssim else 0.0)
+    t0 = time.perf_counter()
+    st.step(cam.viewmat, cam.K, cam.width, cam.height, np.ascontiguousarray(gt_chw))
+    dt = time.perf_counter() - t0
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {"value": round(1.0 / dt, 5), "unit": "it/s", "cores": cores, "kind": "port",
+            "sample": f"1 full step of the same workload ({st.params['means'].shape[0]} Gaussians, "
+                      f"{cam.width}x{cam.height}), OpenMP over Gaussians / tiles / image planes",
+            "seconds": round(dt, 2), "cpu": model, "loss": [round(x, 6) for x in st.loss]}
+
+
+if __name__ == "__main__":
+    main()

@@ -130,11 +130,34 @@ GSX_API int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
     const int32_t* tile_offsets, const int32_t* flatten_ids, float* render_colors, float* render_alphas,
     int32_t* last_ids, void* stream);
 
+/* Pair counts of one forward pass, for turning kernel times into rates (no counterpart in the reference).
+ * stats_out: device uint64[3] = {pairs the forward evaluates, pairs composited, pairs the backward evaluates};
+ * the counts are ADDED to it, so zero it first. */
+GSX_API int gsx_rasterize_pair_stats(uint32_t N, int64_t n_isects, const float* means, const float* quats,
+                                     const float* scales, const float* opacities, uint32_t image_width,
+                                     uint32_t image_height, const float* viewmat, const float* K,
+                                     const int32_t* tile_offsets, const int32_t* flatten_ids,
+                                     unsigned long long* stats_out, void* stream);
+
 /* ---- a8: gsplat::rasterize_to_pixels_from_world_3dgs_bwd (Ops.h:131-166; ...3DGSBwd.cu:16-379) ----
  * channels must be 3.  The five gradient outputs are fully WRITTEN (no zero-fill needed; the reference
  * zero-fills and accumulates, Rasterization.cpp:190-194): v_means [N,3], v_quats [N,4], v_scales [N,3],
  * v_colors [C,N,3], v_opacities [C,N].  The workspace holds 16 floats per Gaussian. */
 GSX_API size_t gsx_rasterize_bwd_workspace_bytes(uint32_t N);
+/* The backward pass is three launches - clear the accumulators, the per-tile kernel, the per-Gaussian epilogue -
+ * that can also be called one by one (a training loop can fold the epilogue into its own per-Gaussian pass). */
+GSX_API int gsx_rasterize_bwd_clear(uint32_t N, void* workspace, size_t workspace_bytes, void* stream);
+GSX_API int gsx_rasterize_bwd_accumulate(
+    uint32_t C, uint32_t N, int64_t n_isects, const float* means, const float* quats, const float* scales,
+    const float* colors, const float* opacities, const float* backgrounds, const uint8_t* masks,
+    uint32_t image_width, uint32_t image_height, uint32_t tile_size, const float* viewmats0, const float* Ks,
+    const int32_t* tile_offsets, const int32_t* flatten_ids, const float* render_alphas, const int32_t* last_ids,
+    const float* v_render_colors, const float* v_render_alphas, void* workspace, size_t workspace_bytes,
+    void* stream);
+GSX_API int gsx_rasterize_bwd_finish(uint32_t N, const float* means, const float* quats, const float* scales,
+                                     const float* viewmats0, const void* workspace, size_t workspace_bytes,
+                                     float* v_means, float* v_quats, float* v_scales, float* v_colors,
+                                     float* v_opacities, void* stream);
 GSX_API int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
     uint32_t C, uint32_t N, int64_t n_isects, const float* means, const float* quats, const float* scales,
     const float* colors, const float* opacities, const float* backgrounds, const uint8_t* masks,
@@ -178,6 +201,12 @@ typedef struct gsx_adam_group {
     const float* grad;
     int64_t n;
     float lr, beta1, beta2, eps, bias_correction1_rcp, bias_correction2_sqrt_rcp;
+    /* Two parameter groups stored interleaved in one tensor (sh0 | shN as one [N,K,3] array): when period > 0,
+     * elements with (index % period) >= split use lr2, and are left untouched (moments too) when skip2 != 0
+     * (fused_adam.cpp:69-70 skips the shN group early in training).  period == 0: plain group. */
+    uint32_t period, split;
+    float lr2;
+    int32_t skip2;
 } gsx_adam_group;
 GSX_API int gsx_adam_step_multi(const gsx_adam_group* groups_host, int n_groups, void* stream);
 

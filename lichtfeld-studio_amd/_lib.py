@@ -41,7 +41,8 @@ class UTParams(ctypes.Structure):
 class AdamGroup(ctypes.Structure):
     _fields_ = [("param", c_p), ("exp_avg", c_p), ("exp_avg_sq", c_p), ("grad", c_p), ("n", c_i64), ("lr", c_f),
                 ("beta1", c_f), ("beta2", c_f), ("eps", c_f), ("bias_correction1_rcp", c_f),
-                ("bias_correction2_sqrt_rcp", c_f)]
+                ("bias_correction2_sqrt_rcp", c_f), ("period", c_u32), ("split", c_u32), ("lr2", c_f),
+                ("skip2", ctypes.c_int32)]
 
 
 class GsxError(RuntimeError):

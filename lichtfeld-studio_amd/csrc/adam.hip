@@ -20,6 +20,9 @@ struct AdamTable {
     uint32_t first_block[GSX_ADAM_MAX_TENSORS + 1];
     float lr[GSX_ADAM_MAX_TENSORS], beta1[GSX_ADAM_MAX_TENSORS], beta2[GSX_ADAM_MAX_TENSORS];
     float eps[GSX_ADAM_MAX_TENSORS], bc1_rcp[GSX_ADAM_MAX_TENSORS], bc2_sqrt_rcp[GSX_ADAM_MAX_TENSORS];
+    uint32_t period[GSX_ADAM_MAX_TENSORS], split[GSX_ADAM_MAX_TENSORS];
+    float lr2[GSX_ADAM_MAX_TENSORS];
+    int32_t skip2[GSX_ADAM_MAX_TENSORS];
     int n_groups;
 };
 
@@ -50,23 +53,43 @@ __global__ void __launch_bounds__(256) adam_multi_kernel(const AdamTable tab) {
     const float* __restrict__ G = tab.grad[gi];
     const float lr = tab.lr[gi], b1 = tab.beta1[gi], b2 = tab.beta2[gi], eps = tab.eps[gi];
     const float c1 = tab.bc1_rcp[gi], c2 = tab.bc2_sqrt_rcp[gi];
+    const uint32_t period = tab.period[gi], split = tab.split[gi];
+    const float lr2 = tab.lr2[gi];
+    const bool skip2 = tab.skip2[gi] != 0;
     const bool aligned = ((((uintptr_t)P) | ((uintptr_t)M) | ((uintptr_t)V) | ((uintptr_t)G)) & 15u) == 0;
     if (aligned && base + kAdamVec <= n) {
         float4 p = *reinterpret_cast<float4*>(P + base);
         float4 m = *reinterpret_cast<float4*>(M + base);
         float4 v = *reinterpret_cast<float4*>(V + base);
         const float4 g = *reinterpret_cast<const float4*>(G + base);
-        adam_one(p.x, m.x, v.x, g.x, lr, b1, b2, eps, c1, c2);
-        adam_one(p.y, m.y, v.y, g.y, lr, b1, b2, eps, c1, c2);
-        adam_one(p.z, m.z, v.z, g.z, lr, b1, b2, eps, c1, c2);
-        adam_one(p.w, m.w, v.w, g.w, lr, b1, b2, eps, c1, c2);
+        float lrs[4] = {lr, lr, lr, lr};
+        bool upd[4] = {true, true, true, true};
+        if (period) {
+#pragma unroll
+            for (uint32_t k = 0; k < 4; ++k) {
+                const bool second = ((base + k) % period) >= split;
+                lrs[k] = second ? lr2 : lr;
+                upd[k] = !(second && skip2);
+            }
+        }
+        if (upd[0])
+            adam_one(p.x, m.x, v.x, g.x, lrs[0], b1, b2, eps, c1, c2);
+        if (upd[1])
+            adam_one(p.y, m.y, v.y, g.y, lrs[1], b1, b2, eps, c1, c2);
+        if (upd[2])
+            adam_one(p.z, m.z, v.z, g.z, lrs[2], b1, b2, eps, c1, c2);
+        if (upd[3])
+            adam_one(p.w, m.w, v.w, g.w, lrs[3], b1, b2, eps, c1, c2);
         *reinterpret_cast<float4*>(P + base) = p;
         *reinterpret_cast<float4*>(M + base) = m;
         *reinterpret_cast<float4*>(V + base) = v;
     } else {
         for (uint32_t i = base; i < n && i < base + kAdamVec; ++i) {
+            const bool second = period && (i % period) >= split;
+            if (second && skip2)
+                continue;
             float p = P[i], m = M[i], v = V[i];
-            adam_one(p, m, v, G[i], lr, b1, b2, eps, c1, c2);
+            adam_one(p, m, v, G[i], second ? lr2 : lr, b1, b2, eps, c1, c2);
             P[i] = p;
             M[i] = m;
             V[i] = v;
@@ -105,6 +128,10 @@ extern "C" int gsx_adam_step_multi(const gsx_adam_group* groups, int n_groups, v
         tab.eps[k] = g.eps;
         tab.bc1_rcp[k] = g.bias_correction1_rcp;
         tab.bc2_sqrt_rcp[k] = g.bias_correction2_sqrt_rcp;
+        tab.period[k] = g.period;
+        tab.split[k] = g.split;
+        tab.lr2[k] = g.lr2;
+        tab.skip2[k] = g.skip2;
         blocks += cdiv((uint64_t)g.n, kAdamChunk);
         ++k;
     }
@@ -136,5 +163,9 @@ extern "C" int gsx_adam_step(float* param, float* exp_avg, float* exp_avg_sq, co
     g.eps = eps;
     g.bias_correction1_rcp = bias_correction1_rcp;
     g.bias_correction2_sqrt_rcp = bias_correction2_sqrt_rcp;
+    g.period = 0;
+    g.split = 0;
+    g.lr2 = 0.f;
+    g.skip2 = 0;
     return gsx_adam_step_multi(&g, 1, stream);
 }

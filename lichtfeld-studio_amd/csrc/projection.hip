@@ -302,10 +302,11 @@ __global__ void __launch_bounds__(256) sh_bwd_kernel(uint32_t N, uint32_t K, uin
             v[c] = v_colors[e * 3 + c];
     }
     for (uint32_t k = 0; k < K; ++k) {
-        const float b = ((int)k < nb) ? B[k < 25 ? k : 24] : 0.f;
-        out[k * 3 + 0] = b * v[0];
-        out[k * 3 + 1] = b * v[1];
-        out[k * 3 + 2] = b * v[2];
+        const bool used = (int)k < nb;
+        const float b = B[k < 25 ? k : 24];
+        out[k * 3 + 0] = used ? b * v[0] : 0.f;
+        out[k * 3 + 1] = used ? b * v[1] : 0.f;
+        out[k * 3 + 2] = used ? b * v[2] : 0.f;
     }
 }
 
@@ -513,10 +514,11 @@ __global__ void __launch_bounds__(256) sh_world_bwd_kernel(uint32_t N, uint32_t 
             v[c] = colors[e * 3 + c] <= 0.0f ? 0.f : v_colors[e * 3 + c];
     }
     for (uint32_t k = 0; k < K; ++k) {
-        const float b = ((int)k < nb) ? B[k < 25 ? k : 24] : 0.f;
-        out[k * 3 + 0] = b * v[0];
-        out[k * 3 + 1] = b * v[1];
-        out[k * 3 + 2] = b * v[2];
+        const bool used = (int)k < nb;
+        const float b = B[k < 25 ? k : 24];
+        out[k * 3 + 0] = used ? b * v[0] : 0.f;
+        out[k * 3 + 1] = used ? b * v[1] : 0.f;
+        out[k * 3 + 2] = used ? b * v[2] : 0.f;
     }
 }
 } // namespace gsx

@@ -321,6 +321,68 @@ using namespace gsx;
 
 extern "C" size_t gsx_rasterize_bwd_workspace_bytes(uint32_t N) { return align_up((size_t)N * kAcc * 4, 256) + 256; }
 
+// stage 1: zero the per-Gaussian accumulators
+extern "C" int gsx_rasterize_bwd_clear(uint32_t N, void* workspace, size_t workspace_bytes, void* stream) {
+    if (N == 0)
+        return GSX_OK;
+    GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 &&
+                    workspace_bytes >= gsx_rasterize_bwd_workspace_bytes(N),
+                GSX_ERR_WORKSPACE, "rasterize bwd: workspace needs %zu bytes, 256-byte aligned",
+                gsx_rasterize_bwd_workspace_bytes(N));
+    const size_t n_acc = (size_t)N * kAcc;
+    hipLaunchKernelGGL(fill_f32_kernel, dim3(cdiv(n_acc, 256)), dim3(256), 0, (hipStream_t)stream, n_acc, 0.f,
+                       (float*)workspace);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+// stage 2: the per-tile kernel, accumulating into the workspace
+extern "C" int gsx_rasterize_bwd_accumulate(
+    uint32_t C, uint32_t N, int64_t n_isects, const float* means, const float* quats, const float* scales,
+    const float* colors, const float* opacities, const float* backgrounds, const uint8_t* masks,
+    uint32_t image_width, uint32_t image_height, uint32_t tile_size, const float* viewmats0, const float* Ks,
+    const int32_t* tile_offsets, const int32_t* flatten_ids, const float* render_alphas, const int32_t* last_ids,
+    const float* v_render_colors, const float* v_render_alphas, void* workspace, size_t workspace_bytes,
+    void* stream) {
+    GSX_REQUIRE(C == 1, GSX_ERR_UNSUPPORTED, "C = %u cameras: only C == 1 is supported", C);
+    if (N == 0 || n_isects == 0 || image_width == 0 || image_height == 0) // ...Bwd.cu:440-443
+        return GSX_OK;
+    GSX_REQUIRE(tile_size == kTile, GSX_ERR_UNSUPPORTED, "rasterize bwd: tile_size %u (only 16 is built)", tile_size);
+    GSX_REQUIRE(n_isects > 0 && n_isects < (1ll << 31), GSX_ERR_OVERFLOW, "rasterize bwd: n_isects out of range");
+    GSX_REQUIRE(means && quats && scales && colors && opacities && viewmats0 && Ks && tile_offsets && flatten_ids &&
+                    render_alphas && last_ids && v_render_colors && v_render_alphas,
+                GSX_ERR_INVALID_ARGUMENT, "rasterize bwd: null tensor");
+    GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 &&
+                    workspace_bytes >= gsx_rasterize_bwd_workspace_bytes(N),
+                GSX_ERR_WORKSPACE, "rasterize bwd: workspace needs %zu bytes, 256-byte aligned",
+                gsx_rasterize_bwd_workspace_bytes(N));
+    const uint32_t tw = cdiv(image_width, kTile), th = cdiv(image_height, kTile);
+    hipLaunchKernelGGL(rasterize_bwd_kernel, dim3(tw * th), dim3(256), 0, (hipStream_t)stream, (uint32_t)n_isects,
+                       means, quats, scales, colors, opacities, backgrounds, masks, image_width, image_height, tw, th,
+                       viewmats0, Ks, tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors,
+                       v_render_alphas, (float*)workspace);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+// stage 3: per-Gaussian epilogue, accumulators -> the five gradient tensors (all elements written)
+extern "C" int gsx_rasterize_bwd_finish(uint32_t N, const float* means, const float* quats, const float* scales,
+                                        const float* viewmats0, const void* workspace, size_t workspace_bytes,
+                                        float* v_means, float* v_quats, float* v_scales, float* v_colors,
+                                        float* v_opacities, void* stream) {
+    if (N == 0)
+        return GSX_OK;
+    GSX_REQUIRE(means && quats && scales && viewmats0 && v_means && v_quats && v_scales && v_colors && v_opacities,
+                GSX_ERR_INVALID_ARGUMENT, "rasterize bwd: null tensor");
+    GSX_REQUIRE(workspace != nullptr && workspace_bytes >= gsx_rasterize_bwd_workspace_bytes(N), GSX_ERR_WORKSPACE,
+                "rasterize bwd: workspace needs %zu bytes", gsx_rasterize_bwd_workspace_bytes(N));
+    hipLaunchKernelGGL(rasterize_bwd_epilogue_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, means,
+                       quats, scales, viewmats0, (const float*)workspace, v_means, v_quats, v_scales, v_colors,
+                       v_opacities);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
 extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
     uint32_t C, uint32_t N, int64_t n_isects, const float* means, const float* quats, const float* scales,
     const float* colors, const float* opacities, const float* backgrounds, const uint8_t* masks,
@@ -331,38 +393,17 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
     const float* v_render_alphas, float* v_means, float* v_quats, float* v_scales, float* v_colors,
     float* v_opacities, void* workspace, size_t workspace_bytes, void* stream) {
     (void)ut;
-    const int rc = check_camera_args(C, viewmats1, camera_model, rs_type, radial_coeffs, tangential_coeffs,
-                                     thin_prism_coeffs);
+    int rc = check_camera_args(C, viewmats1, camera_model, rs_type, radial_coeffs, tangential_coeffs,
+                               thin_prism_coeffs);
     if (rc != GSX_OK)
         return rc;
-    if (N == 0)
-        return GSX_OK;
-    GSX_REQUIRE(tile_size == kTile, GSX_ERR_UNSUPPORTED, "rasterize bwd: tile_size %u (only 16 is built)", tile_size);
-    GSX_REQUIRE(n_isects >= 0 && n_isects < (1ll << 31), GSX_ERR_OVERFLOW, "rasterize bwd: n_isects out of range");
-    GSX_REQUIRE(means && quats && scales && colors && opacities && viewmats0 && Ks && tile_offsets && render_alphas &&
-                    last_ids && v_render_colors && v_render_alphas && v_means && v_quats && v_scales && v_colors &&
-                    v_opacities,
-                GSX_ERR_INVALID_ARGUMENT, "rasterize bwd: null tensor");
-    GSX_REQUIRE(n_isects == 0 || flatten_ids, GSX_ERR_INVALID_ARGUMENT, "rasterize bwd: flatten_ids is null");
-    GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 &&
-                    workspace_bytes >= gsx_rasterize_bwd_workspace_bytes(N),
-                GSX_ERR_WORKSPACE, "rasterize bwd: workspace needs %zu bytes, 256-byte aligned",
-                gsx_rasterize_bwd_workspace_bytes(N));
-    float* gacc = (float*)workspace;
-    hipStream_t s = (hipStream_t)stream;
-    const size_t n_acc = (size_t)N * kAcc;
-    hipLaunchKernelGGL(fill_f32_kernel, dim3(cdiv(n_acc, 256)), dim3(256), 0, s, n_acc, 0.f, gacc);
-    GSX_LAUNCH_CHECK();
-    if (n_isects > 0 && image_width > 0 && image_height > 0) { // ...Bwd.cu:440-443
-        const uint32_t tw = cdiv(image_width, kTile), th = cdiv(image_height, kTile);
-        hipLaunchKernelGGL(rasterize_bwd_kernel, dim3(tw * th), dim3(256), 0, s, (uint32_t)n_isects, means, quats,
-                           scales, colors, opacities, backgrounds, masks, image_width, image_height, tw, th, viewmats0,
-                           Ks, tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors, v_render_alphas,
-                           gacc);
-        GSX_LAUNCH_CHECK();
-    }
-    hipLaunchKernelGGL(rasterize_bwd_epilogue_kernel, dim3(cdiv(N, 256)), dim3(256), 0, s, N, means, quats, scales,
-                       viewmats0, gacc, v_means, v_quats, v_scales, v_colors, v_opacities);
-    GSX_LAUNCH_CHECK();
-    return GSX_OK;
+    if ((rc = gsx_rasterize_bwd_clear(N, workspace, workspace_bytes, stream)) != GSX_OK)
+        return rc;
+    if ((rc = gsx_rasterize_bwd_accumulate(C, N, n_isects, means, quats, scales, colors, opacities, backgrounds,
+                                           masks, image_width, image_height, tile_size, viewmats0, Ks, tile_offsets,
+                                           flatten_ids, render_alphas, last_ids, v_render_colors, v_render_alphas,
+                                           workspace, workspace_bytes, stream)) != GSX_OK)
+        return rc;
+    return gsx_rasterize_bwd_finish(N, means, quats, scales, viewmats0, workspace, workspace_bytes, v_means, v_quats,
+                                    v_scales, v_colors, v_opacities, stream);
 }

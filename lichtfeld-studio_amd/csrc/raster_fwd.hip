@@ -21,7 +21,10 @@ struct StagedGaussian {        // 64 bytes
     float m22, c0, c1, c2;     // colour (channels 0..2)
 };
 
-template <uint32_t CDIM>
+// STATS: also count the (pixel, Gaussian) pairs this launch evaluates / composites (for roofline accounting);
+// stats[0] += pairs evaluated, stats[1] += pairs composited, stats[2] += pairs the backward pass will evaluate
+// (entries up to each pixel's last contributor).
+template <uint32_t CDIM, bool STATS>
 __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
     uint32_t n_isects, const float* __restrict__ means, const float* __restrict__ quats,
     const float* __restrict__ scales, const float* __restrict__ colors, const float* __restrict__ opacities,
@@ -29,7 +32,7 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
     uint32_t image_height, uint32_t tile_width, uint32_t tile_height, const float* __restrict__ viewmat,
     const float* __restrict__ Kmat, const int32_t* __restrict__ tile_offsets,
     const int32_t* __restrict__ flatten_ids, float* __restrict__ render_colors, float* __restrict__ render_alphas,
-    int32_t* __restrict__ last_ids) {
+    int32_t* __restrict__ last_ids, unsigned long long* __restrict__ stats) {
     __shared__ float4 stage[kBatch * 4];
     __shared__ float extra[CDIM > 3 ? kBatch * (CDIM - 3) : 1]; // channels beyond the third
 
@@ -67,6 +70,7 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
 #pragma unroll
     for (uint32_t k = 0; k < CDIM; ++k)
         pix_out[k] = 0.f;
+    uint32_t n_eval = 0, n_comp = 0;
 
     for (uint32_t b = 0; b < num_batches; ++b) {
         // all four waves saturated: nothing left to stage (:190-194)
@@ -104,6 +108,8 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
                 break; // this wave's 64 pixels are all saturated
             if (done)
                 continue;
+            if (STATS)
+                ++n_eval;
             const float4 a = stage[t * 4 + 0];
             const float4 m0 = stage[t * 4 + 1];
             const float4 m1 = stage[t * 4 + 2];
@@ -138,7 +144,18 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
                 pix_out[k] = fma(extra[t * (CDIM > 3 ? CDIM - 3 : 1) + (k - 3)], vis, pix_out[k]);
             cur_idx = batch_start + t;
             T = next_T;
+            if (STATS)
+                ++n_comp;
         }
+    }
+    if (STATS) {
+        if (inside) {
+            atomicAdd(&stats[0], (unsigned long long)n_eval);
+            atomicAdd(&stats[1], (unsigned long long)n_comp);
+            if (n_comp)
+                atomicAdd(&stats[2], (unsigned long long)(cur_idx - (uint32_t)range_start + 1u));
+        }
+        return;
     }
 
     if (inside) {
@@ -179,10 +196,11 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
     const uint32_t tw = cdiv(image_width, kTile), th = cdiv(image_height, kTile);
     const dim3 grid(tw * th), block(256);
     hipStream_t s = (hipStream_t)stream;
-#define GSX_LAUNCH_FWD(CD)                                                                                        \
-    hipLaunchKernelGGL(rasterize_fwd_kernel<CD>, grid, block, 0, s, (uint32_t)n_isects, means, quats, scales, colors, \
-                       opacities, backgrounds, masks, image_width, image_height, tw, th, viewmats0, Ks, tile_offsets, \
-                       flatten_ids, render_colors, render_alphas, last_ids)
+#define GSX_LAUNCH_FWD(CD)                                                                                         \
+    hipLaunchKernelGGL((rasterize_fwd_kernel<CD, false>), grid, block, 0, s, (uint32_t)n_isects, means, quats, scales, \
+                       colors, opacities, backgrounds, masks, image_width, image_height, tw, th, viewmats0, Ks,        \
+                       tile_offsets, flatten_ids, render_colors, render_alphas, last_ids,                              \
+                       (unsigned long long*)nullptr)
     switch (channels) { // the channel counts the render modes of Rasterization.cpp:374-393 produce
     case 1: GSX_LAUNCH_FWD(1); break;
     case 3: GSX_LAUNCH_FWD(3); break;
@@ -192,6 +210,29 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
         return GSX_ERR_UNSUPPORTED;
     }
 #undef GSX_LAUNCH_FWD
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+// Pair counts of one forward pass (no counterpart in the reference; used to turn kernel times into flop rates).
+// stats_out: three device uint64 {pairs evaluated by the forward, pairs composited, pairs the backward evaluates};
+// they are ADDED to, so zero them first.
+extern "C" int gsx_rasterize_pair_stats(uint32_t N, int64_t n_isects, const float* means, const float* quats,
+                                        const float* scales, const float* opacities, uint32_t image_width,
+                                        uint32_t image_height, const float* viewmat, const float* K,
+                                        const int32_t* tile_offsets, const int32_t* flatten_ids,
+                                        unsigned long long* stats_out, void* stream) {
+    (void)N;
+    if (image_width == 0 || image_height == 0 || n_isects <= 0)
+        return GSX_OK;
+    GSX_REQUIRE(means && quats && scales && opacities && viewmat && K && tile_offsets && flatten_ids && stats_out,
+                GSX_ERR_INVALID_ARGUMENT, "rasterize_pair_stats: null tensor");
+    const uint32_t tw = cdiv(image_width, kTile), th = cdiv(image_height, kTile);
+    // colours are not needed for counting: the means array stands in (3 floats per Gaussian, same layout)
+    hipLaunchKernelGGL((rasterize_fwd_kernel<3, true>), dim3(tw * th), dim3(256), 0, (hipStream_t)stream,
+                       (uint32_t)n_isects, means, quats, scales, means, opacities, (const float*)nullptr,
+                       (const uint8_t*)nullptr, image_width, image_height, tw, th, viewmat, K, tile_offsets,
+                       flatten_ids, (float*)nullptr, (float*)nullptr, (int32_t*)nullptr, stats_out);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

@@ -1,0 +1,255 @@
+"""One training iteration of LichtFeld's `--gut` path (Trainer::train_step, src/training/trainer.cpp:599-875) on
+the gfx950 kernels: activations -> fused rasterization with SH (Rasterization.cpp:279-467) -> photometric loss
+(trainer.cpp:126-129) -> backward (Rasterization.cpp:469-642 + the autograd of the activations and of the loss)
+-> fused Adam over the six parameter groups (mcmc.cpp:479-497, fused_adam.cpp:22-95).
+
+Differences in organisation (not in arithmetic): every buffer is allocated once and reused; sh0 and shN live in
+one [N,K,3] tensor (no 192 B/Gaussian concatenation per step, splat_data.cpp:285) whose two learning rates the Adam
+kernel applies by element index; all parameter groups are updated by one launch; the ATen glue passes are fused
+into the kernels that produce or consume their data.
+"""
+import ctypes
+import math
+
+import numpy as np
+import torch
+
+from . import _lib as L
+from ._lib import UTParams, c_f, c_i, c_i64, c_p, c_sz, c_u32, check, lib
+
+# mcmc.cpp:487-492 / include/core/parameters.hpp:19-23
+DEFAULT_LRS = dict(means=1.6e-4, sh0=2.5e-3, shN=2.5e-3 / 20.0, scaling=5e-3, rotation=1e-3, opacity=5e-2)
+
+
+def _p(t):
+    return c_p(None) if t is None else c_p(t.data_ptr())
+
+
+class TrainStep:
+    def __init__(self, scene, device="cuda:0", lrs=None, lambda_dssim=0.2, betas=(0.9, 0.999), eps=1e-15,
+                 scene_scale=1.0, sh_degree=None, use_ssim=True):
+        self.dev = torch.device(device)
+        self.lib = lib()
+        f = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(self.dev)
+        self.N = scene.means.shape[0]
+        self.K = 1 + scene.shN.shape[1]
+        self.sh_degree = scene.sh_degree if sh_degree is None else sh_degree
+        # raw trainable tensors (include/core/splat_data.hpp:68-79); sh0 | shN share one [N,K,3] tensor
+        self.params = dict(
+            means=f(scene.means), shs=f(np.concatenate([scene.sh0, scene.shN], 1)), scaling=f(scene.scaling_raw),
+            rotation=f(scene.rotation_raw), opacity=f(scene.opacity_raw.reshape(-1)))
+        self.grads = {k: torch.zeros_like(v) for k, v in self.params.items()}
+        self.exp_avg = {k: torch.zeros_like(v) for k, v in self.params.items()}
+        self.exp_avg_sq = {k: torch.zeros_like(v) for k, v in self.params.items()}
+        self.step_count = 0
+        self.iteration = 0
+        lrs = dict(DEFAULT_LRS, **(lrs or {}))
+        lrs["means"] = lrs["means"] * scene_scale
+        self.lrs = lrs
+        self.betas, self.eps = betas, eps
+        self.lambda_dssim = lambda_dssim if use_ssim else 0.0
+        self.use_ssim = use_ssim
+        self.ut = UTParams()
+        N = self.N
+        e = lambda *s, dt=torch.float32: torch.empty(s, dtype=dt, device=self.dev)
+        self.act = dict(opacities=e(N), scales=e(N, 3), quats=e(N, 4))
+        self.v_act = dict(opacities=e(N), scales=e(N, 3), quats=e(N, 4))
+        self.proj = dict(radii=e(1, N, 2, dt=torch.int32), means2d=e(1, N, 2), depths=e(1, N), conics=e(1, N, 3))
+        self.colors = e(1, N, 3)
+        self.v_colors = e(1, N, 3)
+        self.tiles_per_gauss = e(N, dt=torch.int32)
+        self.cum = e(N, dt=torch.int64)
+        self.ws_count = e(self.lib.gsx_intersect_tile_count_workspace_bytes(c_u32(1), c_u32(N)), dt=torch.uint8)
+        self.ws_bwd = e(self.lib.gsx_rasterize_bwd_workspace_bytes(c_u32(N)), dt=torch.uint8)
+        self.cap = 0
+        self.img_shape = None
+        self.n_isects = 0
+        self.bg = torch.zeros((1, 3), dtype=torch.float32, device=self.dev)  # trainer.cpp:383-384
+        self.loss_out = e(3)
+
+    # -- buffers that depend on n_isects / image size --------------------------------------------
+    def _ensure_isect_capacity(self, n):
+        if n <= self.cap:
+            return
+        cap = max(int(n * 1.25) + 1024, 1 << 16)
+        e = lambda *s, dt: torch.empty(s, dtype=dt, device=self.dev)
+        self.keys = [e(cap, dt=torch.int64), e(cap, dt=torch.int64)]
+        self.vals = [e(cap, dt=torch.int32), e(cap, dt=torch.int32)]
+        self.ws_sort = e(self.lib.gsx_radix_sort_pairs_workspace_bytes(c_i64(cap)), dt=torch.uint8)
+        self.cap = cap
+
+    def _ensure_image(self, H, W):
+        if self.img_shape == (H, W):
+            return
+        e = lambda *s, dt=torch.float32: torch.empty(s, dtype=dt, device=self.dev)
+        self.tw, self.th = (W + 15) // 16, (H + 15) // 16
+        self.offsets = e(1, self.th, self.tw, dt=torch.int32)
+        self.render = e(1, H, W, 3)
+        self.alpha = e(1, H, W, 1)
+        self.last_ids = e(1, H, W, dt=torch.int32)
+        self.image = e(1, 3, H, W)
+        self.v_render = e(1, H, W, 3)
+        self.v_alpha = torch.zeros((1, H, W, 1), dtype=torch.float32, device=self.dev)
+        nb = self.lib.gsx_image_loss_blocks(c_u32(H), c_u32(W))
+        self.n_partials = nb
+        self.l1_partials, self.ssim_partials = e(nb), e(nb)
+        self.ssim_map, self.dm1, self.dm2, self.dm3 = e(1, 3, H, W), e(1, 3, H, W), e(1, 3, H, W), e(1, 3, H, W)
+        self.dL_dmap, self.dL_dimg = e(1, 3, H, W), e(1, 3, H, W)
+        crop = H > 10 and W > 10
+        count = 3 * (H - 10) * (W - 10) if crop else 3 * H * W
+        # d loss / d map = lambda * d(1 - mean(map_valid)) / d map ; constant per resolution
+        check(self.lib.gsx_ssim_valid_grad_map(c_u32(3), c_u32(H), c_u32(W), c_f(-self.lambda_dssim / count),
+                                               _p(self.dL_dmap), self._stream()))
+        self.img_shape = (H, W)
+
+    def _stream(self):
+        return c_p(torch.cuda.current_stream(self.dev).cuda_stream)
+
+    # per-stage HIP-event timing (events are recorded on the stream the kernels are launched on)
+    timing = None  # None, or a dict name -> list of (start_event, stop_event)
+
+    def _run(self, name, fn, *args):
+        if self.timing is None or (self.timed_names is not None and name not in self.timed_names):
+            check(fn(*args))
+            return
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(torch.cuda.current_stream(self.dev))
+        check(fn(*args))
+        e1.record(torch.cuda.current_stream(self.dev))
+        self.timing.setdefault(name, []).append((e0, e1))
+
+    timed_names = None  # None = every stage; or a set of stage names
+
+    def start_timing(self, names=None):
+        self.timing, self.timed_names = {}, (None if names is None else set(names))
+
+    def stop_timing(self):
+        """-> dict name -> list of milliseconds (synchronises)"""
+        torch.cuda.synchronize(self.dev)
+        out = {k: [a.elapsed_time(b) for a, b in v] for k, v in (self.timing or {}).items()}
+        self.timing = None
+        return out
+
+    # -- forward ----------------------------------------------------------------------------------
+    def forward(self, viewmat, K, W, H):
+        """activations + rasterize_from_world_with_sh_fwd; returns the [1,H,W,3] render (not clamped)."""
+        lb, s, N = self.lib, self._stream(), self.N
+        self._ensure_image(H, W)
+        self.viewmat, self.Kmat, self.W, self.H = viewmat, K, W, H
+        P, A, J = self.params, self.act, self.proj
+        self._run("activate_params", lb.gsx_activate_params, c_u32(N), _p(P["opacity"]), _p(P["scaling"]), _p(P["rotation"]),
+                                     _p(A["opacities"]), _p(A["scales"]), _p(A["quats"]), s)
+        self._run("projection_ut_3dgs_fused", lb.gsx_projection_ut_3dgs_fused, 
+            c_u32(1), c_u32(N), _p(P["means"]), _p(A["quats"]), _p(A["scales"]), _p(A["opacities"]), _p(viewmat),
+            c_p(None), _p(K), c_u32(W), c_u32(H), c_f(0.3), c_f(0.01), c_f(1e4), c_f(0.0), c_i(0), self.ut, c_i(4),
+            c_p(None), c_p(None), c_p(None), _p(J["radii"]), _p(J["means2d"]), _p(J["depths"]), _p(J["conics"]),
+            c_p(None), s)
+        self._run("sh_colors_from_world", lb.gsx_sh_colors_from_world, c_u32(N), c_u32(self.K), c_u32(self.sh_degree), _p(P["means"]), _p(P["shs"]),
+                                          _p(J["radii"]), _p(viewmat), _p(self.colors), s)
+        n_isects = c_i64(0)
+        self._run("intersect_tile_count", lb.gsx_intersect_tile_count, c_u32(1), c_u32(N), _p(J["means2d"]), _p(J["radii"]), c_u32(16),
+                                          c_u32(self.tw), c_u32(self.th), _p(self.tiles_per_gauss), _p(self.cum),
+                                          _p(self.ws_count), c_sz(self.ws_count.numel()), ctypes.byref(n_isects), s)
+        n = self.n_isects = n_isects.value
+        self._ensure_isect_capacity(n)
+        sel = c_i(0)
+        if n:
+            self._run("intersect_tile_emit", lb.gsx_intersect_tile_emit, c_u32(1), c_u32(N), _p(J["means2d"]), _p(J["radii"]), _p(J["depths"]),
+                                             _p(self.cum), c_u32(16), c_u32(self.tw), c_u32(self.th),
+                                             _p(self.keys[0]), _p(self.vals[0]), s)
+            end_bit = 32 + lb.gsx_n_bits(c_u32(self.tw * self.th)) + lb.gsx_n_bits(c_u32(1))
+            self._run("radix_sort_pairs", lb.gsx_radix_sort_pairs, c_i64(n), _p(self.keys[0]), _p(self.vals[0]), _p(self.keys[1]),
+                                          _p(self.vals[1]), c_u32(end_bit), _p(self.ws_sort),
+                                          c_sz(self.ws_sort.numel()), ctypes.byref(sel), s)
+        self.sel = sel.value
+        self.isect_ids, self.flatten_ids = self.keys[self.sel], self.vals[self.sel]
+        self._run("intersect_offset", lb.gsx_intersect_offset, c_i64(n), _p(self.isect_ids), c_u32(1), c_u32(self.tw), c_u32(self.th),
+                                      _p(self.offsets), s)
+        self._run("rasterize_to_pixels_from_world_3dgs_fwd", lb.gsx_rasterize_to_pixels_from_world_3dgs_fwd, 
+            c_u32(1), c_u32(N), c_i64(n), _p(P["means"]), _p(A["quats"]), _p(A["scales"]), _p(self.colors), c_u32(3),
+            _p(A["opacities"]), _p(self.bg), c_p(None), c_u32(W), c_u32(H), c_u32(16), _p(viewmat), c_p(None), _p(K),
+            c_i(0), self.ut, c_i(4), c_p(None), c_p(None), c_p(None), _p(self.offsets), _p(self.flatten_ids),
+            _p(self.render), _p(self.alpha), _p(self.last_ids), s)
+        return self.render
+
+    # -- loss ---------------------------------------------------------------------------------------
+    def loss_forward(self, gt_chw):
+        """image = clamp(render, 0, 1) CHW; loss = (1-l) L1 + l (1 - SSIM_valid); result stays on the device."""
+        lb, s, H, W = self.lib, self._stream(), self.H, self.W
+        self.gt = gt_chw
+        self._run("image_from_render", lb.gsx_image_from_render, c_u32(H), c_u32(W), _p(self.render), _p(gt_chw), _p(self.image),
+                                       _p(self.l1_partials), s)
+        if self.use_ssim:
+            self._run("fusedssim", lb.gsx_fusedssim, c_i(1), c_i(3), c_i(H), c_i(W), c_f(0.01 ** 2), c_f(0.03 ** 2), _p(self.image),
+                                   _p(gt_chw), _p(self.ssim_map), _p(self.dm1), _p(self.dm2), _p(self.dm3), s)
+            self._run("ssim_valid_partials", lb.gsx_ssim_valid_partials, c_u32(3), c_u32(H), c_u32(W), _p(self.ssim_map), _p(self.ssim_partials),
+                                             s)
+        else:
+            self.ssim_partials.zero_()
+        self._run("photometric_loss_finish", lb.gsx_photometric_loss_finish, c_u32(3), c_u32(H), c_u32(W), c_f(self.lambda_dssim),
+                                             _p(self.l1_partials), _p(self.ssim_partials), c_u32(self.n_partials),
+                                             _p(self.loss_out), s)
+        return self.loss_out
+
+    # -- backward -----------------------------------------------------------------------------------
+    def backward(self):
+        lb, s, N, H, W = self.lib, self._stream(), self.N, self.H, self.W
+        P, A, J, G, V = self.params, self.act, self.proj, self.grads, self.v_act
+        dimg = None
+        if self.use_ssim:
+            self._run("fusedssim_backward", lb.gsx_fusedssim_backward, c_i(1), c_i(3), c_i(H), c_i(W), c_f(0.01 ** 2), c_f(0.03 ** 2),
+                                            _p(self.image), _p(self.gt), _p(self.dL_dmap), _p(self.dm1), _p(self.dm2),
+                                            _p(self.dm3), _p(self.dL_dimg), s)
+            dimg = self.dL_dimg
+        self._run("render_grad_from_loss", lb.gsx_render_grad_from_loss, c_u32(H), c_u32(W), c_f(self.lambda_dssim), _p(self.render),
+                                           _p(self.image), _p(self.gt), _p(dimg), _p(self.v_render), s)
+        ws, wsn = _p(self.ws_bwd), c_sz(self.ws_bwd.numel())
+        self._run("rasterize_bwd_clear", lb.gsx_rasterize_bwd_clear, c_u32(N), ws, wsn, s)
+        self._run("rasterize_bwd_accumulate", lb.gsx_rasterize_bwd_accumulate,
+                  c_u32(1), c_u32(N), c_i64(self.n_isects), _p(P["means"]), _p(A["quats"]), _p(A["scales"]),
+                  _p(self.colors), _p(A["opacities"]), _p(self.bg), c_p(None), c_u32(W), c_u32(H), c_u32(16),
+                  _p(self.viewmat), _p(self.Kmat), _p(self.offsets), _p(self.flatten_ids), _p(self.alpha),
+                  _p(self.last_ids), _p(self.v_render), _p(self.v_alpha), ws, wsn, s)
+        self._run("rasterize_bwd_finish", lb.gsx_rasterize_bwd_finish, c_u32(N), _p(P["means"]), _p(A["quats"]),
+                  _p(A["scales"]), _p(self.viewmat), ws, wsn, _p(G["means"]), _p(V["quats"]), _p(V["scales"]),
+                  _p(self.v_colors), _p(V["opacities"]), s)
+        self._run("sh_colors_from_world_bwd", lb.gsx_sh_colors_from_world_bwd, c_u32(N), c_u32(self.K), c_u32(self.sh_degree), _p(P["means"]),
+                                              _p(J["radii"]), _p(self.viewmat), _p(self.colors), _p(self.v_colors),
+                                              _p(G["shs"]), s)
+        self._run("activate_params_bwd", lb.gsx_activate_params_bwd, c_u32(N), _p(P["opacity"]), _p(P["scaling"]), _p(P["rotation"]),
+                                         _p(V["opacities"]), _p(V["scales"]), _p(V["quats"]), _p(G["opacity"]),
+                                         _p(G["scaling"]), _p(G["rotation"]), s)
+
+    # -- optimiser ------------------------------------------------------------------------------------
+    def adam(self):
+        """FusedAdam::step (fused_adam.cpp:22-95): all groups share the step count here (all have gradients every
+        iteration); the shN part of the SH tensor is frozen while iteration <= 1000 (:69-70)."""
+        self.step_count += 1
+        t = self.step_count
+        b1, b2 = self.betas
+        bc1 = 1.0 / (1.0 - math.pow(b1, t))
+        bc2 = 1.0 / math.sqrt(1.0 - math.pow(b2, t))
+        names = ["means", "shs", "scaling", "rotation", "opacity"]
+        lr_of = dict(means=self.lrs["means"], shs=self.lrs["sh0"], scaling=self.lrs["scaling"],
+                     rotation=self.lrs["rotation"], opacity=self.lrs["opacity"])
+        arr = (L.AdamGroup * len(names))()
+        for i, k in enumerate(names):
+            p = self.params[k]
+            g = L.AdamGroup(p.data_ptr(), self.exp_avg[k].data_ptr(), self.exp_avg_sq[k].data_ptr(),
+                            self.grads[k].data_ptr(), p.numel(), lr_of[k], b1, b2, self.eps, bc1, bc2)
+            if k == "shs" and self.K > 1:
+                g.period, g.split = self.K * 3, 3
+                g.lr2 = self.lrs["shN"]
+                g.skip2 = 1 if self.iteration <= 1000 and self.freeze_shN_early else 0
+            arr[i] = g
+        self._run("adam_step_multi", self.lib.gsx_adam_step_multi, arr, c_i(len(names)), self._stream())
+
+    freeze_shN_early = False  # BASELINE's step updates all parameter tensors; set True for the product schedule
+
+    def step(self, viewmat, K, W, H, gt_chw):
+        self.iteration += 1
+        self.forward(viewmat, K, W, H)
+        self.loss_forward(gt_chw)
+        self.backward()
+        self.adam()
+        return self.loss_out

@@ -906,6 +906,234 @@ ORC_API int orc_rasterize_to_pixels_from_world_3dgs_bwd(
     return 0;
 }
 
+// ---------------------------------------------------------------------------------------------
+// float64 evaluation of the same backward pass, for judging fp32 results.
+// Which (pixel, Gaussian) pairs take part is decided by the fp32 path above (thresholds on alpha and
+// the last contributing index), the values are then evaluated in double from the same fp32 inputs.
+// grads[N][14]: mean 3, quat 4 (wxyz), scale 3, colour 3, opacity 1.
+// bound[N][14]: the same expressions evaluated with every product replaced by its absolute value and every
+// difference by a sum (a running error-bound scale: an fp32 evaluation of depth d differs from the exact
+// value by at most about d * 2^-24 * bound).
+// =============================================================================================
+namespace {
+struct d3 {
+    double x, y, z;
+};
+inline d3 dcross(d3 a, d3 b) { return {a.y * b.z - a.z * b.y, a.z * b.x - a.x * b.z, a.x * b.y - a.y * b.x}; }
+inline d3 dcross_abs(d3 a, d3 b) {
+    return {std::fabs(a.y * b.z) + std::fabs(a.z * b.y), std::fabs(a.z * b.x) + std::fabs(a.x * b.z),
+            std::fabs(a.x * b.y) + std::fabs(a.y * b.x)};
+}
+inline double ddot(d3 a, d3 b) { return a.x * b.x + a.y * b.y + a.z * b.z; }
+inline double ddot_abs(d3 a, d3 b) { return std::fabs(a.x * b.x) + std::fabs(a.y * b.y) + std::fabs(a.z * b.z); }
+} // namespace
+
+ORC_API int orc_rasterize_bwd_f64(
+    uint32_t N, int64_t n_isects, const float* means, const float* quats, const float* scales, const float* colors,
+    const float* opacities, const float* backgrounds /*nullable*/, uint32_t image_width, uint32_t image_height,
+    uint32_t tile_size, const float* viewmats0, const float* Ks, const int32_t* tile_offsets,
+    const int32_t* flatten_ids, const float* render_alphas, const int32_t* last_ids, const float* v_render_colors,
+    const float* v_render_alphas, double* grads, double* bound) {
+    const uint32_t tile_width = (image_width + tile_size - 1) / tile_size;
+    const uint32_t tile_height = (image_height + tile_size - 1) / tile_size;
+    const uint32_t n_tiles = tile_width * tile_height;
+    const float fx = Ks[0], fy = Ks[4], cx = Ks[2], cy = Ks[5];
+    const RollingShutter rs = make_rolling_shutter(viewmats0, nullptr);
+    std::fill(grads, grads + (size_t)N * 14, 0.0);
+    std::fill(bound, bound + (size_t)N * 14, 0.0);
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int64_t tile_id = 0; tile_id < (int64_t)n_tiles; ++tile_id) {
+        const uint32_t ty = tile_id / tile_width, tx = tile_id % tile_width;
+        const int32_t range_start = tile_offsets[tile_id];
+        const int32_t range_end = (tile_id == (int64_t)n_tiles - 1) ? (int32_t)n_isects : tile_offsets[tile_id + 1];
+        const int32_t cnt = range_end - range_start;
+        if (cnt <= 0)
+            continue;
+        std::vector<double> local((size_t)cnt * 14, 0.0), lbound((size_t)cnt * 14, 0.0);
+        for (uint32_t ly = 0; ly < tile_size; ++ly)
+            for (uint32_t lx = 0; lx < tile_size; ++lx) {
+                const uint32_t i = ty * tile_size + ly, j = tx * tile_size + lx;
+                if (!(i < image_height && j < image_width))
+                    continue;
+                const int64_t pix_id = (int64_t)i * image_width + j;
+                vec3 ray_of, ray_df;
+                pixel_world_ray((float)j + 0.5f, (float)i + 0.5f, fx, fy, cx, cy, rs, &ray_of, &ray_df);
+                const d3 ray_o = {ray_of.x, ray_of.y, ray_of.z}, ray_d = {ray_df.x, ray_df.y, ray_df.z};
+                const double T_final = 1.0 - (double)render_alphas[pix_id];
+                double T = T_final;
+                double buffer[3] = {0, 0, 0}, buffer_abs[3] = {0, 0, 0};
+                const int32_t bin_final = last_ids[pix_id];
+                const double vrc[3] = {v_render_colors[pix_id * 3], v_render_colors[pix_id * 3 + 1],
+                                       v_render_colors[pix_id * 3 + 2]};
+                const double vra = v_render_alphas[pix_id];
+                for (int32_t idx = std::min(range_end - 1, bin_final); idx >= range_start; --idx) {
+                    const int32_t g = flatten_ids[idx];
+                    // fp32 decision and fp32 alpha (identical to orc_rasterize_to_pixels_from_world_3dgs_bwd): the
+                    // transmittance is recovered by dividing by (1 - alpha) with the alpha the forward pass used
+                    float alphaf;
+                    {
+                        const mat3 Mf = iscl_rot(ld4(quats, g), ld3(scales, g));
+                        const vec3 grof = gsx::mul(Mf, gsx::sub(ray_of, ld3(means, g)));
+                        const vec3 grdf = gsx::safe_normalize(gsx::mul(Mf, ray_df));
+                        const vec3 cf = gsx::cross(grdf, grof);
+                        const float powerf = -0.5f * gsx::dot(cf, cf);
+                        alphaf = gsx::fmin(0.999f, opacities[g] * gsx::exp(powerf));
+                        if (powerf > 0.f || alphaf < 1.f / 255.f)
+                            continue;
+                    }
+                    // values in double
+                    const double qw = quats[g * 4], qx = quats[g * 4 + 1], qy = quats[g * 4 + 2], qz = quats[g * 4 + 3];
+                    const double inv_norm = 1.0 / std::sqrt(qw * qw + qx * qx + qy * qy + qz * qz);
+                    const double w = qw * inv_norm, x = qx * inv_norm, y = qy * inv_norm, z = qz * inv_norm;
+                    double R[3][3];
+                    R[0][0] = 1 - 2 * (y * y + z * z), R[0][1] = 2 * (x * y - w * z), R[0][2] = 2 * (x * z + w * y);
+                    R[1][0] = 2 * (x * y + w * z), R[1][1] = 1 - 2 * (x * x + z * z), R[1][2] = 2 * (y * z - w * x);
+                    R[2][0] = 2 * (x * z - w * y), R[2][1] = 2 * (y * z + w * x), R[2][2] = 1 - 2 * (x * x + y * y);
+                    const double is[3] = {1.0 / scales[g * 3], 1.0 / scales[g * 3 + 1], 1.0 / scales[g * 3 + 2]};
+                    double Mt[3][3];
+                    for (int a = 0; a < 3; ++a)
+                        for (int b = 0; b < 3; ++b)
+                            Mt[a][b] = R[b][a] * is[a];
+                    const double om[3] = {ray_o.x - means[g * 3], ray_o.y - means[g * 3 + 1], ray_o.z - means[g * 3 + 2]};
+                    const double rd[3] = {ray_d.x, ray_d.y, ray_d.z};
+                    double gro_[3], grd_[3];
+                    for (int a = 0; a < 3; ++a) {
+                        gro_[a] = Mt[a][0] * om[0] + Mt[a][1] * om[1] + Mt[a][2] * om[2];
+                        grd_[a] = Mt[a][0] * rd[0] + Mt[a][1] * rd[1] + Mt[a][2] * rd[2];
+                    }
+                    const d3 gro = {gro_[0], gro_[1], gro_[2]}, grd = {grd_[0], grd_[1], grd_[2]};
+                    const double l = ddot(grd, grd);
+                    const double il = 1.0 / std::sqrt(l);
+                    const d3 grd_n = {grd.x * il, grd.y * il, grd.z * il};
+                    const d3 gcrod = dcross(grd_n, gro);
+                    const double power = -0.5 * ddot(gcrod, gcrod);
+                    const double vis = std::exp(power);
+                    const double opac = opacities[g];
+                    const double alpha = (double)alphaf;
+                    const double ra = 1.0 / (double)(1.0f - alphaf);
+                    T *= ra;
+                    const double fac = alpha * T;
+                    const double rgb[3] = {colors[(int64_t)g * 3], colors[(int64_t)g * 3 + 1], colors[(int64_t)g * 3 + 2]};
+                    double v_alpha = 0, v_alpha_abs = 0;
+                    for (int k = 0; k < 3; ++k) {
+                        v_alpha += (rgb[k] * T - buffer[k] * ra) * vrc[k];
+                        v_alpha_abs += (std::fabs(rgb[k] * T) + buffer_abs[k] * ra) * std::fabs(vrc[k]);
+                    }
+                    v_alpha += T_final * ra * vra;
+                    v_alpha_abs += std::fabs(T_final * ra * vra);
+                    if (backgrounds != nullptr) {
+                        double accum = 0, accum_abs = 0;
+                        for (int k = 0; k < 3; ++k) {
+                            accum += backgrounds[k] * vrc[k];
+                            accum_abs += std::fabs(backgrounds[k] * vrc[k]);
+                        }
+                        v_alpha += -T_final * ra * accum;
+                        v_alpha_abs += std::fabs(T_final * ra) * accum_abs;
+                    }
+                    double* a = local.data() + (size_t)(idx - range_start) * 14;
+                    double* ab = lbound.data() + (size_t)(idx - range_start) * 14;
+                    for (int k = 0; k < 3; ++k) {
+                        a[10 + k] += fac * vrc[k];
+                        ab[10 + k] += std::fabs(fac * vrc[k]);
+                    }
+                    if (opac * vis <= 0.999) {
+                        const double v_vis = opac * v_alpha, v_vis_abs = opac * v_alpha_abs;
+                        const double v_gd = -0.5 * vis * v_vis, v_gd_abs = 0.5 * vis * v_vis_abs;
+                        const d3 v_gcrod = {2 * v_gd * gcrod.x, 2 * v_gd * gcrod.y, 2 * v_gd * gcrod.z};
+                        const d3 gcrod_abs = dcross_abs(grd_n, gro);
+                        const d3 v_gcrod_abs = {2 * v_gd_abs * gcrod_abs.x, 2 * v_gd_abs * gcrod_abs.y,
+                                                2 * v_gd_abs * gcrod_abs.z};
+                        d3 v_grd_n = dcross(v_gcrod, gro);
+                        v_grd_n = {-v_grd_n.x, -v_grd_n.y, -v_grd_n.z};
+                        const d3 v_grd_n_abs = dcross_abs(v_gcrod_abs, gro);
+                        const d3 v_gro = dcross(v_gcrod, grd_n);
+                        const d3 v_gro_abs = dcross_abs(v_gcrod_abs, grd_n);
+                        const double il3 = il * il * il;
+                        const double dd = ddot(v_grd_n, grd), dd_abs = ddot_abs(v_grd_n_abs, grd);
+                        const d3 v_grd = {il * v_grd_n.x - il3 * dd * grd.x, il * v_grd_n.y - il3 * dd * grd.y,
+                                          il * v_grd_n.z - il3 * dd * grd.z};
+                        const d3 v_grd_abs = {il * v_grd_n_abs.x + il3 * dd_abs * std::fabs(grd.x),
+                                              il * v_grd_n_abs.y + il3 * dd_abs * std::fabs(grd.y),
+                                              il * v_grd_n_abs.z + il3 * dd_abs * std::fabs(grd.z)};
+                        const double vg[3] = {v_grd.x, v_grd.y, v_grd.z}, vo[3] = {v_gro.x, v_gro.y, v_gro.z};
+                        const double vga[3] = {v_grd_abs.x, v_grd_abs.y, v_grd_abs.z};
+                        const double voa[3] = {v_gro_abs.x, v_gro_abs.y, v_gro_abs.z};
+                        double v_Mt[3][3], v_Mt_abs[3][3];
+                        for (int p = 0; p < 3; ++p)
+                            for (int q = 0; q < 3; ++q) {
+                                v_Mt[p][q] = vg[p] * rd[q] + vo[p] * om[q];
+                                v_Mt_abs[p][q] = vga[p] * std::fabs(rd[q]) + voa[p] * std::fabs(om[q]);
+                            }
+                        for (int q = 0; q < 3; ++q) { // v_mean = -Mt^T v_gro
+                            a[q] += -(Mt[0][q] * vo[0] + Mt[1][q] * vo[1] + Mt[2][q] * vo[2]);
+                            ab[q] += std::fabs(Mt[0][q]) * voa[0] + std::fabs(Mt[1][q]) * voa[1] +
+                                     std::fabs(Mt[2][q]) * voa[2];
+                        }
+                        double vr[3][3], vra_[3][3];
+                        for (int k = 0; k < 3; ++k)
+                            for (int jj = 0; jj < 3; ++jj) {
+                                vr[k][jj] = v_Mt[jj][k] * is[jj];
+                                vra_[k][jj] = v_Mt_abs[jj][k] * is[jj];
+                            }
+                        const double vq_w =
+                            2 * (x * (vr[2][1] - vr[1][2]) + y * (vr[0][2] - vr[2][0]) + z * (vr[1][0] - vr[0][1]));
+                        const double vq_x = 2 * (-2 * x * (vr[1][1] + vr[2][2]) + y * (vr[1][0] + vr[0][1]) +
+                                                 z * (vr[2][0] + vr[0][2]) + w * (vr[2][1] - vr[1][2]));
+                        const double vq_y = 2 * (x * (vr[1][0] + vr[0][1]) - 2 * y * (vr[0][0] + vr[2][2]) +
+                                                 z * (vr[2][1] + vr[1][2]) + w * (vr[0][2] - vr[2][0]));
+                        const double vq_z = 2 * (x * (vr[2][0] + vr[0][2]) + y * (vr[2][1] + vr[1][2]) -
+                                                 2 * z * (vr[0][0] + vr[1][1]) + w * (vr[1][0] - vr[0][1]));
+                        const double ax = std::fabs(x), ay = std::fabs(y), az = std::fabs(z), aw = std::fabs(w);
+                        const double vqa_w = 2 * (ax * (vra_[2][1] + vra_[1][2]) + ay * (vra_[0][2] + vra_[2][0]) +
+                                                  az * (vra_[1][0] + vra_[0][1]));
+                        const double vqa_x = 2 * (2 * ax * (vra_[1][1] + vra_[2][2]) + ay * (vra_[1][0] + vra_[0][1]) +
+                                                  az * (vra_[2][0] + vra_[0][2]) + aw * (vra_[2][1] + vra_[1][2]));
+                        const double vqa_y = 2 * (ax * (vra_[1][0] + vra_[0][1]) + 2 * ay * (vra_[0][0] + vra_[2][2]) +
+                                                  az * (vra_[2][1] + vra_[1][2]) + aw * (vra_[0][2] + vra_[2][0]));
+                        const double vqa_z = 2 * (ax * (vra_[2][0] + vra_[0][2]) + ay * (vra_[2][1] + vra_[1][2]) +
+                                                  2 * az * (vra_[0][0] + vra_[1][1]) + aw * (vra_[1][0] + vra_[0][1]));
+                        const double dq = vq_w * w + vq_x * x + vq_y * y + vq_z * z;
+                        const double dqa = vqa_w * aw + vqa_x * ax + vqa_y * ay + vqa_z * az;
+                        a[3] += (vq_w - dq * w) * inv_norm;
+                        a[4] += (vq_x - dq * x) * inv_norm;
+                        a[5] += (vq_y - dq * y) * inv_norm;
+                        a[6] += (vq_z - dq * z) * inv_norm;
+                        ab[3] += (vqa_w + dqa * aw) * inv_norm;
+                        ab[4] += (vqa_x + dqa * ax) * inv_norm;
+                        ab[5] += (vqa_y + dqa * ay) * inv_norm;
+                        ab[6] += (vqa_z + dqa * az) * inv_norm;
+                        for (int jj = 0; jj < 3; ++jj) {
+                            a[7 + jj] += -is[jj] * is[jj] *
+                                         (R[0][jj] * v_Mt[jj][0] + R[1][jj] * v_Mt[jj][1] + R[2][jj] * v_Mt[jj][2]);
+                            ab[7 + jj] += is[jj] * is[jj] *
+                                          (std::fabs(R[0][jj]) * v_Mt_abs[jj][0] + std::fabs(R[1][jj]) * v_Mt_abs[jj][1] +
+                                           std::fabs(R[2][jj]) * v_Mt_abs[jj][2]);
+                        }
+                        a[13] += vis * v_alpha;
+                        ab[13] += vis * v_alpha_abs;
+                    }
+                    for (int k = 0; k < 3; ++k) {
+                        buffer[k] += rgb[k] * fac;
+                        buffer_abs[k] += std::fabs(rgb[k] * fac);
+                    }
+                }
+            }
+        for (int32_t t = 0; t < cnt; ++t) {
+            const int32_t g = flatten_ids[range_start + t];
+            for (int k = 0; k < 14; ++k) {
+                const double v = local[(size_t)t * 14 + k], vb = lbound[(size_t)t * 14 + k];
+                if (vb != 0.0) {
+#pragma omp atomic
+                    grads[(size_t)g * 14 + k] += v;
+#pragma omp atomic
+                    bound[(size_t)g * 14 + k] += vb;
+                }
+            }
+        }
+    }
+    return 0;
+}
+
 // =============================================================================================
 // k9/k10  fused SSIM  src/training/kernels/ssim.cu:16-27 (window), :64-276 (fwd), :284-424 (bwd)
 // Images are [B, CH, H, W].  dm_* may be null (train == false).
@@ -1197,6 +1425,125 @@ ORC_API int orc_sh_colors_from_world_bwd(uint32_t N, uint32_t K, uint32_t degree
                 out[k * 3 + c] = B[k] * v;
         }
     }
+    return 0;
+}
+
+// =============================================================================================
+// a15  step-driver semantics around the boundary
+// activations: SplatData getters, src/core/splat_data.cpp:271-286 (torch sigmoid / exp / normalize with eps 1e-12)
+// and their VJPs (what LibTorch autograd applies to the gradients Ops.h's backward returns).
+// =============================================================================================
+ORC_API int orc_activate_params(uint32_t N, const float* opacity_raw, const float* scaling_raw,
+                                const float* rotation_raw, float* opacities, float* scales, float* quats) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < (int64_t)N; ++i) {
+        opacities[i] = gsx::sigmoid(opacity_raw[i]);
+        for (int k = 0; k < 3; ++k)
+            scales[3 * i + k] = gsx::exp(scaling_raw[3 * i + k]);
+        const quat q = ld4(rotation_raw, i);
+        const float nrm = gsx::fmax(gsx::sqrt(gsx::qdot(q, q)), 1e-12f);
+        quats[4 * i + 0] = q.w / nrm;
+        quats[4 * i + 1] = q.x / nrm;
+        quats[4 * i + 2] = q.y / nrm;
+        quats[4 * i + 3] = q.z / nrm;
+    }
+    return 0;
+}
+
+ORC_API int orc_activate_params_bwd(uint32_t N, const float* opacity_raw, const float* scaling_raw,
+                                    const float* rotation_raw, const float* v_opacities, const float* v_scales,
+                                    const float* v_quats, float* v_opacity_raw, float* v_scaling_raw,
+                                    float* v_rotation_raw) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < (int64_t)N; ++i) {
+        const float o = gsx::sigmoid(opacity_raw[i]);
+        v_opacity_raw[i] = v_opacities[i] * (o * (1.0f - o));
+        for (int k = 0; k < 3; ++k)
+            v_scaling_raw[3 * i + k] = v_scales[3 * i + k] * gsx::exp(scaling_raw[3 * i + k]);
+        const quat q = ld4(rotation_raw, i);
+        const quat g = ld4(v_quats, i);
+        const float len = gsx::sqrt(gsx::qdot(q, q));
+        if (len > 1e-12f) {
+            const float inv = 1.0f / len;
+            const float yw = q.w * inv, yx = q.x * inv, yy = q.y * inv, yz = q.z * inv;
+            const float d = g.w * yw + g.x * yx + g.y * yy + g.z * yz;
+            v_rotation_raw[4 * i + 0] = (g.w - yw * d) * inv;
+            v_rotation_raw[4 * i + 1] = (g.x - yx * d) * inv;
+            v_rotation_raw[4 * i + 2] = (g.y - yy * d) * inv;
+            v_rotation_raw[4 * i + 3] = (g.z - yz * d) * inv;
+        } else {
+            v_rotation_raw[4 * i + 0] = g.w * 1e12f;
+            v_rotation_raw[4 * i + 1] = g.x * 1e12f;
+            v_rotation_raw[4 * i + 2] = g.y * 1e12f;
+            v_rotation_raw[4 * i + 3] = g.z * 1e12f;
+        }
+    }
+    return 0;
+}
+
+// photometric loss of trainer.cpp:126-129 around the rasterizer output:
+// image = clamp(render[0] HWC -> CHW, 0, 1) (rasterizer.cpp:205); loss = (1-l) mean|image - gt| + l (1 - mean(ssim_valid))
+// with the "valid" crop of fused_ssim.cuh:59-67.  Sums are formed in double.  Returns loss, l1, ssim in out[0..2],
+// the clamped image, and (when v_render != nullptr) d loss / d render [H,W,3] including the SSIM backward
+// (fused_ssim.cuh:74-102) and the clamp VJP.
+ORC_API int orc_photometric_loss(uint32_t H, uint32_t W, float lambda_dssim, const float* render_hwc,
+                                 const float* gt_chw, float* image_chw, double* out, float* v_render_hwc) {
+    const int64_t HW = (int64_t)H * W;
+    double l1 = 0.0;
+#pragma omp parallel for schedule(static) reduction(+ : l1)
+    for (int64_t p = 0; p < HW; ++p)
+        for (int c = 0; c < 3; ++c) {
+            const float r = render_hwc[p * 3 + c];
+            const float v = gsx::fmin(gsx::fmax(r, 0.0f), 1.0f);
+            image_chw[c * HW + p] = v;
+            l1 += (double)gsx::fabs(v - gt_chw[c * HW + p]);
+        }
+    l1 /= (double)(3 * HW);
+    double ss = 0.0;
+    std::vector<float> map, d1, d2, d3;
+    const bool crop = H > 10 && W > 10;
+    const double count = crop ? 3.0 * (H - 10) * (W - 10) : 3.0 * H * W;
+    if (lambda_dssim != 0.f) {
+        map.resize(3 * HW), d1.resize(3 * HW), d2.resize(3 * HW), d3.resize(3 * HW);
+        orc_fusedssim(1, 3, (int)H, (int)W, 0.01f * 0.01f, 0.03f * 0.03f, image_chw, gt_chw, map.data(), d1.data(),
+                      d2.data(), d3.data());
+        for (int c = 0; c < 3; ++c)
+            for (uint32_t y = 0; y < H; ++y)
+                for (uint32_t x = 0; x < W; ++x)
+                    if (!crop || (y >= 5 && y < H - 5 && x >= 5 && x < W - 5))
+                        ss += map[c * HW + (int64_t)y * W + x];
+        ss /= count;
+    }
+    out[0] = (1.0 - lambda_dssim) * l1 + lambda_dssim * (1.0 - ss);
+    out[1] = l1;
+    out[2] = ss;
+    if (v_render_hwc == nullptr)
+        return 0;
+    std::vector<float> dimg;
+    if (lambda_dssim != 0.f) {
+        std::vector<float> dmap(3 * HW, 0.f);
+        const float sc = -lambda_dssim / (float)count;
+        for (int c = 0; c < 3; ++c)
+            for (uint32_t y = 0; y < H; ++y)
+                for (uint32_t x = 0; x < W; ++x)
+                    if (!crop || (y >= 5 && y < H - 5 && x >= 5 && x < W - 5))
+                        dmap[c * HW + (int64_t)y * W + x] = sc;
+        dimg.resize(3 * HW);
+        orc_fusedssim_backward(1, 3, (int)H, (int)W, 0.01f * 0.01f, 0.03f * 0.03f, image_chw, gt_chw, dmap.data(),
+                               d1.data(), d2.data(), d3.data(), dimg.data());
+    }
+    const float l1_scale = (1.f - lambda_dssim) / (3.f * (float)H * (float)W);
+#pragma omp parallel for schedule(static)
+    for (int64_t p = 0; p < HW; ++p)
+        for (int c = 0; c < 3; ++c) {
+            const float r = render_hwc[p * 3 + c];
+            const float d = image_chw[c * HW + p] - gt_chw[c * HW + p];
+            const float sgn = d > 0.f ? 1.f : (d < 0.f ? -1.f : 0.f);
+            float g = l1_scale * sgn;
+            if (!dimg.empty())
+                g += dimg[c * HW + p];
+            v_render_hwc[p * 3 + c] = (r >= 0.f && r <= 1.f) ? g : 0.f;
+        }
     return 0;
 }
 

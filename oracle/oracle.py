@@ -207,6 +207,30 @@ def rasterize_to_pixels_from_world_3dgs_bwd(means, quats, scales, colors, opacit
     return v_means, v_quats, v_scales, v_colors, v_opac
 
 
+def rasterize_bwd_f64(means, quats, scales, colors, opacities, backgrounds, image_width, image_height, tile_size,
+                      viewmats0, Ks, tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors,
+                      v_render_alphas):
+    """float64 evaluation of the rasterizer backward (same pair selection as the fp32 pass) and a running
+    error-bound scale.  -> (grads [N,14], bound [N,14]) float64; columns: mean 3, quat 4, scale 3, colour 3,
+    opacity 1."""
+    means, quats, scales = _f32(means), _f32(quats), _f32(scales)
+    colors, opacities = _f32(colors), _f32(opacities)
+    backgrounds, viewmats0, Ks = _f32(backgrounds), _f32(viewmats0), _f32(Ks)
+    render_alphas, v_render_colors, v_render_alphas = _f32(render_alphas), _f32(v_render_colors), _f32(v_render_alphas)
+    tile_offsets = np.ascontiguousarray(tile_offsets, dtype=np.int32)
+    flatten_ids = np.ascontiguousarray(flatten_ids, dtype=np.int32)
+    last_ids = np.ascontiguousarray(last_ids, dtype=np.int32)
+    N = means.shape[0]
+    grads = np.zeros((N, 14), np.float64)
+    bound = np.zeros((N, 14), np.float64)
+    _chk(lib().orc_rasterize_bwd_f64(
+        c_u32(N), c_i64(flatten_ids.shape[0]), _p(means), _p(quats), _p(scales), _p(colors), _p(opacities),
+        _p(backgrounds), c_u32(image_width), c_u32(image_height), c_u32(tile_size), _p(viewmats0), _p(Ks),
+        _p(tile_offsets), _p(flatten_ids), _p(render_alphas), _p(last_ids), _p(v_render_colors), _p(v_render_alphas),
+        _p(grads), _p(bound)), "rasterize_bwd_f64")
+    return grads, bound
+
+
 def fusedssim(C1, C2, img1, img2, train=True):
     """include/kernels/ssim.cuh:11-19.  img [B,CH,H,W] -> (map, dm_dmu1, dm_dsigma1_sq, dm_dsigma12)."""
     img1, img2 = _f32(img1), _f32(img2)
@@ -331,6 +355,37 @@ def rasterize_from_world_with_sh_bwd(means, quats, scales, opacities, sh_coeffs,
     if scaling_modifier != 1.0:
         v_scales = v_scales * np.float32(scaling_modifier)
     return v_means, v_quats, v_scales, v_opac, v_sh
+
+
+def activate_params(opacity_raw, scaling_raw, rotation_raw):
+    """src/core/splat_data.cpp:271-286 -> (opacities [N], scales [N,3], quats [N,4])"""
+    o, sc, r = _f32(opacity_raw).reshape(-1), _f32(scaling_raw), _f32(rotation_raw)
+    N = o.shape[0]
+    op, scales, quats = np.zeros(N, np.float32), np.zeros((N, 3), np.float32), np.zeros((N, 4), np.float32)
+    _chk(lib().orc_activate_params(c_u32(N), _p(o), _p(sc), _p(r), _p(op), _p(scales), _p(quats)), "activate_params")
+    return op, scales, quats
+
+
+def activate_params_bwd(opacity_raw, scaling_raw, rotation_raw, v_opacities, v_scales, v_quats):
+    o, sc, r = _f32(opacity_raw).reshape(-1), _f32(scaling_raw), _f32(rotation_raw)
+    N = o.shape[0]
+    vo, vs, vr = np.zeros(N, np.float32), np.zeros((N, 3), np.float32), np.zeros((N, 4), np.float32)
+    _chk(lib().orc_activate_params_bwd(c_u32(N), _p(o), _p(sc), _p(r), _p(_f32(v_opacities).reshape(-1)),
+                                       _p(_f32(v_scales)), _p(_f32(v_quats)), _p(vo), _p(vs), _p(vr)),
+         "activate_params_bwd")
+    return vo, vs, vr
+
+
+def photometric_loss(render_hwc, gt_chw, lambda_dssim, with_grad=True):
+    """trainer.cpp:126-129 on clamp(render) -> (loss, l1, ssim, image [3,H,W], v_render [H,W,3] or None)"""
+    render_hwc, gt_chw = _f32(render_hwc), _f32(gt_chw)
+    H, W = render_hwc.shape[0], render_hwc.shape[1]
+    image = np.zeros((3, H, W), np.float32)
+    out = np.zeros(3, np.float64)
+    v = np.zeros((H, W, 3), np.float32) if with_grad else None
+    _chk(lib().orc_photometric_loss(c_u32(H), c_u32(W), c_f(lambda_dssim), _p(render_hwc), _p(gt_chw), _p(image),
+                                    _p(out), _p(v)), "photometric_loss")
+    return float(out[0]), float(out[1]), float(out[2]), image, v
 
 
 def math_unary(which, x):

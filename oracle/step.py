@@ -1,0 +1,80 @@
+"""CPU restatement of one training iteration (Trainer::train_step, src/training/trainer.cpp:599-875, `--gut` path
+with the MCMC strategy's optimiser, mcmc.cpp:479-497), built from the checker's kernels.
+
+TEST INFRASTRUCTURE ONLY (tests/, __graft_entry__.smoke(), bench.py's cpu_baseline leg).
+"""
+import math
+
+import numpy as np
+
+from . import oracle as orc
+
+DEFAULT_LRS = dict(means=1.6e-4, sh0=2.5e-3, shN=2.5e-3 / 20.0, scaling=5e-3, rotation=1e-3, opacity=5e-2)
+
+
+class OracleTrainStep:
+    def __init__(self, scene, lrs=None, lambda_dssim=0.2, betas=(0.9, 0.999), eps=1e-15, sh_degree=None):
+        c = lambda a: np.ascontiguousarray(a, dtype=np.float32).copy()
+        self.params = dict(means=c(scene.means), shs=c(np.concatenate([scene.sh0, scene.shN], 1)),
+                           scaling=c(scene.scaling_raw), rotation=c(scene.rotation_raw),
+                           opacity=c(scene.opacity_raw.reshape(-1)))
+        self.exp_avg = {k: np.zeros_like(v) for k, v in self.params.items()}
+        self.exp_avg_sq = {k: np.zeros_like(v) for k, v in self.params.items()}
+        self.K = self.params["shs"].shape[1]
+        self.sh_degree = scene.sh_degree if sh_degree is None else sh_degree
+        self.lrs = dict(DEFAULT_LRS, **(lrs or {}))
+        self.lambda_dssim, self.betas, self.eps = lambda_dssim, betas, eps
+        self.step_count = 0
+        self.bg = np.zeros((1, 3), np.float32)
+
+    def forward(self, viewmat, K, W, H):
+        P = self.params
+        self.cam = (viewmat, K, W, H)
+        self.act = orc.activate_params(P["opacity"], P["scaling"], P["rotation"])
+        op, scales, quats = self.act
+        self.fwd = orc.rasterize_from_world_with_sh_fwd(P["means"], quats, scales, op, P["shs"], self.sh_degree,
+                                                        self.bg, W, H, 16, viewmat[None], K[None])
+        return self.fwd[0]
+
+    def loss_and_backward(self, gt_chw):
+        P = self.params
+        viewmat, K, W, H = self.cam
+        op, scales, quats = self.act
+        renders, alphas, radii, means2d, depths, colors, offsets, flat, last_ids, comp, ids = self.fwd
+        loss, l1, ss, image, v_render = orc.photometric_loss(renders[0], gt_chw, self.lambda_dssim, True)
+        self.loss, self.image, self.v_render = (loss, l1, ss), image, v_render
+        v_alpha = np.zeros_like(alphas)
+        v_means, v_quats, v_scales, v_op, v_sh = orc.rasterize_from_world_with_sh_bwd(
+            P["means"], quats, scales, op, P["shs"], self.sh_degree, self.bg, W, H, 16, viewmat[None], K[None], 1.0,
+            False, alphas, last_ids, offsets, flat, colors, radii, comp, v_render[None], v_alpha)
+        g_op, g_sc, g_rot = orc.activate_params_bwd(P["opacity"], P["scaling"], P["rotation"], v_op, v_scales,
+                                                    v_quats)
+        self.grads = dict(means=v_means, shs=v_sh, scaling=g_sc, rotation=g_rot, opacity=g_op)
+        return loss
+
+    def adam(self):
+        self.step_count += 1
+        t = self.step_count
+        b1, b2 = self.betas
+        bc1 = 1.0 / (1.0 - math.pow(b1, t))
+        bc2 = 1.0 / math.sqrt(1.0 - math.pow(b2, t))
+        for k in ("means", "scaling", "rotation", "opacity"):
+            lr = self.lrs[{"means": "means", "scaling": "scaling", "rotation": "rotation", "opacity": "opacity"}[k]]
+            orc.adam_step(self.params[k], self.exp_avg[k], self.exp_avg_sq[k], self.grads[k], lr, b1, b2, self.eps,
+                          bc1, bc2)
+        # sh0 and shN are separate parameter groups in the reference (mcmc.cpp:488-489): same arithmetic, two lrs
+        for sl, lr in ((slice(0, 1), self.lrs["sh0"]), (slice(1, self.K), self.lrs["shN"])):
+            if sl.stop <= sl.start:
+                continue
+            p = np.ascontiguousarray(self.params["shs"][:, sl])
+            m = np.ascontiguousarray(self.exp_avg["shs"][:, sl])
+            v = np.ascontiguousarray(self.exp_avg_sq["shs"][:, sl])
+            g = np.ascontiguousarray(self.grads["shs"][:, sl])
+            orc.adam_step(p, m, v, g, lr, b1, b2, self.eps, bc1, bc2)
+            self.params["shs"][:, sl], self.exp_avg["shs"][:, sl], self.exp_avg_sq["shs"][:, sl] = p, m, v
+
+    def step(self, viewmat, K, W, H, gt_chw):
+        self.forward(viewmat, K, W, H)
+        loss = self.loss_and_backward(gt_chw)
+        self.adam()
+        return loss
