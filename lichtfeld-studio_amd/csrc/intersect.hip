@@ -204,7 +204,9 @@ extern "C" int gsx_intersect_tile_count(uint32_t C, uint32_t N, const float* mea
     GSX_REQUIRE(n64 < (1ull << 31), GSX_ERR_INVALID_ARGUMENT, "intersect_tile_count: C*N >= 2^31");
     GSX_REQUIRE(tile_size > 0 && tile_width > 0 && tile_height > 0, GSX_ERR_INVALID_ARGUMENT,
                 "intersect_tile_count: empty tile grid");
-    GSX_REQUIRE(gsx_n_bits(tile_width * tile_height) + gsx_n_bits(C) <= 32, GSX_ERR_INVALID_ARGUMENT,
+    GSX_REQUIRE((uint64_t)tile_width * tile_height < (1ull << 32) &&
+                    gsx_n_bits(tile_width * tile_height) + gsx_n_bits(C) <= 32,
+                GSX_ERR_INVALID_ARGUMENT,
                 "intersect_tile_count: tile and camera ids need more than 32 bits"); // Intersect.cpp:50
     GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 &&
                     workspace_bytes >= gsx_intersect_tile_count_workspace_bytes(C, N),

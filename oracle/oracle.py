@@ -247,11 +247,11 @@ def fusedssim(C1, C2, img1, img2, train=True):
 def fusedssim_backward(C1, C2, img1, img2, dL_dmap, dm_dmu1, dm_dsigma1_sq, dm_dsigma12):
     """include/kernels/ssim.cuh:21-28 -> dL/dimg1."""
     img1, img2, dL_dmap = _f32(img1), _f32(img2), _f32(dL_dmap)
+    d1, d2, d3 = _f32(dm_dmu1), _f32(dm_dsigma1_sq), _f32(dm_dsigma12)  # keep the converted arrays alive
     B, CH, H, W = img1.shape
     out = np.zeros_like(img1)
     _chk(lib().orc_fusedssim_backward(c_i(B), c_i(CH), c_i(H), c_i(W), c_f(C1), c_f(C2), _p(img1), _p(img2),
-                                      _p(dL_dmap), _p(_f32(dm_dmu1)), _p(_f32(dm_dsigma1_sq)), _p(_f32(dm_dsigma12)),
-                                      _p(out)), "fusedssim_backward")
+                                      _p(dL_dmap), _p(d1), _p(d2), _p(d3), _p(out)), "fusedssim_backward")
     return out
 
 
@@ -281,8 +281,9 @@ def relocation(opacities, scales, ratios, binoms, n_max):
 def add_noise(raw_opacities, raw_scales, raw_quats, noise, means, current_lr):
     """gsplat/Ops.h:59-65; means is updated in place."""
     assert means.dtype == np.float32 and means.flags["C_CONTIGUOUS"]
-    _chk(lib().orc_add_noise(c_i(means.shape[0]), _p(_f32(raw_opacities)), _p(_f32(raw_scales)), _p(_f32(raw_quats)),
-                             _p(_f32(noise)), _p(means), c_f(current_lr)), "add_noise")
+    ro, rs, rq, nz = _f32(raw_opacities), _f32(raw_scales), _f32(raw_quats), _f32(noise)
+    _chk(lib().orc_add_noise(c_i(means.shape[0]), _p(ro), _p(rs), _p(rq), _p(nz), _p(means), c_f(current_lr)),
+         "add_noise")
 
 
 def quats_to_rotmats(quats):
@@ -370,8 +371,9 @@ def activate_params_bwd(opacity_raw, scaling_raw, rotation_raw, v_opacities, v_s
     o, sc, r = _f32(opacity_raw).reshape(-1), _f32(scaling_raw), _f32(rotation_raw)
     N = o.shape[0]
     vo, vs, vr = np.zeros(N, np.float32), np.zeros((N, 3), np.float32), np.zeros((N, 4), np.float32)
-    _chk(lib().orc_activate_params_bwd(c_u32(N), _p(o), _p(sc), _p(r), _p(_f32(v_opacities).reshape(-1)),
-                                       _p(_f32(v_scales)), _p(_f32(v_quats)), _p(vo), _p(vs), _p(vr)),
+    g_o, g_s, g_q = _f32(v_opacities).reshape(-1), _f32(v_scales), _f32(v_quats)
+    _chk(lib().orc_activate_params_bwd(c_u32(N), _p(o), _p(sc), _p(r), _p(g_o), _p(g_s), _p(g_q), _p(vo), _p(vs),
+                                       _p(vr)),
          "activate_params_bwd")
     return vo, vs, vr
 

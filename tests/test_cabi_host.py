@@ -1,0 +1,119 @@
+"""CPU-side checks of the shipped library and host layer: libgsx.so loads and exports every symbol include/gsx.h
+declares, argument validation returns the documented status codes before anything is launched, the torch-facing
+mirror of the reference API rejects what the reference's CHECK_INPUT rejects, and the scene generator is
+deterministic.  Nothing here launches a kernel."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "gsx.h")).read()
+    return sorted(set(re.findall(r"GSX_API\s+[\w\s\*]+?\b(gsx_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(gsx):
+    lib = gsx._lib.lib()
+    names = declared_symbols()
+    assert len(names) >= 35 and "gsx_rasterize_to_pixels_from_world_3dgs_bwd" in names
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, missing
+
+
+def test_host_only_entry_points(gsx):
+    L = gsx._lib
+    lib = L.lib()
+    assert lib.gsx_version() >= 100
+    assert [lib.gsx_n_bits(ctypes.c_uint32(t)) for t in (1, 2, 255, 256, 4056, 8160, 32400)] == [1, 2, 8, 9, 12, 13, 15]
+    ut = lib.gsx_ut_defaults()  # gsplat/Cameras.h:33-44
+    assert (round(ut.alpha, 6), ut.beta, ut.kappa, round(ut.in_image_margin_factor, 6),
+            ut.require_all_sigma_points_valid) == (0.1, 2.0, 0.0, 0.1, 1)
+    assert lib.gsx_status_string(0) == b"ok" and b"unsupported" in lib.gsx_status_string(L.GSX_ERR_UNSUPPORTED)
+    assert lib.gsx_rasterize_bwd_workspace_bytes(ctypes.c_uint32(1000)) >= 1000 * 64
+    assert lib.gsx_radix_sort_pairs_workspace_bytes(ctypes.c_int64(10 ** 6)) >= 245 * 256 * 4
+    assert lib.gsx_intersect_tile_count_workspace_bytes(ctypes.c_uint32(1), ctypes.c_uint32(10 ** 6)) >= 489 * 8
+    assert lib.gsx_image_loss_blocks(ctypes.c_uint32(822), ctypes.c_uint32(1237)) == -(-822 * 1237 // 2048)
+
+
+def test_status_codes_without_launch(gsx):
+    L = gsx._lib
+    lib = L.lib()
+    nul = ctypes.c_void_p(None)
+    one = ctypes.c_void_p(256)  # a non-null dummy: the calls below must fail validation before touching it
+    u32, i64, cf, ci = ctypes.c_uint32, ctypes.c_int64, ctypes.c_float, ctypes.c_int
+    # zero-size inputs are accepted and do nothing (ProjectionUT3DGSFused.cu:249-252, IntersectTile.cu:268-271)
+    assert lib.gsx_spherical_harmonics_fwd(u32(0), u32(16), u32(3), nul, nul, nul, nul, nul) == L.GSX_OK
+    assert lib.gsx_adam_step(nul, nul, nul, nul, i64(0), cf(1), cf(.9), cf(.999), cf(1e-15), cf(1), cf(1), nul) == 0
+    assert lib.gsx_relocation(ci(0), nul, nul, nul, nul, ci(51), nul, nul, nul) == L.GSX_OK
+    sel = ci(7)
+    assert lib.gsx_radix_sort_pairs(i64(0), nul, nul, nul, nul, u32(45), nul, ctypes.c_size_t(0),
+                                    ctypes.byref(sel), nul) == L.GSX_OK and sel.value == 0
+    # invalid arguments
+    assert lib.gsx_spherical_harmonics_fwd(u32(10), u32(4), u32(3), one, one, nul, one, nul) == \
+        L.GSX_ERR_INVALID_ARGUMENT  # degree 3 needs K >= 16
+    assert b"K >= 16" in lib.gsx_last_error()
+    assert lib.gsx_spherical_harmonics_fwd(u32(10), u32(16), u32(3), nul, one, nul, one, nul) == \
+        L.GSX_ERR_INVALID_ARGUMENT  # null tensor
+    assert lib.gsx_radix_sort_pairs(i64(100), one, one, one, one, u32(45), nul, ctypes.c_size_t(0), ctypes.byref(sel),
+                                    nul) == L.GSX_ERR_WORKSPACE
+    assert lib.gsx_radix_sort_pairs(i64(1 << 31), one, one, one, one, u32(45), one, ctypes.c_size_t(1 << 40),
+                                    ctypes.byref(sel), nul) == L.GSX_ERR_OVERFLOW
+    ut = L.UTParams()
+    proj = lambda C, model, rs, vm1: lib.gsx_projection_ut_3dgs_fused(
+        u32(C), u32(10), one, one, one, one, one, vm1, one, u32(64), u32(64), cf(.3), cf(.01), cf(1e4), cf(0),
+        ci(model), ut, ci(rs), nul, nul, nul, one, one, one, one, nul, nul)
+    assert proj(2, L.PINHOLE, L.GLOBAL, nul) == L.GSX_ERR_UNSUPPORTED        # C > 1
+    assert proj(1, L.FISHEYE, L.GLOBAL, nul) == L.GSX_ERR_UNSUPPORTED        # camera model
+    assert proj(1, L.PINHOLE, L.ROLLING_TOP_TO_BOTTOM, nul) == L.GSX_ERR_UNSUPPORTED
+    assert proj(1, L.PINHOLE, L.GLOBAL, one) == L.GSX_ERR_UNSUPPORTED        # viewmats1 given
+    n_host = i64(-1)
+    assert lib.gsx_intersect_tile_count(u32(1), u32(10), one, one, u32(16), u32(1 << 20), u32(1 << 11), one, one, one,
+                                        ctypes.c_size_t(1 << 20), ctypes.byref(n_host), nul) == \
+        L.GSX_ERR_INVALID_ARGUMENT  # tile id + camera id need more than 32 bits (Intersect.cpp:50)
+    groups = (L.AdamGroup * 9)()
+    assert lib.gsx_adam_step_multi(groups, ci(9), nul) == L.GSX_ERR_INVALID_ARGUMENT
+
+
+def test_python_mirror_rejects_what_check_input_rejects(gsx):
+    torch = pytest.importorskip("torch")
+    ops = gsx.ops
+    cpu = torch.zeros((4, 3))
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):  # gsplat/Common.h:12
+        ops.quats_to_rotmats(torch.zeros((4, 4)))
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        ops.spherical_harmonics_fwd(3, cpu, torch.zeros((4, 16, 3)), None)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        ops.relocation(torch.zeros(4), cpu, torch.ones(4, dtype=torch.int32), torch.zeros((51, 51)), 51)
+    with pytest.raises(TypeError):
+        ops.intersect_offset(np.zeros(3, np.int64), 1, 4, 4)
+
+
+def test_scene_generator_is_deterministic(gsx):
+    a, b = gsx.scenes.config(3, 1000), gsx.scenes.config(3, 1000)
+    for k, v in a.params().items():
+        assert np.array_equal(v, b.params()[k]) and v.dtype == np.float32
+    assert a.shN.shape == (1000, 15, 3) and a.sh0.shape == (1000, 1, 3) and a.sh_degree == 3
+    assert not np.array_equal(a.means, a.target_scene.means)
+    cam = a.cameras[0]
+    assert (cam.width, cam.height) == (1237, 822) and cam.K[0, 0] == 1150.0
+    R = cam.viewmat[:3, :3].astype(np.float64)
+    np.testing.assert_allclose(R @ R.T, np.eye(3), atol=1e-6)
+    np.testing.assert_allclose(np.linalg.norm(np.linalg.inv(cam.viewmat.astype(np.float64))[:3, 3]), 4.0, rtol=1e-6)
+    c1 = gsx.scenes.config(1)
+    assert c1.n == 10_000 and c1.sh_degree == 0 and c1.target.shape == (3, 256, 256)
+    assert len(gsx.scenes.config(2, 100).cameras) == 8
+
+
+def test_oracle_training_reduces_the_loss(gsx):
+    """the CPU restatement of the whole iteration (forward, loss, backward, Adam) descends"""
+    from oracle.step import OracleTrainStep
+    sc = gsx.scenes.config(1, 3000)
+    cam = sc.cameras[0]
+    st = OracleTrainStep(sc, lambda_dssim=0.2, lrs=dict(sh0=0.05, opacity=0.05))
+    losses = [st.step(cam.viewmat, cam.K, cam.width, cam.height, sc.target) for _ in range(4)]
+    assert losses[-1] < losses[0] - 1e-4, losses

@@ -1,0 +1,339 @@
+"""Pins the checker's projection, spherical harmonics, tile intersection, sort and offsets against independent
+statements of the mathematics (float64 numpy models, closed forms, brute force), since the reference holds no
+golden vectors for this path (its only test, tests/test_render_modes.cpp, checks tensor shapes)."""
+import numpy as np
+import pytest
+from scipy.spatial.transform import Rotation
+
+
+def look_cam(W=640, H=480, f=500.0, z=4.0):
+    V = np.eye(4, dtype=np.float32)
+    V[2, 3] = z
+    K = np.array([[f, 0, W / 2], [0, f, H / 2], [0, 0, 1]], np.float32)
+    return V, K, W, H
+
+
+# ---------------------------------------------------------------------------------------------
+# unscented-transform projection
+# ---------------------------------------------------------------------------------------------
+def ut_project_f64(mean, quat_wxyz, scale, V, K, alpha=0.1, beta=2.0, kappa=0.0, eps2d=0.3):
+    """Unscented transform of N(mean, R diag(s^2) R^T) through the pinhole camera, written from the definition
+    (Wan & van der Merwe 2000 weights; sigma points along the principal axes) in float64."""
+    q = np.asarray(quat_wxyz, np.float64)
+    q = q / np.linalg.norm(q)
+    Rg = Rotation.from_quat([q[1], q[2], q[3], q[0]]).as_matrix()
+    lam = float(np.float32(np.float32(alpha) * np.float32(alpha) * np.float32(3.0 + kappa)) - np.float32(3.0))
+    n = 3.0
+    pts = [np.asarray(mean, np.float64)]
+    for sgn in (+1, -1):
+        for i in range(3):
+            pts.append(mean + sgn * np.sqrt(n + lam) * scale[i] * Rg[:, i])
+    wm = np.array([lam / (n + lam)] + [1 / (2 * (n + lam))] * 6)
+    wc = wm.copy()
+    wc[0] += 1 - alpha * alpha + beta
+    Rc, t = V[:3, :3].astype(np.float64), V[:3, 3].astype(np.float64)
+    uv = []
+    for p in pts:
+        c = Rc @ p + t
+        uv.append(np.array([K[0, 0] * c[0] / c[2] + K[0, 2], K[1, 1] * c[1] / c[2] + K[1, 2]]))
+    uv = np.array(uv)
+    m = (wm[:, None] * uv).sum(0)
+    d = uv - m
+    cov = (wc[:, None, None] * d[:, :, None] * d[:, None, :]).sum(0)
+    det0 = np.linalg.det(cov)
+    cov = cov + eps2d * np.eye(2)
+    comp = np.sqrt(max(0.0, det0 / np.linalg.det(cov)))
+    return m, cov, comp, (Rc @ mean + t)[2]
+
+
+def ewa_cov_f64(mean, quat_wxyz, scale, V, K):
+    """Jacobian (EWA) projection of the same Gaussian: J W Sigma W^T J^T (Zwicker et al. 2001)."""
+    q = np.asarray(quat_wxyz, np.float64)
+    q = q / np.linalg.norm(q)
+    Rg = Rotation.from_quat([q[1], q[2], q[3], q[0]]).as_matrix()
+    Sigma = Rg @ np.diag(np.asarray(scale, np.float64) ** 2) @ Rg.T
+    Wm, t = V[:3, :3].astype(np.float64), V[:3, 3].astype(np.float64)
+    x, y, z = Wm @ mean + t
+    J = np.array([[K[0, 0] / z, 0, -K[0, 0] * x / z ** 2], [0, K[1, 1] / z, -K[1, 1] * y / z ** 2]])
+    return J @ Wm @ Sigma @ Wm.T @ J.T
+
+
+def test_projection_isotropic_on_axis_closed_form(orc):
+    V, K, W, H = look_cam()
+    s, f, z, o = 0.05, 500.0, 4.0, 0.8
+    r = orc.projection_ut_3dgs_fused(np.zeros((1, 3)), [[1, 0, 0, 0]], [[s, s, s]], [o], V[None], K[None], W, H,
+                                     calc_compensations=True)
+    radii, m2, depth, conic, comp = r
+    np.testing.assert_allclose(m2[0, 0], [W / 2, H / 2], atol=2e-2)
+    var = (f * s / z) ** 2  # up to O(s^2/z^2) relative
+    cov = var + 0.3
+    np.testing.assert_allclose(conic[0, 0], [1 / cov, 0, 1 / cov], rtol=2e-3, atol=1e-5)
+    assert depth[0, 0] == np.float32(z)
+    ext = min(3.33, np.sqrt(2 * np.log(o * np.sqrt(var * var / (cov * cov)) * 255)))
+    assert abs(int(radii[0, 0, 0]) - np.ceil(ext * np.sqrt(cov))) <= 1 and radii[0, 0, 0] == radii[0, 0, 1]
+    np.testing.assert_allclose(comp[0, 0], var / cov, rtol=2e-3)
+
+
+def test_projection_matches_float64_unscented_transform_and_ewa_limit(orc):
+    rng = np.random.default_rng(0)
+    V = np.eye(4, dtype=np.float32)
+    V[:3, :3] = Rotation.from_euler("xyz", [0.2, -0.3, 0.1]).as_matrix()
+    V[:3, 3] = [0.1, -0.2, 5.0]
+    K = np.array([[600, 0, 330], [0, 580, 250], [0, 0, 1]], np.float32)
+    W, H = 640, 480
+    n = 300
+    means = rng.uniform(-1, 1, (n, 3)).astype(np.float32)
+    quats = rng.normal(0, 1, (n, 4)).astype(np.float32)
+    scales = np.exp(rng.uniform(np.log(0.05), np.log(0.3), (n, 3))).astype(np.float32)
+    radii, m2, depth, conic, comp = orc.projection_ut_3dgs_fused(means, quats, scales, None, V[None], K[None], W, H,
+                                                                 calc_compensations=True)
+    checked = 0
+    for i in range(n):
+        if radii[0, i, 0] == 0:
+            continue
+        m, cov, c, z = ut_project_f64(means[i].astype(np.float64), quats[i], scales[i].astype(np.float64), V, K)
+        # -99 p0 + 16.7 sum(p_i): the weights amplify fp32 rounding of pixel coordinates (~600) about 100x
+        np.testing.assert_allclose(m2[0, i], m, atol=3e-2)
+        np.testing.assert_allclose(conic[0, i], [np.linalg.inv(cov)[0, 0], np.linalg.inv(cov)[0, 1],
+                                                 np.linalg.inv(cov)[1, 1]], rtol=3e-2, atol=2e-5)
+        np.testing.assert_allclose(depth[0, i], z, rtol=1e-6)
+        np.testing.assert_allclose(comp[0, i], c, rtol=2e-2)
+        ext = 3.33
+        b = 0.5 * (cov[0, 0] + cov[1, 1])
+        v1 = b + np.sqrt(max(0.01, b * b - np.linalg.det(cov)))
+        rx = np.ceil(min(ext * np.sqrt(cov[0, 0]), ext * np.sqrt(v1)))
+        ry = np.ceil(min(ext * np.sqrt(cov[1, 1]), ext * np.sqrt(v1)))
+        assert abs(radii[0, i, 0] - rx) <= 1 and abs(radii[0, i, 1] - ry) <= 1
+        checked += 1
+    assert checked > 100
+    # the float64 model itself: for small Gaussians the unscented transform tends to the Jacobian (EWA) projection
+    for i in range(20):
+        s = scales[i].astype(np.float64) * 0.02
+        _, cov, _, _ = ut_project_f64(means[i].astype(np.float64), quats[i], s, V, K, eps2d=0.0)
+        np.testing.assert_allclose(cov, ewa_cov_f64(means[i].astype(np.float64), quats[i], s, V, K), rtol=2e-3,
+                                   atol=1e-9)
+
+
+def test_projection_culling_cases(orc):
+    V, K, W, H = look_cam()
+    one = lambda mean, s=0.05, o=0.9, **kw: orc.projection_ut_3dgs_fused(
+        [mean], [[1, 0, 0, 0]], [[s, s, s]], None if o is None else [o], V[None], K[None], W, H, **kw)[0][0, 0]
+    assert one([0, 0, 0])[0] > 0
+    assert tuple(one([0, 0, -3.995])) == (0, 0)            # z = 0.005 < near 0.01
+    assert tuple(one([0, 0, 0], far_plane=3.0)) == (0, 0)  # z = 4 > far
+    # a sigma point behind the camera plane: z_c = 0.1, sigma points at z_c -/+ 0.173 * 1.0 along the view axis
+    behind = orc.projection_ut_3dgs_fused([[0, 0, -3.9]], [[1, 0, 0, 0]], [[1e-3, 1e-3, 1.0]], [0.9], V[None], K[None],
+                                          W, H)[0][0, 0]
+    assert tuple(behind) == (0, 0)
+    ahead = orc.projection_ut_3dgs_fused([[0, 0, -3.9]], [[1, 0, 0, 0]], [[1e-3, 1e-3, 0.5]], [0.9], V[None], K[None],
+                                         W, H)[0][0, 0]
+    assert ahead[0] > 0
+    assert tuple(one([2.9, 0, 0])) == (0, 0)               # u = 320 + 500*2.9/4 = 682 >= 1.1 W... outside the margin
+    assert one([2.7, 0, 0])[0] > 0                         # u = 657.5 inside the 10 % margin and bbox touches the image
+    assert tuple(one([0, 0, 0], o=0.003)) == (0, 0)        # opacity * compensation < 1/255
+    assert one([0, 0, 0], o=0.01)[0] > 0
+    assert tuple(one([0, 0, 0], s=1e-4, radius_clip=3.0)) == (0, 0)  # radius <= radius_clip
+    # opacity-aware extent shrinks the radius (Section B.2 of arXiv 2402.00525)
+    assert one([0, 0, 0], o=0.01)[0] < one([0, 0, 0], o=0.9)[0] <= one([0, 0, 0], o=None)[0]
+    # require_all_sigma_points_valid = False keeps a Gaussian with one invalid sigma point
+    ut = dict(require_all_sigma_points_valid=False)
+    assert orc.projection_ut_3dgs_fused([[2.88, 0, 0]], [[1, 0, 0, 0]], [[0.3, 0.3, 0.3]], None, V[None], K[None], W,
+                                        H, ut=ut)[0][0, 0, 0] > 0
+
+
+# ---------------------------------------------------------------------------------------------
+# spherical harmonics
+# ---------------------------------------------------------------------------------------------
+def sh_basis_polynomials(d):
+    """Real SH basis in the explicit polynomial form of the original 3DGS / tiny-cuda-nn code (an algebraically
+    different statement from the Sloan recurrences the reference's gsplat kernel uses), degrees 0-3."""
+    x, y, z = d[..., 0], d[..., 1], d[..., 2]
+    xx, yy, zz, xy, yz, xz = x * x, y * y, z * z, x * y, y * z, x * z
+    return np.stack([
+        0.28209479177387814 * np.ones_like(x),
+        -0.4886025119029199 * y, 0.4886025119029199 * z, -0.4886025119029199 * x,
+        1.0925484305920792 * xy, -1.0925484305920792 * yz, 0.31539156525252005 * (2 * zz - xx - yy),
+        -1.0925484305920792 * xz, 0.5462742152960396 * (xx - yy),
+        -0.5900435899266435 * y * (3 * xx - yy), 2.890611442640554 * xy * z,
+        -0.4570457994644658 * y * (4 * zz - xx - yy), 0.3731763325901154 * z * (2 * zz - 3 * xx - 3 * yy),
+        -0.4570457994644658 * x * (4 * zz - xx - yy), 1.445305721320277 * z * (xx - yy),
+        -0.5900435899266435 * x * (xx - 3 * yy)], -1)
+
+
+def checker_basis(orc, dirs, degree, K=25):
+    """basis values through the checker: colour of a one-hot coefficient vector"""
+    n = dirs.shape[0]
+    B = np.zeros((n, K))
+    for k in range((degree + 1) ** 2):
+        co = np.zeros((n, K, 3), np.float32)
+        co[:, k, 0] = 1.0
+        B[:, k] = orc.spherical_harmonics_fwd(degree, dirs, co)[:, 0]
+    return B
+
+
+def test_sh_basis_matches_polynomial_form(orc):
+    rng = np.random.default_rng(0)
+    d = rng.normal(0, 1, (2000, 3))
+    dn = d / np.linalg.norm(d, axis=1, keepdims=True)
+    scale = rng.uniform(0.1, 10, (2000, 1))  # the kernel normalises the direction itself
+    B = checker_basis(orc, (dn * scale).astype(np.float32), 3)
+    np.testing.assert_allclose(B[:, :16], sh_basis_polynomials(dn), atol=3e-6)
+    # lower degrees use the leading bases only
+    for deg in (0, 1, 2):
+        Bd = checker_basis(orc, dn.astype(np.float32), deg)
+        nb = (deg + 1) ** 2
+        np.testing.assert_allclose(Bd[:, :nb], sh_basis_polynomials(dn)[:, :nb], atol=3e-6)
+        assert np.all(Bd[:, nb:] == 0)
+
+
+def test_sh_basis_degree4_orthonormal_and_harmonic(orc):
+    # Gauss-Legendre x uniform-phi product quadrature integrates polynomials of degree <= 8 on the sphere exactly
+    nt, nphi = 12, 24
+    ct, wt = np.polynomial.legendre.leggauss(nt)
+    phi = (np.arange(nphi) + 0.5) * 2 * np.pi / nphi
+    CT, PH = np.meshgrid(ct, phi, indexing="ij")
+    st = np.sqrt(1 - CT ** 2)
+    d = np.stack([st * np.cos(PH), st * np.sin(PH), CT], -1).reshape(-1, 3)
+    w = (wt[:, None] * np.ones(nphi)[None] * 2 * np.pi / nphi).reshape(-1)
+    B = checker_basis(orc, d.astype(np.float32), 4)
+    G = (B * w[:, None]).T @ B
+    np.testing.assert_allclose(G, np.eye(25), atol=2e-5)
+    # parity (-1)^l under d -> -d pins the degree of each band
+    Bm = checker_basis(orc, (-d).astype(np.float32), 4)
+    deg = np.concatenate([[l] * (2 * l + 1) for l in range(5)])
+    np.testing.assert_allclose(Bm, B * ((-1.0) ** deg)[None], atol=2e-6)
+    # the m = 0 members are the Legendre polynomials in z, with positive sign at the pole
+    pole = checker_basis(orc, np.array([[0, 0, 1.0]], np.float32), 4)[0]
+    for l in range(5):
+        assert abs(pole[l * l + l] - np.sqrt((2 * l + 1) / (4 * np.pi))) < 2e-6
+
+
+def test_sh_colour_and_adjoint(orc):
+    rng = np.random.default_rng(1)
+    n, K = 500, 16
+    dirs = rng.normal(0, 1, (n, 3)).astype(np.float32)
+    co = rng.normal(0, 1, (n, K, 3)).astype(np.float32)
+    masks = rng.uniform(0, 1, n) < 0.7
+    dn = dirs / np.linalg.norm(dirs, axis=1, keepdims=True)
+    for deg in range(4):
+        col = orc.spherical_harmonics_fwd(deg, dirs, co, masks)
+        nb = (deg + 1) ** 2
+        want = np.einsum("nk,nkc->nc", sh_basis_polynomials(dn.astype(np.float64))[:, :nb], co[:, :nb].astype(np.float64))
+        np.testing.assert_allclose(col[masks], want[masks], atol=2e-5)
+        assert np.all(col[~masks] == 0)
+        # backward = transpose of forward:  <v, fwd(c)> == <bwd(v), c>
+        v = rng.normal(0, 1, (n, 3)).astype(np.float32)
+        vc, vd = orc.spherical_harmonics_bwd(K, deg, dirs, co, masks, v, True)
+        lhs = (v[masks].astype(np.float64) * col[masks]).sum()
+        rhs = (vc.astype(np.float64) * co).sum()
+        assert abs(lhs - rhs) < 1e-3 * max(1.0, abs(lhs))
+        assert np.all(vc[~masks] == 0) and np.all(vc[:, nb:] == 0)
+        # direction gradient against central differences of the float64 polynomial form
+        h = 1e-6
+        for j in range(3):
+            dp, dm = dirs.astype(np.float64).copy(), dirs.astype(np.float64).copy()
+            dp[:, j] += h
+            dm[:, j] -= h
+            fp = np.einsum("nk,nkc->nc", sh_basis_polynomials(dp / np.linalg.norm(dp, axis=1, keepdims=True))[:, :nb],
+                           co[:, :nb].astype(np.float64))
+            fm = np.einsum("nk,nkc->nc", sh_basis_polynomials(dm / np.linalg.norm(dm, axis=1, keepdims=True))[:, :nb],
+                           co[:, :nb].astype(np.float64))
+            num = ((fp - fm) / (2 * h) * v).sum(1)
+            np.testing.assert_allclose(vd[masks, j], num[masks], rtol=2e-3, atol=2e-4)
+
+
+def test_sh_colors_from_world_glue(orc):
+    """dirs = means - campos with campos = -R^T t, radii mask, +0.5 and clamp at 0 (Rasterization.cpp:356-378)"""
+    rng = np.random.default_rng(2)
+    n, K = 300, 16
+    V = np.eye(4, dtype=np.float32)
+    V[:3, :3] = Rotation.from_euler("xyz", [0.3, 0.5, -0.2]).as_matrix()
+    V[:3, 3] = [0.3, -0.1, 4.0]
+    campos = np.linalg.inv(V.astype(np.float64))[:3, 3]
+    means = rng.normal(0, 1, (n, 3)).astype(np.float32)
+    co = rng.normal(0, 0.6, (n, K, 3)).astype(np.float32)
+    radii = rng.integers(0, 3, (n, 2)).astype(np.int32)
+    col = orc.sh_colors_from_world(3, means, co, radii, V)
+    d = means.astype(np.float64) - campos
+    want = np.maximum(np.einsum("nk,nkc->nc", sh_basis_polynomials(d / np.linalg.norm(d, axis=1, keepdims=True)),
+                                co.astype(np.float64)) + 0.5, 0)
+    vis = (radii > 0).all(1)
+    np.testing.assert_allclose(col[vis], want[vis], atol=3e-5)
+    assert np.all(col[~vis] == 0) and (col[vis] == 0).any() and (col[vis] > 0).any()
+    v = rng.normal(0, 1, (n, 3)).astype(np.float32)
+    vsh = orc.sh_colors_from_world_bwd(3, means, K, radii, V, col, v)
+    Bm = sh_basis_polynomials(d / np.linalg.norm(d, axis=1, keepdims=True))
+    want_v = Bm[:, :, None] * np.where(col > 0, v, 0)[:, None, :] * vis[:, None, None]
+    np.testing.assert_allclose(vsh, want_v, atol=3e-5)
+
+
+# ---------------------------------------------------------------------------------------------
+# tile intersection, sort, offsets
+# ---------------------------------------------------------------------------------------------
+def brute_force_tiles(means2d, radii, tile, tw, th):
+    out = []
+    for g in range(means2d.shape[0]):
+        rx, ry = radii[g]
+        if rx <= 0 or ry <= 0:
+            out.append([])
+            continue
+        x0 = min(max(0, int(np.floor(np.float32(means2d[g, 0] / tile) - np.float32(rx / tile)))), tw)
+        x1 = min(max(0, int(np.ceil(np.float32(means2d[g, 0] / tile) + np.float32(rx / tile)))), tw)
+        y0 = min(max(0, int(np.floor(np.float32(means2d[g, 1] / tile) - np.float32(ry / tile)))), th)
+        y1 = min(max(0, int(np.ceil(np.float32(means2d[g, 1] / tile) + np.float32(ry / tile)))), th)
+        out.append([i * tw + j for i in range(y0, y1) for j in range(x0, x1)])
+    return out
+
+
+def test_intersect_brute_force_and_invariants(orc):
+    rng = np.random.default_rng(0)
+    n, W, H, tile = 400, 200, 120, 16
+    tw, th = (W + 15) // 16, (H + 15) // 16
+    means2d = rng.uniform(-60, 260, (1, n, 2)).astype(np.float32)  # includes centres left of / above the image
+    radii = rng.integers(0, 40, (1, n, 2)).astype(np.int32)
+    radii[0, ::9] = 0
+    depths = np.exp(rng.normal(1, 0.5, (1, n))).astype(np.float32)
+    tpg, ids, flat = orc.intersect_tile(means2d, radii, depths, 1, tile, tw, th, sort=False)
+    want = brute_force_tiles(means2d[0], radii[0], tile, tw, th)
+    assert [len(t) for t in want] == list(tpg[0])
+    assert tpg.sum() == ids.shape[0] == flat.shape[0] > 0
+    exp_ids = np.array([(t << 32) | int(depths[0, g].view(np.uint32)) for g, ts in enumerate(want) for t in ts],
+                       np.int64)
+    exp_flat = np.array([g for g, ts in enumerate(want) for _ in ts], np.int32)
+    assert np.array_equal(ids, exp_ids) and np.array_equal(flat, exp_flat)
+    # sorted: stable ascending on (tile, depth bits); ties keep emission order
+    _, sid, sflat = orc.intersect_tile(means2d, radii, depths, 1, tile, tw, th, sort=True)
+    order = np.argsort(exp_ids, kind="stable")
+    assert np.array_equal(sid, exp_ids[order]) and np.array_equal(sflat, exp_flat[order])
+    off = orc.intersect_offset(sid, 1, tw, th)
+    tiles = (sid >> 32)
+    cnt = np.bincount(tiles, minlength=tw * th)
+    assert np.array_equal(off.ravel(), np.concatenate([[0], np.cumsum(cnt)[:-1]]))
+    assert np.all(np.diff(off.ravel()) >= 0)
+    assert np.all(orc.intersect_offset(np.zeros(0, np.int64), 1, tw, th) == 0)
+
+
+def test_intersect_key_layout_and_bits(orc):
+    assert [orc.tile_n_bits(t) for t in (1, 2, 255, 256, 4056, 8160, 32400)] == [1, 2, 8, 9, 12, 13, 15]
+    # one Gaussian covering a 2x3 block of tiles: row-major emission, depth bits in the low word
+    m2 = np.array([[[40.0, 24.0]]], np.float32)
+    rad = np.array([[[20, 10]]], np.int32)
+    dep = np.array([[2.5]], np.float32)
+    tpg, ids, flat = orc.intersect_tile(m2, rad, dep, 1, 16, 10, 10, sort=False)
+    # x tiles floor(2.5 - 1.25) = 1 .. ceil(2.5 + 1.25) = 4 -> 1, 2, 3 ; y tiles floor(1.5 - 0.625) = 0 .. ceil(2.125) = 3
+    tiles = [(i * 10 + j) for i in range(0, 3) for j in range(1, 4)]
+    assert tpg[0, 0] == 9 and list(ids >> 32) == tiles and np.all(flat == 0)
+    assert np.all((ids & 0xffffffff) == int(dep.view(np.uint32)[0, 0]))
+
+
+def test_radix_sort_is_stable_on_bit_range(orc):
+    rng = np.random.default_rng(1)
+    n = 20000
+    keys = rng.integers(0, 1 << 50, n, dtype=np.int64)
+    keys[::3] = keys[0]  # many ties
+    vals = np.arange(n, dtype=np.int32)
+    for end_bit in (1, 7, 33, 45, 64):
+        mask = (1 << end_bit) - 1 if end_bit < 64 else -1
+        k, v = orc.radix_sort_pairs(keys, vals, end_bit)
+        order = np.argsort((keys & mask).astype(np.uint64), kind="stable")
+        assert np.array_equal(k, keys[order]) and np.array_equal(v, vals[order])

@@ -1,0 +1,97 @@
+"""Pins the shared fp32 primitives (lichtfeld-studio_amd/csrc/gsx_math.h, host build inside the checker) against
+numpy / scipy, so that a wrong coefficient, sign or index in them fails here."""
+import numpy as np
+import pytest
+from scipy.spatial.transform import Rotation, Slerp
+
+
+def ulps(a, b):
+    b32 = b.astype(np.float32)
+    return np.abs(a.astype(np.float64) - b) / np.spacing(np.abs(b32)).astype(np.float64)
+
+
+def test_exp_log_rsqrt_accuracy(orc):
+    rng = np.random.default_rng(0)
+    x = rng.uniform(-86.9, 88.0, 400_000).astype(np.float32)
+    assert ulps(orc.math_unary("exp", x), np.exp(x.astype(np.float64))).max() <= 2.0
+    assert np.all(orc.math_unary("exp", np.array([-87.5, -1e4, -np.inf], np.float32)) == 0.0)
+    assert np.all(np.isinf(orc.math_unary("exp", np.array([88.8, 1e4], np.float32))))
+    assert orc.math_unary("exp", np.zeros(1, np.float32))[0] == 1.0
+    y = np.exp(rng.uniform(-85, 85, 400_000)).astype(np.float32)
+    lg, ref = orc.math_unary("log", y), np.log(y.astype(np.float64))
+    assert (np.abs(lg - ref) <= 2.0 * np.spacing(np.abs(ref).astype(np.float32)) + 1e-7).all()
+    assert orc.math_unary("log", np.ones(1, np.float32))[0] == 0.0
+    assert ulps(orc.math_unary("rsqrt", y), 1.0 / np.sqrt(y.astype(np.float64))).max() <= 2.0
+    s = rng.uniform(-30, 30, 100_000).astype(np.float32)
+    np.testing.assert_allclose(orc.math_unary("sigmoid", s), 1 / (1 + np.exp(-s.astype(np.float64))), rtol=3e-7,
+                               atol=1e-30)
+    b, e = rng.uniform(1e-4, 1.0, 100_000).astype(np.float32), rng.uniform(0.02, 52, 100_000).astype(np.float32)
+    np.testing.assert_allclose(orc.math_pow(b, e), np.power(b.astype(np.float64), e.astype(np.float64)), rtol=5e-5,
+                               atol=1e-37)
+
+
+def test_sin_acos(orc):
+    rng = np.random.default_rng(1)
+    x = rng.uniform(-np.pi, np.pi, 200_000).astype(np.float32)
+    np.testing.assert_allclose(orc.math_unary("sin", x), np.sin(x.astype(np.float64)), rtol=0, atol=2e-7)
+    c = rng.uniform(-1, 1, 200_000).astype(np.float32)
+    np.testing.assert_allclose(orc.math_unary("acos", c), np.arccos(c.astype(np.float64)), rtol=0, atol=5e-7)
+    near1 = (1.0 - np.exp(rng.uniform(-16, -3, 1000))).astype(np.float32)
+    np.testing.assert_allclose(orc.math_unary("acos", near1), np.arccos(near1.astype(np.float64)), rtol=2e-6, atol=0)
+
+
+def test_sat_u32(orc):
+    x = np.array([-1e9, -1.5, -0.0, 0.0, 0.99, 1.0, 77.7, 4294967040.0, 4294967296.0, 1e20, np.nan, -np.inf, np.inf],
+                 np.float32)
+    want = np.array([0, 0, 0, 0, 0, 1, 77, 4294967040, 4294967295, 4294967295, 0, 0, 4294967295], np.float64)
+    assert np.array_equal(orc.math_unary("sat_u32", x).astype(np.float64), want.astype(np.float32).astype(np.float64))
+
+
+def test_quaternion_helpers_against_scipy(orc):
+    rng = np.random.default_rng(2)
+    for _ in range(200):
+        q = rng.normal(0, 1, 4)
+        q /= np.linalg.norm(q)
+        w, x, y, z = q
+        R = Rotation.from_quat([x, y, z, w]).as_matrix()
+        # mat3_cast (no normalisation) and quat_to_rotmat (normalises): both must give R, row-major
+        np.testing.assert_allclose(orc.math_quat("mat3_cast", q, 9).reshape(3, 3), R, atol=2e-6)
+        np.testing.assert_allclose(orc.math_quat("quat_to_rotmat", 3.7 * q, 9).reshape(3, 3), R, atol=2e-6)
+        # quat_cast: R -> q (up to sign), for all four branches of the largest-component selection
+        qc = orc.math_quat("quat_cast", R.astype(np.float32).ravel(), 4)
+        assert min(np.abs(qc - q).max(), np.abs(qc + q).max()) < 2e-6
+        # rotate(q, v) = R v
+        v = rng.normal(0, 2, 3)
+        np.testing.assert_allclose(orc.math_quat("quat_rotate", np.concatenate([q, v]), 3), R @ v, atol=5e-6)
+    # the four quat_cast branches explicitly: rotations by pi about x, y, z and the identity
+    for axis, idx in (([1, 0, 0], 1), ([0, 1, 0], 2), ([0, 0, 1], 3)):
+        R = Rotation.from_rotvec(np.pi * np.array(axis, float)).as_matrix()
+        qc = orc.math_quat("quat_cast", R.astype(np.float32).ravel(), 4)
+        assert abs(abs(qc[idx]) - 1) < 1e-6
+    assert np.allclose(orc.math_quat("quat_cast", np.eye(3, dtype=np.float32).ravel(), 4), [1, 0, 0, 0])
+
+
+def test_slerp(orc):
+    rng = np.random.default_rng(3)
+    q = rng.normal(0, 1, 4).astype(np.float32)
+    q /= np.float32(np.sqrt((q.astype(np.float64) ** 2).sum()))
+    q32 = q.astype(np.float32)
+    # same end points: glm::slerp takes the lerp branch when |q|^2 > 1 - eps and returns x exactly for a = 0 and 0.5
+    if np.float32(np.dot(q32, q32)) > np.float32(1.0 - 1.1920929e-07):
+        for a in (0.0, 0.5):
+            assert np.array_equal(orc.math_quat("slerp", np.concatenate([q32, q32, [a]]), 4), q32)
+    # a slightly short quaternion takes the trigonometric branch: the result is q rescaled by ~ 1 / cos(theta / 2)
+    qs = (q32 * np.float32(0.999)).astype(np.float32)
+    r = orc.math_quat("slerp", np.concatenate([qs, qs, [0.5]]), 4)
+    theta = np.arccos(np.dot(qs.astype(np.float64), qs.astype(np.float64)))
+    np.testing.assert_allclose(r, qs / np.cos(theta / 2), rtol=2e-6)
+    # general case against scipy (wxyz -> xyzw)
+    for _ in range(50):
+        a, b = rng.normal(0, 1, 4), rng.normal(0, 1, 4)
+        a /= np.linalg.norm(a)
+        b /= np.linalg.norm(b)
+        t = rng.uniform(0, 1)
+        got = orc.math_quat("slerp", np.concatenate([a, b, [t]]), 4)
+        rot = Slerp([0, 1], Rotation.from_quat([[a[1], a[2], a[3], a[0]], [b[1], b[2], b[3], b[0]]]))(t).as_quat()
+        want = np.array([rot[3], rot[0], rot[1], rot[2]])
+        assert min(np.abs(got - want).max(), np.abs(got + want).max()) < 5e-6
