@@ -66,6 +66,8 @@ GSX_API gsx_ut_params gsx_ut_defaults(void);
  * device so that a test can compare it bit for bit with a host build.  which: 0 exp, 1 log, 2 rsqrt, 3 sin, 4 acos,
  * 5 sigmoid, 6 saturating float->u32, 7 pow(x, x2), 8 x / x2, 9 sqrt, 10 fma(x, x2, x). */
 GSX_API int gsx_debug_math(int which, uint32_t n, const float* x, const float* x2, float* y, void* stream);
+/* Test hook: the 64-lane, 16-value wave reduction of the rasterizer backward.  in [n_waves,64,16] -> out [n_waves,16]. */
+GSX_API int gsx_debug_wave_reduce16(uint32_t n_waves, const float* in, float* out, void* stream);
 
 /* ---- a1: gsplat::projection_ut_3dgs_fused (Ops.h:69-98; kernel ProjectionUT3DGSFused.cu:17-210) ----
  * means [N,3] quats [N,4] (wxyz) scales [N,3] opacities [N] nullable, viewmats0 [C,4,4], Ks [C,3,3]

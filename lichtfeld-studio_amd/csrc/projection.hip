@@ -258,58 +258,6 @@ __device__ __forceinline__ float sh_color_channel(uint32_t degree, vec3 dir, con
     return result;
 }
 
-// One lane per element, all three channels (the reference uses one thread per (element, channel),
-// SphericalHarmonicsCUDA.cu:373-399); a lane's coefficient row is 12*K contiguous bytes.
-__global__ void __launch_bounds__(256) sh_fwd_kernel(uint32_t N, uint32_t K, uint32_t degree,
-                                                      const float* __restrict__ dirs,
-                                                      const float* __restrict__ coeffs,
-                                                      const uint8_t* __restrict__ masks,
-                                                      float* __restrict__ colors) {
-    const uint32_t e = blockIdx.x * 256u + threadIdx.x;
-    if (e >= N)
-        return;
-    if (masks != nullptr && !masks[e])
-        return;
-    const vec3 dir = ld3(dirs, e);
-    float B[25];
-    sh_basis(degree, dir, B);
-    const float* co = coeffs + (size_t)e * K * 3;
-#pragma unroll
-    for (uint32_t c = 0; c < 3; ++c)
-        colors[e * 3 + c] = sh_color_channel(degree, dir, B, co, c);
-}
-
-// VJP wrt the coefficients (SphericalHarmonicsCUDA.cu:112-371 with v_dir == nullptr): every entry of the
-// element's [K,3] row is written (zero for masked elements and bands above `degree`), so the caller needs no
-// memset.
-__global__ void __launch_bounds__(256) sh_bwd_kernel(uint32_t N, uint32_t K, uint32_t degree,
-                                                      const float* __restrict__ dirs,
-                                                      const uint8_t* __restrict__ masks,
-                                                      const float* __restrict__ v_colors,
-                                                      float* __restrict__ v_coeffs) {
-    const uint32_t e = blockIdx.x * 256u + threadIdx.x;
-    if (e >= N)
-        return;
-    float* out = v_coeffs + (size_t)e * K * 3;
-    const bool live = masks == nullptr || masks[e];
-    float B[25];
-    int nb = 0;
-    float v[3] = {0.f, 0.f, 0.f};
-    if (live) {
-        nb = sh_basis(degree, ld3(dirs, e), B);
-#pragma unroll
-        for (int c = 0; c < 3; ++c)
-            v[c] = v_colors[e * 3 + c];
-    }
-    for (uint32_t k = 0; k < K; ++k) {
-        const bool used = (int)k < nb;
-        const float b = B[k < 25 ? k : 24];
-        out[k * 3 + 0] = used ? b * v[0] : 0.f;
-        out[k * 3 + 1] = used ? b * v[1] : 0.f;
-        out[k * 3 + 2] = used ? b * v[2] : 0.f;
-    }
-}
-
 // direction gradient (degree <= 3), accumulated over the three channels
 // (sh_coeffs_to_color_fast_vjp with v_dir != nullptr; the reference adds the channels with atomics, :474-478)
 __global__ void __launch_bounds__(256) sh_bwd_dirs_kernel(uint32_t N, uint32_t K, uint32_t degree,
@@ -466,53 +414,163 @@ __device__ __forceinline__ vec3 campos_from_viewmat(const float* __restrict__ vm
     return neg(mul_t(R, mk3(vm[3], vm[7], vm[11])));
 }
 
-// glue of the fused entry point (Rasterization.cpp:356-378): dirs, radii mask, SH, +0.5, clamp in one pass
-__global__ void __launch_bounds__(256) sh_world_fwd_kernel(uint32_t N, uint32_t K, uint32_t degree,
-                                                            const float* __restrict__ means,
-                                                            const float* __restrict__ coeffs,
-                                                            const int32_t* __restrict__ radii,
-                                                            const float* __restrict__ viewmat,
-                                                            float* __restrict__ colors) {
-    const uint32_t e = blockIdx.x * 256u + threadIdx.x;
-    if (e >= N)
-        return;
-    if (!(radii[e * 2] > 0 && radii[e * 2 + 1] > 0)) {
-        colors[e * 3 + 0] = 0.f;
-        colors[e * 3 + 1] = 0.f;
-        colors[e * 3 + 2] = 0.f;
-        return;
-    }
-    const vec3 dir = sub(ld3(means, e), campos_from_viewmat(viewmat));
-    float B[25];
-    sh_basis(degree, dir, B);
-    const float* co = coeffs + (size_t)e * K * 3;
+// ---- coefficient rows through LDS (K = 16) -----------------------------------------------------
+// A lane owns one Gaussian, whose 16x3 coefficients are a 192-byte row; lanes reading or writing their own rows
+// directly touch 64 different cache lines per instruction.  Instead a wave moves its 64 rows (12 KiB, contiguous in
+// memory) with fully coalesced 16-byte accesses and transposes through LDS; rows are padded to 13 x 16 bytes so
+// that the per-lane 16-byte LDS accesses are conflict-free.
+static constexpr uint32_t kShRowF4 = 12;   // float4 per row (K = 16)
+static constexpr uint32_t kShLdsF4 = 13;   // padded row stride in float4
+
+__device__ __forceinline__ void sh16_rows_to_lds(const float* __restrict__ coeffs, uint32_t row0, uint32_t N,
+                                                 float4* wave_lds, uint32_t lane) {
+    const float4* src = reinterpret_cast<const float4*>(coeffs + (size_t)row0 * 48);
+    const uint32_t n_f4 = min(64u, N - row0) * kShRowF4;
 #pragma unroll
-    for (uint32_t c = 0; c < 3; ++c)
-        colors[e * 3 + c] = gsx::fmax(sh_color_channel(degree, dir, B, co, c) + 0.5f, 0.0f);
+    for (uint32_t i = 0; i < kShRowF4; ++i) {
+        const uint32_t q = i * 64u + lane;
+        if (q < n_f4) {
+            const uint32_t r = (q * 43691u) >> 19; // q / 12 for q < 768
+            wave_lds[r * kShLdsF4 + (q - r * kShRowF4)] = src[q];
+        }
+    }
 }
 
-__global__ void __launch_bounds__(256) sh_world_bwd_kernel(uint32_t N, uint32_t K, uint32_t degree,
-                                                            const float* __restrict__ means,
-                                                            const int32_t* __restrict__ radii,
-                                                            const float* __restrict__ viewmat,
-                                                            const float* __restrict__ colors,
-                                                            const float* __restrict__ v_colors,
-                                                            float* __restrict__ v_coeffs) {
+__device__ __forceinline__ void sh16_rows_from_lds(float* __restrict__ v_coeffs, uint32_t row0, uint32_t N,
+                                                   const float4* wave_lds, uint32_t lane) {
+    float4* dst = reinterpret_cast<float4*>(v_coeffs + (size_t)row0 * 48);
+    const uint32_t n_f4 = min(64u, N - row0) * kShRowF4;
+#pragma unroll
+    for (uint32_t i = 0; i < kShRowF4; ++i) {
+        const uint32_t q = i * 64u + lane;
+        if (q < n_f4) {
+            const uint32_t r = (q * 43691u) >> 19;
+            dst[q] = wave_lds[r * kShLdsF4 + (q - r * kShRowF4)];
+        }
+    }
+}
+
+// glue of the fused entry point (Rasterization.cpp:356-378): dirs, radii mask, SH, +0.5, clamp in one pass.
+// WORLD: dirs = means - campos, radii mask, +0.5 and clamp; otherwise the plain operator with an optional mask.
+// LDS16: K == 16 and 16-byte aligned coefficients, rows staged through LDS.
+template <bool WORLD, bool LDS16>
+__global__ void __launch_bounds__(256) sh_fwd_generic_kernel(uint32_t N, uint32_t K, uint32_t degree,
+                                                              const float* __restrict__ dirs_or_means,
+                                                              const float* __restrict__ coeffs,
+                                                              const uint8_t* __restrict__ masks,
+                                                              const int32_t* __restrict__ radii,
+                                                              const float* __restrict__ viewmat,
+                                                              float* __restrict__ colors) {
+    __shared__ float4 lds[LDS16 ? 4 * 64 * kShLdsF4 : 1];
     const uint32_t e = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    float4* wave_lds = lds + (LDS16 ? wave * 64 * kShLdsF4 : 0);
+    if (LDS16) {
+        const uint32_t row0 = blockIdx.x * 256u + wave * 64u;
+        if (row0 < N)
+            sh16_rows_to_lds(coeffs, row0, N, wave_lds, lane);
+        __builtin_amdgcn_wave_barrier();
+    }
     if (e >= N)
         return;
-    float* out = v_coeffs + (size_t)e * K * 3;
-    const bool live = radii[e * 2] > 0 && radii[e * 2 + 1] > 0;
+    bool live;
+    if (WORLD)
+        live = radii[e * 2] > 0 && radii[e * 2 + 1] > 0;
+    else
+        live = masks == nullptr || masks[e];
+    if (!live) {
+        if (WORLD) {
+            colors[e * 3 + 0] = 0.f;
+            colors[e * 3 + 1] = 0.f;
+            colors[e * 3 + 2] = 0.f;
+        }
+        return;
+    }
+    vec3 dir = ld3(dirs_or_means, e);
+    if (WORLD)
+        dir = sub(dir, campos_from_viewmat(viewmat));
+    float B[25];
+    sh_basis(degree, dir, B);
+    float co_reg[48];
+    const float* co;
+    if (LDS16) {
+#pragma unroll
+        for (uint32_t j = 0; j < kShRowF4; ++j) {
+            const float4 t = wave_lds[lane * kShLdsF4 + j];
+            co_reg[4 * j + 0] = t.x;
+            co_reg[4 * j + 1] = t.y;
+            co_reg[4 * j + 2] = t.z;
+            co_reg[4 * j + 3] = t.w;
+        }
+        co = co_reg;
+    } else {
+        co = coeffs + (size_t)e * K * 3;
+    }
+#pragma unroll
+    for (uint32_t c = 0; c < 3; ++c) {
+        float v = sh_color_channel(degree, dir, B, co, c);
+        if (WORLD)
+            v = gsx::fmax(v + 0.5f, 0.0f);
+        colors[e * 3 + c] = v;
+    }
+}
+
+template <bool WORLD, bool LDS16>
+__global__ void __launch_bounds__(256) sh_bwd_generic_kernel(uint32_t N, uint32_t K, uint32_t degree,
+                                                              const float* __restrict__ dirs_or_means,
+                                                              const uint8_t* __restrict__ masks,
+                                                              const int32_t* __restrict__ radii,
+                                                              const float* __restrict__ viewmat,
+                                                              const float* __restrict__ colors,
+                                                              const float* __restrict__ v_colors,
+                                                              float* __restrict__ v_coeffs) {
+    __shared__ float4 lds[LDS16 ? 4 * 64 * kShLdsF4 : 1];
+    const uint32_t e = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    float4* wave_lds = lds + (LDS16 ? wave * 64 * kShLdsF4 : 0);
     float B[25];
     int nb = 0;
     float v[3] = {0.f, 0.f, 0.f};
-    if (live) {
-        const vec3 dir = sub(ld3(means, e), campos_from_viewmat(viewmat));
-        nb = sh_basis(degree, dir, B);
+    if (e < N) {
+        bool live;
+        if (WORLD)
+            live = radii[e * 2] > 0 && radii[e * 2 + 1] > 0;
+        else
+            live = masks == nullptr || masks[e];
+        if (live) {
+            vec3 dir = ld3(dirs_or_means, e);
+            if (WORLD)
+                dir = sub(dir, campos_from_viewmat(viewmat));
+            nb = sh_basis(degree, dir, B);
 #pragma unroll
-        for (int c = 0; c < 3; ++c)
-            v[c] = colors[e * 3 + c] <= 0.0f ? 0.f : v_colors[e * 3 + c];
+            for (int c = 0; c < 3; ++c) {
+                v[c] = v_colors[e * 3 + c];
+                if (WORLD && colors[e * 3 + c] <= 0.0f) // clamp VJP (Rasterization.cpp:609-610)
+                    v[c] = 0.f;
+            }
+        }
     }
+    if (LDS16) {
+        float o[48];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            const bool used = k < nb;
+            o[k * 3 + 0] = used ? B[k] * v[0] : 0.f;
+            o[k * 3 + 1] = used ? B[k] * v[1] : 0.f;
+            o[k * 3 + 2] = used ? B[k] * v[2] : 0.f;
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < kShRowF4; ++j)
+            wave_lds[lane * kShLdsF4 + j] = make_float4(o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]);
+        __builtin_amdgcn_wave_barrier();
+        const uint32_t row0 = blockIdx.x * 256u + wave * 64u;
+        if (row0 < N)
+            sh16_rows_from_lds(v_coeffs, row0, N, wave_lds, lane);
+        return;
+    }
+    if (e >= N)
+        return;
+    float* out = v_coeffs + (size_t)e * K * 3;
     for (uint32_t k = 0; k < K; ++k) {
         const bool used = (int)k < nb;
         const float b = B[k < 25 ? k : 24];
@@ -521,6 +579,33 @@ __global__ void __launch_bounds__(256) sh_world_bwd_kernel(uint32_t N, uint32_t 
         out[k * 3 + 2] = used ? b * v[2] : 0.f;
     }
 }
+
+template <bool WORLD>
+static void launch_sh_fwd(uint32_t N, uint32_t K, uint32_t degree, const float* dirs_or_means, const float* coeffs,
+                          const uint8_t* masks, const int32_t* radii, const float* viewmat, float* colors,
+                          hipStream_t s) {
+    const bool lds16 = K == 16 && (((uintptr_t)coeffs) & 15u) == 0;
+    if (lds16)
+        hipLaunchKernelGGL((sh_fwd_generic_kernel<WORLD, true>), dim3(cdiv(N, 256)), dim3(256), 0, s, N, K, degree,
+                           dirs_or_means, coeffs, masks, radii, viewmat, colors);
+    else
+        hipLaunchKernelGGL((sh_fwd_generic_kernel<WORLD, false>), dim3(cdiv(N, 256)), dim3(256), 0, s, N, K, degree,
+                           dirs_or_means, coeffs, masks, radii, viewmat, colors);
+}
+
+template <bool WORLD>
+static void launch_sh_bwd(uint32_t N, uint32_t K, uint32_t degree, const float* dirs_or_means, const uint8_t* masks,
+                          const int32_t* radii, const float* viewmat, const float* colors, const float* v_colors,
+                          float* v_coeffs, hipStream_t s) {
+    const bool lds16 = K == 16 && (((uintptr_t)v_coeffs) & 15u) == 0;
+    if (lds16)
+        hipLaunchKernelGGL((sh_bwd_generic_kernel<WORLD, true>), dim3(cdiv(N, 256)), dim3(256), 0, s, N, K, degree,
+                           dirs_or_means, masks, radii, viewmat, colors, v_colors, v_coeffs);
+    else
+        hipLaunchKernelGGL((sh_bwd_generic_kernel<WORLD, false>), dim3(cdiv(N, 256)), dim3(256), 0, s, N, K, degree,
+                           dirs_or_means, masks, radii, viewmat, colors, v_colors, v_coeffs);
+}
+
 } // namespace gsx
 
 using namespace gsx;
@@ -572,8 +657,7 @@ extern "C" int gsx_spherical_harmonics_fwd(uint32_t N, uint32_t K, uint32_t degr
     GSX_REQUIRE(degrees_to_use <= 4 && K >= (degrees_to_use + 1) * (degrees_to_use + 1), GSX_ERR_INVALID_ARGUMENT,
                 "spherical_harmonics_fwd: degree %u needs K >= %u (got %u)", degrees_to_use,
                 (degrees_to_use + 1) * (degrees_to_use + 1), K);
-    hipLaunchKernelGGL(sh_fwd_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, K, degrees_to_use,
-                       dirs, coeffs, masks, colors);
+    launch_sh_fwd<false>(N, K, degrees_to_use, dirs, coeffs, masks, nullptr, nullptr, colors, (hipStream_t)stream);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }
@@ -590,8 +674,8 @@ extern "C" int gsx_spherical_harmonics_bwd(uint32_t N, uint32_t K, uint32_t degr
                 (degrees_to_use + 1) * (degrees_to_use + 1), K);
     GSX_REQUIRE(v_dirs == nullptr || degrees_to_use <= 3, GSX_ERR_UNSUPPORTED,
                 "spherical_harmonics_bwd: v_dirs is implemented for degree <= 3");
-    hipLaunchKernelGGL(sh_bwd_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, K, degrees_to_use,
-                       dirs, masks, v_colors, v_coeffs);
+    launch_sh_bwd<false>(N, K, degrees_to_use, dirs, masks, nullptr, nullptr, nullptr, v_colors, v_coeffs,
+                         (hipStream_t)stream);
     GSX_LAUNCH_CHECK();
     if (v_dirs != nullptr) {
         hipLaunchKernelGGL(sh_bwd_dirs_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, K,
@@ -611,8 +695,7 @@ extern "C" int gsx_sh_colors_from_world(uint32_t N, uint32_t K, uint32_t sh_degr
     GSX_REQUIRE(sh_degree <= 4 && K >= (sh_degree + 1) * (sh_degree + 1), GSX_ERR_INVALID_ARGUMENT,
                 "sh_colors_from_world: degree %u needs K >= %u (got %u)", sh_degree, (sh_degree + 1) * (sh_degree + 1),
                 K);
-    hipLaunchKernelGGL(sh_world_fwd_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, K, sh_degree,
-                       means, sh_coeffs, radii, viewmat, colors);
+    launch_sh_fwd<true>(N, K, sh_degree, means, sh_coeffs, nullptr, radii, viewmat, colors, (hipStream_t)stream);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }
@@ -627,8 +710,8 @@ extern "C" int gsx_sh_colors_from_world_bwd(uint32_t N, uint32_t K, uint32_t sh_
     GSX_REQUIRE(sh_degree <= 4 && K >= (sh_degree + 1) * (sh_degree + 1), GSX_ERR_INVALID_ARGUMENT,
                 "sh_colors_from_world_bwd: degree %u needs K >= %u (got %u)", sh_degree,
                 (sh_degree + 1) * (sh_degree + 1), K);
-    hipLaunchKernelGGL(sh_world_bwd_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, K, sh_degree,
-                       means, radii, viewmat, colors, v_colors, v_sh_coeffs);
+    launch_sh_bwd<true>(N, K, sh_degree, means, nullptr, radii, viewmat, colors, v_colors, v_sh_coeffs,
+                        (hipStream_t)stream);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

@@ -22,6 +22,7 @@ namespace gsx {
 
 static constexpr uint32_t kTile = 16;
 static constexpr uint32_t kBatch = 256;
+static constexpr float kPowerCut = -5.55f; // exp(-5.55) = 3.8875e-3 < 1/255 = 3.9216e-3
 static constexpr uint32_t kAcc = 16; // floats accumulated per Gaussian: rgb 3, v_gro 3, v_grd(x)ray_d 9, opacity 1
 
 __global__ void __launch_bounds__(256) fill_f32_kernel(size_t n, float v, float* __restrict__ out) {
@@ -30,24 +31,66 @@ __global__ void __launch_bounds__(256) fill_f32_kernel(size_t n, float v, float*
         out[i] = v;
 }
 
-// sum of 16 values over the 64 lanes of a wave; on return lane L holds, in v[0], the wave total of component
-// ((L>>5)&1)*8 + ((L>>4)&1)*4 + ((L>>3)&1)*2 + ((L>>2)&1)
+// ---- cross-lane helpers -----------------------------------------------------------------------
+// One halving step of a wave reduction: lanes of the lower half want lo_mine + lo_partner, lanes of the upper half
+// want hi_mine + hi_partner.  v_permlane32_swap / v_permlane16_swap exchange the upper (odd-row) lanes of their first
+// operand with the lower (even-row) lanes of the second, so swap(lo, hi) followed by one add is the whole step.
+__device__ __forceinline__ float halve_swap32(float lo, float hi) {
+    const auto r = __builtin_amdgcn_permlane32_swap(f2u(lo), f2u(hi), false, false);
+    return u2f(r[0]) + u2f(r[1]);
+}
+__device__ __forceinline__ float halve_swap16(float lo, float hi) {
+    const auto r = __builtin_amdgcn_permlane16_swap(f2u(lo), f2u(hi), false, false);
+    return u2f(r[0]) + u2f(r[1]);
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp(float v) {
+    return u2f((uint32_t)__builtin_amdgcn_update_dpp(0, (int)f2u(v), CTRL, 0xf, 0xf, true));
+}
+static constexpr int kDppRowMirror = 0x140;     // lane i <-> 15 - i inside a row of 16
+static constexpr int kDppHalfMirror = 0x141;    // lane i <-> 7 - i inside a half row of 8
+static constexpr int kDppQuadXor1 = 0xB1;       // quad_perm [1,0,3,2]
+static constexpr int kDppQuadXor2 = 0x4E;       // quad_perm [2,3,0,1]
+
+// Sum of 16 values over the 64 lanes of a wave with a halving butterfly: 8 + 4 swap steps across the rows, then
+// 2 + 1 mirror steps inside a row, then the quad.  On return lane L holds the wave total of component
+// ((L>>5)&1)*8 + ((L>>4)&1)*4 + ((L>>3)&1)*2 + ((L>>2)&1).
 __device__ __forceinline__ float wave_reduce16(float (&v)[16], uint32_t lane) {
 #pragma unroll
-    for (uint32_t step = 0; step < 4; ++step) {
-        const uint32_t m = 32u >> step;
-        const uint32_t half = 8u >> step;
-        const bool upper = (lane & m) != 0;
+    for (uint32_t i = 0; i < 8; ++i)
+        v[i] = halve_swap32(v[i], v[i + 8]);
 #pragma unroll
-        for (uint32_t i = 0; i < half; ++i) {
-            const float send = upper ? v[i] : v[i + half];
-            const float keep = upper ? v[i + half] : v[i];
-            v[i] = keep + __shfl_xor(send, (int)m, 64);
-        }
+    for (uint32_t i = 0; i < 4; ++i)
+        v[i] = halve_swap16(v[i], v[i + 4]);
+    {
+        const bool upper = (lane & 8u) != 0;
+        const float a0 = v[0] + dpp<kDppRowMirror>(v[0]), b0 = v[2] + dpp<kDppRowMirror>(v[2]);
+        const float a1 = v[1] + dpp<kDppRowMirror>(v[1]), b1 = v[3] + dpp<kDppRowMirror>(v[3]);
+        v[0] = upper ? b0 : a0;
+        v[1] = upper ? b1 : a1;
     }
-    v[0] += __shfl_xor(v[0], 2, 64);
-    v[0] += __shfl_xor(v[0], 1, 64);
+    {
+        const bool upper = (lane & 4u) != 0;
+        const float a0 = v[0] + dpp<kDppHalfMirror>(v[0]), b0 = v[1] + dpp<kDppHalfMirror>(v[1]);
+        v[0] = upper ? b0 : a0;
+    }
+    v[0] += dpp<kDppQuadXor2>(v[0]);
+    v[0] += dpp<kDppQuadXor1>(v[0]);
     return v[0];
+}
+
+// probe of wave_reduce16 for tests: in [n_waves][64 lanes][16], out [n_waves][16]
+__global__ void __launch_bounds__(64) wave_reduce16_probe_kernel(const float* __restrict__ in, float* __restrict__ out) {
+    float v[16];
+    const uint32_t lane = threadIdx.x;
+#pragma unroll
+    for (uint32_t k = 0; k < 16; ++k)
+        v[k] = in[((size_t)blockIdx.x * 64 + lane) * 16 + k];
+    const float total = wave_reduce16(v, lane);
+    if ((lane & 3u) == 0) {
+        const uint32_t comp = ((lane >> 5) & 1u) * 8u + ((lane >> 4) & 1u) * 4u + ((lane >> 3) & 1u) * 2u + ((lane >> 2) & 1u);
+        out[(size_t)blockIdx.x * 16 + comp] = total;
+    }
 }
 
 __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
@@ -131,11 +174,18 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             const mat3 R = quat_to_rotmat(ld4q(quats, g));
             const vec3 s = ld3(scales, g);
             const float is0 = 1.0f / s.x, is1 = 1.0f / s.y, is2 = 1.0f / s.z;
-            stage[tr * 4 + 0] = make_float4(xyz.x, xyz.y, xyz.z, opac);
-            stage[tr * 4 + 1] = make_float4(is0 * R.m[0][0], is0 * R.m[1][0], is0 * R.m[2][0], is1 * R.m[0][1]);
-            stage[tr * 4 + 2] = make_float4(is1 * R.m[1][1], is1 * R.m[2][1], is2 * R.m[0][2], is2 * R.m[1][2]);
+            // M = diag(1/s) R^T and gro = M (ray_o - mean): the ray origin is the same for every pixel of a
+            // global-shutter camera, so this half of the per-pair work is done once per staged Gaussian
+            mat3 M;
+            M.m[0][0] = is0 * R.m[0][0], M.m[0][1] = is0 * R.m[1][0], M.m[0][2] = is0 * R.m[2][0];
+            M.m[1][0] = is1 * R.m[0][1], M.m[1][1] = is1 * R.m[1][1], M.m[1][2] = is1 * R.m[2][1];
+            M.m[2][0] = is2 * R.m[0][2], M.m[2][1] = is2 * R.m[1][2], M.m[2][2] = is2 * R.m[2][2];
+            const vec3 gro = mul(M, sub(ray_o, xyz));
+            stage[tr * 4 + 0] = make_float4(gro.x, gro.y, gro.z, opac);
+            stage[tr * 4 + 1] = make_float4(M.m[0][0], M.m[0][1], M.m[0][2], M.m[1][0]);
+            stage[tr * 4 + 2] = make_float4(M.m[1][1], M.m[1][2], M.m[2][0], M.m[2][1]);
             stage[tr * 4 + 3] =
-                make_float4(is2 * R.m[2][2], colors[(size_t)g * 3], colors[(size_t)g * 3 + 1], colors[(size_t)g * 3 + 2]);
+                make_float4(M.m[2][2], colors[(size_t)g * 3], colors[(size_t)g * 3 + 1], colors[(size_t)g * 3 + 2]);
         }
         __syncthreads();
 
@@ -145,9 +195,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             const float4 m0 = stage[t * 4 + 1];
             const float4 m1 = stage[t * 4 + 2];
             const float4 m2 = stage[t * 4 + 3];
-            const vec3 o = mk3(ray_o.x - a.x, ray_o.y - a.y, ray_o.z - a.z);
-            const vec3 gro = mk3(fma(m0.z, o.z, fma(m0.y, o.y, m0.x * o.x)), fma(m1.y, o.z, fma(m1.x, o.y, m0.w * o.x)),
-                                 fma(m2.x, o.z, fma(m1.w, o.y, m1.z * o.x)));
+            const vec3 gro = mk3(a.x, a.y, a.z);
             const vec3 grd = mk3(fma(m0.z, ray_d.z, fma(m0.y, ray_d.y, m0.x * ray_d.x)),
                                  fma(m1.y, ray_d.z, fma(m1.x, ray_d.y, m0.w * ray_d.x)),
                                  fma(m2.x, ray_d.z, fma(m1.w, ray_d.y, m1.z * ray_d.x)));
@@ -155,6 +203,11 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             const vec3 gcrod = cross(grd_n, gro);
             const float grayDist = dot(gcrod, gcrod);
             const float power = -0.5f * grayDist;
+            // exp(power) < 1/255 below kPowerCut, so alpha < 1/255 for any opacity <= 1: decided without the exp
+            if (power < kPowerCut && a.w <= 1.0f)
+                valid = false;
+            if (__builtin_amdgcn_ballot_w64(valid) == 0)
+                continue;
             const float vis = gsx::exp(power);
             const float alpha = gsx::fmin(0.999f, a.w * vis);
             if (power > 0.f || alpha < 1.f / 255.f)
@@ -318,6 +371,15 @@ __global__ void __launch_bounds__(256) rasterize_bwd_epilogue_kernel(
 } // namespace gsx
 
 using namespace gsx;
+
+extern "C" int gsx_debug_wave_reduce16(uint32_t n_waves, const float* in, float* out, void* stream) {
+    if (n_waves == 0)
+        return GSX_OK;
+    GSX_REQUIRE(in && out, GSX_ERR_INVALID_ARGUMENT, "debug_wave_reduce16: null tensor");
+    hipLaunchKernelGGL(wave_reduce16_probe_kernel, dim3(n_waves), dim3(64), 0, (hipStream_t)stream, in, out);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
 
 extern "C" size_t gsx_rasterize_bwd_workspace_bytes(uint32_t N) { return align_up((size_t)N * kAcc * 4, 256) + 256; }
 

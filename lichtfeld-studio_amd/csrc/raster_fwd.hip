@@ -13,13 +13,7 @@ namespace gsx {
 
 static constexpr uint32_t kTile = 16;
 static constexpr uint32_t kBatch = 256;
-
-struct StagedGaussian {        // 64 bytes
-    float x, y, z, opac;       // mean, opacity
-    float m00, m01, m02, m10;  // M row-major
-    float m11, m12, m20, m21;
-    float m22, c0, c1, c2;     // colour (channels 0..2)
-};
+static constexpr float kPowerCut = -5.55f; // exp(-5.55) = 3.8875e-3 < 1/255 = 3.9216e-3
 
 // STATS: also count the (pixel, Gaussian) pairs this launch evaluates / composites (for roofline accounting);
 // stats[0] += pairs evaluated, stats[1] += pairs composited, stats[2] += pairs the backward pass will evaluate
@@ -92,10 +86,17 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
                 c1 = colors[(size_t)g * CDIM + 1];
             if (CDIM > 2)
                 c2 = colors[(size_t)g * CDIM + 2];
-            stage[tr * 4 + 0] = make_float4(xyz.x, xyz.y, xyz.z, opac);
-            stage[tr * 4 + 1] = make_float4(is0 * R.m[0][0], is0 * R.m[1][0], is0 * R.m[2][0], is1 * R.m[0][1]);
-            stage[tr * 4 + 2] = make_float4(is1 * R.m[1][1], is1 * R.m[2][1], is2 * R.m[0][2], is2 * R.m[1][2]);
-            stage[tr * 4 + 3] = make_float4(is2 * R.m[2][2], c0, c1, c2);
+            // gro = M (ray_o - mean) does not depend on the pixel (one ray origin per global-shutter camera): it is
+            // formed here, once per staged Gaussian, with the arithmetic of the per-pair formula
+            mat3 M;
+            M.m[0][0] = is0 * R.m[0][0], M.m[0][1] = is0 * R.m[1][0], M.m[0][2] = is0 * R.m[2][0];
+            M.m[1][0] = is1 * R.m[0][1], M.m[1][1] = is1 * R.m[1][1], M.m[1][2] = is1 * R.m[2][1];
+            M.m[2][0] = is2 * R.m[0][2], M.m[2][1] = is2 * R.m[1][2], M.m[2][2] = is2 * R.m[2][2];
+            const vec3 gro = mul(M, sub(ray_o, xyz));
+            stage[tr * 4 + 0] = make_float4(gro.x, gro.y, gro.z, opac);
+            stage[tr * 4 + 1] = make_float4(M.m[0][0], M.m[0][1], M.m[0][2], M.m[1][0]);
+            stage[tr * 4 + 2] = make_float4(M.m[1][1], M.m[1][2], M.m[2][0], M.m[2][1]);
+            stage[tr * 4 + 3] = make_float4(M.m[2][2], c0, c1, c2);
 #pragma unroll
             for (uint32_t k = 3; k < CDIM; ++k)
                 extra[tr * (CDIM > 3 ? CDIM - 3 : 1) + (k - 3)] = colors[(size_t)g * CDIM + k];
@@ -114,10 +115,8 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
             const float4 m0 = stage[t * 4 + 1];
             const float4 m1 = stage[t * 4 + 2];
             const float4 m2 = stage[t * 4 + 3];
-            const vec3 o = mk3(ray_o.x - a.x, ray_o.y - a.y, ray_o.z - a.z);
-            // gro = M (ray_o - xyz); grd = normalize(M ray_d)
-            const vec3 gro = mk3(fma(m0.z, o.z, fma(m0.y, o.y, m0.x * o.x)), fma(m1.y, o.z, fma(m1.x, o.y, m0.w * o.x)),
-                                 fma(m2.x, o.z, fma(m1.w, o.y, m1.z * o.x)));
+            const vec3 gro = mk3(a.x, a.y, a.z);
+            // grd = normalize(M ray_d)
             const vec3 gd = mk3(fma(m0.z, ray_d.z, fma(m0.y, ray_d.y, m0.x * ray_d.x)),
                                 fma(m1.y, ray_d.z, fma(m1.x, ray_d.y, m0.w * ray_d.x)),
                                 fma(m2.x, ray_d.z, fma(m1.w, ray_d.y, m1.z * ray_d.x)));
@@ -125,6 +124,10 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
             const vec3 gcrod = cross(grd, gro);
             const float grayDist = dot(gcrod, gcrod);
             const float power = -0.5f * grayDist;
+            // exp(power) < 1/255 below kPowerCut, so alpha < 1/255 for any opacity <= 1: decided without the exp
+            const bool far_away = power < kPowerCut && a.w <= 1.0f;
+            if (__builtin_amdgcn_ballot_w64(!far_away) == 0 || far_away)
+                continue;
             const float alpha = gsx::fmin(0.999f, a.w * gsx::exp(power));
             if (alpha < 1.f / 255.f)
                 continue;

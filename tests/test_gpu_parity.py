@@ -124,11 +124,11 @@ def test_projection_unsupported_and_errors(gsx, cuda):
     assert out[0].shape == (1, 0, 2)
 
 
-@pytest.mark.parametrize("degree", [0, 1, 2, 3, 4])
-def test_spherical_harmonics(gsx, orc, cuda, degree):
+@pytest.mark.parametrize("degree,n,K", [(0, 5000, 25), (1, 5000, 25), (2, 5000, 25), (3, 5000, 25), (4, 5000, 25),
+                                        (3, 4999, 16), (2, 70, 16), (0, 1, 16), (1, 333, 4), (0, 77, 1)])
+def test_spherical_harmonics(gsx, orc, cuda, degree, n, K):
     ops = gsx.ops
     rng = np.random.default_rng(degree)
-    n, K = 5000, 25
     dirs = rng.normal(0, 1, (n, 3)).astype(np.float32) * rng.uniform(0.1, 5, (n, 1)).astype(np.float32)
     coeffs = rng.normal(0, 0.5, (n, K, 3)).astype(np.float32)
     masks = rng.uniform(0, 1, n) < 0.8
@@ -474,3 +474,21 @@ def test_add_noise_and_quats(gsx, orc, cuda):
     bits_equal(N(md), means, '')
     R = ops.quats_to_rotmats(T(rq, cuda))
     bits_equal(N(R), orc.quats_to_rotmats(rq), '')
+
+
+def test_wave_reduce16_probe(gsx, cuda):
+    """the 64-lane x 16-value halving reduction of the backward rasterizer (permlane swaps + DPP mirrors)"""
+    import ctypes
+    L = gsx._lib
+    rng = np.random.default_rng(0)
+    nw = 37
+    x = rng.normal(0, 1, (nw, 64, 16)).astype(np.float32)
+    x[3] = np.arange(64 * 16, dtype=np.float32).reshape(64, 16)  # exact integers: any mis-routed lane shows
+    xd = T(x, cuda)
+    out = torch.zeros((nw, 16), dtype=torch.float32, device=cuda)
+    L.check(L.lib().gsx_debug_wave_reduce16(ctypes.c_uint32(nw), ctypes.c_void_p(xd.data_ptr()),
+                                            ctypes.c_void_p(out.data_ptr()), ctypes.c_void_p(None)))
+    torch.cuda.synchronize()
+    got = N(out)
+    assert np.array_equal(got[3], x[3].sum(0))
+    np.testing.assert_allclose(got, x.astype(np.float64).sum(1), rtol=0, atol=2e-5)
