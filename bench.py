@@ -128,14 +128,14 @@ def main():
     loss = [float(x) for x in ts.loss_out.cpu()]
 
     # pair counts of the last forward (for flop rates)
-    stats = torch.zeros(3, dtype=torch.int64, device=dev)
+    stats = torch.zeros(8, dtype=torch.int64, device=dev)
     L = gsx._lib
     p = lambda t: ctypes.c_void_p(t.data_ptr())
     L.check(L.lib().gsx_rasterize_pair_stats(
         ctypes.c_uint32(ts.N), ctypes.c_int64(ts.n_isects), p(ts.params["means"]), p(ts.act["quats"]),
         p(ts.act["scales"]), p(ts.act["opacities"]), ctypes.c_uint32(W), ctypes.c_uint32(H), p(viewmat), p(Kmat),
         p(ts.offsets), p(ts.flatten_ids), p(stats), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
-    pairs_fwd, pairs_comp, pairs_bwd = [int(x) for x in stats.cpu()]
+    pairs_fwd, pairs_comp, pairs_bwd = [int(x) for x in stats.cpu()[:3]]
 
     # instrumented pass: every stage bracketed by events (not part of the timed region)
     ts.start_timing(None)

@@ -133,8 +133,9 @@ GSX_API int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
     int32_t* last_ids, void* stream);
 
 /* Pair counts of one forward pass, for turning kernel times into rates (no counterpart in the reference).
- * stats_out: device uint64[3] = {pairs the forward evaluates, pairs composited, pairs the backward evaluates};
- * the counts are ADDED to it, so zero it first. */
+ * stats_out: device uint64[8] = {pairs the forward evaluates, pairs composited, pairs the backward evaluates,
+ * (wave, Gaussian) iterations of the forward, those of them with at least one lane above the alpha threshold,
+ * 3 reserved}; the counts are ADDED to it, so zero it first. */
 GSX_API int gsx_rasterize_pair_stats(uint32_t N, int64_t n_isects, const float* means, const float* quats,
                                      const float* scales, const float* opacities, uint32_t image_width,
                                      uint32_t image_height, const float* viewmat, const float* K,

@@ -1,0 +1,489 @@
+// gsplat_ops.cpp - the C++ host layer of the path: at::Tensor in / out with the validation, allocation and error
+// behaviour of LichtFeld-Studio's gsplat/*.cpp host functions (Projection.cpp:16-110, SphericalHarmonics.cpp:15-75,
+// Intersect.cpp:15-137, QuatToRotmat.cpp:14-26, Relocation.cpp:15-50, Rasterization.cpp:20-261,267-642,
+// src/training/kernels/ssim.cu:431-510, fastgs/optimizer/src/adam_api.cu:8-33), calling the gfx950 kernels through
+// the C ABI of gsx.h on torch's current stream.  Torch is used for tensors, the caching allocator and the stream.
+#include "gsplat_api.h"
+
+#include <ATen/Functions.h>
+#include <c10/core/DeviceGuard.h>
+#include <c10/hip/HIPStream.h>
+#include <c10/util/Exception.h>
+
+#include "gsx.h"
+
+namespace {
+
+// gsplat/Common.h:12-19
+#define GSX_CHECK_CUDA(x) TORCH_CHECK((x).is_cuda(), #x " must be a CUDA tensor")
+#define GSX_CHECK_CONTIGUOUS(x) TORCH_CHECK((x).is_contiguous(), #x " must be contiguous")
+#define CHECK_INPUT(x)  \
+    GSX_CHECK_CUDA(x);  \
+    GSX_CHECK_CONTIGUOUS(x)
+#define DEVICE_GUARD(t) const c10::DeviceGuard device_guard((t).device())
+
+using gsplat::OptT;
+
+inline void* cur_stream(const at::Tensor& t) { return (void*)c10::hip::getCurrentHIPStream(t.device().index()).stream(); }
+
+inline void gsx_check(int status) { TORCH_CHECK(status == GSX_OK, "gsx (", gsx_status_string(status), "): ", gsx_last_error()); }
+
+inline bool has(const OptT& t) { return t.has_value() && t->defined() && t->numel() > 0; }
+inline const float* fptr(const OptT& t) { return has(t) ? t->data_ptr<float>() : nullptr; }
+inline const uint8_t* bptr(const OptT& t) { return has(t) ? static_cast<const uint8_t*>(t->data_ptr()) : nullptr; }
+
+inline gsx_ut_params to_gsx(const UnscentedTransformParameters& p) {
+    gsx_ut_params u;
+    u.alpha = p.alpha;
+    u.beta = p.beta;
+    u.kappa = p.kappa;
+    u.in_image_margin_factor = p.in_image_margin_factor;
+    u.require_all_sigma_points_valid = p.require_all_sigma_points_valid ? 1 : 0;
+    return u;
+}
+
+inline at::Tensor workspace(size_t bytes, const at::Tensor& like) {
+    return at::empty({(int64_t)(bytes < 256 ? 256 : bytes)}, like.options().dtype(at::kByte));
+}
+
+} // namespace
+
+namespace gsplat {
+
+at::Tensor spherical_harmonics_fwd(const uint32_t degrees_to_use, const at::Tensor dirs, const at::Tensor coeffs,
+                                   const OptT masks) {
+    DEVICE_GUARD(dirs);
+    CHECK_INPUT(dirs);
+    CHECK_INPUT(coeffs);
+    if (masks.has_value()) {
+        CHECK_INPUT(masks.value());
+    }
+    TORCH_CHECK(coeffs.size(-1) == 3, "coeffs must have last dimension 3");
+    TORCH_CHECK(dirs.size(-1) == 3, "dirs must have last dimension 3");
+    at::Tensor colors = at::empty_like(dirs);
+    gsx_check(gsx_spherical_harmonics_fwd((uint32_t)(dirs.numel() / 3), (uint32_t)coeffs.size(-2), degrees_to_use,
+                                          dirs.data_ptr<float>(), coeffs.data_ptr<float>(), bptr(masks),
+                                          colors.data_ptr<float>(), cur_stream(dirs)));
+    return colors;
+}
+
+std::tuple<at::Tensor, at::Tensor> spherical_harmonics_bwd(const uint32_t K, const uint32_t degrees_to_use,
+                                                           const at::Tensor dirs, const at::Tensor coeffs,
+                                                           const OptT masks, const at::Tensor v_colors,
+                                                           bool compute_v_dirs) {
+    DEVICE_GUARD(dirs);
+    CHECK_INPUT(dirs);
+    CHECK_INPUT(coeffs);
+    CHECK_INPUT(v_colors);
+    if (masks.has_value()) {
+        CHECK_INPUT(masks.value());
+    }
+    TORCH_CHECK(v_colors.size(-1) == 3, "v_colors must have last dimension 3");
+    TORCH_CHECK(coeffs.size(-1) == 3, "coeffs must have last dimension 3");
+    TORCH_CHECK(dirs.size(-1) == 3, "dirs must have last dimension 3");
+    at::Tensor v_coeffs = at::empty_like(coeffs); // the kernel writes every element
+    at::Tensor v_dirs;
+    if (compute_v_dirs)
+        v_dirs = at::zeros_like(dirs);
+    gsx_check(gsx_spherical_harmonics_bwd((uint32_t)(dirs.numel() / 3), K, degrees_to_use, dirs.data_ptr<float>(),
+                                          coeffs.data_ptr<float>(), bptr(masks), v_colors.data_ptr<float>(),
+                                          v_coeffs.data_ptr<float>(),
+                                          compute_v_dirs ? v_dirs.data_ptr<float>() : nullptr, cur_stream(dirs)));
+    return std::make_tuple(v_coeffs, v_dirs);
+}
+
+void radix_sort_double_buffer(const int64_t n_isects, const uint32_t tile_n_bits, const uint32_t cam_n_bits,
+                              at::Tensor isect_ids, at::Tensor flatten_ids, at::Tensor isect_ids_sorted,
+                              at::Tensor flatten_ids_sorted) {
+    if (n_isects <= 0)
+        return;
+    at::Tensor ws = workspace(gsx_radix_sort_pairs_workspace_bytes(n_isects), isect_ids);
+    int selector = 0;
+    gsx_check(gsx_radix_sort_pairs(n_isects, isect_ids.data_ptr<int64_t>(), flatten_ids.data_ptr<int32_t>(),
+                                   isect_ids_sorted.data_ptr<int64_t>(), flatten_ids_sorted.data_ptr<int32_t>(),
+                                   32 + tile_n_bits + cam_n_bits, ws.data_ptr(), (size_t)ws.numel(), &selector,
+                                   cur_stream(isect_ids)));
+    if (selector == 0) { // sorted items ended up in the input buffers (IntersectTile.cu:315-328)
+        isect_ids_sorted.set_(isect_ids);
+        flatten_ids_sorted.set_(flatten_ids);
+    }
+}
+
+std::tuple<at::Tensor, at::Tensor, at::Tensor> intersect_tile(const at::Tensor means2d, const at::Tensor radii,
+                                                              const at::Tensor depths, const OptT camera_ids,
+                                                              const OptT gaussian_ids, const uint32_t C,
+                                                              const uint32_t tile_size, const uint32_t tile_width,
+                                                              const uint32_t tile_height, const bool sort) {
+    DEVICE_GUARD(means2d);
+    CHECK_INPUT(means2d);
+    CHECK_INPUT(radii);
+    CHECK_INPUT(depths);
+    const bool packed = means2d.dim() == 2;
+    if (packed) {
+        TORCH_CHECK(camera_ids.has_value() && gaussian_ids.has_value(),
+                    "When packed is set, camera_ids and gaussian_ids must be provided.");
+        TORCH_CHECK(false, "packed intersect_tile is not built (LichtFeld never uses it: rasterizer.cpp:25)");
+    }
+    const uint32_t N = (uint32_t)means2d.size(1);
+    const uint32_t tile_n_bits = gsx_n_bits(tile_width * tile_height);
+    const uint32_t cam_n_bits = gsx_n_bits(C);
+    at::Tensor tiles_per_gauss = at::empty_like(depths, depths.options().dtype(at::kInt));
+    at::Tensor cum = at::empty({(int64_t)C * N}, depths.options().dtype(at::kLong));
+    at::Tensor ws = workspace(gsx_intersect_tile_count_workspace_bytes(C, N), depths);
+    int64_t n_isects = 0;
+    void* stream = cur_stream(means2d);
+    gsx_check(gsx_intersect_tile_count(C, N, means2d.data_ptr<float>(), radii.data_ptr<int32_t>(), tile_size,
+                                       tile_width, tile_height, tiles_per_gauss.data_ptr<int32_t>(),
+                                       cum.data_ptr<int64_t>(), ws.data_ptr(), (size_t)ws.numel(), &n_isects, stream));
+    at::Tensor isect_ids = at::empty({n_isects}, depths.options().dtype(at::kLong));
+    at::Tensor flatten_ids = at::empty({n_isects}, depths.options().dtype(at::kInt));
+    if (n_isects) {
+        gsx_check(gsx_intersect_tile_emit(C, N, means2d.data_ptr<float>(), radii.data_ptr<int32_t>(),
+                                          depths.data_ptr<float>(), cum.data_ptr<int64_t>(), tile_size, tile_width,
+                                          tile_height, isect_ids.data_ptr<int64_t>(), flatten_ids.data_ptr<int32_t>(),
+                                          stream));
+    }
+    if (n_isects && sort) {
+        at::Tensor isect_ids_sorted = at::empty_like(isect_ids);
+        at::Tensor flatten_ids_sorted = at::empty_like(flatten_ids);
+        radix_sort_double_buffer(n_isects, tile_n_bits, cam_n_bits, isect_ids, flatten_ids, isect_ids_sorted,
+                                 flatten_ids_sorted);
+        return std::make_tuple(tiles_per_gauss, isect_ids_sorted, flatten_ids_sorted);
+    }
+    return std::make_tuple(tiles_per_gauss, isect_ids, flatten_ids);
+}
+
+at::Tensor intersect_offset(const at::Tensor isect_ids, const uint32_t C, const uint32_t tile_width,
+                            const uint32_t tile_height) {
+    DEVICE_GUARD(isect_ids);
+    CHECK_INPUT(isect_ids);
+    at::Tensor offsets = at::empty({C, tile_height, tile_width}, isect_ids.options().dtype(at::kInt));
+    gsx_check(gsx_intersect_offset(isect_ids.size(0), isect_ids.data_ptr<int64_t>(), C, tile_width, tile_height,
+                                   offsets.data_ptr<int32_t>(), cur_stream(isect_ids)));
+    return offsets;
+}
+
+at::Tensor quats_to_rotmats(const at::Tensor quats) {
+    DEVICE_GUARD(quats);
+    CHECK_INPUT(quats);
+    const int64_t N = quats.size(0);
+    at::Tensor rotmats = at::empty({N, 3, 3}, quats.options());
+    gsx_check(gsx_quats_to_rotmats((int)N, quats.data_ptr<float>(), rotmats.data_ptr<float>(), cur_stream(quats)));
+    return rotmats;
+}
+
+std::tuple<at::Tensor, at::Tensor> relocation(at::Tensor opacities, at::Tensor scales, at::Tensor ratios,
+                                              at::Tensor binoms, const int n_max) {
+    DEVICE_GUARD(opacities);
+    CHECK_INPUT(opacities);
+    CHECK_INPUT(scales);
+    CHECK_INPUT(ratios);
+    CHECK_INPUT(binoms);
+    at::Tensor new_opacities = at::empty_like(opacities);
+    at::Tensor new_scales = at::empty_like(scales);
+    gsx_check(gsx_relocation((int)opacities.size(0), opacities.data_ptr<float>(), scales.data_ptr<float>(),
+                             ratios.data_ptr<int32_t>(), binoms.data_ptr<float>(), n_max,
+                             new_opacities.data_ptr<float>(), new_scales.data_ptr<float>(), cur_stream(opacities)));
+    return std::make_tuple(new_opacities, new_scales);
+}
+
+void add_noise(at::Tensor raw_opacities, at::Tensor raw_scales, at::Tensor raw_quats, at::Tensor noise,
+               at::Tensor means, const float current_lr) {
+    DEVICE_GUARD(raw_opacities);
+    CHECK_INPUT(raw_opacities);
+    CHECK_INPUT(raw_scales);
+    CHECK_INPUT(raw_quats);
+    CHECK_INPUT(noise);
+    CHECK_INPUT(means);
+    gsx_check(gsx_add_noise((int)raw_opacities.size(0), raw_opacities.data_ptr<float>(), raw_scales.data_ptr<float>(),
+                            raw_quats.data_ptr<float>(), noise.data_ptr<float>(), means.data_ptr<float>(), current_lr,
+                            cur_stream(means)));
+}
+
+std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> projection_ut_3dgs_fused(
+    const at::Tensor means, const at::Tensor quats, const at::Tensor scales, const OptT opacities,
+    const at::Tensor viewmats0, const OptT viewmats1, const at::Tensor Ks, const uint32_t image_width,
+    const uint32_t image_height, const float eps2d, const float near_plane, const float far_plane,
+    const float radius_clip, const bool calc_compensations, const CameraModelType camera_model,
+    const UnscentedTransformParameters ut_params, ShutterType rs_type, const OptT radial_coeffs,
+    const OptT tangential_coeffs, const OptT thin_prism_coeffs) {
+    DEVICE_GUARD(means);
+    CHECK_INPUT(means);
+    CHECK_INPUT(quats);
+    CHECK_INPUT(scales);
+    if (opacities.has_value()) {
+        CHECK_INPUT(opacities.value());
+    }
+    CHECK_INPUT(viewmats0);
+    if (viewmats1.has_value()) {
+        CHECK_INPUT(viewmats1.value());
+    }
+    CHECK_INPUT(Ks);
+    if (radial_coeffs.has_value()) {
+        CHECK_INPUT(radial_coeffs.value());
+    }
+    if (tangential_coeffs.has_value()) {
+        CHECK_INPUT(tangential_coeffs.value());
+    }
+    if (thin_prism_coeffs.has_value()) {
+        CHECK_INPUT(thin_prism_coeffs.value());
+    }
+    const uint32_t N = (uint32_t)means.size(0), C = (uint32_t)viewmats0.size(0);
+    auto opt = means.options();
+    at::Tensor radii = at::empty({C, N, 2}, opt.dtype(at::kInt));
+    at::Tensor means2d = at::empty({C, N, 2}, opt);
+    at::Tensor depths = at::empty({C, N}, opt);
+    at::Tensor conics = at::empty({C, N, 3}, opt);
+    at::Tensor compensations;
+    if (calc_compensations)
+        compensations = at::zeros({C, N}, opt); // Projection.cpp:77
+    gsx_check(gsx_projection_ut_3dgs_fused(
+        C, N, means.data_ptr<float>(), quats.data_ptr<float>(), scales.data_ptr<float>(), fptr(opacities),
+        viewmats0.data_ptr<float>(), fptr(viewmats1), Ks.data_ptr<float>(), image_width, image_height, eps2d,
+        near_plane, far_plane, radius_clip, (int)camera_model, to_gsx(ut_params), (int)rs_type, fptr(radial_coeffs),
+        fptr(tangential_coeffs), fptr(thin_prism_coeffs), radii.data_ptr<int32_t>(), means2d.data_ptr<float>(),
+        depths.data_ptr<float>(), conics.data_ptr<float>(),
+        calc_compensations ? compensations.data_ptr<float>() : nullptr, cur_stream(means)));
+    return std::make_tuple(radii, means2d, depths, conics, compensations);
+}
+
+std::tuple<at::Tensor, at::Tensor, at::Tensor> rasterize_to_pixels_from_world_3dgs_fwd(
+    const at::Tensor means, const at::Tensor quats, const at::Tensor scales, const at::Tensor colors,
+    const at::Tensor opacities, const OptT backgrounds, const OptT masks, const uint32_t image_width,
+    const uint32_t image_height, const uint32_t tile_size, const at::Tensor viewmats0, const OptT viewmats1,
+    const at::Tensor Ks, const CameraModelType camera_model, const UnscentedTransformParameters ut_params,
+    ShutterType rs_type, const OptT radial_coeffs, const OptT tangential_coeffs, const OptT thin_prism_coeffs,
+    const at::Tensor tile_offsets, const at::Tensor flatten_ids) {
+    DEVICE_GUARD(means);
+    CHECK_INPUT(means);
+    CHECK_INPUT(quats);
+    CHECK_INPUT(scales);
+    CHECK_INPUT(colors);
+    CHECK_INPUT(opacities);
+    CHECK_INPUT(tile_offsets);
+    CHECK_INPUT(flatten_ids);
+    if (has(backgrounds)) {
+        CHECK_INPUT(backgrounds.value());
+    }
+    if (masks.has_value()) {
+        CHECK_INPUT(masks.value());
+    }
+    const uint32_t C = (uint32_t)tile_offsets.size(0), N = (uint32_t)means.size(0);
+    const uint32_t channels = (uint32_t)colors.size(-1);
+    auto opt = means.options();
+    at::Tensor renders = at::empty({C, image_height, image_width, channels}, opt);
+    at::Tensor alphas = at::empty({C, image_height, image_width, 1}, opt);
+    at::Tensor last_ids = at::empty({C, image_height, image_width}, opt.dtype(at::kInt));
+    const int st = gsx_rasterize_to_pixels_from_world_3dgs_fwd(
+        C, N, flatten_ids.size(0), means.data_ptr<float>(), quats.data_ptr<float>(), scales.data_ptr<float>(),
+        colors.data_ptr<float>(), channels, opacities.data_ptr<float>(), fptr(backgrounds), bptr(masks), image_width,
+        image_height, tile_size, viewmats0.data_ptr<float>(), fptr(viewmats1), Ks.data_ptr<float>(), (int)camera_model,
+        to_gsx(ut_params), (int)rs_type, fptr(radial_coeffs), fptr(tangential_coeffs), fptr(thin_prism_coeffs),
+        tile_offsets.data_ptr<int32_t>(), flatten_ids.data_ptr<int32_t>(), renders.data_ptr<float>(),
+        alphas.data_ptr<float>(), last_ids.data_ptr<int32_t>(), cur_stream(means));
+    TORCH_CHECK(st != GSX_ERR_UNSUPPORTED || (channels == 1 || channels == 3 || channels == 4),
+                "Unsupported number of channels: ", channels); // Rasterization.cpp:126-127
+    gsx_check(st);
+    return std::make_tuple(renders, alphas, last_ids);
+}
+
+std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> rasterize_to_pixels_from_world_3dgs_bwd(
+    const at::Tensor means, const at::Tensor quats, const at::Tensor scales, const at::Tensor colors,
+    const at::Tensor opacities, const OptT backgrounds, const OptT masks, const uint32_t image_width,
+    const uint32_t image_height, const uint32_t tile_size, const at::Tensor viewmats0, const OptT viewmats1,
+    const at::Tensor Ks, const CameraModelType camera_model, const UnscentedTransformParameters ut_params,
+    ShutterType rs_type, const OptT radial_coeffs, const OptT tangential_coeffs, const OptT thin_prism_coeffs,
+    const at::Tensor tile_offsets, const at::Tensor flatten_ids, const at::Tensor render_alphas,
+    const at::Tensor last_ids, const at::Tensor v_render_colors, const at::Tensor v_render_alphas) {
+    DEVICE_GUARD(means);
+    CHECK_INPUT(means);
+    CHECK_INPUT(quats);
+    CHECK_INPUT(scales);
+    CHECK_INPUT(colors);
+    CHECK_INPUT(opacities);
+    CHECK_INPUT(tile_offsets);
+    CHECK_INPUT(flatten_ids);
+    CHECK_INPUT(render_alphas);
+    CHECK_INPUT(last_ids);
+    CHECK_INPUT(v_render_colors);
+    CHECK_INPUT(v_render_alphas);
+    if (has(backgrounds)) {
+        CHECK_INPUT(backgrounds.value());
+    }
+    if (masks.has_value()) {
+        CHECK_INPUT(masks.value());
+    }
+    TORCH_CHECK(colors.size(-1) == 3, "Unsupported number of channels: ", colors.size(-1)); // Rasterization.cpp:65
+    const uint32_t C = (uint32_t)tile_offsets.size(0), N = (uint32_t)means.size(0);
+    // the kernels write every element of the five outputs (the reference zero-fills, Rasterization.cpp:190-194)
+    at::Tensor v_means = at::empty_like(means), v_quats = at::empty_like(quats), v_scales = at::empty_like(scales);
+    at::Tensor v_colors = at::empty_like(colors), v_opacities = at::empty_like(opacities);
+    at::Tensor ws = workspace(gsx_rasterize_bwd_workspace_bytes(N), means);
+    gsx_check(gsx_rasterize_to_pixels_from_world_3dgs_bwd(
+        C, N, flatten_ids.size(0), means.data_ptr<float>(), quats.data_ptr<float>(), scales.data_ptr<float>(),
+        colors.data_ptr<float>(), opacities.data_ptr<float>(), fptr(backgrounds), bptr(masks), image_width,
+        image_height, tile_size, viewmats0.data_ptr<float>(), fptr(viewmats1), Ks.data_ptr<float>(), (int)camera_model,
+        to_gsx(ut_params), (int)rs_type, fptr(radial_coeffs), fptr(tangential_coeffs), fptr(thin_prism_coeffs),
+        tile_offsets.data_ptr<int32_t>(), flatten_ids.data_ptr<int32_t>(), render_alphas.data_ptr<float>(),
+        last_ids.data_ptr<int32_t>(), v_render_colors.data_ptr<float>(), v_render_alphas.data_ptr<float>(),
+        v_means.data_ptr<float>(), v_quats.data_ptr<float>(), v_scales.data_ptr<float>(), v_colors.data_ptr<float>(),
+        v_opacities.data_ptr<float>(), ws.data_ptr(), (size_t)ws.numel(), cur_stream(means)));
+    return std::make_tuple(v_means, v_quats, v_scales, v_colors, v_opacities);
+}
+
+std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor,
+           at::Tensor>
+rasterize_from_world_with_sh_fwd(const at::Tensor means, const at::Tensor quats, const at::Tensor scales,
+                                 const at::Tensor opacities, const at::Tensor sh_coeffs, const uint32_t sh_degree,
+                                 const OptT backgrounds, const OptT masks, const uint32_t image_width,
+                                 const uint32_t image_height, const uint32_t tile_size, const at::Tensor viewmats0,
+                                 const OptT viewmats1, const at::Tensor Ks, const CameraModelType camera_model,
+                                 const float eps2d, const float near_plane, const float far_plane,
+                                 const float radius_clip, const float scaling_modifier, const bool calc_compensations,
+                                 const int render_mode, const UnscentedTransformParameters ut_params,
+                                 ShutterType rs_type, const OptT radial_coeffs, const OptT tangential_coeffs,
+                                 const OptT thin_prism_coeffs) {
+    DEVICE_GUARD(means);
+    CHECK_INPUT(means);
+    CHECK_INPUT(quats);
+    CHECK_INPUT(scales);
+    CHECK_INPUT(opacities);
+    CHECK_INPUT(sh_coeffs);
+    CHECK_INPUT(viewmats0);
+    CHECK_INPUT(Ks);
+    TORCH_CHECK(render_mode == 0, "render_mode ", render_mode, ": only RGB (0) is built");
+    const uint32_t N = (uint32_t)means.size(0), C = (uint32_t)viewmats0.size(0);
+    at::Tensor op_flat = opacities.reshape({-1});
+    at::Tensor scaled_scales = scaling_modifier == 1.0f ? scales : at::mul(scales, scaling_modifier); // Rasterization.cpp:327
+    auto proj = projection_ut_3dgs_fused(means, quats, scaled_scales, op_flat, viewmats0, viewmats1, Ks, image_width,
+                                         image_height, eps2d, near_plane, far_plane, radius_clip, calc_compensations,
+                                         camera_model, ut_params, rs_type, radial_coeffs, tangential_coeffs,
+                                         thin_prism_coeffs);
+    at::Tensor radii = std::get<0>(proj), means2d = std::get<1>(proj), depths = std::get<2>(proj);
+    at::Tensor compensations = std::get<4>(proj);
+    // Rasterization.cpp:356-378 in one pass: dirs, radii mask, SH, + 0.5, clamp
+    at::Tensor colors = at::empty({C, N, 3}, means.options());
+    gsx_check(gsx_sh_colors_from_world(N, (uint32_t)sh_coeffs.size(1), sh_degree, means.data_ptr<float>(),
+                                       sh_coeffs.data_ptr<float>(), radii.data_ptr<int32_t>(),
+                                       viewmats0.data_ptr<float>(), colors.data_ptr<float>(), cur_stream(means)));
+    at::Tensor final_opacities = op_flat.unsqueeze(0);
+    if (calc_compensations && compensations.defined() && compensations.numel() > 0)
+        final_opacities = at::mul(final_opacities, compensations).contiguous();
+    const uint32_t tile_width = (image_width + tile_size - 1) / tile_size;
+    const uint32_t tile_height = (image_height + tile_size - 1) / tile_size;
+    auto isect = intersect_tile(means2d, radii, depths, at::nullopt, at::nullopt, C, tile_size, tile_width, tile_height,
+                                true);
+    at::Tensor flatten_ids = std::get<2>(isect);
+    at::Tensor offsets = intersect_offset(std::get<1>(isect), C, tile_width, tile_height);
+    auto r = rasterize_to_pixels_from_world_3dgs_fwd(means, quats, scaled_scales, colors, final_opacities.contiguous(),
+                                                     backgrounds, masks, image_width, image_height, tile_size,
+                                                     viewmats0, viewmats1, Ks, camera_model, ut_params, rs_type,
+                                                     radial_coeffs, tangential_coeffs, thin_prism_coeffs, offsets,
+                                                     flatten_ids);
+    return std::make_tuple(std::get<0>(r), std::get<1>(r), radii, means2d, depths, colors, offsets, flatten_ids,
+                           std::get<2>(r), compensations);
+}
+
+std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> rasterize_from_world_with_sh_bwd(
+    const at::Tensor means, const at::Tensor quats, const at::Tensor scales, const at::Tensor opacities,
+    const at::Tensor sh_coeffs, const uint32_t sh_degree, const OptT backgrounds, const OptT masks,
+    const uint32_t image_width, const uint32_t image_height, const uint32_t tile_size, const at::Tensor viewmats0,
+    const OptT viewmats1, const at::Tensor Ks, const CameraModelType camera_model, const float eps2d,
+    const float near_plane, const float far_plane, const float radius_clip, const float scaling_modifier,
+    const bool calc_compensations, const int render_mode, const UnscentedTransformParameters ut_params,
+    ShutterType rs_type, const OptT radial_coeffs, const OptT tangential_coeffs, const OptT thin_prism_coeffs,
+    const at::Tensor render_alphas, const at::Tensor last_ids, const at::Tensor tile_offsets,
+    const at::Tensor flatten_ids, const at::Tensor colors, const at::Tensor radii, const at::Tensor means2d,
+    const at::Tensor depths, const at::Tensor compensations, const at::Tensor v_render_colors,
+    const at::Tensor v_render_alphas) {
+    (void)eps2d, (void)near_plane, (void)far_plane, (void)radius_clip, (void)means2d, (void)depths;
+    DEVICE_GUARD(means);
+    CHECK_INPUT(means);
+    CHECK_INPUT(quats);
+    CHECK_INPUT(scales);
+    CHECK_INPUT(opacities);
+    CHECK_INPUT(sh_coeffs);
+    CHECK_INPUT(v_render_colors);
+    CHECK_INPUT(v_render_alphas);
+    TORCH_CHECK(render_mode == 0, "render_mode ", render_mode, ": only RGB (0) is built");
+    at::Tensor final_opacities = opacities.reshape({1, -1});
+    if (calc_compensations && compensations.defined() && compensations.numel() > 0)
+        final_opacities = at::mul(final_opacities, compensations).contiguous();
+    at::Tensor scaled_scales = scaling_modifier == 1.0f ? scales : at::mul(scales, scaling_modifier);
+    auto g = rasterize_to_pixels_from_world_3dgs_bwd(means, quats, scaled_scales, colors, final_opacities.contiguous(),
+                                                     backgrounds, masks, image_width, image_height, tile_size,
+                                                     viewmats0, viewmats1, Ks, camera_model, ut_params, rs_type,
+                                                     radial_coeffs, tangential_coeffs, thin_prism_coeffs, tile_offsets,
+                                                     flatten_ids, render_alphas, last_ids, v_render_colors,
+                                                     v_render_alphas);
+    at::Tensor v_sh = at::empty_like(sh_coeffs);
+    gsx_check(gsx_sh_colors_from_world_bwd((uint32_t)means.size(0), (uint32_t)sh_coeffs.size(1), sh_degree,
+                                           means.data_ptr<float>(), radii.data_ptr<int32_t>(),
+                                           viewmats0.data_ptr<float>(), colors.data_ptr<float>(),
+                                           std::get<3>(g).data_ptr<float>(), v_sh.data_ptr<float>(), cur_stream(means)));
+    at::Tensor v_scales = std::get<2>(g);
+    if (scaling_modifier != 1.0f)
+        v_scales = at::mul(v_scales, scaling_modifier); // Rasterization.cpp:633
+    return std::make_tuple(std::get<0>(g), std::get<1>(g), v_scales, std::get<4>(g), v_sh);
+}
+
+} // namespace gsplat
+
+// src/training/kernels/ssim.cu:431-468
+std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor> fusedssim(float C1, float C2, at::Tensor& img1,
+                                                                     at::Tensor& img2, bool train) {
+    const c10::DeviceGuard device_guard(img1.device());
+    const int B = (int)img1.size(0), CH = (int)img1.size(1), H = (int)img1.size(2), W = (int)img1.size(3);
+    at::Tensor a = img1.contiguous(), b = img2.contiguous();
+    at::Tensor ssim_map = at::empty_like(a);
+    at::Tensor d1 = train ? at::empty_like(a) : at::empty({0}, a.options());
+    at::Tensor d2 = train ? at::empty_like(a) : at::empty({0}, a.options());
+    at::Tensor d3 = train ? at::empty_like(a) : at::empty({0}, a.options());
+    gsx_check(gsx_fusedssim(B, CH, H, W, C1, C2, a.data_ptr<float>(), b.data_ptr<float>(), ssim_map.data_ptr<float>(),
+                            train ? d1.data_ptr<float>() : nullptr, train ? d2.data_ptr<float>() : nullptr,
+                            train ? d3.data_ptr<float>() : nullptr, cur_stream(a)));
+    return std::make_tuple(ssim_map, d1, d2, d3);
+}
+
+// src/training/kernels/ssim.cu:476-510
+at::Tensor fusedssim_backward(float C1, float C2, at::Tensor& img1, at::Tensor& img2, at::Tensor& dL_dmap,
+                              at::Tensor& dm_dmu1, at::Tensor& dm_dsigma1_sq, at::Tensor& dm_dsigma12) {
+    const c10::DeviceGuard device_guard(img1.device());
+    const int B = (int)img1.size(0), CH = (int)img1.size(1), H = (int)img1.size(2), W = (int)img1.size(3);
+    at::Tensor a = img1.contiguous(), b = img2.contiguous(), g = dL_dmap.contiguous();
+    at::Tensor d1 = dm_dmu1.contiguous(), d2 = dm_dsigma1_sq.contiguous(), d3 = dm_dsigma12.contiguous();
+    at::Tensor out = at::empty_like(a);
+    gsx_check(gsx_fusedssim_backward(B, CH, H, W, C1, C2, a.data_ptr<float>(), b.data_ptr<float>(), g.data_ptr<float>(),
+                                     d1.data_ptr<float>(), d2.data_ptr<float>(), d3.data_ptr<float>(),
+                                     out.data_ptr<float>(), cur_stream(a)));
+    return out;
+}
+
+// value of fused_ssim(img1, img2, padding) (include/kernels/fused_ssim.cuh:117-122), no autograd node
+at::Tensor fused_ssim_value(at::Tensor img1, at::Tensor img2, const std::string& padding) {
+    TORCH_CHECK(padding == "same" || padding == "valid", "fused_ssim: padding must be \"same\" or \"valid\" (got \"",
+                padding, "\")");
+    if (img1.dim() == 3)
+        img1 = img1.unsqueeze(0);
+    if (img2.dim() == 3)
+        img2 = img2.unsqueeze(0);
+    TORCH_CHECK(img1.dim() == 4 && img2.dim() == 4, "fused_ssim expects 4D tensors [N,C,H,W]");
+    TORCH_CHECK(img1.sizes() == img2.sizes(), "img1 and img2 must have the same shape");
+    img1 = img1.contiguous();
+    img2 = img2.contiguous();
+    at::Tensor map = std::get<0>(fusedssim(0.01f * 0.01f, 0.03f * 0.03f, img1, img2, false));
+    const int64_t h = map.size(2), w = map.size(3);
+    if (padding == "valid" && h > 10 && w > 10)
+        map = map.slice(2, 5, h - 5).slice(3, 5, w - 5);
+    return map.mean();
+}
+
+void fast_gs::optimizer::adam_step_wrapper(at::Tensor& param, at::Tensor& exp_avg, at::Tensor& exp_avg_sq,
+                                           const at::Tensor& param_grad, const float lr, const float beta1,
+                                           const float beta2, const float eps, const float bias_correction1_rcp,
+                                           const float bias_correction2_sqrt_rcp) {
+    const c10::DeviceGuard device_guard(param.device());
+    gsx_check(gsx_adam_step(param.data_ptr<float>(), exp_avg.data_ptr<float>(), exp_avg_sq.data_ptr<float>(),
+                            param_grad.data_ptr<float>(), param.numel(), lr, beta1, beta2, eps, bias_correction1_rcp,
+                            bias_correction2_sqrt_rcp, cur_stream(param)));
+}

@@ -126,6 +126,15 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
             const float power = -0.5f * grayDist;
             // exp(power) < 1/255 below kPowerCut, so alpha < 1/255 for any opacity <= 1: decided without the exp
             const bool far_away = power < kPowerCut && a.w <= 1.0f;
+            if (STATS) {
+                const uint64_t act = __builtin_amdgcn_ballot_w64(true);
+                const uint64_t nearm = __builtin_amdgcn_ballot_w64(!far_away);
+                if ((act & ((1ull << (threadIdx.x & 63u)) - 1ull)) == 0) { // first active lane of the wave
+                    atomicAdd(&stats[3], 1ull);
+                    if (nearm)
+                        atomicAdd(&stats[4], 1ull);
+                }
+            }
             if (__builtin_amdgcn_ballot_w64(!far_away) == 0 || far_away)
                 continue;
             const float alpha = gsx::fmin(0.999f, a.w * gsx::exp(power));

@@ -46,3 +46,14 @@ def cuda():
         pytest.skip("no GPU")
     load_package()._lib.lib()  # fail loudly if libgsx.so is missing
     return torch.device("cuda:0")
+
+
+@pytest.fixture(scope="session")
+def cpp():
+    """gsx_torch_ext: the pybind11 module over the C++ host layer (csrc/host/gsplat_ops.cpp), built in-tree by
+    build_ext.py.  Missing build = failure, not skip."""
+    import torch  # noqa: F401  (libtorch must be loaded first)
+    if PKG_DIR not in sys.path:
+        sys.path.insert(0, PKG_DIR)
+    import gsx_torch_ext
+    return gsx_torch_ext

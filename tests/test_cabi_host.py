@@ -93,6 +93,29 @@ def test_python_mirror_rejects_what_check_input_rejects(gsx):
         ops.intersect_offset(np.zeros(3, np.int64), 1, 4, 4)
 
 
+def test_cpp_host_layer_loads_and_checks_inputs(cpp):
+    """the C++ functions with gsplat/Ops.h's names exist and apply CHECK_INPUT (gsplat/Common.h:12-19) before
+    anything touches a GPU"""
+    torch = pytest.importorskip("torch")
+    for name in ("spherical_harmonics_fwd", "spherical_harmonics_bwd", "intersect_tile", "intersect_offset",
+                 "quats_to_rotmats", "relocation", "add_noise", "projection_ut_3dgs_fused",
+                 "rasterize_to_pixels_from_world_3dgs_fwd", "rasterize_to_pixels_from_world_3dgs_bwd",
+                 "rasterize_from_world_with_sh_fwd", "rasterize_from_world_with_sh_bwd", "fusedssim",
+                 "fusedssim_backward", "adam_step_wrapper"):
+        assert callable(getattr(cpp, name)), name
+    ut = cpp.UnscentedTransformParameters()
+    assert (ut.alpha, ut.beta, ut.kappa, ut.require_all_sigma_points_valid) == (pytest.approx(0.1), 2.0, 0.0, True)
+    assert int(cpp.ShutterType.GLOBAL) == 4 and int(cpp.CameraModelType.PINHOLE) == 0
+    with pytest.raises(RuntimeError, match="quats must be a CUDA tensor"):
+        cpp.quats_to_rotmats(torch.zeros((4, 4)))
+    with pytest.raises(RuntimeError, match="dirs must be a CUDA tensor"):
+        cpp.spherical_harmonics_fwd(3, torch.zeros((4, 3)), torch.zeros((4, 16, 3)), None)
+    with pytest.raises(RuntimeError, match="opacities must be a CUDA tensor"):
+        cpp.relocation(torch.zeros(4), torch.zeros((4, 3)), torch.ones(4, dtype=torch.int32), torch.zeros((51, 51)), 51)
+    with pytest.raises(RuntimeError, match="padding"):
+        cpp.fused_ssim_value(torch.zeros((1, 3, 16, 16)), torch.zeros((1, 3, 16, 16)), "reflect")
+
+
 def test_scene_generator_is_deterministic(gsx):
     a, b = gsx.scenes.config(3, 1000), gsx.scenes.config(3, 1000)
     for k, v in a.params().items():
