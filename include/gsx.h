@@ -216,6 +216,26 @@ GSX_API int gsx_adam_step_multi(const gsx_adam_group* groups_host, int n_groups,
 /* ---- a12: gsplat::relocation (Ops.h:52-57; RelocationCUDA.cu:11-43) ---- */
 GSX_API int gsx_relocation(int M, const float* opacities, const float* scales, const int32_t* ratios,
                            const float* binoms, int n_max, float* new_opacities, float* new_scales, void* stream);
+/* ---- a12 caller glue: MCMC::relocate_gs once the dead and the sampled index sets are chosen (mcmc.cpp:141-187;
+ * the multinomial draw of :132 stays with the caller, random streams cannot be reproduced across libraries) ----
+ *   ratios[i]      = min(1 + #{j : sampled[j] == sampled[i]}, n_max)                               (:141-148)
+ *   new_o, new_s   = relocation(sigmoid(opacity_raw[s]), exp(scaling_raw[s]), ratios)               (:151-156)
+ *   opacity_raw[s] = logit(clamp(new_o, min_opacity, 1 - 1e-7)),  scaling_raw[s] = log(new_s)       (:160-171)
+ *   parameter rows:        row[dead[i]] = row[sampled[i]]  for every tensor with is_optimizer_state == 0  (:175-180)
+ *   optimiser-state rows:  row[sampled[i]] = 0             for every tensor with is_optimizer_state != 0  (:100-104)
+ * sampled_idxs / dead_idxs: i64 [n_idx], disjoint sets, values < N.  opacity_raw [N] and scaling_raw [N,3] must ALSO
+ * be listed in tensors_host to have their rows copied to the dead indices. */
+#define GSX_MCMC_MAX_TENSORS 24
+typedef struct gsx_row_tensor {
+    float* data;         /* [N, row_floats] */
+    uint32_t row_floats; /* floats per Gaussian */
+    int32_t is_optimizer_state;
+} gsx_row_tensor;
+GSX_API size_t gsx_mcmc_relocate_workspace_bytes(uint32_t N, uint32_t n_idx);
+GSX_API int gsx_mcmc_relocate(uint32_t N, uint32_t n_idx, const int64_t* sampled_idxs, const int64_t* dead_idxs,
+                              const float* binoms, int n_max, float min_opacity, float* opacity_raw,
+                              float* scaling_raw, const gsx_row_tensor* tensors_host, int n_tensors, void* workspace,
+                              size_t workspace_bytes, void* stream);
 /* ---- a13: gsplat::add_noise (Ops.h:59-65; RelocationCUDA.cu:112-144); means updated in place ---- */
 GSX_API int gsx_add_noise(int N, const float* raw_opacities, const float* raw_scales, const float* raw_quats,
                           const float* noise, float* means, float current_lr, void* stream);

@@ -45,6 +45,11 @@ class AdamGroup(ctypes.Structure):
                 ("skip2", ctypes.c_int32)]
 
 
+class RowTensor(ctypes.Structure):
+    """gsx_row_tensor"""
+    _fields_ = [("data", c_p), ("row_floats", c_u32), ("is_optimizer_state", ctypes.c_int32)]
+
+
 class GsxError(RuntimeError):
     def __init__(self, status, message):
         super().__init__(f"gsx status {status}: {message}")
@@ -68,7 +73,7 @@ def lib():
         L.gsx_image_loss_blocks.restype = c_u32
         L.gsx_ut_defaults.restype = UTParams
         for name in ("gsx_intersect_tile_count_workspace_bytes", "gsx_radix_sort_pairs_workspace_bytes",
-                     "gsx_rasterize_bwd_workspace_bytes"):
+                     "gsx_rasterize_bwd_workspace_bytes", "gsx_mcmc_relocate_workspace_bytes"):
             getattr(L, name).restype = c_sz
         _lib = L
     return _lib

@@ -1,7 +1,24 @@
 // relocation.hip - MCMC relocation (Eq. 9) and noise injection (gsplat/RelocationCUDA.cu:11-43, 88-144).
 #include "gsx_common.h"
 
+#include <string.h>
+
 namespace gsx {
+
+// Eq. 9 for one Gaussian: opacity and scale factor after splitting it into n copies (RelocationCUDA.cu:25-42)
+__device__ __forceinline__ void relocate_one(float op, int n_idx, const float* __restrict__ binoms, int n_max,
+                                             float& new_o, float& coeff) {
+    float denom_sum = 0.0f;
+    new_o = 1.0f - gsx::pow(1.0f - op, 1.0f / (float)n_idx);
+    for (int i = 1; i <= n_idx; ++i)
+        for (int k = 0; k <= (i - 1); ++k) {
+            const float bin_coeff = binoms[(i - 1) * n_max + k];
+            const float sgn = (k & 1) ? -1.0f : 1.0f;
+            const float term = (sgn / gsx::sqrt((float)(k + 1))) * gsx::pow(new_o, (float)(k + 1));
+            denom_sum += (bin_coeff * term);
+        }
+    coeff = (op / denom_sum);
+}
 
 __global__ void __launch_bounds__(256) relocation_kernel(int M, const float* __restrict__ opacities,
                                                           const float* __restrict__ scales,
@@ -12,22 +29,85 @@ __global__ void __launch_bounds__(256) relocation_kernel(int M, const float* __r
     const int idx = blockIdx.x * 256 + threadIdx.x;
     if (idx >= M)
         return;
-    const int n_idx = ratios[idx];
-    const float op = opacities[idx];
-    float denom_sum = 0.0f;
-    const float new_o = 1.0f - gsx::pow(1.0f - op, 1.0f / (float)n_idx);
+    float new_o, coeff;
+    relocate_one(opacities[idx], ratios[idx], binoms, n_max, new_o, coeff);
     new_opacities[idx] = new_o;
-    for (int i = 1; i <= n_idx; ++i)
-        for (int k = 0; k <= (i - 1); ++k) {
-            const float bin_coeff = binoms[(i - 1) * n_max + k];
-            const float sgn = (k & 1) ? -1.0f : 1.0f;
-            const float term = (sgn / gsx::sqrt((float)(k + 1))) * gsx::pow(new_o, (float)(k + 1));
-            denom_sum += (bin_coeff * term);
-        }
-    const float coeff = (op / denom_sum);
 #pragma unroll
     for (int i = 0; i < 3; ++i)
         new_scales[idx * 3 + i] = coeff * scales[idx * 3 + i];
+}
+
+// ---- MCMC::relocate_gs after the index sets are chosen (mcmc.cpp:141-187) ----
+// pass 0 / 1: occurrences of each sampled index (ratios = 1 + count, mcmc.cpp:141-144)
+__global__ void __launch_bounds__(256) mcmc_count_kernel(uint32_t n, const int64_t* __restrict__ sampled,
+                                                          int32_t* __restrict__ counts, int add) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n)
+        return;
+    if (add)
+        atomicAdd(&counts[sampled[i]], 1);
+    else
+        counts[sampled[i]] = 0;
+}
+
+// pass 2: new opacity / scales of every sampled Gaussian from its CURRENT raw parameters (:136-160); results go to
+// scratch so that no thread reads a row that another one has already rewritten
+__global__ void __launch_bounds__(256) mcmc_relocate_compute_kernel(
+    uint32_t n, const int64_t* __restrict__ sampled, const int32_t* __restrict__ counts,
+    const float* __restrict__ opacity_raw, const float* __restrict__ scaling_raw, const float* __restrict__ binoms,
+    int n_max, float min_opacity, float* __restrict__ new_opacity_raw, float* __restrict__ new_scaling_raw) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n)
+        return;
+    const int64_t s = sampled[i];
+    const int ratio = min(1 + counts[s], n_max); // :147-148
+    const float op = gsx::sigmoid(opacity_raw[s]);
+    float new_o, coeff;
+    relocate_one(op, ratio, binoms, n_max, new_o, coeff);
+    new_o = gsx::fmin(gsx::fmax(new_o, min_opacity), 1.0f - 1e-7f); // :160
+    new_opacity_raw[i] = gsx::log(new_o / (1.0f - new_o));           // torch::logit, :165-169
+#pragma unroll
+    for (int a = 0; a < 3; ++a)
+        new_scaling_raw[i * 3 + a] = gsx::log(coeff * gsx::exp(scaling_raw[s * 3 + a])); // :171
+}
+
+__global__ void __launch_bounds__(256) mcmc_relocate_store_kernel(uint32_t n, const int64_t* __restrict__ sampled,
+                                                                   const float* __restrict__ new_opacity_raw,
+                                                                   const float* __restrict__ new_scaling_raw,
+                                                                   float* __restrict__ opacity_raw,
+                                                                   float* __restrict__ scaling_raw) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n)
+        return;
+    const int64_t s = sampled[i]; // duplicates of one index carry identical values
+    opacity_raw[s] = new_opacity_raw[i];
+#pragma unroll
+    for (int a = 0; a < 3; ++a)
+        scaling_raw[s * 3 + a] = new_scaling_raw[i * 3 + a];
+}
+
+struct RowTable {
+    float* data[GSX_MCMC_MAX_TENSORS];
+    uint32_t row_floats[GSX_MCMC_MAX_TENSORS];
+    uint32_t is_state[GSX_MCMC_MAX_TENSORS];
+};
+
+// pass 4: parameter rows dead[i] <- sampled[i] (:175-180); optimiser-state rows of sampled[i] <- 0 (:100-104).
+// blockIdx.y = tensor; one thread per (i, float of the row)
+__global__ void __launch_bounds__(256) mcmc_rows_kernel(uint32_t n, const int64_t* __restrict__ sampled,
+                                                         const int64_t* __restrict__ dead, RowTable tab) {
+    const uint32_t e = blockIdx.y;
+    const uint32_t r = tab.row_floats[e];
+    const uint64_t t = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= (uint64_t)n * r)
+        return;
+    const uint32_t i = (uint32_t)(t / r), f = (uint32_t)(t % r);
+    float* __restrict__ p = tab.data[e];
+    const int64_t s = sampled[i];
+    if (tab.is_state[e])
+        p[s * r + f] = 0.f;
+    else
+        p[dead[i] * r + f] = p[s * r + f];
 }
 
 __global__ void __launch_bounds__(256) add_noise_kernel(int N, const float* __restrict__ raw_opacities,
@@ -85,6 +165,59 @@ extern "C" int gsx_add_noise(int N, const float* raw_opacities, const float* raw
                 "add_noise: null tensor");
     hipLaunchKernelGGL(add_noise_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, raw_opacities,
                        raw_scales, raw_quats, noise, means, current_lr);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+extern "C" size_t gsx_mcmc_relocate_workspace_bytes(uint32_t N, uint32_t n_idx) {
+    return align_up((size_t)N * 4, 256) + align_up((size_t)n_idx * 4, 256) + align_up((size_t)n_idx * 12, 256);
+}
+
+extern "C" int gsx_mcmc_relocate(uint32_t N, uint32_t n_idx, const int64_t* sampled_idxs, const int64_t* dead_idxs,
+                                 const float* binoms, int n_max, float min_opacity, float* opacity_raw,
+                                 float* scaling_raw, const gsx_row_tensor* tensors_host, int n_tensors,
+                                 void* workspace, size_t workspace_bytes, void* stream) {
+    if (n_idx == 0)
+        return GSX_OK; // mcmc.cpp:126-127
+    GSX_REQUIRE(sampled_idxs && dead_idxs && binoms && opacity_raw && scaling_raw, GSX_ERR_INVALID_ARGUMENT,
+                "mcmc_relocate: null tensor");
+    GSX_REQUIRE(n_max > 0 && n_tensors >= 0 && n_tensors <= GSX_MCMC_MAX_TENSORS && (n_tensors == 0 || tensors_host),
+                GSX_ERR_INVALID_ARGUMENT, "mcmc_relocate: n_max %d, n_tensors %d (max %d)", n_max, n_tensors,
+                GSX_MCMC_MAX_TENSORS);
+    GSX_REQUIRE(workspace && ((uintptr_t)workspace & 255) == 0 &&
+                    workspace_bytes >= gsx_mcmc_relocate_workspace_bytes(N, n_idx),
+                GSX_ERR_WORKSPACE, "mcmc_relocate: workspace of %zu bytes, need %zu (256-byte aligned)",
+                workspace_bytes, gsx_mcmc_relocate_workspace_bytes(N, n_idx));
+    RowTable tab;
+    memset(&tab, 0, sizeof(tab));
+    uint32_t max_row = 0;
+    for (int e = 0; e < n_tensors; ++e) {
+        GSX_REQUIRE(tensors_host[e].data && tensors_host[e].row_floats > 0, GSX_ERR_INVALID_ARGUMENT,
+                    "mcmc_relocate: tensor %d is null or has empty rows", e);
+        tab.data[e] = tensors_host[e].data;
+        tab.row_floats[e] = tensors_host[e].row_floats;
+        tab.is_state[e] = tensors_host[e].is_optimizer_state ? 1u : 0u;
+        max_row = tensors_host[e].row_floats > max_row ? tensors_host[e].row_floats : max_row;
+    }
+    char* ws = (char*)workspace;
+    int32_t* counts = (int32_t*)ws;
+    float* new_op = (float*)(ws + align_up((size_t)N * 4, 256));
+    float* new_sc = (float*)((char*)new_op + align_up((size_t)n_idx * 4, 256));
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 g(cdiv(n_idx, 256)), b(256);
+    hipLaunchKernelGGL(mcmc_count_kernel, g, b, 0, st, n_idx, sampled_idxs, counts, 0);
+    hipLaunchKernelGGL(mcmc_count_kernel, g, b, 0, st, n_idx, sampled_idxs, counts, 1);
+    hipLaunchKernelGGL(mcmc_relocate_compute_kernel, g, b, 0, st, n_idx, sampled_idxs, counts, opacity_raw,
+                       scaling_raw, binoms, n_max, min_opacity, new_op, new_sc);
+    hipLaunchKernelGGL(mcmc_relocate_store_kernel, g, b, 0, st, n_idx, sampled_idxs, new_op, new_sc, opacity_raw,
+                       scaling_raw);
+    if (n_tensors) {
+        const uint64_t per = (uint64_t)n_idx * max_row;
+        GSX_REQUIRE((per + 255) / 256 < (1ull << 31), GSX_ERR_OVERFLOW, "mcmc_relocate: %u rows x %u floats", n_idx,
+                    max_row);
+        hipLaunchKernelGGL(mcmc_rows_kernel, dim3((uint32_t)cdiv(per, (uint64_t)256), n_tensors), b, 0, st, n_idx,
+                           sampled_idxs, dead_idxs, tab);
+    }
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

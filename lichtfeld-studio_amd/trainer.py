@@ -246,6 +246,36 @@ class TrainStep:
 
     freeze_shN_early = False  # BASELINE's step updates all parameter tensors; set True for the product schedule
 
+    # -- MCMC strategy steps that touch the parameters ------------------------------------------------
+    def relocate(self, sampled_idxs, dead_idxs, binoms, min_opacity=0.005):
+        """MCMC::relocate_gs (mcmc.cpp:112-190) for index sets chosen by the caller (the multinomial draw of :132 is
+        the caller's): sampled Gaussians get the Eq. 9 opacity / scales, dead ones become copies of them, the Adam
+        moments of the sampled ones are cleared.  sampled_idxs / dead_idxs: int64 device tensors of equal length."""
+        n = int(sampled_idxs.numel())
+        assert n == int(dead_idxs.numel()) and sampled_idxs.dtype == dead_idxs.dtype == torch.int64
+        if n == 0:
+            return 0
+        names = ["means", "shs", "scaling", "rotation", "opacity"]
+        tensors = [(self.params[k], 0) for k in names]
+        tensors += [(self.exp_avg[k], 1) for k in names] + [(self.exp_avg_sq[k], 1) for k in names]
+        arr = (L.RowTensor * len(tensors))()
+        for i, (t, is_state) in enumerate(tensors):
+            arr[i] = L.RowTensor(t.data_ptr(), t.numel() // self.N, is_state)
+        nbytes = self.lib.gsx_mcmc_relocate_workspace_bytes(c_u32(self.N), c_u32(n))
+        if getattr(self, "ws_mcmc", None) is None or self.ws_mcmc.numel() < nbytes:
+            self.ws_mcmc = torch.empty(nbytes, dtype=torch.uint8, device=self.dev)
+        self._run("mcmc_relocate", self.lib.gsx_mcmc_relocate, c_u32(self.N), c_u32(n), _p(sampled_idxs),
+                  _p(dead_idxs), _p(binoms), c_i(binoms.shape[0]), c_f(min_opacity), _p(self.params["opacity"]),
+                  _p(self.params["scaling"]), arr, c_i(len(tensors)), _p(self.ws_mcmc), c_sz(self.ws_mcmc.numel()),
+                  self._stream())
+        return n
+
+    def inject_noise(self, noise, noise_lr=5e5):
+        """MCMC::inject_noise (mcmc.cpp:349-367) with the caller's N(0,1) draws [N,3]."""
+        self._run("add_noise", self.lib.gsx_add_noise, c_i(self.N), _p(self.params["opacity"]),
+                  _p(self.params["scaling"]), _p(self.params["rotation"]), _p(noise), _p(self.params["means"]),
+                  c_f(self.lrs["means"] * noise_lr), self._stream())
+
     def step(self, viewmat, K, W, H, gt_chw):
         self.iteration += 1
         self.forward(viewmat, K, W, H)

@@ -73,6 +73,33 @@ class OracleTrainStep:
             orc.adam_step(p, m, v, g, lr, b1, b2, self.eps, bc1, bc2)
             self.params["shs"][:, sl], self.exp_avg["shs"][:, sl], self.exp_avg_sq["shs"][:, sl] = p, m, v
 
+    def relocate(self, sampled_idxs, dead_idxs, binoms, min_opacity=0.005):
+        """MCMC::relocate_gs (mcmc.cpp:112-190) line by line, with the caller's index sets."""
+        P = self.params
+        n_max = binoms.shape[0]
+        if sampled_idxs.size == 0:
+            return 0
+        op, scales, _ = orc.activate_params(P["opacity"], P["scaling"], P["rotation"])
+        ratios = np.ones(op.shape[0], np.int32)                                   # :141
+        np.add.at(ratios, sampled_idxs, 1)                                        # :142-143
+        ratios = np.minimum(ratios[sampled_idxs], n_max).astype(np.int32)         # :144-148
+        new_op, new_sc = orc.relocation(op[sampled_idxs], scales[sampled_idxs], ratios, binoms, n_max)  # :151-156
+        new_op = np.clip(new_op, np.float32(min_opacity), np.float32(1.0 - 1e-7))  # :160
+        P["opacity"][sampled_idxs] = orc.math_unary("log", new_op / (np.float32(1.0) - new_op))  # logit, :165-169
+        P["scaling"][sampled_idxs] = orc.math_unary("log", new_sc.reshape(-1)).reshape(-1, 3)    # log, :171
+        for k in ("means", "shs", "scaling", "rotation", "opacity"):               # :175-180
+            P[k][dead_idxs] = P[k][sampled_idxs]
+        for k in P:                                                                # :100-104
+            self.exp_avg[k][sampled_idxs] = 0
+            self.exp_avg_sq[k][sampled_idxs] = 0
+        return sampled_idxs.size
+
+    def inject_noise(self, noise, noise_lr=5e5):
+        """MCMC::inject_noise (mcmc.cpp:349-367)"""
+        P = self.params
+        orc.add_noise(P["opacity"], P["scaling"], P["rotation"], noise, P["means"],
+                      np.float32(self.lrs["means"] * noise_lr))
+
     def step(self, viewmat, K, W, H, gt_chw):
         self.forward(viewmat, K, W, H)
         loss = self.loss_and_backward(gt_chw)
