@@ -64,6 +64,7 @@ def algorithmic_bytes(N, K, H, W, n_isects, sort_bits):
         "fusedssim": P * (24 + 12 + 36),
         "fusedssim_backward": P * (72 + 12),
         "render_grad_from_loss": P * (12 + 12 + 12 + 12 + 12),
+        "pack_raster_records": N * (56 + 80),
         "rasterize_bwd_clear": N * 64,
         "rasterize_bwd_finish": N * (64 + 40 + 56),
         "sh_colors_from_world_bwd": N * (12 + 8 + 12 + 12 + 12 * K),
@@ -132,10 +133,9 @@ def main():
     L = gsx._lib
     p = lambda t: ctypes.c_void_p(t.data_ptr())
     L.check(L.lib().gsx_rasterize_pair_stats(
-        ctypes.c_uint32(ts.N), ctypes.c_int64(ts.n_isects), p(ts.params["means"]), p(ts.act["quats"]),
-        p(ts.act["scales"]), p(ts.act["opacities"]), ctypes.c_uint32(W), ctypes.c_uint32(H), p(viewmat), p(Kmat),
+        ctypes.c_int64(ts.n_isects), p(ts.records), ctypes.c_uint32(W), ctypes.c_uint32(H), p(viewmat), p(Kmat),
         p(ts.offsets), p(ts.flatten_ids), p(stats), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
-    pairs_fwd, pairs_comp, pairs_bwd = [int(x) for x in stats.cpu()[:3]]
+    pairs_fwd, pairs_comp, pairs_bwd, wave_iters, wave_skipped = [int(x) for x in stats.cpu()[:5]]
 
     # instrumented pass: every stage bracketed by events (not part of the timed region)
     ts.start_timing(None)
@@ -143,6 +143,23 @@ def main():
     for _ in range(n_prof):
         ts.step(viewmat, Kmat, W, H, gt)
     stage_ms = {k: float(np.mean(v)) for k, v in ts.stop_timing().items()}
+
+    # known-size copy: the yardstick for byte counters and the measured streaming bandwidth of this GPU
+    copy_bytes = 256 << 20
+    cp_src = torch.empty(copy_bytes, dtype=torch.uint8, device=dev)
+    cp_dst = torch.empty(copy_bytes, dtype=torch.uint8, device=dev)
+    cp_src.zero_()
+    copy_ms = []
+    for _ in range(4):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        L.check(L.lib().gsx_debug_copy(p(cp_src), p(cp_dst), ctypes.c_size_t(copy_bytes),
+                                       ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        e1.record()
+        torch.cuda.synchronize()
+        copy_ms.append(e0.elapsed_time(e1))
+    copy_gbs = 2 * copy_bytes / (min(copy_ms[1:]) * 1e-3) / 1e9
+    del cp_src, cp_dst
 
     tile_bits = int(L.lib().gsx_n_bits(ctypes.c_uint32(ts.tw * ts.th)))
     abytes = algorithmic_bytes(ts.N, ts.K, H, W, ts.n_isects, 32 + tile_bits + 1)
@@ -184,10 +201,14 @@ def main():
                                f"{W}x{H}, fwd + " + ("0.8 L1 + 0.2 (1-SSIM)" if use_ssim else "L1") +
                                " + bwd + fused Adam", "n_gaussians": ts.N, "image": [W, H], "n_isects": ts.n_isects,
                    "tiles": ts.tw * ts.th, "pairs_fwd": pairs_fwd, "pairs_composited": pairs_comp,
-                   "pairs_bwd": pairs_bwd, "loss": loss, "setup_s": round(setup_s, 1)},
+                   "pairs_bwd": pairs_bwd, "wave_iterations": wave_iters,
+                   "wave_iterations_skipped_by_bounds": wave_skipped, "loss": loss, "setup_s": round(setup_s, 1)},
         "raster_fwd_ms": kernels.get("rasterize_to_pixels_from_world_3dgs_fwd", {}).get("ms"),
         "raster_bwd_ms": round(dom_ms, 4),
-        "roofline": roofline, "cpu_baseline": cpu_baseline, "kernels": kernels,
+        "roofline": roofline, "cpu_baseline": cpu_baseline,
+        "copy_probe": {"bytes_moved": 2 * copy_bytes, "GBps": round(copy_gbs, 1),
+                       "note": "gsx_debug_copy, 256 MiB read + 256 MiB written: measured streaming bandwidth"},
+        "kernels": kernels,
     }
     print(json.dumps(out))
 

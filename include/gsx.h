@@ -66,6 +66,9 @@ GSX_API gsx_ut_params gsx_ut_defaults(void);
  * device so that a test can compare it bit for bit with a host build.  which: 0 exp, 1 log, 2 rsqrt, 3 sin, 4 acos,
  * 5 sigmoid, 6 saturating float->u32, 7 pow(x, x2), 8 x / x2, 9 sqrt, 10 fma(x, x2, x). */
 GSX_API int gsx_debug_math(int which, uint32_t n, const float* x, const float* x2, float* y, void* stream);
+/* Measurement hook (no counterpart in the reference): a plain device-to-device copy kernel of `bytes` bytes (a
+ * multiple of 16), the known-size yardstick for HBM byte counters and achieved-bandwidth figures. */
+GSX_API int gsx_debug_copy(const void* src, void* dst, size_t bytes, void* stream);
 /* Test hook: the 64-lane, 16-value wave reduction of the rasterizer backward.  in [n_waves,64,16] -> out [n_waves,16]. */
 GSX_API int gsx_debug_wave_reduce16(uint32_t n_waves, const float* in, float* out, void* stream);
 
@@ -122,7 +125,23 @@ GSX_API int gsx_intersect_offset(int64_t n_isects, const int64_t* isect_ids, uin
 /* ---- a7: gsplat::rasterize_to_pixels_from_world_3dgs_fwd (Ops.h:100-129; ...3DGSFwd.cu:19-285) ----
  * colors [C,N,channels] (channels in {1,3,4}), opacities [C,N], backgrounds [C,channels] nullable,
  * masks u8 [C,Th,Tw] nullable, tile_offsets i32 [C,Th,Tw], flatten_ids i32 [n_isects]
- * -> render_colors [C,H,W,channels], render_alphas [C,H,W,1], last_ids i32 [C,H,W]. tile_size must be 16. */
+ * -> render_colors [C,H,W,channels], render_alphas [C,H,W,1], last_ids i32 [C,H,W]. tile_size must be 16.
+ *
+ * The rasterizers read one 80-byte RECORD per Gaussian (whitening matrix diag(1/s) R^T, camera centre in whitened
+ * coordinates, opacity, first three colour channels, exact pixel bounds of alpha >= 1/255) instead of the five
+ * parameter tensors: gsx_pack_raster_records builds them for one camera, gsx_rasterize_records_fwd renders from
+ * them.  The whole-operator entry point does both and needs gsx_raster_records_bytes(N) of workspace. */
+GSX_API size_t gsx_raster_records_bytes(uint32_t N);
+GSX_API int gsx_pack_raster_records(uint32_t N, const float* means, const float* quats, const float* scales,
+                                    const float* opacities, const float* colors, uint32_t channels,
+                                    const float* viewmat, const float* K, uint32_t image_width,
+                                    uint32_t image_height, void* records, void* stream);
+/* colors is only read for channels beyond the third (channels == 4); nullable otherwise */
+GSX_API int gsx_rasterize_records_fwd(int64_t n_isects, const void* records, const float* colors, uint32_t channels,
+                                      const float* backgrounds, const uint8_t* masks, uint32_t image_width,
+                                      uint32_t image_height, const float* viewmat, const float* K,
+                                      const int32_t* tile_offsets, const int32_t* flatten_ids, float* render_colors,
+                                      float* render_alphas, int32_t* last_ids, void* stream);
 GSX_API int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
     uint32_t C, uint32_t N, int64_t n_isects, const float* means, const float* quats, const float* scales,
     const float* colors, uint32_t channels, const float* opacities, const float* backgrounds, const uint8_t* masks,
@@ -130,14 +149,13 @@ GSX_API int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
     const float* viewmats1 /*must be NULL*/, const float* Ks, int camera_model, gsx_ut_params ut, int rs_type,
     const float* radial_coeffs, const float* tangential_coeffs, const float* thin_prism_coeffs,
     const int32_t* tile_offsets, const int32_t* flatten_ids, float* render_colors, float* render_alphas,
-    int32_t* last_ids, void* stream);
+    int32_t* last_ids, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Pair counts of one forward pass, for turning kernel times into rates (no counterpart in the reference).
- * stats_out: device uint64[8] = {pairs the forward evaluates, pairs composited, pairs the backward evaluates,
- * (wave, Gaussian) iterations of the forward, those of them with at least one lane above the alpha threshold,
- * 3 reserved}; the counts are ADDED to it, so zero it first. */
-GSX_API int gsx_rasterize_pair_stats(uint32_t N, int64_t n_isects, const float* means, const float* quats,
-                                     const float* scales, const float* opacities, uint32_t image_width,
+ * stats_out: device uint64[8] = {(pixel, Gaussian) pairs the forward evaluates, pairs composited, pairs the backward
+ * walks, (wave, Gaussian) iterations executed, (wave, Gaussian) iterations removed by the pixel bounds, 3 reserved};
+ * the counts are ADDED to it, so zero it first. */
+GSX_API int gsx_rasterize_pair_stats(int64_t n_isects, const void* records, uint32_t image_width,
                                      uint32_t image_height, const float* viewmat, const float* K,
                                      const int32_t* tile_offsets, const int32_t* flatten_ids,
                                      unsigned long long* stats_out, void* stream);
@@ -145,18 +163,21 @@ GSX_API int gsx_rasterize_pair_stats(uint32_t N, int64_t n_isects, const float* 
 /* ---- a8: gsplat::rasterize_to_pixels_from_world_3dgs_bwd (Ops.h:131-166; ...3DGSBwd.cu:16-379) ----
  * channels must be 3.  The five gradient outputs are fully WRITTEN (no zero-fill needed; the reference
  * zero-fills and accumulates, Rasterization.cpp:190-194): v_means [N,3], v_quats [N,4], v_scales [N,3],
- * v_colors [C,N,3], v_opacities [C,N].  The workspace holds 16 floats per Gaussian. */
+ * v_colors [C,N,3], v_opacities [C,N].  Workspace of the whole operator: 16 accumulator floats per Gaussian
+ * followed by the records. */
 GSX_API size_t gsx_rasterize_bwd_workspace_bytes(uint32_t N);
+GSX_API size_t gsx_rasterize_bwd_accum_bytes(uint32_t N);
 /* The backward pass is three launches - clear the accumulators, the per-tile kernel, the per-Gaussian epilogue -
- * that can also be called one by one (a training loop can fold the epilogue into its own per-Gaussian pass). */
+ * that can also be called one by one (a training loop shares the forward's records and can fold the epilogue into
+ * its own per-Gaussian pass); these three take the accumulator part (gsx_rasterize_bwd_accum_bytes) only. */
 GSX_API int gsx_rasterize_bwd_clear(uint32_t N, void* workspace, size_t workspace_bytes, void* stream);
-GSX_API int gsx_rasterize_bwd_accumulate(
-    uint32_t C, uint32_t N, int64_t n_isects, const float* means, const float* quats, const float* scales,
-    const float* colors, const float* opacities, const float* backgrounds, const uint8_t* masks,
-    uint32_t image_width, uint32_t image_height, uint32_t tile_size, const float* viewmats0, const float* Ks,
-    const int32_t* tile_offsets, const int32_t* flatten_ids, const float* render_alphas, const int32_t* last_ids,
-    const float* v_render_colors, const float* v_render_alphas, void* workspace, size_t workspace_bytes,
-    void* stream);
+GSX_API int gsx_rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isects, const void* records,
+                                         const float* backgrounds, const uint8_t* masks, uint32_t image_width,
+                                         uint32_t image_height, uint32_t tile_size, const float* viewmats0,
+                                         const float* Ks, const int32_t* tile_offsets, const int32_t* flatten_ids,
+                                         const float* render_alphas, const int32_t* last_ids,
+                                         const float* v_render_colors, const float* v_render_alphas, void* workspace,
+                                         size_t workspace_bytes, void* stream);
 GSX_API int gsx_rasterize_bwd_finish(uint32_t N, const float* means, const float* quats, const float* scales,
                                      const float* viewmats0, const void* workspace, size_t workspace_bytes,
                                      float* v_means, float* v_quats, float* v_scales, float* v_colors,

@@ -73,7 +73,8 @@ def lib():
         L.gsx_image_loss_blocks.restype = c_u32
         L.gsx_ut_defaults.restype = UTParams
         for name in ("gsx_intersect_tile_count_workspace_bytes", "gsx_radix_sort_pairs_workspace_bytes",
-                     "gsx_rasterize_bwd_workspace_bytes", "gsx_mcmc_relocate_workspace_bytes"):
+                     "gsx_rasterize_bwd_workspace_bytes", "gsx_mcmc_relocate_workspace_bytes",
+                     "gsx_raster_records_bytes", "gsx_rasterize_bwd_accum_bytes"):
             getattr(L, name).restype = c_sz
         _lib = L
     return _lib

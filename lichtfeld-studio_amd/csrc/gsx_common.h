@@ -8,6 +8,7 @@
 #define GSX_BUILD 1
 #include "../../include/gsx.h"
 #include "gsx_math.h"
+#include "gsx_record.h"
 
 namespace gsx {
 
@@ -84,6 +85,81 @@ __device__ __forceinline__ void pixel_world_ray(const CamPose& cp, float px, flo
     const mat3 R_inv = mat3_cast(quat_inverse(q));
     *ray_o = neg(mul(R_inv, t));
     *ray_d = mul(R_inv, d_cam);
+}
+
+// camera centre in world space exactly as the rasterizers form it (Cameras.cuh:253-266 with the start pose)
+__device__ __forceinline__ vec3 camera_ray_origin(const CamPose& cp) {
+    quat q;
+    vec3 t;
+    shutter_pose(cp, 0.f, &q, &t);
+    return neg(mul(mat3_cast(quat_inverse(q)), t));
+}
+
+// ---- tile geometry shared by the forward and backward rasterizers ----------------------------
+// One 256-lane workgroup per 16x16 tile; wave w owns the 8x8 pixel block (w & 1, w >> 1), lane l the pixel
+// (l >> 3, l & 7) of it: compact blocks keep a wave's pixels coherent (saturation, bounds rejection).
+static constexpr uint32_t kTile = 16;
+static constexpr uint32_t kBatch = 256;
+static constexpr float kPowerCut = -5.55f; // exp(-5.55) = 3.8875e-3 < 1/255 = 3.9216e-3
+
+struct TilePixel {
+    uint32_t i, j;     // pixel row / column
+    int32_t wi0, wj0;  // first row / column of the wave's 8x8 block
+};
+__device__ __forceinline__ TilePixel tile_pixel(uint32_t tile_id, uint32_t tile_width, uint32_t tr) {
+    const uint32_t ty = tile_id / tile_width, tx = tile_id % tile_width;
+    const uint32_t wave = tr >> 6, lane = tr & 63u;
+    TilePixel p;
+    p.wi0 = (int32_t)(ty * kTile + (wave >> 1) * 8u);
+    p.wj0 = (int32_t)(tx * kTile + (wave & 1u) * 8u);
+    p.i = (uint32_t)p.wi0 + (lane >> 3);
+    p.j = (uint32_t)p.wj0 + (lane & 7u);
+    return p;
+}
+
+// Stage one batch of records (the tile's list entries [first, first + count) in the order given by step = +1 /
+// -1) into LDS, then build, per wave, the ordered list of batch slots whose pixel bounds meet the wave's 8x8
+// block and whose slot index is >= t_start.  Returns the length of the wave's list.  Contains two barriers.
+__device__ __forceinline__ uint32_t stage_and_select(const float4* __restrict__ records,
+                                                     const int32_t* __restrict__ flatten_ids, int32_t first,
+                                                     int32_t step, uint32_t count, uint32_t tr, const TilePixel& px,
+                                                     uint32_t t_start, bool wave_active, float4* stage, int4* boxes,
+                                                     int32_t* ids, uint8_t* wave_list) {
+    if (tr < count) {
+        const int32_t g = flatten_ids[first + step * (int32_t)tr];
+        const float4* __restrict__ r = records + (size_t)g * 5;
+        const float4 r0 = r[0], r1 = r[1], r2 = r[2], r3 = r[3], r4 = r[4];
+        stage[tr * 4 + 0] = r0;
+        stage[tr * 4 + 1] = r1;
+        stage[tr * 4 + 2] = r2;
+        stage[tr * 4 + 3] = r3;
+        boxes[tr] = make_int4((int)f2u(r4.x), (int)f2u(r4.y), (int)f2u(r4.z), (int)f2u(r4.w));
+        if (ids != nullptr)
+            ids[tr] = g;
+    }
+    __syncthreads();
+    uint32_t n = 0;
+    if (wave_active) {
+        const uint32_t lane = tr & 63u;
+#pragma unroll
+        for (uint32_t r = 0; r < kBatch / 64; ++r) {
+            const uint32_t t = r * 64u + lane;
+            bool hit = false;
+            if (t < count && t >= t_start) {
+                const int4 b = boxes[t];
+                hit = b.x <= px.wj0 + 7 && b.z >= px.wj0 && b.y <= px.wi0 + 7 && b.w >= px.wi0;
+            }
+            const uint64_t m = __builtin_amdgcn_ballot_w64(hit);
+            if (hit) {
+                const uint32_t below =
+                    __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+                wave_list[n + below] = (uint8_t)t;
+            }
+            n += (uint32_t)__builtin_popcountll(m);
+        }
+    }
+    __syncthreads();
+    return n;
 }
 
 __device__ __forceinline__ vec3 ld3(const float* __restrict__ p, uint32_t i) {

@@ -274,13 +274,14 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> rasterize_to_pixels_from_world_3d
     at::Tensor renders = at::empty({C, image_height, image_width, channels}, opt);
     at::Tensor alphas = at::empty({C, image_height, image_width, 1}, opt);
     at::Tensor last_ids = at::empty({C, image_height, image_width}, opt.dtype(at::kInt));
+    at::Tensor ws = workspace(gsx_raster_records_bytes(N), means);
     const int st = gsx_rasterize_to_pixels_from_world_3dgs_fwd(
         C, N, flatten_ids.size(0), means.data_ptr<float>(), quats.data_ptr<float>(), scales.data_ptr<float>(),
         colors.data_ptr<float>(), channels, opacities.data_ptr<float>(), fptr(backgrounds), bptr(masks), image_width,
         image_height, tile_size, viewmats0.data_ptr<float>(), fptr(viewmats1), Ks.data_ptr<float>(), (int)camera_model,
         to_gsx(ut_params), (int)rs_type, fptr(radial_coeffs), fptr(tangential_coeffs), fptr(thin_prism_coeffs),
         tile_offsets.data_ptr<int32_t>(), flatten_ids.data_ptr<int32_t>(), renders.data_ptr<float>(),
-        alphas.data_ptr<float>(), last_ids.data_ptr<int32_t>(), cur_stream(means));
+        alphas.data_ptr<float>(), last_ids.data_ptr<int32_t>(), ws.data_ptr(), (size_t)ws.numel(), cur_stream(means));
     TORCH_CHECK(st != GSX_ERR_UNSUPPORTED || (channels == 1 || channels == 3 || channels == 4),
                 "Unsupported number of channels: ", channels); // Rasterization.cpp:126-127
     gsx_check(st);

@@ -20,9 +20,6 @@
 
 namespace gsx {
 
-static constexpr uint32_t kTile = 16;
-static constexpr uint32_t kBatch = 256;
-static constexpr float kPowerCut = -5.55f; // exp(-5.55) = 3.8875e-3 < 1/255 = 3.9216e-3
 static constexpr uint32_t kAcc = 16; // floats accumulated per Gaussian: rgb 3, v_gro 3, v_grd(x)ray_d 9, opacity 1
 
 __global__ void __launch_bounds__(256) fill_f32_kernel(size_t n, float v, float* __restrict__ out) {
@@ -94,15 +91,16 @@ __global__ void __launch_bounds__(64) wave_reduce16_probe_kernel(const float* __
 }
 
 __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
-    uint32_t n_isects, const float* __restrict__ means, const float* __restrict__ quats,
-    const float* __restrict__ scales, const float* __restrict__ colors, const float* __restrict__ opacities,
-    const float* __restrict__ backgrounds, const uint8_t* __restrict__ masks, uint32_t image_width,
-    uint32_t image_height, uint32_t tile_width, uint32_t tile_height, const float* __restrict__ viewmat,
-    const float* __restrict__ Kmat, const int32_t* __restrict__ tile_offsets,
-    const int32_t* __restrict__ flatten_ids, const float* __restrict__ render_alphas,
-    const int32_t* __restrict__ last_ids, const float* __restrict__ v_render_colors,
-    const float* __restrict__ v_render_alphas, float* __restrict__ gacc /*[N,16]*/) {
+    uint32_t n_isects, const float4* __restrict__ records, const float* __restrict__ backgrounds,
+    const uint8_t* __restrict__ masks, uint32_t image_width, uint32_t image_height, uint32_t tile_width,
+    uint32_t tile_height, const float* __restrict__ viewmat, const float* __restrict__ Kmat,
+    const int32_t* __restrict__ tile_offsets, const int32_t* __restrict__ flatten_ids,
+    const float* __restrict__ render_alphas, const int32_t* __restrict__ last_ids,
+    const float* __restrict__ v_render_colors, const float* __restrict__ v_render_alphas,
+    float* __restrict__ gacc /*[N,16]*/) {
     __shared__ float4 stage[kBatch * 4];
+    __shared__ int4 boxes[kBatch];
+    __shared__ uint8_t lists[4][kBatch];
     __shared__ int32_t id_batch[kBatch];
     __shared__ float acc[kBatch * kAcc];
     __shared__ int32_t block_max;
@@ -110,13 +108,13 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     const uint32_t tile_id = blockIdx.x;
     if (masks != nullptr && !masks[tile_id]) // :83-87
         return;
-    const uint32_t ty = tile_id / tile_width, tx = tile_id % tile_width;
     const uint32_t tr = threadIdx.x;
     const uint32_t lane = tr & 63u;
-    const uint32_t i = ty * kTile + (tr >> 4);
-    const uint32_t j = tx * kTile + (tr & 15u);
+    const TilePixel px = tile_pixel(tile_id, tile_width, tr);
+    const uint32_t i = px.i, j = px.j;
     const bool inside = (i < image_height && j < image_width);
     const uint32_t pix_id = min(i * image_width + j, image_width * image_height - 1); // :92-93
+    uint8_t* wave_list = lists[tr >> 6];
 
     const CamPose cp = load_cam_pose(viewmat);
     vec3 ray_o, ray_d;
@@ -162,34 +160,17 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     const uint32_t num_batches = (uint32_t)(range_end - range_start + (int32_t)kBatch - 1) / kBatch;
 
     for (uint32_t b = 0; b < num_batches; ++b) {
-        // back to front: entry 0 of the batch is the farthest Gaussian (:211-216)
+        // back to front: slot 0 of the batch is the farthest Gaussian (:211-216)
         const int32_t batch_end = range_end - 1 - (int32_t)(kBatch * b);
         const int32_t batch_size = min((int32_t)kBatch, batch_end + 1 - range_start);
-        const int32_t idx = batch_end - (int32_t)tr;
-        if (idx >= range_start) {
-            const int32_t g = flatten_ids[idx];
-            id_batch[tr] = g;
-            const vec3 xyz = ld3(means, g);
-            const float opac = opacities[g];
-            const mat3 R = quat_to_rotmat(ld4q(quats, g));
-            const vec3 s = ld3(scales, g);
-            const float is0 = 1.0f / s.x, is1 = 1.0f / s.y, is2 = 1.0f / s.z;
-            // M = diag(1/s) R^T and gro = M (ray_o - mean): the ray origin is the same for every pixel of a
-            // global-shutter camera, so this half of the per-pair work is done once per staged Gaussian
-            mat3 M;
-            M.m[0][0] = is0 * R.m[0][0], M.m[0][1] = is0 * R.m[1][0], M.m[0][2] = is0 * R.m[2][0];
-            M.m[1][0] = is1 * R.m[0][1], M.m[1][1] = is1 * R.m[1][1], M.m[1][2] = is1 * R.m[2][1];
-            M.m[2][0] = is2 * R.m[0][2], M.m[2][1] = is2 * R.m[1][2], M.m[2][2] = is2 * R.m[2][2];
-            const vec3 gro = mul(M, sub(ray_o, xyz));
-            stage[tr * 4 + 0] = make_float4(gro.x, gro.y, gro.z, opac);
-            stage[tr * 4 + 1] = make_float4(M.m[0][0], M.m[0][1], M.m[0][2], M.m[1][0]);
-            stage[tr * 4 + 2] = make_float4(M.m[1][1], M.m[1][2], M.m[2][0], M.m[2][1]);
-            stage[tr * 4 + 3] =
-                make_float4(M.m[2][2], colors[(size_t)g * 3], colors[(size_t)g * 3 + 1], colors[(size_t)g * 3 + 2]);
-        }
-        __syncthreads();
+        // slots in front of t_start lie behind every last contributor of this wave
+        const uint32_t t_start = (uint32_t)max(0, batch_end - wave_bin_final);
+        const uint32_t n_sel = stage_and_select(records, flatten_ids, batch_end, -1, (uint32_t)batch_size, tr, px,
+                                                t_start, t_start < (uint32_t)batch_size, stage, boxes, id_batch,
+                                                wave_list);
 
-        for (int32_t t = max(0, batch_end - wave_bin_final); t < batch_size; ++t) {
+        for (uint32_t sidx = 0; sidx < n_sel; ++sidx) {
+            const int32_t t = (int32_t)wave_list[sidx];
             bool valid = inside && (batch_end - t <= bin_final);
             const float4 a = stage[t * 4 + 0];
             const float4 m0 = stage[t * 4 + 1];
@@ -381,16 +362,20 @@ extern "C" int gsx_debug_wave_reduce16(uint32_t n_waves, const float* in, float*
     return GSX_OK;
 }
 
-extern "C" size_t gsx_rasterize_bwd_workspace_bytes(uint32_t N) { return align_up((size_t)N * kAcc * 4, 256) + 256; }
+// accumulators only (16 floats per Gaussian); the whole-operator entry point also packs the records behind them
+extern "C" size_t gsx_rasterize_bwd_accum_bytes(uint32_t N) { return align_up((size_t)N * kAcc * 4, 256) + 256; }
+extern "C" size_t gsx_rasterize_bwd_workspace_bytes(uint32_t N) {
+    return gsx_rasterize_bwd_accum_bytes(N) + gsx_raster_records_bytes(N);
+}
 
 // stage 1: zero the per-Gaussian accumulators
 extern "C" int gsx_rasterize_bwd_clear(uint32_t N, void* workspace, size_t workspace_bytes, void* stream) {
     if (N == 0)
         return GSX_OK;
     GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 &&
-                    workspace_bytes >= gsx_rasterize_bwd_workspace_bytes(N),
-                GSX_ERR_WORKSPACE, "rasterize bwd: workspace needs %zu bytes, 256-byte aligned",
-                gsx_rasterize_bwd_workspace_bytes(N));
+                    workspace_bytes >= gsx_rasterize_bwd_accum_bytes(N),
+                GSX_ERR_WORKSPACE, "rasterize bwd: accumulators need %zu bytes, 256-byte aligned",
+                gsx_rasterize_bwd_accum_bytes(N));
     const size_t n_acc = (size_t)N * kAcc;
     hipLaunchKernelGGL(fill_f32_kernel, dim3(cdiv(n_acc, 256)), dim3(256), 0, (hipStream_t)stream, n_acc, 0.f,
                        (float*)workspace);
@@ -398,31 +383,33 @@ extern "C" int gsx_rasterize_bwd_clear(uint32_t N, void* workspace, size_t works
     return GSX_OK;
 }
 
-// stage 2: the per-tile kernel, accumulating into the workspace
-extern "C" int gsx_rasterize_bwd_accumulate(
-    uint32_t C, uint32_t N, int64_t n_isects, const float* means, const float* quats, const float* scales,
-    const float* colors, const float* opacities, const float* backgrounds, const uint8_t* masks,
-    uint32_t image_width, uint32_t image_height, uint32_t tile_size, const float* viewmats0, const float* Ks,
-    const int32_t* tile_offsets, const int32_t* flatten_ids, const float* render_alphas, const int32_t* last_ids,
-    const float* v_render_colors, const float* v_render_alphas, void* workspace, size_t workspace_bytes,
-    void* stream) {
+// stage 2: the per-tile kernel, accumulating into the workspace; `records` from gsx_pack_raster_records (or the
+// fused per-Gaussian pass) for the same camera and parameters
+extern "C" int gsx_rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isects, const void* records,
+                                            const float* backgrounds, const uint8_t* masks, uint32_t image_width,
+                                            uint32_t image_height, uint32_t tile_size, const float* viewmats0,
+                                            const float* Ks, const int32_t* tile_offsets, const int32_t* flatten_ids,
+                                            const float* render_alphas, const int32_t* last_ids,
+                                            const float* v_render_colors, const float* v_render_alphas,
+                                            void* workspace, size_t workspace_bytes, void* stream) {
     GSX_REQUIRE(C == 1, GSX_ERR_UNSUPPORTED, "C = %u cameras: only C == 1 is supported", C);
     if (N == 0 || n_isects == 0 || image_width == 0 || image_height == 0) // ...Bwd.cu:440-443
         return GSX_OK;
     GSX_REQUIRE(tile_size == kTile, GSX_ERR_UNSUPPORTED, "rasterize bwd: tile_size %u (only 16 is built)", tile_size);
     GSX_REQUIRE(n_isects > 0 && n_isects < (1ll << 31), GSX_ERR_OVERFLOW, "rasterize bwd: n_isects out of range");
-    GSX_REQUIRE(means && quats && scales && colors && opacities && viewmats0 && Ks && tile_offsets && flatten_ids &&
-                    render_alphas && last_ids && v_render_colors && v_render_alphas,
+    GSX_REQUIRE(records && viewmats0 && Ks && tile_offsets && flatten_ids && render_alphas && last_ids &&
+                    v_render_colors && v_render_alphas,
                 GSX_ERR_INVALID_ARGUMENT, "rasterize bwd: null tensor");
+    GSX_REQUIRE(((uintptr_t)records & 15) == 0, GSX_ERR_WORKSPACE, "rasterize bwd: records need 16-byte alignment");
     GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 &&
-                    workspace_bytes >= gsx_rasterize_bwd_workspace_bytes(N),
-                GSX_ERR_WORKSPACE, "rasterize bwd: workspace needs %zu bytes, 256-byte aligned",
-                gsx_rasterize_bwd_workspace_bytes(N));
+                    workspace_bytes >= gsx_rasterize_bwd_accum_bytes(N),
+                GSX_ERR_WORKSPACE, "rasterize bwd: accumulators need %zu bytes, 256-byte aligned",
+                gsx_rasterize_bwd_accum_bytes(N));
     const uint32_t tw = cdiv(image_width, kTile), th = cdiv(image_height, kTile);
     hipLaunchKernelGGL(rasterize_bwd_kernel, dim3(tw * th), dim3(256), 0, (hipStream_t)stream, (uint32_t)n_isects,
-                       means, quats, scales, colors, opacities, backgrounds, masks, image_width, image_height, tw, th,
-                       viewmats0, Ks, tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors,
-                       v_render_alphas, (float*)workspace);
+                       (const float4*)records, backgrounds, masks, image_width, image_height, tw, th, viewmats0, Ks,
+                       tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors, v_render_alphas,
+                       (float*)workspace);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }
@@ -436,8 +423,8 @@ extern "C" int gsx_rasterize_bwd_finish(uint32_t N, const float* means, const fl
         return GSX_OK;
     GSX_REQUIRE(means && quats && scales && viewmats0 && v_means && v_quats && v_scales && v_colors && v_opacities,
                 GSX_ERR_INVALID_ARGUMENT, "rasterize bwd: null tensor");
-    GSX_REQUIRE(workspace != nullptr && workspace_bytes >= gsx_rasterize_bwd_workspace_bytes(N), GSX_ERR_WORKSPACE,
-                "rasterize bwd: workspace needs %zu bytes", gsx_rasterize_bwd_workspace_bytes(N));
+    GSX_REQUIRE(workspace != nullptr && workspace_bytes >= gsx_rasterize_bwd_accum_bytes(N), GSX_ERR_WORKSPACE,
+                "rasterize bwd: accumulators need %zu bytes", gsx_rasterize_bwd_accum_bytes(N));
     hipLaunchKernelGGL(rasterize_bwd_epilogue_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, means,
                        quats, scales, viewmats0, (const float*)workspace, v_means, v_quats, v_scales, v_colors,
                        v_opacities);
@@ -459,13 +446,26 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
                                thin_prism_coeffs);
     if (rc != GSX_OK)
         return rc;
-    if ((rc = gsx_rasterize_bwd_clear(N, workspace, workspace_bytes, stream)) != GSX_OK)
+    if (N == 0)
+        return GSX_OK;
+    GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 &&
+                    workspace_bytes >= gsx_rasterize_bwd_workspace_bytes(N),
+                GSX_ERR_WORKSPACE, "rasterize bwd: workspace needs %zu bytes, 256-byte aligned",
+                gsx_rasterize_bwd_workspace_bytes(N));
+    GSX_REQUIRE(means && quats && scales && colors && opacities && viewmats0 && Ks, GSX_ERR_INVALID_ARGUMENT,
+                "rasterize bwd: null tensor");
+    const size_t acc_bytes = gsx_rasterize_bwd_accum_bytes(N);
+    void* records = (char*)workspace + acc_bytes;
+    if ((rc = gsx_rasterize_bwd_clear(N, workspace, acc_bytes, stream)) != GSX_OK)
         return rc;
-    if ((rc = gsx_rasterize_bwd_accumulate(C, N, n_isects, means, quats, scales, colors, opacities, backgrounds,
-                                           masks, image_width, image_height, tile_size, viewmats0, Ks, tile_offsets,
-                                           flatten_ids, render_alphas, last_ids, v_render_colors, v_render_alphas,
-                                           workspace, workspace_bytes, stream)) != GSX_OK)
+    if ((rc = gsx_pack_raster_records(N, means, quats, scales, opacities, colors, 3, viewmats0, Ks, image_width,
+                                      image_height, records, stream)) != GSX_OK)
         return rc;
-    return gsx_rasterize_bwd_finish(N, means, quats, scales, viewmats0, workspace, workspace_bytes, v_means, v_quats,
+    if ((rc = gsx_rasterize_bwd_accumulate(C, N, n_isects, records, backgrounds, masks, image_width, image_height,
+                                           tile_size, viewmats0, Ks, tile_offsets, flatten_ids, render_alphas,
+                                           last_ids, v_render_colors, v_render_alphas, workspace, acc_bytes,
+                                           stream)) != GSX_OK)
+        return rc;
+    return gsx_rasterize_bwd_finish(N, means, quats, scales, viewmats0, workspace, acc_bytes, v_means, v_quats,
                                     v_scales, v_colors, v_opacities, stream);
 }

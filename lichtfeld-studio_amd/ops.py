@@ -233,12 +233,14 @@ def rasterize_to_pixels_from_world_3dgs_fwd(means, quats, scales, colors, opacit
     last_ids = torch.empty((C, image_height, image_width), dtype=torch.int32, device=dev)
     m8 = None if masks is None else masks.view(torch.uint8) if masks.dtype == torch.bool else masks
     with torch.cuda.device(dev):
+        ws = _workspace(lib().gsx_raster_records_bytes(c_u32(N)), dev)
         check(lib().gsx_rasterize_to_pixels_from_world_3dgs_fwd(
             c_u32(C), c_u32(N), c_i64(flatten_ids.numel()), _ptr(means), _ptr(quats), _ptr(scales), _ptr(colors),
             c_u32(channels), _ptr(opacities), _ptr(backgrounds), _ptr(m8), c_u32(image_width), c_u32(image_height),
             c_u32(tile_size), _ptr(viewmats0), _ptr(viewmats1), _ptr(Ks), c_i(camera_model), ut_params, c_i(rs_type),
             _ptr(radial_coeffs), _ptr(tangential_coeffs), _ptr(thin_prism_coeffs), _ptr(tile_offsets),
-            _ptr(flatten_ids), _ptr(renders), _ptr(alphas), _ptr(last_ids), _stream(dev)))
+            _ptr(flatten_ids), _ptr(renders), _ptr(alphas), _ptr(last_ids), _ptr(ws), c_sz(ws.numel()),
+            _stream(dev)))
     return renders, alphas, last_ids
 
 

@@ -60,7 +60,8 @@ class TrainStep:
         self.tiles_per_gauss = e(N, dt=torch.int32)
         self.cum = e(N, dt=torch.int64)
         self.ws_count = e(self.lib.gsx_intersect_tile_count_workspace_bytes(c_u32(1), c_u32(N)), dt=torch.uint8)
-        self.ws_bwd = e(self.lib.gsx_rasterize_bwd_workspace_bytes(c_u32(N)), dt=torch.uint8)
+        self.ws_bwd = e(self.lib.gsx_rasterize_bwd_accum_bytes(c_u32(N)), dt=torch.uint8)
+        self.records = e(self.lib.gsx_raster_records_bytes(c_u32(N)), dt=torch.uint8)
         self.cap = 0
         self.img_shape = None
         self.n_isects = 0
@@ -165,11 +166,13 @@ class TrainStep:
         self.isect_ids, self.flatten_ids = self.keys[self.sel], self.vals[self.sel]
         self._run("intersect_offset", lb.gsx_intersect_offset, c_i64(n), _p(self.isect_ids), c_u32(1), c_u32(self.tw), c_u32(self.th),
                                       _p(self.offsets), s)
-        self._run("rasterize_to_pixels_from_world_3dgs_fwd", lb.gsx_rasterize_to_pixels_from_world_3dgs_fwd, 
-            c_u32(1), c_u32(N), c_i64(n), _p(P["means"]), _p(A["quats"]), _p(A["scales"]), _p(self.colors), c_u32(3),
-            _p(A["opacities"]), _p(self.bg), c_p(None), c_u32(W), c_u32(H), c_u32(16), _p(viewmat), c_p(None), _p(K),
-            c_i(0), self.ut, c_i(4), c_p(None), c_p(None), c_p(None), _p(self.offsets), _p(self.flatten_ids),
-            _p(self.render), _p(self.alpha), _p(self.last_ids), s)
+        self._run("pack_raster_records", lb.gsx_pack_raster_records, c_u32(N), _p(P["means"]), _p(A["quats"]),
+                  _p(A["scales"]), _p(A["opacities"]), _p(self.colors), c_u32(3), _p(viewmat), _p(K), c_u32(W),
+                  c_u32(H), _p(self.records), s)
+        self._run("rasterize_to_pixels_from_world_3dgs_fwd", lb.gsx_rasterize_records_fwd, c_i64(n),
+                  _p(self.records), c_p(None), c_u32(3), _p(self.bg), c_p(None), c_u32(W), c_u32(H), _p(viewmat),
+                  _p(K), _p(self.offsets), _p(self.flatten_ids), _p(self.render), _p(self.alpha), _p(self.last_ids),
+                  s)
         return self.render
 
     # -- loss ---------------------------------------------------------------------------------------
@@ -206,8 +209,8 @@ class TrainStep:
         ws, wsn = _p(self.ws_bwd), c_sz(self.ws_bwd.numel())
         self._run("rasterize_bwd_clear", lb.gsx_rasterize_bwd_clear, c_u32(N), ws, wsn, s)
         self._run("rasterize_bwd_accumulate", lb.gsx_rasterize_bwd_accumulate,
-                  c_u32(1), c_u32(N), c_i64(self.n_isects), _p(P["means"]), _p(A["quats"]), _p(A["scales"]),
-                  _p(self.colors), _p(A["opacities"]), _p(self.bg), c_p(None), c_u32(W), c_u32(H), c_u32(16),
+                  c_u32(1), c_u32(N), c_i64(self.n_isects), _p(self.records), _p(self.bg), c_p(None), c_u32(W),
+                  c_u32(H), c_u32(16),
                   _p(self.viewmat), _p(self.Kmat), _p(self.offsets), _p(self.flatten_ids), _p(self.alpha),
                   _p(self.last_ids), _p(self.v_render), _p(self.v_alpha), ws, wsn, s)
         self._run("rasterize_bwd_finish", lb.gsx_rasterize_bwd_finish, c_u32(N), _p(P["means"]), _p(A["quats"]),

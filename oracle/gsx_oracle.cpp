@@ -1617,3 +1617,43 @@ ORC_API void orc_set_num_threads(int n) {
     (void)n;
 #endif
 }
+
+// ---- conservativeness of the rasterizers' per-Gaussian pixel bounds (csrc/gsx_record.h) ----
+// For each Gaussian: the bounds as the kernels compute them, and a brute-force pass over EVERY pixel of the image
+// with the per-pair arithmetic of the forward pass above (RasterizeToPixelsFromWorld3DGSFwd.cu:228-246): how many
+// pixels reach alpha >= 1/255 (true_count) and how many of those lie outside the bounds (violations, must be 0).
+#include "gsx_record.h"
+
+ORC_API int orc_record_bounds_check(uint32_t N, const float* means, const float* quats, const float* scales,
+                                    const float* opacities, const float* viewmat, const float* Ks, uint32_t W,
+                                    uint32_t H, int32_t* bounds, int64_t* true_count, int64_t* violations) {
+    const float fx = Ks[0], fy = Ks[4], cx = Ks[2], cy = Ks[5];
+    const RollingShutter rs = make_rolling_shutter(viewmat, nullptr);
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int64_t g = 0; g < (int64_t)N; ++g) {
+        vec3 ray_o, ray_d;
+        pixel_world_ray(0.5f, 0.5f, fx, fy, cx, cy, rs, &ray_o, &ray_d);
+        const vec3 xyz = ld3(means, g);
+        const mat3 M = gsx::record_whitening(ld4(quats, g), ld3(scales, g));
+        const vec3 gro = gsx::mul(M, gsx::sub(ray_o, xyz));
+        const gsx::RecordBounds b = gsx::record_bounds(gro, M, opacities[g], xyz, viewmat, fx, fy, cx, cy, W, H);
+        bounds[g * 4 + 0] = b.jmin, bounds[g * 4 + 1] = b.imin, bounds[g * 4 + 2] = b.jmax, bounds[g * 4 + 3] = b.imax;
+        int64_t cnt = 0, bad = 0;
+        for (uint32_t i = 0; i < H; ++i)
+            for (uint32_t j = 0; j < W; ++j) {
+                pixel_world_ray((float)j + 0.5f, (float)i + 0.5f, fx, fy, cx, cy, rs, &ray_o, &ray_d);
+                const vec3 grd = gsx::safe_normalize(gsx::mul(M, ray_d));
+                const vec3 gcrod = gsx::cross(grd, gro);
+                const float power = -0.5f * gsx::dot(gcrod, gcrod);
+                const float alpha = gsx::fmin(0.999f, opacities[g] * gsx::exp(power));
+                if (alpha < 1.f / 255.f)
+                    continue;
+                ++cnt;
+                if ((int32_t)j < b.jmin || (int32_t)j > b.jmax || (int32_t)i < b.imin || (int32_t)i > b.imax)
+                    ++bad;
+            }
+        true_count[g] = cnt;
+        violations[g] = bad;
+    }
+    return 0;
+}

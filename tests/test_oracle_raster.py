@@ -195,3 +195,34 @@ def test_backward_matches_finite_differences_of_the_model(orc):
     assert checked == 6 * 14
     # colour gradient closed form: v_colors[g] = sum_pixels alpha T v_render; zero for Gaussians that reach no pixel
     assert np.all(np.abs(g64[:, 10:13]).sum(1)[np.bincount(flat, minlength=24) == 0] == 0)
+
+
+@pytest.mark.parametrize("trial", range(7))
+def test_record_pixel_bounds_are_conservative(gsx, orc, trial):
+    """The per-Gaussian pixel bounds the GPU rasterizers skip by (csrc/gsx_record.h, compiled here for the host) must
+    contain every pixel that reaches alpha >= 1/255 in the checker's per-pair arithmetic: brute force over all pixels
+    for Gaussians from sub-pixel to screen-filling, anisotropy up to ~1e3, opacities from below the threshold to 1,
+    cameras inside the cloud, long focal lengths and an off-centre crop of a large image."""
+    rng = np.random.default_rng(100 + trial)
+    n, W, H = 1200, 160, 120
+    f = [150.0, 400.0, 80.0, 1000.0, 150.0, 150.0, 3200.0][trial]
+    radius = [4.0, 4.0, 2.0, 6.0, 1.0, 4.0, 4.0][trial]
+    cam = gsx.scenes.orbit_camera(0.3 + trial, radius, W, H, f)
+    if trial == 6:  # a 160x120 window far from the principal point of a 3840x2160 image
+        cam.K = gsx.scenes.intrinsics(W, H, f, f, 1900.0, -950.0)
+    spread = [0.6, 0.6, 0.6, 0.3, 0.8, 0.6, 0.5][trial]
+    means = rng.normal(0, spread, (n, 3)).astype(np.float32)
+    if trial == 6:
+        means += np.linalg.inv(cam.viewmat)[:3, :3] @ np.array([-2.2, 1.3, 0.0], np.float32)  # into the window
+    aniso = [0.3, 1.0, 1.5, 0.5, 1.0, 2.0, 1.0][trial]
+    log_s = rng.uniform(np.log(1e-4), np.log(0.5), (n, 1)) + rng.normal(0, aniso, (n, 3))
+    scales = np.exp(log_s).astype(np.float32)
+    quats = rng.normal(0, 1, (n, 4)).astype(np.float32)
+    op = np.exp(rng.uniform(np.log(1 / 300), 0, n)).astype(np.float32)
+    bounds, count, outside = orc.record_bounds_check(means, quats, scales, op, cam.viewmat, cam.K, W, H)
+    assert outside.sum() == 0, f"{(outside > 0).sum()} Gaussians have contributing pixels outside their bounds"
+    assert (count > 0).sum() > 100  # the case is not vacuous
+    box = np.maximum(bounds[:, 2] - bounds[:, 0] + 1, 0) * np.maximum(bounds[:, 3] - bounds[:, 1] + 1, 0)
+    proper = box < W * H
+    assert box[proper].sum() < 3.0 * max(count[proper].sum(), 1) + 16 * proper.sum()  # and they are tight
+    assert (box[op < 1 / 256] == 0).all()  # below the alpha threshold: empty
