@@ -64,7 +64,8 @@ GSX_API const char* gsx_status_string(int status);
 GSX_API gsx_ut_params gsx_ut_defaults(void);
 /* Test hook (no counterpart in the reference): evaluates one of the shared fp32 math primitives element-wise on the
  * device so that a test can compare it bit for bit with a host build.  which: 0 exp, 1 log, 2 rsqrt, 3 sin, 4 acos,
- * 5 sigmoid, 6 saturating float->u32, 7 pow(x, x2), 8 x / x2, 9 sqrt, 10 fma(x, x2, x). */
+ * 5 sigmoid, 6 saturating float->u32, 7 pow(x, x2), 8 x / x2, 9 sqrt, 10 fma(x, x2, x), 11 exp restricted to
+ * -87 <= x <= 0 (the rasterizers' variant; must equal 0 on that range). */
 GSX_API int gsx_debug_math(int which, uint32_t n, const float* x, const float* x2, float* y, void* stream);
 /* Measurement hook (no counterpart in the reference): a plain device-to-device copy kernel of `bytes` bytes (a
  * multiple of 16), the known-size yardstick for HBM byte counters and achieved-bandwidth figures. */
@@ -153,7 +154,8 @@ GSX_API int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
 
 /* Pair counts of one forward pass, for turning kernel times into rates (no counterpart in the reference).
  * stats_out: device uint64[8] = {(pixel, Gaussian) pairs the forward evaluates, pairs composited, pairs the backward
- * walks, (wave, Gaussian) iterations executed, (wave, Gaussian) iterations removed by the pixel bounds, 3 reserved};
+ * walks, (wave, Gaussian) iterations executed, (wave, Gaussian) iterations removed by the pixel bounds, executed
+ * iterations with a contributing pixel, 2 reserved};
  * the counts are ADDED to it, so zero it first. */
 GSX_API int gsx_rasterize_pair_stats(int64_t n_isects, const void* records, uint32_t image_width,
                                      uint32_t image_height, const float* viewmat, const float* K,

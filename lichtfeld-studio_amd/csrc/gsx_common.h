@@ -100,7 +100,6 @@ __device__ __forceinline__ vec3 camera_ray_origin(const CamPose& cp) {
 // (l >> 3, l & 7) of it: compact blocks keep a wave's pixels coherent (saturation, bounds rejection).
 static constexpr uint32_t kTile = 16;
 static constexpr uint32_t kBatch = 256;
-static constexpr float kPowerCut = -5.55f; // exp(-5.55) = 3.8875e-3 < 1/255 = 3.9216e-3
 
 struct TilePixel {
     uint32_t i, j;     // pixel row / column
@@ -117,23 +116,41 @@ __device__ __forceinline__ TilePixel tile_pixel(uint32_t tile_id, uint32_t tile_
     return p;
 }
 
-// Stage one batch of records (the tile's list entries [first, first + count) in the order given by step = +1 /
-// -1) into LDS, then build, per wave, the ordered list of batch slots whose pixel bounds meet the wave's 8x8
-// block and whose slot index is >= t_start.  Returns the length of the wave's list.  Contains two barriers.
+// The record of one Gaussian as the rasterizers read it (gsx_record.h)
+__device__ __forceinline__ void store_record(float4* __restrict__ r, vec3 gro, float opac, const mat3& M, float c0,
+                                             float c1, float c2, const RecordRegion& g) {
+    r[0] = make_float4(gro.x, gro.y, gro.z, opac);
+    r[1] = make_float4(M.m[0][0], M.m[0][1], M.m[0][2], M.m[1][0]);
+    r[2] = make_float4(M.m[1][1], M.m[1][2], M.m[2][0], M.m[2][1]);
+    r[3] = make_float4(M.m[2][2], c0, c1, c2);
+    const bool is_empty = g.jmin > g.jmax || g.imin > g.imax;
+    const uint32_t jb = is_empty ? 1u : ((uint32_t)g.jmin | ((uint32_t)g.jmax << 16)); // empty: min 1 > max 0
+    const uint32_t ib = is_empty ? 1u : ((uint32_t)g.imin | ((uint32_t)g.imax << 16));
+    r[4] = make_float4(u2f(jb), u2f(ib), g.cut, g.a00);
+    r[5] = make_float4(g.a01, g.a11, g.pcx, g.pcy);
+}
+
+// Stage one batch of records (the tile's list entries first, first + step, ... count of them) into LDS: the
+// 64 bytes the per-pair arithmetic reads go to `stage`, the power cut-off to `cuts`, the region test stays in
+// registers of the staging lane's wave via `region`.  Then build, per wave, the ordered list of batch slots whose
+// region meets the wave's 8x8 block and whose slot index is >= t_start.  Returns the length of the wave's list.
+// Contains two barriers.
 __device__ __forceinline__ uint32_t stage_and_select(const float4* __restrict__ records,
                                                      const int32_t* __restrict__ flatten_ids, int32_t first,
                                                      int32_t step, uint32_t count, uint32_t tr, const TilePixel& px,
-                                                     uint32_t t_start, bool wave_active, float4* stage, int4* boxes,
-                                                     int32_t* ids, uint8_t* wave_list) {
+                                                     uint32_t t_start, bool wave_active, float4* stage, float4* region,
+                                                     float* cuts, int32_t* ids, uint8_t* wave_list) {
     if (tr < count) {
         const int32_t g = flatten_ids[first + step * (int32_t)tr];
-        const float4* __restrict__ r = records + (size_t)g * 5;
-        const float4 r0 = r[0], r1 = r[1], r2 = r[2], r3 = r[3], r4 = r[4];
+        const float4* __restrict__ r = records + (size_t)g * kRecordF4;
+        const float4 r0 = r[0], r1 = r[1], r2 = r[2], r3 = r[3], r4 = r[4], r5 = r[5];
         stage[tr * 4 + 0] = r0;
         stage[tr * 4 + 1] = r1;
         stage[tr * 4 + 2] = r2;
         stage[tr * 4 + 3] = r3;
-        boxes[tr] = make_int4((int)f2u(r4.x), (int)f2u(r4.y), (int)f2u(r4.z), (int)f2u(r4.w));
+        region[tr * 2 + 0] = r4;
+        region[tr * 2 + 1] = r5;
+        cuts[tr] = r4.z;
         if (ids != nullptr)
             ids[tr] = g;
     }
@@ -146,8 +163,10 @@ __device__ __forceinline__ uint32_t stage_and_select(const float4* __restrict__ 
             const uint32_t t = r * 64u + lane;
             bool hit = false;
             if (t < count && t >= t_start) {
-                const int4 b = boxes[t];
-                hit = b.x <= px.wj0 + 7 && b.z >= px.wj0 && b.y <= px.wi0 + 7 && b.w >= px.wi0;
+                const float4 q0 = region[t * 2 + 0], q1 = region[t * 2 + 1];
+                const uint32_t jb = f2u(q0.x), ib = f2u(q0.y);
+                hit = record_region_hits_block((int32_t)(jb & 0xffffu), (int32_t)(ib & 0xffffu), (int32_t)(jb >> 16),
+                                               (int32_t)(ib >> 16), q0.w, q1.x, q1.y, q1.z, q1.w, px.wi0, px.wj0);
             }
             const uint64_t m = __builtin_amdgcn_ballot_w64(hit);
             if (hit) {

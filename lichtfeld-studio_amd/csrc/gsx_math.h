@@ -79,6 +79,23 @@ GSX_HD float exp(float x) {
     return y;
 }
 
+// gsx::exp restricted to -87 <= x <= 0, where its two range tests never fire and its two-step scaling is a single
+// exact multiplication by 2^n (n in [-126, 0]): the same bits for fewer instructions.
+GSX_HD float exp_nonpos(float x) {
+    const float n = __builtin_rintf(x * 1.44269504088896341f);
+    float r = fma(n, -0.693359375f, x);
+    r = fma(n, 2.12194440e-4f, r);
+    float p = 1.9875691500e-4f;
+    p = fma(p, r, 1.3981999507e-3f);
+    p = fma(p, r, 8.3334519073e-3f);
+    p = fma(p, r, 4.1665795894e-2f);
+    p = fma(p, r, 1.6666665459e-1f);
+    p = fma(p, r, 5.0000001201e-1f);
+    const float z = r * r;
+    const float y = fma(p, z, r) + 1.0f;
+    return y * u2f((uint32_t)((int)n + 127) << 23);
+}
+
 // natural log of a positive normal float (Cephes logf scheme).
 GSX_HD float log(float x) {
     uint32_t ix = f2u(x);

@@ -99,7 +99,8 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     const float* __restrict__ v_render_colors, const float* __restrict__ v_render_alphas,
     float* __restrict__ gacc /*[N,16]*/) {
     __shared__ float4 stage[kBatch * 4];
-    __shared__ int4 boxes[kBatch];
+    __shared__ float4 region[kBatch * 2];
+    __shared__ float cuts[kBatch];
     __shared__ uint8_t lists[4][kBatch];
     __shared__ int32_t id_batch[kBatch];
     __shared__ float acc[kBatch * kAcc];
@@ -145,6 +146,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1)
         wave_bin_final = max(wave_bin_final, __shfl_xor(wave_bin_final, m, 64));
+    wave_bin_final = __builtin_amdgcn_readfirstlane(wave_bin_final); // the same in every lane: keep it scalar
     if (tr == 0)
         block_max = 0;
     __syncthreads();
@@ -165,9 +167,9 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
         const int32_t batch_size = min((int32_t)kBatch, batch_end + 1 - range_start);
         // slots in front of t_start lie behind every last contributor of this wave
         const uint32_t t_start = (uint32_t)max(0, batch_end - wave_bin_final);
-        const uint32_t n_sel = stage_and_select(records, flatten_ids, batch_end, -1, (uint32_t)batch_size, tr, px,
-                                                t_start, t_start < (uint32_t)batch_size, stage, boxes, id_batch,
-                                                wave_list);
+        const uint32_t n_sel = (uint32_t)__builtin_amdgcn_readfirstlane((int)stage_and_select(
+            records, flatten_ids, batch_end, -1, (uint32_t)batch_size, tr, px, t_start,
+            t_start < (uint32_t)batch_size, stage, region, cuts, id_batch, wave_list));
 
         for (uint32_t sidx = 0; sidx < n_sel; ++sidx) {
             const int32_t t = (int32_t)wave_list[sidx];
@@ -180,65 +182,71 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             const vec3 grd = mk3(fma(m0.z, ray_d.z, fma(m0.y, ray_d.y, m0.x * ray_d.x)),
                                  fma(m1.y, ray_d.z, fma(m1.x, ray_d.y, m0.w * ray_d.x)),
                                  fma(m2.x, ray_d.z, fma(m1.w, ray_d.y, m1.z * ray_d.x)));
-            const vec3 grd_n = safe_normalize(grd);
+            // safe_normalize without a branch: the reciprocal length is reused by the VJP below
+            const float l2 = dot(grd, grd);
+            const float il_any = gsx::rsqrt(l2);
+            const float il = l2 > 0.0f ? il_any : 1.0f;
+            const vec3 grd_n = scale(grd, il);
             const vec3 gcrod = cross(grd_n, gro);
             const float grayDist = dot(gcrod, gcrod);
             const float power = -0.5f * grayDist;
-            // exp(power) < 1/255 below kPowerCut, so alpha < 1/255 for any opacity <= 1: decided without the exp
-            if (power < kPowerCut && a.w <= 1.0f)
+            // below the record's cut-off alpha < 1/255 whatever the rounding: decided without the exp
+            if (power < cuts[t])
                 valid = false;
             if (__builtin_amdgcn_ballot_w64(valid) == 0)
                 continue;
-            const float vis = gsx::exp(power);
+            const float vis = gsx::exp_nonpos(gsx::fmax(power, kPowerFloor)); // lanes that are not valid may be far
             const float alpha = gsx::fmin(0.999f, a.w * vis);
             if (power > 0.f || alpha < 1.f / 255.f)
                 valid = false;
             if (__builtin_amdgcn_ballot_w64(valid) == 0)
                 continue; // no lane of this wave sees the Gaussian (:286-289)
 
+            // From here on without branches: a lane that is not valid carries ra = 1 and fac = v_alpha = 0, which
+            // leaves its T and colour buffer unchanged and makes all 16 of its partials zero.  The decisions above
+            // use the forward pass's exact arithmetic; the derivative chain may use the hardware reciprocal.
             float v[kAcc];
-#pragma unroll
-            for (uint32_t k = 0; k < kAcc; ++k)
-                v[k] = 0.f;
-            if (valid) {
-                const float ra = 1.0f / (1.0f - alpha);
-                T *= ra;
-                const float fac = alpha * T;
-                v[0] = fac * v_render_c[0];
-                v[1] = fac * v_render_c[1];
-                v[2] = fac * v_render_c[2];
-                float v_alpha = 0.f;
-                v_alpha += (m2.y * T - buffer[0] * ra) * v_render_c[0];
-                v_alpha += (m2.z * T - buffer[1] * ra) * v_render_c[1];
-                v_alpha += (m2.w * T - buffer[2] * ra) * v_render_c[2];
-                v_alpha += T_final * ra * v_render_a;
-                if (backgrounds != nullptr)
-                    v_alpha += -T_final * ra * bg_dot;
-                if (a.w * vis <= 0.999f) {
-                    const float v_vis = a.w * v_alpha;
-                    const float v_gradDist = -0.5f * vis * v_vis;
-                    const vec3 v_gcrod = scale(gcrod, 2.0f * v_gradDist);
-                    const vec3 v_grd_n = neg(cross(v_gcrod, gro));
-                    const vec3 v_gro = cross(v_gcrod, grd_n);
-                    const vec3 v_grd = safe_normalize_bw(grd, v_grd_n);
-                    v[3] = v_gro.x;
-                    v[4] = v_gro.y;
-                    v[5] = v_gro.z;
-                    v[6] = v_grd.x * ray_d.x;
-                    v[7] = v_grd.x * ray_d.y;
-                    v[8] = v_grd.x * ray_d.z;
-                    v[9] = v_grd.y * ray_d.x;
-                    v[10] = v_grd.y * ray_d.y;
-                    v[11] = v_grd.y * ray_d.z;
-                    v[12] = v_grd.z * ray_d.x;
-                    v[13] = v_grd.z * ray_d.y;
-                    v[14] = v_grd.z * ray_d.z;
-                    v[15] = vis * v_alpha;
-                }
-                buffer[0] += m2.y * fac;
-                buffer[1] += m2.z * fac;
-                buffer[2] += m2.w * fac;
-            }
+            const float ra = valid ? __builtin_amdgcn_rcpf(1.0f - alpha) : 1.0f;
+            T *= ra;
+            const float fac = valid ? alpha * T : 0.f;
+            v[0] = fac * v_render_c[0];
+            v[1] = fac * v_render_c[1];
+            v[2] = fac * v_render_c[2];
+            float v_alpha = 0.f;
+            v_alpha += (m2.y * T - buffer[0] * ra) * v_render_c[0];
+            v_alpha += (m2.z * T - buffer[1] * ra) * v_render_c[1];
+            v_alpha += (m2.w * T - buffer[2] * ra) * v_render_c[2];
+            v_alpha += T_final * ra * v_render_a;
+            if (backgrounds != nullptr)
+                v_alpha += -T_final * ra * bg_dot;
+            // the clamp at 0.999 has zero derivative (:322)
+            v_alpha = (valid && a.w * vis <= 0.999f) ? v_alpha : 0.f;
+            const float v_vis = a.w * v_alpha;
+            const float v_gradDist = -0.5f * vis * v_vis;
+            const vec3 v_gcrod = scale(gcrod, 2.0f * v_gradDist);
+            const vec3 v_grd_n = neg(cross(v_gcrod, gro));
+            const vec3 v_gro = cross(v_gcrod, grd_n);
+            // VJP of safe_normalize (Utils.cuh:186-194) with the reciprocal length from above
+            const float il3 = il * il * il;
+            const float sdot = il3 * dot(v_grd_n, grd);
+            const vec3 v_grd = mk3(fma(il, v_grd_n.x, -(sdot * grd.x)), fma(il, v_grd_n.y, -(sdot * grd.y)),
+                                   fma(il, v_grd_n.z, -(sdot * grd.z)));
+            v[3] = v_gro.x;
+            v[4] = v_gro.y;
+            v[5] = v_gro.z;
+            v[6] = v_grd.x * ray_d.x;
+            v[7] = v_grd.x * ray_d.y;
+            v[8] = v_grd.x * ray_d.z;
+            v[9] = v_grd.y * ray_d.x;
+            v[10] = v_grd.y * ray_d.y;
+            v[11] = v_grd.y * ray_d.z;
+            v[12] = v_grd.z * ray_d.x;
+            v[13] = v_grd.z * ray_d.y;
+            v[14] = v_grd.z * ray_d.z;
+            v[15] = vis * v_alpha;
+            buffer[0] += m2.y * fac;
+            buffer[1] += m2.z * fac;
+            buffer[2] += m2.w * fac;
             const float total = wave_reduce16(v, lane);
             if ((lane & 3u) == 0) {
                 const uint32_t comp = ((lane >> 5) & 1u) * 8u + ((lane >> 4) & 1u) * 4u + ((lane >> 3) & 1u) * 2u +

@@ -2,7 +2,7 @@
 //
 // One 256-lane workgroup (four 64-lane waves) per 16x16 tile, one lane per pixel; every wave owns an 8x8 pixel
 // block.  What a (pixel, Gaussian) pair needs from the Gaussian - M = diag(1/scale) R(quat)^T, gro = M (ray_o -
-// mean), opacity, colour - does not depend on the tile, so it is built once per Gaussian as an 80-byte record
+// mean), opacity, colour - does not depend on the tile, so it is built once per Gaussian as a 96-byte record
 // (gsx_record.h) by pack_records_kernel (or by the fused per-Gaussian pass of a training step) instead of once per
 // tile the Gaussian touches.  The tile's depth-sorted records are staged through LDS 256 at a time; every wave
 // then keeps the slots whose exact pixel bounds meet its 8x8 block (ballot + prefix count, order preserved) and
@@ -32,21 +32,17 @@ __global__ void __launch_bounds__(256) pack_records_kernel(uint32_t N, const flo
     const float opac = opacities[g];
     const mat3 M = record_whitening(ld4q(quats, g), ld3(scales, g));
     const vec3 gro = mul(M, sub(ray_o, xyz));
-    const RecordBounds b = record_bounds(gro, M, opac, xyz, viewmat, Kmat[0], Kmat[4], Kmat[2], Kmat[5], W, H);
+    const RecordRegion b = record_region(gro, M, opac, xyz, viewmat, Kmat[0], Kmat[4], Kmat[2], Kmat[5], W, H);
     const float c0 = colors[(size_t)g * CDIM];
     const float c1 = CDIM > 1 ? colors[(size_t)g * CDIM + 1] : 0.f;
     const float c2 = CDIM > 2 ? colors[(size_t)g * CDIM + 2] : 0.f;
-    float4* __restrict__ r = records + (size_t)g * 5;
-    r[0] = make_float4(gro.x, gro.y, gro.z, opac);
-    r[1] = make_float4(M.m[0][0], M.m[0][1], M.m[0][2], M.m[1][0]);
-    r[2] = make_float4(M.m[1][1], M.m[1][2], M.m[2][0], M.m[2][1]);
-    r[3] = make_float4(M.m[2][2], c0, c1, c2);
-    r[4] = make_float4(u2f((uint32_t)b.jmin), u2f((uint32_t)b.imin), u2f((uint32_t)b.jmax), u2f((uint32_t)b.imax));
+    store_record(records + (size_t)g * kRecordF4, gro, opac, M, c0, c1, c2, b);
 }
 
 // STATS: count instead of rendering (for roofline accounting); stats[0] += (pixel, Gaussian) pairs evaluated,
 // [1] += pairs composited, [2] += pairs the backward pass walks (entries up to each pixel's last contributor),
-// [3] += (wave, Gaussian) iterations executed, [4] += (wave, Gaussian) iterations removed by the pixel bounds.
+// [3] += (wave, Gaussian) iterations executed, [4] += (wave, Gaussian) iterations removed by the pixel bounds,
+// [5] += executed iterations in which at least one pixel reaches the alpha threshold.
 template <uint32_t CDIM, bool STATS>
 __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
     uint32_t n_isects, const float4* __restrict__ records, const float* __restrict__ colors,
@@ -56,7 +52,8 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
     const int32_t* __restrict__ flatten_ids, float* __restrict__ render_colors, float* __restrict__ render_alphas,
     int32_t* __restrict__ last_ids, unsigned long long* __restrict__ stats) {
     __shared__ float4 stage[kBatch * 4];
-    __shared__ int4 boxes[kBatch];
+    __shared__ float4 region[kBatch * 2];
+    __shared__ float cuts[kBatch];
     __shared__ uint8_t lists[4][kBatch];
     __shared__ int32_t ids[CDIM > 3 ? kBatch : 1];
     __shared__ float extra[CDIM > 3 ? kBatch * (CDIM - 3) : 1]; // channels beyond the third
@@ -95,7 +92,7 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
 #pragma unroll
     for (uint32_t k = 0; k < CDIM; ++k)
         pix_out[k] = 0.f;
-    uint32_t n_eval = 0, n_comp = 0, n_iter = 0, n_skip = 0;
+    uint32_t n_eval = 0, n_comp = 0, n_iter = 0, n_skip = 0, n_hit = 0;
 
     for (uint32_t b = 0; b < num_batches; ++b) {
         // all four waves saturated: nothing left to stage (:190-194)
@@ -105,7 +102,8 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
         const uint32_t batch_size = min(kBatch, (uint32_t)range_end - batch_start);
         const bool wave_active = __builtin_amdgcn_ballot_w64(!done) != 0;
         const uint32_t n_sel = stage_and_select(records, flatten_ids, (int32_t)batch_start, 1, batch_size, tr, px, 0u,
-                                                wave_active, stage, boxes, CDIM > 3 ? ids : nullptr, wave_list);
+                                                wave_active, stage, region, cuts, CDIM > 3 ? ids : nullptr,
+                                                wave_list);
         if (CDIM > 3) {
             if (tr < batch_size) {
 #pragma unroll
@@ -136,15 +134,25 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
             const vec3 gd = mk3(fma(m0.z, ray_d.z, fma(m0.y, ray_d.y, m0.x * ray_d.x)),
                                 fma(m1.y, ray_d.z, fma(m1.x, ray_d.y, m0.w * ray_d.x)),
                                 fma(m2.x, ray_d.z, fma(m1.w, ray_d.y, m1.z * ray_d.x)));
-            const vec3 grd = safe_normalize(gd);
+            // safe_normalize (Utils.cuh:181-184) as a select instead of a branch
+            const float l2 = dot(gd, gd);
+            const float il_any = gsx::rsqrt(l2);
+            const vec3 grd = scale(gd, l2 > 0.0f ? il_any : 1.0f);
             const vec3 gcrod = cross(grd, gro);
             const float grayDist = dot(gcrod, gcrod);
             const float power = -0.5f * grayDist;
-            // exp(power) < 1/255 below kPowerCut, so alpha < 1/255 for any opacity <= 1: decided without the exp
-            const bool far_away = power < kPowerCut && a.w <= 1.0f;
+            // below the record's cut-off alpha < 1/255 whatever the rounding: decided without the exp
+            const bool far_away = power < cuts[t];
+            if (STATS) {
+                const bool contributes = !far_away && gsx::fmin(0.999f, a.w * gsx::exp_nonpos(power)) >= 1.f / 255.f;
+                const uint64_t act = __builtin_amdgcn_ballot_w64(true);
+                if (__builtin_amdgcn_ballot_w64(contributes) != 0 &&
+                    (act & ((1ull << (tr & 63u)) - 1ull)) == 0) // first active lane counts for the wave
+                    ++n_hit;
+            }
             if (__builtin_amdgcn_ballot_w64(!far_away) == 0 || far_away)
                 continue;
-            const float alpha = gsx::fmin(0.999f, a.w * gsx::exp(power));
+            const float alpha = gsx::fmin(0.999f, a.w * gsx::exp_nonpos(power)); // cut <= power <= 0
             if (alpha < 1.f / 255.f)
                 continue;
             const float next_T = T * (1.0f - alpha);
@@ -178,6 +186,7 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
             atomicAdd(&stats[3], (unsigned long long)n_iter);
             atomicAdd(&stats[4], (unsigned long long)n_skip);
         }
+        atomicAdd(&stats[5], (unsigned long long)n_hit);
         return;
     }
 

@@ -1626,9 +1626,11 @@ ORC_API void orc_set_num_threads(int n) {
 
 ORC_API int orc_record_bounds_check(uint32_t N, const float* means, const float* quats, const float* scales,
                                     const float* opacities, const float* viewmat, const float* Ks, uint32_t W,
-                                    uint32_t H, int32_t* bounds, int64_t* true_count, int64_t* violations) {
+                                    uint32_t H, int32_t* bounds, int64_t* true_count, int64_t* violations,
+                                    int64_t* blocks_true, int64_t* blocks_hit) {
     const float fx = Ks[0], fy = Ks[4], cx = Ks[2], cy = Ks[5];
     const RollingShutter rs = make_rolling_shutter(viewmat, nullptr);
+    const uint32_t bw = (W + 7) / 8, bh = (H + 7) / 8;
 #pragma omp parallel for schedule(dynamic, 1)
     for (int64_t g = 0; g < (int64_t)N; ++g) {
         vec3 ray_o, ray_d;
@@ -1636,9 +1638,10 @@ ORC_API int orc_record_bounds_check(uint32_t N, const float* means, const float*
         const vec3 xyz = ld3(means, g);
         const mat3 M = gsx::record_whitening(ld4(quats, g), ld3(scales, g));
         const vec3 gro = gsx::mul(M, gsx::sub(ray_o, xyz));
-        const gsx::RecordBounds b = gsx::record_bounds(gro, M, opacities[g], xyz, viewmat, fx, fy, cx, cy, W, H);
+        const gsx::RecordRegion b = gsx::record_region(gro, M, opacities[g], xyz, viewmat, fx, fy, cx, cy, W, H);
         bounds[g * 4 + 0] = b.jmin, bounds[g * 4 + 1] = b.imin, bounds[g * 4 + 2] = b.jmax, bounds[g * 4 + 3] = b.imax;
-        int64_t cnt = 0, bad = 0;
+        int64_t cnt = 0, bad = 0, bt = 0, bhit = 0;
+        std::vector<uint8_t> block_has(bw * bh, 0);
         for (uint32_t i = 0; i < H; ++i)
             for (uint32_t j = 0; j < W; ++j) {
                 pixel_world_ray((float)j + 0.5f, (float)i + 0.5f, fx, fy, cx, cy, rs, &ray_o, &ray_d);
@@ -1649,11 +1652,25 @@ ORC_API int orc_record_bounds_check(uint32_t N, const float* means, const float*
                 if (alpha < 1.f / 255.f)
                     continue;
                 ++cnt;
+                block_has[(i / 8) * bw + j / 8] = 1;
                 if ((int32_t)j < b.jmin || (int32_t)j > b.jmax || (int32_t)i < b.imin || (int32_t)i > b.imax)
+                    ++bad;
+                if (power < b.cut)
+                    ++bad; // the cut-off must lie below every contributing pair's power
+            }
+        for (uint32_t by = 0; by < bh; ++by)
+            for (uint32_t bx = 0; bx < bw; ++bx) {
+                const bool hit = gsx::record_region_hits_block(b.jmin, b.imin, b.jmax, b.imax, b.a00, b.a01, b.a11,
+                                                               b.pcx, b.pcy, (int32_t)(by * 8), (int32_t)(bx * 8));
+                bhit += hit;
+                bt += block_has[by * bw + bx];
+                if (block_has[by * bw + bx] && !hit)
                     ++bad;
             }
         true_count[g] = cnt;
         violations[g] = bad;
+        blocks_true[g] = bt;
+        blocks_hit[g] = bhit;
     }
     return 0;
 }

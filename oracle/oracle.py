@@ -422,15 +422,16 @@ def math_quat(which, inp, n_out):
 
 
 def record_bounds_check(means, quats, scales, opacities, viewmat, K, W, H):
-    """Per-Gaussian pixel bounds of the rasterizers (csrc/gsx_record.h) and a brute-force count, over every pixel of
-    the image, of the pixels that reach alpha >= 1/255 -> (bounds [N,4] = jmin, imin, jmax, imax; true_count [N];
-    violations [N] = contributing pixels outside the bounds)."""
+    """Per-Gaussian contribution region of the rasterizers (csrc/gsx_record.h: pixel bounds, power cut-off, ellipse
+    test per 8x8 block) against a brute-force pass over every pixel of the image -> (bounds [N,4] = jmin, imin, jmax,
+    imax; true_count [N] pixels with alpha >= 1/255; violations [N] = contributing pixels outside the bounds or below
+    the cut-off + contributing blocks the block test rejects; blocks_true [N]; blocks_hit [N])."""
     means, quats, scales, opacities = _f32(means), _f32(quats), _f32(scales), _f32(opacities)
     viewmat, K = _f32(viewmat), _f32(K)
     N = means.shape[0]
     bounds = np.zeros((N, 4), np.int32)
-    cnt = np.zeros(N, np.int64)
-    bad = np.zeros(N, np.int64)
+    cnt, bad, bt, bh = (np.zeros(N, np.int64) for _ in range(4))
     _chk(lib().orc_record_bounds_check(c_u32(N), _p(means), _p(quats), _p(scales), _p(opacities), _p(viewmat), _p(K),
-                                       c_u32(W), c_u32(H), _p(bounds), _p(cnt), _p(bad)), "record_bounds_check")
-    return bounds, cnt, bad
+                                       c_u32(W), c_u32(H), _p(bounds), _p(cnt), _p(bad), _p(bt), _p(bh)),
+         "record_bounds_check")
+    return bounds, cnt, bad, bt, bh

@@ -62,6 +62,7 @@ def test_math_primitives_bit_exact(gsx, orc, cuda):
         8: (rng.normal(0, 100, n), np.exp(rng.uniform(-30, 30, n)), "div"),
         9: (np.exp(rng.uniform(-80, 80, n)), np.ones(n), "sqrt"),
         10: (rng.normal(0, 1, n), rng.normal(0, 1, n), "fma"),
+        11: (np.concatenate([rng.uniform(-87, 0, n - 3), [0.0, -87.0, -1e-30]]), None, "exp"),  # restricted variant
     }
     for which, (x, x2, name) in cases.items():
         x = x.astype(np.float32)
@@ -72,7 +73,7 @@ def test_math_primitives_bit_exact(gsx, orc, cuda):
                                        ctypes.c_void_p(None if x2d is None else x2d.data_ptr()),
                                        ctypes.c_void_p(y.data_ptr()), ctypes.c_void_p(None)))
         torch.cuda.synchronize()
-        ref = orc.math_unary(name, x) if which < 7 else orc.math_binary(name, x, x2.astype(np.float32))
+        ref = orc.math_unary(name, x) if x2 is None else orc.math_binary(name, x, x2.astype(np.float32))
         got = N(y)
         bits_equal(got, ref, name)
 

@@ -219,10 +219,13 @@ def test_record_pixel_bounds_are_conservative(gsx, orc, trial):
     scales = np.exp(log_s).astype(np.float32)
     quats = rng.normal(0, 1, (n, 4)).astype(np.float32)
     op = np.exp(rng.uniform(np.log(1 / 300), 0, n)).astype(np.float32)
-    bounds, count, outside = orc.record_bounds_check(means, quats, scales, op, cam.viewmat, cam.K, W, H)
-    assert outside.sum() == 0, f"{(outside > 0).sum()} Gaussians have contributing pixels outside their bounds"
+    bounds, count, outside, blocks_true, blocks_hit = orc.record_bounds_check(means, quats, scales, op, cam.viewmat,
+                                                                              cam.K, W, H)
+    assert outside.sum() == 0, f"{(outside > 0).sum()} Gaussians have contributing pixels outside their region"
     assert (count > 0).sum() > 100  # the case is not vacuous
     box = np.maximum(bounds[:, 2] - bounds[:, 0] + 1, 0) * np.maximum(bounds[:, 3] - bounds[:, 1] + 1, 0)
     proper = box < W * H
     assert box[proper].sum() < 3.0 * max(count[proper].sum(), 1) + 16 * proper.sum()  # and they are tight
     assert (box[op < 1 / 256] == 0).all()  # below the alpha threshold: empty
+    assert (blocks_hit >= blocks_true).all()
+    assert blocks_hit[proper].sum() < 2.5 * blocks_true[proper].sum() + 6 * proper.sum()  # 8x8 block test is tight
