@@ -51,13 +51,14 @@ def load_package():
 def algorithmic_bytes(N, K, H, W, n_isects, sort_bits):
     """HBM bytes one launch of each streaming stage has to move (reads + writes), per the cost model."""
     P = H * W
-    passes = (sort_bits + 7) // 8
+    passes = (sort_bits - 32 + 7) // 8  # the pairs are emitted in depth order: only the tile / camera bits are sorted
     return {
         "activate_params": N * (32 + 32),
         "projection_ut_3dgs_fused": N * (44 + 32),
         "sh_colors_from_world": N * (12 + 12 * K + 8 + 12),
-        "intersect_tile_count": N * (16 + 4 + 4 + 8 + 4),
-        "intersect_tile_emit": N * (16 + 4 + 8) + n_isects * 12,
+        "intersect_tile_count": N * (4 + 16 + 4 + 4 + 4 + 8 + 4),
+        "intersect_tile_emit": N * (4 + 16 + 4 + 8) + n_isects * 12,
+        "depth_order": N * (12 + 12 + (8 + 24) * 4),
         "radix_sort_pairs": n_isects * (8 + 24) * passes,
         "intersect_offset": n_isects * 8 + (P // 256) * 4,
         "image_from_render": P * (12 + 12 + 12),

@@ -97,27 +97,40 @@ GSX_API int gsx_spherical_harmonics_bwd(uint32_t N, uint32_t K, uint32_t degrees
 
 /* ---- a4: gsplat::intersect_tile (Ops.h:28-38; Intersect.cpp:15-122; IntersectTile.cu:23-114) ----
  * Two calls, as the reference's two passes: count (+ inclusive scan; blocks until the total is on the
- * host, like Intersect.cpp:76) then emit.  cum_tiles_per_gauss is i64 [C*N]. */
+ * host, like Intersect.cpp:76) then emit.  cum_tiles_per_gauss is i64 [C*N].
+ *
+ * `order` (i32 [N], nullable, C == 1 only) visits the Gaussians in that order instead of by index: position i is
+ * Gaussian order[i], cum_tiles_per_gauss is the prefix sum over POSITIONS and the pairs are emitted position by
+ * position (tiles_per_gauss stays indexed by Gaussian).  With order = gsx_depth_order(...) the emitted pairs are
+ * already sorted by (depth bits, Gaussian index), so the sorted list the reference obtains from one radix sort on
+ * all 32 + tile + camera bits (Intersect.cpp:104-113) is reached by sorting on the tile / camera bits alone
+ * (gsx_radix_sort_pairs with begin_bit = 32): the sort is stable, the result is the same array bit for bit, and
+ * four of its six passes run over N Gaussians instead of n_isects pairs. */
 GSX_API size_t gsx_intersect_tile_count_workspace_bytes(uint32_t C, uint32_t N);
 GSX_API int gsx_intersect_tile_count(uint32_t C, uint32_t N, const float* means2d, const int32_t* radii,
                                      uint32_t tile_size, uint32_t tile_width, uint32_t tile_height,
-                                     int32_t* tiles_per_gauss, int64_t* cum_tiles_per_gauss, void* workspace,
-                                     size_t workspace_bytes, int64_t* n_isects_host, void* stream);
+                                     const int32_t* order, int32_t* tiles_per_gauss, int64_t* cum_tiles_per_gauss,
+                                     void* workspace, size_t workspace_bytes, int64_t* n_isects_host, void* stream);
 GSX_API int gsx_intersect_tile_emit(uint32_t C, uint32_t N, const float* means2d, const int32_t* radii,
-                                    const float* depths, const int64_t* cum_tiles_per_gauss, uint32_t tile_size,
-                                    uint32_t tile_width, uint32_t tile_height, int64_t* isect_ids,
+                                    const float* depths, const int64_t* cum_tiles_per_gauss, const int32_t* order,
+                                    uint32_t tile_size, uint32_t tile_width, uint32_t tile_height, int64_t* isect_ids,
                                     int32_t* flatten_ids, void* stream);
+/* order[i] = index of the Gaussian with the i-th smallest depth bit pattern (ties by index; Gaussians with
+ * radii == 0 last).  One camera. */
+GSX_API size_t gsx_depth_order_workspace_bytes(uint32_t N);
+GSX_API int gsx_depth_order(uint32_t N, const float* depths, const int32_t* radii, int32_t* order, void* workspace,
+                            size_t workspace_bytes, void* stream);
 /* Intersect.cpp:46-47: floor(log2(n)) + 1 */
 GSX_API uint32_t gsx_n_bits(uint32_t n);
 
 /* ---- a5: gsplat::radix_sort_double_buffer (Intersect.h:39-46; IntersectTile.cu:290-328) ----
- * Stable ascending LSD radix sort of (i64 key, i32 value) pairs on key bits [0, end_bit).
- * Buffers 0 (keys0/vals0, the input) and 1 (keys1/vals1) are ping-ponged; *selector_host (host int)
- * says which pair holds the result (like cub::DoubleBuffer::selector). */
+ * Stable ascending LSD radix sort of (i64 key, i32 value) pairs on key bits [begin_bit, end_bit) (the reference
+ * passes begin_bit = 0).  Buffers 0 (keys0/vals0, the input) and 1 (keys1/vals1) are ping-ponged; *selector_host
+ * (host int) says which pair holds the result (like cub::DoubleBuffer::selector). */
 GSX_API size_t gsx_radix_sort_pairs_workspace_bytes(int64_t n);
 GSX_API int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, int64_t* keys1, int32_t* vals1,
-                                 uint32_t end_bit, void* workspace, size_t workspace_bytes, int* selector_host,
-                                 void* stream);
+                                 uint32_t begin_bit, uint32_t end_bit, void* workspace, size_t workspace_bytes,
+                                 int* selector_host, void* stream);
 
 /* ---- a6: gsplat::intersect_offset (Ops.h:39-43; IntersectTile.cu:206-286) -> offsets i32 [C,Th,Tw] ---- */
 GSX_API int gsx_intersect_offset(int64_t n_isects, const int64_t* isect_ids, uint32_t C, uint32_t tile_width,

@@ -92,22 +92,35 @@ std::tuple<at::Tensor, at::Tensor> spherical_harmonics_bwd(const uint32_t K, con
     return std::make_tuple(v_coeffs, v_dirs);
 }
 
+namespace {
+void sort_pairs(const int64_t n_isects, const uint32_t begin_bit, const uint32_t end_bit, at::Tensor& isect_ids,
+                at::Tensor& flatten_ids, at::Tensor& isect_ids_sorted, at::Tensor& flatten_ids_sorted);
+}
+
 void radix_sort_double_buffer(const int64_t n_isects, const uint32_t tile_n_bits, const uint32_t cam_n_bits,
                               at::Tensor isect_ids, at::Tensor flatten_ids, at::Tensor isect_ids_sorted,
                               at::Tensor flatten_ids_sorted) {
+    sort_pairs(n_isects, 0, 32 + tile_n_bits + cam_n_bits, isect_ids, flatten_ids, isect_ids_sorted,
+               flatten_ids_sorted);
+}
+
+namespace {
+void sort_pairs(const int64_t n_isects, const uint32_t begin_bit, const uint32_t end_bit, at::Tensor& isect_ids,
+                at::Tensor& flatten_ids, at::Tensor& isect_ids_sorted, at::Tensor& flatten_ids_sorted) {
     if (n_isects <= 0)
         return;
     at::Tensor ws = workspace(gsx_radix_sort_pairs_workspace_bytes(n_isects), isect_ids);
     int selector = 0;
     gsx_check(gsx_radix_sort_pairs(n_isects, isect_ids.data_ptr<int64_t>(), flatten_ids.data_ptr<int32_t>(),
                                    isect_ids_sorted.data_ptr<int64_t>(), flatten_ids_sorted.data_ptr<int32_t>(),
-                                   32 + tile_n_bits + cam_n_bits, ws.data_ptr(), (size_t)ws.numel(), &selector,
+                                   begin_bit, end_bit, ws.data_ptr(), (size_t)ws.numel(), &selector,
                                    cur_stream(isect_ids)));
     if (selector == 0) { // sorted items ended up in the input buffers (IntersectTile.cu:315-328)
         isect_ids_sorted.set_(isect_ids);
         flatten_ids_sorted.set_(flatten_ids);
     }
 }
+} // namespace
 
 std::tuple<at::Tensor, at::Tensor, at::Tensor> intersect_tile(const at::Tensor means2d, const at::Tensor radii,
                                                               const at::Tensor depths, const OptT camera_ids,
@@ -128,26 +141,38 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> intersect_tile(const at::Tensor m
     const uint32_t tile_n_bits = gsx_n_bits(tile_width * tile_height);
     const uint32_t cam_n_bits = gsx_n_bits(C);
     at::Tensor tiles_per_gauss = at::empty_like(depths, depths.options().dtype(at::kInt));
+    // one camera, sorted output: visit the Gaussians in depth order and sort on the tile bits only (same array as
+    // one sort on every bit, Intersect.cpp:104-113, because the sort is stable)
+    const bool two_level = sort && C == 1;
+    at::Tensor order;
+    const int32_t* order_ptr = nullptr;
+    if (two_level && N > 0) {
+        order = at::empty({(int64_t)N}, depths.options().dtype(at::kInt));
+        at::Tensor ws_o = workspace(gsx_depth_order_workspace_bytes(N), depths);
+        gsx_check(gsx_depth_order(N, depths.data_ptr<float>(), radii.data_ptr<int32_t>(), order.data_ptr<int32_t>(),
+                                  ws_o.data_ptr(), (size_t)ws_o.numel(), cur_stream(means2d)));
+        order_ptr = order.data_ptr<int32_t>();
+    }
     at::Tensor cum = at::empty({(int64_t)C * N}, depths.options().dtype(at::kLong));
     at::Tensor ws = workspace(gsx_intersect_tile_count_workspace_bytes(C, N), depths);
     int64_t n_isects = 0;
     void* stream = cur_stream(means2d);
     gsx_check(gsx_intersect_tile_count(C, N, means2d.data_ptr<float>(), radii.data_ptr<int32_t>(), tile_size,
-                                       tile_width, tile_height, tiles_per_gauss.data_ptr<int32_t>(),
+                                       tile_width, tile_height, order_ptr, tiles_per_gauss.data_ptr<int32_t>(),
                                        cum.data_ptr<int64_t>(), ws.data_ptr(), (size_t)ws.numel(), &n_isects, stream));
     at::Tensor isect_ids = at::empty({n_isects}, depths.options().dtype(at::kLong));
     at::Tensor flatten_ids = at::empty({n_isects}, depths.options().dtype(at::kInt));
     if (n_isects) {
         gsx_check(gsx_intersect_tile_emit(C, N, means2d.data_ptr<float>(), radii.data_ptr<int32_t>(),
-                                          depths.data_ptr<float>(), cum.data_ptr<int64_t>(), tile_size, tile_width,
-                                          tile_height, isect_ids.data_ptr<int64_t>(), flatten_ids.data_ptr<int32_t>(),
-                                          stream));
+                                          depths.data_ptr<float>(), cum.data_ptr<int64_t>(), order_ptr, tile_size,
+                                          tile_width, tile_height, isect_ids.data_ptr<int64_t>(),
+                                          flatten_ids.data_ptr<int32_t>(), stream));
     }
     if (n_isects && sort) {
         at::Tensor isect_ids_sorted = at::empty_like(isect_ids);
         at::Tensor flatten_ids_sorted = at::empty_like(flatten_ids);
-        radix_sort_double_buffer(n_isects, tile_n_bits, cam_n_bits, isect_ids, flatten_ids, isect_ids_sorted,
-                                 flatten_ids_sorted);
+        sort_pairs(n_isects, two_level ? 32u : 0u, 32 + tile_n_bits + cam_n_bits, isect_ids, flatten_ids,
+                   isect_ids_sorted, flatten_ids_sorted);
         return std::make_tuple(tiles_per_gauss, isect_ids_sorted, flatten_ids_sorted);
     }
     return std::make_tuple(tiles_per_gauss, isect_ids, flatten_ids);

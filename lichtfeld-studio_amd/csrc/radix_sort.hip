@@ -1,10 +1,11 @@
-// radix_sort.hip - stable LSD radix sort of (int64 key, int32 value) pairs on key bits [0, end_bit)
+// radix_sort.hip - stable LSD radix sort of (int64 key, int32 value) pairs on key bits [begin_bit, end_bit)
 // (gsplat/IntersectTile.cu:290-328 calls cub::DeviceRadixSort::SortPairs with a DoubleBuffer).
 //
-// 8-bit digits.  Per pass: block histograms -> exclusive scan of the digit-major histogram table ->
-// stable scatter.  A block owns 4096 consecutive pairs; inside the block each 64-lane wave owns 1024
-// consecutive pairs and ranks them 64 at a time with wave-wide match masks built from ballots, so the
-// order (wave, round, lane) equals the input order and the sort is stable.
+// 8-bit digits.  Per pass three launches: block histograms (which also add up the 256 digit totals) -> one scan
+// block per digit turns its row of the digit-major table into global start positions -> stable scatter.  A
+// block owns 4096 consecutive pairs; inside the block each 64-lane wave owns 1024 consecutive pairs and ranks
+// them 64 at a time with wave-wide match masks built from ballots, so the order (wave, round, lane) equals the
+// input order and the sort is stable.
 #include "gsx_common.h"
 
 namespace gsx {
@@ -15,13 +16,20 @@ static constexpr uint32_t kSortItems = 16;
 static constexpr uint32_t kSortTile = 256 * kSortItems; // pairs per block
 static constexpr uint32_t kWaveTile = 64 * kSortItems;  // pairs per wave
 
+__global__ void __launch_bounds__(256) fill_u32_kernel(uint32_t n, uint32_t v, uint32_t* __restrict__ out) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i < n)
+        out[i] = v;
+}
+
 __device__ __forceinline__ uint32_t digit_of(int64_t key, uint32_t shift, uint32_t mask) {
     return (uint32_t)((uint64_t)key >> shift) & mask;
 }
 
 __global__ void __launch_bounds__(256) radix_hist_kernel(uint32_t n, const int64_t* __restrict__ keys,
                                                           uint32_t shift, uint32_t mask, uint32_t nblocks,
-                                                          uint32_t* __restrict__ hist /*[kRadix][nblocks]*/) {
+                                                          uint32_t* __restrict__ hist /*[kRadix][nblocks]*/,
+                                                          uint32_t* __restrict__ digit_total /*[kRadix]*/) {
     __shared__ uint32_t lh[kRadix];
     lh[threadIdx.x] = 0;
     __syncthreads();
@@ -33,77 +41,58 @@ __global__ void __launch_bounds__(256) radix_hist_kernel(uint32_t n, const int64
             atomicAdd(&lh[digit_of(keys[idx], shift, mask)], 1u);
     }
     __syncthreads();
-    hist[threadIdx.x * nblocks + blockIdx.x] = lh[threadIdx.x];
+    const uint32_t c = lh[threadIdx.x];
+    hist[threadIdx.x * nblocks + blockIdx.x] = c;
+    if (c)
+        atomicAdd(&digit_total[threadIdx.x], c);
 }
 
-// ---- exclusive scan of a uint32 array (three passes) ---------------------------------------------
-static constexpr uint32_t kScanItems = 8;
-static constexpr uint32_t kScanTile = 256 * kScanItems;
-
-__device__ __forceinline__ uint32_t block_exclusive_scan_u32(uint32_t v, uint32_t* lds, uint32_t* total) {
-    const uint32_t t = threadIdx.x;
-    lds[t] = v;
-    __syncthreads();
+// ---- per-digit scan --------------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t wave_inclusive_scan_u32(uint32_t v, uint32_t lane) {
 #pragma unroll
-    for (uint32_t off = 1; off < 256; off <<= 1) {
-        const uint32_t add = (t >= off) ? lds[t - off] : 0;
+    for (uint32_t off = 1; off < 64; off <<= 1) {
+        const uint32_t up = __shfl_up(v, off, 64);
+        if (lane >= off)
+            v += up;
+    }
+    return v;
+}
+
+// Block d owns digit d: hist[d][0..nblocks) becomes the global position at which each sort block starts writing
+// its pairs with that digit = (pairs with a smaller digit) + (pairs with digit d in earlier blocks).
+__global__ void __launch_bounds__(256) radix_scan_kernel(uint32_t nblocks, uint32_t* __restrict__ hist,
+                                                          const uint32_t* __restrict__ digit_total) {
+    __shared__ uint32_t wsum[4];
+    __shared__ uint32_t base_s;
+    const uint32_t d = blockIdx.x, t = threadIdx.x, lane = t & 63u, w = t >> 6;
+    // pairs with a smaller digit
+    {
+        const uint32_t v = t < d ? digit_total[t] : 0u;
+        const uint32_t incl = wave_inclusive_scan_u32(v, lane);
+        if (lane == 63)
+            wsum[w] = incl;
         __syncthreads();
-        lds[t] += add;
+        if (t == 0)
+            base_s = wsum[0] + wsum[1] + wsum[2] + wsum[3];
         __syncthreads();
     }
-    const uint32_t incl = lds[t];
-    *total = lds[255];
-    __syncthreads();
-    return incl - v;
-}
-
-__global__ void __launch_bounds__(256) scan_u32_sums_kernel(uint32_t n, const uint32_t* __restrict__ in,
-                                                             uint32_t* __restrict__ sums) {
-    __shared__ uint32_t lds[256];
-    const uint32_t base = blockIdx.x * kScanTile + threadIdx.x * kScanItems;
-    uint32_t s = 0;
+    uint32_t carry = base_s;
+    uint32_t* __restrict__ row = hist + (size_t)d * nblocks;
+    for (uint32_t start = 0; start < nblocks; start += 256) {
+        const uint32_t i = start + t;
+        const uint32_t v = i < nblocks ? row[i] : 0u;
+        const uint32_t incl = wave_inclusive_scan_u32(v, lane);
+        __syncthreads(); // wsum of the previous round has been read
+        if (lane == 63)
+            wsum[w] = incl;
+        __syncthreads();
+        uint32_t before = 0;
 #pragma unroll
-    for (uint32_t i = 0; i < kScanItems; ++i)
-        if (base + i < n)
-            s += in[base + i];
-    uint32_t total;
-    block_exclusive_scan_u32(s, lds, &total);
-    if (threadIdx.x == 0)
-        sums[blockIdx.x] = total;
-}
-
-__global__ void __launch_bounds__(256) scan_u32_offsets_kernel(uint32_t nb, uint32_t* __restrict__ sums) {
-    __shared__ uint32_t lds[256];
-    uint32_t carry = 0;
-    for (uint32_t start = 0; start < nb; start += 256) {
-        const uint32_t i = start + threadIdx.x;
-        const uint32_t v = i < nb ? sums[i] : 0;
-        uint32_t total;
-        const uint32_t ex = block_exclusive_scan_u32(v, lds, &total);
-        if (i < nb)
-            sums[i] = carry + ex;
-        carry += total;
-    }
-}
-
-__global__ void __launch_bounds__(256) scan_u32_apply_kernel(uint32_t n, uint32_t* __restrict__ data,
-                                                              const uint32_t* __restrict__ offsets) {
-    __shared__ uint32_t lds[256];
-    const uint32_t base = blockIdx.x * kScanTile + threadIdx.x * kScanItems;
-    uint32_t v[kScanItems];
-    uint32_t s = 0;
-#pragma unroll
-    for (uint32_t i = 0; i < kScanItems; ++i) {
-        v[i] = (base + i < n) ? data[base + i] : 0;
-        s += v[i];
-    }
-    uint32_t total;
-    uint32_t run = block_exclusive_scan_u32(s, lds, &total) + offsets[blockIdx.x];
-#pragma unroll
-    for (uint32_t i = 0; i < kScanItems; ++i) {
-        if (base + i < n)
-            data[base + i] = run;
-        run += v[i];
+        for (uint32_t k = 0; k < 4; ++k)
+            before += k < w ? wsum[k] : 0u;
+        if (i < nblocks)
+            row[i] = carry + before + incl - v;
+        carry += wsum[0] + wsum[1] + wsum[2] + wsum[3];
     }
 }
 
@@ -183,20 +172,17 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const in
 using namespace gsx;
 
 namespace {
+static constexpr uint32_t kMaxPasses = 8;
 struct SortLayout {
     uint32_t nblocks;
-    uint32_t hist_len;
-    uint32_t scan_blocks;
-    size_t hist_off, sums_off, total;
+    size_t hist_off, totals_off, total;
 };
 SortLayout sort_layout(int64_t n) {
     SortLayout L;
     L.nblocks = cdiv((uint64_t)n, kSortTile);
-    L.hist_len = L.nblocks * kRadix;
-    L.scan_blocks = cdiv(L.hist_len, kScanTile);
     L.hist_off = 0;
-    L.sums_off = align_up((size_t)L.hist_len * 4, 256);
-    L.total = L.sums_off + align_up((size_t)L.scan_blocks * 4, 256);
+    L.totals_off = align_up((size_t)L.nblocks * kRadix * 4, 256);
+    L.total = L.totals_off + (size_t)kMaxPasses * kRadix * 4;
     return L;
 }
 } // namespace
@@ -208,37 +194,39 @@ extern "C" size_t gsx_radix_sort_pairs_workspace_bytes(int64_t n) {
 }
 
 extern "C" int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, int64_t* keys1, int32_t* vals1,
-                                    uint32_t end_bit, void* workspace, size_t workspace_bytes, int* selector_host,
-                                    void* stream) {
+                                    uint32_t begin_bit, uint32_t end_bit, void* workspace, size_t workspace_bytes,
+                                    int* selector_host, void* stream) {
     if (selector_host)
         *selector_host = 0;
     if (n <= 0)
         return GSX_OK; // IntersectTile.cu:298-300
     GSX_REQUIRE(n < (1ll << 31), GSX_ERR_OVERFLOW, "radix_sort_pairs: n = %lld does not fit int32", (long long)n);
     GSX_REQUIRE(keys0 && vals0 && keys1 && vals1, GSX_ERR_INVALID_ARGUMENT, "radix_sort_pairs: null buffer");
-    GSX_REQUIRE(end_bit >= 1 && end_bit <= 64, GSX_ERR_INVALID_ARGUMENT, "radix_sort_pairs: end_bit %u", end_bit);
+    GSX_REQUIRE(end_bit >= 1 && end_bit <= 64 && begin_bit < end_bit, GSX_ERR_INVALID_ARGUMENT,
+                "radix_sort_pairs: bits [%u, %u)", begin_bit, end_bit);
     const SortLayout L = sort_layout(n);
     GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 && workspace_bytes >= L.total,
                 GSX_ERR_WORKSPACE, "radix_sort_pairs: workspace needs %zu bytes, 256-byte aligned", L.total);
     uint32_t* hist = (uint32_t*)((char*)workspace + L.hist_off);
-    uint32_t* sums = (uint32_t*)((char*)workspace + L.sums_off);
+    uint32_t* totals = (uint32_t*)((char*)workspace + L.totals_off);
     hipStream_t s = (hipStream_t)stream;
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(cdiv(kMaxPasses * kRadix, 256)), dim3(256), 0, s, kMaxPasses * kRadix,
+                       0u, totals);
+    GSX_LAUNCH_CHECK();
     int sel = 0;
-    for (uint32_t shift = 0; shift < end_bit; shift += kRadixBits) {
+    uint32_t pass = 0;
+    for (uint32_t shift = begin_bit; shift < end_bit; shift += kRadixBits, ++pass) {
         const uint32_t bits = (end_bit - shift) < kRadixBits ? (end_bit - shift) : kRadixBits;
         const uint32_t mask = (1u << bits) - 1u;
         const int64_t* kin = sel ? keys1 : keys0;
         const int32_t* vin = sel ? vals1 : vals0;
         int64_t* kout = sel ? keys0 : keys1;
         int32_t* vout = sel ? vals0 : vals1;
+        uint32_t* tot = totals + pass * kRadix;
         hipLaunchKernelGGL(radix_hist_kernel, dim3(L.nblocks), dim3(256), 0, s, (uint32_t)n, kin, shift, mask,
-                           L.nblocks, hist);
+                           L.nblocks, hist, tot);
         GSX_LAUNCH_CHECK();
-        hipLaunchKernelGGL(scan_u32_sums_kernel, dim3(L.scan_blocks), dim3(256), 0, s, L.hist_len, hist, sums);
-        GSX_LAUNCH_CHECK();
-        hipLaunchKernelGGL(scan_u32_offsets_kernel, dim3(1), dim3(256), 0, s, L.scan_blocks, sums);
-        GSX_LAUNCH_CHECK();
-        hipLaunchKernelGGL(scan_u32_apply_kernel, dim3(L.scan_blocks), dim3(256), 0, s, L.hist_len, hist, sums);
+        hipLaunchKernelGGL(radix_scan_kernel, dim3(kRadix), dim3(256), 0, s, L.nblocks, hist, tot);
         GSX_LAUNCH_CHECK();
         hipLaunchKernelGGL(radix_scatter_kernel, dim3(L.nblocks), dim3(256), 0, s, (uint32_t)n, kin, vin, kout, vout,
                            shift, mask, L.nblocks, hist);

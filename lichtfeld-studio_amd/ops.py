@@ -99,30 +99,43 @@ def intersect_tile(means2d, radii, depths, camera_ids, gaussian_ids, C, tile_siz
     N = means2d.size(1)
     tiles_per_gauss = torch.empty_like(depths, dtype=torch.int32)
     n_isects = c_i64(0)
+    # sort == True with one camera: depth order first, then a sort on the tile bits only (same result as the
+    # reference's single sort on every bit, Intersect.cpp:104-113; see gsx.h)
+    two_level = bool(sort) and C == 1
     with torch.cuda.device(dev):
+        order = None
+        if two_level:
+            order = torch.empty((N,), dtype=torch.int32, device=dev)
+            ws_o = _workspace(lib().gsx_depth_order_workspace_bytes(c_u32(N)), dev)
+            check(lib().gsx_depth_order(c_u32(N), _ptr(depths), _ptr(radii), _ptr(order), _ptr(ws_o),
+                                        c_sz(ws_o.numel()), _stream(dev)))
         cum = torch.empty((C * N,), dtype=torch.int64, device=dev)
         ws_bytes = lib().gsx_intersect_tile_count_workspace_bytes(c_u32(C), c_u32(N))
         ws = _workspace(ws_bytes, dev)
         check(lib().gsx_intersect_tile_count(c_u32(C), c_u32(N), _ptr(means2d), _ptr(radii), c_u32(tile_size),
-                                             c_u32(tile_width), c_u32(tile_height), _ptr(tiles_per_gauss), _ptr(cum),
-                                             _ptr(ws), c_sz(ws.numel()), ctypes.byref(n_isects), _stream(dev)))
+                                             c_u32(tile_width), c_u32(tile_height), _ptr(order),
+                                             _ptr(tiles_per_gauss), _ptr(cum), _ptr(ws), c_sz(ws.numel()),
+                                             ctypes.byref(n_isects), _stream(dev)))
         n = n_isects.value
         isect_ids = torch.empty((n,), dtype=torch.int64, device=dev)
         flatten_ids = torch.empty((n,), dtype=torch.int32, device=dev)
         if n:
             check(lib().gsx_intersect_tile_emit(c_u32(C), c_u32(N), _ptr(means2d), _ptr(radii), _ptr(depths),
-                                                _ptr(cum), c_u32(tile_size), c_u32(tile_width), c_u32(tile_height),
-                                                _ptr(isect_ids), _ptr(flatten_ids), _stream(dev)))
+                                                _ptr(cum), _ptr(order), c_u32(tile_size), c_u32(tile_width),
+                                                c_u32(tile_height), _ptr(isect_ids), _ptr(flatten_ids),
+                                                _stream(dev)))
         if n and sort:
             tile_n_bits = lib().gsx_n_bits(c_u32(tile_width * tile_height))
             cam_n_bits = lib().gsx_n_bits(c_u32(C))
-            isect_ids, flatten_ids = radix_sort_double_buffer(n, tile_n_bits, cam_n_bits, isect_ids, flatten_ids)
+            isect_ids, flatten_ids = radix_sort_double_buffer(n, tile_n_bits, cam_n_bits, isect_ids, flatten_ids,
+                                                              begin_bit=32 if two_level else 0)
     return tiles_per_gauss, isect_ids, flatten_ids
 
 
-def radix_sort_double_buffer(n_isects, tile_n_bits, cam_n_bits, isect_ids, flatten_ids):
+def radix_sort_double_buffer(n_isects, tile_n_bits, cam_n_bits, isect_ids, flatten_ids, begin_bit=0):
     """Intersect.h:39-46.  Returns the sorted (isect_ids, flatten_ids); like the reference's DoubleBuffer the
-    result may live in either the input tensors or the internally allocated pair."""
+    result may live in either the input tensors or the internally allocated pair.  begin_bit > 0 sorts on the
+    key bits from there up only (stable)."""
     _check_input(isect_ids, "isect_ids"), _check_input(flatten_ids, "flatten_ids")
     if n_isects <= 0:
         return isect_ids, flatten_ids
@@ -132,7 +145,8 @@ def radix_sort_double_buffer(n_isects, tile_n_bits, cam_n_bits, isect_ids, flatt
         ws = _workspace(lib().gsx_radix_sort_pairs_workspace_bytes(c_i64(n_isects)), dev)
         sel = c_i(0)
         check(lib().gsx_radix_sort_pairs(c_i64(n_isects), _ptr(isect_ids), _ptr(flatten_ids), _ptr(k1), _ptr(v1),
-                                         c_u32(32 + tile_n_bits + cam_n_bits), _ptr(ws), c_sz(ws.numel()),
+                                         c_u32(begin_bit), c_u32(32 + tile_n_bits + cam_n_bits), _ptr(ws),
+                                         c_sz(ws.numel()),
                                          ctypes.byref(sel), _stream(dev)))
     return (k1, v1) if sel.value else (isect_ids, flatten_ids)
 

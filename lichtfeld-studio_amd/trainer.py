@@ -60,6 +60,8 @@ class TrainStep:
         self.tiles_per_gauss = e(N, dt=torch.int32)
         self.cum = e(N, dt=torch.int64)
         self.ws_count = e(self.lib.gsx_intersect_tile_count_workspace_bytes(c_u32(1), c_u32(N)), dt=torch.uint8)
+        self.order = e(N, dt=torch.int32)
+        self.ws_order = e(self.lib.gsx_depth_order_workspace_bytes(c_u32(N)), dt=torch.uint8)
         self.ws_bwd = e(self.lib.gsx_rasterize_bwd_accum_bytes(c_u32(N)), dt=torch.uint8)
         self.records = e(self.lib.gsx_raster_records_bytes(c_u32(N)), dt=torch.uint8)
         self.cap = 0
@@ -148,20 +150,25 @@ class TrainStep:
         self._run("sh_colors_from_world", lb.gsx_sh_colors_from_world, c_u32(N), c_u32(self.K), c_u32(self.sh_degree), _p(P["means"]), _p(P["shs"]),
                                           _p(J["radii"]), _p(viewmat), _p(self.colors), s)
         n_isects = c_i64(0)
-        self._run("intersect_tile_count", lb.gsx_intersect_tile_count, c_u32(1), c_u32(N), _p(J["means2d"]), _p(J["radii"]), c_u32(16),
-                                          c_u32(self.tw), c_u32(self.th), _p(self.tiles_per_gauss), _p(self.cum),
-                                          _p(self.ws_count), c_sz(self.ws_count.numel()), ctypes.byref(n_isects), s)
+        # depth order of the Gaussians first: the pairs then leave the emission sorted by depth and only the tile
+        # bits are left for the big sort
+        self._run("depth_order", lb.gsx_depth_order, c_u32(N), _p(J["depths"]), _p(J["radii"]), _p(self.order),
+                  _p(self.ws_order), c_sz(self.ws_order.numel()), s)
+        self._run("intersect_tile_count", lb.gsx_intersect_tile_count, c_u32(1), c_u32(N), _p(J["means2d"]),
+                  _p(J["radii"]), c_u32(16), c_u32(self.tw), c_u32(self.th), _p(self.order),
+                  _p(self.tiles_per_gauss), _p(self.cum), _p(self.ws_count), c_sz(self.ws_count.numel()),
+                  ctypes.byref(n_isects), s)
         n = self.n_isects = n_isects.value
         self._ensure_isect_capacity(n)
         sel = c_i(0)
         if n:
-            self._run("intersect_tile_emit", lb.gsx_intersect_tile_emit, c_u32(1), c_u32(N), _p(J["means2d"]), _p(J["radii"]), _p(J["depths"]),
-                                             _p(self.cum), c_u32(16), c_u32(self.tw), c_u32(self.th),
-                                             _p(self.keys[0]), _p(self.vals[0]), s)
+            self._run("intersect_tile_emit", lb.gsx_intersect_tile_emit, c_u32(1), c_u32(N), _p(J["means2d"]),
+                      _p(J["radii"]), _p(J["depths"]), _p(self.cum), _p(self.order), c_u32(16), c_u32(self.tw),
+                      c_u32(self.th), _p(self.keys[0]), _p(self.vals[0]), s)
             end_bit = 32 + lb.gsx_n_bits(c_u32(self.tw * self.th)) + lb.gsx_n_bits(c_u32(1))
-            self._run("radix_sort_pairs", lb.gsx_radix_sort_pairs, c_i64(n), _p(self.keys[0]), _p(self.vals[0]), _p(self.keys[1]),
-                                          _p(self.vals[1]), c_u32(end_bit), _p(self.ws_sort),
-                                          c_sz(self.ws_sort.numel()), ctypes.byref(sel), s)
+            self._run("radix_sort_pairs", lb.gsx_radix_sort_pairs, c_i64(n), _p(self.keys[0]), _p(self.vals[0]),
+                      _p(self.keys[1]), _p(self.vals[1]), c_u32(32), c_u32(end_bit), _p(self.ws_sort),
+                      c_sz(self.ws_sort.numel()), ctypes.byref(sel), s)
         self.sel = sel.value
         self.isect_ids, self.flatten_ids = self.keys[self.sel], self.vals[self.sel]
         self._run("intersect_offset", lb.gsx_intersect_offset, c_i64(n), _p(self.isect_ids), c_u32(1), c_u32(self.tw), c_u32(self.th),

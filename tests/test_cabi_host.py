@@ -51,7 +51,7 @@ def test_status_codes_without_launch(gsx):
     assert lib.gsx_adam_step(nul, nul, nul, nul, i64(0), cf(1), cf(.9), cf(.999), cf(1e-15), cf(1), cf(1), nul) == 0
     assert lib.gsx_relocation(ci(0), nul, nul, nul, nul, ci(51), nul, nul, nul) == L.GSX_OK
     sel = ci(7)
-    assert lib.gsx_radix_sort_pairs(i64(0), nul, nul, nul, nul, u32(45), nul, ctypes.c_size_t(0),
+    assert lib.gsx_radix_sort_pairs(i64(0), nul, nul, nul, nul, u32(0), u32(45), nul, ctypes.c_size_t(0),
                                     ctypes.byref(sel), nul) == L.GSX_OK and sel.value == 0
     # invalid arguments
     assert lib.gsx_spherical_harmonics_fwd(u32(10), u32(4), u32(3), one, one, nul, one, nul) == \
@@ -59,9 +59,9 @@ def test_status_codes_without_launch(gsx):
     assert b"K >= 16" in lib.gsx_last_error()
     assert lib.gsx_spherical_harmonics_fwd(u32(10), u32(16), u32(3), nul, one, nul, one, nul) == \
         L.GSX_ERR_INVALID_ARGUMENT  # null tensor
-    assert lib.gsx_radix_sort_pairs(i64(100), one, one, one, one, u32(45), nul, ctypes.c_size_t(0), ctypes.byref(sel),
-                                    nul) == L.GSX_ERR_WORKSPACE
-    assert lib.gsx_radix_sort_pairs(i64(1 << 31), one, one, one, one, u32(45), one, ctypes.c_size_t(1 << 40),
+    assert lib.gsx_radix_sort_pairs(i64(100), one, one, one, one, u32(0), u32(45), nul, ctypes.c_size_t(0),
+                                    ctypes.byref(sel), nul) == L.GSX_ERR_WORKSPACE
+    assert lib.gsx_radix_sort_pairs(i64(1 << 31), one, one, one, one, u32(0), u32(45), one, ctypes.c_size_t(1 << 40),
                                     ctypes.byref(sel), nul) == L.GSX_ERR_OVERFLOW
     ut = L.UTParams()
     proj = lambda C, model, rs, vm1: lib.gsx_projection_ut_3dgs_fused(
@@ -72,9 +72,11 @@ def test_status_codes_without_launch(gsx):
     assert proj(1, L.PINHOLE, L.ROLLING_TOP_TO_BOTTOM, nul) == L.GSX_ERR_UNSUPPORTED
     assert proj(1, L.PINHOLE, L.GLOBAL, one) == L.GSX_ERR_UNSUPPORTED        # viewmats1 given
     n_host = i64(-1)
-    assert lib.gsx_intersect_tile_count(u32(1), u32(10), one, one, u32(16), u32(1 << 20), u32(1 << 11), one, one, one,
+    assert lib.gsx_intersect_tile_count(u32(1), u32(10), one, one, u32(16), u32(1 << 20), u32(1 << 11), nul, one, one, one,
                                         ctypes.c_size_t(1 << 20), ctypes.byref(n_host), nul) == \
         L.GSX_ERR_INVALID_ARGUMENT  # tile id + camera id need more than 32 bits (Intersect.cpp:50)
+    assert lib.gsx_radix_sort_pairs(i64(100), one, one, one, one, u32(45), u32(45), one, ctypes.c_size_t(1 << 40),
+                                    ctypes.byref(sel), nul) == L.GSX_ERR_INVALID_ARGUMENT  # empty bit range
     groups = (L.AdamGroup * 9)()
     assert lib.gsx_adam_step_multi(groups, ci(9), nul) == L.GSX_ERR_INVALID_ARGUMENT
 

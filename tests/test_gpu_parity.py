@@ -203,8 +203,11 @@ def test_radix_sort_bit_range(gsx, orc, cuda):
     n = 50_000
     keys = rng.integers(0, 1 << 62, n, dtype=np.int64)
     vals = np.arange(n, dtype=np.int32)
-    for end_bit in (1, 8, 13, 45, 64):
-        ref_k, ref_v = orc.radix_sort_pairs(keys, vals, end_bit)
+    for begin_bit, end_bit in ((0, 1), (0, 8), (0, 13), (0, 45), (0, 64), (32, 45), (5, 6), (40, 64)):
+        # the checker sorts on bits [0, end): shifting the keys right by begin_bit gives the order for [begin, end)
+        order = orc.radix_sort_pairs((keys.view(np.uint64) >> np.uint64(begin_bit)).view(np.int64),
+                                     np.arange(n, dtype=np.int32), end_bit - begin_bit)[1]
+        ref_k, ref_v = keys[order], vals[order]
         k0, v0 = T(keys, cuda), T(vals, cuda)
         k1, v1 = torch.empty_like(k0), torch.empty_like(v0)
         ws = torch.empty((L.lib().gsx_radix_sort_pairs_workspace_bytes(ctypes.c_int64(n)),), dtype=torch.uint8,
@@ -212,12 +215,13 @@ def test_radix_sort_bit_range(gsx, orc, cuda):
         sel = ctypes.c_int(0)
         L.check(L.lib().gsx_radix_sort_pairs(ctypes.c_int64(n), ctypes.c_void_p(k0.data_ptr()),
                                              ctypes.c_void_p(v0.data_ptr()), ctypes.c_void_p(k1.data_ptr()),
-                                             ctypes.c_void_p(v1.data_ptr()), ctypes.c_uint32(end_bit),
+                                             ctypes.c_void_p(v1.data_ptr()), ctypes.c_uint32(begin_bit),
+                                             ctypes.c_uint32(end_bit),
                                              ctypes.c_void_p(ws.data_ptr()), ctypes.c_size_t(ws.numel()),
                                              ctypes.byref(sel), ctypes.c_void_p(None)))
         torch.cuda.synchronize()
         k, v = (k1, v1) if sel.value else (k0, v0)
-        assert np.array_equal(N(k), ref_k) and np.array_equal(N(v), ref_v), end_bit
+        assert np.array_equal(N(k), ref_k) and np.array_equal(N(v), ref_v), (begin_bit, end_bit)
 
 
 # ---------------------------------------------------------------------------------------------
