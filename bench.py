@@ -56,9 +56,8 @@ def algorithmic_bytes(N, K, H, W, n_isects, sort_bits):
         "activate_params": N * (32 + 32),
         "projection_ut_3dgs_fused": N * (44 + 32),
         "sh_colors_from_world": N * (12 + 12 * K + 8 + 12),
-        "intersect_tile_count": N * (4 + 16 + 4 + 4 + 4 + 8 + 4),
         "intersect_tile_emit": N * (4 + 16 + 4 + 8) + n_isects * 12,
-        "depth_order": N * (12 + 12 + (8 + 24) * 4),
+        "intersect_tile_count_ordered": N * (28 + 16 + (8 + 24) * 4 + 8 + 8),
         "radix_sort_pairs": n_isects * (8 + 24) * passes,
         "intersect_offset": n_isects * 8 + (P // 256) * 4,
         "image_from_render": P * (12 + 12 + 12),

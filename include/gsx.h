@@ -97,29 +97,33 @@ GSX_API int gsx_spherical_harmonics_bwd(uint32_t N, uint32_t K, uint32_t degrees
 
 /* ---- a4: gsplat::intersect_tile (Ops.h:28-38; Intersect.cpp:15-122; IntersectTile.cu:23-114) ----
  * Two calls, as the reference's two passes: count (+ inclusive scan; blocks until the total is on the
- * host, like Intersect.cpp:76) then emit.  cum_tiles_per_gauss is i64 [C*N].
- *
- * `order` (i32 [N], nullable, C == 1 only) visits the Gaussians in that order instead of by index: position i is
- * Gaussian order[i], cum_tiles_per_gauss is the prefix sum over POSITIONS and the pairs are emitted position by
- * position (tiles_per_gauss stays indexed by Gaussian).  With order = gsx_depth_order(...) the emitted pairs are
- * already sorted by (depth bits, Gaussian index), so the sorted list the reference obtains from one radix sort on
- * all 32 + tile + camera bits (Intersect.cpp:104-113) is reached by sorting on the tile / camera bits alone
- * (gsx_radix_sort_pairs with begin_bit = 32): the sort is stable, the result is the same array bit for bit, and
- * four of its six passes run over N Gaussians instead of n_isects pairs. */
+ * host, like Intersect.cpp:76) then emit.  cum_tiles_per_gauss is i64 [C*N]. */
 GSX_API size_t gsx_intersect_tile_count_workspace_bytes(uint32_t C, uint32_t N);
 GSX_API int gsx_intersect_tile_count(uint32_t C, uint32_t N, const float* means2d, const int32_t* radii,
                                      uint32_t tile_size, uint32_t tile_width, uint32_t tile_height,
-                                     const int32_t* order, int32_t* tiles_per_gauss, int64_t* cum_tiles_per_gauss,
-                                     void* workspace, size_t workspace_bytes, int64_t* n_isects_host, void* stream);
+                                     int32_t* tiles_per_gauss, int64_t* cum_tiles_per_gauss, void* workspace,
+                                     size_t workspace_bytes, int64_t* n_isects_host, void* stream);
+/* The depth-ordered count (one camera): order[i] = index of the Gaussian with the i-th smallest depth bit pattern
+ * (ties by index; Gaussians that touch no tile last), cum_tiles_per_gauss = prefix sum of the tile counts over
+ * POSITIONS in that order (tiles_per_gauss stays indexed by Gaussian).  Emitting with this order leaves the pairs
+ * sorted by (depth bits, Gaussian index), so the sorted list the reference obtains from one radix sort on all
+ * 32 + tile + camera bits (Intersect.cpp:104-113) is reached by sorting on the tile / camera bits alone
+ * (gsx_radix_sort_pairs with begin_bit = 32): the sort is stable, the result is the same array bit for bit, and
+ * four of its six passes run over N Gaussians instead of n_isects pairs.
+ * wait != 0: returns with *n_isects_host valid (and checked against the int32 index space), like the call above.
+ * wait == 0: nothing blocks; n_isects_host must be PINNED host memory, and the caller reads it (and checks it is
+ * below 2^31) after synchronising with the stream - work that does not need the count can be queued in between. */
+GSX_API size_t gsx_intersect_tile_count_ordered_workspace_bytes(uint32_t N);
+GSX_API int gsx_intersect_tile_count_ordered(uint32_t N, const float* means2d, const int32_t* radii,
+                                             const float* depths, uint32_t tile_size, uint32_t tile_width,
+                                             uint32_t tile_height, int32_t* order, int32_t* tiles_per_gauss,
+                                             int64_t* cum_tiles_per_gauss, void* workspace, size_t workspace_bytes,
+                                             int64_t* n_isects_host, int wait, void* stream);
+/* order: nullable (i32 [N], C == 1): emit position by position in that order, cum_tiles_per_gauss by position */
 GSX_API int gsx_intersect_tile_emit(uint32_t C, uint32_t N, const float* means2d, const int32_t* radii,
                                     const float* depths, const int64_t* cum_tiles_per_gauss, const int32_t* order,
                                     uint32_t tile_size, uint32_t tile_width, uint32_t tile_height, int64_t* isect_ids,
                                     int32_t* flatten_ids, void* stream);
-/* order[i] = index of the Gaussian with the i-th smallest depth bit pattern (ties by index; Gaussians with
- * radii == 0 last).  One camera. */
-GSX_API size_t gsx_depth_order_workspace_bytes(uint32_t N);
-GSX_API int gsx_depth_order(uint32_t N, const float* depths, const int32_t* radii, int32_t* order, void* workspace,
-                            size_t workspace_bytes, void* stream);
 /* Intersect.cpp:46-47: floor(log2(n)) + 1 */
 GSX_API uint32_t gsx_n_bits(uint32_t n);
 
@@ -193,10 +197,12 @@ GSX_API int gsx_rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isect
                                          const float* render_alphas, const int32_t* last_ids,
                                          const float* v_render_colors, const float* v_render_alphas, void* workspace,
                                          size_t workspace_bytes, void* stream);
+/* clear_accumulators != 0: the epilogue zeroes each accumulator row after reading it, so the next backward pass
+ * needs no gsx_rasterize_bwd_clear */
 GSX_API int gsx_rasterize_bwd_finish(uint32_t N, const float* means, const float* quats, const float* scales,
-                                     const float* viewmats0, const void* workspace, size_t workspace_bytes,
-                                     float* v_means, float* v_quats, float* v_scales, float* v_colors,
-                                     float* v_opacities, void* stream);
+                                     const float* viewmats0, void* workspace, size_t workspace_bytes,
+                                     int clear_accumulators, float* v_means, float* v_quats, float* v_scales,
+                                     float* v_colors, float* v_opacities, void* stream);
 GSX_API int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
     uint32_t C, uint32_t N, int64_t n_isects, const float* means, const float* quats, const float* scales,
     const float* colors, const float* opacities, const float* backgrounds, const uint8_t* masks,

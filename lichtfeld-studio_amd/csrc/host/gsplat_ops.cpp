@@ -146,20 +146,25 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> intersect_tile(const at::Tensor m
     const bool two_level = sort && C == 1;
     at::Tensor order;
     const int32_t* order_ptr = nullptr;
-    if (two_level && N > 0) {
-        order = at::empty({(int64_t)N}, depths.options().dtype(at::kInt));
-        at::Tensor ws_o = workspace(gsx_depth_order_workspace_bytes(N), depths);
-        gsx_check(gsx_depth_order(N, depths.data_ptr<float>(), radii.data_ptr<int32_t>(), order.data_ptr<int32_t>(),
-                                  ws_o.data_ptr(), (size_t)ws_o.numel(), cur_stream(means2d)));
-        order_ptr = order.data_ptr<int32_t>();
-    }
     at::Tensor cum = at::empty({(int64_t)C * N}, depths.options().dtype(at::kLong));
-    at::Tensor ws = workspace(gsx_intersect_tile_count_workspace_bytes(C, N), depths);
     int64_t n_isects = 0;
     void* stream = cur_stream(means2d);
-    gsx_check(gsx_intersect_tile_count(C, N, means2d.data_ptr<float>(), radii.data_ptr<int32_t>(), tile_size,
-                                       tile_width, tile_height, order_ptr, tiles_per_gauss.data_ptr<int32_t>(),
-                                       cum.data_ptr<int64_t>(), ws.data_ptr(), (size_t)ws.numel(), &n_isects, stream));
+    if (two_level && N > 0) {
+        order = at::empty({(int64_t)N}, depths.options().dtype(at::kInt));
+        order_ptr = order.data_ptr<int32_t>();
+        at::Tensor ws = workspace(gsx_intersect_tile_count_ordered_workspace_bytes(N), depths);
+        gsx_check(gsx_intersect_tile_count_ordered(N, means2d.data_ptr<float>(), radii.data_ptr<int32_t>(),
+                                                   depths.data_ptr<float>(), tile_size, tile_width, tile_height,
+                                                   order.data_ptr<int32_t>(), tiles_per_gauss.data_ptr<int32_t>(),
+                                                   cum.data_ptr<int64_t>(), ws.data_ptr(), (size_t)ws.numel(),
+                                                   &n_isects, 1, stream));
+    } else {
+        at::Tensor ws = workspace(gsx_intersect_tile_count_workspace_bytes(C, N), depths);
+        gsx_check(gsx_intersect_tile_count(C, N, means2d.data_ptr<float>(), radii.data_ptr<int32_t>(), tile_size,
+                                           tile_width, tile_height, tiles_per_gauss.data_ptr<int32_t>(),
+                                           cum.data_ptr<int64_t>(), ws.data_ptr(), (size_t)ws.numel(), &n_isects,
+                                           stream));
+    }
     at::Tensor isect_ids = at::empty({n_isects}, depths.options().dtype(at::kLong));
     at::Tensor flatten_ids = at::empty({n_isects}, depths.options().dtype(at::kInt));
     if (n_isects) {

@@ -28,38 +28,40 @@ __device__ __forceinline__ bool tile_rect(const float* __restrict__ means2d, con
     return true;
 }
 
-// order == nullptr: position i is Gaussian i.  Otherwise position i is Gaussian order[i]; the count goes to
-// tiles_per_gauss[order[i]] and, for the prefix sum over positions, to counts_by_position[i].
 __global__ void __launch_bounds__(256) tile_count_kernel(uint32_t n, const float* __restrict__ means2d,
                                                           const int32_t* __restrict__ radii, float tile_size,
                                                           uint32_t tile_width, uint32_t tile_height,
-                                                          const int32_t* __restrict__ order,
-                                                          int32_t* __restrict__ tiles_per_gauss,
-                                                          int32_t* __restrict__ counts_by_position) {
-    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
-    if (i >= n)
+                                                          int32_t* __restrict__ tiles_per_gauss) {
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= n)
         return;
-    const uint32_t idx = order != nullptr ? (uint32_t)order[i] : i;
     TileRect r;
     int32_t cnt = 0;
     if (tile_rect(means2d, radii, idx, tile_size, tile_width, tile_height, &r))
         cnt = (int32_t)((r.y1 - r.y0) * (r.x1 - r.x0));
     tiles_per_gauss[idx] = cnt;
-    if (order != nullptr)
-        counts_by_position[i] = cnt;
 }
 
-// sort keys for the depth order of one camera's Gaussians: the depth's bit pattern (what the low word of an
-// intersection key holds), all ones for a Gaussian that touches no tile
-__global__ void __launch_bounds__(256) depth_keys_kernel(uint32_t n, const float* __restrict__ depths,
-                                                          const int32_t* __restrict__ radii,
-                                                          int64_t* __restrict__ keys, int32_t* __restrict__ vals) {
+// Depth-ordered variant, one camera: the tile count rides in the high word of a sort key whose low word is the
+// depth's bit pattern (what the low word of an intersection key holds; all ones for a Gaussian that touches no
+// tile).  Sorting these N keys on their low 32 bits gives the visiting order AND the counts in that order.
+__global__ void __launch_bounds__(256) depth_count_keys_kernel(uint32_t n, const float* __restrict__ means2d,
+                                                                const int32_t* __restrict__ radii,
+                                                                const float* __restrict__ depths, float tile_size,
+                                                                uint32_t tile_width, uint32_t tile_height,
+                                                                int32_t* __restrict__ tiles_per_gauss,
+                                                                int64_t* __restrict__ keys,
+                                                                int32_t* __restrict__ vals) {
     const uint32_t i = blockIdx.x * 256u + threadIdx.x;
     if (i >= n)
         return;
-    const int2 rad = reinterpret_cast<const int2*>(radii)[i];
-    const bool live = rad.x > 0 && rad.y > 0;
-    keys[i] = live ? (int64_t)(uint64_t)f2u(depths[i]) : (int64_t)0xFFFFFFFFll;
+    TileRect r;
+    uint32_t cnt = 0;
+    if (tile_rect(means2d, radii, i, tile_size, tile_width, tile_height, &r))
+        cnt = (r.y1 - r.y0) * (r.x1 - r.x0);
+    tiles_per_gauss[i] = (int32_t)cnt;
+    const uint32_t lo = cnt ? f2u(depths[i]) : 0xFFFFFFFFu;
+    keys[i] = (int64_t)(((uint64_t)cnt << 32) | lo);
     vals[i] = (int32_t)i;
 }
 
@@ -85,7 +87,14 @@ __device__ __forceinline__ int64_t block_exclusive_scan_256(int64_t v, int64_t* 
     return incl - v;
 }
 
+// the scan's input: int32 counts, or (keys != nullptr) the high words of 64-bit keys
+__device__ __forceinline__ int32_t scan_input(const int32_t* __restrict__ in, const int64_t* __restrict__ keys,
+                                              uint32_t i) {
+    return keys != nullptr ? (int32_t)(keys[i] >> 32) : in[i];
+}
+
 __global__ void __launch_bounds__(256) scan_block_sums_kernel(uint32_t n, const int32_t* __restrict__ in,
+                                                               const int64_t* __restrict__ keys,
                                                                int64_t* __restrict__ block_sums) {
     __shared__ int64_t lds[256];
     const uint32_t base = blockIdx.x * kScanTile + threadIdx.x * kScanItems;
@@ -93,7 +102,7 @@ __global__ void __launch_bounds__(256) scan_block_sums_kernel(uint32_t n, const 
 #pragma unroll
     for (uint32_t i = 0; i < kScanItems; ++i)
         if (base + i < n)
-            s += in[base + i];
+            s += scan_input(in, keys, base + i);
     int64_t total;
     block_exclusive_scan_256(s, lds, &total);
     if (threadIdx.x == 0)
@@ -119,6 +128,7 @@ __global__ void __launch_bounds__(256) scan_block_offsets_kernel(uint32_t nb, in
 }
 
 __global__ void __launch_bounds__(256) scan_apply_kernel(uint32_t n, const int32_t* __restrict__ in,
+                                                          const int64_t* __restrict__ keys,
                                                           const int64_t* __restrict__ block_offsets,
                                                           int64_t* __restrict__ out) {
     __shared__ int64_t lds[256];
@@ -127,7 +137,7 @@ __global__ void __launch_bounds__(256) scan_apply_kernel(uint32_t n, const int32
     int64_t s = 0;
 #pragma unroll
     for (uint32_t i = 0; i < kScanItems; ++i) {
-        v[i] = (base + i < n) ? in[base + i] : 0;
+        v[i] = (base + i < n) ? scan_input(in, keys, base + i) : 0;
         s += v[i];
     }
     int64_t total;
@@ -141,9 +151,10 @@ __global__ void __launch_bounds__(256) scan_apply_kernel(uint32_t n, const int32
 }
 
 // IntersectTile.cu:78-113 second pass: keys and values in emission order (ascending position, row-major tiles
-// inside a Gaussian).  A lane writes the tiles of a small Gaussian itself; the tiles of a Gaussian with more than
-// 32 of them are written by the whole wave, 64 at a time, so that one screen-filling Gaussian does not leave
-// 63 lanes idle.
+// inside a Gaussian).  The reference lets every thread write its own Gaussian's run, 64 scattered 8-byte stores per
+// instruction and a serial loop as long as the largest Gaussian.  Here a wave flattens the runs of its 64
+// positions: entry k of the wave's output range belongs to the position whose inclusive count prefix first
+// exceeds k (binary search over 64 prefixes in LDS), so the lanes write consecutive entries.
 __global__ void __launch_bounds__(256) tile_emit_kernel(uint32_t n, uint32_t N, const float* __restrict__ means2d,
                                                          const int32_t* __restrict__ radii,
                                                          const float* __restrict__ depths,
@@ -152,8 +163,9 @@ __global__ void __launch_bounds__(256) tile_emit_kernel(uint32_t n, uint32_t N, 
                                                          uint32_t tile_width, uint32_t tile_height,
                                                          uint32_t tile_n_bits, int64_t* __restrict__ isect_ids,
                                                          int32_t* __restrict__ flatten_ids) {
+    __shared__ uint32_t s_incl[4][64], s_xy[4][64], s_w[4][64], s_idx[4][64], s_lo[4][64], s_hi[4][64];
     const uint32_t i = blockIdx.x * 256u + threadIdx.x;
-    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t lane = threadIdx.x & 63u, wv = threadIdx.x >> 6;
     TileRect r = {0, 0, 0, 0};
     uint32_t idx = 0;
     bool live = false;
@@ -164,39 +176,51 @@ __global__ void __launch_bounds__(256) tile_emit_kernel(uint32_t n, uint32_t N, 
     const uint32_t w = live ? r.x1 - r.x0 : 0u;
     const uint32_t cnt = live ? (r.y1 - r.y0) * w : 0u;
     int64_t key_base = 0;
-    int64_t cur = 0;
     if (cnt) {
         const int64_t cid = idx / N;
         key_base = (cid << (32 + tile_n_bits)) | (int64_t)(uint64_t)f2u(depths[idx]); // zero-extended bits (:96-98)
-        cur = (i == 0) ? 0 : cum_tiles_per_gauss[i - 1];
     }
-    const bool big = cnt > 32u;
-    if (cnt && !big) {
-        for (uint32_t ty = r.y0; ty < r.y1; ++ty)
-            for (uint32_t tx = r.x0; tx < r.x1; ++tx) {
-                const int64_t tile_id = (int64_t)ty * tile_width + tx;
-                isect_ids[cur] = key_base | (tile_id << 32);
-                flatten_ids[cur] = (int32_t)idx;
-                ++cur;
-            }
+    // inclusive prefix of the counts over the wave
+    uint32_t incl = cnt;
+#pragma unroll
+    for (uint32_t off = 1; off < 64; off <<= 1) {
+        const uint32_t up = (uint32_t)__shfl_up((int)incl, off, 64);
+        if (lane >= off)
+            incl += up;
     }
-    uint64_t todo = __builtin_amdgcn_ballot_w64(big);
-    while (todo) {
-        const int src = __builtin_ctzll(todo);
-        todo &= todo - 1;
-        const uint32_t bx0 = (uint32_t)__shfl((int)r.x0, src, 64), by0 = (uint32_t)__shfl((int)r.y0, src, 64);
-        const uint32_t bw = (uint32_t)__shfl((int)w, src, 64), bcnt = (uint32_t)__shfl((int)cnt, src, 64);
-        const int32_t bidx = __shfl((int)idx, src, 64);
-        const int64_t bkey = ((int64_t)__shfl((int)(key_base >> 32), src, 64) << 32) |
-                             (int64_t)(uint32_t)__shfl((int)(uint32_t)key_base, src, 64);
-        const int64_t bcur = ((int64_t)__shfl((int)(cur >> 32), src, 64) << 32) |
-                             (int64_t)(uint32_t)__shfl((int)(uint32_t)cur, src, 64);
-        for (uint32_t k = lane; k < bcnt; k += 64u) {
-            const uint32_t row = k / bw;
-            const int64_t tile_id = (int64_t)(by0 + row) * tile_width + (bx0 + (k - row * bw));
-            isect_ids[bcur + k] = bkey | (tile_id << 32);
-            flatten_ids[bcur + k] = bidx;
+    const uint32_t total = (uint32_t)__shfl((int)incl, 63, 64);
+    s_incl[wv][lane] = incl;
+    s_xy[wv][lane] = r.x0 | (r.y0 << 16);
+    s_w[wv][lane] = w;
+    s_idx[wv][lane] = idx;
+    s_lo[wv][lane] = (uint32_t)key_base;
+    s_hi[wv][lane] = (uint32_t)(key_base >> 32);
+    __syncthreads();
+    if (total == 0)
+        return; // wave-uniform; no barrier follows
+    // where the wave's first position starts in the output
+    const uint32_t i0 = i - lane;
+    const int64_t wave_base = (i0 == 0) ? 0 : cum_tiles_per_gauss[i0 - 1];
+    for (uint32_t k = lane; k < total; k += 64u) {
+        // smallest l with incl[l] > k
+        uint32_t lo = 0, hi = 63;
+#pragma unroll
+        for (uint32_t step = 0; step < 6; ++step) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (s_incl[wv][mid] > k)
+                hi = mid;
+            else
+                lo = mid + 1;
         }
+        const uint32_t l = lo;
+        const uint32_t before = l ? s_incl[wv][l - 1] : 0u;
+        const uint32_t local = k - before;
+        const uint32_t gw = s_w[wv][l], xy = s_xy[wv][l];
+        const uint32_t row = local / gw;
+        const int64_t tile_id = (int64_t)((xy >> 16) + row) * tile_width + ((xy & 0xffffu) + (local - row * gw));
+        const int64_t kb = ((int64_t)s_hi[wv][l] << 32) | (int64_t)s_lo[wv][l];
+        isect_ids[wave_base + k] = kb | (tile_id << 32);
+        flatten_ids[wave_base + k] = (int32_t)s_idx[wv][l];
     }
 }
 
@@ -240,47 +264,38 @@ using namespace gsx;
 extern "C" size_t gsx_intersect_tile_count_workspace_bytes(uint32_t C, uint32_t N) {
     const uint64_t n = (uint64_t)C * N;
     const uint64_t nb = (n + kScanTile - 1) / kScanTile;
-    return align_up((nb + 1) * sizeof(int64_t), 256) + 256 + align_up(n * sizeof(int32_t), 256);
+    return align_up((nb + 1) * sizeof(int64_t), 256) + 256;
 }
 
-// depth order of one camera's Gaussians: keys0 / keys1 (i64 [N] each), vals1 (i32 [N]), then the sort's own scratch
-extern "C" size_t gsx_depth_order_workspace_bytes(uint32_t N) {
-    return 2 * align_up((size_t)N * 8, 256) + align_up((size_t)N * 4, 256) + gsx_radix_sort_pairs_workspace_bytes(N);
-}
-
-extern "C" int gsx_depth_order(uint32_t N, const float* depths, const int32_t* radii, int32_t* order, void* workspace,
-                               size_t workspace_bytes, void* stream) {
-    if (N == 0)
-        return GSX_OK;
-    GSX_REQUIRE(depths && radii && order, GSX_ERR_INVALID_ARGUMENT, "depth_order: null tensor");
-    GSX_REQUIRE(N < (1u << 31), GSX_ERR_INVALID_ARGUMENT, "depth_order: N >= 2^31");
-    GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 &&
-                    workspace_bytes >= gsx_depth_order_workspace_bytes(N),
-                GSX_ERR_WORKSPACE, "depth_order: workspace needs %zu bytes, 256-byte aligned",
-                gsx_depth_order_workspace_bytes(N));
-    char* ws = (char*)workspace;
-    int64_t* keys0 = (int64_t*)ws;
-    int64_t* keys1 = (int64_t*)(ws + align_up((size_t)N * 8, 256));
-    int32_t* vals1 = (int32_t*)(ws + 2 * align_up((size_t)N * 8, 256));
-    char* sort_ws = ws + 2 * align_up((size_t)N * 8, 256) + align_up((size_t)N * 4, 256);
-    hipStream_t s = (hipStream_t)stream;
-    hipLaunchKernelGGL(depth_keys_kernel, dim3(cdiv(N, 256)), dim3(256), 0, s, N, depths, radii, keys0, order);
+namespace {
+// prefix sum of the counts (int32 array, or high words of `keys`) into cum, grand total to *total_dev
+int scan_counts(uint32_t n, const int32_t* counts, const int64_t* keys, int64_t* cum, int64_t* block_sums,
+                int64_t* total_dev, hipStream_t s) {
+    const uint32_t nb = cdiv(n, kScanTile);
+    hipLaunchKernelGGL(scan_block_sums_kernel, dim3(nb), dim3(256), 0, s, n, counts, keys, block_sums);
     GSX_LAUNCH_CHECK();
-    int sel = 0;
-    const int rc = gsx_radix_sort_pairs(N, keys0, order, keys1, vals1, 0, 32, sort_ws,
-                                        gsx_radix_sort_pairs_workspace_bytes(N), &sel, stream);
-    if (rc != GSX_OK)
-        return rc;
-    if (sel) // four 8-bit passes end in buffer 0; kept for a different digit width
-        GSX_HIP_CHECK(hipMemcpyAsync(order, vals1, (size_t)N * 4, hipMemcpyDeviceToDevice, s));
+    hipLaunchKernelGGL(scan_block_offsets_kernel, dim3(1), dim3(256), 0, s, nb, block_sums, total_dev);
+    GSX_LAUNCH_CHECK();
+    hipLaunchKernelGGL(scan_apply_kernel, dim3(nb), dim3(256), 0, s, n, counts, keys, block_sums, cum);
+    GSX_LAUNCH_CHECK();
     return GSX_OK;
 }
 
+int check_tile_grid(const char* who, uint32_t C, uint32_t tile_size, uint32_t tile_width, uint32_t tile_height) {
+    GSX_REQUIRE(tile_size > 0 && tile_width > 0 && tile_height > 0, GSX_ERR_INVALID_ARGUMENT, "%s: empty tile grid",
+                who);
+    GSX_REQUIRE((uint64_t)tile_width * tile_height < (1ull << 32) &&
+                    gsx_n_bits(tile_width * tile_height) + gsx_n_bits(C) <= 32,
+                GSX_ERR_INVALID_ARGUMENT, "%s: tile and camera ids need more than 32 bits", who); // Intersect.cpp:50
+    GSX_REQUIRE(tile_width < 65536 && tile_height < 65536, GSX_ERR_INVALID_ARGUMENT, "%s: tile grid too large", who);
+    return GSX_OK;
+}
+} // namespace
+
 extern "C" int gsx_intersect_tile_count(uint32_t C, uint32_t N, const float* means2d, const int32_t* radii,
                                         uint32_t tile_size, uint32_t tile_width, uint32_t tile_height,
-                                        const int32_t* order, int32_t* tiles_per_gauss,
-                                        int64_t* cum_tiles_per_gauss, void* workspace, size_t workspace_bytes,
-                                        int64_t* n_isects_host, void* stream) {
+                                        int32_t* tiles_per_gauss, int64_t* cum_tiles_per_gauss, void* workspace,
+                                        size_t workspace_bytes, int64_t* n_isects_host, void* stream) {
     GSX_REQUIRE(n_isects_host != nullptr, GSX_ERR_INVALID_ARGUMENT, "intersect_tile_count: n_isects_host is null");
     *n_isects_host = 0;
     const uint64_t n64 = (uint64_t)C * N;
@@ -289,33 +304,23 @@ extern "C" int gsx_intersect_tile_count(uint32_t C, uint32_t N, const float* mea
     GSX_REQUIRE(means2d && radii && tiles_per_gauss && cum_tiles_per_gauss, GSX_ERR_INVALID_ARGUMENT,
                 "intersect_tile_count: null tensor");
     GSX_REQUIRE(n64 < (1ull << 31), GSX_ERR_INVALID_ARGUMENT, "intersect_tile_count: C*N >= 2^31");
-    GSX_REQUIRE(tile_size > 0 && tile_width > 0 && tile_height > 0, GSX_ERR_INVALID_ARGUMENT,
-                "intersect_tile_count: empty tile grid");
-    GSX_REQUIRE((uint64_t)tile_width * tile_height < (1ull << 32) &&
-                    gsx_n_bits(tile_width * tile_height) + gsx_n_bits(C) <= 32,
-                GSX_ERR_INVALID_ARGUMENT,
-                "intersect_tile_count: tile and camera ids need more than 32 bits"); // Intersect.cpp:50
+    int rc = check_tile_grid("intersect_tile_count", C, tile_size, tile_width, tile_height);
+    if (rc != GSX_OK)
+        return rc;
     GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 &&
                     workspace_bytes >= gsx_intersect_tile_count_workspace_bytes(C, N),
                 GSX_ERR_WORKSPACE, "intersect_tile_count: workspace needs %zu bytes, 256-byte aligned",
                 gsx_intersect_tile_count_workspace_bytes(C, N));
     const uint32_t n = (uint32_t)n64;
     const uint32_t nb = cdiv(n, kScanTile);
-    GSX_REQUIRE(order == nullptr || C == 1, GSX_ERR_UNSUPPORTED, "intersect_tile_count: an order needs C == 1");
     int64_t* block_sums = (int64_t*)workspace;
     int64_t* total = block_sums + nb;
-    int32_t* counts_by_position = (int32_t*)((char*)workspace + align_up((nb + 1) * sizeof(int64_t), 256) + 256);
-    const int32_t* scan_in = order != nullptr ? counts_by_position : tiles_per_gauss;
     hipStream_t s = (hipStream_t)stream;
     hipLaunchKernelGGL(tile_count_kernel, dim3(cdiv(n, 256)), dim3(256), 0, s, n, means2d, radii, (float)tile_size,
-                       tile_width, tile_height, order, tiles_per_gauss, counts_by_position);
+                       tile_width, tile_height, tiles_per_gauss);
     GSX_LAUNCH_CHECK();
-    hipLaunchKernelGGL(scan_block_sums_kernel, dim3(nb), dim3(256), 0, s, n, scan_in, block_sums);
-    GSX_LAUNCH_CHECK();
-    hipLaunchKernelGGL(scan_block_offsets_kernel, dim3(1), dim3(256), 0, s, nb, block_sums, total);
-    GSX_LAUNCH_CHECK();
-    hipLaunchKernelGGL(scan_apply_kernel, dim3(nb), dim3(256), 0, s, n, scan_in, block_sums, cum_tiles_per_gauss);
-    GSX_LAUNCH_CHECK();
+    if ((rc = scan_counts(n, tiles_per_gauss, nullptr, cum_tiles_per_gauss, block_sums, total, s)) != GSX_OK)
+        return rc;
     // the one sanctioned host synchronisation of the path (Intersect.cpp:76 `.item<int64_t>()`)
     int64_t host_total = 0;
     GSX_HIP_CHECK(hipMemcpyAsync(&host_total, total, sizeof(int64_t), hipMemcpyDeviceToHost, s));
@@ -323,6 +328,72 @@ extern "C" int gsx_intersect_tile_count(uint32_t C, uint32_t N, const float* mea
     *n_isects_host = host_total;
     GSX_REQUIRE(host_total < (1ll << 31), GSX_ERR_OVERFLOW,
                 "intersect_tile_count: %lld intersections do not fit int32 indices", (long long)host_total);
+    return GSX_OK;
+}
+
+// workspace: keys0, keys1 (i64 [N]), vals1 (i32 [N]), scan block sums + total, then the sort's own scratch
+namespace {
+struct OrderedLayout {
+    size_t keys1_off, vals1_off, sums_off, sort_off, total;
+};
+OrderedLayout ordered_layout(uint32_t N) {
+    OrderedLayout L;
+    const size_t kb = align_up((size_t)N * 8, 256);
+    L.keys1_off = kb;
+    L.vals1_off = 2 * kb;
+    L.sums_off = L.vals1_off + align_up((size_t)N * 4, 256);
+    L.sort_off = L.sums_off + gsx_intersect_tile_count_workspace_bytes(1, N);
+    L.total = L.sort_off + gsx_radix_sort_pairs_workspace_bytes(N);
+    return L;
+}
+} // namespace
+
+extern "C" size_t gsx_intersect_tile_count_ordered_workspace_bytes(uint32_t N) { return ordered_layout(N).total; }
+
+extern "C" int gsx_intersect_tile_count_ordered(uint32_t N, const float* means2d, const int32_t* radii,
+                                                const float* depths, uint32_t tile_size, uint32_t tile_width,
+                                                uint32_t tile_height, int32_t* order, int32_t* tiles_per_gauss,
+                                                int64_t* cum_tiles_per_gauss, void* workspace,
+                                                size_t workspace_bytes, int64_t* n_isects_host, int wait,
+                                                void* stream) {
+    GSX_REQUIRE(n_isects_host != nullptr, GSX_ERR_INVALID_ARGUMENT, "intersect_tile_count_ordered: n_isects_host is null");
+    *n_isects_host = 0;
+    if (N == 0)
+        return GSX_OK;
+    GSX_REQUIRE(means2d && radii && depths && order && tiles_per_gauss && cum_tiles_per_gauss,
+                GSX_ERR_INVALID_ARGUMENT, "intersect_tile_count_ordered: null tensor");
+    GSX_REQUIRE(N < (1u << 31), GSX_ERR_INVALID_ARGUMENT, "intersect_tile_count_ordered: N >= 2^31");
+    int rc = check_tile_grid("intersect_tile_count_ordered", 1, tile_size, tile_width, tile_height);
+    if (rc != GSX_OK)
+        return rc;
+    const OrderedLayout L = ordered_layout(N);
+    GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 && workspace_bytes >= L.total,
+                GSX_ERR_WORKSPACE, "intersect_tile_count_ordered: workspace needs %zu bytes, 256-byte aligned", L.total);
+    char* ws = (char*)workspace;
+    int64_t* keys0 = (int64_t*)ws;
+    int64_t* keys1 = (int64_t*)(ws + L.keys1_off);
+    int32_t* vals1 = (int32_t*)(ws + L.vals1_off);
+    int64_t* block_sums = (int64_t*)(ws + L.sums_off);
+    int64_t* total = block_sums + cdiv(N, kScanTile);
+    hipStream_t s = (hipStream_t)stream;
+    hipLaunchKernelGGL(depth_count_keys_kernel, dim3(cdiv(N, 256)), dim3(256), 0, s, N, means2d, radii, depths,
+                       (float)tile_size, tile_width, tile_height, tiles_per_gauss, keys0, order);
+    GSX_LAUNCH_CHECK();
+    int sel = 0;
+    if ((rc = gsx_radix_sort_pairs(N, keys0, order, keys1, vals1, 0, 32, ws + L.sort_off,
+                                   gsx_radix_sort_pairs_workspace_bytes(N), &sel, stream)) != GSX_OK)
+        return rc;
+    if (sel) // four 8-bit passes end in buffer 0; kept for a different digit width
+        GSX_HIP_CHECK(hipMemcpyAsync(order, vals1, (size_t)N * 4, hipMemcpyDeviceToDevice, s));
+    if ((rc = scan_counts(N, nullptr, sel ? keys1 : keys0, cum_tiles_per_gauss, block_sums, total, s)) != GSX_OK)
+        return rc;
+    GSX_HIP_CHECK(hipMemcpyAsync(n_isects_host, total, sizeof(int64_t), hipMemcpyDeviceToHost, s));
+    if (wait) {
+        GSX_HIP_CHECK(hipStreamSynchronize(s));
+        GSX_REQUIRE(*n_isects_host < (1ll << 31), GSX_ERR_OVERFLOW,
+                    "intersect_tile_count_ordered: %lld intersections do not fit int32 indices",
+                    (long long)*n_isects_host);
+    }
     return GSX_OK;
 }
 

@@ -15,6 +15,7 @@ static constexpr uint32_t kRadix = 1u << kRadixBits;
 static constexpr uint32_t kSortItems = 16;
 static constexpr uint32_t kSortTile = 256 * kSortItems; // pairs per block
 static constexpr uint32_t kWaveTile = 64 * kSortItems;  // pairs per wave
+static constexpr uint32_t kTotalStripes = 32;
 
 __global__ void __launch_bounds__(256) fill_u32_kernel(uint32_t n, uint32_t v, uint32_t* __restrict__ out) {
     const uint32_t i = blockIdx.x * 256u + threadIdx.x;
@@ -29,7 +30,7 @@ __device__ __forceinline__ uint32_t digit_of(int64_t key, uint32_t shift, uint32
 __global__ void __launch_bounds__(256) radix_hist_kernel(uint32_t n, const int64_t* __restrict__ keys,
                                                           uint32_t shift, uint32_t mask, uint32_t nblocks,
                                                           uint32_t* __restrict__ hist /*[kRadix][nblocks]*/,
-                                                          uint32_t* __restrict__ digit_total /*[kRadix]*/) {
+                                                          uint32_t* __restrict__ digit_total /*[kTotalStripes][kRadix]*/) {
     __shared__ uint32_t lh[kRadix];
     lh[threadIdx.x] = 0;
     __syncthreads();
@@ -43,8 +44,8 @@ __global__ void __launch_bounds__(256) radix_hist_kernel(uint32_t n, const int64
     __syncthreads();
     const uint32_t c = lh[threadIdx.x];
     hist[threadIdx.x * nblocks + blockIdx.x] = c;
-    if (c)
-        atomicAdd(&digit_total[threadIdx.x], c);
+    if (c) // the totals are striped over kTotalStripes copies so that the blocks do not queue on 256 addresses
+        atomicAdd(&digit_total[(blockIdx.x % kTotalStripes) * kRadix + threadIdx.x], c);
 }
 
 // ---- per-digit scan --------------------------------------------------------------------------------
@@ -67,7 +68,12 @@ __global__ void __launch_bounds__(256) radix_scan_kernel(uint32_t nblocks, uint3
     const uint32_t d = blockIdx.x, t = threadIdx.x, lane = t & 63u, w = t >> 6;
     // pairs with a smaller digit
     {
-        const uint32_t v = t < d ? digit_total[t] : 0u;
+        uint32_t v = 0;
+        if (t < d) {
+#pragma unroll 8
+            for (uint32_t st = 0; st < kTotalStripes; ++st)
+                v += digit_total[st * kRadix + t];
+        }
         const uint32_t incl = wave_inclusive_scan_u32(v, lane);
         if (lane == 63)
             wsum[w] = incl;
@@ -182,7 +188,7 @@ SortLayout sort_layout(int64_t n) {
     L.nblocks = cdiv((uint64_t)n, kSortTile);
     L.hist_off = 0;
     L.totals_off = align_up((size_t)L.nblocks * kRadix * 4, 256);
-    L.total = L.totals_off + (size_t)kMaxPasses * kRadix * 4;
+    L.total = L.totals_off + (size_t)kMaxPasses * kTotalStripes * kRadix * 4;
     return L;
 }
 } // namespace
@@ -210,19 +216,25 @@ extern "C" int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, i
     uint32_t* hist = (uint32_t*)((char*)workspace + L.hist_off);
     uint32_t* totals = (uint32_t*)((char*)workspace + L.totals_off);
     hipStream_t s = (hipStream_t)stream;
-    hipLaunchKernelGGL(fill_u32_kernel, dim3(cdiv(kMaxPasses * kRadix, 256)), dim3(256), 0, s, kMaxPasses * kRadix,
-                       0u, totals);
+    // digits as equal as possible: ceil(bits / 8) passes of floor or ceil(bits / passes) bits (13 tile bits sort
+    // as 7 + 6, whose longer runs per (block, digit) scatter in fuller cache lines than 8 + 5)
+    const uint32_t n_bits = end_bit - begin_bit;
+    const uint32_t passes = (n_bits + kRadixBits - 1) / kRadixBits;
+    GSX_REQUIRE(passes <= kMaxPasses, GSX_ERR_INVALID_ARGUMENT, "radix_sort_pairs: %u passes", passes);
+    const uint32_t width_lo = n_bits / passes, n_wide = n_bits % passes;
+    const uint32_t n_tot = passes * kTotalStripes * kRadix;
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(cdiv(n_tot, 256)), dim3(256), 0, s, n_tot, 0u, totals);
     GSX_LAUNCH_CHECK();
     int sel = 0;
-    uint32_t pass = 0;
-    for (uint32_t shift = begin_bit; shift < end_bit; shift += kRadixBits, ++pass) {
-        const uint32_t bits = (end_bit - shift) < kRadixBits ? (end_bit - shift) : kRadixBits;
+    uint32_t shift = begin_bit;
+    for (uint32_t pass = 0; pass < passes; ++pass) {
+        const uint32_t bits = width_lo + (pass < n_wide ? 1u : 0u);
         const uint32_t mask = (1u << bits) - 1u;
         const int64_t* kin = sel ? keys1 : keys0;
         const int32_t* vin = sel ? vals1 : vals0;
         int64_t* kout = sel ? keys0 : keys1;
         int32_t* vout = sel ? vals0 : vals1;
-        uint32_t* tot = totals + pass * kRadix;
+        uint32_t* tot = totals + pass * kTotalStripes * kRadix;
         hipLaunchKernelGGL(radix_hist_kernel, dim3(L.nblocks), dim3(256), 0, s, (uint32_t)n, kin, shift, mask,
                            L.nblocks, hist, tot);
         GSX_LAUNCH_CHECK();
@@ -232,6 +244,7 @@ extern "C" int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, i
                            shift, mask, L.nblocks, hist);
         GSX_LAUNCH_CHECK();
         sel ^= 1;
+        shift += bits;
     }
     if (selector_host)
         *selector_host = sel;

@@ -275,14 +275,18 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
 // (v_mean, v_quat, v_scale) - quat_scale_to_preci_half_vjp / quat_to_rotmat_vjp of Utils.cuh:104-158.
 __global__ void __launch_bounds__(256) rasterize_bwd_epilogue_kernel(
     uint32_t N, const float* __restrict__ means, const float* __restrict__ quats, const float* __restrict__ scales,
-    const float* __restrict__ viewmat, const float* __restrict__ gacc, float* __restrict__ v_means,
+    const float* __restrict__ viewmat, float* __restrict__ gacc, int clear, float* __restrict__ v_means,
     float* __restrict__ v_quats, float* __restrict__ v_scales, float* __restrict__ v_colors,
     float* __restrict__ v_opacities) {
     const uint32_t g = blockIdx.x * 256u + threadIdx.x;
     if (g >= N)
         return;
-    const float4* row = reinterpret_cast<const float4*>(gacc + (size_t)g * kAcc);
+    float4* row = reinterpret_cast<float4*>(gacc + (size_t)g * kAcc);
     const float4 r0 = row[0], r1 = row[1], r2 = row[2], r3 = row[3];
+    if (clear) { // leave the accumulators ready for the next backward pass
+        const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+        row[0] = z, row[1] = z, row[2] = z, row[3] = z;
+    }
     // r0 = rgb.xyz, vo.x ; r1 = vo.y, vo.z, G00, G01 ; r2 = G02, G10, G11, G12 ; r3 = G20, G21, G22, v_opacity
     v_colors[(size_t)g * 3 + 0] = r0.x;
     v_colors[(size_t)g * 3 + 1] = r0.y;
@@ -424,9 +428,9 @@ extern "C" int gsx_rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_is
 
 // stage 3: per-Gaussian epilogue, accumulators -> the five gradient tensors (all elements written)
 extern "C" int gsx_rasterize_bwd_finish(uint32_t N, const float* means, const float* quats, const float* scales,
-                                        const float* viewmats0, const void* workspace, size_t workspace_bytes,
-                                        float* v_means, float* v_quats, float* v_scales, float* v_colors,
-                                        float* v_opacities, void* stream) {
+                                        const float* viewmats0, void* workspace, size_t workspace_bytes,
+                                        int clear_accumulators, float* v_means, float* v_quats, float* v_scales,
+                                        float* v_colors, float* v_opacities, void* stream) {
     if (N == 0)
         return GSX_OK;
     GSX_REQUIRE(means && quats && scales && viewmats0 && v_means && v_quats && v_scales && v_colors && v_opacities,
@@ -434,8 +438,8 @@ extern "C" int gsx_rasterize_bwd_finish(uint32_t N, const float* means, const fl
     GSX_REQUIRE(workspace != nullptr && workspace_bytes >= gsx_rasterize_bwd_accum_bytes(N), GSX_ERR_WORKSPACE,
                 "rasterize bwd: accumulators need %zu bytes", gsx_rasterize_bwd_accum_bytes(N));
     hipLaunchKernelGGL(rasterize_bwd_epilogue_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, means,
-                       quats, scales, viewmats0, (const float*)workspace, v_means, v_quats, v_scales, v_colors,
-                       v_opacities);
+                       quats, scales, viewmats0, (float*)workspace, clear_accumulators, v_means, v_quats, v_scales,
+                       v_colors, v_opacities);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }
@@ -474,6 +478,6 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
                                            last_ids, v_render_colors, v_render_alphas, workspace, acc_bytes,
                                            stream)) != GSX_OK)
         return rc;
-    return gsx_rasterize_bwd_finish(N, means, quats, scales, viewmats0, workspace, acc_bytes, v_means, v_quats,
+    return gsx_rasterize_bwd_finish(N, means, quats, scales, viewmats0, workspace, acc_bytes, 0, v_means, v_quats,
                                     v_scales, v_colors, v_opacities, stream);
 }

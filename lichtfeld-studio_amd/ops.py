@@ -104,18 +104,20 @@ def intersect_tile(means2d, radii, depths, camera_ids, gaussian_ids, C, tile_siz
     two_level = bool(sort) and C == 1
     with torch.cuda.device(dev):
         order = None
+        cum = torch.empty((C * N,), dtype=torch.int64, device=dev)
         if two_level:
             order = torch.empty((N,), dtype=torch.int32, device=dev)
-            ws_o = _workspace(lib().gsx_depth_order_workspace_bytes(c_u32(N)), dev)
-            check(lib().gsx_depth_order(c_u32(N), _ptr(depths), _ptr(radii), _ptr(order), _ptr(ws_o),
-                                        c_sz(ws_o.numel()), _stream(dev)))
-        cum = torch.empty((C * N,), dtype=torch.int64, device=dev)
-        ws_bytes = lib().gsx_intersect_tile_count_workspace_bytes(c_u32(C), c_u32(N))
-        ws = _workspace(ws_bytes, dev)
-        check(lib().gsx_intersect_tile_count(c_u32(C), c_u32(N), _ptr(means2d), _ptr(radii), c_u32(tile_size),
-                                             c_u32(tile_width), c_u32(tile_height), _ptr(order),
-                                             _ptr(tiles_per_gauss), _ptr(cum), _ptr(ws), c_sz(ws.numel()),
-                                             ctypes.byref(n_isects), _stream(dev)))
+            ws = _workspace(lib().gsx_intersect_tile_count_ordered_workspace_bytes(c_u32(N)), dev)
+            check(lib().gsx_intersect_tile_count_ordered(
+                c_u32(N), _ptr(means2d), _ptr(radii), _ptr(depths), c_u32(tile_size), c_u32(tile_width),
+                c_u32(tile_height), _ptr(order), _ptr(tiles_per_gauss), _ptr(cum), _ptr(ws), c_sz(ws.numel()),
+                ctypes.byref(n_isects), c_i(1), _stream(dev)))
+        else:
+            ws = _workspace(lib().gsx_intersect_tile_count_workspace_bytes(c_u32(C), c_u32(N)), dev)
+            check(lib().gsx_intersect_tile_count(c_u32(C), c_u32(N), _ptr(means2d), _ptr(radii), c_u32(tile_size),
+                                                 c_u32(tile_width), c_u32(tile_height), _ptr(tiles_per_gauss),
+                                                 _ptr(cum), _ptr(ws), c_sz(ws.numel()), ctypes.byref(n_isects),
+                                                 _stream(dev)))
         n = n_isects.value
         isect_ids = torch.empty((n,), dtype=torch.int64, device=dev)
         flatten_ids = torch.empty((n,), dtype=torch.int32, device=dev)

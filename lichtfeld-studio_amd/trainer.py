@@ -59,10 +59,12 @@ class TrainStep:
         self.v_colors = e(1, N, 3)
         self.tiles_per_gauss = e(N, dt=torch.int32)
         self.cum = e(N, dt=torch.int64)
-        self.ws_count = e(self.lib.gsx_intersect_tile_count_workspace_bytes(c_u32(1), c_u32(N)), dt=torch.uint8)
+        self.ws_count = e(self.lib.gsx_intersect_tile_count_ordered_workspace_bytes(c_u32(N)), dt=torch.uint8)
         self.order = e(N, dt=torch.int32)
-        self.ws_order = e(self.lib.gsx_depth_order_workspace_bytes(c_u32(N)), dt=torch.uint8)
-        self.ws_bwd = e(self.lib.gsx_rasterize_bwd_accum_bytes(c_u32(N)), dt=torch.uint8)
+        self.n_isects_pinned = torch.zeros(1, dtype=torch.int64, pin_memory=True)
+        self.count_done = torch.cuda.Event()
+        self.ws_bwd = torch.zeros(self.lib.gsx_rasterize_bwd_accum_bytes(c_u32(N)), dtype=torch.uint8,
+                                  device=self.dev)  # the backward's epilogue leaves it zeroed for the next pass
         self.records = e(self.lib.gsx_raster_records_bytes(c_u32(N)), dt=torch.uint8)
         self.cap = 0
         self.img_shape = None
@@ -147,18 +149,23 @@ class TrainStep:
             c_p(None), _p(K), c_u32(W), c_u32(H), c_f(0.3), c_f(0.01), c_f(1e4), c_f(0.0), c_i(0), self.ut, c_i(4),
             c_p(None), c_p(None), c_p(None), _p(J["radii"]), _p(J["means2d"]), _p(J["depths"]), _p(J["conics"]),
             c_p(None), s)
-        self._run("sh_colors_from_world", lb.gsx_sh_colors_from_world, c_u32(N), c_u32(self.K), c_u32(self.sh_degree), _p(P["means"]), _p(P["shs"]),
-                                          _p(J["radii"]), _p(viewmat), _p(self.colors), s)
-        n_isects = c_i64(0)
-        # depth order of the Gaussians first: the pairs then leave the emission sorted by depth and only the tile
-        # bits are left for the big sort
-        self._run("depth_order", lb.gsx_depth_order, c_u32(N), _p(J["depths"]), _p(J["radii"]), _p(self.order),
-                  _p(self.ws_order), c_sz(self.ws_order.numel()), s)
-        self._run("intersect_tile_count", lb.gsx_intersect_tile_count, c_u32(1), c_u32(N), _p(J["means2d"]),
-                  _p(J["radii"]), c_u32(16), c_u32(self.tw), c_u32(self.th), _p(self.order),
+        # Tile counts in depth order; the total comes back through pinned memory without blocking, and the SH /
+        # record passes (which do not need it) run while the host waits for it.
+        self._run("intersect_tile_count_ordered", lb.gsx_intersect_tile_count_ordered, c_u32(N), _p(J["means2d"]),
+                  _p(J["radii"]), _p(J["depths"]), c_u32(16), c_u32(self.tw), c_u32(self.th), _p(self.order),
                   _p(self.tiles_per_gauss), _p(self.cum), _p(self.ws_count), c_sz(self.ws_count.numel()),
-                  ctypes.byref(n_isects), s)
-        n = self.n_isects = n_isects.value
+                  c_p(self.n_isects_pinned.data_ptr()), c_i(0), s)
+        self.count_done.record(torch.cuda.current_stream(self.dev))
+        self._run("sh_colors_from_world", lb.gsx_sh_colors_from_world, c_u32(N), c_u32(self.K),
+                  c_u32(self.sh_degree), _p(P["means"]), _p(P["shs"]), _p(J["radii"]), _p(viewmat), _p(self.colors),
+                  s)
+        self._run("pack_raster_records", lb.gsx_pack_raster_records, c_u32(N), _p(P["means"]), _p(A["quats"]),
+                  _p(A["scales"]), _p(A["opacities"]), _p(self.colors), c_u32(3), _p(viewmat), _p(K), c_u32(W),
+                  c_u32(H), _p(self.records), s)
+        self.count_done.synchronize()
+        n = self.n_isects = int(self.n_isects_pinned[0])
+        if n >= 1 << 31:
+            raise L.GsxError(-5, f"{n} intersections do not fit int32 indices")
         self._ensure_isect_capacity(n)
         sel = c_i(0)
         if n:
@@ -173,9 +180,6 @@ class TrainStep:
         self.isect_ids, self.flatten_ids = self.keys[self.sel], self.vals[self.sel]
         self._run("intersect_offset", lb.gsx_intersect_offset, c_i64(n), _p(self.isect_ids), c_u32(1), c_u32(self.tw), c_u32(self.th),
                                       _p(self.offsets), s)
-        self._run("pack_raster_records", lb.gsx_pack_raster_records, c_u32(N), _p(P["means"]), _p(A["quats"]),
-                  _p(A["scales"]), _p(A["opacities"]), _p(self.colors), c_u32(3), _p(viewmat), _p(K), c_u32(W),
-                  c_u32(H), _p(self.records), s)
         self._run("rasterize_to_pixels_from_world_3dgs_fwd", lb.gsx_rasterize_records_fwd, c_i64(n),
                   _p(self.records), c_p(None), c_u32(3), _p(self.bg), c_p(None), c_u32(W), c_u32(H), _p(viewmat),
                   _p(K), _p(self.offsets), _p(self.flatten_ids), _p(self.render), _p(self.alpha), _p(self.last_ids),
@@ -214,14 +218,13 @@ class TrainStep:
         self._run("render_grad_from_loss", lb.gsx_render_grad_from_loss, c_u32(H), c_u32(W), c_f(self.lambda_dssim), _p(self.render),
                                            _p(self.image), _p(self.gt), _p(dimg), _p(self.v_render), s)
         ws, wsn = _p(self.ws_bwd), c_sz(self.ws_bwd.numel())
-        self._run("rasterize_bwd_clear", lb.gsx_rasterize_bwd_clear, c_u32(N), ws, wsn, s)
         self._run("rasterize_bwd_accumulate", lb.gsx_rasterize_bwd_accumulate,
                   c_u32(1), c_u32(N), c_i64(self.n_isects), _p(self.records), _p(self.bg), c_p(None), c_u32(W),
                   c_u32(H), c_u32(16),
                   _p(self.viewmat), _p(self.Kmat), _p(self.offsets), _p(self.flatten_ids), _p(self.alpha),
                   _p(self.last_ids), _p(self.v_render), _p(self.v_alpha), ws, wsn, s)
         self._run("rasterize_bwd_finish", lb.gsx_rasterize_bwd_finish, c_u32(N), _p(P["means"]), _p(A["quats"]),
-                  _p(A["scales"]), _p(self.viewmat), ws, wsn, _p(G["means"]), _p(V["quats"]), _p(V["scales"]),
+                  _p(A["scales"]), _p(self.viewmat), ws, wsn, c_i(1), _p(G["means"]), _p(V["quats"]), _p(V["scales"]),
                   _p(self.v_colors), _p(V["opacities"]), s)
         self._run("sh_colors_from_world_bwd", lb.gsx_sh_colors_from_world_bwd, c_u32(N), c_u32(self.K), c_u32(self.sh_degree), _p(P["means"]),
                                               _p(J["radii"]), _p(self.viewmat), _p(self.colors), _p(self.v_colors),

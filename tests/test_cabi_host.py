@@ -72,7 +72,7 @@ def test_status_codes_without_launch(gsx):
     assert proj(1, L.PINHOLE, L.ROLLING_TOP_TO_BOTTOM, nul) == L.GSX_ERR_UNSUPPORTED
     assert proj(1, L.PINHOLE, L.GLOBAL, one) == L.GSX_ERR_UNSUPPORTED        # viewmats1 given
     n_host = i64(-1)
-    assert lib.gsx_intersect_tile_count(u32(1), u32(10), one, one, u32(16), u32(1 << 20), u32(1 << 11), nul, one, one, one,
+    assert lib.gsx_intersect_tile_count(u32(1), u32(10), one, one, u32(16), u32(1 << 20), u32(1 << 11), one, one, one,
                                         ctypes.c_size_t(1 << 20), ctypes.byref(n_host), nul) == \
         L.GSX_ERR_INVALID_ARGUMENT  # tile id + camera id need more than 32 bits (Intersect.cpp:50)
     assert lib.gsx_radix_sort_pairs(i64(100), one, one, one, one, u32(45), u32(45), one, ctypes.c_size_t(1 << 40),
