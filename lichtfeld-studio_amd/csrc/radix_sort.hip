@@ -3,18 +3,19 @@
 //
 // 8-bit digits.  Per pass three launches: block histograms (which also add up the 256 digit totals) -> one scan
 // block per digit turns its row of the digit-major table into global start positions -> stable scatter.  A
-// block owns 4096 consecutive pairs; inside the block each 64-lane wave owns 1024 consecutive pairs and ranks
-// them 64 at a time with wave-wide match masks built from ballots, so the order (wave, round, lane) equals the
-// input order and the sort is stable.
+// block owns a tile of 256 x ITEMS consecutive pairs; inside the block each 64-lane wave owns a quarter of them
+// and ranks them 64 at a time with wave-wide match masks built from ballots, so the order (wave, round, lane)
+// equals the input order and the sort is stable.  The ranked pairs are first placed in LDS in digit order and then
+// written out by consecutive lanes, so that every (tile, digit) run leaves the block as whole cache lines.
 #include "gsx_common.h"
 
 namespace gsx {
 
 static constexpr uint32_t kRadixBits = 8;
 static constexpr uint32_t kRadix = 1u << kRadixBits;
-static constexpr uint32_t kSortItems = 16;
-static constexpr uint32_t kSortTile = 256 * kSortItems; // pairs per block
-static constexpr uint32_t kWaveTile = 64 * kSortItems;  // pairs per wave
+static constexpr uint32_t kItemsLarge = 16; // pairs per lane: 4096-pair tiles
+static constexpr uint32_t kItemsSmall = 4;  // 1024-pair tiles when there are too few pairs to fill the GPU otherwise
+static constexpr int64_t kSmallSortLimit = 1ll << 21;
 static constexpr uint32_t kTotalStripes = 32;
 
 __global__ void __launch_bounds__(256) fill_u32_kernel(uint32_t n, uint32_t v, uint32_t* __restrict__ out) {
@@ -28,15 +29,16 @@ __device__ __forceinline__ uint32_t digit_of(int64_t key, uint32_t shift, uint32
 }
 
 __global__ void __launch_bounds__(256) radix_hist_kernel(uint32_t n, const int64_t* __restrict__ keys,
-                                                          uint32_t shift, uint32_t mask, uint32_t nblocks,
+                                                          uint32_t items, uint32_t shift, uint32_t mask,
+                                                          uint32_t nblocks,
                                                           uint32_t* __restrict__ hist /*[kRadix][nblocks]*/,
                                                           uint32_t* __restrict__ digit_total /*[kTotalStripes][kRadix]*/) {
     __shared__ uint32_t lh[kRadix];
     lh[threadIdx.x] = 0;
     __syncthreads();
-    const uint32_t base = blockIdx.x * kSortTile;
-#pragma unroll
-    for (uint32_t i = 0; i < kSortItems; ++i) {
+    const uint32_t base = blockIdx.x * 256u * items;
+#pragma unroll 4
+    for (uint32_t i = 0; i < items; ++i) {
         const uint32_t idx = base + i * 256u + threadIdx.x;
         if (idx < n)
             atomicAdd(&lh[digit_of(keys[idx], shift, mask)], 1u);
@@ -103,13 +105,19 @@ __global__ void __launch_bounds__(256) radix_scan_kernel(uint32_t nblocks, uint3
 }
 
 // ---- stable scatter -------------------------------------------------------------------------------
+template <uint32_t ITEMS>
 __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const int64_t* __restrict__ keys_in,
                                                              const int32_t* __restrict__ vals_in,
                                                              int64_t* __restrict__ keys_out,
                                                              int32_t* __restrict__ vals_out, uint32_t shift,
                                                              uint32_t mask, uint32_t nblocks,
                                                              const uint32_t* __restrict__ hist_scanned) {
+    constexpr uint32_t kTileN = 256 * ITEMS, kWaveN = 64 * ITEMS;
     __shared__ uint32_t wave_count[4][kRadix];
+    __shared__ uint32_t to_global[kRadix]; // global position of a pair = to_global[digit] + its slot in the tile
+    __shared__ uint32_t wsum[4];
+    __shared__ int64_t s_keys[kTileN];
+    __shared__ int32_t s_vals[kTileN];
     const uint32_t t = threadIdx.x;
     const uint32_t w = t >> 6, lane = t & 63u;
 #pragma unroll
@@ -117,20 +125,21 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const in
         wave_count[i][t] = 0;
     __syncthreads();
 
-    const uint32_t wave_base = blockIdx.x * kSortTile + w * kWaveTile;
+    const uint32_t tile_base = blockIdx.x * kTileN;
+    const uint32_t wave_base = tile_base + w * kWaveN;
     const uint64_t lt_mask = (1ull << lane) - 1ull;
-    int64_t key[kSortItems];
-    int32_t val[kSortItems];
-    uint32_t rank[kSortItems]; // rank among the wave's pairs with the same digit
+    int64_t key[ITEMS];
+    int32_t val[ITEMS];
+    uint32_t rank[ITEMS]; // rank among the wave's pairs with the same digit
 #pragma unroll
-    for (uint32_t r = 0; r < kSortItems; ++r) {
+    for (uint32_t r = 0; r < ITEMS; ++r) {
         const uint32_t idx = wave_base + r * 64u + lane;
         const bool valid = idx < n;
         key[r] = valid ? keys_in[idx] : 0;
         val[r] = valid ? vals_in[idx] : 0;
     }
 #pragma unroll
-    for (uint32_t r = 0; r < kSortItems; ++r) {
+    for (uint32_t r = 0; r < ITEMS; ++r) {
         const uint32_t idx = wave_base + r * 64u + lane;
         const bool valid = idx < n;
         const uint32_t d = digit_of(key[r], shift, mask);
@@ -151,24 +160,46 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const in
         __builtin_amdgcn_wave_barrier();
     }
     __syncthreads();
-    // digit t: global base of this block + counts of the lower waves
+    // digit t: slot at which each wave's pairs with this digit start inside the tile (digits in ascending order,
+    // waves in ascending order inside a digit), and the offset from tile slots to global positions
     {
-        const uint32_t c0 = wave_count[0][t], c1 = wave_count[1][t], c2 = wave_count[2][t];
-        const uint32_t g = hist_scanned[t * nblocks + blockIdx.x];
+        const uint32_t c0 = wave_count[0][t], c1 = wave_count[1][t], c2 = wave_count[2][t], c3 = wave_count[3][t];
+        const uint32_t tot = c0 + c1 + c2 + c3;
+        const uint32_t incl = wave_inclusive_scan_u32(tot, lane);
+        if (lane == 63)
+            wsum[w] = incl;
         __syncthreads();
-        wave_count[0][t] = g;
-        wave_count[1][t] = g + c0;
-        wave_count[2][t] = g + c0 + c1;
-        wave_count[3][t] = g + c0 + c1 + c2;
+        uint32_t before = 0;
+#pragma unroll
+        for (uint32_t k = 0; k < 4; ++k)
+            before += k < w ? wsum[k] : 0u;
+        const uint32_t start = before + incl - tot;
+        wave_count[0][t] = start;
+        wave_count[1][t] = start + c0;
+        wave_count[2][t] = start + c0 + c1;
+        wave_count[3][t] = start + c0 + c1 + c2;
+        to_global[t] = hist_scanned[t * nblocks + blockIdx.x] - start;
     }
     __syncthreads();
 #pragma unroll
-    for (uint32_t r = 0; r < kSortItems; ++r) {
+    for (uint32_t r = 0; r < ITEMS; ++r) {
         const uint32_t idx = wave_base + r * 64u + lane;
         if (idx < n) {
-            const uint32_t pos = wave_count[w][digit_of(key[r], shift, mask)] + rank[r];
-            keys_out[pos] = key[r];
-            vals_out[pos] = val[r];
+            const uint32_t slot = wave_count[w][digit_of(key[r], shift, mask)] + rank[r];
+            s_keys[slot] = key[r];
+            s_vals[slot] = val[r];
+        }
+    }
+    __syncthreads();
+    const uint32_t count = min(kTileN, n - tile_base);
+#pragma unroll
+    for (uint32_t k = 0; k < ITEMS; ++k) {
+        const uint32_t slot = k * 256u + t;
+        if (slot < count) {
+            const int64_t kk = s_keys[slot];
+            const uint32_t pos = to_global[digit_of(kk, shift, mask)] + slot;
+            keys_out[pos] = kk;
+            vals_out[pos] = s_vals[slot];
         }
     }
 }
@@ -183,9 +214,10 @@ struct SortLayout {
     uint32_t nblocks;
     size_t hist_off, totals_off, total;
 };
+uint32_t sort_items(int64_t n) { return n <= kSmallSortLimit ? kItemsSmall : kItemsLarge; }
 SortLayout sort_layout(int64_t n) {
     SortLayout L;
-    L.nblocks = cdiv((uint64_t)n, kSortTile);
+    L.nblocks = cdiv((uint64_t)n, 256u * sort_items(n));
     L.hist_off = 0;
     L.totals_off = align_up((size_t)L.nblocks * kRadix * 4, 256);
     L.total = L.totals_off + (size_t)kMaxPasses * kTotalStripes * kRadix * 4;
@@ -193,10 +225,13 @@ SortLayout sort_layout(int64_t n) {
 }
 } // namespace
 
+// monotone in n (a workspace sized for a capacity serves every smaller sort, whichever tile size that one uses)
 extern "C" size_t gsx_radix_sort_pairs_workspace_bytes(int64_t n) {
     if (n <= 0)
         return 256;
-    return sort_layout(n).total;
+    const size_t need = sort_layout(n).total;
+    const size_t small_max = sort_layout(kSmallSortLimit).total;
+    return n > kSmallSortLimit && small_max > need ? small_max : need;
 }
 
 extern "C" int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, int64_t* keys1, int32_t* vals1,
@@ -227,6 +262,7 @@ extern "C" int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, i
     GSX_LAUNCH_CHECK();
     int sel = 0;
     uint32_t shift = begin_bit;
+    const uint32_t items = sort_items(n);
     for (uint32_t pass = 0; pass < passes; ++pass) {
         const uint32_t bits = width_lo + (pass < n_wide ? 1u : 0u);
         const uint32_t mask = (1u << bits) - 1u;
@@ -235,13 +271,17 @@ extern "C" int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, i
         int64_t* kout = sel ? keys0 : keys1;
         int32_t* vout = sel ? vals0 : vals1;
         uint32_t* tot = totals + pass * kTotalStripes * kRadix;
-        hipLaunchKernelGGL(radix_hist_kernel, dim3(L.nblocks), dim3(256), 0, s, (uint32_t)n, kin, shift, mask,
+        hipLaunchKernelGGL(radix_hist_kernel, dim3(L.nblocks), dim3(256), 0, s, (uint32_t)n, kin, items, shift, mask,
                            L.nblocks, hist, tot);
         GSX_LAUNCH_CHECK();
         hipLaunchKernelGGL(radix_scan_kernel, dim3(kRadix), dim3(256), 0, s, L.nblocks, hist, tot);
         GSX_LAUNCH_CHECK();
-        hipLaunchKernelGGL(radix_scatter_kernel, dim3(L.nblocks), dim3(256), 0, s, (uint32_t)n, kin, vin, kout, vout,
-                           shift, mask, L.nblocks, hist);
+        if (items == kItemsSmall)
+            hipLaunchKernelGGL((radix_scatter_kernel<kItemsSmall>), dim3(L.nblocks), dim3(256), 0, s, (uint32_t)n, kin,
+                               vin, kout, vout, shift, mask, L.nblocks, hist);
+        else
+            hipLaunchKernelGGL((radix_scatter_kernel<kItemsLarge>), dim3(L.nblocks), dim3(256), 0, s, (uint32_t)n, kin,
+                               vin, kout, vout, shift, mask, L.nblocks, hist);
         GSX_LAUNCH_CHECK();
         sel ^= 1;
         shift += bits;

@@ -283,7 +283,11 @@ __global__ void __launch_bounds__(256) rasterize_bwd_epilogue_kernel(
         return;
     float4* row = reinterpret_cast<float4*>(gacc + (size_t)g * kAcc);
     const float4 r0 = row[0], r1 = row[1], r2 = row[2], r3 = row[3];
-    if (clear) { // leave the accumulators ready for the next backward pass
+    const bool any_geo = (r0.w != 0.f) | (r1.x != 0.f) | (r1.y != 0.f) | (r1.z != 0.f) | (r1.w != 0.f) |
+                         (r2.x != 0.f) | (r2.y != 0.f) | (r2.z != 0.f) | (r2.w != 0.f) | (r3.x != 0.f) |
+                         (r3.y != 0.f) | (r3.z != 0.f);
+    // leave the accumulators ready for the next backward pass; rows no pixel touched are still zero
+    if (clear && (any_geo | (r0.x != 0.f) | (r0.y != 0.f) | (r0.z != 0.f) | (r3.w != 0.f))) {
         const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
         row[0] = z, row[1] = z, row[2] = z, row[3] = z;
     }
@@ -292,9 +296,6 @@ __global__ void __launch_bounds__(256) rasterize_bwd_epilogue_kernel(
     v_colors[(size_t)g * 3 + 1] = r0.y;
     v_colors[(size_t)g * 3 + 2] = r0.z;
     v_opacities[g] = r3.w;
-    const bool any_geo = (r0.w != 0.f) | (r1.x != 0.f) | (r1.y != 0.f) | (r1.z != 0.f) | (r1.w != 0.f) |
-                         (r2.x != 0.f) | (r2.y != 0.f) | (r2.z != 0.f) | (r2.w != 0.f) | (r3.x != 0.f) |
-                         (r3.y != 0.f) | (r3.z != 0.f);
     float vm[3] = {0.f, 0.f, 0.f}, vq[4] = {0.f, 0.f, 0.f, 0.f}, vs[3] = {0.f, 0.f, 0.f};
     if (any_geo) {
         const CamPose cp = load_cam_pose(viewmat);
