@@ -25,6 +25,12 @@ PKG_DIR = os.path.join(ROOT, "lichtfeld-studio_amd")
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+# HBM bytes per launch of the dominant kernel at the default workload, from two rocprofv3 --pmc runs (FETCH_SIZE,
+# WRITE_SIZE, each scaled by what the same counter reads for gsx_debug_copy's known 256 MiB + 256 MiB); the figures
+# and the commands are in profiles/train_step_1M_1237x822_hbm_traffic.txt.  Counters cannot be read from inside
+# this process, so the value is only attached when the workload is the one it was measured on.
+MEASURED_TRAFFIC_BYTES = {("rasterize_bwd_kernel", 3, 1_000_000): 223.7e6}
+
 # published MI355X peaks
 PEAK_HBM_GBS = 8000.0
 PEAK_FP32_TFLOPS = 157.3
@@ -182,10 +188,12 @@ def main():
     dom_tf = flops_bwd / (dom_ms * 1e-3) / 1e12
     roofline = {
         "kernel": "rasterize_bwd_kernel", "bound": "fp32_valu", "achieved": round(dom_tf, 3),
-        "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s", "frac": round(dom_tf / PEAK_FP32_TFLOPS, 4), "traffic": None,
+        "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s", "frac": round(dom_tf / PEAK_FP32_TFLOPS, 4),
+        "traffic": MEASURED_TRAFFIC_BYTES.get(("rasterize_bwd_kernel", args.config, ts.N)),
         "avg_launch_ms": round(dom_ms, 4), "launches": len(in_loop[dominant]),
-        "note": "no MFMA and not HBM-bound: per-pair fp32 vector ALU work; algorithmic flops = 62 x pairs "
-                "evaluated + 180 x pairs composited",
+        "note": "no MFMA and not HBM-bound: per-pair fp32 vector ALU work; algorithmic flops = 62 x pairs the "
+                "backward walks + 180 x pairs composited; traffic = HBM bytes per launch (rocprofv3 FETCH_SIZE + "
+                "WRITE_SIZE, copy-kernel calibrated), far below what 78.6 TFLOP/s non-packed fp32 issue needs",
     }
 
     cpu_baseline = None
