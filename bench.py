@@ -76,6 +76,7 @@ def algorithmic_bytes(N, K, H, W, n_isects, sort_bits):
         "sh_colors_from_world_bwd": N * (12 + 8 + 12 + 12 + 12 * K),
         "activate_params_bwd": N * (32 + 32 + 32),
         "adam_step_multi": N * (11 + 3 * K) * 28,
+        "backward_update_fused": N * ((11 + 3 * K) * 24 + 64 + 64 + 12 + 8),
     }
 
 
@@ -87,6 +88,8 @@ def main():
     ap.add_argument("--config", type=int, default=3, help="BASELINE configuration (3 = the metric's)")
     ap.add_argument("--n", type=int, default=None, help="override the number of Gaussians (parity / debugging)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--separate-update", action="store_true",
+                    help="run epilogue / SH backward / activation VJPs / Adam as separate kernels (default: one pass)")
     ap.add_argument("--cpu-threads", type=int, default=0, help="threads for the CPU baseline (0 = all)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -117,7 +120,7 @@ def main():
     else:
         gt = torch.from_numpy(sc.target[None].copy()).to(dev)
     use_ssim = args.config != 1  # configuration 1 is L1 only
-    ts = TrainStep(sc, dev, use_ssim=use_ssim)
+    ts = TrainStep(sc, dev, use_ssim=use_ssim, fused_update=not args.separate_update)
     setup_s = time.time() - t0
 
     dominant = "rasterize_bwd_accumulate"

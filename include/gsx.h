@@ -295,6 +295,28 @@ GSX_API int gsx_activate_params_bwd(uint32_t N, const float* opacity_raw, const 
                                     const float* rotation_raw, const float* v_opacities, const float* v_scales,
                                     const float* v_quats, float* v_opacity_raw, float* v_scaling_raw,
                                     float* v_rotation_raw, void* stream);
+/* The tail of a training step in ONE pass over the Gaussians (no counterpart in the reference, which runs them as
+ * separate kernels and ATen ops): rasterizer-backward epilogue (as gsx_rasterize_bwd_finish with
+ * clear_accumulators = 1, on the ACTIVATIONS of the raw parameters) -> SH backward with the clamp mask (as
+ * gsx_sh_colors_from_world_bwd) -> activation VJPs (as gsx_activate_params_bwd) -> Adam on the five raw parameter
+ * tensors (as gsx_adam_step_multi with sh0 | shN interleaved in `shs` [N,K,3]).  The 236 B / Gaussian of gradients
+ * never reach memory; parameters and moments come out bit-identical to the separate calls.  Must run before the
+ * parameters change in any other way: it re-derives the activations from the raw parameters. */
+typedef struct gsx_update_args {
+    uint32_t N, K, sh_degree;
+    float *means, *opacity_raw, *scaling_raw, *rotation_raw, *shs;                        /* parameters (in / out) */
+    float *m_means, *m_opacity, *m_scaling, *m_rotation, *m_shs;                          /* exp_avg (in / out) */
+    float *v_means, *v_opacity, *v_scaling, *v_rotation, *v_shs;                          /* exp_avg_sq (in / out) */
+    const int32_t* radii;  /* [N,2] of the forward pass */
+    const float* colors;   /* [N,3] of the forward pass (clamp mask) */
+    const float* viewmat;  /* [4,4] */
+    void* accumulators;    /* gsx_rasterize_bwd_accumulate's workspace; consumed rows are zeroed */
+    float lr_means, lr_sh0, lr_shN, lr_scaling, lr_rotation, lr_opacity;
+    float beta1, beta2, eps, bias_correction1_rcp, bias_correction2_sqrt_rcp;
+    int32_t skip_shN;      /* fused_adam.cpp:69-70 */
+} gsx_update_args;
+GSX_API int gsx_backward_update_fused(const gsx_update_args* args_host, void* stream);
+
 /* image = clamp(render HWC -> CHW, 0, 1) (rasterizer.cpp:205) and the per-pixel part of the photometric
  * loss of trainer.cpp:126-129: partial sums of |image - gt| into l1_partials [gsx_image_loss_blocks()]. */
 GSX_API uint32_t gsx_image_loss_blocks(uint32_t H, uint32_t W);

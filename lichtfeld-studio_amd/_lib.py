@@ -50,6 +50,19 @@ class RowTensor(ctypes.Structure):
     _fields_ = [("data", c_p), ("row_floats", c_u32), ("is_optimizer_state", ctypes.c_int32)]
 
 
+class UpdateArgs(ctypes.Structure):
+    """gsx_update_args"""
+    _fields_ = ([("N", c_u32), ("K", c_u32), ("sh_degree", c_u32)] +
+                [(n, c_p) for n in ("means", "opacity_raw", "scaling_raw", "rotation_raw", "shs", "m_means",
+                                    "m_opacity", "m_scaling", "m_rotation", "m_shs", "v_means", "v_opacity",
+                                    "v_scaling", "v_rotation", "v_shs", "radii", "colors", "viewmat",
+                                    "accumulators")] +
+                [(n, c_f) for n in ("lr_means", "lr_sh0", "lr_shN", "lr_scaling", "lr_rotation", "lr_opacity",
+                                    "beta1", "beta2", "eps", "bias_correction1_rcp",
+                                    "bias_correction2_sqrt_rcp")] +
+                [("skip_shN", ctypes.c_int32)])
+
+
 class GsxError(RuntimeError):
     def __init__(self, status, message):
         super().__init__(f"gsx status {status}: {message}")

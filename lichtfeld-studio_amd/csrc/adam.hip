@@ -5,6 +5,7 @@
 #include <string.h>
 
 #include "gsx_common.h"
+#include "gsx_step.h"
 
 namespace gsx {
 
@@ -25,17 +26,6 @@ struct AdamTable {
     int32_t skip2[GSX_ADAM_MAX_TENSORS];
     int n_groups;
 };
-
-__device__ __forceinline__ void adam_one(float& p, float& m, float& v, float g, float lr, float beta1, float beta2,
-                                         float eps, float bc1_rcp, float bc2_sqrt_rcp) {
-    const float moment1 = beta1 * m + (1.0f - beta1) * g;
-    const float moment2 = beta2 * v + (1.0f - beta2) * g * g;
-    const float denom = gsx::sqrt(moment2) * bc2_sqrt_rcp + eps;
-    const float step_size = lr * bc1_rcp;
-    p -= step_size * moment1 / denom;
-    m = moment1;
-    v = moment2;
-}
 
 __global__ void __launch_bounds__(256) adam_multi_kernel(const AdamTable tab) {
     int gi = 0;

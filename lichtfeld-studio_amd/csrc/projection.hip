@@ -4,6 +4,7 @@
 // All of these touch each Gaussian once and are bound by HBM bandwidth; one lane owns one Gaussian and
 // rows are read with whole-row vector loads.
 #include "gsx_common.h"
+#include "gsx_step.h"
 
 namespace gsx {
 
@@ -179,58 +180,6 @@ __global__ void __launch_bounds__(256) projection_ut_kernel(
 // Spherical harmonics (gsplat/SphericalHarmonicsCUDA.cu:20-110): basis values and the colour of one
 // channel in the reference's summation order.
 // ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ int sh_basis(uint32_t degree, vec3 dir, float* B) {
-    B[0] = 0.2820947917738781f;
-    if (degree < 1)
-        return 1;
-    const float inorm = gsx::rsqrt(dir.x * dir.x + dir.y * dir.y + dir.z * dir.z);
-    const float x = dir.x * inorm, y = dir.y * inorm, z = dir.z * inorm;
-    B[1] = -0.48860251190292f * y;
-    B[2] = 0.48860251190292f * z;
-    B[3] = -0.48860251190292f * x;
-    if (degree < 2)
-        return 4;
-    const float z2 = z * z;
-    const float fTmp0B = -1.092548430592079f * z;
-    const float fC1 = x * x - y * y;
-    const float fS1 = 2.f * x * y;
-    B[6] = (0.9461746957575601f * z2 - 0.3153915652525201f);
-    B[7] = fTmp0B * x;
-    B[5] = fTmp0B * y;
-    B[8] = 0.5462742152960395f * fC1;
-    B[4] = 0.5462742152960395f * fS1;
-    if (degree < 3)
-        return 9;
-    const float fTmp0C = -2.285228997322329f * z2 + 0.4570457994644658f;
-    const float fTmp1B = 1.445305721320277f * z;
-    const float fC2 = x * fC1 - y * fS1;
-    const float fS2 = x * fS1 + y * fC1;
-    B[12] = z * (1.865881662950577f * z2 - 1.119528997770346f);
-    B[13] = fTmp0C * x;
-    B[11] = fTmp0C * y;
-    B[14] = fTmp1B * fC1;
-    B[10] = fTmp1B * fS1;
-    B[15] = -0.5900435899266435f * fC2;
-    B[9] = -0.5900435899266435f * fS2;
-    if (degree < 4)
-        return 16;
-    const float fTmp0D = z * (-4.683325804901025f * z2 + 2.007139630671868f);
-    const float fTmp1C = 3.31161143515146f * z2 - 0.47308734787878f;
-    const float fTmp2B = -1.770130769779931f * z;
-    const float fC3 = x * fC2 - y * fS2;
-    const float fS3 = x * fS2 + y * fC2;
-    B[20] = (1.984313483298443f * z * B[12] - 1.006230589874905f * B[6]);
-    B[21] = fTmp0D * x;
-    B[19] = fTmp0D * y;
-    B[22] = fTmp1C * fC1;
-    B[18] = fTmp1C * fS1;
-    B[23] = fTmp2B * fC2;
-    B[17] = fTmp2B * fS2;
-    B[24] = 0.6258357354491763f * fC3;
-    B[16] = 0.6258357354491763f * fS3;
-    return 25;
-}
-
 // co: the Gaussian's coefficients, element (k, c) at co[k * 3 + c]
 __device__ __forceinline__ float sh_color_channel(uint32_t degree, vec3 dir, const float* B,
                                                   const float* __restrict__ co, uint32_t c) {
@@ -359,15 +308,12 @@ __global__ void __launch_bounds__(256) activate_params_kernel(uint32_t N, const 
     const uint32_t i = blockIdx.x * 256u + threadIdx.x;
     if (i >= N)
         return;
-    opacities[i] = gsx::sigmoid(opacity_raw[i]);
-    const vec3 s = ld3(scaling_raw, i);
-    scales[3 * i + 0] = gsx::exp(s.x);
-    scales[3 * i + 1] = gsx::exp(s.y);
-    scales[3 * i + 2] = gsx::exp(s.z);
-    const quat q = ld4q(rotation_raw, i);
-    // torch::nn::functional::normalize: x / max(||x||_2, eps), eps = 1e-12
-    const float nrm = gsx::fmax(gsx::sqrt(qdot(q, q)), 1e-12f);
-    reinterpret_cast<float4*>(quats)[i] = make_float4(q.w / nrm, q.x / nrm, q.y / nrm, q.z / nrm);
+    const Activated a = activate(opacity_raw[i], ld3(scaling_raw, i), ld4q(rotation_raw, i));
+    opacities[i] = a.opacity;
+    scales[3 * i + 0] = a.scales.x;
+    scales[3 * i + 1] = a.scales.y;
+    scales[3 * i + 2] = a.scales.z;
+    reinterpret_cast<float4*>(quats)[i] = make_float4(a.quat.w, a.quat.x, a.quat.y, a.quat.z);
 }
 
 // VJPs of the three activations (what autograd applies to the gradients Ops.h's backward returns)
@@ -379,75 +325,14 @@ __global__ void __launch_bounds__(256) activate_params_bwd_kernel(
     const uint32_t i = blockIdx.x * 256u + threadIdx.x;
     if (i >= N)
         return;
-    const float o = gsx::sigmoid(opacity_raw[i]);
-    v_opacity_raw[i] = v_opacities[i] * (o * (1.0f - o));
-    const vec3 s = ld3(scaling_raw, i);
-    v_scaling_raw[3 * i + 0] = v_scales[3 * i + 0] * gsx::exp(s.x);
-    v_scaling_raw[3 * i + 1] = v_scales[3 * i + 1] * gsx::exp(s.y);
-    v_scaling_raw[3 * i + 2] = v_scales[3 * i + 2] * gsx::exp(s.z);
-    const quat q = ld4q(rotation_raw, i);
-    const quat g = ld4q(v_quats, i);
-    const float len = gsx::sqrt(qdot(q, q));
-    float4 out;
-    if (len > 1e-12f) {
-        // y = x / len : v_x = (g - y (y . g)) / len
-        const float inv = 1.0f / len;
-        const float yw = q.w * inv, yx = q.x * inv, yy = q.y * inv, yz = q.z * inv;
-        const float d = g.w * yw + g.x * yx + g.y * yy + g.z * yz;
-        out = make_float4((g.w - yw * d) * inv, (g.x - yx * d) * inv, (g.y - yy * d) * inv, (g.z - yz * d) * inv);
-    } else {
-        out = make_float4(g.w * 1e12f, g.x * 1e12f, g.y * 1e12f, g.z * 1e12f);
-    }
-    reinterpret_cast<float4*>(v_rotation_raw)[i] = out;
-}
-
-// campos = translation column of inverse([R|t]) = -R^T t (Rasterization.cpp:358-359 uses at::inverse; for the
-// rigid matrices LichtFeld passes the two agree).  Evaluated per lane from the uniform matrix: the matrix
-// lives in device memory and a host copy would cost a synchronisation.
-__device__ __forceinline__ vec3 campos_from_viewmat(const float* __restrict__ vm) {
-    mat3 R;
-#pragma unroll
-    for (int r = 0; r < 3; ++r)
-#pragma unroll
-        for (int c = 0; c < 3; ++c)
-            R.m[r][c] = vm[r * 4 + c];
-    return neg(mul_t(R, mk3(vm[3], vm[7], vm[11])));
-}
-
-// ---- coefficient rows through LDS (K = 16) -----------------------------------------------------
-// A lane owns one Gaussian, whose 16x3 coefficients are a 192-byte row; lanes reading or writing their own rows
-// directly touch 64 different cache lines per instruction.  Instead a wave moves its 64 rows (12 KiB, contiguous in
-// memory) with fully coalesced 16-byte accesses and transposes through LDS; rows are padded to 13 x 16 bytes so
-// that the per-lane 16-byte LDS accesses are conflict-free.
-static constexpr uint32_t kShRowF4 = 12;   // float4 per row (K = 16)
-static constexpr uint32_t kShLdsF4 = 13;   // padded row stride in float4
-
-__device__ __forceinline__ void sh16_rows_to_lds(const float* __restrict__ coeffs, uint32_t row0, uint32_t N,
-                                                 float4* wave_lds, uint32_t lane) {
-    const float4* src = reinterpret_cast<const float4*>(coeffs + (size_t)row0 * 48);
-    const uint32_t n_f4 = min(64u, N - row0) * kShRowF4;
-#pragma unroll
-    for (uint32_t i = 0; i < kShRowF4; ++i) {
-        const uint32_t q = i * 64u + lane;
-        if (q < n_f4) {
-            const uint32_t r = (q * 43691u) >> 19; // q / 12 for q < 768
-            wave_lds[r * kShLdsF4 + (q - r * kShRowF4)] = src[q];
-        }
-    }
-}
-
-__device__ __forceinline__ void sh16_rows_from_lds(float* __restrict__ v_coeffs, uint32_t row0, uint32_t N,
-                                                   const float4* wave_lds, uint32_t lane) {
-    float4* dst = reinterpret_cast<float4*>(v_coeffs + (size_t)row0 * 48);
-    const uint32_t n_f4 = min(64u, N - row0) * kShRowF4;
-#pragma unroll
-    for (uint32_t i = 0; i < kShRowF4; ++i) {
-        const uint32_t q = i * 64u + lane;
-        if (q < n_f4) {
-            const uint32_t r = (q * 43691u) >> 19;
-            dst[q] = wave_lds[r * kShLdsF4 + (q - r * kShRowF4)];
-        }
-    }
+    const vec3 vs = ld3(v_scales, i);
+    const ActivationVjp a = activation_vjp(opacity_raw[i], ld3(scaling_raw, i), ld4q(rotation_raw, i), v_opacities[i],
+                                           vs, ld4q(v_quats, i));
+    v_opacity_raw[i] = a.opacity;
+    v_scaling_raw[3 * i + 0] = a.scaling.x;
+    v_scaling_raw[3 * i + 1] = a.scaling.y;
+    v_scaling_raw[3 * i + 2] = a.scaling.z;
+    reinterpret_cast<float4*>(v_rotation_raw)[i] = make_float4(a.rotation.w, a.rotation.x, a.rotation.y, a.rotation.z);
 }
 
 // glue of the fused entry point (Rasterization.cpp:356-378): dirs, radii mask, SH, +0.5, clamp in one pass.

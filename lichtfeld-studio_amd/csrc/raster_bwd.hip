@@ -17,6 +17,7 @@
 // Sums are formed in a different order than the reference's warp reduce + atomics (whose order is itself
 // unspecified), so results agree to rounding, not bitwise.
 #include "gsx_common.h"
+#include "gsx_step.h"
 
 namespace gsx {
 
@@ -297,63 +298,8 @@ __global__ void __launch_bounds__(256) rasterize_bwd_epilogue_kernel(
     v_colors[(size_t)g * 3 + 2] = r0.z;
     v_opacities[g] = r3.w;
     float vm[3] = {0.f, 0.f, 0.f}, vq[4] = {0.f, 0.f, 0.f, 0.f}, vs[3] = {0.f, 0.f, 0.f};
-    if (any_geo) {
-        const CamPose cp = load_cam_pose(viewmat);
-        quat qp;
-        vec3 tp;
-        shutter_pose(cp, 0.f, &qp, &tp);
-        const mat3 R_inv = mat3_cast(quat_inverse(qp));
-        const vec3 ray_o = neg(mul(R_inv, tp));
-        const vec3 om = sub(ray_o, ld3(means, g));
-        const quat q = ld4q(quats, g);
-        const mat3 R = quat_to_rotmat(q);
-        const vec3 s = ld3(scales, g);
-        const float is[3] = {1.0f / s.x, 1.0f / s.y, 1.0f / s.z};
-        mat3 Mt;
-#pragma unroll
-        for (int a = 0; a < 3; ++a)
-#pragma unroll
-            for (int b = 0; b < 3; ++b)
-                Mt.m[a][b] = is[a] * R.m[b][a];
-        const vec3 Vo = mk3(r0.w, r1.x, r1.y);
-        const float G[3][3] = {{r1.z, r1.w, r2.x}, {r2.y, r2.z, r2.w}, {r3.x, r3.y, r3.z}};
-        const float vo[3] = {Vo.x, Vo.y, Vo.z};
-        const float omv[3] = {om.x, om.y, om.z};
-        float v_Mt[3][3];
-#pragma unroll
-        for (int a = 0; a < 3; ++a)
-#pragma unroll
-            for (int b = 0; b < 3; ++b)
-                v_Mt[a][b] = fma(vo[a], omv[b], G[a][b]);
-        const vec3 v_o = mul_t(Mt, Vo);
-        vm[0] = -v_o.x;
-        vm[1] = -v_o.y;
-        vm[2] = -v_o.z;
-        float vr[3][3]; // v_R(k,j) = v_M(k,j) / s_j, v_M = v_Mt^T
-#pragma unroll
-        for (int k = 0; k < 3; ++k)
-#pragma unroll
-            for (int jj = 0; jj < 3; ++jj)
-                vr[k][jj] = v_Mt[jj][k] * is[jj];
-        const float inv_norm = gsx::rsqrt(fma(q.w, q.w, fma(q.z, q.z, fma(q.y, q.y, q.x * q.x))));
-        const float x = q.x * inv_norm, y = q.y * inv_norm, z = q.z * inv_norm, w = q.w * inv_norm;
-        const float vq_w = 2.f * (x * (vr[2][1] - vr[1][2]) + y * (vr[0][2] - vr[2][0]) + z * (vr[1][0] - vr[0][1]));
-        const float vq_x = 2.f * (-2.f * x * (vr[1][1] + vr[2][2]) + y * (vr[1][0] + vr[0][1]) +
-                                  z * (vr[2][0] + vr[0][2]) + w * (vr[2][1] - vr[1][2]));
-        const float vq_y = 2.f * (x * (vr[1][0] + vr[0][1]) - 2.f * y * (vr[0][0] + vr[2][2]) +
-                                  z * (vr[2][1] + vr[1][2]) + w * (vr[0][2] - vr[2][0]));
-        const float vq_z = 2.f * (x * (vr[2][0] + vr[0][2]) + y * (vr[2][1] + vr[1][2]) -
-                                  2.f * z * (vr[0][0] + vr[1][1]) + w * (vr[1][0] - vr[0][1]));
-        const float d = vq_w * w + vq_x * x + vq_y * y + vq_z * z;
-        vq[0] = (vq_w - d * w) * inv_norm;
-        vq[1] = (vq_x - d * x) * inv_norm;
-        vq[2] = (vq_y - d * y) * inv_norm;
-        vq[3] = (vq_z - d * z) * inv_norm;
-#pragma unroll
-        for (int jj = 0; jj < 3; ++jj)
-            vs[jj] = -is[jj] * is[jj] *
-                     (R.m[0][jj] * v_Mt[jj][0] + R.m[1][jj] * v_Mt[jj][1] + R.m[2][jj] * v_Mt[jj][2]);
-    }
+    if (any_geo)
+        epilogue_geometry_grads(r0, r1, r2, r3, viewmat, ld3(means, g), ld4q(quats, g), ld3(scales, g), vm, vq, vs);
 #pragma unroll
     for (int k = 0; k < 3; ++k) {
         v_means[(size_t)g * 3 + k] = vm[k];

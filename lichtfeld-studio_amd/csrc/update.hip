@@ -1,0 +1,243 @@
+// update.hip - the tail of a training step in one pass over the Gaussians: rasterizer-backward epilogue
+// (Utils.cuh:104-158) -> SH backward with the clamp mask (Rasterization.cpp:608-624) -> VJPs of the activations
+// (autograd of splat_data.cpp:271-286) -> Adam on all parameter tensors (adam_kernels.cuh:13-36,
+// fused_adam.cpp:22-95).
+//
+// The separate kernels write 236 B of raw-parameter gradients per Gaussian and the optimiser reads them back; here
+// they stay in registers.  Arithmetic is that of the separate kernels (same device functions), so parameters and
+// moments come out bit-identical to epilogue + sh_colors_from_world_bwd + activate_params_bwd + adam_step_multi.
+// The 192-byte SH rows of the parameter and of both moments move through LDS with coalesced 16-byte accesses, one
+// tensor at a time: moment 1, moment 2 (their new values stay in registers), then the parameter.
+#include <string.h>
+
+#include "gsx_common.h"
+#include "gsx_step.h"
+
+namespace gsx {
+
+struct UpdateArgs {
+    uint32_t N, K, sh_degree;
+    float *means, *opacity_raw, *scaling_raw, *rotation_raw, *shs;
+    float *m_means, *m_opacity, *m_scaling, *m_rotation, *m_shs;
+    float *v_means, *v_opacity, *v_scaling, *v_rotation, *v_shs;
+    const int32_t* radii;
+    const float* colors;
+    const float* viewmat;
+    float* acc;
+    float lr_means, lr_sh0, lr_shN, lr_scaling, lr_rotation, lr_opacity;
+    float beta1, beta2, eps, bc1_rcp, bc2_sqrt_rcp;
+    int32_t skip_shN;
+};
+
+// new first / second moment of one element (the first two lines of adam_one)
+__device__ __forceinline__ float adam_m(float m, float g, float beta1) { return beta1 * m + (1.0f - beta1) * g; }
+__device__ __forceinline__ float adam_v(float v, float g, float beta2) { return beta2 * v + (1.0f - beta2) * g * g; }
+__device__ __forceinline__ float adam_p(float p, float m1, float v1, float lr, float eps, float c1, float c2) {
+    const float denom = gsx::sqrt(v1) * c2 + eps;
+    const float step_size = lr * c1;
+    return p - step_size * m1 / denom;
+}
+
+template <int n>
+__device__ __forceinline__ void adam_row(float* __restrict__ P, float* __restrict__ M, float* __restrict__ V,
+                                         uint32_t e, const float (&g)[n], float lr, const UpdateArgs& a) {
+#pragma unroll
+    for (int k = 0; k < n; ++k) {
+        float p = P[(size_t)e * n + k], m = M[(size_t)e * n + k], v = V[(size_t)e * n + k];
+        adam_one(p, m, v, g[k], lr, a.beta1, a.beta2, a.eps, a.bc1_rcp, a.bc2_sqrt_rcp);
+        P[(size_t)e * n + k] = p;
+        M[(size_t)e * n + k] = m;
+        V[(size_t)e * n + k] = v;
+    }
+}
+
+template <bool LDS16>
+__global__ void __launch_bounds__(256) backward_update_kernel(const UpdateArgs a) {
+    __shared__ float4 lds[LDS16 ? 4 * 64 * kShLdsF4 : 1];
+    const uint32_t e = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    float4* wave_lds = lds + (LDS16 ? wave * 64 * kShLdsF4 : 0);
+    const bool in = e < a.N;
+
+    float B[25];
+    int nb = 0;
+    float vc[3] = {0.f, 0.f, 0.f}; // d loss / d colour behind the clamp
+    if (in) {
+        // ---- epilogue of the rasterizer backward ----
+        float4* row = reinterpret_cast<float4*>(a.acc + (size_t)e * 16);
+        const float4 r0 = row[0], r1 = row[1], r2 = row[2], r3 = row[3];
+        const bool any_geo = (r0.w != 0.f) | (r1.x != 0.f) | (r1.y != 0.f) | (r1.z != 0.f) | (r1.w != 0.f) |
+                             (r2.x != 0.f) | (r2.y != 0.f) | (r2.z != 0.f) | (r2.w != 0.f) | (r3.x != 0.f) |
+                             (r3.y != 0.f) | (r3.z != 0.f);
+        if (any_geo | (r0.x != 0.f) | (r0.y != 0.f) | (r0.z != 0.f) | (r3.w != 0.f)) {
+            const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+            row[0] = z, row[1] = z, row[2] = z, row[3] = z; // ready for the next backward pass
+        }
+        const vec3 mean = ld3(a.means, e);
+        const float o_raw = a.opacity_raw[e];
+        const vec3 s_raw = ld3(a.scaling_raw, e);
+        const quat q_raw = ld4q(a.rotation_raw, e);
+        float vm[3] = {0.f, 0.f, 0.f}, vq[4] = {0.f, 0.f, 0.f, 0.f}, vs[3] = {0.f, 0.f, 0.f};
+        if (any_geo) {
+            const Activated act = activate(o_raw, s_raw, q_raw);
+            epilogue_geometry_grads(r0, r1, r2, r3, a.viewmat, mean, act.quat, act.scales, vm, vq, vs);
+        }
+        // ---- VJPs of the activations ----
+        quat gq;
+        gq.w = vq[0], gq.x = vq[1], gq.y = vq[2], gq.z = vq[3];
+        const ActivationVjp av = activation_vjp(o_raw, s_raw, q_raw, r3.w, mk3(vs[0], vs[1], vs[2]), gq);
+        // ---- SH backward inputs (sh_colors_from_world_bwd) ----
+        const bool live = a.radii[e * 2] > 0 && a.radii[e * 2 + 1] > 0;
+        if (live) {
+            nb = sh_basis(a.sh_degree, sub(mean, campos_from_viewmat(a.viewmat)), B);
+            const float v_col[3] = {r0.x, r0.y, r0.z};
+#pragma unroll
+            for (int c = 0; c < 3; ++c)
+                vc[c] = a.colors[e * 3 + c] <= 0.0f ? 0.f : v_col[c]; // clamp VJP (Rasterization.cpp:609-610)
+        }
+        // ---- Adam on the small tensors ----
+        adam_row<3>(a.means, a.m_means, a.v_means, e, vm, a.lr_means, a);
+        const float gs[3] = {av.scaling.x, av.scaling.y, av.scaling.z};
+        adam_row<3>(a.scaling_raw, a.m_scaling, a.v_scaling, e, gs, a.lr_scaling, a);
+        const float gr[4] = {av.rotation.w, av.rotation.x, av.rotation.y, av.rotation.z};
+        adam_row<4>(a.rotation_raw, a.m_rotation, a.v_rotation, e, gr, a.lr_rotation, a);
+        const float go[1] = {av.opacity};
+        adam_row<1>(a.opacity_raw, a.m_opacity, a.v_opacity, e, go, a.lr_opacity, a);
+    }
+
+    // ---- Adam on the SH tensor; gradient of coefficient (k, c) = B[k] * vc[c] for k < nb, else 0 ----
+    if (LDS16) {
+        const uint32_t row0 = blockIdx.x * 256u + wave * 64u;
+        if (row0 >= a.N)
+            return; // whole wave out of range
+        float g[48];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            const bool used = k < nb;
+            g[k * 3 + 0] = used ? B[k] * vc[0] : 0.f;
+            g[k * 3 + 1] = used ? B[k] * vc[1] : 0.f;
+            g[k * 3 + 2] = used ? B[k] * vc[2] : 0.f;
+        }
+        const bool skip = a.skip_shN != 0;
+        float m1[48], v1[48];
+        // first moment
+        sh16_rows_to_lds(a.m_shs, row0, a.N, wave_lds, lane);
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (uint32_t j = 0; j < kShRowF4; ++j) {
+            float4 t = wave_lds[lane * kShLdsF4 + j];
+            float* tv = reinterpret_cast<float*>(&t);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int i = 4 * (int)j + q;
+                const float nm = adam_m(tv[q], g[i], a.beta1);
+                m1[i] = (i >= 3 && skip) ? tv[q] : nm;
+                tv[q] = m1[i];
+            }
+            wave_lds[lane * kShLdsF4 + j] = t;
+        }
+        __builtin_amdgcn_wave_barrier();
+        sh16_rows_from_lds(a.m_shs, row0, a.N, wave_lds, lane);
+        __builtin_amdgcn_wave_barrier();
+        // second moment
+        sh16_rows_to_lds(a.v_shs, row0, a.N, wave_lds, lane);
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (uint32_t j = 0; j < kShRowF4; ++j) {
+            float4 t = wave_lds[lane * kShLdsF4 + j];
+            float* tv = reinterpret_cast<float*>(&t);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int i = 4 * (int)j + q;
+                const float nv = adam_v(tv[q], g[i], a.beta2);
+                v1[i] = (i >= 3 && skip) ? tv[q] : nv;
+                tv[q] = v1[i];
+            }
+            wave_lds[lane * kShLdsF4 + j] = t;
+        }
+        __builtin_amdgcn_wave_barrier();
+        sh16_rows_from_lds(a.v_shs, row0, a.N, wave_lds, lane);
+        __builtin_amdgcn_wave_barrier();
+        // parameter
+        sh16_rows_to_lds(a.shs, row0, a.N, wave_lds, lane);
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (uint32_t j = 0; j < kShRowF4; ++j) {
+            float4 t = wave_lds[lane * kShLdsF4 + j];
+            float* tv = reinterpret_cast<float*>(&t);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int i = 4 * (int)j + q;
+                const float np = adam_p(tv[q], m1[i], v1[i], i < 3 ? a.lr_sh0 : a.lr_shN, a.eps, a.bc1_rcp,
+                                        a.bc2_sqrt_rcp);
+                tv[q] = (i >= 3 && skip) ? tv[q] : np;
+            }
+            wave_lds[lane * kShLdsF4 + j] = t;
+        }
+        __builtin_amdgcn_wave_barrier();
+        sh16_rows_from_lds(a.shs, row0, a.N, wave_lds, lane);
+        return;
+    }
+    if (!in)
+        return;
+    for (uint32_t k = 0; k < a.K; ++k) {
+        const bool used = (int)k < nb;
+        const float b = B[k < 25 ? k : 24];
+        if (k >= 1 && a.skip_shN)
+            break;
+#pragma unroll
+        for (uint32_t c = 0; c < 3; ++c) {
+            const size_t i = ((size_t)e * a.K + k) * 3 + c;
+            float p = a.shs[i], m = a.m_shs[i], v = a.v_shs[i];
+            adam_one(p, m, v, used ? b * vc[c] : 0.f, k == 0 ? a.lr_sh0 : a.lr_shN, a.beta1, a.beta2, a.eps,
+                     a.bc1_rcp, a.bc2_sqrt_rcp);
+            a.shs[i] = p;
+            a.m_shs[i] = m;
+            a.v_shs[i] = v;
+        }
+    }
+}
+
+} // namespace gsx
+
+using namespace gsx;
+
+extern "C" int gsx_backward_update_fused(const gsx_update_args* args, void* stream) {
+    GSX_REQUIRE(args != nullptr, GSX_ERR_INVALID_ARGUMENT, "backward_update_fused: args is null");
+    if (args->N == 0)
+        return GSX_OK;
+    GSX_REQUIRE(args->means && args->opacity_raw && args->scaling_raw && args->rotation_raw && args->shs &&
+                    args->m_means && args->m_opacity && args->m_scaling && args->m_rotation && args->m_shs &&
+                    args->v_means && args->v_opacity && args->v_scaling && args->v_rotation && args->v_shs &&
+                    args->radii && args->colors && args->viewmat && args->accumulators,
+                GSX_ERR_INVALID_ARGUMENT, "backward_update_fused: null tensor");
+    GSX_REQUIRE(args->K >= 1 && args->K <= 25, GSX_ERR_INVALID_ARGUMENT, "backward_update_fused: K = %u", args->K);
+    const uint32_t need = (args->sh_degree + 1) * (args->sh_degree + 1);
+    GSX_REQUIRE(args->sh_degree <= 4 && args->K >= need, GSX_ERR_INVALID_ARGUMENT,
+                "backward_update_fused: degree %u needs K >= %u (K = %u)", args->sh_degree, need, args->K);
+    GSX_REQUIRE((((uintptr_t)args->accumulators) & 15) == 0 && (((uintptr_t)args->rotation_raw) & 15) == 0,
+                GSX_ERR_INVALID_ARGUMENT, "backward_update_fused: accumulators / rotation need 16-byte alignment");
+    UpdateArgs a;
+    memset(&a, 0, sizeof(a));
+    a.N = args->N, a.K = args->K, a.sh_degree = args->sh_degree;
+    a.means = args->means, a.opacity_raw = args->opacity_raw, a.scaling_raw = args->scaling_raw;
+    a.rotation_raw = args->rotation_raw, a.shs = args->shs;
+    a.m_means = args->m_means, a.m_opacity = args->m_opacity, a.m_scaling = args->m_scaling;
+    a.m_rotation = args->m_rotation, a.m_shs = args->m_shs;
+    a.v_means = args->v_means, a.v_opacity = args->v_opacity, a.v_scaling = args->v_scaling;
+    a.v_rotation = args->v_rotation, a.v_shs = args->v_shs;
+    a.radii = args->radii, a.colors = args->colors, a.viewmat = args->viewmat, a.acc = (float*)args->accumulators;
+    a.lr_means = args->lr_means, a.lr_sh0 = args->lr_sh0, a.lr_shN = args->lr_shN, a.lr_scaling = args->lr_scaling;
+    a.lr_rotation = args->lr_rotation, a.lr_opacity = args->lr_opacity;
+    a.beta1 = args->beta1, a.beta2 = args->beta2, a.eps = args->eps;
+    a.bc1_rcp = args->bias_correction1_rcp, a.bc2_sqrt_rcp = args->bias_correction2_sqrt_rcp;
+    a.skip_shN = args->skip_shN;
+    const bool lds16 = a.K == 16 && ((((uintptr_t)a.shs) | ((uintptr_t)a.m_shs) | ((uintptr_t)a.v_shs)) & 15u) == 0;
+    const dim3 grid(cdiv(a.N, 256)), block(256);
+    if (lds16)
+        hipLaunchKernelGGL((backward_update_kernel<true>), grid, block, 0, (hipStream_t)stream, a);
+    else
+        hipLaunchKernelGGL((backward_update_kernel<false>), grid, block, 0, (hipStream_t)stream, a);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}

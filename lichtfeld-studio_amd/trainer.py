@@ -27,7 +27,7 @@ def _p(t):
 
 class TrainStep:
     def __init__(self, scene, device="cuda:0", lrs=None, lambda_dssim=0.2, betas=(0.9, 0.999), eps=1e-15,
-                 scene_scale=1.0, sh_degree=None, use_ssim=True):
+                 scene_scale=1.0, sh_degree=None, use_ssim=True, fused_update=False):
         self.dev = torch.device(device)
         self.lib = lib()
         f = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(self.dev)
@@ -49,6 +49,9 @@ class TrainStep:
         self.betas, self.eps = betas, eps
         self.lambda_dssim = lambda_dssim if use_ssim else 0.0
         self.use_ssim = use_ssim
+        # True: epilogue + SH backward + activation VJPs + Adam run as one pass and the raw-parameter gradients
+        # (self.grads) are never materialised; False: separate kernels (what the parity tests inspect)
+        self.fused_update = fused_update
         self.ut = UTParams()
         N = self.N
         e = lambda *s, dt=torch.float32: torch.empty(s, dtype=dt, device=self.dev)
@@ -223,6 +226,8 @@ class TrainStep:
                   c_u32(H), c_u32(16),
                   _p(self.viewmat), _p(self.Kmat), _p(self.offsets), _p(self.flatten_ids), _p(self.alpha),
                   _p(self.last_ids), _p(self.v_render), _p(self.v_alpha), ws, wsn, s)
+        if self.fused_update:
+            return
         self._run("rasterize_bwd_finish", lb.gsx_rasterize_bwd_finish, c_u32(N), _p(P["means"]), _p(A["quats"]),
                   _p(A["scales"]), _p(self.viewmat), ws, wsn, c_i(1), _p(G["means"]), _p(V["quats"]), _p(V["scales"]),
                   _p(self.v_colors), _p(V["opacities"]), s)
@@ -242,6 +247,19 @@ class TrainStep:
         b1, b2 = self.betas
         bc1 = 1.0 / (1.0 - math.pow(b1, t))
         bc2 = 1.0 / math.sqrt(1.0 - math.pow(b2, t))
+        if self.fused_update:
+            P, M, V = self.params, self.exp_avg, self.exp_avg_sq
+            skip = 1 if self.iteration <= 1000 and self.freeze_shN_early else 0
+            a = L.UpdateArgs(
+                self.N, self.K, self.sh_degree, P["means"].data_ptr(), P["opacity"].data_ptr(),
+                P["scaling"].data_ptr(), P["rotation"].data_ptr(), P["shs"].data_ptr(), M["means"].data_ptr(),
+                M["opacity"].data_ptr(), M["scaling"].data_ptr(), M["rotation"].data_ptr(), M["shs"].data_ptr(),
+                V["means"].data_ptr(), V["opacity"].data_ptr(), V["scaling"].data_ptr(), V["rotation"].data_ptr(),
+                V["shs"].data_ptr(), self.proj["radii"].data_ptr(), self.colors.data_ptr(), self.viewmat.data_ptr(),
+                self.ws_bwd.data_ptr(), self.lrs["means"], self.lrs["sh0"], self.lrs["shN"], self.lrs["scaling"],
+                self.lrs["rotation"], self.lrs["opacity"], b1, b2, self.eps, bc1, bc2, skip)
+            self._run("backward_update_fused", self.lib.gsx_backward_update_fused, ctypes.byref(a), self._stream())
+            return
         names = ["means", "shs", "scaling", "rotation", "opacity"]
         lr_of = dict(means=self.lrs["means"], shs=self.lrs["sh0"], scaling=self.lrs["scaling"],
                      rotation=self.lrs["rotation"], opacity=self.lrs["opacity"])
