@@ -61,6 +61,7 @@ def algorithmic_bytes(N, K, H, W, n_isects, sort_bits):
     return {
         "activate_params": N * (32 + 32),
         "projection_ut_3dgs_fused": N * (44 + 32),
+        "activate_project_ut": N * (44 + 32 + 32),
         "sh_colors_from_world": N * (12 + 12 * K + 8 + 12),
         "intersect_tile_emit": N * (4 + 16 + 4 + 8) + n_isects * 12,
         "intersect_tile_count_ordered": N * (28 + 16 + (8 + 24) * 4 + 8 + 8),
@@ -71,6 +72,7 @@ def algorithmic_bytes(N, K, H, W, n_isects, sort_bits):
         "fusedssim_backward": P * (72 + 12),
         "render_grad_from_loss": P * (12 + 12 + 12 + 12 + 12),
         "pack_raster_records": N * (56 + 96),
+        "sh_colors_records_from_world": N * (12 + 12 * K + 8 + 32 + 12 + 96),
         "rasterize_bwd_clear": N * 64,
         "rasterize_bwd_finish": N * (64 + 40 + 56),
         "sh_colors_from_world_bwd": N * (12 + 8 + 12 + 12 + 12 * K),

@@ -219,6 +219,13 @@ GSX_API int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
 GSX_API int gsx_sh_colors_from_world(uint32_t N, uint32_t K, uint32_t sh_degree, const float* means,
                                      const float* sh_coeffs, const int32_t* radii, const float* viewmat,
                                      float* colors, void* stream);
+/* gsx_sh_colors_from_world + gsx_pack_raster_records (channels = 3) in one pass, same results; records of
+ * Gaussians with radii == 0 are left untouched (no tile lists them) and their SH rows are not read. */
+GSX_API int gsx_sh_colors_records_from_world(uint32_t N, uint32_t K, uint32_t sh_degree, const float* means,
+                                             const float* quats, const float* scales, const float* opacities,
+                                             const float* sh_coeffs, const int32_t* radii, const float* viewmat,
+                                             const float* Kmat, uint32_t image_width, uint32_t image_height,
+                                             float* colors, void* records, void* stream);
 GSX_API int gsx_sh_colors_from_world_bwd(uint32_t N, uint32_t K, uint32_t sh_degree, const float* means,
                                          const int32_t* radii, const float* viewmat, const float* colors,
                                          const float* v_colors, float* v_sh_coeffs, void* stream);
@@ -291,6 +298,14 @@ GSX_API int gsx_quats_to_rotmats(int N, const float* quats, float* rotmats, void
 GSX_API int gsx_activate_params(uint32_t N, const float* opacity_raw, const float* scaling_raw,
                                 const float* rotation_raw, float* opacities, float* scales, float* quats,
                                 void* stream);
+/* gsx_activate_params + gsx_projection_ut_3dgs_fused (one pinhole camera, global shutter, opacities given, no
+ * compensations) in one pass with the same results; conics nullable. */
+GSX_API int gsx_activate_project_ut(uint32_t N, const float* means, const float* opacity_raw,
+                                    const float* scaling_raw, const float* rotation_raw, const float* viewmat,
+                                    const float* K, uint32_t image_width, uint32_t image_height, float eps2d,
+                                    float near_plane, float far_plane, float radius_clip, gsx_ut_params ut,
+                                    float* opacities, float* scales, float* quats, int32_t* radii, float* means2d,
+                                    float* depths, float* conics, void* stream);
 GSX_API int gsx_activate_params_bwd(uint32_t N, const float* opacity_raw, const float* scaling_raw,
                                     const float* rotation_raw, const float* v_opacities, const float* v_scales,
                                     const float* v_quats, float* v_opacity_raw, float* v_scaling_raw,

@@ -3,6 +3,8 @@
 //
 // All of these touch each Gaussian once and are bound by HBM bandwidth; one lane owns one Gaussian and
 // rows are read with whole-row vector loads.
+#include <string.h>
+
 #include "gsx_common.h"
 #include "gsx_step.h"
 
@@ -174,6 +176,45 @@ __global__ void __launch_bounds__(256) projection_ut_kernel(
     conics[idx * 3 + 2] = o.c2;
     if (compensations != nullptr)
         compensations[idx] = o.compensation;
+}
+
+// activate_params + projection in one pass (C == 1): raw parameters in, activated parameters and the projection
+// outputs out - the same values as the two separate kernels.
+__global__ void __launch_bounds__(256) projection_ut_raw_kernel(
+    uint32_t N, const float* __restrict__ means, const float* __restrict__ opacity_raw,
+    const float* __restrict__ scaling_raw, const float* __restrict__ rotation_raw,
+    const float* __restrict__ viewmat, const float* __restrict__ Ks, ProjCfg cfg, float* __restrict__ opacities,
+    float* __restrict__ scales, float* __restrict__ quats, int32_t* __restrict__ radii, float* __restrict__ means2d,
+    float* __restrict__ depths, float* __restrict__ conics) {
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= N)
+        return;
+    const Activated a = activate(opacity_raw[idx], ld3(scaling_raw, idx), ld4q(rotation_raw, idx));
+    opacities[idx] = a.opacity;
+    scales[3 * idx + 0] = a.scales.x;
+    scales[3 * idx + 1] = a.scales.y;
+    scales[3 * idx + 2] = a.scales.z;
+    reinterpret_cast<float4*>(quats)[idx] = make_float4(a.quat.w, a.quat.x, a.quat.y, a.quat.z);
+    cfg.fx = Ks[0];
+    cfg.fy = Ks[4];
+    cfg.cx = Ks[2];
+    cfg.cy = Ks[5];
+    const CamPose cp = load_cam_pose(viewmat);
+    ProjOut o;
+    const bool ok = project_ut(cfg, cp, ld3(means, idx), a.quat, a.scales, true, a.opacity, &o);
+    int2* r2 = reinterpret_cast<int2*>(radii);
+    if (!ok) {
+        r2[idx] = make_int2(0, 0);
+        return;
+    }
+    r2[idx] = make_int2((int32_t)o.rx, (int32_t)o.ry);
+    reinterpret_cast<float2*>(means2d)[idx] = make_float2(o.mx, o.my);
+    depths[idx] = o.depth;
+    if (conics != nullptr) {
+        conics[idx * 3 + 0] = o.c0;
+        conics[idx * 3 + 1] = o.c1;
+        conics[idx * 3 + 2] = o.c2;
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -465,6 +506,81 @@ __global__ void __launch_bounds__(256) sh_bwd_generic_kernel(uint32_t N, uint32_
     }
 }
 
+// Colours AND raster records in one pass (what gsx_sh_colors_from_world followed by gsx_pack_raster_records
+// produce, same arithmetic): the colour goes straight from the SH evaluation into the record, and the coefficient
+// rows of Gaussians that touch no tile are not read at all.
+template <bool LDS16>
+__global__ void __launch_bounds__(256) sh_records_kernel(uint32_t N, uint32_t K, uint32_t degree,
+                                                          const float* __restrict__ means,
+                                                          const float* __restrict__ quats,
+                                                          const float* __restrict__ scales,
+                                                          const float* __restrict__ opacities,
+                                                          const float* __restrict__ coeffs,
+                                                          const int32_t* __restrict__ radii,
+                                                          const float* __restrict__ viewmat,
+                                                          const float* __restrict__ Kmat, uint32_t W, uint32_t H,
+                                                          float* __restrict__ colors, float4* __restrict__ records) {
+    __shared__ float4 lds[LDS16 ? 4 * 64 * kShLdsF4 : 1];
+    const uint32_t e = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    float4* wave_lds = lds + (LDS16 ? wave * 64 * kShLdsF4 : 0);
+    const bool live = e < N && radii[e * 2] > 0 && radii[e * 2 + 1] > 0;
+    if (LDS16) {
+        const uint32_t row0 = blockIdx.x * 256u + wave * 64u;
+        const uint64_t live_rows = __builtin_amdgcn_ballot_w64(live);
+        if (row0 < N && live_rows) {
+            const float4* src = reinterpret_cast<const float4*>(coeffs + (size_t)row0 * 48);
+            const uint32_t n_f4 = min(64u, N - row0) * kShRowF4;
+#pragma unroll
+            for (uint32_t i = 0; i < kShRowF4; ++i) {
+                const uint32_t q = i * 64u + lane;
+                const uint32_t r = (q * 43691u) >> 19; // q / 12 for q < 768
+                if (q < n_f4 && ((live_rows >> r) & 1ull))
+                    wave_lds[r * kShLdsF4 + (q - r * kShRowF4)] = src[q];
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    if (e >= N)
+        return;
+    float c[3] = {0.f, 0.f, 0.f};
+    const vec3 mean = ld3(means, e);
+    if (live) {
+        const vec3 dir = sub(mean, campos_from_viewmat(viewmat));
+        float B[25];
+        sh_basis(degree, dir, B);
+        float co_reg[48];
+        const float* co;
+        if (LDS16) {
+#pragma unroll
+            for (uint32_t j = 0; j < kShRowF4; ++j) {
+                const float4 t = wave_lds[lane * kShLdsF4 + j];
+                co_reg[4 * j + 0] = t.x;
+                co_reg[4 * j + 1] = t.y;
+                co_reg[4 * j + 2] = t.z;
+                co_reg[4 * j + 3] = t.w;
+            }
+            co = co_reg;
+        } else {
+            co = coeffs + (size_t)e * K * 3;
+        }
+#pragma unroll
+        for (uint32_t ch = 0; ch < 3; ++ch)
+            c[ch] = gsx::fmax(sh_color_channel(degree, dir, B, co, ch) + 0.5f, 0.0f);
+    }
+    colors[e * 3 + 0] = c[0];
+    colors[e * 3 + 1] = c[1];
+    colors[e * 3 + 2] = c[2];
+    if (!live)
+        return; // no tile lists this Gaussian: its record is never read
+    const vec3 ray_o = camera_ray_origin(load_cam_pose(viewmat));
+    const float opac = opacities[e];
+    const mat3 M = record_whitening(ld4q(quats, e), ld3(scales, e));
+    const vec3 gro = mul(M, sub(ray_o, mean));
+    const RecordRegion reg = record_region(gro, M, opac, mean, viewmat, Kmat[0], Kmat[4], Kmat[2], Kmat[5], W, H);
+    store_record(records + (size_t)e * kRecordF4, gro, opac, M, c[0], c[1], c[2], reg);
+}
+
 template <bool WORLD>
 static void launch_sh_fwd(uint32_t N, uint32_t K, uint32_t degree, const float* dirs_or_means, const float* coeffs,
                           const uint8_t* masks, const int32_t* radii, const float* viewmat, float* colors,
@@ -534,6 +650,33 @@ extern "C" int gsx_projection_ut_3dgs_fused(
     return GSX_OK;
 }
 
+extern "C" int gsx_activate_project_ut(uint32_t N, const float* means, const float* opacity_raw,
+                                       const float* scaling_raw, const float* rotation_raw, const float* viewmat,
+                                       const float* K, uint32_t image_width, uint32_t image_height, float eps2d,
+                                       float near_plane, float far_plane, float radius_clip, gsx_ut_params ut,
+                                       float* opacities, float* scales, float* quats, int32_t* radii, float* means2d,
+                                       float* depths, float* conics, void* stream) {
+    if (N == 0)
+        return GSX_OK;
+    GSX_REQUIRE(means && opacity_raw && scaling_raw && rotation_raw && viewmat && K && opacities && scales && quats &&
+                    radii && means2d && depths,
+                GSX_ERR_INVALID_ARGUMENT, "activate_project_ut: null tensor");
+    GSX_REQUIRE((((uintptr_t)rotation_raw) & 15) == 0 && (((uintptr_t)quats) & 15) == 0, GSX_ERR_INVALID_ARGUMENT,
+                "activate_project_ut: quaternion tensors need 16-byte alignment");
+    ProjCfg cfg;
+    memset(&cfg, 0, sizeof(cfg));
+    cfg.W = image_width, cfg.H = image_height;
+    cfg.eps2d = eps2d, cfg.near_plane = near_plane, cfg.far_plane = far_plane, cfg.radius_clip = radius_clip;
+    cfg.ut_alpha = ut.alpha, cfg.ut_beta = ut.beta, cfg.ut_kappa = ut.kappa;
+    cfg.ut_margin = ut.in_image_margin_factor;
+    cfg.ut_require_all = ut.require_all_sigma_points_valid;
+    hipLaunchKernelGGL(projection_ut_raw_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, means,
+                       opacity_raw, scaling_raw, rotation_raw, viewmat, K, cfg, opacities, scales, quats, radii,
+                       means2d, depths, conics);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
 extern "C" int gsx_spherical_harmonics_fwd(uint32_t N, uint32_t K, uint32_t degrees_to_use, const float* dirs,
                                            const float* coeffs, const uint8_t* masks, float* colors, void* stream) {
     if (N == 0)
@@ -581,6 +724,34 @@ extern "C" int gsx_sh_colors_from_world(uint32_t N, uint32_t K, uint32_t sh_degr
                 "sh_colors_from_world: degree %u needs K >= %u (got %u)", sh_degree, (sh_degree + 1) * (sh_degree + 1),
                 K);
     launch_sh_fwd<true>(N, K, sh_degree, means, sh_coeffs, nullptr, radii, viewmat, colors, (hipStream_t)stream);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+extern "C" int gsx_sh_colors_records_from_world(uint32_t N, uint32_t K, uint32_t sh_degree, const float* means,
+                                                const float* quats, const float* scales, const float* opacities,
+                                                const float* sh_coeffs, const int32_t* radii, const float* viewmat,
+                                                const float* Kmat, uint32_t image_width, uint32_t image_height,
+                                                float* colors, void* records, void* stream) {
+    if (N == 0)
+        return GSX_OK;
+    GSX_REQUIRE(means && quats && scales && opacities && sh_coeffs && radii && viewmat && Kmat && colors && records,
+                GSX_ERR_INVALID_ARGUMENT, "sh_colors_records_from_world: null tensor");
+    GSX_REQUIRE(sh_degree <= 4 && K >= (sh_degree + 1) * (sh_degree + 1), GSX_ERR_INVALID_ARGUMENT,
+                "sh_colors_records_from_world: degree %u needs K >= %u (got %u)", sh_degree,
+                (sh_degree + 1) * (sh_degree + 1), K);
+    GSX_REQUIRE(((uintptr_t)records & 15) == 0 && ((uintptr_t)quats & 15) == 0, GSX_ERR_INVALID_ARGUMENT,
+                "sh_colors_records_from_world: records / quats need 16-byte alignment");
+    const bool lds16 = K == 16 && (((uintptr_t)sh_coeffs) & 15u) == 0;
+    const dim3 grid(cdiv(N, 256)), block(256);
+    if (lds16)
+        hipLaunchKernelGGL((sh_records_kernel<true>), grid, block, 0, (hipStream_t)stream, N, K, sh_degree, means,
+                           quats, scales, opacities, sh_coeffs, radii, viewmat, Kmat, image_width, image_height, colors,
+                           (float4*)records);
+    else
+        hipLaunchKernelGGL((sh_records_kernel<false>), grid, block, 0, (hipStream_t)stream, N, K, sh_degree, means,
+                           quats, scales, opacities, sh_coeffs, radii, viewmat, Kmat, image_width, image_height, colors,
+                           (float4*)records);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

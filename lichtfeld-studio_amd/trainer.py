@@ -145,13 +145,10 @@ class TrainStep:
         self._ensure_image(H, W)
         self.viewmat, self.Kmat, self.W, self.H = viewmat, K, W, H
         P, A, J = self.params, self.act, self.proj
-        self._run("activate_params", lb.gsx_activate_params, c_u32(N), _p(P["opacity"]), _p(P["scaling"]), _p(P["rotation"]),
-                                     _p(A["opacities"]), _p(A["scales"]), _p(A["quats"]), s)
-        self._run("projection_ut_3dgs_fused", lb.gsx_projection_ut_3dgs_fused, 
-            c_u32(1), c_u32(N), _p(P["means"]), _p(A["quats"]), _p(A["scales"]), _p(A["opacities"]), _p(viewmat),
-            c_p(None), _p(K), c_u32(W), c_u32(H), c_f(0.3), c_f(0.01), c_f(1e4), c_f(0.0), c_i(0), self.ut, c_i(4),
-            c_p(None), c_p(None), c_p(None), _p(J["radii"]), _p(J["means2d"]), _p(J["depths"]), _p(J["conics"]),
-            c_p(None), s)
+        self._run("activate_project_ut", lb.gsx_activate_project_ut, c_u32(N), _p(P["means"]), _p(P["opacity"]),
+                  _p(P["scaling"]), _p(P["rotation"]), _p(viewmat), _p(K), c_u32(W), c_u32(H), c_f(0.3), c_f(0.01),
+                  c_f(1e4), c_f(0.0), self.ut, _p(A["opacities"]), _p(A["scales"]), _p(A["quats"]), _p(J["radii"]),
+                  _p(J["means2d"]), _p(J["depths"]), _p(J["conics"]), s)
         # Tile counts in depth order; the total comes back through pinned memory without blocking, and the SH /
         # record passes (which do not need it) run while the host waits for it.
         self._run("intersect_tile_count_ordered", lb.gsx_intersect_tile_count_ordered, c_u32(N), _p(J["means2d"]),
@@ -159,12 +156,10 @@ class TrainStep:
                   _p(self.tiles_per_gauss), _p(self.cum), _p(self.ws_count), c_sz(self.ws_count.numel()),
                   c_p(self.n_isects_pinned.data_ptr()), c_i(0), s)
         self.count_done.record(torch.cuda.current_stream(self.dev))
-        self._run("sh_colors_from_world", lb.gsx_sh_colors_from_world, c_u32(N), c_u32(self.K),
-                  c_u32(self.sh_degree), _p(P["means"]), _p(P["shs"]), _p(J["radii"]), _p(viewmat), _p(self.colors),
-                  s)
-        self._run("pack_raster_records", lb.gsx_pack_raster_records, c_u32(N), _p(P["means"]), _p(A["quats"]),
-                  _p(A["scales"]), _p(A["opacities"]), _p(self.colors), c_u32(3), _p(viewmat), _p(K), c_u32(W),
-                  c_u32(H), _p(self.records), s)
+        self._run("sh_colors_records_from_world", lb.gsx_sh_colors_records_from_world, c_u32(N), c_u32(self.K),
+                  c_u32(self.sh_degree), _p(P["means"]), _p(A["quats"]), _p(A["scales"]), _p(A["opacities"]),
+                  _p(P["shs"]), _p(J["radii"]), _p(viewmat), _p(K), c_u32(W), c_u32(H), _p(self.colors),
+                  _p(self.records), s)
         self.count_done.synchronize()
         n = self.n_isects = int(self.n_isects_pinned[0])
         if n >= 1 << 31:
