@@ -69,6 +69,8 @@ def algorithmic_bytes(N, K, H, W, n_isects, sort_bits):
         "intersect_offset": n_isects * 8 + (P // 256) * 4,
         "image_from_render": P * (12 + 12 + 12),
         "fusedssim": P * (24 + 12 + 36),
+        "photometric_loss_forward": P * (12 + 12 + 36),
+        "photometric_loss_backward": P * (12 + 12 + 36 + 12),
         "fusedssim_backward": P * (72 + 12),
         "render_grad_from_loss": P * (12 + 12 + 12 + 12 + 12),
         "pack_raster_records": N * (56 + 96),
@@ -122,7 +124,8 @@ def main():
     else:
         gt = torch.from_numpy(sc.target[None].copy()).to(dev)
     use_ssim = args.config != 1  # configuration 1 is L1 only
-    ts = TrainStep(sc, dev, use_ssim=use_ssim, fused_update=not args.separate_update)
+    ts = TrainStep(sc, dev, use_ssim=use_ssim, fused_update=not args.separate_update,
+                   fused_loss=not args.separate_update)
     setup_s = time.time() - t0
 
     dominant = "rasterize_bwd_accumulate"

@@ -345,6 +345,18 @@ GSX_API int gsx_ssim_valid_partials(uint32_t CH, uint32_t H, uint32_t W, const f
 GSX_API int gsx_photometric_loss_finish(uint32_t CH, uint32_t H, uint32_t W, float lambda_dssim,
                                         const float* l1_partials, const float* ssim_partials, uint32_t n_partials,
                                         float* loss_out, void* stream);
+/* The same loss in two kernels for a training loop: forward = clamp + permute on load, SSIM derivative maps and
+ * the per-block partial sums (l1_partials / ssim_partials hold gsx_photometric_partials(H, W) floats each; the
+ * clamped image and the SSIM map are not written), then gsx_photometric_loss_finish; backward = v_render [H,W,3]
+ * from the derivative maps, with d loss / d map of the valid crop formed on the fly.  Per-pixel arithmetic is that
+ * of the separate kernels; the loss value differs from theirs by summation order only. */
+GSX_API uint32_t gsx_photometric_partials(uint32_t H, uint32_t W);
+GSX_API int gsx_photometric_loss_forward(uint32_t H, uint32_t W, float C1, float C2, const float* render_hwc,
+                                         const float* gt_chw, float* dm_dmu1, float* dm_dsigma1_sq,
+                                         float* dm_dsigma12, float* l1_partials, float* ssim_partials, void* stream);
+GSX_API int gsx_photometric_loss_backward(uint32_t H, uint32_t W, float lambda_dssim, const float* render_hwc,
+                                          const float* gt_chw, const float* dm_dmu1, const float* dm_dsigma1_sq,
+                                          const float* dm_dsigma12, float* v_render_hwc, void* stream);
 /* v_render [H,W,3] = d loss / d render: L1 sign term + lambda * SSIM term (dL_dimg_ssim is
  * gsx_fusedssim_backward's output for dL_dmap = -lambda / count on the valid crop, 0 elsewhere), passed through
  * the clamp VJP (zero where render < 0 or > 1) and the CHW -> HWC permute. */

@@ -84,6 +84,7 @@ def lib():
         L.gsx_status_string.restype = ctypes.c_char_p
         L.gsx_n_bits.restype = c_u32
         L.gsx_image_loss_blocks.restype = c_u32
+        L.gsx_photometric_partials.restype = c_u32
         L.gsx_ut_defaults.restype = UTParams
         for name in ("gsx_intersect_tile_count_workspace_bytes", "gsx_radix_sort_pairs_workspace_bytes",
                      "gsx_rasterize_bwd_workspace_bytes", "gsx_mcmc_relocate_workspace_bytes",

@@ -251,10 +251,20 @@ __global__ void __launch_bounds__(256) photometric_loss_finish_kernel(uint32_t C
                                                                        float* __restrict__ loss_out) {
     __shared__ float lds[4];
     float a = 0.f, b = 0.f;
-    for (uint32_t i = threadIdx.x; i < n_partials; i += 256) {
-        a += l1_partials[i];
-        b += ssim_partials[i];
+    // four independent loads in flight per lane: the kernel is one block and pure latency
+    float a4[4] = {0.f, 0.f, 0.f, 0.f}, b4[4] = {0.f, 0.f, 0.f, 0.f};
+    for (uint32_t i = threadIdx.x; i < n_partials; i += 1024) {
+#pragma unroll
+        for (uint32_t k = 0; k < 4; ++k) {
+            const uint32_t j = i + k * 256u;
+            if (j < n_partials) {
+                a4[k] += l1_partials[j];
+                b4[k] += ssim_partials[j];
+            }
+        }
     }
+    a = (a4[0] + a4[1]) + (a4[2] + a4[3]);
+    b = (b4[0] + b4[1]) + (b4[2] + b4[3]);
     const float l1_sum = block_sum_256(a, lds);
     const float ss_sum = block_sum_256(b, lds);
     if (threadIdx.x == 0) {
@@ -303,6 +313,198 @@ __global__ void __launch_bounds__(256) render_grad_from_loss_kernel(uint32_t HW,
             g += dL_dimg_ssim[(size_t)c * HW + p];
         // clamp VJP: gradient passes where 0 <= render <= 1
         v_render_hwc[(size_t)p * 3 + c] = (r >= 0.f && r <= 1.f) ? g : 0.f;
+    }
+}
+
+// ---- the photometric loss of a training step in two kernels ---------------------------------------
+// forward: clamp + HWC -> CHW on load, SSIM moments and derivative maps, per-block partial sums of |image - gt| and
+// of the SSIM map over the valid crop (what image_from_render + fusedssim + ssim_valid_partials do in three passes;
+// the clamped image and the SSIM map themselves are never written).
+__global__ void __launch_bounds__(256) photometric_fwd_kernel(int H, int W, float C1, float C2,
+                                                               const float* __restrict__ render_hwc,
+                                                               const float* __restrict__ gt_chw,
+                                                               float* __restrict__ dm_dmu1,
+                                                               float* __restrict__ dm_dsigma1_sq,
+                                                               float* __restrict__ dm_dsigma12,
+                                                               float* __restrict__ l1_partials,
+                                                               float* __restrict__ ssim_partials) {
+    __shared__ float sTile[SY][SX][2];
+    __shared__ float xconv[CY][BX][5];
+    __shared__ float red[4];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int pix_x = blockIdx.x * BX + tx, pix_y = blockIdx.y * BY + ty;
+    const int c = blockIdx.z;
+    const size_t plane = (size_t)c * H * W;
+
+    for (int tid = threadIdx.x; tid < SY * SX; tid += 256) {
+        const int ly = tid / SX, lx = tid % SX;
+        const int gy = blockIdx.y * BY + ly - HALO, gx = blockIdx.x * BX + lx - HALO;
+        float a = 0.f, b = 0.f;
+        if (gx >= 0 && gx < W && gy >= 0 && gy < H) {
+            a = gsx::fmin(gsx::fmax(render_hwc[((size_t)gy * W + gx) * 3 + c], 0.0f), 1.0f); // rasterizer.cpp:205
+            b = gt_chw[plane + (size_t)gy * W + gx];
+        }
+        sTile[ly][lx][0] = a;
+        sTile[ly][lx][1] = b;
+    }
+    __syncthreads();
+    for (int ly = ty; ly < CY; ly += BY) {
+        const int lx = tx + HALO;
+        float sumX = 0.f, sumX2 = 0.f, sumY = 0.f, sumY2 = 0.f, sumXY = 0.f;
+#pragma unroll
+        for (int d = 1; d <= HALO; ++d) {
+            const float w = cGauss[HALO - d];
+            const float Xl = sTile[ly][lx - d][0], Yl = sTile[ly][lx - d][1];
+            const float Xr = sTile[ly][lx + d][0], Yr = sTile[ly][lx + d][1];
+            sumX += (Xl + Xr) * w;
+            sumX2 += ((Xl * Xl) + (Xr * Xr)) * w;
+            sumY += (Yl + Yr) * w;
+            sumY2 += ((Yl * Yl) + (Yr * Yr)) * w;
+            sumXY += ((Xl * Yl) + (Xr * Yr)) * w;
+        }
+        const float cX = sTile[ly][lx][0], cY = sTile[ly][lx][1];
+        const float wc = cGauss[HALO];
+        sumX += cX * wc;
+        sumX2 += (cX * cX) * wc;
+        sumY += cY * wc;
+        sumY2 += (cY * cY) * wc;
+        sumXY += (cX * cY) * wc;
+        xconv[ly][tx][0] = sumX;
+        xconv[ly][tx][1] = sumX2;
+        xconv[ly][tx][2] = sumY;
+        xconv[ly][tx][3] = sumY2;
+        xconv[ly][tx][4] = sumXY;
+    }
+    __syncthreads();
+    float l1 = 0.f, ss = 0.f;
+    {
+        const int ly = ty + HALO, lx = tx;
+        float out[5] = {0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int d = 1; d <= HALO; ++d) {
+            const float w = cGauss[HALO - d];
+#pragma unroll
+            for (int k = 0; k < 5; ++k)
+                out[k] += (xconv[ly - d][lx][k] + xconv[ly + d][lx][k]) * w;
+        }
+#pragma unroll
+        for (int k = 0; k < 5; ++k)
+            out[k] += xconv[ly][lx][k] * cGauss[HALO];
+        if (pix_x < W && pix_y < H) {
+            const float mu1 = out[0], mu2 = out[2];
+            const float mu1_sq = mu1 * mu1, mu2_sq = mu2 * mu2;
+            const float sigma1_sq = out[1] - mu1_sq, sigma2_sq = out[3] - mu2_sq;
+            const float sigma12 = out[4] - mu1 * mu2;
+            const float A = mu1_sq + mu2_sq + C1;
+            const float B = sigma1_sq + sigma2_sq + C2;
+            const float C_ = 2.f * mu1 * mu2 + C1;
+            const float D_ = 2.f * sigma12 + C2;
+            const size_t gi = plane + (size_t)pix_y * W + pix_x;
+            const bool crop = H > 10 && W > 10;
+            if (!crop || (pix_y >= 5 && pix_y < H - 5 && pix_x >= 5 && pix_x < W - 5))
+                ss = (C_ * D_) / (A * B);
+            dm_dmu1[gi] = ((mu2 * 2.f * D_) / (A * B) - (mu2 * 2.f * C_) / (A * B) -
+                           (mu1 * 2.f * C_ * D_) / (A * A * B) + (mu1 * 2.f * C_ * D_) / (A * B * B));
+            dm_dsigma1_sq[gi] = (-C_ * D_) / (A * B * B);
+            dm_dsigma12[gi] = (2.f * C_) / (A * B);
+            l1 = gsx::fabs(sTile[ty + HALO][tx + HALO][0] - sTile[ty + HALO][tx + HALO][1]);
+        }
+    }
+    const uint32_t bid = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+    const float l1s = block_sum_256(l1, red);
+    const float sss = block_sum_256(ss, red);
+    if (threadIdx.x == 0) {
+        l1_partials[bid] = l1s;
+        ssim_partials[bid] = sss;
+    }
+}
+
+// backward: d loss / d render in one pass - the SSIM chain with d loss / d map = -lambda / count inside the valid crop
+// formed on the fly (fused_ssim.cuh:84-96), the L1 sign term, the clamp VJP and the CHW -> HWC permute (what
+// fusedssim_backward + render_grad_from_loss do in two passes with two intermediate images).  A block walks the
+// three colour planes of its tile and writes the pixel's three gradients together.
+__global__ void __launch_bounds__(256) photometric_bwd_kernel(int H, int W, float ssim_scale, float l1_scale,
+                                                               const float* __restrict__ render_hwc,
+                                                               const float* __restrict__ gt_chw,
+                                                               const float* __restrict__ dm_dmu1,
+                                                               const float* __restrict__ dm_dsigma1_sq,
+                                                               const float* __restrict__ dm_dsigma12,
+                                                               float* __restrict__ v_render_hwc) {
+    __shared__ float sData[3][SY][SX];
+    __shared__ float sScratch[CY][BX][3];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int pix_x = blockIdx.x * BX + tx, pix_y = blockIdx.y * BY + ty;
+    const bool inside = pix_x < W && pix_y < H;
+    const bool crop = H > 10 && W > 10;
+    float g[3] = {0.f, 0.f, 0.f};
+    for (int c = 0; c < 3; ++c) {
+        const size_t plane = (size_t)c * H * W;
+        for (int tid = threadIdx.x; tid < SY * SX; tid += 256) {
+            const int row = tid / SX, col = tid % SX;
+            const int gy = blockIdx.y * BY + row - HALO, gx = blockIdx.x * BX + col - HALO;
+            float d0 = 0.f, d1 = 0.f, d2 = 0.f;
+            if (gx >= 0 && gx < W && gy >= 0 && gy < H) {
+                const bool valid = !crop || (gy >= 5 && gy < H - 5 && gx >= 5 && gx < W - 5);
+                const float chain = valid ? ssim_scale : 0.f;
+                const size_t gi = plane + (size_t)gy * W + gx;
+                d0 = dm_dmu1[gi] * chain;
+                d1 = dm_dsigma1_sq[gi] * chain;
+                d2 = dm_dsigma12[gi] * chain;
+            }
+            sData[0][row][col] = d0;
+            sData[1][row][col] = d1;
+            sData[2][row][col] = d2;
+        }
+        __syncthreads();
+        for (int yy = ty; yy < CY; yy += BY) {
+            const int lx = tx + HALO;
+            float a0 = 0.f, a1 = 0.f, a2 = 0.f;
+#pragma unroll
+            for (int d = 1; d <= HALO; ++d) {
+                const float w = cGauss[HALO - d];
+                a0 += (sData[0][yy][lx - d] + sData[0][yy][lx + d]) * w;
+                a1 += (sData[1][yy][lx - d] + sData[1][yy][lx + d]) * w;
+                a2 += (sData[2][yy][lx - d] + sData[2][yy][lx + d]) * w;
+            }
+            const float wc = cGauss[HALO];
+            a0 += sData[0][yy][lx] * wc;
+            a1 += sData[1][yy][lx] * wc;
+            a2 += sData[2][yy][lx] * wc;
+            sScratch[yy][tx][0] = a0;
+            sScratch[yy][tx][1] = a1;
+            sScratch[yy][tx][2] = a2;
+        }
+        __syncthreads();
+        if (inside) {
+            const int ly = ty + HALO, lx = tx;
+            float s0 = 0.f, s1 = 0.f, s2 = 0.f;
+#pragma unroll
+            for (int d = 1; d <= HALO; ++d) {
+                const float w = cGauss[HALO - d];
+                s0 += (sScratch[ly - d][lx][0] + sScratch[ly + d][lx][0]) * w;
+                s1 += (sScratch[ly - d][lx][1] + sScratch[ly + d][lx][1]) * w;
+                s2 += (sScratch[ly - d][lx][2] + sScratch[ly + d][lx][2]) * w;
+            }
+            const float wc = cGauss[HALO];
+            s0 += sScratch[ly][lx][0] * wc;
+            s1 += sScratch[ly][lx][1] * wc;
+            s2 += sScratch[ly][lx][2] * wc;
+            const size_t p = (size_t)pix_y * W + pix_x;
+            const float r = render_hwc[p * 3 + c];
+            const float p1 = gsx::fmin(gsx::fmax(r, 0.0f), 1.0f), p2 = gt_chw[plane + p];
+            const float dssim = s0 + (2.f * p1) * s1 + (p2)*s2;
+            const float d = p1 - p2;
+            const float sgn = d > 0.f ? 1.f : (d < 0.f ? -1.f : 0.f);
+            const float gg = l1_scale * sgn + dssim;
+            g[c] = (r >= 0.f && r <= 1.f) ? gg : 0.f; // clamp VJP
+        }
+        __syncthreads(); // sData / sScratch are rewritten for the next plane
+    }
+    if (inside) {
+        const size_t p = (size_t)pix_y * W + pix_x;
+        v_render_hwc[p * 3 + 0] = g[0];
+        v_render_hwc[p * 3 + 1] = g[1];
+        v_render_hwc[p * 3 + 2] = g[2];
     }
 }
 
@@ -405,6 +607,44 @@ extern "C" int gsx_render_grad_from_loss(uint32_t H, uint32_t W, float lambda_ds
     hipLaunchKernelGGL(render_grad_from_loss_kernel, dim3(cdiv((uint64_t)H * W, 256)), dim3(256), 0,
                        (hipStream_t)stream, H * W, l1_scale, render_hwc, image_chw, gt_chw, dL_dimg_ssim,
                        v_render_hwc);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+extern "C" uint32_t gsx_photometric_partials(uint32_t H, uint32_t W) {
+    return 3u * cdiv(W, (uint32_t)BX) * cdiv(H, (uint32_t)BY);
+}
+
+extern "C" int gsx_photometric_loss_forward(uint32_t H, uint32_t W, float C1, float C2, const float* render_hwc,
+                                            const float* gt_chw, float* dm_dmu1, float* dm_dsigma1_sq,
+                                            float* dm_dsigma12, float* l1_partials, float* ssim_partials,
+                                            void* stream) {
+    if ((uint64_t)H * W == 0)
+        return GSX_OK;
+    GSX_REQUIRE(render_hwc && gt_chw && dm_dmu1 && dm_dsigma1_sq && dm_dsigma12 && l1_partials && ssim_partials,
+                GSX_ERR_INVALID_ARGUMENT, "photometric_loss_forward: null tensor");
+    GSX_REQUIRE((uint64_t)H * W < (1ull << 30), GSX_ERR_INVALID_ARGUMENT, "photometric_loss_forward: image too large");
+    const dim3 grid(cdiv(W, (uint32_t)BX), cdiv(H, (uint32_t)BY), 3);
+    hipLaunchKernelGGL(photometric_fwd_kernel, grid, dim3(256), 0, (hipStream_t)stream, (int)H, (int)W, C1, C2,
+                       render_hwc, gt_chw, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, l1_partials, ssim_partials);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+extern "C" int gsx_photometric_loss_backward(uint32_t H, uint32_t W, float lambda_dssim, const float* render_hwc,
+                                             const float* gt_chw, const float* dm_dmu1, const float* dm_dsigma1_sq,
+                                             const float* dm_dsigma12, float* v_render_hwc, void* stream) {
+    if ((uint64_t)H * W == 0)
+        return GSX_OK;
+    GSX_REQUIRE(render_hwc && gt_chw && dm_dmu1 && dm_dsigma1_sq && dm_dsigma12 && v_render_hwc,
+                GSX_ERR_INVALID_ARGUMENT, "photometric_loss_backward: null tensor");
+    const bool crop = H > 10 && W > 10;
+    const float count = crop ? 3.f * (float)(H - 10) * (float)(W - 10) : 3.f * (float)H * (float)W;
+    const float ssim_scale = -lambda_dssim / count;
+    const float l1_scale = (1.f - lambda_dssim) / (3.f * (float)H * (float)W);
+    const dim3 grid(cdiv(W, (uint32_t)BX), cdiv(H, (uint32_t)BY));
+    hipLaunchKernelGGL(photometric_bwd_kernel, grid, dim3(256), 0, (hipStream_t)stream, (int)H, (int)W, ssim_scale,
+                       l1_scale, render_hwc, gt_chw, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, v_render_hwc);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

@@ -27,7 +27,7 @@ def _p(t):
 
 class TrainStep:
     def __init__(self, scene, device="cuda:0", lrs=None, lambda_dssim=0.2, betas=(0.9, 0.999), eps=1e-15,
-                 scene_scale=1.0, sh_degree=None, use_ssim=True, fused_update=False):
+                 scene_scale=1.0, sh_degree=None, use_ssim=True, fused_update=False, fused_loss=False):
         self.dev = torch.device(device)
         self.lib = lib()
         f = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(self.dev)
@@ -52,6 +52,8 @@ class TrainStep:
         # True: epilogue + SH backward + activation VJPs + Adam run as one pass and the raw-parameter gradients
         # (self.grads) are never materialised; False: separate kernels (what the parity tests inspect)
         self.fused_update = fused_update
+        # True (needs use_ssim): the loss runs as two kernels and neither the clamped image nor the SSIM map exist
+        self.fused_loss = fused_loss and use_ssim
         self.ut = UTParams()
         N = self.N
         e = lambda *s, dt=torch.float32: torch.empty(s, dtype=dt, device=self.dev)
@@ -98,8 +100,9 @@ class TrainStep:
         self.image = e(1, 3, H, W)
         self.v_render = e(1, H, W, 3)
         self.v_alpha = torch.zeros((1, H, W, 1), dtype=torch.float32, device=self.dev)
-        nb = self.lib.gsx_image_loss_blocks(c_u32(H), c_u32(W))
-        self.n_partials = nb
+        nb = max(self.lib.gsx_image_loss_blocks(c_u32(H), c_u32(W)), self.lib.gsx_photometric_partials(c_u32(H), c_u32(W)))
+        self.n_partials = self.lib.gsx_image_loss_blocks(c_u32(H), c_u32(W))
+        self.n_partials_fused = self.lib.gsx_photometric_partials(c_u32(H), c_u32(W))
         self.l1_partials, self.ssim_partials = e(nb), e(nb)
         self.ssim_map, self.dm1, self.dm2, self.dm3 = e(1, 3, H, W), e(1, 3, H, W), e(1, 3, H, W), e(1, 3, H, W)
         self.dL_dmap, self.dL_dimg = e(1, 3, H, W), e(1, 3, H, W)
@@ -189,6 +192,14 @@ class TrainStep:
         """image = clamp(render, 0, 1) CHW; loss = (1-l) L1 + l (1 - SSIM_valid); result stays on the device."""
         lb, s, H, W = self.lib, self._stream(), self.H, self.W
         self.gt = gt_chw
+        if self.fused_loss:
+            self._run("photometric_loss_forward", lb.gsx_photometric_loss_forward, c_u32(H), c_u32(W),
+                      c_f(0.01 ** 2), c_f(0.03 ** 2), _p(self.render), _p(gt_chw), _p(self.dm1), _p(self.dm2),
+                      _p(self.dm3), _p(self.l1_partials), _p(self.ssim_partials), s)
+            self._run("photometric_loss_finish", lb.gsx_photometric_loss_finish, c_u32(3), c_u32(H), c_u32(W),
+                      c_f(self.lambda_dssim), _p(self.l1_partials), _p(self.ssim_partials),
+                      c_u32(self.n_partials_fused), _p(self.loss_out), s)
+            return self.loss_out
         self._run("image_from_render", lb.gsx_image_from_render, c_u32(H), c_u32(W), _p(self.render), _p(gt_chw), _p(self.image),
                                        _p(self.l1_partials), s)
         if self.use_ssim:
@@ -208,13 +219,19 @@ class TrainStep:
         lb, s, N, H, W = self.lib, self._stream(), self.N, self.H, self.W
         P, A, J, G, V = self.params, self.act, self.proj, self.grads, self.v_act
         dimg = None
-        if self.use_ssim:
+        if self.fused_loss:
+            self._run("photometric_loss_backward", lb.gsx_photometric_loss_backward, c_u32(H), c_u32(W),
+                      c_f(self.lambda_dssim), _p(self.render), _p(self.gt), _p(self.dm1), _p(self.dm2), _p(self.dm3),
+                      _p(self.v_render), s)
+        elif self.use_ssim:
             self._run("fusedssim_backward", lb.gsx_fusedssim_backward, c_i(1), c_i(3), c_i(H), c_i(W), c_f(0.01 ** 2), c_f(0.03 ** 2),
                                             _p(self.image), _p(self.gt), _p(self.dL_dmap), _p(self.dm1), _p(self.dm2),
                                             _p(self.dm3), _p(self.dL_dimg), s)
             dimg = self.dL_dimg
-        self._run("render_grad_from_loss", lb.gsx_render_grad_from_loss, c_u32(H), c_u32(W), c_f(self.lambda_dssim), _p(self.render),
-                                           _p(self.image), _p(self.gt), _p(dimg), _p(self.v_render), s)
+        if not self.fused_loss:
+            self._run("render_grad_from_loss", lb.gsx_render_grad_from_loss, c_u32(H), c_u32(W),
+                      c_f(self.lambda_dssim), _p(self.render), _p(self.image), _p(self.gt), _p(dimg),
+                      _p(self.v_render), s)
         ws, wsn = _p(self.ws_bwd), c_sz(self.ws_bwd.numel())
         self._run("rasterize_bwd_accumulate", lb.gsx_rasterize_bwd_accumulate,
                   c_u32(1), c_u32(N), c_i64(self.n_isects), _p(self.records), _p(self.bg), c_p(None), c_u32(W),

@@ -117,3 +117,32 @@ def test_fused_update_equals_separate_kernels(gsx, cuda, cfg, n, freeze):
                 assert torch.equal(x.view(torch.int32), y.view(torch.int32)), f"{name} {k} iteration {it}"
         assert float(b2.ws_bwd.view(torch.float32).abs().max()) == 0.0  # accumulators left cleared
         # keep the two states identical for the next iteration (they are, bit for bit)
+
+
+@pytest.mark.parametrize("W,H", [(309, 205), (64, 48), (9, 7)])
+def test_fused_loss_equals_separate_kernels(gsx, cuda, W, H):
+    """gsx_photometric_loss_forward / _backward against image_from_render + fusedssim + partials + fusedssim_backward
+    + render_grad_from_loss: same d loss / d render per pixel, same loss up to summation order (ragged image sizes,
+    an image smaller than the SSIM window: no valid crop)"""
+    from lichtfeld_studio_amd.trainer import TrainStep
+    sc = gsx.scenes.config(3, 20_000)
+    sc.scaling_raw += 1.2
+    cam = gsx.scenes.orbit_camera(0.7, 4.0, W, H, 0.93 * W)
+    vm = torch.from_numpy(cam.viewmat[None].copy()).to(cuda)
+    Km = torch.from_numpy(cam.K[None].copy()).to(cuda)
+    gt = torch.rand((1, 3, H, W), generator=torch.Generator().manual_seed(5)).to(cuda)
+    a = TrainStep(sc, cuda, fused_loss=False)
+    b = TrainStep(sc, cuda, fused_loss=True)
+    for ts in (a, b):
+        ts.forward(vm, Km, W, H)
+        # push part of the render outside [0, 1] so that the clamp and its VJP matter
+        ts.render.mul_(1.6).sub_(0.1)
+        ts.loss_forward(gt)
+        ts.backward()
+    torch.cuda.synchronize()
+    la, lb = a.loss_out.cpu().numpy(), b.loss_out.cpu().numpy()
+    assert np.abs(la - lb).max() <= 2e-6, (la, lb)
+    va, vb = a.v_render.cpu().numpy(), b.v_render.cpu().numpy()
+    assert (va != 0).mean() > 0.3
+    assert np.abs(va - vb).max() <= 1e-6 * np.abs(va).max()
+    assert np.array_equal(va == 0, vb == 0)  # the clamp mask
