@@ -180,18 +180,20 @@ GSX_API int gsx_rasterize_pair_stats(int64_t n_isects, const void* records, uint
                                      unsigned long long* stats_out, void* stream);
 
 /* ---- a8: gsplat::rasterize_to_pixels_from_world_3dgs_bwd (Ops.h:131-166; ...3DGSBwd.cu:16-379) ----
- * channels must be 3.  The five gradient outputs are fully WRITTEN (no zero-fill needed; the reference
+ * channels in {1, 3, 4} (RGB, and the depth render modes of Rasterization.cpp:374-393).  The five gradient outputs are fully WRITTEN (no zero-fill needed; the reference
  * zero-fills and accumulates, Rasterization.cpp:190-194): v_means [N,3], v_quats [N,4], v_scales [N,3],
- * v_colors [C,N,3], v_opacities [C,N].  Workspace of the whole operator: 16 accumulator floats per Gaussian
- * followed by the records. */
+ * v_colors [C,N,channels], v_opacities [C,N].  Workspace of the whole operator: 16 + 1 accumulator floats per
+ * Gaussian followed by the records. */
 GSX_API size_t gsx_rasterize_bwd_workspace_bytes(uint32_t N);
 GSX_API size_t gsx_rasterize_bwd_accum_bytes(uint32_t N);
 /* The backward pass is three launches - clear the accumulators, the per-tile kernel, the per-Gaussian epilogue -
  * that can also be called one by one (a training loop shares the forward's records and can fold the epilogue into
  * its own per-Gaussian pass); these three take the accumulator part (gsx_rasterize_bwd_accum_bytes) only. */
 GSX_API int gsx_rasterize_bwd_clear(uint32_t N, void* workspace, size_t workspace_bytes, void* stream);
+/* colors [N,channels] is read for a fourth channel only (nullable otherwise) */
 GSX_API int gsx_rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isects, const void* records,
-                                         const float* backgrounds, const uint8_t* masks, uint32_t image_width,
+                                         const float* colors, uint32_t channels, const float* backgrounds,
+                                         const uint8_t* masks, uint32_t image_width,
                                          uint32_t image_height, uint32_t tile_size, const float* viewmats0,
                                          const float* Ks, const int32_t* tile_offsets, const int32_t* flatten_ids,
                                          const float* render_alphas, const int32_t* last_ids,
@@ -201,11 +203,11 @@ GSX_API int gsx_rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isect
  * needs no gsx_rasterize_bwd_clear */
 GSX_API int gsx_rasterize_bwd_finish(uint32_t N, const float* means, const float* quats, const float* scales,
                                      const float* viewmats0, void* workspace, size_t workspace_bytes,
-                                     int clear_accumulators, float* v_means, float* v_quats, float* v_scales,
-                                     float* v_colors, float* v_opacities, void* stream);
+                                     int clear_accumulators, uint32_t channels, float* v_means, float* v_quats,
+                                     float* v_scales, float* v_colors, float* v_opacities, void* stream);
 GSX_API int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
     uint32_t C, uint32_t N, int64_t n_isects, const float* means, const float* quats, const float* scales,
-    const float* colors, const float* opacities, const float* backgrounds, const uint8_t* masks,
+    const float* colors, uint32_t channels, const float* opacities, const float* backgrounds, const uint8_t* masks,
     uint32_t image_width, uint32_t image_height, uint32_t tile_size, const float* viewmats0,
     const float* viewmats1 /*must be NULL*/, const float* Ks, int camera_model, gsx_ut_params ut, int rs_type,
     const float* radial_coeffs, const float* tangential_coeffs, const float* thin_prism_coeffs,

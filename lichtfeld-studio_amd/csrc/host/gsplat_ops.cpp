@@ -344,7 +344,8 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> rasterize
     if (masks.has_value()) {
         CHECK_INPUT(masks.value());
     }
-    TORCH_CHECK(colors.size(-1) == 3, "Unsupported number of channels: ", colors.size(-1)); // Rasterization.cpp:65
+    const uint32_t channels = (uint32_t)colors.size(-1);
+    TORCH_CHECK(channels == 1 || channels == 3 || channels == 4, "Unsupported number of channels: ", channels);
     const uint32_t C = (uint32_t)tile_offsets.size(0), N = (uint32_t)means.size(0);
     // the kernels write every element of the five outputs (the reference zero-fills, Rasterization.cpp:190-194)
     at::Tensor v_means = at::empty_like(means), v_quats = at::empty_like(quats), v_scales = at::empty_like(scales);
@@ -352,7 +353,7 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> rasterize
     at::Tensor ws = workspace(gsx_rasterize_bwd_workspace_bytes(N), means);
     gsx_check(gsx_rasterize_to_pixels_from_world_3dgs_bwd(
         C, N, flatten_ids.size(0), means.data_ptr<float>(), quats.data_ptr<float>(), scales.data_ptr<float>(),
-        colors.data_ptr<float>(), opacities.data_ptr<float>(), fptr(backgrounds), bptr(masks), image_width,
+        colors.data_ptr<float>(), channels, opacities.data_ptr<float>(), fptr(backgrounds), bptr(masks), image_width,
         image_height, tile_size, viewmats0.data_ptr<float>(), fptr(viewmats1), Ks.data_ptr<float>(), (int)camera_model,
         to_gsx(ut_params), (int)rs_type, fptr(radial_coeffs), fptr(tangential_coeffs), fptr(thin_prism_coeffs),
         tile_offsets.data_ptr<int32_t>(), flatten_ids.data_ptr<int32_t>(), render_alphas.data_ptr<float>(),
@@ -382,7 +383,7 @@ rasterize_from_world_with_sh_fwd(const at::Tensor means, const at::Tensor quats,
     CHECK_INPUT(sh_coeffs);
     CHECK_INPUT(viewmats0);
     CHECK_INPUT(Ks);
-    TORCH_CHECK(render_mode == 0, "render_mode ", render_mode, ": only RGB (0) is built");
+    TORCH_CHECK(render_mode >= 0 && render_mode <= 4, "render_mode ", render_mode, ": must be 0 .. 4");
     const uint32_t N = (uint32_t)means.size(0), C = (uint32_t)viewmats0.size(0);
     at::Tensor op_flat = opacities.reshape({-1});
     at::Tensor scaled_scales = scaling_modifier == 1.0f ? scales : at::mul(scales, scaling_modifier); // Rasterization.cpp:327
@@ -392,11 +393,18 @@ rasterize_from_world_with_sh_fwd(const at::Tensor means, const at::Tensor quats,
                                          thin_prism_coeffs);
     at::Tensor radii = std::get<0>(proj), means2d = std::get<1>(proj), depths = std::get<2>(proj);
     at::Tensor compensations = std::get<4>(proj);
-    // Rasterization.cpp:356-378 in one pass: dirs, radii mask, SH, + 0.5, clamp
-    at::Tensor colors = at::empty({C, N, 3}, means.options());
-    gsx_check(gsx_sh_colors_from_world(N, (uint32_t)sh_coeffs.size(1), sh_degree, means.data_ptr<float>(),
-                                       sh_coeffs.data_ptr<float>(), radii.data_ptr<int32_t>(),
-                                       viewmats0.data_ptr<float>(), colors.data_ptr<float>(), cur_stream(means)));
+    at::Tensor colors;
+    if (render_mode == 0 || render_mode == 3 || render_mode == 4) {
+        // Rasterization.cpp:356-378 in one pass: dirs, radii mask, SH, + 0.5, clamp
+        colors = at::empty({C, N, 3}, means.options());
+        gsx_check(gsx_sh_colors_from_world(N, (uint32_t)sh_coeffs.size(1), sh_degree, means.data_ptr<float>(),
+                                           sh_coeffs.data_ptr<float>(), radii.data_ptr<int32_t>(),
+                                           viewmats0.data_ptr<float>(), colors.data_ptr<float>(), cur_stream(means)));
+        if (render_mode != 0) // RGB + depth (:385-387)
+            colors = at::cat({colors, depths.unsqueeze(-1)}, -1).contiguous();
+    } else { // depth only (:389-392)
+        colors = depths.unsqueeze(-1).contiguous();
+    }
     at::Tensor final_opacities = op_flat.unsqueeze(0);
     if (calc_compensations && compensations.defined() && compensations.numel() > 0)
         final_opacities = at::mul(final_opacities, compensations).contiguous();
@@ -436,7 +444,7 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> rasterize
     CHECK_INPUT(sh_coeffs);
     CHECK_INPUT(v_render_colors);
     CHECK_INPUT(v_render_alphas);
-    TORCH_CHECK(render_mode == 0, "render_mode ", render_mode, ": only RGB (0) is built");
+    TORCH_CHECK(render_mode >= 0 && render_mode <= 4, "render_mode ", render_mode, ": must be 0 .. 4");
     at::Tensor final_opacities = opacities.reshape({1, -1});
     if (calc_compensations && compensations.defined() && compensations.numel() > 0)
         final_opacities = at::mul(final_opacities, compensations).contiguous();
@@ -447,11 +455,21 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> rasterize
                                                      radial_coeffs, tangential_coeffs, thin_prism_coeffs, tile_offsets,
                                                      flatten_ids, render_alphas, last_ids, v_render_colors,
                                                      v_render_alphas);
-    at::Tensor v_sh = at::empty_like(sh_coeffs);
-    gsx_check(gsx_sh_colors_from_world_bwd((uint32_t)means.size(0), (uint32_t)sh_coeffs.size(1), sh_degree,
-                                           means.data_ptr<float>(), radii.data_ptr<int32_t>(),
-                                           viewmats0.data_ptr<float>(), colors.data_ptr<float>(),
-                                           std::get<3>(g).data_ptr<float>(), v_sh.data_ptr<float>(), cur_stream(means)));
+    at::Tensor v_sh;
+    if (render_mode == 0 || render_mode == 3 || render_mode == 4) {
+        at::Tensor rgb = colors, v_rgb = std::get<3>(g);
+        if (render_mode != 0) { // the depth channel's gradient is dropped (:587-606)
+            rgb = colors.slice(-1, 0, 3).contiguous();
+            v_rgb = v_rgb.slice(-1, 0, 3).contiguous();
+        }
+        v_sh = at::empty_like(sh_coeffs);
+        gsx_check(gsx_sh_colors_from_world_bwd((uint32_t)means.size(0), (uint32_t)sh_coeffs.size(1), sh_degree,
+                                               means.data_ptr<float>(), radii.data_ptr<int32_t>(),
+                                               viewmats0.data_ptr<float>(), rgb.data_ptr<float>(),
+                                               v_rgb.data_ptr<float>(), v_sh.data_ptr<float>(), cur_stream(means)));
+    } else {
+        v_sh = at::zeros_like(sh_coeffs); // :625-629
+    }
     at::Tensor v_scales = std::get<2>(g);
     if (scaling_modifier != 1.0f)
         v_scales = at::mul(v_scales, scaling_modifier); // Rasterization.cpp:633

@@ -91,15 +91,23 @@ __global__ void __launch_bounds__(64) wave_reduce16_probe_kernel(const float* __
     }
 }
 
+// CDIM = 3: the RGB training path.  CDIM = 1 / 4: the depth render modes (Rasterization.cpp:374-393) - one colour
+// channel, or RGB plus a fourth channel that is staged from `colors` and whose per-Gaussian gradient is reduced
+// on its own into gextra [N].
+template <uint32_t CDIM>
 __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
-    uint32_t n_isects, const float4* __restrict__ records, const float* __restrict__ backgrounds,
+    uint32_t n_isects, const float4* __restrict__ records, const float* __restrict__ colors,
+    const float* __restrict__ backgrounds,
     const uint8_t* __restrict__ masks, uint32_t image_width, uint32_t image_height, uint32_t tile_width,
     uint32_t tile_height, const float* __restrict__ viewmat, const float* __restrict__ Kmat,
     const int32_t* __restrict__ tile_offsets, const int32_t* __restrict__ flatten_ids,
     const float* __restrict__ render_alphas, const int32_t* __restrict__ last_ids,
     const float* __restrict__ v_render_colors, const float* __restrict__ v_render_alphas,
-    float* __restrict__ gacc /*[N,16]*/) {
+    float* __restrict__ gacc /*[N,16]*/, float* __restrict__ gextra /*[N], CDIM == 4*/) {
+    constexpr uint32_t NC = CDIM < 3 ? CDIM : 3; // channels carried by the record
     __shared__ float4 stage[kBatch * 4];
+    __shared__ float extra[CDIM > 3 ? kBatch : 1];
+    __shared__ float acc_extra[CDIM > 3 ? kBatch : 1];
     __shared__ float4 region[kBatch * 2];
     __shared__ float cuts[kBatch];
     __shared__ uint8_t lists[4][kBatch];
@@ -127,17 +135,19 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
 
     const float T_final = 1.0f - render_alphas[pix_id];
     float T = T_final;
-    float buffer[3] = {0.f, 0.f, 0.f};
+    float buffer[CDIM];
     const int32_t bin_final = inside ? last_ids[pix_id] : 0;
-    float v_render_c[3];
+    float v_render_c[CDIM];
 #pragma unroll
-    for (uint32_t k = 0; k < 3; ++k)
-        v_render_c[k] = v_render_colors[(size_t)pix_id * 3 + k];
+    for (uint32_t k = 0; k < CDIM; ++k) {
+        buffer[k] = 0.f;
+        v_render_c[k] = v_render_colors[(size_t)pix_id * CDIM + k];
+    }
     const float v_render_a = v_render_alphas[pix_id];
     float bg_dot = 0.f;
     if (backgrounds != nullptr) {
 #pragma unroll
-        for (uint32_t k = 0; k < 3; ++k)
+        for (uint32_t k = 0; k < CDIM; ++k)
             bg_dot += backgrounds[k] * v_render_c[k];
     }
 
@@ -156,6 +166,8 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
 #pragma unroll
     for (uint32_t k = 0; k < kAcc; ++k)
         acc[tr * kAcc + k] = 0.f;
+    if (CDIM > 3)
+        acc_extra[tr] = 0.f;
     __syncthreads();
     range_end = min(range_end, block_max + 1);
     if (range_end <= range_start)
@@ -171,6 +183,11 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
         const uint32_t n_sel = (uint32_t)__builtin_amdgcn_readfirstlane((int)stage_and_select(
             records, flatten_ids, batch_end, -1, (uint32_t)batch_size, tr, px, t_start,
             t_start < (uint32_t)batch_size, stage, region, cuts, id_batch, wave_list));
+        if (CDIM > 3) {
+            if ((int32_t)tr < batch_size)
+                extra[tr] = colors[(size_t)id_batch[tr] * CDIM + 3];
+            __syncthreads();
+        }
 
         for (uint32_t sidx = 0; sidx < n_sel; ++sidx) {
             const int32_t t = (int32_t)wave_list[sidx];
@@ -210,13 +227,14 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             const float ra = valid ? __builtin_amdgcn_rcpf(1.0f - alpha) : 1.0f;
             T *= ra;
             const float fac = valid ? alpha * T : 0.f;
+            const float col[4] = {m2.y, m2.z, m2.w, CDIM > 3 ? extra[t] : 0.f};
             v[0] = fac * v_render_c[0];
-            v[1] = fac * v_render_c[1];
-            v[2] = fac * v_render_c[2];
+            v[1] = NC > 1 ? fac * v_render_c[NC > 1 ? 1 : 0] : 0.f;
+            v[2] = NC > 2 ? fac * v_render_c[NC > 2 ? 2 : 0] : 0.f;
             float v_alpha = 0.f;
-            v_alpha += (m2.y * T - buffer[0] * ra) * v_render_c[0];
-            v_alpha += (m2.z * T - buffer[1] * ra) * v_render_c[1];
-            v_alpha += (m2.w * T - buffer[2] * ra) * v_render_c[2];
+#pragma unroll
+            for (uint32_t k = 0; k < CDIM; ++k)
+                v_alpha += (col[k] * T - buffer[k] * ra) * v_render_c[k];
             v_alpha += T_final * ra * v_render_a;
             if (backgrounds != nullptr)
                 v_alpha += -T_final * ra * bg_dot;
@@ -245,9 +263,17 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             v[13] = v_grd.z * ray_d.y;
             v[14] = v_grd.z * ray_d.z;
             v[15] = vis * v_alpha;
-            buffer[0] += m2.y * fac;
-            buffer[1] += m2.z * fac;
-            buffer[2] += m2.w * fac;
+#pragma unroll
+            for (uint32_t k = 0; k < CDIM; ++k)
+                buffer[k] += col[k] * fac;
+            if (CDIM > 3) { // the fourth channel's gradient: its own wave sum
+                float e = fac * v_render_c[CDIM > 3 ? 3 : 0];
+#pragma unroll
+                for (int m = 32; m >= 1; m >>= 1)
+                    e += __shfl_xor(e, m, 64);
+                if (lane == 0)
+                    atomicAdd(&acc_extra[t], e);
+            }
             const float total = wave_reduce16(v, lane);
             if ((lane & 3u) == 0) {
                 const uint32_t comp = ((lane >> 5) & 1u) * 8u + ((lane >> 4) & 1u) * 4u + ((lane >> 3) & 1u) * 2u +
@@ -268,6 +294,12 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
                     unsafeAtomicAdd(&gacc[(size_t)id_batch[gi] * kAcc + k], val);
             }
         }
+        if (CDIM > 3 && (int32_t)tr < batch_size) {
+            const float val = acc_extra[tr];
+            acc_extra[tr] = 0.f;
+            if (val != 0.f)
+                unsafeAtomicAdd(&gextra[id_batch[tr]], val);
+        }
         __syncthreads();
     }
 }
@@ -276,9 +308,9 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
 // (v_mean, v_quat, v_scale) - quat_scale_to_preci_half_vjp / quat_to_rotmat_vjp of Utils.cuh:104-158.
 __global__ void __launch_bounds__(256) rasterize_bwd_epilogue_kernel(
     uint32_t N, const float* __restrict__ means, const float* __restrict__ quats, const float* __restrict__ scales,
-    const float* __restrict__ viewmat, float* __restrict__ gacc, int clear, float* __restrict__ v_means,
-    float* __restrict__ v_quats, float* __restrict__ v_scales, float* __restrict__ v_colors,
-    float* __restrict__ v_opacities) {
+    const float* __restrict__ viewmat, float* __restrict__ gacc, float* __restrict__ gextra, uint32_t channels,
+    int clear, float* __restrict__ v_means, float* __restrict__ v_quats, float* __restrict__ v_scales,
+    float* __restrict__ v_colors, float* __restrict__ v_opacities) {
     const uint32_t g = blockIdx.x * 256u + threadIdx.x;
     if (g >= N)
         return;
@@ -293,9 +325,17 @@ __global__ void __launch_bounds__(256) rasterize_bwd_epilogue_kernel(
         row[0] = z, row[1] = z, row[2] = z, row[3] = z;
     }
     // r0 = rgb.xyz, vo.x ; r1 = vo.y, vo.z, G00, G01 ; r2 = G02, G10, G11, G12 ; r3 = G20, G21, G22, v_opacity
-    v_colors[(size_t)g * 3 + 0] = r0.x;
-    v_colors[(size_t)g * 3 + 1] = r0.y;
-    v_colors[(size_t)g * 3 + 2] = r0.z;
+    v_colors[(size_t)g * channels + 0] = r0.x;
+    if (channels > 1)
+        v_colors[(size_t)g * channels + 1] = r0.y;
+    if (channels > 2)
+        v_colors[(size_t)g * channels + 2] = r0.z;
+    if (channels > 3) {
+        const float e = gextra[g];
+        v_colors[(size_t)g * channels + 3] = e;
+        if (clear && e != 0.f)
+            gextra[g] = 0.f;
+    }
     v_opacities[g] = r3.w;
     float vm[3] = {0.f, 0.f, 0.f}, vq[4] = {0.f, 0.f, 0.f, 0.f}, vs[3] = {0.f, 0.f, 0.f};
     if (any_geo)
@@ -321,8 +361,12 @@ extern "C" int gsx_debug_wave_reduce16(uint32_t n_waves, const float* in, float*
     return GSX_OK;
 }
 
-// accumulators only (16 floats per Gaussian); the whole-operator entry point also packs the records behind them
-extern "C" size_t gsx_rasterize_bwd_accum_bytes(uint32_t N) { return align_up((size_t)N * kAcc * 4, 256) + 256; }
+// accumulators only: 16 floats per Gaussian, then one float per Gaussian for a fourth colour channel; the
+// whole-operator entry point also packs the records behind them
+static size_t accum_extra_offset(uint32_t N) { return align_up((size_t)N * kAcc * 4, 256) + 256; }
+extern "C" size_t gsx_rasterize_bwd_accum_bytes(uint32_t N) {
+    return accum_extra_offset(N) + align_up((size_t)N * 4, 256);
+}
 extern "C" size_t gsx_rasterize_bwd_workspace_bytes(uint32_t N) {
     return gsx_rasterize_bwd_accum_bytes(N) + gsx_raster_records_bytes(N);
 }
@@ -335,7 +379,7 @@ extern "C" int gsx_rasterize_bwd_clear(uint32_t N, void* workspace, size_t works
                     workspace_bytes >= gsx_rasterize_bwd_accum_bytes(N),
                 GSX_ERR_WORKSPACE, "rasterize bwd: accumulators need %zu bytes, 256-byte aligned",
                 gsx_rasterize_bwd_accum_bytes(N));
-    const size_t n_acc = (size_t)N * kAcc;
+    const size_t n_acc = gsx_rasterize_bwd_accum_bytes(N) / 4;
     hipLaunchKernelGGL(fill_f32_kernel, dim3(cdiv(n_acc, 256)), dim3(256), 0, (hipStream_t)stream, n_acc, 0.f,
                        (float*)workspace);
     GSX_LAUNCH_CHECK();
@@ -345,7 +389,8 @@ extern "C" int gsx_rasterize_bwd_clear(uint32_t N, void* workspace, size_t works
 // stage 2: the per-tile kernel, accumulating into the workspace; `records` from gsx_pack_raster_records (or the
 // fused per-Gaussian pass) for the same camera and parameters
 extern "C" int gsx_rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isects, const void* records,
-                                            const float* backgrounds, const uint8_t* masks, uint32_t image_width,
+                                            const float* colors, uint32_t channels, const float* backgrounds,
+                                            const uint8_t* masks, uint32_t image_width,
                                             uint32_t image_height, uint32_t tile_size, const float* viewmats0,
                                             const float* Ks, const int32_t* tile_offsets, const int32_t* flatten_ids,
                                             const float* render_alphas, const int32_t* last_ids,
@@ -364,11 +409,22 @@ extern "C" int gsx_rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_is
                     workspace_bytes >= gsx_rasterize_bwd_accum_bytes(N),
                 GSX_ERR_WORKSPACE, "rasterize bwd: accumulators need %zu bytes, 256-byte aligned",
                 gsx_rasterize_bwd_accum_bytes(N));
+    GSX_REQUIRE(channels == 1 || channels == 3 || channels == 4, GSX_ERR_UNSUPPORTED,
+                "rasterize bwd: %u channels (built: 1, 3, 4)", channels);
+    GSX_REQUIRE(channels <= 3 || colors != nullptr, GSX_ERR_INVALID_ARGUMENT, "rasterize bwd: colors is null");
     const uint32_t tw = cdiv(image_width, kTile), th = cdiv(image_height, kTile);
-    hipLaunchKernelGGL(rasterize_bwd_kernel, dim3(tw * th), dim3(256), 0, (hipStream_t)stream, (uint32_t)n_isects,
-                       (const float4*)records, backgrounds, masks, image_width, image_height, tw, th, viewmats0, Ks,
-                       tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors, v_render_alphas,
-                       (float*)workspace);
+    float* gextra = (float*)((char*)workspace + accum_extra_offset(N));
+#define GSX_LAUNCH_BWD(CD)                                                                                           \
+    hipLaunchKernelGGL((rasterize_bwd_kernel<CD>), dim3(tw * th), dim3(256), 0, (hipStream_t)stream,                 \
+                       (uint32_t)n_isects, (const float4*)records, colors, backgrounds, masks, image_width,          \
+                       image_height, tw, th, viewmats0, Ks, tile_offsets, flatten_ids, render_alphas, last_ids,      \
+                       v_render_colors, v_render_alphas, (float*)workspace, gextra)
+    switch (channels) {
+    case 1: GSX_LAUNCH_BWD(1); break;
+    case 3: GSX_LAUNCH_BWD(3); break;
+    default: GSX_LAUNCH_BWD(4); break;
+    }
+#undef GSX_LAUNCH_BWD
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }
@@ -376,24 +432,26 @@ extern "C" int gsx_rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_is
 // stage 3: per-Gaussian epilogue, accumulators -> the five gradient tensors (all elements written)
 extern "C" int gsx_rasterize_bwd_finish(uint32_t N, const float* means, const float* quats, const float* scales,
                                         const float* viewmats0, void* workspace, size_t workspace_bytes,
-                                        int clear_accumulators, float* v_means, float* v_quats, float* v_scales,
-                                        float* v_colors, float* v_opacities, void* stream) {
+                                        int clear_accumulators, uint32_t channels, float* v_means, float* v_quats,
+                                        float* v_scales, float* v_colors, float* v_opacities, void* stream) {
     if (N == 0)
         return GSX_OK;
     GSX_REQUIRE(means && quats && scales && viewmats0 && v_means && v_quats && v_scales && v_colors && v_opacities,
                 GSX_ERR_INVALID_ARGUMENT, "rasterize bwd: null tensor");
     GSX_REQUIRE(workspace != nullptr && workspace_bytes >= gsx_rasterize_bwd_accum_bytes(N), GSX_ERR_WORKSPACE,
                 "rasterize bwd: accumulators need %zu bytes", gsx_rasterize_bwd_accum_bytes(N));
+    GSX_REQUIRE(channels == 1 || channels == 3 || channels == 4, GSX_ERR_UNSUPPORTED,
+                "rasterize bwd: %u channels (built: 1, 3, 4)", channels);
     hipLaunchKernelGGL(rasterize_bwd_epilogue_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, means,
-                       quats, scales, viewmats0, (float*)workspace, clear_accumulators, v_means, v_quats, v_scales,
-                       v_colors, v_opacities);
+                       quats, scales, viewmats0, (float*)workspace, (float*)((char*)workspace + accum_extra_offset(N)),
+                       channels, clear_accumulators, v_means, v_quats, v_scales, v_colors, v_opacities);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }
 
 extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
     uint32_t C, uint32_t N, int64_t n_isects, const float* means, const float* quats, const float* scales,
-    const float* colors, const float* opacities, const float* backgrounds, const uint8_t* masks,
+    const float* colors, uint32_t channels, const float* opacities, const float* backgrounds, const uint8_t* masks,
     uint32_t image_width, uint32_t image_height, uint32_t tile_size, const float* viewmats0, const float* viewmats1,
     const float* Ks, int camera_model, gsx_ut_params ut, int rs_type, const float* radial_coeffs,
     const float* tangential_coeffs, const float* thin_prism_coeffs, const int32_t* tile_offsets,
@@ -417,14 +475,14 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
     void* records = (char*)workspace + acc_bytes;
     if ((rc = gsx_rasterize_bwd_clear(N, workspace, acc_bytes, stream)) != GSX_OK)
         return rc;
-    if ((rc = gsx_pack_raster_records(N, means, quats, scales, opacities, colors, 3, viewmats0, Ks, image_width,
+    if ((rc = gsx_pack_raster_records(N, means, quats, scales, opacities, colors, channels, viewmats0, Ks, image_width,
                                       image_height, records, stream)) != GSX_OK)
         return rc;
-    if ((rc = gsx_rasterize_bwd_accumulate(C, N, n_isects, records, backgrounds, masks, image_width, image_height,
-                                           tile_size, viewmats0, Ks, tile_offsets, flatten_ids, render_alphas,
-                                           last_ids, v_render_colors, v_render_alphas, workspace, acc_bytes,
-                                           stream)) != GSX_OK)
+    if ((rc = gsx_rasterize_bwd_accumulate(C, N, n_isects, records, colors, channels, backgrounds, masks, image_width,
+                                           image_height, tile_size, viewmats0, Ks, tile_offsets, flatten_ids,
+                                           render_alphas, last_ids, v_render_colors, v_render_alphas, workspace,
+                                           acc_bytes, stream)) != GSX_OK)
         return rc;
-    return gsx_rasterize_bwd_finish(N, means, quats, scales, viewmats0, workspace, acc_bytes, 0, v_means, v_quats,
-                                    v_scales, v_colors, v_opacities, stream);
+    return gsx_rasterize_bwd_finish(N, means, quats, scales, viewmats0, workspace, acc_bytes, 0, channels, v_means,
+                                    v_quats, v_scales, v_colors, v_opacities, stream);
 }

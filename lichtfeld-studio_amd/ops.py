@@ -272,8 +272,8 @@ def rasterize_to_pixels_from_world_3dgs_bwd(means, quats, scales, colors, opacit
         _f32(t, n)
     _check_input(tile_offsets, "tile_offsets"), _check_input(flatten_ids, "flatten_ids")
     _check_input(last_ids, "last_ids")
-    if colors.size(-1) != 3:
-        raise RuntimeError("Unsupported number of channels: only 3 is built for the backward pass")
+    if colors.size(-1) not in (1, 3, 4):
+        raise RuntimeError("Unsupported number of channels: %d (built: 1, 3, 4)" % colors.size(-1))
     if backgrounds is not None and backgrounds.numel() == 0:
         backgrounds = None
     dev = means.device
@@ -285,7 +285,8 @@ def rasterize_to_pixels_from_world_3dgs_bwd(means, quats, scales, colors, opacit
         ws = _workspace(lib().gsx_rasterize_bwd_workspace_bytes(c_u32(N)), dev)
         check(lib().gsx_rasterize_to_pixels_from_world_3dgs_bwd(
             c_u32(C), c_u32(N), c_i64(flatten_ids.numel()), _ptr(means), _ptr(quats), _ptr(scales), _ptr(colors),
-            _ptr(opacities), _ptr(backgrounds), _ptr(m8), c_u32(image_width), c_u32(image_height), c_u32(tile_size),
+            c_u32(colors.size(-1)), _ptr(opacities), _ptr(backgrounds), _ptr(m8), c_u32(image_width),
+            c_u32(image_height), c_u32(tile_size),
             _ptr(viewmats0), _ptr(viewmats1), _ptr(Ks), c_i(camera_model), ut_params, c_i(rs_type),
             _ptr(radial_coeffs), _ptr(tangential_coeffs), _ptr(thin_prism_coeffs), _ptr(tile_offsets),
             _ptr(flatten_ids), _ptr(render_alphas), _ptr(last_ids), _ptr(v_render_colors), _ptr(v_render_alphas),
@@ -300,12 +301,13 @@ def rasterize_from_world_with_sh_fwd(means, quats, scales, opacities, sh_coeffs,
                                      render_mode, ut_params, rs_type, radial_coeffs=None, tangential_coeffs=None,
                                      thin_prism_coeffs=None, return_isect_ids=False):
     """Ops.h:174-220 (Rasterization.cpp:279-467).  -> (render_colors, render_alphas, radii, means2d, depths, colors,
-    tile_offsets, flatten_ids, last_ids, compensations).  render_mode 0 (RGB) is built."""
+    tile_offsets, flatten_ids, last_ids, compensations).  render_mode: 0 RGB, 1 / 2 depth (one channel), 3 / 4
+    RGB + depth (four channels), as Rasterization.cpp:372-393."""
     for t, n in ((means, "means"), (quats, "quats"), (scales, "scales"), (opacities, "opacities"),
                  (sh_coeffs, "sh_coeffs"), (viewmats0, "viewmats0"), (Ks, "Ks")):
         _f32(t, n)
-    if render_mode != 0:
-        raise NotImplementedError("render_mode %d: only RGB (0) is built" % render_mode)
+    if render_mode not in (0, 1, 2, 3, 4):
+        raise RuntimeError("render_mode %d: must be 0 (RGB), 1 (D), 2 (ED), 3 (RGB_D) or 4 (RGB_ED)" % render_mode)
     dev = means.device
     N, C = means.size(0), viewmats0.size(0)
     opacities = opacities.reshape(-1)
@@ -315,10 +317,15 @@ def rasterize_from_world_with_sh_fwd(means, quats, scales, opacities, sh_coeffs,
         near_plane, far_plane, radius_clip, calc_compensations, camera_model, ut_params, rs_type, radial_coeffs,
         tangential_coeffs, thin_prism_coeffs)
     K = sh_coeffs.size(1)
-    colors = torch.empty((C, N, 3), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
-        check(lib().gsx_sh_colors_from_world(c_u32(N), c_u32(K), c_u32(sh_degree), _ptr(means), _ptr(sh_coeffs),
-                                             _ptr(radii), _ptr(viewmats0), _ptr(colors), _stream(dev)))
+    if render_mode in (0, 3, 4):
+        colors = torch.empty((C, N, 3), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            check(lib().gsx_sh_colors_from_world(c_u32(N), c_u32(K), c_u32(sh_degree), _ptr(means), _ptr(sh_coeffs),
+                                                 _ptr(radii), _ptr(viewmats0), _ptr(colors), _stream(dev)))
+        if render_mode != 0:  # RGB + depth (Rasterization.cpp:385-387)
+            colors = torch.cat([colors, depths.unsqueeze(-1)], -1).contiguous()
+    else:  # depth only (:389-392)
+        colors = depths.unsqueeze(-1).contiguous()
     final_opacities = opacities.unsqueeze(0)
     if calc_compensations and comp is not None:
         final_opacities = (final_opacities * comp).contiguous()
@@ -346,8 +353,8 @@ def rasterize_from_world_with_sh_bwd(means, quats, scales, opacities, sh_coeffs,
                  (sh_coeffs, "sh_coeffs"), (v_render_colors, "v_render_colors"),
                  (v_render_alphas, "v_render_alphas")):
         _f32(t, n)
-    if render_mode != 0:
-        raise NotImplementedError("render_mode %d: only RGB (0) is built" % render_mode)
+    if render_mode not in (0, 1, 2, 3, 4):
+        raise RuntimeError("render_mode %d: must be 0 (RGB), 1 (D), 2 (ED), 3 (RGB_D) or 4 (RGB_ED)" % render_mode)
     dev = means.device
     N = means.size(0)
     final_opacities = opacities.reshape(1, -1)
@@ -359,11 +366,17 @@ def rasterize_from_world_with_sh_bwd(means, quats, scales, opacities, sh_coeffs,
         tile_size, viewmats0, viewmats1, Ks, camera_model, ut_params, rs_type, radial_coeffs, tangential_coeffs,
         thin_prism_coeffs, tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors, v_render_alphas)
     K = sh_coeffs.size(1)
-    v_sh = torch.empty_like(sh_coeffs)
-    with torch.cuda.device(dev):
-        check(lib().gsx_sh_colors_from_world_bwd(c_u32(N), c_u32(K), c_u32(sh_degree), _ptr(means), _ptr(radii),
-                                                 _ptr(viewmats0), _ptr(colors), _ptr(v_colors), _ptr(v_sh),
-                                                 _stream(dev)))
+    if render_mode in (0, 3, 4):
+        rgb, v_rgb = colors, v_colors
+        if render_mode != 0:  # the depth channel's gradient is dropped (Rasterization.cpp:587-606)
+            rgb, v_rgb = colors[..., :3].contiguous(), v_colors[..., :3].contiguous()
+        v_sh = torch.empty_like(sh_coeffs)
+        with torch.cuda.device(dev):
+            check(lib().gsx_sh_colors_from_world_bwd(c_u32(N), c_u32(K), c_u32(sh_degree), _ptr(means), _ptr(radii),
+                                                     _ptr(viewmats0), _ptr(rgb), _ptr(v_rgb), _ptr(v_sh),
+                                                     _stream(dev)))
+    else:
+        v_sh = torch.zeros_like(sh_coeffs)  # :625-629
     if scaling_modifier != 1.0:
         v_scales = v_scales * scaling_modifier  # Rasterization.cpp:633
     return v_means, v_quats, v_scales, v_opacities, v_sh

@@ -234,14 +234,15 @@ class TrainStep:
                       _p(self.v_render), s)
         ws, wsn = _p(self.ws_bwd), c_sz(self.ws_bwd.numel())
         self._run("rasterize_bwd_accumulate", lb.gsx_rasterize_bwd_accumulate,
-                  c_u32(1), c_u32(N), c_i64(self.n_isects), _p(self.records), _p(self.bg), c_p(None), c_u32(W),
-                  c_u32(H), c_u32(16),
+                  c_u32(1), c_u32(N), c_i64(self.n_isects), _p(self.records), c_p(None), c_u32(3), _p(self.bg),
+                  c_p(None), c_u32(W), c_u32(H), c_u32(16),
                   _p(self.viewmat), _p(self.Kmat), _p(self.offsets), _p(self.flatten_ids), _p(self.alpha),
                   _p(self.last_ids), _p(self.v_render), _p(self.v_alpha), ws, wsn, s)
         if self.fused_update:
             return
         self._run("rasterize_bwd_finish", lb.gsx_rasterize_bwd_finish, c_u32(N), _p(P["means"]), _p(A["quats"]),
-                  _p(A["scales"]), _p(self.viewmat), ws, wsn, c_i(1), _p(G["means"]), _p(V["quats"]), _p(V["scales"]),
+                  _p(A["scales"]), _p(self.viewmat), ws, wsn, c_i(1), c_u32(3), _p(G["means"]), _p(V["quats"]),
+                  _p(V["scales"]),
                   _p(self.v_colors), _p(V["opacities"]), s)
         self._run("sh_colors_from_world_bwd", lb.gsx_sh_colors_from_world_bwd, c_u32(N), c_u32(self.K), c_u32(self.sh_degree), _p(P["means"]),
                                               _p(J["radii"]), _p(self.viewmat), _p(self.colors), _p(self.v_colors),

@@ -184,7 +184,8 @@ def rasterize_to_pixels_from_world_3dgs_fwd(means, quats, scales, colors, opacit
 def rasterize_to_pixels_from_world_3dgs_bwd(means, quats, scales, colors, opacities, backgrounds, masks, image_width,
                                             image_height, tile_size, viewmats0, Ks, tile_offsets, flatten_ids,
                                             render_alphas, last_ids, v_render_colors, v_render_alphas):
-    """gsplat/Ops.h:131-166 (C == 1, CDIM == 3) -> v_means, v_quats, v_scales, v_colors [1,N,3], v_opacities [1,N]."""
+    """gsplat/Ops.h:131-166 (C == 1, 1 to 4 channels) -> v_means, v_quats, v_scales, v_colors [1,N,CDIM],
+    v_opacities [1,N]."""
     means, quats, scales = _f32(means), _f32(quats), _f32(scales)
     colors, opacities = _f32(colors), _f32(opacities)
     backgrounds, viewmats0, Ks = _f32(backgrounds), _f32(viewmats0), _f32(Ks)
@@ -194,13 +195,15 @@ def rasterize_to_pixels_from_world_3dgs_bwd(means, quats, scales, colors, opacit
     last_ids = np.ascontiguousarray(last_ids, dtype=np.int32)
     m = None if masks is None else np.ascontiguousarray(masks, dtype=np.uint8)
     N = means.shape[0]
+    cdim = colors.shape[-1]
     v_means = np.zeros((N, 3), np.float32)
     v_quats = np.zeros((N, 4), np.float32)
     v_scales = np.zeros((N, 3), np.float32)
-    v_colors = np.zeros((1, N, 3), np.float32)
+    v_colors = np.zeros((1, N, cdim), np.float32)
     v_opac = np.zeros((1, N), np.float32)
     _chk(lib().orc_rasterize_to_pixels_from_world_3dgs_bwd(
-        c_u32(1), c_u32(N), c_i64(flatten_ids.shape[0]), _p(means), _p(quats), _p(scales), _p(colors), _p(opacities),
+        c_u32(1), c_u32(N), c_i64(flatten_ids.shape[0]), _p(means), _p(quats), _p(scales), _p(colors), c_u32(cdim),
+        _p(opacities),
         _p(backgrounds), _p(m), c_u32(image_width), c_u32(image_height), c_u32(tile_size), _p(viewmats0), _p(Ks),
         _p(tile_offsets), _p(flatten_ids), _p(render_alphas), _p(last_ids), _p(v_render_colors), _p(v_render_alphas),
         _p(v_means), _p(v_quats), _p(v_scales), _p(v_colors), _p(v_opac)), "rasterize_bwd")
@@ -318,14 +321,21 @@ def sh_colors_from_world_bwd(sh_degree, means, K, radii, viewmat, colors, v_colo
 
 def rasterize_from_world_with_sh_fwd(means, quats, scales, opacities, sh_coeffs, sh_degree, backgrounds, image_width,
                                      image_height, tile_size, viewmats0, Ks, eps2d=0.3, near_plane=0.01, far_plane=1e4,
-                                     radius_clip=0.0, scaling_modifier=1.0, calc_compensations=False, ut=None):
-    """gsplat/Ops.h:174-220 (render_mode RGB, C == 1, no masks).  Returns the reference's 10-tuple plus the sorted
-    isect_ids (for key parity checks) as an 11th element."""
+                                     radius_clip=0.0, scaling_modifier=1.0, calc_compensations=False, ut=None,
+                                     render_mode=0):
+    """gsplat/Ops.h:174-220 (C == 1, no masks; render_mode 0 RGB, 1 / 2 depth, 3 / 4 RGB + depth,
+    Rasterization.cpp:372-393).  Returns the reference's 10-tuple plus the sorted isect_ids (for key parity checks)
+    as an 11th element."""
     scaled = _f32(scales) * np.float32(scaling_modifier) if scaling_modifier != 1.0 else _f32(scales)
     radii, means2d, depths, conics, comp = projection_ut_3dgs_fused(
         means, quats, scaled, opacities, viewmats0, Ks, image_width, image_height, eps2d, near_plane, far_plane,
         radius_clip, calc_compensations, ut)
-    colors = sh_colors_from_world(sh_degree, means, sh_coeffs, radii[0], viewmats0[0])[None]
+    if render_mode in (0, 3, 4):
+        colors = sh_colors_from_world(sh_degree, means, sh_coeffs, radii[0], viewmats0[0])[None]
+        if render_mode != 0:
+            colors = np.ascontiguousarray(np.concatenate([colors, depths[..., None]], -1))  # :385-387
+    else:
+        colors = np.ascontiguousarray(depths[..., None])  # :389-392
     final_op = _f32(opacities).reshape(1, -1)
     if calc_compensations:
         final_op = final_op * comp
@@ -342,7 +352,7 @@ def rasterize_from_world_with_sh_fwd(means, quats, scales, opacities, sh_coeffs,
 def rasterize_from_world_with_sh_bwd(means, quats, scales, opacities, sh_coeffs, sh_degree, backgrounds, image_width,
                                      image_height, tile_size, viewmats0, Ks, scaling_modifier, calc_compensations,
                                      render_alphas, last_ids, tile_offsets, flatten_ids, colors, radii, compensations,
-                                     v_render_colors, v_render_alphas):
+                                     v_render_colors, v_render_alphas, render_mode=0):
     """gsplat/Ops.h:222-270 -> v_means, v_quats, v_scales, v_opacities [1,N], v_sh_coeffs [N,K,3]."""
     scaled = _f32(scales) * np.float32(scaling_modifier) if scaling_modifier != 1.0 else _f32(scales)
     final_op = _f32(opacities).reshape(1, -1)
@@ -352,7 +362,11 @@ def rasterize_from_world_with_sh_bwd(means, quats, scales, opacities, sh_coeffs,
         means, quats, scaled, colors, final_op, backgrounds, None, image_width, image_height, tile_size, viewmats0, Ks,
         tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors, v_render_alphas)
     K = sh_coeffs.shape[1]
-    v_sh = sh_colors_from_world_bwd(sh_degree, means, K, radii[0], viewmats0[0], colors[0], v_colors[0])
+    if render_mode in (0, 3, 4):  # Rasterization.cpp:581-624: the depth channel's gradient is dropped
+        v_sh = sh_colors_from_world_bwd(sh_degree, means, K, radii[0], viewmats0[0],
+                                        np.ascontiguousarray(colors[0][:, :3]), np.ascontiguousarray(v_colors[0][:, :3]))
+    else:
+        v_sh = np.zeros((means.shape[0], K, 3), np.float32)  # :625-629
     if scaling_modifier != 1.0:
         v_scales = v_scales * np.float32(scaling_modifier)
     return v_means, v_quats, v_scales, v_opac, v_sh

@@ -497,3 +497,62 @@ def test_wave_reduce16_probe(gsx, cuda):
     got = N(out)
     assert np.array_equal(got[3], x[3].sum(0))
     np.testing.assert_allclose(got, x.astype(np.float64).sum(1), rtol=0, atol=2e-5)
+
+
+@pytest.mark.parametrize("render_mode", [1, 3, 4])
+def test_depth_render_modes(gsx, orc, cuda, render_mode):
+    """render modes D / RGB_D / RGB_ED of the fused entry (Rasterization.cpp:372-393, 581-629): one or four colour
+    channels whose last one is the camera depth; forward bit-exact, gradients within the usual bars, the depth
+    channel's own gradient is dropped and the SH gradient is zero for depth-only rendering"""
+    ops = gsx.ops
+    sc, cam, h, d = _fused_inputs(gsx, cuda, 6000)
+    ch = 1 if render_mode in (1, 2) else 4
+    bg_h = np.linspace(0.1, 0.4, ch, dtype=np.float32)[None]
+    bg_d = T(bg_h, cuda)
+    ut = ops.UnscentedTransformParameters()
+    ref = orc.rasterize_from_world_with_sh_fwd(h["means"], h["quats"], h["scales"], h["op"], h["shs"], 3, bg_h,
+                                               cam.width, cam.height, 16, h["vm"], h["K"], render_mode=render_mode)
+    got = ops.rasterize_from_world_with_sh_fwd(d["means"], d["quats"], d["scales"], d["op"], d["shs"], 3, bg_d, None,
+                                               cam.width, cam.height, 16, d["vm"], None, d["K"], 0, 0.3, 0.01, 1e4,
+                                               0.0, 1.0, False, render_mode, ut, 4)
+    renders, alphas, radii, means2d, depths, colors, offsets, flat, last_ids, comp = got
+    assert renders.shape[-1] == ch and colors.shape[-1] == ch
+    bits_equal(N(renders), ref[0], "image")
+    bits_equal(N(alphas), ref[1], "alpha")
+    bits_equal(N(last_ids), ref[8], "last ids")
+    vis = ref[2][0, :, 0] > 0
+    bits_equal(N(colors)[0][vis], ref[5][0][vis], "colours incl. depth channel")
+    assert np.abs(ref[0][..., -1]).max() > 1.0  # the depth channel really holds depths
+
+    rng = np.random.default_rng(render_mode)
+    v_img = rng.standard_normal(ref[0].shape).astype(np.float32)
+    v_alpha = rng.standard_normal(ref[1].shape).astype(np.float32)
+    g = ops.rasterize_from_world_with_sh_bwd(d["means"], d["quats"], d["scales"], d["op"], d["shs"], 3, bg_d, None,
+                                             cam.width, cam.height, 16, d["vm"], None, d["K"], 0, 0.3, 0.01, 1e4, 0.0,
+                                             1.0, False, render_mode, ut, 4, None, None, None, alphas, last_ids,
+                                             offsets, flat, colors, radii, means2d, depths, None, T(v_img, cuda),
+                                             T(v_alpha, cuda))
+    colors_ref = ref[5].copy()
+    o = orc.rasterize_from_world_with_sh_bwd(h["means"], h["quats"], h["scales"], h["op"], h["shs"], 3, bg_h,
+                                             cam.width, cam.height, 16, h["vm"], h["K"], 1.0, False, ref[1], ref[8],
+                                             ref[6], ref[7], colors_ref, ref[2], None, v_img, v_alpha,
+                                             render_mode=render_mode)
+    for name, a, b in zip(("v_means", "v_quats", "v_scales", "v_opacities", "v_sh"), g, o):
+        a, b = N(a).reshape(b.shape), b
+        if name == "v_sh" and render_mode in (1, 2):
+            assert np.abs(a).max() == 0.0 and np.abs(b).max() == 0.0
+            continue
+        scale = float(np.abs(b).max())
+        tol = 1e-3 if name in ("v_means", "v_opacities", "v_sh") else 5e-3  # quats / scales: see check_raster_gradients
+        assert np.abs(a - b).max() <= tol * scale, f"{name}: {np.abs(a - b).max()} vs {scale}"
+    # the operator itself returns the gradient of every colour channel
+    gc = ops.rasterize_to_pixels_from_world_3dgs_bwd(d["means"], d["quats"], d["scales"], colors, d["op"][None], bg_d,
+                                                     None, cam.width, cam.height, 16, d["vm"], None, d["K"], 0, ut, 4,
+                                                     None, None, None, offsets, flat, alphas, last_ids,
+                                                     T(v_img, cuda), T(v_alpha, cuda))[3]
+    oc = orc.rasterize_to_pixels_from_world_3dgs_bwd(h["means"], h["quats"], h["scales"], colors_ref, h["op"][None],
+                                                     bg_h, None, cam.width, cam.height, 16, h["vm"], h["K"], ref[6],
+                                                     ref[7], ref[1], ref[8], v_img, v_alpha)[3]
+    assert gc.shape[-1] == ch
+    assert np.abs(N(gc) - oc).max() <= 1e-3 * np.abs(oc).max()
+    assert np.abs(oc[..., -1]).max() > 0

@@ -100,8 +100,8 @@ def test_fused_update_equals_separate_kernels(gsx, cuda, cfg, n, freeze):
         P, A, J, G, V = a2.params, a2.act, a2.proj, a2.grads, a2.v_act
         ws, wsn = _p(a2.ws_bwd), c_sz(a2.ws_bwd.numel())
         check(lb.gsx_rasterize_bwd_finish(c_u32(N_), _p(P["means"]), _p(A["quats"]), _p(A["scales"]), _p(a2.viewmat),
-                                          ws, wsn, c_i(1), _p(G["means"]), _p(V["quats"]), _p(V["scales"]),
-                                          _p(a2.v_colors), _p(V["opacities"]), s))
+                                          ws, wsn, c_i(1), c_u32(3), _p(G["means"]), _p(V["quats"]),
+                                          _p(V["scales"]), _p(a2.v_colors), _p(V["opacities"]), s))
         check(lb.gsx_sh_colors_from_world_bwd(c_u32(N_), c_u32(a2.K), c_u32(a2.sh_degree), _p(P["means"]),
                                               _p(J["radii"]), _p(a2.viewmat), _p(a2.colors), _p(a2.v_colors),
                                               _p(G["shs"]), s))
