@@ -273,14 +273,17 @@ GSX_API int gsx_relocation(int M, const float* opacities, const float* scales, c
  *   new_o, new_s   = relocation(sigmoid(opacity_raw[s]), exp(scaling_raw[s]), ratios)               (:151-156)
  *   opacity_raw[s] = logit(clamp(new_o, min_opacity, 1 - 1e-7)),  scaling_raw[s] = log(new_s)       (:160-171)
  *   parameter rows:        row[dead[i]] = row[sampled[i]]  for every tensor with is_optimizer_state == 0  (:175-180)
- *   optimiser-state rows:  row[sampled[i]] = 0             for every tensor with is_optimizer_state != 0  (:100-104)
+ *   optimiser-state rows:  row[sampled[i]] = 0             for every tensor with is_optimizer_state == 1  (:100-104)
+ * MCMC::add_new_gs (mcmc.cpp:192-347) is the same computation with the "dead" indices being the rows appended to
+ * the (re-allocated, N = old N + n_idx) tensors, except that the moments of the sampled Gaussians are kept and the
+ * new rows' moments are zero: state tensors take is_optimizer_state == 2 (row[dead[i]] = 0) there.
  * sampled_idxs / dead_idxs: i64 [n_idx], disjoint sets, values < N.  opacity_raw [N] and scaling_raw [N,3] must ALSO
  * be listed in tensors_host to have their rows copied to the dead indices. */
 #define GSX_MCMC_MAX_TENSORS 24
 typedef struct gsx_row_tensor {
     float* data;         /* [N, row_floats] */
     uint32_t row_floats; /* floats per Gaussian */
-    int32_t is_optimizer_state;
+    int32_t is_optimizer_state; /* 0 parameter, 1 state cleared at sampled[i], 2 state cleared at dead[i] */
 } gsx_row_tensor;
 GSX_API size_t gsx_mcmc_relocate_workspace_bytes(uint32_t N, uint32_t n_idx);
 GSX_API int gsx_mcmc_relocate(uint32_t N, uint32_t n_idx, const int64_t* sampled_idxs, const int64_t* dead_idxs,
@@ -312,6 +315,16 @@ GSX_API int gsx_activate_params_bwd(uint32_t N, const float* opacity_raw, const 
                                     const float* rotation_raw, const float* v_opacities, const float* v_scales,
                                     const float* v_quats, float* v_opacity_raw, float* v_scaling_raw,
                                     float* v_rotation_raw, void* stream);
+/* ---- scale / opacity L1 regularisation (include/kernels/regularization.cuh:12-48; regularization.cu:20-289;
+ * trainer.cpp:136-174) ----  loss = weight * mean(f(params)), f = exp (scaling_raw) / sigmoid (opacity_raw);
+ * param_grads (nullable) += (weight / n) f'(params).  partials: gsx_l1_regularization_partials() floats of scratch;
+ * loss_out: one float in DEVICE memory (the reference blocks on a cudaMemcpy of it per call).  weight == 0: no-op. */
+GSX_API uint32_t gsx_l1_regularization_partials(void);
+GSX_API int gsx_exp_l1_regularization(const float* params, float* param_grads, int64_t n, float weight,
+                                      float* partials, float* loss_out, void* stream);
+GSX_API int gsx_sigmoid_l1_regularization(const float* params, float* param_grads, int64_t n, float weight,
+                                          float* partials, float* loss_out, void* stream);
+
 /* The tail of a training step in ONE pass over the Gaussians (no counterpart in the reference, which runs them as
  * separate kernels and ATen ops): rasterizer-backward epilogue (as gsx_rasterize_bwd_finish with
  * clear_accumulators = 1, on the ACTIVATIONS of the raw parameters) -> SH backward with the clamp mask (as
@@ -331,6 +344,9 @@ typedef struct gsx_update_args {
     float lr_means, lr_sh0, lr_shN, lr_scaling, lr_rotation, lr_opacity;
     float beta1, beta2, eps, bias_correction1_rcp, bias_correction2_sqrt_rcp;
     int32_t skip_shN;      /* fused_adam.cpp:69-70 */
+    /* regularisation gradients folded in: scaling grad += reg_scaling * exp(scaling_raw), opacity grad +=
+     * reg_opacity * s (1 - s); reg_* = weight / element count as in gsx_*_l1_regularization (0 = off) */
+    float reg_scaling, reg_opacity;
 } gsx_update_args;
 GSX_API int gsx_backward_update_fused(const gsx_update_args* args_host, void* stream);
 

@@ -60,7 +60,7 @@ class UpdateArgs(ctypes.Structure):
                 [(n, c_f) for n in ("lr_means", "lr_sh0", "lr_shN", "lr_scaling", "lr_rotation", "lr_opacity",
                                     "beta1", "beta2", "eps", "bias_correction1_rcp",
                                     "bias_correction2_sqrt_rcp")] +
-                [("skip_shN", ctypes.c_int32)])
+                [("skip_shN", ctypes.c_int32), ("reg_scaling", c_f), ("reg_opacity", c_f)])
 
 
 class GsxError(RuntimeError):
@@ -85,6 +85,7 @@ def lib():
         L.gsx_n_bits.restype = c_u32
         L.gsx_image_loss_blocks.restype = c_u32
         L.gsx_photometric_partials.restype = c_u32
+        L.gsx_l1_regularization_partials.restype = c_u32
         L.gsx_ut_defaults.restype = UTParams
         for name in ("gsx_intersect_tile_count_workspace_bytes", "gsx_radix_sort_pairs_workspace_bytes",
                      "gsx_rasterize_bwd_workspace_bytes", "gsx_mcmc_relocate_workspace_bytes",

@@ -104,8 +104,10 @@ __global__ void __launch_bounds__(256) mcmc_rows_kernel(uint32_t n, const int64_
     const uint32_t i = (uint32_t)(t / r), f = (uint32_t)(t % r);
     float* __restrict__ p = tab.data[e];
     const int64_t s = sampled[i];
-    if (tab.is_state[e])
-        p[s * r + f] = 0.f;
+    if (tab.is_state[e] == 1u)
+        p[s * r + f] = 0.f; // relocate_gs: moments of the sampled Gaussian restart
+    else if (tab.is_state[e] == 2u)
+        p[dead[i] * r + f] = 0.f; // add_new_gs: moments of the new row start at zero
     else
         p[dead[i] * r + f] = p[s * r + f];
 }
@@ -192,11 +194,12 @@ extern "C" int gsx_mcmc_relocate(uint32_t N, uint32_t n_idx, const int64_t* samp
     memset(&tab, 0, sizeof(tab));
     uint32_t max_row = 0;
     for (int e = 0; e < n_tensors; ++e) {
-        GSX_REQUIRE(tensors_host[e].data && tensors_host[e].row_floats > 0, GSX_ERR_INVALID_ARGUMENT,
-                    "mcmc_relocate: tensor %d is null or has empty rows", e);
+        GSX_REQUIRE(tensors_host[e].data && tensors_host[e].row_floats > 0 &&
+                        tensors_host[e].is_optimizer_state >= 0 && tensors_host[e].is_optimizer_state <= 2,
+                    GSX_ERR_INVALID_ARGUMENT, "mcmc_relocate: tensor %d is null, has empty rows or a bad role", e);
         tab.data[e] = tensors_host[e].data;
         tab.row_floats[e] = tensors_host[e].row_floats;
-        tab.is_state[e] = tensors_host[e].is_optimizer_state ? 1u : 0u;
+        tab.is_state[e] = (uint32_t)tensors_host[e].is_optimizer_state;
         max_row = tensors_host[e].row_floats > max_row ? tensors_host[e].row_floats : max_row;
     }
     char* ws = (char*)workspace;

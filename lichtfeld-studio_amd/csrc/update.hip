@@ -27,6 +27,7 @@ struct UpdateArgs {
     float lr_means, lr_sh0, lr_shN, lr_scaling, lr_rotation, lr_opacity;
     float beta1, beta2, eps, bc1_rcp, bc2_sqrt_rcp;
     int32_t skip_shN;
+    float reg_scaling, reg_opacity;
 };
 
 // new first / second moment of one element (the first two lines of adam_one)
@@ -97,11 +98,20 @@ __global__ void __launch_bounds__(256) backward_update_kernel(const UpdateArgs a
         }
         // ---- Adam on the small tensors ----
         adam_row<3>(a.means, a.m_means, a.v_means, e, vm, a.lr_means, a);
-        const float gs[3] = {av.scaling.x, av.scaling.y, av.scaling.z};
+        float gs[3] = {av.scaling.x, av.scaling.y, av.scaling.z};
+        float go[1] = {av.opacity};
+        if (a.reg_scaling != 0.f) { // += (w / n) exp(x), as the regularisation kernel adds it to the finished gradient
+            gs[0] += a.reg_scaling * gsx::exp(s_raw.x);
+            gs[1] += a.reg_scaling * gsx::exp(s_raw.y);
+            gs[2] += a.reg_scaling * gsx::exp(s_raw.z);
+        }
+        if (a.reg_opacity != 0.f) {
+            const float sg = gsx::sigmoid(o_raw);
+            go[0] += a.reg_opacity * (sg * (1.0f - sg));
+        }
         adam_row<3>(a.scaling_raw, a.m_scaling, a.v_scaling, e, gs, a.lr_scaling, a);
         const float gr[4] = {av.rotation.w, av.rotation.x, av.rotation.y, av.rotation.z};
         adam_row<4>(a.rotation_raw, a.m_rotation, a.v_rotation, e, gr, a.lr_rotation, a);
-        const float go[1] = {av.opacity};
         adam_row<1>(a.opacity_raw, a.m_opacity, a.v_opacity, e, go, a.lr_opacity, a);
     }
 
@@ -232,6 +242,7 @@ extern "C" int gsx_backward_update_fused(const gsx_update_args* args, void* stre
     a.beta1 = args->beta1, a.beta2 = args->beta2, a.eps = args->eps;
     a.bc1_rcp = args->bias_correction1_rcp, a.bc2_sqrt_rcp = args->bias_correction2_sqrt_rcp;
     a.skip_shN = args->skip_shN;
+    a.reg_scaling = args->reg_scaling, a.reg_opacity = args->reg_opacity;
     const bool lds16 = a.K == 16 && ((((uintptr_t)a.shs) | ((uintptr_t)a.m_shs) | ((uintptr_t)a.v_shs)) & 15u) == 0;
     const dim3 grid(cdiv(a.N, 256)), block(256);
     if (lds16)

@@ -27,7 +27,8 @@ def _p(t):
 
 class TrainStep:
     def __init__(self, scene, device="cuda:0", lrs=None, lambda_dssim=0.2, betas=(0.9, 0.999), eps=1e-15,
-                 scene_scale=1.0, sh_degree=None, use_ssim=True, fused_update=False, fused_loss=False):
+                 scene_scale=1.0, sh_degree=None, use_ssim=True, fused_update=False, fused_loss=False,
+                 scale_reg=0.0, opacity_reg=0.0):
         self.dev = torch.device(device)
         self.lib = lib()
         f = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(self.dev)
@@ -55,7 +56,21 @@ class TrainStep:
         # True (needs use_ssim): the loss runs as two kernels and neither the clamped image nor the SSIM map exist
         self.fused_loss = fused_loss and use_ssim
         self.ut = UTParams()
-        N = self.N
+        # trainer.cpp:136-174 (weights of the L1 terms on exp(scaling_raw) and sigmoid(opacity_raw); 0 = off)
+        self.scale_reg, self.opacity_reg = float(scale_reg), float(opacity_reg)
+        self.reg_partials = torch.empty(self.lib.gsx_l1_regularization_partials(), dtype=torch.float32,
+                                        device=self.dev)
+        self.reg_losses = torch.zeros(2, dtype=torch.float32, device=self.dev)  # [scale term, opacity term]
+        self._allocate_per_gaussian(self.N)
+        self.cap = 0
+        self.img_shape = None
+        self.n_isects = 0
+        self.bg = torch.zeros((1, 3), dtype=torch.float32, device=self.dev)  # trainer.cpp:383-384
+        self.loss_out = torch.empty(3, dtype=torch.float32, device=self.dev)
+
+    def _allocate_per_gaussian(self, N):
+        """every buffer whose size follows the number of Gaussians"""
+        self.N = N
         e = lambda *s, dt=torch.float32: torch.empty(s, dtype=dt, device=self.dev)
         self.act = dict(opacities=e(N), scales=e(N, 3), quats=e(N, 4))
         self.v_act = dict(opacities=e(N), scales=e(N, 3), quats=e(N, 4))
@@ -71,11 +86,6 @@ class TrainStep:
         self.ws_bwd = torch.zeros(self.lib.gsx_rasterize_bwd_accum_bytes(c_u32(N)), dtype=torch.uint8,
                                   device=self.dev)  # the backward's epilogue leaves it zeroed for the next pass
         self.records = e(self.lib.gsx_raster_records_bytes(c_u32(N)), dt=torch.uint8)
-        self.cap = 0
-        self.img_shape = None
-        self.n_isects = 0
-        self.bg = torch.zeros((1, 3), dtype=torch.float32, device=self.dev)  # trainer.cpp:383-384
-        self.loss_out = e(3)
 
     # -- buffers that depend on n_isects / image size --------------------------------------------
     def _ensure_isect_capacity(self, n):
@@ -250,6 +260,23 @@ class TrainStep:
         self._run("activate_params_bwd", lb.gsx_activate_params_bwd, c_u32(N), _p(P["opacity"]), _p(P["scaling"]), _p(P["rotation"]),
                                          _p(V["opacities"]), _p(V["scales"]), _p(V["quats"]), _p(G["opacity"]),
                                          _p(G["scaling"]), _p(G["rotation"]), s)
+        self.regularization_losses(with_grads=True)
+
+    def regularization_losses(self, with_grads=False):
+        """Trainer::compute_scale_reg_loss / compute_opacity_reg_loss (trainer.cpp:136-174): the two loss values land
+        in self.reg_losses (device); with_grads adds their gradients onto self.grads (the fused update adds them
+        itself and only needs this call when the loss values are wanted)."""
+        s = self._stream()
+        P, G = self.params, self.grads
+        if self.scale_reg > 0.0:
+            self._run("exp_l1_regularization", self.lib.gsx_exp_l1_regularization, _p(P["scaling"]),
+                      _p(G["scaling"]) if with_grads else c_p(None), c_i64(P["scaling"].numel()),
+                      c_f(self.scale_reg), _p(self.reg_partials), c_p(self.reg_losses.data_ptr()), s)
+        if self.opacity_reg > 0.0:
+            self._run("sigmoid_l1_regularization", self.lib.gsx_sigmoid_l1_regularization, _p(P["opacity"]),
+                      _p(G["opacity"]) if with_grads else c_p(None), c_i64(P["opacity"].numel()),
+                      c_f(self.opacity_reg), _p(self.reg_partials), c_p(self.reg_losses.data_ptr() + 4), s)
+        return self.reg_losses
 
     # -- optimiser ------------------------------------------------------------------------------------
     def adam(self):
@@ -270,7 +297,10 @@ class TrainStep:
                 V["means"].data_ptr(), V["opacity"].data_ptr(), V["scaling"].data_ptr(), V["rotation"].data_ptr(),
                 V["shs"].data_ptr(), self.proj["radii"].data_ptr(), self.colors.data_ptr(), self.viewmat.data_ptr(),
                 self.ws_bwd.data_ptr(), self.lrs["means"], self.lrs["sh0"], self.lrs["shN"], self.lrs["scaling"],
-                self.lrs["rotation"], self.lrs["opacity"], b1, b2, self.eps, bc1, bc2, skip)
+                self.lrs["rotation"], self.lrs["opacity"], b1, b2, self.eps, bc1, bc2, skip,
+                # weight / element count in float32, as the separate regularisation kernels form it
+                float(np.float32(self.scale_reg) / np.float32(3 * self.N)) if self.scale_reg > 0.0 else 0.0,
+                float(np.float32(self.opacity_reg) / np.float32(self.N)) if self.opacity_reg > 0.0 else 0.0)
             self._run("backward_update_fused", self.lib.gsx_backward_update_fused, ctypes.byref(a), self._stream())
             return
         names = ["means", "shs", "scaling", "rotation", "opacity"]
@@ -291,7 +321,22 @@ class TrainStep:
     freeze_shN_early = False  # BASELINE's step updates all parameter tensors; set True for the product schedule
 
     # -- MCMC strategy steps that touch the parameters ------------------------------------------------
-    def relocate(self, sampled_idxs, dead_idxs, binoms, min_opacity=0.005):
+    def add_new_gs(self, sampled_idxs, binoms, min_opacity=0.005):
+        """MCMC::add_new_gs (mcmc.cpp:192-347) for sampled sources chosen by the caller: the tensors grow by
+        len(sampled_idxs) rows (copies of the sampled Gaussians after the Eq. 9 rebalancing, zero moments)."""
+        n_new = int(sampled_idxs.numel())
+        if n_new == 0:
+            return 0
+        old_n = self.N
+        grow = lambda t: torch.cat([t, torch.zeros((n_new,) + tuple(t.shape[1:]), dtype=t.dtype, device=t.device)])
+        for d in (self.params, self.exp_avg, self.exp_avg_sq, self.grads):
+            for k in d:
+                d[k] = grow(d[k])
+        self._allocate_per_gaussian(old_n + n_new)
+        new_rows = torch.arange(old_n, old_n + n_new, dtype=torch.int64, device=self.dev)
+        return self.relocate(sampled_idxs, new_rows, binoms, min_opacity, state_role=2)
+
+    def relocate(self, sampled_idxs, dead_idxs, binoms, min_opacity=0.005, state_role=1):
         """MCMC::relocate_gs (mcmc.cpp:112-190) for index sets chosen by the caller (the multinomial draw of :132 is
         the caller's): sampled Gaussians get the Eq. 9 opacity / scales, dead ones become copies of them, the Adam
         moments of the sampled ones are cleared.  sampled_idxs / dead_idxs: int64 device tensors of equal length."""
@@ -301,7 +346,7 @@ class TrainStep:
             return 0
         names = ["means", "shs", "scaling", "rotation", "opacity"]
         tensors = [(self.params[k], 0) for k in names]
-        tensors += [(self.exp_avg[k], 1) for k in names] + [(self.exp_avg_sq[k], 1) for k in names]
+        tensors += [(self.exp_avg[k], state_role) for k in names] + [(self.exp_avg_sq[k], state_role) for k in names]
         arr = (L.RowTensor * len(tensors))()
         for i, (t, is_state) in enumerate(tensors):
             arr[i] = L.RowTensor(t.data_ptr(), t.numel() // self.N, is_state)

@@ -1453,6 +1453,30 @@ ORC_API int orc_activate_params(uint32_t N, const float* opacity_raw, const floa
     return 0;
 }
 
+// regularization.cu:20-57 (exp) / 60-90 (sigmoid): loss = weight * mean(f(x)); grads += (weight / n) f'(x).
+// mode 0: f = exp; mode 1: f = sigmoid.  The sum is taken in double (the kernels' block order is not part of the
+// contract; the loss value is compared with a tolerance, the gradients bit for bit).
+ORC_API double orc_l1_regularization(int mode, const float* params, float* grads, int64_t n, float weight) {
+    if (weight == 0.0f || n <= 0)
+        return 0.0;
+    const float grad_scale = weight / (float)n;
+    double sum = 0.0;
+    for (int64_t i = 0; i < n; ++i) {
+        float value, deriv;
+        if (mode == 0) {
+            value = gsx::exp(params[i]);
+            deriv = value;
+        } else {
+            value = gsx::sigmoid(params[i]);
+            deriv = value * (1.0f - value);
+        }
+        sum += (double)value;
+        if (grads)
+            grads[i] += grad_scale * deriv;
+    }
+    return (double)weight * (sum / (double)n);
+}
+
 ORC_API int orc_activate_params_bwd(uint32_t N, const float* opacity_raw, const float* scaling_raw,
                                     const float* rotation_raw, const float* v_opacities, const float* v_scales,
                                     const float* v_quats, float* v_opacity_raw, float* v_scaling_raw,

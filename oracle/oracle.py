@@ -392,6 +392,18 @@ def activate_params_bwd(opacity_raw, scaling_raw, rotation_raw, v_opacities, v_s
     return vo, vs, vr
 
 
+def l1_regularization(mode, params, grads, weight):
+    """regularization.cu:20-90: mode "exp" (scaling_raw) or "sigmoid" (opacity_raw); grads (float32 array of the same
+    size, or None) is updated in place; returns the loss value weight * mean(f(params))."""
+    x = _f32(params).reshape(-1)
+    if grads is not None:
+        assert grads.dtype == np.float32 and grads.flags.c_contiguous and grads.size == x.size
+    f = lib().orc_l1_regularization
+    f.restype = ctypes.c_double
+    return float(f(c_i(0 if mode == "exp" else 1), _p(x), _p(grads) if grads is not None else None,
+                   ctypes.c_int64(x.size), ctypes.c_float(weight)))
+
+
 def photometric_loss(render_hwc, gt_chw, lambda_dssim, with_grad=True):
     """trainer.cpp:126-129 on clamp(render) -> (loss, l1, ssim, image [3,H,W], v_render [H,W,3] or None)"""
     render_hwc, gt_chw = _f32(render_hwc), _f32(gt_chw)

@@ -13,7 +13,8 @@ DEFAULT_LRS = dict(means=1.6e-4, sh0=2.5e-3, shN=2.5e-3 / 20.0, scaling=5e-3, ro
 
 
 class OracleTrainStep:
-    def __init__(self, scene, lrs=None, lambda_dssim=0.2, betas=(0.9, 0.999), eps=1e-15, sh_degree=None):
+    def __init__(self, scene, lrs=None, lambda_dssim=0.2, betas=(0.9, 0.999), eps=1e-15, sh_degree=None,
+                 scale_reg=0.0, opacity_reg=0.0):
         c = lambda a: np.ascontiguousarray(a, dtype=np.float32).copy()
         self.params = dict(means=c(scene.means), shs=c(np.concatenate([scene.sh0, scene.shN], 1)),
                            scaling=c(scene.scaling_raw), rotation=c(scene.rotation_raw),
@@ -25,6 +26,7 @@ class OracleTrainStep:
         self.lrs = dict(DEFAULT_LRS, **(lrs or {}))
         self.lambda_dssim, self.betas, self.eps = lambda_dssim, betas, eps
         self.step_count = 0
+        self.scale_reg, self.opacity_reg = scale_reg, opacity_reg
         self.bg = np.zeros((1, 3), np.float32)
 
     def forward(self, viewmat, K, W, H):
@@ -50,6 +52,10 @@ class OracleTrainStep:
         g_op, g_sc, g_rot = orc.activate_params_bwd(P["opacity"], P["scaling"], P["rotation"], v_op, v_scales,
                                                     v_quats)
         self.grads = dict(means=v_means, shs=v_sh, scaling=g_sc, rotation=g_rot, opacity=g_op)
+        # trainer.cpp:136-174: the two L1 terms add their gradients onto the finished ones
+        self.reg_losses = (orc.l1_regularization("exp", P["scaling"], g_sc, self.scale_reg) if self.scale_reg > 0 else 0.0,
+                           orc.l1_regularization("sigmoid", P["opacity"], g_op, self.opacity_reg)
+                           if self.opacity_reg > 0 else 0.0)
         return loss
 
     def adam(self):
@@ -92,6 +98,27 @@ class OracleTrainStep:
         for k in P:                                                                # :100-104
             self.exp_avg[k][sampled_idxs] = 0
             self.exp_avg_sq[k][sampled_idxs] = 0
+        return sampled_idxs.size
+
+    def add_new_gs(self, sampled_idxs, binoms, min_opacity=0.005):
+        """MCMC::add_new_gs (mcmc.cpp:192-347) line by line, with the caller's sampled sources."""
+        P = self.params
+        n_max = binoms.shape[0]
+        if sampled_idxs.size == 0:
+            return 0
+        op, scales, _ = orc.activate_params(P["opacity"], P["scaling"], P["rotation"])
+        ratios = np.zeros(op.shape[0], np.float32)                                 # :217
+        np.add.at(ratios, sampled_idxs, 1.0)                                       # :218
+        ratios = np.clip(ratios[sampled_idxs] + 1, 1, n_max).astype(np.int32)      # :219-224
+        new_op, new_sc = orc.relocation(op[sampled_idxs], scales[sampled_idxs], ratios, binoms, n_max)
+        new_op = np.clip(new_op, np.float32(min_opacity), np.float32(1.0 - 1e-7))  # :236
+        P["opacity"][sampled_idxs] = orc.math_unary("log", new_op / (np.float32(1.0) - new_op))
+        P["scaling"][sampled_idxs] = orc.math_unary("log", new_sc.reshape(-1)).reshape(-1, 3)
+        for k in list(P):                                                          # :247-260, 285-291
+            P[k] = np.ascontiguousarray(np.concatenate([P[k], P[k][sampled_idxs]], 0))
+            zeros = np.zeros((sampled_idxs.size,) + P[k].shape[1:], np.float32)
+            self.exp_avg[k] = np.ascontiguousarray(np.concatenate([self.exp_avg[k], zeros], 0))
+            self.exp_avg_sq[k] = np.ascontiguousarray(np.concatenate([self.exp_avg_sq[k], zeros], 0))
         return sampled_idxs.size
 
     def inject_noise(self, noise, noise_lr=5e5):

@@ -199,3 +199,38 @@ def test_config5_literal_scales_overflow_is_reported(gsx, cuda):
     with pytest.raises(gsx._lib.GsxError, match="do not fit int32") as e:
         ts.forward(T(cam.viewmat[None], cuda), T(cam.K[None], cuda), cam.width, cam.height)
     assert e.value.status == -5
+
+
+def test_mcmc_add_new_gs_bit_exact(gsx, orc, cuda):
+    """MCMC::add_new_gs: 5 % growth from identical parameters on both sides (sampled sources given to both): the grown
+    parameter and moment tensors are bit-identical, and a training step runs on the grown state"""
+    from lichtfeld_studio_amd.trainer import TrainStep
+    from oracle.step import OracleTrainStep
+    sc = gsx.scenes.config(3, 100_000)
+    sc.scaling_raw += 0.8
+    cam = gsx.scenes.orbit_camera(0.7, 4.0, 309, 205, 287.0)
+    ts, ref = TrainStep(sc, cuda), OracleTrainStep(sc)
+    rng = np.random.default_rng(17)
+    for k in ts.params:
+        m = rng.standard_normal(ref.exp_avg[k].shape).astype(np.float32)
+        ref.exp_avg[k][...] = m
+        ref.exp_avg_sq[k][...] = m * m
+        ts.exp_avg[k].copy_(T(m, cuda))
+        ts.exp_avg_sq[k].copy_(T(m * m, cuda))
+    n_new = ts.N // 20
+    sampled = rng.integers(0, 2000, n_new).astype(np.int64)  # few sources: ratios up to the clamp
+    b = binoms(51)
+    ts.add_new_gs(T(sampled, cuda), T(b, cuda))
+    ref.add_new_gs(sampled, b)
+    torch.cuda.synchronize()
+    assert ts.N == 105_000
+    for k in ts.params:
+        assert np.array_equal(N(ts.params[k]).view(np.uint32), ref.params[k].view(np.uint32)), k
+        assert np.array_equal(N(ts.exp_avg[k]).view(np.uint32), ref.exp_avg[k].view(np.uint32)), k
+        assert np.array_equal(N(ts.exp_avg_sq[k]).view(np.uint32), ref.exp_avg_sq[k].view(np.uint32)), k
+    vm, Km = T(cam.viewmat[None], cuda), T(cam.K[None], cuda)
+    gt = torch.rand((1, 3, cam.height, cam.width), generator=torch.Generator().manual_seed(1)).to(cuda)
+    ts.step(vm, Km, cam.width, cam.height, gt)
+    ref.step(cam.viewmat, cam.K, cam.width, cam.height, N(gt)[0])
+    torch.cuda.synchronize()
+    check_forward_bit_exact(ts, ref, min_isects=10_000)

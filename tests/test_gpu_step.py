@@ -10,8 +10,9 @@ torch = pytest.importorskip("torch")
 from step_checks import check_first_step, check_forward_bit_exact, check_loss, check_params_close  # noqa: E402
 
 
-@pytest.mark.parametrize("cfg,n,use_ssim", [(1, 10_000, False), (3, 30_000, True)])
-def test_train_step_matches_oracle(gsx, orc, cuda, cfg, n, use_ssim):
+@pytest.mark.parametrize("cfg,n,use_ssim,reg", [(1, 10_000, False, 0.0), (3, 30_000, True, 0.0),
+                                                (3, 20_000, True, 0.01)])
+def test_train_step_matches_oracle(gsx, orc, cuda, cfg, n, use_ssim, reg):
     from lichtfeld_studio_amd.trainer import TrainStep
     from oracle.step import OracleTrainStep
     sc = gsx.scenes.config(cfg, n)
@@ -29,8 +30,9 @@ def test_train_step_matches_oracle(gsx, orc, cuda, cfg, n, use_ssim):
     else:
         tg = OracleTrainStep(sc.target_scene)
         gt = np.ascontiguousarray(np.clip(tg.forward(cam.viewmat, cam.K, W, H)[0], 0, 1).transpose(2, 0, 1))
-    ts = TrainStep(sc, cuda, use_ssim=use_ssim)
-    ref = OracleTrainStep(sc, lambda_dssim=0.2 if use_ssim else 0.0)
+    # reg: the MCMC defaults of the scale / opacity L1 terms (trainer.cpp:136-174)
+    ts = TrainStep(sc, cuda, use_ssim=use_ssim, scale_reg=reg, opacity_reg=reg)
+    ref = OracleTrainStep(sc, lambda_dssim=0.2 if use_ssim else 0.0, scale_reg=reg, opacity_reg=reg)
     gt_d = torch.from_numpy(gt[None].copy()).to(cuda)
 
     for it in range(2):
@@ -41,6 +43,12 @@ def test_train_step_matches_oracle(gsx, orc, cuda, cfg, n, use_ssim):
             check_forward_bit_exact(ts, ref)
             check_loss(ts, ref)
             check_first_step(ts, ref)
+            if reg:
+                # loss values of the two terms on the updated parameters (which agree to the Adam tolerance)
+                got = [float(x) for x in ts.regularization_losses().cpu()]
+                want = [orc.l1_regularization("exp", ref.params["scaling"], None, reg),
+                        orc.l1_regularization("sigmoid", ref.params["opacity"], None, reg)]
+                assert np.allclose(got, want, rtol=1e-4, atol=0), (got, want)
         else:
             # the second iteration starts from parameters that already differ in the last bits (Adam state is only
             # toleranced), so a few alpha-threshold decisions may differ: loss and parameters are compared, the
@@ -50,11 +58,13 @@ def test_train_step_matches_oracle(gsx, orc, cuda, cfg, n, use_ssim):
             check_params_close(ts, ref, 2, 5e-3)
 
 
-@pytest.mark.parametrize("cfg,n,freeze", [(1, 10_000, False), (3, 30_000, False), (3, 30_001, True)])
-def test_fused_update_equals_separate_kernels(gsx, cuda, cfg, n, freeze):
+@pytest.mark.parametrize("cfg,n,freeze,reg", [(1, 10_000, False, 0.0), (3, 30_000, False, 0.0),
+                                              (3, 30_001, True, 0.0), (3, 20_003, False, 0.01)])
+def test_fused_update_equals_separate_kernels(gsx, cuda, cfg, n, freeze, reg):
     """epilogue + SH backward + activation VJPs + Adam in one pass (gsx_backward_update_fused) leaves parameters and
     both moments bit-identical to the separate kernels, over three iterations (K = 1 and K = 16 paths, with and
-    without the frozen shN group, a Gaussian count that is not a multiple of the block size)"""
+    without the frozen shN group, a Gaussian count that is not a multiple of the block size, with the scale / opacity
+    regularisation gradients folded in)"""
     from lichtfeld_studio_amd.trainer import TrainStep
     sc = gsx.scenes.config(cfg, n)
     if cfg == 3:
@@ -65,8 +75,8 @@ def test_fused_update_equals_separate_kernels(gsx, cuda, cfg, n, freeze):
     vm = torch.from_numpy(cam.viewmat[None].copy()).to(cuda)
     Km = torch.from_numpy(cam.K[None].copy()).to(cuda)
     gt = torch.rand((1, 3, H, W), generator=torch.Generator().manual_seed(3)).to(cuda)
-    a = TrainStep(sc, cuda, use_ssim=cfg != 1, fused_update=False)
-    b = TrainStep(sc, cuda, use_ssim=cfg != 1, fused_update=True)
+    a = TrainStep(sc, cuda, use_ssim=cfg != 1, fused_update=False, scale_reg=reg, opacity_reg=reg)
+    b = TrainStep(sc, cuda, use_ssim=cfg != 1, fused_update=True, scale_reg=reg, opacity_reg=reg)
     a.freeze_shN_early = b.freeze_shN_early = freeze
     for it in range(3):
         a.step(vm, Km, W, H, gt)
@@ -79,8 +89,8 @@ def test_fused_update_equals_separate_kernels(gsx, cuda, cfg, n, freeze):
                 d = (a.params[k] - b.params[k]).abs().max().item()
                 assert d <= 2.1 * max(a.lrs.values()), k
     # exact comparison of the two tails on identical inputs
-    a2 = TrainStep(sc, cuda, use_ssim=cfg != 1, fused_update=False)
-    b2 = TrainStep(sc, cuda, use_ssim=cfg != 1, fused_update=True)
+    a2 = TrainStep(sc, cuda, use_ssim=cfg != 1, fused_update=False, scale_reg=reg, opacity_reg=reg)
+    b2 = TrainStep(sc, cuda, use_ssim=cfg != 1, fused_update=True, scale_reg=reg, opacity_reg=reg)
     a2.freeze_shN_early = b2.freeze_shN_early = freeze
     for it in range(2):
         for ts in (a2, b2):
@@ -108,6 +118,7 @@ def test_fused_update_equals_separate_kernels(gsx, cuda, cfg, n, freeze):
         check(lb.gsx_activate_params_bwd(c_u32(N_), _p(P["opacity"]), _p(P["scaling"]), _p(P["rotation"]),
                                          _p(V["opacities"]), _p(V["scales"]), _p(V["quats"]), _p(G["opacity"]),
                                          _p(G["scaling"]), _p(G["rotation"]), s))
+        a2.regularization_losses(with_grads=True)
         a2.adam()
         b2.adam()
         torch.cuda.synchronize()
@@ -146,3 +157,38 @@ def test_fused_loss_equals_separate_kernels(gsx, cuda, W, H):
     assert (va != 0).mean() > 0.3
     assert np.abs(va - vb).max() <= 1e-6 * np.abs(va).max()
     assert np.array_equal(va == 0, vb == 0)  # the clamp mask
+
+
+@pytest.mark.parametrize("n", [1, 255, 300_001, 3_000_000])
+def test_l1_regularization_kernels(gsx, orc, cuda, n):
+    """gsx_exp_l1_regularization / gsx_sigmoid_l1_regularization: gradients added onto existing ones bit for bit as
+    the checker adds them, loss = weight * mean to 2e-6 relative (summation order differs); without a gradient
+    tensor only the loss is produced; weight 0 touches nothing"""
+    from lichtfeld_studio_amd._lib import c_f, c_i64, c_p, check, lib
+    L = lib()
+    rng = np.random.default_rng(n)
+    x = rng.normal(-2.0, 2.0, n).astype(np.float32)
+    g0 = rng.normal(0, 1e-3, n).astype(np.float32)
+    xd = torch.from_numpy(x).to(cuda)
+    partials = torch.empty(L.gsx_l1_regularization_partials(), dtype=torch.float32, device=cuda)
+    s = c_p(torch.cuda.current_stream(cuda).cuda_stream)
+    for mode, fn in (("exp", L.gsx_exp_l1_regularization), ("sigmoid", L.gsx_sigmoid_l1_regularization)):
+        want_g = g0.copy()
+        want_loss = orc.l1_regularization(mode, x, want_g, 0.01)
+        gd = torch.from_numpy(g0).to(cuda)
+        out = torch.full((2,), -7.0, dtype=torch.float32, device=cuda)
+        check(fn(c_p(xd.data_ptr()), c_p(gd.data_ptr()), c_i64(n), c_f(0.01), c_p(partials.data_ptr()),
+                 c_p(out.data_ptr()), s))
+        check(fn(c_p(xd.data_ptr()), c_p(None), c_i64(n), c_f(0.01), c_p(partials.data_ptr()),
+                 c_p(out.data_ptr() + 4), s))
+        torch.cuda.synchronize()
+        assert np.array_equal(gd.cpu().numpy().view(np.int32), want_g.view(np.int32)), mode
+        got = out.cpu().numpy()
+        assert got[0] == got[1]
+        assert abs(got[0] - want_loss) <= 2e-6 * abs(want_loss), (mode, got, want_loss)
+        before = gd.clone()
+        out.fill_(-7.0)
+        check(fn(c_p(xd.data_ptr()), c_p(gd.data_ptr()), c_i64(n), c_f(0.0), c_p(partials.data_ptr()),
+                 c_p(out.data_ptr()), s))
+        torch.cuda.synchronize()
+        assert torch.equal(before, gd) and float(out[0]) == -7.0

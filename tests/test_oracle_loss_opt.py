@@ -215,3 +215,25 @@ def test_photometric_loss_against_torch(orc):
     inside = (render >= 0) & (render <= 1)
     np.testing.assert_allclose(v0[inside], (np.sign(np.clip(render, 0, 1) - gt.transpose(1, 2, 0)) / (3 * H * W))[inside],
                                rtol=1e-6)
+
+
+def test_l1_regularization_matches_autograd(orc):
+    """regularization.cu:20-90 pinned by autograd of the definition: loss = w mean(exp(x)) resp. w mean(sigmoid(x)),
+    gradients ADDED onto what the tensor already holds (a dropped 1/n, a missing chain-rule factor or an overwrite
+    instead of an accumulation fails)"""
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(5)
+    x = rng.normal(-1.0, 1.5, (4001, 3)).astype(np.float32)
+    g0 = rng.normal(0, 1e-4, x.shape).astype(np.float32)
+    for mode, f in (("exp", torch.exp), ("sigmoid", torch.sigmoid)):
+        t = torch.from_numpy(x.astype(np.float64)).requires_grad_(True)
+        loss = 0.013 * f(t).mean()
+        loss.backward()
+        g = g0.copy()
+        got = orc.l1_regularization(mode, x, g, 0.013)
+        assert abs(got - loss.item()) <= 1e-6 * loss.item()
+        want = g0.astype(np.float64) + t.grad.numpy()
+        assert np.abs(g - want).max() <= 2e-6 * np.abs(want).max()
+        assert orc.l1_regularization(mode, x, None, 0.013) == got
+        g2 = g0.copy()
+        assert orc.l1_regularization(mode, x, g2, 0.0) == 0.0 and np.array_equal(g2, g0)
