@@ -383,6 +383,43 @@ GSX_API int gsx_render_grad_from_loss(uint32_t H, uint32_t W, float lambda_dssim
                                       const float* image_chw, const float* gt_chw, const float* dL_dimg_ssim,
                                       float* v_render_hwc, void* stream);
 
+/* ---- trained model on disk: binary little-endian PLY, one float32 row per Gaussian ----
+ * writer: SplatData::save_ply / to_point_cloud / get_attribute_names / write_ply_impl (src/core/splat_data.cpp:
+ * 113-169, 402-418, 484-506); reader: load_ply / parse_header / extract_* (src/loader/formats/ply.cpp:185-323,
+ * 446-496, 500-637).  Row of the writer (gsx_ply_row_floats(K) = 14 + 3K floats): x y z nx ny nz f_dc_0..2
+ * f_rest_0..3(K-1)-1 opacity scale_0..2 rot_0..3 with normals 0, f_rest channel-major (all R, then G, then B),
+ * opacity / scales raw (logit / log), rotation normalised.  shs here is [N,K,3] (sh0 and shN concatenated).
+ * The row image is assembled / taken apart on the GPU; the *_file functions only move whole buffers. */
+typedef struct gsx_ply_layout {
+    uint64_t vertex_count;
+    uint64_t data_offset;   /* byte offset of the first vertex row */
+    uint32_t stride_floats; /* floats per vertex row */
+    int32_t pos[3];         /* float index inside a row; -1 = property absent */
+    int32_t opacity;
+    int32_t scale[3];
+    int32_t rot[4];
+    int32_t dc_start, dc_count, rest_start, rest_count;
+} gsx_ply_layout;
+GSX_API uint32_t gsx_ply_row_floats(uint32_t K);
+/* header text of the writer; returns its length (buf may be null to query), negative status on error */
+GSX_API int64_t gsx_ply_format_header(uint64_t N, uint32_t K, char* buf, size_t capacity);
+/* parse_header (ply.cpp:185-323): LF or CRLF lines, '#' / empty lines skipped, properties found by name in any
+ * order, unknown float properties skipped over.  Errors as the reference's (missing magic, not binary little
+ * endian, no vertex element, no end_header, > 10000 lines); a non-float vertex property is GSX_ERR_UNSUPPORTED
+ * (the reference would misread the rows). */
+GSX_API int gsx_ply_parse_header(const char* data, size_t size, gsx_ply_layout* layout);
+/* K of the tensors a file unpacks to: dc_count/3 (1 if absent) + rest_count/3 (15 if absent, ply.cpp:554) */
+GSX_API uint32_t gsx_ply_layout_sh_coeffs(const gsx_ply_layout* layout);
+GSX_API int gsx_ply_pack_rows(uint64_t N, uint32_t K, const float* means, const float* shs, const float* opacity_raw,
+                              const float* scaling_raw, const float* rotation_raw, float* rows, void* stream);
+/* rows: device copy of the vertex rows (vertex_count * stride_floats floats).  Absent properties get the
+ * reference's defaults: 0, log-scale -5 (ply.cpp:583), rotation (1,0,0,0) (ply.cpp:608). */
+GSX_API int gsx_ply_unpack_rows(const gsx_ply_layout* layout, const float* rows, float* means, float* shs,
+                                float* opacity_raw, float* scaling_raw, float* rotation_raw, void* stream);
+GSX_API int gsx_ply_write_file(const char* path, uint64_t N, uint32_t K, const float* rows_host);
+GSX_API int gsx_ply_read_file_header(const char* path, gsx_ply_layout* layout);
+GSX_API int gsx_ply_read_file_rows(const char* path, const gsx_ply_layout* layout, float* rows_host);
+
 #ifdef __cplusplus
 }
 #endif

@@ -50,6 +50,14 @@ class RowTensor(ctypes.Structure):
     _fields_ = [("data", c_p), ("row_floats", c_u32), ("is_optimizer_state", ctypes.c_int32)]
 
 
+class PlyLayout(ctypes.Structure):
+    """gsx_ply_layout"""
+    _fields_ = [("vertex_count", ctypes.c_uint64), ("data_offset", ctypes.c_uint64),
+                ("stride_floats", ctypes.c_uint32), ("pos", ctypes.c_int32 * 3), ("opacity", ctypes.c_int32),
+                ("scale", ctypes.c_int32 * 3), ("rot", ctypes.c_int32 * 4), ("dc_start", ctypes.c_int32),
+                ("dc_count", ctypes.c_int32), ("rest_start", ctypes.c_int32), ("rest_count", ctypes.c_int32)]
+
+
 class UpdateArgs(ctypes.Structure):
     """gsx_update_args"""
     _fields_ = ([("N", c_u32), ("K", c_u32), ("sh_degree", c_u32)] +
@@ -86,6 +94,9 @@ def lib():
         L.gsx_image_loss_blocks.restype = c_u32
         L.gsx_photometric_partials.restype = c_u32
         L.gsx_l1_regularization_partials.restype = c_u32
+        L.gsx_ply_row_floats.restype = c_u32
+        L.gsx_ply_layout_sh_coeffs.restype = c_u32
+        L.gsx_ply_format_header.restype = ctypes.c_int64
         L.gsx_ut_defaults.restype = UTParams
         for name in ("gsx_intersect_tile_count_workspace_bytes", "gsx_radix_sort_pairs_workspace_bytes",
                      "gsx_rasterize_bwd_workspace_bytes", "gsx_mcmc_relocate_workspace_bytes",
