@@ -132,6 +132,8 @@ GSX_API uint32_t gsx_n_bits(uint32_t n);
  * passes begin_bit = 0).  Buffers 0 (keys0/vals0, the input) and 1 (keys1/vals1) are ping-ponged; *selector_host
  * (host int) says which pair holds the result (like cub::DoubleBuffer::selector). */
 GSX_API size_t gsx_radix_sort_pairs_workspace_bytes(int64_t n);
+/* the selector gsx_radix_sort_pairs will report for this size and bit range (known before the sort runs) */
+GSX_API int gsx_radix_sort_pairs_selector(int64_t n, uint32_t begin_bit, uint32_t end_bit);
 GSX_API int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, int64_t* keys1, int32_t* vals1,
                                  uint32_t begin_bit, uint32_t end_bit, void* workspace, size_t workspace_bytes,
                                  int* selector_host, void* stream);

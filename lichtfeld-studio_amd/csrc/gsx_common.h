@@ -38,6 +38,13 @@ void set_error(const char* fmt, ...);
 static inline uint32_t cdiv(uint64_t a, uint64_t b) { return (uint32_t)((a + b - 1) / b); }
 static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
+// intersect.hip: the depth-ordered tile count from ready-made keys.  ordered_keys(ws) is where the N
+// (tile count << 32 | depth bits) keys go inside a gsx_intersect_tile_count_ordered workspace; the second call sorts
+// them on the depth bits, scans the counts in that order into cum (inclusive) and starts the copy of the total.
+int64_t* ordered_keys(void* workspace);
+int ordered_counts_from_keys(const char* who, uint32_t N, int32_t* order, int64_t* cum_tiles_per_gauss, void* workspace,
+                             size_t workspace_bytes, int64_t* n_isects_host, int wait, void* stream);
+
 int check_camera_args(uint32_t C, const float* viewmats1, int camera_model, int rs_type, const float* radial,
                       const float* tangential, const float* thin_prism);
 

@@ -350,6 +350,41 @@ OrderedLayout ordered_layout(uint32_t N) {
 
 extern "C" size_t gsx_intersect_tile_count_ordered_workspace_bytes(uint32_t N) { return ordered_layout(N).total; }
 
+namespace gsx {
+int64_t* ordered_keys(void* workspace) { return (int64_t*)workspace; }
+
+// The part after the keys are written: sort the N (count << 32 | depth bits) keys in workspace on their low word,
+// scan the counts in that order, start the copy of the total.  order must hold 0..N-1 on entry.
+int ordered_counts_from_keys(const char* who, uint32_t N, int32_t* order, int64_t* cum_tiles_per_gauss, void* workspace,
+                             size_t workspace_bytes, int64_t* n_isects_host, int wait, void* stream) {
+    const OrderedLayout L = ordered_layout(N);
+    GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 && workspace_bytes >= L.total,
+                GSX_ERR_WORKSPACE, "%s: workspace needs %zu bytes, 256-byte aligned", who, L.total);
+    char* ws = (char*)workspace;
+    int64_t* keys0 = (int64_t*)ws;
+    int64_t* keys1 = (int64_t*)(ws + L.keys1_off);
+    int32_t* vals1 = (int32_t*)(ws + L.vals1_off);
+    int64_t* block_sums = (int64_t*)(ws + L.sums_off);
+    int64_t* total = block_sums + cdiv(N, kScanTile);
+    hipStream_t s = (hipStream_t)stream;
+    int rc, sel = 0;
+    if ((rc = gsx_radix_sort_pairs(N, keys0, order, keys1, vals1, 0, 32, ws + L.sort_off,
+                                   gsx_radix_sort_pairs_workspace_bytes(N), &sel, stream)) != GSX_OK)
+        return rc;
+    if (sel) // four 8-bit passes end in buffer 0; kept for a different digit width
+        GSX_HIP_CHECK(hipMemcpyAsync(order, vals1, (size_t)N * 4, hipMemcpyDeviceToDevice, s));
+    if ((rc = scan_counts(N, nullptr, sel ? keys1 : keys0, cum_tiles_per_gauss, block_sums, total, s)) != GSX_OK)
+        return rc;
+    GSX_HIP_CHECK(hipMemcpyAsync(n_isects_host, total, sizeof(int64_t), hipMemcpyDeviceToHost, s));
+    if (wait) {
+        GSX_HIP_CHECK(hipStreamSynchronize(s));
+        GSX_REQUIRE(*n_isects_host < (1ll << 31), GSX_ERR_OVERFLOW, "%s: %lld intersections do not fit int32 indices",
+                    who, (long long)*n_isects_host);
+    }
+    return GSX_OK;
+}
+} // namespace gsx
+
 extern "C" int gsx_intersect_tile_count_ordered(uint32_t N, const float* means2d, const int32_t* radii,
                                                 const float* depths, uint32_t tile_size, uint32_t tile_width,
                                                 uint32_t tile_height, int32_t* order, int32_t* tiles_per_gauss,
@@ -366,35 +401,16 @@ extern "C" int gsx_intersect_tile_count_ordered(uint32_t N, const float* means2d
     int rc = check_tile_grid("intersect_tile_count_ordered", 1, tile_size, tile_width, tile_height);
     if (rc != GSX_OK)
         return rc;
-    const OrderedLayout L = ordered_layout(N);
-    GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 && workspace_bytes >= L.total,
-                GSX_ERR_WORKSPACE, "intersect_tile_count_ordered: workspace needs %zu bytes, 256-byte aligned", L.total);
-    char* ws = (char*)workspace;
-    int64_t* keys0 = (int64_t*)ws;
-    int64_t* keys1 = (int64_t*)(ws + L.keys1_off);
-    int32_t* vals1 = (int32_t*)(ws + L.vals1_off);
-    int64_t* block_sums = (int64_t*)(ws + L.sums_off);
-    int64_t* total = block_sums + cdiv(N, kScanTile);
-    hipStream_t s = (hipStream_t)stream;
-    hipLaunchKernelGGL(depth_count_keys_kernel, dim3(cdiv(N, 256)), dim3(256), 0, s, N, means2d, radii, depths,
-                       (float)tile_size, tile_width, tile_height, tiles_per_gauss, keys0, order);
+    GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 &&
+                    workspace_bytes >= ordered_layout(N).total,
+                GSX_ERR_WORKSPACE, "intersect_tile_count_ordered: workspace needs %zu bytes, 256-byte aligned",
+                ordered_layout(N).total);
+    hipLaunchKernelGGL(depth_count_keys_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, means2d,
+                       radii, depths, (float)tile_size, tile_width, tile_height, tiles_per_gauss,
+                       gsx::ordered_keys(workspace), order);
     GSX_LAUNCH_CHECK();
-    int sel = 0;
-    if ((rc = gsx_radix_sort_pairs(N, keys0, order, keys1, vals1, 0, 32, ws + L.sort_off,
-                                   gsx_radix_sort_pairs_workspace_bytes(N), &sel, stream)) != GSX_OK)
-        return rc;
-    if (sel) // four 8-bit passes end in buffer 0; kept for a different digit width
-        GSX_HIP_CHECK(hipMemcpyAsync(order, vals1, (size_t)N * 4, hipMemcpyDeviceToDevice, s));
-    if ((rc = scan_counts(N, nullptr, sel ? keys1 : keys0, cum_tiles_per_gauss, block_sums, total, s)) != GSX_OK)
-        return rc;
-    GSX_HIP_CHECK(hipMemcpyAsync(n_isects_host, total, sizeof(int64_t), hipMemcpyDeviceToHost, s));
-    if (wait) {
-        GSX_HIP_CHECK(hipStreamSynchronize(s));
-        GSX_REQUIRE(*n_isects_host < (1ll << 31), GSX_ERR_OVERFLOW,
-                    "intersect_tile_count_ordered: %lld intersections do not fit int32 indices",
-                    (long long)*n_isects_host);
-    }
-    return GSX_OK;
+    return gsx::ordered_counts_from_keys("intersect_tile_count_ordered", N, order, cum_tiles_per_gauss, workspace,
+                                         workspace_bytes, n_isects_host, wait, stream);
 }
 
 extern "C" int gsx_intersect_tile_emit(uint32_t C, uint32_t N, const float* means2d, const int32_t* radii,

@@ -234,6 +234,12 @@ extern "C" size_t gsx_radix_sort_pairs_workspace_bytes(int64_t n) {
     return n > kSmallSortLimit && small_max > need ? small_max : need;
 }
 
+extern "C" int gsx_radix_sort_pairs_selector(int64_t n, uint32_t begin_bit, uint32_t end_bit) {
+    if (n <= 0 || end_bit <= begin_bit)
+        return 0;
+    return (int)(((end_bit - begin_bit + kRadixBits - 1) / kRadixBits) & 1u); // one ping-pong per digit pass
+}
+
 extern "C" int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, int64_t* keys1, int32_t* vals1,
                                     uint32_t begin_bit, uint32_t end_bit, void* workspace, size_t workspace_bytes,
                                     int* selector_host, void* stream) {

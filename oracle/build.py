@@ -1,4 +1,4 @@
-"""Build the CPU checker (oracle/gsx_oracle.cpp) into oracle/libgsx_oracle.so.
+"""Build the CPU checker (oracle/gsx_oracle.cpp, oracle/fastgs_oracle.cpp) into oracle/libgsx_oracle.so.
 
 Test infrastructure only: nothing in the shipped package imports this.
 
@@ -11,7 +11,7 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
-SRC = os.path.join(HERE, "gsx_oracle.cpp")
+SRCS = [os.path.join(HERE, "gsx_oracle.cpp"), os.path.join(HERE, "fastgs_oracle.cpp")]
 OUT = os.path.join(HERE, "libgsx_oracle.so")
 MATH_INC = os.path.join(ROOT, "lichtfeld-studio_amd", "csrc")
 
@@ -23,9 +23,9 @@ FLAGS = ["-O2", "-march=x86-64-v3", "-ffp-contract=off", "-fno-fast-math", "-fop
 
 def build(force=True):
     if not force and os.path.exists(OUT) and os.path.getmtime(OUT) >= max(
-            os.path.getmtime(SRC), os.path.getmtime(os.path.join(MATH_INC, "gsx_math.h"))):
+            *[os.path.getmtime(s) for s in SRCS], os.path.getmtime(os.path.join(MATH_INC, "gsx_math.h"))):
         return OUT
-    cmd = ["g++", *FLAGS, "-I", MATH_INC, SRC, "-o", OUT]
+    cmd = ["g++", *FLAGS, "-I", MATH_INC, *SRCS, "-o", OUT]
     subprocess.run(cmd, check=True)
     return OUT
 

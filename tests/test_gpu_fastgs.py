@@ -1,0 +1,168 @@
+"""GPU parity of the fastgs (Jacobian-EWA) backend against its CPU restatement: the forward bit for bit (tile lists,
+image, alpha, per-pixel state), the backward to 1e-3 of each tensor's scale, through the host mirror of
+forward_wrapper / backward_wrapper over the C ABI."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+
+from oracle import fastgs as ofg  # noqa: E402
+
+
+def _scene(gsx, n, W, H, f, seed=2, bigger=0.0, degree=3):
+    sc = gsx.scenes.config(3, n)
+    K = (degree + 1) ** 2
+    P = dict(means=sc.means.astype(np.float32), scales_raw=(sc.scaling_raw + bigger).astype(np.float32),
+             rotations_raw=(sc.rotation_raw * np.linspace(0.5, 2.0, n)[:, None]).astype(np.float32),
+             opacities_raw=sc.opacity_raw.reshape(-1, 1).astype(np.float32), sh0=sc.sh0.astype(np.float32),
+             shN=np.ascontiguousarray(sc.shN[:, :max(K - 1, 0)]).astype(np.float32))
+    cam = gsx.scenes.orbit_camera(0.7, 4.0, W, H, f)
+    V = cam.viewmat.astype(np.float32)
+    cam_pos = (-V[:3, :3].T @ V[:3, 3]).astype(np.float32)
+    return P, V, cam_pos
+
+
+def _to(P, cuda):
+    return {k: torch.from_numpy(v).to(cuda) for k, v in P.items()}
+
+
+def _forward(gsx, D, V, cam_pos, bases, W, H, f, bg=None):
+    from lichtfeld_studio_amd import fastgs
+    return fastgs.forward_wrapper(D["means"], D["scales_raw"], D["rotations_raw"], D["opacities_raw"], D["sh0"],
+                                  D["shN"], V, cam_pos, bases, W, H, f, 1.02 * f, W / 2 + 0.5, H / 2 - 0.25, 0.01, 1e10,
+                                  background=bg)
+
+
+@pytest.mark.parametrize("n,W,H,bigger,degree", [(20_000, 309, 205, 1.2, 3), (3_000, 200, 136, 3.0, 1),
+                                                 (50_000, 640, 360, 0.8, 0)])
+def test_forward_bit_exact(gsx, cuda, n, W, H, bigger, degree):
+    """tile lists, image, alpha, final transmittance and last-contributor positions equal the checker's bit for
+    bit (small Gaussians: the sequential tile path; large ones: the wave-cooperative path); the footprint box the
+    per-wave selection uses is conservative; a second run is identical"""
+    from lichtfeld_studio_amd import fastgs
+    f = 0.93 * W
+    P, V, cam_pos = _scene(gsx, n, W, H, f, bigger=bigger, degree=degree)
+    P["means"][100:110] = P["means"][90:100]  # equal depths
+    bases = (degree + 1) ** 2
+    S = ofg.settings(bases, P["shN"].shape[1], W, H, f, 1.02 * f, W / 2 + 0.5, H / 2 - 0.25)
+    F = ofg.forward(P["means"], P["scales_raw"], P["rotations_raw"], P["opacities_raw"], P["sh0"], P["shN"], V,
+                    cam_pos, S)
+    D = _to(P, cuda)
+    out = _forward(gsx, D, V, cam_pos, bases, W, H, f)
+    torch.cuda.synchronize()
+    image, alpha, prim, pix, inst_state, _, _, n_inst = out[:8]
+    assert n_inst == F["instance_primitive"].size and n_inst > 10 * n // 4
+    rec, cnt = fastgs.primitive_records(prim, n)
+    assert np.array_equal(cnt.cpu().numpy().astype(np.uint32), F["n_touched"])
+    vis = F["n_touched"] > 0
+    rec = rec.cpu().numpy()
+    for got, want in ((rec[:, 0:2], F["mean2d"]), (rec[:, [2, 3, 4, 5]], F["conic_opacity"]), (rec[:, 6:9], F["color"]),
+                      (rec[:, 11], F["depth"])):
+        assert np.array_equal(got[vis].view(np.int32), np.ascontiguousarray(want[vis]).view(np.int32))
+    inst, offs = fastgs.instance_list(inst_state, n_inst, W, H)
+    assert np.array_equal(inst.cpu().numpy().astype(np.uint32), F["instance_primitive"])
+    ranges = F["tile_ranges"]
+    offs = offs.cpu().numpy()
+    nonempty = ranges[:, 1] > ranges[:, 0]
+    assert np.array_equal(offs[nonempty], ranges[nonempty, 0].astype(np.int32))
+    ends = np.append(offs[1:], n_inst)
+    assert np.array_equal((ends - offs)[~nonempty], np.zeros((~nonempty).sum(), np.int32))
+    assert np.array_equal(image.cpu().numpy().view(np.int32), F["image"].view(np.int32))
+    assert np.array_equal(alpha.cpu().numpy().view(np.int32), F["alpha"].view(np.int32))
+    px = W * H
+    t_final = pix.view(torch.float32)[:px].cpu().numpy().reshape(H, W)
+    off2 = ((px * 4 + 255) // 256 * 256) // 4
+    n_contrib = pix.view(torch.int32)[off2:off2 + px].cpu().numpy().reshape(H, W)
+    assert np.array_equal(t_final.view(np.int32), F["transmittance"].view(np.int32))
+    assert np.array_equal(n_contrib.astype(np.uint32), F["n_contributions"])
+    *_, violations = ofg.blend(F, F["instance_primitive"], ranges, S, extents=rec[:, 9:11])
+    assert violations == 0
+    out2 = _forward(gsx, D, V, cam_pos, bases, W, H, f)
+    assert torch.equal(out2[0], image) and torch.equal(out2[1], alpha)
+
+
+@pytest.mark.parametrize("n,W,H,bigger,degree,bg", [(20_000, 309, 205, 1.2, 3, True), (3_000, 200, 136, 3.0, 1, False),
+                                                    (4_000, 160, 120, 1.5, 0, True)])
+def test_backward_matches_oracle(gsx, cuda, n, W, H, bigger, degree, bg):
+    """gradients of every parameter tensor, the camera gradient and the densification statistic against the
+    checker (1e-3 of each tensor's largest entry: the sums over pixels run in another order), with and without a
+    background; the accumulator is left zeroed, so a second backward gives the same result"""
+    from lichtfeld_studio_amd import fastgs
+    f = 0.93 * W
+    P, V, cam_pos = _scene(gsx, n, W, H, f, bigger=bigger, degree=degree)
+    bases = (degree + 1) ** 2
+    S = ofg.settings(bases, P["shN"].shape[1], W, H, f, 1.02 * f, W / 2 + 0.5, H / 2 - 0.25)
+    F = ofg.forward(P["means"], P["scales_raw"], P["rotations_raw"], P["opacities_raw"], P["sh0"], P["shN"], V,
+                    cam_pos, S)
+    r = np.random.default_rng(4)
+    g_img = r.normal(0, 1, (3, H, W)).astype(np.float32)
+    g_a = r.normal(0, 1, (1, H, W)).astype(np.float32)
+    bgc = np.array([0.2, 0.7, 0.4], np.float32)
+    # image_out = image + T * bg: the background reaches the parameters through alpha only
+    g_a_ref = g_a - (bgc[:, None, None] * g_img).sum(0, keepdims=True) if bg else g_a
+    info_ref = np.full((2, n), 0.5, np.float32)
+    G = ofg.backward(F, P["means"], P["scales_raw"], P["rotations_raw"], P["shN"], V, cam_pos, S, g_img, g_a_ref, True,
+                     info_ref)
+    D = _to(P, cuda)
+    bg_d = torch.from_numpy(bgc).to(cuda) if bg else None
+    out = _forward(gsx, D, V, cam_pos, bases, W, H, f, bg=bg_d)
+    if bg:
+        want = F["image"] + F["transmittance"][None] * bgc[:, None, None]
+        assert np.abs(out[0].cpu().numpy() - want).max() < 1e-6
+    info = torch.full((2, n), 0.5, dtype=torch.float32, device=cuda)
+    args = (torch.from_numpy(g_img).to(cuda), torch.from_numpy(g_a).to(cuda), out[0], out[1], D["means"],
+            D["scales_raw"], D["rotations_raw"], D["shN"], out[2], out[3], out[4], out[5], V, cam_pos, bases, W, H, f,
+            1.02 * f, W / 2 + 0.5, H / 2 - 0.25, 0.01, 1e10, out[6], out[7], out[8], out[9], out[10])
+    got = fastgs.backward_wrapper(info, *args, w2c_requires_grad=True, background=bg_d)
+    torch.cuda.synchronize()
+    names = ("means", "scales_raw", "rotations_raw", "opacities_raw", "sh0", "shN")
+    for name, g in zip(names, got[:6]):
+        want = G[name].reshape(g.shape)
+        if want.size == 0:
+            continue
+        scale = np.abs(want).max()
+        assert scale > 0, name
+        err = np.abs(g.cpu().numpy() - want).max()
+        assert err <= 1e-3 * scale, (name, err, scale)
+    culled = F["n_touched"] == 0
+    assert culled.any() and not got[0].cpu().numpy()[culled].any() and not got[5].cpu().numpy()[culled].any()
+    w2c_want = G["w2c"]
+    assert np.abs(got[6].cpu().numpy() - w2c_want).max() <= 2e-3 * np.abs(w2c_want).max()
+    assert np.allclose(info.cpu().numpy(), info_ref, rtol=2e-3, atol=1e-4)
+    got2 = fastgs.backward_wrapper(None, *args, w2c_requires_grad=False, background=bg_d)
+    for a, b in zip(got[:6], got2[:6]):
+        if a.numel() == 0:
+            continue
+        scale = float(a.abs().max())
+        assert float((a - b).abs().max()) <= 1e-4 * scale  # atomics: equal up to summation order
+    assert got2[6] is None
+
+
+def test_wrapper_rejects_bad_inputs(gsx, cuda):
+    from lichtfeld_studio_amd import fastgs
+    from lichtfeld_studio_amd._lib import GsxError
+    P, V, cam_pos = _scene(gsx, 1000, 64, 48, 60.0)
+    D = _to(P, cuda)
+    with pytest.raises(ValueError, match="contiguous CUDA float"):
+        fastgs.forward_wrapper(D["means"].cpu(), D["scales_raw"], D["rotations_raw"], D["opacities_raw"], D["sh0"],
+                               D["shN"], V, cam_pos, 16, 64, 48, 60.0, 60.0, 32.0, 24.0, 0.01, 1e10)
+    with pytest.raises(ValueError, match="contiguous CUDA float"):
+        fastgs.forward_wrapper(D["means"], D["scales_raw"].t().contiguous().t(), D["rotations_raw"],
+                               D["opacities_raw"], D["sh0"], D["shN"], V, cam_pos, 16, 64, 48, 60.0, 60.0, 32.0, 24.0,
+                               0.01, 1e10)
+    with pytest.raises(GsxError):  # more active bases than stored
+        fastgs.forward_wrapper(D["means"], D["scales_raw"], D["rotations_raw"], D["opacities_raw"], D["sh0"],
+                               D["shN"][:, :3].contiguous(), V, cam_pos, 16, 64, 48, 60.0, 60.0, 32.0, 24.0, 0.01, 1e10)
+    with pytest.raises(GsxError):  # more than 65536 tiles
+        fastgs.forward_wrapper(D["means"], D["scales_raw"], D["rotations_raw"], D["opacities_raw"], D["sh0"],
+                               D["shN"], V, cam_pos, 16, 8192, 4096, 60.0, 60.0, 32.0, 24.0, 0.01, 1e10)
+    # nothing visible: empty instance list, zero image, zero gradients
+    far = D["means"] + 1000.0
+    out = fastgs.forward_wrapper(far, D["scales_raw"], D["rotations_raw"], D["opacities_raw"], D["sh0"], D["shN"], V,
+                                 cam_pos, 16, 64, 48, 60.0, 60.0, 32.0, 24.0, 0.01, 1e10)
+    assert out[7] == 0 and float(out[0].abs().max()) == 0.0 and float(out[1].abs().max()) == 0.0
+    g = fastgs.backward_wrapper(None, torch.ones_like(out[0]), torch.ones_like(out[1]), out[0], out[1], far,
+                                D["scales_raw"], D["rotations_raw"], D["shN"], out[2], out[3], out[4], out[5], V, cam_pos,
+                                16, 64, 48, 60.0, 60.0, 32.0, 24.0, 0.01, 1e10, *out[6:11])
+    assert all(float(t.abs().max()) == 0.0 for t in g[:6])
