@@ -166,3 +166,53 @@ def test_wrapper_rejects_bad_inputs(gsx, cuda):
                                 D["scales_raw"], D["rotations_raw"], D["shN"], out[2], out[3], out[4], out[5], V, cam_pos,
                                 16, 64, 48, 60.0, 60.0, 32.0, 24.0, 0.01, 1e10, *out[6:11])
     assert all(float(t.abs().max()) == 0.0 for t in g[:6])
+
+
+def test_full_size_1m_gaussians(gsx, cuda):
+    """the measured configuration's shape (1M SH3 Gaussians, 1237x822): forward bit for bit against the checker,
+    backward to 1e-3, and the properties that hold at any size (instance total = sum of tile counts, ranges
+    partition the list, every tile's list is depth ordered, alpha in [0, 1])"""
+    from lichtfeld_studio_amd import fastgs
+    n, W, H, f = 1_000_000, 1237, 822, 1150.0
+    sc = gsx.scenes.config(3, n)
+    cam = sc.cameras[0]
+    V = cam.viewmat.astype(np.float32)
+    cam_pos = (-V[:3, :3].T @ V[:3, 3]).astype(np.float32)
+    P = dict(means=sc.means.astype(np.float32), scales_raw=sc.scaling_raw.astype(np.float32),
+             rotations_raw=sc.rotation_raw.astype(np.float32), opacities_raw=sc.opacity_raw.reshape(-1, 1).astype(np.float32),
+             sh0=sc.sh0.astype(np.float32), shN=sc.shN.astype(np.float32))
+    fx, fy, cx, cy = float(cam.K[0, 0]), float(cam.K[1, 1]), float(cam.K[0, 2]), float(cam.K[1, 2])
+    S = ofg.settings(16, 15, W, H, fx, fy, cx, cy)
+    F = ofg.forward(P["means"], P["scales_raw"], P["rotations_raw"], P["opacities_raw"], P["sh0"], P["shN"], V,
+                    cam_pos, S)
+    D = _to(P, cuda)
+    out = fastgs.forward_wrapper(D["means"], D["scales_raw"], D["rotations_raw"], D["opacities_raw"], D["sh0"], D["shN"],
+                                 V, cam_pos, 16, W, H, fx, fy, cx, cy, 0.01, 1e10)
+    torch.cuda.synchronize()
+    n_inst = out[7]
+    assert n_inst == F["instance_primitive"].size and n_inst > 2_000_000
+    rec, cnt = fastgs.primitive_records(out[2], n)
+    assert int(cnt.sum()) == n_inst
+    inst, offs = fastgs.instance_list(out[4], n_inst, W, H)
+    assert np.array_equal(inst.cpu().numpy().astype(np.uint32), F["instance_primitive"])
+    ends = torch.cat([offs[1:], torch.tensor([n_inst], dtype=torch.int32, device=cuda)])
+    assert bool((ends >= offs).all()) and int(offs[0]) == 0
+    depth_bits = rec[:, 11].contiguous().view(torch.int32)[inst.long()].long()
+    tile_of = torch.repeat_interleave(torch.arange(offs.numel(), device=cuda), (ends - offs).long())
+    key = tile_of * (1 << 32) + depth_bits
+    assert bool((key[1:] >= key[:-1]).all())
+    assert np.array_equal(out[0].cpu().numpy().view(np.int32), F["image"].view(np.int32))
+    assert np.array_equal(out[1].cpu().numpy().view(np.int32), F["alpha"].view(np.int32))
+    assert float(out[1].min()) >= 0.0 and float(out[1].max()) <= 1.0
+    r = np.random.default_rng(8)
+    g_img, g_a = r.normal(0, 1, (3, H, W)).astype(np.float32), r.normal(0, 1, (1, H, W)).astype(np.float32)
+    G = ofg.backward(F, P["means"], P["scales_raw"], P["rotations_raw"], P["shN"], V, cam_pos, S, g_img, g_a)
+    got = fastgs.backward_wrapper(None, torch.from_numpy(g_img).to(cuda), torch.from_numpy(g_a).to(cuda), out[0], out[1],
+                                  D["means"], D["scales_raw"], D["rotations_raw"], D["shN"], out[2], out[3], out[4], out[5],
+                                  V, cam_pos, 16, W, H, fx, fy, cx, cy, 0.01, 1e10, *out[6:11])
+    torch.cuda.synchronize()
+    for name, g in zip(("means", "scales_raw", "rotations_raw", "opacities_raw", "sh0", "shN"), got[:6]):
+        want = G[name].reshape(g.shape)
+        scale = np.abs(want).max()
+        err = np.abs(g.cpu().numpy() - want).max()
+        assert err <= 1e-3 * scale, (name, err, scale)
