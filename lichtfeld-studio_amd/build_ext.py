@@ -1,5 +1,5 @@
-"""Build gsx_torch_ext.so: the C++ host layer (csrc/host/gsplat_ops.cpp, the at::Tensor functions of gsplat/Ops.h
-over the C ABI) plus its pybind11 module, in-tree, linked against libgsx.so (rpath $ORIGIN) and LibTorch.
+"""Build gsx_torch_ext.so: the C++ host layer (csrc/host/gsplat_ops.cpp: the at::Tensor functions of gsplat/Ops.h;
+csrc/host/fastgs_api.cpp: fast_gs::rasterization::forward_wrapper / backward_wrapper; both over the C ABI) plus its pybind11 module, in-tree, linked against libgsx.so (rpath $ORIGIN) and LibTorch.
 
     python build_ext.py
 
@@ -53,8 +53,8 @@ def build():
         raise RuntimeError("libgsx.so is missing: run build.py first")
     os.makedirs(OBJ, exist_ok=True)
     cflags, ldflags = _flags()
-    srcs = [os.path.join(HOST, "gsplat_ops.cpp"), os.path.join(HOST, "bindings.cpp")]
-    with ThreadPoolExecutor(max_workers=2) as ex:
+    srcs = [os.path.join(HOST, "gsplat_ops.cpp"), os.path.join(HOST, "fastgs_api.cpp"), os.path.join(HOST, "bindings.cpp")]
+    with ThreadPoolExecutor(max_workers=3) as ex:
         objs = list(ex.map(_compile, [(s, cflags) for s in srcs]))
     subprocess.run([CXX, *objs, *ldflags, "-o", OUT], check=True)
     return OUT

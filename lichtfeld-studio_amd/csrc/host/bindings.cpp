@@ -2,6 +2,7 @@
 // drive the functions a LichtFeld build would link.  Names and argument order are those of gsplat/Ops.h.
 #include <torch/extension.h>
 
+#include "fastgs_api.h"
 #include "gsplat_api.h"
 
 namespace py = pybind11;
@@ -51,4 +52,6 @@ PYBIND11_MODULE(gsx_torch_ext, m) {
         fast_gs::optimizer::adam_step_wrapper(param, exp_avg, exp_avg_sq, param_grad, lr, beta1, beta2, eps, bc1_rcp,
                                               bc2_sqrt_rcp);
     });
+    m.def("fastgs_forward_wrapper", &fast_gs::rasterization::forward_wrapper);
+    m.def("fastgs_backward_wrapper", &fast_gs::rasterization::backward_wrapper);
 }

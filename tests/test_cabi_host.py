@@ -103,7 +103,7 @@ def test_cpp_host_layer_loads_and_checks_inputs(cpp):
                  "quats_to_rotmats", "relocation", "add_noise", "projection_ut_3dgs_fused",
                  "rasterize_to_pixels_from_world_3dgs_fwd", "rasterize_to_pixels_from_world_3dgs_bwd",
                  "rasterize_from_world_with_sh_fwd", "rasterize_from_world_with_sh_bwd", "fusedssim",
-                 "fusedssim_backward", "adam_step_wrapper"):
+                 "fusedssim_backward", "adam_step_wrapper", "fastgs_forward_wrapper", "fastgs_backward_wrapper"):
         assert callable(getattr(cpp, name)), name
     ut = cpp.UnscentedTransformParameters()
     assert (ut.alpha, ut.beta, ut.kappa, ut.require_all_sigma_points_valid) == (pytest.approx(0.1), 2.0, 0.0, True)
@@ -116,6 +116,10 @@ def test_cpp_host_layer_loads_and_checks_inputs(cpp):
         cpp.relocation(torch.zeros(4), torch.zeros((4, 3)), torch.ones(4, dtype=torch.int32), torch.zeros((51, 51)), 51)
     with pytest.raises(RuntimeError, match="padding"):
         cpp.fused_ssim_value(torch.zeros((1, 3, 16, 16)), torch.zeros((1, 3, 16, 16)), "reflect")
+    z = torch.zeros
+    with pytest.raises(RuntimeError, match="means must be a contiguous CUDA float tensor"):
+        cpp.fastgs_forward_wrapper(z((4, 3)), z((4, 3)), z((4, 4)), z((4, 1)), z((4, 1, 3)), z((4, 15, 3)), torch.eye(4),
+                                   z(3), 16, 64, 48, 60.0, 60.0, 32.0, 24.0, 0.01, 1e10)
 
 
 def test_scene_generator_is_deterministic(gsx):

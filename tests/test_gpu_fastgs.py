@@ -216,3 +216,41 @@ def test_full_size_1m_gaussians(gsx, cuda):
         scale = np.abs(want).max()
         err = np.abs(g.cpu().numpy() - want).max()
         assert err <= 1e-3 * scale, (name, err, scale)
+
+
+def test_cpp_wrappers_equal_python_wrappers(gsx, cpp, cuda):
+    """fast_gs::rasterization::forward_wrapper / backward_wrapper of the C++ host layer: same image / alpha bit for
+    bit and the same gradients (up to the order of the atomic sums) as the ctypes path, w2c gradient only when
+    w2c.requires_grad(), densification_info updated in place, errors as c10::Error"""
+    from lichtfeld_studio_amd import fastgs
+    n, W, H, f = 20_000, 309, 205, 287.0
+    P, V, cam_pos = _scene(gsx, n, W, H, f, bigger=1.2)
+    D = _to(P, cuda)
+    scal = (16, W, H, f, 1.02 * f, W / 2 + 0.5, H / 2 - 0.25, 0.01, 1e10)
+    ref = fastgs.forward_wrapper(D["means"], D["scales_raw"], D["rotations_raw"], D["opacities_raw"], D["sh0"], D["shN"],
+                                 V, cam_pos, *scal)
+    w2c = torch.from_numpy(V).to(cuda).requires_grad_(True)
+    cp = torch.from_numpy(cam_pos).to(cuda)
+    out = cpp.fastgs_forward_wrapper(D["means"], D["scales_raw"], D["rotations_raw"], D["opacities_raw"], D["sh0"],
+                                     D["shN"], w2c, cp, *scal)
+    assert torch.equal(out[0], ref[0]) and torch.equal(out[1], ref[1]) and out[7] == ref[7]
+    assert out[5].numel() == 0 and out[6] == -1 and out[8:] == (0, 0, 0)
+    g_img, g_a = torch.randn(3, H, W, device=cuda), torch.randn(1, H, W, device=cuda)
+    info = torch.zeros((2, n), device=cuda)
+    got = cpp.fastgs_backward_wrapper(info, g_img, g_a, out[0], out[1], D["means"], D["scales_raw"], D["rotations_raw"],
+                                      D["shN"], out[2], out[3], out[4], out[5], w2c, cp, *scal, *out[6:11])
+    info_ref = torch.zeros((2, n), device=cuda)
+    want = fastgs.backward_wrapper(info_ref, g_img, g_a, ref[0], ref[1], D["means"], D["scales_raw"], D["rotations_raw"],
+                                   D["shN"], ref[2], ref[3], ref[4], ref[5], V, cam_pos, *scal, *ref[6:11],
+                                   w2c_requires_grad=True)
+    torch.cuda.synchronize()
+    for a, b in zip(got, want):
+        assert a.shape == b.shape and float((a - b).abs().max()) <= 1e-4 * float(b.abs().max())
+    assert float((info - info_ref).abs().max()) <= 1e-4 * float(info_ref.abs().max()) and float(info[0].max()) == 1.0
+    got = cpp.fastgs_backward_wrapper(torch.empty(0, device=cuda), g_img, g_a, out[0], out[1], D["means"], D["scales_raw"],
+                                      D["rotations_raw"], D["shN"], out[2], out[3], out[4], out[5], w2c.detach(), cp,
+                                      *scal, *out[6:11])
+    assert got[6] is None  # an undefined at::Tensor comes back as None
+    with pytest.raises(RuntimeError, match="gsx"):
+        cpp.fastgs_forward_wrapper(D["means"], D["scales_raw"], D["rotations_raw"], D["opacities_raw"], D["sh0"],
+                                   D["shN"][:, :3].contiguous(), w2c, cp, *scal)
