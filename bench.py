@@ -95,6 +95,9 @@ def main():
     ap.add_argument("--separate-update", action="store_true",
                     help="run epilogue / SH backward / activation VJPs / Adam as separate kernels (default: one pass)")
     ap.add_argument("--cpu-threads", type=int, default=0, help="threads for the CPU baseline (0 = all)")
+    ap.add_argument("--workload", choices=["gut", "fastgs"], default="gut",
+                    help="gut: the training step of the metric (default); fastgs: forward + backward of the "
+                         "reference's default rasterizer on the same scene (a secondary line, not the metric)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the path has no multi-GPU part); use --gpus 1", file=sys.stderr)
@@ -112,6 +115,8 @@ def main():
     sc = gsx.scenes.config(args.config, args.n)
     cam = sc.cameras[0]
     W, H = cam.width, cam.height
+    if args.workload == "fastgs":
+        return run_fastgs(args, gsx, sc, cam, dev)
     viewmat = torch.from_numpy(cam.viewmat[None].copy()).to(dev)
     Kmat = torch.from_numpy(cam.K[None].copy()).to(dev)
     # target: render of the independently seeded target scene by the same forward, clamped, CHW
@@ -227,6 +232,47 @@ def main():
         "kernels": kernels,
     }
     print(json.dumps(out))
+
+
+def run_fastgs(args, gsx, sc, cam, dev):
+    """forward_wrapper + backward_wrapper of the fastgs backend on the scene of the metric: a secondary line"""
+    import numpy as np
+    import torch
+    from lichtfeld_studio_amd import fastgs
+    W, H = cam.width, cam.height
+    V = cam.viewmat.astype(np.float32)
+    cam_pos = (-V[:3, :3].T @ V[:3, 3]).astype(np.float32)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(dev)
+    D = dict(means=t(sc.means), scales_raw=t(sc.scaling_raw), rotations_raw=t(sc.rotation_raw),
+             opacities_raw=t(sc.opacity_raw.reshape(-1, 1)), sh0=t(sc.sh0), shN=t(sc.shN))
+    bases = (sc.sh_degree + 1) ** 2
+    scal = (bases, W, H, float(cam.K[0, 0]), float(cam.K[1, 1]), float(cam.K[0, 2]), float(cam.K[1, 2]), 0.01, 1e10)
+    g = torch.Generator(device=dev).manual_seed(1)
+    g_img = torch.randn((3, H, W), generator=g, device=dev)
+    g_a = torch.randn((1, H, W), generator=g, device=dev)
+
+    def step():
+        out = fastgs.forward_wrapper(D["means"], D["scales_raw"], D["rotations_raw"], D["opacities_raw"], D["sh0"],
+                                     D["shN"], V, cam_pos, *scal)
+        fastgs.backward_wrapper(None, g_img, g_a, out[0], out[1], D["means"], D["scales_raw"], D["rotations_raw"],
+                                D["shN"], out[2], out[3], out[4], out[5], V, cam_pos, *scal, *out[6:11])
+        return out
+
+    for _ in range(args.warmup):
+        out = step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for _ in range(args.steps):
+        out = step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t1
+    print(json.dumps({
+        "metric": "fastgs rasterization forward + backward it/s (secondary; not the BASELINE metric)",
+        "value": round(args.steps / elapsed, 3), "unit": "it/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(1e3 * elapsed / args.steps, 3), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"fastgs forward_wrapper + backward_wrapper, {sc.means.shape[0]} Gaussians SH degree "
+                               f"{sc.sh_degree}, {W}x{H}", "n_instances": out[7]}}))
 
 
 def run_cpu_baseline(gsx, sc, cam, gt_chw, use_ssim, threads):
