@@ -77,12 +77,106 @@ __device__ __forceinline__ void shutter_pose(const CamPose& cp, float rel, quat*
     *q = slerp(cp.q_start, cp.q_start, rel);
 }
 
-// world ray through a pixel centre, perfect pinhole, global shutter
-// (Cameras.cuh:457-470 unproject, :253-266 camera_ray_to_world_ray, :322-339)
-__device__ __forceinline__ void pixel_world_ray(const CamPose& cp, float px, float py, float fx, float fy, float cx,
-                                                float cy, vec3* ray_o, vec3* ray_d) {
-    const float u = (px - cx) / fx;
-    const float v = (py - cy) / fy;
+// ---- OpenCV pinhole distortion (gsplat/Cameras.cuh:473-815) ------------------------------------
+// radial [6], tangential [2], thin prism [4]; `on` when the caller gave any of the three coefficient arrays (the
+// reference's dispatch, ProjectionUT3DGSFused.cu:86-113).
+struct Distortion {
+    bool on;
+    float k[6], p[2], s[4];
+};
+
+__device__ __forceinline__ Distortion load_distortion(const float* __restrict__ radial,
+                                                      const float* __restrict__ tangential,
+                                                      const float* __restrict__ thin_prism) {
+    Distortion d;
+    d.on = radial != nullptr || tangential != nullptr || thin_prism != nullptr;
+#pragma unroll
+    for (int i = 0; i < 6; ++i)
+        d.k[i] = radial != nullptr ? radial[i] : 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+        d.p[i] = tangential != nullptr ? tangential[i] : 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        d.s[i] = thin_prism != nullptr ? thin_prism[i] : 0.f;
+    return d;
+}
+
+// Cameras.cuh:504-533
+__device__ __forceinline__ void compute_distortion(const Distortion& d, float u, float v, float* icD, float* delta_x,
+                                                   float* delta_y) {
+    const float uu = u * u, vv = v * v;
+    const float r2 = uu + vv;
+    const float a1 = 2.f * u * v;
+    const float a2 = r2 + 2.f * uu;
+    const float a3 = r2 + 2.f * vv;
+    const float num = 1.f + r2 * (d.k[0] + r2 * (d.k[1] + r2 * d.k[2]));
+    const float den = 1.f + r2 * (d.k[3] + r2 * (d.k[4] + r2 * d.k[5]));
+    *icD = num / den;
+    *delta_x = d.p[0] * a1 + d.p[1] * a2 + r2 * (d.s[0] + r2 * d.s[1]);
+    *delta_y = d.p[0] * a3 + d.p[1] * a1 + r2 * (d.s[2] + r2 * d.s[3]);
+}
+
+// Cameras.cuh:635-740: Newton undistortion, at most 5 steps.  The reference's double literals make parts of the
+// Jacobian double arithmetic; the expressions are kept as written there.  Returns "converged".
+__device__ __forceinline__ bool opencv_undistort_newton(const Distortion& d, float xd, float yd, float* xo, float* yo) {
+    const float k1 = d.k[0], k2 = d.k[1], k3 = d.k[2], k4 = d.k[3], k5 = d.k[4], k6 = d.k[5];
+    const float p1 = d.p[0], p2 = d.p[1], s1 = d.s[0], s2 = d.s[1], s3 = d.s[2], s4 = d.s[3];
+    float x = xd, y = yd;
+    const float eps = 1e-6f;
+    bool converged = false;
+    for (int iter = 0; iter < 5; ++iter) {
+        const float r = x * x + y * y;
+        const float r2 = r * r;
+        const float alpha = 1.0f + r * (k1 + r * (k2 + r * k3));
+        const float beta = 1.0f + r * (k4 + r * (k5 + r * k6));
+        const float dd = alpha / beta;
+        if (dd <= 0.f)
+            break;
+        const float fx = dd * x + 2 * p1 * x * y + p2 * (r + 2 * x * x) + s1 * r + s2 * r2 - xd;
+        const float fy = dd * y + 2 * p2 * x * y + p1 * (r + 2 * y * y) + s3 * r + s4 * r2 - yd;
+        const float alpha_r = k1 + r * (2.0 * k2 + r * (3.0 * k3));
+        const float beta_r = k4 + r * (2.0 * k5 + r * (3.0 * k6));
+        const float d_r = (alpha_r * beta - alpha * beta_r) / (beta * beta);
+        const float d_x = 2.0 * x * d_r;
+        const float d_y = 2.0 * y * d_r;
+        float fx_x = dd + d_x * x + 2.0 * p1 * y + 6.0 * p2 * x;
+        fx_x += 2.0 * x * (s1 + 2.0 * s2 * r);
+        float fx_y = d_y * x + 2.0 * p1 * x + 2.0 * p2 * y;
+        fx_y += 2.0 * y * (s1 + 2.0 * s2 * r);
+        float fy_x = d_x * y + 2.0 * p2 * y + 2.0 * p1 * x;
+        fy_x += 2.0 * x * (s3 + 2.0 * s4 * r);
+        float fy_y = dd + d_y * y + 2.0 * p2 * x + 6.0 * p1 * y;
+        fy_y += 2.0 * y * (s3 + 2.0 * s4 * r);
+        const float det = fx_y * fy_x - fx_x * fy_y;
+        if (gsx::fabs(det) < eps)
+            break;
+        const float dx = (fx * fy_y - fy * fx_y) / det;
+        const float dy = (fy * fx_x - fx * fy_x) / det;
+        x += dx;
+        y += dy;
+        if (gsx::fabs(dx) < eps && gsx::fabs(dy) < eps) {
+            converged = true;
+            break;
+        }
+    }
+    *xo = x;
+    *yo = y;
+    return converged;
+}
+
+// world ray through a pixel centre, (distorted) pinhole, global shutter (Cameras.cuh:457-470 / 742-755 unproject,
+// :253-266 camera_ray_to_world_ray, :322-339).  Returns the ray's valid flag: false only when an undistortion did
+// not converge (the ray is then zero, :330-333, and the pixel takes no part in either pass).
+__device__ __forceinline__ bool pixel_world_ray(const CamPose& cp, float px, float py, float fx, float fy, float cx,
+                                                float cy, const Distortion& dist, vec3* ray_o, vec3* ray_d) {
+    float u = (px - cx) / fx;
+    float v = (py - cy) / fy;
+    if (dist.on && !opencv_undistort_newton(dist, u, v, &u, &v)) {
+        *ray_o = mk3(0.f, 0.f, 0.f);
+        *ray_d = mk3(0.f, 0.f, 0.f);
+        return false;
+    }
     const vec3 cr = mk3(u, v, 1.f);
     const float len = gsx::sqrt(dot(cr, cr));
     const vec3 d_cam = mk3(cr.x / len, cr.y / len, cr.z / len);
@@ -92,6 +186,7 @@ __device__ __forceinline__ void pixel_world_ray(const CamPose& cp, float px, flo
     const mat3 R_inv = mat3_cast(quat_inverse(q));
     *ray_o = neg(mul(R_inv, t));
     *ray_d = mul(R_inv, d_cam);
+    return true;
 }
 
 // camera centre in world space exactly as the rasterizers form it (Cameras.cuh:253-266 with the start pose)

@@ -40,8 +40,10 @@ struct RecordRegion {
 };
 
 // viewmat: row-major [4,4] world->camera.  gro / M as stored in the record.
+// pinhole = false (a distorted camera: straight lines of rays are not straight lines of pixels): only the power
+// cut-off is claimed, the pixel region is "everywhere".
 GSX_HD RecordRegion record_region(vec3 gro, const mat3& M, float opacity, vec3 mean, const float* viewmat, float fx,
-                                  float fy, float cx, float cy, uint32_t W, uint32_t H) {
+                                  float fy, float cx, float cy, uint32_t W, uint32_t H, bool pinhole = true) {
     RecordRegion full = {0, 0, (int32_t)W - 1, (int32_t)H - 1, kPowerFloor, 0.f, 0.f, 0.f, 0.f, 0.f};
     RecordRegion empty = {1, 1, 0, 0, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     if (!(opacity > 0.f))
@@ -56,6 +58,8 @@ GSX_HD RecordRegion record_region(vec3 gro, const mat3& M, float opacity, vec3 m
     // the cut-off is compared with the power the kernel itself computes, so it only needs room for the rounding of
     // exp and log: o exp(cut) < 1/255 by 0.4 %
     full.cut = gsx::fmax(fma(-0.5f, k, -0.004f), kPowerFloor);
+    if (!pinhole)
+        return full;
     // the geometric region is derived in exact arithmetic: inflate k for the rounding of the kernel's d^2
     const float g2 = dot(gro, gro);
     k = fma(k, 1.002f, 0.004f) + 4e-6f * gsx::sqrt(g2 * k);

@@ -30,6 +30,7 @@ struct ProjCfg {
     float ut_alpha, ut_beta, ut_kappa, ut_margin;
     int ut_require_all;
     float fx, fy, cx, cy;
+    Distortion dist; // OpenCV pinhole distortion; dist.on = false: the perfect pinhole model
 };
 
 __device__ __forceinline__ bool pinhole_project(vec3 cam, const ProjCfg& cfg, vec2* out) {
@@ -42,6 +43,26 @@ __device__ __forceinline__ bool pinhole_project(vec3 cam, const ProjCfg& cfg, ve
     const float mx = (float)cfg.W * cfg.ut_margin;
     const float my = (float)cfg.H * cfg.ut_margin;
     bool valid = true;
+    valid &= (-mx) <= out->x && out->x < ((float)cfg.W + mx);
+    valid &= (-my) <= out->y && out->y < ((float)cfg.H + my);
+    return valid;
+}
+
+// Cameras.cuh:535-597: camera_ray_to_image_point of the distorted model
+__device__ __forceinline__ bool opencv_project(vec3 cam, const ProjCfg& cfg, vec2* out) {
+    out->x = 0.f;
+    out->y = 0.f;
+    if (cam.z <= 0.f)
+        return false;
+    const float u = cam.x / cam.z, v = cam.y / cam.z;
+    float icD, dx, dy;
+    compute_distortion(cfg.dist, u, v, &icD, &dx, &dy);
+    const bool valid_radial = icD > 0.8f;
+    out->x = (icD * u + dx) * cfg.fx + cfg.cx;
+    out->y = (icD * v + dy) * cfg.fy + cfg.cy;
+    const float mx = (float)cfg.W * cfg.ut_margin;
+    const float my = (float)cfg.H * cfg.ut_margin;
+    bool valid = valid_radial;
     valid &= (-mx) <= out->x && out->x < ((float)cfg.W + mx);
     valid &= (-my) <= out->y && out->y < ((float)cfg.H + my);
     return valid;
@@ -82,7 +103,7 @@ __device__ __forceinline__ bool project_ut(const ProjCfg& cfg, const CamPose& cp
         }
         const vec3 pc = add(quat_rotate(cp.q_start, p), cp.t_start);
         vec2 uv;
-        const bool pv = pinhole_project(pc, cfg, &uv);
+        const bool pv = cfg.dist.on ? opencv_project(pc, cfg, &uv) : pinhole_project(pc, cfg, &uv);
         if (cfg.ut_require_all) {
             valid &= pv;
             if (!pv)
@@ -149,12 +170,16 @@ __device__ __forceinline__ bool project_ut(const ProjCfg& cfg, const CamPose& cp
 __global__ void __launch_bounds__(256) projection_ut_kernel(
     uint32_t C, uint32_t N, const float* __restrict__ means, const float* __restrict__ quats,
     const float* __restrict__ scales, const float* __restrict__ opacities, const float* __restrict__ viewmats0,
-    const float* __restrict__ Ks, ProjCfg cfg, int32_t* __restrict__ radii, float* __restrict__ means2d,
+    const float* __restrict__ Ks, const float* __restrict__ radial, const float* __restrict__ tangential,
+    const float* __restrict__ thin_prism, ProjCfg cfg, int32_t* __restrict__ radii, float* __restrict__ means2d,
     float* __restrict__ depths, float* __restrict__ conics, float* __restrict__ compensations) {
     const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
     if (idx >= C * N)
         return;
     const uint32_t cid = idx / N, gid = idx % N;
+    cfg.dist = load_distortion(radial != nullptr ? radial + cid * 6 : nullptr,
+                               tangential != nullptr ? tangential + cid * 2 : nullptr,
+                               thin_prism != nullptr ? thin_prism + cid * 4 : nullptr);
     cfg.fx = Ks[cid * 9 + 0];
     cfg.fy = Ks[cid * 9 + 4];
     cfg.cx = Ks[cid * 9 + 2];
@@ -643,9 +668,10 @@ extern "C" int gsx_projection_ut_3dgs_fused(
     cfg.ut_margin = ut.in_image_margin_factor;
     cfg.ut_require_all = ut.require_all_sigma_points_valid;
     cfg.fx = cfg.fy = cfg.cx = cfg.cy = 0.f;
+    memset(&cfg.dist, 0, sizeof(cfg.dist));
     hipLaunchKernelGGL(projection_ut_kernel, dim3(cdiv((uint64_t)C * N, 256)), dim3(256), 0, (hipStream_t)stream, C,
-                       N, means, quats, scales, opacities, viewmats0, Ks, cfg, radii, means2d, depths, conics,
-                       compensations);
+                       N, means, quats, scales, opacities, viewmats0, Ks, radial_coeffs, tangential_coeffs,
+                       thin_prism_coeffs, cfg, radii, means2d, depths, conics, compensations);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

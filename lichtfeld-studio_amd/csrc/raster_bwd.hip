@@ -47,12 +47,13 @@ __global__ void __launch_bounds__(64) wave_reduce16_probe_kernel(const float* __
 // CDIM = 3: the RGB training path.  CDIM = 1 / 4: the depth render modes (Rasterization.cpp:374-393) - one colour
 // channel, or RGB plus a fourth channel that is staged from `colors` and whose per-Gaussian gradient is reduced
 // on its own into gextra [N].
-template <uint32_t CDIM>
+template <uint32_t CDIM, bool DIST>
 __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     uint32_t n_isects, const float4* __restrict__ records, const float* __restrict__ colors,
     const float* __restrict__ backgrounds,
     const uint8_t* __restrict__ masks, uint32_t image_width, uint32_t image_height, uint32_t tile_width,
     uint32_t tile_height, const float* __restrict__ viewmat, const float* __restrict__ Kmat,
+    const float* __restrict__ radial, const float* __restrict__ tangential, const float* __restrict__ thin_prism,
     const int32_t* __restrict__ tile_offsets, const int32_t* __restrict__ flatten_ids,
     const float* __restrict__ render_alphas, const int32_t* __restrict__ last_ids,
     const float* __restrict__ v_render_colors, const float* __restrict__ v_render_alphas,
@@ -75,13 +76,19 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     const uint32_t lane = tr & 63u;
     const TilePixel px = tile_pixel(tile_id, tile_width, tr);
     const uint32_t i = px.i, j = px.j;
-    const bool inside = (i < image_height && j < image_width);
+    bool inside = (i < image_height && j < image_width);
     const uint32_t pix_id = min(i * image_width + j, image_width * image_height - 1); // :92-93
     uint8_t* wave_list = lists[tr >> 6];
 
     const CamPose cp = load_cam_pose(viewmat);
     vec3 ray_o, ray_d;
-    pixel_world_ray(cp, (float)j + 0.5f, (float)i + 0.5f, Kmat[0], Kmat[4], Kmat[2], Kmat[5], &ray_o, &ray_d);
+    Distortion dist;
+    dist.on = false;
+    if (DIST)
+        dist = load_distortion(radial, tangential, thin_prism);
+    // a pixel without a valid ray takes no part (RasterizeToPixelsFromWorld3DGSBwd.cu:157)
+    inside &= pixel_world_ray(cp, (float)j + 0.5f, (float)i + 0.5f, Kmat[0], Kmat[4], Kmat[2], Kmat[5], dist, &ray_o,
+                              &ray_d);
 
     const int32_t range_start = tile_offsets[tile_id];
     int32_t range_end = (tile_id == tile_width * tile_height - 1) ? (int32_t)n_isects : tile_offsets[tile_id + 1];
@@ -339,16 +346,20 @@ extern "C" int gsx_rasterize_bwd_clear(uint32_t N, void* workspace, size_t works
     return GSX_OK;
 }
 
-// stage 2: the per-tile kernel, accumulating into the workspace; `records` from gsx_pack_raster_records (or the
-// fused per-Gaussian pass) for the same camera and parameters
-extern "C" int gsx_rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isects, const void* records,
-                                            const float* colors, uint32_t channels, const float* backgrounds,
-                                            const uint8_t* masks, uint32_t image_width,
-                                            uint32_t image_height, uint32_t tile_size, const float* viewmats0,
-                                            const float* Ks, const int32_t* tile_offsets, const int32_t* flatten_ids,
-                                            const float* render_alphas, const int32_t* last_ids,
-                                            const float* v_render_colors, const float* v_render_alphas,
-                                            void* workspace, size_t workspace_bytes, void* stream) {
+namespace gsx {
+int pack_raster_records(uint32_t N, const float* means, const float* quats, const float* scales,
+                        const float* opacities, const float* colors, uint32_t channels, const float* viewmat,
+                        const float* K, uint32_t image_width, uint32_t image_height, bool pinhole, void* records,
+                        void* stream); // raster_fwd.hip
+
+static int rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isects, const void* records,
+                                    const float* colors, uint32_t channels, const float* backgrounds,
+                                    const uint8_t* masks, uint32_t image_width, uint32_t image_height,
+                                    uint32_t tile_size, const float* viewmats0, const float* Ks, const float* radial,
+                                    const float* tangential, const float* thin_prism, const int32_t* tile_offsets,
+                                    const int32_t* flatten_ids, const float* render_alphas, const int32_t* last_ids,
+                                    const float* v_render_colors, const float* v_render_alphas, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
     GSX_REQUIRE(C == 1, GSX_ERR_UNSUPPORTED, "C = %u cameras: only C == 1 is supported", C);
     if (N == 0 || n_isects == 0 || image_width == 0 || image_height == 0) // ...Bwd.cu:440-443
         return GSX_OK;
@@ -367,19 +378,44 @@ extern "C" int gsx_rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_is
     GSX_REQUIRE(channels <= 3 || colors != nullptr, GSX_ERR_INVALID_ARGUMENT, "rasterize bwd: colors is null");
     const uint32_t tw = cdiv(image_width, kTile), th = cdiv(image_height, kTile);
     float* gextra = (float*)((char*)workspace + accum_extra_offset(N));
-#define GSX_LAUNCH_BWD(CD)                                                                                           \
-    hipLaunchKernelGGL((rasterize_bwd_kernel<CD>), dim3(tw * th), dim3(256), 0, (hipStream_t)stream,                 \
+    const bool distorted = radial != nullptr || tangential != nullptr || thin_prism != nullptr;
+#define GSX_LAUNCH_BWD(CD, DI)                                                                                       \
+    hipLaunchKernelGGL((rasterize_bwd_kernel<CD, DI>), dim3(tw * th), dim3(256), 0, (hipStream_t)stream,             \
                        (uint32_t)n_isects, (const float4*)records, colors, backgrounds, masks, image_width,          \
-                       image_height, tw, th, viewmats0, Ks, tile_offsets, flatten_ids, render_alphas, last_ids,      \
-                       v_render_colors, v_render_alphas, (float*)workspace, gextra)
+                       image_height, tw, th, viewmats0, Ks, radial, tangential, thin_prism, tile_offsets,            \
+                       flatten_ids, render_alphas, last_ids, v_render_colors, v_render_alphas, (float*)workspace,    \
+                       gextra)
+#define GSX_LAUNCH_BWD2(CD)       \
+    if (distorted)                \
+        GSX_LAUNCH_BWD(CD, true); \
+    else                          \
+        GSX_LAUNCH_BWD(CD, false)
     switch (channels) {
-    case 1: GSX_LAUNCH_BWD(1); break;
-    case 3: GSX_LAUNCH_BWD(3); break;
-    default: GSX_LAUNCH_BWD(4); break;
+    case 1: GSX_LAUNCH_BWD2(1); break;
+    case 3: GSX_LAUNCH_BWD2(3); break;
+    default: GSX_LAUNCH_BWD2(4); break;
     }
+#undef GSX_LAUNCH_BWD2
 #undef GSX_LAUNCH_BWD
     GSX_LAUNCH_CHECK();
     return GSX_OK;
+}
+} // namespace gsx
+
+// stage 2: the per-tile kernel, accumulating into the workspace; `records` from gsx_pack_raster_records (or the
+// fused per-Gaussian pass) for the same camera and parameters
+extern "C" int gsx_rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isects, const void* records,
+                                            const float* colors, uint32_t channels, const float* backgrounds,
+                                            const uint8_t* masks, uint32_t image_width,
+                                            uint32_t image_height, uint32_t tile_size, const float* viewmats0,
+                                            const float* Ks, const int32_t* tile_offsets, const int32_t* flatten_ids,
+                                            const float* render_alphas, const int32_t* last_ids,
+                                            const float* v_render_colors, const float* v_render_alphas,
+                                            void* workspace, size_t workspace_bytes, void* stream) {
+    return rasterize_bwd_accumulate(C, N, n_isects, records, colors, channels, backgrounds, masks, image_width,
+                                    image_height, tile_size, viewmats0, Ks, nullptr, nullptr, nullptr, tile_offsets,
+                                    flatten_ids, render_alphas, last_ids, v_render_colors, v_render_alphas, workspace,
+                                    workspace_bytes, stream);
 }
 
 // stage 3: per-Gaussian epilogue, accumulators -> the five gradient tensors (all elements written)
@@ -428,13 +464,14 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
     void* records = (char*)workspace + acc_bytes;
     if ((rc = gsx_rasterize_bwd_clear(N, workspace, acc_bytes, stream)) != GSX_OK)
         return rc;
-    if ((rc = gsx_pack_raster_records(N, means, quats, scales, opacities, colors, channels, viewmats0, Ks, image_width,
-                                      image_height, records, stream)) != GSX_OK)
+    const bool pinhole = !(radial_coeffs || tangential_coeffs || thin_prism_coeffs);
+    if ((rc = pack_raster_records(N, means, quats, scales, opacities, colors, channels, viewmats0, Ks, image_width,
+                                  image_height, pinhole, records, stream)) != GSX_OK)
         return rc;
-    if ((rc = gsx_rasterize_bwd_accumulate(C, N, n_isects, records, colors, channels, backgrounds, masks, image_width,
-                                           image_height, tile_size, viewmats0, Ks, tile_offsets, flatten_ids,
-                                           render_alphas, last_ids, v_render_colors, v_render_alphas, workspace,
-                                           acc_bytes, stream)) != GSX_OK)
+    if ((rc = rasterize_bwd_accumulate(C, N, n_isects, records, colors, channels, backgrounds, masks, image_width,
+                                       image_height, tile_size, viewmats0, Ks, radial_coeffs, tangential_coeffs,
+                                       thin_prism_coeffs, tile_offsets, flatten_ids, render_alphas, last_ids,
+                                       v_render_colors, v_render_alphas, workspace, acc_bytes, stream)) != GSX_OK)
         return rc;
     return gsx_rasterize_bwd_finish(N, means, quats, scales, viewmats0, workspace, acc_bytes, 0, channels, v_means,
                                     v_quats, v_scales, v_colors, v_opacities, stream);

@@ -23,7 +23,7 @@ __global__ void __launch_bounds__(256) pack_records_kernel(uint32_t N, const flo
                                                             const float* __restrict__ colors,
                                                             const float* __restrict__ viewmat,
                                                             const float* __restrict__ Kmat, uint32_t W, uint32_t H,
-                                                            float4* __restrict__ records) {
+                                                            bool pinhole, float4* __restrict__ records) {
     const uint32_t g = blockIdx.x * 256u + threadIdx.x;
     if (g >= N)
         return;
@@ -32,7 +32,8 @@ __global__ void __launch_bounds__(256) pack_records_kernel(uint32_t N, const flo
     const float opac = opacities[g];
     const mat3 M = record_whitening(ld4q(quats, g), ld3(scales, g));
     const vec3 gro = mul(M, sub(ray_o, xyz));
-    const RecordRegion b = record_region(gro, M, opac, xyz, viewmat, Kmat[0], Kmat[4], Kmat[2], Kmat[5], W, H);
+    const RecordRegion b =
+        record_region(gro, M, opac, xyz, viewmat, Kmat[0], Kmat[4], Kmat[2], Kmat[5], W, H, pinhole);
     const float c0 = colors[(size_t)g * CDIM];
     const float c1 = CDIM > 1 ? colors[(size_t)g * CDIM + 1] : 0.f;
     const float c2 = CDIM > 2 ? colors[(size_t)g * CDIM + 2] : 0.f;
@@ -43,12 +44,15 @@ __global__ void __launch_bounds__(256) pack_records_kernel(uint32_t N, const flo
 // [1] += pairs composited, [2] += pairs the backward pass walks (entries up to each pixel's last contributor),
 // [3] += (wave, Gaussian) iterations executed, [4] += (wave, Gaussian) iterations removed by the pixel bounds,
 // [5] += executed iterations in which at least one pixel reaches the alpha threshold.
-template <uint32_t CDIM, bool STATS>
+// DIST: OpenCV pinhole distortion (each pixel's ray comes from a Newton undistortion; a pixel whose undistortion
+// does not converge is done from the start, RasterizeToPixelsFromWorld3DGSFwd.cu:145).
+template <uint32_t CDIM, bool STATS, bool DIST>
 __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
     uint32_t n_isects, const float4* __restrict__ records, const float* __restrict__ colors,
     const float* __restrict__ backgrounds, const uint8_t* __restrict__ masks, uint32_t image_width,
     uint32_t image_height, uint32_t tile_width, uint32_t tile_height, const float* __restrict__ viewmat,
-    const float* __restrict__ Kmat, const int32_t* __restrict__ tile_offsets,
+    const float* __restrict__ Kmat, const float* __restrict__ radial, const float* __restrict__ tangential,
+    const float* __restrict__ thin_prism, const int32_t* __restrict__ tile_offsets,
     const int32_t* __restrict__ flatten_ids, float* __restrict__ render_colors, float* __restrict__ render_alphas,
     int32_t* __restrict__ last_ids, unsigned long long* __restrict__ stats) {
     __shared__ float4 stage[kBatch * 4];
@@ -78,14 +82,19 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
 
     const CamPose cp = load_cam_pose(viewmat);
     vec3 ray_o, ray_d;
-    pixel_world_ray(cp, (float)j + 0.5f, (float)i + 0.5f, Kmat[0], Kmat[4], Kmat[2], Kmat[5], &ray_o, &ray_d);
+    Distortion dist;
+    dist.on = false;
+    if (DIST)
+        dist = load_distortion(radial, tangential, thin_prism);
+    const bool ray_ok =
+        pixel_world_ray(cp, (float)j + 0.5f, (float)i + 0.5f, Kmat[0], Kmat[4], Kmat[2], Kmat[5], dist, &ray_o, &ray_d);
 
     const int32_t range_start = tile_offsets[tile_id];
     const int32_t range_end =
         (tile_id == tile_width * tile_height - 1) ? (int32_t)n_isects : tile_offsets[tile_id + 1];
     const uint32_t num_batches = (uint32_t)(range_end - range_start + (int32_t)kBatch - 1) / kBatch;
 
-    bool done = !inside;
+    bool done = !inside || !ray_ok;
     float T = 1.0f;
     uint32_t cur_idx = 0;
     float pix_out[CDIM];
@@ -206,10 +215,11 @@ using namespace gsx;
 
 extern "C" size_t gsx_raster_records_bytes(uint32_t N) { return align_up((size_t)N * kRecordFloats * 4, 256); }
 
-extern "C" int gsx_pack_raster_records(uint32_t N, const float* means, const float* quats, const float* scales,
-                                       const float* opacities, const float* colors, uint32_t channels,
-                                       const float* viewmat, const float* K, uint32_t image_width,
-                                       uint32_t image_height, void* records, void* stream) {
+namespace gsx {
+int pack_raster_records(uint32_t N, const float* means, const float* quats, const float* scales,
+                        const float* opacities, const float* colors, uint32_t channels, const float* viewmat,
+                        const float* K, uint32_t image_width, uint32_t image_height, bool pinhole, void* records,
+                        void* stream) {
     if (N == 0)
         return GSX_OK;
     GSX_REQUIRE(means && quats && scales && opacities && colors && viewmat && K && records, GSX_ERR_INVALID_ARGUMENT,
@@ -219,7 +229,7 @@ extern "C" int gsx_pack_raster_records(uint32_t N, const float* means, const flo
     hipStream_t s = (hipStream_t)stream;
 #define GSX_LAUNCH_PACK(CD)                                                                                         \
     hipLaunchKernelGGL((pack_records_kernel<CD>), grid, block, 0, s, N, means, quats, scales, opacities, colors,    \
-                       viewmat, K, image_width, image_height, (float4*)records)
+                       viewmat, K, image_width, image_height, pinhole, (float4*)records)
     switch (channels) {
     case 1: GSX_LAUNCH_PACK(1); break;
     case 3: GSX_LAUNCH_PACK(3); break;
@@ -233,12 +243,11 @@ extern "C" int gsx_pack_raster_records(uint32_t N, const float* means, const flo
     return GSX_OK;
 }
 
-extern "C" int gsx_rasterize_records_fwd(int64_t n_isects, const void* records, const float* colors,
-                                         uint32_t channels, const float* backgrounds, const uint8_t* masks,
-                                         uint32_t image_width, uint32_t image_height, const float* viewmat,
-                                         const float* K, const int32_t* tile_offsets, const int32_t* flatten_ids,
-                                         float* render_colors, float* render_alphas, int32_t* last_ids,
-                                         void* stream) {
+int rasterize_records_fwd(int64_t n_isects, const void* records, const float* colors, uint32_t channels,
+                          const float* backgrounds, const uint8_t* masks, uint32_t image_width, uint32_t image_height,
+                          const float* viewmat, const float* K, const float* radial, const float* tangential,
+                          const float* thin_prism, const int32_t* tile_offsets, const int32_t* flatten_ids,
+                          float* render_colors, float* render_alphas, int32_t* last_ids, void* stream) {
     if (image_width == 0 || image_height == 0)
         return GSX_OK;
     GSX_REQUIRE(n_isects >= 0 && n_isects < (1ll << 31), GSX_ERR_OVERFLOW, "rasterize fwd: n_isects out of range");
@@ -249,22 +258,49 @@ extern "C" int gsx_rasterize_records_fwd(int64_t n_isects, const void* records, 
     const uint32_t tw = cdiv(image_width, kTile), th = cdiv(image_height, kTile);
     const dim3 grid(tw * th), block(256);
     hipStream_t s = (hipStream_t)stream;
-#define GSX_LAUNCH_FWD(CD)                                                                                          \
-    hipLaunchKernelGGL((rasterize_fwd_kernel<CD, false>), grid, block, 0, s, (uint32_t)n_isects,                    \
+    const bool distorted = radial != nullptr || tangential != nullptr || thin_prism != nullptr;
+#define GSX_LAUNCH_FWD(CD, DI)                                                                                      \
+    hipLaunchKernelGGL((rasterize_fwd_kernel<CD, false, DI>), grid, block, 0, s, (uint32_t)n_isects,                \
                        (const float4*)records, colors, backgrounds, masks, image_width, image_height, tw, th,       \
-                       viewmat, K, tile_offsets, flatten_ids, render_colors, render_alphas, last_ids,               \
-                       (unsigned long long*)nullptr)
+                       viewmat, K, radial, tangential, thin_prism, tile_offsets, flatten_ids, render_colors,        \
+                       render_alphas, last_ids, (unsigned long long*)nullptr)
+#define GSX_LAUNCH_FWD2(CD)     \
+    if (distorted)              \
+        GSX_LAUNCH_FWD(CD, true); \
+    else                        \
+        GSX_LAUNCH_FWD(CD, false)
     switch (channels) { // the channel counts the render modes of Rasterization.cpp:374-393 produce
-    case 1: GSX_LAUNCH_FWD(1); break;
-    case 3: GSX_LAUNCH_FWD(3); break;
-    case 4: GSX_LAUNCH_FWD(4); break;
+    case 1: GSX_LAUNCH_FWD2(1); break;
+    case 3: GSX_LAUNCH_FWD2(3); break;
+    case 4: GSX_LAUNCH_FWD2(4); break;
     default:
         set_error("rasterize fwd: %u channels (built: 1, 3, 4)", channels);
         return GSX_ERR_UNSUPPORTED;
     }
+#undef GSX_LAUNCH_FWD2
 #undef GSX_LAUNCH_FWD
     GSX_LAUNCH_CHECK();
     return GSX_OK;
+}
+} // namespace gsx
+
+extern "C" int gsx_pack_raster_records(uint32_t N, const float* means, const float* quats, const float* scales,
+                                       const float* opacities, const float* colors, uint32_t channels,
+                                       const float* viewmat, const float* K, uint32_t image_width,
+                                       uint32_t image_height, void* records, void* stream) {
+    return pack_raster_records(N, means, quats, scales, opacities, colors, channels, viewmat, K, image_width,
+                               image_height, true, records, stream);
+}
+
+extern "C" int gsx_rasterize_records_fwd(int64_t n_isects, const void* records, const float* colors,
+                                         uint32_t channels, const float* backgrounds, const uint8_t* masks,
+                                         uint32_t image_width, uint32_t image_height, const float* viewmat,
+                                         const float* K, const int32_t* tile_offsets, const int32_t* flatten_ids,
+                                         float* render_colors, float* render_alphas, int32_t* last_ids,
+                                         void* stream) {
+    return rasterize_records_fwd(n_isects, records, colors, channels, backgrounds, masks, image_width, image_height,
+                                 viewmat, K, nullptr, nullptr, nullptr, tile_offsets, flatten_ids, render_colors,
+                                 render_alphas, last_ids, stream);
 }
 
 extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
@@ -293,13 +329,14 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
                         workspace_bytes >= gsx_raster_records_bytes(N),
                     GSX_ERR_WORKSPACE, "rasterize fwd: workspace needs %zu bytes, 256-byte aligned",
                     gsx_raster_records_bytes(N));
-        if ((rc = gsx_pack_raster_records(N, means, quats, scales, opacities, colors, channels, viewmats0, Ks,
-                                          image_width, image_height, workspace, stream)) != GSX_OK)
+        const bool pinhole = !(radial_coeffs || tangential_coeffs || thin_prism_coeffs);
+        if ((rc = pack_raster_records(N, means, quats, scales, opacities, colors, channels, viewmats0, Ks, image_width,
+                                      image_height, pinhole, workspace, stream)) != GSX_OK)
             return rc;
     }
-    return gsx_rasterize_records_fwd(n_isects, workspace, colors, channels, backgrounds, masks, image_width,
-                                     image_height, viewmats0, Ks, tile_offsets, flatten_ids, render_colors,
-                                     render_alphas, last_ids, stream);
+    return rasterize_records_fwd(n_isects, workspace, colors, channels, backgrounds, masks, image_width, image_height,
+                                 viewmats0, Ks, radial_coeffs, tangential_coeffs, thin_prism_coeffs, tile_offsets,
+                                 flatten_ids, render_colors, render_alphas, last_ids, stream);
 }
 
 // Pair counts of one forward pass (no counterpart in the reference; used to turn kernel times into flop rates).
@@ -312,10 +349,11 @@ extern "C" int gsx_rasterize_pair_stats(int64_t n_isects, const void* records, u
     GSX_REQUIRE(records && viewmat && K && tile_offsets && flatten_ids && stats_out, GSX_ERR_INVALID_ARGUMENT,
                 "rasterize_pair_stats: null tensor");
     const uint32_t tw = cdiv(image_width, kTile), th = cdiv(image_height, kTile);
-    hipLaunchKernelGGL((rasterize_fwd_kernel<3, true>), dim3(tw * th), dim3(256), 0, (hipStream_t)stream,
+    hipLaunchKernelGGL((rasterize_fwd_kernel<3, true, false>), dim3(tw * th), dim3(256), 0, (hipStream_t)stream,
                        (uint32_t)n_isects, (const float4*)records, (const float*)nullptr, (const float*)nullptr,
-                       (const uint8_t*)nullptr, image_width, image_height, tw, th, viewmat, K, tile_offsets,
-                       flatten_ids, (float*)nullptr, (float*)nullptr, (int32_t*)nullptr, stats_out);
+                       (const uint8_t*)nullptr, image_width, image_height, tw, th, viewmat, K, (const float*)nullptr,
+                       (const float*)nullptr, (const float*)nullptr, tile_offsets, flatten_ids, (float*)nullptr,
+                       (float*)nullptr, (int32_t*)nullptr, stats_out);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

@@ -106,12 +106,117 @@ bool pinhole_project(vec3 cam, float fx, float fy, float cx, float cy, uint32_t 
     return valid;
 }
 
-// Cameras.cuh:457-470 + 253-266 + 322-339 : pixel centre -> world ray, global shutter
-// (relative frame time 0 because shutter_relative_frame_time has no GLOBAL case, :293-320).
-void pixel_world_ray(float px, float py, float fx, float fy, float cx, float cy,
+// OpenCV pinhole model with radial (6), tangential (2) and thin-prism (4) distortion (Cameras.cuh:473-815).  The
+// coefficients are process-wide checker state set by orc_set_distortion (off = the perfect pinhole model): every
+// function below that projects a point or casts a pixel ray consults it, like the reference's dispatch on
+// "any coefficient pointer given" (ProjectionUT3DGSFused.cu:86-113, RasterizeToPixelsFromWorld3DGSFwd.cu:90-116).
+struct Distortion {
+    bool on = false;
+    float k[6] = {0, 0, 0, 0, 0, 0}, p[2] = {0, 0}, s[4] = {0, 0, 0, 0};
+};
+Distortion g_dist;
+
+// Cameras.cuh:504-533
+void compute_distortion(const Distortion& d, float u, float v, float* icD, float* delta_x, float* delta_y) {
+    const float uu = u * u, vv = v * v;
+    const float r2 = uu + vv;
+    const float a1 = 2.f * u * v;
+    const float a2 = r2 + 2.f * uu;
+    const float a3 = r2 + 2.f * vv;
+    const float num = 1.f + r2 * (d.k[0] + r2 * (d.k[1] + r2 * d.k[2]));
+    const float den = 1.f + r2 * (d.k[3] + r2 * (d.k[4] + r2 * d.k[5]));
+    *icD = num / den;
+    *delta_x = d.p[0] * a1 + d.p[1] * a2 + r2 * (d.s[0] + r2 * d.s[1]);
+    *delta_y = d.p[0] * a3 + d.p[1] * a1 + r2 * (d.s[2] + r2 * d.s[3]);
+}
+
+// Cameras.cuh:535-597 : camera_ray_to_image_point of the distorted model
+bool opencv_project(const Distortion& d, vec3 cam, float fx, float fy, float cx, float cy, uint32_t W, uint32_t H,
+                    float margin_factor, vec2* out) {
+    out->x = 0.f;
+    out->y = 0.f;
+    if (cam.z <= 0.f)
+        return false;
+    const float u = cam.x / cam.z, v = cam.y / cam.z;
+    float icD, dx, dy;
+    compute_distortion(d, u, v, &icD, &dx, &dy);
+    const bool valid_radial = icD > 0.8f;
+    out->x = (icD * u + dx) * fx + cx;
+    out->y = (icD * v + dy) * fy + cy;
+    const float mx = (float)W * margin_factor;
+    const float my = (float)H * margin_factor;
+    bool valid = valid_radial;
+    valid &= (-mx) <= out->x && out->x < ((float)W + mx);
+    valid &= (-my) <= out->y && out->y < ((float)H + my);
+    return valid;
+}
+
+bool project_point(vec3 cam, float fx, float fy, float cx, float cy, uint32_t W, uint32_t H, float margin_factor,
+                   vec2* out) {
+    return g_dist.on ? opencv_project(g_dist, cam, fx, fy, cx, cy, W, H, margin_factor, out)
+                     : pinhole_project(cam, fx, fy, cx, cy, W, H, margin_factor, out);
+}
+
+// Cameras.cuh:635-740 : Newton undistortion (at most 5 steps, stop at |step| < 1e-6).  The reference's double
+// literals make parts of the Jacobian double arithmetic; the expressions are kept as written there.
+bool opencv_undistort_newton(const Distortion& d, float xd, float yd, float* xo, float* yo) {
+    const float k1 = d.k[0], k2 = d.k[1], k3 = d.k[2], k4 = d.k[3], k5 = d.k[4], k6 = d.k[5];
+    const float p1 = d.p[0], p2 = d.p[1], s1 = d.s[0], s2 = d.s[1], s3 = d.s[2], s4 = d.s[3];
+    float x = xd, y = yd;
+    const float eps = 1e-6f;
+    bool converged = false;
+    for (int iter = 0; iter < 5; ++iter) {
+        const float r = x * x + y * y;
+        const float r2 = r * r;
+        const float alpha = 1.0f + r * (k1 + r * (k2 + r * k3));
+        const float beta = 1.0f + r * (k4 + r * (k5 + r * k6));
+        const float dd = alpha / beta;
+        if (dd <= 0.f)
+            break;
+        const float fx = dd * x + 2 * p1 * x * y + p2 * (r + 2 * x * x) + s1 * r + s2 * r2 - xd;
+        const float fy = dd * y + 2 * p2 * x * y + p1 * (r + 2 * y * y) + s3 * r + s4 * r2 - yd;
+        const float alpha_r = k1 + r * (2.0 * k2 + r * (3.0 * k3));
+        const float beta_r = k4 + r * (2.0 * k5 + r * (3.0 * k6));
+        const float d_r = (alpha_r * beta - alpha * beta_r) / (beta * beta);
+        const float d_x = 2.0 * x * d_r;
+        const float d_y = 2.0 * y * d_r;
+        float fx_x = dd + d_x * x + 2.0 * p1 * y + 6.0 * p2 * x;
+        fx_x += 2.0 * x * (s1 + 2.0 * s2 * r);
+        float fx_y = d_y * x + 2.0 * p1 * x + 2.0 * p2 * y;
+        fx_y += 2.0 * y * (s1 + 2.0 * s2 * r);
+        float fy_x = d_x * y + 2.0 * p2 * y + 2.0 * p1 * x;
+        fy_x += 2.0 * x * (s3 + 2.0 * s4 * r);
+        float fy_y = dd + d_y * y + 2.0 * p2 * x + 6.0 * p1 * y;
+        fy_y += 2.0 * y * (s3 + 2.0 * s4 * r);
+        const float det = fx_y * fy_x - fx_x * fy_y;
+        if (gsx::fabs(det) < eps)
+            break;
+        const float dx = (fx * fy_y - fy * fx_y) / det;
+        const float dy = (fy * fx_x - fx * fy_x) / det;
+        x += dx;
+        y += dy;
+        if (gsx::fabs(dx) < eps && gsx::fabs(dy) < eps) {
+            converged = true;
+            break;
+        }
+    }
+    *xo = x;
+    *yo = y;
+    return converged;
+}
+
+// Cameras.cuh:457-470 / 742-755 + 253-266 + 322-339 : pixel centre -> world ray, global shutter (relative frame
+// time 0 because shutter_relative_frame_time has no GLOBAL case, :293-320).  Returns the ray's valid flag (false
+// only when the undistortion did not converge; then the ray is zero, :330-333).
+bool pixel_world_ray(float px, float py, float fx, float fy, float cx, float cy,
                      const RollingShutter& rs, vec3* ray_o, vec3* ray_d) {
-    const float u = (px - cx) / fx;
-    const float v = (py - cy) / fy;
+    float u = (px - cx) / fx;
+    float v = (py - cy) / fy;
+    if (g_dist.on && !opencv_undistort_newton(g_dist, u, v, &u, &v)) {
+        *ray_o = gsx::mk3(0.f, 0.f, 0.f);
+        *ray_d = gsx::mk3(0.f, 0.f, 0.f);
+        return false;
+    }
     const vec3 cr = gsx::mk3(u, v, 1.f);
     const float len = gsx::sqrt(gsx::dot(cr, cr));
     const vec3 d_cam = gsx::mk3(cr.x / len, cr.y / len, cr.z / len);
@@ -119,6 +224,7 @@ void pixel_world_ray(float px, float py, float fx, float fy, float cx, float cy,
     const mat3 R_inv = gsx::mat3_cast(gsx::quat_inverse(pose.q));
     *ray_o = gsx::neg(gsx::mul(R_inv, pose.t));
     *ray_d = gsx::mul(R_inv, d_cam);
+    return true;
 }
 
 // M = diag(1/scale) * R(quat)^T  (RasterizeToPixelsFromWorld3DGSFwd.cu:214-226)
@@ -204,7 +310,7 @@ ORC_API int orc_projection_ut_3dgs_fused(
         for (int i = 0; i < 7; ++i) {
             const vec3 pc = gsx::add(gsx::quat_rotate(rs.q_start, pts[i]), rs.t_start);
             vec2 p;
-            const bool pv = pinhole_project(pc, fx, fy, cx, cy, image_width, image_height, ut_margin, &p);
+            const bool pv = project_point(pc, fx, fy, cx, cy, image_width, image_height, ut_margin, &p);
             if (ut_require_all) {
                 valid &= pv;
                 if (!pv) {
@@ -667,11 +773,13 @@ ORC_API int orc_rasterize_to_pixels_from_world_3dgs_fwd(
                     continue;
                 }
                 vec3 ray_o, ray_d;
-                pixel_world_ray((float)j + 0.5f, (float)i + 0.5f, fx, fy, cx, cy, rs, &ray_o, &ray_d);
+                const bool ray_ok =
+                    pixel_world_ray((float)j + 0.5f, (float)i + 0.5f, fx, fy, cx, cy, rs, &ray_o, &ray_d);
                 float T = 1.0f;
                 uint32_t cur_idx = 0;
                 float pix_out[8] = {0.f};
-                for (int32_t t = 0; t < cnt; ++t) {
+                // a pixel without a valid ray is done from the start (RasterizeToPixelsFromWorld3DGSFwd.cu:145)
+                for (int32_t t = 0; t < (ray_ok ? cnt : 0); ++t) {
                     ++pairs;
                     const int32_t g = flatten_ids[range_start + t];
                     const vec3 xyz = ld3(means, g);
@@ -751,7 +859,8 @@ ORC_API int orc_rasterize_to_pixels_from_world_3dgs_bwd(
                     continue;
                 const int64_t pix_id = (int64_t)i * image_width + j;
                 vec3 ray_o, ray_d;
-                pixel_world_ray((float)j + 0.5f, (float)i + 0.5f, fx, fy, cx, cy, rs, &ray_o, &ray_d);
+                if (!pixel_world_ray((float)j + 0.5f, (float)i + 0.5f, fx, fy, cx, cy, rs, &ray_o, &ray_d))
+                    continue; // RasterizeToPixelsFromWorld3DGSBwd.cu:157
                 const float T_final = 1.0f - render_alphas[pix_id];
                 float T = T_final;
                 float buffer[kMaxC] = {0.f, 0.f, 0.f, 0.f};
@@ -960,7 +1069,8 @@ ORC_API int orc_rasterize_bwd_f64(
                     continue;
                 const int64_t pix_id = (int64_t)i * image_width + j;
                 vec3 ray_of, ray_df;
-                pixel_world_ray((float)j + 0.5f, (float)i + 0.5f, fx, fy, cx, cy, rs, &ray_of, &ray_df);
+                if (!pixel_world_ray((float)j + 0.5f, (float)i + 0.5f, fx, fy, cx, cy, rs, &ray_of, &ray_df))
+                    continue;
                 const d3 ray_o = {ray_of.x, ray_of.y, ray_of.z}, ray_d = {ray_df.x, ray_df.y, ray_df.z};
                 const double T_final = 1.0 - (double)render_alphas[pix_id];
                 double T = T_final;
@@ -1700,4 +1810,41 @@ ORC_API int orc_record_bounds_check(uint32_t N, const float* means, const float*
         blocks_hit[g] = bhit;
     }
     return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// camera model state and probes
+// ---------------------------------------------------------------------------------------------
+// radial [6], tangential [2], thin_prism [4], each nullable; all null = perfect pinhole.
+ORC_API void orc_set_distortion(const float* radial, const float* tangential, const float* thin_prism) {
+    g_dist = Distortion();
+    g_dist.on = radial != nullptr || tangential != nullptr || thin_prism != nullptr;
+    for (int i = 0; i < 6 && radial; ++i)
+        g_dist.k[i] = radial[i];
+    for (int i = 0; i < 2 && tangential; ++i)
+        g_dist.p[i] = tangential[i];
+    for (int i = 0; i < 4 && thin_prism; ++i)
+        g_dist.s[i] = thin_prism[i];
+}
+
+// camera-space points [n,3] -> image points [n,2] + valid [n] under the current camera model
+ORC_API void orc_camera_project(int64_t n, const float* pts, float fx, float fy, float cx, float cy, uint32_t W,
+                                uint32_t H, float margin, float* out, uint8_t* valid) {
+    for (int64_t i = 0; i < n; ++i) {
+        vec2 p;
+        valid[i] = project_point(ld3(pts, i), fx, fy, cx, cy, W, H, margin, &p) ? 1 : 0;
+        out[2 * i] = p.x, out[2 * i + 1] = p.y;
+    }
+}
+
+// image points [n,2] -> unit camera rays [n,3] + valid [n] (identity pose) under the current camera model
+ORC_API void orc_camera_unproject(int64_t n, const float* image_points, float fx, float fy, float cx, float cy,
+                                  float* rays, uint8_t* valid) {
+    const float eye[16] = {1, 0, 0, 0, 0, 1, 0, 0, 0, 0, 1, 0, 0, 0, 0, 1};
+    const RollingShutter rs = make_rolling_shutter(eye, nullptr);
+    for (int64_t i = 0; i < n; ++i) {
+        vec3 o, d;
+        valid[i] = pixel_world_ray(image_points[2 * i], image_points[2 * i + 1], fx, fy, cx, cy, rs, &o, &d) ? 1 : 0;
+        rays[3 * i] = d.x, rays[3 * i + 1] = d.y, rays[3 * i + 2] = d.z;
+    }
 }

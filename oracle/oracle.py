@@ -53,6 +53,43 @@ def _chk(rc, name):
 UT_DEFAULT = dict(alpha=0.1, beta=2.0, kappa=0.0, in_image_margin_factor=0.1, require_all_sigma_points_valid=True)
 
 
+class distortion:
+    """Context manager: OpenCV pinhole distortion coefficients (radial [6], tangential [2], thin_prism [4], each
+    optional) for every projection / pixel-ray inside the block, as the reference dispatches on "any coefficient
+    tensor given" (ProjectionUT3DGSFused.cu:86-113)."""
+
+    def __init__(self, radial=None, tangential=None, thin_prism=None):
+        f = lambda a, n: None if a is None else np.ascontiguousarray(np.asarray(a, np.float32).reshape(-1)[:n])
+        self.args = (f(radial, 6), f(tangential, 2), f(thin_prism, 4))
+
+    def __enter__(self):
+        lib().orc_set_distortion(*[_p(a) for a in self.args])
+        return self
+
+    def __exit__(self, *exc):
+        lib().orc_set_distortion(None, None, None)
+        return False
+
+
+def camera_project(points, fx, fy, cx, cy, W, H, margin=0.1):
+    """camera-space points [n,3] -> (image points [n,2], valid [n]) under the current camera model"""
+    pts = _f32(points)
+    n = pts.shape[0]
+    out, valid = np.zeros((n, 2), np.float32), np.zeros(n, np.uint8)
+    lib().orc_camera_project(c_i64(n), _p(pts), c_f(fx), c_f(fy), c_f(cx), c_f(cy), c_u32(W), c_u32(H), c_f(margin),
+                             _p(out), _p(valid))
+    return out, valid.astype(bool)
+
+
+def camera_unproject(image_points, fx, fy, cx, cy):
+    """image points [n,2] -> (unit camera rays [n,3], valid [n]) under the current camera model"""
+    ip = _f32(image_points)
+    n = ip.shape[0]
+    rays, valid = np.zeros((n, 3), np.float32), np.zeros(n, np.uint8)
+    lib().orc_camera_unproject(c_i64(n), _p(ip), c_f(fx), c_f(fy), c_f(cx), c_f(cy), _p(rays), _p(valid))
+    return rays, valid.astype(bool)
+
+
 def num_threads():
     return lib().orc_num_threads()
 

@@ -556,3 +556,92 @@ def test_depth_render_modes(gsx, orc, cuda, render_mode):
     assert gc.shape[-1] == ch
     assert np.abs(N(gc) - oc).max() <= 1e-3 * np.abs(oc).max()
     assert np.abs(oc[..., -1]).max() > 0
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# OpenCV pinhole distortion (radial / tangential / thin-prism coefficients given): Cameras.cuh:473-815
+# ---------------------------------------------------------------------------------------------------------------
+_DIST = dict(radial=[-0.12, 0.03, -0.004, 0.02, -0.005, 0.001], tangential=[8e-4, -6e-4],
+             thin_prism=[3e-4, -1e-4, -2e-4, 1e-4])
+
+
+@pytest.mark.parametrize("which", ["all", "radial", "tangential+thin", "strong"])
+def test_opencv_distortion_fused_forward_backward(gsx, orc, cuda, which):
+    """the fused forward (projection through the distorted model, per-pixel Newton undistortion) is bit-identical to
+    the checker; the backward meets the gradient bar.  "strong": barrel distortion large enough that icD <= 0.8
+    culls Gaussians near the border and some pixel undistortions do not converge (those pixels stay background)."""
+    ops = gsx.ops
+    sc, cam, h, d = _fused_inputs(gsx, cuda, 20000)
+    coeffs = {"all": _DIST, "radial": dict(radial=_DIST["radial"]),
+              "tangential+thin": dict(tangential=[6e-3, -4e-3], thin_prism=[3e-3, -1e-3, -2e-3, 1e-3]),
+              "strong": dict(radial=[-0.9, 0.5, 0.0, 0.0, 0.0, 0.0])}[which]
+    dev = {k: T(np.asarray(v, np.float32)[None], cuda) for k, v in coeffs.items()}
+    co = (dev.get("radial"), dev.get("tangential"), dev.get("thin_prism"))
+    ut = ops.UnscentedTransformParameters()
+    with orc.distortion(**coeffs):
+        ref = orc.rasterize_from_world_with_sh_fwd(h["means"], h["quats"], h["scales"], h["op"], h["shs"], 3, h["bg"],
+                                                   cam.width, cam.height, 16, h["vm"], h["K"])
+    plain = orc.rasterize_from_world_with_sh_fwd(h["means"], h["quats"], h["scales"], h["op"], h["shs"], 3, h["bg"],
+                                                 cam.width, cam.height, 16, h["vm"], h["K"])
+    assert np.abs(ref[0] - plain[0]).max() > 0.02  # the coefficients matter
+    got = ops.rasterize_from_world_with_sh_fwd(d["means"], d["quats"], d["scales"], d["op"], d["shs"], 3, d["bg"], None,
+                                               cam.width, cam.height, 16, d["vm"], None, d["K"], 0, 0.3, 0.01, 1e4, 0.0,
+                                               1.0, False, 0, ut, 4, *co, return_isect_ids=True)
+    renders, alphas, radii, means2d, depths, colors, offsets, flat, last_ids, comp, ids = got
+    bits_equal(N(radii), ref[2], "radii")
+    vis = ref[2][0, :, 0] > 0
+    bits_equal(N(means2d)[0][vis], ref[3][0][vis], "means2d")
+    bits_equal(N(ids), ref[10], "sorted tile keys")
+    bits_equal(N(flat), ref[7], "sort order")
+    bits_equal(N(offsets), ref[6], "per-tile ranges")
+    bits_equal(N(last_ids), ref[8], "last ids")
+    bits_equal(N(renders), ref[0], "image")
+    bits_equal(N(alphas), ref[1], "alpha")
+    assert ref[1].mean() > 0.05
+    if which == "strong":
+        assert vis.sum() < (plain[2][0, :, 0] > 0).sum()
+
+    rng = np.random.default_rng(3)
+    v_r = rng.normal(0, 1, tuple(renders.shape)).astype(np.float32)
+    v_a = rng.normal(0, 1, tuple(alphas.shape)).astype(np.float32)
+    op1 = d["op"][None].contiguous()
+    got5 = ops.rasterize_to_pixels_from_world_3dgs_bwd(d["means"], d["quats"], d["scales"], colors, op1, d["bg"], None,
+                                                       cam.width, cam.height, 16, d["vm"], None, d["K"], 0, ut, 4, *co,
+                                                       offsets, flat, alphas, last_ids, T(v_r, cuda), T(v_a, cuda))
+    args = (h["means"], h["quats"], h["scales"], N(colors), h["op"][None], h["bg"])
+    with orc.distortion(**coeffs):
+        o32 = orc.rasterize_to_pixels_from_world_3dgs_bwd(*args, None, cam.width, cam.height, 16, h["vm"], h["K"],
+                                                          N(offsets), N(flat), N(alphas), N(last_ids), v_r, v_a)
+        g64, _ = orc.rasterize_bwd_f64(*args, cam.width, cam.height, 16, h["vm"], h["K"], N(offsets), N(flat),
+                                       N(alphas), N(last_ids), v_r, v_a)
+    check_raster_gradients([N(x) for x in got5], o32, g64, tag=which + " ")
+
+
+def test_opencv_distortion_projection_and_errors(gsx, orc, cuda):
+    """gsx_projection_ut_3dgs_fused with coefficients: radii / means2d / depths / conics bit-identical to the checker;
+    zero coefficients give the perfect pinhole's results; other camera models and rolling shutter stay unsupported"""
+    ops = gsx.ops
+    sc, cam, h, d = _fused_inputs(gsx, cuda, 30000)
+    ut = ops.UnscentedTransformParameters()
+    dev = {k: T(np.asarray(v, np.float32)[None], cuda) for k, v in _DIST.items()}
+    call = lambda *co, **kw: ops.projection_ut_3dgs_fused(d["means"], d["quats"], d["scales"], d["op"], d["vm"], None,
+                                                          d["K"], cam.width, cam.height, 0.3, 0.01, 1e4, 0.0, False,
+                                                          kw.get("model", 0), ut, kw.get("rs", 4), *co)
+    got = call(dev["radial"], dev["tangential"], dev["thin_prism"])
+    with orc.distortion(**_DIST):
+        ref = orc.projection_ut_3dgs_fused(h["means"], h["quats"], h["scales"], h["op"], h["vm"], h["K"], cam.width,
+                                           cam.height)
+    bits_equal(N(got[0]), ref[0], "radii")
+    vis = ref[0][0, :, 0] > 0
+    assert vis.sum() > 5000
+    for k, name in ((1, "means2d"), (2, "depths"), (3, "conics")):
+        bits_equal(N(got[k])[0][vis], ref[k][0][vis], name)
+    zero = [torch.zeros_like(dev[k]) for k in ("radial", "tangential", "thin_prism")]
+    a, b = call(*zero), call(None, None, None)
+    assert torch.equal(a[0], b[0])
+    vis = (b[0][0, :, 0] > 0)
+    assert torch.equal(a[1][0][vis], b[1][0][vis]) and torch.equal(a[3][0][vis], b[3][0][vis])
+    with pytest.raises(RuntimeError, match="only PINHOLE"):
+        call(None, None, None, model=2)  # FISHEYE
+    with pytest.raises(RuntimeError, match="rolling shutter"):
+        call(None, None, None, rs=0)  # ROLLING_TOP_TO_BOTTOM

@@ -337,3 +337,83 @@ def test_radix_sort_is_stable_on_bit_range(orc):
         k, v = orc.radix_sort_pairs(keys, vals, end_bit)
         order = np.argsort((keys & mask).astype(np.uint64), kind="stable")
         assert np.array_equal(k, keys[order]) and np.array_equal(v, vals[order])
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# OpenCV pinhole distortion (Cameras.cuh:473-815)
+# ---------------------------------------------------------------------------------------------------------------
+_RADIAL = [-0.12, 0.03, -0.004, 0.02, -0.005, 0.001]
+_TANGENTIAL = [8e-4, -6e-4]
+_THIN_PRISM = [3e-4, -1e-4, -2e-4, 1e-4]
+
+
+def _rays(n, seed, half_fov=0.6):
+    r = np.random.default_rng(seed)
+    uv = r.uniform(-np.tan(half_fov), np.tan(half_fov), (n, 2))
+    z = r.uniform(0.5, 6.0, (n, 1))
+    return np.concatenate([uv * z, z], 1).astype(np.float32)
+
+
+def test_distortion_off_is_the_pinhole_model(orc):
+    """all coefficients zero: image points, rays and the whole UT projection equal the perfect pinhole's bit for bit"""
+    pts = _rays(2000, 0)
+    a, va = orc.camera_project(pts, 300.0, 310.0, 200.0, 150.0, 400, 300)
+    with orc.distortion([0] * 6, [0] * 2, [0] * 4):
+        b, vb = orc.camera_project(pts, 300.0, 310.0, 200.0, 150.0, 400, 300)
+        rb, okb = orc.camera_unproject(a, 300.0, 310.0, 200.0, 150.0)
+    ra, oka = orc.camera_unproject(a, 300.0, 310.0, 200.0, 150.0)
+    assert np.array_equal(a.view(np.int32), b.view(np.int32)) and np.array_equal(va, vb)
+    assert okb.all() and oka.all() and np.abs(ra - rb).max() <= 1.2e-7  # one Newton step of size 0 later
+
+
+def test_distortion_special_cases(orc):
+    """radial-only: the image radius is f r (1 + k1 r^2 + k2 r^4 + k3 r^6) / (1 + k4 r^2 + ...) along the ray's own
+    direction; tangential / thin-prism terms on the axes; validity: icD <= 0.8 and z <= 0 are invalid"""
+    f, c = 250.0, 160.0
+    pts = _rays(500, 1)
+    u, v = pts[:, 0] / pts[:, 2], pts[:, 1] / pts[:, 2]
+    r2 = (u.astype(np.float64) ** 2 + v.astype(np.float64) ** 2)
+    k = np.array(_RADIAL, np.float64)
+    with orc.distortion(radial=_RADIAL):
+        ip, _ = orc.camera_project(pts, f, f, c, c, 320, 320, margin=10.0)
+    scale = (1 + r2 * (k[0] + r2 * (k[1] + r2 * k[2]))) / (1 + r2 * (k[3] + r2 * (k[4] + r2 * k[5])))
+    assert np.abs(ip[:, 0] - (f * u * scale + c)).max() < 2e-4 and np.abs(ip[:, 1] - (f * v * scale + c)).max() < 2e-4
+    x = np.linspace(-0.5, 0.5, 11).astype(np.float32)
+    on_x = np.stack([x, np.zeros_like(x), np.ones_like(x)], 1)
+    with orc.distortion(tangential=[2e-3, -3e-3], thin_prism=[1e-3, 2e-3, -1e-3, 5e-4]):
+        ip, _ = orc.camera_project(on_x, 1.0, 1.0, 0.0, 0.0, 4, 4, margin=10.0)
+    xx = x.astype(np.float64) ** 2
+    assert np.allclose(ip[:, 0], x + (-3e-3) * 3 * xx + xx * (1e-3 + xx * 2e-3), atol=1e-7)
+    assert np.allclose(ip[:, 1], 2e-3 * xx + xx * (-1e-3 + xx * 5e-4), atol=1e-7)
+    with orc.distortion(radial=[-0.5, 0, 0, 0, 0, 0]):  # icD = 1 - 0.5 r^2 <= 0.8 beyond r^2 = 0.4
+        p = np.array([[0.5, 0, 1], [0.7, 0, 1], [0.1, 0, -1]], np.float32)
+        _, ok = orc.camera_project(p, 100.0, 100.0, 100.0, 100.0, 200, 200)
+    assert list(ok) == [True, False, False]
+
+
+def test_undistortion_inverts_the_projection(orc):
+    """Newton undistortion of projected rays returns the rays (a wrong Jacobian entry stalls the 5 iterations), and
+    agrees with an independent solve of the float64 forward model by scipy"""
+    from scipy.optimize import fsolve
+    f, c = 400.0, 320.0
+    pts = _rays(3000, 2)
+    with orc.distortion(_RADIAL, _TANGENTIAL, _THIN_PRISM):
+        ip, ok = orc.camera_project(pts, f, 1.1 * f, c, c - 40, 640, 560, margin=0.5)
+        rays, conv = orc.camera_unproject(ip, f, 1.1 * f, c, c - 40)
+    assert ok.sum() > 2500 and conv[ok].all()
+    want = pts / np.linalg.norm(pts, axis=1, keepdims=True)
+    assert np.abs(rays[ok] - want[ok]).max() < 3e-6
+    k, p, s = (np.array(a, np.float64) for a in (_RADIAL, _TANGENTIAL, _THIN_PRISM))
+
+    def forward(uv):
+        u, v = uv
+        r2 = u * u + v * v
+        icd = (1 + r2 * (k[0] + r2 * (k[1] + r2 * k[2]))) / (1 + r2 * (k[3] + r2 * (k[4] + r2 * k[5])))
+        return np.array([icd * u + 2 * p[0] * u * v + p[1] * (r2 + 2 * u * u) + r2 * (s[0] + r2 * s[1]),
+                         icd * v + p[0] * (r2 + 2 * v * v) + 2 * p[1] * u * v + r2 * (s[2] + r2 * s[3])])
+
+    for i in np.nonzero(ok)[0][:40]:
+        target = np.array([(ip[i, 0] - c) / f, (ip[i, 1] - (c - 40)) / (1.1 * f)], np.float64)
+        sol = fsolve(lambda uv: forward(uv) - target, target, xtol=1e-12)
+        ray = np.array([sol[0], sol[1], 1.0]) / np.linalg.norm([sol[0], sol[1], 1.0])
+        assert np.abs(rays[i] - ray).max() < 3e-6
