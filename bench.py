@@ -94,6 +94,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--separate-update", action="store_true",
                     help="run epilogue / SH backward / activation VJPs / Adam as separate kernels (default: one pass)")
+    ap.add_argument("--no-overlap", action="store_true",
+                    help="keep every kernel of the step on one stream (default: the SH / record pass and the loss "
+                         "reduction run on a second stream beside the sort chain / the backward rasterizer)")
     ap.add_argument("--cpu-threads", type=int, default=0, help="threads for the CPU baseline (0 = all)")
     ap.add_argument("--workload", choices=["gut", "fastgs"], default="gut",
                     help="gut: the training step of the metric (default); fastgs: forward + backward of the "
@@ -130,7 +133,7 @@ def main():
         gt = torch.from_numpy(sc.target[None].copy()).to(dev)
     use_ssim = args.config != 1  # configuration 1 is L1 only
     ts = TrainStep(sc, dev, use_ssim=use_ssim, fused_update=not args.separate_update,
-                   fused_loss=not args.separate_update)
+                   fused_loss=not args.separate_update, overlap=not args.no_overlap)
     setup_s = time.time() - t0
 
     dominant = "rasterize_bwd_accumulate"

@@ -124,6 +124,13 @@ GSX_API int gsx_intersect_tile_emit(uint32_t C, uint32_t N, const float* means2d
                                     const float* depths, const int64_t* cum_tiles_per_gauss, const int32_t* order,
                                     uint32_t tile_size, uint32_t tile_width, uint32_t tile_height, int64_t* isect_ids,
                                     int32_t* flatten_ids, void* stream);
+/* The same with the writes bounded to the first `capacity` entries: lets a caller that reuses its buffers emit
+ * while the total is still on its way to the host, and repeat the call only if the total exceeded the buffers. */
+GSX_API int gsx_intersect_tile_emit_capped(uint32_t C, uint32_t N, const float* means2d, const int32_t* radii,
+                                           const float* depths, const int64_t* cum_tiles_per_gauss,
+                                           const int32_t* order, uint32_t tile_size, uint32_t tile_width,
+                                           uint32_t tile_height, int64_t capacity, int64_t* isect_ids,
+                                           int32_t* flatten_ids, void* stream);
 /* Intersect.cpp:46-47: floor(log2(n)) + 1 */
 GSX_API uint32_t gsx_n_bits(uint32_t n);
 

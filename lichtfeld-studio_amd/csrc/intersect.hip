@@ -161,7 +161,8 @@ __global__ void __launch_bounds__(256) tile_emit_kernel(uint32_t n, uint32_t N, 
                                                          const int64_t* __restrict__ cum_tiles_per_gauss,
                                                          const int32_t* __restrict__ order, float tile_size,
                                                          uint32_t tile_width, uint32_t tile_height,
-                                                         uint32_t tile_n_bits, int64_t* __restrict__ isect_ids,
+                                                         uint32_t tile_n_bits, int64_t capacity,
+                                                         int64_t* __restrict__ isect_ids,
                                                          int32_t* __restrict__ flatten_ids) {
     __shared__ uint32_t s_incl[4][64], s_xy[4][64], s_w[4][64], s_idx[4][64], s_lo[4][64], s_hi[4][64];
     const uint32_t i = blockIdx.x * 256u + threadIdx.x;
@@ -219,8 +220,10 @@ __global__ void __launch_bounds__(256) tile_emit_kernel(uint32_t n, uint32_t N, 
         const uint32_t row = local / gw;
         const int64_t tile_id = (int64_t)((xy >> 16) + row) * tile_width + ((xy & 0xffffu) + (local - row * gw));
         const int64_t kb = ((int64_t)s_hi[wv][l] << 32) | (int64_t)s_lo[wv][l];
-        isect_ids[wave_base + k] = kb | (tile_id << 32);
-        flatten_ids[wave_base + k] = (int32_t)s_idx[wv][l];
+        if (wave_base + k < capacity) { // a caller that emits before it knows the total bounds the writes
+            isect_ids[wave_base + k] = kb | (tile_id << 32);
+            flatten_ids[wave_base + k] = (int32_t)s_idx[wv][l];
+        }
     }
 }
 
@@ -418,6 +421,15 @@ extern "C" int gsx_intersect_tile_emit(uint32_t C, uint32_t N, const float* mean
                                        const int32_t* order, uint32_t tile_size, uint32_t tile_width,
                                        uint32_t tile_height, int64_t* isect_ids, int32_t* flatten_ids,
                                        void* stream) {
+    return gsx_intersect_tile_emit_capped(C, N, means2d, radii, depths, cum_tiles_per_gauss, order, tile_size,
+                                          tile_width, tile_height, INT64_MAX, isect_ids, flatten_ids, stream);
+}
+
+extern "C" int gsx_intersect_tile_emit_capped(uint32_t C, uint32_t N, const float* means2d, const int32_t* radii,
+                                              const float* depths, const int64_t* cum_tiles_per_gauss,
+                                              const int32_t* order, uint32_t tile_size, uint32_t tile_width,
+                                              uint32_t tile_height, int64_t capacity, int64_t* isect_ids,
+                                              int32_t* flatten_ids, void* stream) {
     const uint64_t n64 = (uint64_t)C * N;
     if (n64 == 0)
         return GSX_OK;
@@ -428,7 +440,7 @@ extern "C" int gsx_intersect_tile_emit(uint32_t C, uint32_t N, const float* mean
     GSX_REQUIRE(order == nullptr || C == 1, GSX_ERR_UNSUPPORTED, "intersect_tile_emit: an order needs C == 1");
     hipLaunchKernelGGL(tile_emit_kernel, dim3(cdiv(n, 256)), dim3(256), 0, (hipStream_t)stream, n, N, means2d, radii,
                        depths, cum_tiles_per_gauss, order, (float)tile_size, tile_width, tile_height,
-                       gsx_n_bits(tile_width * tile_height), isect_ids, flatten_ids);
+                       gsx_n_bits(tile_width * tile_height), capacity, isect_ids, flatten_ids);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

@@ -28,7 +28,7 @@ def _p(t):
 class TrainStep:
     def __init__(self, scene, device="cuda:0", lrs=None, lambda_dssim=0.2, betas=(0.9, 0.999), eps=1e-15,
                  scene_scale=1.0, sh_degree=None, use_ssim=True, fused_update=False, fused_loss=False,
-                 scale_reg=0.0, opacity_reg=0.0):
+                 scale_reg=0.0, opacity_reg=0.0, overlap=False):
         self.dev = torch.device(device)
         self.lib = lib()
         f = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(self.dev)
@@ -66,6 +66,12 @@ class TrainStep:
         self.img_shape = None
         self.n_isects = 0
         self.bg = torch.zeros((1, 3), dtype=torch.float32, device=self.dev)  # trainer.cpp:383-384
+        # A second stream (default priority) for work that is independent of the launch-latency-bound sort chain:
+        # the SH / record pass runs beside the depth-ordered count, the loss reduction beside the backward rasterizer.
+        self.overlap = overlap
+        self.side = torch.cuda.Stream(self.dev) if overlap else None
+        self.ev_fork, self.ev_join = torch.cuda.Event(), torch.cuda.Event()
+        self.ev_loss_fork, self.ev_loss_join = torch.cuda.Event(), torch.cuda.Event()
         self.loss_out = torch.empty(3, dtype=torch.float32, device=self.dev)
 
     def _allocate_per_gaussian(self, N):
@@ -162,6 +168,8 @@ class TrainStep:
                   _p(P["scaling"]), _p(P["rotation"]), _p(viewmat), _p(K), c_u32(W), c_u32(H), c_f(0.3), c_f(0.01),
                   c_f(1e4), c_f(0.0), self.ut, _p(A["opacities"]), _p(A["scales"]), _p(A["quats"]), _p(J["radii"]),
                   _p(J["means2d"]), _p(J["depths"]), _p(J["conics"]), s)
+        if self.side is not None:
+            self.ev_fork.record(torch.cuda.current_stream(self.dev))
         # Tile counts in depth order; the total comes back through pinned memory without blocking, and the SH /
         # record passes (which do not need it) run while the host waits for it.
         self._run("intersect_tile_count_ordered", lb.gsx_intersect_tile_count_ordered, c_u32(N), _p(J["means2d"]),
@@ -169,10 +177,26 @@ class TrainStep:
                   _p(self.tiles_per_gauss), _p(self.cum), _p(self.ws_count), c_sz(self.ws_count.numel()),
                   c_p(self.n_isects_pinned.data_ptr()), c_i(0), s)
         self.count_done.record(torch.cuda.current_stream(self.dev))
-        self._run("sh_colors_records_from_world", lb.gsx_sh_colors_records_from_world, c_u32(N), c_u32(self.K),
-                  c_u32(self.sh_degree), _p(P["means"]), _p(A["quats"]), _p(A["scales"]), _p(A["opacities"]),
-                  _p(P["shs"]), _p(J["radii"]), _p(viewmat), _p(K), c_u32(W), c_u32(H), _p(self.colors),
-                  _p(self.records), s)
+        sh_args = (c_u32(N), c_u32(self.K), c_u32(self.sh_degree), _p(P["means"]), _p(A["quats"]), _p(A["scales"]),
+                   _p(A["opacities"]), _p(P["shs"]), _p(J["radii"]), _p(viewmat), _p(K), c_u32(W), c_u32(H),
+                   _p(self.colors), _p(self.records))
+        if self.side is None:
+            self._run("sh_colors_records_from_world", lb.gsx_sh_colors_records_from_world, *sh_args, s)
+        else:
+            self.side.wait_event(self.ev_fork)  # recorded after the activation / projection pass
+            with torch.cuda.stream(self.side):
+                self._run("sh_colors_records_from_world", lb.gsx_sh_colors_records_from_world, *sh_args,
+                          self._stream())
+                self.ev_join.record(self.side)
+        # The emission does not need the total, only room for it: with buffers from an earlier step it is queued now
+        # (writes bounded to the buffers) and the host's wake-up from the wait below hides behind it.
+        emit = lambda cap: self._run(
+            "intersect_tile_emit", lb.gsx_intersect_tile_emit_capped, c_u32(1), c_u32(N), _p(J["means2d"]),
+            _p(J["radii"]), _p(J["depths"]), _p(self.cum), _p(self.order), c_u32(16), c_u32(self.tw), c_u32(self.th),
+            c_i64(cap), _p(self.keys[0]), _p(self.vals[0]), s)
+        emitted_cap = self.cap
+        if emitted_cap:
+            emit(emitted_cap)
         self.count_done.synchronize()
         n = self.n_isects = int(self.n_isects_pinned[0])
         if n >= 1 << 31:
@@ -180,9 +204,8 @@ class TrainStep:
         self._ensure_isect_capacity(n)
         sel = c_i(0)
         if n:
-            self._run("intersect_tile_emit", lb.gsx_intersect_tile_emit, c_u32(1), c_u32(N), _p(J["means2d"]),
-                      _p(J["radii"]), _p(J["depths"]), _p(self.cum), _p(self.order), c_u32(16), c_u32(self.tw),
-                      c_u32(self.th), _p(self.keys[0]), _p(self.vals[0]), s)
+            if n > emitted_cap:  # first step, or the buffers had to grow
+                emit(self.cap)
             end_bit = 32 + lb.gsx_n_bits(c_u32(self.tw * self.th)) + lb.gsx_n_bits(c_u32(1))
             self._run("radix_sort_pairs", lb.gsx_radix_sort_pairs, c_i64(n), _p(self.keys[0]), _p(self.vals[0]),
                       _p(self.keys[1]), _p(self.vals[1]), c_u32(32), c_u32(end_bit), _p(self.ws_sort),
@@ -191,6 +214,8 @@ class TrainStep:
         self.isect_ids, self.flatten_ids = self.keys[self.sel], self.vals[self.sel]
         self._run("intersect_offset", lb.gsx_intersect_offset, c_i64(n), _p(self.isect_ids), c_u32(1), c_u32(self.tw), c_u32(self.th),
                                       _p(self.offsets), s)
+        if self.side is not None:
+            torch.cuda.current_stream(self.dev).wait_event(self.ev_join)  # colours and records are ready
         self._run("rasterize_to_pixels_from_world_3dgs_fwd", lb.gsx_rasterize_records_fwd, c_i64(n),
                   _p(self.records), c_p(None), c_u32(3), _p(self.bg), c_p(None), c_u32(W), c_u32(H), _p(viewmat),
                   _p(K), _p(self.offsets), _p(self.flatten_ids), _p(self.render), _p(self.alpha), _p(self.last_ids),
@@ -206,9 +231,17 @@ class TrainStep:
             self._run("photometric_loss_forward", lb.gsx_photometric_loss_forward, c_u32(H), c_u32(W),
                       c_f(0.01 ** 2), c_f(0.03 ** 2), _p(self.render), _p(gt_chw), _p(self.dm1), _p(self.dm2),
                       _p(self.dm3), _p(self.l1_partials), _p(self.ssim_partials), s)
-            self._run("photometric_loss_finish", lb.gsx_photometric_loss_finish, c_u32(3), c_u32(H), c_u32(W),
-                      c_f(self.lambda_dssim), _p(self.l1_partials), _p(self.ssim_partials),
-                      c_u32(self.n_partials_fused), _p(self.loss_out), s)
+            fin = (c_u32(3), c_u32(H), c_u32(W), c_f(self.lambda_dssim), _p(self.l1_partials), _p(self.ssim_partials),
+                   c_u32(self.n_partials_fused), _p(self.loss_out))
+            if self.side is None:
+                self._run("photometric_loss_finish", lb.gsx_photometric_loss_finish, *fin, s)
+            else:  # the value is only reported: its reduction runs beside the backward pass
+                self.ev_loss_fork.record(torch.cuda.current_stream(self.dev))
+                self.side.wait_event(self.ev_loss_fork)
+                with torch.cuda.stream(self.side):
+                    self._run("photometric_loss_finish", lb.gsx_photometric_loss_finish, *fin, self._stream())
+                    self.ev_loss_join.record(self.side)
+                self.loss_pending = True
             return self.loss_out
         self._run("image_from_render", lb.gsx_image_from_render, c_u32(H), c_u32(W), _p(self.render), _p(gt_chw), _p(self.image),
                                        _p(self.l1_partials), s)
@@ -365,10 +398,15 @@ class TrainStep:
                   _p(self.params["scaling"]), _p(self.params["rotation"]), _p(noise), _p(self.params["means"]),
                   c_f(self.lrs["means"] * noise_lr), self._stream())
 
+    loss_pending = False
+
     def step(self, viewmat, K, W, H, gt_chw):
         self.iteration += 1
         self.forward(viewmat, K, W, H)
         self.loss_forward(gt_chw)
         self.backward()
         self.adam()
+        if self.loss_pending:  # the next step's loss pass overwrites the partial sums: rejoin the side stream
+            torch.cuda.current_stream(self.dev).wait_event(self.ev_loss_join)
+            self.loss_pending = False
         return self.loss_out
