@@ -192,3 +192,44 @@ def test_l1_regularization_kernels(gsx, orc, cuda, n):
                  c_p(out.data_ptr()), s))
         torch.cuda.synchronize()
         assert torch.equal(before, gd) and float(out[0]) == -7.0
+
+
+def test_speculative_emission_and_overlap_change_nothing(gsx, cuda):
+    """the step with the second stream and the early, capacity-bounded tile emission produces the same image and
+    parameters bit for bit as the single-stream step; when the buffers turn out too small (capacity forced down)
+    only their first `capacity` entries are written early and the emission is repeated after they have grown"""
+    from lichtfeld_studio_amd.trainer import TrainStep
+    sc = gsx.scenes.config(3, 20_000)
+    sc.scaling_raw += 1.2
+    cam = gsx.scenes.orbit_camera(0.7, 4.0, 309, 205, 287.0)
+    W, H = cam.width, cam.height
+    vm = torch.from_numpy(cam.viewmat[None].copy()).to(cuda)
+    Km = torch.from_numpy(cam.K[None].copy()).to(cuda)
+    gt = torch.rand((1, 3, H, W), generator=torch.Generator().manual_seed(3)).to(cuda)
+    a = TrainStep(sc, cuda, fused_update=True, fused_loss=True, overlap=False)
+    b = TrainStep(sc, cuda, fused_update=True, fused_loss=True, overlap=True)
+    for it in range(3):
+        if it == 2:
+            b.cap = 1000  # far below the ~1e5 intersections: the early emission must stop at 1000 entries
+            b.keys[0][1000:].fill_(-1)
+        a.forward(vm, Km, W, H)
+        b.forward(vm, Km, W, H)
+        torch.cuda.synchronize()
+        assert a.n_isects == b.n_isects and a.n_isects > 50_000
+        assert torch.equal(a.isect_ids[:a.n_isects], b.isect_ids[:b.n_isects])
+        assert torch.equal(a.flatten_ids[:a.n_isects], b.flatten_ids[:b.n_isects])
+        assert torch.equal(a.render, b.render)
+        for ts in (a, b):
+            ts.iteration += 1
+            ts.loss_forward(gt)
+            ts.backward()
+        b.ws_bwd.copy_(a.ws_bwd)  # the accumulators are atomic sums: give both tails the same ones
+        a.adam()
+        b.adam()
+        if b.loss_pending:
+            torch.cuda.current_stream(cuda).wait_event(b.ev_loss_join)
+            b.loss_pending = False
+        torch.cuda.synchronize()
+        assert torch.equal(a.loss_out, b.loss_out)
+        for k in a.params:
+            assert torch.equal(a.params[k], b.params[k]), k
