@@ -157,7 +157,8 @@ def main():
     L.check(L.lib().gsx_rasterize_pair_stats(
         ctypes.c_int64(ts.n_isects), p(ts.records), ctypes.c_uint32(W), ctypes.c_uint32(H), p(viewmat), p(Kmat),
         p(ts.offsets), p(ts.flatten_ids), p(stats), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
-    pairs_fwd, pairs_comp, pairs_bwd, wave_iters, wave_skipped, wave_hits = [int(x) for x in stats.cpu()[:6]]
+    pairs_fwd, pairs_comp, pairs_bwd, wave_iters, wave_skipped, wave_hits, half_rows, half_cols = [
+        int(x) for x in stats.cpu()[:8]]
 
     # instrumented pass: every stage bracketed by events (not part of the timed region)
     ts.start_timing(None)
@@ -226,7 +227,8 @@ def main():
                                " + bwd + fused Adam", "n_gaussians": ts.N, "image": [W, H], "n_isects": ts.n_isects,
                    "tiles": ts.tw * ts.th, "pairs_fwd": pairs_fwd, "pairs_composited": pairs_comp,
                    "pairs_bwd": pairs_bwd, "wave_iterations": wave_iters,
-                   "wave_iterations_skipped_by_bounds": wave_skipped, "wave_iterations_contributing": wave_hits, "loss": loss, "setup_s": round(setup_s, 1)},
+                   "wave_iterations_skipped_by_bounds": wave_skipped, "wave_iterations_contributing": wave_hits,
+                   "contributing_half_blocks_8x4": half_rows, "contributing_half_blocks_4x8": half_cols, "loss": loss, "setup_s": round(setup_s, 1)},
         "raster_fwd_ms": kernels.get("rasterize_to_pixels_from_world_3dgs_fwd", {}).get("ms"),
         "raster_bwd_ms": round(dom_ms, 4),
         "roofline": roofline, "cpu_baseline": cpu_baseline,

@@ -50,8 +50,9 @@ GSX_API int gsx_fastgs_preprocess(uint32_t N, const float* means, const float* s
  * background (nullable, 3 floats on the device): image += (1 - alpha) * background as fast_rasterizer.cpp:63 does
  * after the kernel. */
 GSX_API int gsx_fastgs_render(uint32_t N, const gsx_fastgs_settings* settings, const void* primitive_state,
-                              int64_t n_instances, void* instance_state, size_t instance_state_bytes,
-                              const float* background, float* image, float* alpha, void* pixel_state, void* stream);
+                              size_t primitive_state_bytes, int64_t n_instances, void* instance_state,
+                              size_t instance_state_bytes, const float* background, float* image, float* alpha,
+                              void* pixel_state, size_t pixel_state_bytes, void* stream);
 /* where gsx_fastgs_preprocess left the per-primitive records ([N,12] floats: mean2d 2, conic 3, opacity, colour 3
  * (not clamped), footprint box half-widths 2, depth; unspecified for culled primitives) and the number of tiles each
  * primitive contributes to (0 = culled) inside primitive_state (device pointers; for inspection and tests) */
@@ -64,13 +65,15 @@ GSX_API int gsx_fastgs_instance_list(const gsx_fastgs_settings* settings, int64_
                                      const int32_t** tile_offsets);
 /* blend_backward_cu + preprocess_backward_cu (kernels_backward.cuh:17-449; src/backward.cu:14-116).  Every output
  * is fully written (zeros for culled primitives; the reference zero-fills them first).  background: the one given
- * to gsx_fastgs_render (its gradient path through alpha is included).  grad_w2c (nullable, 16 floats on the device):
+ * to gsx_fastgs_render (its gradient path through alpha is included).  The three state buffers are checked against
+ * the sizes N, n_instances and the image size require (GSX_ERR_WORKSPACE).  grad_w2c (nullable, 16 floats on the device):
  * rows 0-2 as kernels_backward.cuh:177-190.  densification_info (nullable, [2,N]): += as :233-236. */
 GSX_API int gsx_fastgs_backward(uint32_t N, const float* means, const float* scales_raw, const float* rotations_raw,
                                 const float* sh_coefficients_rest, const float* w2c_host,
                                 const float* cam_position_host, const gsx_fastgs_settings* settings,
-                                const void* primitive_state, int64_t n_instances, const void* instance_state,
-                                const void* pixel_state, const float* background, const float* grad_image,
+                                const void* primitive_state, size_t primitive_state_bytes, int64_t n_instances,
+                                const void* instance_state, size_t instance_state_bytes, const void* pixel_state,
+                                size_t pixel_state_bytes, const float* background, const float* grad_image,
                                 const float* grad_alpha, void* accum, size_t accum_bytes, float* grad_means,
                                 float* grad_scales_raw, float* grad_rotations_raw, float* grad_opacities_raw,
                                 float* grad_sh_coefficients_0, float* grad_sh_coefficients_rest, float* grad_w2c,

@@ -915,15 +915,21 @@ extern "C" int gsx_fastgs_preprocess(uint32_t N, const float* means, const float
 }
 
 extern "C" int gsx_fastgs_render(uint32_t N, const gsx_fastgs_settings* settings, const void* primitive_state,
-                                 int64_t n_instances, void* instance_state, size_t instance_state_bytes,
-                                 const float* background, float* image, float* alpha, void* pixel_state, void* stream) {
+                                 size_t primitive_state_bytes, int64_t n_instances, void* instance_state,
+                                 size_t instance_state_bytes, const float* background, float* image, float* alpha,
+                                 void* pixel_state, size_t pixel_state_bytes, void* stream) {
     GSX_REQUIRE(settings && image && alpha && pixel_state, GSX_ERR_INVALID_ARGUMENT, "fastgs_render: null argument");
     const uint32_t W = settings->width, H = settings->height;
     const uint32_t gw = (W + kTile - 1) / kTile, gh = (H + kTile - 1) / kTile, n_tiles = gw * gh;
     GSX_REQUIRE(W > 0 && H > 0 && (uint64_t)gw * gh <= 65536, GSX_ERR_INVALID_ARGUMENT, "fastgs_render: image %u x %u", W, H);
     GSX_REQUIRE(n_instances >= 0 && n_instances < (1ll << 31), GSX_ERR_OVERFLOW,
                 "fastgs_render: %lld instances do not fit int32 indices", (long long)n_instances);
-    GSX_REQUIRE(N == 0 || primitive_state, GSX_ERR_INVALID_ARGUMENT, "fastgs_render: null primitive state");
+    GSX_REQUIRE(N == 0 || (primitive_state && primitive_state_bytes >= fgs_prim_layout(N).total), GSX_ERR_WORKSPACE,
+                "fastgs_render: primitive state of %zu bytes, %zu needed", primitive_state_bytes,
+                fgs_prim_layout(N).total);
+    GSX_REQUIRE(pixel_state_bytes >= gsx_fastgs_pixel_state_bytes(W, H) && ((uintptr_t)pixel_state & 255) == 0,
+                GSX_ERR_WORKSPACE, "fastgs_render: pixel state needs %zu bytes, 256-byte aligned",
+                gsx_fastgs_pixel_state_bytes(W, H));
     const FgsInstLayout IL = fgs_inst_layout(n_instances, n_tiles);
     GSX_REQUIRE(instance_state && ((uintptr_t)instance_state & 255) == 0 && instance_state_bytes >= IL.total,
                 GSX_ERR_WORKSPACE, "fastgs_render: instance state needs %zu bytes, 256-byte aligned", IL.total);
@@ -988,8 +994,9 @@ extern "C" int gsx_fastgs_instance_list(const gsx_fastgs_settings* settings, int
 extern "C" int gsx_fastgs_backward(uint32_t N, const float* means, const float* scales_raw, const float* rotations_raw,
                                    const float* sh_coefficients_rest, const float* w2c_host,
                                    const float* cam_position_host, const gsx_fastgs_settings* settings,
-                                   const void* primitive_state, int64_t n_instances, const void* instance_state,
-                                   const void* pixel_state, const float* background, const float* grad_image,
+                                   const void* primitive_state, size_t primitive_state_bytes, int64_t n_instances,
+                                   const void* instance_state, size_t instance_state_bytes, const void* pixel_state,
+                                   size_t pixel_state_bytes, const float* background, const float* grad_image,
                                    const float* grad_alpha, void* accum, size_t accum_bytes, float* grad_means,
                                    float* grad_scales_raw, float* grad_rotations_raw, float* grad_opacities_raw,
                                    float* grad_sh_coefficients_0, float* grad_sh_coefficients_rest, float* grad_w2c,
@@ -1016,6 +1023,13 @@ extern "C" int gsx_fastgs_backward(uint32_t N, const float* means, const float* 
                 (long long)n_instances);
     const uint32_t W = settings->width, H = settings->height, n_tiles = c.grid_w * c.grid_h;
     const FgsPrimLayout L = fgs_prim_layout(N);
+    GSX_REQUIRE(primitive_state_bytes >= L.total && instance_state_bytes >= fgs_inst_layout(n_instances, n_tiles).total &&
+                    pixel_state_bytes >= gsx_fastgs_pixel_state_bytes(W, H),
+                GSX_ERR_WORKSPACE,
+                "fastgs_backward: state buffers of %zu / %zu / %zu bytes, %zu / %zu / %zu needed (primitive / instance / "
+                "pixel): not the ones the forward filled for this N, instance count and image size",
+                primitive_state_bytes, instance_state_bytes, pixel_state_bytes, L.total,
+                fgs_inst_layout(n_instances, n_tiles).total, gsx_fastgs_pixel_state_bytes(W, H));
     const char* ps = (const char*)primitive_state;
     const int32_t *inst, *offsets;
     if ((rc = gsx_fastgs_instance_list(settings, n_instances, instance_state, &inst, &offsets)) != GSX_OK)

@@ -76,8 +76,9 @@ forward_wrapper(const at::Tensor& means, const at::Tensor& scales_raw, const at:
                                     prim.data_ptr(), (size_t)prim.numel(), &n_instances, /*wait=*/1, stream));
     at::Tensor inst = bytes(gsx_fastgs_instance_state_bytes(n_instances, S.width, S.height), means);
     at::Tensor pix = bytes(gsx_fastgs_pixel_state_bytes(S.width, S.height), means);
-    gsx_check(gsx_fastgs_render(N, &S, prim.data_ptr(), n_instances, inst.data_ptr(), (size_t)inst.numel(), nullptr,
-                                image.data_ptr<float>(), alpha.data_ptr<float>(), pix.data_ptr(), stream));
+    gsx_check(gsx_fastgs_render(N, &S, prim.data_ptr(), (size_t)prim.numel(), n_instances, inst.data_ptr(),
+                                (size_t)inst.numel(), nullptr, image.data_ptr<float>(), alpha.data_ptr<float>(),
+                                pix.data_ptr(), (size_t)pix.numel(), stream));
     at::Tensor bucket = at::empty({0}, means.options().dtype(at::kByte));
     return {image, alpha, prim, pix, inst, bucket, -1, (int)n_instances, 0, 0, 0};
 }
@@ -118,12 +119,21 @@ backward_wrapper(at::Tensor& densification_info, const at::Tensor& grad_image, c
                         densification_info.numel() == 2 * n,
                     "densification_info must be a contiguous CUDA tensor [2, N]");
     }
+    for (const at::Tensor* t : {&per_primitive_buffers, &per_tile_buffers, &per_instance_buffers})
+        TORCH_CHECK(t->is_cuda() && t->is_contiguous() && t->scalar_type() == at::kByte,
+                    "the state buffers must be the byte tensors forward_wrapper returned");
+    TORCH_CHECK(grad_image.is_cuda() && grad_image.scalar_type() == at::kFloat && grad_image.numel() == 3ll * width * height,
+                "grad_image must be a CUDA float tensor [3, H, W]");
+    TORCH_CHECK(grad_alpha.is_cuda() && grad_alpha.scalar_type() == at::kFloat && grad_alpha.numel() == 1ll * width * height,
+                "grad_alpha must be a CUDA float tensor [1, H, W]");
     const at::Tensor gi = grad_image.contiguous(), ga = grad_alpha.contiguous();
     at::Tensor accum = at::zeros({(int64_t)gsx_fastgs_accum_bytes((uint32_t)n)}, means.options().dtype(at::kByte));
     gsx_check(gsx_fastgs_backward((uint32_t)n, means.data_ptr<float>(), scales_raw.data_ptr<float>(),
                                   rotations_raw.data_ptr<float>(), opt_ptr(sh_coefficients_rest), cam.w2c.data_ptr<float>(),
-                                  cam.cam.data_ptr<float>(), &S, per_primitive_buffers.data_ptr(), n_instances,
-                                  per_instance_buffers.data_ptr(), per_tile_buffers.data_ptr(), nullptr, gi.data_ptr<float>(),
+                                  cam.cam.data_ptr<float>(), &S, per_primitive_buffers.data_ptr(),
+                                  (size_t)per_primitive_buffers.numel(), n_instances, per_instance_buffers.data_ptr(),
+                                  (size_t)per_instance_buffers.numel(), per_tile_buffers.data_ptr(),
+                                  (size_t)per_tile_buffers.numel(), nullptr, gi.data_ptr<float>(),
                                   ga.data_ptr<float>(), accum.data_ptr(), (size_t)accum.numel(), grad_means.data_ptr<float>(),
                                   grad_scales_raw.data_ptr<float>(), grad_rotations_raw.data_ptr<float>(),
                                   grad_opacities_raw.data_ptr<float>(), grad_sh0.data_ptr<float>(), opt_ptr(grad_shN),

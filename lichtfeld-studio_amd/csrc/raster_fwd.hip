@@ -43,7 +43,8 @@ __global__ void __launch_bounds__(256) pack_records_kernel(uint32_t N, const flo
 // STATS: count instead of rendering (for roofline accounting); stats[0] += (pixel, Gaussian) pairs evaluated,
 // [1] += pairs composited, [2] += pairs the backward pass walks (entries up to each pixel's last contributor),
 // [3] += (wave, Gaussian) iterations executed, [4] += (wave, Gaussian) iterations removed by the pixel bounds,
-// [5] += executed iterations in which at least one pixel reaches the alpha threshold.
+// [5] += executed iterations in which at least one pixel reaches the alpha threshold, [6] / [7] += the halves
+// (8x4 rows / 4x8 columns) of those iterations' blocks that hold such a pixel.
 // DIST: OpenCV pinhole distortion (each pixel's ray comes from a Newton undistortion; a pixel whose undistortion
 // does not converge is done from the start, RasterizeToPixelsFromWorld3DGSFwd.cu:145).
 template <uint32_t CDIM, bool STATS, bool DIST>
@@ -101,7 +102,7 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
 #pragma unroll
     for (uint32_t k = 0; k < CDIM; ++k)
         pix_out[k] = 0.f;
-    uint32_t n_eval = 0, n_comp = 0, n_iter = 0, n_skip = 0, n_hit = 0;
+    uint32_t n_eval = 0, n_comp = 0, n_iter = 0, n_skip = 0, n_hit = 0, n_half_rows = 0, n_half_cols = 0;
 
     for (uint32_t b = 0; b < num_batches; ++b) {
         // all four waves saturated: nothing left to stage (:190-194)
@@ -155,9 +156,13 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
             if (STATS) {
                 const bool contributes = !far_away && gsx::fmin(0.999f, a.w * gsx::exp_nonpos(power)) >= 1.f / 255.f;
                 const uint64_t act = __builtin_amdgcn_ballot_w64(true);
-                if (__builtin_amdgcn_ballot_w64(contributes) != 0 &&
-                    (act & ((1ull << (tr & 63u)) - 1ull)) == 0) // first active lane counts for the wave
+                const uint64_t cm = __builtin_amdgcn_ballot_w64(contributes);
+                if (cm != 0 && (act & ((1ull << (tr & 63u)) - 1ull)) == 0) { // first active lane counts for the wave
                     ++n_hit;
+                    // how many 8x4 (rows 0-3 / 4-7) and 4x8 (columns 0-3 / 4-7) halves of the block hold one
+                    n_half_rows += ((cm & 0xffffffffull) != 0) + ((cm >> 32) != 0);
+                    n_half_cols += ((cm & 0x0f0f0f0f0f0f0f0full) != 0) + ((cm & 0xf0f0f0f0f0f0f0f0ull) != 0);
+                }
             }
             if (__builtin_amdgcn_ballot_w64(!far_away) == 0 || far_away)
                 continue;
@@ -196,6 +201,8 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
             atomicAdd(&stats[4], (unsigned long long)n_skip);
         }
         atomicAdd(&stats[5], (unsigned long long)n_hit);
+        atomicAdd(&stats[6], (unsigned long long)n_half_rows);
+        atomicAdd(&stats[7], (unsigned long long)n_half_cols);
         return;
     }
 

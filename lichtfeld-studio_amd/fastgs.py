@@ -98,8 +98,9 @@ def forward_wrapper(means, scales_raw, rotations_raw, opacities_raw, sh_coeffici
         inst = e(lb.gsx_fastgs_instance_state_bytes(c_i64(n_instances), c_u32(width), c_u32(height)), dt=torch.uint8)
         pix = e(lb.gsx_fastgs_pixel_state_bytes(c_u32(width), c_u32(height)), dt=torch.uint8)
         image, alpha = e(3, height, width), e(1, height, width)
-        check(lb.gsx_fastgs_render(c_u32(N), ctypes.byref(S), _p(prim), c_i64(n_instances), _p(inst),
-                                   c_sz(inst.numel()), _p(background), _p(image), _p(alpha), _p(pix), s))
+        check(lb.gsx_fastgs_render(c_u32(N), ctypes.byref(S), _p(prim), c_sz(prim.numel()), c_i64(n_instances),
+                                   _p(inst), c_sz(inst.numel()), _p(background), _p(image), _p(alpha), _p(pix),
+                                   c_sz(pix.numel()), s))
     return (image, alpha, prim, pix, inst, e(0, dt=torch.uint8), -1, n_instances, 0, 0, 0)
 
 
@@ -125,12 +126,22 @@ def backward_wrapper(densification_info, grad_image, grad_alpha, image, alpha, m
     if info is not None and tuple(info.shape) != (2, N):
         raise ValueError("densification_info must be [2, N]")
     acc = _accumulator(dev, N)
+    for t, name, shape in ((grad_image, "grad_image", (3, height, width)), (grad_alpha, "grad_alpha", (1, height, width))):
+        if not (t.is_cuda and t.dtype == torch.float32 and tuple(t.shape) == shape):
+            raise ValueError(f"{name} must be a CUDA float tensor of shape {shape}")
+    for t, name in ((per_primitive_buffers, "per_primitive_buffers"), (per_tile_buffers, "per_tile_buffers"),
+                    (per_instance_buffers, "per_instance_buffers")):
+        if not (t.is_cuda and t.dtype == torch.uint8 and t.is_contiguous()):
+            raise ValueError(f"{name} must be the byte tensor forward_wrapper returned")
     gi, ga = grad_image.contiguous(), grad_alpha.contiguous()
     with torch.cuda.device(dev):
         check(lb.gsx_fastgs_backward(c_u32(N), _p(means), _p(scales_raw), _p(rotations_raw), _p(sh_coefficients_rest),
                                      c_p(w.ctypes.data), c_p(c.ctypes.data), ctypes.byref(S),
-                                     _p(per_primitive_buffers), c_i64(n_instances), _p(per_instance_buffers),
-                                     _p(per_tile_buffers), _p(background), _p(gi), _p(ga), _p(acc), c_sz(acc.numel()),
+                                     _p(per_primitive_buffers), c_sz(per_primitive_buffers.numel()),
+                                     c_i64(n_instances), _p(per_instance_buffers),
+                                     c_sz(per_instance_buffers.numel()), _p(per_tile_buffers),
+                                     c_sz(per_tile_buffers.numel()), _p(background), _p(gi), _p(ga), _p(acc),
+                                     c_sz(acc.numel()),
                                      _p(g_means), _p(g_scales), _p(g_rot), _p(g_op), _p(g_sh0), _p(g_shN), _p(g_w2c),
                                      _p(info), _stream(dev)))
     return g_means, g_scales, g_rot, g_op, g_sh0, g_shN, g_w2c

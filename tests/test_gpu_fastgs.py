@@ -166,6 +166,17 @@ def test_wrapper_rejects_bad_inputs(gsx, cuda):
                                 D["scales_raw"], D["rotations_raw"], D["shN"], out[2], out[3], out[4], out[5], V, cam_pos,
                                 16, 64, 48, 60.0, 60.0, 32.0, 24.0, 0.01, 1e10, *out[6:11])
     assert all(float(t.abs().max()) == 0.0 for t in g[:6])
+    # state buffers that do not belong to this call are refused before any kernel runs
+    ok = fastgs.forward_wrapper(D["means"], D["scales_raw"], D["rotations_raw"], D["opacities_raw"], D["sh0"], D["shN"],
+                                V, cam_pos, 16, 64, 48, 60.0, 60.0, 32.0, 24.0, 0.01, 1e10)
+    with pytest.raises(GsxError, match="state buffers"):
+        fastgs.backward_wrapper(None, torch.ones_like(ok[0]), torch.ones_like(ok[1]), ok[0], ok[1], D["means"],
+                                D["scales_raw"], D["rotations_raw"], D["shN"], ok[2][:1024], ok[3], ok[4], ok[5], V,
+                                cam_pos, 16, 64, 48, 60.0, 60.0, 32.0, 24.0, 0.01, 1e10, *ok[6:11])
+    with pytest.raises(ValueError, match="grad_image"):
+        fastgs.backward_wrapper(None, torch.ones((3, 10, 10), device=cuda), torch.ones_like(ok[1]), ok[0], ok[1],
+                                D["means"], D["scales_raw"], D["rotations_raw"], D["shN"], ok[2], ok[3], ok[4], ok[5], V,
+                                cam_pos, 16, 64, 48, 60.0, 60.0, 32.0, 24.0, 0.01, 1e10, *ok[6:11])
 
 
 def test_full_size_1m_gaussians(gsx, cuda):
