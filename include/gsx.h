@@ -302,6 +302,14 @@ GSX_API int gsx_mcmc_relocate(uint32_t N, uint32_t n_idx, const int64_t* sampled
 /* ---- a13: gsplat::add_noise (Ops.h:59-65; RelocationCUDA.cu:112-144); means updated in place ---- */
 GSX_API int gsx_add_noise(int N, const float* raw_opacities, const float* raw_scales, const float* raw_quats,
                           const float* noise, float* means, float current_lr, void* stream);
+/* The same with the N(0,1) draws of mcmc.cpp:358 (torch::randn_like) generated where they are consumed: row i of the
+ * noise is a function of (seed, offset, i) only - Philox4x32-10 with counter (i, offset) and key seed, two Box-Muller
+ * pairs - so no [N,3] tensor is written and read back.  A caller advances `offset` per call.  The stream of values
+ * is not torch's (no implementation outside torch reproduces that); gsx_philox_randn3 writes the same rows out for
+ * callers that want them (out [N,3]): gsx_add_noise with that tensor equals gsx_add_noise_philox bit for bit. */
+GSX_API int gsx_philox_randn3(uint32_t N, uint64_t seed, uint64_t offset, float* out, void* stream);
+GSX_API int gsx_add_noise_philox(int N, const float* raw_opacities, const float* raw_scales, const float* raw_quats,
+                                 float* means, float current_lr, uint64_t seed, uint64_t offset, void* stream);
 /* ---- a14: gsplat::quats_to_rotmats (Ops.h:46-48; QuatToRotmatCUDA.cu:14-39) -> [N,3,3] row-major ---- */
 GSX_API int gsx_quats_to_rotmats(int N, const float* quats, float* rotmats, void* stream);
 

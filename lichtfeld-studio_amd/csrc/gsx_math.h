@@ -163,6 +163,9 @@ GSX_HD float sin(float x) {
     return sgn * r;
 }
 
+// cos on [-pi, pi] through the same cores: cos(x) = sin(pi/2 - |x|), whose argument stays inside [-pi/2, pi/2].
+GSX_HD float cos(float x) { return gsx::sin(1.57079632679489661923f - gsx::fabs(x)); }
+
 // acos on [-1, 1] (Cephes asinf core).
 GSX_HD float asin_core(float a) { // 0 <= a <= 0.5
     const float z = a * a;

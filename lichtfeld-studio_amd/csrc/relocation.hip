@@ -112,11 +112,50 @@ __global__ void __launch_bounds__(256) mcmc_rows_kernel(uint32_t n, const int64_
         p[dead[i] * r + f] = p[s * r + f];
 }
 
+// ---- counter-based normal draws (torch::randn_like of mcmc.cpp:358 generated where it is consumed) ----
+// Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3", SC'11), counter
+// (row, offset lo, offset hi, 0), key = seed; two Box-Muller pairs give the row's three N(0,1) values.
+__device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
+                                              uint32_t k1, uint32_t* out) {
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+        const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n1 = (uint32_t)p1;
+        const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1, n3 = (uint32_t)p0;
+        c0 = n0, c1 = n1, c2 = n2, c3 = n3;
+        k0 += 0x9E3779B9u, k1 += 0xBB67AE85u;
+    }
+    out[0] = c0, out[1] = c1, out[2] = c2, out[3] = c3;
+}
+
+__device__ __forceinline__ vec3 philox_normal3(uint32_t row, uint64_t seed, uint64_t offset) {
+    uint32_t u[4];
+    philox4x32_10(row, (uint32_t)offset, (uint32_t)(offset >> 32), 0u, (uint32_t)seed, (uint32_t)(seed >> 32), u);
+    const float scale = 5.9604644775390625e-8f; // 2^-24
+    // radius from a uniform in (0, 1], angle pi (2 v - 1) with v uniform in [0, 1)
+    const float ra = gsx::sqrt(-2.0f * gsx::log((float)((u[0] >> 8) + 1u) * scale));
+    const float rb = gsx::sqrt(-2.0f * gsx::log((float)((u[2] >> 8) + 1u) * scale));
+    const float pa = 3.14159265358979323846f * (2.0f * ((float)(u[1] >> 8) * scale) - 1.0f);
+    const float pb = 3.14159265358979323846f * (2.0f * ((float)(u[3] >> 8) * scale) - 1.0f);
+    return mk3(ra * gsx::cos(pa), ra * gsx::sin(pa), rb * gsx::cos(pb));
+}
+
+__global__ void __launch_bounds__(256) philox_randn3_kernel(uint32_t N, uint64_t seed, uint64_t offset,
+                                                             float* __restrict__ out) {
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= N)
+        return;
+    const vec3 z = philox_normal3(idx, seed, offset);
+    out[3 * (size_t)idx] = z.x, out[3 * (size_t)idx + 1] = z.y, out[3 * (size_t)idx + 2] = z.z;
+}
+
+// NOISE_FROM_RNG: the N(0,1) row is drawn in the kernel (noise == nullptr) instead of read
+template <bool NOISE_FROM_RNG>
 __global__ void __launch_bounds__(256) add_noise_kernel(int N, const float* __restrict__ raw_opacities,
                                                          const float* __restrict__ raw_scales,
                                                          const float* __restrict__ raw_quats,
                                                          const float* __restrict__ noise, float* __restrict__ means,
-                                                         float current_lr) {
+                                                         float current_lr, uint64_t seed, uint64_t offset) {
     const int idx = blockIdx.x * 256 + threadIdx.x;
     if (idx >= N)
         return;
@@ -133,7 +172,7 @@ __global__ void __launch_bounds__(256) add_noise_kernel(int N, const float* __re
             a = fma(R.m[i][2] * s2[2], R.m[j][2], a);
             cov.m[i][j] = a;
         }
-    const vec3 tn = mul(cov, ld3(noise, idx));
+    const vec3 tn = mul(cov, NOISE_FROM_RNG ? philox_normal3((uint32_t)idx, seed, offset) : ld3(noise, idx));
     const float opacity = 1.0f / (1.f + gsx::exp(-raw_opacities[idx]));
     const float op_sigmoid = 1.0f / (1.f + gsx::exp(100.f * opacity - 0.5f));
     const float noise_factor = current_lr * op_sigmoid;
@@ -165,8 +204,30 @@ extern "C" int gsx_add_noise(int N, const float* raw_opacities, const float* raw
         return GSX_OK;
     GSX_REQUIRE(raw_opacities && raw_scales && raw_quats && noise && means, GSX_ERR_INVALID_ARGUMENT,
                 "add_noise: null tensor");
-    hipLaunchKernelGGL(add_noise_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, raw_opacities,
-                       raw_scales, raw_quats, noise, means, current_lr);
+    hipLaunchKernelGGL(add_noise_kernel<false>, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N,
+                       raw_opacities, raw_scales, raw_quats, noise, means, current_lr, (uint64_t)0, (uint64_t)0);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+extern "C" int gsx_philox_randn3(uint32_t N, uint64_t seed, uint64_t offset, float* out, void* stream) {
+    if (N == 0)
+        return GSX_OK;
+    GSX_REQUIRE(out != nullptr, GSX_ERR_INVALID_ARGUMENT, "philox_randn3: null tensor");
+    hipLaunchKernelGGL(philox_randn3_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, seed, offset, out);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+extern "C" int gsx_add_noise_philox(int N, const float* raw_opacities, const float* raw_scales,
+                                    const float* raw_quats, float* means, float current_lr, uint64_t seed,
+                                    uint64_t offset, void* stream) {
+    if (N <= 0)
+        return GSX_OK;
+    GSX_REQUIRE(raw_opacities && raw_scales && raw_quats && means, GSX_ERR_INVALID_ARGUMENT,
+                "add_noise_philox: null tensor");
+    hipLaunchKernelGGL(add_noise_kernel<true>, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N,
+                       raw_opacities, raw_scales, raw_quats, (const float*)nullptr, means, current_lr, seed, offset);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

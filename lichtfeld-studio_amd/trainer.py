@@ -392,11 +392,17 @@ class TrainStep:
                   self._stream())
         return n
 
-    def inject_noise(self, noise, noise_lr=5e5):
-        """MCMC::inject_noise (mcmc.cpp:349-367) with the caller's N(0,1) draws [N,3]."""
-        self._run("add_noise", self.lib.gsx_add_noise, c_i(self.N), _p(self.params["opacity"]),
-                  _p(self.params["scaling"]), _p(self.params["rotation"]), _p(noise), _p(self.params["means"]),
-                  c_f(self.lrs["means"] * noise_lr), self._stream())
+    def inject_noise(self, noise=None, noise_lr=5e5, seed=0):
+        """MCMC::inject_noise (mcmc.cpp:349-367): with the caller's N(0,1) draws [N,3], or (noise = None) with draws
+        generated inside the kernel from (seed, iteration, row) - no [N,3] tensor is written and read back."""
+        P = self.params
+        if noise is None:
+            self._run("add_noise_philox", self.lib.gsx_add_noise_philox, c_i(self.N), _p(P["opacity"]),
+                      _p(P["scaling"]), _p(P["rotation"]), _p(P["means"]), c_f(self.lrs["means"] * noise_lr),
+                      ctypes.c_uint64(seed), ctypes.c_uint64(self.iteration), self._stream())
+            return
+        self._run("add_noise", self.lib.gsx_add_noise, c_i(self.N), _p(P["opacity"]), _p(P["scaling"]),
+                  _p(P["rotation"]), _p(noise), _p(P["means"]), c_f(self.lrs["means"] * noise_lr), self._stream())
 
     loss_pending = False
 

@@ -1848,3 +1848,38 @@ ORC_API void orc_camera_unproject(int64_t n, const float* image_points, float fx
         rays[3 * i] = d.x, rays[3 * i + 1] = d.y, rays[3 * i + 2] = d.z;
     }
 }
+
+// ---------------------------------------------------------------------------------------------
+// counter-based normal draws: Philox4x32-10 (Salmon et al., SC'11; known-answer vectors of the Random123
+// distribution in tests/test_oracle_loss_opt.py) + Box-Muller.  Stands in for torch::randn_like of mcmc.cpp:358,
+// whose stream no implementation outside torch reproduces: "parity unpinned" against the reference's values, pinned
+// as a generator (known answers, moments, Kolmogorov-Smirnov).
+// ---------------------------------------------------------------------------------------------
+ORC_API void orc_philox4x32_10(const uint32_t* ctr, const uint32_t* key, uint32_t* out) {
+    uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3], k0 = key[0], k1 = key[1];
+    for (int r = 0; r < 10; ++r) {
+        const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+        const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n1 = (uint32_t)p1;
+        const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1, n3 = (uint32_t)p0;
+        c0 = n0, c1 = n1, c2 = n2, c3 = n3;
+        k0 += 0x9E3779B9u, k1 += 0xBB67AE85u;
+    }
+    out[0] = c0, out[1] = c1, out[2] = c2, out[3] = c3;
+}
+
+ORC_API void orc_philox_randn3(uint32_t N, uint64_t seed, uint64_t offset, float* out) {
+    const float scale = 5.9604644775390625e-8f; // 2^-24
+    for (uint32_t i = 0; i < N; ++i) {
+        const uint32_t ctr[4] = {i, (uint32_t)offset, (uint32_t)(offset >> 32), 0u};
+        const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+        uint32_t u[4];
+        orc_philox4x32_10(ctr, key, u);
+        const float ra = gsx::sqrt(-2.0f * gsx::log((float)((u[0] >> 8) + 1u) * scale));
+        const float rb = gsx::sqrt(-2.0f * gsx::log((float)((u[2] >> 8) + 1u) * scale));
+        const float pa = 3.14159265358979323846f * (2.0f * ((float)(u[1] >> 8) * scale) - 1.0f);
+        const float pb = 3.14159265358979323846f * (2.0f * ((float)(u[3] >> 8) * scale) - 1.0f);
+        out[3 * (size_t)i] = ra * gsx::cos(pa);
+        out[3 * (size_t)i + 1] = ra * gsx::sin(pa);
+        out[3 * (size_t)i + 2] = rb * gsx::cos(pb);
+    }
+}

@@ -90,6 +90,20 @@ def camera_unproject(image_points, fx, fy, cx, cy):
     return rays, valid.astype(bool)
 
 
+def philox4x32_10(ctr, key):
+    c, k = np.asarray(ctr, np.uint32).copy(), np.asarray(key, np.uint32).copy()
+    out = np.zeros(4, np.uint32)
+    lib().orc_philox4x32_10(_p(c), _p(k), _p(out))
+    return out
+
+
+def philox_randn3(n, seed, offset):
+    """[n,3] N(0,1) rows, row i a function of (seed, offset, i): the draws gsx_add_noise_philox consumes"""
+    out = np.zeros((n, 3), np.float32)
+    lib().orc_philox_randn3(c_u32(n), ctypes.c_uint64(seed), ctypes.c_uint64(offset), _p(out))
+    return out
+
+
 def num_threads():
     return lib().orc_num_threads()
 

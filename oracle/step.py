@@ -121,9 +121,11 @@ class OracleTrainStep:
             self.exp_avg_sq[k] = np.ascontiguousarray(np.concatenate([self.exp_avg_sq[k], zeros], 0))
         return sampled_idxs.size
 
-    def inject_noise(self, noise, noise_lr=5e5):
-        """MCMC::inject_noise (mcmc.cpp:349-367)"""
+    def inject_noise(self, noise=None, noise_lr=5e5, seed=0, iteration=0):
+        """MCMC::inject_noise (mcmc.cpp:349-367); noise = None: the counter-based draws for (seed, iteration)"""
         P = self.params
+        if noise is None:
+            noise = orc.philox_randn3(P["means"].shape[0], seed, iteration)
         orc.add_noise(P["opacity"], P["scaling"], P["rotation"], noise, P["means"],
                       np.float32(self.lrs["means"] * noise_lr))
 

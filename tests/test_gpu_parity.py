@@ -645,3 +645,27 @@ def test_opencv_distortion_projection_and_errors(gsx, orc, cuda):
         call(None, None, None, model=2)  # FISHEYE
     with pytest.raises(RuntimeError, match="rolling shutter"):
         call(None, None, None, rs=0)  # ROLLING_TOP_TO_BOTTOM
+
+
+def test_philox_noise_on_device(gsx, orc, cuda):
+    """gsx_philox_randn3 equals the checker's counter-based draws bit for bit; gsx_add_noise_philox equals gsx_add_noise
+    fed with those rows bit for bit (the [N,3] noise tensor never has to exist)"""
+    import ctypes
+    from lichtfeld_studio_amd._lib import c_f, c_i, c_p, c_u32, check, lib
+    L = lib()
+    n = 100_003
+    s = c_p(torch.cuda.current_stream(cuda).cuda_stream)
+    out = torch.empty((n, 3), dtype=torch.float32, device=cuda)
+    check(L.gsx_philox_randn3(c_u32(n), ctypes.c_uint64(0x123456789abcdef), ctypes.c_uint64(77), c_p(out.data_ptr()), s))
+    want = orc.philox_randn3(n, 0x123456789abcdef, 77)
+    bits_equal(N(out), want, "philox rows")
+    sc = gsx.scenes.config(3, n)
+    P = {k: T(v, cuda) for k, v in dict(op=sc.opacity_raw.reshape(-1), sc=sc.scaling_raw, q=sc.rotation_raw,
+                                        m=sc.means).items()}
+    m2 = P["m"].clone()
+    p = lambda t: c_p(t.data_ptr())
+    check(L.gsx_add_noise(c_i(n), p(P["op"]), p(P["sc"]), p(P["q"]), p(out), p(P["m"]), c_f(0.3), s))
+    check(L.gsx_add_noise_philox(c_i(n), p(P["op"]), p(P["sc"]), p(P["q"]), p(m2), c_f(0.3),
+                                 ctypes.c_uint64(0x123456789abcdef), ctypes.c_uint64(77), s))
+    torch.cuda.synchronize()
+    assert torch.equal(P["m"], m2) and not torch.equal(m2, T(sc.means, cuda))

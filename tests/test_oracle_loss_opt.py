@@ -237,3 +237,26 @@ def test_l1_regularization_matches_autograd(orc):
         assert orc.l1_regularization(mode, x, None, 0.013) == got
         g2 = g0.copy()
         assert orc.l1_regularization(mode, x, g2, 0.0) == 0.0 and np.array_equal(g2, g0)
+
+
+def test_philox_known_answers_and_normal_draws(orc):
+    """Philox4x32-10 against the known-answer vectors of the Random123 distribution (kat_vectors: zero, all-ones and
+    pi-digit inputs); the Box-Muller rows: moments, independence of the three columns, Kolmogorov-Smirnov against
+    N(0,1), different (seed, offset) give different rows, the same give the same"""
+    from scipy import stats
+    kat = [([0, 0, 0, 0], [0, 0], "6627e8d5 e169c58d bc57ac4c 9b00dbd8"),
+           ([0xffffffff] * 4, [0xffffffff] * 2, "408f276d 41c83b0e a20bc7c6 6d5451fd"),
+           ([0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344], [0xa4093822, 0x299f31d0],
+            "d16cfe09 94fdcceb 5001e420 24126ea1")]
+    for ctr, key, want in kat:
+        assert " ".join("%08x" % v for v in orc.philox4x32_10(ctr, key)) == want
+    z = orc.philox_randn3(400_000, 11, 5)
+    assert np.isfinite(z).all() and np.abs(z).max() < 6.0  # |z| <= sqrt(2 * 24 ln 2) = 5.77
+    assert np.abs(z.mean(0)).max() < 6e-3 and np.abs(z.std(0) - 1).max() < 4e-3
+    c = np.corrcoef(z.T)
+    assert np.abs(c - np.eye(3)).max() < 6e-3
+    for k in range(3):
+        assert stats.kstest(z[:100_000, k].astype(np.float64), "norm").pvalue > 1e-3
+    assert np.array_equal(z, orc.philox_randn3(400_000, 11, 5))
+    assert not np.array_equal(z[:100], orc.philox_randn3(100, 11, 6))
+    assert not np.array_equal(z[:100], orc.philox_randn3(100, 12, 5))
