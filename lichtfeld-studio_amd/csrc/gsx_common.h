@@ -8,6 +8,7 @@
 #define GSX_BUILD 1
 #include "../../include/gsx.h"
 #include "gsx_math.h"
+#include "gsx_camera.h"
 #include "gsx_record.h"
 
 namespace gsx {
@@ -165,21 +166,56 @@ __device__ __forceinline__ bool opencv_undistort_newton(const Distortion& d, flo
     return converged;
 }
 
-// world ray through a pixel centre, (distorted) pinhole, global shutter (Cameras.cuh:457-470 / 742-755 unproject,
-// :253-266 camera_ray_to_world_ray, :322-339).  Returns the ray's valid flag: false only when an undistortion did
-// not converge (the ray is then zero, :330-333, and the pixel takes no part in either pass).
+// The camera model of one call: the (distorted) pinhole, the OpenCV fisheye or the equirectangular model
+// (gsx_camera_model values; the reference's dispatch, ProjectionUT3DGSFused.cu:86-136).
+struct CameraModel {
+    int type; // 0 pinhole (dist.on: with distortion), 2 fisheye, 3 equirectangular
+    Distortion dist;
+    Fisheye fe;
+    float W, H;
+};
+
+__device__ __forceinline__ CameraModel load_camera_model(int type, const float* __restrict__ radial,
+                                                         const float* __restrict__ tangential,
+                                                         const float* __restrict__ thin_prism, float fx, float fy,
+                                                         float cx, float cy, uint32_t W, uint32_t H) {
+    CameraModel m;
+    m.type = type;
+    m.W = (float)W, m.H = (float)H;
+    m.dist.on = false;
+    if (type == 2)
+        m.fe = fisheye_setup(radial, fx, fy, cx, cy, W, H);
+    else if (type == 0)
+        m.dist = load_distortion(radial, tangential, thin_prism);
+    return m;
+}
+
+// world ray through a pixel centre, global shutter (Cameras.cuh:457-470 / 742-755 / 961-1000 / 1027-1036
+// unproject, :253-266 camera_ray_to_world_ray, :322-339).  Returns the ray's valid flag: false when an undistortion
+// or the fisheye inverse did not converge or left the field of view (the ray is then zero, :330-333, and the pixel
+// takes no part in either pass).
 __device__ __forceinline__ bool pixel_world_ray(const CamPose& cp, float px, float py, float fx, float fy, float cx,
-                                                float cy, const Distortion& dist, vec3* ray_o, vec3* ray_d) {
-    float u = (px - cx) / fx;
-    float v = (py - cy) / fy;
-    if (dist.on && !opencv_undistort_newton(dist, u, v, &u, &v)) {
+                                                float cy, const CameraModel& cam, vec3* ray_o, vec3* ray_d) {
+    vec3 d_cam;
+    bool ok = true;
+    if (cam.type == 2) {
+        ok = fisheye_unproject(cam.fe, px, py, &d_cam);
+    } else if (cam.type == 3) {
+        equirect_unproject(cam.W, cam.H, px, py, &d_cam);
+    } else {
+        float u = (px - cx) / fx;
+        float v = (py - cy) / fy;
+        if (cam.dist.on)
+            ok = opencv_undistort_newton(cam.dist, u, v, &u, &v);
+        const vec3 cr = mk3(u, v, 1.f);
+        const float len = gsx::sqrt(dot(cr, cr));
+        d_cam = mk3(cr.x / len, cr.y / len, cr.z / len);
+    }
+    if (!ok) {
         *ray_o = mk3(0.f, 0.f, 0.f);
         *ray_d = mk3(0.f, 0.f, 0.f);
         return false;
     }
-    const vec3 cr = mk3(u, v, 1.f);
-    const float len = gsx::sqrt(dot(cr, cr));
-    const vec3 d_cam = mk3(cr.x / len, cr.y / len, cr.z / len);
     quat q;
     vec3 t;
     shutter_pose(cp, 0.f, &q, &t);

@@ -300,6 +300,9 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> rasterize_to_pixels_from_world_3d
     }
     const uint32_t C = (uint32_t)tile_offsets.size(0), N = (uint32_t)means.size(0);
     const uint32_t channels = (uint32_t)colors.size(-1);
+    TORCH_CHECK(!has(backgrounds) || (backgrounds->dim() == 2 && backgrounds->size(0) == C &&
+                                      backgrounds->size(1) == channels),
+                "backgrounds must be [C, channels] = [", C, ", ", channels, "], got ", backgrounds->sizes());
     auto opt = means.options();
     at::Tensor renders = at::empty({C, image_height, image_width, channels}, opt);
     at::Tensor alphas = at::empty({C, image_height, image_width, 1}, opt);
@@ -346,6 +349,10 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> rasterize
     }
     const uint32_t channels = (uint32_t)colors.size(-1);
     TORCH_CHECK(channels == 1 || channels == 3 || channels == 4, "Unsupported number of channels: ", channels);
+    TORCH_CHECK(!has(backgrounds) || (backgrounds->dim() == 2 && backgrounds->size(0) == tile_offsets.size(0) &&
+                                      backgrounds->size(1) == channels),
+                "backgrounds must be [C, channels] = [", tile_offsets.size(0), ", ", channels, "], got ",
+                backgrounds->sizes());
     const uint32_t C = (uint32_t)tile_offsets.size(0), N = (uint32_t)means.size(0);
     // the kernels write every element of the five outputs (the reference zero-fills, Rasterization.cpp:190-194)
     at::Tensor v_means = at::empty_like(means), v_quats = at::empty_like(quats), v_scales = at::empty_like(scales);
@@ -361,6 +368,25 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> rasterize
         v_means.data_ptr<float>(), v_quats.data_ptr<float>(), v_scales.data_ptr<float>(), v_colors.data_ptr<float>(),
         v_opacities.data_ptr<float>(), ws.data_ptr(), (size_t)ws.numel(), cur_stream(means)));
     return std::make_tuple(v_means, v_quats, v_scales, v_colors, v_opacities);
+}
+
+// The fused operators hand the caller's background ([C,3] from gs::training::rasterize, rasterizer.cpp:84-87, 147)
+// to a kernel that blends `channels` values per pixel (Rasterization.cpp:401-407): with RGB + depth it would read one
+// float past each row.  Here the missing channels' background is 0 and surplus ones are dropped (for one camera the
+// values the reference's kernel reads).
+static OptT fit_backgrounds(const OptT& backgrounds, int64_t channels) {
+    if (!backgrounds.has_value() || !backgrounds->defined() || backgrounds->numel() == 0)
+        return at::nullopt;
+    const at::Tensor& b = backgrounds.value();
+    const int64_t have = b.size(-1);
+    if (have > channels)
+        return b.slice(-1, 0, channels).contiguous();
+    if (have < channels) {
+        auto shape = b.sizes().vec();
+        shape.back() = channels - have;
+        return at::cat({b, at::zeros(shape, b.options())}, -1).contiguous();
+    }
+    return b;
 }
 
 std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor,
@@ -415,7 +441,7 @@ rasterize_from_world_with_sh_fwd(const at::Tensor means, const at::Tensor quats,
     at::Tensor flatten_ids = std::get<2>(isect);
     at::Tensor offsets = intersect_offset(std::get<1>(isect), C, tile_width, tile_height);
     auto r = rasterize_to_pixels_from_world_3dgs_fwd(means, quats, scaled_scales, colors, final_opacities.contiguous(),
-                                                     backgrounds, masks, image_width, image_height, tile_size,
+                                                     fit_backgrounds(backgrounds, colors.size(-1)), masks, image_width, image_height, tile_size,
                                                      viewmats0, viewmats1, Ks, camera_model, ut_params, rs_type,
                                                      radial_coeffs, tangential_coeffs, thin_prism_coeffs, offsets,
                                                      flatten_ids);
@@ -450,7 +476,7 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> rasterize
         final_opacities = at::mul(final_opacities, compensations).contiguous();
     at::Tensor scaled_scales = scaling_modifier == 1.0f ? scales : at::mul(scales, scaling_modifier);
     auto g = rasterize_to_pixels_from_world_3dgs_bwd(means, quats, scaled_scales, colors, final_opacities.contiguous(),
-                                                     backgrounds, masks, image_width, image_height, tile_size,
+                                                     fit_backgrounds(backgrounds, colors.size(-1)), masks, image_width, image_height, tile_size,
                                                      viewmats0, viewmats1, Ks, camera_model, ut_params, rs_type,
                                                      radial_coeffs, tangential_coeffs, thin_prism_coeffs, tile_offsets,
                                                      flatten_ids, render_alphas, last_ids, v_render_colors,

@@ -30,7 +30,7 @@ struct ProjCfg {
     float ut_alpha, ut_beta, ut_kappa, ut_margin;
     int ut_require_all;
     float fx, fy, cx, cy;
-    Distortion dist; // OpenCV pinhole distortion; dist.on = false: the perfect pinhole model
+    CameraModel cam; // type 0 with cam.dist.on = false: the perfect pinhole model
 };
 
 __device__ __forceinline__ bool pinhole_project(vec3 cam, const ProjCfg& cfg, vec2* out) {
@@ -56,7 +56,7 @@ __device__ __forceinline__ bool opencv_project(vec3 cam, const ProjCfg& cfg, vec
         return false;
     const float u = cam.x / cam.z, v = cam.y / cam.z;
     float icD, dx, dy;
-    compute_distortion(cfg.dist, u, v, &icD, &dx, &dy);
+    compute_distortion(cfg.cam.dist, u, v, &icD, &dx, &dy);
     const bool valid_radial = icD > 0.8f;
     out->x = (icD * u + dx) * cfg.fx + cfg.cx;
     out->y = (icD * v + dy) * cfg.fy + cfg.cy;
@@ -103,7 +103,15 @@ __device__ __forceinline__ bool project_ut(const ProjCfg& cfg, const CamPose& cp
         }
         const vec3 pc = add(quat_rotate(cp.q_start, p), cp.t_start);
         vec2 uv;
-        const bool pv = cfg.dist.on ? opencv_project(pc, cfg, &uv) : pinhole_project(pc, cfg, &uv);
+        bool pv;
+        if (cfg.cam.type == 2) {
+            pv = fisheye_project(cfg.cam.fe, pc, cfg.ut_margin, &uv);
+        } else if (cfg.cam.type == 3) {
+            equirect_project((float)cfg.W, (float)cfg.H, pc, &uv);
+            pv = true; // Cameras.cuh:1013-1025 returns valid for every point
+        } else {
+            pv = cfg.cam.dist.on ? opencv_project(pc, cfg, &uv) : pinhole_project(pc, cfg, &uv);
+        }
         if (cfg.ut_require_all) {
             valid &= pv;
             if (!pv)
@@ -170,20 +178,23 @@ __device__ __forceinline__ bool project_ut(const ProjCfg& cfg, const CamPose& cp
 __global__ void __launch_bounds__(256) projection_ut_kernel(
     uint32_t C, uint32_t N, const float* __restrict__ means, const float* __restrict__ quats,
     const float* __restrict__ scales, const float* __restrict__ opacities, const float* __restrict__ viewmats0,
-    const float* __restrict__ Ks, const float* __restrict__ radial, const float* __restrict__ tangential,
-    const float* __restrict__ thin_prism, ProjCfg cfg, int32_t* __restrict__ radii, float* __restrict__ means2d,
+    const float* __restrict__ Ks, int camera_model, const float* __restrict__ radial,
+    const float* __restrict__ tangential, const float* __restrict__ thin_prism, ProjCfg cfg,
+    int32_t* __restrict__ radii, float* __restrict__ means2d,
     float* __restrict__ depths, float* __restrict__ conics, float* __restrict__ compensations) {
     const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
     if (idx >= C * N)
         return;
     const uint32_t cid = idx / N, gid = idx % N;
-    cfg.dist = load_distortion(radial != nullptr ? radial + cid * 6 : nullptr,
-                               tangential != nullptr ? tangential + cid * 2 : nullptr,
-                               thin_prism != nullptr ? thin_prism + cid * 4 : nullptr);
     cfg.fx = Ks[cid * 9 + 0];
     cfg.fy = Ks[cid * 9 + 4];
     cfg.cx = Ks[cid * 9 + 2];
     cfg.cy = Ks[cid * 9 + 5];
+    const uint32_t n_radial = camera_model == GSX_FISHEYE ? 4u : 6u; // ProjectionUT3DGSFused.cu:103, 124
+    cfg.cam = load_camera_model(camera_model, radial != nullptr ? radial + cid * n_radial : nullptr,
+                                tangential != nullptr ? tangential + cid * 2 : nullptr,
+                                thin_prism != nullptr ? thin_prism + cid * 4 : nullptr, cfg.fx, cfg.fy, cfg.cx, cfg.cy,
+                                cfg.W, cfg.H);
     const CamPose cp = load_cam_pose(viewmats0 + cid * 16);
     ProjOut o;
     const bool ok = project_ut(cfg, cp, ld3(means, gid), ld4q(quats, gid), ld3(scales, gid), opacities != nullptr,
@@ -668,10 +679,10 @@ extern "C" int gsx_projection_ut_3dgs_fused(
     cfg.ut_margin = ut.in_image_margin_factor;
     cfg.ut_require_all = ut.require_all_sigma_points_valid;
     cfg.fx = cfg.fy = cfg.cx = cfg.cy = 0.f;
-    memset(&cfg.dist, 0, sizeof(cfg.dist));
+    memset(&cfg.cam, 0, sizeof(cfg.cam));
     hipLaunchKernelGGL(projection_ut_kernel, dim3(cdiv((uint64_t)C * N, 256)), dim3(256), 0, (hipStream_t)stream, C,
-                       N, means, quats, scales, opacities, viewmats0, Ks, radial_coeffs, tangential_coeffs,
-                       thin_prism_coeffs, cfg, radii, means2d, depths, conics, compensations);
+                       N, means, quats, scales, opacities, viewmats0, Ks, camera_model, radial_coeffs,
+                       tangential_coeffs, thin_prism_coeffs, cfg, radii, means2d, depths, conics, compensations);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

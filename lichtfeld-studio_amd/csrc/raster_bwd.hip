@@ -53,8 +53,9 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     const float* __restrict__ backgrounds,
     const uint8_t* __restrict__ masks, uint32_t image_width, uint32_t image_height, uint32_t tile_width,
     uint32_t tile_height, const float* __restrict__ viewmat, const float* __restrict__ Kmat,
-    const float* __restrict__ radial, const float* __restrict__ tangential, const float* __restrict__ thin_prism,
-    const int32_t* __restrict__ tile_offsets, const int32_t* __restrict__ flatten_ids,
+    int camera_model, const float* __restrict__ radial, const float* __restrict__ tangential,
+    const float* __restrict__ thin_prism, const int32_t* __restrict__ tile_offsets,
+    const int32_t* __restrict__ flatten_ids,
     const float* __restrict__ render_alphas, const int32_t* __restrict__ last_ids,
     const float* __restrict__ v_render_colors, const float* __restrict__ v_render_alphas,
     float* __restrict__ gacc /*[N,16]*/, float* __restrict__ gextra /*[N], CDIM == 4*/) {
@@ -82,12 +83,13 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
 
     const CamPose cp = load_cam_pose(viewmat);
     vec3 ray_o, ray_d;
-    Distortion dist;
-    dist.on = false;
+    CameraModel cam;
+    cam.type = 0, cam.dist.on = false;
     if (DIST)
-        dist = load_distortion(radial, tangential, thin_prism);
+        cam = load_camera_model(camera_model, radial, tangential, thin_prism, Kmat[0], Kmat[4], Kmat[2], Kmat[5],
+                                image_width, image_height);
     // a pixel without a valid ray takes no part (RasterizeToPixelsFromWorld3DGSBwd.cu:157)
-    inside &= pixel_world_ray(cp, (float)j + 0.5f, (float)i + 0.5f, Kmat[0], Kmat[4], Kmat[2], Kmat[5], dist, &ray_o,
+    inside &= pixel_world_ray(cp, (float)j + 0.5f, (float)i + 0.5f, Kmat[0], Kmat[4], Kmat[2], Kmat[5], cam, &ray_o,
                               &ray_d);
 
     const int32_t range_start = tile_offsets[tile_id];
@@ -355,8 +357,9 @@ int pack_raster_records(uint32_t N, const float* means, const float* quats, cons
 static int rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isects, const void* records,
                                     const float* colors, uint32_t channels, const float* backgrounds,
                                     const uint8_t* masks, uint32_t image_width, uint32_t image_height,
-                                    uint32_t tile_size, const float* viewmats0, const float* Ks, const float* radial,
-                                    const float* tangential, const float* thin_prism, const int32_t* tile_offsets,
+                                    uint32_t tile_size, const float* viewmats0, const float* Ks, int camera_model,
+                                    const float* radial, const float* tangential, const float* thin_prism,
+                                    const int32_t* tile_offsets,
                                     const int32_t* flatten_ids, const float* render_alphas, const int32_t* last_ids,
                                     const float* v_render_colors, const float* v_render_alphas, void* workspace,
                                     size_t workspace_bytes, void* stream) {
@@ -378,13 +381,14 @@ static int rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isects, co
     GSX_REQUIRE(channels <= 3 || colors != nullptr, GSX_ERR_INVALID_ARGUMENT, "rasterize bwd: colors is null");
     const uint32_t tw = cdiv(image_width, kTile), th = cdiv(image_height, kTile);
     float* gextra = (float*)((char*)workspace + accum_extra_offset(N));
-    const bool distorted = radial != nullptr || tangential != nullptr || thin_prism != nullptr;
+    const bool distorted =
+        camera_model != GSX_PINHOLE || radial != nullptr || tangential != nullptr || thin_prism != nullptr;
 #define GSX_LAUNCH_BWD(CD, DI)                                                                                       \
     hipLaunchKernelGGL((rasterize_bwd_kernel<CD, DI>), dim3(tw * th), dim3(256), 0, (hipStream_t)stream,             \
                        (uint32_t)n_isects, (const float4*)records, colors, backgrounds, masks, image_width,          \
-                       image_height, tw, th, viewmats0, Ks, radial, tangential, thin_prism, tile_offsets,            \
-                       flatten_ids, render_alphas, last_ids, v_render_colors, v_render_alphas, (float*)workspace,    \
-                       gextra)
+                       image_height, tw, th, viewmats0, Ks, camera_model, radial, tangential, thin_prism,            \
+                       tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors, v_render_alphas,         \
+                       (float*)workspace, gextra)
 #define GSX_LAUNCH_BWD2(CD)       \
     if (distorted)                \
         GSX_LAUNCH_BWD(CD, true); \
@@ -413,9 +417,9 @@ extern "C" int gsx_rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_is
                                             const float* v_render_colors, const float* v_render_alphas,
                                             void* workspace, size_t workspace_bytes, void* stream) {
     return rasterize_bwd_accumulate(C, N, n_isects, records, colors, channels, backgrounds, masks, image_width,
-                                    image_height, tile_size, viewmats0, Ks, nullptr, nullptr, nullptr, tile_offsets,
-                                    flatten_ids, render_alphas, last_ids, v_render_colors, v_render_alphas, workspace,
-                                    workspace_bytes, stream);
+                                    image_height, tile_size, viewmats0, Ks, GSX_PINHOLE, nullptr, nullptr, nullptr,
+                                    tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors,
+                                    v_render_alphas, workspace, workspace_bytes, stream);
 }
 
 // stage 3: per-Gaussian epilogue, accumulators -> the five gradient tensors (all elements written)
@@ -464,13 +468,13 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
     void* records = (char*)workspace + acc_bytes;
     if ((rc = gsx_rasterize_bwd_clear(N, workspace, acc_bytes, stream)) != GSX_OK)
         return rc;
-    const bool pinhole = !(radial_coeffs || tangential_coeffs || thin_prism_coeffs);
+    const bool pinhole = camera_model == GSX_PINHOLE && !(radial_coeffs || tangential_coeffs || thin_prism_coeffs);
     if ((rc = pack_raster_records(N, means, quats, scales, opacities, colors, channels, viewmats0, Ks, image_width,
                                   image_height, pinhole, records, stream)) != GSX_OK)
         return rc;
     if ((rc = rasterize_bwd_accumulate(C, N, n_isects, records, colors, channels, backgrounds, masks, image_width,
-                                       image_height, tile_size, viewmats0, Ks, radial_coeffs, tangential_coeffs,
-                                       thin_prism_coeffs, tile_offsets, flatten_ids, render_alphas, last_ids,
+                                       image_height, tile_size, viewmats0, Ks, camera_model, radial_coeffs,
+                                       tangential_coeffs, thin_prism_coeffs, tile_offsets, flatten_ids, render_alphas, last_ids,
                                        v_render_colors, v_render_alphas, workspace, acc_bytes, stream)) != GSX_OK)
         return rc;
     return gsx_rasterize_bwd_finish(N, means, quats, scales, viewmats0, workspace, acc_bytes, 0, channels, v_means,

@@ -45,15 +45,17 @@ __global__ void __launch_bounds__(256) pack_records_kernel(uint32_t N, const flo
 // [3] += (wave, Gaussian) iterations executed, [4] += (wave, Gaussian) iterations removed by the pixel bounds,
 // [5] += executed iterations in which at least one pixel reaches the alpha threshold, [6] / [7] += the halves
 // (8x4 rows / 4x8 columns) of those iterations' blocks that hold such a pixel.
-// DIST: OpenCV pinhole distortion (each pixel's ray comes from a Newton undistortion; a pixel whose undistortion
-// does not converge is done from the start, RasterizeToPixelsFromWorld3DGSFwd.cu:145).
+// DIST: any camera but the perfect pinhole - OpenCV distortion, fisheye, equirectangular (each pixel's ray comes
+// from the model's unprojection; a pixel without a valid ray is done from the start,
+// RasterizeToPixelsFromWorld3DGSFwd.cu:145).
 template <uint32_t CDIM, bool STATS, bool DIST>
 __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
     uint32_t n_isects, const float4* __restrict__ records, const float* __restrict__ colors,
     const float* __restrict__ backgrounds, const uint8_t* __restrict__ masks, uint32_t image_width,
     uint32_t image_height, uint32_t tile_width, uint32_t tile_height, const float* __restrict__ viewmat,
-    const float* __restrict__ Kmat, const float* __restrict__ radial, const float* __restrict__ tangential,
-    const float* __restrict__ thin_prism, const int32_t* __restrict__ tile_offsets,
+    const float* __restrict__ Kmat, int camera_model, const float* __restrict__ radial,
+    const float* __restrict__ tangential, const float* __restrict__ thin_prism,
+    const int32_t* __restrict__ tile_offsets,
     const int32_t* __restrict__ flatten_ids, float* __restrict__ render_colors, float* __restrict__ render_alphas,
     int32_t* __restrict__ last_ids, unsigned long long* __restrict__ stats) {
     __shared__ float4 stage[kBatch * 4];
@@ -83,12 +85,13 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
 
     const CamPose cp = load_cam_pose(viewmat);
     vec3 ray_o, ray_d;
-    Distortion dist;
-    dist.on = false;
+    CameraModel cam;
+    cam.type = 0, cam.dist.on = false;
     if (DIST)
-        dist = load_distortion(radial, tangential, thin_prism);
+        cam = load_camera_model(camera_model, radial, tangential, thin_prism, Kmat[0], Kmat[4], Kmat[2], Kmat[5],
+                                image_width, image_height);
     const bool ray_ok =
-        pixel_world_ray(cp, (float)j + 0.5f, (float)i + 0.5f, Kmat[0], Kmat[4], Kmat[2], Kmat[5], dist, &ray_o, &ray_d);
+        pixel_world_ray(cp, (float)j + 0.5f, (float)i + 0.5f, Kmat[0], Kmat[4], Kmat[2], Kmat[5], cam, &ray_o, &ray_d);
 
     const int32_t range_start = tile_offsets[tile_id];
     const int32_t range_end =
@@ -252,8 +255,9 @@ int pack_raster_records(uint32_t N, const float* means, const float* quats, cons
 
 int rasterize_records_fwd(int64_t n_isects, const void* records, const float* colors, uint32_t channels,
                           const float* backgrounds, const uint8_t* masks, uint32_t image_width, uint32_t image_height,
-                          const float* viewmat, const float* K, const float* radial, const float* tangential,
-                          const float* thin_prism, const int32_t* tile_offsets, const int32_t* flatten_ids,
+                          const float* viewmat, const float* K, int camera_model, const float* radial,
+                          const float* tangential, const float* thin_prism, const int32_t* tile_offsets,
+                          const int32_t* flatten_ids,
                           float* render_colors, float* render_alphas, int32_t* last_ids, void* stream) {
     if (image_width == 0 || image_height == 0)
         return GSX_OK;
@@ -265,12 +269,13 @@ int rasterize_records_fwd(int64_t n_isects, const void* records, const float* co
     const uint32_t tw = cdiv(image_width, kTile), th = cdiv(image_height, kTile);
     const dim3 grid(tw * th), block(256);
     hipStream_t s = (hipStream_t)stream;
-    const bool distorted = radial != nullptr || tangential != nullptr || thin_prism != nullptr;
+    const bool distorted =
+        camera_model != GSX_PINHOLE || radial != nullptr || tangential != nullptr || thin_prism != nullptr;
 #define GSX_LAUNCH_FWD(CD, DI)                                                                                      \
     hipLaunchKernelGGL((rasterize_fwd_kernel<CD, false, DI>), grid, block, 0, s, (uint32_t)n_isects,                \
                        (const float4*)records, colors, backgrounds, masks, image_width, image_height, tw, th,       \
-                       viewmat, K, radial, tangential, thin_prism, tile_offsets, flatten_ids, render_colors,        \
-                       render_alphas, last_ids, (unsigned long long*)nullptr)
+                       viewmat, K, camera_model, radial, tangential, thin_prism, tile_offsets, flatten_ids,         \
+                       render_colors, render_alphas, last_ids, (unsigned long long*)nullptr)
 #define GSX_LAUNCH_FWD2(CD)     \
     if (distorted)              \
         GSX_LAUNCH_FWD(CD, true); \
@@ -306,8 +311,8 @@ extern "C" int gsx_rasterize_records_fwd(int64_t n_isects, const void* records, 
                                          float* render_colors, float* render_alphas, int32_t* last_ids,
                                          void* stream) {
     return rasterize_records_fwd(n_isects, records, colors, channels, backgrounds, masks, image_width, image_height,
-                                 viewmat, K, nullptr, nullptr, nullptr, tile_offsets, flatten_ids, render_colors,
-                                 render_alphas, last_ids, stream);
+                                 viewmat, K, GSX_PINHOLE, nullptr, nullptr, nullptr, tile_offsets, flatten_ids,
+                                 render_colors, render_alphas, last_ids, stream);
 }
 
 extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
@@ -336,14 +341,14 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
                         workspace_bytes >= gsx_raster_records_bytes(N),
                     GSX_ERR_WORKSPACE, "rasterize fwd: workspace needs %zu bytes, 256-byte aligned",
                     gsx_raster_records_bytes(N));
-        const bool pinhole = !(radial_coeffs || tangential_coeffs || thin_prism_coeffs);
+        const bool pinhole = camera_model == GSX_PINHOLE && !(radial_coeffs || tangential_coeffs || thin_prism_coeffs);
         if ((rc = pack_raster_records(N, means, quats, scales, opacities, colors, channels, viewmats0, Ks, image_width,
                                       image_height, pinhole, workspace, stream)) != GSX_OK)
             return rc;
     }
     return rasterize_records_fwd(n_isects, workspace, colors, channels, backgrounds, masks, image_width, image_height,
-                                 viewmats0, Ks, radial_coeffs, tangential_coeffs, thin_prism_coeffs, tile_offsets,
-                                 flatten_ids, render_colors, render_alphas, last_ids, stream);
+                                 viewmats0, Ks, camera_model, radial_coeffs, tangential_coeffs, thin_prism_coeffs,
+                                 tile_offsets, flatten_ids, render_colors, render_alphas, last_ids, stream);
 }
 
 // Pair counts of one forward pass (no counterpart in the reference; used to turn kernel times into flop rates).
@@ -358,8 +363,9 @@ extern "C" int gsx_rasterize_pair_stats(int64_t n_isects, const void* records, u
     const uint32_t tw = cdiv(image_width, kTile), th = cdiv(image_height, kTile);
     hipLaunchKernelGGL((rasterize_fwd_kernel<3, true, false>), dim3(tw * th), dim3(256), 0, (hipStream_t)stream,
                        (uint32_t)n_isects, (const float4*)records, (const float*)nullptr, (const float*)nullptr,
-                       (const uint8_t*)nullptr, image_width, image_height, tw, th, viewmat, K, (const float*)nullptr,
-                       (const float*)nullptr, (const float*)nullptr, tile_offsets, flatten_ids, (float*)nullptr,
+                       (const uint8_t*)nullptr, image_width, image_height, tw, th, viewmat, K, (int)GSX_PINHOLE,
+                       (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, tile_offsets, flatten_ids,
+                       (float*)nullptr,
                        (float*)nullptr, (int32_t*)nullptr, stats_out);
     GSX_LAUNCH_CHECK();
     return GSX_OK;

@@ -226,6 +226,28 @@ def projection_ut_3dgs_fused(means, quats, scales, opacities, viewmats0, viewmat
     return radii, means2d, depths, conics, comp
 
 
+def _fit_backgrounds(backgrounds, channels):
+    """The fused operators hand the caller's background ([C,3] from gs::training::rasterize, rasterizer.cpp:84-87,
+    147) to a kernel that blends `channels` values per pixel (Rasterization.cpp:401-407): with RGB + depth it would
+    read one float past each row.  Here the missing channels' background is 0 and surplus ones are dropped (for one
+    camera the values the reference's kernel reads)."""
+    if backgrounds is None or backgrounds.numel() == 0:
+        return None
+    have = backgrounds.size(-1)
+    if have > channels:
+        return backgrounds[..., :channels].contiguous()
+    if have < channels:
+        pad = torch.zeros(backgrounds.shape[:-1] + (channels - have,), dtype=backgrounds.dtype,
+                          device=backgrounds.device)
+        return torch.cat([backgrounds, pad], -1).contiguous()
+    return backgrounds
+
+
+def _check_backgrounds(backgrounds, C, channels):
+    if backgrounds is not None and tuple(backgrounds.shape) != (C, channels):
+        raise RuntimeError(f"backgrounds must be [C, channels] = [{C}, {channels}], got {tuple(backgrounds.shape)}")
+
+
 def rasterize_to_pixels_from_world_3dgs_fwd(means, quats, scales, colors, opacities, backgrounds, masks, image_width,
                                             image_height, tile_size, viewmats0, viewmats1, Ks, camera_model,
                                             ut_params, rs_type, radial_coeffs, tangential_coeffs, thin_prism_coeffs,
@@ -244,6 +266,7 @@ def rasterize_to_pixels_from_world_3dgs_fwd(means, quats, scales, colors, opacit
     dev = means.device
     C, N = tile_offsets.size(0), means.size(0)
     channels = colors.size(-1)
+    _check_backgrounds(backgrounds, C, channels)
     renders = torch.empty((C, image_height, image_width, channels), dtype=torch.float32, device=dev)
     alphas = torch.empty((C, image_height, image_width, 1), dtype=torch.float32, device=dev)
     last_ids = torch.empty((C, image_height, image_width), dtype=torch.int32, device=dev)
@@ -278,6 +301,7 @@ def rasterize_to_pixels_from_world_3dgs_bwd(means, quats, scales, colors, opacit
         backgrounds = None
     dev = means.device
     C, N = tile_offsets.size(0), means.size(0)
+    _check_backgrounds(backgrounds, C, colors.size(-1))
     v_means, v_quats, v_scales = torch.empty_like(means), torch.empty_like(quats), torch.empty_like(scales)
     v_colors, v_opacities = torch.empty_like(colors), torch.empty_like(opacities)
     m8 = None if masks is None else masks.view(torch.uint8) if masks.dtype == torch.bool else masks
@@ -335,7 +359,7 @@ def rasterize_from_world_with_sh_fwd(means, quats, scales, opacities, sh_coeffs,
                                                tile_height, True)
     offsets = intersect_offset(isect_ids, C, tile_width, tile_height)
     renders, alphas, last_ids = rasterize_to_pixels_from_world_3dgs_fwd(
-        means, quats, scaled_scales, colors, final_opacities, backgrounds, masks, image_width, image_height,
+        means, quats, scaled_scales, colors, final_opacities, _fit_backgrounds(backgrounds, colors.size(-1)), masks, image_width, image_height,
         tile_size, viewmats0, viewmats1, Ks, camera_model, ut_params, rs_type, radial_coeffs, tangential_coeffs,
         thin_prism_coeffs, offsets, flatten_ids)
     out = (renders, alphas, radii, means2d, depths, colors, offsets, flatten_ids, last_ids, comp)
@@ -362,7 +386,7 @@ def rasterize_from_world_with_sh_bwd(means, quats, scales, opacities, sh_coeffs,
         final_opacities = (final_opacities * compensations).contiguous()
     scaled_scales = scales if scaling_modifier == 1.0 else scales * scaling_modifier
     v_means, v_quats, v_scales, v_colors, v_opacities = rasterize_to_pixels_from_world_3dgs_bwd(
-        means, quats, scaled_scales, colors, final_opacities, backgrounds, masks, image_width, image_height,
+        means, quats, scaled_scales, colors, final_opacities, _fit_backgrounds(backgrounds, colors.size(-1)), masks, image_width, image_height,
         tile_size, viewmats0, viewmats1, Ks, camera_model, ut_params, rs_type, radial_coeffs, tangential_coeffs,
         thin_prism_coeffs, tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors, v_render_alphas)
     K = sh_coeffs.size(1)

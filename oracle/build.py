@@ -23,7 +23,8 @@ FLAGS = ["-O2", "-march=x86-64-v3", "-ffp-contract=off", "-fno-fast-math", "-fop
 
 def build(force=True):
     if not force and os.path.exists(OUT) and os.path.getmtime(OUT) >= max(
-            *[os.path.getmtime(s) for s in SRCS], os.path.getmtime(os.path.join(MATH_INC, "gsx_math.h"))):
+            *[os.path.getmtime(s) for s in SRCS],
+            *[os.path.getmtime(os.path.join(MATH_INC, h)) for h in ("gsx_math.h", "gsx_camera.h", "gsx_record.h")]):
         return OUT
     cmd = ["g++", *FLAGS, "-I", MATH_INC, *SRCS, "-o", OUT]
     subprocess.run(cmd, check=True)

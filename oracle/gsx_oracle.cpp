@@ -27,6 +27,7 @@
 #include <vector>
 
 #include "gsx_math.h"
+#include "gsx_camera.h"
 
 #if defined(_OPENMP)
 #include <omp.h>
@@ -115,6 +116,10 @@ struct Distortion {
     float k[6] = {0, 0, 0, 0, 0, 0}, p[2] = {0, 0}, s[4] = {0, 0, 0, 0};
 };
 Distortion g_dist;
+// camera model (gsx_camera_model values): 0 pinhole (g_dist), 2 OpenCV fisheye (g_dist.k[0..3] = radial), 3
+// equirectangular - the two latter through the model code shared with the kernels (gsx_camera.h)
+int g_model = 0;
+bool g_fisheye_has_coeffs = false;
 
 // Cameras.cuh:504-533
 void compute_distortion(const Distortion& d, float u, float v, float* icD, float* delta_x, float* delta_y) {
@@ -153,9 +158,18 @@ bool opencv_project(const Distortion& d, vec3 cam, float fx, float fy, float cx,
 
 bool project_point(vec3 cam, float fx, float fy, float cx, float cy, uint32_t W, uint32_t H, float margin_factor,
                    vec2* out) {
+    if (g_model == 2) {
+        const gsx::Fisheye fe = gsx::fisheye_setup(g_fisheye_has_coeffs ? g_dist.k : nullptr, fx, fy, cx, cy, W, H);
+        return gsx::fisheye_project(fe, cam, margin_factor, out);
+    }
+    if (g_model == 3) {
+        gsx::equirect_project((float)W, (float)H, cam, out);
+        return true;
+    }
     return g_dist.on ? opencv_project(g_dist, cam, fx, fy, cx, cy, W, H, margin_factor, out)
                      : pinhole_project(cam, fx, fy, cx, cy, W, H, margin_factor, out);
 }
+uint32_t g_W = 0, g_H = 0; // image size for the models whose unprojection needs it (set by the rasterizers)
 
 // Cameras.cuh:635-740 : Newton undistortion (at most 5 steps, stop at |step| < 1e-6).  The reference's double
 // literals make parts of the Jacobian double arithmetic; the expressions are kept as written there.
@@ -210,16 +224,27 @@ bool opencv_undistort_newton(const Distortion& d, float xd, float yd, float* xo,
 // only when the undistortion did not converge; then the ray is zero, :330-333).
 bool pixel_world_ray(float px, float py, float fx, float fy, float cx, float cy,
                      const RollingShutter& rs, vec3* ray_o, vec3* ray_d) {
-    float u = (px - cx) / fx;
-    float v = (py - cy) / fy;
-    if (g_dist.on && !opencv_undistort_newton(g_dist, u, v, &u, &v)) {
+    vec3 d_cam;
+    bool ok = true;
+    if (g_model == 2) {
+        const gsx::Fisheye fe = gsx::fisheye_setup(g_fisheye_has_coeffs ? g_dist.k : nullptr, fx, fy, cx, cy, g_W, g_H);
+        ok = gsx::fisheye_unproject(fe, px, py, &d_cam);
+    } else if (g_model == 3) {
+        gsx::equirect_unproject((float)g_W, (float)g_H, px, py, &d_cam);
+    } else {
+        float u = (px - cx) / fx;
+        float v = (py - cy) / fy;
+        if (g_dist.on)
+            ok = opencv_undistort_newton(g_dist, u, v, &u, &v);
+        const vec3 cr = gsx::mk3(u, v, 1.f);
+        const float len = gsx::sqrt(gsx::dot(cr, cr));
+        d_cam = gsx::mk3(cr.x / len, cr.y / len, cr.z / len);
+    }
+    if (!ok) {
         *ray_o = gsx::mk3(0.f, 0.f, 0.f);
         *ray_d = gsx::mk3(0.f, 0.f, 0.f);
         return false;
     }
-    const vec3 cr = gsx::mk3(u, v, 1.f);
-    const float len = gsx::sqrt(gsx::dot(cr, cr));
-    const vec3 d_cam = gsx::mk3(cr.x / len, cr.y / len, cr.z / len);
     const ShutterPose pose = interpolate_shutter_pose(0.f, rs);
     const mat3 R_inv = gsx::mat3_cast(gsx::quat_inverse(pose.q));
     *ray_o = gsx::neg(gsx::mul(R_inv, pose.t));
@@ -1706,6 +1731,20 @@ ORC_API void orc_math_pow(int64_t n, const float* x, const float* e, float* y) {
         y[i] = gsx::pow(x[i], e[i]);
 }
 // which: 7 pow, 8 x / x2, 9 sqrt(x), 10 fma(x, x2, x)  (same numbering as the device probe)
+// probes of the camera-model primitives of gsx_camera.h: 0 atan2(x, x2), 1 cbrt(x), 2 asin(x), 3 cos(x),
+// 4 fisheye_max_angle_sq(x, x2, x3)
+ORC_API void orc_math_camera(int which, int64_t n, const float* x, const float* x2, const float* x3, float* y) {
+    for (int64_t i = 0; i < n; ++i) {
+        switch (which) {
+        case 0: y[i] = gsx::atan2(x[i], x2[i]); break;
+        case 1: y[i] = gsx::cbrt(x[i]); break;
+        case 2: y[i] = gsx::asin(x[i]); break;
+        case 3: y[i] = gsx::cos(x[i]); break;
+        default: y[i] = gsx::fisheye_max_angle_sq(x[i], x2[i], x3[i]); break;
+        }
+    }
+}
+
 ORC_API void orc_math_binary(int which, int64_t n, const float* x, const float* x2, float* y) {
     for (int64_t i = 0; i < n; ++i) {
         switch (which) {
@@ -1816,8 +1855,25 @@ ORC_API int orc_record_bounds_check(uint32_t N, const float* means, const float*
 // camera model state and probes
 // ---------------------------------------------------------------------------------------------
 // radial [6], tangential [2], thin_prism [4], each nullable; all null = perfect pinhole.
+ORC_API void orc_set_camera_model(int model, const float* radial, const float* tangential, const float* thin_prism,
+                                  uint32_t W, uint32_t H);
 ORC_API void orc_set_distortion(const float* radial, const float* tangential, const float* thin_prism) {
+    orc_set_camera_model(0, radial, tangential, thin_prism, 0, 0);
+}
+
+// model: 0 pinhole (coefficients: radial [6], tangential [2], thin_prism [4]), 2 fisheye (radial [4]), 3
+// equirectangular.  W, H: the image size (the fisheye and equirectangular unprojections need it).
+ORC_API void orc_set_camera_model(int model, const float* radial, const float* tangential, const float* thin_prism,
+                                  uint32_t W, uint32_t H) {
+    g_model = model;
+    g_W = W, g_H = H;
     g_dist = Distortion();
+    g_fisheye_has_coeffs = model == 2 && radial != nullptr;
+    if (model != 0) {
+        for (int i = 0; i < 4 && radial && model == 2; ++i)
+            g_dist.k[i] = radial[i];
+        return;
+    }
     g_dist.on = radial != nullptr || tangential != nullptr || thin_prism != nullptr;
     for (int i = 0; i < 6 && radial; ++i)
         g_dist.k[i] = radial[i];

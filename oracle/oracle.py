@@ -71,6 +71,34 @@ class distortion:
         return False
 
 
+class camera_model:
+    """Context manager: the OpenCV fisheye (model 2, radial [4] optional) or the equirectangular model (3) for every
+    projection / pixel ray inside the block; W, H = the image size."""
+
+    def __init__(self, model, W, H, radial=None):
+        self.model, self.W, self.H = int(model), int(W), int(H)
+        self.radial = None if radial is None else np.ascontiguousarray(np.asarray(radial, np.float32).reshape(-1)[:4])
+
+    def __enter__(self):
+        lib().orc_set_camera_model(c_i(self.model), _p(self.radial), None, None, c_u32(self.W), c_u32(self.H))
+        return self
+
+    def __exit__(self, *exc):
+        lib().orc_set_camera_model(c_i(0), None, None, None, c_u32(0), c_u32(0))
+        return False
+
+
+def math_camera(which, x, x2=None, x3=None):
+    """probes of gsx_camera.h's primitives: "atan2" (x, x2), "cbrt", "asin", "cos", "max_angle_sq" (x, x2, x3)"""
+    idx = {"atan2": 0, "cbrt": 1, "asin": 2, "cos": 3, "max_angle_sq": 4}[which]
+    x = _f32(x).reshape(-1)
+    x2 = x if x2 is None else _f32(x2).reshape(-1)
+    x3 = x if x3 is None else _f32(x3).reshape(-1)
+    y = np.zeros_like(x)
+    lib().orc_math_camera(c_i(idx), c_i64(x.size), _p(x), _p(x2), _p(x3), _p(y))
+    return y
+
+
 def camera_project(points, fx, fy, cx, cy, W, H, margin=0.1):
     """camera-space points [n,3] -> (image points [n,2], valid [n]) under the current camera model"""
     pts = _f32(points)
@@ -370,6 +398,19 @@ def sh_colors_from_world_bwd(sh_degree, means, K, radii, viewmat, colors, v_colo
     return out
 
 
+def _fit_backgrounds(backgrounds, channels):
+    """[C,3] background under a render with another channel count: zeros for missing channels, surplus ones dropped
+    (Rasterization.cpp:401-407 passes it on as it is, and its kernel then reads past each row's end)"""
+    if backgrounds is None:
+        return None
+    b = _f32(backgrounds)
+    if b.shape[-1] > channels:
+        return np.ascontiguousarray(b[..., :channels])
+    if b.shape[-1] < channels:
+        return np.ascontiguousarray(np.concatenate([b, np.zeros(b.shape[:-1] + (channels - b.shape[-1],), np.float32)], -1))
+    return b
+
+
 def rasterize_from_world_with_sh_fwd(means, quats, scales, opacities, sh_coeffs, sh_degree, backgrounds, image_width,
                                      image_height, tile_size, viewmats0, Ks, eps2d=0.3, near_plane=0.01, far_plane=1e4,
                                      radius_clip=0.0, scaling_modifier=1.0, calc_compensations=False, ut=None,
@@ -395,8 +436,8 @@ def rasterize_from_world_with_sh_fwd(means, quats, scales, opacities, sh_coeffs,
     _, isect_ids, flatten_ids = intersect_tile(means2d, radii, depths, 1, tile_size, tw, th, True)
     offsets = intersect_offset(isect_ids, 1, tw, th)
     renders, alphas, last_ids = rasterize_to_pixels_from_world_3dgs_fwd(
-        means, quats, scaled, colors, final_op, backgrounds, None, image_width, image_height, tile_size, viewmats0,
-        Ks, offsets, flatten_ids)
+        means, quats, scaled, colors, final_op, _fit_backgrounds(backgrounds, colors.shape[-1]), None, image_width,
+        image_height, tile_size, viewmats0, Ks, offsets, flatten_ids)
     return renders, alphas, radii, means2d, depths, colors, offsets, flatten_ids, last_ids, comp, isect_ids
 
 
@@ -410,7 +451,8 @@ def rasterize_from_world_with_sh_bwd(means, quats, scales, opacities, sh_coeffs,
     if calc_compensations:
         final_op = final_op * compensations
     v_means, v_quats, v_scales, v_colors, v_opac = rasterize_to_pixels_from_world_3dgs_bwd(
-        means, quats, scaled, colors, final_op, backgrounds, None, image_width, image_height, tile_size, viewmats0, Ks,
+        means, quats, scaled, colors, final_op, _fit_backgrounds(backgrounds, np.shape(colors)[-1]), None, image_width,
+        image_height, tile_size, viewmats0, Ks,
         tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors, v_render_alphas)
     K = sh_coeffs.shape[1]
     if render_mode in (0, 3, 4):  # Rasterization.cpp:581-624: the depth channel's gradient is dropped

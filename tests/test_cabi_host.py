@@ -68,7 +68,7 @@ def test_status_codes_without_launch(gsx):
         u32(C), u32(10), one, one, one, one, one, vm1, one, u32(64), u32(64), cf(.3), cf(.01), cf(1e4), cf(0),
         ci(model), ut, ci(rs), nul, nul, nul, one, one, one, one, nul, nul)
     assert proj(2, L.PINHOLE, L.GLOBAL, nul) == L.GSX_ERR_UNSUPPORTED        # C > 1
-    assert proj(1, L.FISHEYE, L.GLOBAL, nul) == L.GSX_ERR_UNSUPPORTED        # camera model
+    assert proj(1, L.ORTHO, L.GLOBAL, nul) == L.GSX_ERR_UNSUPPORTED          # camera model
     assert proj(1, L.PINHOLE, L.ROLLING_TOP_TO_BOTTOM, nul) == L.GSX_ERR_UNSUPPORTED
     assert proj(1, L.PINHOLE, L.GLOBAL, one) == L.GSX_ERR_UNSUPPORTED        # viewmats1 given
     n_host = i64(-1)

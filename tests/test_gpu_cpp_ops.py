@@ -168,7 +168,7 @@ def test_cpp_errors_on_device(gsx, cpp, cuda):
                                      cpp.ShutterType.GLOBAL, None, None, None)
     with pytest.raises(RuntimeError, match="gsx"):
         cpp.projection_ut_3dgs_fused(d["means"], d["quats"], d["scales"], d["op"], d["vm"], None, d["K"], cam.width,
-                                     cam.height, 0.3, 0.01, 1e4, 0.0, False, cpp.CameraModelType.FISHEYE, ut,
+                                     cam.height, 0.3, 0.01, 1e4, 0.0, False, cpp.CameraModelType.ORTHO, ut,
                                      cpp.ShutterType.GLOBAL, None, None, None)
     with pytest.raises(RuntimeError, match="contiguous"):
         cpp.quats_to_rotmats(d["quats"].t().contiguous().t())

@@ -109,8 +109,8 @@ def test_projection_unsupported_and_errors(gsx, cuda):
     means, quats, scales, op, shs = gsx.scenes.activate(sc)
     args = [T(means, cuda), T(quats, cuda), T(scales, cuda), T(op, cuda), T(cam.viewmat[None], cuda), None,
             T(cam.K[None], cuda), cam.width, cam.height, 0.3, 0.01, 1e4, 0.0, False]
-    with pytest.raises(gsx._lib.GsxError):  # fisheye model is not built
-        ops.projection_ut_3dgs_fused(*args, 2, ops.UnscentedTransformParameters(), 4)
+    with pytest.raises(gsx._lib.GsxError):  # the orthographic model is not built
+        ops.projection_ut_3dgs_fused(*args, 1, ops.UnscentedTransformParameters(), 4)
     with pytest.raises(gsx._lib.GsxError):  # rolling shutter is not built
         ops.projection_ut_3dgs_fused(*args, 0, ops.UnscentedTransformParameters(), 0)
     with pytest.raises(RuntimeError):  # CHECK_INPUT: CPU tensor
@@ -367,6 +367,12 @@ def test_raster_masks_and_channels(gsx, orc, cuda):
                                                     torch.zeros((1, 4000, 5), device=cuda), T(h["op"][None], cuda),
                                                     None, None, cam.width, cam.height, 16, d["vm"], None, d["K"], 0,
                                                     ut, 4, None, None, None, T(off, cuda), T(flat, cuda))
+    with pytest.raises(RuntimeError, match=r"backgrounds must be \[C, channels\]"):  # a [1,3] row under 4 channels
+        ops.rasterize_to_pixels_from_world_3dgs_fwd(d["means"], d["quats"], d["scales"],
+                                                    torch.zeros((1, 4000, 4), device=cuda), T(h["op"][None], cuda),
+                                                    torch.zeros((1, 3), device=cuda), None, cam.width, cam.height, 16,
+                                                    d["vm"], None, d["K"], 0, ut, 4, None, None, None, T(off, cuda),
+                                                    T(flat, cuda))
 
 
 # ---------------------------------------------------------------------------------------------
@@ -641,10 +647,64 @@ def test_opencv_distortion_projection_and_errors(gsx, orc, cuda):
     assert torch.equal(a[0], b[0])
     vis = (b[0][0, :, 0] > 0)
     assert torch.equal(a[1][0][vis], b[1][0][vis]) and torch.equal(a[3][0][vis], b[3][0][vis])
-    with pytest.raises(RuntimeError, match="only PINHOLE"):
-        call(None, None, None, model=2)  # FISHEYE
+    with pytest.raises(RuntimeError, match="PINHOLE, FISHEYE and EQUIRECTANGULAR are supported"):
+        call(None, None, None, model=1)  # ORTHO
     with pytest.raises(RuntimeError, match="rolling shutter"):
         call(None, None, None, rs=0)  # ROLLING_TOP_TO_BOTTOM
+
+
+@pytest.mark.parametrize("which", ["fisheye", "fisheye+coeffs", "equirectangular"])
+def test_fisheye_and_equirectangular_fused_forward_backward(gsx, orc, cuda, which):
+    """OpenCV fisheye (with and without its four radial coefficients) and the equirectangular panorama: UT projection
+    through the model and per-pixel unprojection, fused forward bit-identical to the checker, backward at the gradient
+    bar (Cameras.cuh:757-1037)"""
+    ops = gsx.ops
+    sc, cam, h, d = _fused_inputs(gsx, cuda, 20000)
+    model = 3 if which == "equirectangular" else 2
+    radial = [0.04, -0.006, 0.0008, -0.00005] if which == "fisheye+coeffs" else None
+    co = (None if radial is None else T(np.asarray(radial, np.float32)[None], cuda), None, None)
+    ut = ops.UnscentedTransformParameters()
+    with orc.camera_model(model, cam.width, cam.height, radial=radial):
+        ref = orc.rasterize_from_world_with_sh_fwd(h["means"], h["quats"], h["scales"], h["op"], h["shs"], 3, h["bg"],
+                                                   cam.width, cam.height, 16, h["vm"], h["K"])
+    plain = orc.rasterize_from_world_with_sh_fwd(h["means"], h["quats"], h["scales"], h["op"], h["shs"], 3, h["bg"],
+                                                 cam.width, cam.height, 16, h["vm"], h["K"])
+    assert np.abs(ref[0] - plain[0]).max() > 0.05  # another image than the pinhole's
+    got = ops.rasterize_from_world_with_sh_fwd(d["means"], d["quats"], d["scales"], d["op"], d["shs"], 3, d["bg"], None,
+                                               cam.width, cam.height, 16, d["vm"], None, d["K"], model, 0.3, 0.01, 1e4,
+                                               0.0, 1.0, False, 0, ut, 4, *co, return_isect_ids=True)
+    renders, alphas, radii, means2d, depths, colors, offsets, flat, last_ids, comp, ids = got
+    bits_equal(N(radii), ref[2], "radii")
+    vis = ref[2][0, :, 0] > 0
+    assert vis.sum() > 2000
+    bits_equal(N(means2d)[0][vis], ref[3][0][vis], "means2d")
+    bits_equal(N(ids), ref[10], "sorted tile keys")
+    bits_equal(N(flat), ref[7], "sort order")
+    bits_equal(N(offsets), ref[6], "per-tile ranges")
+    bits_equal(N(last_ids), ref[8], "last ids")
+    bits_equal(N(renders), ref[0], "image")
+    bits_equal(N(alphas), ref[1], "alpha")
+    assert ref[1].mean() > 0.01
+
+    rng = np.random.default_rng(3)
+    v_r = rng.normal(0, 1, tuple(renders.shape)).astype(np.float32)
+    v_a = rng.normal(0, 1, tuple(alphas.shape)).astype(np.float32)
+    op1 = d["op"][None].contiguous()
+    got5 = ops.rasterize_to_pixels_from_world_3dgs_bwd(d["means"], d["quats"], d["scales"], colors, op1, d["bg"], None,
+                                                       cam.width, cam.height, 16, d["vm"], None, d["K"], model, ut, 4,
+                                                       *co, offsets, flat, alphas, last_ids, T(v_r, cuda), T(v_a, cuda))
+    args = (h["means"], h["quats"], h["scales"], N(colors), h["op"][None], h["bg"])
+    with orc.camera_model(model, cam.width, cam.height, radial=radial):
+        o32 = orc.rasterize_to_pixels_from_world_3dgs_bwd(*args, None, cam.width, cam.height, 16, h["vm"], h["K"],
+                                                          N(offsets), N(flat), N(alphas), N(last_ids), v_r, v_a)
+        g64, _ = orc.rasterize_bwd_f64(*args, cam.width, cam.height, 16, h["vm"], h["K"], N(offsets), N(flat),
+                                       N(alphas), N(last_ids), v_r, v_a)
+    check_raster_gradients([N(x) for x in got5], o32, g64, tag=which + " ")
+
+    pr = ops.projection_ut_3dgs_fused(d["means"], d["quats"], d["scales"], d["op"], d["vm"], None, d["K"], cam.width,
+                                      cam.height, 0.3, 0.01, 1e4, 0.0, False, model, ut, 4, *co)
+    bits_equal(N(pr[0]), ref[2], "standalone projection radii")
+    bits_equal(N(pr[1])[0][vis], ref[3][0][vis], "standalone projection means2d")
 
 
 def test_philox_noise_on_device(gsx, orc, cuda):

@@ -83,3 +83,11 @@ def test_rasterize_checks_and_options(gsx, cuda):
     assert float((zero.image - base.image).abs().max()) <= 1e-6
     bent = rasterize(*args, d["bg"], radial_distortion=torch.tensor([-0.2, 0.05], device=cuda))
     assert float((bent.image - base.image).abs().max()) > 0.005
+    # gs::Camera::camera_model_type() reaches the kernels (rasterizer.cpp:135): the fisheye image is another one, and
+    # the mirror's output is the operator's
+    fish = rasterize(*args, d["bg"], camera_model=2, radial_distortion=torch.tensor([0.02, -0.003], device=cuda))
+    assert float((fish.image - base.image).abs().max()) > 0.005 and float(fish.alpha.mean()) > 0.01
+    pano = rasterize(*args, d["bg"], camera_model=3)
+    assert float((pano.image - base.image).abs().max()) > 0.005 and float(pano.alpha.sum()) > 0
+    with pytest.raises(RuntimeError, match="PINHOLE, FISHEYE and EQUIRECTANGULAR"):
+        rasterize(*args, d["bg"], camera_model=1)

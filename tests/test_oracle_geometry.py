@@ -417,3 +417,92 @@ def test_undistortion_inverts_the_projection(orc):
         sol = fsolve(lambda uv: forward(uv) - target, target, xtol=1e-12)
         ray = np.array([sol[0], sol[1], 1.0]) / np.linalg.norm([sol[0], sol[1], 1.0])
         assert np.abs(rays[i] - ray).max() < 3e-6
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# OpenCV fisheye and equirectangular models (Cameras.cuh:757-1037; gsx_camera.h)
+# ---------------------------------------------------------------------------------------------------------------
+def test_camera_primitives(orc):
+    """atan2 on the whole plane, cbrt, asin, cos against numpy in float64 (<= 2e-7 absolute / 3e-7 relative)"""
+    r = np.random.default_rng(0)
+    y, x = r.normal(0, 1, 20000).astype(np.float32), r.normal(0, 1, 20000).astype(np.float32)
+    y[:100], x[100:200] = 0.0, 0.0
+    y[200:300] *= 1e-6
+    x[300:400] *= 1e6
+    assert np.abs(orc.math_camera("atan2", y, x) - np.arctan2(y.astype(np.float64), x)).max() < 3e-7
+    assert orc.math_camera("atan2", [0.0], [0.0])[0] == 0.0
+    v = np.concatenate([r.normal(0, 100, 5000), r.normal(0, 1e-3, 5000), [0.0, 8.0, -27.0]]).astype(np.float32)
+    got = orc.math_camera("cbrt", v)
+    assert np.abs(got - np.cbrt(v.astype(np.float64))).max() <= 3e-7 * np.abs(np.cbrt(v)).max()
+    assert np.all(np.abs(got - np.cbrt(v.astype(np.float64))) <= 3e-7 * np.abs(np.cbrt(v.astype(np.float64))) + 1e-30)
+    s = r.uniform(-1, 1, 20000).astype(np.float32)
+    assert np.abs(orc.math_camera("asin", s) - np.arcsin(s.astype(np.float64))).max() < 4e-7
+    a = r.uniform(-np.pi, np.pi, 20000).astype(np.float32)
+    assert np.abs(orc.math_camera("cos", a) - np.cos(a.astype(np.float64))).max() < 2.5e-7
+
+
+def test_fisheye_field_of_view_limit(orc):
+    """the limit is the smallest positive root of the derivative 1 + 3 k1 t^2 + 5 k2 t^4 + 7 k3 t^6 (+ 9 k4 t^8) of
+    the forward polynomial (beyond it the mapping folds back): numpy's roots of the same polynomial"""
+    cases = [(-0.05, 0.0, 0.0), (0.1, -0.02, 0.0), (-0.02, 0.003, -0.0004), (0.05, 0.01, 0.001), (0.2, -0.05, 0.004),
+             (-0.3, 0.05, -0.01), (0.0, -0.01, 0.0), (0.0, 0.0, -1e-3)]
+    for k1, k2, k3 in cases:
+        a, b, c = 3 * k1, 5 * k2, 7 * k3
+        got = float(orc.math_camera("max_angle_sq", [a], [b], [c])[0])
+        roots = np.roots([c, b, a, 1.0])  # in x = t^2
+        pos = sorted(float(z.real) for z in roots if abs(z.imag) < 1e-9 and z.real > 0)
+        if pos:
+            assert abs(got - pos[0]) <= 2e-5 * pos[0], (k1, k2, k3, got, pos)
+        else:
+            assert got > 1e38, (k1, k2, k3, got)
+
+
+def _fisheye_rays(n, seed, max_theta):
+    r = np.random.default_rng(seed)
+    theta = r.uniform(0.0, max_theta, n)
+    phi = r.uniform(-np.pi, np.pi, n)
+    d = r.uniform(0.5, 5.0, n)
+    return (d[:, None] * np.stack([np.sin(theta) * np.cos(phi), np.sin(theta) * np.sin(phi), np.cos(theta)], 1)), theta
+
+
+@pytest.mark.parametrize("k", [None, [0.03, -0.004, 0.0006, 0.0], [-0.02, 0.003, -0.0004, 0.00003]])
+def test_fisheye_projection_closed_form_and_round_trip(orc, k):
+    """image radius = f (theta + k1 theta^3 + k2 theta^5 + k3 theta^7 + k4 theta^9) along the ray's azimuth (the
+    equidistant model when k = 0), in float64; the Newton inverse returns the unit ray; rays beyond the field of
+    view / behind the camera are invalid or clamped onto the rim"""
+    W, H, f = 640, 480, 200.0
+    pts, theta = _fisheye_rays(4000, 3, 1.3)
+    with orc.camera_model(2, W, H, radial=k):
+        ip, ok = orc.camera_project(pts.astype(np.float32), f, f, W / 2, H / 2, W, H, margin=0.1)
+        rays, conv = orc.camera_unproject(ip, f, f, W / 2, H / 2)
+        behind, okb = orc.camera_project(np.array([[0.1, 0.2, -1.0]], np.float32), f, f, W / 2, H / 2, W, H)
+    kk = np.zeros(4) if k is None else np.array(k, np.float64)
+    rad = theta + kk[0] * theta ** 3 + kk[1] * theta ** 5 + kk[2] * theta ** 7 + kk[3] * theta ** 9
+    az = np.arctan2(pts[:, 1], pts[:, 0])
+    want = np.stack([f * rad * np.cos(az) + W / 2, f * rad * np.sin(az) + H / 2], 1)
+    assert np.abs(ip - want).max() < 2e-3  # pixels; float32 at a few hundred pixels
+    inside = (want[:, 0] >= -0.1 * W) & (want[:, 0] < 1.1 * W) & (want[:, 1] >= -0.1 * H) & (want[:, 1] < 1.1 * H)
+    edge = np.minimum(np.abs(want[:, 0] + 0.1 * W), np.abs(want[:, 0] - 1.1 * W)) < 1e-2
+    assert np.array_equal(ok[~edge], inside[~edge]) and ok.sum() > 1000
+    assert not okb[0]
+    unit = pts / np.linalg.norm(pts, axis=1, keepdims=True)
+    assert conv[ok].all() and np.abs(rays[ok] - unit[ok]).max() < 5e-6
+
+
+def test_equirectangular_closed_form_and_round_trip(orc):
+    """pixel = ((azimuth / 2 pi + 1/2) W, (elevation / pi + 1/2) H) with azimuth = atan2(x, z), elevation =
+    asin(y / |p|): every direction is valid, including behind the camera; the unprojection returns the unit ray"""
+    W, H = 1024, 512
+    r = np.random.default_rng(5)
+    pts = r.normal(0, 1, (5000, 3))
+    pts *= r.uniform(0.5, 4.0, (5000, 1)) / np.linalg.norm(pts, axis=1, keepdims=True)
+    with orc.camera_model(3, W, H):
+        ip, ok = orc.camera_project(pts.astype(np.float32), 1.0, 1.0, 0.0, 0.0, W, H)
+        rays, conv = orc.camera_unproject(ip, 1.0, 1.0, 0.0, 0.0)
+    az, el = np.arctan2(pts[:, 0], pts[:, 2]), np.arcsin(pts[:, 1] / np.linalg.norm(pts, axis=1))
+    want = np.stack([(az / (2 * np.pi) + 0.5) * W, (el / np.pi + 0.5) * H], 1)
+    assert ok.all() and conv.all() and np.abs(ip[:, 0] - want[:, 0]).max() < 1.5e-4
+    # asin is ill-conditioned at the poles: one float32 rounding of y / |p| moves the elevation by 6e-8 / cos(el)
+    assert np.all(np.abs(ip[:, 1] - want[:, 1]) < 1.5e-4 + H / np.pi * 1.2e-7 / np.cos(el))
+    unit = pts / np.linalg.norm(pts, axis=1, keepdims=True)
+    assert np.abs(rays - unit).max() < 3e-6
