@@ -11,7 +11,8 @@
  *    (workspace, workspace_bytes) pair is handed to the op.  Workspaces need 256-byte alignment.
  *  - Return value: GSX_OK or a negative gsx_status.  gsx_last_error() gives a thread-local message.
  *  - Optional pointers may be NULL where the comment says "nullable".
- *  - C = 1 camera and a global shutter; camera models GSX_PINHOLE (radial [6], tangential [2], thin prism [4]
+ *  - C = 1 camera; global or rolling shutter (gsx_shutter_type; viewmats1 = the end-of-frame pose, nullable = the
+ *    start pose); camera models GSX_PINHOLE (radial [6], tangential [2], thin prism [4]
  *    coefficients, each nullable; LichtFeld's trainer uses the perfect pinhole: rasterizer.cpp:33-35,
  *    rasterizer_autograd.cpp:59-60), GSX_FISHEYE (radial [4], nullable) and GSX_EQUIRECTANGULAR.  Other values
  *    return GSX_ERR_UNSUPPORTED.  backgrounds, where given, is [C, channels] of the colours being blended.
@@ -37,7 +38,7 @@ extern "C" {
 typedef enum gsx_status {
     GSX_OK = 0,
     GSX_ERR_INVALID_ARGUMENT = -1, /* null pointer, bad size, bad enum */
-    GSX_ERR_UNSUPPORTED = -2,      /* C > 1, orthographic camera, rolling shutter, CDIM not built */
+    GSX_ERR_UNSUPPORTED = -2,      /* C > 1, orthographic camera, CDIM not built */
     GSX_ERR_WORKSPACE = -3,        /* workspace too small or misaligned */
     GSX_ERR_HIP = -4,              /* a HIP runtime call failed (message has the HIP error) */
     GSX_ERR_OVERFLOW = -5          /* n_isects does not fit the int32 index space */

@@ -17,15 +17,17 @@ void set_error(const char* fmt, ...) {
 // One camera per call (the reference's rasterizer indexes per-Gaussian arrays with the flattened [C*N] id,
 // RasterizeToPixelsFromWorld3DGSFwd.cu:203-210, so C > 1 is not usable there either); the pinhole model with or
 // without OpenCV distortion coefficients (radial [6], tangential [2], thin prism [4]), the OpenCV fisheye model
-// (radial [4]) and the equirectangular model; global shutter.
+// (radial [4]) and the equirectangular model; global or rolling shutter (viewmats1 = the end-of-frame pose, null =
+// the start pose).
 int check_camera_args(uint32_t C, const float* viewmats1, int camera_model, int rs_type, const float* radial,
                       const float* tangential, const float* thin_prism) {
     GSX_REQUIRE(C == 1, GSX_ERR_UNSUPPORTED, "C = %u cameras: only C == 1 is supported", C);
     GSX_REQUIRE(camera_model == GSX_PINHOLE || camera_model == GSX_FISHEYE || camera_model == GSX_EQUIRECTANGULAR,
                 GSX_ERR_UNSUPPORTED, "camera model %d: PINHOLE, FISHEYE and EQUIRECTANGULAR are supported", camera_model);
     (void)radial, (void)tangential, (void)thin_prism;
-    GSX_REQUIRE(rs_type == GSX_GLOBAL && viewmats1 == nullptr, GSX_ERR_UNSUPPORTED,
-                "rolling shutter (rs_type %d / viewmats1): only a global shutter is supported", rs_type);
+    (void)viewmats1;
+    GSX_REQUIRE(rs_type >= GSX_ROLLING_TOP_TO_BOTTOM && rs_type <= GSX_GLOBAL, GSX_ERR_INVALID_ARGUMENT,
+                "shutter type %d: must be 0 .. 4 (gsx_shutter_type)", rs_type);
     return GSX_OK;
 }
 

@@ -55,9 +55,15 @@ int check_camera_args(uint32_t C, const float* viewmats1, int camera_model, int 
 struct CamPose {
     quat q_start;
     vec3 t_start;
+    quat q_end; // = the start pose for a global shutter or when no end-of-frame pose is given
+    vec3 t_end;
+    int rs_type;   // gsx_shutter_type
+    uint32_t W, H; // image size: the exposure time of a pixel is its row / column over H - 1 / W - 1
 };
 
-__device__ __forceinline__ CamPose load_cam_pose(const float* __restrict__ vm) {
+// RollingShutterParameters (Cameras.cuh:33-71): row-major [4,4] world->camera matrices; vm1 nullable
+__device__ __forceinline__ CamPose load_cam_pose(const float* __restrict__ vm, const float* __restrict__ vm1 = nullptr,
+                                                 int rs_type = 4 /*GLOBAL*/, uint32_t W = 0, uint32_t H = 0) {
     mat3 R;
 #pragma unroll
     for (int r = 0; r < 3; ++r)
@@ -67,15 +73,39 @@ __device__ __forceinline__ CamPose load_cam_pose(const float* __restrict__ vm) {
     CamPose p;
     p.q_start = quat_cast(R);
     p.t_start = mk3(vm[3], vm[7], vm[11]);
+    p.q_end = p.q_start;
+    p.t_end = p.t_start;
+    if (vm1 != nullptr) {
+#pragma unroll
+        for (int r = 0; r < 3; ++r)
+#pragma unroll
+            for (int c = 0; c < 3; ++c)
+                R.m[r][c] = vm1[r * 4 + c];
+        p.q_end = quat_cast(R);
+        p.t_end = mk3(vm1[3], vm1[7], vm1[11]);
+    }
+    p.rs_type = rs_type;
+    p.W = W, p.H = H;
     return p;
 }
 
-// interpolate_shutter_pose(rel, {start, end = start})
+// interpolate_shutter_pose (Cameras.cuh:268-280)
 __device__ __forceinline__ void shutter_pose(const CamPose& cp, float rel, quat* q, vec3* t) {
-    t->x = (1.f - rel) * cp.t_start.x + rel * cp.t_start.x;
-    t->y = (1.f - rel) * cp.t_start.y + rel * cp.t_start.y;
-    t->z = (1.f - rel) * cp.t_start.z + rel * cp.t_start.z;
-    *q = slerp(cp.q_start, cp.q_start, rel);
+    t->x = (1.f - rel) * cp.t_start.x + rel * cp.t_end.x;
+    t->y = (1.f - rel) * cp.t_start.y + rel * cp.t_end.y;
+    t->z = (1.f - rel) * cp.t_start.z + rel * cp.t_end.z;
+    *q = slerp(cp.q_start, cp.q_end, rel);
+}
+
+// shutter_relative_frame_time (Cameras.cuh:293-320): 0 for a global shutter
+__device__ __forceinline__ float shutter_relative_frame_time(const CamPose& cp, float x, float y) {
+    switch (cp.rs_type) {
+    case 0: return gsx::floor(y) / (float)(cp.H - 1);
+    case 1: return gsx::floor(x) / (float)(cp.W - 1);
+    case 2: return ((float)cp.H - gsx::ceil(y)) / (float)(cp.H - 1);
+    case 3: return ((float)cp.W - gsx::ceil(x)) / (float)(cp.W - 1);
+    default: return 0.f;
+    }
 }
 
 // ---- OpenCV pinhole distortion (gsplat/Cameras.cuh:473-815) ------------------------------------
@@ -190,7 +220,7 @@ __device__ __forceinline__ CameraModel load_camera_model(int type, const float* 
     return m;
 }
 
-// world ray through a pixel centre, global shutter (Cameras.cuh:457-470 / 742-755 / 961-1000 / 1027-1036
+// world ray through a pixel centre under the pose of the pixel's exposure time (Cameras.cuh:457-470 / 742-755 / 961-1000 / 1027-1036
 // unproject, :253-266 camera_ray_to_world_ray, :322-339).  Returns the ray's valid flag: false when an undistortion
 // or the fisheye inverse did not converge or left the field of view (the ray is then zero, :330-333, and the pixel
 // takes no part in either pass).
@@ -218,7 +248,7 @@ __device__ __forceinline__ bool pixel_world_ray(const CamPose& cp, float px, flo
     }
     quat q;
     vec3 t;
-    shutter_pose(cp, 0.f, &q, &t);
+    shutter_pose(cp, shutter_relative_frame_time(cp, px, py), &q, &t);
     const mat3 R_inv = mat3_cast(quat_inverse(q));
     *ray_o = neg(mul(R_inv, t));
     *ray_d = mul(R_inv, d_cam);

@@ -68,6 +68,66 @@ __device__ __forceinline__ bool opencv_project(vec3 cam, const ProjCfg& cfg, vec
     return valid;
 }
 
+// camera_ray_to_image_point of the configured model
+template <bool GENERAL>
+__device__ __forceinline__ bool project_cam_point(const ProjCfg& cfg, vec3 pc, vec2* uv) {
+    if (GENERAL) {
+        if (cfg.cam.type == 2)
+            return fisheye_project(cfg.cam.fe, pc, cfg.ut_margin, uv);
+        if (cfg.cam.type == 3) {
+            equirect_project((float)cfg.W, (float)cfg.H, pc, uv);
+            return true; // Cameras.cuh:1013-1025 returns valid for every point
+        }
+        if (cfg.cam.dist.on)
+            return opencv_project(pc, cfg, uv);
+    }
+    return pinhole_project(pc, cfg, uv);
+}
+
+// world_point_to_image_point_shutter_pose (Cameras.cuh:346-414).  Global shutter: the start pose's projection.
+// Rolling shutter: from the start-pose projection (the end-pose one if only that is valid; neither valid = invalid)
+// ten rounds of "exposure time of the current image point -> pose -> projection"; the last point is returned as
+// valid.  One loop, one projection call site: round 0 = start pose, 1 = end pose, 2 .. 11 = the iteration.
+template <bool GENERAL>
+__device__ __forceinline__ bool project_world_point(const ProjCfg& cfg, const CamPose& cp, vec3 p, vec2* uv) {
+    if (!GENERAL || cp.rs_type == GSX_GLOBAL)
+        return project_cam_point<GENERAL>(cfg, add(quat_rotate(cp.q_start, p), cp.t_start), uv);
+    vec2 prev = {0.f, 0.f}, p_start = {0.f, 0.f};
+    bool valid_start = false;
+#pragma unroll 1
+    for (int round = 0; round < 12; ++round) {
+        quat q = cp.q_start;
+        vec3 t = cp.t_start;
+        if (round == 1) {
+            q = cp.q_end;
+            t = cp.t_end;
+        } else if (round > 1) {
+            shutter_pose(cp, shutter_relative_frame_time(cp, prev.x, prev.y), &q, &t);
+        }
+        vec2 pt;
+        const bool pv = project_cam_point<GENERAL>(cfg, add(quat_rotate(q, p), t), &pt);
+        if (round == 0) {
+            p_start = pt;
+            valid_start = pv;
+        } else if (round == 1) {
+            if (valid_start) {
+                prev = p_start;
+            } else if (pv) {
+                prev = pt;
+            } else {
+                *uv = pt;
+                return false;
+            }
+        } else {
+            prev = pt;
+        }
+    }
+    *uv = prev;
+    return true;
+}
+
+// GENERAL = false: the perfect pinhole with a global shutter (the training step's camera), decided at compile time
+template <bool GENERAL>
 __device__ __forceinline__ bool project_ut(const ProjCfg& cfg, const CamPose& cp, vec3 mean, quat q_in, vec3 scl,
                                            bool has_opacity, float opacity_in, ProjOut* o) {
     const quat q = quat_normalize(q_in);
@@ -75,7 +135,8 @@ __device__ __forceinline__ bool project_ut(const ProjCfg& cfg, const CamPose& cp
     vec3 tc;
     shutter_pose(cp, 0.5f, &qc, &tc);
     const vec3 mean_c = add(quat_rotate(qc, mean), tc);
-    if (mean_c.z < cfg.near_plane || mean_c.z > cfg.far_plane)
+    // the equirectangular model sees behind the camera (ProjectionUT3DGSFused.cu:78)
+    if ((mean_c.z < cfg.near_plane && !(GENERAL && cfg.cam.type == 3)) || mean_c.z > cfg.far_plane)
         return false;
 
     const float D = 3.0f;
@@ -101,17 +162,8 @@ __device__ __forceinline__ bool project_ut(const ProjCfg& cfg, const CamPose& cp
             const vec3 delta = mk3(s * Rg.m[0][a], s * Rg.m[1][a], s * Rg.m[2][a]);
             p = (i <= 3) ? add(mean, delta) : sub(mean, delta);
         }
-        const vec3 pc = add(quat_rotate(cp.q_start, p), cp.t_start);
         vec2 uv;
-        bool pv;
-        if (cfg.cam.type == 2) {
-            pv = fisheye_project(cfg.cam.fe, pc, cfg.ut_margin, &uv);
-        } else if (cfg.cam.type == 3) {
-            equirect_project((float)cfg.W, (float)cfg.H, pc, &uv);
-            pv = true; // Cameras.cuh:1013-1025 returns valid for every point
-        } else {
-            pv = cfg.cam.dist.on ? opencv_project(pc, cfg, &uv) : pinhole_project(pc, cfg, &uv);
-        }
+        const bool pv = project_world_point<GENERAL>(cfg, cp, p, &uv);
         if (cfg.ut_require_all) {
             valid &= pv;
             if (!pv)
@@ -178,8 +230,9 @@ __device__ __forceinline__ bool project_ut(const ProjCfg& cfg, const CamPose& cp
 __global__ void __launch_bounds__(256) projection_ut_kernel(
     uint32_t C, uint32_t N, const float* __restrict__ means, const float* __restrict__ quats,
     const float* __restrict__ scales, const float* __restrict__ opacities, const float* __restrict__ viewmats0,
-    const float* __restrict__ Ks, int camera_model, const float* __restrict__ radial,
-    const float* __restrict__ tangential, const float* __restrict__ thin_prism, ProjCfg cfg,
+    const float* __restrict__ viewmats1, int rs_type, const float* __restrict__ Ks, int camera_model,
+    const float* __restrict__ radial, const float* __restrict__ tangential, const float* __restrict__ thin_prism,
+    ProjCfg cfg,
     int32_t* __restrict__ radii, float* __restrict__ means2d,
     float* __restrict__ depths, float* __restrict__ conics, float* __restrict__ compensations) {
     const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
@@ -195,9 +248,10 @@ __global__ void __launch_bounds__(256) projection_ut_kernel(
                                 tangential != nullptr ? tangential + cid * 2 : nullptr,
                                 thin_prism != nullptr ? thin_prism + cid * 4 : nullptr, cfg.fx, cfg.fy, cfg.cx, cfg.cy,
                                 cfg.W, cfg.H);
-    const CamPose cp = load_cam_pose(viewmats0 + cid * 16);
+    const CamPose cp = load_cam_pose(viewmats0 + cid * 16, viewmats1 != nullptr ? viewmats1 + cid * 16 : nullptr,
+                                     rs_type, cfg.W, cfg.H);
     ProjOut o;
-    const bool ok = project_ut(cfg, cp, ld3(means, gid), ld4q(quats, gid), ld3(scales, gid), opacities != nullptr,
+    const bool ok = project_ut<true>(cfg, cp, ld3(means, gid), ld4q(quats, gid), ld3(scales, gid), opacities != nullptr,
                                opacities != nullptr ? opacities[gid] : 0.f, &o);
     int2* r2 = reinterpret_cast<int2*>(radii);
     if (!ok) {
@@ -237,7 +291,7 @@ __global__ void __launch_bounds__(256) projection_ut_raw_kernel(
     cfg.cy = Ks[5];
     const CamPose cp = load_cam_pose(viewmat);
     ProjOut o;
-    const bool ok = project_ut(cfg, cp, ld3(means, idx), a.quat, a.scales, true, a.opacity, &o);
+    const bool ok = project_ut<false>(cfg, cp, ld3(means, idx), a.quat, a.scales, true, a.opacity, &o);
     int2* r2 = reinterpret_cast<int2*>(radii);
     if (!ok) {
         r2[idx] = make_int2(0, 0);
@@ -681,8 +735,9 @@ extern "C" int gsx_projection_ut_3dgs_fused(
     cfg.fx = cfg.fy = cfg.cx = cfg.cy = 0.f;
     memset(&cfg.cam, 0, sizeof(cfg.cam));
     hipLaunchKernelGGL(projection_ut_kernel, dim3(cdiv((uint64_t)C * N, 256)), dim3(256), 0, (hipStream_t)stream, C,
-                       N, means, quats, scales, opacities, viewmats0, Ks, camera_model, radial_coeffs,
-                       tangential_coeffs, thin_prism_coeffs, cfg, radii, means2d, depths, conics, compensations);
+                       N, means, quats, scales, opacities, viewmats0, viewmats1, rs_type, Ks, camera_model,
+                       radial_coeffs, tangential_coeffs, thin_prism_coeffs, cfg, radii, means2d, depths, conics,
+                       compensations);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

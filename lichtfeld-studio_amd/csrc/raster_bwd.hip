@@ -54,7 +54,8 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     const uint8_t* __restrict__ masks, uint32_t image_width, uint32_t image_height, uint32_t tile_width,
     uint32_t tile_height, const float* __restrict__ viewmat, const float* __restrict__ Kmat,
     int camera_model, const float* __restrict__ radial, const float* __restrict__ tangential,
-    const float* __restrict__ thin_prism, const int32_t* __restrict__ tile_offsets,
+    const float* __restrict__ thin_prism, const float* __restrict__ viewmat1, int rs_type,
+    const int32_t* __restrict__ tile_offsets,
     const int32_t* __restrict__ flatten_ids,
     const float* __restrict__ render_alphas, const int32_t* __restrict__ last_ids,
     const float* __restrict__ v_render_colors, const float* __restrict__ v_render_alphas,
@@ -81,7 +82,9 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     const uint32_t pix_id = min(i * image_width + j, image_width * image_height - 1); // :92-93
     uint8_t* wave_list = lists[tr >> 6];
 
-    const CamPose cp = load_cam_pose(viewmat);
+    const CamPose cp = DIST ? load_cam_pose(viewmat, viewmat1, rs_type, image_width, image_height) : load_cam_pose(viewmat);
+    // rolling shutter: the records carry the means and every pixel has its own ray origin
+    const bool rolling = DIST && rs_type != GSX_GLOBAL;
     vec3 ray_o, ray_d;
     CameraModel cam;
     cam.type = 0, cam.dist.on = false;
@@ -91,6 +94,12 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     // a pixel without a valid ray takes no part (RasterizeToPixelsFromWorld3DGSBwd.cu:157)
     inside &= pixel_world_ray(cp, (float)j + 0.5f, (float)i + 0.5f, Kmat[0], Kmat[4], Kmat[2], Kmat[5], cam, &ray_o,
                               &ray_d);
+    // v_M = v_grd (x) ray_d + v_gro (x) (ray_o - mean) (RasterizeToPixelsFromWorld3DGSBwd.cu:330-340); the epilogue
+    // adds (sum v_gro) (x) (o_ref - mean) with the start pose's centre o_ref, so under a rolling shutter the nine
+    // accumulators also take v_gro (x) (ray_o - o_ref) of this pixel
+    vec3 o_shift = mk3(0.f, 0.f, 0.f);
+    if (rolling)
+        o_shift = sub(ray_o, camera_ray_origin(load_cam_pose(viewmat)));
 
     const int32_t range_start = tile_offsets[tile_id];
     int32_t range_end = (tile_id == tile_width * tile_height - 1) ? (int32_t)n_isects : tile_offsets[tile_id + 1];
@@ -158,7 +167,12 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             const float4 m0 = stage[t * 4 + 1];
             const float4 m1 = stage[t * 4 + 2];
             const float4 m2 = stage[t * 4 + 3];
-            const vec3 gro = mk3(a.x, a.y, a.z);
+            vec3 gro = mk3(a.x, a.y, a.z);
+            if (rolling) { // M (ray_o - mean), the record's arithmetic
+                const vec3 d = sub(ray_o, gro);
+                gro = mk3(fma(m0.z, d.z, fma(m0.y, d.y, m0.x * d.x)), fma(m1.y, d.z, fma(m1.x, d.y, m0.w * d.x)),
+                          fma(m2.x, d.z, fma(m1.w, d.y, m1.z * d.x)));
+            }
             const vec3 grd = mk3(fma(m0.z, ray_d.z, fma(m0.y, ray_d.y, m0.x * ray_d.x)),
                                  fma(m1.y, ray_d.z, fma(m1.x, ray_d.y, m0.w * ray_d.x)),
                                  fma(m2.x, ray_d.z, fma(m1.w, ray_d.y, m1.z * ray_d.x)));
@@ -225,6 +239,13 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             v[13] = v_grd.z * ray_d.y;
             v[14] = v_grd.z * ray_d.z;
             v[15] = vis * v_alpha;
+            if (rolling) {
+                v[6] = fma(v_gro.x, o_shift.x, v[6]), v[7] = fma(v_gro.x, o_shift.y, v[7]);
+                v[8] = fma(v_gro.x, o_shift.z, v[8]), v[9] = fma(v_gro.y, o_shift.x, v[9]);
+                v[10] = fma(v_gro.y, o_shift.y, v[10]), v[11] = fma(v_gro.y, o_shift.z, v[11]);
+                v[12] = fma(v_gro.z, o_shift.x, v[12]), v[13] = fma(v_gro.z, o_shift.y, v[13]);
+                v[14] = fma(v_gro.z, o_shift.z, v[14]);
+            }
 #pragma unroll
             for (uint32_t k = 0; k < CDIM; ++k)
                 buffer[k] += col[k] * fac;
@@ -351,15 +372,15 @@ extern "C" int gsx_rasterize_bwd_clear(uint32_t N, void* workspace, size_t works
 namespace gsx {
 int pack_raster_records(uint32_t N, const float* means, const float* quats, const float* scales,
                         const float* opacities, const float* colors, uint32_t channels, const float* viewmat,
-                        const float* K, uint32_t image_width, uint32_t image_height, bool pinhole, void* records,
-                        void* stream); // raster_fwd.hip
+                        const float* K, uint32_t image_width, uint32_t image_height, bool pinhole, bool rolling,
+                        void* records, void* stream); // raster_fwd.hip
 
 static int rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isects, const void* records,
                                     const float* colors, uint32_t channels, const float* backgrounds,
                                     const uint8_t* masks, uint32_t image_width, uint32_t image_height,
                                     uint32_t tile_size, const float* viewmats0, const float* Ks, int camera_model,
                                     const float* radial, const float* tangential, const float* thin_prism,
-                                    const int32_t* tile_offsets,
+                                    const float* viewmats1, int rs_type, const int32_t* tile_offsets,
                                     const int32_t* flatten_ids, const float* render_alphas, const int32_t* last_ids,
                                     const float* v_render_colors, const float* v_render_alphas, void* workspace,
                                     size_t workspace_bytes, void* stream) {
@@ -381,14 +402,14 @@ static int rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isects, co
     GSX_REQUIRE(channels <= 3 || colors != nullptr, GSX_ERR_INVALID_ARGUMENT, "rasterize bwd: colors is null");
     const uint32_t tw = cdiv(image_width, kTile), th = cdiv(image_height, kTile);
     float* gextra = (float*)((char*)workspace + accum_extra_offset(N));
-    const bool distorted =
-        camera_model != GSX_PINHOLE || radial != nullptr || tangential != nullptr || thin_prism != nullptr;
+    const bool distorted = camera_model != GSX_PINHOLE || radial != nullptr || tangential != nullptr ||
+                           thin_prism != nullptr || rs_type != GSX_GLOBAL || viewmats1 != nullptr;
 #define GSX_LAUNCH_BWD(CD, DI)                                                                                       \
     hipLaunchKernelGGL((rasterize_bwd_kernel<CD, DI>), dim3(tw * th), dim3(256), 0, (hipStream_t)stream,             \
                        (uint32_t)n_isects, (const float4*)records, colors, backgrounds, masks, image_width,          \
                        image_height, tw, th, viewmats0, Ks, camera_model, radial, tangential, thin_prism,            \
-                       tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors, v_render_alphas,         \
-                       (float*)workspace, gextra)
+                       viewmats1, rs_type, tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors,      \
+                       v_render_alphas, (float*)workspace, gextra)
 #define GSX_LAUNCH_BWD2(CD)       \
     if (distorted)                \
         GSX_LAUNCH_BWD(CD, true); \
@@ -418,7 +439,7 @@ extern "C" int gsx_rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_is
                                             void* workspace, size_t workspace_bytes, void* stream) {
     return rasterize_bwd_accumulate(C, N, n_isects, records, colors, channels, backgrounds, masks, image_width,
                                     image_height, tile_size, viewmats0, Ks, GSX_PINHOLE, nullptr, nullptr, nullptr,
-                                    tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors,
+                                    nullptr, GSX_GLOBAL, tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors,
                                     v_render_alphas, workspace, workspace_bytes, stream);
 }
 
@@ -468,13 +489,16 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
     void* records = (char*)workspace + acc_bytes;
     if ((rc = gsx_rasterize_bwd_clear(N, workspace, acc_bytes, stream)) != GSX_OK)
         return rc;
-    const bool pinhole = camera_model == GSX_PINHOLE && !(radial_coeffs || tangential_coeffs || thin_prism_coeffs);
+    const bool rolling = rs_type != GSX_GLOBAL;
+    const bool pinhole =
+        camera_model == GSX_PINHOLE && !(radial_coeffs || tangential_coeffs || thin_prism_coeffs) && !rolling;
     if ((rc = pack_raster_records(N, means, quats, scales, opacities, colors, channels, viewmats0, Ks, image_width,
-                                  image_height, pinhole, records, stream)) != GSX_OK)
+                                  image_height, pinhole, rolling, records, stream)) != GSX_OK)
         return rc;
     if ((rc = rasterize_bwd_accumulate(C, N, n_isects, records, colors, channels, backgrounds, masks, image_width,
                                        image_height, tile_size, viewmats0, Ks, camera_model, radial_coeffs,
-                                       tangential_coeffs, thin_prism_coeffs, tile_offsets, flatten_ids, render_alphas, last_ids,
+                                       tangential_coeffs, thin_prism_coeffs, viewmats1, rs_type, tile_offsets,
+                                       flatten_ids, render_alphas, last_ids,
                                        v_render_colors, v_render_alphas, workspace, acc_bytes, stream)) != GSX_OK)
         return rc;
     return gsx_rasterize_bwd_finish(N, means, quats, scales, viewmats0, workspace, acc_bytes, 0, channels, v_means,

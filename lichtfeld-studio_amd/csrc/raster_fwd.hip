@@ -23,7 +23,8 @@ __global__ void __launch_bounds__(256) pack_records_kernel(uint32_t N, const flo
                                                             const float* __restrict__ colors,
                                                             const float* __restrict__ viewmat,
                                                             const float* __restrict__ Kmat, uint32_t W, uint32_t H,
-                                                            bool pinhole, float4* __restrict__ records) {
+                                                            bool pinhole, bool rolling,
+                                                            float4* __restrict__ records) {
     const uint32_t g = blockIdx.x * 256u + threadIdx.x;
     if (g >= N)
         return;
@@ -37,7 +38,9 @@ __global__ void __launch_bounds__(256) pack_records_kernel(uint32_t N, const flo
     const float c0 = colors[(size_t)g * CDIM];
     const float c1 = CDIM > 1 ? colors[(size_t)g * CDIM + 1] : 0.f;
     const float c2 = CDIM > 2 ? colors[(size_t)g * CDIM + 2] : 0.f;
-    store_record(records + (size_t)g * kRecordF4, gro, opac, M, c0, c1, c2, b);
+    // rolling shutter: every pixel row / column has its own ray origin, so the record carries the mean and the
+    // rasterizers form M (ray_o - mean) per pixel
+    store_record(records + (size_t)g * kRecordF4, rolling ? xyz : gro, opac, M, c0, c1, c2, b);
 }
 
 // STATS: count instead of rendering (for roofline accounting); stats[0] += (pixel, Gaussian) pairs evaluated,
@@ -45,9 +48,9 @@ __global__ void __launch_bounds__(256) pack_records_kernel(uint32_t N, const flo
 // [3] += (wave, Gaussian) iterations executed, [4] += (wave, Gaussian) iterations removed by the pixel bounds,
 // [5] += executed iterations in which at least one pixel reaches the alpha threshold, [6] / [7] += the halves
 // (8x4 rows / 4x8 columns) of those iterations' blocks that hold such a pixel.
-// DIST: any camera but the perfect pinhole - OpenCV distortion, fisheye, equirectangular (each pixel's ray comes
-// from the model's unprojection; a pixel without a valid ray is done from the start,
-// RasterizeToPixelsFromWorld3DGSFwd.cu:145).
+// DIST: any camera but the perfect pinhole with a global shutter - OpenCV distortion, fisheye, equirectangular,
+// rolling shutter (each pixel's ray comes from the model's unprojection under the pose of its exposure time; a pixel
+// without a valid ray is done from the start, RasterizeToPixelsFromWorld3DGSFwd.cu:145).
 template <uint32_t CDIM, bool STATS, bool DIST>
 __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
     uint32_t n_isects, const float4* __restrict__ records, const float* __restrict__ colors,
@@ -55,7 +58,7 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
     uint32_t image_height, uint32_t tile_width, uint32_t tile_height, const float* __restrict__ viewmat,
     const float* __restrict__ Kmat, int camera_model, const float* __restrict__ radial,
     const float* __restrict__ tangential, const float* __restrict__ thin_prism,
-    const int32_t* __restrict__ tile_offsets,
+    const float* __restrict__ viewmat1, int rs_type, const int32_t* __restrict__ tile_offsets,
     const int32_t* __restrict__ flatten_ids, float* __restrict__ render_colors, float* __restrict__ render_alphas,
     int32_t* __restrict__ last_ids, unsigned long long* __restrict__ stats) {
     __shared__ float4 stage[kBatch * 4];
@@ -83,7 +86,9 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
         return;
     }
 
-    const CamPose cp = load_cam_pose(viewmat);
+    const CamPose cp = DIST ? load_cam_pose(viewmat, viewmat1, rs_type, image_width, image_height) : load_cam_pose(viewmat);
+    // rolling shutter: the records carry the means and every pixel has its own ray origin
+    const bool rolling = DIST && rs_type != GSX_GLOBAL;
     vec3 ray_o, ray_d;
     CameraModel cam;
     cam.type = 0, cam.dist.on = false;
@@ -142,7 +147,12 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
             const float4 m0 = stage[t * 4 + 1];
             const float4 m1 = stage[t * 4 + 2];
             const float4 m2 = stage[t * 4 + 3];
-            const vec3 gro = mk3(a.x, a.y, a.z);
+            vec3 gro = mk3(a.x, a.y, a.z);
+            if (rolling) { // M (ray_o - mean), the record's arithmetic
+                const vec3 d = sub(ray_o, gro);
+                gro = mk3(fma(m0.z, d.z, fma(m0.y, d.y, m0.x * d.x)), fma(m1.y, d.z, fma(m1.x, d.y, m0.w * d.x)),
+                          fma(m2.x, d.z, fma(m1.w, d.y, m1.z * d.x)));
+            }
             // grd = normalize(M ray_d)
             const vec3 gd = mk3(fma(m0.z, ray_d.z, fma(m0.y, ray_d.y, m0.x * ray_d.x)),
                                 fma(m1.y, ray_d.z, fma(m1.x, ray_d.y, m0.w * ray_d.x)),
@@ -228,8 +238,8 @@ extern "C" size_t gsx_raster_records_bytes(uint32_t N) { return align_up((size_t
 namespace gsx {
 int pack_raster_records(uint32_t N, const float* means, const float* quats, const float* scales,
                         const float* opacities, const float* colors, uint32_t channels, const float* viewmat,
-                        const float* K, uint32_t image_width, uint32_t image_height, bool pinhole, void* records,
-                        void* stream) {
+                        const float* K, uint32_t image_width, uint32_t image_height, bool pinhole, bool rolling,
+                        void* records, void* stream) {
     if (N == 0)
         return GSX_OK;
     GSX_REQUIRE(means && quats && scales && opacities && colors && viewmat && K && records, GSX_ERR_INVALID_ARGUMENT,
@@ -239,7 +249,7 @@ int pack_raster_records(uint32_t N, const float* means, const float* quats, cons
     hipStream_t s = (hipStream_t)stream;
 #define GSX_LAUNCH_PACK(CD)                                                                                         \
     hipLaunchKernelGGL((pack_records_kernel<CD>), grid, block, 0, s, N, means, quats, scales, opacities, colors,    \
-                       viewmat, K, image_width, image_height, pinhole, (float4*)records)
+                       viewmat, K, image_width, image_height, pinhole, rolling, (float4*)records)
     switch (channels) {
     case 1: GSX_LAUNCH_PACK(1); break;
     case 3: GSX_LAUNCH_PACK(3); break;
@@ -256,9 +266,9 @@ int pack_raster_records(uint32_t N, const float* means, const float* quats, cons
 int rasterize_records_fwd(int64_t n_isects, const void* records, const float* colors, uint32_t channels,
                           const float* backgrounds, const uint8_t* masks, uint32_t image_width, uint32_t image_height,
                           const float* viewmat, const float* K, int camera_model, const float* radial,
-                          const float* tangential, const float* thin_prism, const int32_t* tile_offsets,
-                          const int32_t* flatten_ids,
-                          float* render_colors, float* render_alphas, int32_t* last_ids, void* stream) {
+                          const float* tangential, const float* thin_prism, const float* viewmat1, int rs_type,
+                          const int32_t* tile_offsets, const int32_t* flatten_ids, float* render_colors,
+                          float* render_alphas, int32_t* last_ids, void* stream) {
     if (image_width == 0 || image_height == 0)
         return GSX_OK;
     GSX_REQUIRE(n_isects >= 0 && n_isects < (1ll << 31), GSX_ERR_OVERFLOW, "rasterize fwd: n_isects out of range");
@@ -269,13 +279,13 @@ int rasterize_records_fwd(int64_t n_isects, const void* records, const float* co
     const uint32_t tw = cdiv(image_width, kTile), th = cdiv(image_height, kTile);
     const dim3 grid(tw * th), block(256);
     hipStream_t s = (hipStream_t)stream;
-    const bool distorted =
-        camera_model != GSX_PINHOLE || radial != nullptr || tangential != nullptr || thin_prism != nullptr;
+    const bool distorted = camera_model != GSX_PINHOLE || radial != nullptr || tangential != nullptr ||
+                           thin_prism != nullptr || rs_type != GSX_GLOBAL || viewmat1 != nullptr;
 #define GSX_LAUNCH_FWD(CD, DI)                                                                                      \
     hipLaunchKernelGGL((rasterize_fwd_kernel<CD, false, DI>), grid, block, 0, s, (uint32_t)n_isects,                \
                        (const float4*)records, colors, backgrounds, masks, image_width, image_height, tw, th,       \
-                       viewmat, K, camera_model, radial, tangential, thin_prism, tile_offsets, flatten_ids,         \
-                       render_colors, render_alphas, last_ids, (unsigned long long*)nullptr)
+                       viewmat, K, camera_model, radial, tangential, thin_prism, viewmat1, rs_type, tile_offsets,   \
+                       flatten_ids, render_colors, render_alphas, last_ids, (unsigned long long*)nullptr)
 #define GSX_LAUNCH_FWD2(CD)     \
     if (distorted)              \
         GSX_LAUNCH_FWD(CD, true); \
@@ -301,7 +311,7 @@ extern "C" int gsx_pack_raster_records(uint32_t N, const float* means, const flo
                                        const float* viewmat, const float* K, uint32_t image_width,
                                        uint32_t image_height, void* records, void* stream) {
     return pack_raster_records(N, means, quats, scales, opacities, colors, channels, viewmat, K, image_width,
-                               image_height, true, records, stream);
+                               image_height, true, false, records, stream);
 }
 
 extern "C" int gsx_rasterize_records_fwd(int64_t n_isects, const void* records, const float* colors,
@@ -311,8 +321,8 @@ extern "C" int gsx_rasterize_records_fwd(int64_t n_isects, const void* records, 
                                          float* render_colors, float* render_alphas, int32_t* last_ids,
                                          void* stream) {
     return rasterize_records_fwd(n_isects, records, colors, channels, backgrounds, masks, image_width, image_height,
-                                 viewmat, K, GSX_PINHOLE, nullptr, nullptr, nullptr, tile_offsets, flatten_ids,
-                                 render_colors, render_alphas, last_ids, stream);
+                                 viewmat, K, GSX_PINHOLE, nullptr, nullptr, nullptr, nullptr, GSX_GLOBAL, tile_offsets,
+                                 flatten_ids, render_colors, render_alphas, last_ids, stream);
 }
 
 extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
@@ -341,14 +351,17 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
                         workspace_bytes >= gsx_raster_records_bytes(N),
                     GSX_ERR_WORKSPACE, "rasterize fwd: workspace needs %zu bytes, 256-byte aligned",
                     gsx_raster_records_bytes(N));
-        const bool pinhole = camera_model == GSX_PINHOLE && !(radial_coeffs || tangential_coeffs || thin_prism_coeffs);
+        const bool rolling = rs_type != GSX_GLOBAL;
+        const bool pinhole = camera_model == GSX_PINHOLE && !(radial_coeffs || tangential_coeffs || thin_prism_coeffs) &&
+                             !rolling;
         if ((rc = pack_raster_records(N, means, quats, scales, opacities, colors, channels, viewmats0, Ks, image_width,
-                                      image_height, pinhole, workspace, stream)) != GSX_OK)
+                                      image_height, pinhole, rolling, workspace, stream)) != GSX_OK)
             return rc;
     }
     return rasterize_records_fwd(n_isects, workspace, colors, channels, backgrounds, masks, image_width, image_height,
                                  viewmats0, Ks, camera_model, radial_coeffs, tangential_coeffs, thin_prism_coeffs,
-                                 tile_offsets, flatten_ids, render_colors, render_alphas, last_ids, stream);
+                                 viewmats1, rs_type, tile_offsets, flatten_ids, render_colors, render_alphas, last_ids,
+                                 stream);
 }
 
 // Pair counts of one forward pass (no counterpart in the reference; used to turn kernel times into flop rates).
@@ -364,8 +377,8 @@ extern "C" int gsx_rasterize_pair_stats(int64_t n_isects, const void* records, u
     hipLaunchKernelGGL((rasterize_fwd_kernel<3, true, false>), dim3(tw * th), dim3(256), 0, (hipStream_t)stream,
                        (uint32_t)n_isects, (const float4*)records, (const float*)nullptr, (const float*)nullptr,
                        (const uint8_t*)nullptr, image_width, image_height, tw, th, viewmat, K, (int)GSX_PINHOLE,
-                       (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, tile_offsets, flatten_ids,
-                       (float*)nullptr,
+                       (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
+                       (int)GSX_GLOBAL, tile_offsets, flatten_ids, (float*)nullptr,
                        (float*)nullptr, (int32_t*)nullptr, stats_out);
     GSX_LAUNCH_CHECK();
     return GSX_OK;

@@ -58,6 +58,13 @@ struct RollingShutter {
     quat q_start, q_end;
 };
 
+// Rolling-shutter state of the one camera (set by orc_set_rolling_shutter; GLOBAL = 4 and no end pose by default):
+// the operators' `rs_type` / `viewmats1` arguments (Ops.h:69-98), kept out of every signature.
+int g_rs_type = 4;
+bool g_has_end_pose = false;
+float g_end_pose[16];
+uint32_t g_W = 0, g_H = 0; // image size for the unprojections and the shutter time (set with the camera model)
+
 // Cameras.cuh:39-70 : rotation part of the row-major [4,4] world->camera matrix as a quaternion.
 RollingShutter make_rolling_shutter(const float* se3_start, const float* se3_end) {
     RollingShutter rs;
@@ -67,6 +74,8 @@ RollingShutter make_rolling_shutter(const float* se3_start, const float* se3_end
             R.m[r][c] = se3_start[r * 4 + c];
     rs.q_start = gsx::quat_cast(R);
     rs.t_start = gsx::mk3(se3_start[3], se3_start[7], se3_start[11]);
+    if (se3_end == nullptr && g_has_end_pose)
+        se3_end = g_end_pose;
     if (se3_end == nullptr) {
         rs.q_end = rs.q_start;
         rs.t_end = rs.t_start;
@@ -88,6 +97,17 @@ ShutterPose interpolate_shutter_pose(float rel, const RollingShutter& rs) {
     p.t.z = (1.f - rel) * rs.t_start.z + rel * rs.t_end.z;
     p.q = gsx::slerp(rs.q_start, rs.q_end, rel);
     return p;
+}
+
+// Cameras.cuh:293-320 : when a pixel is exposed, as a fraction of the frame time (0 for a global shutter)
+float shutter_relative_frame_time(float x, float y, uint32_t W, uint32_t H) {
+    switch (g_rs_type) {
+    case 0: return gsx::floor(y) / (float)(H - 1);
+    case 1: return gsx::floor(x) / (float)(W - 1);
+    case 2: return ((float)H - gsx::ceil(y)) / (float)(H - 1);
+    case 3: return ((float)W - gsx::ceil(x)) / (float)(W - 1);
+    default: return 0.f;
+    }
 }
 
 // Cameras.cuh:416-455 : perfect pinhole projection with the 10 % margin validity test (:228-240)
@@ -169,7 +189,41 @@ bool project_point(vec3 cam, float fx, float fy, float cx, float cy, uint32_t W,
     return g_dist.on ? opencv_project(g_dist, cam, fx, fy, cx, cy, W, H, margin_factor, out)
                      : pinhole_project(cam, fx, fy, cx, cy, W, H, margin_factor, out);
 }
-uint32_t g_W = 0, g_H = 0; // image size for the models whose unprojection needs it (set by the rasterizers)
+
+// Cameras.cuh:346-414 world_point_to_image_point_shutter_pose: a global shutter projects under the start pose; a
+// rolling shutter starts from the start-pose projection (the end-pose one if only that is valid; neither valid =
+// invalid) and iterates 10 times "exposure time of the current image point -> pose -> projection", returning the
+// last image point as valid.
+bool project_world_point_shutter(vec3 world, const RollingShutter& rs, float fx, float fy, float cx, float cy,
+                                 uint32_t W, uint32_t H, float margin_factor, vec2* out) {
+    vec2 p_start;
+    const bool valid_start = project_point(gsx::add(gsx::quat_rotate(rs.q_start, world), rs.t_start), fx, fy, cx,
+                                           cy, W, H, margin_factor, &p_start);
+    if (g_rs_type == 4) {
+        *out = p_start;
+        return valid_start;
+    }
+    vec2 p_end;
+    const bool valid_end =
+        project_point(gsx::add(gsx::quat_rotate(rs.q_end, world), rs.t_end), fx, fy, cx, cy, W, H, margin_factor, &p_end);
+    vec2 prev;
+    if (valid_start) {
+        prev = p_start;
+    } else if (valid_end) {
+        prev = p_end;
+    } else {
+        *out = p_end;
+        return false;
+    }
+    for (int j = 0; j < 10; ++j) {
+        const ShutterPose pose = interpolate_shutter_pose(shutter_relative_frame_time(prev.x, prev.y, W, H), rs);
+        vec2 p;
+        project_point(gsx::add(gsx::quat_rotate(pose.q, world), pose.t), fx, fy, cx, cy, W, H, margin_factor, &p);
+        prev = p;
+    }
+    *out = prev;
+    return true;
+}
 
 // Cameras.cuh:635-740 : Newton undistortion (at most 5 steps, stop at |step| < 1e-6).  The reference's double
 // literals make parts of the Jacobian double arithmetic; the expressions are kept as written there.
@@ -219,8 +273,8 @@ bool opencv_undistort_newton(const Distortion& d, float xd, float yd, float* xo,
     return converged;
 }
 
-// Cameras.cuh:457-470 / 742-755 + 253-266 + 322-339 : pixel centre -> world ray, global shutter (relative frame
-// time 0 because shutter_relative_frame_time has no GLOBAL case, :293-320).  Returns the ray's valid flag (false
+// Cameras.cuh:457-470 / 742-755 + 253-266 + 322-339 : pixel centre -> world ray under the pose of the pixel's
+// exposure time (the start pose for a global shutter: shutter_relative_frame_time has no GLOBAL case).  Returns the ray's valid flag (false
 // only when the undistortion did not converge; then the ray is zero, :330-333).
 bool pixel_world_ray(float px, float py, float fx, float fy, float cx, float cy,
                      const RollingShutter& rs, vec3* ray_o, vec3* ray_d) {
@@ -245,7 +299,7 @@ bool pixel_world_ray(float px, float py, float fx, float fy, float cx, float cy,
         *ray_d = gsx::mk3(0.f, 0.f, 0.f);
         return false;
     }
-    const ShutterPose pose = interpolate_shutter_pose(0.f, rs);
+    const ShutterPose pose = interpolate_shutter_pose(shutter_relative_frame_time(px, py, g_W, g_H), rs);
     const mat3 R_inv = gsx::mat3_cast(gsx::quat_inverse(pose.q));
     *ray_o = gsx::neg(gsx::mul(R_inv, pose.t));
     *ray_d = gsx::mul(R_inv, d_cam);
@@ -299,7 +353,7 @@ ORC_API int orc_projection_ut_3dgs_fused(
         // :76-82 centre-of-shutter pose, near/far cull
         const ShutterPose pose = interpolate_shutter_pose(0.5f, rs);
         const vec3 mean_c = gsx::add(gsx::quat_rotate(pose.q, mean), pose.t);
-        if (mean_c.z < near_plane || mean_c.z > far_plane) {
+        if ((mean_c.z < near_plane && g_model != 3) || mean_c.z > far_plane) { // :78
             radii[idx * 2] = 0;
             radii[idx * 2 + 1] = 0;
             continue;
@@ -333,9 +387,9 @@ ORC_API int orc_projection_ut_3dgs_fused(
         vec2 ip[7];
         vec2 m2 = {0.f, 0.f};
         for (int i = 0; i < 7; ++i) {
-            const vec3 pc = gsx::add(gsx::quat_rotate(rs.q_start, pts[i]), rs.t_start);
             vec2 p;
-            const bool pv = project_point(pc, fx, fy, cx, cy, image_width, image_height, ut_margin, &p);
+            const bool pv = project_world_point_shutter(pts[i], rs, fx, fy, cx, cy, image_width, image_height,
+                                                        ut_margin, &p);
             if (ut_require_all) {
                 valid &= pv;
                 if (!pv) {
@@ -1881,6 +1935,40 @@ ORC_API void orc_set_camera_model(int model, const float* radial, const float* t
         g_dist.p[i] = tangential[i];
     for (int i = 0; i < 4 && thin_prism; ++i)
         g_dist.s[i] = thin_prism[i];
+}
+
+ORC_API void orc_set_image_size(uint32_t W, uint32_t H) { g_W = W, g_H = H; }
+ORC_API uint32_t orc_get_image_size(int axis) { return axis == 0 ? g_W : g_H; }
+
+// rs_type: gsplat/Cameras.h:16-22 (4 = GLOBAL); viewmat1: the end-of-frame pose [4,4] or null (= the start pose)
+ORC_API void orc_set_rolling_shutter(int rs_type, const float* viewmat1) {
+    g_rs_type = rs_type;
+    g_has_end_pose = viewmat1 != nullptr;
+    if (viewmat1 != nullptr)
+        std::memcpy(g_end_pose, viewmat1, sizeof(g_end_pose));
+}
+
+// world points [n,3] -> image points [n,2] + valid [n] under the current camera model and shutter, viewmat [4,4]
+ORC_API void orc_world_project(int64_t n, const float* pts, const float* viewmat, float fx, float fy, float cx,
+                               float cy, uint32_t W, uint32_t H, float margin, float* out, uint8_t* valid) {
+    const RollingShutter rs = make_rolling_shutter(viewmat, nullptr);
+    for (int64_t i = 0; i < n; ++i) {
+        vec2 p;
+        valid[i] = project_world_point_shutter(ld3(pts, i), rs, fx, fy, cx, cy, W, H, margin, &p) ? 1 : 0;
+        out[2 * i] = p.x, out[2 * i + 1] = p.y;
+    }
+}
+
+// pixel positions [n,2] -> world rays (origin [n,3], direction [n,3]) + valid [n] under the current model and shutter
+ORC_API void orc_pixel_world_rays(int64_t n, const float* image_points, const float* viewmat, float fx, float fy,
+                                  float cx, float cy, float* origins, float* dirs, uint8_t* valid) {
+    const RollingShutter rs = make_rolling_shutter(viewmat, nullptr);
+    for (int64_t i = 0; i < n; ++i) {
+        vec3 o, d;
+        valid[i] = pixel_world_ray(image_points[2 * i], image_points[2 * i + 1], fx, fy, cx, cy, rs, &o, &d) ? 1 : 0;
+        origins[3 * i] = o.x, origins[3 * i + 1] = o.y, origins[3 * i + 2] = o.z;
+        dirs[3 * i] = d.x, dirs[3 * i + 1] = d.y, dirs[3 * i + 2] = d.z;
+    }
 }
 
 // camera-space points [n,3] -> image points [n,2] + valid [n] under the current camera model

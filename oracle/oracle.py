@@ -31,6 +31,7 @@ def lib():
         _lib = ctypes.CDLL(_LIB_PATH)
         _lib.orc_tile_n_bits.restype = c_u32
         _lib.orc_num_threads.restype = c_i
+        _lib.orc_get_image_size.restype = c_u32
     return _lib
 
 
@@ -86,6 +87,48 @@ class camera_model:
     def __exit__(self, *exc):
         lib().orc_set_camera_model(c_i(0), None, None, None, c_u32(0), c_u32(0))
         return False
+
+
+class rolling_shutter:
+    """Context manager: shutter type (gsplat/Cameras.h:16-22: 0 top-to-bottom, 1 left-to-right, 2 bottom-to-top,
+    3 right-to-left, 4 global) and end-of-frame pose viewmat1 [4,4] for every projection / pixel ray inside the block;
+    W, H = the image size (the exposure time of a pixel is its row / column over H - 1 / W - 1)."""
+
+    def __init__(self, rs_type, viewmat1, W, H):
+        self.rs_type, self.W, self.H = int(rs_type), int(W), int(H)
+        self.vm1 = None if viewmat1 is None else np.ascontiguousarray(np.asarray(viewmat1, np.float32).reshape(4, 4))
+
+    def __enter__(self):
+        L = lib()
+        self.prev = (L.orc_get_image_size(0), L.orc_get_image_size(1))
+        L.orc_set_image_size(c_u32(self.W), c_u32(self.H))
+        L.orc_set_rolling_shutter(c_i(self.rs_type), _p(self.vm1))
+        return self
+
+    def __exit__(self, *exc):
+        lib().orc_set_rolling_shutter(c_i(4), None)
+        lib().orc_set_image_size(c_u32(self.prev[0]), c_u32(self.prev[1]))
+        return False
+
+
+def world_project(points, viewmat, fx, fy, cx, cy, W, H, margin=0.1):
+    """world points [n,3] -> (image points [n,2], valid [n]) under the current camera model and shutter"""
+    pts, vm = _f32(points).reshape(-1, 3), _f32(viewmat).reshape(4, 4)
+    out = np.zeros((pts.shape[0], 2), np.float32)
+    valid = np.zeros(pts.shape[0], np.uint8)
+    lib().orc_world_project(c_i64(pts.shape[0]), _p(pts), _p(vm), c_f(fx), c_f(fy), c_f(cx), c_f(cy), c_u32(W),
+                            c_u32(H), c_f(margin), _p(out), _p(valid))
+    return out, valid.astype(bool)
+
+
+def pixel_world_rays(image_points, viewmat, fx, fy, cx, cy):
+    """pixel positions [n,2] -> (origins [n,3], directions [n,3], valid [n]) under the current model and shutter"""
+    ip, vm = _f32(image_points).reshape(-1, 2), _f32(viewmat).reshape(4, 4)
+    o, d = np.zeros((ip.shape[0], 3), np.float32), np.zeros((ip.shape[0], 3), np.float32)
+    valid = np.zeros(ip.shape[0], np.uint8)
+    lib().orc_pixel_world_rays(c_i64(ip.shape[0]), _p(ip), _p(vm), c_f(fx), c_f(fy), c_f(cx), c_f(cy), _p(o), _p(d),
+                               _p(valid))
+    return o, d, valid.astype(bool)
 
 
 def math_camera(which, x, x2=None, x3=None):

@@ -69,8 +69,8 @@ def test_status_codes_without_launch(gsx):
         ci(model), ut, ci(rs), nul, nul, nul, one, one, one, one, nul, nul)
     assert proj(2, L.PINHOLE, L.GLOBAL, nul) == L.GSX_ERR_UNSUPPORTED        # C > 1
     assert proj(1, L.ORTHO, L.GLOBAL, nul) == L.GSX_ERR_UNSUPPORTED          # camera model
-    assert proj(1, L.PINHOLE, L.ROLLING_TOP_TO_BOTTOM, nul) == L.GSX_ERR_UNSUPPORTED
-    assert proj(1, L.PINHOLE, L.GLOBAL, one) == L.GSX_ERR_UNSUPPORTED        # viewmats1 given
+    assert proj(1, L.PINHOLE, 5, nul) == L.GSX_ERR_INVALID_ARGUMENT          # not a shutter type
+    assert b"shutter type 5" in lib.gsx_last_error()
     n_host = i64(-1)
     assert lib.gsx_intersect_tile_count(u32(1), u32(10), one, one, u32(16), u32(1 << 20), u32(1 << 11), one, one, one,
                                         ctypes.c_size_t(1 << 20), ctypes.byref(n_host), nul) == \

@@ -111,8 +111,8 @@ def test_projection_unsupported_and_errors(gsx, cuda):
             T(cam.K[None], cuda), cam.width, cam.height, 0.3, 0.01, 1e4, 0.0, False]
     with pytest.raises(gsx._lib.GsxError):  # the orthographic model is not built
         ops.projection_ut_3dgs_fused(*args, 1, ops.UnscentedTransformParameters(), 4)
-    with pytest.raises(gsx._lib.GsxError):  # rolling shutter is not built
-        ops.projection_ut_3dgs_fused(*args, 0, ops.UnscentedTransformParameters(), 0)
+    with pytest.raises(gsx._lib.GsxError):  # not a shutter type
+        ops.projection_ut_3dgs_fused(*args, 0, ops.UnscentedTransformParameters(), 5)
     with pytest.raises(RuntimeError):  # CHECK_INPUT: CPU tensor
         ops.projection_ut_3dgs_fused(torch.from_numpy(means), *args[1:], 0, ops.UnscentedTransformParameters(), 4)
     with pytest.raises(RuntimeError):  # CHECK_INPUT: non-contiguous
@@ -649,18 +649,24 @@ def test_opencv_distortion_projection_and_errors(gsx, orc, cuda):
     assert torch.equal(a[1][0][vis], b[1][0][vis]) and torch.equal(a[3][0][vis], b[3][0][vis])
     with pytest.raises(RuntimeError, match="PINHOLE, FISHEYE and EQUIRECTANGULAR are supported"):
         call(None, None, None, model=1)  # ORTHO
-    with pytest.raises(RuntimeError, match="rolling shutter"):
-        call(None, None, None, rs=0)  # ROLLING_TOP_TO_BOTTOM
+    with pytest.raises(RuntimeError, match="shutter type 7"):
+        call(None, None, None, rs=7)
 
 
-@pytest.mark.parametrize("which", ["fisheye", "fisheye+coeffs", "equirectangular"])
+@pytest.mark.parametrize("which", ["fisheye", "fisheye+coeffs", "equirectangular", "equirectangular-inside"])
 def test_fisheye_and_equirectangular_fused_forward_backward(gsx, orc, cuda, which):
     """OpenCV fisheye (with and without its four radial coefficients) and the equirectangular panorama: UT projection
     through the model and per-pixel unprojection, fused forward bit-identical to the checker, backward at the gradient
     bar (Cameras.cuh:757-1037)"""
     ops = gsx.ops
     sc, cam, h, d = _fused_inputs(gsx, cuda, 20000)
-    model = 3 if which == "equirectangular" else 2
+    model = 3 if which.startswith("equirectangular") else 2
+    if which == "equirectangular-inside":
+        # the camera inside the cloud: Gaussians behind it stay (no near-plane cull for this model,
+        # ProjectionUT3DGSFused.cu:78) and sort by the raw bits of their negative depth
+        h["vm"] = h["vm"].copy()
+        h["vm"][0, :3, 3] = [0.3, -0.2, 0.1]
+        d["vm"] = T(h["vm"], cuda)
     radial = [0.04, -0.006, 0.0008, -0.00005] if which == "fisheye+coeffs" else None
     co = (None if radial is None else T(np.asarray(radial, np.float32)[None], cuda), None, None)
     ut = ops.UnscentedTransformParameters()
@@ -677,6 +683,8 @@ def test_fisheye_and_equirectangular_fused_forward_backward(gsx, orc, cuda, whic
     bits_equal(N(radii), ref[2], "radii")
     vis = ref[2][0, :, 0] > 0
     assert vis.sum() > 2000
+    if which == "equirectangular-inside":
+        assert (ref[4][0][vis] < 0).sum() > 1000
     bits_equal(N(means2d)[0][vis], ref[3][0][vis], "means2d")
     bits_equal(N(ids), ref[10], "sorted tile keys")
     bits_equal(N(flat), ref[7], "sort order")
@@ -705,6 +713,80 @@ def test_fisheye_and_equirectangular_fused_forward_backward(gsx, orc, cuda, whic
                                       cam.height, 0.3, 0.01, 1e4, 0.0, False, model, ut, 4, *co)
     bits_equal(N(pr[0]), ref[2], "standalone projection radii")
     bits_equal(N(pr[1])[0][vis], ref[3][0][vis], "standalone projection means2d")
+
+
+@pytest.mark.parametrize("rs_type,which", [(0, "pinhole"), (1, "pinhole"), (2, "distorted"), (3, "fisheye"),
+                                           (4, "pinhole")])
+def test_rolling_shutter_fused_forward_backward(gsx, orc, cuda, rs_type, which):
+    """rolling shutter (viewmats1 = end-of-frame pose, the four directions of gsplat/Cameras.h:16-22): iterated UT
+    projection, per-pixel pose in both rasterizers; fused forward bit-identical to the checker, backward at the
+    gradient bar.  rs_type 4 with viewmats1: a global shutter, the end pose only moves the centre-of-shutter depth."""
+    from contextlib import ExitStack
+    from scipy.spatial.transform import Rotation
+    ops = gsx.ops
+    sc, cam, h, d = _fused_inputs(gsx, cuda, 20000)
+    step = np.eye(4)
+    step[:3, :3] = Rotation.from_rotvec([0.01, -0.015, 0.02]).as_matrix()
+    step[:3, 3] = [0.05, -0.03, 0.08]
+    vm1 = (step @ h["vm"][0].astype(np.float64)).astype(np.float32)[None]
+    dvm1 = T(vm1, cuda)
+    model = 2 if which == "fisheye" else 0
+    coeffs = dict(radial=_DIST["radial"], tangential=_DIST["tangential"]) if which == "distorted" else {}
+    radial = [0.03, -0.004, 0.0006, 0.0] if which == "fisheye" else coeffs.get("radial")
+    co = (None if radial is None else T(np.asarray(radial, np.float32)[None], cuda),
+          None if "tangential" not in coeffs else T(np.asarray(coeffs["tangential"], np.float32)[None], cuda), None)
+    ut = ops.UnscentedTransformParameters()
+
+    def checker():
+        st = ExitStack()
+        if which == "fisheye":
+            st.enter_context(orc.camera_model(2, cam.width, cam.height, radial=radial))
+        elif coeffs:
+            st.enter_context(orc.distortion(**coeffs))
+        st.enter_context(orc.rolling_shutter(rs_type, vm1[0], cam.width, cam.height))
+        return st
+
+    with checker():
+        ref = orc.rasterize_from_world_with_sh_fwd(h["means"], h["quats"], h["scales"], h["op"], h["shs"], 3, h["bg"],
+                                                   cam.width, cam.height, 16, h["vm"], h["K"])
+    with orc.rolling_shutter(4, None, cam.width, cam.height):
+        pass
+    got = ops.rasterize_from_world_with_sh_fwd(d["means"], d["quats"], d["scales"], d["op"], d["shs"], 3, d["bg"], None,
+                                               cam.width, cam.height, 16, d["vm"], dvm1, d["K"], model, 0.3, 0.01, 1e4,
+                                               0.0, 1.0, False, 0, ut, rs_type, *co, return_isect_ids=True)
+    renders, alphas, radii, means2d, depths, colors, offsets, flat, last_ids, comp, ids = got
+    bits_equal(N(radii), ref[2], "radii")
+    vis = ref[2][0, :, 0] > 0
+    assert vis.sum() > 2000
+    bits_equal(N(means2d)[0][vis], ref[3][0][vis], "means2d")
+    bits_equal(N(depths)[0][vis], ref[4][0][vis], "depths")
+    bits_equal(N(ids), ref[10], "sorted tile keys")
+    bits_equal(N(flat), ref[7], "sort order")
+    bits_equal(N(offsets), ref[6], "per-tile ranges")
+    bits_equal(N(last_ids), ref[8], "last ids")
+    bits_equal(N(renders), ref[0], "image")
+    bits_equal(N(alphas), ref[1], "alpha")
+    assert ref[1].mean() > 0.01
+    if rs_type != 4 and which == "pinhole":  # the motion matters: another image than the start pose's
+        still = orc.rasterize_from_world_with_sh_fwd(h["means"], h["quats"], h["scales"], h["op"], h["shs"], 3,
+                                                     h["bg"], cam.width, cam.height, 16, h["vm"], h["K"])
+        assert np.abs(still[0] - ref[0]).max() > 0.05
+
+    rng = np.random.default_rng(3)
+    v_r = rng.normal(0, 1, tuple(renders.shape)).astype(np.float32)
+    v_a = rng.normal(0, 1, tuple(alphas.shape)).astype(np.float32)
+    op1 = d["op"][None].contiguous()
+    got5 = ops.rasterize_to_pixels_from_world_3dgs_bwd(d["means"], d["quats"], d["scales"], colors, op1, d["bg"], None,
+                                                       cam.width, cam.height, 16, d["vm"], dvm1, d["K"], model, ut,
+                                                       rs_type, *co, offsets, flat, alphas, last_ids, T(v_r, cuda),
+                                                       T(v_a, cuda))
+    args = (h["means"], h["quats"], h["scales"], N(colors), h["op"][None], h["bg"])
+    with checker():
+        o32 = orc.rasterize_to_pixels_from_world_3dgs_bwd(*args, None, cam.width, cam.height, 16, h["vm"], h["K"],
+                                                          N(offsets), N(flat), N(alphas), N(last_ids), v_r, v_a)
+        g64, _ = orc.rasterize_bwd_f64(*args, cam.width, cam.height, 16, h["vm"], h["K"], N(offsets), N(flat),
+                                       N(alphas), N(last_ids), v_r, v_a)
+    check_raster_gradients([N(x) for x in got5], o32, g64, tag=f"rs {rs_type} {which} ")
 
 
 def test_philox_noise_on_device(gsx, orc, cuda):

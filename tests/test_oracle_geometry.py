@@ -506,3 +506,90 @@ def test_equirectangular_closed_form_and_round_trip(orc):
     assert np.all(np.abs(ip[:, 1] - want[:, 1]) < 1.5e-4 + H / np.pi * 1.2e-7 / np.cos(el))
     unit = pts / np.linalg.norm(pts, axis=1, keepdims=True)
     assert np.abs(rays - unit).max() < 3e-6
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# rolling shutter (Cameras.cuh:268-414)
+# ---------------------------------------------------------------------------------------------------------------
+def _pose(rotvec, t):
+    from scipy.spatial.transform import Rotation
+    vm = np.eye(4)
+    vm[:3, :3] = Rotation.from_rotvec(rotvec).as_matrix()
+    vm[:3, 3] = t
+    return vm
+
+
+def _pose_at(vm0, vm1, rel):
+    """float64 model of the pose at a relative frame time: translation lerp, rotation slerp as the geodesic
+    R1 (R1^T R0)^(1 - rel) ... written through the rotation vector so that times outside [0, 1] (image points in the
+    margin around the image) extrapolate, as the quaternion formula does"""
+    from scipy.spatial.transform import Rotation
+    R0, R1 = Rotation.from_matrix(vm0[:3, :3]), Rotation.from_matrix(vm1[:3, :3])
+    # quaternion slerp q0 (q0^-1 q1)^rel; the view rotation is that quaternion's matrix
+    R = (R0 * Rotation.from_rotvec(rel * (R0.inv() * R1).as_rotvec())).as_matrix()
+    return R, (1 - rel) * vm0[:3, 3] + rel * vm1[:3, 3]
+
+
+def _rel_time(rs_type, x, y, W, H):
+    return [np.floor(y) / (H - 1), np.floor(x) / (W - 1), (H - np.ceil(y)) / (H - 1), (W - np.ceil(x)) / (W - 1)][rs_type]
+
+
+@pytest.mark.parametrize("rs_type", [0, 1, 2, 3])
+def test_rolling_shutter_pixel_rays(orc, rs_type):
+    """a pixel's world ray is the global-shutter ray under the pose interpolated to the pixel's exposure time (row or
+    column over H - 1 / W - 1, in the shutter's direction): numpy / scipy Slerp in float64"""
+    W, H, f = 320, 240, 300.0
+    vm0, vm1 = _pose([0.02, -0.01, 0.03], [0.1, -0.2, 4.0]), _pose([-0.05, 0.06, -0.02], [0.4, 0.1, 3.7])
+    r = np.random.default_rng(rs_type)
+    ip = np.stack([r.integers(0, W, 400) + 0.5, r.integers(0, H, 400) + 0.5], 1)
+    with orc.rolling_shutter(rs_type, vm1, W, H):
+        o, d, ok = orc.pixel_world_rays(ip, vm0, f, f, W / 2, H / 2)
+    assert ok.all()
+    for k in range(ip.shape[0]):
+        R, t = _pose_at(vm0, vm1, _rel_time(rs_type, ip[k, 0], ip[k, 1], W, H))
+        cam = np.array([(ip[k, 0] - W / 2) / f, (ip[k, 1] - H / 2) / f, 1.0])
+        assert np.abs(o[k] - (-R.T @ t)).max() < 3e-6
+        assert np.abs(d[k] - R.T @ (cam / np.linalg.norm(cam))).max() < 1e-6
+    # first / last row (column) are exposed under the start / end pose exactly
+    ends = {0: ([[5.5, 0.5]], [[5.5, H - 0.5]]), 1: ([[0.5, 7.5]], [[W - 0.5, 7.5]]),
+            2: ([[5.5, H - 0.5]], [[5.5, 0.5]]), 3: ([[W - 0.5, 7.5]], [[0.5, 7.5]])}[rs_type]
+    with orc.rolling_shutter(rs_type, vm1, W, H):
+        o0 = orc.pixel_world_rays(ends[0], vm0, f, f, W / 2, H / 2)[0][0]
+        o1 = orc.pixel_world_rays(ends[1], vm0, f, f, W / 2, H / 2)[0][0]
+    if rs_type in (0, 1):
+        assert np.abs(o0 - (-vm0[:3, :3].T @ vm0[:3, 3])).max() < 3e-6
+        assert np.abs(o1 - (-vm1[:3, :3].T @ vm1[:3, 3])).max() < 3e-6
+    else:  # (H - ceil(y)) / (H - 1): the last row is at time 0, the first at 1 + 1 / (H - 1) of the frame
+        assert np.abs(o0 - (-vm0[:3, :3].T @ vm0[:3, 3])).max() < 3e-6
+
+
+@pytest.mark.parametrize("rs_type", [0, 1, 2, 3])
+def test_rolling_shutter_projection_is_a_fixed_point(orc, rs_type):
+    """the image point of a world point satisfies p = project(pose(time(p)) X) (float64 model): the iteration of
+    Cameras.cuh:346-414 converges for a moderate motion; with the end pose = the start pose, and for GLOBAL, the
+    plain projection comes back bit for bit"""
+    W, H, f = 320, 240, 300.0
+    vm0, vm1 = _pose([0.02, -0.01, 0.03], [0.1, -0.2, 4.0]), _pose([0.01, 0.01, 0.02], [0.15, -0.15, 3.9])
+    r = np.random.default_rng(10 + rs_type)
+    X = r.normal(0, 0.6, (500, 3))
+    with orc.rolling_shutter(rs_type, vm1, W, H):
+        ip, ok = orc.world_project(X.astype(np.float32), vm0, f, f, W / 2, H / 2, W, H)
+    with orc.rolling_shutter(rs_type, vm0, W, H):
+        same, ok_same = orc.world_project(X.astype(np.float32), vm0, f, f, W / 2, H / 2, W, H)
+    with orc.rolling_shutter(4, vm1, W, H):
+        glob, ok_glob = orc.world_project(X.astype(np.float32), vm0, f, f, W / 2, H / 2, W, H)
+    plain, ok_plain = orc.world_project(X.astype(np.float32), vm0, f, f, W / 2, H / 2, W, H)
+    assert np.array_equal(glob, plain) and np.array_equal(ok_glob, ok_plain)
+    assert np.array_equal(ok_same, ok_plain)
+    assert np.abs(same[ok_plain] - plain[ok_plain]).max() < 2e-4  # slerp(q, q, t) and the lerp round differently
+    assert ok.sum() > 300
+    moved = 0
+    for k in np.flatnonzero(ok):
+        R, t = _pose_at(vm0, vm1, _rel_time(rs_type, ip[k, 0], ip[k, 1], W, H))
+        c = R @ X[k].astype(np.float32).astype(np.float64) + t
+        want = np.array([f * c[0] / c[2] + W / 2, f * c[1] / c[2] + H / 2])
+        # the time is a step function of the pixel: at a row / column boundary the iteration may alternate between two
+        # neighbouring times; the fixed point is then met to one row's worth of motion
+        assert np.abs(ip[k] - want).max() < 0.05, (k, ip[k], want)
+        moved += np.abs(ip[k] - plain[k]).max() > 0.5
+    assert moved > 100  # the motion matters
