@@ -29,6 +29,9 @@ struct ProjCfg {
     float eps2d, near_plane, far_plane, radius_clip;
     float ut_alpha, ut_beta, ut_kappa, ut_margin;
     int ut_require_all;
+    // sigma-point spread and weights (Cameras.cuh:1070-1119), the same for every Gaussian: formed once on the host
+    // from the three parameters above with correctly rounded fp32 operations (what the device would compute)
+    float ut_sq, ut_w0m, ut_w0c, ut_wi;
     float fx, fy, cx, cy;
     CameraModel cam; // type 0 with cam.dist.on = false: the perfect pinhole model
 };
@@ -128,24 +131,17 @@ __device__ __forceinline__ bool project_world_point(const ProjCfg& cfg, const Ca
 
 // GENERAL = false: the perfect pinhole with a global shutter (the training step's camera), decided at compile time
 template <bool GENERAL>
-__device__ __forceinline__ bool project_ut(const ProjCfg& cfg, const CamPose& cp, vec3 mean, quat q_in, vec3 scl,
-                                           bool has_opacity, float opacity_in, ProjOut* o) {
+__device__ __forceinline__ bool project_ut(const ProjCfg& cfg, const CamPose& cp, quat qc, vec3 tc, vec3 mean,
+                                           quat q_in, vec3 scl, bool has_opacity, float opacity_in, ProjOut* o) {
+    // qc, tc: the centre-of-shutter pose shutter_pose(cp, 0.5) (ProjectionUT3DGSFused.cu:76-77)
     const quat q = quat_normalize(q_in);
-    quat qc;
-    vec3 tc;
-    shutter_pose(cp, 0.5f, &qc, &tc);
     const vec3 mean_c = add(quat_rotate(qc, mean), tc);
     // the equirectangular model sees behind the camera (ProjectionUT3DGSFused.cu:78)
     if ((mean_c.z < cfg.near_plane && !(GENERAL && cfg.cam.type == 3)) || mean_c.z > cfg.far_plane)
         return false;
 
-    const float D = 3.0f;
-    const float lambda = cfg.ut_alpha * cfg.ut_alpha * (D + cfg.ut_kappa) - D;
     const mat3 Rg = mat3_cast(q);
-    const float sq = gsx::sqrt(D + lambda);
-    const float w0m = lambda / (D + lambda);
-    const float w0c = lambda / (D + lambda) + (1.f - cfg.ut_alpha * cfg.ut_alpha + cfg.ut_beta);
-    const float wi = 1.f / (2.f * (D + lambda));
+    const float sq = cfg.ut_sq, w0m = cfg.ut_w0m, w0c = cfg.ut_w0c, wi = cfg.ut_wi;
     const float sc[3] = {scl.x, scl.y, scl.z};
 
     vec2 ip[7];
@@ -251,7 +247,10 @@ __global__ void __launch_bounds__(256) projection_ut_kernel(
     const CamPose cp = load_cam_pose(viewmats0 + cid * 16, viewmats1 != nullptr ? viewmats1 + cid * 16 : nullptr,
                                      rs_type, cfg.W, cfg.H);
     ProjOut o;
-    const bool ok = project_ut<true>(cfg, cp, ld3(means, gid), ld4q(quats, gid), ld3(scales, gid), opacities != nullptr,
+    quat qc;
+    vec3 tc;
+    shutter_pose(cp, 0.5f, &qc, &tc);
+    const bool ok = project_ut<true>(cfg, cp, qc, tc, ld3(means, gid), ld4q(quats, gid), ld3(scales, gid), opacities != nullptr,
                                opacities != nullptr ? opacities[gid] : 0.f, &o);
     int2* r2 = reinterpret_cast<int2*>(radii);
     if (!ok) {
@@ -290,8 +289,11 @@ __global__ void __launch_bounds__(256) projection_ut_raw_kernel(
     cfg.cx = Ks[2];
     cfg.cy = Ks[5];
     const CamPose cp = load_cam_pose(viewmat);
+    quat qc;
+    vec3 tc;
+    shutter_pose(cp, 0.5f, &qc, &tc);
     ProjOut o;
-    const bool ok = project_ut<false>(cfg, cp, ld3(means, idx), a.quat, a.scales, true, a.opacity, &o);
+    const bool ok = project_ut<false>(cfg, cp, qc, tc, ld3(means, idx), a.quat, a.scales, true, a.opacity, &o);
     int2* r2 = reinterpret_cast<int2*>(radii);
     if (!ok) {
         r2[idx] = make_int2(0, 0);
@@ -615,6 +617,13 @@ __global__ void __launch_bounds__(256) sh_records_kernel(uint32_t N, uint32_t K,
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     float4* wave_lds = lds + (LDS16 ? wave * 64 * kShLdsF4 : 0);
     const bool live = e < N && radii[e * 2] > 0 && radii[e * 2 + 1] > 0;
+    // everything the record needs is requested now, together with the coefficient rows below: one memory round
+    // trip instead of one per phase (the 44 bytes are read for Gaussians without a tile too)
+    const uint32_t ec = min(e, N - 1);
+    const vec3 mean = ld3(means, ec);
+    const float opac = opacities[ec];
+    const quat q_in = ld4q(quats, ec);
+    const vec3 scl = ld3(scales, ec);
     if (LDS16) {
         const uint32_t row0 = blockIdx.x * 256u + wave * 64u;
         const uint64_t live_rows = __builtin_amdgcn_ballot_w64(live);
@@ -634,7 +643,6 @@ __global__ void __launch_bounds__(256) sh_records_kernel(uint32_t N, uint32_t K,
     if (e >= N)
         return;
     float c[3] = {0.f, 0.f, 0.f};
-    const vec3 mean = ld3(means, e);
     if (live) {
         const vec3 dir = sub(mean, campos_from_viewmat(viewmat));
         float B[25];
@@ -664,8 +672,7 @@ __global__ void __launch_bounds__(256) sh_records_kernel(uint32_t N, uint32_t K,
     if (!live)
         return; // no tile lists this Gaussian: its record is never read
     const vec3 ray_o = camera_ray_origin(load_cam_pose(viewmat));
-    const float opac = opacities[e];
-    const mat3 M = record_whitening(ld4q(quats, e), ld3(scales, e));
+    const mat3 M = record_whitening(q_in, scl);
     const vec3 gro = mul(M, sub(ray_o, mean));
     const RecordRegion reg = record_region(gro, M, opac, mean, viewmat, Kmat[0], Kmat[4], Kmat[2], Kmat[5], W, H);
     store_record(records + (size_t)e * kRecordF4, gro, opac, M, c[0], c[1], c[2], reg);
@@ -705,6 +712,19 @@ using namespace gsx;
 // C ABI
 // =============================================================================================
 
+// Cameras.cuh:1070-1119: lambda = alpha^2 (D + kappa) - D, spread sqrt(D + lambda), weights; D = 3
+static void set_ut_constants(ProjCfg& cfg, const gsx_ut_params& ut) {
+    cfg.ut_alpha = ut.alpha, cfg.ut_beta = ut.beta, cfg.ut_kappa = ut.kappa;
+    cfg.ut_margin = ut.in_image_margin_factor;
+    cfg.ut_require_all = ut.require_all_sigma_points_valid;
+    const float D = 3.0f;
+    const float lambda = cfg.ut_alpha * cfg.ut_alpha * (D + cfg.ut_kappa) - D;
+    cfg.ut_sq = gsx::sqrt(D + lambda);
+    cfg.ut_w0m = lambda / (D + lambda);
+    cfg.ut_w0c = lambda / (D + lambda) + (1.f - cfg.ut_alpha * cfg.ut_alpha + cfg.ut_beta);
+    cfg.ut_wi = 1.f / (2.f * (D + lambda));
+}
+
 extern "C" int gsx_projection_ut_3dgs_fused(
     uint32_t C, uint32_t N, const float* means, const float* quats, const float* scales, const float* opacities,
     const float* viewmats0, const float* viewmats1, const float* Ks, uint32_t image_width, uint32_t image_height,
@@ -727,11 +747,7 @@ extern "C" int gsx_projection_ut_3dgs_fused(
     cfg.near_plane = near_plane;
     cfg.far_plane = far_plane;
     cfg.radius_clip = radius_clip;
-    cfg.ut_alpha = ut.alpha;
-    cfg.ut_beta = ut.beta;
-    cfg.ut_kappa = ut.kappa;
-    cfg.ut_margin = ut.in_image_margin_factor;
-    cfg.ut_require_all = ut.require_all_sigma_points_valid;
+    set_ut_constants(cfg, ut);
     cfg.fx = cfg.fy = cfg.cx = cfg.cy = 0.f;
     memset(&cfg.cam, 0, sizeof(cfg.cam));
     hipLaunchKernelGGL(projection_ut_kernel, dim3(cdiv((uint64_t)C * N, 256)), dim3(256), 0, (hipStream_t)stream, C,
@@ -759,9 +775,7 @@ extern "C" int gsx_activate_project_ut(uint32_t N, const float* means, const flo
     memset(&cfg, 0, sizeof(cfg));
     cfg.W = image_width, cfg.H = image_height;
     cfg.eps2d = eps2d, cfg.near_plane = near_plane, cfg.far_plane = far_plane, cfg.radius_clip = radius_clip;
-    cfg.ut_alpha = ut.alpha, cfg.ut_beta = ut.beta, cfg.ut_kappa = ut.kappa;
-    cfg.ut_margin = ut.in_image_margin_factor;
-    cfg.ut_require_all = ut.require_all_sigma_points_valid;
+    set_ut_constants(cfg, ut);
     hipLaunchKernelGGL(projection_ut_raw_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, means,
                        opacity_raw, scaling_raw, rotation_raw, viewmat, K, cfg, opacities, scales, quats, radii,
                        means2d, depths, conics);
