@@ -42,6 +42,35 @@ inline gsx_ut_params to_gsx(const UnscentedTransformParameters& p) {
     return u;
 }
 
+// The kernels index by these extents: a tensor of another shape would be read or written out of bounds.
+// -1 leaves an extent free.
+inline void sized(const at::Tensor& t, const char* name, std::initializer_list<int64_t> shape) {
+    bool ok = t.dim() == (int64_t)shape.size();
+    int64_t i = 0;
+    for (const int64_t want : shape) {
+        ok = ok && (want < 0 || t.size(i) == want);
+        ++i;
+    }
+    TORCH_CHECK(ok, name, " must be ", c10::IntArrayRef(shape.begin(), shape.size()), " (-1 = any), got ", t.sizes());
+}
+inline void sized(const OptT& t, const char* name, std::initializer_list<int64_t> shape) {
+    if (has(t))
+        sized(t.value(), name, shape);
+}
+
+// [C,4,4] poses, [C,3,3] intrinsics; coefficient rows as the kernels read them (ProjectionUT3DGSFused.cu:101-126):
+// radial [C,6] (pinhole) or [C,4] (fisheye), tangential [C,2], thin prism [C,4]
+inline void check_camera_tensors(int64_t C, gsplat::CameraModelType camera_model, const at::Tensor& viewmats0,
+                                 const OptT& viewmats1, const at::Tensor& Ks, const OptT& radial_coeffs,
+                                 const OptT& tangential_coeffs, const OptT& thin_prism_coeffs) {
+    sized(viewmats0, "viewmats0", {C, 4, 4});
+    sized(viewmats1, "viewmats1", {C, 4, 4});
+    sized(Ks, "Ks", {C, 3, 3});
+    sized(radial_coeffs, "radial_coeffs", {C, camera_model == gsplat::FISHEYE ? 4 : 6});
+    sized(tangential_coeffs, "tangential_coeffs", {C, 2});
+    sized(thin_prism_coeffs, "thin_prism_coeffs", {C, 4});
+}
+
 inline at::Tensor workspace(size_t bytes, const at::Tensor& like) {
     return at::empty({(int64_t)(bytes < 256 ? 256 : bytes)}, like.options().dtype(at::kByte));
 }
@@ -197,6 +226,7 @@ at::Tensor quats_to_rotmats(const at::Tensor quats) {
     DEVICE_GUARD(quats);
     CHECK_INPUT(quats);
     const int64_t N = quats.size(0);
+    sized(quats, "quats", {N, 4});
     at::Tensor rotmats = at::empty({N, 3, 3}, quats.options());
     gsx_check(gsx_quats_to_rotmats((int)N, quats.data_ptr<float>(), rotmats.data_ptr<float>(), cur_stream(quats)));
     return rotmats;
@@ -209,6 +239,11 @@ std::tuple<at::Tensor, at::Tensor> relocation(at::Tensor opacities, at::Tensor s
     CHECK_INPUT(scales);
     CHECK_INPUT(ratios);
     CHECK_INPUT(binoms);
+    const int64_t n = opacities.size(0);
+    sized(opacities, "opacities", {n});
+    sized(scales, "scales", {n, 3});
+    sized(ratios, "ratios", {n});
+    sized(binoms, "binoms", {n_max, n_max});
     at::Tensor new_opacities = at::empty_like(opacities);
     at::Tensor new_scales = at::empty_like(scales);
     gsx_check(gsx_relocation((int)opacities.size(0), opacities.data_ptr<float>(), scales.data_ptr<float>(),
@@ -225,6 +260,12 @@ void add_noise(at::Tensor raw_opacities, at::Tensor raw_scales, at::Tensor raw_q
     CHECK_INPUT(raw_quats);
     CHECK_INPUT(noise);
     CHECK_INPUT(means);
+    const int64_t n = means.size(0);
+    sized(means, "means", {n, 3});
+    sized(noise, "noise", {n, 3});
+    sized(raw_quats, "raw_quats", {n, 4});
+    sized(raw_scales, "raw_scales", {n, 3});
+    TORCH_CHECK(raw_opacities.numel() == n, "raw_opacities must hold ", n, " values, got ", raw_opacities.sizes());
     gsx_check(gsx_add_noise((int)raw_opacities.size(0), raw_opacities.data_ptr<float>(), raw_scales.data_ptr<float>(),
                             raw_quats.data_ptr<float>(), noise.data_ptr<float>(), means.data_ptr<float>(), current_lr,
                             cur_stream(means)));
@@ -259,6 +300,12 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> projectio
         CHECK_INPUT(thin_prism_coeffs.value());
     }
     const uint32_t N = (uint32_t)means.size(0), C = (uint32_t)viewmats0.size(0);
+    sized(means, "means", {N, 3});
+    sized(quats, "quats", {N, 4});
+    sized(scales, "scales", {N, 3});
+    sized(opacities, "opacities", {N});
+    check_camera_tensors(C, camera_model, viewmats0, viewmats1, Ks, radial_coeffs, tangential_coeffs,
+                         thin_prism_coeffs);
     auto opt = means.options();
     at::Tensor radii = at::empty({C, N, 2}, opt.dtype(at::kInt));
     at::Tensor means2d = at::empty({C, N, 2}, opt);
@@ -303,6 +350,17 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> rasterize_to_pixels_from_world_3d
     TORCH_CHECK(!has(backgrounds) || (backgrounds->dim() == 2 && backgrounds->size(0) == C &&
                                       backgrounds->size(1) == channels),
                 "backgrounds must be [C, channels] = [", C, ", ", channels, "], got ", backgrounds->sizes());
+    const int64_t th = tile_size ? (image_height + tile_size - 1) / tile_size : 0;
+    const int64_t tw = tile_size ? (image_width + tile_size - 1) / tile_size : 0;
+    sized(means, "means", {N, 3});
+    sized(quats, "quats", {N, 4});
+    sized(scales, "scales", {N, 3});
+    sized(colors, "colors", {C, N, channels});
+    sized(opacities, "opacities", {C, N});
+    sized(tile_offsets, "tile_offsets", {C, th, tw});
+    sized(masks, "masks", {C, th, tw});
+    check_camera_tensors(C, camera_model, viewmats0, viewmats1, Ks, radial_coeffs, tangential_coeffs,
+                         thin_prism_coeffs);
     auto opt = means.options();
     at::Tensor renders = at::empty({C, image_height, image_width, channels}, opt);
     at::Tensor alphas = at::empty({C, image_height, image_width, 1}, opt);
@@ -354,6 +412,21 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> rasterize
                 "backgrounds must be [C, channels] = [", tile_offsets.size(0), ", ", channels, "], got ",
                 backgrounds->sizes());
     const uint32_t C = (uint32_t)tile_offsets.size(0), N = (uint32_t)means.size(0);
+    const int64_t th = tile_size ? (image_height + tile_size - 1) / tile_size : 0;
+    const int64_t tw = tile_size ? (image_width + tile_size - 1) / tile_size : 0;
+    sized(means, "means", {N, 3});
+    sized(quats, "quats", {N, 4});
+    sized(scales, "scales", {N, 3});
+    sized(colors, "colors", {C, N, channels});
+    sized(opacities, "opacities", {C, N});
+    sized(tile_offsets, "tile_offsets", {C, th, tw});
+    sized(masks, "masks", {C, th, tw});
+    sized(render_alphas, "render_alphas", {C, image_height, image_width, 1});
+    sized(last_ids, "last_ids", {C, image_height, image_width});
+    sized(v_render_colors, "v_render_colors", {C, image_height, image_width, channels});
+    sized(v_render_alphas, "v_render_alphas", {C, image_height, image_width, 1});
+    check_camera_tensors(C, camera_model, viewmats0, viewmats1, Ks, radial_coeffs, tangential_coeffs,
+                         thin_prism_coeffs);
     // the kernels write every element of the five outputs (the reference zero-fills, Rasterization.cpp:190-194)
     at::Tensor v_means = at::empty_like(means), v_quats = at::empty_like(quats), v_scales = at::empty_like(scales);
     at::Tensor v_colors = at::empty_like(colors), v_opacities = at::empty_like(opacities);

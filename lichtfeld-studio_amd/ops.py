@@ -47,6 +47,25 @@ def _f32(x, name):
     return x
 
 
+def _sized(x, name, *shape):
+    """The kernels index by these extents: a tensor of another shape would be read or written out of bounds.  None
+    in `shape` leaves that extent free; a None tensor passes."""
+    if x is None:
+        return
+    if x.dim() != len(shape) or any(s is not None and int(d) != int(s) for d, s in zip(x.shape, shape)):
+        want = ", ".join("*" if s is None else str(int(s)) for s in shape)
+        raise RuntimeError(f"{name} must be [{want}], got {tuple(x.shape)}")
+
+
+def _check_camera_tensors(C, camera_model, viewmats0, viewmats1, Ks, radial_coeffs, tangential_coeffs,
+                          thin_prism_coeffs):
+    """[C,4,4] poses, [C,3,3] intrinsics; coefficient rows as the kernels read them (ProjectionUT3DGSFused.cu:101-
+    126): radial [C,6] (pinhole) or [C,4] (fisheye), tangential [C,2], thin prism [C,4]"""
+    _sized(viewmats0, "viewmats0", C, 4, 4), _sized(viewmats1, "viewmats1", C, 4, 4), _sized(Ks, "Ks", C, 3, 3)
+    _sized(radial_coeffs, "radial_coeffs", C, 4 if camera_model == CameraModelType.FISHEYE else 6)
+    _sized(tangential_coeffs, "tangential_coeffs", C, 2), _sized(thin_prism_coeffs, "thin_prism_coeffs", C, 4)
+
+
 # ------------------------------------------------------------------------------------------------
 def spherical_harmonics_fwd(degrees_to_use, dirs, coeffs, masks=None):
     """Ops.h:12-17"""
@@ -59,6 +78,9 @@ def spherical_harmonics_fwd(degrees_to_use, dirs, coeffs, masks=None):
         raise RuntimeError("dirs must have last dimension 3")
     K = coeffs.size(-2)
     N = dirs.numel() // 3
+    if coeffs.numel() != N * K * 3 or (masks is not None and masks.numel() != N):
+        raise RuntimeError(f"coeffs must be [..., K, 3] and masks [...] over the {N} directions, got "
+                           f"{tuple(coeffs.shape)}" + ("" if masks is None else f" / {tuple(masks.shape)}"))
     colors = torch.empty_like(dirs)
     m8 = None if masks is None else masks.view(torch.uint8) if masks.dtype == torch.bool else masks
     with torch.cuda.device(dirs.device):
@@ -75,6 +97,9 @@ def spherical_harmonics_bwd(K, degrees_to_use, dirs, coeffs, masks, v_colors, co
     if v_colors.size(-1) != 3 or coeffs.size(-1) != 3 or dirs.size(-1) != 3:
         raise RuntimeError("last dimension must be 3")
     N = dirs.numel() // 3
+    if coeffs.size(-2) != K or coeffs.numel() != N * K * 3 or v_colors.numel() != N * 3 or \
+            (masks is not None and masks.numel() != N):
+        raise RuntimeError(f"coeffs must be [..., {K}, 3], v_colors [..., 3] and masks [...] over the {N} directions")
     v_coeffs = torch.empty_like(coeffs)
     v_dirs = torch.empty_like(dirs) if compute_v_dirs else None
     m8 = None if masks is None else masks.view(torch.uint8) if masks.dtype == torch.bool else masks
@@ -97,6 +122,7 @@ def intersect_tile(means2d, radii, depths, camera_ids, gaussian_ids, C, tile_siz
         raise RuntimeError("radii must be int32")
     dev = means2d.device
     N = means2d.size(1)
+    _sized(means2d, "means2d", C, N, 2), _sized(radii, "radii", C, N, 2), _sized(depths, "depths", C, N)
     tiles_per_gauss = torch.empty_like(depths, dtype=torch.int32)
     n_isects = c_i64(0)
     # sort == True with one camera: depth order first, then a sort on the tile bits only (same result as the
@@ -141,6 +167,9 @@ def radix_sort_double_buffer(n_isects, tile_n_bits, cam_n_bits, isect_ids, flatt
     _check_input(isect_ids, "isect_ids"), _check_input(flatten_ids, "flatten_ids")
     if n_isects <= 0:
         return isect_ids, flatten_ids
+    if isect_ids.dtype != torch.int64 or flatten_ids.dtype != torch.int32 or isect_ids.numel() < n_isects or \
+            flatten_ids.numel() < n_isects:
+        raise RuntimeError(f"isect_ids (int64) and flatten_ids (int32) must hold {n_isects} entries")
     dev = isect_ids.device
     with torch.cuda.device(dev):
         k1, v1 = torch.empty_like(isect_ids), torch.empty_like(flatten_ids)
@@ -156,6 +185,8 @@ def radix_sort_double_buffer(n_isects, tile_n_bits, cam_n_bits, isect_ids, flatt
 def intersect_offset(isect_ids, C, tile_width, tile_height):
     """Ops.h:39-43 -> offsets [C, tile_height, tile_width] i32"""
     _check_input(isect_ids, "isect_ids")
+    if isect_ids.dtype != torch.int64:
+        raise RuntimeError("isect_ids must be int64")
     dev = isect_ids.device
     offsets = torch.empty((C, tile_height, tile_width), dtype=torch.int32, device=dev)
     with torch.cuda.device(dev):
@@ -168,6 +199,7 @@ def quats_to_rotmats(quats):
     """Ops.h:46-48"""
     _f32(quats, "quats")
     N = quats.size(0)
+    _sized(quats, "quats", N, 4)
     out = torch.empty((N, 3, 3), dtype=quats.dtype, device=quats.device)
     with torch.cuda.device(quats.device):
         check(lib().gsx_quats_to_rotmats(c_i(N), _ptr(quats), _ptr(out), _stream(quats.device)))
@@ -179,6 +211,9 @@ def relocation(opacities, scales, ratios, binoms, n_max):
     _f32(opacities, "opacities"), _f32(scales, "scales"), _check_input(ratios, "ratios"), _f32(binoms, "binoms")
     if ratios.dtype != torch.int32:
         raise RuntimeError("ratios must be int32")
+    n = opacities.size(0)
+    _sized(opacities, "opacities", n), _sized(scales, "scales", n, 3), _sized(ratios, "ratios", n)
+    _sized(binoms, "binoms", n_max, n_max)
     new_opacities, new_scales = torch.empty_like(opacities), torch.empty_like(scales)
     with torch.cuda.device(opacities.device):
         check(lib().gsx_relocation(c_i(opacities.size(0)), _ptr(opacities), _ptr(scales), _ptr(ratios), _ptr(binoms),
@@ -191,6 +226,11 @@ def add_noise(raw_opacities, raw_scales, raw_quats, noise, means, current_lr):
     for t, n in ((raw_opacities, "raw_opacities"), (raw_scales, "raw_scales"), (raw_quats, "raw_quats"),
                  (noise, "noise"), (means, "means")):
         _f32(t, n)
+    n = means.size(0)
+    _sized(means, "means", n, 3), _sized(noise, "noise", n, 3), _sized(raw_quats, "raw_quats", n, 4)
+    _sized(raw_scales, "raw_scales", n, 3)
+    if raw_opacities.numel() != n:
+        raise RuntimeError(f"raw_opacities must hold {n} values, got {tuple(raw_opacities.shape)}")
     with torch.cuda.device(means.device):
         check(lib().gsx_add_noise(c_i(means.size(0)), _ptr(raw_opacities), _ptr(raw_scales), _ptr(raw_quats),
                                   _ptr(noise), _ptr(means), c_f(current_lr), _stream(means.device)))
@@ -211,6 +251,10 @@ def projection_ut_3dgs_fused(means, quats, scales, opacities, viewmats0, viewmat
             _f32(t, n)
     dev = means.device
     N, C = means.size(0), viewmats0.size(0)
+    _sized(means, "means", N, 3), _sized(quats, "quats", N, 4), _sized(scales, "scales", N, 3)
+    _sized(opacities, "opacities", N)
+    _check_camera_tensors(C, camera_model, viewmats0, viewmats1, Ks, radial_coeffs, tangential_coeffs,
+                          thin_prism_coeffs)
     radii = torch.empty((C, N, 2), dtype=torch.int32, device=dev)
     means2d = torch.empty((C, N, 2), dtype=torch.float32, device=dev)
     depths = torch.empty((C, N), dtype=torch.float32, device=dev)
@@ -267,6 +311,14 @@ def rasterize_to_pixels_from_world_3dgs_fwd(means, quats, scales, colors, opacit
     C, N = tile_offsets.size(0), means.size(0)
     channels = colors.size(-1)
     _check_backgrounds(backgrounds, C, channels)
+    th, tw = (image_height + tile_size - 1) // tile_size, (image_width + tile_size - 1) // tile_size
+    _sized(means, "means", N, 3), _sized(quats, "quats", N, 4), _sized(scales, "scales", N, 3)
+    _sized(colors, "colors", C, N, channels), _sized(opacities, "opacities", C, N)
+    _sized(tile_offsets, "tile_offsets", C, th, tw), _sized(masks, "masks", C, th, tw)
+    _check_camera_tensors(C, camera_model, viewmats0, viewmats1, Ks, radial_coeffs, tangential_coeffs,
+                          thin_prism_coeffs)
+    if tile_offsets.dtype != torch.int32 or flatten_ids.dtype != torch.int32:
+        raise RuntimeError("tile_offsets and flatten_ids must be int32")
     renders = torch.empty((C, image_height, image_width, channels), dtype=torch.float32, device=dev)
     alphas = torch.empty((C, image_height, image_width, 1), dtype=torch.float32, device=dev)
     last_ids = torch.empty((C, image_height, image_width), dtype=torch.int32, device=dev)
@@ -301,7 +353,20 @@ def rasterize_to_pixels_from_world_3dgs_bwd(means, quats, scales, colors, opacit
         backgrounds = None
     dev = means.device
     C, N = tile_offsets.size(0), means.size(0)
-    _check_backgrounds(backgrounds, C, colors.size(-1))
+    channels = colors.size(-1)
+    _check_backgrounds(backgrounds, C, channels)
+    th, tw = (image_height + tile_size - 1) // tile_size, (image_width + tile_size - 1) // tile_size
+    _sized(means, "means", N, 3), _sized(quats, "quats", N, 4), _sized(scales, "scales", N, 3)
+    _sized(colors, "colors", C, N, channels), _sized(opacities, "opacities", C, N)
+    _sized(tile_offsets, "tile_offsets", C, th, tw), _sized(masks, "masks", C, th, tw)
+    _sized(render_alphas, "render_alphas", C, image_height, image_width, 1)
+    _sized(last_ids, "last_ids", C, image_height, image_width)
+    _sized(v_render_colors, "v_render_colors", C, image_height, image_width, channels)
+    _sized(v_render_alphas, "v_render_alphas", C, image_height, image_width, 1)
+    _check_camera_tensors(C, camera_model, viewmats0, viewmats1, Ks, radial_coeffs, tangential_coeffs,
+                          thin_prism_coeffs)
+    if tile_offsets.dtype != torch.int32 or flatten_ids.dtype != torch.int32 or last_ids.dtype != torch.int32:
+        raise RuntimeError("tile_offsets, flatten_ids and last_ids must be int32")
     v_means, v_quats, v_scales = torch.empty_like(means), torch.empty_like(quats), torch.empty_like(scales)
     v_colors, v_opacities = torch.empty_like(colors), torch.empty_like(opacities)
     m8 = None if masks is None else masks.view(torch.uint8) if masks.dtype == torch.bool else masks
@@ -340,6 +405,7 @@ def rasterize_from_world_with_sh_fwd(means, quats, scales, opacities, sh_coeffs,
         means, quats, scaled_scales, opacities, viewmats0, viewmats1, Ks, image_width, image_height, eps2d,
         near_plane, far_plane, radius_clip, calc_compensations, camera_model, ut_params, rs_type, radial_coeffs,
         tangential_coeffs, thin_prism_coeffs)
+    _sized(sh_coeffs, "sh_coeffs", N, None, 3)
     K = sh_coeffs.size(1)
     if render_mode in (0, 3, 4):
         colors = torch.empty((C, N, 3), dtype=torch.float32, device=dev)
@@ -359,8 +425,8 @@ def rasterize_from_world_with_sh_fwd(means, quats, scales, opacities, sh_coeffs,
                                                tile_height, True)
     offsets = intersect_offset(isect_ids, C, tile_width, tile_height)
     renders, alphas, last_ids = rasterize_to_pixels_from_world_3dgs_fwd(
-        means, quats, scaled_scales, colors, final_opacities, _fit_backgrounds(backgrounds, colors.size(-1)), masks, image_width, image_height,
-        tile_size, viewmats0, viewmats1, Ks, camera_model, ut_params, rs_type, radial_coeffs, tangential_coeffs,
+        means, quats, scaled_scales, colors, final_opacities, _fit_backgrounds(backgrounds, colors.size(-1)), masks,
+        image_width, image_height, tile_size, viewmats0, viewmats1, Ks, camera_model, ut_params, rs_type, radial_coeffs, tangential_coeffs,
         thin_prism_coeffs, offsets, flatten_ids)
     out = (renders, alphas, radii, means2d, depths, colors, offsets, flatten_ids, last_ids, comp)
     return out + (isect_ids,) if return_isect_ids else out
@@ -386,9 +452,10 @@ def rasterize_from_world_with_sh_bwd(means, quats, scales, opacities, sh_coeffs,
         final_opacities = (final_opacities * compensations).contiguous()
     scaled_scales = scales if scaling_modifier == 1.0 else scales * scaling_modifier
     v_means, v_quats, v_scales, v_colors, v_opacities = rasterize_to_pixels_from_world_3dgs_bwd(
-        means, quats, scaled_scales, colors, final_opacities, _fit_backgrounds(backgrounds, colors.size(-1)), masks, image_width, image_height,
-        tile_size, viewmats0, viewmats1, Ks, camera_model, ut_params, rs_type, radial_coeffs, tangential_coeffs,
+        means, quats, scaled_scales, colors, final_opacities, _fit_backgrounds(backgrounds, colors.size(-1)), masks,
+        image_width, image_height, tile_size, viewmats0, viewmats1, Ks, camera_model, ut_params, rs_type, radial_coeffs, tangential_coeffs,
         thin_prism_coeffs, tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors, v_render_alphas)
+    _sized(sh_coeffs, "sh_coeffs", N, None, 3), _sized(radii, "radii", 1, N, 2)
     K = sh_coeffs.size(1)
     if render_mode in (0, 3, 4):
         rgb, v_rgb = colors, v_colors
@@ -410,6 +477,9 @@ def rasterize_from_world_with_sh_bwd(means, quats, scales, opacities, sh_coeffs,
 def fusedssim(C1, C2, img1, img2, train):
     """include/kernels/ssim.cuh:11-19 -> (ssim_map, dm_dmu1, dm_dsigma1_sq, dm_dsigma12)"""
     _f32(img1, "img1"), _f32(img2, "img2")
+    if img1.dim() != 4 or img1.shape != img2.shape:
+        raise RuntimeError(f"img1 and img2 must be [B, C, H, W] of one shape, got {tuple(img1.shape)} / "
+                           f"{tuple(img2.shape)}")
     B, CH, H, W = img1.shape
     ssim_map = torch.empty_like(img1)
     if train:
@@ -428,6 +498,8 @@ def fusedssim_backward(C1, C2, img1, img2, dL_dmap, dm_dmu1, dm_dsigma1_sq, dm_d
     for t, n in ((img1, "img1"), (img2, "img2"), (dL_dmap, "dL_dmap"), (dm_dmu1, "dm_dmu1"),
                  (dm_dsigma1_sq, "dm_dsigma1_sq"), (dm_dsigma12, "dm_dsigma12")):
         _f32(t, n)
+        if t.shape != img1.shape or t.dim() != 4:
+            raise RuntimeError(f"{n} must be [B, C, H, W] like img1 {tuple(img1.shape)}, got {tuple(t.shape)}")
     B, CH, H, W = img1.shape
     out = torch.empty_like(img1)
     with torch.cuda.device(img1.device):
@@ -442,6 +514,8 @@ def adam_step(param, exp_avg, exp_avg_sq, param_grad, lr, beta1, beta2, eps, bia
     """fast_gs::optimizer::adam_step_wrapper (fastgs/optimizer/src/adam_api.cu:8-33); in place"""
     for t, n in ((param, "param"), (exp_avg, "exp_avg"), (exp_avg_sq, "exp_avg_sq"), (param_grad, "param_grad")):
         _f32(t, n)
+        if t.numel() != param.numel():
+            raise RuntimeError(f"{n} must hold {param.numel()} elements like param, got {t.numel()}")
     with torch.cuda.device(param.device):
         check(lib().gsx_adam_step(_ptr(param), _ptr(exp_avg), _ptr(exp_avg_sq), _ptr(param_grad),
                                   c_i64(param.numel()), c_f(lr), c_f(beta1), c_f(beta2), c_f(eps),
@@ -463,6 +537,9 @@ def adam_step_multi(groups):
         grad = g.get("param_grad")
         if grad is not None:
             _f32(grad, "param_grad")
+        for n, t in (("exp_avg", g["exp_avg"]), ("exp_avg_sq", g["exp_avg_sq"]), ("param_grad", grad)):
+            if t is not None and t.numel() != p.numel():
+                raise RuntimeError(f"group {i}: {n} must hold {p.numel()} elements like param, got {t.numel()}")
         arr[i] = L.AdamGroup(p.data_ptr(), g["exp_avg"].data_ptr(), g["exp_avg_sq"].data_ptr(),
                              None if grad is None else grad.data_ptr(), p.numel(), g["lr"], g["beta1"], g["beta2"],
                              g["eps"], g["bias_correction1_rcp"], g["bias_correction2_sqrt_rcp"])

@@ -38,8 +38,9 @@ def _check(cond, msg):
 
 
 def _pad(t, n, dev):
-    """rasterizer.cpp:97-120 pads the coefficient vectors with zeros; the kernel reads 6 radial / 2 tangential
-    values (ProjectionUT3DGSFused.cu:101-106), so the radial vector is padded to 6 here (the reference pads to 4)"""
+    """rasterizer.cpp:97-120 pads the coefficient vectors with zeros; the pinhole kernel reads 6 radial / 2 tangential
+    values (ProjectionUT3DGSFused.cu:101-106), the fisheye one 4 radial (:124), so the radial vector is padded to 6
+    or 4 here (the reference always pads to 4)"""
     if t is None or t.numel() == 0:
         return None
     _check(t.dim() == 1, f"distortion coefficients must be 1D, got {tuple(t.shape)}")
@@ -87,7 +88,8 @@ def rasterize(viewmat, K, image_width, image_height, means3D, opacities, scales,
         means3D.contiguous(), rotations.contiguous(), scales.contiguous(), opacities.contiguous(),
         sh_coeffs.contiguous(), sh_degree, bg, None, image_width, image_height, 16, viewmat.contiguous(), None,
         K.contiguous(), int(camera_model), 0.3, 0.01, 10000.0, 0.0, float(scaling_modifier), bool(antialiased),
-        int(mode), ops.UnscentedTransformParameters(), 4, _pad(radial_distortion, 6, dev),
+        int(mode), ops.UnscentedTransformParameters(), 4,
+        _pad(radial_distortion, 4 if int(camera_model) == ops.CameraModelType.FISHEYE else 6, dev),
         _pad(tangential_distortion, 2, dev), None)
     rendered, alpha, radii, means2d, depths = out[0], out[1], out[2], out[3], out[4]
     image = depth = None

@@ -172,3 +172,11 @@ def test_cpp_errors_on_device(gsx, cpp, cuda):
                                      cpp.ShutterType.GLOBAL, None, None, None)
     with pytest.raises(RuntimeError, match="contiguous"):
         cpp.quats_to_rotmats(d["quats"].t().contiguous().t())
+    with pytest.raises(RuntimeError, match="radial_coeffs must be"):  # the pinhole model reads six per camera
+        cpp.projection_ut_3dgs_fused(d["means"], d["quats"], d["scales"], d["op"], d["vm"], None, d["K"], cam.width,
+                                     cam.height, 0.3, 0.01, 1e4, 0.0, False, cpp.CameraModelType.PINHOLE, ut,
+                                     cpp.ShutterType.GLOBAL, torch.zeros((1, 4), device=cuda), None, None)
+    with pytest.raises(RuntimeError, match="scales must be"):
+        cpp.projection_ut_3dgs_fused(d["means"], d["quats"], d["scales"][:100].contiguous(), d["op"], d["vm"], None,
+                                     d["K"], cam.width, cam.height, 0.3, 0.01, 1e4, 0.0, False,
+                                     cpp.CameraModelType.PINHOLE, ut, cpp.ShutterType.GLOBAL, None, None, None)

@@ -113,6 +113,17 @@ def test_projection_unsupported_and_errors(gsx, cuda):
         ops.projection_ut_3dgs_fused(*args, 1, ops.UnscentedTransformParameters(), 4)
     with pytest.raises(gsx._lib.GsxError):  # not a shutter type
         ops.projection_ut_3dgs_fused(*args, 0, ops.UnscentedTransformParameters(), 5)
+    # extents the kernels index by: four radial coefficients are a fisheye row, the pinhole model reads six
+    four = torch.zeros((1, 4), device=cuda)
+    with pytest.raises(RuntimeError, match=r"radial_coeffs must be \[1, 6\]"):
+        ops.projection_ut_3dgs_fused(*args, 0, ops.UnscentedTransformParameters(), 4, four)
+    ops.projection_ut_3dgs_fused(*args, 2, ops.UnscentedTransformParameters(), 4, four)
+    with pytest.raises(RuntimeError, match=r"quats must be \[100, 4\]"):
+        ops.projection_ut_3dgs_fused(args[0], args[1][:50].contiguous(), *args[2:], 0,
+                                     ops.UnscentedTransformParameters(), 4)
+    with pytest.raises(RuntimeError, match=r"viewmats1 must be \[1, 4, 4\]"):
+        ops.projection_ut_3dgs_fused(*args[:5], torch.eye(4, device=cuda), *args[6:], 0,
+                                     ops.UnscentedTransformParameters(), 0)
     with pytest.raises(RuntimeError):  # CHECK_INPUT: CPU tensor
         ops.projection_ut_3dgs_fused(torch.from_numpy(means), *args[1:], 0, ops.UnscentedTransformParameters(), 4)
     with pytest.raises(RuntimeError):  # CHECK_INPUT: non-contiguous
@@ -367,6 +378,12 @@ def test_raster_masks_and_channels(gsx, orc, cuda):
                                                     torch.zeros((1, 4000, 5), device=cuda), T(h["op"][None], cuda),
                                                     None, None, cam.width, cam.height, 16, d["vm"], None, d["K"], 0,
                                                     ut, 4, None, None, None, T(off, cuda), T(flat, cuda))
+    with pytest.raises(RuntimeError, match=r"tile_offsets must be \[1, "):  # ranges of another tile grid
+        ops.rasterize_to_pixels_from_world_3dgs_fwd(d["means"], d["quats"], d["scales"],
+                                                    torch.zeros((1, 4000, 3), device=cuda), T(h["op"][None], cuda),
+                                                    None, None, cam.width, cam.height, 16, d["vm"], None, d["K"], 0,
+                                                    ut, 4, None, None, None, T(off[:, :-1].copy(), cuda),
+                                                    T(flat, cuda))
     with pytest.raises(RuntimeError, match=r"backgrounds must be \[C, channels\]"):  # a [1,3] row under 4 channels
         ops.rasterize_to_pixels_from_world_3dgs_fwd(d["means"], d["quats"], d["scales"],
                                                     torch.zeros((1, 4000, 4), device=cuda), T(h["op"][None], cuda),
