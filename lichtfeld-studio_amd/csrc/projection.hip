@@ -612,10 +612,12 @@ __global__ void __launch_bounds__(256) sh_records_kernel(uint32_t N, uint32_t K,
                                                           const float* __restrict__ viewmat,
                                                           const float* __restrict__ Kmat, uint32_t W, uint32_t H,
                                                           float* __restrict__ colors, float4* __restrict__ records) {
-    __shared__ float4 lds[LDS16 ? 4 * 64 * kShLdsF4 : 1];
+    // a wave stages its 64 coefficient rows 32 at a time: half the LDS per wave, more waves per CU to cover the
+    // memory round trips of this latency-bound pass
+    __shared__ float4 lds[LDS16 ? 4 * 32 * kShLdsF4 : 1];
     const uint32_t e = blockIdx.x * 256u + threadIdx.x;
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    float4* wave_lds = lds + (LDS16 ? wave * 64 * kShLdsF4 : 0);
+    float4* wave_lds = lds + (LDS16 ? wave * 32 * kShLdsF4 : 0);
     const bool live = e < N && radii[e * 2] > 0 && radii[e * 2 + 1] > 0;
     // everything the record needs is requested now, together with the coefficient rows below: one memory round
     // trip instead of one per phase (the 44 bytes are read for Gaussians without a tile too)
@@ -624,21 +626,44 @@ __global__ void __launch_bounds__(256) sh_records_kernel(uint32_t N, uint32_t K,
     const float opac = opacities[ec];
     const quat q_in = ld4q(quats, ec);
     const vec3 scl = ld3(scales, ec);
+    float co_reg[48];
     if (LDS16) {
         const uint32_t row0 = blockIdx.x * 256u + wave * 64u;
         const uint64_t live_rows = __builtin_amdgcn_ballot_w64(live);
         if (row0 < N && live_rows) {
             const float4* src = reinterpret_cast<const float4*>(coeffs + (size_t)row0 * 48);
             const uint32_t n_f4 = min(64u, N - row0) * kShRowF4;
+            float4 tmp[kShRowF4]; // all twelve requests leave before the first is needed
 #pragma unroll
             for (uint32_t i = 0; i < kShRowF4; ++i) {
                 const uint32_t q = i * 64u + lane;
                 const uint32_t r = (q * 43691u) >> 19; // q / 12 for q < 768
+                tmp[i] = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (q < n_f4 && ((live_rows >> r) & 1ull))
-                    wave_lds[r * kShLdsF4 + (q - r * kShRowF4)] = src[q];
+                    tmp[i] = src[q];
+            }
+#pragma unroll
+            for (uint32_t half = 0; half < 2; ++half) {
+#pragma unroll
+                for (uint32_t i = 0; i < kShRowF4 / 2; ++i) {
+                    const uint32_t q = i * 64u + lane;     // position inside this half's 32 rows
+                    const uint32_t r = (q * 43691u) >> 19; // q / 12
+                    wave_lds[r * kShLdsF4 + (q - r * kShRowF4)] = tmp[half * (kShRowF4 / 2) + i];
+                }
+                __builtin_amdgcn_wave_barrier();
+                if ((lane >> 5) == half) {
+#pragma unroll
+                    for (uint32_t k = 0; k < kShRowF4; ++k) {
+                        const float4 t = wave_lds[(lane & 31u) * kShLdsF4 + k];
+                        co_reg[4 * k + 0] = t.x;
+                        co_reg[4 * k + 1] = t.y;
+                        co_reg[4 * k + 2] = t.z;
+                        co_reg[4 * k + 3] = t.w;
+                    }
+                }
+                __builtin_amdgcn_wave_barrier();
             }
         }
-        __builtin_amdgcn_wave_barrier();
     }
     if (e >= N)
         return;
@@ -647,21 +672,7 @@ __global__ void __launch_bounds__(256) sh_records_kernel(uint32_t N, uint32_t K,
         const vec3 dir = sub(mean, campos_from_viewmat(viewmat));
         float B[25];
         sh_basis(degree, dir, B);
-        float co_reg[48];
-        const float* co;
-        if (LDS16) {
-#pragma unroll
-            for (uint32_t j = 0; j < kShRowF4; ++j) {
-                const float4 t = wave_lds[lane * kShLdsF4 + j];
-                co_reg[4 * j + 0] = t.x;
-                co_reg[4 * j + 1] = t.y;
-                co_reg[4 * j + 2] = t.z;
-                co_reg[4 * j + 3] = t.w;
-            }
-            co = co_reg;
-        } else {
-            co = coeffs + (size_t)e * K * 3;
-        }
+        const float* co = LDS16 ? co_reg : coeffs + (size_t)e * K * 3;
 #pragma unroll
         for (uint32_t ch = 0; ch < 3; ++ch)
             c[ch] = gsx::fmax(sh_color_channel(degree, dir, B, co, ch) + 0.5f, 0.0f);
