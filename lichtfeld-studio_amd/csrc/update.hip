@@ -6,8 +6,8 @@
 // The separate kernels write 236 B of raw-parameter gradients per Gaussian and the optimiser reads them back; here
 // they stay in registers.  Arithmetic is that of the separate kernels (same device functions), so parameters and
 // moments come out bit-identical to epilogue + sh_colors_from_world_bwd + activate_params_bwd + adam_step_multi.
-// The 192-byte SH rows of the parameter and of both moments move through LDS with coalesced 16-byte accesses, one
-// tensor at a time: moment 1, moment 2 (their new values stay in registers), then the parameter.
+// The SH parameter and its two moments are updated where they lie with coalesced 16-byte accesses; the per-Gaussian
+// gradient rows reach that layout through LDS.
 #include <string.h>
 
 #include "gsx_common.h"
@@ -54,10 +54,10 @@ __device__ __forceinline__ void adam_row(float* __restrict__ P, float* __restric
 
 template <bool LDS16>
 __global__ void __launch_bounds__(256) backward_update_kernel(const UpdateArgs a) {
-    __shared__ float4 lds[LDS16 ? 4 * 64 * kShLdsF4 : 1];
+    __shared__ float4 lds[LDS16 ? 4 * 32 * kShLdsF4 : 1];
     const uint32_t e = blockIdx.x * 256u + threadIdx.x;
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    float4* wave_lds = lds + (LDS16 ? wave * 64 * kShLdsF4 : 0);
+    float4* wave_lds = lds + (LDS16 ? wave * 32 * kShLdsF4 : 0);
     const bool in = e < a.N;
 
     float B[25];
@@ -116,76 +116,81 @@ __global__ void __launch_bounds__(256) backward_update_kernel(const UpdateArgs a
     }
 
     // ---- Adam on the SH tensor; gradient of coefficient (k, c) = B[k] * vc[c] for k < nb, else 0 ----
+    // The update is elementwise, so the parameter and both moments are processed where they lie, with coalesced
+    // 16-byte accesses; only the gradient rows (one per lane) are turned into that layout through LDS, 32 rows at a
+    // time.  Position q of a half = float4 (q % 12) of row (q / 12).
     if (LDS16) {
         const uint32_t row0 = blockIdx.x * 256u + wave * 64u;
         if (row0 >= a.N)
             return; // whole wave out of range
-        float g[48];
-#pragma unroll
-        for (int k = 0; k < 16; ++k) {
-            const bool used = k < nb;
-            g[k * 3 + 0] = used ? B[k] * vc[0] : 0.f;
-            g[k * 3 + 1] = used ? B[k] * vc[1] : 0.f;
-            g[k * 3 + 2] = used ? B[k] * vc[2] : 0.f;
-        }
         const bool skip = a.skip_shN != 0;
-        float m1[48], v1[48];
-        // first moment
-        sh16_rows_to_lds(a.m_shs, row0, a.N, wave_lds, lane);
-        __builtin_amdgcn_wave_barrier();
+        const uint32_t n_f4 = min(64u, a.N - row0) * kShRowF4;
 #pragma unroll
-        for (uint32_t j = 0; j < kShRowF4; ++j) {
-            float4 t = wave_lds[lane * kShLdsF4 + j];
-            float* tv = reinterpret_cast<float*>(&t);
+        for (uint32_t half = 0; half < 2; ++half) {
+            if ((lane >> 5) == half) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int i = 4 * (int)j + q;
-                const float nm = adam_m(tv[q], g[i], a.beta1);
-                m1[i] = (i >= 3 && skip) ? tv[q] : nm;
-                tv[q] = m1[i];
+                for (uint32_t j = 0; j < kShRowF4; ++j) {
+                    float t[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int i = 4 * (int)j + q, k = i / 3, c = i - 3 * k;
+                        t[q] = k < nb ? B[k] * vc[c] : 0.f;
+                    }
+                    wave_lds[(lane & 31u) * kShLdsF4 + j] = make_float4(t[0], t[1], t[2], t[3]);
+                }
             }
-            wave_lds[lane * kShLdsF4 + j] = t;
-        }
-        __builtin_amdgcn_wave_barrier();
-        sh16_rows_from_lds(a.m_shs, row0, a.N, wave_lds, lane);
-        __builtin_amdgcn_wave_barrier();
-        // second moment
-        sh16_rows_to_lds(a.v_shs, row0, a.N, wave_lds, lane);
-        __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_wave_barrier();
+            const uint32_t base = half * 32u * kShRowF4; // first float4 of this half inside the wave's rows
+            const size_t g0 = (size_t)row0 * kShRowF4 + base;
+            float4* __restrict__ P4 = reinterpret_cast<float4*>(a.shs) + g0;
+            float4* __restrict__ M4 = reinterpret_cast<float4*>(a.m_shs) + g0;
+            float4* __restrict__ V4 = reinterpret_cast<float4*>(a.v_shs) + g0;
+            constexpr uint32_t kPer = 3; // float4 per lane and batch (two batches per half)
+#pragma unroll 1
+            for (uint32_t batch = 0; batch < 2; ++batch) {
+            float4 p4[kPer], m4[kPer], v4[kPer];
+            bool act[kPer];
 #pragma unroll
-        for (uint32_t j = 0; j < kShRowF4; ++j) {
-            float4 t = wave_lds[lane * kShLdsF4 + j];
-            float* tv = reinterpret_cast<float*>(&t);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int i = 4 * (int)j + q;
-                const float nv = adam_v(tv[q], g[i], a.beta2);
-                v1[i] = (i >= 3 && skip) ? tv[q] : nv;
-                tv[q] = v1[i];
+            for (uint32_t i = 0; i < kPer; ++i) { // the batch's requests leave before the first result is used
+                const uint32_t q = (batch * kPer + i) * 64u + lane;
+                const uint32_t col = q - ((q * 43691u) >> 19) * kShRowF4;
+                // with the higher bands frozen only the first float4 of a row (DC + one more element) is touched
+                act[i] = base + q < n_f4 && !(skip && col != 0);
+                if (act[i]) {
+                    p4[i] = P4[q];
+                    m4[i] = M4[q];
+                    v4[i] = V4[q];
+                }
             }
-            wave_lds[lane * kShLdsF4 + j] = t;
-        }
-        __builtin_amdgcn_wave_barrier();
-        sh16_rows_from_lds(a.v_shs, row0, a.N, wave_lds, lane);
-        __builtin_amdgcn_wave_barrier();
-        // parameter
-        sh16_rows_to_lds(a.shs, row0, a.N, wave_lds, lane);
-        __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (uint32_t j = 0; j < kShRowF4; ++j) {
-            float4 t = wave_lds[lane * kShLdsF4 + j];
-            float* tv = reinterpret_cast<float*>(&t);
+            for (uint32_t i = 0; i < kPer; ++i) {
+                const uint32_t q = (batch * kPer + i) * 64u + lane;
+                const uint32_t r = (q * 43691u) >> 19, col = q - r * kShRowF4;
+                if (!act[i])
+                    continue;
+                const float4 g4 = wave_lds[r * kShLdsF4 + col];
+                const float* gv = reinterpret_cast<const float*>(&g4);
+                float* pv = reinterpret_cast<float*>(&p4[i]);
+                float* mv = reinterpret_cast<float*>(&m4[i]);
+                float* vv = reinterpret_cast<float*>(&v4[i]);
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int i = 4 * (int)j + q;
-                const float np = adam_p(tv[q], m1[i], v1[i], i < 3 ? a.lr_sh0 : a.lr_shN, a.eps, a.bc1_rcp,
-                                        a.bc2_sqrt_rcp);
-                tv[q] = (i >= 3 && skip) ? tv[q] : np;
+                for (int t = 0; t < 4; ++t) {
+                    const bool dc = col == 0 && t < 3; // elements 0..2 of a row: the DC coefficient
+                    if (!dc && skip)
+                        continue;
+                    const float m1 = adam_m(mv[t], gv[t], a.beta1);
+                    const float v1 = adam_v(vv[t], gv[t], a.beta2);
+                    pv[t] = adam_p(pv[t], m1, v1, dc ? a.lr_sh0 : a.lr_shN, a.eps, a.bc1_rcp, a.bc2_sqrt_rcp);
+                    mv[t] = m1;
+                    vv[t] = v1;
+                }
+                P4[q] = p4[i];
+                M4[q] = m4[i];
+                V4[q] = v4[i];
             }
-            wave_lds[lane * kShLdsF4 + j] = t;
+            }
+            __builtin_amdgcn_wave_barrier();
         }
-        __builtin_amdgcn_wave_barrier();
-        sh16_rows_from_lds(a.shs, row0, a.N, wave_lds, lane);
         return;
     }
     if (!in)
