@@ -78,11 +78,13 @@ GSX_API int gsx_debug_wave_reduce16(uint32_t n_waves, const float* in, float* ou
 /* ---- a1: gsplat::projection_ut_3dgs_fused (Ops.h:69-98; kernel ProjectionUT3DGSFused.cu:17-210) ----
  * means [N,3] quats [N,4] (wxyz) scales [N,3] opacities [N] nullable, viewmats0 [C,4,4], Ks [C,3,3]
  * -> radii i32 [C,N,2], means2d [C,N,2], depths [C,N], conics [C,N,3], compensations [C,N] nullable.
+ * radial_coeffs [C,6] (GSX_PINHOLE) or [C,4] (GSX_FISHEYE), tangential_coeffs [C,2], thin_prism_coeffs [C,4], each
+ * nullable; rs_type: gsx_shutter_type (a rolling shutter iterates every sigma point's projection, Cameras.cuh:346-414).
  * Rows of culled Gaussians (radii 0) are left untouched in means2d/depths/conics/compensations. */
 GSX_API int gsx_projection_ut_3dgs_fused(
     uint32_t C, uint32_t N, const float* means, const float* quats, const float* scales, const float* opacities,
-    const float* viewmats0, const float* viewmats1 /*must be NULL*/, const float* Ks, uint32_t image_width,
-    uint32_t image_height, float eps2d, float near_plane, float far_plane, float radius_clip, int camera_model,
+    const float* viewmats0, const float* viewmats1 /*[C,4,4] end-of-frame pose, nullable*/, const float* Ks,
+    uint32_t image_width, uint32_t image_height, float eps2d, float near_plane, float far_plane, float radius_clip, int camera_model,
     gsx_ut_params ut, int rs_type, const float* radial_coeffs, const float* tangential_coeffs,
     const float* thin_prism_coeffs, int32_t* radii, float* means2d, float* depths, float* conics,
     float* compensations, void* stream);
@@ -175,7 +177,7 @@ GSX_API int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
     uint32_t C, uint32_t N, int64_t n_isects, const float* means, const float* quats, const float* scales,
     const float* colors, uint32_t channels, const float* opacities, const float* backgrounds, const uint8_t* masks,
     uint32_t image_width, uint32_t image_height, uint32_t tile_size, const float* viewmats0,
-    const float* viewmats1 /*must be NULL*/, const float* Ks, int camera_model, gsx_ut_params ut, int rs_type,
+    const float* viewmats1 /*[C,4,4] end-of-frame pose, nullable*/, const float* Ks, int camera_model, gsx_ut_params ut, int rs_type,
     const float* radial_coeffs, const float* tangential_coeffs, const float* thin_prism_coeffs,
     const int32_t* tile_offsets, const int32_t* flatten_ids, float* render_colors, float* render_alphas,
     int32_t* last_ids, void* workspace, size_t workspace_bytes, void* stream);
@@ -220,7 +222,7 @@ GSX_API int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
     uint32_t C, uint32_t N, int64_t n_isects, const float* means, const float* quats, const float* scales,
     const float* colors, uint32_t channels, const float* opacities, const float* backgrounds, const uint8_t* masks,
     uint32_t image_width, uint32_t image_height, uint32_t tile_size, const float* viewmats0,
-    const float* viewmats1 /*must be NULL*/, const float* Ks, int camera_model, gsx_ut_params ut, int rs_type,
+    const float* viewmats1 /*[C,4,4] end-of-frame pose, nullable*/, const float* Ks, int camera_model, gsx_ut_params ut, int rs_type,
     const float* radial_coeffs, const float* tangential_coeffs, const float* thin_prism_coeffs,
     const int32_t* tile_offsets, const int32_t* flatten_ids, const float* render_alphas, const int32_t* last_ids,
     const float* v_render_colors, const float* v_render_alphas, float* v_means, float* v_quats, float* v_scales,
