@@ -135,6 +135,15 @@ GSX_API int gsx_intersect_tile_emit_capped(uint32_t C, uint32_t N, const float* 
                                            const int32_t* order, uint32_t tile_size, uint32_t tile_width,
                                            uint32_t tile_height, int64_t capacity, int64_t* isect_ids,
                                            int32_t* flatten_ids, void* stream);
+/* The emission after gsx_intersect_tile_count_ordered, given that call's workspace (unchanged since): for tile grids
+ * up to 255 x 255 the sorted depth keys in it carry every Gaussian's tile rectangle, so positions are emitted from
+ * sequential reads of (key, order, cum) alone - nothing is gathered in sorted order; larger grids take the path of
+ * gsx_intersect_tile_emit_capped.  Same outputs either way; capacity as above (INT64_MAX = unbounded). */
+GSX_API int gsx_intersect_tile_emit_ordered(uint32_t N, const float* means2d, const int32_t* radii,
+                                            const float* depths, const int64_t* cum_tiles_per_gauss,
+                                            const int32_t* order, const void* ordered_workspace, uint32_t tile_size,
+                                            uint32_t tile_width, uint32_t tile_height, int64_t capacity,
+                                            int64_t* isect_ids, int32_t* flatten_ids, void* stream);
 /* Intersect.cpp:46-47: floor(log2(n)) + 1 */
 GSX_API uint32_t gsx_n_bits(uint32_t n);
 

@@ -41,10 +41,13 @@ static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; 
 
 // intersect.hip: the depth-ordered tile count from ready-made keys.  ordered_keys(ws) is where the N
 // (tile count << 32 | depth bits) keys go inside a gsx_intersect_tile_count_ordered workspace; the second call sorts
-// them on the depth bits, scans the counts in that order into cum (inclusive) and starts the copy of the total.
+// them on the depth bits, scans the counts in that order into cum (inclusive) and starts the copy of the total; the
+// sorted keys stay in ordered_keys(ws).  rect_keys: the high words are packed tile rectangles
+// (x0 | y0 << 8 | x1 << 16 | y1 << 24, 0 = none) instead of counts.
 int64_t* ordered_keys(void* workspace);
 int ordered_counts_from_keys(const char* who, uint32_t N, int32_t* order, int64_t* cum_tiles_per_gauss, void* workspace,
-                             size_t workspace_bytes, int64_t* n_isects_host, int wait, void* stream);
+                             size_t workspace_bytes, int64_t* n_isects_host, int wait, void* stream,
+                             bool rect_keys = false);
 
 int check_camera_args(uint32_t C, const float* viewmats1, int camera_model, int rs_type, const float* radial,
                       const float* tangential, const float* thin_prism);

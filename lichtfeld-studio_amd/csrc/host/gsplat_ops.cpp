@@ -178,10 +178,12 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> intersect_tile(const at::Tensor m
     at::Tensor cum = at::empty({(int64_t)C * N}, depths.options().dtype(at::kLong));
     int64_t n_isects = 0;
     void* stream = cur_stream(means2d);
+    at::Tensor ordered_ws; // holds the sorted depth keys the emission reads: alive until that launch is queued
     if (two_level && N > 0) {
         order = at::empty({(int64_t)N}, depths.options().dtype(at::kInt));
         order_ptr = order.data_ptr<int32_t>();
-        at::Tensor ws = workspace(gsx_intersect_tile_count_ordered_workspace_bytes(N), depths);
+        ordered_ws = workspace(gsx_intersect_tile_count_ordered_workspace_bytes(N), depths);
+        at::Tensor& ws = ordered_ws;
         gsx_check(gsx_intersect_tile_count_ordered(N, means2d.data_ptr<float>(), radii.data_ptr<int32_t>(),
                                                    depths.data_ptr<float>(), tile_size, tile_width, tile_height,
                                                    order.data_ptr<int32_t>(), tiles_per_gauss.data_ptr<int32_t>(),
@@ -196,7 +198,13 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> intersect_tile(const at::Tensor m
     }
     at::Tensor isect_ids = at::empty({n_isects}, depths.options().dtype(at::kLong));
     at::Tensor flatten_ids = at::empty({n_isects}, depths.options().dtype(at::kInt));
-    if (n_isects) {
+    if (n_isects && ordered_ws.defined()) {
+        gsx_check(gsx_intersect_tile_emit_ordered(N, means2d.data_ptr<float>(), radii.data_ptr<int32_t>(),
+                                                  depths.data_ptr<float>(), cum.data_ptr<int64_t>(), order_ptr,
+                                                  ordered_ws.data_ptr(), tile_size, tile_width, tile_height, INT64_MAX,
+                                                  isect_ids.data_ptr<int64_t>(), flatten_ids.data_ptr<int32_t>(),
+                                                  stream));
+    } else if (n_isects) {
         gsx_check(gsx_intersect_tile_emit(C, N, means2d.data_ptr<float>(), radii.data_ptr<int32_t>(),
                                           depths.data_ptr<float>(), cum.data_ptr<int64_t>(), order_ptr, tile_size,
                                           tile_width, tile_height, isect_ids.data_ptr<int64_t>(),

@@ -45,6 +45,13 @@ __global__ void __launch_bounds__(256) tile_count_kernel(uint32_t n, const float
 // Depth-ordered variant, one camera: the tile count rides in the high word of a sort key whose low word is the
 // depth's bit pattern (what the low word of an intersection key holds; all ones for a Gaussian that touches no
 // tile).  Sorting these N keys on their low 32 bits gives the visiting order AND the counts in that order.
+// RECT (tile grids up to 255 x 255): the high word holds the tile rectangle x0 | y0 << 8 | x1 << 16 | y1 << 24
+// instead (0 = no tile), from which both the count and the emission follow without going back to the Gaussian.
+__device__ __forceinline__ uint32_t packed_rect_count(uint32_t hi) {
+    return (((hi >> 24) & 255u) - ((hi >> 8) & 255u)) * (((hi >> 16) & 255u) - (hi & 255u));
+}
+
+template <bool RECT>
 __global__ void __launch_bounds__(256) depth_count_keys_kernel(uint32_t n, const float* __restrict__ means2d,
                                                                 const int32_t* __restrict__ radii,
                                                                 const float* __restrict__ depths, float tile_size,
@@ -61,7 +68,8 @@ __global__ void __launch_bounds__(256) depth_count_keys_kernel(uint32_t n, const
         cnt = (r.y1 - r.y0) * (r.x1 - r.x0);
     tiles_per_gauss[i] = (int32_t)cnt;
     const uint32_t lo = cnt ? f2u(depths[i]) : 0xFFFFFFFFu;
-    keys[i] = (int64_t)(((uint64_t)cnt << 32) | lo);
+    const uint32_t hi = !RECT ? cnt : cnt ? (r.x0 | (r.y0 << 8) | (r.x1 << 16) | (r.y1 << 24)) : 0u;
+    keys[i] = (int64_t)(((uint64_t)hi << 32) | lo);
     vals[i] = (int32_t)i;
 }
 
@@ -87,14 +95,18 @@ __device__ __forceinline__ int64_t block_exclusive_scan_256(int64_t v, int64_t* 
     return incl - v;
 }
 
-// the scan's input: int32 counts, or (keys != nullptr) the high words of 64-bit keys
+// the scan's input: int32 counts, or (keys != nullptr) the high words of 64-bit keys - counts themselves, or
+// packed tile rectangles (rect_keys)
 __device__ __forceinline__ int32_t scan_input(const int32_t* __restrict__ in, const int64_t* __restrict__ keys,
-                                              uint32_t i) {
-    return keys != nullptr ? (int32_t)(keys[i] >> 32) : in[i];
+                                              bool rect_keys, uint32_t i) {
+    if (keys == nullptr)
+        return in[i];
+    const uint32_t hi = (uint32_t)((uint64_t)keys[i] >> 32);
+    return (int32_t)(rect_keys ? packed_rect_count(hi) : hi);
 }
 
 __global__ void __launch_bounds__(256) scan_block_sums_kernel(uint32_t n, const int32_t* __restrict__ in,
-                                                               const int64_t* __restrict__ keys,
+                                                               const int64_t* __restrict__ keys, bool rect_keys,
                                                                int64_t* __restrict__ block_sums) {
     __shared__ int64_t lds[256];
     const uint32_t base = blockIdx.x * kScanTile + threadIdx.x * kScanItems;
@@ -102,7 +114,7 @@ __global__ void __launch_bounds__(256) scan_block_sums_kernel(uint32_t n, const 
 #pragma unroll
     for (uint32_t i = 0; i < kScanItems; ++i)
         if (base + i < n)
-            s += scan_input(in, keys, base + i);
+            s += scan_input(in, keys, rect_keys, base + i);
     int64_t total;
     block_exclusive_scan_256(s, lds, &total);
     if (threadIdx.x == 0)
@@ -128,7 +140,7 @@ __global__ void __launch_bounds__(256) scan_block_offsets_kernel(uint32_t nb, in
 }
 
 __global__ void __launch_bounds__(256) scan_apply_kernel(uint32_t n, const int32_t* __restrict__ in,
-                                                          const int64_t* __restrict__ keys,
+                                                          const int64_t* __restrict__ keys, bool rect_keys,
                                                           const int64_t* __restrict__ block_offsets,
                                                           int64_t* __restrict__ out) {
     __shared__ int64_t lds[256];
@@ -137,7 +149,7 @@ __global__ void __launch_bounds__(256) scan_apply_kernel(uint32_t n, const int32
     int64_t s = 0;
 #pragma unroll
     for (uint32_t i = 0; i < kScanItems; ++i) {
-        v[i] = (base + i < n) ? scan_input(in, keys, base + i) : 0;
+        v[i] = (base + i < n) ? scan_input(in, keys, rect_keys, base + i) : 0;
         s += v[i];
     }
     int64_t total;
@@ -155,9 +167,13 @@ __global__ void __launch_bounds__(256) scan_apply_kernel(uint32_t n, const int32
 // instruction and a serial loop as long as the largest Gaussian.  Here a wave flattens the runs of its 64
 // positions: entry k of the wave's output range belongs to the position whose inclusive count prefix first
 // exceeds k (binary search over 64 prefixes in LDS), so the lanes write consecutive entries.
+// FROM_KEYS: position i's Gaussian is order[i] and its rectangle and depth bits are the words of sorted_keys[i]
+// (depth_count_keys_kernel<true>): sequential reads only, nothing is gathered in sorted order.
+template <bool FROM_KEYS>
 __global__ void __launch_bounds__(256) tile_emit_kernel(uint32_t n, uint32_t N, const float* __restrict__ means2d,
                                                          const int32_t* __restrict__ radii,
                                                          const float* __restrict__ depths,
+                                                         const int64_t* __restrict__ sorted_keys,
                                                          const int64_t* __restrict__ cum_tiles_per_gauss,
                                                          const int32_t* __restrict__ order, float tile_size,
                                                          uint32_t tile_width, uint32_t tile_height,
@@ -170,16 +186,27 @@ __global__ void __launch_bounds__(256) tile_emit_kernel(uint32_t n, uint32_t N, 
     TileRect r = {0, 0, 0, 0};
     uint32_t idx = 0;
     bool live = false;
+    uint32_t depth_bits = 0;
     if (i < n) {
         idx = order != nullptr ? (uint32_t)order[i] : i;
-        live = tile_rect(means2d, radii, idx, tile_size, tile_width, tile_height, &r);
+        if (FROM_KEYS) {
+            const uint64_t key = (uint64_t)sorted_keys[i];
+            const uint32_t hi = (uint32_t)(key >> 32);
+            r.x0 = hi & 255u, r.y0 = (hi >> 8) & 255u, r.x1 = (hi >> 16) & 255u, r.y1 = hi >> 24;
+            live = hi != 0u;
+            depth_bits = (uint32_t)key;
+        } else {
+            live = tile_rect(means2d, radii, idx, tile_size, tile_width, tile_height, &r);
+        }
     }
     const uint32_t w = live ? r.x1 - r.x0 : 0u;
     const uint32_t cnt = live ? (r.y1 - r.y0) * w : 0u;
     int64_t key_base = 0;
     if (cnt) {
         const int64_t cid = idx / N;
-        key_base = (cid << (32 + tile_n_bits)) | (int64_t)(uint64_t)f2u(depths[idx]); // zero-extended bits (:96-98)
+        if (!FROM_KEYS)
+            depth_bits = f2u(depths[idx]);
+        key_base = (cid << (32 + tile_n_bits)) | (int64_t)(uint64_t)depth_bits; // zero-extended bits (:96-98)
     }
     // inclusive prefix of the counts over the wave
     uint32_t incl = cnt;
@@ -272,17 +299,20 @@ extern "C" size_t gsx_intersect_tile_count_workspace_bytes(uint32_t C, uint32_t 
 
 namespace {
 // prefix sum of the counts (int32 array, or high words of `keys`) into cum, grand total to *total_dev
-int scan_counts(uint32_t n, const int32_t* counts, const int64_t* keys, int64_t* cum, int64_t* block_sums,
-                int64_t* total_dev, hipStream_t s) {
+int scan_counts(uint32_t n, const int32_t* counts, const int64_t* keys, bool rect_keys, int64_t* cum,
+                int64_t* block_sums, int64_t* total_dev, hipStream_t s) {
     const uint32_t nb = cdiv(n, kScanTile);
-    hipLaunchKernelGGL(scan_block_sums_kernel, dim3(nb), dim3(256), 0, s, n, counts, keys, block_sums);
+    hipLaunchKernelGGL(scan_block_sums_kernel, dim3(nb), dim3(256), 0, s, n, counts, keys, rect_keys, block_sums);
     GSX_LAUNCH_CHECK();
     hipLaunchKernelGGL(scan_block_offsets_kernel, dim3(1), dim3(256), 0, s, nb, block_sums, total_dev);
     GSX_LAUNCH_CHECK();
-    hipLaunchKernelGGL(scan_apply_kernel, dim3(nb), dim3(256), 0, s, n, counts, keys, block_sums, cum);
+    hipLaunchKernelGGL(scan_apply_kernel, dim3(nb), dim3(256), 0, s, n, counts, keys, rect_keys, block_sums, cum);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }
+
+// tile grids whose rectangle corners fit a byte each: the depth keys then carry the rectangle
+bool rect_keys_fit(uint32_t tile_width, uint32_t tile_height) { return tile_width <= 255 && tile_height <= 255; }
 
 int check_tile_grid(const char* who, uint32_t C, uint32_t tile_size, uint32_t tile_width, uint32_t tile_height) {
     GSX_REQUIRE(tile_size > 0 && tile_width > 0 && tile_height > 0, GSX_ERR_INVALID_ARGUMENT, "%s: empty tile grid",
@@ -322,7 +352,7 @@ extern "C" int gsx_intersect_tile_count(uint32_t C, uint32_t N, const float* mea
     hipLaunchKernelGGL(tile_count_kernel, dim3(cdiv(n, 256)), dim3(256), 0, s, n, means2d, radii, (float)tile_size,
                        tile_width, tile_height, tiles_per_gauss);
     GSX_LAUNCH_CHECK();
-    if ((rc = scan_counts(n, tiles_per_gauss, nullptr, cum_tiles_per_gauss, block_sums, total, s)) != GSX_OK)
+    if ((rc = scan_counts(n, tiles_per_gauss, nullptr, false, cum_tiles_per_gauss, block_sums, total, s)) != GSX_OK)
         return rc;
     // the one sanctioned host synchronisation of the path (Intersect.cpp:76 `.item<int64_t>()`)
     int64_t host_total = 0;
@@ -357,9 +387,10 @@ namespace gsx {
 int64_t* ordered_keys(void* workspace) { return (int64_t*)workspace; }
 
 // The part after the keys are written: sort the N (count << 32 | depth bits) keys in workspace on their low word,
-// scan the counts in that order, start the copy of the total.  order must hold 0..N-1 on entry.
+// scan the counts in that order, start the copy of the total.  order must hold 0..N-1 on entry.  rect_keys: the
+// high words are packed tile rectangles (depth_count_keys_kernel<true>) instead of counts.
 int ordered_counts_from_keys(const char* who, uint32_t N, int32_t* order, int64_t* cum_tiles_per_gauss, void* workspace,
-                             size_t workspace_bytes, int64_t* n_isects_host, int wait, void* stream) {
+                             size_t workspace_bytes, int64_t* n_isects_host, int wait, void* stream, bool rect_keys) {
     const OrderedLayout L = ordered_layout(N);
     GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 && workspace_bytes >= L.total,
                 GSX_ERR_WORKSPACE, "%s: workspace needs %zu bytes, 256-byte aligned", who, L.total);
@@ -374,9 +405,12 @@ int ordered_counts_from_keys(const char* who, uint32_t N, int32_t* order, int64_
     if ((rc = gsx_radix_sort_pairs(N, keys0, order, keys1, vals1, 0, 32, ws + L.sort_off,
                                    gsx_radix_sort_pairs_workspace_bytes(N), &sel, stream)) != GSX_OK)
         return rc;
-    if (sel) // four 8-bit passes end in buffer 0; kept for a different digit width
+    if (sel) { // four 8-bit passes end in buffer 0; kept for a different digit width
         GSX_HIP_CHECK(hipMemcpyAsync(order, vals1, (size_t)N * 4, hipMemcpyDeviceToDevice, s));
-    if ((rc = scan_counts(N, nullptr, sel ? keys1 : keys0, cum_tiles_per_gauss, block_sums, total, s)) != GSX_OK)
+        GSX_HIP_CHECK(hipMemcpyAsync(keys0, keys1, (size_t)N * 8, hipMemcpyDeviceToDevice, s));
+    }
+    // the sorted keys stay in ordered_keys(workspace) for an emission that reads them
+    if ((rc = scan_counts(N, nullptr, keys0, rect_keys, cum_tiles_per_gauss, block_sums, total, s)) != GSX_OK)
         return rc;
     GSX_HIP_CHECK(hipMemcpyAsync(n_isects_host, total, sizeof(int64_t), hipMemcpyDeviceToHost, s));
     if (wait) {
@@ -408,12 +442,18 @@ extern "C" int gsx_intersect_tile_count_ordered(uint32_t N, const float* means2d
                     workspace_bytes >= ordered_layout(N).total,
                 GSX_ERR_WORKSPACE, "intersect_tile_count_ordered: workspace needs %zu bytes, 256-byte aligned",
                 ordered_layout(N).total);
-    hipLaunchKernelGGL(depth_count_keys_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, means2d,
-                       radii, depths, (float)tile_size, tile_width, tile_height, tiles_per_gauss,
-                       gsx::ordered_keys(workspace), order);
+    const bool rect_keys = rect_keys_fit(tile_width, tile_height);
+    if (rect_keys)
+        hipLaunchKernelGGL(depth_count_keys_kernel<true>, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N,
+                           means2d, radii, depths, (float)tile_size, tile_width, tile_height, tiles_per_gauss,
+                           gsx::ordered_keys(workspace), order);
+    else
+        hipLaunchKernelGGL(depth_count_keys_kernel<false>, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N,
+                           means2d, radii, depths, (float)tile_size, tile_width, tile_height, tiles_per_gauss,
+                           gsx::ordered_keys(workspace), order);
     GSX_LAUNCH_CHECK();
     return gsx::ordered_counts_from_keys("intersect_tile_count_ordered", N, order, cum_tiles_per_gauss, workspace,
-                                         workspace_bytes, n_isects_host, wait, stream);
+                                         workspace_bytes, n_isects_host, wait, stream, rect_keys);
 }
 
 extern "C" int gsx_intersect_tile_emit(uint32_t C, uint32_t N, const float* means2d, const int32_t* radii,
@@ -438,9 +478,34 @@ extern "C" int gsx_intersect_tile_emit_capped(uint32_t C, uint32_t N, const floa
     GSX_REQUIRE(n64 < (1ull << 31), GSX_ERR_INVALID_ARGUMENT, "intersect_tile_emit: C*N >= 2^31");
     const uint32_t n = (uint32_t)n64;
     GSX_REQUIRE(order == nullptr || C == 1, GSX_ERR_UNSUPPORTED, "intersect_tile_emit: an order needs C == 1");
-    hipLaunchKernelGGL(tile_emit_kernel, dim3(cdiv(n, 256)), dim3(256), 0, (hipStream_t)stream, n, N, means2d, radii,
-                       depths, cum_tiles_per_gauss, order, (float)tile_size, tile_width, tile_height,
-                       gsx_n_bits(tile_width * tile_height), capacity, isect_ids, flatten_ids);
+    hipLaunchKernelGGL(tile_emit_kernel<false>, dim3(cdiv(n, 256)), dim3(256), 0, (hipStream_t)stream, n, N, means2d,
+                       radii, depths, (const int64_t*)nullptr, cum_tiles_per_gauss, order, (float)tile_size, tile_width,
+                       tile_height, gsx_n_bits(tile_width * tile_height), capacity, isect_ids, flatten_ids);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+extern "C" int gsx_intersect_tile_emit_ordered(uint32_t N, const float* means2d, const int32_t* radii,
+                                               const float* depths, const int64_t* cum_tiles_per_gauss,
+                                               const int32_t* order, const void* ordered_workspace,
+                                               uint32_t tile_size, uint32_t tile_width, uint32_t tile_height,
+                                               int64_t capacity, int64_t* isect_ids, int32_t* flatten_ids,
+                                               void* stream) {
+    if (N == 0)
+        return GSX_OK;
+    GSX_REQUIRE(order && ordered_workspace, GSX_ERR_INVALID_ARGUMENT,
+                "intersect_tile_emit_ordered: order / workspace of gsx_intersect_tile_count_ordered is null");
+    if (!rect_keys_fit(tile_width, tile_height)) // the keys hold counts: rectangles come from the Gaussians
+        return gsx_intersect_tile_emit_capped(1, N, means2d, radii, depths, cum_tiles_per_gauss, order, tile_size,
+                                              tile_width, tile_height, capacity, isect_ids, flatten_ids, stream);
+    GSX_REQUIRE(cum_tiles_per_gauss && isect_ids && flatten_ids, GSX_ERR_INVALID_ARGUMENT,
+                "intersect_tile_emit_ordered: null tensor");
+    GSX_REQUIRE(N < (1u << 31), GSX_ERR_INVALID_ARGUMENT, "intersect_tile_emit_ordered: N >= 2^31");
+    hipLaunchKernelGGL(tile_emit_kernel<true>, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, N,
+                       (const float*)nullptr, (const int32_t*)nullptr, (const float*)nullptr,
+                       (const int64_t*)gsx::ordered_keys(const_cast<void*>(ordered_workspace)), cum_tiles_per_gauss,
+                       order, (float)tile_size, tile_width, tile_height, gsx_n_bits(tile_width * tile_height),
+                       capacity, isect_ids, flatten_ids);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

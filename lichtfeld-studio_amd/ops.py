@@ -147,7 +147,12 @@ def intersect_tile(means2d, radii, depths, camera_ids, gaussian_ids, C, tile_siz
         n = n_isects.value
         isect_ids = torch.empty((n,), dtype=torch.int64, device=dev)
         flatten_ids = torch.empty((n,), dtype=torch.int32, device=dev)
-        if n:
+        if n and two_level:  # ws still holds the sorted depth keys (with the tile rectangles) the emission reads
+            check(lib().gsx_intersect_tile_emit_ordered(
+                c_u32(N), _ptr(means2d), _ptr(radii), _ptr(depths), _ptr(cum), _ptr(order), _ptr(ws),
+                c_u32(tile_size), c_u32(tile_width), c_u32(tile_height), c_i64((1 << 63) - 1), _ptr(isect_ids),
+                _ptr(flatten_ids), _stream(dev)))
+        elif n:
             check(lib().gsx_intersect_tile_emit(c_u32(C), c_u32(N), _ptr(means2d), _ptr(radii), _ptr(depths),
                                                 _ptr(cum), _ptr(order), c_u32(tile_size), c_u32(tile_width),
                                                 c_u32(tile_height), _ptr(isect_ids), _ptr(flatten_ids),

@@ -191,9 +191,9 @@ class TrainStep:
         # The emission does not need the total, only room for it: with buffers from an earlier step it is queued now
         # (writes bounded to the buffers) and the host's wake-up from the wait below hides behind it.
         emit = lambda cap: self._run(
-            "intersect_tile_emit", lb.gsx_intersect_tile_emit_capped, c_u32(1), c_u32(N), _p(J["means2d"]),
-            _p(J["radii"]), _p(J["depths"]), _p(self.cum), _p(self.order), c_u32(16), c_u32(self.tw), c_u32(self.th),
-            c_i64(cap), _p(self.keys[0]), _p(self.vals[0]), s)
+            "intersect_tile_emit", lb.gsx_intersect_tile_emit_ordered, c_u32(N), _p(J["means2d"]), _p(J["radii"]),
+            _p(J["depths"]), _p(self.cum), _p(self.order), _p(self.ws_count), c_u32(16), c_u32(self.tw),
+            c_u32(self.th), c_i64(cap), _p(self.keys[0]), _p(self.vals[0]), s)
         emitted_cap = self.cap
         if emitted_cap:
             emit(emitted_cap)

@@ -190,6 +190,35 @@ def test_intersect_sort_offsets_bit_exact(gsx, orc, cuda):
     assert ids.numel() == 0 and flat.numel() == 0 and int(tpg.sum()) == 0
 
 
+@pytest.mark.parametrize("grid", [(255, 40), (256, 40), (40, 300), (255, 255)])
+def test_intersect_wide_tile_grids(gsx, orc, cuda, grid):
+    """tile grids at and beyond 255 tiles per side: up to 255 x 255 the depth keys carry each Gaussian's tile rectangle
+    and the emission reads nothing else; wider grids fall back to rectangles from the Gaussians.  Same keys, order and
+    counts as the checker either way (rectangles touching the last column / row included)."""
+    ops = gsx.ops
+    tw, th = grid
+    W, H = tw * 16 - 3, th * 16 - 5
+    rng = np.random.default_rng(tw * 1000 + th)
+    n = 20000
+    means2d = np.stack([rng.uniform(-20, W + 20, n), rng.uniform(-20, H + 20, n)], 1).astype(np.float32)[None]
+    radii = rng.integers(0, 40, (1, n, 2)).astype(np.int32)
+    radii[0, ::7] = 0
+    means2d[0, :50] = [W - 1.0, H - 1.0]  # rectangles that end at the grid's last tile
+    radii[0, :50] = 30
+    depths = rng.uniform(0.1, 50.0, (1, n)).astype(np.float32)
+    depths[0, 100:200] = depths[0, 100]  # ties: broken by index
+    for sort in (True, False):
+        ref_tpg, ref_ids, ref_flat = orc.intersect_tile(means2d, radii, depths, 1, 16, tw, th, sort)
+        tpg, ids, flat = ops.intersect_tile(T(means2d, cuda), T(radii, cuda), T(depths, cuda), None, None, 1, 16, tw,
+                                            th, sort)
+        assert ref_ids.shape[0] > 100000
+        bits_equal(N(tpg), ref_tpg, "tiles_per_gauss")
+        bits_equal(N(ids), ref_ids, f"keys (sort={sort})")
+        bits_equal(N(flat), ref_flat, f"values (sort={sort})")
+    _, s_ids, _ = ops.intersect_tile(T(means2d, cuda), T(radii, cuda), T(depths, cuda), None, None, 1, 16, tw, th, True)
+    bits_equal(N(ops.intersect_offset(s_ids, 1, tw, th)), orc.intersect_offset(N(s_ids), 1, tw, th), "per-tile ranges")
+
+
 @pytest.mark.parametrize("n", [1, 63, 64, 65, 4095, 4096, 4097, 100_003, 3_000_000])
 def test_radix_sort_stable(gsx, orc, cuda, n):
     ops = gsx.ops
