@@ -74,7 +74,8 @@ __global__ void __launch_bounds__(256) depth_count_keys_kernel(uint32_t n, const
 }
 
 // ---- inclusive scan int32 -> int64 (at::cumsum of Intersect.cpp:75) -----------------------------
-// three passes: per-block sums, scan of the sums (one block), per-block scan + offset
+// per-block sums, then per-block scan + the total of the earlier blocks (summed by each block itself, or for very
+// long inputs scanned by one block in a launch of its own)
 static constexpr uint32_t kScanItems = 8;
 static constexpr uint32_t kScanTile = 256 * kScanItems;
 
@@ -139,10 +140,14 @@ __global__ void __launch_bounds__(256) scan_block_offsets_kernel(uint32_t nb, in
         *total_out = carry;
 }
 
+// Per-block scan plus the total of the earlier blocks.  SUMS: block_sums holds the blocks' own totals and every block
+// adds up the ones in front of it for itself (a few hundred to a few thousand values from L2: cheaper than a launch
+// of its own; the last block also leaves the grand total); otherwise it holds the exclusive prefixes already.
+template <bool SUMS>
 __global__ void __launch_bounds__(256) scan_apply_kernel(uint32_t n, const int32_t* __restrict__ in,
                                                           const int64_t* __restrict__ keys, bool rect_keys,
-                                                          const int64_t* __restrict__ block_offsets,
-                                                          int64_t* __restrict__ out) {
+                                                          const int64_t* __restrict__ block_sums,
+                                                          int64_t* __restrict__ out, int64_t* __restrict__ total_out) {
     __shared__ int64_t lds[256];
     const uint32_t base = blockIdx.x * kScanTile + threadIdx.x * kScanItems;
     int32_t v[kScanItems];
@@ -152,14 +157,25 @@ __global__ void __launch_bounds__(256) scan_apply_kernel(uint32_t n, const int32
         v[i] = (base + i < n) ? scan_input(in, keys, rect_keys, base + i) : 0;
         s += v[i];
     }
+    int64_t offset = 0; // total of the blocks in front of this one
+    if (SUMS) {
+        int64_t before = 0;
+        for (uint32_t b = threadIdx.x; b < blockIdx.x; b += 256)
+            before += block_sums[b];
+        block_exclusive_scan_256(before, lds, &offset);
+    } else {
+        offset = block_sums[blockIdx.x];
+    }
     int64_t total;
-    int64_t run = block_exclusive_scan_256(s, lds, &total) + block_offsets[blockIdx.x];
+    int64_t run = block_exclusive_scan_256(s, lds, &total) + offset;
 #pragma unroll
     for (uint32_t i = 0; i < kScanItems; ++i) {
         run += v[i];
         if (base + i < n)
             out[base + i] = run;
     }
+    if (SUMS && blockIdx.x == gridDim.x - 1 && threadIdx.x == 0)
+        *total_out = offset + total;
 }
 
 // IntersectTile.cu:78-113 second pass: keys and values in emission order (ascending position, row-major tiles
@@ -304,9 +320,15 @@ int scan_counts(uint32_t n, const int32_t* counts, const int64_t* keys, bool rec
     const uint32_t nb = cdiv(n, kScanTile);
     hipLaunchKernelGGL(scan_block_sums_kernel, dim3(nb), dim3(256), 0, s, n, counts, keys, rect_keys, block_sums);
     GSX_LAUNCH_CHECK();
-    hipLaunchKernelGGL(scan_block_offsets_kernel, dim3(1), dim3(256), 0, s, nb, block_sums, total_dev);
-    GSX_LAUNCH_CHECK();
-    hipLaunchKernelGGL(scan_apply_kernel, dim3(nb), dim3(256), 0, s, n, counts, keys, rect_keys, block_sums, cum);
+    if (nb <= 4096) { // every block sums the totals in front of it: at most 8 M additions in all
+        hipLaunchKernelGGL(scan_apply_kernel<true>, dim3(nb), dim3(256), 0, s, n, counts, keys, rect_keys, block_sums,
+                           cum, total_dev);
+    } else {
+        hipLaunchKernelGGL(scan_block_offsets_kernel, dim3(1), dim3(256), 0, s, nb, block_sums, total_dev);
+        GSX_LAUNCH_CHECK();
+        hipLaunchKernelGGL(scan_apply_kernel<false>, dim3(nb), dim3(256), 0, s, n, counts, keys, rect_keys, block_sums,
+                           cum, total_dev);
+    }
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

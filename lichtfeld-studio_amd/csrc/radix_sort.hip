@@ -1,8 +1,9 @@
 // radix_sort.hip - stable LSD radix sort of (int64 key, int32 value) pairs on key bits [begin_bit, end_bit)
 // (gsplat/IntersectTile.cu:290-328 calls cub::DeviceRadixSort::SortPairs with a DoubleBuffer).
 //
-// 8-bit digits.  Per pass three launches: block histograms (which also add up the 256 digit totals) -> one scan
-// block per digit turns its row of the digit-major table into global start positions -> stable scatter.  A
+// 8-bit digits.  Per pass three launches: block histograms -> one scan block per digit turns its row of the
+// digit-major table into running counts and leaves the digit's total -> stable scatter (every block adds the
+// exclusive scan of the 256 totals itself; no atomics between blocks, nothing to zero).  A
 // block owns a tile of 256 x ITEMS consecutive pairs; inside the block each 64-lane wave owns a quarter of them
 // and ranks them 64 at a time with wave-wide match masks built from ballots, so the order (wave, round, lane)
 // equals the input order and the sort is stable.  The ranked pairs are first placed in LDS in digit order and then
@@ -16,13 +17,6 @@ static constexpr uint32_t kRadix = 1u << kRadixBits;
 static constexpr uint32_t kItemsLarge = 16; // pairs per lane: 4096-pair tiles
 static constexpr uint32_t kItemsSmall = 4;  // 1024-pair tiles when there are too few pairs to fill the GPU otherwise
 static constexpr int64_t kSmallSortLimit = 1ll << 21;
-static constexpr uint32_t kTotalStripes = 32;
-
-__global__ void __launch_bounds__(256) fill_u32_kernel(uint32_t n, uint32_t v, uint32_t* __restrict__ out) {
-    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
-    if (i < n)
-        out[i] = v;
-}
 
 __device__ __forceinline__ uint32_t digit_of(int64_t key, uint32_t shift, uint32_t mask) {
     return (uint32_t)((uint64_t)key >> shift) & mask;
@@ -31,8 +25,7 @@ __device__ __forceinline__ uint32_t digit_of(int64_t key, uint32_t shift, uint32
 __global__ void __launch_bounds__(256) radix_hist_kernel(uint32_t n, const int64_t* __restrict__ keys,
                                                           uint32_t items, uint32_t shift, uint32_t mask,
                                                           uint32_t nblocks,
-                                                          uint32_t* __restrict__ hist /*[kRadix][nblocks]*/,
-                                                          uint32_t* __restrict__ digit_total /*[kTotalStripes][kRadix]*/) {
+                                                          uint32_t* __restrict__ hist /*[kRadix][nblocks]*/) {
     __shared__ uint32_t lh[kRadix];
     lh[threadIdx.x] = 0;
     __syncthreads();
@@ -44,10 +37,7 @@ __global__ void __launch_bounds__(256) radix_hist_kernel(uint32_t n, const int64
             atomicAdd(&lh[digit_of(keys[idx], shift, mask)], 1u);
     }
     __syncthreads();
-    const uint32_t c = lh[threadIdx.x];
-    hist[threadIdx.x * nblocks + blockIdx.x] = c;
-    if (c) // the totals are striped over kTotalStripes copies so that the blocks do not queue on 256 addresses
-        atomicAdd(&digit_total[(blockIdx.x % kTotalStripes) * kRadix + threadIdx.x], c);
+    hist[threadIdx.x * nblocks + blockIdx.x] = lh[threadIdx.x];
 }
 
 // ---- per-digit scan --------------------------------------------------------------------------------
@@ -61,30 +51,14 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan_u32(uint32_t v, uint32_t
     return v;
 }
 
-// Block d owns digit d: hist[d][0..nblocks) becomes the global position at which each sort block starts writing
-// its pairs with that digit = (pairs with a smaller digit) + (pairs with digit d in earlier blocks).
+// Block d owns digit d: hist[d][0..nblocks) becomes the number of pairs with digit d in earlier sort blocks, and
+// digit_total[d] the number of pairs with digit d.  (The scatter adds the pairs with a smaller digit: an exclusive
+// scan of the 256 totals, which every sort block forms for itself - no atomics, nothing to zero beforehand.)
 __global__ void __launch_bounds__(256) radix_scan_kernel(uint32_t nblocks, uint32_t* __restrict__ hist,
-                                                          const uint32_t* __restrict__ digit_total) {
+                                                          uint32_t* __restrict__ digit_total /*[kRadix]*/) {
     __shared__ uint32_t wsum[4];
-    __shared__ uint32_t base_s;
     const uint32_t d = blockIdx.x, t = threadIdx.x, lane = t & 63u, w = t >> 6;
-    // pairs with a smaller digit
-    {
-        uint32_t v = 0;
-        if (t < d) {
-#pragma unroll 8
-            for (uint32_t st = 0; st < kTotalStripes; ++st)
-                v += digit_total[st * kRadix + t];
-        }
-        const uint32_t incl = wave_inclusive_scan_u32(v, lane);
-        if (lane == 63)
-            wsum[w] = incl;
-        __syncthreads();
-        if (t == 0)
-            base_s = wsum[0] + wsum[1] + wsum[2] + wsum[3];
-        __syncthreads();
-    }
-    uint32_t carry = base_s;
+    uint32_t carry = 0;
     uint32_t* __restrict__ row = hist + (size_t)d * nblocks;
     for (uint32_t start = 0; start < nblocks; start += 256) {
         const uint32_t i = start + t;
@@ -102,6 +76,8 @@ __global__ void __launch_bounds__(256) radix_scan_kernel(uint32_t nblocks, uint3
             row[i] = carry + before + incl - v;
         carry += wsum[0] + wsum[1] + wsum[2] + wsum[3];
     }
+    if (t == 0)
+        digit_total[d] = carry;
 }
 
 // ---- stable scatter -------------------------------------------------------------------------------
@@ -111,11 +87,12 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const in
                                                              int64_t* __restrict__ keys_out,
                                                              int32_t* __restrict__ vals_out, uint32_t shift,
                                                              uint32_t mask, uint32_t nblocks,
-                                                             const uint32_t* __restrict__ hist_scanned) {
+                                                             const uint32_t* __restrict__ hist_scanned,
+                                                             const uint32_t* __restrict__ digit_total) {
     constexpr uint32_t kTileN = 256 * ITEMS, kWaveN = 64 * ITEMS;
     __shared__ uint32_t wave_count[4][kRadix];
     __shared__ uint32_t to_global[kRadix]; // global position of a pair = to_global[digit] + its slot in the tile
-    __shared__ uint32_t wsum[4];
+    __shared__ uint32_t wsum[4], gsum[4];
     __shared__ int64_t s_keys[kTileN];
     __shared__ int32_t s_vals[kTileN];
     const uint32_t t = threadIdx.x;
@@ -165,20 +142,27 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const in
     {
         const uint32_t c0 = wave_count[0][t], c1 = wave_count[1][t], c2 = wave_count[2][t], c3 = wave_count[3][t];
         const uint32_t tot = c0 + c1 + c2 + c3;
+        const uint32_t gtot = digit_total[t]; // pairs with digit t in the whole input
         const uint32_t incl = wave_inclusive_scan_u32(tot, lane);
-        if (lane == 63)
+        const uint32_t gincl = wave_inclusive_scan_u32(gtot, lane);
+        if (lane == 63) {
             wsum[w] = incl;
+            gsum[w] = gincl;
+        }
         __syncthreads();
-        uint32_t before = 0;
+        uint32_t before = 0, gbefore = 0;
 #pragma unroll
-        for (uint32_t k = 0; k < 4; ++k)
+        for (uint32_t k = 0; k < 4; ++k) {
             before += k < w ? wsum[k] : 0u;
+            gbefore += k < w ? gsum[k] : 0u;
+        }
         const uint32_t start = before + incl - tot;
+        const uint32_t smaller = gbefore + gincl - gtot; // pairs with a smaller digit
         wave_count[0][t] = start;
         wave_count[1][t] = start + c0;
         wave_count[2][t] = start + c0 + c1;
         wave_count[3][t] = start + c0 + c1 + c2;
-        to_global[t] = hist_scanned[t * nblocks + blockIdx.x] - start;
+        to_global[t] = smaller + hist_scanned[t * nblocks + blockIdx.x] - start;
     }
     __syncthreads();
 #pragma unroll
@@ -220,7 +204,7 @@ SortLayout sort_layout(int64_t n) {
     L.nblocks = cdiv((uint64_t)n, 256u * sort_items(n));
     L.hist_off = 0;
     L.totals_off = align_up((size_t)L.nblocks * kRadix * 4, 256);
-    L.total = L.totals_off + (size_t)kMaxPasses * kTotalStripes * kRadix * 4;
+    L.total = L.totals_off + (size_t)kRadix * 4;
     return L;
 }
 } // namespace
@@ -263,9 +247,6 @@ extern "C" int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, i
     const uint32_t passes = (n_bits + kRadixBits - 1) / kRadixBits;
     GSX_REQUIRE(passes <= kMaxPasses, GSX_ERR_INVALID_ARGUMENT, "radix_sort_pairs: %u passes", passes);
     const uint32_t width_lo = n_bits / passes, n_wide = n_bits % passes;
-    const uint32_t n_tot = passes * kTotalStripes * kRadix;
-    hipLaunchKernelGGL(fill_u32_kernel, dim3(cdiv(n_tot, 256)), dim3(256), 0, s, n_tot, 0u, totals);
-    GSX_LAUNCH_CHECK();
     int sel = 0;
     uint32_t shift = begin_bit;
     const uint32_t items = sort_items(n);
@@ -276,18 +257,17 @@ extern "C" int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, i
         const int32_t* vin = sel ? vals1 : vals0;
         int64_t* kout = sel ? keys0 : keys1;
         int32_t* vout = sel ? vals0 : vals1;
-        uint32_t* tot = totals + pass * kTotalStripes * kRadix;
         hipLaunchKernelGGL(radix_hist_kernel, dim3(L.nblocks), dim3(256), 0, s, (uint32_t)n, kin, items, shift, mask,
-                           L.nblocks, hist, tot);
+                           L.nblocks, hist);
         GSX_LAUNCH_CHECK();
-        hipLaunchKernelGGL(radix_scan_kernel, dim3(kRadix), dim3(256), 0, s, L.nblocks, hist, tot);
+        hipLaunchKernelGGL(radix_scan_kernel, dim3(kRadix), dim3(256), 0, s, L.nblocks, hist, totals);
         GSX_LAUNCH_CHECK();
         if (items == kItemsSmall)
             hipLaunchKernelGGL((radix_scatter_kernel<kItemsSmall>), dim3(L.nblocks), dim3(256), 0, s, (uint32_t)n, kin,
-                               vin, kout, vout, shift, mask, L.nblocks, hist);
+                               vin, kout, vout, shift, mask, L.nblocks, hist, totals);
         else
             hipLaunchKernelGGL((radix_scatter_kernel<kItemsLarge>), dim3(L.nblocks), dim3(256), 0, s, (uint32_t)n, kin,
-                               vin, kout, vout, shift, mask, L.nblocks, hist);
+                               vin, kout, vout, shift, mask, L.nblocks, hist, totals);
         GSX_LAUNCH_CHECK();
         sel ^= 1;
         shift += bits;

@@ -219,6 +219,31 @@ def test_intersect_wide_tile_grids(gsx, orc, cuda, grid):
     bits_equal(N(ops.intersect_offset(s_ids, 1, tw, th)), orc.intersect_offset(N(s_ids), 1, tw, th), "per-tile ranges")
 
 
+@pytest.mark.parametrize("n", [2047, 2048, 2049, 700_001, 9_000_000])
+def test_tile_count_prefix_sums(gsx, cuda, n):
+    """the inclusive prefix of the tile counts and the total equal numpy's cumsum at the scan's block boundaries, in
+    the middle, and beyond 4096 scan blocks (where the block totals are scanned by a launch of their own)"""
+    import ctypes
+    from lichtfeld_studio_amd._lib import c_p, c_sz, c_u32, check, lib
+    L = lib()
+    rng = np.random.default_rng(n)
+    tw, th = 78, 52
+    means2d = torch.from_numpy(np.stack([rng.uniform(0, tw * 16, n), rng.uniform(0, th * 16, n)], 1)
+                               .astype(np.float32)).to(cuda)
+    radii = torch.from_numpy(rng.integers(0, 30, (n, 2)).astype(np.int32)).to(cuda)
+    tpg = torch.empty(n, dtype=torch.int32, device=cuda)
+    cum = torch.empty(n, dtype=torch.int64, device=cuda)
+    ws = torch.empty(L.gsx_intersect_tile_count_workspace_bytes(c_u32(1), c_u32(n)), dtype=torch.uint8, device=cuda)
+    total = ctypes.c_int64(0)
+    p = lambda t: c_p(t.data_ptr())
+    check(L.gsx_intersect_tile_count(c_u32(1), c_u32(n), p(means2d), p(radii), c_u32(16), c_u32(tw), c_u32(th), p(tpg),
+                                     p(cum), p(ws), c_sz(ws.numel()), ctypes.byref(total),
+                                     c_p(torch.cuda.current_stream(cuda).cuda_stream)))
+    want = np.cumsum(tpg.cpu().numpy().astype(np.int64))
+    assert total.value == int(want[-1]) and total.value > n
+    assert np.array_equal(cum.cpu().numpy(), want)
+
+
 @pytest.mark.parametrize("n", [1, 63, 64, 65, 4095, 4096, 4097, 100_003, 3_000_000])
 def test_radix_sort_stable(gsx, orc, cuda, n):
     ops = gsx.ops
