@@ -454,6 +454,8 @@ extern "C" int gsx_intersect_tile_count_ordered(uint32_t N, const float* means2d
     *n_isects_host = 0;
     if (N == 0)
         return GSX_OK;
+    if (!wait)
+        *n_isects_host = -1; // "not there yet": the device-to-host copy queued below overwrites it with the total
     GSX_REQUIRE(means2d && radii && depths && order && tiles_per_gauss && cum_tiles_per_gauss,
                 GSX_ERR_INVALID_ARGUMENT, "intersect_tile_count_ordered: null tensor");
     GSX_REQUIRE(N < (1u << 31), GSX_ERR_INVALID_ARGUMENT, "intersect_tile_count_ordered: N >= 2^31");

@@ -88,12 +88,27 @@ class TrainStep:
         self.ws_count = e(self.lib.gsx_intersect_tile_count_ordered_workspace_bytes(c_u32(N)), dt=torch.uint8)
         self.order = e(N, dt=torch.int32)
         self.n_isects_pinned = torch.zeros(1, dtype=torch.int64, pin_memory=True)
+        self._n_slot = ctypes.c_int64.from_address(self.n_isects_pinned.data_ptr())
         self.count_done = torch.cuda.Event()
         self.ws_bwd = torch.zeros(self.lib.gsx_rasterize_bwd_accum_bytes(c_u32(N)), dtype=torch.uint8,
                                   device=self.dev)  # the backward's epilogue leaves it zeroed for the next pass
         self.records = e(self.lib.gsx_raster_records_bytes(c_u32(N)), dt=torch.uint8)
 
     # -- buffers that depend on n_isects / image size --------------------------------------------
+    def _await_count(self):
+        """The intersection total: the pinned slot reads -1 until the device's copy has landed.  Watching the slot
+        costs the host no driver call on the way out of the wait (the kernels behind it are queued sooner)."""
+        slot = self._n_slot
+        for _ in range(2_000_000):
+            n = slot.value
+            if n >= 0:
+                break
+        else:
+            self.count_done.synchronize()
+            n = slot.value
+        self.n_isects = n
+        return n
+
     def _ensure_isect_capacity(self, n):
         if n <= self.cap:
             return
@@ -109,6 +124,7 @@ class TrainStep:
             return
         e = lambda *s, dt=torch.float32: torch.empty(s, dtype=dt, device=self.dev)
         self.tw, self.th = (W + 15) // 16, (H + 15) // 16
+        self._end_bit = 32 + self.lib.gsx_n_bits(c_u32(self.tw * self.th)) + self.lib.gsx_n_bits(c_u32(1))
         self.offsets = e(1, self.th, self.tw, dt=torch.int32)
         self.render = e(1, H, W, 3)
         self.alpha = e(1, H, W, 1)
@@ -197,8 +213,7 @@ class TrainStep:
         emitted_cap = self.cap
         if emitted_cap:
             emit(emitted_cap)
-        self.count_done.synchronize()
-        n = self.n_isects = int(self.n_isects_pinned[0])
+        n = self._await_count()
         if n >= 1 << 31:
             raise L.GsxError(-5, f"{n} intersections do not fit int32 indices")
         self._ensure_isect_capacity(n)
@@ -206,7 +221,7 @@ class TrainStep:
         if n:
             if n > emitted_cap:  # first step, or the buffers had to grow
                 emit(self.cap)
-            end_bit = 32 + lb.gsx_n_bits(c_u32(self.tw * self.th)) + lb.gsx_n_bits(c_u32(1))
+            end_bit = self._end_bit  # 32 + tile bits + camera bits, fixed with the image size
             self._run("radix_sort_pairs", lb.gsx_radix_sort_pairs, c_i64(n), _p(self.keys[0]), _p(self.vals[0]),
                       _p(self.keys[1]), _p(self.vals[1]), c_u32(32), c_u32(end_bit), _p(self.ws_sort),
                       c_sz(self.ws_sort.numel()), ctypes.byref(sel), s)
