@@ -89,8 +89,8 @@ __device__ __forceinline__ bool project_cam_point(const ProjCfg& cfg, vec3 pc, v
 
 // world_point_to_image_point_shutter_pose (Cameras.cuh:346-414).  Global shutter: the start pose's projection.
 // Rolling shutter: from the start-pose projection (the end-pose one if only that is valid; neither valid = invalid)
-// ten rounds of "exposure time of the current image point -> pose -> projection"; the last point is returned as
-// valid.  One loop, one projection call site: round 0 = start pose, 1 = end pose, 2 .. 11 = the iteration.
+// ten passes of "exposure time of the current image point -> pose -> projection"; the last point is returned as
+// valid.  One loop, one projection call site: pass 0 = start pose, 1 = end pose, 2 .. 11 = the iteration.
 template <bool GENERAL>
 __device__ __forceinline__ bool project_world_point(const ProjCfg& cfg, const CamPose& cp, vec3 p, vec2* uv) {
     if (!GENERAL || cp.rs_type == GSX_GLOBAL)
@@ -98,21 +98,21 @@ __device__ __forceinline__ bool project_world_point(const ProjCfg& cfg, const Ca
     vec2 prev = {0.f, 0.f}, p_start = {0.f, 0.f};
     bool valid_start = false;
 #pragma unroll 1
-    for (int round = 0; round < 12; ++round) {
+    for (int pass = 0; pass < 12; ++pass) {
         quat q = cp.q_start;
         vec3 t = cp.t_start;
-        if (round == 1) {
+        if (pass == 1) {
             q = cp.q_end;
             t = cp.t_end;
-        } else if (round > 1) {
+        } else if (pass > 1) {
             shutter_pose(cp, shutter_relative_frame_time(cp, prev.x, prev.y), &q, &t);
         }
         vec2 pt;
         const bool pv = project_cam_point<GENERAL>(cfg, add(quat_rotate(q, p), t), &pt);
-        if (round == 0) {
+        if (pass == 0) {
             p_start = pt;
             valid_start = pv;
-        } else if (round == 1) {
+        } else if (pass == 1) {
             if (valid_start) {
                 prev = p_start;
             } else if (pv) {
