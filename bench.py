@@ -97,6 +97,7 @@ def main():
     ap.add_argument("--no-overlap", action="store_true",
                     help="keep every kernel of the step on one stream (default: the SH / record pass and the loss "
                          "reduction run on a second stream beside the sort chain / the backward rasterizer)")
+    ap.add_argument("--no-tile-order", action="store_true", help="rasterize the tiles in index order")
     ap.add_argument("--cpu-threads", type=int, default=0, help="threads for the CPU baseline (0 = all)")
     ap.add_argument("--workload", choices=["gut", "fastgs"], default="gut",
                     help="gut: the training step of the metric (default); fastgs: forward + backward of the "
@@ -134,6 +135,7 @@ def main():
     use_ssim = args.config != 1  # configuration 1 is L1 only
     ts = TrainStep(sc, dev, use_ssim=use_ssim, fused_update=not args.separate_update,
                    fused_loss=not args.separate_update, overlap=not args.no_overlap)
+    ts.order_tiles = not args.no_tile_order
     setup_s = time.time() - t0
 
     dominant = "rasterize_bwd_accumulate"

@@ -177,12 +177,19 @@ GSX_API int gsx_pack_raster_records(uint32_t N, const float* means, const float*
                                     const float* opacities, const float* colors, uint32_t channels,
                                     const float* viewmat, const float* K, uint32_t image_width,
                                     uint32_t image_height, void* records, void* stream);
-/* colors is only read for channels beyond the third (channels == 4); nullable otherwise */
+/* The order in which the rasterizers visit the tiles (no counterpart in the reference): tile ids, longest lists
+ * first, so that the short lists fill the end of a launch instead of a few long ones running on alone.  tile_order:
+ * u32 [tile_width * tile_height]; no result depends on it (within a length class the order is unspecified). */
+GSX_API int gsx_tile_order(int64_t n_isects, const int32_t* tile_offsets, uint32_t tile_width, uint32_t tile_height,
+                           uint32_t* tile_order, void* stream);
+/* colors is only read for channels beyond the third (channels == 4); nullable otherwise.  tile_order: nullable (tiles
+ * in index order), else gsx_tile_order's output for these tile_offsets. */
 GSX_API int gsx_rasterize_records_fwd(int64_t n_isects, const void* records, const float* colors, uint32_t channels,
                                       const float* backgrounds, const uint8_t* masks, uint32_t image_width,
                                       uint32_t image_height, const float* viewmat, const float* K,
-                                      const int32_t* tile_offsets, const int32_t* flatten_ids, float* render_colors,
-                                      float* render_alphas, int32_t* last_ids, void* stream);
+                                      const int32_t* tile_offsets, const int32_t* flatten_ids,
+                                      const uint32_t* tile_order, float* render_colors, float* render_alphas,
+                                      int32_t* last_ids, void* stream);
 GSX_API int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
     uint32_t C, uint32_t N, int64_t n_isects, const float* means, const float* quats, const float* scales,
     const float* colors, uint32_t channels, const float* opacities, const float* backgrounds, const uint8_t* masks,
@@ -213,13 +220,15 @@ GSX_API size_t gsx_rasterize_bwd_accum_bytes(uint32_t N);
  * that can also be called one by one (a training loop shares the forward's records and can fold the epilogue into
  * its own per-Gaussian pass); these three take the accumulator part (gsx_rasterize_bwd_accum_bytes) only. */
 GSX_API int gsx_rasterize_bwd_clear(uint32_t N, void* workspace, size_t workspace_bytes, void* stream);
-/* colors [N,channels] is read for a fourth channel only (nullable otherwise) */
+/* colors [N,channels] is read for a fourth channel only (nullable otherwise); tile_order: nullable, see
+ * gsx_tile_order */
 GSX_API int gsx_rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isects, const void* records,
                                          const float* colors, uint32_t channels, const float* backgrounds,
                                          const uint8_t* masks, uint32_t image_width,
                                          uint32_t image_height, uint32_t tile_size, const float* viewmats0,
                                          const float* Ks, const int32_t* tile_offsets, const int32_t* flatten_ids,
-                                         const float* render_alphas, const int32_t* last_ids,
+                                         const uint32_t* tile_order, const float* render_alphas,
+                                         const int32_t* last_ids,
                                          const float* v_render_colors, const float* v_render_alphas, void* workspace,
                                          size_t workspace_bytes, void* stream);
 /* clear_accumulators != 0: the epilogue zeroes each accumulator row after reading it, so the next backward pass

@@ -270,6 +270,47 @@ __global__ void __launch_bounds__(256) tile_emit_kernel(uint32_t n, uint32_t N, 
     }
 }
 
+// ---- visiting order of the tiles for the rasterizers: longest lists first -----------------------------------------
+// The rasterizers' workgroups are handed out in launch order as slots free up; with the long lists first the short
+// ones fill the end of the launch instead of a few long ones running on alone.  Counting sort on a logarithmic
+// length class (16 classes per octave), descending; the order inside a class is whatever the atomics give (no
+// result depends on the order tiles are visited in).
+static constexpr uint32_t kLenClasses = 512;
+__device__ __forceinline__ uint32_t tile_len_class(uint32_t len) {
+    if (len == 0)
+        return 0;
+    const uint32_t e = 31u - (uint32_t)__clz((int)len);
+    const uint32_t m = e >= 4 ? (len >> (e - 4)) & 15u : (len << (4 - e)) & 15u; // four bits below the leading one
+    return e * 16u + m + 1u;
+}
+
+__global__ void __launch_bounds__(1024) tile_order_kernel(uint32_t n_tiles, uint32_t n_isects,
+                                                           const int32_t* __restrict__ tile_offsets,
+                                                           uint32_t* __restrict__ tile_order) {
+    __shared__ uint32_t cursor[kLenClasses];
+    for (uint32_t c = threadIdx.x; c < kLenClasses; c += 1024)
+        cursor[c] = 0;
+    __syncthreads();
+    auto length = [&](uint32_t t) {
+        const uint32_t end = t + 1 < n_tiles ? (uint32_t)tile_offsets[t + 1] : n_isects;
+        return end - (uint32_t)tile_offsets[t];
+    };
+    for (uint32_t t = threadIdx.x; t < n_tiles; t += 1024)
+        atomicAdd(&cursor[tile_len_class(length(t))], 1u);
+    __syncthreads();
+    if (threadIdx.x == 0) { // first position of every class, longest class first
+        uint32_t run = 0;
+        for (int c = (int)kLenClasses - 1; c >= 0; --c) {
+            const uint32_t n = cursor[c];
+            cursor[c] = run;
+            run += n;
+        }
+    }
+    __syncthreads();
+    for (uint32_t t = threadIdx.x; t < n_tiles; t += 1024)
+        tile_order[atomicAdd(&cursor[tile_len_class(length(t))], 1u)] = t;
+}
+
 // IntersectTile.cu:206-252
 __global__ void __launch_bounds__(256) intersect_offset_kernel(uint32_t n_isects,
                                                                 const int64_t* __restrict__ isect_ids, uint32_t C,
@@ -530,6 +571,20 @@ extern "C" int gsx_intersect_tile_emit_ordered(uint32_t N, const float* means2d,
                        (const int64_t*)gsx::ordered_keys(const_cast<void*>(ordered_workspace)), cum_tiles_per_gauss,
                        order, (float)tile_size, tile_width, tile_height, gsx_n_bits(tile_width * tile_height),
                        capacity, isect_ids, flatten_ids);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+extern "C" int gsx_tile_order(int64_t n_isects, const int32_t* tile_offsets, uint32_t tile_width, uint32_t tile_height,
+                              uint32_t* tile_order, void* stream) {
+    const uint64_t n_tiles = (uint64_t)tile_width * tile_height;
+    if (n_tiles == 0)
+        return GSX_OK;
+    GSX_REQUIRE(tile_offsets && tile_order, GSX_ERR_INVALID_ARGUMENT, "tile_order: null tensor");
+    GSX_REQUIRE(n_isects >= 0 && n_isects < (1ll << 31) && n_tiles < (1ull << 31), GSX_ERR_OVERFLOW,
+                "tile_order: sizes out of range");
+    hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, (uint32_t)n_tiles,
+                       (uint32_t)n_isects, tile_offsets, tile_order);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

@@ -55,7 +55,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     uint32_t tile_height, const float* __restrict__ viewmat, const float* __restrict__ Kmat,
     int camera_model, const float* __restrict__ radial, const float* __restrict__ tangential,
     const float* __restrict__ thin_prism, const float* __restrict__ viewmat1, int rs_type,
-    const int32_t* __restrict__ tile_offsets,
+    const int32_t* __restrict__ tile_offsets, const uint32_t* __restrict__ tile_order /*nullable*/,
     const int32_t* __restrict__ flatten_ids,
     const float* __restrict__ render_alphas, const int32_t* __restrict__ last_ids,
     const float* __restrict__ v_render_colors, const float* __restrict__ v_render_alphas,
@@ -71,7 +71,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     __shared__ float acc[kBatch * kAcc];
     __shared__ int32_t block_max;
 
-    const uint32_t tile_id = blockIdx.x;
+    const uint32_t tile_id = tile_order != nullptr ? tile_order[blockIdx.x] : blockIdx.x;
     if (masks != nullptr && !masks[tile_id]) // :83-87
         return;
     const uint32_t tr = threadIdx.x;
@@ -381,7 +381,8 @@ static int rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isects, co
                                     uint32_t tile_size, const float* viewmats0, const float* Ks, int camera_model,
                                     const float* radial, const float* tangential, const float* thin_prism,
                                     const float* viewmats1, int rs_type, const int32_t* tile_offsets,
-                                    const int32_t* flatten_ids, const float* render_alphas, const int32_t* last_ids,
+                                    const uint32_t* tile_order, const int32_t* flatten_ids,
+                                    const float* render_alphas, const int32_t* last_ids,
                                     const float* v_render_colors, const float* v_render_alphas, void* workspace,
                                     size_t workspace_bytes, void* stream) {
     GSX_REQUIRE(C == 1, GSX_ERR_UNSUPPORTED, "C = %u cameras: only C == 1 is supported", C);
@@ -408,8 +409,8 @@ static int rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isects, co
     hipLaunchKernelGGL((rasterize_bwd_kernel<CD, DI>), dim3(tw * th), dim3(256), 0, (hipStream_t)stream,             \
                        (uint32_t)n_isects, (const float4*)records, colors, backgrounds, masks, image_width,          \
                        image_height, tw, th, viewmats0, Ks, camera_model, radial, tangential, thin_prism,            \
-                       viewmats1, rs_type, tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors,      \
-                       v_render_alphas, (float*)workspace, gextra)
+                       viewmats1, rs_type, tile_offsets, tile_order, flatten_ids, render_alphas, last_ids,           \
+                       v_render_colors, v_render_alphas, (float*)workspace, gextra)
 #define GSX_LAUNCH_BWD2(CD)       \
     if (distorted)                \
         GSX_LAUNCH_BWD(CD, true); \
@@ -434,12 +435,14 @@ extern "C" int gsx_rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_is
                                             const uint8_t* masks, uint32_t image_width,
                                             uint32_t image_height, uint32_t tile_size, const float* viewmats0,
                                             const float* Ks, const int32_t* tile_offsets, const int32_t* flatten_ids,
-                                            const float* render_alphas, const int32_t* last_ids,
-                                            const float* v_render_colors, const float* v_render_alphas,
-                                            void* workspace, size_t workspace_bytes, void* stream) {
+                                            const uint32_t* tile_order, const float* render_alphas,
+                                            const int32_t* last_ids, const float* v_render_colors,
+                                            const float* v_render_alphas, void* workspace, size_t workspace_bytes,
+                                            void* stream) {
     return rasterize_bwd_accumulate(C, N, n_isects, records, colors, channels, backgrounds, masks, image_width,
                                     image_height, tile_size, viewmats0, Ks, GSX_PINHOLE, nullptr, nullptr, nullptr,
-                                    nullptr, GSX_GLOBAL, tile_offsets, flatten_ids, render_alphas, last_ids, v_render_colors,
+                                    nullptr, GSX_GLOBAL, tile_offsets, tile_order, flatten_ids, render_alphas, last_ids,
+                                    v_render_colors,
                                     v_render_alphas, workspace, workspace_bytes, stream);
 }
 
@@ -497,7 +500,7 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
         return rc;
     if ((rc = rasterize_bwd_accumulate(C, N, n_isects, records, colors, channels, backgrounds, masks, image_width,
                                        image_height, tile_size, viewmats0, Ks, camera_model, radial_coeffs,
-                                       tangential_coeffs, thin_prism_coeffs, viewmats1, rs_type, tile_offsets,
+                                       tangential_coeffs, thin_prism_coeffs, viewmats1, rs_type, tile_offsets, nullptr,
                                        flatten_ids, render_alphas, last_ids,
                                        v_render_colors, v_render_alphas, workspace, acc_bytes, stream)) != GSX_OK)
         return rc;

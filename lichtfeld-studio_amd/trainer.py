@@ -126,6 +126,7 @@ class TrainStep:
         self.tw, self.th = (W + 15) // 16, (H + 15) // 16
         self._end_bit = 32 + self.lib.gsx_n_bits(c_u32(self.tw * self.th)) + self.lib.gsx_n_bits(c_u32(1))
         self.offsets = e(1, self.th, self.tw, dt=torch.int32)
+        self.tile_order = e(self.th * self.tw, dt=torch.int32)  # the rasterizers' tile visiting order
         self.render = e(1, H, W, 3)
         self.alpha = e(1, H, W, 1)
         self.last_ids = e(1, H, W, dt=torch.int32)
@@ -229,12 +230,18 @@ class TrainStep:
         self.isect_ids, self.flatten_ids = self.keys[self.sel], self.vals[self.sel]
         self._run("intersect_offset", lb.gsx_intersect_offset, c_i64(n), _p(self.isect_ids), c_u32(1), c_u32(self.tw), c_u32(self.th),
                                       _p(self.offsets), s)
+        order = c_p(None)
+        if self.order_tiles:  # longest tile lists first: both rasterizers end with short lists instead of a long tail
+            self._run("tile_order", lb.gsx_tile_order, c_i64(n), _p(self.offsets), c_u32(self.tw), c_u32(self.th),
+                      _p(self.tile_order), s)
+            order = _p(self.tile_order)
+        self._tile_order_arg = order
         if self.side is not None:
             torch.cuda.current_stream(self.dev).wait_event(self.ev_join)  # colours and records are ready
         self._run("rasterize_to_pixels_from_world_3dgs_fwd", lb.gsx_rasterize_records_fwd, c_i64(n),
                   _p(self.records), c_p(None), c_u32(3), _p(self.bg), c_p(None), c_u32(W), c_u32(H), _p(viewmat),
-                  _p(K), _p(self.offsets), _p(self.flatten_ids), _p(self.render), _p(self.alpha), _p(self.last_ids),
-                  s)
+                  _p(K), _p(self.offsets), _p(self.flatten_ids), order, _p(self.render), _p(self.alpha),
+                  _p(self.last_ids), s)
         return self.render
 
     # -- loss ---------------------------------------------------------------------------------------
@@ -294,8 +301,8 @@ class TrainStep:
         self._run("rasterize_bwd_accumulate", lb.gsx_rasterize_bwd_accumulate,
                   c_u32(1), c_u32(N), c_i64(self.n_isects), _p(self.records), c_p(None), c_u32(3), _p(self.bg),
                   c_p(None), c_u32(W), c_u32(H), c_u32(16),
-                  _p(self.viewmat), _p(self.Kmat), _p(self.offsets), _p(self.flatten_ids), _p(self.alpha),
-                  _p(self.last_ids), _p(self.v_render), _p(self.v_alpha), ws, wsn, s)
+                  _p(self.viewmat), _p(self.Kmat), _p(self.offsets), _p(self.flatten_ids), self._tile_order_arg,
+                  _p(self.alpha), _p(self.last_ids), _p(self.v_render), _p(self.v_alpha), ws, wsn, s)
         if self.fused_update:
             return
         self._run("rasterize_bwd_finish", lb.gsx_rasterize_bwd_finish, c_u32(N), _p(P["means"]), _p(A["quats"]),
@@ -366,6 +373,7 @@ class TrainStep:
             arr[i] = g
         self._run("adam_step_multi", self.lib.gsx_adam_step_multi, arr, c_i(len(names)), self._stream())
 
+    order_tiles = True  # visit the tiles longest list first (gsx_tile_order)
     freeze_shN_early = False  # BASELINE's step updates all parameter tensors; set True for the product schedule
 
     # -- MCMC strategy steps that touch the parameters ------------------------------------------------

@@ -233,3 +233,63 @@ def test_speculative_emission_and_overlap_change_nothing(gsx, cuda):
         assert torch.equal(a.loss_out, b.loss_out)
         for k in a.params:
             assert torch.equal(a.params[k], b.params[k]), k
+
+
+def test_tile_visiting_order(gsx, cuda):
+    """gsx_tile_order returns a permutation of the tiles with the list lengths falling from class to class (16 classes
+    per octave); rasterizing in that order changes nothing: forward outputs bit for bit, backward accumulators to
+    atomic-order rounding"""
+    from lichtfeld_studio_amd.trainer import TrainStep
+    sc = gsx.scenes.config(3, 30_000)
+    sc.scaling_raw += 1.0
+    cam = gsx.scenes.orbit_camera(0.4, 4.0, 413, 277, 380.0)
+    W, H = cam.width, cam.height
+    vm = torch.from_numpy(cam.viewmat[None].copy()).to(cuda)
+    Km = torch.from_numpy(cam.K[None].copy()).to(cuda)
+    gt = torch.rand((1, 3, H, W), generator=torch.Generator().manual_seed(5)).to(cuda)
+    a = TrainStep(sc, cuda, fused_update=True, fused_loss=True)
+    b = TrainStep(sc, cuda, fused_update=True, fused_loss=True)
+    a.order_tiles, b.order_tiles = False, True
+    for ts in (a, b):
+        ts.forward(vm, Km, W, H)
+        ts.iteration += 1
+        ts.loss_forward(gt)
+        ts.backward()
+    torch.cuda.synchronize()
+    T = a.tw * a.th
+    order = b.tile_order.cpu().numpy().astype(np.int64)
+    assert np.array_equal(np.sort(order), np.arange(T))
+    off = b.offsets.cpu().numpy().reshape(-1).astype(np.int64)
+    lens = np.diff(np.concatenate([off, [b.n_isects]]))
+    assert lens.max() > 2 * max(1, int(np.median(lens)))  # uneven lists
+    visited = lens[order]
+
+    def klass(n):  # 16 classes per octave
+        if n == 0:
+            return 0
+        e = int(n).bit_length() - 1
+        m = (n >> (e - 4)) & 15 if e >= 4 else (n << (4 - e)) & 15
+        return e * 16 + m + 1
+    classes = np.array([klass(int(n)) for n in visited])
+    assert np.all(np.diff(classes) <= 0)
+    # lists of every size class, empty ones and a few very long ones, through the C ABI alone
+    import ctypes
+    from lichtfeld_studio_amd._lib import c_i64, c_p, c_u32, check, lib
+    rng = np.random.default_rng(1)
+    lens2 = np.concatenate([np.zeros(300, np.int64), rng.integers(0, 40, 3000), rng.integers(0, 5000, 700),
+                            [1, 15, 16, 17, 31, 32, 33, 1 << 20, (1 << 20) + 1, 3 << 19]])
+    rng.shuffle(lens2)
+    tw2, th2 = 401, 10
+    assert lens2.size == tw2 * th2
+    off2 = torch.from_numpy(np.concatenate([[0], np.cumsum(lens2)[:-1]]).astype(np.int32)).to(cuda)
+    out2 = torch.full((lens2.size,), -1, dtype=torch.int32, device=cuda)
+    check(lib().gsx_tile_order(c_i64(int(lens2.sum())), c_p(off2.data_ptr()), c_u32(tw2), c_u32(th2),
+                               c_p(out2.data_ptr()), c_p(torch.cuda.current_stream(cuda).cuda_stream)))
+    o2 = out2.cpu().numpy().astype(np.int64)
+    assert np.array_equal(np.sort(o2), np.arange(lens2.size))
+    assert np.all(np.diff(np.array([klass(int(n)) for n in lens2[o2]])) <= 0)
+    assert lens2[o2[0]] == (1 << 20) + 1 or klass(int(lens2[o2[0]])) == klass(3 << 19)
+    assert torch.equal(a.render, b.render) and torch.equal(a.alpha, b.alpha) and torch.equal(a.last_ids, b.last_ids)
+    ga = a.ws_bwd.view(torch.float32).cpu().numpy().astype(np.float64)
+    gb = b.ws_bwd.view(torch.float32).cpu().numpy().astype(np.float64)
+    assert np.abs(ga).max() > 0 and np.abs(ga - gb).max() <= 1e-4 * np.abs(ga).max()
