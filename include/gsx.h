@@ -177,19 +177,23 @@ GSX_API int gsx_pack_raster_records(uint32_t N, const float* means, const float*
                                     const float* opacities, const float* colors, uint32_t channels,
                                     const float* viewmat, const float* K, uint32_t image_width,
                                     uint32_t image_height, void* records, void* stream);
-/* The order in which the rasterizers visit the tiles (no counterpart in the reference): tile ids, longest lists
- * first, so that the short lists fill the end of a launch instead of a few long ones running on alone.  tile_order:
- * u32 [tile_width * tile_height]; no result depends on it (within a length class the order is unspecified). */
-GSX_API int gsx_tile_order(int64_t n_isects, const int32_t* tile_offsets, uint32_t tile_width, uint32_t tile_height,
-                           uint32_t* tile_order, void* stream);
+/* The order in which the rasterizers visit the tiles (no counterpart in the reference): tile ids, dearest first, so
+ * that the cheap tiles fill the end of a launch instead of a few dear ones running on alone.  A tile's cost is
+ * tile_cost[tile] (u32, e.g. the tile_walk a forward pass left), or with tile_cost == NULL the length of its list in
+ * tile_offsets.  tile_order: u32 [tile_width * tile_height]; no result depends on it (the order inside one of the
+ * logarithmic cost classes is unspecified). */
+GSX_API int gsx_tile_order(int64_t n_isects, const int32_t* tile_offsets, const uint32_t* tile_cost,
+                           uint32_t tile_width, uint32_t tile_height, uint32_t* tile_order, void* stream);
 /* colors is only read for channels beyond the third (channels == 4); nullable otherwise.  tile_order: nullable (tiles
- * in index order), else gsx_tile_order's output for these tile_offsets. */
+ * in index order), else any permutation of the tile ids (gsx_tile_order).  tile_walk: nullable, u32 [tiles]: receives
+ * per tile how far its pixels went into the list (entries up to the last contributor, 0 = none) - what the tile cost
+ * this pass and will cost the backward pass. */
 GSX_API int gsx_rasterize_records_fwd(int64_t n_isects, const void* records, const float* colors, uint32_t channels,
                                       const float* backgrounds, const uint8_t* masks, uint32_t image_width,
                                       uint32_t image_height, const float* viewmat, const float* K,
                                       const int32_t* tile_offsets, const int32_t* flatten_ids,
-                                      const uint32_t* tile_order, float* render_colors, float* render_alphas,
-                                      int32_t* last_ids, void* stream);
+                                      const uint32_t* tile_order, uint32_t* tile_walk, float* render_colors,
+                                      float* render_alphas, int32_t* last_ids, void* stream);
 GSX_API int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
     uint32_t C, uint32_t N, int64_t n_isects, const float* means, const float* quats, const float* scales,
     const float* colors, uint32_t channels, const float* opacities, const float* backgrounds, const uint8_t* masks,

@@ -286,12 +286,15 @@ __device__ __forceinline__ uint32_t tile_len_class(uint32_t len) {
 
 __global__ void __launch_bounds__(1024) tile_order_kernel(uint32_t n_tiles, uint32_t n_isects,
                                                            const int32_t* __restrict__ tile_offsets,
+                                                           const uint32_t* __restrict__ tile_cost /*nullable*/,
                                                            uint32_t* __restrict__ tile_order) {
     __shared__ uint32_t cursor[kLenClasses];
     for (uint32_t c = threadIdx.x; c < kLenClasses; c += 1024)
         cursor[c] = 0;
     __syncthreads();
     auto length = [&](uint32_t t) {
+        if (tile_cost != nullptr)
+            return tile_cost[t];
         const uint32_t end = t + 1 < n_tiles ? (uint32_t)tile_offsets[t + 1] : n_isects;
         return end - (uint32_t)tile_offsets[t];
     };
@@ -575,16 +578,16 @@ extern "C" int gsx_intersect_tile_emit_ordered(uint32_t N, const float* means2d,
     return GSX_OK;
 }
 
-extern "C" int gsx_tile_order(int64_t n_isects, const int32_t* tile_offsets, uint32_t tile_width, uint32_t tile_height,
-                              uint32_t* tile_order, void* stream) {
+extern "C" int gsx_tile_order(int64_t n_isects, const int32_t* tile_offsets, const uint32_t* tile_cost,
+                              uint32_t tile_width, uint32_t tile_height, uint32_t* tile_order, void* stream) {
     const uint64_t n_tiles = (uint64_t)tile_width * tile_height;
     if (n_tiles == 0)
         return GSX_OK;
-    GSX_REQUIRE(tile_offsets && tile_order, GSX_ERR_INVALID_ARGUMENT, "tile_order: null tensor");
+    GSX_REQUIRE((tile_offsets || tile_cost) && tile_order, GSX_ERR_INVALID_ARGUMENT, "tile_order: null tensor");
     GSX_REQUIRE(n_isects >= 0 && n_isects < (1ll << 31) && n_tiles < (1ull << 31), GSX_ERR_OVERFLOW,
                 "tile_order: sizes out of range");
     hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, (uint32_t)n_tiles,
-                       (uint32_t)n_isects, tile_offsets, tile_order);
+                       (uint32_t)n_isects, tile_offsets, tile_cost, tile_order);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

@@ -60,7 +60,8 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
     const float* __restrict__ tangential, const float* __restrict__ thin_prism,
     const float* __restrict__ viewmat1, int rs_type, const int32_t* __restrict__ tile_offsets,
     const int32_t* __restrict__ flatten_ids, const uint32_t* __restrict__ tile_order /*nullable*/,
-    float* __restrict__ render_colors, float* __restrict__ render_alphas,
+    uint32_t* __restrict__ tile_walk /*nullable*/, float* __restrict__ render_colors,
+    float* __restrict__ render_alphas,
     int32_t* __restrict__ last_ids, unsigned long long* __restrict__ stats) {
     __shared__ float4 stage[kBatch * 4];
     __shared__ float4 region[kBatch * 2];
@@ -228,6 +229,24 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
                 backgrounds == nullptr ? pix_out[k] : fma(T, backgrounds[k], pix_out[k]);
         last_ids[pix_id] = (int32_t)cur_idx;
     }
+    if (tile_walk != nullptr) {
+        // how far into its list this tile's pixels went (entries up to the last contributor): what the tile costs
+        // either rasterizer, for the visiting order of later launches
+        __shared__ uint32_t walk_s;
+        if (tr == 0)
+            walk_s = 0;
+        __syncthreads();
+        uint32_t w = (inside && cur_idx >= (uint32_t)range_start && range_end > range_start && T < 1.0f)
+                         ? cur_idx - (uint32_t)range_start + 1u : 0u;
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1)
+            w = max(w, (uint32_t)__shfl_xor((int)w, m, 64));
+        if ((tr & 63u) == 0)
+            atomicMax(&walk_s, w);
+        __syncthreads();
+        if (tr == 0)
+            tile_walk[tile_id] = walk_s;
+    }
 }
 
 } // namespace gsx
@@ -269,7 +288,8 @@ int rasterize_records_fwd(int64_t n_isects, const void* records, const float* co
                           const float* viewmat, const float* K, int camera_model, const float* radial,
                           const float* tangential, const float* thin_prism, const float* viewmat1, int rs_type,
                           const int32_t* tile_offsets, const int32_t* flatten_ids, const uint32_t* tile_order,
-                          float* render_colors, float* render_alphas, int32_t* last_ids, void* stream) {
+                          uint32_t* tile_walk, float* render_colors, float* render_alphas, int32_t* last_ids,
+                          void* stream) {
     if (image_width == 0 || image_height == 0)
         return GSX_OK;
     GSX_REQUIRE(n_isects >= 0 && n_isects < (1ll << 31), GSX_ERR_OVERFLOW, "rasterize fwd: n_isects out of range");
@@ -286,7 +306,8 @@ int rasterize_records_fwd(int64_t n_isects, const void* records, const float* co
     hipLaunchKernelGGL((rasterize_fwd_kernel<CD, false, DI>), grid, block, 0, s, (uint32_t)n_isects,                \
                        (const float4*)records, colors, backgrounds, masks, image_width, image_height, tw, th,       \
                        viewmat, K, camera_model, radial, tangential, thin_prism, viewmat1, rs_type, tile_offsets,   \
-                       flatten_ids, tile_order, render_colors, render_alphas, last_ids, (unsigned long long*)nullptr)
+                       flatten_ids, tile_order, tile_walk, render_colors, render_alphas, last_ids,                  \
+                       (unsigned long long*)nullptr)
 #define GSX_LAUNCH_FWD2(CD)     \
     if (distorted)              \
         GSX_LAUNCH_FWD(CD, true); \
@@ -319,11 +340,11 @@ extern "C" int gsx_rasterize_records_fwd(int64_t n_isects, const void* records, 
                                          uint32_t channels, const float* backgrounds, const uint8_t* masks,
                                          uint32_t image_width, uint32_t image_height, const float* viewmat,
                                          const float* K, const int32_t* tile_offsets, const int32_t* flatten_ids,
-                                         const uint32_t* tile_order, float* render_colors, float* render_alphas,
-                                         int32_t* last_ids, void* stream) {
+                                         const uint32_t* tile_order, uint32_t* tile_walk, float* render_colors,
+                                         float* render_alphas, int32_t* last_ids, void* stream) {
     return rasterize_records_fwd(n_isects, records, colors, channels, backgrounds, masks, image_width, image_height,
                                  viewmat, K, GSX_PINHOLE, nullptr, nullptr, nullptr, nullptr, GSX_GLOBAL, tile_offsets,
-                                 flatten_ids, tile_order, render_colors, render_alphas, last_ids, stream);
+                                 flatten_ids, tile_order, tile_walk, render_colors, render_alphas, last_ids, stream);
 }
 
 extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
@@ -361,8 +382,8 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
     }
     return rasterize_records_fwd(n_isects, workspace, colors, channels, backgrounds, masks, image_width, image_height,
                                  viewmats0, Ks, camera_model, radial_coeffs, tangential_coeffs, thin_prism_coeffs,
-                                 viewmats1, rs_type, tile_offsets, flatten_ids, nullptr, render_colors, render_alphas,
-                                 last_ids, stream);
+                                 viewmats1, rs_type, tile_offsets, flatten_ids, nullptr, nullptr, render_colors,
+                                 render_alphas, last_ids, stream);
 }
 
 // Pair counts of one forward pass (no counterpart in the reference; used to turn kernel times into flop rates).
@@ -379,7 +400,8 @@ extern "C" int gsx_rasterize_pair_stats(int64_t n_isects, const void* records, u
                        (uint32_t)n_isects, (const float4*)records, (const float*)nullptr, (const float*)nullptr,
                        (const uint8_t*)nullptr, image_width, image_height, tw, th, viewmat, K, (int)GSX_PINHOLE,
                        (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
-                       (int)GSX_GLOBAL, tile_offsets, flatten_ids, (const uint32_t*)nullptr, (float*)nullptr,
+                       (int)GSX_GLOBAL, tile_offsets, flatten_ids, (const uint32_t*)nullptr, (uint32_t*)nullptr,
+                       (float*)nullptr,
                        (float*)nullptr, (int32_t*)nullptr, stats_out);
     GSX_LAUNCH_CHECK();
     return GSX_OK;

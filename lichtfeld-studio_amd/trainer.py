@@ -127,6 +127,8 @@ class TrainStep:
         self._end_bit = 32 + self.lib.gsx_n_bits(c_u32(self.tw * self.th)) + self.lib.gsx_n_bits(c_u32(1))
         self.offsets = e(1, self.th, self.tw, dt=torch.int32)
         self.tile_order = e(self.th * self.tw, dt=torch.int32)  # the rasterizers' tile visiting order
+        self.tile_walk = e(self.th * self.tw, dt=torch.int32)   # per tile: entries up to its last contributor
+        self.have_walk = False
         self.render = e(1, H, W, 3)
         self.alpha = e(1, H, W, 1)
         self.last_ids = e(1, H, W, dt=torch.int32)
@@ -230,18 +232,26 @@ class TrainStep:
         self.isect_ids, self.flatten_ids = self.keys[self.sel], self.vals[self.sel]
         self._run("intersect_offset", lb.gsx_intersect_offset, c_i64(n), _p(self.isect_ids), c_u32(1), c_u32(self.tw), c_u32(self.th),
                                       _p(self.offsets), s)
+        # Dearest tiles first: both rasterizers then end with cheap tiles instead of a long tail.  What a tile costs is
+        # how far its pixels go into the list, which the forward pass itself reports; the forward pass therefore
+        # uses the order of the previous step (the first one: by list length), the backward pass this step's.
         order = c_p(None)
-        if self.order_tiles:  # longest tile lists first: both rasterizers end with short lists instead of a long tail
-            self._run("tile_order", lb.gsx_tile_order, c_i64(n), _p(self.offsets), c_u32(self.tw), c_u32(self.th),
-                      _p(self.tile_order), s)
+        if self.order_tiles:
+            if not self.have_walk:
+                self._run("tile_order", lb.gsx_tile_order, c_i64(n), _p(self.offsets), c_p(None), c_u32(self.tw),
+                          c_u32(self.th), _p(self.tile_order), s)
             order = _p(self.tile_order)
         self._tile_order_arg = order
         if self.side is not None:
             torch.cuda.current_stream(self.dev).wait_event(self.ev_join)  # colours and records are ready
         self._run("rasterize_to_pixels_from_world_3dgs_fwd", lb.gsx_rasterize_records_fwd, c_i64(n),
                   _p(self.records), c_p(None), c_u32(3), _p(self.bg), c_p(None), c_u32(W), c_u32(H), _p(viewmat),
-                  _p(K), _p(self.offsets), _p(self.flatten_ids), order, _p(self.render), _p(self.alpha),
-                  _p(self.last_ids), s)
+                  _p(K), _p(self.offsets), _p(self.flatten_ids), order, _p(self.tile_walk) if self.order_tiles else
+                  c_p(None), _p(self.render), _p(self.alpha), _p(self.last_ids), s)
+        if self.order_tiles:
+            self._run("tile_order", lb.gsx_tile_order, c_i64(n), c_p(None), _p(self.tile_walk), c_u32(self.tw),
+                      c_u32(self.th), _p(self.tile_order), s)
+            self.have_walk = True
         return self.render
 
     # -- loss ---------------------------------------------------------------------------------------

@@ -259,10 +259,20 @@ def test_tile_visiting_order(gsx, cuda):
     T = a.tw * a.th
     order = b.tile_order.cpu().numpy().astype(np.int64)
     assert np.array_equal(np.sort(order), np.arange(T))
+    # after the forward pass the order is by what the pass reported per tile: entries up to the last contributor
     off = b.offsets.cpu().numpy().reshape(-1).astype(np.int64)
-    lens = np.diff(np.concatenate([off, [b.n_isects]]))
-    assert lens.max() > 2 * max(1, int(np.median(lens)))  # uneven lists
-    visited = lens[order]
+    last = b.last_ids.cpu().numpy()[0].astype(np.int64)
+    alpha = b.alpha.cpu().numpy()[0, :, :, 0]
+    walk = np.zeros(T, np.int64)
+    for ty in range(b.th):
+        for tx in range(b.tw):
+            blk = (slice(ty * 16, (ty + 1) * 16), slice(tx * 16, (tx + 1) * 16))
+            hit = alpha[blk] > 0
+            if hit.any():
+                walk[ty * b.tw + tx] = last[blk][hit].max() - off[ty * b.tw + tx] + 1
+    assert np.array_equal(b.tile_walk.cpu().numpy().astype(np.int64), walk)
+    assert walk.max() > 2 * max(1, int(np.median(walk)))  # uneven costs
+    visited = walk[order]
 
     def klass(n):  # 16 classes per octave
         if n == 0:
@@ -283,12 +293,16 @@ def test_tile_visiting_order(gsx, cuda):
     assert lens2.size == tw2 * th2
     off2 = torch.from_numpy(np.concatenate([[0], np.cumsum(lens2)[:-1]]).astype(np.int32)).to(cuda)
     out2 = torch.full((lens2.size,), -1, dtype=torch.int32, device=cuda)
-    check(lib().gsx_tile_order(c_i64(int(lens2.sum())), c_p(off2.data_ptr()), c_u32(tw2), c_u32(th2),
-                               c_p(out2.data_ptr()), c_p(torch.cuda.current_stream(cuda).cuda_stream)))
-    o2 = out2.cpu().numpy().astype(np.int64)
-    assert np.array_equal(np.sort(o2), np.arange(lens2.size))
-    assert np.all(np.diff(np.array([klass(int(n)) for n in lens2[o2]])) <= 0)
-    assert lens2[o2[0]] == (1 << 20) + 1 or klass(int(lens2[o2[0]])) == klass(3 << 19)
+    stream = c_p(torch.cuda.current_stream(cuda).cuda_stream)
+    cost2 = torch.from_numpy(lens2.astype(np.int32)).to(cuda)
+    for offsets_arg, cost_arg in ((c_p(off2.data_ptr()), c_p(None)), (c_p(None), c_p(cost2.data_ptr()))):
+        out2.fill_(-1)
+        check(lib().gsx_tile_order(c_i64(int(lens2.sum())), offsets_arg, cost_arg, c_u32(tw2), c_u32(th2),
+                                   c_p(out2.data_ptr()), stream))
+        o2 = out2.cpu().numpy().astype(np.int64)
+        assert np.array_equal(np.sort(o2), np.arange(lens2.size))
+        assert np.all(np.diff(np.array([klass(int(n)) for n in lens2[o2]])) <= 0)
+        assert klass(int(lens2[o2[0]])) == klass(3 << 19)
     assert torch.equal(a.render, b.render) and torch.equal(a.alpha, b.alpha) and torch.equal(a.last_ids, b.last_ids)
     ga = a.ws_bwd.view(torch.float32).cpu().numpy().astype(np.float64)
     gb = b.ws_bwd.view(torch.float32).cpu().numpy().astype(np.float64)
