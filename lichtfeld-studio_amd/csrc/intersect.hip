@@ -301,12 +301,26 @@ __global__ void __launch_bounds__(1024) tile_order_kernel(uint32_t n_tiles, uint
     for (uint32_t t = threadIdx.x; t < n_tiles; t += 1024)
         atomicAdd(&cursor[tile_len_class(length(t))], 1u);
     __syncthreads();
-    if (threadIdx.x == 0) { // first position of every class, longest class first
-        uint32_t run = 0;
-        for (int c = (int)kLenClasses - 1; c >= 0; --c) {
-            const uint32_t n = cursor[c];
-            cursor[c] = run;
-            run += n;
+    { // first position of every class, dearest class first: an exclusive scan over the classes in descending order
+        __shared__ uint32_t wave_total[kLenClasses / 64];
+        const uint32_t t = threadIdx.x, lane = t & 63u, w = t >> 6;
+        const uint32_t c = kLenClasses - 1u - t; // thread t owns class c (t < kLenClasses)
+        const uint32_t n = t < kLenClasses ? cursor[c] : 0u;
+        uint32_t incl = n;
+#pragma unroll
+        for (uint32_t off = 1; off < 64; off <<= 1) {
+            const uint32_t up = (uint32_t)__shfl_up((int)incl, off, 64);
+            if (lane >= off)
+                incl += up;
+        }
+        if (lane == 63 && w < kLenClasses / 64)
+            wave_total[w] = incl;
+        __syncthreads();
+        if (t < kLenClasses) {
+            uint32_t before = 0;
+            for (uint32_t k = 0; k < w; ++k)
+                before += wave_total[k];
+            cursor[c] = before + incl - n;
         }
     }
     __syncthreads();
