@@ -48,7 +48,9 @@ GSX_API int gsx_fastgs_preprocess(uint32_t N, const float* means, const float* s
                                   int wait, void* stream);
 /* create_instances_cu, tile sort, instance ranges, blend_cu (kernels_forward.cuh:220-459; src/forward.cu:125-196).
  * background (nullable, 3 floats on the device): image += (1 - alpha) * background as fast_rasterizer.cpp:63 does
- * after the kernel. */
+ * after the kernel.  pixel_state receives per pixel the final transmittance and the number of list entries the
+ * backward replays, and per tile how far its pixels went into the list plus the tile order the backward visits
+ * (dearest tiles first, so that its launch ends with cheap tiles). */
 GSX_API int gsx_fastgs_render(uint32_t N, const gsx_fastgs_settings* settings, const void* primitive_state,
                               size_t primitive_state_bytes, int64_t n_instances, void* instance_state,
                               size_t instance_state_bytes, const float* background, float* image, float* alpha,

@@ -409,9 +409,10 @@ __global__ void __launch_bounds__(256) fgs_blend_fwd_kernel(
     uint32_t n_instances, const float4* __restrict__ prims, const int32_t* __restrict__ tile_offsets,
     const int32_t* __restrict__ inst, uint32_t width, uint32_t height, uint32_t grid_w, uint32_t n_tiles,
     const float* __restrict__ background, float* __restrict__ image, float* __restrict__ alpha_map,
-    float* __restrict__ t_final, uint32_t* __restrict__ n_contributions) {
+    float* __restrict__ t_final, uint32_t* __restrict__ n_contributions, uint32_t* __restrict__ tile_walk) {
     __shared__ float4 stage[kBatch * kFgsPrimF4];
     __shared__ uint8_t lists[4][kBatch];
+    __shared__ uint32_t walk_s;
     const uint32_t tile_id = blockIdx.x;
     const uint32_t tr = threadIdx.x;
     const TilePixel px = tile_pixel(tile_id, grid_w, tr);
@@ -472,6 +473,19 @@ __global__ void __launch_bounds__(256) fgs_blend_fwd_kernel(
         t_final[p] = T;
         n_contributions[p] = n_contrib;
     }
+    // how far into its list the tile's pixels went: what the tile costs the backward pass
+    if (tr == 0)
+        walk_s = 0;
+    __syncthreads();
+    uint32_t w = inside ? n_contrib : 0u;
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1)
+        w = max(w, (uint32_t)__shfl_xor((int)w, m, 64));
+    if ((tr & 63u) == 0)
+        atomicMax(&walk_s, w);
+    __syncthreads();
+    if (tr == 0)
+        tile_walk[tile_id] = walk_s;
 }
 
 // blend_backward_cu (kernels_backward.cuh:240-449) as a back-to-front walk per pixel; per Gaussian and wave the
@@ -481,13 +495,14 @@ __global__ void __launch_bounds__(256) fgs_blend_bwd_kernel(
     uint32_t n_instances, const float4* __restrict__ prims, const int32_t* __restrict__ tile_offsets,
     const int32_t* __restrict__ inst, uint32_t width, uint32_t height, uint32_t grid_w, uint32_t n_tiles,
     const float* __restrict__ background, const float* __restrict__ t_final, const uint32_t* __restrict__ n_contributions,
-    const float* __restrict__ grad_image, const float* __restrict__ grad_alpha, float* __restrict__ gacc) {
+    const float* __restrict__ grad_image, const float* __restrict__ grad_alpha,
+    const uint32_t* __restrict__ tile_order, float* __restrict__ gacc) {
     __shared__ float4 stage[kBatch * kFgsPrimF4];
     __shared__ uint8_t lists[4][kBatch];
     __shared__ int32_t id_batch[kBatch];
     __shared__ float acc[kBatch * kFgsAcc];
     __shared__ int32_t block_max;
-    const uint32_t tile_id = blockIdx.x;
+    const uint32_t tile_id = tile_order[blockIdx.x]; // dearest tiles first
     const uint32_t tr = threadIdx.x, lane = tr & 63u;
     const TilePixel px = tile_pixel(tile_id, grid_w, tr);
     const bool inside = px.i < height && px.j < width;
@@ -877,8 +892,11 @@ extern "C" size_t gsx_fastgs_primitive_state_bytes(uint32_t N) { return fgs_prim
 extern "C" size_t gsx_fastgs_instance_state_bytes(int64_t n_instances, uint32_t width, uint32_t height) {
     return fgs_inst_layout(n_instances, ((width + kTile - 1) / kTile) * ((height + kTile - 1) / kTile)).total;
 }
+// final transmittance, number of list entries replayed per pixel; per tile how far its pixels went into the list
+// and the order in which the backward visits the tiles (dearest first)
 extern "C" size_t gsx_fastgs_pixel_state_bytes(uint32_t width, uint32_t height) {
-    return 2 * align_up((size_t)width * height * 4, 256);
+    const size_t n_tiles = (size_t)((width + kTile - 1) / kTile) * ((height + kTile - 1) / kTile);
+    return 2 * align_up((size_t)width * height * 4, 256) + 2 * align_up(n_tiles * 4, 256);
 }
 extern "C" size_t gsx_fastgs_accum_bytes(uint32_t N) { return align_up((size_t)N * kFgsAcc * 4, 256) + 256; }
 
@@ -959,12 +977,17 @@ extern "C" int gsx_fastgs_render(uint32_t N, const gsx_fastgs_settings* settings
     if ((rc = gsx_intersect_offset(n_instances, sel ? keys1 : keys0, 1, gw, gh, offsets, stream)) != GSX_OK)
         return rc;
     char* px = (char*)pixel_state;
+    const size_t plane = align_up((size_t)W * H * 4, 256);
     float* t_final = (float*)px;
-    uint32_t* n_contrib = (uint32_t*)(px + align_up((size_t)W * H * 4, 256));
+    uint32_t* n_contrib = (uint32_t*)(px + plane);
+    uint32_t* tile_walk = (uint32_t*)(px + 2 * plane);
+    uint32_t* tile_order = (uint32_t*)(px + 2 * plane + align_up((size_t)n_tiles * 4, 256));
     hipLaunchKernelGGL(fgs_blend_fwd_kernel, dim3(n_tiles), dim3(256), 0, s, (uint32_t)n_instances, (const float4*)ps,
-                       offsets, sel ? vals1 : vals0, W, H, gw, n_tiles, background, image, alpha, t_final, n_contrib);
+                       offsets, sel ? vals1 : vals0, W, H, gw, n_tiles, background, image, alpha, t_final, n_contrib,
+                       tile_walk);
     GSX_LAUNCH_CHECK();
-    return GSX_OK;
+    // the backward's visiting order: tiles whose pixels went furthest into their lists first
+    return gsx_tile_order(n_instances, nullptr, tile_walk, gw, gh, tile_order, stream);
 }
 
 extern "C" int gsx_fastgs_primitive_records(uint32_t N, const void* primitive_state, const float** records,
@@ -1039,6 +1062,8 @@ extern "C" int gsx_fastgs_backward(uint32_t N, const float* means, const float* 
         hipLaunchKernelGGL(fgs_blend_bwd_kernel, dim3(n_tiles), dim3(256), 0, s, (uint32_t)n_instances, (const float4*)ps,
                            offsets, inst, W, H, c.grid_w, n_tiles, background, (const float*)px,
                            (const uint32_t*)(px + align_up((size_t)W * H * 4, 256)), grad_image, grad_alpha,
+                           (const uint32_t*)(px + 2 * align_up((size_t)W * H * 4, 256) +
+                                             align_up((size_t)n_tiles * 4, 256)),
                            (float*)accum);
         GSX_LAUNCH_CHECK();
     }
