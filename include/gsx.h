@@ -184,6 +184,10 @@ GSX_API int gsx_pack_raster_records(uint32_t N, const float* means, const float*
  * logarithmic cost classes is unspecified). */
 GSX_API int gsx_tile_order(int64_t n_isects, const int32_t* tile_offsets, const uint32_t* tile_cost,
                            uint32_t tile_width, uint32_t tile_height, uint32_t* tile_order, void* stream);
+/* The whole-operator rasterizer entry points (gsx_rasterize_to_pixels_from_world_3dgs_fwd / _bwd) order their tiles
+ * themselves when the workspace they are given is this much larger than their own requirement: the forward by list
+ * length, the backward by the cost read from render_alphas / last_ids. */
+GSX_API size_t gsx_tile_order_bytes(uint32_t tile_width, uint32_t tile_height);
 /* colors is only read for channels beyond the third (channels == 4); nullable otherwise.  tile_order: nullable (tiles
  * in index order), else any permutation of the tile ids (gsx_tile_order).  tile_walk: nullable, u32 [tiles]: receives
  * per tile how far its pixels went into the list (entries up to the last contributor, 0 = none) - what the tile cost

@@ -45,6 +45,10 @@ static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; 
 // sorted keys stay in ordered_keys(ws).  rect_keys: the high words are packed tile rectangles
 // (x0 | y0 << 8 | x1 << 16 | y1 << 24, 0 = none) instead of counts.
 int64_t* ordered_keys(void* workspace);
+// intersect.hip: the tile visiting order of a backward pass from the forward pass's per-pixel outputs
+int tile_order_from_pixels(int64_t n_isects, uint32_t image_width, uint32_t image_height, const int32_t* tile_offsets,
+                           const float* render_alphas, const int32_t* last_ids, void* scratch,
+                           const uint32_t** tile_order, void* stream);
 int ordered_counts_from_keys(const char* who, uint32_t N, int32_t* order, int64_t* cum_tiles_per_gauss, void* workspace,
                              size_t workspace_bytes, int64_t* n_isects_host, int wait, void* stream,
                              bool rect_keys = false);

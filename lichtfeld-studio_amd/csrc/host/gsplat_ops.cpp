@@ -373,7 +373,8 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> rasterize_to_pixels_from_world_3d
     at::Tensor renders = at::empty({C, image_height, image_width, channels}, opt);
     at::Tensor alphas = at::empty({C, image_height, image_width, 1}, opt);
     at::Tensor last_ids = at::empty({C, image_height, image_width}, opt.dtype(at::kInt));
-    at::Tensor ws = workspace(gsx_raster_records_bytes(N), means);
+    // records + room for the tile visiting order
+    at::Tensor ws = workspace(gsx_raster_records_bytes(N) + gsx_tile_order_bytes((uint32_t)tw, (uint32_t)th), means);
     const int st = gsx_rasterize_to_pixels_from_world_3dgs_fwd(
         C, N, flatten_ids.size(0), means.data_ptr<float>(), quats.data_ptr<float>(), scales.data_ptr<float>(),
         colors.data_ptr<float>(), channels, opacities.data_ptr<float>(), fptr(backgrounds), bptr(masks), image_width,
@@ -438,7 +439,8 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> rasterize
     // the kernels write every element of the five outputs (the reference zero-fills, Rasterization.cpp:190-194)
     at::Tensor v_means = at::empty_like(means), v_quats = at::empty_like(quats), v_scales = at::empty_like(scales);
     at::Tensor v_colors = at::empty_like(colors), v_opacities = at::empty_like(opacities);
-    at::Tensor ws = workspace(gsx_rasterize_bwd_workspace_bytes(N), means);
+    at::Tensor ws = workspace(gsx_rasterize_bwd_workspace_bytes(N) + gsx_tile_order_bytes((uint32_t)tw, (uint32_t)th),
+                              means); // + room for the tile visiting order
     gsx_check(gsx_rasterize_to_pixels_from_world_3dgs_bwd(
         C, N, flatten_ids.size(0), means.data_ptr<float>(), quats.data_ptr<float>(), scales.data_ptr<float>(),
         colors.data_ptr<float>(), channels, opacities.data_ptr<float>(), fptr(backgrounds), bptr(masks), image_width,

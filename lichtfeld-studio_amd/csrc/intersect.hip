@@ -328,6 +328,36 @@ __global__ void __launch_bounds__(1024) tile_order_kernel(uint32_t n_tiles, uint
         tile_order[atomicAdd(&cursor[tile_len_class(length(t))], 1u)] = t;
 }
 
+// What a forward pass leaves per pixel (alpha, position of the last contributor) gives the tile cost too: how far
+// the tile's pixels went into its list.  One workgroup per tile.
+__global__ void __launch_bounds__(256) tile_walk_kernel(uint32_t image_width, uint32_t image_height,
+                                                         uint32_t tile_width, const int32_t* __restrict__ tile_offsets,
+                                                         const float* __restrict__ render_alphas,
+                                                         const int32_t* __restrict__ last_ids,
+                                                         uint32_t* __restrict__ tile_walk) {
+    __shared__ uint32_t walk_s;
+    const uint32_t tile_id = blockIdx.x, tr = threadIdx.x;
+    if (tr == 0)
+        walk_s = 0;
+    __syncthreads();
+    const TilePixel px = tile_pixel(tile_id, tile_width, tr);
+    uint32_t w = 0;
+    if (px.i < image_height && px.j < image_width) {
+        const size_t p = (size_t)px.i * image_width + px.j;
+        const int32_t start = tile_offsets[tile_id];
+        if (render_alphas[p] > 0.0f && last_ids[p] >= start)
+            w = (uint32_t)(last_ids[p] - start) + 1u;
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1)
+        w = max(w, (uint32_t)__shfl_xor((int)w, m, 64));
+    if ((tr & 63u) == 0)
+        atomicMax(&walk_s, w);
+    __syncthreads();
+    if (tr == 0)
+        tile_walk[tile_id] = walk_s;
+}
+
 // IntersectTile.cu:206-252
 __global__ void __launch_bounds__(256) intersect_offset_kernel(uint32_t n_isects,
                                                                 const int64_t* __restrict__ isect_ids, uint32_t C,
@@ -591,6 +621,26 @@ extern "C" int gsx_intersect_tile_emit_ordered(uint32_t N, const float* means2d,
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }
+
+extern "C" size_t gsx_tile_order_bytes(uint32_t tile_width, uint32_t tile_height) {
+    return 2 * align_up((size_t)tile_width * tile_height * 4, 256);
+}
+
+namespace gsx {
+// the order for a backward pass from what the forward pass left per pixel; scratch: gsx_tile_order_bytes
+int tile_order_from_pixels(int64_t n_isects, uint32_t image_width, uint32_t image_height, const int32_t* tile_offsets,
+                           const float* render_alphas, const int32_t* last_ids, void* scratch,
+                           const uint32_t** tile_order, void* stream) {
+    const uint32_t tw = cdiv(image_width, kTile), th = cdiv(image_height, kTile);
+    uint32_t* walk = (uint32_t*)scratch;
+    uint32_t* order = (uint32_t*)((char*)scratch + align_up((size_t)tw * th * 4, 256));
+    hipLaunchKernelGGL(tile_walk_kernel, dim3(tw * th), dim3(256), 0, (hipStream_t)stream, image_width, image_height,
+                       tw, tile_offsets, render_alphas, last_ids, walk);
+    GSX_LAUNCH_CHECK();
+    *tile_order = order;
+    return gsx_tile_order(n_isects, nullptr, walk, tw, th, order, stream);
+}
+} // namespace gsx
 
 extern "C" int gsx_tile_order(int64_t n_isects, const int32_t* tile_offsets, const uint32_t* tile_cost,
                               uint32_t tile_width, uint32_t tile_height, uint32_t* tile_order, void* stream) {

@@ -498,10 +498,19 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
     if ((rc = pack_raster_records(N, means, quats, scales, opacities, colors, channels, viewmats0, Ks, image_width,
                                   image_height, pinhole, rolling, records, stream)) != GSX_OK)
         return rc;
+    // room behind the records for a tile order: visit the tiles dearest first (cost from the forward's outputs)
+    const uint32_t* tile_order = nullptr;
+    const size_t base_bytes = gsx_rasterize_bwd_workspace_bytes(N);
+    if (n_isects > 0 && tile_size == kTile && tile_offsets && render_alphas && last_ids &&
+        workspace_bytes >= base_bytes + gsx_tile_order_bytes(cdiv(image_width, kTile), cdiv(image_height, kTile))) {
+        if ((rc = tile_order_from_pixels(n_isects, image_width, image_height, tile_offsets, render_alphas, last_ids,
+                                         (char*)workspace + base_bytes, &tile_order, stream)) != GSX_OK)
+            return rc;
+    }
     if ((rc = rasterize_bwd_accumulate(C, N, n_isects, records, colors, channels, backgrounds, masks, image_width,
                                        image_height, tile_size, viewmats0, Ks, camera_model, radial_coeffs,
-                                       tangential_coeffs, thin_prism_coeffs, viewmats1, rs_type, tile_offsets, nullptr,
-                                       flatten_ids, render_alphas, last_ids,
+                                       tangential_coeffs, thin_prism_coeffs, viewmats1, rs_type, tile_offsets,
+                                       tile_order, flatten_ids, render_alphas, last_ids,
                                        v_render_colors, v_render_alphas, workspace, acc_bytes, stream)) != GSX_OK)
         return rc;
     return gsx_rasterize_bwd_finish(N, means, quats, scales, viewmats0, workspace, acc_bytes, 0, channels, v_means,

@@ -380,9 +380,19 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
                                       image_height, pinhole, rolling, workspace, stream)) != GSX_OK)
             return rc;
     }
+    // room behind the records for a tile order: visit the tiles longest list first
+    const uint32_t* tile_order = nullptr;
+    const uint32_t tw = cdiv(image_width, kTile), th = cdiv(image_height, kTile);
+    const size_t rec_bytes = gsx_raster_records_bytes(N);
+    if (n_isects > 0 && tile_offsets != nullptr && workspace_bytes >= rec_bytes + gsx_tile_order_bytes(tw, th)) {
+        uint32_t* order = (uint32_t*)((char*)workspace + rec_bytes);
+        if ((rc = gsx_tile_order(n_isects, tile_offsets, nullptr, tw, th, order, stream)) != GSX_OK)
+            return rc;
+        tile_order = order;
+    }
     return rasterize_records_fwd(n_isects, workspace, colors, channels, backgrounds, masks, image_width, image_height,
                                  viewmats0, Ks, camera_model, radial_coeffs, tangential_coeffs, thin_prism_coeffs,
-                                 viewmats1, rs_type, tile_offsets, flatten_ids, nullptr, nullptr, render_colors,
+                                 viewmats1, rs_type, tile_offsets, flatten_ids, tile_order, nullptr, render_colors,
                                  render_alphas, last_ids, stream);
 }
 

@@ -329,7 +329,8 @@ def rasterize_to_pixels_from_world_3dgs_fwd(means, quats, scales, colors, opacit
     last_ids = torch.empty((C, image_height, image_width), dtype=torch.int32, device=dev)
     m8 = None if masks is None else masks.view(torch.uint8) if masks.dtype == torch.bool else masks
     with torch.cuda.device(dev):
-        ws = _workspace(lib().gsx_raster_records_bytes(c_u32(N)), dev)
+        ws = _workspace(lib().gsx_raster_records_bytes(c_u32(N)) + lib().gsx_tile_order_bytes(c_u32(tw), c_u32(th)),
+                        dev)  # records + room for the tile visiting order
         check(lib().gsx_rasterize_to_pixels_from_world_3dgs_fwd(
             c_u32(C), c_u32(N), c_i64(flatten_ids.numel()), _ptr(means), _ptr(quats), _ptr(scales), _ptr(colors),
             c_u32(channels), _ptr(opacities), _ptr(backgrounds), _ptr(m8), c_u32(image_width), c_u32(image_height),
@@ -376,7 +377,8 @@ def rasterize_to_pixels_from_world_3dgs_bwd(means, quats, scales, colors, opacit
     v_colors, v_opacities = torch.empty_like(colors), torch.empty_like(opacities)
     m8 = None if masks is None else masks.view(torch.uint8) if masks.dtype == torch.bool else masks
     with torch.cuda.device(dev):
-        ws = _workspace(lib().gsx_rasterize_bwd_workspace_bytes(c_u32(N)), dev)
+        ws = _workspace(lib().gsx_rasterize_bwd_workspace_bytes(c_u32(N)) +
+                        lib().gsx_tile_order_bytes(c_u32(tw), c_u32(th)), dev)  # + room for the tile visiting order
         check(lib().gsx_rasterize_to_pixels_from_world_3dgs_bwd(
             c_u32(C), c_u32(N), c_i64(flatten_ids.numel()), _ptr(means), _ptr(quats), _ptr(scales), _ptr(colors),
             c_u32(colors.size(-1)), _ptr(opacities), _ptr(backgrounds), _ptr(m8), c_u32(image_width),
