@@ -72,6 +72,8 @@ class TrainStep:
         self.side = torch.cuda.Stream(self.dev) if overlap else None
         self.ev_fork, self.ev_join = torch.cuda.Event(), torch.cuda.Event()
         self.ev_loss_fork, self.ev_loss_join = torch.cuda.Event(), torch.cuda.Event()
+        self.ev_order_fork, self.ev_order_join = torch.cuda.Event(), torch.cuda.Event()
+        self.order_pending = False
         self.loss_out = torch.empty(3, dtype=torch.float32, device=self.dev)
 
     def _allocate_per_gaussian(self, N):
@@ -148,6 +150,11 @@ class TrainStep:
                                                _p(self.dL_dmap), self._stream()))
         self.img_shape = (H, W)
 
+    def _join_tile_order(self):
+        if self.order_pending:  # the tile order was formed on the second stream
+            torch.cuda.current_stream(self.dev).wait_event(self.ev_order_join)
+            self.order_pending = False
+
     def _stream(self):
         return c_p(torch.cuda.current_stream(self.dev).cuda_stream)
 
@@ -180,6 +187,7 @@ class TrainStep:
     def forward(self, viewmat, K, W, H):
         """activations + rasterize_from_world_with_sh_fwd; returns the [1,H,W,3] render (not clamped)."""
         lb, s, N = self.lib, self._stream(), self.N
+        self._join_tile_order()  # a forward pass with no backward after it leaves the order kernel unjoined
         self._ensure_image(H, W)
         self.viewmat, self.Kmat, self.W, self.H = viewmat, K, W, H
         P, A, J = self.params, self.act, self.proj
@@ -249,8 +257,17 @@ class TrainStep:
                   _p(K), _p(self.offsets), _p(self.flatten_ids), order, _p(self.tile_walk) if self.order_tiles else
                   c_p(None), _p(self.render), _p(self.alpha), _p(self.last_ids), s)
         if self.order_tiles:
-            self._run("tile_order", lb.gsx_tile_order, c_i64(n), c_p(None), _p(self.tile_walk), c_u32(self.tw),
-                      c_u32(self.th), _p(self.tile_order), s)
+            order_args = (c_i64(n), c_p(None), _p(self.tile_walk), c_u32(self.tw), c_u32(self.th),
+                          _p(self.tile_order))
+            if self.side is None:
+                self._run("tile_order", lb.gsx_tile_order, *order_args, s)
+            else:  # beside the loss kernels: the backward pass, its first reader, waits for it
+                self.ev_order_fork.record(torch.cuda.current_stream(self.dev))
+                self.side.wait_event(self.ev_order_fork)
+                with torch.cuda.stream(self.side):
+                    self._run("tile_order", lb.gsx_tile_order, *order_args, self._stream())
+                    self.ev_order_join.record(self.side)
+                self.order_pending = True
             self.have_walk = True
         return self.render
 
@@ -308,6 +325,7 @@ class TrainStep:
                       c_f(self.lambda_dssim), _p(self.render), _p(self.image), _p(self.gt), _p(dimg),
                       _p(self.v_render), s)
         ws, wsn = _p(self.ws_bwd), c_sz(self.ws_bwd.numel())
+        self._join_tile_order()
         self._run("rasterize_bwd_accumulate", lb.gsx_rasterize_bwd_accumulate,
                   c_u32(1), c_u32(N), c_i64(self.n_isects), _p(self.records), c_p(None), c_u32(3), _p(self.bg),
                   c_p(None), c_u32(W), c_u32(H), c_u32(16),
