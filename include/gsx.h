@@ -163,12 +163,32 @@ GSX_API int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, int6
 GSX_API int gsx_intersect_offset(int64_t n_isects, const int64_t* isect_ids, uint32_t C, uint32_t tile_width,
                                  uint32_t tile_height, int32_t* offsets, void* stream);
 
+/* ---- a4-a6 for a caller that only wants the per-tile lists (one camera, grids up to 255 x 255) ----
+ * After gsx_intersect_tile_count_ordered the pairs leave in depth order, so the sort only ever looks at their tile
+ * bits and the ranges only at the tile index: the key of a pair can be its 16-bit tile index alone (the reference's
+ * other backend sorts u16 tile keys the same way, src/training/fastgs/rasterization/src/forward.cu:141-147).
+ * tile_keys u16 [n_isects] + flatten_ids i32 [n_isects] -> sorted on bits [0, n_bits) -> offsets i32 [Th,Tw].
+ * flatten_ids and offsets equal, element for element, what gsx_intersect_tile_emit_ordered +
+ * gsx_radix_sort_pairs(32, 32 + n_bits) + gsx_intersect_offset produce; a pass moves 6 instead of 12 bytes a pair.
+ * gsx_intersect_tile_pairs_fit: 1 when the grid is within the limit (else GSX_ERR_UNSUPPORTED from the emission);
+ * the sort's workspace is gsx_radix_sort_pairs_workspace_bytes(n). */
+GSX_API int gsx_intersect_tile_pairs_fit(uint32_t tile_width, uint32_t tile_height);
+GSX_API int gsx_intersect_tile_emit_pairs(uint32_t N, const int64_t* cum_tiles_per_gauss, const int32_t* order,
+                                          const void* ordered_workspace, uint32_t tile_size, uint32_t tile_width,
+                                          uint32_t tile_height, int64_t capacity, uint16_t* tile_keys,
+                                          int32_t* flatten_ids, void* stream);
+GSX_API int gsx_radix_sort_tile_pairs(int64_t n, uint16_t* keys0, int32_t* vals0, uint16_t* keys1, int32_t* vals1,
+                                      uint32_t n_bits, void* workspace, size_t workspace_bytes, int* selector_host,
+                                      void* stream);
+GSX_API int gsx_intersect_tile_pairs_offset(int64_t n_isects, const uint16_t* tile_keys, uint32_t tile_width,
+                                            uint32_t tile_height, int32_t* offsets, void* stream);
+
 /* ---- a7: gsplat::rasterize_to_pixels_from_world_3dgs_fwd (Ops.h:100-129; ...3DGSFwd.cu:19-285) ----
  * colors [C,N,channels] (channels in {1,3,4}), opacities [C,N], backgrounds [C,channels] nullable,
  * masks u8 [C,Th,Tw] nullable, tile_offsets i32 [C,Th,Tw], flatten_ids i32 [n_isects]
  * -> render_colors [C,H,W,channels], render_alphas [C,H,W,1], last_ids i32 [C,H,W]. tile_size must be 16.
  *
- * The rasterizers read one 80-byte RECORD per Gaussian (whitening matrix diag(1/s) R^T, camera centre in whitened
+ * The rasterizers read one 96-byte RECORD per Gaussian (whitening matrix diag(1/s) R^T, camera centre in whitened
  * coordinates, opacity, first three colour channels, exact pixel bounds of alpha >= 1/255) instead of the five
  * parameter tensors: gsx_pack_raster_records builds them for one camera, gsx_rasterize_records_fwd renders from
  * them.  The whole-operator entry point does both and needs gsx_raster_records_bytes(N) of workspace. */

@@ -185,7 +185,9 @@ __global__ void __launch_bounds__(256) scan_apply_kernel(uint32_t n, const int32
 // exceeds k (binary search over 64 prefixes in LDS), so the lanes write consecutive entries.
 // FROM_KEYS: position i's Gaussian is order[i] and its rectangle and depth bits are the words of sorted_keys[i]
 // (depth_count_keys_kernel<true>): sequential reads only, nothing is gathered in sorted order.
-template <bool FROM_KEYS>
+// COMPACT (one camera, at most 65 536 tiles): the output key is the 16-bit tile index alone - pairs emitted in depth
+// order only ever sort on their tile bits, and the per-tile ranges need nothing else.
+template <bool FROM_KEYS, bool COMPACT = false>
 __global__ void __launch_bounds__(256) tile_emit_kernel(uint32_t n, uint32_t N, const float* __restrict__ means2d,
                                                          const int32_t* __restrict__ radii,
                                                          const float* __restrict__ depths,
@@ -195,8 +197,10 @@ __global__ void __launch_bounds__(256) tile_emit_kernel(uint32_t n, uint32_t N, 
                                                          uint32_t tile_width, uint32_t tile_height,
                                                          uint32_t tile_n_bits, int64_t capacity,
                                                          int64_t* __restrict__ isect_ids,
+                                                         uint16_t* __restrict__ tile_keys /*COMPACT*/,
                                                          int32_t* __restrict__ flatten_ids) {
-    __shared__ uint32_t s_incl[4][64], s_xy[4][64], s_w[4][64], s_idx[4][64], s_lo[4][64], s_hi[4][64];
+    __shared__ uint32_t s_incl[4][64], s_xy[4][64], s_w[4][64], s_idx[4][64], s_lo[COMPACT ? 1 : 4][64],
+        s_hi[COMPACT ? 1 : 4][64];
     const uint32_t i = blockIdx.x * 256u + threadIdx.x;
     const uint32_t lane = threadIdx.x & 63u, wv = threadIdx.x >> 6;
     TileRect r = {0, 0, 0, 0};
@@ -237,8 +241,10 @@ __global__ void __launch_bounds__(256) tile_emit_kernel(uint32_t n, uint32_t N, 
     s_xy[wv][lane] = r.x0 | (r.y0 << 16);
     s_w[wv][lane] = w;
     s_idx[wv][lane] = idx;
-    s_lo[wv][lane] = (uint32_t)key_base;
-    s_hi[wv][lane] = (uint32_t)(key_base >> 32);
+    if (!COMPACT) {
+        s_lo[wv][lane] = (uint32_t)key_base;
+        s_hi[wv][lane] = (uint32_t)(key_base >> 32);
+    }
     __syncthreads();
     if (total == 0)
         return; // wave-uniform; no barrier follows
@@ -262,9 +268,13 @@ __global__ void __launch_bounds__(256) tile_emit_kernel(uint32_t n, uint32_t N, 
         const uint32_t gw = s_w[wv][l], xy = s_xy[wv][l];
         const uint32_t row = local / gw;
         const int64_t tile_id = (int64_t)((xy >> 16) + row) * tile_width + ((xy & 0xffffu) + (local - row * gw));
-        const int64_t kb = ((int64_t)s_hi[wv][l] << 32) | (int64_t)s_lo[wv][l];
         if (wave_base + k < capacity) { // a caller that emits before it knows the total bounds the writes
-            isect_ids[wave_base + k] = kb | (tile_id << 32);
+            if (COMPACT) {
+                tile_keys[wave_base + k] = (uint16_t)tile_id;
+            } else {
+                const int64_t kb = ((int64_t)s_hi[wv][l] << 32) | (int64_t)s_lo[wv][l];
+                isect_ids[wave_base + k] = kb | (tile_id << 32);
+            }
             flatten_ids[wave_base + k] = (int32_t)s_idx[wv][l];
         }
     }
@@ -382,6 +392,41 @@ __global__ void __launch_bounds__(256) intersect_offset_kernel(uint32_t n_isects
         const int64_t id_prev = (isect_id_prev >> tile_n_bits) * n_tiles + (isect_id_prev & tile_mask);
         for (int64_t i = id_prev + 1; i < id_curr + 1; ++i)
             offsets[i] = (int32_t)idx;
+    }
+}
+
+// the same ranges from sorted 16-bit tile indices of one camera; a thread takes `per` consecutive pairs (8 with one
+// 16-byte load when the array is aligned for it)
+__global__ void __launch_bounds__(256) tile_pairs_offset_kernel(uint32_t n_isects,
+                                                                 const uint16_t* __restrict__ tile_keys,
+                                                                 uint32_t n_tiles, uint32_t per,
+                                                                 int32_t* __restrict__ offsets) {
+    const uint32_t first = (blockIdx.x * 256u + threadIdx.x) * per;
+    if (first >= n_isects)
+        return;
+    uint32_t k[8];
+    const uint32_t cnt = min(per, n_isects - first);
+    if (cnt == 8) {
+        const uint4 q = *reinterpret_cast<const uint4*>(tile_keys + first);
+        k[0] = q.x & 0xffffu, k[1] = q.x >> 16, k[2] = q.y & 0xffffu, k[3] = q.y >> 16;
+        k[4] = q.z & 0xffffu, k[5] = q.z >> 16, k[6] = q.w & 0xffffu, k[7] = q.w >> 16;
+    } else {
+        for (uint32_t e = 0; e < cnt; ++e)
+            k[e] = tile_keys[first + e];
+    }
+    uint32_t prev = first ? (uint32_t)tile_keys[first - 1] : 0u;
+    if (first == 0)
+        for (uint32_t i = 0; i < k[0] + 1; ++i)
+            offsets[i] = 0;
+    for (uint32_t e = 0; e < cnt; ++e) {
+        const uint32_t idx = first + e, curr = k[e];
+        if (idx > 0)
+            for (uint32_t i = prev + 1; i < curr + 1; ++i)
+                offsets[i] = (int32_t)idx;
+        if (idx == n_isects - 1)
+            for (uint32_t i = curr + 1; i < n_tiles; ++i)
+                offsets[i] = (int32_t)n_isects;
+        prev = curr;
     }
 }
 
@@ -592,7 +637,8 @@ extern "C" int gsx_intersect_tile_emit_capped(uint32_t C, uint32_t N, const floa
     GSX_REQUIRE(order == nullptr || C == 1, GSX_ERR_UNSUPPORTED, "intersect_tile_emit: an order needs C == 1");
     hipLaunchKernelGGL(tile_emit_kernel<false>, dim3(cdiv(n, 256)), dim3(256), 0, (hipStream_t)stream, n, N, means2d,
                        radii, depths, (const int64_t*)nullptr, cum_tiles_per_gauss, order, (float)tile_size, tile_width,
-                       tile_height, gsx_n_bits(tile_width * tile_height), capacity, isect_ids, flatten_ids);
+                       tile_height, gsx_n_bits(tile_width * tile_height), capacity, isect_ids, (uint16_t*)nullptr,
+                       flatten_ids);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }
@@ -617,7 +663,33 @@ extern "C" int gsx_intersect_tile_emit_ordered(uint32_t N, const float* means2d,
                        (const float*)nullptr, (const int32_t*)nullptr, (const float*)nullptr,
                        (const int64_t*)gsx::ordered_keys(const_cast<void*>(ordered_workspace)), cum_tiles_per_gauss,
                        order, (float)tile_size, tile_width, tile_height, gsx_n_bits(tile_width * tile_height),
-                       capacity, isect_ids, flatten_ids);
+                       capacity, isect_ids, (uint16_t*)nullptr, flatten_ids);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+extern "C" int gsx_intersect_tile_pairs_fit(uint32_t tile_width, uint32_t tile_height) {
+    return rect_keys_fit(tile_width, tile_height) ? 1 : 0;
+}
+
+extern "C" int gsx_intersect_tile_emit_pairs(uint32_t N, const int64_t* cum_tiles_per_gauss, const int32_t* order,
+                                             const void* ordered_workspace, uint32_t tile_size, uint32_t tile_width,
+                                             uint32_t tile_height, int64_t capacity, uint16_t* tile_keys,
+                                             int32_t* flatten_ids, void* stream) {
+    if (N == 0)
+        return GSX_OK;
+    GSX_REQUIRE(order && ordered_workspace, GSX_ERR_INVALID_ARGUMENT,
+                "intersect_tile_emit_pairs: order / workspace of gsx_intersect_tile_count_ordered is null");
+    GSX_REQUIRE(rect_keys_fit(tile_width, tile_height), GSX_ERR_UNSUPPORTED,
+                "intersect_tile_emit_pairs: a %u x %u tile grid needs the 64-bit keys", tile_width, tile_height);
+    GSX_REQUIRE(cum_tiles_per_gauss && tile_keys && flatten_ids, GSX_ERR_INVALID_ARGUMENT,
+                "intersect_tile_emit_pairs: null tensor");
+    GSX_REQUIRE(N < (1u << 31), GSX_ERR_INVALID_ARGUMENT, "intersect_tile_emit_pairs: N >= 2^31");
+    hipLaunchKernelGGL((tile_emit_kernel<true, true>), dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, N,
+                       (const float*)nullptr, (const int32_t*)nullptr, (const float*)nullptr,
+                       (const int64_t*)gsx::ordered_keys(const_cast<void*>(ordered_workspace)), cum_tiles_per_gauss,
+                       order, (float)tile_size, tile_width, tile_height, gsx_n_bits(tile_width * tile_height),
+                       capacity, (int64_t*)nullptr, tile_keys, flatten_ids);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }
@@ -674,6 +746,29 @@ extern "C" int gsx_intersect_offset(int64_t n_isects, const int64_t* isect_ids, 
     GSX_REQUIRE(isect_ids != nullptr, GSX_ERR_INVALID_ARGUMENT, "intersect_offset: isect_ids is null");
     hipLaunchKernelGGL(intersect_offset_kernel, dim3(cdiv(n_isects, 256)), dim3(256), 0, s, (uint32_t)n_isects,
                        isect_ids, C, tile_width * tile_height, gsx_n_bits(tile_width * tile_height), offsets);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+extern "C" int gsx_intersect_tile_pairs_offset(int64_t n_isects, const uint16_t* tile_keys, uint32_t tile_width,
+                                               uint32_t tile_height, int32_t* offsets, void* stream) {
+    const uint64_t n_tiles = (uint64_t)tile_width * tile_height;
+    if (n_tiles == 0)
+        return GSX_OK;
+    GSX_REQUIRE(offsets != nullptr, GSX_ERR_INVALID_ARGUMENT, "intersect_tile_pairs_offset: offsets is null");
+    GSX_REQUIRE(n_isects >= 0 && n_isects < (1ll << 31), GSX_ERR_OVERFLOW,
+                "intersect_tile_pairs_offset: n_isects out of range");
+    GSX_REQUIRE(n_tiles <= 65536, GSX_ERR_UNSUPPORTED, "intersect_tile_pairs_offset: more than 65536 tiles");
+    hipStream_t s = (hipStream_t)stream;
+    if (n_isects == 0) {
+        hipLaunchKernelGGL(fill_i32_kernel, dim3(cdiv(n_tiles, 256)), dim3(256), 0, s, (uint32_t)n_tiles, 0, offsets);
+        GSX_LAUNCH_CHECK();
+        return GSX_OK;
+    }
+    GSX_REQUIRE(tile_keys != nullptr, GSX_ERR_INVALID_ARGUMENT, "intersect_tile_pairs_offset: tile_keys is null");
+    const uint32_t per = ((uintptr_t)tile_keys & 15u) == 0 ? 8u : 1u;
+    hipLaunchKernelGGL(tile_pairs_offset_kernel, dim3(cdiv(n_isects, 256 * per)), dim3(256), 0, s,
+                       (uint32_t)n_isects, tile_keys, (uint32_t)n_tiles, per, offsets);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

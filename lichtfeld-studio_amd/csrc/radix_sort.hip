@@ -1,5 +1,6 @@
 // radix_sort.hip - stable LSD radix sort of (int64 key, int32 value) pairs on key bits [begin_bit, end_bit)
-// (gsplat/IntersectTile.cu:290-328 calls cub::DeviceRadixSort::SortPairs with a DoubleBuffer).
+// (gsplat/IntersectTile.cu:290-328 calls cub::DeviceRadixSort::SortPairs with a DoubleBuffer), and the same sort
+// for (uint16 tile index, int32 value) pairs.
 //
 // 8-bit digits.  Per pass three launches: block histograms -> one scan block per digit turns its row of the
 // digit-major table into running counts and leaves the digit's total -> stable scatter (every block adds the
@@ -21,8 +22,12 @@ static constexpr int64_t kSmallSortLimit = 1ll << 21;
 __device__ __forceinline__ uint32_t digit_of(int64_t key, uint32_t shift, uint32_t mask) {
     return (uint32_t)((uint64_t)key >> shift) & mask;
 }
+__device__ __forceinline__ uint32_t digit_of(uint16_t key, uint32_t shift, uint32_t mask) {
+    return ((uint32_t)key >> shift) & mask;
+}
 
-__global__ void __launch_bounds__(256) radix_hist_kernel(uint32_t n, const int64_t* __restrict__ keys,
+template <typename KeyT>
+__global__ void __launch_bounds__(256) radix_hist_kernel(uint32_t n, const KeyT* __restrict__ keys,
                                                           uint32_t items, uint32_t shift, uint32_t mask,
                                                           uint32_t nblocks,
                                                           uint32_t* __restrict__ hist /*[kRadix][nblocks]*/) {
@@ -30,11 +35,31 @@ __global__ void __launch_bounds__(256) radix_hist_kernel(uint32_t n, const int64
     lh[threadIdx.x] = 0;
     __syncthreads();
     const uint32_t base = blockIdx.x * 256u * items;
+    if (sizeof(KeyT) == 2 && ((uintptr_t)keys & 15u) == 0) {
+        // 16-bit keys, eight to a 16-byte load (a tile starts at a multiple of 1024 keys)
+        const uint4* __restrict__ k8 = reinterpret_cast<const uint4*>(keys + base);
+        for (uint32_t v = threadIdx.x; v < 32u * items; v += 256u) {
+            const uint32_t first = base + v * 8u;
+            if (first + 8u <= n) {
+                const uint4 q = k8[v];
+                const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+                for (uint32_t h = 0; h < 4; ++h) {
+                    atomicAdd(&lh[((w[h] & 0xffffu) >> shift) & mask], 1u);
+                    atomicAdd(&lh[((w[h] >> 16) >> shift) & mask], 1u);
+                }
+            } else {
+                for (uint32_t idx = first; idx < n && idx < first + 8u; ++idx)
+                    atomicAdd(&lh[digit_of(keys[idx], shift, mask)], 1u);
+            }
+        }
+    } else {
 #pragma unroll 4
-    for (uint32_t i = 0; i < items; ++i) {
-        const uint32_t idx = base + i * 256u + threadIdx.x;
-        if (idx < n)
-            atomicAdd(&lh[digit_of(keys[idx], shift, mask)], 1u);
+        for (uint32_t i = 0; i < items; ++i) {
+            const uint32_t idx = base + i * 256u + threadIdx.x;
+            if (idx < n)
+                atomicAdd(&lh[digit_of(keys[idx], shift, mask)], 1u);
+        }
     }
     __syncthreads();
     hist[threadIdx.x * nblocks + blockIdx.x] = lh[threadIdx.x];
@@ -81,10 +106,10 @@ __global__ void __launch_bounds__(256) radix_scan_kernel(uint32_t nblocks, uint3
 }
 
 // ---- stable scatter -------------------------------------------------------------------------------
-template <uint32_t ITEMS>
-__global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const int64_t* __restrict__ keys_in,
+template <typename KeyT, uint32_t ITEMS>
+__global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const KeyT* __restrict__ keys_in,
                                                              const int32_t* __restrict__ vals_in,
-                                                             int64_t* __restrict__ keys_out,
+                                                             KeyT* __restrict__ keys_out,
                                                              int32_t* __restrict__ vals_out, uint32_t shift,
                                                              uint32_t mask, uint32_t nblocks,
                                                              const uint32_t* __restrict__ hist_scanned,
@@ -93,7 +118,7 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const in
     __shared__ uint32_t wave_count[4][kRadix];
     __shared__ uint32_t to_global[kRadix]; // global position of a pair = to_global[digit] + its slot in the tile
     __shared__ uint32_t wsum[4], gsum[4];
-    __shared__ int64_t s_keys[kTileN];
+    __shared__ KeyT s_keys[kTileN];
     __shared__ int32_t s_vals[kTileN];
     const uint32_t t = threadIdx.x;
     const uint32_t w = t >> 6, lane = t & 63u;
@@ -105,7 +130,7 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const in
     const uint32_t tile_base = blockIdx.x * kTileN;
     const uint32_t wave_base = tile_base + w * kWaveN;
     const uint64_t lt_mask = (1ull << lane) - 1ull;
-    int64_t key[ITEMS];
+    KeyT key[ITEMS];
     int32_t val[ITEMS];
     uint32_t rank[ITEMS]; // rank among the wave's pairs with the same digit
 #pragma unroll
@@ -180,7 +205,7 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const in
     for (uint32_t k = 0; k < ITEMS; ++k) {
         const uint32_t slot = k * 256u + t;
         if (slot < count) {
-            const int64_t kk = s_keys[slot];
+            const KeyT kk = s_keys[slot];
             const uint32_t pos = to_global[digit_of(kk, shift, mask)] + slot;
             keys_out[pos] = kk;
             vals_out[pos] = s_vals[slot];
@@ -224,20 +249,22 @@ extern "C" int gsx_radix_sort_pairs_selector(int64_t n, uint32_t begin_bit, uint
     return (int)(((end_bit - begin_bit + kRadixBits - 1) / kRadixBits) & 1u); // one ping-pong per digit pass
 }
 
-extern "C" int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, int64_t* keys1, int32_t* vals1,
-                                    uint32_t begin_bit, uint32_t end_bit, void* workspace, size_t workspace_bytes,
-                                    int* selector_host, void* stream) {
+namespace {
+template <typename KeyT>
+int sort_pairs(const char* what, int64_t n, KeyT* keys0, int32_t* vals0, KeyT* keys1, int32_t* vals1,
+               uint32_t begin_bit, uint32_t end_bit, void* workspace, size_t workspace_bytes, int* selector_host,
+               void* stream) {
     if (selector_host)
         *selector_host = 0;
     if (n <= 0)
         return GSX_OK; // IntersectTile.cu:298-300
-    GSX_REQUIRE(n < (1ll << 31), GSX_ERR_OVERFLOW, "radix_sort_pairs: n = %lld does not fit int32", (long long)n);
-    GSX_REQUIRE(keys0 && vals0 && keys1 && vals1, GSX_ERR_INVALID_ARGUMENT, "radix_sort_pairs: null buffer");
-    GSX_REQUIRE(end_bit >= 1 && end_bit <= 64 && begin_bit < end_bit, GSX_ERR_INVALID_ARGUMENT,
-                "radix_sort_pairs: bits [%u, %u)", begin_bit, end_bit);
+    GSX_REQUIRE(n < (1ll << 31), GSX_ERR_OVERFLOW, "%s: n = %lld does not fit int32", what, (long long)n);
+    GSX_REQUIRE(keys0 && vals0 && keys1 && vals1, GSX_ERR_INVALID_ARGUMENT, "%s: null buffer", what);
+    GSX_REQUIRE(end_bit >= 1 && end_bit <= 8 * sizeof(KeyT) && begin_bit < end_bit, GSX_ERR_INVALID_ARGUMENT,
+                "%s: bits [%u, %u)", what, begin_bit, end_bit);
     const SortLayout L = sort_layout(n);
     GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 && workspace_bytes >= L.total,
-                GSX_ERR_WORKSPACE, "radix_sort_pairs: workspace needs %zu bytes, 256-byte aligned", L.total);
+                GSX_ERR_WORKSPACE, "%s: workspace needs %zu bytes, 256-byte aligned", what, L.total);
     uint32_t* hist = (uint32_t*)((char*)workspace + L.hist_off);
     uint32_t* totals = (uint32_t*)((char*)workspace + L.totals_off);
     hipStream_t s = (hipStream_t)stream;
@@ -245,7 +272,7 @@ extern "C" int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, i
     // as 7 + 6, whose longer runs per (block, digit) scatter in fuller cache lines than 8 + 5)
     const uint32_t n_bits = end_bit - begin_bit;
     const uint32_t passes = (n_bits + kRadixBits - 1) / kRadixBits;
-    GSX_REQUIRE(passes <= kMaxPasses, GSX_ERR_INVALID_ARGUMENT, "radix_sort_pairs: %u passes", passes);
+    GSX_REQUIRE(passes <= kMaxPasses, GSX_ERR_INVALID_ARGUMENT, "%s: %u passes", what, passes);
     const uint32_t width_lo = n_bits / passes, n_wide = n_bits % passes;
     int sel = 0;
     uint32_t shift = begin_bit;
@@ -253,21 +280,21 @@ extern "C" int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, i
     for (uint32_t pass = 0; pass < passes; ++pass) {
         const uint32_t bits = width_lo + (pass < n_wide ? 1u : 0u);
         const uint32_t mask = (1u << bits) - 1u;
-        const int64_t* kin = sel ? keys1 : keys0;
+        const KeyT* kin = sel ? keys1 : keys0;
         const int32_t* vin = sel ? vals1 : vals0;
-        int64_t* kout = sel ? keys0 : keys1;
+        KeyT* kout = sel ? keys0 : keys1;
         int32_t* vout = sel ? vals0 : vals1;
-        hipLaunchKernelGGL(radix_hist_kernel, dim3(L.nblocks), dim3(256), 0, s, (uint32_t)n, kin, items, shift, mask,
-                           L.nblocks, hist);
+        hipLaunchKernelGGL(radix_hist_kernel<KeyT>, dim3(L.nblocks), dim3(256), 0, s, (uint32_t)n, kin, items, shift,
+                           mask, L.nblocks, hist);
         GSX_LAUNCH_CHECK();
         hipLaunchKernelGGL(radix_scan_kernel, dim3(kRadix), dim3(256), 0, s, L.nblocks, hist, totals);
         GSX_LAUNCH_CHECK();
         if (items == kItemsSmall)
-            hipLaunchKernelGGL((radix_scatter_kernel<kItemsSmall>), dim3(L.nblocks), dim3(256), 0, s, (uint32_t)n, kin,
-                               vin, kout, vout, shift, mask, L.nblocks, hist, totals);
+            hipLaunchKernelGGL((radix_scatter_kernel<KeyT, kItemsSmall>), dim3(L.nblocks), dim3(256), 0, s,
+                               (uint32_t)n, kin, vin, kout, vout, shift, mask, L.nblocks, hist, totals);
         else
-            hipLaunchKernelGGL((radix_scatter_kernel<kItemsLarge>), dim3(L.nblocks), dim3(256), 0, s, (uint32_t)n, kin,
-                               vin, kout, vout, shift, mask, L.nblocks, hist, totals);
+            hipLaunchKernelGGL((radix_scatter_kernel<KeyT, kItemsLarge>), dim3(L.nblocks), dim3(256), 0, s,
+                               (uint32_t)n, kin, vin, kout, vout, shift, mask, L.nblocks, hist, totals);
         GSX_LAUNCH_CHECK();
         sel ^= 1;
         shift += bits;
@@ -275,4 +302,20 @@ extern "C" int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, i
     if (selector_host)
         *selector_host = sel;
     return GSX_OK;
+}
+} // namespace
+
+extern "C" int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, int64_t* keys1, int32_t* vals1,
+                                    uint32_t begin_bit, uint32_t end_bit, void* workspace, size_t workspace_bytes,
+                                    int* selector_host, void* stream) {
+    return sort_pairs<int64_t>("radix_sort_pairs", n, keys0, vals0, keys1, vals1, begin_bit, end_bit, workspace,
+                               workspace_bytes, selector_host, stream);
+}
+
+// The same sort for 16-bit keys (tile indices of one camera, bits [0, n_bits)): a third of the bytes per pass.
+extern "C" int gsx_radix_sort_tile_pairs(int64_t n, uint16_t* keys0, int32_t* vals0, uint16_t* keys1, int32_t* vals1,
+                                         uint32_t n_bits, void* workspace, size_t workspace_bytes,
+                                         int* selector_host, void* stream) {
+    return sort_pairs<uint16_t>("radix_sort_tile_pairs", n, keys0, vals0, keys1, vals1, 0, n_bits, workspace,
+                                workspace_bytes, selector_host, stream);
 }

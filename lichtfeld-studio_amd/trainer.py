@@ -28,9 +28,10 @@ def _p(t):
 class TrainStep:
     def __init__(self, scene, device="cuda:0", lrs=None, lambda_dssim=0.2, betas=(0.9, 0.999), eps=1e-15,
                  scene_scale=1.0, sh_degree=None, use_ssim=True, fused_update=False, fused_loss=False,
-                 scale_reg=0.0, opacity_reg=0.0, overlap=False):
+                 scale_reg=0.0, opacity_reg=0.0, overlap=False, tile_pairs=True):
         self.dev = torch.device(device)
         self.lib = lib()
+        self.tile_pairs = tile_pairs  # sort (u16 tile index, id) pairs where the tile grid allows it
         f = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(self.dev)
         self.N = scene.means.shape[0]
         self.K = 1 + scene.shN.shape[1]
@@ -63,6 +64,7 @@ class TrainStep:
         self.reg_losses = torch.zeros(2, dtype=torch.float32, device=self.dev)  # [scale term, opacity term]
         self._allocate_per_gaussian(self.N)
         self.cap = 0
+        self.compact = False
         self.img_shape = None
         self.n_isects = 0
         self.bg = torch.zeros((1, 3), dtype=torch.float32, device=self.dev)  # trainer.cpp:383-384
@@ -112,11 +114,12 @@ class TrainStep:
         return n
 
     def _ensure_isect_capacity(self, n):
-        if n <= self.cap:
+        if n <= self.cap and self.cap:
             return
         cap = max(int(n * 1.25) + 1024, 1 << 16)
         e = lambda *s, dt: torch.empty(s, dtype=dt, device=self.dev)
-        self.keys = [e(cap, dt=torch.int64), e(cap, dt=torch.int64)]
+        kt = torch.int16 if self.compact else torch.int64
+        self.keys = [e(cap, dt=kt), e(cap, dt=kt)]
         self.vals = [e(cap, dt=torch.int32), e(cap, dt=torch.int32)]
         self.ws_sort = e(self.lib.gsx_radix_sort_pairs_workspace_bytes(c_i64(cap)), dt=torch.uint8)
         self.cap = cap
@@ -126,7 +129,11 @@ class TrainStep:
             return
         e = lambda *s, dt=torch.float32: torch.empty(s, dtype=dt, device=self.dev)
         self.tw, self.th = (W + 15) // 16, (H + 15) // 16
+        self._tile_bits = self.lib.gsx_n_bits(c_u32(self.tw * self.th))
         self._end_bit = 32 + self.lib.gsx_n_bits(c_u32(self.tw * self.th)) + self.lib.gsx_n_bits(c_u32(1))
+        compact = bool(self.tile_pairs and self.lib.gsx_intersect_tile_pairs_fit(c_u32(self.tw), c_u32(self.th)))
+        if compact != self.compact:  # the key buffers change their element type
+            self.compact, self.cap = compact, 0
         self.offsets = e(1, self.th, self.tw, dt=torch.int32)
         self.tile_order = e(self.th * self.tw, dt=torch.int32)  # the rasterizers' tile visiting order
         self.tile_walk = e(self.th * self.tw, dt=torch.int32)   # per tile: entries up to its last contributor
@@ -217,10 +224,16 @@ class TrainStep:
                 self.ev_join.record(self.side)
         # The emission does not need the total, only room for it: with buffers from an earlier step it is queued now
         # (writes bounded to the buffers) and the host's wake-up from the wait below hides behind it.
-        emit = lambda cap: self._run(
-            "intersect_tile_emit", lb.gsx_intersect_tile_emit_ordered, c_u32(N), _p(J["means2d"]), _p(J["radii"]),
-            _p(J["depths"]), _p(self.cum), _p(self.order), _p(self.ws_count), c_u32(16), c_u32(self.tw),
-            c_u32(self.th), c_i64(cap), _p(self.keys[0]), _p(self.vals[0]), s)
+        if self.compact:  # pairs in depth order sort on their tile bits only: 16-bit tile indices as keys
+            emit = lambda cap: self._run(
+                "intersect_tile_emit", lb.gsx_intersect_tile_emit_pairs, c_u32(N), _p(self.cum), _p(self.order),
+                _p(self.ws_count), c_u32(16), c_u32(self.tw), c_u32(self.th), c_i64(cap), _p(self.keys[0]),
+                _p(self.vals[0]), s)
+        else:
+            emit = lambda cap: self._run(
+                "intersect_tile_emit", lb.gsx_intersect_tile_emit_ordered, c_u32(N), _p(J["means2d"]),
+                _p(J["radii"]), _p(J["depths"]), _p(self.cum), _p(self.order), _p(self.ws_count), c_u32(16),
+                c_u32(self.tw), c_u32(self.th), c_i64(cap), _p(self.keys[0]), _p(self.vals[0]), s)
         emitted_cap = self.cap
         if emitted_cap:
             emit(emitted_cap)
@@ -233,13 +246,22 @@ class TrainStep:
             if n > emitted_cap:  # first step, or the buffers had to grow
                 emit(self.cap)
             end_bit = self._end_bit  # 32 + tile bits + camera bits, fixed with the image size
-            self._run("radix_sort_pairs", lb.gsx_radix_sort_pairs, c_i64(n), _p(self.keys[0]), _p(self.vals[0]),
-                      _p(self.keys[1]), _p(self.vals[1]), c_u32(32), c_u32(end_bit), _p(self.ws_sort),
-                      c_sz(self.ws_sort.numel()), ctypes.byref(sel), s)
+            if self.compact:
+                self._run("radix_sort_pairs", lb.gsx_radix_sort_tile_pairs, c_i64(n), _p(self.keys[0]),
+                          _p(self.vals[0]), _p(self.keys[1]), _p(self.vals[1]), c_u32(self._tile_bits),
+                          _p(self.ws_sort), c_sz(self.ws_sort.numel()), ctypes.byref(sel), s)
+            else:
+                self._run("radix_sort_pairs", lb.gsx_radix_sort_pairs, c_i64(n), _p(self.keys[0]),
+                          _p(self.vals[0]), _p(self.keys[1]), _p(self.vals[1]), c_u32(32), c_u32(end_bit),
+                          _p(self.ws_sort), c_sz(self.ws_sort.numel()), ctypes.byref(sel), s)
         self.sel = sel.value
-        self.isect_ids, self.flatten_ids = self.keys[self.sel], self.vals[self.sel]
-        self._run("intersect_offset", lb.gsx_intersect_offset, c_i64(n), _p(self.isect_ids), c_u32(1), c_u32(self.tw), c_u32(self.th),
-                                      _p(self.offsets), s)
+        self.flatten_ids = self.vals[self.sel]
+        if self.compact:
+            self._run("intersect_offset", lb.gsx_intersect_tile_pairs_offset, c_i64(n), _p(self.keys[self.sel]),
+                      c_u32(self.tw), c_u32(self.th), _p(self.offsets), s)
+        else:
+            self._run("intersect_offset", lb.gsx_intersect_offset, c_i64(n), _p(self.keys[self.sel]), c_u32(1),
+                      c_u32(self.tw), c_u32(self.th), _p(self.offsets), s)
         # Dearest tiles first: both rasterizers then end with cheap tiles instead of a long tail.  What a tile costs is
         # how far its pixels go into the list, which the forward pass itself reports; the forward pass therefore
         # uses the order of the previous step (the first one: by list length), the backward pass this step's.
@@ -270,6 +292,17 @@ class TrainStep:
                 self.order_pending = True
             self.have_walk = True
         return self.render
+
+    @property
+    def isect_ids(self):
+        """The sorted 64-bit keys (tile << 32 | depth bits) of the last forward pass.  On the 16-bit path they are not
+        formed by the step: rebuilt here, for inspection, from the sorted tile indices and the depths."""
+        if not self.compact:
+            return self.keys[self.sel]
+        n = self.n_isects
+        tiles = self.keys[self.sel][:n].to(torch.int64) & 0xFFFF
+        depth = self.proj["depths"].view(torch.int32).reshape(-1)[self.vals[self.sel][:n].long()]
+        return (tiles << 32) | (depth.to(torch.int64) & 0xFFFFFFFF)
 
     # -- loss ---------------------------------------------------------------------------------------
     def loss_forward(self, gt_chw):

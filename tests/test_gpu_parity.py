@@ -244,6 +244,139 @@ def test_tile_count_prefix_sums(gsx, cuda, n):
     assert np.array_equal(cum.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("n,bits", [(1, 12), (65, 1), (4097, 8), (100_003, 12), (3_000_000, 13), (2_500_000, 16)])
+def test_tile_pair_sort_stable(gsx, cuda, n, bits):
+    """the 16-bit-key sort is the stable sort on bits [0, bits): numpy's stable argsort of the masked keys (bits above
+    the range do not take part and travel with their pair)"""
+    import ctypes
+    from lichtfeld_studio_amd._lib import c_i64, c_p, c_sz, c_u32, check, lib
+    L = lib()
+    rng = np.random.default_rng(n + bits)
+    keys = rng.integers(0, 1 << 16, n).astype(np.uint16)
+    if n > 1000:
+        keys[: n // 2] &= 0x0F0F  # many ties
+    vals = rng.permutation(n).astype(np.int32)
+    order = np.argsort(keys & np.uint16((1 << bits) - 1), kind="stable")
+    k = [T(keys.view(np.int16), cuda), torch.empty(n, dtype=torch.int16, device=cuda)]
+    v = [T(vals, cuda), torch.empty(n, dtype=torch.int32, device=cuda)]
+    ws = torch.empty(L.gsx_radix_sort_pairs_workspace_bytes(c_i64(n)), dtype=torch.uint8, device=cuda)
+    sel = ctypes.c_int(-1)
+    p = lambda t: c_p(t.data_ptr())
+    check(L.gsx_radix_sort_tile_pairs(c_i64(n), p(k[0]), p(v[0]), p(k[1]), p(v[1]), c_u32(bits), p(ws),
+                                      c_sz(ws.numel()), ctypes.byref(sel),
+                                      c_p(torch.cuda.current_stream(cuda).cuda_stream)))
+    assert sel.value == (1 if bits <= 8 else 0)
+    bits_equal(N(k[sel.value]).view(np.uint16), keys[order], "keys")
+    bits_equal(N(v[sel.value]), vals[order], "values")
+    with pytest.raises(gsx._lib.GsxError, match="bits"):
+        check(L.gsx_radix_sort_tile_pairs(c_i64(n), p(k[0]), p(v[0]), p(k[1]), p(v[1]), c_u32(17), p(ws),
+                                          c_sz(ws.numel()), ctypes.byref(sel), c_p(0)))
+
+
+@pytest.mark.parametrize("grid,n", [((78, 52), 60_000), ((255, 255), 20_000), ((3, 2), 0), ((3, 2), 500)])
+def test_tile_pairs_match_the_64_bit_keys(gsx, cuda, grid, n):
+    """(u16 tile index, id) pairs emitted in depth order, sorted on their tile bits, and their per-tile ranges: the
+    values and ranges equal, element for element, those of the 64-bit (tile << 32 | depth) path"""
+    import ctypes
+    from lichtfeld_studio_amd._lib import c_i, c_i64, c_p, c_sz, c_u32, check, lib
+    L = lib()
+    ops = gsx.ops
+    tw, th = grid
+    W, H = tw * 16 - 3, th * 16 - 5
+    rng = np.random.default_rng(tw * 1000 + th + n)
+    means2d = np.stack([rng.uniform(-20, W + 20, n), rng.uniform(-20, H + 20, n)], 1).astype(np.float32)[None]
+    radii = rng.integers(0, 40, (1, n, 2)).astype(np.int32)
+    radii[0, ::7] = 0
+    depths = rng.uniform(0.1, 50.0, (1, n)).astype(np.float32)
+    depths[0, 100:200] = depths[0, 100:101]  # ties: broken by index
+    m, r, d = T(means2d, cuda), T(radii, cuda), T(depths, cuda)
+    stream = c_p(torch.cuda.current_stream(cuda).cuda_stream)
+    p = lambda t: c_p(t.data_ptr())
+    assert L.gsx_intersect_tile_pairs_fit(c_u32(tw), c_u32(th)) == 1
+    if n:
+        _, ids, flat = ops.intersect_tile(m, r, d, None, None, 1, 16, tw, th, True)
+        want_off = ops.intersect_offset(ids, 1, tw, th)
+    else:
+        flat = torch.empty(0, dtype=torch.int32, device=cuda)
+        want_off = torch.zeros((1, th, tw), dtype=torch.int32, device=cuda)
+    order = torch.empty(max(n, 1), dtype=torch.int32, device=cuda)
+    tpg = torch.empty(max(n, 1), dtype=torch.int32, device=cuda)
+    cum = torch.empty(max(n, 1), dtype=torch.int64, device=cuda)
+    ws = torch.empty(L.gsx_intersect_tile_count_ordered_workspace_bytes(c_u32(max(n, 1))), dtype=torch.uint8,
+                     device=cuda)
+    total = ctypes.c_int64(-7)
+    check(L.gsx_intersect_tile_count_ordered(c_u32(n), p(m), p(r), p(d), c_u32(16), c_u32(tw), c_u32(th), p(order),
+                                             p(tpg), p(cum), p(ws), c_sz(ws.numel()), ctypes.byref(total), c_i(1),
+                                             stream))
+    ni = total.value if n else 0
+    assert ni == flat.numel()
+    cap = max(ni, 1)
+    k = [torch.full((cap,), -1, dtype=torch.int16, device=cuda), torch.empty(cap, dtype=torch.int16, device=cuda)]
+    v = [torch.full((cap,), -1, dtype=torch.int32, device=cuda), torch.empty(cap, dtype=torch.int32, device=cuda)]
+    check(L.gsx_intersect_tile_emit_pairs(c_u32(n), p(cum), p(order), p(ws), c_u32(16), c_u32(tw), c_u32(th),
+                                          c_i64(ni), p(k[0]), p(v[0]), stream))
+    ws2 = torch.empty(L.gsx_radix_sort_pairs_workspace_bytes(c_i64(cap)), dtype=torch.uint8, device=cuda)
+    sel = ctypes.c_int(0)
+    check(L.gsx_radix_sort_tile_pairs(c_i64(ni), p(k[0]), p(v[0]), p(k[1]), p(v[1]), L.gsx_n_bits(c_u32(tw * th)),
+                                      p(ws2), c_sz(ws2.numel()), ctypes.byref(sel), stream))
+    off = torch.full((1, th, tw), -1, dtype=torch.int32, device=cuda)
+    check(L.gsx_intersect_tile_pairs_offset(c_i64(ni), p(k[sel.value]), c_u32(tw), c_u32(th), p(off), stream))
+    bits_equal(N(v[sel.value][:ni]), N(flat), "values")
+    bits_equal(N(off), N(want_off), "per-tile ranges")
+    if n:
+        bits_equal(N(k[sel.value][:ni]).view(np.uint16).astype(np.int64), N(ids) >> 32, "tile indices")
+        # a bounded emission writes nothing beyond its capacity
+        k0 = torch.full((cap,), -1, dtype=torch.int16, device=cuda)
+        v0 = torch.full((cap,), -1, dtype=torch.int32, device=cuda)
+        check(L.gsx_intersect_tile_emit_pairs(c_u32(n), p(cum), p(order), p(ws), c_u32(16), c_u32(tw), c_u32(th),
+                                              c_i64(ni // 2), p(k0), p(v0), stream))
+        assert (N(k0[ni // 2:]) == -1).all() and (N(v0[ni // 2:]) == -1).all()
+        assert (N(v0[: ni // 2]) >= 0).all()
+
+
+def test_tile_pairs_unaligned_arrays(gsx, cuda):
+    """key arrays that do not start on a 16-byte boundary take the element-wise loads: same results"""
+    import ctypes
+    from lichtfeld_studio_amd._lib import c_i64, c_p, c_sz, c_u32, check, lib
+    L = lib()
+    rng = np.random.default_rng(77)
+    n, tw, th = 70_001, 78, 52
+    keys = rng.integers(0, tw * th, n).astype(np.uint16)
+    keys[keys == 17] = 18  # an empty tile
+    vals = rng.permutation(n).astype(np.int32)
+    order = np.argsort(keys, kind="stable")
+    big = [torch.empty(n + 8, dtype=torch.int16, device=cuda) for _ in range(2)]
+    k = [b[3:3 + n] for b in big]
+    k[0].copy_(T(keys.view(np.int16), cuda))
+    v = [T(vals, cuda), torch.empty(n, dtype=torch.int32, device=cuda)]
+    ws = torch.empty(L.gsx_radix_sort_pairs_workspace_bytes(c_i64(n)), dtype=torch.uint8, device=cuda)
+    sel = ctypes.c_int(-1)
+    p = lambda t: c_p(t.data_ptr())
+    stream = c_p(torch.cuda.current_stream(cuda).cuda_stream)
+    assert k[0].data_ptr() % 16 != 0
+    check(L.gsx_radix_sort_tile_pairs(c_i64(n), p(k[0]), p(v[0]), p(k[1]), p(v[1]), c_u32(12), p(ws),
+                                      c_sz(ws.numel()), ctypes.byref(sel), stream))
+    bits_equal(N(k[sel.value]).view(np.uint16), keys[order], "keys")
+    bits_equal(N(v[sel.value]), vals[order], "values")
+    want = np.searchsorted(keys[order], np.arange(tw * th)).astype(np.int32)
+    for arr in (k[sel.value], k[sel.value].clone()):  # unaligned, then aligned
+        off = torch.full((th * tw,), -1, dtype=torch.int32, device=cuda)
+        check(L.gsx_intersect_tile_pairs_offset(c_i64(n), p(arr), c_u32(tw), c_u32(th), p(off), stream))
+        bits_equal(N(off), want, "per-tile ranges")
+
+
+def test_tile_pairs_need_a_small_grid(gsx, cuda):
+    import ctypes
+    from lichtfeld_studio_amd._lib import c_i64, c_p, c_u32, check, lib
+    L = lib()
+    assert L.gsx_intersect_tile_pairs_fit(c_u32(256), c_u32(10)) == 0
+    x = torch.zeros(64, dtype=torch.int64, device=cuda)
+    with pytest.raises(gsx._lib.GsxError, match="64-bit keys"):
+        check(L.gsx_intersect_tile_emit_pairs(c_u32(4), c_p(x.data_ptr()), c_p(x.data_ptr()), c_p(x.data_ptr()),
+                                              c_u32(16), c_u32(256), c_u32(10), c_i64(8), c_p(x.data_ptr()),
+                                              c_p(x.data_ptr()), c_p(0)))
+
+
 @pytest.mark.parametrize("n", [1, 63, 64, 65, 4095, 4096, 4097, 100_003, 3_000_000])
 def test_radix_sort_stable(gsx, orc, cuda, n):
     ops = gsx.ops
