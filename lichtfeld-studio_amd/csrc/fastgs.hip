@@ -7,7 +7,8 @@
 //    with wave-cooperative counting for large footprints.  No atomic compaction: every Gaussian writes a
 //    (tile count << 32 | depth bits) key and the N keys are sorted on the depth bits, which gives the visiting
 //    order and the counts in that order deterministically (ties by index).
-//  * instances: emitted in depth order, so only the tile bits of the (tile << 32) keys are sorted afterwards.
+//  * instances: emitted in depth order with their 16-bit tile index as the key, which is all that is sorted
+//    afterwards.
 //  * blend forward / backward: one 256-lane workgroup per 16x16 tile, each wave owns an 8x8 pixel block and keeps
 //    its own ordered list of the batch's Gaussians whose footprint box meets the block.  The backward walks back
 //    to front from the last contributor with the final transmittance (no per-bucket checkpoints are stored: the
@@ -291,12 +292,12 @@ __global__ void __launch_bounds__(256) fgs_preprocess_kernel(
 }
 
 // ---- instances (create_instances_cu, kernels_forward.cuh:220-321) -----------------------------------
-// One lane per depth-ordered position; keys are (tile << 32) so that the pair sorter's bit range
-// [32, 32 + tile bits) orders them, values the primitive index.
+// One lane per depth-ordered position; keys are the 16-bit tile index (the reference's ushort keys,
+// buffer_utils.h:90), values the primitive index.
 __global__ void __launch_bounds__(256) fgs_create_instances_kernel(
     uint32_t N, const int32_t* __restrict__ order, const int64_t* __restrict__ cum /*inclusive*/,
     const uint32_t* __restrict__ n_touched, const ushort4* __restrict__ bounds, const float4* __restrict__ prims,
-    uint32_t grid_w, int64_t* __restrict__ keys, int32_t* __restrict__ vals) {
+    uint32_t grid_w, uint16_t* __restrict__ keys, int32_t* __restrict__ vals) {
     const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
     const uint32_t lane = threadIdx.x & 63u;
     bool active = idx < N;
@@ -321,7 +322,7 @@ __global__ void __launch_bounds__(256) fgs_create_instances_kernel(
         for (uint32_t k = 0; k < tile_count && k < kFgsSequential; ++k) {
             const uint32_t tx = b[0] + k % bw, ty = b[2] + k / bw;
             if (fgs_will_contribute(mx, my, c0, c1, c2, tx, ty, pt)) {
-                keys[write] = (int64_t)((uint64_t)(ty * grid_w + tx) << 32);
+                keys[write] = (uint16_t)(ty * grid_w + tx);
                 vals[write] = (int32_t)prim;
                 ++write;
             }
@@ -347,7 +348,7 @@ __global__ void __launch_bounds__(256) fgs_create_instances_kernel(
             if (hit) {
                 const uint32_t below =
                     __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
-                keys[at + below] = (int64_t)((uint64_t)(ty * grid_w + tx) << 32);
+                keys[at + below] = (uint16_t)(ty * grid_w + tx);
                 vals[at + below] = sprim;
             }
             at += (uint32_t)__builtin_popcountll(m);
@@ -848,11 +849,16 @@ static FgsPrimLayout fgs_prim_layout(uint32_t N) {
 struct FgsInstLayout {
     size_t keys1_off, vals0_off, vals1_off, offsets_off, sel_off, ws_off, total;
 };
+// bits of the tile index the instance sort looks at (at most 65 536 tiles)
+static uint32_t fgs_tile_bits(uint32_t n_tiles) {
+    const uint32_t b = gsx_n_bits(n_tiles);
+    return b < 16u ? b : 16u;
+}
 static FgsInstLayout fgs_inst_layout(int64_t n, uint32_t n_tiles) {
     FgsInstLayout L;
     const size_t m = (size_t)(n > 0 ? n : 1);
-    size_t at = align_up(m * 8, 256);
-    L.keys1_off = at, at += align_up(m * 8, 256);
+    size_t at = align_up(m * 2, 256);
+    L.keys1_off = at, at += align_up(m * 2, 256);
     L.vals0_off = at, at += align_up(m * 4, 256);
     L.vals1_off = at, at += align_up(m * 4, 256);
     L.offsets_off = at, at += align_up((size_t)n_tiles * 4, 256);
@@ -954,8 +960,8 @@ extern "C" int gsx_fastgs_render(uint32_t N, const gsx_fastgs_settings* settings
     const FgsPrimLayout L = fgs_prim_layout(N);
     const char* ps = (const char*)primitive_state;
     char* is = (char*)instance_state;
-    int64_t* keys0 = (int64_t*)is;
-    int64_t* keys1 = (int64_t*)(is + IL.keys1_off);
+    uint16_t* keys0 = (uint16_t*)is;
+    uint16_t* keys1 = (uint16_t*)(is + IL.keys1_off);
     int32_t* vals0 = (int32_t*)(is + IL.vals0_off);
     int32_t* vals1 = (int32_t*)(is + IL.vals1_off);
     int32_t* offsets = (int32_t*)(is + IL.offsets_off);
@@ -967,14 +973,14 @@ extern "C" int gsx_fastgs_render(uint32_t N, const gsx_fastgs_settings* settings
                            (const uint32_t*)(ps + L.n_touched_off), (const ushort4*)(ps + L.bounds_off),
                            (const float4*)ps, gw, keys0, vals0);
         GSX_LAUNCH_CHECK();
-        if ((rc = gsx_radix_sort_pairs(n_instances, keys0, vals0, keys1, vals1, 32, 32 + gsx_n_bits(n_tiles),
-                                       is + IL.ws_off, gsx_radix_sort_pairs_workspace_bytes(n_instances), &sel,
-                                       stream)) != GSX_OK)
+        if ((rc = gsx_radix_sort_tile_pairs(n_instances, keys0, vals0, keys1, vals1, fgs_tile_bits(n_tiles),
+                                            is + IL.ws_off, gsx_radix_sort_pairs_workspace_bytes(n_instances), &sel,
+                                            stream)) != GSX_OK)
             return rc;
     }
     // which buffer holds the sorted list: kept in the state for the backward (a host-side int in the first bytes
     // of a slot the kernels never touch would not survive a device buffer; it is recomputed there instead)
-    if ((rc = gsx_intersect_offset(n_instances, sel ? keys1 : keys0, 1, gw, gh, offsets, stream)) != GSX_OK)
+    if ((rc = gsx_intersect_tile_pairs_offset(n_instances, sel ? keys1 : keys0, gw, gh, offsets, stream)) != GSX_OK)
         return rc;
     char* px = (char*)pixel_state;
     const size_t plane = align_up((size_t)W * H * 4, 256);
@@ -1007,7 +1013,7 @@ extern "C" int gsx_fastgs_instance_list(const gsx_fastgs_settings* settings, int
     const uint32_t gw = (settings->width + kTile - 1) / kTile, gh = (settings->height + kTile - 1) / kTile;
     const FgsInstLayout IL = fgs_inst_layout(n_instances, gw * gh);
     // the pair sorter ping-pongs once per digit pass; its pass count for this bit range fixes the final buffer
-    const int sel = n_instances > 0 ? gsx_radix_sort_pairs_selector(n_instances, 32, 32 + gsx_n_bits(gw * gh)) : 0;
+    const int sel = n_instances > 0 ? gsx_radix_sort_pairs_selector(n_instances, 0, fgs_tile_bits(gw * gh)) : 0;
     const char* is = (const char*)instance_state;
     *instance_primitive = (const int32_t*)(is + (sel ? IL.vals1_off : IL.vals0_off));
     *tile_offsets = (const int32_t*)(is + IL.offsets_off);
