@@ -54,19 +54,23 @@ def load_package():
     return mod
 
 
-def algorithmic_bytes(N, K, H, W, n_isects, sort_bits):
-    """HBM bytes one launch of each streaming stage has to move (reads + writes), per the cost model."""
+def algorithmic_bytes(N, K, H, W, n_isects, sort_bits, key_bytes=8):
+    """HBM bytes one launch of each streaming stage has to move (reads + writes), per the cost model.
+    key_bytes: 8 for (tile << 32 | depth) keys, 2 for the 16-bit tile indices (sort_bits then counts from bit 0)."""
     P = H * W
-    passes = (sort_bits - 32 + 7) // 8  # the pairs are emitted in depth order: only the tile / camera bits are sorted
+    # the pairs are emitted in depth order: only the tile (/ camera) bits are sorted
+    passes = (sort_bits - (32 if key_bytes == 8 else 0) + 7) // 8
+    pair = key_bytes + 4
     return {
         "activate_params": N * (32 + 32),
         "projection_ut_3dgs_fused": N * (44 + 32),
         "activate_project_ut": N * (44 + 32 + 32),
+        "activate_project_sh_records": N * (44 + 32 + 32 + 12 * K + 12 + 96),
         "sh_colors_from_world": N * (12 + 12 * K + 8 + 12),
-        "intersect_tile_emit": N * (4 + 16 + 4 + 8) + n_isects * 12,
+        "intersect_tile_emit": N * (4 + 16 + 4 + 8) + n_isects * pair,
         "intersect_tile_count_ordered": N * (28 + 16 + (8 + 24) * 4 + 8 + 8),
-        "radix_sort_pairs": n_isects * (8 + 24) * passes,
-        "intersect_offset": n_isects * 8 + (P // 256) * 4,
+        "radix_sort_pairs": n_isects * (key_bytes + 2 * pair) * passes,
+        "intersect_offset": n_isects * key_bytes + (P // 256) * 4,
         "image_from_render": P * (12 + 12 + 12),
         "fusedssim": P * (24 + 12 + 36),
         "photometric_loss_forward": P * (12 + 12 + 36),
@@ -97,6 +101,8 @@ def main():
     ap.add_argument("--no-overlap", action="store_true",
                     help="keep every kernel of the step on one stream (default: the SH / record pass and the loss "
                          "reduction run on a second stream beside the sort chain / the backward rasterizer)")
+    ap.add_argument("--one-front-pass", action="store_true",
+                    help="activations + projection + SH colours + records as one launch")
     ap.add_argument("--no-tile-order", action="store_true", help="rasterize the tiles in index order")
     ap.add_argument("--cpu-threads", type=int, default=0, help="threads for the CPU baseline (0 = all)")
     ap.add_argument("--workload", choices=["gut", "fastgs"], default="gut",
@@ -134,7 +140,8 @@ def main():
         gt = torch.from_numpy(sc.target[None].copy()).to(dev)
     use_ssim = args.config != 1  # configuration 1 is L1 only
     ts = TrainStep(sc, dev, use_ssim=use_ssim, fused_update=not args.separate_update,
-                   fused_loss=not args.separate_update, overlap=not args.no_overlap)
+                   fused_loss=not args.separate_update, overlap=not args.no_overlap,
+                   one_front_pass=args.one_front_pass)
     ts.order_tiles = not args.no_tile_order
     setup_s = time.time() - t0
 
@@ -187,7 +194,8 @@ def main():
     del cp_src, cp_dst
 
     tile_bits = int(L.lib().gsx_n_bits(ctypes.c_uint32(ts.tw * ts.th)))
-    abytes = algorithmic_bytes(ts.N, ts.K, H, W, ts.n_isects, 32 + tile_bits + 1)
+    abytes = (algorithmic_bytes(ts.N, ts.K, H, W, ts.n_isects, tile_bits, 2) if ts.compact else
+              algorithmic_bytes(ts.N, ts.K, H, W, ts.n_isects, 32 + tile_bits + 1))
     kernels = {}
     for k, ms in stage_ms.items():
         e = {"ms": round(ms, 4)}

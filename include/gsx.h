@@ -379,6 +379,19 @@ GSX_API int gsx_activate_project_ut(uint32_t N, const float* means, const float*
                                     float near_plane, float far_plane, float radius_clip, gsx_ut_params ut,
                                     float* opacities, float* scales, float* quats, int32_t* radii, float* means2d,
                                     float* depths, float* conics, void* stream);
+/* gsx_activate_project_ut + gsx_sh_colors_records_from_world: the whole per-Gaussian front of a forward pass
+ * (splat_data.cpp:271-286 activations, ProjectionUT3DGSFused.cu:17-210, Rasterization.cpp:356-378 colours, the raster
+ * records) with the same results.  For K = 16 coefficient rows on a 16-byte boundary it is one pass over the Gaussians
+ * - the activated parameters and the visibility stay in registers, the parameters are read once - otherwise the two
+ * launches. */
+GSX_API int gsx_activate_project_sh_records(uint32_t N, uint32_t K, uint32_t sh_degree, const float* means,
+                                            const float* opacity_raw, const float* scaling_raw,
+                                            const float* rotation_raw, const float* sh_coeffs, const float* viewmat,
+                                            const float* Kmat, uint32_t image_width, uint32_t image_height,
+                                            float eps2d, float near_plane, float far_plane, float radius_clip,
+                                            gsx_ut_params ut, float* opacities, float* scales, float* quats,
+                                            int32_t* radii, float* means2d, float* depths, float* conics,
+                                            float* colors, void* records, void* stream);
 GSX_API int gsx_activate_params_bwd(uint32_t N, const float* opacity_raw, const float* scaling_raw,
                                     const float* rotation_raw, const float* v_opacities, const float* v_scales,
                                     const float* v_quats, float* v_opacity_raw, float* v_scaling_raw,

@@ -220,6 +220,50 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> intersect_tile(const at::Tensor m
     return std::make_tuple(tiles_per_gauss, isect_ids, flatten_ids);
 }
 
+namespace {
+// flatten_ids and offsets of one camera as intersect_tile(sort = true) + intersect_offset return them, without
+// forming the 64-bit keys: pairs in depth order with their 16-bit tile index as the sort key (the fused forward
+// keeps no isect_ids, Rasterization.cpp:413-424).  false where the grid needs the 64-bit keys.
+bool tile_lists(const at::Tensor& means2d, const at::Tensor& radii, const at::Tensor& depths, uint32_t tile_size,
+                uint32_t tile_width, uint32_t tile_height, at::Tensor* flatten_ids, at::Tensor* offsets) {
+    if (means2d.size(0) != 1 || !gsx_intersect_tile_pairs_fit(tile_width, tile_height))
+        return false;
+    const uint32_t N = (uint32_t)means2d.size(1);
+    void* stream = cur_stream(means2d);
+    const auto i32 = depths.options().dtype(at::kInt);
+    *offsets = at::empty({1, (int64_t)tile_height, (int64_t)tile_width}, i32);
+    int64_t n = 0;
+    at::Tensor order = at::empty({(int64_t)N}, i32), tiles_per_gauss = at::empty({(int64_t)N}, i32);
+    at::Tensor cum = at::empty({(int64_t)N}, depths.options().dtype(at::kLong));
+    at::Tensor ws = workspace(gsx_intersect_tile_count_ordered_workspace_bytes(N), depths);
+    if (N > 0)
+        gsx_check(gsx_intersect_tile_count_ordered(N, means2d.data_ptr<float>(), radii.data_ptr<int32_t>(),
+                                                   depths.data_ptr<float>(), tile_size, tile_width, tile_height,
+                                                   order.data_ptr<int32_t>(), tiles_per_gauss.data_ptr<int32_t>(),
+                                                   cum.data_ptr<int64_t>(), ws.data_ptr(), (size_t)ws.numel(), &n, 1,
+                                                   stream));
+    at::Tensor keys[2] = {at::empty({n}, depths.options().dtype(at::kShort)),
+                          at::empty({n}, depths.options().dtype(at::kShort))};
+    at::Tensor vals[2] = {at::empty({n}, i32), at::empty({n}, i32)};
+    int sel = 0;
+    if (n > 0) {
+        gsx_check(gsx_intersect_tile_emit_pairs(N, cum.data_ptr<int64_t>(), order.data_ptr<int32_t>(), ws.data_ptr(),
+                                                tile_size, tile_width, tile_height, n,
+                                                (uint16_t*)keys[0].data_ptr<int16_t>(), vals[0].data_ptr<int32_t>(),
+                                                stream));
+        at::Tensor ws2 = workspace(gsx_radix_sort_pairs_workspace_bytes(n), depths);
+        gsx_check(gsx_radix_sort_tile_pairs(n, (uint16_t*)keys[0].data_ptr<int16_t>(), vals[0].data_ptr<int32_t>(),
+                                            (uint16_t*)keys[1].data_ptr<int16_t>(), vals[1].data_ptr<int32_t>(),
+                                            gsx_n_bits(tile_width * tile_height), ws2.data_ptr(),
+                                            (size_t)ws2.numel(), &sel, stream));
+    }
+    gsx_check(gsx_intersect_tile_pairs_offset(n, (const uint16_t*)keys[sel].data_ptr<int16_t>(), tile_width,
+                                              tile_height, offsets->data_ptr<int32_t>(), stream));
+    *flatten_ids = vals[sel];
+    return true;
+}
+} // namespace
+
 at::Tensor intersect_offset(const at::Tensor isect_ids, const uint32_t C, const uint32_t tile_width,
                             const uint32_t tile_height) {
     DEVICE_GUARD(isect_ids);
@@ -519,10 +563,13 @@ rasterize_from_world_with_sh_fwd(const at::Tensor means, const at::Tensor quats,
         final_opacities = at::mul(final_opacities, compensations).contiguous();
     const uint32_t tile_width = (image_width + tile_size - 1) / tile_size;
     const uint32_t tile_height = (image_height + tile_size - 1) / tile_size;
-    auto isect = intersect_tile(means2d, radii, depths, at::nullopt, at::nullopt, C, tile_size, tile_width, tile_height,
-                                true);
-    at::Tensor flatten_ids = std::get<2>(isect);
-    at::Tensor offsets = intersect_offset(std::get<1>(isect), C, tile_width, tile_height);
+    at::Tensor flatten_ids, offsets;
+    if (!tile_lists(means2d, radii, depths, tile_size, tile_width, tile_height, &flatten_ids, &offsets)) {
+        auto isect = intersect_tile(means2d, radii, depths, at::nullopt, at::nullopt, C, tile_size, tile_width,
+                                    tile_height, true);
+        flatten_ids = std::get<2>(isect);
+        offsets = intersect_offset(std::get<1>(isect), C, tile_width, tile_height);
+    }
     auto r = rasterize_to_pixels_from_world_3dgs_fwd(means, quats, scaled_scales, colors, final_opacities.contiguous(),
                                                      fit_backgrounds(backgrounds, colors.size(-1)), masks, image_width, image_height, tile_size,
                                                      viewmats0, viewmats1, Ks, camera_model, ut_params, rs_type,

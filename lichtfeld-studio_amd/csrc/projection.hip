@@ -598,81 +598,69 @@ __global__ void __launch_bounds__(256) sh_bwd_generic_kernel(uint32_t N, uint32_
     }
 }
 
-// Colours AND raster records in one pass (what gsx_sh_colors_from_world followed by gsx_pack_raster_records
-// produce, same arithmetic): the colour goes straight from the SH evaluation into the record, and the coefficient
-// rows of Gaussians that touch no tile are not read at all.
-template <bool LDS16>
-__global__ void __launch_bounds__(256) sh_records_kernel(uint32_t N, uint32_t K, uint32_t degree,
-                                                          const float* __restrict__ means,
-                                                          const float* __restrict__ quats,
-                                                          const float* __restrict__ scales,
-                                                          const float* __restrict__ opacities,
-                                                          const float* __restrict__ coeffs,
-                                                          const int32_t* __restrict__ radii,
-                                                          const float* __restrict__ viewmat,
-                                                          const float* __restrict__ Kmat, uint32_t W, uint32_t H,
-                                                          float* __restrict__ colors, float4* __restrict__ records) {
-    // a wave stages its 64 coefficient rows 32 at a time: half the LDS per wave, more waves per CU to cover the
-    // memory round trips of this latency-bound pass
-    __shared__ float4 lds[LDS16 ? 4 * 32 * kShLdsF4 : 1];
-    const uint32_t e = blockIdx.x * 256u + threadIdx.x;
-    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    float4* wave_lds = lds + (LDS16 ? wave * 32 * kShLdsF4 : 0);
-    const bool live = e < N && radii[e * 2] > 0 && radii[e * 2 + 1] > 0;
-    // everything the record needs is requested now, together with the coefficient rows below: one memory round
-    // trip instead of one per phase (the 44 bytes are read for Gaussians without a tile too)
-    const uint32_t ec = min(e, N - 1);
-    const vec3 mean = ld3(means, ec);
-    const float opac = opacities[ec];
-    const quat q_in = ld4q(quats, ec);
-    const vec3 scl = ld3(scales, ec);
-    float co_reg[48];
-    if (LDS16) {
-        const uint32_t row0 = blockIdx.x * 256u + wave * 64u;
-        const uint64_t live_rows = __builtin_amdgcn_ballot_w64(live);
-        if (row0 < N && live_rows) {
-            const float4* src = reinterpret_cast<const float4*>(coeffs + (size_t)row0 * 48);
-            const uint32_t n_f4 = min(64u, N - row0) * kShRowF4;
-            float4 tmp[kShRowF4]; // all twelve requests leave before the first is needed
+// A wave's 64 consecutive coefficient rows (K = 16: 48 floats each, 16-byte aligned) -> the 48 coefficients of
+// every live lane's own row in registers.  Rows are read by consecutive lanes (request_coefficient_rows: the twelve
+// requests per lane leave together; rows of lanes that are not live are not read) and turned through LDS 32 at a
+// time (turn_coefficient_rows: half the LDS per wave, more waves per CU).  wave_lds: 32 * kShLdsF4 float4 owned by
+// the wave.
+__device__ __forceinline__ void request_coefficient_rows(const float* __restrict__ coeffs, uint32_t N, uint32_t row0,
+                                                         uint64_t live_rows, uint32_t lane, float4* tmp) {
+    const float4* src = reinterpret_cast<const float4*>(coeffs + (size_t)min(row0, N - 1) * 48);
+    const uint32_t n_f4 = row0 < N ? min(64u, N - row0) * kShRowF4 : 0u;
 #pragma unroll
-            for (uint32_t i = 0; i < kShRowF4; ++i) {
-                const uint32_t q = i * 64u + lane;
-                const uint32_t r = (q * 43691u) >> 19; // q / 12 for q < 768
-                tmp[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (q < n_f4 && ((live_rows >> r) & 1ull))
-                    tmp[i] = src[q];
-            }
+    for (uint32_t i = 0; i < kShRowF4; ++i) {
+        const uint32_t q = i * 64u + lane;
+        const uint32_t r = (q * 43691u) >> 19; // q / 12 for q < 768
+        tmp[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (q < n_f4 && ((live_rows >> r) & 1ull))
+            tmp[i] = src[q];
+    }
+}
+__device__ __forceinline__ void turn_coefficient_rows(const float4* tmp, uint32_t lane, float4* wave_lds,
+                                                      float* co_reg) {
 #pragma unroll
-            for (uint32_t half = 0; half < 2; ++half) {
+    for (uint32_t half = 0; half < 2; ++half) {
 #pragma unroll
-                for (uint32_t i = 0; i < kShRowF4 / 2; ++i) {
-                    const uint32_t q = i * 64u + lane;     // position inside this half's 32 rows
-                    const uint32_t r = (q * 43691u) >> 19; // q / 12
-                    wave_lds[r * kShLdsF4 + (q - r * kShRowF4)] = tmp[half * (kShRowF4 / 2) + i];
-                }
-                __builtin_amdgcn_wave_barrier();
-                if ((lane >> 5) == half) {
+        for (uint32_t i = 0; i < kShRowF4 / 2; ++i) {
+            const uint32_t q = i * 64u + lane;     // position inside this half's 32 rows
+            const uint32_t r = (q * 43691u) >> 19; // q / 12
+            wave_lds[r * kShLdsF4 + (q - r * kShRowF4)] = tmp[half * (kShRowF4 / 2) + i];
+        }
+        __builtin_amdgcn_wave_barrier();
+        if ((lane >> 5) == half) {
 #pragma unroll
-                    for (uint32_t k = 0; k < kShRowF4; ++k) {
-                        const float4 t = wave_lds[(lane & 31u) * kShLdsF4 + k];
-                        co_reg[4 * k + 0] = t.x;
-                        co_reg[4 * k + 1] = t.y;
-                        co_reg[4 * k + 2] = t.z;
-                        co_reg[4 * k + 3] = t.w;
-                    }
-                }
-                __builtin_amdgcn_wave_barrier();
+            for (uint32_t k = 0; k < kShRowF4; ++k) {
+                const float4 t = wave_lds[(lane & 31u) * kShLdsF4 + k];
+                co_reg[4 * k + 0] = t.x;
+                co_reg[4 * k + 1] = t.y;
+                co_reg[4 * k + 2] = t.z;
+                co_reg[4 * k + 3] = t.w;
             }
         }
+        __builtin_amdgcn_wave_barrier();
     }
-    if (e >= N)
+}
+__device__ __forceinline__ void wave_coefficient_rows(const float* __restrict__ coeffs, uint32_t N, uint32_t row0,
+                                                      bool live, uint32_t lane, float4* wave_lds, float* co_reg) {
+    const uint64_t live_rows = __builtin_amdgcn_ballot_w64(live);
+    if (row0 >= N || !live_rows)
         return;
+    float4 tmp[kShRowF4];
+    request_coefficient_rows(coeffs, N, row0, live_rows, lane, tmp);
+    turn_coefficient_rows(tmp, lane, wave_lds, co_reg);
+}
+
+// Gaussian e's colour (clamped SH colour of the direction camera -> mean) and, if it touches a tile, its record
+__device__ __forceinline__ void color_and_record(uint32_t e, bool live, uint32_t degree, vec3 mean, float opac,
+                                                 quat q_in, vec3 scl, const float* co,
+                                                 const float* __restrict__ viewmat, const float* __restrict__ Kmat,
+                                                 uint32_t W, uint32_t H, float* __restrict__ colors,
+                                                 float4* __restrict__ records) {
     float c[3] = {0.f, 0.f, 0.f};
     if (live) {
         const vec3 dir = sub(mean, campos_from_viewmat(viewmat));
         float B[25];
         sh_basis(degree, dir, B);
-        const float* co = LDS16 ? co_reg : coeffs + (size_t)e * K * 3;
 #pragma unroll
         for (uint32_t ch = 0; ch < 3; ++ch)
             c[ch] = gsx::fmax(sh_color_channel(degree, dir, B, co, ch) + 0.5f, 0.0f);
@@ -687,6 +675,147 @@ __global__ void __launch_bounds__(256) sh_records_kernel(uint32_t N, uint32_t K,
     const vec3 gro = mul(M, sub(ray_o, mean));
     const RecordRegion reg = record_region(gro, M, opac, mean, viewmat, Kmat[0], Kmat[4], Kmat[2], Kmat[5], W, H);
     store_record(records + (size_t)e * kRecordF4, gro, opac, M, c[0], c[1], c[2], reg);
+}
+
+// The same for a whole wave (lane = Gaussian row0 + lane; lanes beyond N are not live): the 96-byte records are
+// turned through LDS and leave as runs of consecutive 16-byte pieces instead of 64 strided ones per store.
+// wave_lds: kShWaveLdsF4 float4 owned by the wave (free again after wave_coefficient_rows).
+static constexpr uint32_t kRecLdsF4 = 7; // padded record stride in LDS: conflict-free 16-byte accesses
+static constexpr uint32_t kShWaveLdsF4 = 64 * kRecLdsF4 > 32 * kShLdsF4 ? 64 * kRecLdsF4 : 32 * kShLdsF4;
+__device__ __forceinline__ void wave_color_and_record(uint32_t row0, uint32_t N, uint32_t lane, bool live,
+                                                      uint32_t degree, vec3 mean, float opac, quat q_in, vec3 scl,
+                                                      const float* co, const float* __restrict__ viewmat,
+                                                      const float* __restrict__ Kmat, uint32_t W, uint32_t H,
+                                                      float* __restrict__ colors, float4* __restrict__ records,
+                                                      float4* wave_lds) {
+    const uint32_t e = row0 + lane;
+    float c[3] = {0.f, 0.f, 0.f};
+    if (live) {
+        const vec3 dir = sub(mean, campos_from_viewmat(viewmat));
+        float B[25];
+        sh_basis(degree, dir, B);
+#pragma unroll
+        for (uint32_t ch = 0; ch < 3; ++ch)
+            c[ch] = gsx::fmax(sh_color_channel(degree, dir, B, co, ch) + 0.5f, 0.0f);
+        const vec3 ray_o = camera_ray_origin(load_cam_pose(viewmat));
+        const mat3 M = record_whitening(q_in, scl);
+        const vec3 gro = mul(M, sub(ray_o, mean));
+        const RecordRegion reg = record_region(gro, M, opac, mean, viewmat, Kmat[0], Kmat[4], Kmat[2], Kmat[5], W, H);
+        store_record(wave_lds + lane * kRecLdsF4, gro, opac, M, c[0], c[1], c[2], reg);
+    }
+    if (e < N) {
+        colors[e * 3 + 0] = c[0];
+        colors[e * 3 + 1] = c[1];
+        colors[e * 3 + 2] = c[2];
+    }
+    const uint64_t live_rows = __builtin_amdgcn_ballot_w64(live);
+    __builtin_amdgcn_wave_barrier();
+    float4* dst = records + (size_t)row0 * kRecordF4;
+#pragma unroll
+    for (uint32_t i = 0; i < kRecordF4; ++i) {
+        const uint32_t q = i * 64u + lane;     // piece q of the wave's 64 * 6
+        const uint32_t r = (q * 43691u) >> 18; // q / 6 for q < 384
+        if ((live_rows >> r) & 1ull)           // a Gaussian no tile lists keeps its record untouched
+            dst[q] = wave_lds[r * kRecLdsF4 + (q - r * kRecordF4)];
+    }
+}
+
+// Colours AND raster records in one pass (what gsx_sh_colors_from_world followed by gsx_pack_raster_records
+// produce, same arithmetic): the colour goes straight from the SH evaluation into the record, and the coefficient
+// rows of Gaussians that touch no tile are not read at all.
+template <bool LDS16>
+__global__ void __launch_bounds__(256) sh_records_kernel(uint32_t N, uint32_t K, uint32_t degree,
+                                                          const float* __restrict__ means,
+                                                          const float* __restrict__ quats,
+                                                          const float* __restrict__ scales,
+                                                          const float* __restrict__ opacities,
+                                                          const float* __restrict__ coeffs,
+                                                          const int32_t* __restrict__ radii,
+                                                          const float* __restrict__ viewmat,
+                                                          const float* __restrict__ Kmat, uint32_t W, uint32_t H,
+                                                          float* __restrict__ colors, float4* __restrict__ records) {
+    __shared__ float4 lds[LDS16 ? 4 * kShWaveLdsF4 : 1];
+    const uint32_t e = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const bool live = e < N && radii[e * 2] > 0 && radii[e * 2 + 1] > 0;
+    // everything the record needs is requested now, together with the coefficient rows below: one memory round
+    // trip instead of one per phase (the 44 bytes are read for Gaussians without a tile too)
+    const uint32_t ec = min(e, N - 1);
+    const vec3 mean = ld3(means, ec);
+    const float opac = opacities[ec];
+    const quat q_in = ld4q(quats, ec);
+    const vec3 scl = ld3(scales, ec);
+    float co_reg[48];
+    if (LDS16) {
+        const uint32_t row0 = blockIdx.x * 256u + wave * 64u;
+        float4* wave_lds = lds + wave * kShWaveLdsF4;
+        wave_coefficient_rows(coeffs, N, row0, live, lane, wave_lds, co_reg);
+        wave_color_and_record(row0, N, lane, live, degree, mean, opac, q_in, scl, co_reg, viewmat, Kmat, W, H, colors,
+                              records, wave_lds);
+        return;
+    }
+    if (e >= N)
+        return;
+    color_and_record(e, live, degree, mean, opac, q_in, scl, coeffs + (size_t)e * K * 3, viewmat, Kmat, W, H, colors,
+                     records);
+}
+
+// The whole per-Gaussian front of a training step in one pass (one camera, K = 16): activations, UT projection,
+// SH colour and raster record - what projection_ut_raw_kernel followed by sh_records_kernel<true> produce, same
+// arithmetic; the activated parameters, the radii and the visibility stay in registers between the two halves.
+// (Requesting a chunk's coefficient rows while the next chunk is projected - a software pipeline inside the wave -
+// needs about 300 live registers as the compiler schedules it and runs slower than this plain sequence.)
+__global__ void __launch_bounds__(256) project_sh_records_kernel(
+    uint32_t N, uint32_t degree, const float* __restrict__ means, const float* __restrict__ opacity_raw,
+    const float* __restrict__ scaling_raw, const float* __restrict__ rotation_raw, const float* __restrict__ coeffs,
+    const float* __restrict__ viewmat, const float* __restrict__ Ks, ProjCfg cfg, float* __restrict__ opacities,
+    float* __restrict__ scales, float* __restrict__ quats, int32_t* __restrict__ radii, float* __restrict__ means2d,
+    float* __restrict__ depths, float* __restrict__ conics, float* __restrict__ colors,
+    float4* __restrict__ records) {
+    __shared__ float4 lds[4 * kShWaveLdsF4];
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t ic = min(idx, N - 1);
+    const vec3 mean = ld3(means, ic);
+    const Activated a = activate(opacity_raw[ic], ld3(scaling_raw, ic), ld4q(rotation_raw, ic));
+    bool live = false;
+    if (idx < N) {
+        opacities[idx] = a.opacity;
+        scales[3 * idx + 0] = a.scales.x;
+        scales[3 * idx + 1] = a.scales.y;
+        scales[3 * idx + 2] = a.scales.z;
+        reinterpret_cast<float4*>(quats)[idx] = make_float4(a.quat.w, a.quat.x, a.quat.y, a.quat.z);
+        cfg.fx = Ks[0];
+        cfg.fy = Ks[4];
+        cfg.cx = Ks[2];
+        cfg.cy = Ks[5];
+        const CamPose cp = load_cam_pose(viewmat);
+        quat qc;
+        vec3 tc;
+        shutter_pose(cp, 0.5f, &qc, &tc);
+        ProjOut o;
+        live = project_ut<false>(cfg, cp, qc, tc, mean, a.quat, a.scales, true, a.opacity, &o);
+        int2* r2 = reinterpret_cast<int2*>(radii);
+        if (!live) {
+            r2[idx] = make_int2(0, 0);
+        } else {
+            r2[idx] = make_int2((int32_t)o.rx, (int32_t)o.ry);
+            reinterpret_cast<float2*>(means2d)[idx] = make_float2(o.mx, o.my);
+            depths[idx] = o.depth;
+            if (conics != nullptr) {
+                conics[idx * 3 + 0] = o.c0;
+                conics[idx * 3 + 1] = o.c1;
+                conics[idx * 3 + 2] = o.c2;
+            }
+            live = o.rx > 0.f && o.ry > 0.f; // what sh_records_kernel reads back from radii
+        }
+    }
+    float co_reg[48];
+    const uint32_t row0 = blockIdx.x * 256u + wave * 64u;
+    float4* wave_lds = lds + wave * kShWaveLdsF4;
+    wave_coefficient_rows(coeffs, N, row0, live, lane, wave_lds, co_reg);
+    wave_color_and_record(row0, N, lane, live, degree, mean, a.opacity, a.quat, a.scales, co_reg, viewmat, Ks, cfg.W,
+                          cfg.H, colors, records, wave_lds);
 }
 
 template <bool WORLD>
@@ -869,6 +998,48 @@ extern "C" int gsx_sh_colors_records_from_world(uint32_t N, uint32_t K, uint32_t
         hipLaunchKernelGGL((sh_records_kernel<false>), grid, block, 0, (hipStream_t)stream, N, K, sh_degree, means,
                            quats, scales, opacities, sh_coeffs, radii, viewmat, Kmat, image_width, image_height, colors,
                            (float4*)records);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+// gsx_activate_project_ut followed by gsx_sh_colors_records_from_world, as one pass over the Gaussians where the
+// coefficient layout allows it (K = 16, 16-byte aligned rows), as those two launches otherwise: same outputs.
+extern "C" int gsx_activate_project_sh_records(uint32_t N, uint32_t K, uint32_t sh_degree, const float* means,
+                                               const float* opacity_raw, const float* scaling_raw,
+                                               const float* rotation_raw, const float* sh_coeffs,
+                                               const float* viewmat, const float* Kmat, uint32_t image_width,
+                                               uint32_t image_height, float eps2d, float near_plane, float far_plane,
+                                               float radius_clip, gsx_ut_params ut, float* opacities, float* scales,
+                                               float* quats, int32_t* radii, float* means2d, float* depths,
+                                               float* conics, float* colors, void* records, void* stream) {
+    if (N == 0)
+        return GSX_OK;
+    const bool one_pass = K == 16 && (((uintptr_t)sh_coeffs) & 15u) == 0;
+    if (!one_pass) {
+        const int rc = gsx_activate_project_ut(N, means, opacity_raw, scaling_raw, rotation_raw, viewmat, Kmat,
+                                               image_width, image_height, eps2d, near_plane, far_plane, radius_clip,
+                                               ut, opacities, scales, quats, radii, means2d, depths, conics, stream);
+        if (rc != GSX_OK)
+            return rc;
+        return gsx_sh_colors_records_from_world(N, K, sh_degree, means, quats, scales, opacities, sh_coeffs, radii,
+                                                viewmat, Kmat, image_width, image_height, colors, records, stream);
+    }
+    GSX_REQUIRE(means && opacity_raw && scaling_raw && rotation_raw && sh_coeffs && viewmat && Kmat && opacities &&
+                    scales && quats && radii && means2d && depths && colors && records,
+                GSX_ERR_INVALID_ARGUMENT, "activate_project_sh_records: null tensor");
+    GSX_REQUIRE((((uintptr_t)rotation_raw) & 15) == 0 && (((uintptr_t)quats) & 15) == 0 &&
+                    ((uintptr_t)records & 15) == 0,
+                GSX_ERR_INVALID_ARGUMENT, "activate_project_sh_records: quaternions / records need 16-byte alignment");
+    GSX_REQUIRE(sh_degree <= 3, GSX_ERR_INVALID_ARGUMENT, "activate_project_sh_records: degree %u needs K >= %u (got %u)",
+                sh_degree, (sh_degree + 1) * (sh_degree + 1), K);
+    ProjCfg cfg;
+    memset(&cfg, 0, sizeof(cfg));
+    cfg.W = image_width, cfg.H = image_height;
+    cfg.eps2d = eps2d, cfg.near_plane = near_plane, cfg.far_plane = far_plane, cfg.radius_clip = radius_clip;
+    set_ut_constants(cfg, ut);
+    hipLaunchKernelGGL(project_sh_records_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, sh_degree,
+                       means, opacity_raw, scaling_raw, rotation_raw, sh_coeffs, viewmat, Kmat, cfg, opacities, scales,
+                       quats, radii, means2d, depths, conics, colors, (float4*)records);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

@@ -165,6 +165,47 @@ def intersect_tile(means2d, radii, depths, camera_ids, gaussian_ids, C, tile_siz
     return tiles_per_gauss, isect_ids, flatten_ids
 
 
+def _tile_lists(means2d, radii, depths, tile_size, tile_width, tile_height):
+    """(flatten_ids [I] i32, offsets [1,Th,Tw] i32) of one camera, as intersect_tile(sort=True) + intersect_offset
+    return them, without forming the 64-bit keys: pairs in depth order with their 16-bit tile index as the sort key
+    (for a caller that keeps no isect_ids: Rasterization.cpp:413-424).  None where the grid needs the 64-bit keys."""
+    if means2d.size(0) != 1 or not lib().gsx_intersect_tile_pairs_fit(c_u32(tile_width), c_u32(tile_height)):
+        return None
+    dev = means2d.device
+    N = means2d.size(1)
+    _sized(means2d, "means2d", 1, N, 2), _sized(radii, "radii", 1, N, 2), _sized(depths, "depths", 1, N)
+    if radii.dtype != torch.int32:
+        raise RuntimeError("radii must be int32")
+    offsets = torch.empty((1, tile_height, tile_width), dtype=torch.int32, device=dev)
+    n_isects = c_i64(0)
+    with torch.cuda.device(dev):
+        st = _stream(dev)
+        order = torch.empty((N,), dtype=torch.int32, device=dev)
+        tiles_per_gauss = torch.empty((N,), dtype=torch.int32, device=dev)
+        cum = torch.empty((N,), dtype=torch.int64, device=dev)
+        ws = _workspace(lib().gsx_intersect_tile_count_ordered_workspace_bytes(c_u32(N)), dev)
+        check(lib().gsx_intersect_tile_count_ordered(
+            c_u32(N), _ptr(means2d), _ptr(radii), _ptr(depths), c_u32(tile_size), c_u32(tile_width),
+            c_u32(tile_height), _ptr(order), _ptr(tiles_per_gauss), _ptr(cum), _ptr(ws), c_sz(ws.numel()),
+            ctypes.byref(n_isects), c_i(1), st))
+        n = n_isects.value if N else 0
+        keys = [torch.empty((n,), dtype=torch.int16, device=dev) for _ in range(2)]
+        vals = [torch.empty((n,), dtype=torch.int32, device=dev) for _ in range(2)]
+        sel = c_i(0)
+        if n:
+            check(lib().gsx_intersect_tile_emit_pairs(
+                c_u32(N), _ptr(cum), _ptr(order), _ptr(ws), c_u32(tile_size), c_u32(tile_width), c_u32(tile_height),
+                c_i64(n), _ptr(keys[0]), _ptr(vals[0]), st))
+            ws2 = _workspace(lib().gsx_radix_sort_pairs_workspace_bytes(c_i64(n)), dev)
+            check(lib().gsx_radix_sort_tile_pairs(
+                c_i64(n), _ptr(keys[0]), _ptr(vals[0]), _ptr(keys[1]), _ptr(vals[1]),
+                c_u32(lib().gsx_n_bits(c_u32(tile_width * tile_height))), _ptr(ws2), c_sz(ws2.numel()),
+                ctypes.byref(sel), st))
+        check(lib().gsx_intersect_tile_pairs_offset(c_i64(n), _ptr(keys[sel.value]), c_u32(tile_width),
+                                                    c_u32(tile_height), _ptr(offsets), st))
+    return vals[sel.value], offsets
+
+
 def radix_sort_double_buffer(n_isects, tile_n_bits, cam_n_bits, isect_ids, flatten_ids, begin_bit=0):
     """Intersect.h:39-46.  Returns the sorted (isect_ids, flatten_ids); like the reference's DoubleBuffer the
     result may live in either the input tensors or the internally allocated pair.  begin_bit > 0 sorts on the
@@ -428,9 +469,14 @@ def rasterize_from_world_with_sh_fwd(means, quats, scales, opacities, sh_coeffs,
         final_opacities = (final_opacities * comp).contiguous()
     tile_width = (image_width + tile_size - 1) // tile_size
     tile_height = (image_height + tile_size - 1) // tile_size
-    _, isect_ids, flatten_ids = intersect_tile(means2d, radii, depths, None, None, C, tile_size, tile_width,
-                                               tile_height, True)
-    offsets = intersect_offset(isect_ids, C, tile_width, tile_height)
+    lists = None if return_isect_ids else _tile_lists(means2d, radii, depths, tile_size, tile_width, tile_height)
+    if lists is not None:
+        isect_ids = None
+        flatten_ids, offsets = lists
+    else:
+        _, isect_ids, flatten_ids = intersect_tile(means2d, radii, depths, None, None, C, tile_size, tile_width,
+                                                   tile_height, True)
+        offsets = intersect_offset(isect_ids, C, tile_width, tile_height)
     renders, alphas, last_ids = rasterize_to_pixels_from_world_3dgs_fwd(
         means, quats, scaled_scales, colors, final_opacities, _fit_backgrounds(backgrounds, colors.size(-1)), masks,
         image_width, image_height, tile_size, viewmats0, viewmats1, Ks, camera_model, ut_params, rs_type, radial_coeffs, tangential_coeffs,

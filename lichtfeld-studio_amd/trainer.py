@@ -28,9 +28,10 @@ def _p(t):
 class TrainStep:
     def __init__(self, scene, device="cuda:0", lrs=None, lambda_dssim=0.2, betas=(0.9, 0.999), eps=1e-15,
                  scene_scale=1.0, sh_degree=None, use_ssim=True, fused_update=False, fused_loss=False,
-                 scale_reg=0.0, opacity_reg=0.0, overlap=False, tile_pairs=True):
+                 scale_reg=0.0, opacity_reg=0.0, overlap=False, tile_pairs=True, one_front_pass=False):
         self.dev = torch.device(device)
         self.lib = lib()
+        self.one_front_pass = one_front_pass  # activations + projection + SH colours + records as one launch
         self.tile_pairs = tile_pairs  # sort (u16 tile index, id) pairs where the tile grid allows it
         f = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(self.dev)
         self.N = scene.means.shape[0]
@@ -198,11 +199,24 @@ class TrainStep:
         self._ensure_image(H, W)
         self.viewmat, self.Kmat, self.W, self.H = viewmat, K, W, H
         P, A, J = self.params, self.act, self.proj
-        self._run("activate_project_ut", lb.gsx_activate_project_ut, c_u32(N), _p(P["means"]), _p(P["opacity"]),
-                  _p(P["scaling"]), _p(P["rotation"]), _p(viewmat), _p(K), c_u32(W), c_u32(H), c_f(0.3), c_f(0.01),
-                  c_f(1e4), c_f(0.0), self.ut, _p(A["opacities"]), _p(A["scales"]), _p(A["quats"]), _p(J["radii"]),
-                  _p(J["means2d"]), _p(J["depths"]), _p(J["conics"]), s)
-        if self.side is not None:
+        sh_args = (c_u32(N), c_u32(self.K), c_u32(self.sh_degree), _p(P["means"]), _p(A["quats"]), _p(A["scales"]),
+                   _p(A["opacities"]), _p(P["shs"]), _p(J["radii"]), _p(viewmat), _p(K), c_u32(W), c_u32(H),
+                   _p(self.colors), _p(self.records))
+        if self.one_front_pass:
+            # activations, projection, SH colours and records in one pass over the Gaussians: nothing runs beside
+            # the latency-bound sort chain
+            self._run("activate_project_sh_records", lb.gsx_activate_project_sh_records, c_u32(N), c_u32(self.K),
+                      c_u32(self.sh_degree), _p(P["means"]), _p(P["opacity"]), _p(P["scaling"]), _p(P["rotation"]),
+                      _p(P["shs"]), _p(viewmat), _p(K), c_u32(W), c_u32(H), c_f(0.3), c_f(0.01), c_f(1e4), c_f(0.0),
+                      self.ut, _p(A["opacities"]), _p(A["scales"]), _p(A["quats"]), _p(J["radii"]), _p(J["means2d"]),
+                      _p(J["depths"]), _p(J["conics"]), _p(self.colors), _p(self.records), s)
+        else:
+            self._run("activate_project_ut", lb.gsx_activate_project_ut, c_u32(N), _p(P["means"]), _p(P["opacity"]),
+                      _p(P["scaling"]), _p(P["rotation"]), _p(viewmat), _p(K), c_u32(W), c_u32(H), c_f(0.3),
+                      c_f(0.01), c_f(1e4), c_f(0.0), self.ut, _p(A["opacities"]), _p(A["scales"]), _p(A["quats"]),
+                      _p(J["radii"]), _p(J["means2d"]), _p(J["depths"]), _p(J["conics"]), s)
+        side_sh = self.side is not None and not self.one_front_pass
+        if side_sh:
             self.ev_fork.record(torch.cuda.current_stream(self.dev))
         # Tile counts in depth order; the total comes back through pinned memory without blocking, and the SH /
         # record passes (which do not need it) run while the host waits for it.
@@ -211,10 +225,9 @@ class TrainStep:
                   _p(self.tiles_per_gauss), _p(self.cum), _p(self.ws_count), c_sz(self.ws_count.numel()),
                   c_p(self.n_isects_pinned.data_ptr()), c_i(0), s)
         self.count_done.record(torch.cuda.current_stream(self.dev))
-        sh_args = (c_u32(N), c_u32(self.K), c_u32(self.sh_degree), _p(P["means"]), _p(A["quats"]), _p(A["scales"]),
-                   _p(A["opacities"]), _p(P["shs"]), _p(J["radii"]), _p(viewmat), _p(K), c_u32(W), c_u32(H),
-                   _p(self.colors), _p(self.records))
-        if self.side is None:
+        if self.one_front_pass:
+            pass
+        elif not side_sh:
             self._run("sh_colors_records_from_world", lb.gsx_sh_colors_records_from_world, *sh_args, s)
         else:
             self.side.wait_event(self.ev_fork)  # recorded after the activation / projection pass
@@ -272,7 +285,7 @@ class TrainStep:
                           c_u32(self.th), _p(self.tile_order), s)
             order = _p(self.tile_order)
         self._tile_order_arg = order
-        if self.side is not None:
+        if side_sh:
             torch.cuda.current_stream(self.dev).wait_event(self.ev_join)  # colours and records are ready
         self._run("rasterize_to_pixels_from_world_3dgs_fwd", lb.gsx_rasterize_records_fwd, c_i64(n),
                   _p(self.records), c_p(None), c_u32(3), _p(self.bg), c_p(None), c_u32(W), c_u32(H), _p(viewmat),

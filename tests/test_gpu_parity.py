@@ -458,6 +458,17 @@ def test_fused_forward_bit_exact(gsx, orc, cuda, n, bg):
     bits_equal(N(renders), r_renders, "image is expected bit-exact")
     bits_equal(N(alphas), r_alphas, '')
     assert r_alphas.mean() > 0.05  # the scene actually covers the image
+    # the operator as the reference declares it (no keys returned) builds its lists from 16-bit tile pairs: same tuple
+    plain = ops.rasterize_from_world_with_sh_fwd(d["means"], d["quats"], d["scales"], d["op"], d["shs"], 3,
+                                                 d["bg"] if bg else None, None, cam.width, cam.height, 16, d["vm"],
+                                                 None, d["K"], 0, 0.3, 0.01, 1e4, 0.0, 1.0, False, 0,
+                                                 ops.UnscentedTransformParameters(), 4)
+    assert len(plain) == 10
+    for name, a, b in zip(("renders", "alphas", "radii", "means2d", "depths", "colors", "offsets", "flatten_ids",
+                           "last_ids"), plain, got):
+        if name in ("means2d", "depths", "colors"):  # rows of culled Gaussians are not written
+            a, b = a[0][torch.from_numpy(vis).to(cuda)], b[0][torch.from_numpy(vis).to(cuda)]
+        assert torch.equal(a, b), name
 
 
 def check_raster_gradients(got5, o32_5, g64, tag=""):

@@ -235,6 +235,39 @@ def test_speculative_emission_and_overlap_change_nothing(gsx, cuda):
             assert torch.equal(a.params[k], b.params[k]), k
 
 
+@pytest.mark.parametrize("n,degree", [(1, 3), (300, 0), (70_001, 3), (40_000, 2)])
+def test_one_front_pass(gsx, cuda, n, degree):
+    """activations + projection + SH colours + records as one launch: every output equals, bit for bit, what the
+    separate launches write (records and projection outputs of Gaussians that touch no tile are never written by
+    either and are not compared)"""
+    from lichtfeld_studio_amd.trainer import TrainStep
+    sc = gsx.scenes.config(3, n)
+    sc.scaling_raw += 0.8
+    cam = gsx.scenes.orbit_camera(1.1, 4.0, 413, 277, 380.0)
+    W, H = cam.width, cam.height
+    vm = torch.from_numpy(cam.viewmat[None].copy()).to(cuda)
+    Km = torch.from_numpy(cam.K[None].copy()).to(cuda)
+    a = TrainStep(sc, cuda, fused_update=True, fused_loss=True, sh_degree=degree, one_front_pass=False)
+    b = TrainStep(sc, cuda, fused_update=True, fused_loss=True, sh_degree=degree, one_front_pass=True)
+    for ts in (a, b):
+        ts.records.zero_()
+        for t in ts.proj.values():
+            t.zero_()
+        ts.forward(vm, Km, W, H)
+    torch.cuda.synchronize()
+    assert a.n_isects == b.n_isects
+    for k in ("opacities", "scales", "quats"):
+        assert torch.equal(a.act[k], b.act[k]), k
+    for k in a.proj:
+        assert torch.equal(a.proj[k], b.proj[k]), k
+    assert torch.equal(a.colors, b.colors)
+    assert torch.equal(a.records, b.records)
+    assert torch.equal(a.render, b.render) and torch.equal(a.last_ids, b.last_ids)
+    if n > 1000:
+        live = (a.proj["radii"].reshape(-1, 2) > 0).all(-1)
+        assert 0.05 < float(live.float().mean()) < 0.95  # both kinds of Gaussian are present
+
+
 def test_tile_visiting_order(gsx, cuda):
     """gsx_tile_order returns a permutation of the tiles with the list lengths falling from class to class (16 classes
     per octave); rasterizing in that order changes nothing: forward outputs bit for bit, backward accumulators to
