@@ -103,6 +103,9 @@ def main():
                          "reduction run on a second stream beside the sort chain / the backward rasterizer)")
     ap.add_argument("--one-front-pass", action="store_true",
                     help="activations + projection + SH colours + records as one launch")
+    ap.add_argument("--alternate-cameras", action="store_true",
+                    help="hand the step two camera tensors in turn (same pose): the forward pass then cannot reuse "
+                         "the previous step's tile costs, as in a training loop that changes camera every step")
     ap.add_argument("--no-tile-order", action="store_true", help="rasterize the tiles in index order")
     ap.add_argument("--cpu-threads", type=int, default=0, help="threads for the CPU baseline (0 = all)")
     ap.add_argument("--workload", choices=["gut", "fastgs"], default="gut",
@@ -146,13 +149,14 @@ def main():
     setup_s = time.time() - t0
 
     dominant = "rasterize_bwd_accumulate"
-    for _ in range(args.warmup):
-        ts.step(viewmat, Kmat, W, H, gt)
+    views = [viewmat, viewmat.clone()] if args.alternate_cameras else [viewmat]
+    for i in range(args.warmup):
+        ts.step(views[i % len(views)], Kmat, W, H, gt)
     torch.cuda.synchronize()
     ts.start_timing([dominant, "rasterize_to_pixels_from_world_3dgs_fwd"])
     t1 = time.perf_counter()
-    for _ in range(args.steps):
-        ts.step(viewmat, Kmat, W, H, gt)
+    for i in range(args.steps):
+        ts.step(views[i % len(views)], Kmat, W, H, gt)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t1
     in_loop = ts.stop_timing()

@@ -136,8 +136,8 @@ __global__ void __launch_bounds__(256) scan_block_offsets_kernel(uint32_t nb, in
             block_sums[i] = carry + ex;
         carry += total;
     }
-    if (threadIdx.x == 0)
-        *total_out = carry;
+    if (threadIdx.x == 0) // total_out may be pinned host memory: one 8-byte store at system scope
+        __hip_atomic_store(total_out, carry, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 // Per-block scan plus the total of the earlier blocks.  SUMS: block_sums holds the blocks' own totals and every block
@@ -175,7 +175,7 @@ __global__ void __launch_bounds__(256) scan_apply_kernel(uint32_t n, const int32
             out[base + i] = run;
     }
     if (SUMS && blockIdx.x == gridDim.x - 1 && threadIdx.x == 0)
-        *total_out = offset + total;
+        __hip_atomic_store(total_out, offset + total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 // IntersectTile.cu:78-113 second pass: keys and values in emission order (ascending position, row-major tiles
@@ -466,6 +466,18 @@ int scan_counts(uint32_t n, const int32_t* counts, const int64_t* keys, bool rec
     return GSX_OK;
 }
 
+// The address under which kernels of the current device can write a pinned host slot, or nullptr for pageable memory.
+int64_t* device_view_of_host_slot(int64_t* slot) {
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, slot) != hipSuccess) {
+        (void)hipGetLastError(); // not known to the runtime: pageable
+        return nullptr;
+    }
+    if (attr.type != hipMemoryTypeHost || attr.devicePointer == nullptr)
+        return nullptr;
+    return (int64_t*)attr.devicePointer;
+}
+
 // tile grids whose rectangle corners fit a byte each: the depth keys then carry the rectangle
 bool rect_keys_fit(uint32_t tile_width, uint32_t tile_height) { return tile_width <= 255 && tile_height <= 255; }
 
@@ -564,10 +576,14 @@ int ordered_counts_from_keys(const char* who, uint32_t N, int32_t* order, int64_
         GSX_HIP_CHECK(hipMemcpyAsync(order, vals1, (size_t)N * 4, hipMemcpyDeviceToDevice, s));
         GSX_HIP_CHECK(hipMemcpyAsync(keys0, keys1, (size_t)N * 8, hipMemcpyDeviceToDevice, s));
     }
-    // the sorted keys stay in ordered_keys(workspace) for an emission that reads them
-    if ((rc = scan_counts(N, nullptr, keys0, rect_keys, cum_tiles_per_gauss, block_sums, total, s)) != GSX_OK)
+    // the sorted keys stay in ordered_keys(workspace) for an emission that reads them.  A caller that does not wait
+    // passes a pinned slot: the scan's last block writes the total there itself (no copy launch behind the scan).
+    int64_t* slot = wait ? nullptr : device_view_of_host_slot(n_isects_host);
+    if ((rc = scan_counts(N, nullptr, keys0, rect_keys, cum_tiles_per_gauss, block_sums, slot ? slot : total, s)) !=
+        GSX_OK)
         return rc;
-    GSX_HIP_CHECK(hipMemcpyAsync(n_isects_host, total, sizeof(int64_t), hipMemcpyDeviceToHost, s));
+    if (slot == nullptr)
+        GSX_HIP_CHECK(hipMemcpyAsync(n_isects_host, total, sizeof(int64_t), hipMemcpyDeviceToHost, s));
     if (wait) {
         GSX_HIP_CHECK(hipStreamSynchronize(s));
         GSX_REQUIRE(*n_isects_host < (1ll << 31), GSX_ERR_OVERFLOW, "%s: %lld intersections do not fit int32 indices",

@@ -138,7 +138,7 @@ class TrainStep:
         self.offsets = e(1, self.th, self.tw, dt=torch.int32)
         self.tile_order = e(self.th * self.tw, dt=torch.int32)  # the rasterizers' tile visiting order
         self.tile_walk = e(self.th * self.tw, dt=torch.int32)   # per tile: entries up to its last contributor
-        self.have_walk = False
+        self.have_walk, self._walk_cam = False, None
         self.render = e(1, H, W, 3)
         self.alpha = e(1, H, W, 1)
         self.last_ids = e(1, H, W, dt=torch.int32)
@@ -280,7 +280,9 @@ class TrainStep:
         # uses the order of the previous step (the first one: by list length), the backward pass this step's.
         order = c_p(None)
         if self.order_tiles:
-            if not self.have_walk:
+            # the previous pass's costs say something about this one only for the same camera (the same tensors)
+            cam_key = (viewmat.data_ptr(), K.data_ptr(), W, H)
+            if not self.have_walk or cam_key != self._walk_cam:
                 self._run("tile_order", lb.gsx_tile_order, c_i64(n), _p(self.offsets), c_p(None), c_u32(self.tw),
                           c_u32(self.th), _p(self.tile_order), s)
             order = _p(self.tile_order)
@@ -303,7 +305,7 @@ class TrainStep:
                     self._run("tile_order", lb.gsx_tile_order, *order_args, self._stream())
                     self.ev_order_join.record(self.side)
                 self.order_pending = True
-            self.have_walk = True
+            self.have_walk, self._walk_cam = True, (viewmat.data_ptr(), K.data_ptr(), W, H)
         return self.render
 
     @property
