@@ -51,7 +51,16 @@ int tile_order_from_pixels(int64_t n_isects, uint32_t image_width, uint32_t imag
                            const uint32_t** tile_order, void* stream);
 int ordered_counts_from_keys(const char* who, uint32_t N, int32_t* order, int64_t* cum_tiles_per_gauss, void* workspace,
                              size_t workspace_bytes, int64_t* n_isects_host, int wait, void* stream,
-                             bool rect_keys = false);
+                             bool rect_keys = false, bool first_hist_done = false);
+// radix_sort.hip: the table of the first 8-bit pass of a 32-bit sort, for a key-writing kernel that fills it itself
+struct RadixFirstPass {
+    uint32_t items, nblocks; // sort block b covers keys [b * 256 * items, (b + 1) * 256 * items)
+    uint32_t* table;         // [256][nblocks], digit-major
+};
+RadixFirstPass radix_first_pass_table(int64_t n, void* sort_workspace);
+int radix_sort_pairs_32_bits(int64_t n, int64_t* keys0, int32_t* vals0, int64_t* keys1, int32_t* vals1,
+                             uint32_t begin_bit, void* workspace, size_t workspace_bytes, int* selector_host,
+                             void* stream, bool first_hist_done);
 
 int check_camera_args(uint32_t C, const float* viewmats1, int camera_model, int rs_type, const float* radial,
                       const float* tangential, const float* thin_prism);

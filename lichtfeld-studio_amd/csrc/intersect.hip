@@ -51,26 +51,39 @@ __device__ __forceinline__ uint32_t packed_rect_count(uint32_t hi) {
     return (((hi >> 24) & 255u) - ((hi >> 8) & 255u)) * (((hi >> 16) & 255u) - (hi & 255u));
 }
 
+// A workgroup writes the keys of one block of the sort that follows (256 * items consecutive Gaussians) and leaves
+// that block's column of the sort's first histogram table (digit = low byte of the depth bits): the sort starts
+// with its scan.
 template <bool RECT>
 __global__ void __launch_bounds__(256) depth_count_keys_kernel(uint32_t n, const float* __restrict__ means2d,
                                                                 const int32_t* __restrict__ radii,
                                                                 const float* __restrict__ depths, float tile_size,
                                                                 uint32_t tile_width, uint32_t tile_height,
+                                                                uint32_t items, uint32_t nblocks,
                                                                 int32_t* __restrict__ tiles_per_gauss,
                                                                 int64_t* __restrict__ keys,
-                                                                int32_t* __restrict__ vals) {
-    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
-    if (i >= n)
-        return;
-    TileRect r;
-    uint32_t cnt = 0;
-    if (tile_rect(means2d, radii, i, tile_size, tile_width, tile_height, &r))
-        cnt = (r.y1 - r.y0) * (r.x1 - r.x0);
-    tiles_per_gauss[i] = (int32_t)cnt;
-    const uint32_t lo = cnt ? f2u(depths[i]) : 0xFFFFFFFFu;
-    const uint32_t hi = !RECT ? cnt : cnt ? (r.x0 | (r.y0 << 8) | (r.x1 << 16) | (r.y1 << 24)) : 0u;
-    keys[i] = (int64_t)(((uint64_t)hi << 32) | lo);
-    vals[i] = (int32_t)i;
+                                                                int32_t* __restrict__ vals,
+                                                                uint32_t* __restrict__ hist /*[256][nblocks]*/) {
+    __shared__ uint32_t lh[256];
+    lh[threadIdx.x] = 0;
+    __syncthreads();
+    for (uint32_t k = 0; k < items; ++k) {
+        const uint32_t i = (blockIdx.x * items + k) * 256u + threadIdx.x;
+        if (i >= n)
+            break;
+        TileRect r;
+        uint32_t cnt = 0;
+        if (tile_rect(means2d, radii, i, tile_size, tile_width, tile_height, &r))
+            cnt = (r.y1 - r.y0) * (r.x1 - r.x0);
+        tiles_per_gauss[i] = (int32_t)cnt;
+        const uint32_t lo = cnt ? f2u(depths[i]) : 0xFFFFFFFFu;
+        const uint32_t hi = !RECT ? cnt : cnt ? (r.x0 | (r.y0 << 8) | (r.x1 << 16) | (r.y1 << 24)) : 0u;
+        keys[i] = (int64_t)(((uint64_t)hi << 32) | lo);
+        vals[i] = (int32_t)i;
+        atomicAdd(&lh[lo & 255u], 1u);
+    }
+    __syncthreads();
+    hist[threadIdx.x * nblocks + blockIdx.x] = lh[threadIdx.x];
 }
 
 // ---- inclusive scan int32 -> int64 (at::cumsum of Intersect.cpp:75) -----------------------------
@@ -557,7 +570,8 @@ int64_t* ordered_keys(void* workspace) { return (int64_t*)workspace; }
 // scan the counts in that order, start the copy of the total.  order must hold 0..N-1 on entry.  rect_keys: the
 // high words are packed tile rectangles (depth_count_keys_kernel<true>) instead of counts.
 int ordered_counts_from_keys(const char* who, uint32_t N, int32_t* order, int64_t* cum_tiles_per_gauss, void* workspace,
-                             size_t workspace_bytes, int64_t* n_isects_host, int wait, void* stream, bool rect_keys) {
+                             size_t workspace_bytes, int64_t* n_isects_host, int wait, void* stream, bool rect_keys,
+                             bool first_hist_done) {
     const OrderedLayout L = ordered_layout(N);
     GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 && workspace_bytes >= L.total,
                 GSX_ERR_WORKSPACE, "%s: workspace needs %zu bytes, 256-byte aligned", who, L.total);
@@ -569,8 +583,9 @@ int ordered_counts_from_keys(const char* who, uint32_t N, int32_t* order, int64_
     int64_t* total = block_sums + cdiv(N, kScanTile);
     hipStream_t s = (hipStream_t)stream;
     int rc, sel = 0;
-    if ((rc = gsx_radix_sort_pairs(N, keys0, order, keys1, vals1, 0, 32, ws + L.sort_off,
-                                   gsx_radix_sort_pairs_workspace_bytes(N), &sel, stream)) != GSX_OK)
+    if ((rc = radix_sort_pairs_32_bits(N, keys0, order, keys1, vals1, 0, ws + L.sort_off,
+                                       gsx_radix_sort_pairs_workspace_bytes(N), &sel, stream, first_hist_done)) !=
+        GSX_OK)
         return rc;
     if (sel) { // four 8-bit passes end in buffer 0; kept for a different digit width
         GSX_HIP_CHECK(hipMemcpyAsync(order, vals1, (size_t)N * 4, hipMemcpyDeviceToDevice, s));
@@ -616,17 +631,20 @@ extern "C" int gsx_intersect_tile_count_ordered(uint32_t N, const float* means2d
                 GSX_ERR_WORKSPACE, "intersect_tile_count_ordered: workspace needs %zu bytes, 256-byte aligned",
                 ordered_layout(N).total);
     const bool rect_keys = rect_keys_fit(tile_width, tile_height);
+    // the key kernel's workgroups are the sort's blocks: each leaves its column of the first pass's histogram
+    const gsx::RadixFirstPass fp =
+        gsx::radix_first_pass_table(N, (char*)workspace + ordered_layout(N).sort_off);
     if (rect_keys)
-        hipLaunchKernelGGL(depth_count_keys_kernel<true>, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N,
-                           means2d, radii, depths, (float)tile_size, tile_width, tile_height, tiles_per_gauss,
-                           gsx::ordered_keys(workspace), order);
+        hipLaunchKernelGGL(depth_count_keys_kernel<true>, dim3(fp.nblocks), dim3(256), 0, (hipStream_t)stream, N,
+                           means2d, radii, depths, (float)tile_size, tile_width, tile_height, fp.items, fp.nblocks,
+                           tiles_per_gauss, gsx::ordered_keys(workspace), order, fp.table);
     else
-        hipLaunchKernelGGL(depth_count_keys_kernel<false>, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N,
-                           means2d, radii, depths, (float)tile_size, tile_width, tile_height, tiles_per_gauss,
-                           gsx::ordered_keys(workspace), order);
+        hipLaunchKernelGGL(depth_count_keys_kernel<false>, dim3(fp.nblocks), dim3(256), 0, (hipStream_t)stream, N,
+                           means2d, radii, depths, (float)tile_size, tile_width, tile_height, fp.items, fp.nblocks,
+                           tiles_per_gauss, gsx::ordered_keys(workspace), order, fp.table);
     GSX_LAUNCH_CHECK();
     return gsx::ordered_counts_from_keys("intersect_tile_count_ordered", N, order, cum_tiles_per_gauss, workspace,
-                                         workspace_bytes, n_isects_host, wait, stream, rect_keys);
+                                         workspace_bytes, n_isects_host, wait, stream, rect_keys, true);
 }
 
 extern "C" int gsx_intersect_tile_emit(uint32_t C, uint32_t N, const float* means2d, const int32_t* radii,

@@ -250,10 +250,12 @@ extern "C" int gsx_radix_sort_pairs_selector(int64_t n, uint32_t begin_bit, uint
 }
 
 namespace {
+// first_hist_done: the caller's own kernel has already left the first pass's histogram table in the workspace
+// (gsx::radix_first_pass_table)
 template <typename KeyT>
 int sort_pairs(const char* what, int64_t n, KeyT* keys0, int32_t* vals0, KeyT* keys1, int32_t* vals1,
                uint32_t begin_bit, uint32_t end_bit, void* workspace, size_t workspace_bytes, int* selector_host,
-               void* stream) {
+               void* stream, bool first_hist_done = false) {
     if (selector_host)
         *selector_host = 0;
     if (n <= 0)
@@ -284,9 +286,11 @@ int sort_pairs(const char* what, int64_t n, KeyT* keys0, int32_t* vals0, KeyT* k
         const int32_t* vin = sel ? vals1 : vals0;
         KeyT* kout = sel ? keys0 : keys1;
         int32_t* vout = sel ? vals0 : vals1;
-        hipLaunchKernelGGL(radix_hist_kernel<KeyT>, dim3(L.nblocks), dim3(256), 0, s, (uint32_t)n, kin, items, shift,
-                           mask, L.nblocks, hist);
-        GSX_LAUNCH_CHECK();
+        if (!(first_hist_done && pass == 0)) {
+            hipLaunchKernelGGL(radix_hist_kernel<KeyT>, dim3(L.nblocks), dim3(256), 0, s, (uint32_t)n, kin, items,
+                               shift, mask, L.nblocks, hist);
+            GSX_LAUNCH_CHECK();
+        }
         hipLaunchKernelGGL(radix_scan_kernel, dim3(kRadix), dim3(256), 0, s, L.nblocks, hist, totals);
         GSX_LAUNCH_CHECK();
         if (items == kItemsSmall)
@@ -304,6 +308,26 @@ int sort_pairs(const char* what, int64_t n, KeyT* keys0, int32_t* vals0, KeyT* k
     return GSX_OK;
 }
 } // namespace
+
+namespace gsx {
+// Where a kernel that writes the keys of a sort on bits [begin_bit, begin_bit + 32) can leave the first pass's
+// histogram itself: sort block b covers keys [b * 256 * items, (b + 1) * 256 * items) and table[d * nblocks + b]
+// counts its keys whose bits [begin_bit, begin_bit + 8) equal d.
+RadixFirstPass radix_first_pass_table(int64_t n, void* workspace) {
+    const SortLayout L = sort_layout(n);
+    RadixFirstPass f;
+    f.items = sort_items(n);
+    f.nblocks = L.nblocks;
+    f.table = (uint32_t*)((char*)workspace + L.hist_off);
+    return f;
+}
+int radix_sort_pairs_32_bits(int64_t n, int64_t* keys0, int32_t* vals0, int64_t* keys1, int32_t* vals1,
+                             uint32_t begin_bit, void* workspace, size_t workspace_bytes, int* selector_host,
+                             void* stream, bool first_hist_done) {
+    return sort_pairs<int64_t>("radix_sort_pairs", n, keys0, vals0, keys1, vals1, begin_bit, begin_bit + 32, workspace,
+                               workspace_bytes, selector_host, stream, first_hist_done);
+}
+} // namespace gsx
 
 extern "C" int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, int64_t* keys1, int32_t* vals1,
                                     uint32_t begin_bit, uint32_t end_bit, void* workspace, size_t workspace_bytes,
