@@ -6,8 +6,8 @@
 // digit-major table into running counts and leaves the digit's total -> stable scatter (every block adds the
 // exclusive scan of the 256 totals itself; no atomics between blocks, nothing to zero).  A
 // block owns a tile of 256 x ITEMS consecutive pairs; inside the block each 64-lane wave owns a quarter of them
-// and ranks them 64 at a time with wave-wide match masks built from ballots, so the order (wave, round, lane)
-// equals the input order and the sort is stable.  The ranked pairs are first placed in LDS in digit order and then
+// and ranks them 64 at a time with wave-wide match masks (one 64-bit mask per digit in LDS, set by atomic OR), so
+// the order (wave, round, lane) equals the input order and the sort is stable.  The ranked pairs are first placed in LDS in digit order and then
 // written out by consecutive lanes, so that every (tile, digit) run leaves the block as whole cache lines.
 #include "gsx_common.h"
 
@@ -118,13 +118,19 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const Ke
     __shared__ uint32_t wave_count[4][kRadix];
     __shared__ uint32_t to_global[kRadix]; // global position of a pair = to_global[digit] + its slot in the tile
     __shared__ uint32_t wsum[4], gsum[4];
-    __shared__ KeyT s_keys[kTileN];
-    __shared__ int32_t s_vals[kTileN];
+    // the match masks of the ranking phase and the reordered tile of the output phase share their bytes
+    constexpr uint32_t kMatchBytes = 4 * kRadix * 8, kTileBytes = kTileN * (sizeof(KeyT) + 4);
+    __shared__ __align__(16) unsigned char overlay[kMatchBytes > kTileBytes ? kMatchBytes : kTileBytes];
+    unsigned long long(*match)[kRadix] = reinterpret_cast<unsigned long long(*)[kRadix]>(overlay);
+    int32_t* s_vals = reinterpret_cast<int32_t*>(overlay);
+    KeyT* s_keys = reinterpret_cast<KeyT*>(overlay + kTileN * 4);
     const uint32_t t = threadIdx.x;
     const uint32_t w = t >> 6, lane = t & 63u;
 #pragma unroll
-    for (uint32_t i = 0; i < 4; ++i)
+    for (uint32_t i = 0; i < 4; ++i) {
         wave_count[i][t] = 0;
+        match[i][t] = 0ull;
+    }
     __syncthreads();
 
     const uint32_t tile_base = blockIdx.x * kTileN;
@@ -145,12 +151,23 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const Ke
         const uint32_t idx = wave_base + r * 64u + lane;
         const bool valid = idx < n;
         const uint32_t d = digit_of(key[r], shift, mask);
-        uint64_t peers = __ballot(valid);
-#pragma unroll
-        for (uint32_t b = 0; b < kRadixBits; ++b) {
-            const bool bit = (d >> b) & 1u;
-            const uint64_t m = __ballot(bit);
-            peers &= bit ? m : ~m;
+        // peers: the wave's lanes whose pair has this lane's digit.  Every lane sets its bit in the digit's mask in
+        // LDS and reads the mask back (LDS serves one wave's instructions in order); the lowest peer clears it for
+        // the next round.  A wave whose pairs all share one digit (sorted or constant input) skips the LDS trip.
+        const uint64_t valid_lanes = __ballot(valid);
+        uint64_t peers = valid_lanes;
+        if (valid_lanes) {
+            const uint32_t d_first = (uint32_t)__builtin_amdgcn_readlane((int)d, __builtin_ctzll(valid_lanes));
+            if (__ballot(valid && d != d_first)) {
+                if (valid)
+                    atomicOr(&match[w][d], 1ull << lane);
+                __builtin_amdgcn_wave_barrier();
+                peers = valid ? match[w][d] : 0ull;
+                __builtin_amdgcn_wave_barrier();
+                if (valid && (peers & lt_mask) == 0)
+                    match[w][d] = 0ull;
+                __builtin_amdgcn_wave_barrier();
+            }
         }
         uint32_t pre = 0;
         if (valid)
