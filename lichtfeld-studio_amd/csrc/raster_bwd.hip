@@ -22,11 +22,6 @@
 
 namespace gsx {
 
-// a x b with one rounding per component
-__device__ __forceinline__ vec3 cross_fma(vec3 a, vec3 b) {
-    return mk3(fma(a.y, b.z, -(a.z * b.y)), fma(a.z, b.x, -(a.x * b.z)), fma(a.x, b.y, -(a.y * b.x)));
-}
-
 static constexpr uint32_t kAcc = 16; // floats accumulated per Gaussian: rgb 3, v_gro 3, v_grd(x)ray_d 9, opacity 1
 
 __global__ void __launch_bounds__(256) fill_f32_kernel(size_t n, float v, float* __restrict__ out) {
@@ -111,14 +106,12 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
 
     const float T_final = 1.0f - render_alphas[pix_id];
     float T = T_final;
-    float buffer[CDIM];
+    float bdot = 0.f; // sum_k buffer_k v_render_k (:186, :309; see the loop)
     const int32_t bin_final = inside ? last_ids[pix_id] : 0;
     float v_render_c[CDIM];
 #pragma unroll
-    for (uint32_t k = 0; k < CDIM; ++k) {
-        buffer[k] = 0.f;
+    for (uint32_t k = 0; k < CDIM; ++k)
         v_render_c[k] = v_render_colors[(size_t)pix_id * CDIM + k];
-    }
     const float v_render_a = v_render_alphas[pix_id];
     float bg_dot = 0.f;
     if (backgrounds != nullptr) {
@@ -126,6 +119,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
         for (uint32_t k = 0; k < CDIM; ++k)
             bg_dot += backgrounds[k] * v_render_c[k];
     }
+    const float v_alpha_bg = v_render_a - bg_dot; // what T_final ra multiplies in v_alpha (:313-321)
 
     // last contributing list entry over the wave (:201-203) and over the workgroup: entries behind the
     // workgroup's maximum are needed by no pixel, so the walk starts there
@@ -212,28 +206,28 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             v[0] = fac * v_render_c[0];
             v[1] = NC > 1 ? fac * v_render_c[NC > 1 ? 1 : 0] : 0.f;
             v[2] = NC > 2 ? fac * v_render_c[NC > 2 ? 2 : 0] : 0.f;
-            // the derivative chain is written with fused multiply-adds (one rounding instead of two per term; the
-            // compiler does not contract on its own here): fewer instructions in the loop that bounds the step
-            float v_alpha = 0.f;
+            // The derivative chain is written with fused multiply-adds (the compiler does not contract on its own
+            // here) and with the colour sums folded: sum_k (c_k T - buffer_k ra) v_render_k (:306-311) is
+            // T cdot - ra bdot with cdot = sum_k c_k v_render_k and bdot = sum_k buffer_k v_render_k, and since
+            // buffer_k grows by c_k fac per Gaussian (:343), bdot grows by cdot fac: one running scalar per pixel instead of
+            // one per channel.  Fewer instructions in the loop that bounds the step; same value up to rounding.
+            float cdot = col[0] * v_render_c[0];
 #pragma unroll
-            for (uint32_t k = 0; k < CDIM; ++k)
-                v_alpha = fma(fma(col[k], T, -(buffer[k] * ra)), v_render_c[k], v_alpha);
-            const float tfr = T_final * ra;
-            v_alpha = fma(tfr, v_render_a, v_alpha);
-            if (backgrounds != nullptr)
-                v_alpha = fma(-tfr, bg_dot, v_alpha);
+            for (uint32_t k = 1; k < CDIM; ++k)
+                cdot = fma(col[k], v_render_c[k], cdot);
+            float v_alpha = fma(T, cdot, -(ra * bdot));
+            v_alpha = fma(T_final * ra, v_alpha_bg, v_alpha); // + T_final ra (v_render_a - bg . v_render)
             // the clamp at 0.999 has zero derivative (:322)
             v_alpha = (valid && a.w * vis <= 0.999f) ? v_alpha : 0.f;
             const float v_vis = a.w * v_alpha;
-            const float v_gradDist = -0.5f * vis * v_vis;
-            const vec3 v_gcrod = scale(gcrod, 2.0f * v_gradDist);
-            const vec3 v_grd_n = cross_fma(gro, v_gcrod); // = -(v_gcrod x gro)
-            const vec3 v_gro = cross_fma(v_gcrod, grd_n);
-            // VJP of safe_normalize (Utils.cuh:186-194) with the reciprocal length from above
-            const float il3 = il * il * il;
-            const float sdot = il3 * fma(v_grd_n.z, grd.z, fma(v_grd_n.y, grd.y, v_grd_n.x * grd.x));
-            const vec3 v_grd = mk3(fma(il, v_grd_n.x, -(sdot * grd.x)), fma(il, v_grd_n.y, -(sdot * grd.y)),
-                                   fma(il, v_grd_n.z, -(sdot * grd.z)));
+            const vec3 v_gcrod = scale(gcrod, -(vis * v_vis)); // 2 v_gradDist, v_gradDist = -0.5 vis v_vis
+            const vec3 v_grd_n = cross(gro, v_gcrod);          // = -(v_gcrod x gro)
+            const vec3 v_gro = cross(v_gcrod, grd_n);
+            // VJP of safe_normalize (Utils.cuh:186-194) with the reciprocal length from above:
+            // (v - (v . n) n) / |grd| with n = grd / |grd|
+            const float along = dot(v_grd_n, grd_n);
+            const vec3 v_grd = mk3(il * fma(-along, grd_n.x, v_grd_n.x), il * fma(-along, grd_n.y, v_grd_n.y),
+                                   il * fma(-along, grd_n.z, v_grd_n.z));
             v[3] = v_gro.x;
             v[4] = v_gro.y;
             v[5] = v_gro.z;
@@ -254,9 +248,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
                 v[12] = fma(v_gro.z, o_shift.x, v[12]), v[13] = fma(v_gro.z, o_shift.y, v[13]);
                 v[14] = fma(v_gro.z, o_shift.z, v[14]);
             }
-#pragma unroll
-            for (uint32_t k = 0; k < CDIM; ++k)
-                buffer[k] = fma(col[k], fac, buffer[k]);
+            bdot = fma(cdot, fac, bdot);
             if (CDIM > 3) { // the fourth channel's gradient: its own wave sum
                 float e = fac * v_render_c[CDIM > 3 ? 3 : 0];
 #pragma unroll
