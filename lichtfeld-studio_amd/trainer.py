@@ -75,8 +75,8 @@ class TrainStep:
         self.side = torch.cuda.Stream(self.dev) if overlap else None
         self.ev_fork, self.ev_join = torch.cuda.Event(), torch.cuda.Event()
         self.ev_loss_fork, self.ev_loss_join = torch.cuda.Event(), torch.cuda.Event()
-        self.ev_order_fork, self.ev_order_join = torch.cuda.Event(), torch.cuda.Event()
-        self.order_pending = False
+        self.ev_order_join = torch.cuda.Event()
+        self.order_pending, self._order_due = False, None
         self.loss_out = torch.empty(3, dtype=torch.float32, device=self.dev)
 
     def _allocate_per_gaussian(self, N):
@@ -159,9 +159,20 @@ class TrainStep:
         self.img_shape = (H, W)
 
     def _join_tile_order(self):
-        if self.order_pending:  # the tile order was formed on the second stream
+        """The tile order from the last forward pass's costs is in place for what the current stream runs next."""
+        if self._order_due is not None:  # nobody has queued it yet
+            self._run("tile_order", self.lib.gsx_tile_order, *self._order_due, self._stream())
+            self._order_due = None
+        if self.order_pending:  # it was formed on the second stream
             torch.cuda.current_stream(self.dev).wait_event(self.ev_order_join)
             self.order_pending = False
+
+    def _order_on_side_stream(self):
+        """Called with the second stream current and already waiting for the forward pass."""
+        if self._order_due is not None:
+            self._run("tile_order", self.lib.gsx_tile_order, *self._order_due, self._stream())
+            self.ev_order_join.record(self.side)
+            self._order_due, self.order_pending = None, True
 
     def _stream(self):
         return c_p(torch.cuda.current_stream(self.dev).cuda_stream)
@@ -294,17 +305,10 @@ class TrainStep:
                   _p(K), _p(self.offsets), _p(self.flatten_ids), order, _p(self.tile_walk) if self.order_tiles else
                   c_p(None), _p(self.render), _p(self.alpha), _p(self.last_ids), s)
         if self.order_tiles:
-            order_args = (c_i64(n), c_p(None), _p(self.tile_walk), c_u32(self.tw), c_u32(self.th),
-                          _p(self.tile_order))
-            if self.side is None:
-                self._run("tile_order", lb.gsx_tile_order, *order_args, s)
-            else:  # beside the loss kernels: the backward pass, its first reader, waits for it
-                self.ev_order_fork.record(torch.cuda.current_stream(self.dev))
-                self.side.wait_event(self.ev_order_fork)
-                with torch.cuda.stream(self.side):
-                    self._run("tile_order", lb.gsx_tile_order, *order_args, self._stream())
-                    self.ev_order_join.record(self.side)
-                self.order_pending = True
+            # the order for the backward pass (and for the next forward pass from this camera): queued by the loss
+            # pass on the second stream, or by whoever needs it first
+            self._order_due = (c_i64(n), c_p(None), _p(self.tile_walk), c_u32(self.tw), c_u32(self.th),
+                               _p(self.tile_order))
             self.have_walk, self._walk_cam = True, (viewmat.data_ptr(), K.data_ptr(), W, H)
         return self.render
 
@@ -336,6 +340,7 @@ class TrainStep:
                 self.ev_loss_fork.record(torch.cuda.current_stream(self.dev))
                 self.side.wait_event(self.ev_loss_fork)
                 with torch.cuda.stream(self.side):
+                    self._order_on_side_stream()  # the backward pass waits for this one, not for the reduction
                     self._run("photometric_loss_finish", lb.gsx_photometric_loss_finish, *fin, self._stream())
                     self.ev_loss_join.record(self.side)
                 self.loss_pending = True
