@@ -538,7 +538,7 @@ __global__ void __launch_bounds__(256) fgs_blend_bwd_kernel(
     range_end = min(range_end, range_start + block_max);
     if (range_end <= range_start)
         return;
-    float T = T_final, a0 = 0.f, a1 = 0.f, a2 = 0.f; // colour behind the current Gaussian
+    float T = T_final, adot = 0.f; // adot: colour behind the current Gaussian, dotted with the pixel's colour gradient
     const uint32_t num_batches = (uint32_t)(range_end - range_start + (int32_t)kBatch - 1) / kBatch;
     for (uint32_t b = 0; b < num_batches; ++b) {
         const int32_t batch_end = range_end - 1 - (int32_t)(kBatch * b); // slot 0: the farthest entry
@@ -571,11 +571,11 @@ __global__ void __launch_bounds__(256) fgs_blend_bwd_kernel(
             const float w = valid ? T * alpha : 0.f;
             const float col0 = q1.z > 0.0f ? q1.z : 0.0f, col1 = q1.w > 0.0f ? q1.w : 0.0f,
                         col2 = q2.x > 0.0f ? q2.x : 0.0f;
-            float dL_dalpha = ga_common * ra;
-            dL_dalpha += (T * col0 - a0 * ra) * g0;
-            dL_dalpha += (T * col1 - a1 * ra) * g1;
-            dL_dalpha += (T * col2 - a2 * ra) * g2;
-            a0 += w * col0, a1 += w * col1, a2 += w * col2;
+            // sum_k (T c_k - a_k ra) g_k with the colour sums folded: cdot = sum_k c_k g_k, and since a_k grows by
+            // w c_k per Gaussian, adot = sum_k a_k g_k grows by w cdot (one running scalar instead of three)
+            const float cdot = fma(col2, g2, fma(col1, g1, col0 * g0));
+            const float dL_dalpha = fma(T, cdot, ra * (ga_common - adot));
+            adot = fma(w, cdot, adot);
             const float ad = valid ? alpha * dL_dalpha : 0.f;
             const float helper = -ad;
             float v[16];
