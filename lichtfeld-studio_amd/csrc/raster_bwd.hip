@@ -106,7 +106,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
 
     const float T_final = 1.0f - render_alphas[pix_id];
     float T = T_final;
-    float bdot = 0.f; // sum_k buffer_k v_render_k (:186, :309; see the loop)
+
     const int32_t bin_final = inside ? last_ids[pix_id] : 0;
     float v_render_c[CDIM];
 #pragma unroll
@@ -119,7 +119,9 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
         for (uint32_t k = 0; k < CDIM; ++k)
             bg_dot += backgrounds[k] * v_render_c[k];
     }
-    const float v_alpha_bg = v_render_a - bg_dot; // what T_final ra multiplies in v_alpha (:313-321)
+    // what ra multiplies in v_alpha: T_final (v_render_a - bg . v_render) (:313-321) minus sum_k buffer_k v_render_k
+    // (:186, :309), which starts at zero and is updated in the loop
+    float behind = T_final * (v_render_a - bg_dot);
 
     // last contributing list entry over the wave (:201-203) and over the workgroup: entries behind the
     // workgroup's maximum are needed by no pixel, so the walk starts there
@@ -207,21 +209,26 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             v[1] = NC > 1 ? fac * v_render_c[NC > 1 ? 1 : 0] : 0.f;
             v[2] = NC > 2 ? fac * v_render_c[NC > 2 ? 2 : 0] : 0.f;
             // The derivative chain is written with fused multiply-adds (the compiler does not contract on its own
-            // here) and with the colour sums folded: sum_k (c_k T - buffer_k ra) v_render_k (:306-311) is
-            // T cdot - ra bdot with cdot = sum_k c_k v_render_k and bdot = sum_k buffer_k v_render_k, and since
-            // buffer_k grows by c_k fac per Gaussian (:343), bdot grows by cdot fac: one running scalar per pixel instead of
-            // one per channel.  Fewer instructions in the loop that bounds the step; same value up to rounding.
+            // here) and folded algebraically; same values as the reference's chain up to rounding, fewer instructions
+            // in the loop that bounds the step.
+            // Colours: sum_k (c_k T - buffer_k ra) v_render_k (:306-311) = T cdot - ra bdot with cdot = sum_k c_k
+            // v_render_k and bdot = sum_k buffer_k v_render_k; buffer_k grows by c_k fac per Gaussian (:343), so bdot
+            // grows by cdot fac.  `behind` = T_final (v_render_a - bg . v_render) - bdot collects everything ra
+            // multiplies (:313-321): one running scalar per pixel instead of one per channel.
             float cdot = col[0] * v_render_c[0];
 #pragma unroll
             for (uint32_t k = 1; k < CDIM; ++k)
                 cdot = fma(col[k], v_render_c[k], cdot);
-            float v_alpha = fma(T, cdot, -(ra * bdot));
-            v_alpha = fma(T_final * ra, v_alpha_bg, v_alpha); // + T_final ra (v_render_a - bg . v_render)
+            float v_alpha = fma(T, cdot, ra * behind);
             // the clamp at 0.999 has zero derivative (:322)
             v_alpha = (valid && a.w * vis <= 0.999f) ? v_alpha : 0.f;
-            const float v_vis = a.w * v_alpha;
-            const vec3 v_gcrod = scale(gcrod, -(vis * v_vis)); // 2 v_gradDist, v_gradDist = -0.5 vis v_vis
-            const vec3 v_grd_n = cross(gro, v_gcrod);          // = -(v_gcrod x gro)
+            const float v_opac = vis * v_alpha;
+            // Geometry (:325-336), in the reference's order of operations: v_gro and v_grd are sums over the footprint
+            // that nearly cancel, and their fp32 rounding pattern is part of what the result is compared with (the
+            // closed form v_gro = s q, v_grd = -s (g . n) q / |grd| with q = g - (g . n) n, eight instructions
+            // shorter, differs from it by up to 6 % of the tolerance floor at rare ill-conditioned Gaussians).
+            const vec3 v_gcrod = scale(gcrod, -(a.w * v_opac)); // 2 v_gradDist, v_gradDist = -0.5 vis opac v_alpha
+            const vec3 v_grd_n = cross(gro, v_gcrod);           // = -(v_gcrod x gro)
             const vec3 v_gro = cross(v_gcrod, grd_n);
             // VJP of safe_normalize (Utils.cuh:186-194) with the reciprocal length from above:
             // (v - (v . n) n) / |grd| with n = grd / |grd|
@@ -240,7 +247,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             v[12] = v_grd.z * ray_d.x;
             v[13] = v_grd.z * ray_d.y;
             v[14] = v_grd.z * ray_d.z;
-            v[15] = vis * v_alpha;
+            v[15] = v_opac;
             if (rolling) {
                 v[6] = fma(v_gro.x, o_shift.x, v[6]), v[7] = fma(v_gro.x, o_shift.y, v[7]);
                 v[8] = fma(v_gro.x, o_shift.z, v[8]), v[9] = fma(v_gro.y, o_shift.x, v[9]);
@@ -248,7 +255,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
                 v[12] = fma(v_gro.z, o_shift.x, v[12]), v[13] = fma(v_gro.z, o_shift.y, v[13]);
                 v[14] = fma(v_gro.z, o_shift.z, v[14]);
             }
-            bdot = fma(cdot, fac, bdot);
+            behind = fma(-cdot, fac, behind);
             if (CDIM > 3) { // the fourth channel's gradient: its own wave sum
                 float e = fac * v_render_c[CDIM > 3 ? 3 : 0];
 #pragma unroll
