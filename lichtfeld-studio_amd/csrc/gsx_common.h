@@ -300,6 +300,18 @@ __device__ __forceinline__ TilePixel tile_pixel(uint32_t tile_id, uint32_t tile_
     return p;
 }
 
+// 16-byte accesses with the non-temporal hint, for arrays a kernel streams through once (measured on a seven-stream
+// Adam-like kernel over 1.8 GB: 5.75 instead of 5.32 TB/s when both the loads and the stores carry it)
+typedef float gsx_float4_nt __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 load_streaming(const float4* p) {
+    const gsx_float4_nt v = __builtin_nontemporal_load(reinterpret_cast<const gsx_float4_nt*>(p));
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void store_streaming(float4* p, float4 v) {
+    const gsx_float4_nt t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, reinterpret_cast<gsx_float4_nt*>(p));
+}
+
 // The record of one Gaussian as the rasterizers read it (gsx_record.h)
 __device__ __forceinline__ void store_record(float4* __restrict__ r, vec3 gro, float opac, const mat3& M, float c0,
                                              float c1, float c2, const RecordRegion& g) {

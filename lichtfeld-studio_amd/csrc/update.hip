@@ -156,10 +156,10 @@ __global__ void __launch_bounds__(256) backward_update_kernel(const UpdateArgs a
                 const uint32_t col = q - ((q * 43691u) >> 19) * kShRowF4;
                 // with the higher bands frozen only the first float4 of a row (DC + one more element) is touched
                 act[i] = base + q < n_f4 && !(skip && col != 0);
-                if (act[i]) {
-                    p4[i] = P4[q];
-                    m4[i] = M4[q];
-                    v4[i] = V4[q];
+                if (act[i]) { // read once, written once: streamed past the caches
+                    p4[i] = load_streaming(P4 + q);
+                    m4[i] = load_streaming(M4 + q);
+                    v4[i] = load_streaming(V4 + q);
                 }
             }
 #pragma unroll
@@ -184,9 +184,9 @@ __global__ void __launch_bounds__(256) backward_update_kernel(const UpdateArgs a
                     mv[t] = m1;
                     vv[t] = v1;
                 }
-                P4[q] = p4[i];
-                M4[q] = m4[i];
-                V4[q] = v4[i];
+                store_streaming(P4 + q, p4[i]);
+                store_streaming(M4 + q, m4[i]);
+                store_streaming(V4 + q, v4[i]);
             }
             }
             __builtin_amdgcn_wave_barrier();
