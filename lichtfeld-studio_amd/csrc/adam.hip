@@ -48,10 +48,11 @@ __global__ void __launch_bounds__(256) adam_multi_kernel(const AdamTable tab) {
     const bool skip2 = tab.skip2[gi] != 0;
     const bool aligned = ((((uintptr_t)P) | ((uintptr_t)M) | ((uintptr_t)V) | ((uintptr_t)G)) & 15u) == 0;
     if (aligned && base + kAdamVec <= n) {
-        float4 p = *reinterpret_cast<float4*>(P + base);
-        float4 m = *reinterpret_cast<float4*>(M + base);
-        float4 v = *reinterpret_cast<float4*>(V + base);
-        const float4 g = *reinterpret_cast<const float4*>(G + base);
+        // every array is read once and written once per step: streamed past the caches
+        float4 p = load_streaming(reinterpret_cast<const float4*>(P + base));
+        float4 m = load_streaming(reinterpret_cast<const float4*>(M + base));
+        float4 v = load_streaming(reinterpret_cast<const float4*>(V + base));
+        const float4 g = load_streaming(reinterpret_cast<const float4*>(G + base));
         float lrs[4] = {lr, lr, lr, lr};
         bool upd[4] = {true, true, true, true};
         if (period) {
@@ -70,9 +71,9 @@ __global__ void __launch_bounds__(256) adam_multi_kernel(const AdamTable tab) {
             adam_one(p.z, m.z, v.z, g.z, lrs[2], b1, b2, eps, c1, c2);
         if (upd[3])
             adam_one(p.w, m.w, v.w, g.w, lrs[3], b1, b2, eps, c1, c2);
-        *reinterpret_cast<float4*>(P + base) = p;
-        *reinterpret_cast<float4*>(M + base) = m;
-        *reinterpret_cast<float4*>(V + base) = v;
+        store_streaming(reinterpret_cast<float4*>(P + base), p);
+        store_streaming(reinterpret_cast<float4*>(M + base), m);
+        store_streaming(reinterpret_cast<float4*>(V + base), v);
     } else {
         for (uint32_t i = base; i < n && i < base + kAdamVec; ++i) {
             const bool second = period && (i % period) >= split;

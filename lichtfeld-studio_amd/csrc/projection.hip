@@ -613,7 +613,7 @@ __device__ __forceinline__ void request_coefficient_rows(const float* __restrict
         const uint32_t r = (q * 43691u) >> 19; // q / 12 for q < 768
         tmp[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         if (q < n_f4 && ((live_rows >> r) & 1ull))
-            tmp[i] = src[q];
+            tmp[i] = load_streaming(src + q); // read once per pass
     }
 }
 __device__ __forceinline__ void turn_coefficient_rows(const float4* tmp, uint32_t lane, float4* wave_lds,
