@@ -26,7 +26,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 # HBM bytes per launch of the dominant kernel at the default workload, from two rocprofv3 --pmc runs (FETCH_SIZE,
-# WRITE_SIZE, each scaled by what the same counter reads for gsx_debug_copy's known 256 MiB + 256 MiB); the figures
+# WRITE_SIZE, each scaled by what the same counter reads for gsx_debug_copy's known 1 GiB + 1 GiB); the figures
 # and the commands are in profiles/train_step_1M_1237x822_hbm_traffic.txt.  Counters cannot be read from inside
 # this process, so the value is only attached when the workload is the one it was measured on.
 MEASURED_TRAFFIC_BYTES = {("rasterize_bwd_kernel", 3, 1_000_000): 246.1e6}
@@ -181,7 +181,7 @@ def main():
     stage_ms = {k: float(np.mean(v)) for k, v in ts.stop_timing().items()}
 
     # known-size copy: the yardstick for byte counters and the measured streaming bandwidth of this GPU
-    copy_bytes = 256 << 20
+    copy_bytes = 1 << 30  # well beyond the 256 MB last-level cache
     cp_src = torch.empty(copy_bytes, dtype=torch.uint8, device=dev)
     cp_dst = torch.empty(copy_bytes, dtype=torch.uint8, device=dev)
     cp_src.zero_()
@@ -247,7 +247,7 @@ def main():
         "raster_bwd_ms": round(dom_ms, 4),
         "roofline": roofline, "cpu_baseline": cpu_baseline,
         "copy_probe": {"bytes_moved": 2 * copy_bytes, "GBps": round(copy_gbs, 1),
-                       "note": "gsx_debug_copy, 256 MiB read + 256 MiB written: measured streaming bandwidth"},
+                       "note": "gsx_debug_copy, 1 GiB read + 1 GiB written: measured streaming bandwidth"},
         "kernels": kernels,
     }
     print(json.dumps(out))

@@ -57,11 +57,13 @@ __global__ void __launch_bounds__(256) math_unary_kernel(int which, uint32_t n, 
     y[i] = r;
 }
 
-// plain streaming copy of known size: the yardstick that HBM byte counters and achieved bandwidths are scaled by
+// streaming copy of known size: the yardstick that HBM byte counters and achieved bandwidths are scaled by.  One
+// 16-byte element per lane, loads and stores with the non-temporal hint: the fastest copy found on this GPU.
 __global__ void __launch_bounds__(256) copy_probe_kernel(const float4* __restrict__ src, float4* __restrict__ dst,
                                                           size_t n16) {
-    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256)
-        dst[i] = src[i];
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n16)
+        store_streaming(dst + i, load_streaming(src + i));
 }
 
 } // namespace gsx
@@ -73,8 +75,9 @@ extern "C" int gsx_debug_copy(const void* src, void* dst, size_t bytes, void* st
                 GSX_ERR_INVALID_ARGUMENT, "debug_copy: null / unaligned buffers or size %zu not a multiple of 16", bytes);
     const size_t n16 = bytes / 16;
     const size_t blocks = (n16 + 255) / 256;
-    hipLaunchKernelGGL(gsx::copy_probe_kernel, dim3((uint32_t)(blocks < 16384 ? blocks : 16384)), dim3(256), 0,
-                       (hipStream_t)stream, (const float4*)src, (float4*)dst, n16);
+    GSX_REQUIRE(blocks < (1ull << 31), GSX_ERR_INVALID_ARGUMENT, "debug_copy: %zu bytes in one call", bytes);
+    hipLaunchKernelGGL(gsx::copy_probe_kernel, dim3((uint32_t)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const float4*)src, (float4*)dst, n16);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }
