@@ -115,9 +115,11 @@ GSX_API int gsx_intersect_tile_count(uint32_t C, uint32_t N, const float* means2
  * (gsx_radix_sort_pairs with begin_bit = 32): the sort is stable, the result is the same array bit for bit, and
  * four of its six passes run over N Gaussians instead of n_isects pairs.
  * wait != 0: returns with *n_isects_host valid (and checked against the int32 index space), like the call above.
- * wait == 0: nothing blocks; n_isects_host must be PINNED host memory.  It reads -1 from the return of this call
- * until the total has arrived (0 at once when N == 0): the caller synchronises with the stream or simply watches
- * the slot, checks the value is below 2^31, and may queue work that does not need the count in between. */
+ * wait == 0: nothing blocks; n_isects_host must be PINNED host memory (the scan's last workgroup stores the total
+ * into it directly; memory the runtime does not know as pinned gets an asynchronous copy instead).  It reads -1
+ * from the return of this call until the total has arrived (0 at once when N == 0): the caller synchronises with
+ * the stream or simply watches the slot, checks the value is below 2^31, and may queue work that does not need the
+ * count in between. */
 GSX_API size_t gsx_intersect_tile_count_ordered_workspace_bytes(uint32_t N);
 GSX_API int gsx_intersect_tile_count_ordered(uint32_t N, const float* means2d, const int32_t* radii,
                                              const float* depths, uint32_t tile_size, uint32_t tile_width,
