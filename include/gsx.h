@@ -160,6 +160,17 @@ GSX_API int gsx_radix_sort_pairs_selector(int64_t n, uint32_t begin_bit, uint32_
 GSX_API int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, int64_t* keys1, int32_t* vals1,
                                  uint32_t begin_bit, uint32_t end_bit, void* workspace, size_t workspace_bytes,
                                  int* selector_host, void* stream);
+/* The same sort for callers that cannot allocate device memory and so cannot bring a workspace: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference (its sort takes
+ * its temporary storage from the caching allocator, IntersectTile.cu:305-327).  The histogram table lives in an
+ * array built into the library: 4 MiB + 1.25 KiB of device memory on every GPU the library runs on, held until the
+ * process ends.  n > GSX_RADIX_SORT_STATIC_MAX_PAIRS returns GSX_ERR_WORKSPACE.  The call allocates and frees
+ * nothing and does not synchronise; its first use on a device looks the array's address up once (make that call
+ * outside a capture).  All calls on one GPU share the one array: calls that overlap on a GPU (two streams, two
+ * threads) race - serialise them.  Nothing in the array has to start at zero, so no clearing is queued. */
+#define GSX_RADIX_SORT_STATIC_MAX_PAIRS (1ll << 24)
+GSX_API int gsx_radix_sort_pairs_static(int64_t n, int64_t* keys0, int32_t* vals0, int64_t* keys1, int32_t* vals1,
+                                        uint32_t begin_bit, uint32_t end_bit, int* selector_host, void* stream);
 
 /* ---- a6: gsplat::intersect_offset (Ops.h:39-43; IntersectTile.cu:206-286) -> offsets i32 [C,Th,Tw] ---- */
 GSX_API int gsx_intersect_offset(int64_t n_isects, const int64_t* isect_ids, uint32_t C, uint32_t tile_width,

@@ -9,6 +9,8 @@
 // and ranks them 64 at a time with wave-wide match masks (one 64-bit mask per digit in LDS, set by atomic OR), so
 // the order (wave, round, lane) equals the input order and the sort is stable.  The ranked pairs are first placed in LDS in digit order and then
 // written out by consecutive lanes, so that every (tile, digit) run leaves the block as whole cache lines.
+#include <mutex>
+
 #include "gsx_common.h"
 
 namespace gsx {
@@ -359,4 +361,56 @@ extern "C" int gsx_radix_sort_tile_pairs(int64_t n, uint16_t* keys0, int32_t* va
                                          int* selector_host, void* stream) {
     return sort_pairs<uint16_t>("radix_sort_tile_pairs", n, keys0, vals0, keys1, vals1, 0, n_bits, workspace,
                                 workspace_bytes, selector_host, stream);
+}
+
+// ---- the pair sort for callers that cannot allocate (and so cannot bring a workspace) ----------------------------
+// The histogram table and the digit totals live in a file-scope device array.  Every GPU the library runs on holds
+// its own copy of the array at its own address (4 MiB + 1.25 KiB until the process ends); the address is looked up
+// once per device and only that pointer is ever handed to kernels.
+namespace {
+static constexpr size_t kStaticScratchBytes =
+    (size_t)(GSX_RADIX_SORT_STATIC_MAX_PAIRS / (256 * kItemsLarge)) * kRadix * 4 + 256 + kRadix * 4;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+static constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices] = {};
+
+// the device address of `scratch` on the current device
+int static_scratch(void** out) {
+    int dev = -1;
+    GSX_HIP_CHECK(hipGetDevice(&dev));
+    GSX_REQUIRE(dev >= 0 && dev < kMaxDevices, GSX_ERR_UNSUPPORTED, "radix_sort_pairs_static: device ordinal %d", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        GSX_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        GSX_REQUIRE(p != nullptr && ((uintptr_t)p & 255) == 0, GSX_ERR_HIP,
+                    "radix_sort_pairs_static: the scratch array's device address %p is unusable", p);
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return GSX_OK;
+}
+} // namespace
+
+extern "C" int gsx_radix_sort_pairs_static(int64_t n, int64_t* keys0, int32_t* vals0, int64_t* keys1, int32_t* vals1,
+                                           uint32_t begin_bit, uint32_t end_bit, int* selector_host, void* stream) {
+    if (selector_host)
+        *selector_host = 0;
+    if (n <= 0)
+        return GSX_OK;
+    GSX_REQUIRE(n <= (int64_t)GSX_RADIX_SORT_STATIC_MAX_PAIRS, GSX_ERR_WORKSPACE,
+                "radix_sort_pairs_static: n = %lld exceeds the built-in scratch's limit of %lld pairs "
+                "(use gsx_radix_sort_pairs with a workspace)",
+                (long long)n, (long long)GSX_RADIX_SORT_STATIC_MAX_PAIRS);
+    GSX_REQUIRE(gsx_radix_sort_pairs_workspace_bytes(n) <= kStaticScratchBytes, GSX_ERR_WORKSPACE,
+                "radix_sort_pairs_static: %zu bytes of scratch needed, %zu built in",
+                gsx_radix_sort_pairs_workspace_bytes(n), kStaticScratchBytes);
+    void* ws = nullptr;
+    const int st = static_scratch(&ws);
+    if (st != GSX_OK)
+        return st;
+    return sort_pairs<int64_t>("radix_sort_pairs_static", n, keys0, vals0, keys1, vals1, begin_bit, end_bit, ws,
+                               kStaticScratchBytes, selector_host, stream);
 }
