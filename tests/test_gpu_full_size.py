@@ -6,6 +6,7 @@ import time
 import numpy as np
 import pytest
 
+from oracle.checks import step_with_truth
 from step_checks import N, check_first_step, check_forward_bit_exact, check_loss
 from test_golden import binoms
 
@@ -90,20 +91,55 @@ def _full_step(gsx, cuda, cfg):
     ts.step(vm, Km, cam.width, cam.height, gt_d)
     torch.cuda.synchronize()
     t2 = time.time()
-    ref.step(cam.viewmat, cam.K, cam.width, cam.height, gt)
+    truth = step_with_truth(ref, cam.viewmat, cam.K, cam.width, cam.height, gt)
     t3 = time.time()
-    print(f"cfg{cfg}: setup {t1 - t0:.1f}s gpu step {t2 - t1:.2f}s cpu step {t3 - t2:.1f}s n_isects {ts.n_isects}",
-          flush=True)
+    print(f"cfg{cfg}: setup {t1 - t0:.1f}s gpu step {t2 - t1:.2f}s cpu step + float64 backward {t3 - t2:.1f}s "
+          f"n_isects {ts.n_isects}", flush=True)
     n = stage_properties(ts)
     check_forward_bit_exact(ts, ref, min_isects=1_000_000)
     check_loss(ts, ref)
-    check_first_step(ts, ref)
+    check_first_step(ts, ref, truth, tag=f"cfg{cfg} full size: ")
     return sc, cam, ts, ref, n
 
 
 def test_config3_full_step(gsx, orc, cuda):
     """1M Gaussians, 1237x822: forward + 0.8 L1 + 0.2 (1 - SSIM) + backward + Adam"""
     _full_step(gsx, cuda, 3)
+
+
+def test_config3_full_size_on_the_benchmarked_path(gsx, orc, cuda):
+    """Configuration 3 at full size through exactly the code path bench.py times: one-pass backward + update
+    (fused_update), two-kernel loss (fused_loss), second stream (overlap), tile visiting order on.  Two iterations
+    from the same camera tensors, so the second forward pass reuses the tile order formed from the first one's costs
+    and both side-stream joins are exercised.  Before the second iteration the GPU state is set to the checker's, so
+    that it, too, starts from identical parameters and moments: keys / order / ranges / image bit-exact, loss <= 1e-5,
+    parameters and both moments by the element-wise bars, in both iterations."""
+    from lichtfeld_studio_amd.trainer import TrainStep
+    from oracle.step import OracleTrainStep
+    sc = gsx.scenes.config(3)
+    cam = sc.cameras[0]
+    gt_d = target_image(gsx, sc, cam, cuda)
+    gt = N(gt_d)[0]
+    ts = TrainStep(sc, cuda, fused_update=True, fused_loss=True, overlap=True)
+    assert ts.order_tiles and ts.fused_loss and ts.side is not None
+    ref = OracleTrainStep(sc)
+    vm, Km = T(cam.viewmat[None], cuda), T(cam.K[None], cuda)
+    prev = None
+    for it in range(2):
+        reused = getattr(ts, "have_walk", False) and ts._walk_cam == (vm.data_ptr(), Km.data_ptr(), cam.width, cam.height)
+        assert reused == (it == 1), "the second forward pass must run with the order left by the first"
+        ts.step(vm, Km, cam.width, cam.height, gt_d)
+        torch.cuda.synchronize()
+        truth = step_with_truth(ref, cam.viewmat, cam.K, cam.width, cam.height, gt)
+        stage_properties(ts)
+        check_forward_bit_exact(ts, ref, min_isects=1_000_000)
+        check_loss(ts, ref)
+        check_first_step(ts, ref, truth, tag=f"cfg3 bench path, iteration {it + 1}: ", prev=prev)
+        prev = ({k: v.copy() for k, v in ref.exp_avg.items()}, {k: v.copy() for k, v in ref.exp_avg_sq.items()})
+        for k in ts.params:  # identical state for the next iteration
+            ts.params[k].copy_(T(ref.params[k], cuda))
+            ts.exp_avg[k].copy_(T(ref.exp_avg[k], cuda))
+            ts.exp_avg_sq[k].copy_(T(ref.exp_avg_sq[k], cuda))
 
 
 def test_config4_step_relocation_noise(gsx, orc, cuda):

@@ -35,14 +35,15 @@ def test_train_step_matches_oracle(gsx, orc, cuda, cfg, n, use_ssim, reg):
     ref = OracleTrainStep(sc, lambda_dssim=0.2 if use_ssim else 0.0, scale_reg=reg, opacity_reg=reg)
     gt_d = torch.from_numpy(gt[None].copy()).to(cuda)
 
+    from oracle.checks import step_with_truth
     for it in range(2):
         ts.step(vm, Km, W, H, gt_d)
-        ref.step(cam.viewmat, cam.K, W, H, gt)
+        truth = step_with_truth(ref, cam.viewmat, cam.K, W, H, gt)
         torch.cuda.synchronize()
         if it == 0:
             check_forward_bit_exact(ts, ref)
             check_loss(ts, ref)
-            check_first_step(ts, ref)
+            check_first_step(ts, ref, truth, tag=f"step cfg{cfg} n={n} reg={reg}: ")
             if reg:
                 # loss values of the two terms on the updated parameters (which agree to the Adam tolerance)
                 got = [float(x) for x in ts.regularization_losses().cpu()]

@@ -163,8 +163,15 @@ def test_backward_matches_finite_differences_of_the_model(orc):
     g32 = orc.rasterize_to_pixels_from_world_3dgs_bwd(*args, None, W, H, TILE, s["V"][None], s["K"][None], off, flat, a,
                                                       last, w_img[None].astype(np.float32),
                                                       w_al[None, :, :, None].astype(np.float32))
-    g64, _ = orc.rasterize_bwd_f64(*args, W, H, TILE, s["V"][None], s["K"][None], off, flat, a, last,
-                                   w_img[None].astype(np.float32), w_al[None, :, :, None].astype(np.float32))
+    g64, b64 = orc.rasterize_bwd_f64(*args, W, H, TILE, s["V"][None], s["K"][None], off, flat, a, last,
+                                     w_img[None].astype(np.float32), w_al[None, :, :, None].astype(np.float32))
+    # the absolute-value chain: never below the value, zero only where the value is, and u * bound is the scale of the
+    # fp32 evaluation's own error (it would not be if a term were missing from the chain or the chain were inflated)
+    assert (b64 >= np.abs(g64) * (1 - 1e-12)).all() and ((b64 == 0) == (g64 == 0)).all()
+    c32 = np.concatenate([g32[0], g32[1], g32[2], g32[3][0], g32[4].reshape(-1, 1)], 1).astype(np.float64)
+    need = (np.abs(c32 - g64) - 1e-3 * np.abs(g64)) / np.maximum(2.0 ** -24 * b64, 1e-300)
+    assert need.max() < 64, need.max()
+    assert np.quantile(np.abs(c32 - g64)[b64 > 0] / (2.0 ** -24 * b64[b64 > 0]), 0.99) > 0.05
     w32i, w32a = w_img.astype(np.float32).astype(np.float64), w_al.astype(np.float32).astype(np.float64)
 
     def loss(p):
