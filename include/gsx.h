@@ -196,6 +196,41 @@ GSX_API int gsx_radix_sort_tile_pairs(int64_t n, uint16_t* keys0, int32_t* vals0
 GSX_API int gsx_intersect_tile_pairs_offset(int64_t n_isects, const uint16_t* tile_keys, uint32_t tile_width,
                                             uint32_t tile_height, int32_t* offsets, void* stream);
 
+/* ---- a4-a6 as one call whose pair count never crosses to the host (one camera, grids up to 255 x 255) ----
+ * No single counterpart in the reference: this is intersect_tile + radix_sort_double_buffer + intersect_offset
+ * (Intersect.cpp:41-137, IntersectTile.cu:23-114, 206-252, 290-328) for the caller that only feeds the rasterizers,
+ * without the `.item()` of Intersect.cpp:76.  Ten launches: depth keys (+ byte histograms + tile-rectangle corners),
+ * tile table (a 2-D prefix sum over the corners gives every list's length, hence tile_offsets and the count, before a
+ * pair exists), four one-launch radix passes over the N depth keys, the emission of (u16 tile, id) pairs in depth
+ * order, two one-launch radix passes over the tile bits.  The one-launch passes chain their workgroups by a bounded
+ * look-back over per-workgroup counts.
+ *   flatten_ids  i32 [capacity]            out: element for element the flatten_ids of the separate operators
+ *   tile_offsets i32 [Th * Tw + 1]         out: the operators' tile_offsets, and the pair count in the last entry
+ *   n_isects_host_slot                     nullable; pinned host memory (hipHostMalloc): receives the pair count
+ *                                          with one 8-byte store from the device (write -1 there first to see it land)
+ * Consumers take the count from the device: pass n_isects = GSX_COUNT_IN_OFFSETS to gsx_tile_order,
+ * gsx_rasterize_records_fwd and gsx_rasterize_bwd_accumulate together with this tile_offsets.
+ * If the pairs exceed `capacity` (or 2^30 - 1) every list is left empty (tile_offsets all zero), bit 0 of the error
+ * word is set and the true count is still reported: grow the buffers and run the step again.  Nothing is read or
+ * written out of bounds in that case.  Bit 1 of the error word: a look-back's bounded wait ran out (results invalid).
+ * The workspace's head must be zeroed once by gsx_tile_lists_init; every call leaves it ready for the next one.  Calls
+ * that share a workspace must not overlap. */
+#define GSX_COUNT_IN_OFFSETS (-1ll)
+GSX_API size_t gsx_tile_lists_workspace_bytes(uint32_t N, int64_t capacity, uint32_t tile_width,
+                                              uint32_t tile_height);
+GSX_API int gsx_tile_lists_init(uint32_t N, int64_t capacity, uint32_t tile_width, uint32_t tile_height,
+                                void* workspace, size_t workspace_bytes, void* stream);
+GSX_API int gsx_tile_lists(uint32_t N, const float* means2d, const int32_t* radii, const float* depths,
+                           uint32_t tile_size, uint32_t tile_width, uint32_t tile_height, int64_t capacity,
+                           void* workspace, size_t workspace_bytes, int32_t* flatten_ids, int32_t* tile_offsets,
+                           int64_t* n_isects_host_slot, void* stream);
+/* device addresses inside the workspace: counts i64 [2] = {pairs in the lists (0 if they did not fit), pairs there
+ * are}; error u32 (bits above; sticky until the caller clears it or calls gsx_tile_lists_init) */
+GSX_API const int64_t* gsx_tile_lists_counts(uint32_t N, int64_t capacity, uint32_t tile_width,
+                                             uint32_t tile_height, const void* workspace);
+GSX_API uint32_t* gsx_tile_lists_error(uint32_t N, int64_t capacity, uint32_t tile_width, uint32_t tile_height,
+                                       void* workspace);
+
 /* ---- a7: gsplat::rasterize_to_pixels_from_world_3dgs_fwd (Ops.h:100-129; ...3DGSFwd.cu:19-285) ----
  * colors [C,N,channels] (channels in {1,3,4}), opacities [C,N], backgrounds [C,channels] nullable,
  * masks u8 [C,Th,Tw] nullable, tile_offsets i32 [C,Th,Tw], flatten_ids i32 [n_isects]

@@ -62,6 +62,25 @@ int radix_sort_pairs_32_bits(int64_t n, int64_t* keys0, int32_t* vals0, int64_t*
                              uint32_t begin_bit, void* workspace, size_t workspace_bytes, int* selector_host,
                              void* stream, bool first_hist_done);
 
+// radix_sort.hip: one stable 1..8-bit radix pass as ONE launch (chained look-back between the workgroups).  The
+// caller provides digit_total[256] = how many of the pairs carry each digit, a status table of
+// radix_chained_rows(n_max) x 256 empty (zero) words and a zero ticket word; the launch can clear the table and ticket
+// of the pass that follows it.  n_dev (nullable): the number of pairs is min(*n_dev, n_max), read on the device.
+// Limit: n_max < 2^30.  error: device word, bit 1 is set if a look-back's bounded wait ran out.
+struct RadixChainArgs {
+    const int64_t* n_dev;
+    uint32_t *status, *ticket, *clear_status;
+    uint32_t clear_rows;
+    uint32_t *clear_ticket, *error;
+};
+uint32_t radix_chained_rows(int64_t n_max);
+int radix_chained_pass_i64(uint32_t n_max, const int64_t* kin, const int32_t* vin, int64_t* kout, int32_t* vout,
+                           uint32_t shift, uint32_t bits, const uint32_t* digit_total, const RadixChainArgs& a,
+                           void* stream);
+int radix_chained_pass_u16(uint32_t n_max, const uint16_t* kin, const int32_t* vin, uint16_t* kout, int32_t* vout,
+                           uint32_t shift, uint32_t bits, const uint32_t* digit_total, const RadixChainArgs& a,
+                           bool write_keys, void* stream);
+
 int check_camera_args(uint32_t C, const float* viewmats1, int camera_model, int rs_type, const float* radial,
                       const float* tangential, const float* thin_prism);
 
@@ -283,6 +302,8 @@ __device__ __forceinline__ vec3 camera_ray_origin(const CamPose& cp) {
 // One 256-lane workgroup per 16x16 tile; wave w owns the 8x8 pixel block (w & 1, w >> 1), lane l the pixel
 // (l >> 3, l & 7) of it: compact blocks keep a wave's pixels coherent (saturation, bounds rejection).
 static constexpr uint32_t kTile = 16;
+// what (uint32_t)GSX_COUNT_IN_OFFSETS is inside the kernels
+static constexpr uint32_t kCountInOffsets = 0xFFFFFFFFu;
 static constexpr uint32_t kBatch = 256;
 
 struct TilePixel {

@@ -2,31 +2,9 @@
 // per-tile ranges of the sorted keys (gsplat/IntersectTile.cu:23-114, 206-252; gsplat/Intersect.cpp:41-137).
 // Integer work: every output is bit-exact given the inputs.
 #include "gsx_common.h"
+#include "gsx_tiles.h"
 
 namespace gsx {
-
-struct TileRect {
-    uint32_t x0, y0, x1, y1;
-};
-
-// IntersectTile.cu:56-76.  The float -> uint32 conversions saturate (negative -> 0): that is what the
-// reference's hardware conversion does, and plain C++ casts of negative floats are undefined.
-__device__ __forceinline__ bool tile_rect(const float* __restrict__ means2d, const int32_t* __restrict__ radii,
-                                          uint32_t idx, float tile_size, uint32_t tile_width, uint32_t tile_height,
-                                          TileRect* r) {
-    const int2 rad = reinterpret_cast<const int2*>(radii)[idx];
-    const float radius_x = (float)rad.x, radius_y = (float)rad.y;
-    if (radius_x <= 0 || radius_y <= 0)
-        return false;
-    const float2 m = reinterpret_cast<const float2*>(means2d)[idx];
-    const float tile_radius_x = radius_x / tile_size, tile_radius_y = radius_y / tile_size;
-    const float tile_x = m.x / tile_size, tile_y = m.y / tile_size;
-    r->x0 = min(sat_u32(gsx::floor(tile_x - tile_radius_x)), tile_width);
-    r->y0 = min(sat_u32(gsx::floor(tile_y - tile_radius_y)), tile_height);
-    r->x1 = min(sat_u32(gsx::ceil(tile_x + tile_radius_x)), tile_width);
-    r->y1 = min(sat_u32(gsx::ceil(tile_y + tile_radius_y)), tile_height);
-    return true;
-}
 
 __global__ void __launch_bounds__(256) tile_count_kernel(uint32_t n, const float* __restrict__ means2d,
                                                           const int32_t* __restrict__ radii, float tile_size,
@@ -40,15 +18,6 @@ __global__ void __launch_bounds__(256) tile_count_kernel(uint32_t n, const float
     if (tile_rect(means2d, radii, idx, tile_size, tile_width, tile_height, &r))
         cnt = (int32_t)((r.y1 - r.y0) * (r.x1 - r.x0));
     tiles_per_gauss[idx] = cnt;
-}
-
-// Depth-ordered variant, one camera: the tile count rides in the high word of a sort key whose low word is the
-// depth's bit pattern (what the low word of an intersection key holds; all ones for a Gaussian that touches no
-// tile).  Sorting these N keys on their low 32 bits gives the visiting order AND the counts in that order.
-// RECT (tile grids up to 255 x 255): the high word holds the tile rectangle x0 | y0 << 8 | x1 << 16 | y1 << 24
-// instead (0 = no tile), from which both the count and the emission follow without going back to the Gaussian.
-__device__ __forceinline__ uint32_t packed_rect_count(uint32_t hi) {
-    return (((hi >> 24) & 255u) - ((hi >> 8) & 255u)) * (((hi >> 16) & 255u) - (hi & 255u));
 }
 
 // A workgroup writes the keys of one block of the sort that follows (256 * items consecutive Gaussians) and leaves
@@ -304,7 +273,7 @@ __device__ __forceinline__ uint32_t tile_len_class(uint32_t len) {
         return 0;
     const uint32_t e = 31u - (uint32_t)__clz((int)len);
     const uint32_t m = e >= 4 ? (len >> (e - 4)) & 15u : (len << (4 - e)) & 15u; // four bits below the leading one
-    return e * 16u + m + 1u;
+    return min(e * 16u + m + 1u, kLenClasses - 1u);
 }
 
 __global__ void __launch_bounds__(1024) tile_order_kernel(uint32_t n_tiles, uint32_t n_isects,
@@ -318,7 +287,7 @@ __global__ void __launch_bounds__(1024) tile_order_kernel(uint32_t n_tiles, uint
     auto length = [&](uint32_t t) {
         if (tile_cost != nullptr)
             return tile_cost[t];
-        const uint32_t end = t + 1 < n_tiles ? (uint32_t)tile_offsets[t + 1] : n_isects;
+        const uint32_t end = (t + 1 < n_tiles || n_isects == kCountInOffsets) ? (uint32_t)tile_offsets[t + 1] : n_isects;
         return end - (uint32_t)tile_offsets[t];
     };
     for (uint32_t t = threadIdx.x; t < n_tiles; t += 1024)
@@ -754,8 +723,8 @@ extern "C" int gsx_tile_order(int64_t n_isects, const int32_t* tile_offsets, con
     if (n_tiles == 0)
         return GSX_OK;
     GSX_REQUIRE((tile_offsets || tile_cost) && tile_order, GSX_ERR_INVALID_ARGUMENT, "tile_order: null tensor");
-    GSX_REQUIRE(n_isects >= 0 && n_isects < (1ll << 31) && n_tiles < (1ull << 31), GSX_ERR_OVERFLOW,
-                "tile_order: sizes out of range");
+    GSX_REQUIRE(n_isects >= GSX_COUNT_IN_OFFSETS && n_isects < (1ll << 31) && n_tiles < (1ull << 31),
+                GSX_ERR_OVERFLOW, "tile_order: sizes out of range");
     hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, (uint32_t)n_tiles,
                        (uint32_t)n_isects, tile_offsets, tile_cost, tile_order);
     GSX_LAUNCH_CHECK();

@@ -12,6 +12,7 @@
 #include <mutex>
 
 #include "gsx_common.h"
+#include "gsx_lookback.h"
 
 namespace gsx {
 
@@ -108,18 +109,35 @@ __global__ void __launch_bounds__(256) radix_scan_kernel(uint32_t nblocks, uint3
 }
 
 // ---- stable scatter -------------------------------------------------------------------------------
-template <typename KeyT, uint32_t ITEMS>
+// CHAINED = false: the positions come from the scanned histogram table of the two launches before (hist_scanned,
+// digit_total).  CHAINED = true: one launch per pass - digit_total holds the digit counts of the whole input (left by
+// whoever wrote the keys), every workgroup takes its place in the input from a ticket, publishes its 256 digit counts
+// and obtains the counts of the workgroups in front of it by a chained look-back (gsx_lookback.h); the number of
+// pairs is read from device memory, and the launch also clears the status words the NEXT pass will use.
+struct RadixChain {
+    const int64_t* n_dev;   // number of pairs (device); the launch covers min(*n_dev, n) pairs
+    uint32_t* status;       // [workgroups][256], empty on entry
+    uint32_t* ticket;       // 0 on entry
+    uint32_t* clear_status; // status words of the next pass (nullable): clear_rows rows are cleared by this launch
+    uint32_t clear_rows;
+    uint32_t* clear_ticket; // nullable
+    uint32_t* error;        // bit 1 is set when a look-back gave up
+};
+
+template <typename KeyT, uint32_t ITEMS, bool CHAINED, bool WRITE_KEYS>
 __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const KeyT* __restrict__ keys_in,
                                                              const int32_t* __restrict__ vals_in,
                                                              KeyT* __restrict__ keys_out,
                                                              int32_t* __restrict__ vals_out, uint32_t shift,
                                                              uint32_t mask, uint32_t nblocks,
                                                              const uint32_t* __restrict__ hist_scanned,
-                                                             const uint32_t* __restrict__ digit_total) {
+                                                             const uint32_t* __restrict__ digit_total,
+                                                             RadixChain chain) {
     constexpr uint32_t kTileN = 256 * ITEMS, kWaveN = 64 * ITEMS;
     __shared__ uint32_t wave_count[4][kRadix];
     __shared__ uint32_t to_global[kRadix]; // global position of a pair = to_global[digit] + its slot in the tile
     __shared__ uint32_t wsum[4], gsum[4];
+    __shared__ uint32_t place_s;
     // the match masks of the ranking phase and the reordered tile of the output phase share their bytes
     constexpr uint32_t kMatchBytes = 4 * kRadix * 8, kTileBytes = kTileN * (sizeof(KeyT) + 4);
     __shared__ __align__(16) unsigned char overlay[kMatchBytes > kTileBytes ? kMatchBytes : kTileBytes];
@@ -128,6 +146,22 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const Ke
     KeyT* s_keys = reinterpret_cast<KeyT*>(overlay + kTileN * 4);
     const uint32_t t = threadIdx.x;
     const uint32_t w = t >> 6, lane = t & 63u;
+    uint32_t place = blockIdx.x;
+    if (CHAINED) {
+        place = lb_take_ticket(chain.ticket, &place_s);
+        if (chain.n_dev != nullptr) {
+            const int64_t nd = *chain.n_dev;
+            n = nd < (int64_t)n ? (uint32_t)(nd < 0 ? 0 : nd) : n;
+        }
+        // housekeeping for the pass after this one (its launch starts after this one has ended)
+        if (chain.clear_status != nullptr)
+            for (uint32_t row = place; row < chain.clear_rows; row += gridDim.x)
+                chain.clear_status[(size_t)row * kRadix + t] = 0u;
+        if (chain.clear_ticket != nullptr && place == 0 && t == 0)
+            *chain.clear_ticket = 0u;
+        if ((uint64_t)place * kTileN >= n)
+            return; // uniform over the workgroup; later places are empty too
+    }
 #pragma unroll
     for (uint32_t i = 0; i < 4; ++i) {
         wave_count[i][t] = 0;
@@ -135,7 +169,7 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const Ke
     }
     __syncthreads();
 
-    const uint32_t tile_base = blockIdx.x * kTileN;
+    const uint32_t tile_base = place * kTileN;
     const uint32_t wave_base = tile_base + w * kWaveN;
     const uint64_t lt_mask = (1ull << lane) - 1ull;
     KeyT key[ITEMS];
@@ -186,6 +220,8 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const Ke
     {
         const uint32_t c0 = wave_count[0][t], c1 = wave_count[1][t], c2 = wave_count[2][t], c3 = wave_count[3][t];
         const uint32_t tot = c0 + c1 + c2 + c3;
+        if (CHAINED) // the first place has nobody in front of it: its counts are a complete prefix already
+            lb_publish(chain.status + (size_t)place * kRadix + t, place == 0 ? kLbPrefix : kLbAggregate, tot);
         const uint32_t gtot = digit_total[t]; // pairs with digit t in the whole input
         const uint32_t incl = wave_inclusive_scan_u32(tot, lane);
         const uint32_t gincl = wave_inclusive_scan_u32(gtot, lane);
@@ -206,7 +242,18 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const Ke
         wave_count[1][t] = start + c0;
         wave_count[2][t] = start + c0 + c1;
         wave_count[3][t] = start + c0 + c1 + c2;
-        to_global[t] = smaller + hist_scanned[t * nblocks + blockIdx.x] - start;
+        uint32_t earlier; // pairs with digit t in the workgroups in front of this one
+        if (CHAINED) {
+            uint32_t gave_up = 0;
+            earlier = lb_exclusive(chain.status, place, kRadix, t, &gave_up);
+            if (place != 0)
+                lb_publish(chain.status + (size_t)place * kRadix + t, kLbPrefix, earlier + tot);
+            if (gave_up)
+                atomicOr(chain.error, 2u);
+        } else {
+            earlier = hist_scanned[t * nblocks + blockIdx.x];
+        }
+        to_global[t] = smaller + earlier - start;
     }
     __syncthreads();
 #pragma unroll
@@ -226,8 +273,12 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const Ke
         if (slot < count) {
             const KeyT kk = s_keys[slot];
             const uint32_t pos = to_global[digit_of(kk, shift, mask)] + slot;
-            keys_out[pos] = kk;
-            vals_out[pos] = s_vals[slot];
+            // chained: digit totals that disagree with the keys (a caller's mistake) must not write out of bounds
+            if (!CHAINED || pos < n) {
+                if (WRITE_KEYS)
+                    keys_out[pos] = kk;
+                vals_out[pos] = s_vals[slot];
+            }
         }
     }
 }
@@ -313,11 +364,13 @@ int sort_pairs(const char* what, int64_t n, KeyT* keys0, int32_t* vals0, KeyT* k
         hipLaunchKernelGGL(radix_scan_kernel, dim3(kRadix), dim3(256), 0, s, L.nblocks, hist, totals);
         GSX_LAUNCH_CHECK();
         if (items == kItemsSmall)
-            hipLaunchKernelGGL((radix_scatter_kernel<KeyT, kItemsSmall>), dim3(L.nblocks), dim3(256), 0, s,
-                               (uint32_t)n, kin, vin, kout, vout, shift, mask, L.nblocks, hist, totals);
+            hipLaunchKernelGGL((radix_scatter_kernel<KeyT, kItemsSmall, false, true>), dim3(L.nblocks), dim3(256), 0,
+                               s, (uint32_t)n, kin, vin, kout, vout, shift, mask, L.nblocks, hist, totals,
+                               RadixChain{});
         else
-            hipLaunchKernelGGL((radix_scatter_kernel<KeyT, kItemsLarge>), dim3(L.nblocks), dim3(256), 0, s,
-                               (uint32_t)n, kin, vin, kout, vout, shift, mask, L.nblocks, hist, totals);
+            hipLaunchKernelGGL((radix_scatter_kernel<KeyT, kItemsLarge, false, true>), dim3(L.nblocks), dim3(256), 0,
+                               s, (uint32_t)n, kin, vin, kout, vout, shift, mask, L.nblocks, hist, totals,
+                               RadixChain{});
         GSX_LAUNCH_CHECK();
         sel ^= 1;
         shift += bits;
@@ -345,6 +398,57 @@ int radix_sort_pairs_32_bits(int64_t n, int64_t* keys0, int32_t* vals0, int64_t*
                              void* stream, bool first_hist_done) {
     return sort_pairs<int64_t>("radix_sort_pairs", n, keys0, vals0, keys1, vals1, begin_bit, begin_bit + 32, workspace,
                                workspace_bytes, selector_host, stream, first_hist_done);
+}
+} // namespace gsx
+
+namespace gsx {
+// ---- one launch per pass (declared in gsx_common.h) ------------------------------------------------
+uint32_t radix_chained_rows(int64_t n_max) { return n_max <= 0 ? 1u : cdiv((uint64_t)n_max, 256u * sort_items(n_max)); }
+
+namespace {
+template <typename KeyT>
+int chained_pass(uint32_t n_max, const KeyT* kin, const int32_t* vin, KeyT* kout, int32_t* vout, uint32_t shift,
+                 uint32_t bits, const uint32_t* digit_total, const RadixChainArgs& a, bool write_keys, void* stream) {
+    GSX_REQUIRE(n_max > 0 && n_max < (1u << kLbValueBits), GSX_ERR_OVERFLOW,
+                "chained radix pass: %u pairs (limit 2^30 - 1)", n_max);
+    GSX_REQUIRE(bits >= 1 && bits <= kRadixBits && kin && vin && vout && (kout || !write_keys) && digit_total &&
+                    a.status && a.ticket && a.error,
+                GSX_ERR_INVALID_ARGUMENT, "chained radix pass: bad argument");
+    const uint32_t items = sort_items(n_max), rows = radix_chained_rows(n_max);
+    const uint32_t mask = (1u << bits) - 1u;
+    RadixChain c;
+    c.n_dev = a.n_dev, c.status = a.status, c.ticket = a.ticket, c.clear_status = a.clear_status;
+    c.clear_rows = a.clear_rows, c.clear_ticket = a.clear_ticket, c.error = a.error;
+    hipStream_t s = (hipStream_t)stream;
+#define GSX_CHAINED(IT, WK)                                                                                       \
+    hipLaunchKernelGGL((radix_scatter_kernel<KeyT, IT, true, WK>), dim3(rows), dim3(256), 0, s, n_max, kin, vin, \
+                       kout, vout, shift, mask, rows, (const uint32_t*)nullptr, digit_total, c)
+    if (items == kItemsSmall) {
+        if (write_keys)
+            GSX_CHAINED(kItemsSmall, true);
+        else
+            GSX_CHAINED(kItemsSmall, false);
+    } else {
+        if (write_keys)
+            GSX_CHAINED(kItemsLarge, true);
+        else
+            GSX_CHAINED(kItemsLarge, false);
+    }
+#undef GSX_CHAINED
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+} // namespace
+
+int radix_chained_pass_i64(uint32_t n_max, const int64_t* kin, const int32_t* vin, int64_t* kout, int32_t* vout,
+                           uint32_t shift, uint32_t bits, const uint32_t* digit_total, const RadixChainArgs& a,
+                           void* stream) {
+    return chained_pass<int64_t>(n_max, kin, vin, kout, vout, shift, bits, digit_total, a, true, stream);
+}
+int radix_chained_pass_u16(uint32_t n_max, const uint16_t* kin, const int32_t* vin, uint16_t* kout, int32_t* vout,
+                           uint32_t shift, uint32_t bits, const uint32_t* digit_total, const RadixChainArgs& a,
+                           bool write_keys, void* stream) {
+    return chained_pass<uint16_t>(n_max, kin, vin, kout, vout, shift, bits, digit_total, a, write_keys, stream);
 }
 } // namespace gsx
 

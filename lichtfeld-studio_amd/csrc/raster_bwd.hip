@@ -102,7 +102,9 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
         o_shift = sub(ray_o, camera_ray_origin(load_cam_pose(viewmat)));
 
     const int32_t range_start = tile_offsets[tile_id];
-    int32_t range_end = (tile_id == tile_width * tile_height - 1) ? (int32_t)n_isects : tile_offsets[tile_id + 1];
+    int32_t range_end = (tile_id == tile_width * tile_height - 1 && n_isects != kCountInOffsets)
+                            ? (int32_t)n_isects
+                            : tile_offsets[tile_id + 1];
 
     const float T_final = 1.0f - render_alphas[pix_id];
     float T = T_final;
@@ -396,7 +398,8 @@ static int rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isects, co
     if (N == 0 || n_isects == 0 || image_width == 0 || image_height == 0) // ...Bwd.cu:440-443
         return GSX_OK;
     GSX_REQUIRE(tile_size == kTile, GSX_ERR_UNSUPPORTED, "rasterize bwd: tile_size %u (only 16 is built)", tile_size);
-    GSX_REQUIRE(n_isects > 0 && n_isects < (1ll << 31), GSX_ERR_OVERFLOW, "rasterize bwd: n_isects out of range");
+    GSX_REQUIRE(n_isects >= GSX_COUNT_IN_OFFSETS && n_isects < (1ll << 31), GSX_ERR_OVERFLOW,
+                "rasterize bwd: n_isects out of range");
     GSX_REQUIRE(records && viewmats0 && Ks && tile_offsets && flatten_ids && render_alphas && last_ids &&
                     v_render_colors && v_render_alphas,
                 GSX_ERR_INVALID_ARGUMENT, "rasterize bwd: null tensor");

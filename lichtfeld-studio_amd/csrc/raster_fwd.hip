@@ -85,6 +85,8 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
             for (uint32_t k = 0; k < CDIM; ++k)
                 render_colors[(size_t)pix_id * CDIM + k] = backgrounds == nullptr ? 0.0f : backgrounds[k];
         }
+        if (tile_walk != nullptr && tr == 0 && !STATS)
+            tile_walk[tile_id] = 0u; // a masked tile costs nothing
         return;
     }
 
@@ -101,8 +103,10 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
         pixel_world_ray(cp, (float)j + 0.5f, (float)i + 0.5f, Kmat[0], Kmat[4], Kmat[2], Kmat[5], cam, &ray_o, &ray_d);
 
     const int32_t range_start = tile_offsets[tile_id];
-    const int32_t range_end =
-        (tile_id == tile_width * tile_height - 1) ? (int32_t)n_isects : tile_offsets[tile_id + 1];
+    // n_isects == kCountInOffsets: tile_offsets has one entry more, the count itself (read on the device)
+    const int32_t range_end = (tile_id == tile_width * tile_height - 1 && n_isects != kCountInOffsets)
+                                  ? (int32_t)n_isects
+                                  : tile_offsets[tile_id + 1];
     const uint32_t num_batches = (uint32_t)(range_end - range_start + (int32_t)kBatch - 1) / kBatch;
 
     bool done = !inside || !ray_ok;
@@ -292,7 +296,8 @@ int rasterize_records_fwd(int64_t n_isects, const void* records, const float* co
                           void* stream) {
     if (image_width == 0 || image_height == 0)
         return GSX_OK;
-    GSX_REQUIRE(n_isects >= 0 && n_isects < (1ll << 31), GSX_ERR_OVERFLOW, "rasterize fwd: n_isects out of range");
+    GSX_REQUIRE(n_isects >= GSX_COUNT_IN_OFFSETS && n_isects < (1ll << 31), GSX_ERR_OVERFLOW,
+                "rasterize fwd: n_isects out of range");
     GSX_REQUIRE(viewmat && K && tile_offsets && render_colors && render_alphas && last_ids, GSX_ERR_INVALID_ARGUMENT,
                 "rasterize fwd: null tensor");
     GSX_REQUIRE(n_isects == 0 || (records && flatten_ids && (channels <= 3 || colors)), GSX_ERR_INVALID_ARGUMENT,

@@ -1,0 +1,467 @@
+// tile_lists.hip - the per-tile lists of one camera in ten launches, without the pair count crossing to the host.
+//
+// What gsplat::intersect_tile + radix_sort_double_buffer + intersect_offset produce for one camera
+// (gsplat/Intersect.cpp:41-137, IntersectTile.cu:23-114, 206-252, 290-328) and what the rasterizers read of it:
+// flatten_ids (Gaussian ids, grouped by tile, depth order inside a tile, ties by id) and tile_offsets.  The result is
+// element for element the one of the separate operators; the organisation is not:
+//
+//  1. depth_keys_kernel      per Gaussian: tile rectangle, key (rectangle << 32 | depth bits), the four byte
+//                            histograms of the depth bits, and +1 / -1 at the rectangle's corners in a
+//                            (Th + 1) x (Tw + 1) grid;
+//  2. four chained radix passes (radix_sort.hip) order the N keys by depth, one launch each;
+//  3. tile_table_kernel      a 2-D prefix sum over the corner grid gives every tile's list length, hence
+//                            tile_offsets, the pair count, and the digit histograms of the pair sort - before a
+//                            single pair exists;
+//  4. tile_emit_chained_kernel  writes (16-bit tile index, id) pairs in depth order; a workgroup's position in the
+//                            output comes from a chained look-back over the workgroups' pair counts;
+//  5. two chained radix passes over the tile bits (the second one writes flatten_ids only).
+//
+// Everything downstream sizes its work by `capacity` and reads the actual count from device memory.  If the count
+// exceeds the capacity, every tile's list is left EMPTY (tile_offsets all zero), bit 0 of the error word is set and
+// the true count is still reported, so that the caller can grow its buffers and run the step again; nothing is
+// written or read out of bounds.
+#include "gsx_common.h"
+#include "gsx_lookback.h"
+#include "gsx_tiles.h"
+
+namespace gsx {
+
+static constexpr uint32_t kKeysPerBlock = 1024; // depth_keys_kernel: 4 Gaussians per lane
+
+// adds `count` to hist[digit] for every lane; one LDS atomic per wave when all its lanes share the digit (nine in
+// ten Gaussians of a training scene are culled and share the key 0xFFFFFFFF)
+__device__ __forceinline__ void wave_hist_add(uint32_t* hist, uint32_t digit, bool live) {
+    const uint64_t lanes = __ballot(live);
+    if (lanes == 0)
+        return;
+    const uint32_t first = (uint32_t)__builtin_amdgcn_readlane((int)digit, __builtin_ctzll(lanes));
+    if (__ballot(live && digit != first) == 0) {
+        if ((threadIdx.x & 63u) == (uint32_t)__builtin_ctzll(lanes))
+            atomicAdd(&hist[first], (uint32_t)__popcll(lanes));
+    } else if (live) {
+        atomicAdd(&hist[digit], 1u);
+    }
+}
+
+__global__ void __launch_bounds__(256) depth_keys_kernel(
+    uint32_t n, const float* __restrict__ means2d, const int32_t* __restrict__ radii,
+    const float* __restrict__ depths, float tile_size, uint32_t tile_width, uint32_t tile_height,
+    int64_t* __restrict__ keys, int32_t* __restrict__ vals, uint32_t* __restrict__ depth_hist /*[4][256], += */,
+    int32_t* __restrict__ corner_grid /*[(Th+1)(Tw+1)], += */, uint32_t* __restrict__ clear_status,
+    uint32_t clear_rows, uint32_t* __restrict__ clear_ticket, uint32_t* __restrict__ clear_emit_status,
+    uint32_t clear_emit_words, uint32_t* __restrict__ clear_emit_ticket) {
+    __shared__ uint32_t lh[4][256];
+    const uint32_t t = threadIdx.x;
+#pragma unroll
+    for (uint32_t k = 0; k < 4; ++k)
+        lh[k][t] = 0;
+    // housekeeping for the launches behind this one
+    for (uint32_t row = blockIdx.x; row < clear_rows; row += gridDim.x)
+        clear_status[(size_t)row * 256u + t] = 0u;
+    for (uint32_t wd = blockIdx.x * 256u + t; wd < clear_emit_words; wd += gridDim.x * 256u)
+        clear_emit_status[wd] = 0u;
+    if (blockIdx.x == 0 && t == 0) {
+        *clear_ticket = 0u;
+        *clear_emit_ticket = 0u;
+    }
+    __syncthreads();
+    const uint32_t gw = tile_width + 1u;
+#pragma unroll
+    for (uint32_t k = 0; k < kKeysPerBlock / 256; ++k) {
+        const uint32_t i = blockIdx.x * kKeysPerBlock + k * 256u + t;
+        const bool live = i < n;
+        uint32_t lo = 0xFFFFFFFFu, hi = 0;
+        if (live) {
+            TileRect r;
+            if (tile_rect(means2d, radii, i, tile_size, tile_width, tile_height, &r) && r.y1 > r.y0 && r.x1 > r.x0) {
+                lo = f2u(depths[i]);
+                hi = r.x0 | (r.y0 << 8) | (r.x1 << 16) | (r.y1 << 24);
+                atomicAdd(&corner_grid[r.y0 * gw + r.x0], 1);
+                atomicAdd(&corner_grid[r.y0 * gw + r.x1], -1);
+                atomicAdd(&corner_grid[r.y1 * gw + r.x0], -1);
+                atomicAdd(&corner_grid[r.y1 * gw + r.x1], 1);
+            }
+            keys[i] = (int64_t)(((uint64_t)hi << 32) | lo);
+            vals[i] = (int32_t)i;
+        }
+#pragma unroll
+        for (uint32_t b = 0; b < 4; ++b)
+            wave_hist_add(lh[b], (lo >> (8u * b)) & 255u, live);
+    }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t b = 0; b < 4; ++b)
+        if (lh[b][t] != 0u)
+            atomicAdd(&depth_hist[b * 256u + t], lh[b][t]);
+}
+
+// One workgroup of 1024 lanes.  corner_grid -> per-tile counts (2-D inclusive prefix sum) -> tile_offsets
+// [n_tiles + 1] (exclusive prefix in row-major tile order, the count in the last entry), counts[0] = the count the
+// launches behind this one use (0 when it exceeds the capacity), counts[1] = the true count, the two digit histograms
+// of the pair sort; the corner grid is left zeroed for the next call.
+__global__ void __launch_bounds__(1024) tile_table_kernel(uint32_t tile_width, uint32_t tile_height,
+                                                           int32_t* __restrict__ corner_grid,
+                                                           uint32_t* __restrict__ tile_counts /*[n_tiles] scratch*/,
+                                                           int64_t capacity, uint32_t bits0, uint32_t bits1,
+                                                           int32_t* __restrict__ tile_offsets,
+                                                           uint32_t* __restrict__ pair_hist /*[2][256]*/,
+                                                           int64_t* __restrict__ counts, int64_t* host_slot,
+                                                           uint32_t* __restrict__ error) {
+    __shared__ unsigned long long wave_tot[16];
+    __shared__ uint32_t h0[256], h1[256];
+    const uint32_t t = threadIdx.x, lane = t & 63u, wv = t >> 6;
+    const uint32_t gw = tile_width + 1u, gh = tile_height + 1u, n_tiles = tile_width * tile_height;
+    // rows (a wave per row, 64 entries at a time), then columns (a lane per column; the loads of a column do not
+    // depend on its running sum, so they are in flight together)
+    for (uint32_t y = wv; y < gh; y += 16u) {
+        int32_t carry = 0;
+        for (uint32_t xb = 0; xb < gw; xb += 64u) {
+            const uint32_t x = xb + lane;
+            int32_t v = x < gw ? corner_grid[y * gw + x] : 0;
+#pragma unroll
+            for (uint32_t off = 1; off < 64; off <<= 1) {
+                const int32_t up = __shfl_up(v, off, 64);
+                if (lane >= off)
+                    v += up;
+            }
+            v += carry;
+            if (x < gw)
+                corner_grid[y * gw + x] = v;
+            carry = __shfl(v, 63, 64);
+        }
+    }
+    __syncthreads();
+    for (uint32_t x = t; x < tile_width; x += 1024u) {
+        int32_t run = 0;
+#pragma unroll 8
+        for (uint32_t y = 0; y < tile_height; ++y) {
+            run += corner_grid[y * gw + x];
+            tile_counts[y * tile_width + x] = (uint32_t)run;
+        }
+    }
+    __syncthreads();
+    for (uint32_t i = t; i < gw * gh; i += 1024u)
+        corner_grid[i] = 0;
+    if (t < 256) {
+        h0[t] = 0;
+        h1[t] = 0;
+    }
+    // exclusive prefix over the tiles: a contiguous chunk per lane
+    const uint32_t chunk = (n_tiles + 1023u) / 1024u;
+    const uint32_t first = min(t * chunk, n_tiles), last = min(first + chunk, n_tiles);
+    unsigned long long mine = 0;
+    for (uint32_t i = first; i < last; ++i)
+        mine += tile_counts[i];
+    unsigned long long incl = mine;
+#pragma unroll
+    for (uint32_t off = 1; off < 64; off <<= 1) {
+        const unsigned long long up = __shfl_up(incl, off, 64);
+        if (lane >= off)
+            incl += up;
+    }
+    if (lane == 63)
+        wave_tot[wv] = incl;
+    __syncthreads();
+    unsigned long long before = 0, total = 0;
+#pragma unroll
+    for (uint32_t k = 0; k < 16; ++k) {
+        before += k < wv ? wave_tot[k] : 0ull;
+        total += wave_tot[k];
+    }
+    const bool fits = total <= (unsigned long long)capacity && total <= (unsigned long long)kLbValueMask;
+    const uint32_t mask0 = (1u << bits0) - 1u, mask1 = bits1 ? (1u << bits1) - 1u : 0u;
+    unsigned long long run = before + incl - mine;
+    for (uint32_t i = first; i < last; ++i) {
+        const uint32_t c = tile_counts[i];
+        tile_offsets[i] = fits ? (int32_t)run : 0;
+        run += c;
+        if (fits && c) {
+            atomicAdd(&h0[i & mask0], c);
+            atomicAdd(&h1[(i >> bits0) & mask1], c);
+        }
+    }
+    __syncthreads();
+    if (t < 256) {
+        pair_hist[t] = h0[t];
+        pair_hist[256u + t] = h1[t];
+    }
+    if (t == 0) {
+        tile_offsets[n_tiles] = fits ? (int32_t)total : 0;
+        counts[0] = fits ? (int64_t)total : 0;
+        counts[1] = (int64_t)total;
+        if (!fits)
+            atomicOr(error, 1u);
+        if (host_slot != nullptr) // pinned host memory: one 8-byte store at system scope
+            __hip_atomic_store(host_slot, (int64_t)total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+}
+
+// (16-bit tile index, id) pairs in depth order from the sorted keys.  Workgroup `place` (ticket order) covers sorted
+// positions [256 place, 256 place + 256); its first output position is the pair count of all positions in front of
+// it, obtained by a chained look-back over the workgroups' counts.  Inside the workgroup a wave flattens the runs of
+// its 64 positions so that consecutive lanes write consecutive pairs.
+__global__ void __launch_bounds__(256) tile_emit_chained_kernel(
+    uint32_t n, const int64_t* __restrict__ sorted_keys, const int32_t* __restrict__ order, uint32_t tile_width,
+    const int64_t* __restrict__ counts, uint32_t* __restrict__ status, uint32_t* __restrict__ ticket,
+    uint16_t* __restrict__ tile_keys, int32_t* __restrict__ ids, uint32_t* __restrict__ clear_status,
+    uint32_t clear_rows, uint32_t* __restrict__ clear_ticket, uint32_t* __restrict__ clear_depth_hist,
+    uint32_t* __restrict__ error) {
+    __shared__ uint32_t s_incl[4][64], s_xy[4][64], s_w[4][64], s_idx[4][64];
+    __shared__ uint32_t wave_total[4];
+    __shared__ uint32_t place_s, base_s;
+    const uint32_t t = threadIdx.x, lane = t & 63u, wv = t >> 6;
+    const uint32_t place = lb_take_ticket(ticket, &place_s);
+    for (uint32_t row = place; row < clear_rows; row += gridDim.x)
+        clear_status[(size_t)row * 256u + t] = 0u;
+    if (place == 0) {
+#pragma unroll
+        for (uint32_t k = 0; k < 4; ++k)
+            clear_depth_hist[k * 256u + t] = 0u;
+        if (t == 0)
+            *clear_ticket = 0u;
+    }
+    const uint32_t limit = (uint32_t)counts[0]; // 0 when the pairs do not fit: nothing is written
+    const uint32_t i = place * 256u + t;
+    uint32_t x0 = 0, y0 = 0, w = 0, cnt = 0, idx = 0;
+    if (i < n) {
+        const uint32_t hi = (uint32_t)((uint64_t)sorted_keys[i] >> 32);
+        x0 = hi & 255u, y0 = (hi >> 8) & 255u;
+        w = ((hi >> 16) & 255u) - x0;
+        cnt = ((hi >> 24) - y0) * w;
+        idx = (uint32_t)order[i];
+    }
+    uint32_t incl = cnt;
+#pragma unroll
+    for (uint32_t off = 1; off < 64; off <<= 1) {
+        const uint32_t up = (uint32_t)__shfl_up((int)incl, off, 64);
+        if (lane >= off)
+            incl += up;
+    }
+    s_incl[wv][lane] = incl;
+    s_xy[wv][lane] = x0 | (y0 << 16);
+    s_w[wv][lane] = w;
+    s_idx[wv][lane] = idx;
+    if (lane == 63)
+        wave_total[wv] = incl;
+    __syncthreads();
+    const uint32_t block_total = wave_total[0] + wave_total[1] + wave_total[2] + wave_total[3];
+    if (t == 0) {
+        // values saturate at the 30-bit field: beyond it the count does not fit and `limit` is 0 anyway
+        lb_publish(status + place, place == 0 ? kLbPrefix : kLbAggregate, min(block_total, kLbValueMask));
+        uint32_t gave_up = 0;
+        const uint32_t before = lb_exclusive(status, place, 1u, 0u, &gave_up);
+        if (place != 0)
+            lb_publish(status + place, kLbPrefix, min(before + block_total, kLbValueMask));
+        if (gave_up)
+            atomicOr(error, 2u);
+        base_s = before;
+    }
+    __syncthreads();
+    uint32_t wave_base = base_s;
+#pragma unroll
+    for (uint32_t k = 0; k < 4; ++k)
+        wave_base += k < wv ? wave_total[k] : 0u;
+    const uint32_t total = wave_total[wv];
+    for (uint32_t k = lane; k < total; k += 64u) {
+        uint32_t lo = 0, hi = 63; // smallest l with incl[l] > k
+#pragma unroll
+        for (uint32_t step = 0; step < 6; ++step) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (s_incl[wv][mid] > k)
+                hi = mid;
+            else
+                lo = mid + 1;
+        }
+        const uint32_t l = lo;
+        const uint32_t local = k - (l ? s_incl[wv][l - 1] : 0u);
+        const uint32_t gw = s_w[wv][l], xy = s_xy[wv][l];
+        const uint32_t row = local / gw;
+        const uint32_t tile_id = ((xy >> 16) + row) * tile_width + ((xy & 0xffffu) + (local - row * gw));
+        const uint32_t pos = wave_base + k;
+        if (pos < limit) {
+            tile_keys[pos] = (uint16_t)tile_id;
+            ids[pos] = (int32_t)s_idx[wv][l];
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256) zero_words_kernel(size_t n, uint32_t* __restrict__ out) {
+    const size_t i = (size_t)blockIdx.x * 256u + threadIdx.x;
+    if (i < n)
+        out[i] = 0u;
+}
+
+} // namespace gsx
+
+using namespace gsx;
+
+namespace {
+struct ListsLayout {
+    size_t keys0, keys1, vals0, vals1;         // depth sort: i64 [N] x 2, i32 [N] x 2
+    size_t depth_hist, corner_grid, tile_counts, pair_hist, counts, error;
+    size_t dstatus0, dstatus1, estatus, pstatus0, pstatus1, tickets; // tickets: 5 words
+    size_t tkeys0, tkeys1, ids0, ids1;         // pairs: u16 [capacity] x 2, i32 [capacity] x 2
+    size_t total;
+    uint32_t drows, prows, ewords;
+};
+ListsLayout lists_layout(uint32_t N, int64_t capacity, uint32_t tw, uint32_t th) {
+    ListsLayout L;
+    size_t o = 0;
+    auto take = [&](size_t bytes) {
+        const size_t at = o;
+        o += align_up(bytes, 256);
+        return at;
+    };
+    L.drows = radix_chained_rows(N);
+    L.prows = radix_chained_rows(capacity);
+    L.ewords = cdiv(N, 256);
+    L.depth_hist = take(4 * 256 * 4);
+    L.corner_grid = take((size_t)(tw + 1) * (th + 1) * 4);
+    L.counts = take(16);
+    L.error = take(4);
+    L.tickets = take(5 * 4);
+    L.tile_counts = take((size_t)tw * th * 4);
+    L.pair_hist = take(2 * 256 * 4);
+    L.keys0 = take((size_t)N * 8);
+    L.keys1 = take((size_t)N * 8);
+    L.vals0 = take((size_t)N * 4);
+    L.vals1 = take((size_t)N * 4);
+    L.dstatus0 = take((size_t)L.drows * 1024);
+    L.dstatus1 = take((size_t)L.drows * 1024);
+    L.estatus = take((size_t)L.ewords * 4);
+    L.pstatus0 = take((size_t)L.prows * 1024);
+    L.pstatus1 = take((size_t)L.prows * 1024);
+    L.tkeys0 = take((size_t)capacity * 2);
+    L.tkeys1 = take((size_t)capacity * 2);
+    L.ids0 = take((size_t)capacity * 4);
+    L.ids1 = take((size_t)capacity * 4);
+    L.total = o;
+    return L;
+}
+int check_lists_args(const char* who, uint32_t N, int64_t capacity, uint32_t tw, uint32_t th) {
+    GSX_REQUIRE(tw >= 1 && th >= 1 && tw <= 255 && th <= 255, GSX_ERR_UNSUPPORTED,
+                "%s: a %u x %u tile grid (limit 255 x 255: the keys carry the tile rectangle in four bytes)", who, tw,
+                th);
+    GSX_REQUIRE(N >= 1 && N < (1u << kLbValueBits), GSX_ERR_OVERFLOW, "%s: N = %u (limit 2^30 - 1)", who, N);
+    GSX_REQUIRE(capacity >= 1 && capacity < (1ll << kLbValueBits), GSX_ERR_OVERFLOW,
+                "%s: capacity = %lld pairs (limit 2^30 - 1)", who, (long long)capacity);
+    return GSX_OK;
+}
+} // namespace
+
+extern "C" size_t gsx_tile_lists_workspace_bytes(uint32_t N, int64_t capacity, uint32_t tile_width,
+                                                 uint32_t tile_height) {
+    if (N == 0 || capacity <= 0 || tile_width == 0 || tile_height == 0)
+        return 256;
+    return lists_layout(N, capacity, tile_width, tile_height).total;
+}
+
+// the head of the workspace (digit histograms, corner grid, counts, error word, tickets) must be zero before the
+// first call; every call leaves it as the next one needs it
+extern "C" int gsx_tile_lists_init(uint32_t N, int64_t capacity, uint32_t tile_width, uint32_t tile_height,
+                                   void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_lists_args("tile_lists_init", N, capacity, tile_width, tile_height);
+    if (rc != GSX_OK)
+        return rc;
+    const ListsLayout L = lists_layout(N, capacity, tile_width, tile_height);
+    GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 && workspace_bytes >= L.total,
+                GSX_ERR_WORKSPACE, "tile_lists_init: workspace needs %zu bytes, 256-byte aligned", L.total);
+    const size_t words = L.tile_counts / 4;
+    hipLaunchKernelGGL(zero_words_kernel, dim3(cdiv(words, 256)), dim3(256), 0, (hipStream_t)stream, words,
+                       (uint32_t*)workspace);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+extern "C" int gsx_tile_lists(uint32_t N, const float* means2d, const int32_t* radii, const float* depths,
+                              uint32_t tile_size, uint32_t tile_width, uint32_t tile_height, int64_t capacity,
+                              void* workspace, size_t workspace_bytes, int32_t* flatten_ids, int32_t* tile_offsets,
+                              int64_t* n_isects_host_slot, void* stream) {
+    int rc = check_lists_args("tile_lists", N, capacity, tile_width, tile_height);
+    if (rc != GSX_OK)
+        return rc;
+    GSX_REQUIRE(means2d && radii && depths && flatten_ids && tile_offsets, GSX_ERR_INVALID_ARGUMENT,
+                "tile_lists: null tensor");
+    GSX_REQUIRE(tile_size > 0, GSX_ERR_INVALID_ARGUMENT, "tile_lists: tile_size is 0");
+    const ListsLayout L = lists_layout(N, capacity, tile_width, tile_height);
+    GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 && workspace_bytes >= L.total,
+                GSX_ERR_WORKSPACE, "tile_lists: workspace needs %zu bytes, 256-byte aligned", L.total);
+    int64_t* slot = nullptr;
+    if (n_isects_host_slot != nullptr) {
+        hipPointerAttribute_t attr;
+        const bool known = hipPointerGetAttributes(&attr, n_isects_host_slot) == hipSuccess;
+        if (!known)
+            (void)hipGetLastError();
+        GSX_REQUIRE(known && attr.type == hipMemoryTypeHost && attr.devicePointer != nullptr, GSX_ERR_INVALID_ARGUMENT,
+                    "tile_lists: n_isects_host_slot must be pinned host memory (hipHostMalloc)");
+        slot = (int64_t*)attr.devicePointer;
+    }
+    char* ws = (char*)workspace;
+    auto u32p = [&](size_t off) { return (uint32_t*)(ws + off); };
+    int64_t* keys[2] = {(int64_t*)(ws + L.keys0), (int64_t*)(ws + L.keys1)};
+    int32_t* vals[2] = {(int32_t*)(ws + L.vals0), (int32_t*)(ws + L.vals1)};
+    uint32_t* dstatus[2] = {u32p(L.dstatus0), u32p(L.dstatus1)};
+    uint32_t* pstatus[2] = {u32p(L.pstatus0), u32p(L.pstatus1)};
+    uint32_t* tickets = u32p(L.tickets); // [0], [1]: depth passes; [2]: emission; [3], [4]: pair passes
+    uint32_t* error = u32p(L.error);
+    int64_t* counts = (int64_t*)(ws + L.counts);
+    hipStream_t s = (hipStream_t)stream;
+
+    hipLaunchKernelGGL(depth_keys_kernel, dim3(cdiv(N, kKeysPerBlock)), dim3(256), 0, s, N, means2d, radii, depths,
+                       (float)tile_size, tile_width, tile_height, keys[0], vals[0], u32p(L.depth_hist),
+                       (int32_t*)(ws + L.corner_grid), dstatus[0], L.drows, tickets + 0, u32p(L.estatus), L.ewords,
+                       tickets + 2);
+    GSX_LAUNCH_CHECK();
+    // the tile table needs the corner grid only: it is queued first so that the count reaches the host early
+    const uint32_t tile_bits = gsx_n_bits(tile_width * tile_height);
+    const uint32_t passes = tile_bits > 8 ? 2u : 1u;
+    const uint32_t bits0 = passes == 2 ? (tile_bits + 1) / 2 : (tile_bits ? tile_bits : 1u);
+    const uint32_t bits1 = passes == 2 ? tile_bits - bits0 : 0u;
+    hipLaunchKernelGGL(tile_table_kernel, dim3(1), dim3(1024), 0, s, tile_width, tile_height,
+                       (int32_t*)(ws + L.corner_grid), u32p(L.tile_counts), capacity, bits0, bits1, tile_offsets,
+                       u32p(L.pair_hist), counts, slot, error);
+    GSX_LAUNCH_CHECK();
+    for (uint32_t pass = 0; pass < 4; ++pass) { // depth bits, a byte per pass; the result ends in keys[0] / vals[0]
+        const uint32_t in = pass & 1u, out = in ^ 1u;
+        RadixChainArgs a;
+        a.n_dev = nullptr, a.status = dstatus[in], a.ticket = tickets + in, a.error = error;
+        a.clear_status = pass < 3 ? dstatus[out] : nullptr, a.clear_rows = L.drows;
+        a.clear_ticket = pass < 3 ? tickets + out : nullptr;
+        if ((rc = radix_chained_pass_i64(N, keys[in], vals[in], keys[out], vals[out], 8u * pass, 8u,
+                                         u32p(L.depth_hist) + 256u * pass, a, s)) != GSX_OK)
+            return rc;
+    }
+    uint16_t* tkeys[2] = {(uint16_t*)(ws + L.tkeys0), (uint16_t*)(ws + L.tkeys1)};
+    int32_t* ids[2] = {(int32_t*)(ws + L.ids0), (int32_t*)(ws + L.ids1)};
+    hipLaunchKernelGGL(tile_emit_chained_kernel, dim3(L.ewords), dim3(256), 0, s, N, keys[0], vals[0], tile_width,
+                       counts, u32p(L.estatus), tickets + 2, tkeys[0], ids[0], pstatus[0], L.prows, tickets + 3,
+                       u32p(L.depth_hist), error);
+    GSX_LAUNCH_CHECK();
+    for (uint32_t pass = 0; pass < passes; ++pass) {
+        const bool last = pass + 1 == passes;
+        RadixChainArgs a;
+        a.n_dev = counts, a.status = pstatus[pass], a.ticket = tickets + 3 + pass, a.error = error;
+        a.clear_status = last ? nullptr : pstatus[1], a.clear_rows = L.prows;
+        a.clear_ticket = last ? nullptr : tickets + 4;
+        if ((rc = radix_chained_pass_u16((uint32_t)capacity, tkeys[pass], ids[pass], tkeys[pass ^ 1u],
+                                         last ? flatten_ids : ids[pass ^ 1u], pass ? bits0 : 0u, pass ? bits1 : bits0,
+                                         u32p(L.pair_hist) + 256u * pass, a, !last, s)) != GSX_OK)
+            return rc;
+    }
+    return GSX_OK;
+}
+
+// where a caller can read the outcome of the last call on the device: counts[0] = pairs in the lists (0 if they did
+// not fit), counts[1] = pairs there are; error: bit 0 = capacity exceeded, bit 1 = a look-back gave up
+extern "C" const int64_t* gsx_tile_lists_counts(uint32_t N, int64_t capacity, uint32_t tile_width,
+                                                uint32_t tile_height, const void* workspace) {
+    if (workspace == nullptr || N == 0 || capacity <= 0)
+        return nullptr;
+    return (const int64_t*)((const char*)workspace + lists_layout(N, capacity, tile_width, tile_height).counts);
+}
+extern "C" uint32_t* gsx_tile_lists_error(uint32_t N, int64_t capacity, uint32_t tile_width, uint32_t tile_height,
+                                          void* workspace) {
+    if (workspace == nullptr || N == 0 || capacity <= 0)
+        return nullptr;
+    return (uint32_t*)((char*)workspace + lists_layout(N, capacity, tile_width, tile_height).error);
+}
