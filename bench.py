@@ -107,6 +107,8 @@ def main():
                     help="hand the step two camera tensors in turn (same pose): the forward pass then cannot reuse "
                          "the previous step's tile costs, as in a training loop that changes camera every step")
     ap.add_argument("--no-tile-order", action="store_true", help="rasterize the tiles in index order")
+    ap.add_argument("--host-count", action="store_true",
+                    help="fetch the pair count to the host in every step (default: it stays on the device)")
     ap.add_argument("--cpu-threads", type=int, default=0, help="threads for the CPU baseline (0 = all)")
     ap.add_argument("--workload", choices=["gut", "fastgs"], default="gut",
                     help="gut: the training step of the metric (default); fastgs: forward + backward of the "
@@ -144,7 +146,7 @@ def main():
     use_ssim = args.config != 1  # configuration 1 is L1 only
     ts = TrainStep(sc, dev, use_ssim=use_ssim, fused_update=not args.separate_update,
                    fused_loss=not args.separate_update, overlap=not args.no_overlap,
-                   one_front_pass=args.one_front_pass)
+                   one_front_pass=args.one_front_pass, device_count=not args.host_count)
     ts.order_tiles = not args.no_tile_order
     setup_s = time.time() - t0
 

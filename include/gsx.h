@@ -476,6 +476,14 @@ typedef struct gsx_update_args {
     /* regularisation gradients folded in: scaling grad += reg_scaling * exp(scaling_raw), opacity grad +=
      * reg_opacity * s (1 - s); reg_* = weight / element count as in gsx_*_l1_regularization (0 = off) */
     float reg_scaling, reg_opacity;
+    /* nullable, device u32 [2] (e.g. gsx_tile_lists_error): while hold[0] != 0 the call changes no parameter or
+     * moment (it still clears the accumulator rows) and adds 1 to hold[1] - a step whose tile lists did not fit its
+     * buffers must not reach the optimiser */
+    uint32_t* hold;
+    /* nullable, device f32 [3] = {bias_correction1_rcp, bias_correction2_sqrt_rcp, skip_shN as 0 / 1}: read when the
+     * kernel runs, in place of the three fields above (a launch replayed from a HIP graph keeps its by-value
+     * arguments; the step's scalars change every iteration) */
+    const float* step_scalars;
 } gsx_update_args;
 GSX_API int gsx_backward_update_fused(const gsx_update_args* args_host, void* stream);
 

@@ -68,7 +68,8 @@ class UpdateArgs(ctypes.Structure):
                 [(n, c_f) for n in ("lr_means", "lr_sh0", "lr_shN", "lr_scaling", "lr_rotation", "lr_opacity",
                                     "beta1", "beta2", "eps", "bias_correction1_rcp",
                                     "bias_correction2_sqrt_rcp")] +
-                [("skip_shN", ctypes.c_int32), ("reg_scaling", c_f), ("reg_opacity", c_f)])
+                [("skip_shN", ctypes.c_int32), ("reg_scaling", c_f), ("reg_opacity", c_f), ("hold", c_p),
+                 ("step_scalars", c_p)])
 
 
 class GsxError(RuntimeError):

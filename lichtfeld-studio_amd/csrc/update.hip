@@ -28,6 +28,8 @@ struct UpdateArgs {
     float beta1, beta2, eps, bc1_rcp, bc2_sqrt_rcp;
     int32_t skip_shN;
     float reg_scaling, reg_opacity;
+    uint32_t* hold;             // nullable: [0] != 0 -> change nothing and count the call in [1]
+    const float* step_scalars;  // nullable: device [3] = bc1_rcp, bc2_sqrt_rcp, skip_shN (0 / 1), read at run time
 };
 
 // new first / second moment of one element (the first two lines of adam_one)
@@ -53,9 +55,27 @@ __device__ __forceinline__ void adam_row(float* __restrict__ P, float* __restric
 }
 
 template <bool LDS16>
-__global__ void __launch_bounds__(256) backward_update_kernel(const UpdateArgs a) {
+__global__ void __launch_bounds__(256) backward_update_kernel(const UpdateArgs a_in) {
     __shared__ float4 lds[LDS16 ? 4 * 32 * kShLdsF4 : 1];
     const uint32_t e = blockIdx.x * 256u + threadIdx.x;
+    UpdateArgs a = a_in;
+    if (a.step_scalars != nullptr) { // a replayed launch takes the step's scalars from memory
+        a.bc1_rcp = a.step_scalars[0];
+        a.bc2_sqrt_rcp = a.step_scalars[1];
+        a.skip_shN = a.step_scalars[2] != 0.f ? 1 : 0;
+    }
+    if (a.hold != nullptr && a.hold[0] != 0u) {
+        // the step's render is not valid (its tile lists did not fit): parameters and moments stay as they are; the
+        // accumulator rows are cleared all the same
+        if (e == 0)
+            atomicAdd(&a.hold[1], 1u);
+        if (e < a.N) {
+            float4* row = reinterpret_cast<float4*>(a.acc + (size_t)e * 16);
+            const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+            row[0] = z, row[1] = z, row[2] = z, row[3] = z;
+        }
+        return;
+    }
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     float4* wave_lds = lds + (LDS16 ? wave * 32 * kShLdsF4 : 0);
     const bool in = e < a.N;
@@ -248,6 +268,7 @@ extern "C" int gsx_backward_update_fused(const gsx_update_args* args, void* stre
     a.bc1_rcp = args->bias_correction1_rcp, a.bc2_sqrt_rcp = args->bias_correction2_sqrt_rcp;
     a.skip_shN = args->skip_shN;
     a.reg_scaling = args->reg_scaling, a.reg_opacity = args->reg_opacity;
+    a.hold = args->hold, a.step_scalars = args->step_scalars;
     const bool lds16 = a.K == 16 && ((((uintptr_t)a.shs) | ((uintptr_t)a.m_shs) | ((uintptr_t)a.v_shs)) & 15u) == 0;
     const dim3 grid(cdiv(a.N, 256)), block(256);
     if (lds16)

@@ -28,11 +28,19 @@ def _p(t):
 class TrainStep:
     def __init__(self, scene, device="cuda:0", lrs=None, lambda_dssim=0.2, betas=(0.9, 0.999), eps=1e-15,
                  scene_scale=1.0, sh_degree=None, use_ssim=True, fused_update=False, fused_loss=False,
-                 scale_reg=0.0, opacity_reg=0.0, overlap=False, tile_pairs=True, one_front_pass=False):
+                 scale_reg=0.0, opacity_reg=0.0, overlap=False, tile_pairs=True, one_front_pass=False,
+                 device_count=False):
         self.dev = torch.device(device)
         self.lib = lib()
         self.one_front_pass = one_front_pass  # activations + projection + SH colours + records as one launch
         self.tile_pairs = tile_pairs  # sort (u16 tile index, id) pairs where the tile grid allows it
+        # True (needs fused_update and a grid of at most 255 x 255 tiles): after the first step, which sizes the
+        # buffers, the tile lists come from gsx_tile_lists and the pair count stays on the device - no host wait
+        # inside a step; a step whose pairs outgrow the buffers renders nothing, is held back from the optimiser
+        # and is made up for by _check_capacity at the start of the next one
+        self.device_count = bool(device_count and fused_update)
+        self.lists_ws, self._lists_dims, self._lists_active = None, None, False
+        self.steps_held = 0
         f = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(self.dev)
         self.N = scene.means.shape[0]
         self.K = 1 + scene.shN.shape[1]
@@ -67,7 +75,7 @@ class TrainStep:
         self.cap = 0
         self.compact = False
         self.img_shape = None
-        self.n_isects = 0
+        self._n_host = 0
         self.bg = torch.zeros((1, 3), dtype=torch.float32, device=self.dev)  # trainer.cpp:383-384
         # A second stream (default priority) for work that is independent of the launch-latency-bound sort chain:
         # the SH / record pass runs beside the depth-ordered count, the loss reduction beside the backward rasterizer.
@@ -111,8 +119,57 @@ class TrainStep:
         else:
             self.count_done.synchronize()
             n = slot.value
-        self.n_isects = n
+        self._n_host = n
         return n
+
+    @property
+    def n_isects(self):
+        """pairs of the last forward pass (with the count on the device: the last value that has landed in the pinned
+        slot - synchronise first to be sure it is the last pass's)"""
+        return self._n_slot.value if self._lists_active else self._n_host
+
+    # -- tile lists with the count on the device -----------------------------------------------------
+    def _lists_ready(self):
+        dims = (self.N, self.cap, self.tw, self.th)
+        if self._lists_dims == dims:
+            return
+        a = (c_u32(self.N), c_i64(self.cap), c_u32(self.tw), c_u32(self.th))
+        nbytes = self.lib.gsx_tile_lists_workspace_bytes(*a)
+        self.lists_ws = torch.empty(nbytes, dtype=torch.uint8, device=self.dev)
+        check(self.lib.gsx_tile_lists_init(*a, _p(self.lists_ws), c_sz(nbytes), self._stream()))
+        base = self.lists_ws.data_ptr()
+        self._lists_error = self.lib.gsx_tile_lists_error(*a, c_p(base))  # device address of u32 [2]
+        self._lists_error_at = self._lists_error - base
+        self.flat_out = torch.empty(self.cap, dtype=torch.int32, device=self.dev)
+        self._lists_dims = dims
+
+    def lists_error(self):
+        """(error bits, optimiser calls held back) of the tile lists so far; synchronises"""
+        if self.lists_ws is None:
+            return 0, 0
+        torch.cuda.synchronize(self.dev)
+        w = self.lists_ws[self._lists_error_at:self._lists_error_at + 8].cpu().numpy().view(np.uint32)
+        return int(w[0]), int(w[1])
+
+    def _check_capacity(self):
+        """Start of a step with the count on the device: the last count that reached the host decides whether the
+        buffers grow.  More pairs than the buffers held means that step (and every step queued behind it) rendered
+        nothing and was held back from the optimiser: they are counted back out of the iteration counters."""
+        if not self._lists_active:
+            return
+        n = self._n_slot.value
+        if n <= int(self.cap * 0.9):
+            return
+        if n > self.cap:
+            bits, held = self.lists_error()
+            self.steps_held += held
+            self.step_count -= held
+            self.iteration -= held
+        else:
+            torch.cuda.synchronize(self.dev)  # kernels in flight still use the buffers that are about to go
+        self.cap = 0
+        self._ensure_isect_capacity(max(n, self._n_slot.value))
+        self._lists_ready()
 
     def _ensure_isect_capacity(self, n):
         if n <= self.cap and self.cap:
@@ -135,7 +192,8 @@ class TrainStep:
         compact = bool(self.tile_pairs and self.lib.gsx_intersect_tile_pairs_fit(c_u32(self.tw), c_u32(self.th)))
         if compact != self.compact:  # the key buffers change their element type
             self.compact, self.cap = compact, 0
-        self.offsets = e(1, self.th, self.tw, dt=torch.int32)
+        self.offsets_full = e(self.th * self.tw + 1, dt=torch.int32)  # the last entry: room for the pair count
+        self.offsets = self.offsets_full[:-1].view(1, self.th, self.tw)
         self.tile_order = e(self.th * self.tw, dt=torch.int32)  # the rasterizers' tile visiting order
         self.tile_walk = e(self.th * self.tw, dt=torch.int32)   # per tile: entries up to its last contributor
         self.have_walk, self._walk_cam = False, None
@@ -229,6 +287,63 @@ class TrainStep:
         side_sh = self.side is not None and not self.one_front_pass
         if side_sh:
             self.ev_fork.record(torch.cuda.current_stream(self.dev))
+
+        def sh_pass():
+            if self.one_front_pass:
+                return
+            if not side_sh:
+                self._run("sh_colors_records_from_world", lb.gsx_sh_colors_records_from_world, *sh_args, s)
+                return
+            self.side.wait_event(self.ev_fork)  # recorded after the activation / projection pass
+            with torch.cuda.stream(self.side):
+                self._run("sh_colors_records_from_world", lb.gsx_sh_colors_records_from_world, *sh_args,
+                          self._stream())
+                self.ev_join.record(self.side)
+
+        self._lists_active = self.device_count and self.compact and self.cap > 0
+        if self._lists_active:
+            # every launch sized by the buffers, the count read on the device: nothing waits for the host
+            self._lists_ready()
+            self._run("tile_lists", lb.gsx_tile_lists, c_u32(N), _p(J["means2d"]), _p(J["radii"]), _p(J["depths"]),
+                      c_u32(16), c_u32(self.tw), c_u32(self.th), c_i64(self.cap), _p(self.lists_ws),
+                      c_sz(self.lists_ws.numel()), _p(self.flat_out), _p(self.offsets_full),
+                      c_p(self.n_isects_pinned.data_ptr()), s)
+            sh_pass()
+            self.flatten_ids = self.flat_out
+            n = -1  # GSX_COUNT_IN_OFFSETS
+        else:
+            n = self._host_counted_lists(sh_pass)
+        self._n_arg = n
+        # Dearest tiles first: both rasterizers then end with cheap tiles instead of a long tail.  What a tile costs is
+        # how far its pixels go into the list, which the forward pass itself reports; the forward pass therefore
+        # uses the order of the previous step (the first one: by list length), the backward pass this step's.
+        order = c_p(None)
+        if self.order_tiles:
+            # the previous pass's costs say something about this one only for the same camera (the same tensors)
+            cam_key = (viewmat.data_ptr(), K.data_ptr(), W, H)
+            if not self.have_walk or cam_key != self._walk_cam:
+                self._run("tile_order", lb.gsx_tile_order, c_i64(n), _p(self.offsets), c_p(None), c_u32(self.tw),
+                          c_u32(self.th), _p(self.tile_order), s)
+            order = _p(self.tile_order)
+        self._tile_order_arg = order
+        if side_sh:
+            torch.cuda.current_stream(self.dev).wait_event(self.ev_join)  # colours and records are ready
+        self._run("rasterize_to_pixels_from_world_3dgs_fwd", lb.gsx_rasterize_records_fwd, c_i64(n),
+                  _p(self.records), c_p(None), c_u32(3), _p(self.bg), c_p(None), c_u32(W), c_u32(H), _p(viewmat),
+                  _p(K), _p(self.offsets), _p(self.flatten_ids), order, _p(self.tile_walk) if self.order_tiles else
+                  c_p(None), _p(self.render), _p(self.alpha), _p(self.last_ids), s)
+        if self.order_tiles:
+            # the order for the backward pass (and for the next forward pass from this camera): queued by the loss
+            # pass on the second stream, or by whoever needs it first
+            self._order_due = (c_i64(n), c_p(None), _p(self.tile_walk), c_u32(self.tw), c_u32(self.th),
+                               _p(self.tile_order))
+            self.have_walk, self._walk_cam = True, (viewmat.data_ptr(), K.data_ptr(), W, H)
+        return self.render
+
+    def _host_counted_lists(self, sh_pass):
+        """intersect_tile (depth-ordered count, emission) + pair sort + intersect_offset with the pair count crossing
+        to the host, which sizes the buffers and the launches by it; returns the count"""
+        lb, s, N, J = self.lib, self._stream(), self.N, self.proj
         # Tile counts in depth order; the total comes back through pinned memory without blocking, and the SH /
         # record passes (which do not need it) run while the host waits for it.
         self._run("intersect_tile_count_ordered", lb.gsx_intersect_tile_count_ordered, c_u32(N), _p(J["means2d"]),
@@ -236,16 +351,7 @@ class TrainStep:
                   _p(self.tiles_per_gauss), _p(self.cum), _p(self.ws_count), c_sz(self.ws_count.numel()),
                   c_p(self.n_isects_pinned.data_ptr()), c_i(0), s)
         self.count_done.record(torch.cuda.current_stream(self.dev))
-        if self.one_front_pass:
-            pass
-        elif not side_sh:
-            self._run("sh_colors_records_from_world", lb.gsx_sh_colors_records_from_world, *sh_args, s)
-        else:
-            self.side.wait_event(self.ev_fork)  # recorded after the activation / projection pass
-            with torch.cuda.stream(self.side):
-                self._run("sh_colors_records_from_world", lb.gsx_sh_colors_records_from_world, *sh_args,
-                          self._stream())
-                self.ev_join.record(self.side)
+        sh_pass()
         # The emission does not need the total, only room for it: with buffers from an earlier step it is queued now
         # (writes bounded to the buffers) and the host's wake-up from the wait below hides behind it.
         if self.compact:  # pairs in depth order sort on their tile bits only: 16-bit tile indices as keys
@@ -286,31 +392,7 @@ class TrainStep:
         else:
             self._run("intersect_offset", lb.gsx_intersect_offset, c_i64(n), _p(self.keys[self.sel]), c_u32(1),
                       c_u32(self.tw), c_u32(self.th), _p(self.offsets), s)
-        # Dearest tiles first: both rasterizers then end with cheap tiles instead of a long tail.  What a tile costs is
-        # how far its pixels go into the list, which the forward pass itself reports; the forward pass therefore
-        # uses the order of the previous step (the first one: by list length), the backward pass this step's.
-        order = c_p(None)
-        if self.order_tiles:
-            # the previous pass's costs say something about this one only for the same camera (the same tensors)
-            cam_key = (viewmat.data_ptr(), K.data_ptr(), W, H)
-            if not self.have_walk or cam_key != self._walk_cam:
-                self._run("tile_order", lb.gsx_tile_order, c_i64(n), _p(self.offsets), c_p(None), c_u32(self.tw),
-                          c_u32(self.th), _p(self.tile_order), s)
-            order = _p(self.tile_order)
-        self._tile_order_arg = order
-        if side_sh:
-            torch.cuda.current_stream(self.dev).wait_event(self.ev_join)  # colours and records are ready
-        self._run("rasterize_to_pixels_from_world_3dgs_fwd", lb.gsx_rasterize_records_fwd, c_i64(n),
-                  _p(self.records), c_p(None), c_u32(3), _p(self.bg), c_p(None), c_u32(W), c_u32(H), _p(viewmat),
-                  _p(K), _p(self.offsets), _p(self.flatten_ids), order, _p(self.tile_walk) if self.order_tiles else
-                  c_p(None), _p(self.render), _p(self.alpha), _p(self.last_ids), s)
-        if self.order_tiles:
-            # the order for the backward pass (and for the next forward pass from this camera): queued by the loss
-            # pass on the second stream, or by whoever needs it first
-            self._order_due = (c_i64(n), c_p(None), _p(self.tile_walk), c_u32(self.tw), c_u32(self.th),
-                               _p(self.tile_order))
-            self.have_walk, self._walk_cam = True, (viewmat.data_ptr(), K.data_ptr(), W, H)
-        return self.render
+        return n
 
     @property
     def isect_ids(self):
@@ -319,8 +401,12 @@ class TrainStep:
         if not self.compact:
             return self.keys[self.sel]
         n = self.n_isects
-        tiles = self.keys[self.sel][:n].to(torch.int64) & 0xFFFF
-        depth = self.proj["depths"].view(torch.int32).reshape(-1)[self.vals[self.sel][:n].long()]
+        if self._lists_active:  # no sorted keys either: an entry's tile is the list it lies in
+            bounds = self.offsets_full[1:].to(torch.int64).contiguous()
+            tiles = torch.searchsorted(bounds, torch.arange(n, dtype=torch.int64, device=self.dev), right=True)
+        else:
+            tiles = self.keys[self.sel][:n].to(torch.int64) & 0xFFFF
+        depth = self.proj["depths"].view(torch.int32).reshape(-1)[self.flatten_ids[:n].long()]
         return (tiles << 32) | (depth.to(torch.int64) & 0xFFFFFFFF)
 
     # -- loss ---------------------------------------------------------------------------------------
@@ -380,7 +466,7 @@ class TrainStep:
         ws, wsn = _p(self.ws_bwd), c_sz(self.ws_bwd.numel())
         self._join_tile_order()
         self._run("rasterize_bwd_accumulate", lb.gsx_rasterize_bwd_accumulate,
-                  c_u32(1), c_u32(N), c_i64(self.n_isects), _p(self.records), c_p(None), c_u32(3), _p(self.bg),
+                  c_u32(1), c_u32(N), c_i64(self._n_arg), _p(self.records), c_p(None), c_u32(3), _p(self.bg),
                   c_p(None), c_u32(W), c_u32(H), c_u32(16),
                   _p(self.viewmat), _p(self.Kmat), _p(self.offsets), _p(self.flatten_ids), self._tile_order_arg,
                   _p(self.alpha), _p(self.last_ids), _p(self.v_render), _p(self.v_alpha), ws, wsn, s)
@@ -436,7 +522,8 @@ class TrainStep:
                 self.lrs["rotation"], self.lrs["opacity"], b1, b2, self.eps, bc1, bc2, skip,
                 # weight / element count in float32, as the separate regularisation kernels form it
                 float(np.float32(self.scale_reg) / np.float32(3 * self.N)) if self.scale_reg > 0.0 else 0.0,
-                float(np.float32(self.opacity_reg) / np.float32(self.N)) if self.opacity_reg > 0.0 else 0.0)
+                float(np.float32(self.opacity_reg) / np.float32(self.N)) if self.opacity_reg > 0.0 else 0.0,
+                self._lists_error if self._lists_active else None, None)
             self._run("backward_update_fused", self.lib.gsx_backward_update_fused, ctypes.byref(a), self._stream())
             return
         names = ["means", "shs", "scaling", "rotation", "opacity"]
@@ -511,6 +598,7 @@ class TrainStep:
     loss_pending = False
 
     def step(self, viewmat, K, W, H, gt_chw):
+        self._check_capacity()
         self.iteration += 1
         self.forward(viewmat, K, W, H)
         self.loss_forward(gt_chw)

@@ -24,7 +24,8 @@ def stage_properties(ts):
     ids = N(ts.isect_ids[:n])
     flat = N(ts.flatten_ids[:n])
     off = N(ts.offsets).reshape(-1)
-    tiles_per_gauss = N(ts.tiles_per_gauss)
+    # with the pair count on the device no per-Gaussian tile counts exist: how often the lists name each Gaussian
+    tiles_per_gauss = np.bincount(flat, minlength=ts.N) if ts._lists_active else N(ts.tiles_per_gauss)
     radii = N(ts.proj["radii"])[0]
     assert int(tiles_per_gauss.sum(dtype=np.int64)) == n, "sum of tile counts = number of intersections"
     assert (tiles_per_gauss[(radii <= 0).any(-1)] == 0).all(), "culled Gaussians touch no tile"
@@ -120,8 +121,8 @@ def test_config3_full_size_on_the_benchmarked_path(gsx, orc, cuda):
     cam = sc.cameras[0]
     gt_d = target_image(gsx, sc, cam, cuda)
     gt = N(gt_d)[0]
-    ts = TrainStep(sc, cuda, fused_update=True, fused_loss=True, overlap=True)
-    assert ts.order_tiles and ts.fused_loss and ts.side is not None
+    ts = TrainStep(sc, cuda, fused_update=True, fused_loss=True, overlap=True, device_count=True)
+    assert ts.order_tiles and ts.fused_loss and ts.side is not None and ts.device_count
     ref = OracleTrainStep(sc)
     vm, Km = T(cam.viewmat[None], cuda), T(cam.K[None], cuda)
     prev = None
@@ -131,6 +132,7 @@ def test_config3_full_size_on_the_benchmarked_path(gsx, orc, cuda):
         ts.step(vm, Km, cam.width, cam.height, gt_d)
         torch.cuda.synchronize()
         truth = step_with_truth(ref, cam.viewmat, cam.K, cam.width, cam.height, gt)
+        assert ts._lists_active == (it == 1), "from the second iteration on the pair count stays on the device"
         stage_properties(ts)
         check_forward_bit_exact(ts, ref, min_isects=1_000_000)
         check_loss(ts, ref)
@@ -140,6 +142,7 @@ def test_config3_full_size_on_the_benchmarked_path(gsx, orc, cuda):
             ts.params[k].copy_(T(ref.params[k], cuda))
             ts.exp_avg[k].copy_(T(ref.exp_avg[k], cuda))
             ts.exp_avg_sq[k].copy_(T(ref.exp_avg_sq[k], cuda))
+    assert ts.lists_error() == (0, 0)
 
 
 def test_config4_step_relocation_noise(gsx, orc, cuda):

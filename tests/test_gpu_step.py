@@ -236,6 +236,90 @@ def test_speculative_emission_and_overlap_change_nothing(gsx, cuda):
             assert torch.equal(a.params[k], b.params[k]), k
 
 
+def test_pair_count_on_the_device_changes_nothing(gsx, cuda):
+    """the step whose tile lists come from gsx_tile_lists (count on the device, no host wait) against the step that
+    fetches the count: keys, order, ranges, image and loss bit for bit in every iteration; parameters bit for bit
+    when both tails are given the same accumulators"""
+    from lichtfeld_studio_amd.trainer import TrainStep
+    sc = gsx.scenes.config(3, 20_000)
+    sc.scaling_raw += 1.2
+    cam = gsx.scenes.orbit_camera(0.7, 4.0, 309, 205, 287.0)
+    W, H = cam.width, cam.height
+    vm = torch.from_numpy(cam.viewmat[None].copy()).to(cuda)
+    Km = torch.from_numpy(cam.K[None].copy()).to(cuda)
+    gt = torch.rand((1, 3, H, W), generator=torch.Generator().manual_seed(3)).to(cuda)
+    a = TrainStep(sc, cuda, fused_update=True, fused_loss=True, overlap=False)
+    b = TrainStep(sc, cuda, fused_update=True, fused_loss=True, overlap=True, device_count=True)
+    for it in range(4):
+        a.forward(vm, Km, W, H)
+        b._check_capacity()
+        b.forward(vm, Km, W, H)
+        torch.cuda.synchronize()
+        assert b._lists_active == (it > 0), "the first iteration sizes the buffers with the count on the host"
+        assert a.n_isects == b.n_isects and a.n_isects > 50_000
+        assert torch.equal(a.isect_ids[:a.n_isects], b.isect_ids[:b.n_isects])
+        assert torch.equal(a.flatten_ids[:a.n_isects], b.flatten_ids[:b.n_isects])
+        assert torch.equal(a.offsets, b.offsets) and int(b.offsets_full[-1]) == a.n_isects or it == 0
+        assert torch.equal(a.render, b.render) and torch.equal(a.last_ids, b.last_ids)
+        for ts in (a, b):
+            ts.iteration += 1
+            ts.loss_forward(gt)
+            ts.backward()
+        b.ws_bwd.copy_(a.ws_bwd)  # the accumulators are atomic sums: give both tails the same ones
+        a.adam()
+        b.adam()
+        if b.loss_pending:
+            torch.cuda.current_stream(cuda).wait_event(b.ev_loss_join)
+            b.loss_pending = False
+        torch.cuda.synchronize()
+        assert torch.equal(a.loss_out, b.loss_out)
+        for k in a.params:
+            assert torch.equal(a.params[k], b.params[k]), k
+    assert b.lists_error() == (0, 0)
+
+
+def test_pairs_outgrowing_the_buffers_hold_the_step_back(gsx, cuda):
+    """count on the device, and a camera that suddenly sees several times the pairs the buffers hold: that step
+    renders nothing, the optimiser leaves parameters and moments untouched, and the next step starts with larger
+    buffers and with the held step counted back out - after which the state equals the one of a run whose buffers
+    were large enough from the start"""
+    from lichtfeld_studio_amd.trainer import TrainStep
+    sc = gsx.scenes.config(3, 20_000)
+    sc.scaling_raw += 1.2
+    far = gsx.scenes.orbit_camera(0.7, 9.0, 309, 205, 287.0)
+    near = gsx.scenes.orbit_camera(0.7, 3.0, 309, 205, 287.0)
+    W, H = far.width, far.height
+    t = lambda a: torch.from_numpy(a[None].copy()).to(cuda)
+    cams = [(t(far.viewmat), t(far.K)), (t(near.viewmat), t(near.K))]
+    gt = torch.rand((1, 3, H, W), generator=torch.Generator().manual_seed(3)).to(cuda)
+    a = TrainStep(sc, cuda, fused_update=True, fused_loss=True, overlap=True, device_count=True)
+    b = TrainStep(sc, cuda, fused_update=True, fused_loss=True, overlap=True)
+    a.step(*cams[0], W, H, gt)
+    b.step(*cams[0], W, H, gt)
+    torch.cuda.synchronize()
+    n_far, cap_far = a.n_isects, a.cap
+    before = {k: v.clone() for k, v in a.params.items()}
+    m_before = {k: v.clone() for k, v in a.exp_avg.items()}
+    a.step(*cams[1], W, H, gt)  # does not fit
+    torch.cuda.synchronize()
+    assert a.n_isects > cap_far > n_far, (a.n_isects, cap_far, n_far)
+    assert a.lists_error() == (1, 1)
+    assert float(a.alpha.max()) == 0.0, "a step that does not fit renders nothing"
+    for k in before:
+        assert torch.equal(a.params[k], before[k]) and torch.equal(a.exp_avg[k], m_before[k]), k
+    assert a.step_count == 2
+    a.step(*cams[1], W, H, gt)  # grows the buffers, forgets the held step, runs it again
+    b.step(*cams[1], W, H, gt)
+    torch.cuda.synchronize()
+    assert a.steps_held == 1 and a.step_count == b.step_count == 2 and a.iteration == b.iteration == 2
+    assert a.cap >= a.n_isects == b.n_isects and a.lists_error() == (0, 0)
+    assert torch.equal(a.render, b.render)
+    for k in a.params:  # the two runs add up their gradients in different (atomic) orders
+        assert torch.allclose(a.params[k], b.params[k], rtol=0, atol=2.2 * a.lrs["opacity"]), k
+        close = (a.params[k] - b.params[k]).abs() <= 1e-6 + 1e-3 * a.lrs["opacity"]
+        assert close.float().mean() > 0.999, k
+
+
 @pytest.mark.parametrize("n,degree,cfg", [(1, 3, 3), (300, 0, 3), (70_001, 3, 3), (40_000, 2, 3), (5_000, 0, 1)])
 def test_one_front_pass(gsx, cuda, n, degree, cfg):
     """activations + projection + SH colours + records as one launch: every output equals, bit for bit, what the
