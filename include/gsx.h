@@ -213,6 +213,9 @@ GSX_API int gsx_intersect_tile_pairs_offset(int64_t n_isects, const uint16_t* ti
  * If the pairs exceed `capacity` (or 2^30 - 1) every list is left empty (tile_offsets all zero), bit 0 of the error
  * word is set and the true count is still reported: grow the buffers and run the step again.  Nothing is read or
  * written out of bounds in that case.  Bit 1 of the error word: a look-back's bounded wait ran out (results invalid).
+ * side_stream: nullable; a second stream of the same device (default priority) on which the tile table is formed
+ * while the depth sort runs on `stream` (forked and joined with events inside the call; all results are ordered on
+ * `stream` when the call returns).
  * The workspace's head must be zeroed once by gsx_tile_lists_init; every call leaves it ready for the next one.  Calls
  * that share a workspace must not overlap. */
 #define GSX_COUNT_IN_OFFSETS (-1ll)
@@ -223,7 +226,7 @@ GSX_API int gsx_tile_lists_init(uint32_t N, int64_t capacity, uint32_t tile_widt
 GSX_API int gsx_tile_lists(uint32_t N, const float* means2d, const int32_t* radii, const float* depths,
                            uint32_t tile_size, uint32_t tile_width, uint32_t tile_height, int64_t capacity,
                            void* workspace, size_t workspace_bytes, int32_t* flatten_ids, int32_t* tile_offsets,
-                           int64_t* n_isects_host_slot, void* stream);
+                           int64_t* n_isects_host_slot, void* stream, void* side_stream);
 /* device addresses inside the workspace: counts i64 [2] = {pairs in the lists (0 if they did not fit), pairs there
  * are}; error u32 (bits above; sticky until the caller clears it or calls gsx_tile_lists_init) */
 GSX_API const int64_t* gsx_tile_lists_counts(uint32_t N, int64_t capacity, uint32_t tile_width,

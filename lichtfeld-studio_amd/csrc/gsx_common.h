@@ -64,14 +64,14 @@ int radix_sort_pairs_32_bits(int64_t n, int64_t* keys0, int32_t* vals0, int64_t*
 
 // radix_sort.hip: one stable 1..8-bit radix pass as ONE launch (chained look-back between the workgroups).  The
 // caller provides digit_total[256] = how many of the pairs carry each digit, a status table of
-// radix_chained_rows(n_max) x 256 empty (zero) words and a zero ticket word; the launch can clear the table and ticket
-// of the pass that follows it.  n_dev (nullable): the number of pairs is min(*n_dev, n_max), read on the device.
+// radix_chained_rows(n_max) x 256 empty (zero) words; the launch can clear the table of the pass that follows it.  n_dev (nullable): the number of pairs is min(*n_dev, n_max), read on the device.
 // Limit: n_max < 2^30.  error: device word, bit 1 is set if a look-back's bounded wait ran out.
 struct RadixChainArgs {
     const int64_t* n_dev;
-    uint32_t *status, *ticket, *clear_status;
+    uint32_t *status, *clear_status;
     uint32_t clear_rows;
-    uint32_t *clear_ticket, *error;
+    uint32_t* error;
+    uint32_t total_replicas, total_stride; // digit_total is the sum of this many tables, total_stride words apart
 };
 uint32_t radix_chained_rows(int64_t n_max);
 int radix_chained_pass_i64(uint32_t n_max, const int64_t* kin, const int32_t* vin, int64_t* kout, int32_t* vout,

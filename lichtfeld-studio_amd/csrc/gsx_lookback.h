@@ -5,11 +5,13 @@
 // Value and state share one 32-bit word (2 state bits + 30 value bits), written and read with relaxed device-scope
 // atomics, so no fence is needed: a word is either empty or complete.
 //
-// Forward progress: workgroups take their place p from a ticket counter when they start running, so every
-// predecessor of a running workgroup is itself running or finished, and a running wave is never starved by a
-// spinning one (the look-back only waits for work that is already resident).  The wait is bounded all the same: after
-// kLbSpinLimit empty reads a lane gives up, reports it, and returns the partial sum it has - which only ever
-// under-counts, so positions derived from it stay inside the output.
+// Forward progress: a workgroup's place p is its index in a one-dimensional grid.  The dispatcher of each XCD starts
+// the workgroups it is given in ascending index order, so the unfinished workgroup with the smallest index never
+// waits for anyone and is either running or next in line on an XCD whose running workgroups all have smaller
+// indices - i.e. are finished: it always gets to run.  (A ticket counter would make the order explicit, but one
+// returning atomic on a single address per workgroup costs ~20 ns each, serialised: 80 us for 4000 workgroups.)
+// The wait is bounded all the same: after kLbSpinLimit empty reads a lane gives up, reports it, and returns the
+// partial sum it has - which only ever under-counts, so positions derived from it stay inside the output.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -18,42 +20,97 @@ namespace gsx {
 
 static constexpr uint32_t kLbEmpty = 0u, kLbAggregate = 1u, kLbPrefix = 2u;
 static constexpr uint32_t kLbValueBits = 30u, kLbValueMask = (1u << kLbValueBits) - 1u;
-static constexpr uint32_t kLbSpinLimit = 1u << 22;
+static constexpr uint32_t kLbSpinLimit = 1u << 20;
 
 __device__ __forceinline__ void lb_publish(uint32_t* slot, uint32_t state, uint32_t value) {
     __hip_atomic_store(slot, (state << kLbValueBits) | value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Sum of the values of places p-1, p-2, ... down to and including the first one in state PREFIX.  Place q's word is
-// status[q * stride + column].  *gave_up is set (never cleared) when the bounded wait ran out.
+// Whether a waiting lane should give up: the bounded wait ran out here, or somewhere else already (then every lane
+// still waiting ends too, so a launch that cannot make progress ends after about one wait, not one per workgroup).
+__device__ __forceinline__ bool lb_give_up(uint32_t spins, uint32_t* error) {
+    if (spins > kLbSpinLimit ||
+        ((spins & 255u) == 0 && (__hip_atomic_load(error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & 2u) != 0)) {
+        atomicOr(error, 2u);
+        return true;
+    }
+    return false;
+}
+
+// Sum of the values of places p-1, p-2, ... down to and including the first one in state PREFIX, for one column of a
+// table with `stride` words per place (place q's word is status[q * stride + column]); every lane walks its own
+// column.  Eight predecessors are requested at a time: a status word that another XCD wrote comes from memory, not
+// from this XCD's L2, and the walk is as long as the prefixes have not caught up with the aggregates.
+// When the bounded wait runs out, bit 1 of *error is set and the partial sum returned.
 __device__ __forceinline__ uint32_t lb_exclusive(const uint32_t* status, uint32_t p, uint32_t stride,
-                                                 uint32_t column, uint32_t* gave_up) {
-    uint32_t sum = 0;
-    for (int64_t q = (int64_t)p - 1; q >= 0; --q) {
-        const uint32_t* slot = status + (size_t)q * stride + column;
-        uint32_t word = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        uint32_t spins = 0;
-        while ((word >> kLbValueBits) == kLbEmpty) {
-            if (++spins > kLbSpinLimit) {
-                *gave_up = 1u;
-                return sum;
+                                                 uint32_t column, uint32_t* error) {
+    constexpr int kWindow = 8;
+    uint32_t sum = 0, spins = 0;
+    int64_t q = (int64_t)p - 1;
+    while (q >= 0) {
+        uint32_t word[kWindow];
+#pragma unroll
+        for (int j = 0; j < kWindow; ++j)
+            word[j] = q - j >= 0 ? __hip_atomic_load(status + (size_t)(q - j) * stride + column, __ATOMIC_RELAXED,
+                                                     __HIP_MEMORY_SCOPE_AGENT)
+                                 : (kLbPrefix << kLbValueBits);
+        int used = 0;
+        bool done = false;
+#pragma unroll
+        for (int j = 0; j < kWindow; ++j) {
+            const uint32_t state = word[j] >> kLbValueBits;
+            if (!done && used == j && state != kLbEmpty) {
+                sum += word[j] & kLbValueMask;
+                ++used;
+                done = state == kLbPrefix;
             }
-            __builtin_amdgcn_s_sleep(1);
-            word = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        sum += word & kLbValueMask;
-        if ((word >> kLbValueBits) == kLbPrefix)
+        if (done)
             break;
+        q -= used;
+        if (used == 0) {
+            if (lb_give_up(++spins, error))
+                break;
+            __builtin_amdgcn_s_sleep(1);
+        }
     }
     return sum;
 }
 
-// the place of this workgroup in the chain (one ticket per workgroup; all lanes get the value)
-__device__ __forceinline__ uint32_t lb_take_ticket(uint32_t* ticket, uint32_t* lds_slot) {
-    if (threadIdx.x == 0)
-        *lds_slot = atomicAdd(ticket, 1u);
-    __syncthreads();
-    return *lds_slot;
+// The same sum for a table with one word per place, formed by a whole wave (all 64 lanes must call; all receive the
+// sum): lane l looks at place p - 1 - l, so 64 predecessors are inspected per round.
+__device__ __forceinline__ uint32_t lb_exclusive_wave(const uint32_t* status, uint32_t p, uint32_t* error) {
+    const uint32_t lane = threadIdx.x & 63u;
+    uint32_t sum = 0, spins = 0;
+    int64_t top = (int64_t)p - 1; // the nearest place not yet added
+    while (top >= 0) {
+        const int64_t q = top - (int64_t)lane;
+        const uint32_t word = q >= 0 ? __hip_atomic_load(status + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                     : (kLbPrefix << kLbValueBits);
+        const uint32_t state = word >> kLbValueBits;
+        const uint64_t prefixes = __ballot(state == kLbPrefix), empties = __ballot(state == kLbEmpty);
+        const uint32_t first_prefix = prefixes ? (uint32_t)__builtin_ctzll(prefixes) : 64u;
+        const uint32_t first_empty = empties ? (uint32_t)__builtin_ctzll(empties) : 64u;
+        // the lanes in front of the first empty word can be added now; the walk ends at a prefix among them
+        const uint32_t usable = first_empty < first_prefix ? first_empty : (first_prefix < 64u ? first_prefix + 1u : 64u);
+        uint32_t v = lane < usable ? (word & kLbValueMask) : 0u;
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1)
+            v += (uint32_t)__shfl_xor((int)v, m, 64);
+        sum += v;
+        if (first_prefix < first_empty)
+            break;
+        top -= usable;
+        if (usable == 0) {
+            bool stop = false;
+            if (lane == 0)
+                stop = lb_give_up(++spins, error);
+            if (__ballot(stop))
+                break;
+            __builtin_amdgcn_s_sleep(1);
+        }
+    }
+    return sum;
 }
 
 } // namespace gsx

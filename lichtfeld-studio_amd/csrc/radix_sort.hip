@@ -111,17 +111,15 @@ __global__ void __launch_bounds__(256) radix_scan_kernel(uint32_t nblocks, uint3
 // ---- stable scatter -------------------------------------------------------------------------------
 // CHAINED = false: the positions come from the scanned histogram table of the two launches before (hist_scanned,
 // digit_total).  CHAINED = true: one launch per pass - digit_total holds the digit counts of the whole input (left by
-// whoever wrote the keys), every workgroup takes its place in the input from a ticket, publishes its 256 digit counts
-// and obtains the counts of the workgroups in front of it by a chained look-back (gsx_lookback.h); the number of
+// whoever wrote the keys), every workgroup publishes its 256 digit counts and obtains the counts of the workgroups in front of it by a chained look-back (gsx_lookback.h); the number of
 // pairs is read from device memory, and the launch also clears the status words the NEXT pass will use.
 struct RadixChain {
     const int64_t* n_dev;   // number of pairs (device); the launch covers min(*n_dev, n) pairs
     uint32_t* status;       // [workgroups][256], empty on entry
-    uint32_t* ticket;       // 0 on entry
     uint32_t* clear_status; // status words of the next pass (nullable): clear_rows rows are cleared by this launch
     uint32_t clear_rows;
-    uint32_t* clear_ticket; // nullable
     uint32_t* error;        // bit 1 is set when a look-back gave up
+    uint32_t total_replicas, total_stride; // digit_total = sum of this many tables, total_stride words apart
 };
 
 template <typename KeyT, uint32_t ITEMS, bool CHAINED, bool WRITE_KEYS>
@@ -137,7 +135,6 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const Ke
     __shared__ uint32_t wave_count[4][kRadix];
     __shared__ uint32_t to_global[kRadix]; // global position of a pair = to_global[digit] + its slot in the tile
     __shared__ uint32_t wsum[4], gsum[4];
-    __shared__ uint32_t place_s;
     // the match masks of the ranking phase and the reordered tile of the output phase share their bytes
     constexpr uint32_t kMatchBytes = 4 * kRadix * 8, kTileBytes = kTileN * (sizeof(KeyT) + 4);
     __shared__ __align__(16) unsigned char overlay[kMatchBytes > kTileBytes ? kMatchBytes : kTileBytes];
@@ -146,9 +143,31 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const Ke
     KeyT* s_keys = reinterpret_cast<KeyT*>(overlay + kTileN * 4);
     const uint32_t t = threadIdx.x;
     const uint32_t w = t >> 6, lane = t & 63u;
-    uint32_t place = blockIdx.x;
+    const uint32_t place = blockIdx.x;
+    const uint32_t tile_base = place * kTileN;
+    const uint32_t wave_base = tile_base + w * kWaveN;
+    const uint64_t lt_mask = (1ull << lane) - 1ull;
+    KeyT key[ITEMS];
+    int32_t val[ITEMS];
+    uint32_t rank[ITEMS]; // rank among the wave's pairs with the same digit
+    // requested before the count is known (chained: it comes from memory too); the buffers hold n entries at least
+#pragma unroll
+    for (uint32_t r = 0; r < ITEMS; ++r) {
+        const uint32_t idx = wave_base + r * 64u + lane;
+        const bool in_buffer = idx < n;
+        key[r] = in_buffer ? keys_in[idx] : 0;
+        val[r] = in_buffer ? vals_in[idx] : 0;
+    }
+    // the digit totals are requested now as well and first used after the ranking
+    uint32_t gtot = digit_total[t]; // pairs with digit t in the whole input
+    if (CHAINED && chain.total_replicas > 1) { // up to four tables: the loads are issued together
+        uint32_t part[3];
+#pragma unroll
+        for (uint32_t r = 0; r < 3; ++r)
+            part[r] = r + 1 < chain.total_replicas ? digit_total[(r + 1) * chain.total_stride + t] : 0u;
+        gtot += part[0] + part[1] + part[2];
+    }
     if (CHAINED) {
-        place = lb_take_ticket(chain.ticket, &place_s);
         if (chain.n_dev != nullptr) {
             const int64_t nd = *chain.n_dev;
             n = nd < (int64_t)n ? (uint32_t)(nd < 0 ? 0 : nd) : n;
@@ -157,8 +176,6 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const Ke
         if (chain.clear_status != nullptr)
             for (uint32_t row = place; row < chain.clear_rows; row += gridDim.x)
                 chain.clear_status[(size_t)row * kRadix + t] = 0u;
-        if (chain.clear_ticket != nullptr && place == 0 && t == 0)
-            *chain.clear_ticket = 0u;
         if ((uint64_t)place * kTileN >= n)
             return; // uniform over the workgroup; later places are empty too
     }
@@ -169,19 +186,6 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const Ke
     }
     __syncthreads();
 
-    const uint32_t tile_base = place * kTileN;
-    const uint32_t wave_base = tile_base + w * kWaveN;
-    const uint64_t lt_mask = (1ull << lane) - 1ull;
-    KeyT key[ITEMS];
-    int32_t val[ITEMS];
-    uint32_t rank[ITEMS]; // rank among the wave's pairs with the same digit
-#pragma unroll
-    for (uint32_t r = 0; r < ITEMS; ++r) {
-        const uint32_t idx = wave_base + r * 64u + lane;
-        const bool valid = idx < n;
-        key[r] = valid ? keys_in[idx] : 0;
-        val[r] = valid ? vals_in[idx] : 0;
-    }
 #pragma unroll
     for (uint32_t r = 0; r < ITEMS; ++r) {
         const uint32_t idx = wave_base + r * 64u + lane;
@@ -222,7 +226,6 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const Ke
         const uint32_t tot = c0 + c1 + c2 + c3;
         if (CHAINED) // the first place has nobody in front of it: its counts are a complete prefix already
             lb_publish(chain.status + (size_t)place * kRadix + t, place == 0 ? kLbPrefix : kLbAggregate, tot);
-        const uint32_t gtot = digit_total[t]; // pairs with digit t in the whole input
         const uint32_t incl = wave_inclusive_scan_u32(tot, lane);
         const uint32_t gincl = wave_inclusive_scan_u32(gtot, lane);
         if (lane == 63) {
@@ -244,12 +247,9 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const Ke
         wave_count[3][t] = start + c0 + c1 + c2;
         uint32_t earlier; // pairs with digit t in the workgroups in front of this one
         if (CHAINED) {
-            uint32_t gave_up = 0;
-            earlier = lb_exclusive(chain.status, place, kRadix, t, &gave_up);
+            earlier = lb_exclusive(chain.status, place, kRadix, t, chain.error);
             if (place != 0)
                 lb_publish(chain.status + (size_t)place * kRadix + t, kLbPrefix, earlier + tot);
-            if (gave_up)
-                atomicOr(chain.error, 2u);
         } else {
             earlier = hist_scanned[t * nblocks + blockIdx.x];
         }
@@ -403,7 +403,8 @@ int radix_sort_pairs_32_bits(int64_t n, int64_t* keys0, int32_t* vals0, int64_t*
 
 namespace gsx {
 // ---- one launch per pass (declared in gsx_common.h) ------------------------------------------------
-uint32_t radix_chained_rows(int64_t n_max) { return n_max <= 0 ? 1u : cdiv((uint64_t)n_max, 256u * sort_items(n_max)); }
+// chained passes always take 4096-pair tiles: the look-back walks as many places as there are workgroups with work
+uint32_t radix_chained_rows(int64_t n_max) { return n_max <= 0 ? 1u : cdiv((uint64_t)n_max, 256u * kItemsLarge); }
 
 namespace {
 template <typename KeyT>
@@ -412,13 +413,15 @@ int chained_pass(uint32_t n_max, const KeyT* kin, const int32_t* vin, KeyT* kout
     GSX_REQUIRE(n_max > 0 && n_max < (1u << kLbValueBits), GSX_ERR_OVERFLOW,
                 "chained radix pass: %u pairs (limit 2^30 - 1)", n_max);
     GSX_REQUIRE(bits >= 1 && bits <= kRadixBits && kin && vin && vout && (kout || !write_keys) && digit_total &&
-                    a.status && a.ticket && a.error,
+                    a.status && a.error,
                 GSX_ERR_INVALID_ARGUMENT, "chained radix pass: bad argument");
-    const uint32_t items = sort_items(n_max), rows = radix_chained_rows(n_max);
+    const uint32_t items = kItemsLarge, rows = radix_chained_rows(n_max);
     const uint32_t mask = (1u << bits) - 1u;
     RadixChain c;
-    c.n_dev = a.n_dev, c.status = a.status, c.ticket = a.ticket, c.clear_status = a.clear_status;
-    c.clear_rows = a.clear_rows, c.clear_ticket = a.clear_ticket, c.error = a.error;
+    c.n_dev = a.n_dev, c.status = a.status, c.clear_status = a.clear_status;
+    c.clear_rows = a.clear_rows, c.error = a.error;
+    GSX_REQUIRE(a.total_replicas <= 4, GSX_ERR_INVALID_ARGUMENT, "chained radix pass: at most 4 total tables");
+    c.total_replicas = a.total_replicas ? a.total_replicas : 1u, c.total_stride = a.total_stride;
     hipStream_t s = (hipStream_t)stream;
 #define GSX_CHAINED(IT, WK)                                                                                       \
     hipLaunchKernelGGL((radix_scatter_kernel<KeyT, IT, true, WK>), dim3(rows), dim3(256), 0, s, n_max, kin, vin, \

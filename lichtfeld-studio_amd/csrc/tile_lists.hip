@@ -5,13 +5,13 @@
 // flatten_ids (Gaussian ids, grouped by tile, depth order inside a tile, ties by id) and tile_offsets.  The result is
 // element for element the one of the separate operators; the organisation is not:
 //
-//  1. depth_keys_kernel      per Gaussian: tile rectangle, key (rectangle << 32 | depth bits), the four byte
-//                            histograms of the depth bits, and +1 / -1 at the rectangle's corners in a
-//                            (Th + 1) x (Tw + 1) grid;
-//  2. four chained radix passes (radix_sort.hip) order the N keys by depth, one launch each;
-//  3. tile_table_kernel      a 2-D prefix sum over the corner grid gives every tile's list length, hence
-//                            tile_offsets, the pair count, and the digit histograms of the pair sort - before a
-//                            single pair exists;
+//  1. depth_keys_kernel      keys (tile rectangle << 32 | depth bits) of the Gaussians that touch a tile, compacted
+//                            in index order (nine in ten Gaussians of a training view touch none);
+//                            depth_hist_kernel counts the bytes of their depth bits;
+//  2. four chained radix passes (radix_sort.hip) order the keys by depth, one launch each;
+//  3. tile_table_kernel      +1 / -1 at every rectangle's corners in a (Th + 1) x (Tw + 1) grid and a 2-D prefix
+//                            sum over it give every tile's list length, hence tile_offsets, the pair count, and the
+//                            digit histograms of the pair sort - before a single pair exists;
 //  4. tile_emit_chained_kernel  writes (16-bit tile index, id) pairs in depth order; a workgroup's position in the
 //                            output comes from a chained look-back over the workgroups' pair counts;
 //  5. two chained radix passes over the tile bits (the second one writes flatten_ids only).
@@ -20,16 +20,25 @@
 // exceeds the capacity, every tile's list is left EMPTY (tile_offsets all zero), bit 0 of the error word is set and
 // the true count is still reported, so that the caller can grow its buffers and run the step again; nothing is
 // written or read out of bounds.
+//
+// Atomics on addresses that many workgroups share are kept out of these kernels: on this GPU they cost far more
+// than the work around them (1.1 M additions onto 5 000 counters took 0.32 ms, one returning addition per workgroup
+// on a single word 20 ns each, serialised).  Counts meet through per-workgroup rows and replicas instead.
+#include <algorithm>
+#include <mutex>
+
 #include "gsx_common.h"
 #include "gsx_lookback.h"
 #include "gsx_tiles.h"
 
 namespace gsx {
 
-static constexpr uint32_t kKeysPerBlock = 1024; // depth_keys_kernel: 4 Gaussians per lane
+static constexpr uint32_t kKeysPerBlock = 1024; // depth_keys_kernel: 4 consecutive Gaussians per lane
+static constexpr uint32_t kTableBlocks = 32;    // tile_table_kernel: workgroups that share the corner counting
+static constexpr uint32_t kMaxLdsCells = 36 * 1024; // corner grids up to this many cells are counted in LDS
+static constexpr uint32_t kHistReplicas = 4;    // copies of the depth-byte histograms (fewer additions per address)
 
-// adds `count` to hist[digit] for every lane; one LDS atomic per wave when all its lanes share the digit (nine in
-// ten Gaussians of a training scene are culled and share the key 0xFFFFFFFF)
+// adds 1 to hist[digit] for every live lane; one LDS atomic per wave when all its live lanes share the digit
 __device__ __forceinline__ void wave_hist_add(uint32_t* hist, uint32_t digit, bool live) {
     const uint64_t lanes = __ballot(live);
     if (lanes == 0)
@@ -43,47 +52,94 @@ __device__ __forceinline__ void wave_hist_add(uint32_t* hist, uint32_t digit, bo
     }
 }
 
+// Keys of the Gaussians that touch a tile, in index order (a chained look-back over the workgroups' counts places
+// them).
 __global__ void __launch_bounds__(256) depth_keys_kernel(
     uint32_t n, const float* __restrict__ means2d, const int32_t* __restrict__ radii,
     const float* __restrict__ depths, float tile_size, uint32_t tile_width, uint32_t tile_height,
-    int64_t* __restrict__ keys, int32_t* __restrict__ vals, uint32_t* __restrict__ depth_hist /*[4][256], += */,
-    int32_t* __restrict__ corner_grid /*[(Th+1)(Tw+1)], += */, uint32_t* __restrict__ clear_status,
-    uint32_t clear_rows, uint32_t* __restrict__ clear_ticket, uint32_t* __restrict__ clear_emit_status,
-    uint32_t clear_emit_words, uint32_t* __restrict__ clear_emit_ticket) {
-    __shared__ uint32_t lh[4][256];
-    const uint32_t t = threadIdx.x;
-#pragma unroll
-    for (uint32_t k = 0; k < 4; ++k)
-        lh[k][t] = 0;
+    int64_t* __restrict__ keys, int32_t* __restrict__ vals, uint32_t* __restrict__ rects,
+    uint32_t* __restrict__ status /*[blocks]*/, int64_t* __restrict__ counts, uint32_t* __restrict__ error,
+    uint32_t* __restrict__ clear_status, uint32_t clear_rows, uint32_t* __restrict__ clear_emit_status,
+    uint32_t clear_emit_words) {
+    __shared__ uint32_t wave_total[4];
+    __shared__ uint32_t base_s;
+    const uint32_t t = threadIdx.x, lane = t & 63u, wv = t >> 6;
     // housekeeping for the launches behind this one
     for (uint32_t row = blockIdx.x; row < clear_rows; row += gridDim.x)
         clear_status[(size_t)row * 256u + t] = 0u;
     for (uint32_t wd = blockIdx.x * 256u + t; wd < clear_emit_words; wd += gridDim.x * 256u)
         clear_emit_status[wd] = 0u;
-    if (blockIdx.x == 0 && t == 0) {
-        *clear_ticket = 0u;
-        *clear_emit_ticket = 0u;
+    uint32_t lo[4], hi[4];
+    uint32_t mine = 0;
+#pragma unroll
+    for (uint32_t k = 0; k < 4; ++k) {
+        const uint32_t i = blockIdx.x * kKeysPerBlock + t * 4u + k;
+        lo[k] = 0, hi[k] = 0;
+        TileRect r;
+        if (i < n && tile_rect(means2d, radii, i, tile_size, tile_width, tile_height, &r) && r.y1 > r.y0 &&
+            r.x1 > r.x0) {
+            lo[k] = f2u(depths[i]);
+            hi[k] = r.x0 | (r.y0 << 8) | (r.x1 << 16) | (r.y1 << 24); // non-zero: x1 > x0 >= 0
+            ++mine;
+        }
+    }
+    uint32_t incl = mine;
+#pragma unroll
+    for (uint32_t off = 1; off < 64; off <<= 1) {
+        const uint32_t up = (uint32_t)__shfl_up((int)incl, off, 64);
+        if (lane >= off)
+            incl += up;
+    }
+    if (lane == 63)
+        wave_total[wv] = incl;
+    __syncthreads();
+    const uint32_t block_total = wave_total[0] + wave_total[1] + wave_total[2] + wave_total[3];
+    if (wv == 0) {
+        if (lane == 0)
+            lb_publish(status + blockIdx.x, blockIdx.x == 0 ? kLbPrefix : kLbAggregate, block_total);
+        const uint32_t before = lb_exclusive_wave(status, blockIdx.x, error);
+        if (lane == 0) {
+            if (blockIdx.x != 0)
+                lb_publish(status + blockIdx.x, kLbPrefix, before + block_total);
+            if (blockIdx.x == gridDim.x - 1)
+                counts[2] = (int64_t)(before + block_total); // Gaussians that touch a tile
+            base_s = before;
+        }
     }
     __syncthreads();
-    const uint32_t gw = tile_width + 1u;
+    uint32_t pos = base_s + incl - mine;
 #pragma unroll
-    for (uint32_t k = 0; k < kKeysPerBlock / 256; ++k) {
-        const uint32_t i = blockIdx.x * kKeysPerBlock + k * 256u + t;
-        const bool live = i < n;
-        uint32_t lo = 0xFFFFFFFFu, hi = 0;
-        if (live) {
-            TileRect r;
-            if (tile_rect(means2d, radii, i, tile_size, tile_width, tile_height, &r) && r.y1 > r.y0 && r.x1 > r.x0) {
-                lo = f2u(depths[i]);
-                hi = r.x0 | (r.y0 << 8) | (r.x1 << 16) | (r.y1 << 24);
-                atomicAdd(&corner_grid[r.y0 * gw + r.x0], 1);
-                atomicAdd(&corner_grid[r.y0 * gw + r.x1], -1);
-                atomicAdd(&corner_grid[r.y1 * gw + r.x0], -1);
-                atomicAdd(&corner_grid[r.y1 * gw + r.x1], 1);
-            }
-            keys[i] = (int64_t)(((uint64_t)hi << 32) | lo);
-            vals[i] = (int32_t)i;
+    for (uint32_t k = 0; k < 4; ++k)
+        pos += k < wv ? wave_total[k] : 0u;
+#pragma unroll
+    for (uint32_t k = 0; k < 4; ++k)
+        if (hi[k] != 0u) {
+            keys[pos] = (int64_t)(((uint64_t)hi[k] << 32) | lo[k]);
+            vals[pos] = (int32_t)(blockIdx.x * kKeysPerBlock + t * 4u + k);
+            rects[pos] = hi[k]; // a copy the sort does not move: the tile table is formed beside the sort
+            ++pos;
         }
+}
+
+// the four byte histograms of the compacted keys' depth bits: 4096 keys per workgroup, counted in LDS, added to
+// one of kHistReplicas copies of depth_hist [4][256] (n / 4096 / kHistReplicas additions per address)
+__global__ void __launch_bounds__(256) depth_hist_kernel(const int64_t* __restrict__ keys,
+                                                          const int64_t* __restrict__ counts,
+                                                          uint32_t* __restrict__ depth_hist) {
+    __shared__ uint32_t lh[4][256];
+    const uint32_t t = threadIdx.x;
+    const uint32_t n = (uint32_t)counts[2];
+    if (blockIdx.x * 4096u >= n)
+        return;
+#pragma unroll
+    for (uint32_t b = 0; b < 4; ++b)
+        lh[b][t] = 0;
+    __syncthreads();
+#pragma unroll 4
+    for (uint32_t k = 0; k < 16; ++k) {
+        const uint32_t i = blockIdx.x * 4096u + k * 256u + t;
+        const bool live = i < n;
+        const uint32_t lo = live ? (uint32_t)(uint64_t)keys[i] : 0u;
 #pragma unroll
         for (uint32_t b = 0; b < 4; ++b)
             wave_hist_add(lh[b], (lo >> (8u * b)) & 255u, live);
@@ -92,32 +148,107 @@ __global__ void __launch_bounds__(256) depth_keys_kernel(
 #pragma unroll
     for (uint32_t b = 0; b < 4; ++b)
         if (lh[b][t] != 0u)
-            atomicAdd(&depth_hist[b * 256u + t], lh[b][t]);
+            atomicAdd(&depth_hist[(blockIdx.x % kHistReplicas) * 1024u + b * 256u + t], lh[b][t]);
 }
 
-// One workgroup of 1024 lanes.  corner_grid -> per-tile counts (2-D inclusive prefix sum) -> tile_offsets
-// [n_tiles + 1] (exclusive prefix in row-major tile order, the count in the last entry), counts[0] = the count the
-// launches behind this one use (0 when it exceeds the capacity), counts[1] = the true count, the two digit histograms
-// of the pair sort; the corner grid is left zeroed for the next call.
-__global__ void __launch_bounds__(1024) tile_table_kernel(uint32_t tile_width, uint32_t tile_height,
-                                                           int32_t* __restrict__ corner_grid,
-                                                           uint32_t* __restrict__ tile_counts /*[n_tiles] scratch*/,
-                                                           int64_t capacity, uint32_t bits0, uint32_t bits1,
-                                                           int32_t* __restrict__ tile_offsets,
-                                                           uint32_t* __restrict__ pair_hist /*[2][256]*/,
-                                                           int64_t* __restrict__ counts, int64_t* host_slot,
-                                                           uint32_t* __restrict__ error) {
+// Up to kTableBlocks workgroups of 1024 lanes.  Every workgroup counts the rectangle corners (+1 / -1) of its share of the
+// keys into a private grid (LDS; a shared grid in global memory when the grid is too large for that) and leaves
+// it in `replicas`; the last one to finish adds the replicas up and turns the corner counts into per-tile counts
+// (2-D inclusive prefix sum), tile_offsets [n_tiles + 1] (exclusive prefix in row-major tile order, the count in the
+// last entry), counts[0] = the count the launches behind this one use (0 when it exceeds the capacity), counts[1] =
+// the true count, and the two digit histograms of the pair sort.
+template <bool in_lds>
+__global__ void __launch_bounds__(1024) tile_table_kernel(
+    const uint32_t* __restrict__ rects, uint32_t tile_width, uint32_t tile_height,
+    int32_t* __restrict__ replicas /*[kTableBlocks][cells], or [cells] zeroed when !in_lds*/,
+    uint32_t* __restrict__ done_counter, int64_t capacity,
+    uint32_t bits0, uint32_t bits1, int32_t* __restrict__ tile_offsets, uint32_t* __restrict__ pair_hist /*[2][256]*/,
+    int64_t* __restrict__ counts, int64_t* host_slot, uint32_t* __restrict__ error) {
+    extern __shared__ int32_t lds_grid[];
     __shared__ unsigned long long wave_tot[16];
     __shared__ uint32_t h0[256], h1[256];
+    __shared__ uint32_t last_s;
     const uint32_t t = threadIdx.x, lane = t & 63u, wv = t >> 6;
     const uint32_t gw = tile_width + 1u, gh = tile_height + 1u, n_tiles = tile_width * tile_height;
-    // rows (a wave per row, 64 entries at a time), then columns (a lane per column; the loads of a column do not
-    // depend on its running sum, so they are in flight together)
+    const uint32_t cells = gw * gh;
+    // the grid is named by its address space so that the LDS instance counts with LDS instructions
+#define GSX_GRID(i) (*(in_lds ? &lds_grid[i] : &replicas[i]))
+    if (in_lds) {
+        for (uint32_t i = t; i < cells; i += 1024u)
+            GSX_GRID(i) = 0;
+        __syncthreads();
+    }
+    const uint32_t n = (uint32_t)counts[2];
+    for (uint32_t i0 = blockIdx.x * 1024u + t; i0 < n; i0 += gridDim.x * 8192u) {
+        uint32_t hi8[8]; // eight keys requested together: every one comes from memory
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) {
+            const uint32_t i = i0 + j * gridDim.x * 1024u;
+            hi8[j] = i < n ? rects[i] : 0u;
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) {
+            const uint32_t hi = hi8[j];
+            if (hi == 0u)
+                continue; // no key: a rectangle has x1 > 0
+            const uint32_t x0 = hi & 255u, y0 = (hi >> 8) & 255u, x1 = (hi >> 16) & 255u, y1 = hi >> 24;
+            if (in_lds) {
+                atomicAdd(&lds_grid[y0 * gw + x0], 1);
+                atomicAdd(&lds_grid[y0 * gw + x1], -1);
+                atomicAdd(&lds_grid[y1 * gw + x0], -1);
+                atomicAdd(&lds_grid[y1 * gw + x1], 1);
+            } else {
+                atomicAdd(&replicas[y0 * gw + x0], 1);
+                atomicAdd(&replicas[y0 * gw + x1], -1);
+                atomicAdd(&replicas[y1 * gw + x0], -1);
+                atomicAdd(&replicas[y1 * gw + x1], 1);
+            }
+        }
+    }
+    __syncthreads();
+    // (a shared grid in global memory: its cells are only ever touched by device-scope atomics and, below, read by
+    // the last workgroup with device-scope loads)
+    // The replicas cross between workgroups (and XCDs) through device-scope stores and loads of the words
+    // themselves; a fence here would write back and invalidate this XCD's whole L2, dirty with the sort's keys.
+    if (in_lds && gridDim.x > 1)
+        for (uint32_t i = t; i < cells; i += 1024u)
+            __hip_atomic_store(&replicas[(size_t)blockIdx.x * cells + i], GSX_GRID(i), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads(); // every lane's stores have been acknowledged
+    if (t == 0)
+        last_s = atomicAdd(done_counter, 1u) == gridDim.x - 1u ? 1u : 0u;
+    __syncthreads();
+    if (!last_s)
+        return;
+    if (t == 0)
+        *done_counter = 0u;
+    if (in_lds && gridDim.x > 1) {
+        for (uint32_t i = t; i < cells; i += 1024u) {
+            int32_t sum = 0;
+            for (uint32_t r0 = 0; r0 < gridDim.x; r0 += 8u) { // eight loads in flight, then their sum
+                int32_t v[8];
+#pragma unroll
+                for (uint32_t j = 0; j < 8; ++j)
+                    v[j] = r0 + j < gridDim.x ? __hip_atomic_load(&replicas[(size_t)(r0 + j) * cells + i],
+                                                                  __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                              : 0;
+#pragma unroll
+                for (uint32_t j = 0; j < 8; ++j)
+                    sum += v[j];
+            }
+            GSX_GRID(i) = sum;
+        }
+        __syncthreads();
+    }
+    // rows (a wave per row, 64 entries at a time), then columns (a lane per column)
     for (uint32_t y = wv; y < gh; y += 16u) {
         int32_t carry = 0;
         for (uint32_t xb = 0; xb < gw; xb += 64u) {
             const uint32_t x = xb + lane;
-            int32_t v = x < gw ? corner_grid[y * gw + x] : 0;
+            int32_t v = 0;
+            if (x < gw)
+                v = in_lds ? lds_grid[y * gw + x]
+                           : __hip_atomic_load(&replicas[y * gw + x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
             for (uint32_t off = 1; off < 64; off <<= 1) {
                 const int32_t up = __shfl_up(v, off, 64);
@@ -126,22 +257,21 @@ __global__ void __launch_bounds__(1024) tile_table_kernel(uint32_t tile_width, u
             }
             v += carry;
             if (x < gw)
-                corner_grid[y * gw + x] = v;
+                GSX_GRID(y * gw + x) = v;
             carry = __shfl(v, 63, 64);
         }
     }
     __syncthreads();
-    for (uint32_t x = t; x < tile_width; x += 1024u) {
+    for (uint32_t x = t; x < tile_width; x += 1024u) { // in place: cell (y, x) becomes the length of tile (y, x)'s list
         int32_t run = 0;
 #pragma unroll 8
         for (uint32_t y = 0; y < tile_height; ++y) {
-            run += corner_grid[y * gw + x];
-            tile_counts[y * tile_width + x] = (uint32_t)run;
+            run += GSX_GRID(y * gw + x);
+            GSX_GRID(y * gw + x) = run;
         }
     }
     __syncthreads();
-    for (uint32_t i = t; i < gw * gh; i += 1024u)
-        corner_grid[i] = 0;
+    auto tile_count = [&](uint32_t i) { return (uint32_t)GSX_GRID((i / tile_width) * gw + i % tile_width); };
     if (t < 256) {
         h0[t] = 0;
         h1[t] = 0;
@@ -151,7 +281,7 @@ __global__ void __launch_bounds__(1024) tile_table_kernel(uint32_t tile_width, u
     const uint32_t first = min(t * chunk, n_tiles), last = min(first + chunk, n_tiles);
     unsigned long long mine = 0;
     for (uint32_t i = first; i < last; ++i)
-        mine += tile_counts[i];
+        mine += tile_count(i);
     unsigned long long incl = mine;
 #pragma unroll
     for (uint32_t off = 1; off < 64; off <<= 1) {
@@ -172,7 +302,7 @@ __global__ void __launch_bounds__(1024) tile_table_kernel(uint32_t tile_width, u
     const uint32_t mask0 = (1u << bits0) - 1u, mask1 = bits1 ? (1u << bits1) - 1u : 0u;
     unsigned long long run = before + incl - mine;
     for (uint32_t i = first; i < last; ++i) {
-        const uint32_t c = tile_counts[i];
+        const uint32_t c = tile_count(i);
         tile_offsets[i] = fits ? (int32_t)run : 0;
         run += c;
         if (fits && c) {
@@ -181,6 +311,9 @@ __global__ void __launch_bounds__(1024) tile_table_kernel(uint32_t tile_width, u
         }
     }
     __syncthreads();
+    if (!in_lds) // the shared grid in global memory is left zeroed for the next call
+        for (uint32_t i = t; i < cells; i += 1024u)
+            GSX_GRID(i) = 0;
     if (t < 256) {
         pair_hist[t] = h0[t];
         pair_hist[256u + t] = h1[t];
@@ -195,32 +328,36 @@ __global__ void __launch_bounds__(1024) tile_table_kernel(uint32_t tile_width, u
             __hip_atomic_store(host_slot, (int64_t)total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
 }
+#undef GSX_GRID
 
-// (16-bit tile index, id) pairs in depth order from the sorted keys.  Workgroup `place` (ticket order) covers sorted
-// positions [256 place, 256 place + 256); its first output position is the pair count of all positions in front of
-// it, obtained by a chained look-back over the workgroups' counts.  Inside the workgroup a wave flattens the runs of
-// its 64 positions so that consecutive lanes write consecutive pairs.
+// (16-bit tile index, id) pairs in depth order from the sorted keys.  Workgroup p covers sorted positions
+// [256 p, 256 p + 256); its first output position is the pair count of all positions in front of it, obtained by a
+// chained look-back over the workgroups' counts.  Inside the workgroup a wave flattens the runs of its 64 positions so
+// that consecutive lanes write consecutive pairs.
 __global__ void __launch_bounds__(256) tile_emit_chained_kernel(
-    uint32_t n, const int64_t* __restrict__ sorted_keys, const int32_t* __restrict__ order, uint32_t tile_width,
-    const int64_t* __restrict__ counts, uint32_t* __restrict__ status, uint32_t* __restrict__ ticket,
-    uint16_t* __restrict__ tile_keys, int32_t* __restrict__ ids, uint32_t* __restrict__ clear_status,
-    uint32_t clear_rows, uint32_t* __restrict__ clear_ticket, uint32_t* __restrict__ clear_depth_hist,
+    const int64_t* __restrict__ sorted_keys, const int32_t* __restrict__ order, uint32_t tile_width,
+    const int64_t* __restrict__ counts, uint32_t* __restrict__ status, uint16_t* __restrict__ tile_keys,
+    int32_t* __restrict__ ids, uint32_t* __restrict__ clear_status, uint32_t clear_rows,
+    uint32_t* __restrict__ clear_key_status, uint32_t clear_key_words, uint32_t* __restrict__ clear_depth_hist,
     uint32_t* __restrict__ error) {
     __shared__ uint32_t s_incl[4][64], s_xy[4][64], s_w[4][64], s_idx[4][64];
     __shared__ uint32_t wave_total[4];
-    __shared__ uint32_t place_s, base_s;
+    __shared__ uint32_t base_s;
     const uint32_t t = threadIdx.x, lane = t & 63u, wv = t >> 6;
-    const uint32_t place = lb_take_ticket(ticket, &place_s);
+    const uint32_t place = blockIdx.x;
     for (uint32_t row = place; row < clear_rows; row += gridDim.x)
         clear_status[(size_t)row * 256u + t] = 0u;
-    if (place == 0) {
+    for (uint32_t wd = place * 256u + t; wd < clear_key_words; wd += gridDim.x * 256u)
+        clear_key_status[wd] = 0u;
+    if (place < kHistReplicas) {
 #pragma unroll
         for (uint32_t k = 0; k < 4; ++k)
-            clear_depth_hist[k * 256u + t] = 0u;
-        if (t == 0)
-            *clear_ticket = 0u;
+            clear_depth_hist[place * 1024u + k * 256u + t] = 0u;
     }
     const uint32_t limit = (uint32_t)counts[0]; // 0 when the pairs do not fit: nothing is written
+    const uint32_t n = (uint32_t)counts[2];     // Gaussians that touch a tile
+    if (place * 256u >= n || limit == 0)
+        return; // nobody behind this workgroup needs its (empty) contribution
     const uint32_t i = place * 256u + t;
     uint32_t x0 = 0, y0 = 0, w = 0, cnt = 0, idx = 0;
     if (i < n) {
@@ -245,16 +382,15 @@ __global__ void __launch_bounds__(256) tile_emit_chained_kernel(
         wave_total[wv] = incl;
     __syncthreads();
     const uint32_t block_total = wave_total[0] + wave_total[1] + wave_total[2] + wave_total[3];
-    if (t == 0) {
-        // values saturate at the 30-bit field: beyond it the count does not fit and `limit` is 0 anyway
-        lb_publish(status + place, place == 0 ? kLbPrefix : kLbAggregate, min(block_total, kLbValueMask));
-        uint32_t gave_up = 0;
-        const uint32_t before = lb_exclusive(status, place, 1u, 0u, &gave_up);
-        if (place != 0)
-            lb_publish(status + place, kLbPrefix, min(before + block_total, kLbValueMask));
-        if (gave_up)
-            atomicOr(error, 2u);
-        base_s = before;
+    if (wv == 0) {
+        if (lane == 0)
+            lb_publish(status + place, place == 0 ? kLbPrefix : kLbAggregate, block_total);
+        const uint32_t before = lb_exclusive_wave(status, place, error);
+        if (lane == 0) {
+            if (place != 0)
+                lb_publish(status + place, kLbPrefix, before + block_total);
+            base_s = before;
+        }
     }
     __syncthreads();
     uint32_t wave_base = base_s;
@@ -297,12 +433,15 @@ using namespace gsx;
 
 namespace {
 struct ListsLayout {
-    size_t keys0, keys1, vals0, vals1;         // depth sort: i64 [N] x 2, i32 [N] x 2
-    size_t depth_hist, corner_grid, tile_counts, pair_hist, counts, error;
-    size_t dstatus0, dstatus1, estatus, pstatus0, pstatus1, tickets; // tickets: 5 words
-    size_t tkeys0, tkeys1, ids0, ids1;         // pairs: u16 [capacity] x 2, i32 [capacity] x 2
+    // zeroed by gsx_tile_lists_init and left zero by every call: the head of the workspace
+    size_t depth_hist, counts, error, done_counter, kstatus, shared_grid, head_end;
+    size_t keys0, keys1, vals0, vals1, rects; // depth sort: i64 [N] x 2, i32 [N] x 2; u32 [N]
+    size_t replicas, pair_hist;
+    size_t dstatus0, dstatus1, estatus, pstatus0, pstatus1;
+    size_t tkeys0, tkeys1, ids0, ids1; // pairs: u16 [capacity] x 2, i32 [capacity] x 2
     size_t total;
-    uint32_t drows, prows, ewords;
+    uint32_t kblocks, drows, prows, ewords, cells, table_blocks;
+    bool grid_in_lds;
 };
 ListsLayout lists_layout(uint32_t N, int64_t capacity, uint32_t tw, uint32_t th) {
     ListsLayout L;
@@ -312,20 +451,27 @@ ListsLayout lists_layout(uint32_t N, int64_t capacity, uint32_t tw, uint32_t th)
         o += align_up(bytes, 256);
         return at;
     };
+    L.kblocks = cdiv(N, kKeysPerBlock);
     L.drows = radix_chained_rows(N);
     L.prows = radix_chained_rows(capacity);
     L.ewords = cdiv(N, 256);
-    L.depth_hist = take(4 * 256 * 4);
-    L.corner_grid = take((size_t)(tw + 1) * (th + 1) * 4);
-    L.counts = take(16);
-    L.error = take(4);
-    L.tickets = take(5 * 4);
-    L.tile_counts = take((size_t)tw * th * 4);
+    L.cells = (tw + 1) * (th + 1);
+    L.grid_in_lds = L.cells <= kMaxLdsCells;
+    L.table_blocks = std::min(kTableBlocks, std::max(1u, N / (128u * 1024u)));
+    L.depth_hist = take((size_t)kHistReplicas * 4 * 256 * 4);
+    L.counts = take(3 * 8);
+    L.error = take(2 * 4);
+    L.done_counter = take(4);
+    L.kstatus = take((size_t)L.kblocks * 4);
+    L.shared_grid = take(L.grid_in_lds ? 0 : (size_t)L.cells * 4);
+    L.head_end = o;
+    L.replicas = take(L.grid_in_lds ? (size_t)kTableBlocks * L.cells * 4 : 0);
     L.pair_hist = take(2 * 256 * 4);
     L.keys0 = take((size_t)N * 8);
     L.keys1 = take((size_t)N * 8);
     L.vals0 = take((size_t)N * 4);
     L.vals1 = take((size_t)N * 4);
+    L.rects = take((size_t)N * 4);
     L.dstatus0 = take((size_t)L.drows * 1024);
     L.dstatus1 = take((size_t)L.drows * 1024);
     L.estatus = take((size_t)L.ewords * 4);
@@ -337,6 +483,26 @@ ListsLayout lists_layout(uint32_t N, int64_t capacity, uint32_t tw, uint32_t th)
     L.ids1 = take((size_t)capacity * 4);
     L.total = o;
     return L;
+}
+// two events per device for the fork / join with a caller's second stream (created once, never destroyed)
+struct SideEvents {
+    hipEvent_t keys_done, table_done;
+};
+int side_events(SideEvents** out) {
+    static std::mutex mutex;
+    static SideEvents events[64];
+    static bool made[64] = {};
+    int dev = -1;
+    GSX_HIP_CHECK(hipGetDevice(&dev));
+    GSX_REQUIRE(dev >= 0 && dev < 64, GSX_ERR_UNSUPPORTED, "tile_lists: device ordinal %d", dev);
+    std::lock_guard<std::mutex> lock(mutex);
+    if (!made[dev]) {
+        GSX_HIP_CHECK(hipEventCreateWithFlags(&events[dev].keys_done, hipEventDisableTiming));
+        GSX_HIP_CHECK(hipEventCreateWithFlags(&events[dev].table_done, hipEventDisableTiming));
+        made[dev] = true;
+    }
+    *out = &events[dev];
+    return GSX_OK;
 }
 int check_lists_args(const char* who, uint32_t N, int64_t capacity, uint32_t tw, uint32_t th) {
     GSX_REQUIRE(tw >= 1 && th >= 1 && tw <= 255 && th <= 255, GSX_ERR_UNSUPPORTED,
@@ -356,8 +522,8 @@ extern "C" size_t gsx_tile_lists_workspace_bytes(uint32_t N, int64_t capacity, u
     return lists_layout(N, capacity, tile_width, tile_height).total;
 }
 
-// the head of the workspace (digit histograms, corner grid, counts, error word, tickets) must be zero before the
-// first call; every call leaves it as the next one needs it
+// the head of the workspace (digit histogram, counts, error words, look-back words of the first launch, ...) must be
+// zero before the first call; every call leaves it as the next one needs it
 extern "C" int gsx_tile_lists_init(uint32_t N, int64_t capacity, uint32_t tile_width, uint32_t tile_height,
                                    void* workspace, size_t workspace_bytes, void* stream) {
     int rc = check_lists_args("tile_lists_init", N, capacity, tile_width, tile_height);
@@ -366,7 +532,7 @@ extern "C" int gsx_tile_lists_init(uint32_t N, int64_t capacity, uint32_t tile_w
     const ListsLayout L = lists_layout(N, capacity, tile_width, tile_height);
     GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 && workspace_bytes >= L.total,
                 GSX_ERR_WORKSPACE, "tile_lists_init: workspace needs %zu bytes, 256-byte aligned", L.total);
-    const size_t words = L.tile_counts / 4;
+    const size_t words = L.head_end / 4;
     hipLaunchKernelGGL(zero_words_kernel, dim3(cdiv(words, 256)), dim3(256), 0, (hipStream_t)stream, words,
                        (uint32_t*)workspace);
     GSX_LAUNCH_CHECK();
@@ -376,7 +542,7 @@ extern "C" int gsx_tile_lists_init(uint32_t N, int64_t capacity, uint32_t tile_w
 extern "C" int gsx_tile_lists(uint32_t N, const float* means2d, const int32_t* radii, const float* depths,
                               uint32_t tile_size, uint32_t tile_width, uint32_t tile_height, int64_t capacity,
                               void* workspace, size_t workspace_bytes, int32_t* flatten_ids, int32_t* tile_offsets,
-                              int64_t* n_isects_host_slot, void* stream) {
+                              int64_t* n_isects_host_slot, void* stream, void* side_stream) {
     int rc = check_lists_args("tile_lists", N, capacity, tile_width, tile_height);
     if (rc != GSX_OK)
         return rc;
@@ -396,53 +562,80 @@ extern "C" int gsx_tile_lists(uint32_t N, const float* means2d, const int32_t* r
                     "tile_lists: n_isects_host_slot must be pinned host memory (hipHostMalloc)");
         slot = (int64_t*)attr.devicePointer;
     }
+    const size_t table_lds = L.grid_in_lds ? (size_t)L.cells * 4 : 0;
+    if (table_lds > 48 * 1024) { // beyond the default limit of dynamically sized LDS
+        static bool raised = false; // per process; the attribute is idempotent
+        if (!raised) {
+            GSX_HIP_CHECK(hipFuncSetAttribute((const void*)tile_table_kernel<true>,
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsCells * 4));
+            raised = true;
+        }
+    }
     char* ws = (char*)workspace;
     auto u32p = [&](size_t off) { return (uint32_t*)(ws + off); };
     int64_t* keys[2] = {(int64_t*)(ws + L.keys0), (int64_t*)(ws + L.keys1)};
     int32_t* vals[2] = {(int32_t*)(ws + L.vals0), (int32_t*)(ws + L.vals1)};
     uint32_t* dstatus[2] = {u32p(L.dstatus0), u32p(L.dstatus1)};
     uint32_t* pstatus[2] = {u32p(L.pstatus0), u32p(L.pstatus1)};
-    uint32_t* tickets = u32p(L.tickets); // [0], [1]: depth passes; [2]: emission; [3], [4]: pair passes
     uint32_t* error = u32p(L.error);
     int64_t* counts = (int64_t*)(ws + L.counts);
     hipStream_t s = (hipStream_t)stream;
 
-    hipLaunchKernelGGL(depth_keys_kernel, dim3(cdiv(N, kKeysPerBlock)), dim3(256), 0, s, N, means2d, radii, depths,
-                       (float)tile_size, tile_width, tile_height, keys[0], vals[0], u32p(L.depth_hist),
-                       (int32_t*)(ws + L.corner_grid), dstatus[0], L.drows, tickets + 0, u32p(L.estatus), L.ewords,
-                       tickets + 2);
+    hipLaunchKernelGGL(depth_keys_kernel, dim3(L.kblocks), dim3(256), 0, s, N, means2d, radii, depths,
+                       (float)tile_size, tile_width, tile_height, keys[0], vals[0], u32p(L.rects), u32p(L.kstatus),
+                       counts, error, dstatus[0], L.drows, u32p(L.estatus), L.ewords);
     GSX_LAUNCH_CHECK();
-    // the tile table needs the corner grid only: it is queued first so that the count reaches the host early
+    // The tile table needs the rectangles only, not their depth order: with a second stream it is formed while the
+    // sort runs.
     const uint32_t tile_bits = gsx_n_bits(tile_width * tile_height);
     const uint32_t passes = tile_bits > 8 ? 2u : 1u;
     const uint32_t bits0 = passes == 2 ? (tile_bits + 1) / 2 : (tile_bits ? tile_bits : 1u);
     const uint32_t bits1 = passes == 2 ? tile_bits - bits0 : 0u;
-    hipLaunchKernelGGL(tile_table_kernel, dim3(1), dim3(1024), 0, s, tile_width, tile_height,
-                       (int32_t*)(ws + L.corner_grid), u32p(L.tile_counts), capacity, bits0, bits1, tile_offsets,
-                       u32p(L.pair_hist), counts, slot, error);
+    hipStream_t ts = side_stream != nullptr && side_stream != stream ? (hipStream_t)side_stream : s;
+    SideEvents* ev = nullptr;
+    if (ts != s) {
+        if ((rc = side_events(&ev)) != GSX_OK)
+            return rc;
+        GSX_HIP_CHECK(hipEventRecord(ev->keys_done, s));
+        GSX_HIP_CHECK(hipStreamWaitEvent(ts, ev->keys_done, 0));
+    }
+    if (L.grid_in_lds)
+        hipLaunchKernelGGL(tile_table_kernel<true>, dim3(L.table_blocks), dim3(1024), table_lds, ts, u32p(L.rects),
+                           tile_width, tile_height, (int32_t*)(ws + L.replicas), u32p(L.done_counter), capacity, bits0,
+                           bits1, tile_offsets, u32p(L.pair_hist), counts, slot, error);
+    else
+        hipLaunchKernelGGL(tile_table_kernel<false>, dim3(L.table_blocks), dim3(1024), 0, ts, u32p(L.rects),
+                           tile_width, tile_height, (int32_t*)(ws + L.shared_grid), u32p(L.done_counter), capacity,
+                           bits0, bits1, tile_offsets, u32p(L.pair_hist), counts, slot, error);
+    GSX_LAUNCH_CHECK();
+    if (ts != s)
+        GSX_HIP_CHECK(hipEventRecord(ev->table_done, ts));
+    hipLaunchKernelGGL(depth_hist_kernel, dim3(cdiv(N, 4096)), dim3(256), 0, s, keys[0], counts, u32p(L.depth_hist));
     GSX_LAUNCH_CHECK();
     for (uint32_t pass = 0; pass < 4; ++pass) { // depth bits, a byte per pass; the result ends in keys[0] / vals[0]
         const uint32_t in = pass & 1u, out = in ^ 1u;
         RadixChainArgs a;
-        a.n_dev = nullptr, a.status = dstatus[in], a.ticket = tickets + in, a.error = error;
+        a.n_dev = counts + 2, a.status = dstatus[in], a.error = error;
+        a.total_replicas = kHistReplicas, a.total_stride = 1024;
         a.clear_status = pass < 3 ? dstatus[out] : nullptr, a.clear_rows = L.drows;
-        a.clear_ticket = pass < 3 ? tickets + out : nullptr;
         if ((rc = radix_chained_pass_i64(N, keys[in], vals[in], keys[out], vals[out], 8u * pass, 8u,
                                          u32p(L.depth_hist) + 256u * pass, a, s)) != GSX_OK)
             return rc;
     }
+    if (ts != s)
+        GSX_HIP_CHECK(hipStreamWaitEvent(s, ev->table_done, 0));
     uint16_t* tkeys[2] = {(uint16_t*)(ws + L.tkeys0), (uint16_t*)(ws + L.tkeys1)};
     int32_t* ids[2] = {(int32_t*)(ws + L.ids0), (int32_t*)(ws + L.ids1)};
-    hipLaunchKernelGGL(tile_emit_chained_kernel, dim3(L.ewords), dim3(256), 0, s, N, keys[0], vals[0], tile_width,
-                       counts, u32p(L.estatus), tickets + 2, tkeys[0], ids[0], pstatus[0], L.prows, tickets + 3,
+    hipLaunchKernelGGL(tile_emit_chained_kernel, dim3(L.ewords), dim3(256), 0, s, keys[0], vals[0], tile_width,
+                       counts, u32p(L.estatus), tkeys[0], ids[0], pstatus[0], L.prows, u32p(L.kstatus), L.kblocks,
                        u32p(L.depth_hist), error);
     GSX_LAUNCH_CHECK();
     for (uint32_t pass = 0; pass < passes; ++pass) {
         const bool last = pass + 1 == passes;
         RadixChainArgs a;
-        a.n_dev = counts, a.status = pstatus[pass], a.ticket = tickets + 3 + pass, a.error = error;
+        a.n_dev = counts, a.status = pstatus[pass], a.error = error;
+        a.total_replicas = 1, a.total_stride = 0;
         a.clear_status = last ? nullptr : pstatus[1], a.clear_rows = L.prows;
-        a.clear_ticket = last ? nullptr : tickets + 4;
         if ((rc = radix_chained_pass_u16((uint32_t)capacity, tkeys[pass], ids[pass], tkeys[pass ^ 1u],
                                          last ? flatten_ids : ids[pass ^ 1u], pass ? bits0 : 0u, pass ? bits1 : bits0,
                                          u32p(L.pair_hist) + 256u * pass, a, !last, s)) != GSX_OK)
@@ -452,7 +645,8 @@ extern "C" int gsx_tile_lists(uint32_t N, const float* means2d, const int32_t* r
 }
 
 // where a caller can read the outcome of the last call on the device: counts[0] = pairs in the lists (0 if they did
-// not fit), counts[1] = pairs there are; error: bit 0 = capacity exceeded, bit 1 = a look-back gave up
+// not fit), counts[1] = pairs there are, counts[2] = Gaussians that touch a tile; error[0]: bit 0 = capacity
+// exceeded, bit 1 = a look-back gave up; error[1]: free for the caller (gsx_update_args.hold counts there)
 extern "C" const int64_t* gsx_tile_lists_counts(uint32_t N, int64_t capacity, uint32_t tile_width,
                                                 uint32_t tile_height, const void* workspace) {
     if (workspace == nullptr || N == 0 || capacity <= 0)

@@ -304,11 +304,12 @@ class TrainStep:
         if self._lists_active:
             # every launch sized by the buffers, the count read on the device: nothing waits for the host
             self._lists_ready()
+            sh_pass()  # queued first: the tile table goes behind it on the second stream
             self._run("tile_lists", lb.gsx_tile_lists, c_u32(N), _p(J["means2d"]), _p(J["radii"]), _p(J["depths"]),
                       c_u32(16), c_u32(self.tw), c_u32(self.th), c_i64(self.cap), _p(self.lists_ws),
                       c_sz(self.lists_ws.numel()), _p(self.flat_out), _p(self.offsets_full),
-                      c_p(self.n_isects_pinned.data_ptr()), s)
-            sh_pass()
+                      c_p(self.n_isects_pinned.data_ptr()), s,
+                      c_p(self.side.cuda_stream if self.side is not None else None))
             self.flatten_ids = self.flat_out
             n = -1  # GSX_COUNT_IN_OFFSETS
         else:

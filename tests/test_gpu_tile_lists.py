@@ -33,7 +33,8 @@ def inputs(tw, th, n, seed, big=0.0):
 
 
 class Lists:
-    def __init__(self, gsx, cuda, n, tw, th, cap):
+    def __init__(self, gsx, cuda, n, tw, th, cap, side=False):
+        self.side = torch.cuda.Stream(cuda) if side else None
         from lichtfeld_studio_amd._lib import c_i64, c_p, c_sz, c_u32, check, lib
         self.L, self.check = lib(), check
         self.n, self.tw, self.th, self.cap, self.dev = n, tw, th, cap, cuda
@@ -52,7 +53,8 @@ class Lists:
         self.slot[0] = -1
         self.check(self.L.gsx_tile_lists(c_u32(self.n), p(m), p(r), p(d), c_u32(16), c_u32(self.tw), c_u32(self.th),
                                          c_i64(self.cap), p(self.ws), c_sz(self.ws.numel()), p(self.flat), p(self.off),
-                                         c_p(self.slot.data_ptr()), self.stream))
+                                         c_p(self.slot.data_ptr()), self.stream,
+                                         c_p(self.side.cuda_stream if self.side is not None else None)))
         torch.cuda.synchronize()
         base = self.ws.data_ptr()
         c_at = self.L.gsx_tile_lists_counts(*self.dims, c_p(base)) - base
@@ -78,7 +80,7 @@ def test_tile_lists_match_the_separate_operators(gsx, orc, cuda, grid, n, big):
     _, o_ids, o_flat = orc.intersect_tile(means2d, radii, depths, 1, 16, tw, th, sort=True)
     assert np.array_equal(N(want_flat), o_flat)
 
-    lists = Lists(gsx, cuda, n, tw, th, cap=ni + 1000)
+    lists = Lists(gsx, cuda, n, tw, th, cap=ni + 1000, side=(n % 2 == 0))  # half the cases with a second stream
     for rep in range(3):  # the workspace is left ready for the next call
         counts, err = lists.run(m, r, d)
         assert err == 0 and counts[0] == ni and counts[1] == ni and int(lists.slot[0]) == ni, (rep, counts, err)
