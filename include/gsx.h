@@ -64,17 +64,6 @@ GSX_API int gsx_version(void);
 GSX_API const char* gsx_last_error(void);
 GSX_API const char* gsx_status_string(int status);
 GSX_API gsx_ut_params gsx_ut_defaults(void);
-/* Test hook (no counterpart in the reference): evaluates one of the shared fp32 math primitives element-wise on the
- * device so that a test can compare it bit for bit with a host build.  which: 0 exp, 1 log, 2 rsqrt, 3 sin, 4 acos,
- * 5 sigmoid, 6 saturating float->u32, 7 pow(x, x2), 8 x / x2, 9 sqrt, 10 fma(x, x2, x), 11 exp restricted to
- * -87 <= x <= 0 (the rasterizers' variant; must equal 0 on that range). */
-GSX_API int gsx_debug_math(int which, uint32_t n, const float* x, const float* x2, float* y, void* stream);
-/* Measurement hook (no counterpart in the reference): a plain device-to-device copy kernel of `bytes` bytes (a
- * multiple of 16), the known-size yardstick for HBM byte counters and achieved-bandwidth figures. */
-GSX_API int gsx_debug_copy(const void* src, void* dst, size_t bytes, void* stream);
-/* Test hook: the 64-lane, 16-value wave reduction of the rasterizer backward.  in [n_waves,64,16] -> out [n_waves,16]. */
-GSX_API int gsx_debug_wave_reduce16(uint32_t n_waves, const float* in, float* out, void* stream);
-
 /* ---- a1: gsplat::projection_ut_3dgs_fused (Ops.h:69-98; kernel ProjectionUT3DGSFused.cu:17-210) ----
  * means [N,3] quats [N,4] (wxyz) scales [N,3] opacities [N] nullable, viewmats0 [C,4,4], Ks [C,3,3]
  * -> radii i32 [C,N,2], means2d [C,N,2], depths [C,N], conics [C,N,3], compensations [C,N] nullable.
@@ -277,16 +266,6 @@ GSX_API int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
     const float* radial_coeffs, const float* tangential_coeffs, const float* thin_prism_coeffs,
     const int32_t* tile_offsets, const int32_t* flatten_ids, float* render_colors, float* render_alphas,
     int32_t* last_ids, void* workspace, size_t workspace_bytes, void* stream);
-
-/* Pair counts of one forward pass, for turning kernel times into rates (no counterpart in the reference).
- * stats_out: device uint64[8] = {(pixel, Gaussian) pairs the forward evaluates, pairs composited, pairs the backward
- * walks, (wave, Gaussian) iterations executed, (wave, Gaussian) iterations removed by the pixel bounds, executed
- * iterations with a contributing pixel, 2 reserved};
- * the counts are ADDED to it, so zero it first. */
-GSX_API int gsx_rasterize_pair_stats(int64_t n_isects, const void* records, uint32_t image_width,
-                                     uint32_t image_height, const float* viewmat, const float* K,
-                                     const int32_t* tile_offsets, const int32_t* flatten_ids,
-                                     unsigned long long* stats_out, void* stream);
 
 /* ---- a8: gsplat::rasterize_to_pixels_from_world_3dgs_bwd (Ops.h:131-166; ...3DGSBwd.cu:16-379) ----
  * channels in {1, 3, 4} (RGB, and the depth render modes of Rasterization.cpp:374-393).  The five gradient outputs are fully WRITTEN (no zero-fill needed; the reference

@@ -7,6 +7,7 @@
 
 #define GSX_BUILD 1
 #include "../../include/gsx.h"
+#include "../../include/gsx_debug.h"
 #include "gsx_math.h"
 #include "gsx_camera.h"
 #include "gsx_record.h"

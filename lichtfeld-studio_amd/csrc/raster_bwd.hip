@@ -47,7 +47,9 @@ __global__ void __launch_bounds__(64) wave_reduce16_probe_kernel(const float* __
 // CDIM = 3: the RGB training path.  CDIM = 1 / 4: the depth render modes (Rasterization.cpp:374-393) - one colour
 // channel, or RGB plus a fourth channel that is staged from `colors` and whose per-Gaussian gradient is reduced
 // on its own into gextra [N].
-template <uint32_t CDIM, bool DIST>
+// STATS: count instead of differentiating (for roofline accounting): stats[0] += pairs whose alpha is evaluated,
+// [1] += valid pairs, [2] += (wave, Gaussian) iterations executed.
+template <uint32_t CDIM, bool DIST, bool STATS = false>
 __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     uint32_t n_isects, const float4* __restrict__ records, const float* __restrict__ colors,
     const float* __restrict__ backgrounds,
@@ -59,7 +61,8 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     const int32_t* __restrict__ flatten_ids,
     const float* __restrict__ render_alphas, const int32_t* __restrict__ last_ids,
     const float* __restrict__ v_render_colors, const float* __restrict__ v_render_alphas,
-    float* __restrict__ gacc /*[N,16]*/, float* __restrict__ gextra /*[N], CDIM == 4*/) {
+    float* __restrict__ gacc /*[N,16]*/, float* __restrict__ gextra /*[N], CDIM == 4*/,
+    unsigned long long* __restrict__ stats = nullptr) {
     constexpr uint32_t NC = CDIM < 3 ? CDIM : 3; // channels carried by the record
     __shared__ float4 stage[kBatch * 4];
     __shared__ float extra[CDIM > 3 ? kBatch : 1];
@@ -113,8 +116,8 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     float v_render_c[CDIM];
 #pragma unroll
     for (uint32_t k = 0; k < CDIM; ++k)
-        v_render_c[k] = v_render_colors[(size_t)pix_id * CDIM + k];
-    const float v_render_a = v_render_alphas[pix_id];
+        v_render_c[k] = STATS ? 0.f : v_render_colors[(size_t)pix_id * CDIM + k];
+    const float v_render_a = STATS ? 0.f : v_render_alphas[pix_id];
     float bg_dot = 0.f;
     if (backgrounds != nullptr) {
 #pragma unroll
@@ -147,6 +150,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     if (range_end <= range_start)
         return;
     const uint32_t num_batches = (uint32_t)(range_end - range_start + (int32_t)kBatch - 1) / kBatch;
+    uint32_t n_eval = 0, n_valid = 0, n_iter = 0;
 
     for (uint32_t b = 0; b < num_batches; ++b) {
         // back to front: slot 0 of the batch is the farthest Gaussian (:211-216)
@@ -166,6 +170,10 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
         for (uint32_t sidx = 0; sidx < n_sel; ++sidx) {
             const int32_t t = (int32_t)wave_list[sidx];
             bool valid = inside && (batch_end - t <= bin_final);
+            if (STATS) {
+                n_eval += (uint32_t)__popcll(__builtin_amdgcn_ballot_w64(valid));
+                ++n_iter;
+            }
             const float4 a = stage[t * 4 + 0];
             const float4 m0 = stage[t * 4 + 1];
             const float4 m1 = stage[t * 4 + 2];
@@ -198,6 +206,10 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
                 valid = false;
             if (__builtin_amdgcn_ballot_w64(valid) == 0)
                 continue; // no lane of this wave sees the Gaussian (:286-289)
+            if (STATS) {
+                n_valid += (uint32_t)__popcll(__builtin_amdgcn_ballot_w64(valid));
+                continue;
+            }
 
             // From here on without branches: a lane that is not valid carries ra = 1 and fac = v_alpha = 0, which
             // leaves its T and colour buffer unchanged and makes all 16 of its partials zero.  The decisions above
@@ -274,6 +286,8 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             }
         }
         __syncthreads();
+        if (STATS)
+            continue;
         // flush: 16 lanes per Gaussian, one 64-byte row each
 #pragma unroll 4
         for (uint32_t s = 0; s < kBatch / 16; ++s) {
@@ -293,6 +307,11 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
                 unsafeAtomicAdd(&gextra[id_batch[tr]], val);
         }
         __syncthreads();
+    }
+    if (STATS && lane == 0) { // the counters are the same in every lane of a wave
+        atomicAdd(&stats[0], (unsigned long long)n_eval);
+        atomicAdd(&stats[1], (unsigned long long)n_valid);
+        atomicAdd(&stats[2], (unsigned long long)n_iter);
     }
 }
 
@@ -454,6 +473,30 @@ extern "C" int gsx_rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_is
                                     nullptr, GSX_GLOBAL, tile_offsets, tile_order, flatten_ids, render_alphas, last_ids,
                                     v_render_colors,
                                     v_render_alphas, workspace, workspace_bytes, stream);
+}
+
+extern "C" int gsx_rasterize_bwd_pair_stats(int64_t n_isects, const void* records, uint32_t image_width,
+                                            uint32_t image_height, const float* viewmat, const float* K,
+                                            const int32_t* tile_offsets, const int32_t* flatten_ids,
+                                            const float* render_alphas, const int32_t* last_ids,
+                                            unsigned long long* stats_out, void* stream) {
+    if (image_width == 0 || image_height == 0 || n_isects == 0)
+        return GSX_OK;
+    GSX_REQUIRE(records && viewmat && K && tile_offsets && flatten_ids && render_alphas && last_ids && stats_out,
+                GSX_ERR_INVALID_ARGUMENT, "rasterize_bwd_pair_stats: null tensor");
+    GSX_REQUIRE(n_isects >= GSX_COUNT_IN_OFFSETS && n_isects < (1ll << 31), GSX_ERR_OVERFLOW,
+                "rasterize_bwd_pair_stats: n_isects out of range");
+    const uint32_t tw = cdiv(image_width, kTile), th = cdiv(image_height, kTile);
+    // the gradient inputs are read but do not matter for the counts: the alphas (one float per pixel; the kernel
+    // reads three) cannot stand in for them, so the counts use a kernel instance that never touches them
+    hipLaunchKernelGGL((rasterize_bwd_kernel<3, false, true>), dim3(tw * th), dim3(256), 0, (hipStream_t)stream,
+                       (uint32_t)n_isects, (const float4*)records, (const float*)nullptr, (const float*)nullptr,
+                       (const uint8_t*)nullptr, image_width, image_height, tw, th, viewmat, K, (int)GSX_PINHOLE,
+                       (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
+                       (int)GSX_GLOBAL, tile_offsets, (const uint32_t*)nullptr, flatten_ids, render_alphas, last_ids,
+                       (const float*)nullptr, (const float*)nullptr, (float*)nullptr, (float*)nullptr, stats_out);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
 }
 
 // stage 3: per-Gaussian epilogue, accumulators -> the five gradient tensors (all elements written)

@@ -1,5 +1,5 @@
-"""CPU-side checks of the shipped library and host layer: libgsx.so loads and exports every symbol include/gsx.h
-declares, argument validation returns the documented status codes before anything is launched, the torch-facing
+"""CPU-side checks of the shipped library and host layer: libgsx.so loads and exports every symbol include/gsx.h and
+include/gsx_debug.h declare, argument validation returns the documented status codes before anything is launched, the torch-facing
 mirror of the reference API rejects what the reference's CHECK_INPUT rejects, and the scene generator is
 deterministic.  Nothing here launches a kernel."""
 import ctypes
@@ -13,7 +13,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "gsx.h")).read()
+    text = "".join(open(os.path.join(ROOT, "include", h)).read() for h in ("gsx.h", "gsx_debug.h"))
     return sorted(set(re.findall(r"GSX_API\s+[\w\s\*]+?\b(gsx_\w+)\s*\(", text)))
 
 
