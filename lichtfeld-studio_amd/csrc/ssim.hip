@@ -1,178 +1,309 @@
-// ssim.hip - fused separable 11x11 SSIM forward / backward (src/training/kernels/ssim.cu:16-27, 64-276, 284-424)
-// and the per-pixel parts of the photometric loss around it (src/training/trainer.cpp:126-129,
-// include/kernels/fused_ssim.cuh:59-67,84-96,117-122, src/training/rasterization/rasterizer.cpp:205).
+// ssim.hip - separable 11x11 SSIM forward / backward as column strips streamed through registers, and the per-pixel
+// parts of the photometric loss around it.  What is computed: src/training/kernels/ssim.cu:16-27 (window), :64-276
+// (forward), :284-424 (backward); src/training/trainer.cpp:126-129, include/kernels/fused_ssim.cuh:59-67,84-96,117-122
+// (valid crop, mean), src/training/rasterization/rasterizer.cpp:205 (clamp).
 //
-// One 256-lane workgroup per 16x16 pixel tile and image plane; the 26x26 halo tile is staged in LDS, convolved
-// horizontally into a 26x16 intermediate (five moments forward, three chains backward), then vertically.
-// Planes are independent workgroups (the reference loops the channels inside one block and re-synchronises).
-// Both kernels write every output element, so no zero-fill of the outputs is needed.
+// Organisation (gfx950).  A wave owns a strip of one image plane: 64 adjacent columns (one per lane) by kFwdRows /
+// output rows, and walks it top to bottom, one INPUT row per step:
+//   * the row's 64 + 10 values per image go through two wave-private LDS rows, from which every lane reads its
+//     eleven horizontal taps with unit stride across the lanes (no bank conflicts, no workgroup barrier: the four
+//     waves of a workgroup never talk to each other);
+//   * the horizontally filtered moments of the last eleven input rows stay in REGISTERS (a sliding window per lane);
+//     once the window is full every further input row completes one output row - the vertical filter reads no
+//     memory at all;
+//   * input rows are requested from memory two steps before they are processed.
+// A strip re-reads 10 halo rows per strip and 10 halo columns per 64; neighbouring strips run at the same time
+// and meet in L2, and the three colour planes of the interleaved render are three waves of one workgroup, so the
+// render's cache lines are fetched once.
+// Each output applies the taps in the reference's order (symmetric pairs from the centre outwards, then the centre;
+// rows after columns) and the reference's quotients, so results do not depend on the strip geometry and equal the CPU
+// checker's to the last bit.  (Sharing two reciprocals between the seven divisions of a pixel saves a seventh of the
+// instructions and moves d loss / d render by a few units in the last place - which the gradients of Gaussians that
+// vanish by cancellation then show at 13 times their rounding scale: not taken.)
 #include "gsx_common.h"
 
 namespace gsx {
 
-static constexpr int BX = 16, BY = 16, HALO = 5;
-static constexpr int SX = BX + 2 * HALO, SY = BY + 2 * HALO; // 26 x 26
-static constexpr int CY = SY;                                // rows of the horizontal-pass result
+static constexpr int HALO = 5;
+static constexpr int kStripCols = 64;  // one per lane
+static constexpr int kFwdRows = 12;    // output rows per forward strip: (12 + 10) / 12 input rows per output row
+static constexpr int kBwdRows = 8;     // backward strips: little arithmetic, more waves to hide the loads behind
+static constexpr int kRowFloats = kStripCols + 2 * HALO + 6; // an LDS row, padded to 80 floats
 
 __constant__ float cGauss[11] = {0.001028380123898387f, 0.0075987582094967365f, 0.036000773310661316f,
                                  0.10936068743467331f,  0.21300552785396576f,   0.26601171493530273f,
                                  0.21300552785396576f,  0.10936068743467331f,   0.036000773310661316f,
                                  0.0075987582094967365f, 0.001028380123898387f};
 
-__device__ __forceinline__ float pix(const float* __restrict__ img, size_t plane, int y, int x, int H, int W) {
-    if (x < 0 || x >= W || y < 0 || y >= H)
-        return 0.0f;
-    return img[plane + (size_t)y * W + x];
+// where a strip lies
+struct Strip {
+    int col0, row0; // first output column / row
+    int H, W;
+};
+
+// One value per lane for the columns col0 - 5 + lane (lane 0..63) and, in the lanes below 10, a second one for the
+// columns col0 + 59 + lane: the 74 columns an input row contributes to a strip.  Outside the image: 0.
+template <class Load>
+__device__ __forceinline__ void request_row(const Strip& st, int row, int lane, const Load& load, float* main_v,
+                                            float* halo_v) {
+    const bool row_in = row >= 0 && row < st.H;
+    const int cm = st.col0 - HALO + lane, ch = st.col0 + kStripCols - HALO + lane;
+    *main_v = (row_in && cm >= 0 && cm < st.W) ? load(row, cm) : 0.0f;
+    *halo_v = (lane < 2 * HALO && row_in && ch < st.W) ? load(row, ch) : 0.0f;
 }
 
-__global__ void __launch_bounds__(256) fusedssim_kernel(int H, int W, float C1, float C2,
-                                                         const float* __restrict__ img1,
-                                                         const float* __restrict__ img2, float* __restrict__ ssim_map,
-                                                         float* __restrict__ dm_dmu1,
-                                                         float* __restrict__ dm_dsigma1_sq,
-                                                         float* __restrict__ dm_dsigma12) {
-    __shared__ float sTile[SY][SX][2];
-    __shared__ float xconv[CY][BX][5];
-    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
-    const int pix_x = blockIdx.x * BX + tx, pix_y = blockIdx.y * BY + ty;
-    const size_t plane = (size_t)blockIdx.z * H * W;
+// the wave's LDS row receives the 74 values; afterwards lane l finds column col0 + l + d at index l + 5 + d
+__device__ __forceinline__ void publish_row(float* lds_row, int lane, float main_v, float halo_v) {
+    __builtin_amdgcn_wave_barrier(); // the previous row's taps have been read
+    lds_row[lane] = main_v;
+    if (lane < 2 * HALO)
+        lds_row[kStripCols + lane] = halo_v;
+    __builtin_amdgcn_wave_barrier();
+}
 
-    // 1) tile + halo, zero padded (:94-119)
-    for (int tid = threadIdx.x; tid < SY * SX; tid += 256) {
-        const int ly = tid / SX, lx = tid % SX;
-        const int gy = blockIdx.y * BY + ly - HALO, gx = blockIdx.x * BX + lx - HALO;
-        sTile[ly][lx][0] = pix(img1, plane, gy, gx, H, W);
-        sTile[ly][lx][1] = pix(img2, plane, gy, gx, H, W);
+// eleven-tap filter of one window (index 0 = oldest = top row): pairs from the centre outwards, then the centre
+template <int N>
+__device__ __forceinline__ void filter_window(const float (&win)[N][11], float (&out)[N]) {
+#pragma unroll
+    for (int k = 0; k < N; ++k)
+        out[k] = 0.f;
+#pragma unroll
+    for (int d = 1; d <= HALO; ++d) {
+        const float w = cGauss[HALO - d];
+#pragma unroll
+        for (int k = 0; k < N; ++k)
+            out[k] += (win[k][HALO - d] + win[k][HALO + d]) * w;
     }
-    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < N; ++k)
+        out[k] += win[k][HALO] * cGauss[HALO];
+}
 
-    // 2) horizontal 11-tap on the 26 rows (:121-213): symmetric pairs d = 1..5, then the centre
-    for (int ly = ty; ly < CY; ly += BY) {
-        const int lx = tx + HALO;
+// The window slides by register moves (ten per moment and row).  Unrolling the row loop eleven times makes every
+// slot a fixed register and removes the moves, but the eleven copies of the loop body no longer fit the instruction
+// cache two CUs share: measured 60 / 67 us against 56 / 46 us for the two loss kernels at 1237 x 822.
+template <int N>
+__device__ __forceinline__ void push_window(float (&win)[N][11], const float (&row)[N]) {
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+#pragma unroll
+        for (int j = 0; j < 10; ++j)
+            win[k][j] = win[k][j + 1];
+        win[k][10] = row[k];
+    }
+}
+
+// ---- forward -----------------------------------------------------------------------------------------------------
+// X / Y: loaders of the two images for this plane (row, column) -> value.  Per output pixel `emit(row, col, ssim,
+// dmu1, dsigma1_sq, dsigma12)` is called (image pixels only); returns the lane's sum of |X - Y| over its output pixels.
+// lds: two rows of kRowFloats (X and Y of the current input row).  Input rows are requested two steps ahead of their use.
+template <int ROWS, class LoadX, class LoadY, class Emit>
+__device__ __forceinline__ float ssim_forward_strip(const Strip& st, float C1, float C2, float* lds,
+                                                    const LoadX& loadx, const LoadY& loady, const Emit& emit) {
+    const int lane = threadIdx.x & 63;
+    const int col = st.col0 + lane;
+    const int row_end = min(st.row0 + ROWS, st.H); // one past the last output row
+    const int last_in = row_end + HALO;             // one past the last input row
+    float* lds_x = lds;
+    float* lds_y = lds + kRowFloats;
+    float win[5][11];
+#pragma unroll
+    for (int k = 0; k < 5; ++k)
+#pragma unroll
+        for (int j = 0; j < 11; ++j)
+            win[k][j] = 0.f;
+    float l1 = 0.f;
+    float xm[2], xh[2], ym[2], yh[2]; // [0]: the next row to publish, [1]: the one after it
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        request_row(st, st.row0 - HALO + k, lane, loadx, &xm[k], &xh[k]);
+        request_row(st, st.row0 - HALO + k, lane, loady, &ym[k], &yh[k]);
+    }
+    for (int row = st.row0 - HALO; row < last_in; ++row) {
+        publish_row(lds_x, lane, xm[0], xh[0]);
+        publish_row(lds_y, lane, ym[0], yh[0]);
+        xm[0] = xm[1], xh[0] = xh[1], ym[0] = ym[1], yh[0] = yh[1];
+        if (row + 2 < last_in) { // on its way while this row and the next are filtered
+            request_row(st, row + 2, lane, loadx, &xm[1], &xh[1]);
+            request_row(st, row + 2, lane, loady, &ym[1], &yh[1]);
+        }
+        // horizontal taps of this row (ssim.cu:121-213)
+        const int c = lane + HALO;
         float sumX = 0.f, sumX2 = 0.f, sumY = 0.f, sumY2 = 0.f, sumXY = 0.f;
 #pragma unroll
         for (int d = 1; d <= HALO; ++d) {
             const float w = cGauss[HALO - d];
-            const float Xl = sTile[ly][lx - d][0], Yl = sTile[ly][lx - d][1];
-            const float Xr = sTile[ly][lx + d][0], Yr = sTile[ly][lx + d][1];
+            const float Xl = lds_x[c - d], Yl = lds_y[c - d];
+            const float Xr = lds_x[c + d], Yr = lds_y[c + d];
             sumX += (Xl + Xr) * w;
             sumX2 += ((Xl * Xl) + (Xr * Xr)) * w;
             sumY += (Yl + Yr) * w;
             sumY2 += ((Yl * Yl) + (Yr * Yr)) * w;
             sumXY += ((Xl * Yl) + (Xr * Yr)) * w;
         }
-        const float cX = sTile[ly][lx][0], cY = sTile[ly][lx][1];
+        const float cX = lds_x[c], cY = lds_y[c];
         const float wc = cGauss[HALO];
         sumX += cX * wc;
         sumX2 += (cX * cX) * wc;
         sumY += cY * wc;
         sumY2 += (cY * cY) * wc;
         sumXY += (cX * cY) * wc;
-        xconv[ly][tx][0] = sumX;
-        xconv[ly][tx][1] = sumX2;
-        xconv[ly][tx][2] = sumY;
-        xconv[ly][tx][3] = sumY2;
-        xconv[ly][tx][4] = sumXY;
-    }
-    __syncthreads();
-
-    // 3) vertical 11-tap + SSIM and its partial derivatives (:215-274)
-    {
-        const int ly = ty + HALO, lx = tx;
-        float out[5] = {0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int d = 1; d <= HALO; ++d) {
-            const float w = cGauss[HALO - d];
-#pragma unroll
-            for (int k = 0; k < 5; ++k)
-                out[k] += (xconv[ly - d][lx][k] + xconv[ly + d][lx][k]) * w;
-        }
-#pragma unroll
-        for (int k = 0; k < 5; ++k)
-            out[k] += xconv[ly][lx][k] * cGauss[HALO];
-
-        if (pix_x < W && pix_y < H) {
-            const float mu1 = out[0], mu2 = out[2];
+        if (row >= st.row0 && row < row_end && col < st.W)
+            l1 += gsx::fabs(cX - cY);
+        const float moments[5] = {sumX, sumX2, sumY, sumY2, sumXY};
+        push_window(win, moments);
+        const int out_row = row - HALO; // the window now spans out_row - 5 .. out_row + 5
+        if (out_row >= st.row0 && col < st.W) {
+            float m[5];
+            filter_window(win, m);
+            // ssim.cu:215-274
+            const float mu1 = m[0], mu2 = m[2];
             const float mu1_sq = mu1 * mu1, mu2_sq = mu2 * mu2;
-            const float sigma1_sq = out[1] - mu1_sq, sigma2_sq = out[3] - mu2_sq;
-            const float sigma12 = out[4] - mu1 * mu2;
+            const float sigma1_sq = m[1] - mu1_sq, sigma2_sq = m[3] - mu2_sq;
+            const float sigma12 = m[4] - mu1 * mu2;
             const float A = mu1_sq + mu2_sq + C1;
             const float B = sigma1_sq + sigma2_sq + C2;
             const float C_ = 2.f * mu1 * mu2 + C1;
             const float D_ = 2.f * sigma12 + C2;
-            const size_t gi = plane + (size_t)pix_y * W + pix_x;
-            ssim_map[gi] = (C_ * D_) / (A * B);
-            if (dm_dmu1) {
-                dm_dmu1[gi] = ((mu2 * 2.f * D_) / (A * B) - (mu2 * 2.f * C_) / (A * B) -
-                               (mu1 * 2.f * C_ * D_) / (A * A * B) + (mu1 * 2.f * C_ * D_) / (A * B * B));
-                dm_dsigma1_sq[gi] = (-C_ * D_) / (A * B * B);
-                dm_dsigma12[gi] = (2.f * C_) / (A * B);
-            }
+            emit(out_row, col, (C_ * D_) / (A * B),
+                 ((mu2 * 2.f * D_) / (A * B) - (mu2 * 2.f * C_) / (A * B) - (mu1 * 2.f * C_ * D_) / (A * A * B) +
+                  (mu1 * 2.f * C_ * D_) / (A * B * B)),
+                 (-C_ * D_) / (A * B * B), (2.f * C_) / (A * B));
+        }
+    }
+    return l1;
+}
+
+// ---- backward ----------------------------------------------------------------------------------------------------
+// chain(row, col, &d0, &d1, &d2): the three derivative maps times d loss / d map at an image pixel (ssim.cu:305-337);
+// emit(row, col, s0, s1, s2): the three filtered sums of an output pixel (:385-421).
+template <int ROWS, class Chain, class Emit>
+__device__ __forceinline__ void ssim_backward_strip(const Strip& st, float* lds0, float* lds1, float* lds2,
+                                                    const Chain& chain, const Emit& emit) {
+    const int lane = threadIdx.x & 63;
+    const int col = st.col0 + lane;
+    const int row_end = min(st.row0 + ROWS, st.H);
+    const int last_in = row_end + HALO;
+    float win[3][11];
+#pragma unroll
+    for (int k = 0; k < 3; ++k)
+#pragma unroll
+        for (int j = 0; j < 11; ++j)
+            win[k][j] = 0.f;
+    auto request = [&](int row, float (&mv)[3], float (&hv)[3]) {
+        const bool row_in = row >= 0 && row < st.H;
+        const int cm = st.col0 - HALO + lane, ch = st.col0 + kStripCols - HALO + lane;
+        mv[0] = mv[1] = mv[2] = hv[0] = hv[1] = hv[2] = 0.f;
+        if (row_in && cm >= 0 && cm < st.W)
+            chain(row, cm, &mv[0], &mv[1], &mv[2]);
+        if (lane < 2 * HALO && row_in && ch < st.W)
+            chain(row, ch, &hv[0], &hv[1], &hv[2]);
+    };
+    float mv[3], hv[3], mv2[3], hv2[3]; // the next row to publish and the one after it
+    request(st.row0 - HALO, mv, hv);
+    request(st.row0 - HALO + 1, mv2, hv2);
+    for (int row = st.row0 - HALO; row < last_in; ++row) {
+        publish_row(lds0, lane, mv[0], hv[0]);
+        publish_row(lds1, lane, mv[1], hv[1]);
+        publish_row(lds2, lane, mv[2], hv[2]);
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+            mv[k] = mv2[k], hv[k] = hv2[k];
+        if (row + 2 < last_in)
+            request(row + 2, mv2, hv2);
+        const int c = lane + HALO;
+        float a0 = 0.f, a1 = 0.f, a2 = 0.f; // ssim.cu:339-383
+#pragma unroll
+        for (int d = 1; d <= HALO; ++d) {
+            const float w = cGauss[HALO - d];
+            a0 += (lds0[c - d] + lds0[c + d]) * w;
+            a1 += (lds1[c - d] + lds1[c + d]) * w;
+            a2 += (lds2[c - d] + lds2[c + d]) * w;
+        }
+        const float wc = cGauss[HALO];
+        a0 += lds0[c] * wc;
+        a1 += lds1[c] * wc;
+        a2 += lds2[c] * wc;
+        const float sums[3] = {a0, a1, a2};
+        push_window(win, sums);
+        const int out_row = row - HALO;
+        if (out_row >= st.row0 && col < st.W) {
+            float f[3];
+            filter_window(win, f);
+            emit(out_row, col, f[0], f[1], f[2]);
         }
     }
 }
 
+// the strip of wave `w` (over all waves of the launch): plane-major so that the planes of one strip are neighbours
+__device__ __forceinline__ Strip strip_of(uint32_t w, int planes, int H, int W, int rows, int* plane) {
+    const int strips_x = (W + kStripCols - 1) / kStripCols;
+    *plane = (int)(w % (uint32_t)planes);
+    const uint32_t s = w / (uint32_t)planes;
+    Strip st;
+    st.col0 = (int)(s % (uint32_t)strips_x) * kStripCols;
+    st.row0 = (int)(s / (uint32_t)strips_x) * rows;
+    st.H = H, st.W = W;
+    return st;
+}
+__host__ __device__ static inline uint32_t strip_count(uint32_t H, uint32_t W, uint32_t rows) {
+    return ((W + kStripCols - 1) / kStripCols) * ((H + rows - 1) / rows);
+}
+
+// gsplat-style operator (include/kernels/ssim.cuh:11-19): img1 / img2 [planes,H,W] -> map and the derivative maps
+__global__ void __launch_bounds__(256) fusedssim_kernel(int planes, int H, int W, float C1, float C2,
+                                                         const float* __restrict__ img1,
+                                                         const float* __restrict__ img2, float* __restrict__ ssim_map,
+                                                         float* __restrict__ dm_dmu1,
+                                                         float* __restrict__ dm_dsigma1_sq,
+                                                         float* __restrict__ dm_dsigma12) {
+    __shared__ float rows[4][2 * kRowFloats];
+    const uint32_t wave = threadIdx.x >> 6, w = blockIdx.x * 4u + wave;
+    if (w >= strip_count(H, W, kFwdRows) * (uint32_t)planes)
+        return;
+    int plane;
+    const Strip st = strip_of(w, planes, H, W, kFwdRows, &plane);
+    const size_t base = (size_t)plane * H * W;
+    ssim_forward_strip<kFwdRows>(
+        st, C1, C2, rows[wave], [&](int y, int x) { return img1[base + (size_t)y * W + x]; },
+        [&](int y, int x) { return img2[base + (size_t)y * W + x]; },
+        [&](int y, int x, float ssim, float dmu1, float ds1, float ds12) {
+            const size_t gi = base + (size_t)y * W + x;
+            ssim_map[gi] = ssim;
+            if (dm_dmu1) {
+                dm_dmu1[gi] = dmu1;
+                dm_dsigma1_sq[gi] = ds1;
+                dm_dsigma12[gi] = ds12;
+            }
+        });
+}
+
+// include/kernels/ssim.cuh:21-28 -> d loss / d img1
 __global__ void __launch_bounds__(256) fusedssim_backward_kernel(
-    int H, int W, const float* __restrict__ img1, const float* __restrict__ img2, const float* __restrict__ dL_dmap,
-    const float* __restrict__ dm_dmu1, const float* __restrict__ dm_dsigma1_sq, const float* __restrict__ dm_dsigma12,
-    float* __restrict__ dL_dimg1) {
-    __shared__ float sData[3][SY][SX];
-    __shared__ float sScratch[CY][BX][3];
-    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
-    const int pix_x = blockIdx.x * BX + tx, pix_y = blockIdx.y * BY + ty;
-    const size_t plane = (size_t)blockIdx.z * H * W;
-
-    // (1) load + fuse the chain multiplication (:305-337)
-    for (int tid = threadIdx.x; tid < SY * SX; tid += 256) {
-        const int row = tid / SX, col = tid % SX;
-        const int gy = blockIdx.y * BY + row - HALO, gx = blockIdx.x * BX + col - HALO;
-        const float chain = pix(dL_dmap, plane, gy, gx, H, W);
-        sData[0][row][col] = pix(dm_dmu1, plane, gy, gx, H, W) * chain;
-        sData[1][row][col] = pix(dm_dsigma1_sq, plane, gy, gx, H, W) * chain;
-        sData[2][row][col] = pix(dm_dsigma12, plane, gy, gx, H, W) * chain;
-    }
-    __syncthreads();
-
-    // (2) horizontal pass (:339-383)
-    for (int yy = ty; yy < CY; yy += BY) {
-        const int lx = tx + HALO;
-        float a0 = 0.f, a1 = 0.f, a2 = 0.f;
-#pragma unroll
-        for (int d = 1; d <= HALO; ++d) {
-            const float w = cGauss[HALO - d];
-            a0 += (sData[0][yy][lx - d] + sData[0][yy][lx + d]) * w;
-            a1 += (sData[1][yy][lx - d] + sData[1][yy][lx + d]) * w;
-            a2 += (sData[2][yy][lx - d] + sData[2][yy][lx + d]) * w;
-        }
-        const float wc = cGauss[HALO];
-        a0 += sData[0][yy][lx] * wc;
-        a1 += sData[1][yy][lx] * wc;
-        a2 += sData[2][yy][lx] * wc;
-        sScratch[yy][tx][0] = a0;
-        sScratch[yy][tx][1] = a1;
-        sScratch[yy][tx][2] = a2;
-    }
-    __syncthreads();
-
-    // (3) vertical pass -> dL/d(img1) (:385-421)
-    if (pix_x < W && pix_y < H) {
-        const int ly = ty + HALO, lx = tx;
-        float s0 = 0.f, s1 = 0.f, s2 = 0.f;
-#pragma unroll
-        for (int d = 1; d <= HALO; ++d) {
-            const float w = cGauss[HALO - d];
-            s0 += (sScratch[ly - d][lx][0] + sScratch[ly + d][lx][0]) * w;
-            s1 += (sScratch[ly - d][lx][1] + sScratch[ly + d][lx][1]) * w;
-            s2 += (sScratch[ly - d][lx][2] + sScratch[ly + d][lx][2]) * w;
-        }
-        const float wc = cGauss[HALO];
-        s0 += sScratch[ly][lx][0] * wc;
-        s1 += sScratch[ly][lx][1] * wc;
-        s2 += sScratch[ly][lx][2] * wc;
-        const size_t gi = plane + (size_t)pix_y * W + pix_x;
-        const float p1 = img1[gi], p2 = img2[gi];
-        dL_dimg1[gi] = s0 + (2.f * p1) * s1 + (p2)*s2;
-    }
+    int planes, int H, int W, const float* __restrict__ img1, const float* __restrict__ img2,
+    const float* __restrict__ dL_dmap, const float* __restrict__ dm_dmu1, const float* __restrict__ dm_dsigma1_sq,
+    const float* __restrict__ dm_dsigma12, float* __restrict__ dL_dimg1) {
+    __shared__ float rows[4][3][kRowFloats];
+    const uint32_t wave = threadIdx.x >> 6, w = blockIdx.x * 4u + wave;
+    if (w >= strip_count(H, W, kBwdRows) * (uint32_t)planes)
+        return;
+    int plane;
+    const Strip st = strip_of(w, planes, H, W, kBwdRows, &plane);
+    const size_t base = (size_t)plane * H * W;
+    ssim_backward_strip<kBwdRows>(
+        st, rows[wave][0], rows[wave][1], rows[wave][2],
+        [&](int y, int x, float* d0, float* d1, float* d2) {
+            const size_t gi = base + (size_t)y * W + x;
+            const float ch = dL_dmap[gi];
+            *d0 = dm_dmu1[gi] * ch;
+            *d1 = dm_dsigma1_sq[gi] * ch;
+            *d2 = dm_dsigma12[gi] * ch;
+        },
+        [&](int y, int x, float s0, float s1, float s2) {
+            const size_t gi = base + (size_t)y * W + x;
+            const float p1 = img1[gi], p2 = img2[gi];
+            dL_dimg1[gi] = s0 + (2.f * p1) * s1 + (p2)*s2;
+        });
 }
 
 // ---- loss-side passes ---------------------------------------------------------------------------
@@ -317,9 +448,9 @@ __global__ void __launch_bounds__(256) render_grad_from_loss_kernel(uint32_t HW,
 }
 
 // ---- the photometric loss of a training step in two kernels ---------------------------------------
-// forward: clamp + HWC -> CHW on load, SSIM moments and derivative maps, per-block partial sums of |image - gt| and
-// of the SSIM map over the valid crop (what image_from_render + fusedssim + ssim_valid_partials do in three passes;
-// the clamped image and the SSIM map themselves are never written).
+// forward: clamp + HWC -> CHW on load, SSIM moments and derivative maps, and per wave the sums of |image - gt| and of
+// the SSIM map over the valid crop (what image_from_render + fusedssim + ssim_valid_partials do in three passes; the
+// clamped image and the SSIM map themselves are never written).
 __global__ void __launch_bounds__(256) photometric_fwd_kernel(int H, int W, float C1, float C2,
                                                                const float* __restrict__ render_hwc,
                                                                const float* __restrict__ gt_chw,
@@ -328,101 +459,43 @@ __global__ void __launch_bounds__(256) photometric_fwd_kernel(int H, int W, floa
                                                                float* __restrict__ dm_dsigma12,
                                                                float* __restrict__ l1_partials,
                                                                float* __restrict__ ssim_partials) {
-    __shared__ float sTile[SY][SX][2];
-    __shared__ float xconv[CY][BX][5];
-    __shared__ float red[4];
-    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
-    const int pix_x = blockIdx.x * BX + tx, pix_y = blockIdx.y * BY + ty;
-    const int c = blockIdx.z;
-    const size_t plane = (size_t)c * H * W;
-
-    for (int tid = threadIdx.x; tid < SY * SX; tid += 256) {
-        const int ly = tid / SX, lx = tid % SX;
-        const int gy = blockIdx.y * BY + ly - HALO, gx = blockIdx.x * BX + lx - HALO;
-        float a = 0.f, b = 0.f;
-        if (gx >= 0 && gx < W && gy >= 0 && gy < H) {
-            a = gsx::fmin(gsx::fmax(render_hwc[((size_t)gy * W + gx) * 3 + c], 0.0f), 1.0f); // rasterizer.cpp:205
-            b = gt_chw[plane + (size_t)gy * W + gx];
-        }
-        sTile[ly][lx][0] = a;
-        sTile[ly][lx][1] = b;
+    __shared__ float rows[4][2 * kRowFloats];
+    const uint32_t wave = threadIdx.x >> 6, w = blockIdx.x * 4u + wave;
+    if (w >= strip_count(H, W, kFwdRows) * 3u)
+        return;
+    int c;
+    const Strip st = strip_of(w, 3, H, W, kFwdRows, &c);
+    const size_t base = (size_t)c * H * W;
+    const bool crop = H > 10 && W > 10;
+    float ss = 0.f;
+    float l1 = ssim_forward_strip<kFwdRows>(
+        st, C1, C2, rows[wave],
+        [&](int y, int x) { // rasterizer.cpp:205
+            return gsx::fmin(gsx::fmax(render_hwc[((size_t)y * W + x) * 3 + c], 0.0f), 1.0f);
+        },
+        [&](int y, int x) { return gt_chw[base + (size_t)y * W + x]; },
+        [&](int y, int x, float ssim, float dmu1, float ds1, float ds12) {
+            const size_t gi = base + (size_t)y * W + x;
+            if (!crop || (y >= 5 && y < H - 5 && x >= 5 && x < W - 5))
+                ss += ssim;
+            dm_dmu1[gi] = dmu1;
+            dm_dsigma1_sq[gi] = ds1;
+            dm_dsigma12[gi] = ds12;
+        });
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        l1 += __shfl_xor(l1, m, 64);
+        ss += __shfl_xor(ss, m, 64);
     }
-    __syncthreads();
-    for (int ly = ty; ly < CY; ly += BY) {
-        const int lx = tx + HALO;
-        float sumX = 0.f, sumX2 = 0.f, sumY = 0.f, sumY2 = 0.f, sumXY = 0.f;
-#pragma unroll
-        for (int d = 1; d <= HALO; ++d) {
-            const float w = cGauss[HALO - d];
-            const float Xl = sTile[ly][lx - d][0], Yl = sTile[ly][lx - d][1];
-            const float Xr = sTile[ly][lx + d][0], Yr = sTile[ly][lx + d][1];
-            sumX += (Xl + Xr) * w;
-            sumX2 += ((Xl * Xl) + (Xr * Xr)) * w;
-            sumY += (Yl + Yr) * w;
-            sumY2 += ((Yl * Yl) + (Yr * Yr)) * w;
-            sumXY += ((Xl * Yl) + (Xr * Yr)) * w;
-        }
-        const float cX = sTile[ly][lx][0], cY = sTile[ly][lx][1];
-        const float wc = cGauss[HALO];
-        sumX += cX * wc;
-        sumX2 += (cX * cX) * wc;
-        sumY += cY * wc;
-        sumY2 += (cY * cY) * wc;
-        sumXY += (cX * cY) * wc;
-        xconv[ly][tx][0] = sumX;
-        xconv[ly][tx][1] = sumX2;
-        xconv[ly][tx][2] = sumY;
-        xconv[ly][tx][3] = sumY2;
-        xconv[ly][tx][4] = sumXY;
-    }
-    __syncthreads();
-    float l1 = 0.f, ss = 0.f;
-    {
-        const int ly = ty + HALO, lx = tx;
-        float out[5] = {0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int d = 1; d <= HALO; ++d) {
-            const float w = cGauss[HALO - d];
-#pragma unroll
-            for (int k = 0; k < 5; ++k)
-                out[k] += (xconv[ly - d][lx][k] + xconv[ly + d][lx][k]) * w;
-        }
-#pragma unroll
-        for (int k = 0; k < 5; ++k)
-            out[k] += xconv[ly][lx][k] * cGauss[HALO];
-        if (pix_x < W && pix_y < H) {
-            const float mu1 = out[0], mu2 = out[2];
-            const float mu1_sq = mu1 * mu1, mu2_sq = mu2 * mu2;
-            const float sigma1_sq = out[1] - mu1_sq, sigma2_sq = out[3] - mu2_sq;
-            const float sigma12 = out[4] - mu1 * mu2;
-            const float A = mu1_sq + mu2_sq + C1;
-            const float B = sigma1_sq + sigma2_sq + C2;
-            const float C_ = 2.f * mu1 * mu2 + C1;
-            const float D_ = 2.f * sigma12 + C2;
-            const size_t gi = plane + (size_t)pix_y * W + pix_x;
-            const bool crop = H > 10 && W > 10;
-            if (!crop || (pix_y >= 5 && pix_y < H - 5 && pix_x >= 5 && pix_x < W - 5))
-                ss = (C_ * D_) / (A * B);
-            dm_dmu1[gi] = ((mu2 * 2.f * D_) / (A * B) - (mu2 * 2.f * C_) / (A * B) -
-                           (mu1 * 2.f * C_ * D_) / (A * A * B) + (mu1 * 2.f * C_ * D_) / (A * B * B));
-            dm_dsigma1_sq[gi] = (-C_ * D_) / (A * B * B);
-            dm_dsigma12[gi] = (2.f * C_) / (A * B);
-            l1 = gsx::fabs(sTile[ty + HALO][tx + HALO][0] - sTile[ty + HALO][tx + HALO][1]);
-        }
-    }
-    const uint32_t bid = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
-    const float l1s = block_sum_256(l1, red);
-    const float sss = block_sum_256(ss, red);
-    if (threadIdx.x == 0) {
-        l1_partials[bid] = l1s;
-        ssim_partials[bid] = sss;
+    if ((threadIdx.x & 63u) == 0) {
+        l1_partials[w] = l1;
+        ssim_partials[w] = ss;
     }
 }
 
 // backward: d loss / d render in one pass - the SSIM chain with d loss / d map = -lambda / count inside the valid crop
 // formed on the fly (fused_ssim.cuh:84-96), the L1 sign term, the clamp VJP and the CHW -> HWC permute (what
-// fusedssim_backward + render_grad_from_loss do in two passes with two intermediate images).  A block walks the
-// three colour planes of its tile and writes the pixel's three gradients together.
+// fusedssim_backward + render_grad_from_loss do in two passes with two intermediate images).
 __global__ void __launch_bounds__(256) photometric_bwd_kernel(int H, int W, float ssim_scale, float l1_scale,
                                                                const float* __restrict__ render_hwc,
                                                                const float* __restrict__ gt_chw,
@@ -430,82 +503,34 @@ __global__ void __launch_bounds__(256) photometric_bwd_kernel(int H, int W, floa
                                                                const float* __restrict__ dm_dsigma1_sq,
                                                                const float* __restrict__ dm_dsigma12,
                                                                float* __restrict__ v_render_hwc) {
-    __shared__ float sData[3][SY][SX];
-    __shared__ float sScratch[CY][BX][3];
-    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
-    const int pix_x = blockIdx.x * BX + tx, pix_y = blockIdx.y * BY + ty;
-    const bool inside = pix_x < W && pix_y < H;
+    __shared__ float rows[4][3][kRowFloats];
+    const uint32_t wave = threadIdx.x >> 6, w = blockIdx.x * 4u + wave;
+    if (w >= strip_count(H, W, kBwdRows) * 3u)
+        return;
+    int c;
+    const Strip st = strip_of(w, 3, H, W, kBwdRows, &c);
+    const size_t base = (size_t)c * H * W;
     const bool crop = H > 10 && W > 10;
-    float g[3] = {0.f, 0.f, 0.f};
-    for (int c = 0; c < 3; ++c) {
-        const size_t plane = (size_t)c * H * W;
-        for (int tid = threadIdx.x; tid < SY * SX; tid += 256) {
-            const int row = tid / SX, col = tid % SX;
-            const int gy = blockIdx.y * BY + row - HALO, gx = blockIdx.x * BX + col - HALO;
-            float d0 = 0.f, d1 = 0.f, d2 = 0.f;
-            if (gx >= 0 && gx < W && gy >= 0 && gy < H) {
-                const bool valid = !crop || (gy >= 5 && gy < H - 5 && gx >= 5 && gx < W - 5);
-                const float chain = valid ? ssim_scale : 0.f;
-                const size_t gi = plane + (size_t)gy * W + gx;
-                d0 = dm_dmu1[gi] * chain;
-                d1 = dm_dsigma1_sq[gi] * chain;
-                d2 = dm_dsigma12[gi] * chain;
-            }
-            sData[0][row][col] = d0;
-            sData[1][row][col] = d1;
-            sData[2][row][col] = d2;
-        }
-        __syncthreads();
-        for (int yy = ty; yy < CY; yy += BY) {
-            const int lx = tx + HALO;
-            float a0 = 0.f, a1 = 0.f, a2 = 0.f;
-#pragma unroll
-            for (int d = 1; d <= HALO; ++d) {
-                const float w = cGauss[HALO - d];
-                a0 += (sData[0][yy][lx - d] + sData[0][yy][lx + d]) * w;
-                a1 += (sData[1][yy][lx - d] + sData[1][yy][lx + d]) * w;
-                a2 += (sData[2][yy][lx - d] + sData[2][yy][lx + d]) * w;
-            }
-            const float wc = cGauss[HALO];
-            a0 += sData[0][yy][lx] * wc;
-            a1 += sData[1][yy][lx] * wc;
-            a2 += sData[2][yy][lx] * wc;
-            sScratch[yy][tx][0] = a0;
-            sScratch[yy][tx][1] = a1;
-            sScratch[yy][tx][2] = a2;
-        }
-        __syncthreads();
-        if (inside) {
-            const int ly = ty + HALO, lx = tx;
-            float s0 = 0.f, s1 = 0.f, s2 = 0.f;
-#pragma unroll
-            for (int d = 1; d <= HALO; ++d) {
-                const float w = cGauss[HALO - d];
-                s0 += (sScratch[ly - d][lx][0] + sScratch[ly + d][lx][0]) * w;
-                s1 += (sScratch[ly - d][lx][1] + sScratch[ly + d][lx][1]) * w;
-                s2 += (sScratch[ly - d][lx][2] + sScratch[ly + d][lx][2]) * w;
-            }
-            const float wc = cGauss[HALO];
-            s0 += sScratch[ly][lx][0] * wc;
-            s1 += sScratch[ly][lx][1] * wc;
-            s2 += sScratch[ly][lx][2] * wc;
-            const size_t p = (size_t)pix_y * W + pix_x;
+    ssim_backward_strip<kBwdRows>(
+        st, rows[wave][0], rows[wave][1], rows[wave][2],
+        [&](int y, int x, float* d0, float* d1, float* d2) {
+            const bool valid = !crop || (y >= 5 && y < H - 5 && x >= 5 && x < W - 5);
+            const float ch = valid ? ssim_scale : 0.f;
+            const size_t gi = base + (size_t)y * W + x;
+            *d0 = dm_dmu1[gi] * ch;
+            *d1 = dm_dsigma1_sq[gi] * ch;
+            *d2 = dm_dsigma12[gi] * ch;
+        },
+        [&](int y, int x, float s0, float s1, float s2) {
+            const size_t p = (size_t)y * W + x;
             const float r = render_hwc[p * 3 + c];
-            const float p1 = gsx::fmin(gsx::fmax(r, 0.0f), 1.0f), p2 = gt_chw[plane + p];
+            const float p1 = gsx::fmin(gsx::fmax(r, 0.0f), 1.0f), p2 = gt_chw[base + p];
             const float dssim = s0 + (2.f * p1) * s1 + (p2)*s2;
             const float d = p1 - p2;
             const float sgn = d > 0.f ? 1.f : (d < 0.f ? -1.f : 0.f);
             const float gg = l1_scale * sgn + dssim;
-            g[c] = (r >= 0.f && r <= 1.f) ? gg : 0.f; // clamp VJP
-        }
-        __syncthreads(); // sData / sScratch are rewritten for the next plane
-    }
-    if (inside) {
-        const size_t p = (size_t)pix_y * W + pix_x;
-        v_render_hwc[p * 3 + 0] = g[0];
-        v_render_hwc[p * 3 + 1] = g[1];
-        v_render_hwc[p * 3 + 2] = g[2];
-    }
+            v_render_hwc[p * 3 + c] = (r >= 0.f && r <= 1.f) ? gg : 0.f; // clamp VJP
+        });
 }
 
 } // namespace gsx
@@ -521,10 +546,11 @@ extern "C" int gsx_fusedssim(int B, int CH, int H, int W, float C1, float C2, co
     const bool train = dm_dmu1 != nullptr;
     GSX_REQUIRE(train == (dm_dsigma1_sq != nullptr) && train == (dm_dsigma12 != nullptr), GSX_ERR_INVALID_ARGUMENT,
                 "fusedssim: the three derivative maps must be given together");
-    GSX_REQUIRE((int64_t)B * CH <= 65535, GSX_ERR_INVALID_ARGUMENT, "fusedssim: B*CH too large");
-    const dim3 grid((W + BX - 1) / BX, (H + BY - 1) / BY, B * CH);
-    hipLaunchKernelGGL(fusedssim_kernel, grid, dim3(256), 0, (hipStream_t)stream, H, W, C1, C2, img1, img2, ssim_map,
-                       dm_dmu1, dm_dsigma1_sq, dm_dsigma12);
+    GSX_REQUIRE((int64_t)B * CH * strip_count((uint32_t)H, (uint32_t)W, kBwdRows) < (1ll << 31),
+                GSX_ERR_INVALID_ARGUMENT, "fusedssim: B*CH*H*W too large");
+    const uint32_t waves = strip_count((uint32_t)H, (uint32_t)W, kFwdRows) * (uint32_t)(B * CH);
+    hipLaunchKernelGGL(fusedssim_kernel, dim3(cdiv(waves, 4)), dim3(256), 0, (hipStream_t)stream, B * CH, H, W, C1, C2,
+                       img1, img2, ssim_map, dm_dmu1, dm_dsigma1_sq, dm_dsigma12);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }
@@ -539,10 +565,11 @@ extern "C" int gsx_fusedssim_backward(int B, int CH, int H, int W, float C1, flo
         return GSX_OK;
     GSX_REQUIRE(img1 && img2 && dL_dmap && dm_dmu1 && dm_dsigma1_sq && dm_dsigma12 && dL_dimg1,
                 GSX_ERR_INVALID_ARGUMENT, "fusedssim_backward: null tensor");
-    GSX_REQUIRE((int64_t)B * CH <= 65535, GSX_ERR_INVALID_ARGUMENT, "fusedssim_backward: B*CH too large");
-    const dim3 grid((W + BX - 1) / BX, (H + BY - 1) / BY, B * CH);
-    hipLaunchKernelGGL(fusedssim_backward_kernel, grid, dim3(256), 0, (hipStream_t)stream, H, W, img1, img2, dL_dmap,
-                       dm_dmu1, dm_dsigma1_sq, dm_dsigma12, dL_dimg1);
+    GSX_REQUIRE((int64_t)B * CH * strip_count((uint32_t)H, (uint32_t)W, kBwdRows) < (1ll << 31),
+                GSX_ERR_INVALID_ARGUMENT, "fusedssim_backward: B*CH*H*W too large");
+    const uint32_t waves = strip_count((uint32_t)H, (uint32_t)W, kBwdRows) * (uint32_t)(B * CH);
+    hipLaunchKernelGGL(fusedssim_backward_kernel, dim3(cdiv(waves, 4)), dim3(256), 0, (hipStream_t)stream, B * CH, H,
+                       W, img1, img2, dL_dmap, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, dL_dimg1);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }
@@ -612,7 +639,7 @@ extern "C" int gsx_render_grad_from_loss(uint32_t H, uint32_t W, float lambda_ds
 }
 
 extern "C" uint32_t gsx_photometric_partials(uint32_t H, uint32_t W) {
-    return 3u * cdiv(W, (uint32_t)BX) * cdiv(H, (uint32_t)BY);
+    return 3u * strip_count(H, W, kFwdRows); // one pair of sums per wave
 }
 
 extern "C" int gsx_photometric_loss_forward(uint32_t H, uint32_t W, float C1, float C2, const float* render_hwc,
@@ -624,8 +651,8 @@ extern "C" int gsx_photometric_loss_forward(uint32_t H, uint32_t W, float C1, fl
     GSX_REQUIRE(render_hwc && gt_chw && dm_dmu1 && dm_dsigma1_sq && dm_dsigma12 && l1_partials && ssim_partials,
                 GSX_ERR_INVALID_ARGUMENT, "photometric_loss_forward: null tensor");
     GSX_REQUIRE((uint64_t)H * W < (1ull << 30), GSX_ERR_INVALID_ARGUMENT, "photometric_loss_forward: image too large");
-    const dim3 grid(cdiv(W, (uint32_t)BX), cdiv(H, (uint32_t)BY), 3);
-    hipLaunchKernelGGL(photometric_fwd_kernel, grid, dim3(256), 0, (hipStream_t)stream, (int)H, (int)W, C1, C2,
+    hipLaunchKernelGGL(photometric_fwd_kernel, dim3(cdiv(3u * strip_count(H, W, kFwdRows), 4)), dim3(256),
+                       0, (hipStream_t)stream, (int)H, (int)W, C1, C2,
                        render_hwc, gt_chw, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, l1_partials, ssim_partials);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
@@ -642,8 +669,8 @@ extern "C" int gsx_photometric_loss_backward(uint32_t H, uint32_t W, float lambd
     const float count = crop ? 3.f * (float)(H - 10) * (float)(W - 10) : 3.f * (float)H * (float)W;
     const float ssim_scale = -lambda_dssim / count;
     const float l1_scale = (1.f - lambda_dssim) / (3.f * (float)H * (float)W);
-    const dim3 grid(cdiv(W, (uint32_t)BX), cdiv(H, (uint32_t)BY));
-    hipLaunchKernelGGL(photometric_bwd_kernel, grid, dim3(256), 0, (hipStream_t)stream, (int)H, (int)W, ssim_scale,
+    hipLaunchKernelGGL(photometric_bwd_kernel, dim3(cdiv(3u * strip_count(H, W, kBwdRows), 4)), dim3(256),
+                       0, (hipStream_t)stream, (int)H, (int)W, ssim_scale,
                        l1_scale, render_hwc, gt_chw, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, v_render_hwc);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
