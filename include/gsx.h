@@ -224,7 +224,8 @@ GSX_API uint32_t* gsx_tile_lists_error(uint32_t N, int64_t capacity, uint32_t ti
                                        void* workspace);
 
 /* ---- a7: gsplat::rasterize_to_pixels_from_world_3dgs_fwd (Ops.h:100-129; ...3DGSFwd.cu:19-285) ----
- * colors [C,N,channels] (channels in {1,3,4}), opacities [C,N], backgrounds [C,channels] nullable,
+ * colors [C,N,channels] (channels in {1,2,3,4,5,8,9,16,17,32}: Rasterization.cpp:106-128 up to 32; beyond that
+ * GSX_ERR_UNSUPPORTED), opacities [C,N], backgrounds [C,channels] nullable,
  * masks u8 [C,Th,Tw] nullable, tile_offsets i32 [C,Th,Tw], flatten_ids i32 [n_isects]
  * -> render_colors [C,H,W,channels], render_alphas [C,H,W,1], last_ids i32 [C,H,W]. tile_size must be 16.
  *
@@ -248,7 +249,7 @@ GSX_API int gsx_tile_order(int64_t n_isects, const int32_t* tile_offsets, const 
  * themselves when the workspace they are given is this much larger than their own requirement: the forward by list
  * length, the backward by the cost read from render_alphas / last_ids. */
 GSX_API size_t gsx_tile_order_bytes(uint32_t tile_width, uint32_t tile_height);
-/* colors is only read for channels beyond the third (channels == 4); nullable otherwise.  tile_order: nullable (tiles
+/* colors is only read for channels beyond the third (channels > 3); nullable otherwise.  tile_order: nullable (tiles
  * in index order), else any permutation of the tile ids (gsx_tile_order).  tile_walk: nullable, u32 [tiles]: receives
  * per tile how far its pixels went into the list (entries up to the last contributor, 0 = none) - what the tile cost
  * this pass and will cost the backward pass. */
@@ -268,17 +269,22 @@ GSX_API int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
     int32_t* last_ids, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- a8: gsplat::rasterize_to_pixels_from_world_3dgs_bwd (Ops.h:131-166; ...3DGSBwd.cu:16-379) ----
- * channels in {1, 3, 4} (RGB, and the depth render modes of Rasterization.cpp:374-393).  The five gradient outputs are fully WRITTEN (no zero-fill needed; the reference
+ * channels as in the forward pass (LichtFeld itself uses 1, 3, 4: RGB and the depth render modes of
+ * Rasterization.cpp:374-393).  The five gradient outputs are fully WRITTEN (no zero-fill needed; the reference
  * zero-fills and accumulates, Rasterization.cpp:190-194): v_means [N,3], v_quats [N,4], v_scales [N,3],
- * v_colors [C,N,channels], v_opacities [C,N].  Workspace of the whole operator: 16 + 1 accumulator floats per
- * Gaussian followed by the records. */
-GSX_API size_t gsx_rasterize_bwd_workspace_bytes(uint32_t N);
-GSX_API size_t gsx_rasterize_bwd_accum_bytes(uint32_t N);
+ * v_colors [C,N,channels], v_opacities [C,N].  Workspace of the whole operator: 16 + max(1, channels - 3) accumulator
+ * floats per Gaussian followed by the records (the ..._for functions; the two without a channel count serve up to
+ * four channels). */
+GSX_API size_t gsx_rasterize_bwd_workspace_bytes(uint32_t N);           /* up to four channels */
+GSX_API size_t gsx_rasterize_bwd_accum_bytes(uint32_t N);               /* up to four channels */
+GSX_API size_t gsx_rasterize_bwd_workspace_bytes_for(uint32_t N, uint32_t channels);
+GSX_API size_t gsx_rasterize_bwd_accum_bytes_for(uint32_t N, uint32_t channels);
 /* The backward pass is three launches - clear the accumulators, the per-tile kernel, the per-Gaussian epilogue -
  * that can also be called one by one (a training loop shares the forward's records and can fold the epilogue into
- * its own per-Gaussian pass); these three take the accumulator part (gsx_rasterize_bwd_accum_bytes) only. */
+ * its own per-Gaussian pass); these three take the accumulator part (gsx_rasterize_bwd_accum_bytes[_for]) only;
+ * gsx_rasterize_bwd_clear zeroes all workspace_bytes it is given. */
 GSX_API int gsx_rasterize_bwd_clear(uint32_t N, void* workspace, size_t workspace_bytes, void* stream);
-/* colors [N,channels] is read for a fourth channel only (nullable otherwise); tile_order: nullable, see
+/* colors [N,channels] is read for channels beyond the third only (nullable otherwise); tile_order: nullable, see
  * gsx_tile_order */
 GSX_API int gsx_rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isects, const void* records,
                                          const float* colors, uint32_t channels, const float* backgrounds,

@@ -102,7 +102,8 @@ def lib():
         for name in ("gsx_intersect_tile_count_workspace_bytes", "gsx_radix_sort_pairs_workspace_bytes",
                      "gsx_rasterize_bwd_workspace_bytes", "gsx_mcmc_relocate_workspace_bytes",
                      "gsx_raster_records_bytes", "gsx_rasterize_bwd_accum_bytes", "gsx_tile_order_bytes",
-                     "gsx_intersect_tile_count_ordered_workspace_bytes", "gsx_tile_lists_workspace_bytes"):
+                     "gsx_intersect_tile_count_ordered_workspace_bytes", "gsx_tile_lists_workspace_bytes",
+                     "gsx_rasterize_bwd_workspace_bytes_for", "gsx_rasterize_bwd_accum_bytes_for"):
             getattr(L, name).restype = c_sz
         L.gsx_tile_lists_counts.restype = c_p
         L.gsx_tile_lists_error.restype = c_p

@@ -302,6 +302,10 @@ __device__ __forceinline__ vec3 camera_ray_origin(const CamPose& cp) {
 // ---- tile geometry shared by the forward and backward rasterizers ----------------------------
 // One 256-lane workgroup per 16x16 tile; wave w owns the 8x8 pixel block (w & 1, w >> 1), lane l the pixel
 // (l >> 3, l & 7) of it: compact blocks keep a wave's pixels coherent (saturation, bounds rejection).
+// colour channel counts the rasterizers are instantiated for (gsplat/Rasterization.cpp:106-128 up to 32)
+static inline bool raster_channels_built(uint32_t c) {
+    return c == 1 || c == 2 || c == 3 || c == 4 || c == 5 || c == 8 || c == 9 || c == 16 || c == 17 || c == 32;
+}
 static constexpr uint32_t kTile = 16;
 // what (uint32_t)GSX_COUNT_IN_OFFSETS is inside the kernels
 static constexpr uint32_t kCountInOffsets = 0xFFFFFFFFu;

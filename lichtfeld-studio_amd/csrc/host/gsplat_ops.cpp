@@ -26,6 +26,10 @@ using gsplat::OptT;
 
 inline void* cur_stream(const at::Tensor& t) { return (void*)c10::hip::getCurrentHIPStream(t.device().index()).stream(); }
 
+// the channel counts the rasterizers are built for (Rasterization.cpp:106-128 lists up to 513)
+inline bool channels_built(uint32_t c) {
+    return c == 1 || c == 2 || c == 3 || c == 4 || c == 5 || c == 8 || c == 9 || c == 16 || c == 17 || c == 32;
+}
 inline void gsx_check(int status) { TORCH_CHECK(status == GSX_OK, "gsx (", gsx_status_string(status), "): ", gsx_last_error()); }
 
 inline bool has(const OptT& t) { return t.has_value() && t->defined() && t->numel() > 0; }
@@ -426,8 +430,8 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> rasterize_to_pixels_from_world_3d
         to_gsx(ut_params), (int)rs_type, fptr(radial_coeffs), fptr(tangential_coeffs), fptr(thin_prism_coeffs),
         tile_offsets.data_ptr<int32_t>(), flatten_ids.data_ptr<int32_t>(), renders.data_ptr<float>(),
         alphas.data_ptr<float>(), last_ids.data_ptr<int32_t>(), ws.data_ptr(), (size_t)ws.numel(), cur_stream(means));
-    TORCH_CHECK(st != GSX_ERR_UNSUPPORTED || (channels == 1 || channels == 3 || channels == 4),
-                "Unsupported number of channels: ", channels); // Rasterization.cpp:126-127
+    TORCH_CHECK(st != GSX_ERR_UNSUPPORTED || channels_built(channels), "Unsupported number of channels: ",
+                channels); // Rasterization.cpp:126-127
     gsx_check(st);
     return std::make_tuple(renders, alphas, last_ids);
 }
@@ -459,7 +463,7 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> rasterize
         CHECK_INPUT(masks.value());
     }
     const uint32_t channels = (uint32_t)colors.size(-1);
-    TORCH_CHECK(channels == 1 || channels == 3 || channels == 4, "Unsupported number of channels: ", channels);
+    TORCH_CHECK(channels_built(channels), "Unsupported number of channels: ", channels);
     TORCH_CHECK(!has(backgrounds) || (backgrounds->dim() == 2 && backgrounds->size(0) == tile_offsets.size(0) &&
                                       backgrounds->size(1) == channels),
                 "backgrounds must be [C, channels] = [", tile_offsets.size(0), ", ", channels, "], got ",
@@ -483,7 +487,8 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> rasterize
     // the kernels write every element of the five outputs (the reference zero-fills, Rasterization.cpp:190-194)
     at::Tensor v_means = at::empty_like(means), v_quats = at::empty_like(quats), v_scales = at::empty_like(scales);
     at::Tensor v_colors = at::empty_like(colors), v_opacities = at::empty_like(opacities);
-    at::Tensor ws = workspace(gsx_rasterize_bwd_workspace_bytes(N) + gsx_tile_order_bytes((uint32_t)tw, (uint32_t)th),
+    at::Tensor ws = workspace(gsx_rasterize_bwd_workspace_bytes_for(N, channels) +
+                                  gsx_tile_order_bytes((uint32_t)tw, (uint32_t)th),
                               means); // + room for the tile visiting order
     gsx_check(gsx_rasterize_to_pixels_from_world_3dgs_bwd(
         C, N, flatten_ids.size(0), means.data_ptr<float>(), quats.data_ptr<float>(), scales.data_ptr<float>(),

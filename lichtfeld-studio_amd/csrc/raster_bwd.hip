@@ -44,9 +44,9 @@ __global__ void __launch_bounds__(64) wave_reduce16_probe_kernel(const float* __
     }
 }
 
-// CDIM = 3: the RGB training path.  CDIM = 1 / 4: the depth render modes (Rasterization.cpp:374-393) - one colour
-// channel, or RGB plus a fourth channel that is staged from `colors` and whose per-Gaussian gradient is reduced
-// on its own into gextra [N].
+// CDIM = 3: the RGB training path.  CDIM = 1 / 4: the depth render modes (Rasterization.cpp:374-393).  Channels
+// beyond the third are staged from `colors`, and their per-Gaussian gradients are reduced on their own into gextra
+// [N, CDIM - 3].
 // STATS: count instead of differentiating (for roofline accounting): stats[0] += pairs whose alpha is evaluated,
 // [1] += valid pairs, [2] += (wave, Gaussian) iterations executed.
 template <uint32_t CDIM, bool DIST, bool STATS = false>
@@ -61,12 +61,16 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     const int32_t* __restrict__ flatten_ids,
     const float* __restrict__ render_alphas, const int32_t* __restrict__ last_ids,
     const float* __restrict__ v_render_colors, const float* __restrict__ v_render_alphas,
-    float* __restrict__ gacc /*[N,16]*/, float* __restrict__ gextra /*[N], CDIM == 4*/,
+    float* __restrict__ gacc /*[N,16]*/, float* __restrict__ gextra /*[N, CDIM - 3]*/,
     unsigned long long* __restrict__ stats = nullptr) {
     constexpr uint32_t NC = CDIM < 3 ? CDIM : 3; // channels carried by the record
     __shared__ float4 stage[kBatch * 4];
-    __shared__ float extra[CDIM > 3 ? kBatch : 1];
-    __shared__ float acc_extra[CDIM > 3 ? kBatch : 1];
+    constexpr uint32_t NX = CDIM > 3 ? CDIM - 3 : 0; // channels beyond the record's three
+    // up to six of them are staged and accumulated in LDS; beyond that (16 channels and more: not a training path)
+    // their colours are read from memory in the loop and every wave adds its sums to memory itself
+    constexpr bool XLDS = NX > 0 && NX <= 6;
+    __shared__ float extra[XLDS ? kBatch * NX : 1];
+    __shared__ float acc_extra[XLDS ? kBatch * NX : 1];
     __shared__ float4 region[kBatch * 2];
     __shared__ float cuts[kBatch];
     __shared__ uint8_t lists[4][kBatch];
@@ -143,8 +147,11 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
 #pragma unroll
     for (uint32_t k = 0; k < kAcc; ++k)
         acc[tr * kAcc + k] = 0.f;
-    if (CDIM > 3)
-        acc_extra[tr] = 0.f;
+    if (XLDS) {
+#pragma unroll
+        for (uint32_t k = 0; k < NX; ++k)
+            acc_extra[tr * (NX ? NX : 1) + k] = 0.f;
+    }
     __syncthreads();
     range_end = min(range_end, block_max + 1);
     if (range_end <= range_start)
@@ -161,9 +168,12 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
         const uint32_t n_sel = (uint32_t)__builtin_amdgcn_readfirstlane((int)stage_and_select(
             records, flatten_ids, batch_end, -1, (uint32_t)batch_size, tr, px, t_start,
             t_start < (uint32_t)batch_size, stage, region, cuts, id_batch, wave_list));
-        if (CDIM > 3) {
-            if ((int32_t)tr < batch_size)
-                extra[tr] = colors[(size_t)id_batch[tr] * CDIM + 3];
+        if (XLDS) {
+            if ((int32_t)tr < batch_size) {
+#pragma unroll
+                for (uint32_t k = 0; k < NX; ++k)
+                    extra[tr * (NX ? NX : 1) + k] = colors[(size_t)id_batch[tr] * CDIM + 3 + k];
+            }
             __syncthreads();
         }
 
@@ -218,7 +228,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             const float ra = valid ? __builtin_amdgcn_rcpf(1.0f - alpha) : 1.0f;
             T *= ra;
             const float fac = valid ? alpha * T : 0.f;
-            const float col[4] = {m2.y, m2.z, m2.w, CDIM > 3 ? extra[t] : 0.f};
+            const float col[3] = {m2.y, m2.z, m2.w};
             v[0] = fac * v_render_c[0];
             v[1] = NC > 1 ? fac * v_render_c[NC > 1 ? 1 : 0] : 0.f;
             v[2] = NC > 2 ? fac * v_render_c[NC > 2 ? 2 : 0] : 0.f;
@@ -231,8 +241,13 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             // multiplies (:313-321): one running scalar per pixel instead of one per channel.
             float cdot = col[0] * v_render_c[0];
 #pragma unroll
-            for (uint32_t k = 1; k < CDIM; ++k)
+            for (uint32_t k = 1; k < NC; ++k)
                 cdot = fma(col[k], v_render_c[k], cdot);
+#pragma unroll
+            for (uint32_t k = 0; k < NX; ++k)
+                cdot = fma(XLDS ? extra[(uint32_t)t * (NX ? NX : 1) + k]
+                                : colors[(size_t)id_batch[t] * CDIM + 3 + k],
+                           v_render_c[CDIM > 3 ? 3 + k : 0], cdot);
             float v_alpha = fma(T, cdot, ra * behind);
             // the clamp at 0.999 has zero derivative (:322)
             v_alpha = (valid && a.w * vis <= 0.999f) ? v_alpha : 0.f;
@@ -270,13 +285,18 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
                 v[14] = fma(v_gro.z, o_shift.z, v[14]);
             }
             behind = fma(-cdot, fac, behind);
-            if (CDIM > 3) { // the fourth channel's gradient: its own wave sum
-                float e = fac * v_render_c[CDIM > 3 ? 3 : 0];
+#pragma unroll
+            for (uint32_t k = 0; k < NX; ++k) { // the gradients of the channels beyond the third: their own wave sums
+                float e = fac * v_render_c[CDIM > 3 ? 3 + k : 0];
 #pragma unroll
                 for (int m = 32; m >= 1; m >>= 1)
                     e += __shfl_xor(e, m, 64);
-                if (lane == 0)
-                    atomicAdd(&acc_extra[t], e);
+                if (lane == 0) {
+                    if (XLDS)
+                        atomicAdd(&acc_extra[(uint32_t)t * (NX ? NX : 1) + k], e);
+                    else if (e != 0.f)
+                        unsafeAtomicAdd(&gextra[(size_t)id_batch[t] * (NX ? NX : 1) + k], e);
+                }
             }
             const float total = wave_reduce16(v, lane);
             if ((lane & 3u) == 0) {
@@ -300,11 +320,14 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
                     unsafeAtomicAdd(&gacc[(size_t)id_batch[gi] * kAcc + k], val);
             }
         }
-        if (CDIM > 3 && (int32_t)tr < batch_size) {
-            const float val = acc_extra[tr];
-            acc_extra[tr] = 0.f;
-            if (val != 0.f)
-                unsafeAtomicAdd(&gextra[id_batch[tr]], val);
+        if (XLDS && (int32_t)tr < batch_size) {
+#pragma unroll
+            for (uint32_t k = 0; k < NX; ++k) {
+                const float val = acc_extra[tr * (NX ? NX : 1) + k];
+                acc_extra[tr * (NX ? NX : 1) + k] = 0.f;
+                if (val != 0.f)
+                    unsafeAtomicAdd(&gextra[(size_t)id_batch[tr] * (NX ? NX : 1) + k], val);
+            }
         }
         __syncthreads();
     }
@@ -341,11 +364,12 @@ __global__ void __launch_bounds__(256) rasterize_bwd_epilogue_kernel(
         v_colors[(size_t)g * channels + 1] = r0.y;
     if (channels > 2)
         v_colors[(size_t)g * channels + 2] = r0.z;
-    if (channels > 3) {
-        const float e = gextra[g];
-        v_colors[(size_t)g * channels + 3] = e;
+    for (uint32_t k = 3; k < channels; ++k) {
+        const size_t at = (size_t)g * (channels - 3) + (k - 3);
+        const float e = gextra[at];
+        v_colors[(size_t)g * channels + k] = e;
         if (clear && e != 0.f)
-            gextra[g] = 0.f;
+            gextra[at] = 0.f;
     }
     v_opacities[g] = r3.w;
     float vm[3] = {0.f, 0.f, 0.f}, vq[4] = {0.f, 0.f, 0.f, 0.f}, vs[3] = {0.f, 0.f, 0.f};
@@ -375,12 +399,15 @@ extern "C" int gsx_debug_wave_reduce16(uint32_t n_waves, const float* in, float*
 // accumulators only: 16 floats per Gaussian, then one float per Gaussian for a fourth colour channel; the
 // whole-operator entry point also packs the records behind them
 static size_t accum_extra_offset(uint32_t N) { return align_up((size_t)N * kAcc * 4, 256) + 256; }
-extern "C" size_t gsx_rasterize_bwd_accum_bytes(uint32_t N) {
-    return accum_extra_offset(N) + align_up((size_t)N * 4, 256);
+extern "C" size_t gsx_rasterize_bwd_accum_bytes_for(uint32_t N, uint32_t channels) {
+    return accum_extra_offset(N) + align_up((size_t)N * (channels > 4 ? channels - 3 : 1) * 4, 256);
 }
-extern "C" size_t gsx_rasterize_bwd_workspace_bytes(uint32_t N) {
-    return gsx_rasterize_bwd_accum_bytes(N) + gsx_raster_records_bytes(N);
+extern "C" size_t gsx_rasterize_bwd_workspace_bytes_for(uint32_t N, uint32_t channels) {
+    return gsx_rasterize_bwd_accum_bytes_for(N, channels) + gsx_raster_records_bytes(N);
 }
+// up to four channels
+extern "C" size_t gsx_rasterize_bwd_accum_bytes(uint32_t N) { return gsx_rasterize_bwd_accum_bytes_for(N, 4); }
+extern "C" size_t gsx_rasterize_bwd_workspace_bytes(uint32_t N) { return gsx_rasterize_bwd_workspace_bytes_for(N, 4); }
 
 // stage 1: zero the per-Gaussian accumulators
 extern "C" int gsx_rasterize_bwd_clear(uint32_t N, void* workspace, size_t workspace_bytes, void* stream) {
@@ -390,7 +417,7 @@ extern "C" int gsx_rasterize_bwd_clear(uint32_t N, void* workspace, size_t works
                     workspace_bytes >= gsx_rasterize_bwd_accum_bytes(N),
                 GSX_ERR_WORKSPACE, "rasterize bwd: accumulators need %zu bytes, 256-byte aligned",
                 gsx_rasterize_bwd_accum_bytes(N));
-    const size_t n_acc = gsx_rasterize_bwd_accum_bytes(N) / 4;
+    const size_t n_acc = workspace_bytes / 4; // everything that was given: more than four channels need more
     hipLaunchKernelGGL(fill_f32_kernel, dim3(cdiv(n_acc, 256)), dim3(256), 0, (hipStream_t)stream, n_acc, 0.f,
                        (float*)workspace);
     GSX_LAUNCH_CHECK();
@@ -423,12 +450,12 @@ static int rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isects, co
                     v_render_colors && v_render_alphas,
                 GSX_ERR_INVALID_ARGUMENT, "rasterize bwd: null tensor");
     GSX_REQUIRE(((uintptr_t)records & 15) == 0, GSX_ERR_WORKSPACE, "rasterize bwd: records need 16-byte alignment");
+    GSX_REQUIRE(raster_channels_built(channels), GSX_ERR_UNSUPPORTED,
+                "rasterize bwd: %u channels (built: 1, 2, 3, 4, 5, 8, 9, 16, 17, 32)", channels);
     GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 &&
-                    workspace_bytes >= gsx_rasterize_bwd_accum_bytes(N),
+                    workspace_bytes >= gsx_rasterize_bwd_accum_bytes_for(N, channels),
                 GSX_ERR_WORKSPACE, "rasterize bwd: accumulators need %zu bytes, 256-byte aligned",
-                gsx_rasterize_bwd_accum_bytes(N));
-    GSX_REQUIRE(channels == 1 || channels == 3 || channels == 4, GSX_ERR_UNSUPPORTED,
-                "rasterize bwd: %u channels (built: 1, 3, 4)", channels);
+                gsx_rasterize_bwd_accum_bytes_for(N, channels));
     GSX_REQUIRE(channels <= 3 || colors != nullptr, GSX_ERR_INVALID_ARGUMENT, "rasterize bwd: colors is null");
     const uint32_t tw = cdiv(image_width, kTile), th = cdiv(image_height, kTile);
     float* gextra = (float*)((char*)workspace + accum_extra_offset(N));
@@ -447,8 +474,15 @@ static int rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isects, co
         GSX_LAUNCH_BWD(CD, false)
     switch (channels) {
     case 1: GSX_LAUNCH_BWD2(1); break;
+    case 2: GSX_LAUNCH_BWD2(2); break;
     case 3: GSX_LAUNCH_BWD2(3); break;
-    default: GSX_LAUNCH_BWD2(4); break;
+    case 4: GSX_LAUNCH_BWD2(4); break;
+    case 5: GSX_LAUNCH_BWD2(5); break;
+    case 8: GSX_LAUNCH_BWD2(8); break;
+    case 9: GSX_LAUNCH_BWD2(9); break;
+    case 16: GSX_LAUNCH_BWD2(16); break;
+    case 17: GSX_LAUNCH_BWD2(17); break;
+    default: GSX_LAUNCH_BWD2(32); break;
     }
 #undef GSX_LAUNCH_BWD2
 #undef GSX_LAUNCH_BWD
@@ -508,10 +542,11 @@ extern "C" int gsx_rasterize_bwd_finish(uint32_t N, const float* means, const fl
         return GSX_OK;
     GSX_REQUIRE(means && quats && scales && viewmats0 && v_means && v_quats && v_scales && v_colors && v_opacities,
                 GSX_ERR_INVALID_ARGUMENT, "rasterize bwd: null tensor");
-    GSX_REQUIRE(workspace != nullptr && workspace_bytes >= gsx_rasterize_bwd_accum_bytes(N), GSX_ERR_WORKSPACE,
-                "rasterize bwd: accumulators need %zu bytes", gsx_rasterize_bwd_accum_bytes(N));
-    GSX_REQUIRE(channels == 1 || channels == 3 || channels == 4, GSX_ERR_UNSUPPORTED,
-                "rasterize bwd: %u channels (built: 1, 3, 4)", channels);
+    GSX_REQUIRE(raster_channels_built(channels), GSX_ERR_UNSUPPORTED,
+                "rasterize bwd: %u channels (built: 1, 2, 3, 4, 5, 8, 9, 16, 17, 32)", channels);
+    GSX_REQUIRE(workspace != nullptr && workspace_bytes >= gsx_rasterize_bwd_accum_bytes_for(N, channels),
+                GSX_ERR_WORKSPACE, "rasterize bwd: accumulators need %zu bytes",
+                gsx_rasterize_bwd_accum_bytes_for(N, channels));
     hipLaunchKernelGGL(rasterize_bwd_epilogue_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, means,
                        quats, scales, viewmats0, (float*)workspace, (float*)((char*)workspace + accum_extra_offset(N)),
                        channels, clear_accumulators, v_means, v_quats, v_scales, v_colors, v_opacities);
@@ -535,13 +570,15 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
         return rc;
     if (N == 0)
         return GSX_OK;
+    GSX_REQUIRE(raster_channels_built(channels), GSX_ERR_UNSUPPORTED,
+                "rasterize bwd: %u channels (built: 1, 2, 3, 4, 5, 8, 9, 16, 17, 32)", channels);
     GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 &&
-                    workspace_bytes >= gsx_rasterize_bwd_workspace_bytes(N),
+                    workspace_bytes >= gsx_rasterize_bwd_workspace_bytes_for(N, channels),
                 GSX_ERR_WORKSPACE, "rasterize bwd: workspace needs %zu bytes, 256-byte aligned",
-                gsx_rasterize_bwd_workspace_bytes(N));
+                gsx_rasterize_bwd_workspace_bytes_for(N, channels));
     GSX_REQUIRE(means && quats && scales && colors && opacities && viewmats0 && Ks, GSX_ERR_INVALID_ARGUMENT,
                 "rasterize bwd: null tensor");
-    const size_t acc_bytes = gsx_rasterize_bwd_accum_bytes(N);
+    const size_t acc_bytes = gsx_rasterize_bwd_accum_bytes_for(N, channels);
     void* records = (char*)workspace + acc_bytes;
     if ((rc = gsx_rasterize_bwd_clear(N, workspace, acc_bytes, stream)) != GSX_OK)
         return rc;
@@ -553,7 +590,7 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
         return rc;
     // room behind the records for a tile order: visit the tiles dearest first (cost from the forward's outputs)
     const uint32_t* tile_order = nullptr;
-    const size_t base_bytes = gsx_rasterize_bwd_workspace_bytes(N);
+    const size_t base_bytes = gsx_rasterize_bwd_workspace_bytes_for(N, channels);
     if (n_isects > 0 && tile_size == kTile && tile_offsets && render_alphas && last_ids &&
         workspace_bytes >= base_bytes + gsx_tile_order_bytes(cdiv(image_width, kTile), cdiv(image_height, kTile))) {
         if ((rc = tile_order_from_pixels(n_isects, image_width, image_height, tile_offsets, render_alphas, last_ids,

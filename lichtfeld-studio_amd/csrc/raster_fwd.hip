@@ -15,8 +15,8 @@
 namespace gsx {
 
 // One record per Gaussian (all N: rows of Gaussians that no tile lists are never read).
-template <uint32_t CDIM>
-__global__ void __launch_bounds__(256) pack_records_kernel(uint32_t N, const float* __restrict__ means,
+__global__ void __launch_bounds__(256) pack_records_kernel(uint32_t N, uint32_t CDIM,
+                                                            const float* __restrict__ means,
                                                             const float* __restrict__ quats,
                                                             const float* __restrict__ scales,
                                                             const float* __restrict__ opacities,
@@ -271,18 +271,10 @@ int pack_raster_records(uint32_t N, const float* means, const float* quats, cons
     GSX_REQUIRE(((uintptr_t)records & 15) == 0, GSX_ERR_WORKSPACE, "pack_raster_records: records need 16-byte alignment");
     const dim3 grid(cdiv(N, 256)), block(256);
     hipStream_t s = (hipStream_t)stream;
-#define GSX_LAUNCH_PACK(CD)                                                                                         \
-    hipLaunchKernelGGL((pack_records_kernel<CD>), grid, block, 0, s, N, means, quats, scales, opacities, colors,    \
-                       viewmat, K, image_width, image_height, pinhole, rolling, (float4*)records)
-    switch (channels) {
-    case 1: GSX_LAUNCH_PACK(1); break;
-    case 3: GSX_LAUNCH_PACK(3); break;
-    case 4: GSX_LAUNCH_PACK(4); break;
-    default:
-        set_error("pack_raster_records: %u channels (built: 1, 3, 4)", channels);
-        return GSX_ERR_UNSUPPORTED;
-    }
-#undef GSX_LAUNCH_PACK
+    GSX_REQUIRE(raster_channels_built(channels), GSX_ERR_UNSUPPORTED,
+                "pack_raster_records: %u channels (built: 1, 2, 3, 4, 5, 8, 9, 16, 17, 32)", channels);
+    hipLaunchKernelGGL(pack_records_kernel, grid, block, 0, s, N, channels, means, quats, scales, opacities, colors,
+                       viewmat, K, image_width, image_height, pinhole, rolling, (float4*)records);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }
@@ -318,12 +310,19 @@ int rasterize_records_fwd(int64_t n_isects, const void* records, const float* co
         GSX_LAUNCH_FWD(CD, true); \
     else                        \
         GSX_LAUNCH_FWD(CD, false)
-    switch (channels) { // the channel counts the render modes of Rasterization.cpp:374-393 produce
+    switch (channels) { // Rasterization.cpp:106-128 up to 32 channels (LichtFeld's render modes use 1, 3, 4)
     case 1: GSX_LAUNCH_FWD2(1); break;
+    case 2: GSX_LAUNCH_FWD2(2); break;
     case 3: GSX_LAUNCH_FWD2(3); break;
     case 4: GSX_LAUNCH_FWD2(4); break;
+    case 5: GSX_LAUNCH_FWD2(5); break;
+    case 8: GSX_LAUNCH_FWD2(8); break;
+    case 9: GSX_LAUNCH_FWD2(9); break;
+    case 16: GSX_LAUNCH_FWD2(16); break;
+    case 17: GSX_LAUNCH_FWD2(17); break;
+    case 32: GSX_LAUNCH_FWD2(32); break;
     default:
-        set_error("rasterize fwd: %u channels (built: 1, 3, 4)", channels);
+        set_error("rasterize fwd: %u channels (built: 1, 2, 3, 4, 5, 8, 9, 16, 17, 32)", channels);
         return GSX_ERR_UNSUPPORTED;
     }
 #undef GSX_LAUNCH_FWD2
@@ -368,8 +367,8 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
     if (image_width == 0 || image_height == 0)
         return GSX_OK;
     GSX_REQUIRE(tile_size == kTile, GSX_ERR_UNSUPPORTED, "rasterize fwd: tile_size %u (only 16 is built)", tile_size);
-    GSX_REQUIRE(channels == 1 || channels == 3 || channels == 4, GSX_ERR_UNSUPPORTED,
-                "rasterize fwd: %u channels (built: 1, 3, 4)", channels);
+    GSX_REQUIRE(raster_channels_built(channels), GSX_ERR_UNSUPPORTED,
+                "rasterize fwd: %u channels (built: 1, 2, 3, 4, 5, 8, 9, 16, 17, 32)", channels);
     GSX_REQUIRE(viewmats0 && Ks, GSX_ERR_INVALID_ARGUMENT, "rasterize fwd: null tensor");
     GSX_REQUIRE(n_isects == 0 || (means && quats && scales && colors && opacities && flatten_ids),
                 GSX_ERR_INVALID_ARGUMENT, "rasterize fwd: null Gaussian tensor");

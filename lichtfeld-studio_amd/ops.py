@@ -316,6 +316,10 @@ def projection_ut_3dgs_fused(means, quats, scales, opacities, viewmats0, viewmat
     return radii, means2d, depths, conics, comp
 
 
+# colour channel counts the rasterizers are built for (gsplat/Rasterization.cpp:106-128 lists up to 513)
+RASTER_CHANNELS = (1, 2, 3, 4, 5, 8, 9, 16, 17, 32)
+
+
 def _fit_backgrounds(backgrounds, channels):
     """The fused operators hand the caller's background ([C,3] from gs::training::rasterize, rasterizer.cpp:84-87,
     147) to a kernel that blends `channels` values per pixel (Rasterization.cpp:401-407): with RGB + depth it would
@@ -394,8 +398,8 @@ def rasterize_to_pixels_from_world_3dgs_bwd(means, quats, scales, colors, opacit
         _f32(t, n)
     _check_input(tile_offsets, "tile_offsets"), _check_input(flatten_ids, "flatten_ids")
     _check_input(last_ids, "last_ids")
-    if colors.size(-1) not in (1, 3, 4):
-        raise RuntimeError("Unsupported number of channels: %d (built: 1, 3, 4)" % colors.size(-1))
+    if colors.size(-1) not in RASTER_CHANNELS:
+        raise RuntimeError("Unsupported number of channels: %d (built: %s)" % (colors.size(-1), RASTER_CHANNELS))
     if backgrounds is not None and backgrounds.numel() == 0:
         backgrounds = None
     dev = means.device
@@ -418,7 +422,7 @@ def rasterize_to_pixels_from_world_3dgs_bwd(means, quats, scales, colors, opacit
     v_colors, v_opacities = torch.empty_like(colors), torch.empty_like(opacities)
     m8 = None if masks is None else masks.view(torch.uint8) if masks.dtype == torch.bool else masks
     with torch.cuda.device(dev):
-        ws = _workspace(lib().gsx_rasterize_bwd_workspace_bytes(c_u32(N)) +
+        ws = _workspace(lib().gsx_rasterize_bwd_workspace_bytes_for(c_u32(N), c_u32(channels)) +
                         lib().gsx_tile_order_bytes(c_u32(tw), c_u32(th)), dev)  # + room for the tile visiting order
         check(lib().gsx_rasterize_to_pixels_from_world_3dgs_bwd(
             c_u32(C), c_u32(N), c_i64(flatten_ids.numel()), _ptr(means), _ptr(quats), _ptr(scales), _ptr(colors),

@@ -819,7 +819,7 @@ ORC_API int orc_rasterize_to_pixels_from_world_3dgs_fwd(
     const uint8_t* masks /*nullable*/, uint32_t image_width, uint32_t image_height, uint32_t tile_size,
     const float* viewmats0, const float* Ks, const int32_t* tile_offsets, const int32_t* flatten_ids,
     float* render_colors, float* render_alphas, int32_t* last_ids, int64_t* pairs_evaluated) {
-    if (C != 1 || CDIM > 8)
+    if (C != 1 || CDIM > 64)
         return -2;
     (void)N;
     const uint32_t tile_width = (image_width + tile_size - 1) / tile_size;
@@ -856,7 +856,7 @@ ORC_API int orc_rasterize_to_pixels_from_world_3dgs_fwd(
                     pixel_world_ray((float)j + 0.5f, (float)i + 0.5f, fx, fy, cx, cy, rs, &ray_o, &ray_d);
                 float T = 1.0f;
                 uint32_t cur_idx = 0;
-                float pix_out[8] = {0.f};
+                float pix_out[64] = {};
                 // a pixel without a valid ray is done from the start (RasterizeToPixelsFromWorld3DGSFwd.cu:145)
                 for (int32_t t = 0; t < (ray_ok ? cnt : 0); ++t) {
                     ++pairs;
@@ -908,16 +908,16 @@ ORC_API int orc_rasterize_to_pixels_from_world_3dgs_bwd(
     const float* render_alphas, const int32_t* last_ids, const float* v_render_colors,
     const float* v_render_alphas, float* v_means, float* v_quats, float* v_scales, float* v_colors,
     float* v_opacities) {
-    if (C != 1 || CDIM < 1 || CDIM > 4)
+    constexpr uint32_t kMaxC = 64;
+    if (C != 1 || CDIM < 1 || CDIM > kMaxC)
         return -2;
-    constexpr uint32_t kMaxC = 4;
+    const size_t kRow = 11 + CDIM; // mean 3, quat 4, scale 3, opacity 1, then the colour channels
     const uint32_t tile_width = (image_width + tile_size - 1) / tile_size;
     const uint32_t tile_height = (image_height + tile_size - 1) / tile_size;
     const uint32_t n_tiles = tile_width * tile_height;
     const float fx = Ks[0], fy = Ks[4], cx = Ks[2], cy = Ks[5];
     const RollingShutter rs = make_rolling_shutter(viewmats0, nullptr);
-    // 15 = mean 3, quat 4, scale 3, colour 3, opacity 1, fourth colour channel 1
-    std::vector<double> acc((size_t)N * 15, 0.0);
+    std::vector<double> acc((size_t)N * kRow, 0.0);
     // tiles that share a Gaussian would race on acc: process tiles in parallel with per-Gaussian
     // atomic double adds (order-independent to ~1e-16, far below the fp32 comparison tolerance)
 #pragma omp parallel for schedule(dynamic, 1)
@@ -930,7 +930,7 @@ ORC_API int orc_rasterize_to_pixels_from_world_3dgs_bwd(
         const int32_t cnt = range_end - range_start;
         if (cnt <= 0)
             continue;
-        std::vector<double> local((size_t)cnt * 15, 0.0);
+        std::vector<double> local((size_t)cnt * kRow, 0.0);
         for (uint32_t ly = 0; ly < tile_size; ++ly)
             for (uint32_t lx = 0; lx < tile_size; ++lx) {
                 const uint32_t i = ty * tile_size + ly, j = tx * tile_size + lx;
@@ -942,9 +942,9 @@ ORC_API int orc_rasterize_to_pixels_from_world_3dgs_bwd(
                     continue; // RasterizeToPixelsFromWorld3DGSBwd.cu:157
                 const float T_final = 1.0f - render_alphas[pix_id];
                 float T = T_final;
-                float buffer[kMaxC] = {0.f, 0.f, 0.f, 0.f};
+                float buffer[kMaxC] = {};
                 const int32_t bin_final = last_ids[pix_id];
-                float v_render_c[kMaxC] = {0.f, 0.f, 0.f, 0.f};
+                float v_render_c[kMaxC] = {};
                 for (uint32_t k = 0; k < CDIM; ++k)
                     v_render_c[k] = v_render_colors[pix_id * CDIM + k];
                 const float v_render_a = v_render_alphas[pix_id];
@@ -976,7 +976,7 @@ ORC_API int orc_rasterize_to_pixels_from_world_3dgs_bwd(
                     const float ra = 1.0f / (1.0f - alpha);
                     T *= ra;
                     const float fac = alpha * T;
-                    float v_rgb_local[kMaxC] = {0.f, 0.f, 0.f, 0.f};
+                    float v_rgb_local[kMaxC] = {};
                     for (uint32_t k = 0; k < CDIM; ++k)
                         v_rgb_local[k] = fac * v_render_c[k];
                     float v_alpha = 0.f;
@@ -1050,7 +1050,7 @@ ORC_API int orc_rasterize_to_pixels_from_world_3dgs_bwd(
                     for (uint32_t k = 0; k < CDIM; ++k)
                         buffer[k] += colors[(int64_t)g * CDIM + k] * fac;
 
-                    double* a = local.data() + (size_t)(idx - range_start) * 15;
+                    double* a = local.data() + (size_t)(idx - range_start) * kRow;
                     a[0] += v_mean_local.x;
                     a[1] += v_mean_local.y;
                     a[2] += v_mean_local.z;
@@ -1061,38 +1061,34 @@ ORC_API int orc_rasterize_to_pixels_from_world_3dgs_bwd(
                     a[7] += v_scale_local[0];
                     a[8] += v_scale_local[1];
                     a[9] += v_scale_local[2];
-                    a[10] += v_rgb_local[0];
-                    a[11] += v_rgb_local[1];
-                    a[12] += v_rgb_local[2];
-                    a[13] += v_opacity_local;
-                    a[14] += v_rgb_local[3];
+                    a[10] += v_opacity_local;
+                    for (uint32_t k = 0; k < CDIM; ++k)
+                        a[11 + k] += v_rgb_local[k];
                 }
             }
         for (int32_t t = 0; t < cnt; ++t) {
             const int32_t g = flatten_ids[range_start + t];
-            for (int k = 0; k < 15; ++k) {
-                const double v = local[(size_t)t * 15 + k];
+            for (size_t k = 0; k < kRow; ++k) {
+                const double v = local[(size_t)t * kRow + k];
                 if (v != 0.0) {
 #pragma omp atomic
-                    acc[(size_t)g * 15 + k] += v;
+                    acc[(size_t)g * kRow + k] += v;
                 }
             }
         }
     }
 #pragma omp parallel for schedule(static)
     for (int64_t g = 0; g < (int64_t)N; ++g) {
-        const double* a = acc.data() + (size_t)g * 15;
+        const double* a = acc.data() + (size_t)g * kRow;
         for (int k = 0; k < 3; ++k)
             v_means[g * 3 + k] += (float)a[k];
         for (int k = 0; k < 4; ++k)
             v_quats[g * 4 + k] += (float)a[3 + k];
         for (int k = 0; k < 3; ++k)
             v_scales[g * 3 + k] += (float)a[7 + k];
-        for (uint32_t k = 0; k < CDIM && k < 3; ++k)
-            v_colors[g * CDIM + k] += (float)a[10 + k];
-        if (CDIM > 3)
-            v_colors[g * CDIM + 3] += (float)a[14];
-        v_opacities[g] += (float)a[13];
+        for (uint32_t k = 0; k < CDIM; ++k)
+            v_colors[g * CDIM + k] += (float)a[11 + k];
+        v_opacities[g] += (float)a[10];
     }
     return 0;
 }
