@@ -340,7 +340,7 @@ __device__ __forceinline__ float sh_color_channel(uint32_t degree, vec3 dir, con
     return result;
 }
 
-// direction gradient (degree <= 3), accumulated over the three channels
+// direction gradient, accumulated over the three channels
 // (sh_coeffs_to_color_fast_vjp with v_dir != nullptr; the reference adds the channels with atomics, :474-478)
 __global__ void __launch_bounds__(256) sh_bwd_dirs_kernel(uint32_t N, uint32_t K, uint32_t degree,
                                                            const float* __restrict__ dirs,
@@ -407,6 +407,41 @@ __global__ void __launch_bounds__(256) sh_bwd_dirs_kernel(uint32_t N, uint32_t K
                             pSH14_y * co[14 * 3 + c] + pSH11_y * co[11 * 3 + c]);
                 v_z += v * (pSH12_z * co[12 * 3 + c] + pSH13_z * co[13 * 3 + c] + pSH11_z * co[11 * 3 + c] +
                             pSH14_z * co[14 * 3 + c] + pSH10_z * co[10 * 3 + c]);
+                if (degree >= 4) { // SphericalHarmonicsCUDA.cu:288-360
+                    const float fC2 = x * fC1 - y * fS1, fS2 = x * fS1 + y * fC1;
+                    const float pSH6 = (0.9461746957575601f * z2 - 0.3153915652525201f);
+                    const float pSH6_z4 = 2.f * 0.9461746957575601f * z;
+                    const float pSH12 = z * (1.865881662950577f * z2 - 1.119528997770346f);
+                    const float fTmp0D = z * (-4.683325804901025f * z2 + 2.007139630671868f);
+                    const float fTmp1C = 3.31161143515146f * z2 - 0.47308734787878f;
+                    const float fTmp2B = -1.770130769779931f * z;
+                    const float fTmp0D_z = 3.f * -4.683325804901025f * z2 + 2.007139630671868f;
+                    const float fTmp1C_z = 2.f * 3.31161143515146f * z;
+                    const float fTmp2B_z = -1.770130769779931f;
+                    const float fC3_x = fC2 + x * fC2_x - y * fS2_x;
+                    const float fC3_y = x * fC2_y - fS2 - y * fS2_y;
+                    const float fS3_x = fS2 + y * fC2_x + x * fS2_x;
+                    const float fS3_y = x * fS2_y + fC2 + y * fC2_y;
+                    const float pSH20_z = 1.984313483298443f * (pSH12 + z * pSH12_z) + -1.006230589874905f * pSH6_z4;
+                    const float pSH21_x = fTmp0D, pSH21_z = fTmp0D_z * x;
+                    const float pSH19_y = fTmp0D, pSH19_z = fTmp0D_z * y;
+                    const float pSH22_x = fTmp1C * fC1_x, pSH22_y = fTmp1C * fC1_y, pSH22_z = fTmp1C_z * fC1;
+                    const float pSH18_x = fTmp1C * fS1_x, pSH18_y = fTmp1C * fS1_y, pSH18_z = fTmp1C_z * fS1;
+                    const float pSH23_x = fTmp2B * fC2_x, pSH23_y = fTmp2B * fC2_y, pSH23_z = fTmp2B_z * fC2;
+                    const float pSH17_x = fTmp2B * fS2_x, pSH17_y = fTmp2B * fS2_y, pSH17_z = fTmp2B_z * fS2;
+                    const float pSH24_x = 0.6258357354491763f * fC3_x, pSH24_y = 0.6258357354491763f * fC3_y;
+                    const float pSH16_x = 0.6258357354491763f * fS3_x, pSH16_y = 0.6258357354491763f * fS3_y;
+                    (void)pSH6;
+                    v_x += v * (pSH16_x * co[16 * 3 + c] + pSH24_x * co[24 * 3 + c] + pSH17_x * co[17 * 3 + c] +
+                                pSH23_x * co[23 * 3 + c] + pSH18_x * co[18 * 3 + c] + pSH22_x * co[22 * 3 + c] +
+                                pSH21_x * co[21 * 3 + c]);
+                    v_y += v * (pSH16_y * co[16 * 3 + c] + pSH24_y * co[24 * 3 + c] + pSH17_y * co[17 * 3 + c] +
+                                pSH23_y * co[23 * 3 + c] + pSH18_y * co[18 * 3 + c] + pSH22_y * co[22 * 3 + c] +
+                                pSH19_y * co[19 * 3 + c]);
+                    v_z += v * (pSH20_z * co[20 * 3 + c] + pSH21_z * co[21 * 3 + c] + pSH19_z * co[19 * 3 + c] +
+                                pSH22_z * co[22 * 3 + c] + pSH18_z * co[18 * 3 + c] + pSH23_z * co[23 * 3 + c] +
+                                pSH17_z * co[17 * 3 + c]);
+                }
             }
             const float d = v_x * x + v_y * y + v_z * z;
             vx += (v_x - d * x) * inorm;
@@ -946,8 +981,7 @@ extern "C" int gsx_spherical_harmonics_bwd(uint32_t N, uint32_t K, uint32_t degr
     GSX_REQUIRE(degrees_to_use <= 4 && K >= (degrees_to_use + 1) * (degrees_to_use + 1), GSX_ERR_INVALID_ARGUMENT,
                 "spherical_harmonics_bwd: degree %u needs K >= %u (got %u)", degrees_to_use,
                 (degrees_to_use + 1) * (degrees_to_use + 1), K);
-    GSX_REQUIRE(v_dirs == nullptr || degrees_to_use <= 3, GSX_ERR_UNSUPPORTED,
-                "spherical_harmonics_bwd: v_dirs is implemented for degree <= 3");
+
     launch_sh_bwd<false>(N, K, degrees_to_use, dirs, masks, nullptr, nullptr, nullptr, v_colors, v_coeffs,
                          (hipStream_t)stream);
     GSX_LAUNCH_CHECK();

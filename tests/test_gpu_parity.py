@@ -148,12 +148,11 @@ def test_spherical_harmonics(gsx, orc, cuda, degree, n, K):
     ref = orc.spherical_harmonics_fwd(degree, dirs, coeffs, masks)
     got = N(ops.spherical_harmonics_fwd(degree, T(dirs, cuda), T(coeffs, cuda), T(masks, cuda)))
     bits_equal(got[masks], ref[masks], '')
-    ref_vc, ref_vd = orc.spherical_harmonics_bwd(K, degree, dirs, coeffs, masks, v_colors, degree <= 3)
+    ref_vc, ref_vd = orc.spherical_harmonics_bwd(K, degree, dirs, coeffs, masks, v_colors, True)
     vc, vd = ops.spherical_harmonics_bwd(K, degree, T(dirs, cuda), T(coeffs, cuda), T(masks, cuda), T(v_colors, cuda),
-                                         degree <= 3)
+                                         True)
     bits_equal(N(vc), ref_vc, '')
-    if degree <= 3:
-        np.testing.assert_allclose(N(vd)[masks], ref_vd[masks], rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(N(vd)[masks], ref_vd[masks], rtol=1e-5, atol=1e-6)
     # no mask
     got = N(ops.spherical_harmonics_fwd(degree, T(dirs, cuda), T(coeffs, cuda), None))
     bits_equal(got, orc.spherical_harmonics_fwd(degree, dirs, coeffs, None), '')

@@ -160,6 +160,32 @@ def sh_basis_polynomials(d):
         -0.5900435899266435 * x * (xx - 3 * yy)], -1)
 
 
+def sh_band4_scipy(d):
+    """The nine real spherical harmonics of degree 4 in float64 from scipy's complex ones (an independent statement
+    of the band: sqrt(2) Im / Re parts, m = -4 .. 4), without the reference's sign convention - callers fix the nine
+    signs against the checker's forward basis, which test_sh_basis_* pin."""
+    from scipy import special
+    x, y, z = d[..., 0], d[..., 1], d[..., 2]
+    theta, phi = np.arccos(np.clip(z, -1, 1)), np.arctan2(y, x)
+    out = []
+    for m in range(-4, 5):
+        Y = special.sph_harm_y(4, abs(m), theta, phi)
+        out.append(Y.real if m == 0 else np.sqrt(2) * (Y.imag if m < 0 else Y.real))
+    return np.stack(out, -1)
+
+
+def sh_basis_25(orc, d):
+    """float64 basis of degrees 0-4: the polynomial form for 0-3, scipy's band for 4 with the signs of the checker"""
+    dn = d / np.linalg.norm(d, axis=-1, keepdims=True)
+    probe = np.random.default_rng(5).normal(0, 1, (64, 3))
+    probe /= np.linalg.norm(probe, axis=1, keepdims=True)
+    got = checker_basis(orc, probe.astype(np.float32), 4)[:, 16:25]
+    raw = sh_band4_scipy(probe)
+    sign = np.sign((got * raw).sum(0))
+    np.testing.assert_allclose(got, raw * sign, atol=5e-6)  # the band itself, up to the nine signs
+    return np.concatenate([sh_basis_polynomials(dn), sh_band4_scipy(dn) * sign], -1)
+
+
 def checker_basis(orc, dirs, degree, K=25):
     """basis values through the checker: colour of a one-hot coefficient vector"""
     n = dirs.shape[0]
@@ -210,15 +236,15 @@ def test_sh_basis_degree4_orthonormal_and_harmonic(orc):
 
 def test_sh_colour_and_adjoint(orc):
     rng = np.random.default_rng(1)
-    n, K = 500, 16
+    n, K = 500, 25
     dirs = rng.normal(0, 1, (n, 3)).astype(np.float32)
     co = rng.normal(0, 1, (n, K, 3)).astype(np.float32)
     masks = rng.uniform(0, 1, n) < 0.7
     dn = dirs / np.linalg.norm(dirs, axis=1, keepdims=True)
-    for deg in range(4):
+    for deg in range(5):
         col = orc.spherical_harmonics_fwd(deg, dirs, co, masks)
         nb = (deg + 1) ** 2
-        want = np.einsum("nk,nkc->nc", sh_basis_polynomials(dn.astype(np.float64))[:, :nb], co[:, :nb].astype(np.float64))
+        want = np.einsum("nk,nkc->nc", sh_basis_25(orc, dn.astype(np.float64))[:, :nb], co[:, :nb].astype(np.float64))
         np.testing.assert_allclose(col[masks], want[masks], atol=2e-5)
         assert np.all(col[~masks] == 0)
         # backward = transpose of forward:  <v, fwd(c)> == <bwd(v), c>
@@ -234,10 +260,8 @@ def test_sh_colour_and_adjoint(orc):
             dp, dm = dirs.astype(np.float64).copy(), dirs.astype(np.float64).copy()
             dp[:, j] += h
             dm[:, j] -= h
-            fp = np.einsum("nk,nkc->nc", sh_basis_polynomials(dp / np.linalg.norm(dp, axis=1, keepdims=True))[:, :nb],
-                           co[:, :nb].astype(np.float64))
-            fm = np.einsum("nk,nkc->nc", sh_basis_polynomials(dm / np.linalg.norm(dm, axis=1, keepdims=True))[:, :nb],
-                           co[:, :nb].astype(np.float64))
+            fp = np.einsum("nk,nkc->nc", sh_basis_25(orc, dp)[:, :nb], co[:, :nb].astype(np.float64))
+            fm = np.einsum("nk,nkc->nc", sh_basis_25(orc, dm)[:, :nb], co[:, :nb].astype(np.float64))
             num = ((fp - fm) / (2 * h) * v).sum(1)
             np.testing.assert_allclose(vd[masks, j], num[masks], rtol=2e-3, atol=2e-4)
 
