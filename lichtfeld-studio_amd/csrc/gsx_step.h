@@ -177,18 +177,19 @@ __device__ __forceinline__ void adam_one(float& p, float& m, float& v, float g, 
 }
 
 // ---------------------------------------------------------------------------------------------
-// Rasterizer-backward epilogue: the linear map from the accumulated (v_gro, v_grd (x) ray_d) of one Gaussian to
-// (v_mean, v_quat, v_scale) - quat_scale_to_preci_half_vjp / quat_to_rotmat_vjp of gsplat/Utils.cuh:104-158.
-// Accumulator row: r0 = rgb.xyz, vo.x ; r1 = vo.y, vo.z, G00, G01 ; r2 = G02, G10, G11, G12 ; r3 = G20, G21, G22,
+// Rasterizer-backward epilogue: the linear map from one Gaussian's accumulated vo = sum k q and S = sum k q (x) q
+// (symmetric) to (v_mean, v_quat, v_scale).  d L / d M^T = S M^-T with M^-1 = R diag(s), then
+// quat_scale_to_preci_half_vjp / quat_to_rotmat_vjp of gsplat/Utils.cuh:104-158.  Because R is orthonormal the scale
+// gradient collapses to v_scale_j = -S_jj / s_j.
+// Accumulator row: r0 = rgb.xyz, vo.x ; r1 = vo.y, vo.z, Sxx, Sxy ; r2 = Sxz, Syy, Syz, Szz ; r3 = -, -, -,
 // v_opacity.  quats / scales are the ACTIVATED ones the rasterizer saw.
 // ---------------------------------------------------------------------------------------------
 __device__ __forceinline__ void epilogue_geometry_grads(float4 r0, float4 r1, float4 r2, float4 r3,
                                                         const float* __restrict__ viewmat, vec3 mean, quat q, vec3 s,
                                                         float (&vm)[3], float (&vq)[4], float (&vs)[3]) {
-    const CamPose cp = load_cam_pose(viewmat);
-    const vec3 ray_o = camera_ray_origin(cp);
-    const vec3 om = sub(ray_o, mean);
+    (void)viewmat, (void)mean, (void)r3;
     const mat3 R = quat_to_rotmat(q);
+    const float sv[3] = {s.x, s.y, s.z};
     const float is[3] = {1.0f / s.x, 1.0f / s.y, 1.0f / s.z};
     mat3 Mt;
 #pragma unroll
@@ -197,15 +198,14 @@ __device__ __forceinline__ void epilogue_geometry_grads(float4 r0, float4 r1, fl
         for (int b = 0; b < 3; ++b)
             Mt.m[a][b] = is[a] * R.m[b][a];
     const vec3 Vo = mk3(r0.w, r1.x, r1.y);
-    const float G[3][3] = {{r1.z, r1.w, r2.x}, {r2.y, r2.z, r2.w}, {r3.x, r3.y, r3.z}};
-    const float vo[3] = {Vo.x, Vo.y, Vo.z};
-    const float omv[3] = {om.x, om.y, om.z};
+    const float S[3][3] = {{r1.z, r1.w, r2.x}, {r1.w, r2.y, r2.z}, {r2.x, r2.z, r2.w}};
+    // v_Mt[a][b] = sum_c S[a][c] s_c R[b][c]
     float v_Mt[3][3];
 #pragma unroll
     for (int a = 0; a < 3; ++a)
 #pragma unroll
         for (int b = 0; b < 3; ++b)
-            v_Mt[a][b] = fma(vo[a], omv[b], G[a][b]);
+            v_Mt[a][b] = fma(S[a][2], sv[2] * R.m[b][2], fma(S[a][1], sv[1] * R.m[b][1], S[a][0] * (sv[0] * R.m[b][0])));
     const vec3 v_o = mul_t(Mt, Vo);
     vm[0] = -v_o.x;
     vm[1] = -v_o.y;
@@ -230,9 +230,10 @@ __device__ __forceinline__ void epilogue_geometry_grads(float4 r0, float4 r1, fl
     vq[1] = (vq_x - d * x) * inv_norm;
     vq[2] = (vq_y - d * y) * inv_norm;
     vq[3] = (vq_z - d * z) * inv_norm;
+    // v_scale_j = -is_j^2 sum_k R(k,j) v_M(k,j) (Utils.cuh:147-157) = -S_jj / s_j, the columns of R being orthonormal
 #pragma unroll
     for (int jj = 0; jj < 3; ++jj)
-        vs[jj] = -is[jj] * is[jj] * (R.m[0][jj] * v_Mt[jj][0] + R.m[1][jj] * v_Mt[jj][1] + R.m[2][jj] * v_Mt[jj][2]);
+        vs[jj] = -(S[jj][jj] * is[jj]);
 }
 
 } // namespace gsx

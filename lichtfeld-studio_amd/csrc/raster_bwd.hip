@@ -6,9 +6,10 @@
 //
 //  1. What is summed per Gaussian.  The reference pushes every (pixel, Gaussian) pair through the whole chain
 //     down to (v_mean, v_quat, v_scale) and reduces those 10 numbers.  That chain is linear in v_M = d L / d M
-//     (M = diag(1/s) R^T), and v_M = v_grd (x) ray_d + v_gro (x) (ray_o - mean) where ray_o is one constant per
-//     camera.  So the per-pair work stops at v_gro (3) and v_grd (x) ray_d (9); those are summed per Gaussian
-//     (with colour 3 and opacity 1: 16 floats) and a per-Gaussian epilogue applies the linear map once.
+//     (M = diag(1/s) R^T), and v_M = v_grd (x) ray_d + v_gro (x) (ray_o - mean) reduces exactly to k q (x) M^-1 q
+//     with q the nearest point of the pixel's ray to the centre in the Gaussian's frame (derivation at the loop).
+//     So the per-pair work stops at k q (3) and the symmetric k q (x) q (6); those are summed per Gaussian (with
+//     colour 3 and opacity 1: 13 of the 16 floats of a row) and a per-Gaussian epilogue applies the linear map once.
 //  2. How it is summed.  A 64-lane wave reduces its 16 partials with a halving butterfly (the array is split in
 //     two at each of the first four steps, so 8+4+2+1+1+1 = 17 exchanges instead of 16*6), after which 16 lanes
 //     hold one total each and add it to the workgroup's LDS accumulators; the workgroup flushes one 64-byte row
@@ -22,7 +23,7 @@
 
 namespace gsx {
 
-static constexpr uint32_t kAcc = 16; // floats accumulated per Gaussian: rgb 3, v_gro 3, v_grd(x)ray_d 9, opacity 1
+static constexpr uint32_t kAcc = 16; // floats per Gaussian: rgb 3, k q 3, k q (x) q 6 (symmetric), 3 unused, opacity 1
 
 __global__ void __launch_bounds__(256) fill_f32_kernel(size_t n, float v, float* __restrict__ out) {
     const size_t i = (size_t)blockIdx.x * 256u + threadIdx.x;
@@ -101,12 +102,6 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     // a pixel without a valid ray takes no part (RasterizeToPixelsFromWorld3DGSBwd.cu:157)
     inside &= pixel_world_ray(cp, (float)j + 0.5f, (float)i + 0.5f, Kmat[0], Kmat[4], Kmat[2], Kmat[5], cam, &ray_o,
                               &ray_d);
-    // v_M = v_grd (x) ray_d + v_gro (x) (ray_o - mean) (RasterizeToPixelsFromWorld3DGSBwd.cu:330-340); the epilogue
-    // adds (sum v_gro) (x) (o_ref - mean) with the start pose's centre o_ref, so under a rolling shutter the nine
-    // accumulators also take v_gro (x) (ray_o - o_ref) of this pixel
-    vec3 o_shift = mk3(0.f, 0.f, 0.f);
-    if (rolling)
-        o_shift = sub(ray_o, camera_ray_origin(load_cam_pose(viewmat)));
 
     const int32_t range_start = tile_offsets[tile_id];
     int32_t range_end = (tile_id == tile_width * tile_height - 1 && n_isects != kCountInOffsets)
@@ -252,38 +247,34 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             // the clamp at 0.999 has zero derivative (:322)
             v_alpha = (valid && a.w * vis <= 0.999f) ? v_alpha : 0.f;
             const float v_opac = vis * v_alpha;
-            // Geometry (:325-336), in the reference's order of operations: v_gro and v_grd are sums over the footprint
-            // that nearly cancel, and their fp32 rounding pattern is part of what the result is compared with (the
-            // closed form v_gro = s q, v_grd = -s (g . n) q / |grd| with q = g - (g . n) n, eight instructions
-            // shorter, differs from it by up to 6 % of the tolerance floor at rare ill-conditioned Gaussians).
-            const vec3 v_gcrod = scale(gcrod, -(a.w * v_opac)); // 2 v_gradDist, v_gradDist = -0.5 vis opac v_alpha
-            const vec3 v_grd_n = cross(gro, v_gcrod);           // = -(v_gcrod x gro)
-            const vec3 v_gro = cross(v_gcrod, grd_n);
-            // VJP of safe_normalize (Utils.cuh:186-194) with the reciprocal length from above:
-            // (v - (v . n) n) / |grd| with n = grd / |grd|
-            const float along = dot(v_grd_n, grd_n);
-            const vec3 v_grd = mk3(il * fma(-along, grd_n.x, v_grd_n.x), il * fma(-along, grd_n.y, v_grd_n.y),
-                                   il * fma(-along, grd_n.z, v_grd_n.z));
+            // Geometry (:325-345).  With n = grd / |grd|, g = gro and q = g - (g . n) n (the point of the pixel's ray
+            // nearest the Gaussian's centre, in the Gaussian's frame) the reference's chain is, exactly,
+            //   v_gro = k q,   v_grd = t v_gro,   k = -opacity v_opacity,   t = -(g . n) / |grd|,
+            // and t is the ray parameter of that nearest point p: ray_o + t ray_d = p, p - mean = M^-1 q.  Hence
+            //   v_M = v_grd (x) ray_d + v_gro (x) (ray_o - mean) = v_gro (x) (p - mean) = k q (x) M^-1 q:
+            // the two terms of the reference's sum, each ~ distance / sigma times larger than the result, cancel
+            // identically.  Only k q (for v_mean) and the symmetric k q (x) q are summed per Gaussian - small,
+            // well-conditioned terms - and the epilogue applies M^-1 once.  (The reference forms both large terms in
+            // fp32 per pair; this evaluation is closer to the exact value than the reference's own, and no ray
+            // origin appears in it: a rolling shutter needs nothing extra.)
+            // q as (n x g) x n, from the cross product the forward arithmetic already formed: it is then orthogonal
+            // to n to rounding (g - (g . n) n leaves an error ALONG n, the one direction in which the sum over a
+            // footprint should vanish, and showed 7 times the reference order's error on v_means)
+            const vec3 q = cross(gcrod, grd_n);
+            const vec3 v_gro = scale(q, -(a.w * v_opac));
             v[3] = v_gro.x;
             v[4] = v_gro.y;
             v[5] = v_gro.z;
-            v[6] = v_grd.x * ray_d.x;
-            v[7] = v_grd.x * ray_d.y;
-            v[8] = v_grd.x * ray_d.z;
-            v[9] = v_grd.y * ray_d.x;
-            v[10] = v_grd.y * ray_d.y;
-            v[11] = v_grd.y * ray_d.z;
-            v[12] = v_grd.z * ray_d.x;
-            v[13] = v_grd.z * ray_d.y;
-            v[14] = v_grd.z * ray_d.z;
+            v[6] = v_gro.x * q.x;
+            v[7] = v_gro.x * q.y;
+            v[8] = v_gro.x * q.z;
+            v[9] = v_gro.y * q.y;
+            v[10] = v_gro.y * q.z;
+            v[11] = v_gro.z * q.z;
+            v[12] = 0.f;
+            v[13] = 0.f;
+            v[14] = 0.f;
             v[15] = v_opac;
-            if (rolling) {
-                v[6] = fma(v_gro.x, o_shift.x, v[6]), v[7] = fma(v_gro.x, o_shift.y, v[7]);
-                v[8] = fma(v_gro.x, o_shift.z, v[8]), v[9] = fma(v_gro.y, o_shift.x, v[9]);
-                v[10] = fma(v_gro.y, o_shift.y, v[10]), v[11] = fma(v_gro.y, o_shift.z, v[11]);
-                v[12] = fma(v_gro.z, o_shift.x, v[12]), v[13] = fma(v_gro.z, o_shift.y, v[13]);
-                v[14] = fma(v_gro.z, o_shift.z, v[14]);
-            }
             behind = fma(-cdot, fac, behind);
 #pragma unroll
             for (uint32_t k = 0; k < NX; ++k) { // the gradients of the channels beyond the third: their own wave sums
@@ -338,7 +329,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     }
 }
 
-// Per-Gaussian epilogue: the linear map from the accumulated (v_gro, v_grd (x) ray_d) to
+// Per-Gaussian epilogue: the linear map from the accumulated (sum k q, sum k q (x) q) to
 // (v_mean, v_quat, v_scale) - quat_scale_to_preci_half_vjp / quat_to_rotmat_vjp of Utils.cuh:104-158.
 __global__ void __launch_bounds__(256) rasterize_bwd_epilogue_kernel(
     uint32_t N, const float* __restrict__ means, const float* __restrict__ quats, const float* __restrict__ scales,
@@ -358,7 +349,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_epilogue_kernel(
         const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
         row[0] = z, row[1] = z, row[2] = z, row[3] = z;
     }
-    // r0 = rgb.xyz, vo.x ; r1 = vo.y, vo.z, G00, G01 ; r2 = G02, G10, G11, G12 ; r3 = G20, G21, G22, v_opacity
+    // r0 = rgb.xyz, vo.x ; r1 = vo.y, vo.z, Sxx, Sxy ; r2 = Sxz, Syy, Syz, Szz ; r3 = -, -, -, v_opacity
     v_colors[(size_t)g * channels + 0] = r0.x;
     if (channels > 1)
         v_colors[(size_t)g * channels + 1] = r0.y;
