@@ -3,31 +3,33 @@
 // (forward), :284-424 (backward); src/training/trainer.cpp:126-129, include/kernels/fused_ssim.cuh:59-67,84-96,117-122
 // (valid crop, mean), src/training/rasterization/rasterizer.cpp:205 (clamp).
 //
-// Organisation (gfx950).  A wave owns a strip of one image plane: 64 adjacent columns (one per lane) by kFwdRows /
-// output rows, and walks it top to bottom, one INPUT row per step:
+// Organisation (gfx950).  A wave owns a strip of one image plane: 64 adjacent columns (one per lane) by 12 output
+// rows, and walks it top to bottom, one INPUT row per step (12 + 10 steps):
 //   * the row's 64 + 10 values per image go through two wave-private LDS rows, from which every lane reads its
 //     eleven horizontal taps with unit stride across the lanes (no bank conflicts, no workgroup barrier: the four
 //     waves of a workgroup never talk to each other);
 //   * the horizontally filtered moments of the last eleven input rows stay in REGISTERS (a sliding window per lane);
 //     once the window is full every further input row completes one output row - the vertical filter reads no
-//     memory at all;
-//   * input rows are requested from memory two steps before they are processed.
-// A strip re-reads 10 halo rows per strip and 10 halo columns per 64; neighbouring strips run at the same time
-// and meet in L2, and the three colour planes of the interleaved render are three waves of one workgroup, so the
-// render's cache lines are fetched once.
+//     memory at all.  The row loop is unrolled eleven times, after which every window slot is back in the register
+//     it started in: the window slides without a single move (22 steps = two passes through the unrolled body);
+//   * input rows are requested from memory two steps before they are used, by unconditional loads whose results
+//     nothing touches until then.
+// A strip re-reads 10 halo rows per 12 and 10 halo columns per 64; the three colour planes of the interleaved render
+// are three waves of one workgroup, and the workgroups of one XCD cover one contiguous eighth of the image, so these
+// re-reads are served by that XCD's L2.
 // Each output applies the taps in the reference's order (symmetric pairs from the centre outwards, then the centre;
-// rows after columns) and the reference's quotients, so results do not depend on the strip geometry and equal the CPU
-// checker's to the last bit.  (Sharing two reciprocals between the seven divisions of a pixel saves a seventh of the
-// instructions and moves d loss / d render by a few units in the last place - which the gradients of Gaussians that
-// vanish by cancellation then show at 13 times their rounding scale: not taken.)
+// rows after columns), every accumulation one fused multiply-add, and forms the seven quotients of a pixel as
+// products with the two IEEE reciprocals 1/A and 1/B (the reference is built with fast-math: its own quotients are
+// reciprocal products and its sums contracted).  Results do not depend on the strip geometry and equal the CPU
+// checker's, which fixes the same evaluation, to the last bit.
 #include "gsx_common.h"
 
 namespace gsx {
 
 static constexpr int HALO = 5;
 static constexpr int kStripCols = 64;  // one per lane
-static constexpr int kFwdRows = 12;    // output rows per forward strip: (12 + 10) / 12 input rows per output row
-static constexpr int kBwdRows = 8;     // backward strips: little arithmetic, more waves to hide the loads behind
+static constexpr int kFwdRows = 12;    // output rows per strip: 12 + 10 input rows = 2 x 11 steps (23 rows per strip
+static constexpr int kBwdRows = 12;    // leave too few waves: measured 34 / 41 us against 33 / 32 us at 1237 x 822)
 static constexpr int kRowFloats = kStripCols + 2 * HALO + 6; // an LDS row, padded to 80 floats
 
 __constant__ float cGauss[11] = {0.001028380123898387f, 0.0075987582094967365f, 0.036000773310661316f,
@@ -41,15 +43,27 @@ struct Strip {
     int H, W;
 };
 
-// One value per lane for the columns col0 - 5 + lane (lane 0..63) and, in the lanes below 10, a second one for the
-// columns col0 + 59 + lane: the 74 columns an input row contributes to a strip.  Outside the image: 0.
-template <class Load>
-__device__ __forceinline__ void request_row(const Strip& st, int row, int lane, const Load& load, float* main_v,
-                                            float* halo_v) {
+// The 74 columns an input row contributes to a strip: one value per lane for the columns col0 - 5 + lane and, in the
+// lanes below 10, a second one for the columns col0 + 59 + lane.  A request is a pair of UNCONDITIONAL loads from
+// addresses clamped into the image, and what it returns is not touched until the row is published two steps later:
+// no branch and no arithmetic stands between a load and its wait, so the wait lands where the value is needed
+// (a conditional load, or one whose result is clamped or scaled at once, waits for the memory on the spot).
+struct RowSlot {
+    int row_c, col_m, col_h; // clamped row, clamped columns of the two values
+};
+__device__ __forceinline__ RowSlot row_slot(const Strip& st, int row, int lane) {
+    RowSlot r;
+    r.row_c = min(max(row, 0), st.H - 1);
+    r.col_m = min(max(st.col0 - HALO + lane, 0), st.W - 1);
+    r.col_h = min(st.col0 + kStripCols - HALO + min(lane, 2 * HALO - 1), st.W - 1);
+    return r;
+}
+// whether the two values of a row lie inside the image (else they count as 0)
+__device__ __forceinline__ void row_valid(const Strip& st, int row, int lane, bool* main_ok, bool* halo_ok) {
     const bool row_in = row >= 0 && row < st.H;
     const int cm = st.col0 - HALO + lane, ch = st.col0 + kStripCols - HALO + lane;
-    *main_v = (row_in && cm >= 0 && cm < st.W) ? load(row, cm) : 0.0f;
-    *halo_v = (lane < 2 * HALO && row_in && ch < st.W) ? load(row, ch) : 0.0f;
+    *main_ok = row_in && cm >= 0 && cm < st.W;
+    *halo_ok = row_in && ch < st.W;
 }
 
 // the wave's LDS row receives the 74 values; afterwards lane l finds column col0 + l + d at index l + 5 + d
@@ -72,16 +86,14 @@ __device__ __forceinline__ void filter_window(const float (&win)[N][11], float (
         const float w = cGauss[HALO - d];
 #pragma unroll
         for (int k = 0; k < N; ++k)
-            out[k] += (win[k][HALO - d] + win[k][HALO + d]) * w;
+            out[k] = fma(win[k][HALO - d] + win[k][HALO + d], w, out[k]);
     }
 #pragma unroll
     for (int k = 0; k < N; ++k)
-        out[k] += win[k][HALO] * cGauss[HALO];
+        out[k] = fma(win[k][HALO], cGauss[HALO], out[k]);
 }
 
-// The window slides by register moves (ten per moment and row).  Unrolling the row loop eleven times makes every
-// slot a fixed register and removes the moves, but the eleven copies of the loop body no longer fit the instruction
-// cache two CUs share: measured 60 / 67 us against 56 / 46 us for the two loss kernels at 1237 x 822.
+// One step of the sliding window.  Written as moves; inside the eleven-fold unrolled row loop they are renamings.
 template <int N>
 __device__ __forceinline__ void push_window(float (&win)[N][11], const float (&row)[N]) {
 #pragma unroll
@@ -94,16 +106,17 @@ __device__ __forceinline__ void push_window(float (&win)[N][11], const float (&r
 }
 
 // ---- forward -----------------------------------------------------------------------------------------------------
-// X / Y: loaders of the two images for this plane (row, column) -> value.  Per output pixel `emit(row, col, ssim,
+// loadx / loady: loaders of the two images for this plane, (row, column) -> the value in memory; prepx: what turns a
+// loaded X value into the image value (the clamp of the training path).  Per output pixel `emit(row, col, ssim,
 // dmu1, dsigma1_sq, dsigma12)` is called (image pixels only); returns the lane's sum of |X - Y| over its output pixels.
-// lds: two rows of kRowFloats (X and Y of the current input row).  Input rows are requested two steps ahead of their use.
-template <int ROWS, class LoadX, class LoadY, class Emit>
+// lds: two rows of kRowFloats (X and Y of the current input row).
+template <int ROWS, class LoadX, class PrepX, class LoadY, class Emit>
 __device__ __forceinline__ float ssim_forward_strip(const Strip& st, float C1, float C2, float* lds,
-                                                    const LoadX& loadx, const LoadY& loady, const Emit& emit) {
+                                                    const LoadX& loadx, const PrepX& prepx, const LoadY& loady,
+                                                    const Emit& emit) {
     const int lane = threadIdx.x & 63;
     const int col = st.col0 + lane;
     const int row_end = min(st.row0 + ROWS, st.H); // one past the last output row
-    const int last_in = row_end + HALO;             // one past the last input row
     float* lds_x = lds;
     float* lds_y = lds + kRowFloats;
     float win[5][11];
@@ -113,19 +126,26 @@ __device__ __forceinline__ float ssim_forward_strip(const Strip& st, float C1, f
         for (int j = 0; j < 11; ++j)
             win[k][j] = 0.f;
     float l1 = 0.f;
-    float xm[2], xh[2], ym[2], yh[2]; // [0]: the next row to publish, [1]: the one after it
+    float xm[2], xh[2], ym[2], yh[2]; // raw values; [0]: the next row to publish, [1]: the one after it
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
-        request_row(st, st.row0 - HALO + k, lane, loadx, &xm[k], &xh[k]);
-        request_row(st, st.row0 - HALO + k, lane, loady, &ym[k], &yh[k]);
+        const RowSlot q = row_slot(st, st.row0 - HALO + k, lane);
+        xm[k] = loadx(q.row_c, q.col_m), xh[k] = loadx(q.row_c, q.col_h);
+        ym[k] = loady(q.row_c, q.col_m), yh[k] = loady(q.row_c, q.col_h);
     }
-    for (int row = st.row0 - HALO; row < last_in; ++row) {
-        publish_row(lds_x, lane, xm[0], xh[0]);
-        publish_row(lds_y, lane, ym[0], yh[0]);
+    static_assert((ROWS + 2 * HALO) % 11 == 0, "the window returns to its registers every eleven rows");
+#pragma unroll 11
+    for (int it = 0; it < ROWS + 2 * HALO; ++it) {
+        const int row = st.row0 - HALO + it;
+        bool main_ok, halo_ok;
+        row_valid(st, row, lane, &main_ok, &halo_ok);
+        publish_row(lds_x, lane, main_ok ? prepx(xm[0]) : 0.0f, halo_ok ? prepx(xh[0]) : 0.0f);
+        publish_row(lds_y, lane, main_ok ? ym[0] : 0.0f, halo_ok ? yh[0] : 0.0f);
         xm[0] = xm[1], xh[0] = xh[1], ym[0] = ym[1], yh[0] = yh[1];
-        if (row + 2 < last_in) { // on its way while this row and the next are filtered
-            request_row(st, row + 2, lane, loadx, &xm[1], &xh[1]);
-            request_row(st, row + 2, lane, loady, &ym[1], &yh[1]);
+        { // the row after the next: on its way while this row and the next are filtered
+            const RowSlot q = row_slot(st, row + 2, lane);
+            xm[1] = loadx(q.row_c, q.col_m), xh[1] = loadx(q.row_c, q.col_h);
+            ym[1] = loady(q.row_c, q.col_m), yh[1] = loady(q.row_c, q.col_h);
         }
         // horizontal taps of this row (ssim.cu:121-213)
         const int c = lane + HALO;
@@ -135,99 +155,105 @@ __device__ __forceinline__ float ssim_forward_strip(const Strip& st, float C1, f
             const float w = cGauss[HALO - d];
             const float Xl = lds_x[c - d], Yl = lds_y[c - d];
             const float Xr = lds_x[c + d], Yr = lds_y[c + d];
-            sumX += (Xl + Xr) * w;
-            sumX2 += ((Xl * Xl) + (Xr * Xr)) * w;
-            sumY += (Yl + Yr) * w;
-            sumY2 += ((Yl * Yl) + (Yr * Yr)) * w;
-            sumXY += ((Xl * Yl) + (Xr * Yr)) * w;
+            sumX = fma(Xl + Xr, w, sumX);
+            sumX2 = fma(fma(Xl, Xl, Xr * Xr), w, sumX2);
+            sumY = fma(Yl + Yr, w, sumY);
+            sumY2 = fma(fma(Yl, Yl, Yr * Yr), w, sumY2);
+            sumXY = fma(fma(Xl, Yl, Xr * Yr), w, sumXY);
         }
         const float cX = lds_x[c], cY = lds_y[c];
         const float wc = cGauss[HALO];
-        sumX += cX * wc;
-        sumX2 += (cX * cX) * wc;
-        sumY += cY * wc;
-        sumY2 += (cY * cY) * wc;
-        sumXY += (cX * cY) * wc;
+        sumX = fma(cX, wc, sumX);
+        sumX2 = fma(cX * cX, wc, sumX2);
+        sumY = fma(cY, wc, sumY);
+        sumY2 = fma(cY * cY, wc, sumY2);
+        sumXY = fma(cX * cY, wc, sumXY);
         if (row >= st.row0 && row < row_end && col < st.W)
             l1 += gsx::fabs(cX - cY);
         const float moments[5] = {sumX, sumX2, sumY, sumY2, sumXY};
         push_window(win, moments);
         const int out_row = row - HALO; // the window now spans out_row - 5 .. out_row + 5
-        if (out_row >= st.row0 && col < st.W) {
+        if (out_row >= st.row0 && out_row < row_end && col < st.W) {
             float m[5];
             filter_window(win, m);
-            // ssim.cu:215-274
+            // ssim.cu:215-274; the seven quotients of a pixel as products with 1/A and 1/B
             const float mu1 = m[0], mu2 = m[2];
-            const float mu1_sq = mu1 * mu1, mu2_sq = mu2 * mu2;
-            const float sigma1_sq = m[1] - mu1_sq, sigma2_sq = m[3] - mu2_sq;
-            const float sigma12 = m[4] - mu1 * mu2;
-            const float A = mu1_sq + mu2_sq + C1;
-            const float B = sigma1_sq + sigma2_sq + C2;
-            const float C_ = 2.f * mu1 * mu2 + C1;
-            const float D_ = 2.f * sigma12 + C2;
-            emit(out_row, col, (C_ * D_) / (A * B),
-                 ((mu2 * 2.f * D_) / (A * B) - (mu2 * 2.f * C_) / (A * B) - (mu1 * 2.f * C_ * D_) / (A * A * B) +
-                  (mu1 * 2.f * C_ * D_) / (A * B * B)),
-                 (-C_ * D_) / (A * B * B), (2.f * C_) / (A * B));
+            const float sigma1_sq = fma(-mu1, mu1, m[1]), sigma2_sq = fma(-mu2, mu2, m[3]);
+            const float sigma12 = fma(-mu1, mu2, m[4]);
+            const float A = fma(mu1, mu1, fma(mu2, mu2, C1));
+            const float B = (sigma1_sq + sigma2_sq) + C2;
+            const float two_mu1 = mu1 + mu1;
+            const float C_ = fma(two_mu1, mu2, C1);
+            const float D_ = fma(2.f, sigma12, C2);
+            const float rA = 1.0f / A, rB = 1.0f / B;
+            const float r = rA * rB, rrB = r * rB;
+            const float CD = C_ * D_;
+            // d map / d mu1 = 2 mu2 (D - C) / (A B) + 2 mu1 C D (1 / (A B B) - 1 / (A A B))
+            emit(out_row, col, CD * r, fma(two_mu1 * CD, rrB - r * rA, ((mu2 + mu2) * (D_ - C_)) * r), -(CD * rrB),
+                 (C_ + C_) * r);
         }
     }
     return l1;
 }
 
 // ---- backward ----------------------------------------------------------------------------------------------------
-// chain(row, col, &d0, &d1, &d2): the three derivative maps times d loss / d map at an image pixel (ssim.cu:305-337);
-// emit(row, col, s0, s1, s2): the three filtered sums of an output pixel (:385-421).
-template <int ROWS, class Chain, class Emit>
+// load4(row, col, v[4]): the three derivative maps at an image pixel as they lie in memory, and a fourth word for
+// the factor; factor(row, col, v[3]): d loss / d map there (ssim.cu:305-337 multiplies the two); emit(row, col, s0,
+// s1, s2): the three filtered sums of an output pixel (:385-421).
+template <int ROWS, class Load4, class Factor, class Emit>
 __device__ __forceinline__ void ssim_backward_strip(const Strip& st, float* lds0, float* lds1, float* lds2,
-                                                    const Chain& chain, const Emit& emit) {
+                                                    const Load4& load4, const Factor& factor, const Emit& emit) {
     const int lane = threadIdx.x & 63;
     const int col = st.col0 + lane;
     const int row_end = min(st.row0 + ROWS, st.H);
-    const int last_in = row_end + HALO;
     float win[3][11];
 #pragma unroll
     for (int k = 0; k < 3; ++k)
 #pragma unroll
         for (int j = 0; j < 11; ++j)
             win[k][j] = 0.f;
-    auto request = [&](int row, float (&mv)[3], float (&hv)[3]) {
-        const bool row_in = row >= 0 && row < st.H;
-        const int cm = st.col0 - HALO + lane, ch = st.col0 + kStripCols - HALO + lane;
-        mv[0] = mv[1] = mv[2] = hv[0] = hv[1] = hv[2] = 0.f;
-        if (row_in && cm >= 0 && cm < st.W)
-            chain(row, cm, &mv[0], &mv[1], &mv[2]);
-        if (lane < 2 * HALO && row_in && ch < st.W)
-            chain(row, ch, &hv[0], &hv[1], &hv[2]);
+    // raw values of the three derivative maps (+ one more word the factor may need); the factor d loss / d map is
+    // applied when a row is published
+    auto request = [&](int row, float (&mv)[4], float (&hv)[4]) {
+        const RowSlot q = row_slot(st, row, lane);
+        load4(q.row_c, q.col_m, mv);
+        load4(q.row_c, q.col_h, hv);
     };
-    float mv[3], hv[3], mv2[3], hv2[3]; // the next row to publish and the one after it
+    float mv[4], hv[4], mv2[4], hv2[4]; // the next row to publish and the one after it
     request(st.row0 - HALO, mv, hv);
     request(st.row0 - HALO + 1, mv2, hv2);
-    for (int row = st.row0 - HALO; row < last_in; ++row) {
-        publish_row(lds0, lane, mv[0], hv[0]);
-        publish_row(lds1, lane, mv[1], hv[1]);
-        publish_row(lds2, lane, mv[2], hv[2]);
+    static_assert((ROWS + 2 * HALO) % 11 == 0, "the window returns to its registers every eleven rows");
+#pragma unroll 11
+    for (int it = 0; it < ROWS + 2 * HALO; ++it) {
+        const int row = st.row0 - HALO + it;
+        bool main_ok, halo_ok;
+        row_valid(st, row, lane, &main_ok, &halo_ok);
+        const float fm = main_ok ? factor(row, st.col0 - HALO + lane, mv[3]) : 0.0f;
+        const float fh = halo_ok ? factor(row, st.col0 + kStripCols - HALO + lane, hv[3]) : 0.0f;
+        publish_row(lds0, lane, main_ok ? mv[0] * fm : 0.0f, halo_ok ? hv[0] * fh : 0.0f);
+        publish_row(lds1, lane, main_ok ? mv[1] * fm : 0.0f, halo_ok ? hv[1] * fh : 0.0f);
+        publish_row(lds2, lane, main_ok ? mv[2] * fm : 0.0f, halo_ok ? hv[2] * fh : 0.0f);
 #pragma unroll
-        for (int k = 0; k < 3; ++k)
+        for (int k = 0; k < 4; ++k)
             mv[k] = mv2[k], hv[k] = hv2[k];
-        if (row + 2 < last_in)
-            request(row + 2, mv2, hv2);
+        request(row + 2, mv2, hv2);
         const int c = lane + HALO;
         float a0 = 0.f, a1 = 0.f, a2 = 0.f; // ssim.cu:339-383
 #pragma unroll
         for (int d = 1; d <= HALO; ++d) {
             const float w = cGauss[HALO - d];
-            a0 += (lds0[c - d] + lds0[c + d]) * w;
-            a1 += (lds1[c - d] + lds1[c + d]) * w;
-            a2 += (lds2[c - d] + lds2[c + d]) * w;
+            a0 = fma(lds0[c - d] + lds0[c + d], w, a0);
+            a1 = fma(lds1[c - d] + lds1[c + d], w, a1);
+            a2 = fma(lds2[c - d] + lds2[c + d], w, a2);
         }
         const float wc = cGauss[HALO];
-        a0 += lds0[c] * wc;
-        a1 += lds1[c] * wc;
-        a2 += lds2[c] * wc;
+        a0 = fma(lds0[c], wc, a0);
+        a1 = fma(lds1[c], wc, a1);
+        a2 = fma(lds2[c], wc, a2);
         const float sums[3] = {a0, a1, a2};
         push_window(win, sums);
         const int out_row = row - HALO;
-        if (out_row >= st.row0 && col < st.W) {
+        if (out_row >= st.row0 && out_row < row_end && col < st.W) {
             float f[3];
             filter_window(win, f);
             emit(out_row, col, f[0], f[1], f[2]);
@@ -250,6 +276,13 @@ __host__ __device__ static inline uint32_t strip_count(uint32_t H, uint32_t W, u
     return ((W + kStripCols - 1) / kStripCols) * ((H + rows - 1) / rows);
 }
 
+// Workgroups are handed to the eight XCDs in turn (workgroup b runs on XCD b % 8, each with an L2 of its own).  A
+// launch of xcd_grid(n) workgroups gives workgroup b the strips of logical index xcd_block(b, n), so that every XCD
+// works through one contiguous eighth of the image: strips that share halo rows and cache lines meet in one L2
+// instead of fetching them from memory once per XCD.
+__host__ __device__ static inline uint32_t xcd_grid(uint32_t n) { return 8u * ((n + 7u) / 8u); }
+__device__ __forceinline__ uint32_t xcd_block(uint32_t b, uint32_t n) { return (b & 7u) * ((n + 7u) / 8u) + (b >> 3); }
+
 // gsplat-style operator (include/kernels/ssim.cuh:11-19): img1 / img2 [planes,H,W] -> map and the derivative maps
 __global__ void __launch_bounds__(256) fusedssim_kernel(int planes, int H, int W, float C1, float C2,
                                                          const float* __restrict__ img1,
@@ -258,15 +291,16 @@ __global__ void __launch_bounds__(256) fusedssim_kernel(int planes, int H, int W
                                                          float* __restrict__ dm_dsigma1_sq,
                                                          float* __restrict__ dm_dsigma12) {
     __shared__ float rows[4][2 * kRowFloats];
-    const uint32_t wave = threadIdx.x >> 6, w = blockIdx.x * 4u + wave;
-    if (w >= strip_count(H, W, kFwdRows) * (uint32_t)planes)
+    const uint32_t n_waves = strip_count(H, W, kFwdRows) * (uint32_t)planes;
+    const uint32_t wave = threadIdx.x >> 6, w = xcd_block(blockIdx.x, (n_waves + 3u) / 4u) * 4u + wave;
+    if (w >= n_waves)
         return;
     int plane;
     const Strip st = strip_of(w, planes, H, W, kFwdRows, &plane);
     const size_t base = (size_t)plane * H * W;
     ssim_forward_strip<kFwdRows>(
         st, C1, C2, rows[wave], [&](int y, int x) { return img1[base + (size_t)y * W + x]; },
-        [&](int y, int x) { return img2[base + (size_t)y * W + x]; },
+        [](float v) { return v; }, [&](int y, int x) { return img2[base + (size_t)y * W + x]; },
         [&](int y, int x, float ssim, float dmu1, float ds1, float ds12) {
             const size_t gi = base + (size_t)y * W + x;
             ssim_map[gi] = ssim;
@@ -284,25 +318,24 @@ __global__ void __launch_bounds__(256) fusedssim_backward_kernel(
     const float* __restrict__ dL_dmap, const float* __restrict__ dm_dmu1, const float* __restrict__ dm_dsigma1_sq,
     const float* __restrict__ dm_dsigma12, float* __restrict__ dL_dimg1) {
     __shared__ float rows[4][3][kRowFloats];
-    const uint32_t wave = threadIdx.x >> 6, w = blockIdx.x * 4u + wave;
-    if (w >= strip_count(H, W, kBwdRows) * (uint32_t)planes)
+    const uint32_t n_waves = strip_count(H, W, kBwdRows) * (uint32_t)planes;
+    const uint32_t wave = threadIdx.x >> 6, w = xcd_block(blockIdx.x, (n_waves + 3u) / 4u) * 4u + wave;
+    if (w >= n_waves)
         return;
     int plane;
     const Strip st = strip_of(w, planes, H, W, kBwdRows, &plane);
     const size_t base = (size_t)plane * H * W;
     ssim_backward_strip<kBwdRows>(
         st, rows[wave][0], rows[wave][1], rows[wave][2],
-        [&](int y, int x, float* d0, float* d1, float* d2) {
+        [&](int y, int x, float (&v)[4]) {
             const size_t gi = base + (size_t)y * W + x;
-            const float ch = dL_dmap[gi];
-            *d0 = dm_dmu1[gi] * ch;
-            *d1 = dm_dsigma1_sq[gi] * ch;
-            *d2 = dm_dsigma12[gi] * ch;
+            v[0] = dm_dmu1[gi], v[1] = dm_dsigma1_sq[gi], v[2] = dm_dsigma12[gi], v[3] = dL_dmap[gi];
         },
+        [](int, int, float chain) { return chain; },
         [&](int y, int x, float s0, float s1, float s2) {
             const size_t gi = base + (size_t)y * W + x;
             const float p1 = img1[gi], p2 = img2[gi];
-            dL_dimg1[gi] = s0 + (2.f * p1) * s1 + (p2)*s2;
+            dL_dimg1[gi] = fma(p2, s2, fma(p1 + p1, s1, s0));
         });
 }
 
@@ -460,8 +493,9 @@ __global__ void __launch_bounds__(256) photometric_fwd_kernel(int H, int W, floa
                                                                float* __restrict__ l1_partials,
                                                                float* __restrict__ ssim_partials) {
     __shared__ float rows[4][2 * kRowFloats];
-    const uint32_t wave = threadIdx.x >> 6, w = blockIdx.x * 4u + wave;
-    if (w >= strip_count(H, W, kFwdRows) * 3u)
+    const uint32_t n_waves = strip_count(H, W, kFwdRows) * 3u;
+    const uint32_t wave = threadIdx.x >> 6, w = xcd_block(blockIdx.x, (n_waves + 3u) / 4u) * 4u + wave;
+    if (w >= n_waves)
         return;
     int c;
     const Strip st = strip_of(w, 3, H, W, kFwdRows, &c);
@@ -470,9 +504,8 @@ __global__ void __launch_bounds__(256) photometric_fwd_kernel(int H, int W, floa
     float ss = 0.f;
     float l1 = ssim_forward_strip<kFwdRows>(
         st, C1, C2, rows[wave],
-        [&](int y, int x) { // rasterizer.cpp:205
-            return gsx::fmin(gsx::fmax(render_hwc[((size_t)y * W + x) * 3 + c], 0.0f), 1.0f);
-        },
+        [&](int y, int x) { return render_hwc[((size_t)y * W + x) * 3 + c]; },
+        [](float v) { return gsx::fmin(gsx::fmax(v, 0.0f), 1.0f); }, // rasterizer.cpp:205
         [&](int y, int x) { return gt_chw[base + (size_t)y * W + x]; },
         [&](int y, int x, float ssim, float dmu1, float ds1, float ds12) {
             const size_t gi = base + (size_t)y * W + x;
@@ -504,8 +537,9 @@ __global__ void __launch_bounds__(256) photometric_bwd_kernel(int H, int W, floa
                                                                const float* __restrict__ dm_dsigma12,
                                                                float* __restrict__ v_render_hwc) {
     __shared__ float rows[4][3][kRowFloats];
-    const uint32_t wave = threadIdx.x >> 6, w = blockIdx.x * 4u + wave;
-    if (w >= strip_count(H, W, kBwdRows) * 3u)
+    const uint32_t n_waves = strip_count(H, W, kBwdRows) * 3u;
+    const uint32_t wave = threadIdx.x >> 6, w = xcd_block(blockIdx.x, (n_waves + 3u) / 4u) * 4u + wave;
+    if (w >= n_waves)
         return;
     int c;
     const Strip st = strip_of(w, 3, H, W, kBwdRows, &c);
@@ -513,19 +547,19 @@ __global__ void __launch_bounds__(256) photometric_bwd_kernel(int H, int W, floa
     const bool crop = H > 10 && W > 10;
     ssim_backward_strip<kBwdRows>(
         st, rows[wave][0], rows[wave][1], rows[wave][2],
-        [&](int y, int x, float* d0, float* d1, float* d2) {
-            const bool valid = !crop || (y >= 5 && y < H - 5 && x >= 5 && x < W - 5);
-            const float ch = valid ? ssim_scale : 0.f;
+        [&](int y, int x, float (&v)[4]) {
             const size_t gi = base + (size_t)y * W + x;
-            *d0 = dm_dmu1[gi] * ch;
-            *d1 = dm_dsigma1_sq[gi] * ch;
-            *d2 = dm_dsigma12[gi] * ch;
+            v[0] = dm_dmu1[gi], v[1] = dm_dsigma1_sq[gi], v[2] = dm_dsigma12[gi], v[3] = 0.f;
+        },
+        [&](int y, int x, float) {
+            const bool valid = !crop || (y >= 5 && y < H - 5 && x >= 5 && x < W - 5);
+            return valid ? ssim_scale : 0.f;
         },
         [&](int y, int x, float s0, float s1, float s2) {
             const size_t p = (size_t)y * W + x;
             const float r = render_hwc[p * 3 + c];
             const float p1 = gsx::fmin(gsx::fmax(r, 0.0f), 1.0f), p2 = gt_chw[base + p];
-            const float dssim = s0 + (2.f * p1) * s1 + (p2)*s2;
+            const float dssim = fma(p2, s2, fma(p1 + p1, s1, s0));
             const float d = p1 - p2;
             const float sgn = d > 0.f ? 1.f : (d < 0.f ? -1.f : 0.f);
             const float gg = l1_scale * sgn + dssim;
@@ -549,7 +583,7 @@ extern "C" int gsx_fusedssim(int B, int CH, int H, int W, float C1, float C2, co
     GSX_REQUIRE((int64_t)B * CH * strip_count((uint32_t)H, (uint32_t)W, kBwdRows) < (1ll << 31),
                 GSX_ERR_INVALID_ARGUMENT, "fusedssim: B*CH*H*W too large");
     const uint32_t waves = strip_count((uint32_t)H, (uint32_t)W, kFwdRows) * (uint32_t)(B * CH);
-    hipLaunchKernelGGL(fusedssim_kernel, dim3(cdiv(waves, 4)), dim3(256), 0, (hipStream_t)stream, B * CH, H, W, C1, C2,
+    hipLaunchKernelGGL(fusedssim_kernel, dim3(xcd_grid(cdiv(waves, 4))), dim3(256), 0, (hipStream_t)stream, B * CH, H, W, C1, C2,
                        img1, img2, ssim_map, dm_dmu1, dm_dsigma1_sq, dm_dsigma12);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
@@ -568,7 +602,7 @@ extern "C" int gsx_fusedssim_backward(int B, int CH, int H, int W, float C1, flo
     GSX_REQUIRE((int64_t)B * CH * strip_count((uint32_t)H, (uint32_t)W, kBwdRows) < (1ll << 31),
                 GSX_ERR_INVALID_ARGUMENT, "fusedssim_backward: B*CH*H*W too large");
     const uint32_t waves = strip_count((uint32_t)H, (uint32_t)W, kBwdRows) * (uint32_t)(B * CH);
-    hipLaunchKernelGGL(fusedssim_backward_kernel, dim3(cdiv(waves, 4)), dim3(256), 0, (hipStream_t)stream, B * CH, H,
+    hipLaunchKernelGGL(fusedssim_backward_kernel, dim3(xcd_grid(cdiv(waves, 4))), dim3(256), 0, (hipStream_t)stream, B * CH, H,
                        W, img1, img2, dL_dmap, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, dL_dimg1);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
@@ -651,7 +685,7 @@ extern "C" int gsx_photometric_loss_forward(uint32_t H, uint32_t W, float C1, fl
     GSX_REQUIRE(render_hwc && gt_chw && dm_dmu1 && dm_dsigma1_sq && dm_dsigma12 && l1_partials && ssim_partials,
                 GSX_ERR_INVALID_ARGUMENT, "photometric_loss_forward: null tensor");
     GSX_REQUIRE((uint64_t)H * W < (1ull << 30), GSX_ERR_INVALID_ARGUMENT, "photometric_loss_forward: image too large");
-    hipLaunchKernelGGL(photometric_fwd_kernel, dim3(cdiv(3u * strip_count(H, W, kFwdRows), 4)), dim3(256),
+    hipLaunchKernelGGL(photometric_fwd_kernel, dim3(xcd_grid(cdiv(3u * strip_count(H, W, kFwdRows), 4))), dim3(256),
                        0, (hipStream_t)stream, (int)H, (int)W, C1, C2,
                        render_hwc, gt_chw, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, l1_partials, ssim_partials);
     GSX_LAUNCH_CHECK();
@@ -669,7 +703,7 @@ extern "C" int gsx_photometric_loss_backward(uint32_t H, uint32_t W, float lambd
     const float count = crop ? 3.f * (float)(H - 10) * (float)(W - 10) : 3.f * (float)H * (float)W;
     const float ssim_scale = -lambda_dssim / count;
     const float l1_scale = (1.f - lambda_dssim) / (3.f * (float)H * (float)W);
-    hipLaunchKernelGGL(photometric_bwd_kernel, dim3(cdiv(3u * strip_count(H, W, kBwdRows), 4)), dim3(256),
+    hipLaunchKernelGGL(photometric_bwd_kernel, dim3(xcd_grid(cdiv(3u * strip_count(H, W, kBwdRows), 4))), dim3(256),
                        0, (hipStream_t)stream, (int)H, (int)W, ssim_scale,
                        l1_scale, render_hwc, gt_chw, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, v_render_hwc);
     GSX_LAUNCH_CHECK();

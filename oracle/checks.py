@@ -3,9 +3,9 @@
 TEST INFRASTRUCTURE ONLY (tests/, __graft_entry__.smoke(), bench.py's parity leg): nothing shipped imports this.
 
 The stated bar is "gradients and Adam state within 1e-3 relative".  Every per-Gaussian gradient is a sum of signed
-per-pixel terms, and d/d(quat, scale, mean) goes through v_M = v_grd (x) ray_d + v_gro (x) (ray_o - mean), two terms
-~ (distance / sigma) times larger than their sum (RasterizeToPixelsFromWorld3DGSBwd.cu:300-345), so ANY fp32
-evaluation - the reference's own order included - misses 1e-3 relative on the elements that are small by
+per-pixel terms, and the reference forms d/d(quat, scale) through v_M = v_grd (x) ray_d + v_gro (x) (ray_o - mean), two
+terms ~ (distance / sigma) times larger than their sum (RasterizeToPixelsFromWorld3DGSBwd.cu:300-345), so an fp32
+evaluation - the reference's own order first of all - misses 1e-3 relative on the elements that are small by
 cancellation.  The float64 evaluation (orc_rasterize_bwd_f64) therefore also returns, per element, BOUND = the same
 chain evaluated with every term replaced by its absolute value: u * BOUND (u = 2^-24) is the first-order forward error
 of one rounding applied to every term, the textbook scale of what an fp32 evaluation in any order can lose.  Each check
@@ -25,11 +25,18 @@ of one rounding applied to every term, the textbook scale of what an fp32 evalua
 
 Where no BOUND exists for a tensor, step 3 uses the fp32 checker's own error as the yardstick:
 max(FLOOR_MULT * E999, MAX_MULT * EMAX), its 99.9th percentile and maximum |error| against float64 on that tensor.
-The multipliers are the smallest that pass every test of the suite with about 2 x head-room over the largest ratio
-measured: MISS_RATIO 6.5 = 2 x 3.26 and L2_MULT 8 = 2 x 4.09, both on the scale gradients of the 3 M-Gaussian
-configuration (1.19 % of the elements against the checker's 0.36 %; L2 5.8e-6 against 1.4e-6).  Cause: the kernel sums
-v_grd (x) ray_d and v_gro per Gaussian in fp32 and lets the two large terms cancel once, in its epilogue, whereas the
-checker cancels them per pair and adds the small remainders in double.  Means, colours, opacities: ratios 1.0 - 1.1.
+
+Measured over every test of the suite (operator tests of all camera models, configurations 1, 3 and 5 at full size,
+two iterations of the benchmarked path), largest figure of each kind:
+  miss fraction   GPU 1.01 x the fp32 checker's (means, opacities, colours 0.98 - 1.01; quaternions and scales 0.2 - 0.5:
+                  the kernel sums k q (x) q per Gaussian and never forms the two large terms, the checker follows the
+                  reference and cancels them in fp32 for every pair)
+  L2              GPU 1.00 x the fp32 checker's (quaternions 0.5 - 0.9, scales 0.7 - 0.9), SH coefficients up to 4.4 x on
+                  tensors whose whole error is 2.4e-7, i.e. two roundings: what L2_EPS is for
+  per element     c needed by the GPU within 1.05 x of what the fp32 checker needs (opacity gradients of long lists:
+                  215 against 214), and below 2.0 where the checker needs less than 2
+The multipliers leave head-room for the order of the atomic additions, which changes from run to run:
+MISS_RATIO 1.5, L2_MULT 2, COND_RATIO 1.5 with COND_MULT 4 as the least bar.
 """
 import numpy as np
 
@@ -38,12 +45,12 @@ from . import oracle as orc
 REL = 1e-3
 U32 = 2.0 ** -24
 COND_MULT = 4.0
-COND_RATIO = 2.0
+COND_RATIO = 1.5
 FLOOR_MULT = 8.0
 MAX_MULT = 4.0
-L2_MULT = 8.0
+L2_MULT = 2.0
 L2_EPS = 4 * 1.1920929e-07
-MISS_RATIO = 6.5
+MISS_RATIO = 1.5
 MISS_SLACK = 2e-4
 
 REPORT = []  # lines for the end-of-session summary (tests/conftest.py prints them)

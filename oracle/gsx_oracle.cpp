@@ -1360,6 +1360,11 @@ ORC_API int orc_rasterize_bwd_f64(
 // =============================================================================================
 // k9/k10  fused SSIM  src/training/kernels/ssim.cu:16-27 (window), :64-276 (fwd), :284-424 (bwd)
 // Images are [B, CH, H, W].  dm_* may be null (train == false).
+// The reference is compiled with --use_fast_math (fused multiply-adds wherever nvcc finds them, approximate
+// quotients), so the bits of its sums and quotients are not defined by its source.  This restatement fixes one
+// evaluation of the same expressions: taps in the reference's order (symmetric pairs from the centre outwards, then the
+// centre; rows after columns), every accumulation a fused multiply-add, and the seven quotients of a pixel as
+// products with the two IEEE reciprocals 1/A and 1/B.  Pinned by the float64 definitions, not by this choice.
 // =============================================================================================
 namespace {
 const float cGauss[11] = {0.001028380123898387f, 0.0075987582094967365f, 0.036000773310661316f,
@@ -1388,19 +1393,19 @@ ORC_API int orc_fusedssim(int B, int CH, int H, int W, float C1, float C2, const
                     const float w = cGauss[5 - d];
                     const float Xl = pix(img1, plane, y, x - d, H, W), Yl = pix(img2, plane, y, x - d, H, W);
                     const float Xr = pix(img1, plane, y, x + d, H, W), Yr = pix(img2, plane, y, x + d, H, W);
-                    sumX += (Xl + Xr) * w;
-                    sumX2 += ((Xl * Xl) + (Xr * Xr)) * w;
-                    sumY += (Yl + Yr) * w;
-                    sumY2 += ((Yl * Yl) + (Yr * Yr)) * w;
-                    sumXY += ((Xl * Yl) + (Xr * Yr)) * w;
+                    sumX = gsx::fma(Xl + Xr, w, sumX);
+                    sumX2 = gsx::fma(gsx::fma(Xl, Xl, Xr * Xr), w, sumX2);
+                    sumY = gsx::fma(Yl + Yr, w, sumY);
+                    sumY2 = gsx::fma(gsx::fma(Yl, Yl, Yr * Yr), w, sumY2);
+                    sumXY = gsx::fma(gsx::fma(Xl, Yl, Xr * Yr), w, sumXY);
                 }
                 const float cX = pix(img1, plane, y, x, H, W), cY = pix(img2, plane, y, x, H, W);
                 const float wc = cGauss[5];
-                sumX += cX * wc;
-                sumX2 += (cX * cX) * wc;
-                sumY += cY * wc;
-                sumY2 += (cY * cY) * wc;
-                sumXY += (cX * cY) * wc;
+                sumX = gsx::fma(cX, wc, sumX);
+                sumX2 = gsx::fma(cX * cX, wc, sumX2);
+                sumY = gsx::fma(cY, wc, sumY);
+                sumY2 = gsx::fma(cY * cY, wc, sumY2);
+                sumXY = gsx::fma(cX * cY, wc, sumXY);
                 float* o = &xconv[((size_t)y * W + x) * 5];
                 o[0] = sumX;
                 o[1] = sumX2;
@@ -1417,26 +1422,31 @@ ORC_API int orc_fusedssim(int B, int CH, int H, int W, float C1, float C2, const
                     const float* top = (y - d >= 0) ? &xconv[((size_t)(y - d) * W + x) * 5] : zero5;
                     const float* bot = (y + d < H) ? &xconv[((size_t)(y + d) * W + x) * 5] : zero5;
                     for (int k = 0; k < 5; ++k)
-                        out[k] += (top[k] + bot[k]) * w;
+                        out[k] = gsx::fma(top[k] + bot[k], w, out[k]);
                 }
                 const float* ctr = &xconv[((size_t)y * W + x) * 5];
                 for (int k = 0; k < 5; ++k)
-                    out[k] += ctr[k] * cGauss[5];
+                    out[k] = gsx::fma(ctr[k], cGauss[5], out[k]);
+                // ssim.cu:215-274 with the quotients as products of two reciprocals
                 const float mu1 = out[0], mu2 = out[2];
-                const float mu1_sq = mu1 * mu1, mu2_sq = mu2 * mu2;
-                const float sigma1_sq = out[1] - mu1_sq, sigma2_sq = out[3] - mu2_sq;
-                const float sigma12 = out[4] - mu1 * mu2;
-                const float A = mu1_sq + mu2_sq + C1;
-                const float Bv = sigma1_sq + sigma2_sq + C2;
-                const float C_ = 2.f * mu1 * mu2 + C1;
-                const float D_ = 2.f * sigma12 + C2;
+                const float sigma1_sq = gsx::fma(-mu1, mu1, out[1]), sigma2_sq = gsx::fma(-mu2, mu2, out[3]);
+                const float sigma12 = gsx::fma(-mu1, mu2, out[4]);
+                const float A = gsx::fma(mu1, mu1, gsx::fma(mu2, mu2, C1));
+                const float Bv = (sigma1_sq + sigma2_sq) + C2;
+                const float two_mu1 = mu1 + mu1;
+                const float C_ = gsx::fma(two_mu1, mu2, C1);
+                const float D_ = gsx::fma(2.f, sigma12, C2);
+                const float rA = 1.0f / A, rB = 1.0f / Bv;
+                const float r = rA * rB;
+                const float CD = C_ * D_;
                 const int64_t gi = plane + (int64_t)y * W + x;
-                ssim_map[gi] = (C_ * D_) / (A * Bv);
+                ssim_map[gi] = CD * r;
                 if (dm_dmu1) {
-                    dm_dmu1[gi] = ((mu2 * 2.f * D_) / (A * Bv) - (mu2 * 2.f * C_) / (A * Bv) -
-                                   (mu1 * 2.f * C_ * D_) / (A * A * Bv) + (mu1 * 2.f * C_ * D_) / (A * Bv * Bv));
-                    dm_dsigma1_sq[gi] = (-C_ * D_) / (A * Bv * Bv);
-                    dm_dsigma12[gi] = (2.f * C_) / (A * Bv);
+                    // 2 mu2 (D - C) / (A B) + 2 mu1 C D (1 / (A B B) - 1 / (A A B))
+                    const float rrB = r * rB;
+                    dm_dmu1[gi] = gsx::fma(two_mu1 * CD, rrB - r * rA, ((mu2 + mu2) * (D_ - C_)) * r);
+                    dm_dsigma1_sq[gi] = -(CD * rrB);
+                    dm_dsigma12[gi] = (C_ + C_) * r;
                 }
             }
     }
@@ -1466,15 +1476,15 @@ ORC_API int orc_fusedssim_backward(int B, int CH, int H, int W, float C1, float 
                     float l[3], r[3];
                     fused(x - d, l);
                     fused(x + d, r);
-                    a0 += (l[0] + r[0]) * w;
-                    a1 += (l[1] + r[1]) * w;
-                    a2 += (l[2] + r[2]) * w;
+                    a0 = gsx::fma(l[0] + r[0], w, a0);
+                    a1 = gsx::fma(l[1] + r[1], w, a1);
+                    a2 = gsx::fma(l[2] + r[2], w, a2);
                 }
                 float c[3];
                 fused(x, c);
-                a0 += c[0] * cGauss[5];
-                a1 += c[1] * cGauss[5];
-                a2 += c[2] * cGauss[5];
+                a0 = gsx::fma(c[0], cGauss[5], a0);
+                a1 = gsx::fma(c[1], cGauss[5], a1);
+                a2 = gsx::fma(c[2], cGauss[5], a2);
                 float* o = &sc[((size_t)y * W + x) * 3];
                 o[0] = a0;
                 o[1] = a1;
@@ -1489,14 +1499,14 @@ ORC_API int orc_fusedssim_backward(int B, int CH, int H, int W, float C1, float 
                     const float* top = (y - d >= 0) ? &sc[((size_t)(y - d) * W + x) * 3] : zero3;
                     const float* bot = (y + d < H) ? &sc[((size_t)(y + d) * W + x) * 3] : zero3;
                     for (int k = 0; k < 3; ++k)
-                        s[k] += (top[k] + bot[k]) * w;
+                        s[k] = gsx::fma(top[k] + bot[k], w, s[k]);
                 }
                 const float* ctr = &sc[((size_t)y * W + x) * 3];
                 for (int k = 0; k < 3; ++k)
-                    s[k] += ctr[k] * cGauss[5];
+                    s[k] = gsx::fma(ctr[k], cGauss[5], s[k]);
                 const int64_t gi = plane + (int64_t)y * W + x;
                 const float p1 = img1[gi], p2 = img2[gi];
-                dL_dimg1[gi] = s[0] + (2.f * p1) * s[1] + (p2)*s[2];
+                dL_dimg1[gi] = gsx::fma(p2, s[2], gsx::fma(p1 + p1, s[1], s[0]));
             }
     }
     return 0;

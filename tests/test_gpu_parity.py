@@ -796,8 +796,7 @@ def test_rasterizer_channel_counts(gsx, orc, cuda, channels):
     assert got5[3].shape == colors_d.shape
     for name, a, b in zip(("v_means", "v_quats", "v_scales", "v_colors", "v_opacities"), got5, o5):
         a, b = N(a).reshape(np.asarray(b).shape), np.asarray(b)
-        tol = 1e-3 if name in ("v_means", "v_colors", "v_opacities") else 5e-3  # quats / scales: see checks.py
-        assert np.abs(a - b).max() <= tol * np.abs(b).max(), f"{name}: {np.abs(a - b).max()} vs {np.abs(b).max()}"
+        assert np.abs(a - b).max() <= 1e-3 * np.abs(b).max(), f"{name}: {np.abs(a - b).max()} vs {np.abs(b).max()}"
         assert np.abs(b).max() > 0
     per_channel = np.abs(N(got5[3]) - o5[3]).reshape(-1, channels).max(0) / np.abs(o5[3]).reshape(-1, channels).max(0)
     assert per_channel.max() <= 1e-3, per_channel
