@@ -146,3 +146,19 @@ def test_oracle_training_reduces_the_loss(gsx):
     st = OracleTrainStep(sc, lambda_dssim=0.2, lrs=dict(sh0=0.05, opacity=0.05))
     losses = [st.step(cam.viewmat, cam.K, cam.width, cam.height, sc.target) for _ in range(4)]
     assert losses[-1] < losses[0] - 1e-4, losses
+
+
+def test_bench_finds_its_kernel_in_the_committed_traffic_summary():
+    """bench.py attaches the dominant kernel's measured HBM bytes from profiles/: the row it looks for must exist and
+    hold a plausible figure (the kernel's template arguments are part of the row's name)"""
+    import importlib.util
+    import os
+    import re
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("gsx_bench_module", os.path.join(root, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    src = open(os.path.join(root, "bench.py")).read()
+    prefix = re.search(r'measured_traffic_bytes\("([^"]+)"\)', src).group(1)
+    nbytes = bench.measured_traffic_bytes(prefix)
+    assert nbytes is not None and 5e7 < nbytes < 2e9, (prefix, nbytes)
