@@ -323,8 +323,16 @@ class TrainStep:
             # the previous pass's costs say something about this one only for the same camera (the same tensors)
             cam_key = (viewmat.data_ptr(), K.data_ptr(), W, H)
             if not self.have_walk or cam_key != self._walk_cam:
-                self._run("tile_order", lb.gsx_tile_order, c_i64(n), _p(self.offsets), c_p(None), c_u32(self.tw),
-                          c_u32(self.th), _p(self.tile_order), s)
+                order_args = (c_i64(n), _p(self.offsets), c_p(None), c_u32(self.tw), c_u32(self.th),
+                              _p(self.tile_order))
+                if self._lists_active and side_sh:
+                    # by list length: the offsets are complete when the tile table is, long before the pair passes
+                    # end - the order goes behind the table on the second stream, off the chain's critical path
+                    with torch.cuda.stream(self.side):
+                        self._run("tile_order", lb.gsx_tile_order, *order_args, self._stream())
+                        self.ev_join.record(self.side)
+                else:
+                    self._run("tile_order", lb.gsx_tile_order, *order_args, s)
             order = _p(self.tile_order)
         self._tile_order_arg = order
         if side_sh:
