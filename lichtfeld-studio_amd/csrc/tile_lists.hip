@@ -1,4 +1,4 @@
-// tile_lists.hip - the per-tile lists of one camera in ten launches, without the pair count crossing to the host.
+// tile_lists.hip - the per-tile lists of one camera in nine launches, without the pair count crossing to the host.
 //
 // What gsplat::intersect_tile + radix_sort_double_buffer + intersect_offset produce for one camera
 // (gsplat/Intersect.cpp:41-137, IntersectTile.cu:23-114, 206-252, 290-328) and what the rasterizers read of it:
@@ -6,8 +6,8 @@
 // element for element the one of the separate operators; the organisation is not:
 //
 //  1. depth_keys_kernel      keys (tile rectangle << 32 | depth bits) of the Gaussians that touch a tile, compacted
-//                            in index order (nine in ten Gaussians of a training view touch none);
-//                            depth_hist_kernel counts the bytes of their depth bits;
+//                            in index order (nine in ten Gaussians of a training view touch none), and the four
+//                            byte histograms of their depth bits (counted while the look-back waits);
 //  2. four chained radix passes (radix_sort.hip) order the keys by depth, one launch each;
 //  3. tile_table_kernel      +1 / -1 at every rectangle's corners in a (Th + 1) x (Tw + 1) grid and a 2-D prefix
 //                            sum over it give every tile's list length, hence tile_offsets, the pair count, and the
@@ -33,7 +33,8 @@
 
 namespace gsx {
 
-static constexpr uint32_t kKeysPerBlock = 1024; // depth_keys_kernel: 4 consecutive Gaussians per lane
+static constexpr uint32_t kKeysThreads = 1024;  // depth_keys_kernel: few, large workgroups keep the look-back short
+static constexpr uint32_t kKeysPerBlock = 4 * kKeysThreads; // 4 consecutive Gaussians per lane
 static constexpr uint32_t kTableBlocks = 32;    // tile_table_kernel: workgroups that share the corner counting
 static constexpr uint32_t kMaxLdsCells = 36 * 1024; // corner grids up to this many cells are counted in LDS
 static constexpr uint32_t kHistReplicas = 4;    // copies of the depth-byte histograms (fewer additions per address)
@@ -54,31 +55,56 @@ __device__ __forceinline__ void wave_hist_add(uint32_t* hist, uint32_t digit, bo
 
 // Keys of the Gaussians that touch a tile, in index order (a chained look-back over the workgroups' counts places
 // them).
-__global__ void __launch_bounds__(256) depth_keys_kernel(
+__global__ void __launch_bounds__(kKeysThreads) depth_keys_kernel(
     uint32_t n, const float* __restrict__ means2d, const int32_t* __restrict__ radii,
     const float* __restrict__ depths, float tile_size, uint32_t tile_width, uint32_t tile_height,
     int64_t* __restrict__ keys, int32_t* __restrict__ vals, uint32_t* __restrict__ rects,
     uint32_t* __restrict__ status /*[blocks]*/, int64_t* __restrict__ counts, uint32_t* __restrict__ error,
     uint32_t* __restrict__ clear_status, uint32_t clear_rows, uint32_t* __restrict__ clear_emit_status,
-    uint32_t clear_emit_words) {
-    __shared__ uint32_t wave_total[4];
+    uint32_t clear_emit_words, uint32_t* __restrict__ depth_hist) {
+    constexpr uint32_t kWaves = kKeysThreads / 64u;
+    __shared__ uint32_t wave_total[kWaves];
     __shared__ uint32_t base_s;
+    __shared__ uint32_t lh[4][256]; // the four byte histograms of this workgroup's depth bits
     const uint32_t t = threadIdx.x, lane = t & 63u, wv = t >> 6;
+    static_assert(kKeysThreads == 1024, "one histogram word per lane");
+    lh[t >> 8][t & 255u] = 0u;
     // housekeeping for the launches behind this one
-    for (uint32_t row = blockIdx.x; row < clear_rows; row += gridDim.x)
-        clear_status[(size_t)row * 256u + t] = 0u;
-    for (uint32_t wd = blockIdx.x * 256u + t; wd < clear_emit_words; wd += gridDim.x * 256u)
+    for (uint32_t wd = blockIdx.x * kKeysThreads + t; wd < clear_rows * 256u; wd += gridDim.x * kKeysThreads)
+        clear_status[wd] = 0u;
+    for (uint32_t wd = blockIdx.x * kKeysThreads + t; wd < clear_emit_words; wd += gridDim.x * kKeysThreads)
         clear_emit_status[wd] = 0u;
     uint32_t lo[4], hi[4];
     uint32_t mine = 0;
+    // the lane's four Gaussians: every load leaves before the first result is used (indices clamped, results
+    // discarded beyond n) - a load inside a condition would be waited for on the spot, twelve times in a row
+    const uint32_t i0 = blockIdx.x * kKeysPerBlock + t * 4u;
+    float2 m4[4];
+    int2 r4[4];
+    float d4[4];
+    if (i0 + 3u < n) {
+        const float4 ma = reinterpret_cast<const float4*>(means2d)[i0 / 2u], mb = reinterpret_cast<const float4*>(means2d)[i0 / 2u + 1u];
+        const int4 ra = reinterpret_cast<const int4*>(radii)[i0 / 2u], rb = reinterpret_cast<const int4*>(radii)[i0 / 2u + 1u];
+        const float4 dd = reinterpret_cast<const float4*>(depths)[i0 / 4u];
+        m4[0] = make_float2(ma.x, ma.y), m4[1] = make_float2(ma.z, ma.w), m4[2] = make_float2(mb.x, mb.y), m4[3] = make_float2(mb.z, mb.w);
+        r4[0] = make_int2(ra.x, ra.y), r4[1] = make_int2(ra.z, ra.w), r4[2] = make_int2(rb.x, rb.y), r4[3] = make_int2(rb.z, rb.w);
+        d4[0] = dd.x, d4[1] = dd.y, d4[2] = dd.z, d4[3] = dd.w;
+    } else {
+#pragma unroll
+        for (uint32_t k = 0; k < 4; ++k) {
+            const uint32_t i = min(i0 + k, n - 1u);
+            m4[k] = reinterpret_cast<const float2*>(means2d)[i];
+            r4[k] = reinterpret_cast<const int2*>(radii)[i];
+            d4[k] = depths[i];
+        }
+    }
 #pragma unroll
     for (uint32_t k = 0; k < 4; ++k) {
-        const uint32_t i = blockIdx.x * kKeysPerBlock + t * 4u + k;
         lo[k] = 0, hi[k] = 0;
         TileRect r;
-        if (i < n && tile_rect(means2d, radii, i, tile_size, tile_width, tile_height, &r) && r.y1 > r.y0 &&
+        if (i0 + k < n && tile_rect_of(m4[k], r4[k], tile_size, tile_width, tile_height, &r) && r.y1 > r.y0 &&
             r.x1 > r.x0) {
-            lo[k] = f2u(depths[i]);
+            lo[k] = f2u(d4[k]);
             hi[k] = r.x0 | (r.y0 << 8) | (r.x1 << 16) | (r.y1 << 24); // non-zero: x1 > x0 >= 0
             ++mine;
         }
@@ -92,11 +118,20 @@ __global__ void __launch_bounds__(256) depth_keys_kernel(
     }
     if (lane == 63)
         wave_total[wv] = incl;
-    __syncthreads();
-    const uint32_t block_total = wave_total[0] + wave_total[1] + wave_total[2] + wave_total[3];
+    __syncthreads(); // also: the histograms are zeroed
+    uint32_t block_total = 0;
+#pragma unroll
+    for (uint32_t k = 0; k < kWaves; ++k)
+        block_total += wave_total[k];
+    if (wv == 0 && lane == 0)
+        lb_publish(status + blockIdx.x, blockIdx.x == 0 ? kLbPrefix : kLbAggregate, block_total);
+    // the byte histograms do not depend on where the keys go: counted while the look-back waits
+#pragma unroll
+    for (uint32_t k = 0; k < 4; ++k)
+#pragma unroll
+        for (uint32_t b = 0; b < 4; ++b)
+            wave_hist_add(lh[b], (lo[k] >> (8u * b)) & 255u, hi[k] != 0u);
     if (wv == 0) {
-        if (lane == 0)
-            lb_publish(status + blockIdx.x, blockIdx.x == 0 ? kLbPrefix : kLbAggregate, block_total);
         const uint32_t before = lb_exclusive_wave(status, blockIdx.x, error);
         if (lane == 0) {
             if (blockIdx.x != 0)
@@ -109,7 +144,7 @@ __global__ void __launch_bounds__(256) depth_keys_kernel(
     __syncthreads();
     uint32_t pos = base_s + incl - mine;
 #pragma unroll
-    for (uint32_t k = 0; k < 4; ++k)
+    for (uint32_t k = 0; k < kWaves; ++k)
         pos += k < wv ? wave_total[k] : 0u;
 #pragma unroll
     for (uint32_t k = 0; k < 4; ++k)
@@ -119,36 +154,10 @@ __global__ void __launch_bounds__(256) depth_keys_kernel(
             rects[pos] = hi[k]; // a copy the sort does not move: the tile table is formed beside the sort
             ++pos;
         }
-}
-
-// the four byte histograms of the compacted keys' depth bits: 4096 keys per workgroup, counted in LDS, added to
-// one of kHistReplicas copies of depth_hist [4][256] (n / 4096 / kHistReplicas additions per address)
-__global__ void __launch_bounds__(256) depth_hist_kernel(const int64_t* __restrict__ keys,
-                                                          const int64_t* __restrict__ counts,
-                                                          uint32_t* __restrict__ depth_hist) {
-    __shared__ uint32_t lh[4][256];
-    const uint32_t t = threadIdx.x;
-    const uint32_t n = (uint32_t)counts[2];
-    if (blockIdx.x * 4096u >= n)
-        return;
-#pragma unroll
-    for (uint32_t b = 0; b < 4; ++b)
-        lh[b][t] = 0;
-    __syncthreads();
-#pragma unroll 4
-    for (uint32_t k = 0; k < 16; ++k) {
-        const uint32_t i = blockIdx.x * 4096u + k * 256u + t;
-        const bool live = i < n;
-        const uint32_t lo = live ? (uint32_t)(uint64_t)keys[i] : 0u;
-#pragma unroll
-        for (uint32_t b = 0; b < 4; ++b)
-            wave_hist_add(lh[b], (lo >> (8u * b)) & 255u, live);
-    }
-    __syncthreads();
-#pragma unroll
-    for (uint32_t b = 0; b < 4; ++b)
-        if (lh[b][t] != 0u)
-            atomicAdd(&depth_hist[(blockIdx.x % kHistReplicas) * 1024u + b * 256u + t], lh[b][t]);
+    // (the barrier behind the look-back also orders every wave's histogram additions before this read)
+    const uint32_t hv = lh[t >> 8][t & 255u];
+    if (hv != 0u)
+        atomicAdd(&depth_hist[(blockIdx.x % kHistReplicas) * 1024u + t], hv);
 }
 
 // Up to kTableBlocks workgroups of 1024 lanes.  Every workgroup counts the rectangle corners (+1 / -1) of its share of the
@@ -381,7 +390,10 @@ __global__ void __launch_bounds__(256) tile_emit_chained_kernel(
     if (lane == 63)
         wave_total[wv] = incl;
     __syncthreads();
-    const uint32_t block_total = wave_total[0] + wave_total[1] + wave_total[2] + wave_total[3];
+    uint32_t block_total = 0;
+#pragma unroll
+    for (uint32_t k = 0; k < 4u; ++k)
+        block_total += wave_total[k];
     if (wv == 0) {
         if (lane == 0)
             lb_publish(status + place, place == 0 ? kLbPrefix : kLbAggregate, block_total);
@@ -549,6 +561,8 @@ extern "C" int gsx_tile_lists(uint32_t N, const float* means2d, const int32_t* r
     GSX_REQUIRE(means2d && radii && depths && flatten_ids && tile_offsets, GSX_ERR_INVALID_ARGUMENT,
                 "tile_lists: null tensor");
     GSX_REQUIRE(tile_size > 0, GSX_ERR_INVALID_ARGUMENT, "tile_lists: tile_size is 0");
+    GSX_REQUIRE(((((uintptr_t)means2d) | ((uintptr_t)radii) | ((uintptr_t)depths)) & 15u) == 0, GSX_ERR_INVALID_ARGUMENT,
+                "tile_lists: means2d / radii / depths need 16-byte alignment");
     const ListsLayout L = lists_layout(N, capacity, tile_width, tile_height);
     GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 && workspace_bytes >= L.total,
                 GSX_ERR_WORKSPACE, "tile_lists: workspace needs %zu bytes, 256-byte aligned", L.total);
@@ -581,9 +595,9 @@ extern "C" int gsx_tile_lists(uint32_t N, const float* means2d, const int32_t* r
     int64_t* counts = (int64_t*)(ws + L.counts);
     hipStream_t s = (hipStream_t)stream;
 
-    hipLaunchKernelGGL(depth_keys_kernel, dim3(L.kblocks), dim3(256), 0, s, N, means2d, radii, depths,
+    hipLaunchKernelGGL(depth_keys_kernel, dim3(L.kblocks), dim3(kKeysThreads), 0, s, N, means2d, radii, depths,
                        (float)tile_size, tile_width, tile_height, keys[0], vals[0], u32p(L.rects), u32p(L.kstatus),
-                       counts, error, dstatus[0], L.drows, u32p(L.estatus), L.ewords);
+                       counts, error, dstatus[0], L.drows, u32p(L.estatus), L.ewords, u32p(L.depth_hist));
     GSX_LAUNCH_CHECK();
     // The tile table needs the rectangles only, not their depth order: with a second stream it is formed while the
     // sort runs.
@@ -610,8 +624,6 @@ extern "C" int gsx_tile_lists(uint32_t N, const float* means2d, const int32_t* r
     GSX_LAUNCH_CHECK();
     if (ts != s)
         GSX_HIP_CHECK(hipEventRecord(ev->table_done, ts));
-    hipLaunchKernelGGL(depth_hist_kernel, dim3(cdiv(N, 4096)), dim3(256), 0, s, keys[0], counts, u32p(L.depth_hist));
-    GSX_LAUNCH_CHECK();
     for (uint32_t pass = 0; pass < 4; ++pass) { // depth bits, a byte per pass; the result ends in keys[0] / vals[0]
         const uint32_t in = pass & 1u, out = in ^ 1u;
         RadixChainArgs a;
