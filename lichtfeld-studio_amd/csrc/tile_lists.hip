@@ -35,6 +35,7 @@ namespace gsx {
 
 static constexpr uint32_t kKeysThreads = 1024;  // depth_keys_kernel: few, large workgroups keep the look-back short
 static constexpr uint32_t kKeysPerBlock = 4 * kKeysThreads; // 4 consecutive Gaussians per lane
+static constexpr uint32_t kEmitThreads = 1024;  // tile_emit_chained_kernel: likewise
 static constexpr uint32_t kTableBlocks = 32;    // tile_table_kernel: workgroups that share the corner counting
 static constexpr uint32_t kMaxLdsCells = 36 * 1024; // corner grids up to this many cells are counted in LDS
 static constexpr uint32_t kHistReplicas = 4;    // copies of the depth-byte histograms (fewer additions per address)
@@ -340,34 +341,33 @@ __global__ void __launch_bounds__(1024) tile_table_kernel(
 #undef GSX_GRID
 
 // (16-bit tile index, id) pairs in depth order from the sorted keys.  Workgroup p covers sorted positions
-// [256 p, 256 p + 256); its first output position is the pair count of all positions in front of it, obtained by a
+// [1024 p, 1024 p + 1024); its first output position is the pair count of all positions in front of it, obtained by a
 // chained look-back over the workgroups' counts.  Inside the workgroup a wave flattens the runs of its 64 positions so
 // that consecutive lanes write consecutive pairs.
-__global__ void __launch_bounds__(256) tile_emit_chained_kernel(
+__global__ void __launch_bounds__(kEmitThreads) tile_emit_chained_kernel(
     const int64_t* __restrict__ sorted_keys, const int32_t* __restrict__ order, uint32_t tile_width,
     const int64_t* __restrict__ counts, uint32_t* __restrict__ status, uint16_t* __restrict__ tile_keys,
     int32_t* __restrict__ ids, uint32_t* __restrict__ clear_status, uint32_t clear_rows,
     uint32_t* __restrict__ clear_key_status, uint32_t clear_key_words, uint32_t* __restrict__ clear_depth_hist,
     uint32_t* __restrict__ error) {
-    __shared__ uint32_t s_incl[4][64], s_xy[4][64], s_w[4][64], s_idx[4][64];
-    __shared__ uint32_t wave_total[4];
+    constexpr uint32_t kWaves = kEmitThreads / 64u;
+    __shared__ uint32_t s_incl[kWaves][64], s_xy[kWaves][64], s_w[kWaves][64], s_idx[kWaves][64];
+    __shared__ uint32_t wave_total[kWaves];
     __shared__ uint32_t base_s;
     const uint32_t t = threadIdx.x, lane = t & 63u, wv = t >> 6;
     const uint32_t place = blockIdx.x;
-    for (uint32_t row = place; row < clear_rows; row += gridDim.x)
-        clear_status[(size_t)row * 256u + t] = 0u;
-    for (uint32_t wd = place * 256u + t; wd < clear_key_words; wd += gridDim.x * 256u)
+    for (uint32_t wd = place * kEmitThreads + t; wd < clear_rows * 256u; wd += gridDim.x * kEmitThreads)
+        clear_status[wd] = 0u;
+    for (uint32_t wd = place * kEmitThreads + t; wd < clear_key_words; wd += gridDim.x * kEmitThreads)
         clear_key_status[wd] = 0u;
-    if (place < kHistReplicas) {
-#pragma unroll
-        for (uint32_t k = 0; k < 4; ++k)
-            clear_depth_hist[place * 1024u + k * 256u + t] = 0u;
-    }
+    static_assert(kEmitThreads == 1024, "one histogram word per lane");
+    for (uint32_t r = place; r < kHistReplicas; r += gridDim.x)
+        clear_depth_hist[r * 1024u + t] = 0u;
     const uint32_t limit = (uint32_t)counts[0]; // 0 when the pairs do not fit: nothing is written
     const uint32_t n = (uint32_t)counts[2];     // Gaussians that touch a tile
-    if (place * 256u >= n || limit == 0)
+    if (place * kEmitThreads >= n || limit == 0)
         return; // nobody behind this workgroup needs its (empty) contribution
-    const uint32_t i = place * 256u + t;
+    const uint32_t i = place * kEmitThreads + t;
     uint32_t x0 = 0, y0 = 0, w = 0, cnt = 0, idx = 0;
     if (i < n) {
         const uint32_t hi = (uint32_t)((uint64_t)sorted_keys[i] >> 32);
@@ -392,7 +392,7 @@ __global__ void __launch_bounds__(256) tile_emit_chained_kernel(
     __syncthreads();
     uint32_t block_total = 0;
 #pragma unroll
-    for (uint32_t k = 0; k < 4u; ++k)
+    for (uint32_t k = 0; k < kWaves; ++k)
         block_total += wave_total[k];
     if (wv == 0) {
         if (lane == 0)
@@ -407,7 +407,7 @@ __global__ void __launch_bounds__(256) tile_emit_chained_kernel(
     __syncthreads();
     uint32_t wave_base = base_s;
 #pragma unroll
-    for (uint32_t k = 0; k < 4; ++k)
+    for (uint32_t k = 0; k < kWaves; ++k)
         wave_base += k < wv ? wave_total[k] : 0u;
     const uint32_t total = wave_total[wv];
     for (uint32_t k = lane; k < total; k += 64u) {
@@ -466,7 +466,7 @@ ListsLayout lists_layout(uint32_t N, int64_t capacity, uint32_t tw, uint32_t th)
     L.kblocks = cdiv(N, kKeysPerBlock);
     L.drows = radix_chained_rows(N);
     L.prows = radix_chained_rows(capacity);
-    L.ewords = cdiv(N, 256);
+    L.ewords = cdiv(N, kEmitThreads);
     L.cells = (tw + 1) * (th + 1);
     L.grid_in_lds = L.cells <= kMaxLdsCells;
     L.table_blocks = std::min(kTableBlocks, std::max(1u, N / (128u * 1024u)));
@@ -638,7 +638,7 @@ extern "C" int gsx_tile_lists(uint32_t N, const float* means2d, const int32_t* r
         GSX_HIP_CHECK(hipStreamWaitEvent(s, ev->table_done, 0));
     uint16_t* tkeys[2] = {(uint16_t*)(ws + L.tkeys0), (uint16_t*)(ws + L.tkeys1)};
     int32_t* ids[2] = {(int32_t*)(ws + L.ids0), (int32_t*)(ws + L.ids1)};
-    hipLaunchKernelGGL(tile_emit_chained_kernel, dim3(L.ewords), dim3(256), 0, s, keys[0], vals[0], tile_width,
+    hipLaunchKernelGGL(tile_emit_chained_kernel, dim3(L.ewords), dim3(kEmitThreads), 0, s, keys[0], vals[0], tile_width,
                        counts, u32p(L.estatus), tkeys[0], ids[0], pstatus[0], L.prows, u32p(L.kstatus), L.kblocks,
                        u32p(L.depth_hist), error);
     GSX_LAUNCH_CHECK();
