@@ -122,8 +122,10 @@ struct RadixChain {
     uint32_t total_replicas, total_stride; // digit_total = sum of this many tables, total_stride words apart
 };
 
-template <typename KeyT, uint32_t ITEMS, bool CHAINED, bool WRITE_KEYS>
-__global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const KeyT* __restrict__ keys_in,
+// NW waves per workgroup (a tile of 64 NW ITEMS pairs): chained passes take eight, which halves the number of places a
+// look-back walks; threads 0..255 double as the digits.
+template <typename KeyT, uint32_t ITEMS, bool CHAINED, bool WRITE_KEYS, uint32_t NW = 4>
+__global__ void __launch_bounds__(64 * NW) radix_scatter_kernel(uint32_t n, const KeyT* __restrict__ keys_in,
                                                              const int32_t* __restrict__ vals_in,
                                                              KeyT* __restrict__ keys_out,
                                                              int32_t* __restrict__ vals_out, uint32_t shift,
@@ -131,12 +133,12 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const Ke
                                                              const uint32_t* __restrict__ hist_scanned,
                                                              const uint32_t* __restrict__ digit_total,
                                                              RadixChain chain) {
-    constexpr uint32_t kTileN = 256 * ITEMS, kWaveN = 64 * ITEMS;
-    __shared__ uint32_t wave_count[4][kRadix];
+    constexpr uint32_t kThreads = 64 * NW, kTileN = kThreads * ITEMS, kWaveN = 64 * ITEMS;
+    __shared__ uint32_t wave_count[NW][kRadix];
     __shared__ uint32_t to_global[kRadix]; // global position of a pair = to_global[digit] + its slot in the tile
     __shared__ uint32_t wsum[4], gsum[4];
     // the match masks of the ranking phase and the reordered tile of the output phase share their bytes
-    constexpr uint32_t kMatchBytes = 4 * kRadix * 8, kTileBytes = kTileN * (sizeof(KeyT) + 4);
+    constexpr uint32_t kMatchBytes = NW * kRadix * 8, kTileBytes = kTileN * (sizeof(KeyT) + 4);
     __shared__ __align__(16) unsigned char overlay[kMatchBytes > kTileBytes ? kMatchBytes : kTileBytes];
     unsigned long long(*match)[kRadix] = reinterpret_cast<unsigned long long(*)[kRadix]>(overlay);
     int32_t* s_vals = reinterpret_cast<int32_t*>(overlay);
@@ -159,8 +161,9 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const Ke
         val[r] = in_buffer ? vals_in[idx] : 0;
     }
     // the digit totals are requested now as well and first used after the ranking
-    uint32_t gtot = digit_total[t]; // pairs with digit t in the whole input
-    if (CHAINED && chain.total_replicas > 1) { // up to four tables: the loads are issued together
+    const bool is_digit = NW == 4 || t < kRadix; // this thread also stands for digit t
+    uint32_t gtot = is_digit ? digit_total[t] : 0u; // pairs with digit t in the whole input
+    if (CHAINED && chain.total_replicas > 1 && is_digit) { // up to four tables: the loads are issued together
         uint32_t part[3];
 #pragma unroll
         for (uint32_t r = 0; r < 3; ++r)
@@ -174,15 +177,18 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const Ke
         }
         // housekeeping for the pass after this one (its launch starts after this one has ended)
         if (chain.clear_status != nullptr)
-            for (uint32_t row = place; row < chain.clear_rows; row += gridDim.x)
-                chain.clear_status[(size_t)row * kRadix + t] = 0u;
+            for (size_t wd = (size_t)place * kThreads + t; wd < (size_t)chain.clear_rows * kRadix;
+                 wd += (size_t)gridDim.x * kThreads)
+                chain.clear_status[wd] = 0u;
         if ((uint64_t)place * kTileN >= n)
             return; // uniform over the workgroup; later places are empty too
     }
+    if (is_digit) {
 #pragma unroll
-    for (uint32_t i = 0; i < 4; ++i) {
-        wave_count[i][t] = 0;
-        match[i][t] = 0ull;
+        for (uint32_t i = 0; i < NW; ++i) {
+            wave_count[i][t] = 0;
+            match[i][t] = 0ull;
+        }
     }
     __syncthreads();
 
@@ -222,38 +228,49 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const Ke
     // digit t: slot at which each wave's pairs with this digit start inside the tile (digits in ascending order,
     // waves in ascending order inside a digit), and the offset from tile slots to global positions
     {
-        const uint32_t c0 = wave_count[0][t], c1 = wave_count[1][t], c2 = wave_count[2][t], c3 = wave_count[3][t];
-        const uint32_t tot = c0 + c1 + c2 + c3;
-        if (CHAINED) // the first place has nobody in front of it: its counts are a complete prefix already
-            lb_publish(chain.status + (size_t)place * kRadix + t, place == 0 ? kLbPrefix : kLbAggregate, tot);
+        uint32_t c[NW];
+        uint32_t tot = 0;
+        if (is_digit) {
+#pragma unroll
+            for (uint32_t k = 0; k < NW; ++k) {
+                c[k] = wave_count[k][t];
+                tot += c[k];
+            }
+            if (CHAINED) // the first place has nobody in front of it: its counts are a complete prefix already
+                lb_publish(chain.status + (size_t)place * kRadix + t, place == 0 ? kLbPrefix : kLbAggregate, tot);
+        }
         const uint32_t incl = wave_inclusive_scan_u32(tot, lane);
         const uint32_t gincl = wave_inclusive_scan_u32(gtot, lane);
-        if (lane == 63) {
+        if (is_digit && lane == 63) {
             wsum[w] = incl;
             gsum[w] = gincl;
         }
         __syncthreads();
-        uint32_t before = 0, gbefore = 0;
+        if (is_digit) {
+            uint32_t before = 0, gbefore = 0;
 #pragma unroll
-        for (uint32_t k = 0; k < 4; ++k) {
-            before += k < w ? wsum[k] : 0u;
-            gbefore += k < w ? gsum[k] : 0u;
+            for (uint32_t k = 0; k < 4; ++k) {
+                before += k < w ? wsum[k] : 0u;
+                gbefore += k < w ? gsum[k] : 0u;
+            }
+            const uint32_t start = before + incl - tot;
+            const uint32_t smaller = gbefore + gincl - gtot; // pairs with a smaller digit
+            uint32_t run = start;
+#pragma unroll
+            for (uint32_t k = 0; k < NW; ++k) {
+                wave_count[k][t] = run;
+                run += c[k];
+            }
+            uint32_t earlier; // pairs with digit t in the workgroups in front of this one
+            if (CHAINED) {
+                earlier = lb_exclusive(chain.status, place, kRadix, t, chain.error);
+                if (place != 0)
+                    lb_publish(chain.status + (size_t)place * kRadix + t, kLbPrefix, earlier + tot);
+            } else {
+                earlier = hist_scanned[t * nblocks + blockIdx.x];
+            }
+            to_global[t] = smaller + earlier - start;
         }
-        const uint32_t start = before + incl - tot;
-        const uint32_t smaller = gbefore + gincl - gtot; // pairs with a smaller digit
-        wave_count[0][t] = start;
-        wave_count[1][t] = start + c0;
-        wave_count[2][t] = start + c0 + c1;
-        wave_count[3][t] = start + c0 + c1 + c2;
-        uint32_t earlier; // pairs with digit t in the workgroups in front of this one
-        if (CHAINED) {
-            earlier = lb_exclusive(chain.status, place, kRadix, t, chain.error);
-            if (place != 0)
-                lb_publish(chain.status + (size_t)place * kRadix + t, kLbPrefix, earlier + tot);
-        } else {
-            earlier = hist_scanned[t * nblocks + blockIdx.x];
-        }
-        to_global[t] = smaller + earlier - start;
     }
     __syncthreads();
 #pragma unroll
@@ -269,7 +286,7 @@ __global__ void __launch_bounds__(256) radix_scatter_kernel(uint32_t n, const Ke
     const uint32_t count = min(kTileN, n - tile_base);
 #pragma unroll
     for (uint32_t k = 0; k < ITEMS; ++k) {
-        const uint32_t slot = k * 256u + t;
+        const uint32_t slot = k * kThreads + t;
         if (slot < count) {
             const KeyT kk = s_keys[slot];
             const uint32_t pos = to_global[digit_of(kk, shift, mask)] + slot;
@@ -403,7 +420,10 @@ int radix_sort_pairs_32_bits(int64_t n, int64_t* keys0, int32_t* vals0, int64_t*
 
 namespace gsx {
 // ---- one launch per pass (declared in gsx_common.h) ------------------------------------------------
-// chained passes always take 4096-pair tiles: the look-back walks as many places as there are workgroups with work
+// chained passes always take the large tiles: the look-back walks as many places as there are workgroups with work.
+// The status table is sized for tiles of 4096 pairs; the passes take tiles of 64 kChainedWaves 16 pairs and use its
+// first rows.
+static constexpr uint32_t kChainedWaves = 8;
 uint32_t radix_chained_rows(int64_t n_max) { return n_max <= 0 ? 1u : cdiv((uint64_t)n_max, 256u * kItemsLarge); }
 
 namespace {
@@ -415,7 +435,7 @@ int chained_pass(uint32_t n_max, const KeyT* kin, const int32_t* vin, KeyT* kout
     GSX_REQUIRE(bits >= 1 && bits <= kRadixBits && kin && vin && vout && (kout || !write_keys) && digit_total &&
                     a.status && a.error,
                 GSX_ERR_INVALID_ARGUMENT, "chained radix pass: bad argument");
-    const uint32_t items = kItemsLarge, rows = radix_chained_rows(n_max);
+    const uint32_t items = kItemsLarge, rows = cdiv((uint64_t)n_max, 64u * kChainedWaves * kItemsLarge);
     const uint32_t mask = (1u << bits) - 1u;
     RadixChain c;
     c.n_dev = a.n_dev, c.status = a.status, c.clear_status = a.clear_status;
@@ -424,8 +444,8 @@ int chained_pass(uint32_t n_max, const KeyT* kin, const int32_t* vin, KeyT* kout
     c.total_replicas = a.total_replicas ? a.total_replicas : 1u, c.total_stride = a.total_stride;
     hipStream_t s = (hipStream_t)stream;
 #define GSX_CHAINED(IT, WK)                                                                                       \
-    hipLaunchKernelGGL((radix_scatter_kernel<KeyT, IT, true, WK>), dim3(rows), dim3(256), 0, s, n_max, kin, vin, \
-                       kout, vout, shift, mask, rows, (const uint32_t*)nullptr, digit_total, c)
+    hipLaunchKernelGGL((radix_scatter_kernel<KeyT, IT, true, WK, kChainedWaves>), dim3(rows), dim3(64 * kChainedWaves), \
+                       0, s, n_max, kin, vin, kout, vout, shift, mask, rows, (const uint32_t*)nullptr, digit_total, c)
     if (items == kItemsSmall) {
         if (write_keys)
             GSX_CHAINED(kItemsSmall, true);
