@@ -184,10 +184,8 @@ __device__ __forceinline__ void adam_one(float& p, float& m, float& v, float g, 
 // Accumulator row: r0 = rgb.xyz, vo.x ; r1 = vo.y, vo.z, Sxx, Sxy ; r2 = Sxz, Syy, Syz, Szz ; r3 = -, -, -,
 // v_opacity.  quats / scales are the ACTIVATED ones the rasterizer saw.
 // ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ void epilogue_geometry_grads(float4 r0, float4 r1, float4 r2, float4 r3,
-                                                        const float* __restrict__ viewmat, vec3 mean, quat q, vec3 s,
+__device__ __forceinline__ void epilogue_geometry_grads(float4 r0, float4 r1, float4 r2, quat q, vec3 s,
                                                         float (&vm)[3], float (&vq)[4], float (&vs)[3]) {
-    (void)viewmat, (void)mean, (void)r3;
     const mat3 R = quat_to_rotmat(q);
     const float sv[3] = {s.x, s.y, s.z};
     const float is[3] = {1.0f / s.x, 1.0f / s.y, 1.0f / s.z};

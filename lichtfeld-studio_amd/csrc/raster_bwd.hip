@@ -365,7 +365,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_epilogue_kernel(
     v_opacities[g] = r3.w;
     float vm[3] = {0.f, 0.f, 0.f}, vq[4] = {0.f, 0.f, 0.f, 0.f}, vs[3] = {0.f, 0.f, 0.f};
     if (any_geo)
-        epilogue_geometry_grads(r0, r1, r2, r3, viewmat, ld3(means, g), ld4q(quats, g), ld3(scales, g), vm, vq, vs);
+        epilogue_geometry_grads(r0, r1, r2, ld4q(quats, g), ld3(scales, g), vm, vq, vs);
 #pragma unroll
     for (int k = 0; k < 3; ++k) {
         v_means[(size_t)g * 3 + k] = vm[k];

@@ -101,7 +101,7 @@ __global__ void __launch_bounds__(256) backward_update_kernel(const UpdateArgs a
         float vm[3] = {0.f, 0.f, 0.f}, vq[4] = {0.f, 0.f, 0.f, 0.f}, vs[3] = {0.f, 0.f, 0.f};
         if (any_geo) {
             const Activated act = activate(o_raw, s_raw, q_raw);
-            epilogue_geometry_grads(r0, r1, r2, r3, a.viewmat, mean, act.quat, act.scales, vm, vq, vs);
+            epilogue_geometry_grads(r0, r1, r2, act.quat, act.scales, vm, vq, vs);
         }
         // ---- VJPs of the activations ----
         quat gq;
