@@ -153,6 +153,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
         return;
     const uint32_t num_batches = (uint32_t)(range_end - range_start + (int32_t)kBatch - 1) / kBatch;
     uint32_t n_eval = 0, n_valid = 0, n_iter = 0;
+    const uint64_t inside_mask = __builtin_amdgcn_ballot_w64(inside);
 
     for (uint32_t b = 0; b < num_batches; ++b) {
         // back to front: slot 0 of the batch is the farthest Gaussian (:211-216)
@@ -175,6 +176,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
         for (uint32_t sidx = 0; sidx < n_sel; ++sidx) {
             const int32_t t = (int32_t)wave_list[sidx];
             bool valid = inside && (batch_end - t <= bin_final);
+            const uint64_t reach_mask = __builtin_amdgcn_ballot_w64(batch_end - t <= bin_final) & inside_mask;
             if (STATS) {
                 n_eval += (uint32_t)__popcll(__builtin_amdgcn_ballot_w64(valid));
                 ++n_iter;
@@ -201,15 +203,20 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             const float grayDist = dot(gcrod, gcrod);
             const float power = -0.5f * grayDist;
             // below the record's cut-off alpha < 1/255 whatever the rounding: decided without the exp
+            // (the wave-wide tests combine the comparisons' own lane masks: a ballot of the combined flag would first
+            // turn it into a register and compare that again)
+            const uint64_t near_mask = __builtin_amdgcn_ballot_w64(!(power < cuts[t]));
             if (power < cuts[t])
                 valid = false;
-            if (__builtin_amdgcn_ballot_w64(valid) == 0)
+            if ((reach_mask & near_mask) == 0)
                 continue;
             const float vis = gsx::exp_nonpos(gsx::fmax(power, kPowerFloor)); // lanes that are not valid may be far
             const float alpha = gsx::fmin(0.999f, a.w * vis);
+            const uint64_t alpha_mask =
+                __builtin_amdgcn_ballot_w64(!(power > 0.f)) & __builtin_amdgcn_ballot_w64(!(alpha < 1.f / 255.f));
             if (power > 0.f || alpha < 1.f / 255.f)
                 valid = false;
-            if (__builtin_amdgcn_ballot_w64(valid) == 0)
+            if ((reach_mask & near_mask & alpha_mask) == 0)
                 continue; // no lane of this wave sees the Gaussian (:286-289)
             if (STATS) {
                 n_valid += (uint32_t)__popcll(__builtin_amdgcn_ballot_w64(valid));
