@@ -37,6 +37,15 @@ GSX_HD float floor(float a) { return __builtin_floorf(a); }
 GSX_HD float ceil(float a) { return __builtin_ceilf(a); }
 GSX_HD float sqrt(float a) { return __builtin_sqrtf(a); } // IEEE, correctly rounded
 GSX_HD float rcp(float a) { return 1.0f / a; }            // IEEE, correctly rounded
+// 1 / a to one unit in the last place on the GPU (v_rcp_f32), correctly rounded on the host: only for heuristics
+// whose outcome may differ between the two without changing a result (the rasterizers' conservative block test)
+GSX_HD float rcp_approx(float a) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_amdgcn_rcpf(a);
+#else
+    return 1.0f / a;
+#endif
+}
 
 GSX_HD uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
 GSX_HD float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }

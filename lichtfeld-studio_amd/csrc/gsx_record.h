@@ -129,16 +129,19 @@ GSX_HD bool record_region_hits_block(int32_t jmin, int32_t imin, int32_t jmax, i
     const float y0 = ((float)wi0 - 0.5f) - pcy, y1 = ((float)wi0 + 8.5f) - pcy;
     if (x0 <= 0.f && x1 >= 0.f && y0 <= 0.f && y1 >= 0.f)
         return true; // centre inside
-    // minimum of q over the four edges (q is convex, its unconstrained minimum lies outside the rectangle)
+    // minimum of q over the four edges (q is convex, its unconstrained minimum lies outside the rectangle).  Where
+    // along an edge the minimum lies needs no more than an approximate quotient: q is stationary there, so an error
+    // of one unit in the last place in the position changes q by its square, far inside the ellipse's 0.4 % margin
+    const float r11 = gsx::rcp_approx(a11), r00 = gsx::rcp_approx(a00);
     float qmin = 3.0e38f;
 #pragma unroll
     for (int e = 0; e < 2; ++e) {
         const float x = e ? x1 : x0;
-        float y = -(a01 * x) / a11; // minimiser along the vertical edge
+        float y = -(a01 * x) * r11; // minimiser along the vertical edge
         y = gsx::fmin(gsx::fmax(y, y0), y1);
         qmin = gsx::fmin(qmin, fma(a11 * y, y, fma(2.0f * a01 * x, y, a00 * x * x)));
         const float yy = e ? y1 : y0;
-        float xx = -(a01 * yy) / a00; // along the horizontal edge
+        float xx = -(a01 * yy) * r00; // along the horizontal edge
         xx = gsx::fmin(gsx::fmax(xx, x0), x1);
         qmin = gsx::fmin(qmin, fma(a00 * xx, xx, fma(2.0f * a01 * xx, yy, a11 * yy * yy)));
     }
