@@ -273,3 +273,27 @@ def test_mcmc_add_new_gs_bit_exact(gsx, orc, cuda):
     ref.step(cam.viewmat, cam.K, cam.width, cam.height, N(gt)[0])
     torch.cuda.synchronize()
     check_forward_bit_exact(ts, ref, min_isects=10_000)
+
+
+def test_config5_tile_lists_in_one_call(gsx, cuda):
+    """gsx_tile_lists at the stress configuration (1.7e8 pairs, tile lists up to 1e5 entries, 20 000 workgroups per
+    chained pass): flatten_ids and tile_offsets element for element those of the separate operators, which the step
+    test above holds against the CPU checker"""
+    from lichtfeld_studio_amd.trainer import TrainStep
+    from test_gpu_tile_lists import Lists
+    sc = gsx.scenes.config(5)
+    cam = sc.cameras[0]
+    ts = TrainStep(sc, cuda)
+    ts.forward(T(cam.viewmat[None], cuda), T(cam.K[None], cuda), cam.width, cam.height)
+    torch.cuda.synchronize()
+    n = ts.n_isects
+    assert n > 100_000_000
+    want_flat, want_off = ts.flatten_ids[:n].clone(), ts.offsets.reshape(-1).clone()
+    J = ts.proj
+    lists = Lists(gsx, cuda, ts.N, ts.tw, ts.th, cap=n + 4096, side=True)
+    for rep in range(2):
+        counts, err = lists.run(J["means2d"], J["radii"], J["depths"])
+        assert err == 0 and counts[0] == n and counts[1] == n, (rep, counts, err)
+        assert torch.equal(lists.flat[:n], want_flat), f"flatten_ids, call {rep}"
+        assert torch.equal(lists.off[:-1], want_off), f"tile_offsets, call {rep}"
+        assert int(lists.off[-1]) == n
