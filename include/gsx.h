@@ -501,6 +501,14 @@ GSX_API int gsx_photometric_loss_forward(uint32_t H, uint32_t W, float C1, float
 GSX_API int gsx_photometric_loss_backward(uint32_t H, uint32_t W, float lambda_dssim, const float* render_hwc,
                                           const float* gt_chw, const float* dm_dmu1, const float* dm_dsigma1_sq,
                                           const float* dm_dsigma12, float* v_render_hwc, void* stream);
+/* the same launch, which also does gsx_photometric_loss_finish's work on the way (its first workgroup adds up the
+ * forward pass's partial sums; loss_out[0..2] as there, same bits): a step that differentiates needs no launch for
+ * the loss value */
+GSX_API int gsx_photometric_loss_backward_finish(uint32_t H, uint32_t W, float lambda_dssim, const float* render_hwc,
+                                                 const float* gt_chw, const float* dm_dmu1,
+                                                 const float* dm_dsigma1_sq, const float* dm_dsigma12,
+                                                 const float* l1_partials, const float* ssim_partials,
+                                                 float* loss_out, float* v_render_hwc, void* stream);
 /* v_render [H,W,3] = d loss / d render: L1 sign term + lambda * SSIM term (dL_dimg_ssim is
  * gsx_fusedssim_backward's output for dL_dmap = -lambda / count on the valid crop, 0 elsewhere), passed through
  * the clamp VJP (zero where render < 0 or > 1) and the CHW -> HWC permute. */

@@ -407,15 +407,13 @@ __global__ void __launch_bounds__(256) ssim_valid_partials_kernel(uint32_t CH, u
         partials[blockIdx.x] = s;
 }
 
-__global__ void __launch_bounds__(256) photometric_loss_finish_kernel(uint32_t CH, uint32_t H, uint32_t W,
-                                                                       float lambda_dssim,
-                                                                       const float* __restrict__ l1_partials,
-                                                                       const float* __restrict__ ssim_partials,
-                                                                       uint32_t n_partials,
-                                                                       float* __restrict__ loss_out) {
-    __shared__ float lds[4];
+// the whole loss from the partial sums, by one workgroup of 256 lanes (contains barriers)
+__device__ __forceinline__ void loss_from_partials(uint32_t CH, uint32_t H, uint32_t W, float lambda_dssim,
+                                                   const float* __restrict__ l1_partials,
+                                                   const float* __restrict__ ssim_partials, uint32_t n_partials,
+                                                   float* __restrict__ loss_out, float* lds) {
     float a = 0.f, b = 0.f;
-    // four independent loads in flight per lane: the kernel is one block and pure latency
+    // four independent loads in flight per lane: one workgroup, pure latency
     float a4[4] = {0.f, 0.f, 0.f, 0.f}, b4[4] = {0.f, 0.f, 0.f, 0.f};
     for (uint32_t i = threadIdx.x; i < n_partials; i += 1024) {
 #pragma unroll
@@ -441,6 +439,16 @@ __global__ void __launch_bounds__(256) photometric_loss_finish_kernel(uint32_t C
         loss_out[1] = l1;
         loss_out[2] = ss;
     }
+}
+
+__global__ void __launch_bounds__(256) photometric_loss_finish_kernel(uint32_t CH, uint32_t H, uint32_t W,
+                                                                       float lambda_dssim,
+                                                                       const float* __restrict__ l1_partials,
+                                                                       const float* __restrict__ ssim_partials,
+                                                                       uint32_t n_partials,
+                                                                       float* __restrict__ loss_out) {
+    __shared__ float lds[4];
+    loss_from_partials(CH, H, W, lambda_dssim, l1_partials, ssim_partials, n_partials, loss_out, lds);
 }
 
 // dL/dmap of mean(map[valid crop]) scaled: `scale` inside the crop, 0 outside (fused_ssim.cuh:84-96)
@@ -535,8 +543,19 @@ __global__ void __launch_bounds__(256) photometric_bwd_kernel(int H, int W, floa
                                                                const float* __restrict__ dm_dmu1,
                                                                const float* __restrict__ dm_dsigma1_sq,
                                                                const float* __restrict__ dm_dsigma12,
-                                                               float* __restrict__ v_render_hwc) {
+                                                               float* __restrict__ v_render_hwc,
+                                                               float lambda_dssim,
+                                                               const float* __restrict__ l1_partials,
+                                                               const float* __restrict__ ssim_partials,
+                                                               uint32_t n_partials, float* __restrict__ loss_out) {
     __shared__ float rows[4][3][kRowFloats];
+    if (loss_out != nullptr && blockIdx.x == 0) {
+        // the loss value itself, which only gets reported: the forward kernel's partial sums are complete when this
+        // launch starts, so its first workgroup adds them up on the way (no launch and no stream of its own)
+        __shared__ float lds[4];
+        loss_from_partials(3u, (uint32_t)H, (uint32_t)W, lambda_dssim, l1_partials, ssim_partials, n_partials,
+                           loss_out, lds);
+    }
     const uint32_t n_waves = strip_count(H, W, kBwdRows) * 3u;
     const uint32_t wave = threadIdx.x >> 6, w = xcd_block(blockIdx.x, (n_waves + 3u) / 4u) * 4u + wave;
     if (w >= n_waves)
@@ -692,20 +711,42 @@ extern "C" int gsx_photometric_loss_forward(uint32_t H, uint32_t W, float C1, fl
     return GSX_OK;
 }
 
-extern "C" int gsx_photometric_loss_backward(uint32_t H, uint32_t W, float lambda_dssim, const float* render_hwc,
-                                             const float* gt_chw, const float* dm_dmu1, const float* dm_dsigma1_sq,
-                                             const float* dm_dsigma12, float* v_render_hwc, void* stream) {
+static int photometric_backward(uint32_t H, uint32_t W, float lambda_dssim, const float* render_hwc,
+                                const float* gt_chw, const float* dm_dmu1, const float* dm_dsigma1_sq,
+                                const float* dm_dsigma12, float* v_render_hwc, const float* l1_partials,
+                                const float* ssim_partials, float* loss_out, void* stream) {
     if ((uint64_t)H * W == 0)
         return GSX_OK;
     GSX_REQUIRE(render_hwc && gt_chw && dm_dmu1 && dm_dsigma1_sq && dm_dsigma12 && v_render_hwc,
                 GSX_ERR_INVALID_ARGUMENT, "photometric_loss_backward: null tensor");
+    GSX_REQUIRE(loss_out == nullptr || (l1_partials && ssim_partials), GSX_ERR_INVALID_ARGUMENT,
+                "photometric_loss_backward: the loss needs the forward pass's partial sums");
     const bool crop = H > 10 && W > 10;
     const float count = crop ? 3.f * (float)(H - 10) * (float)(W - 10) : 3.f * (float)H * (float)W;
     const float ssim_scale = -lambda_dssim / count;
     const float l1_scale = (1.f - lambda_dssim) / (3.f * (float)H * (float)W);
     hipLaunchKernelGGL(photometric_bwd_kernel, dim3(xcd_grid(cdiv(3u * strip_count(H, W, kBwdRows), 4))), dim3(256),
                        0, (hipStream_t)stream, (int)H, (int)W, ssim_scale,
-                       l1_scale, render_hwc, gt_chw, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, v_render_hwc);
+                       l1_scale, render_hwc, gt_chw, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, v_render_hwc, lambda_dssim,
+                       l1_partials, ssim_partials, gsx_photometric_partials(H, W), loss_out);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
+}
+
+extern "C" int gsx_photometric_loss_backward(uint32_t H, uint32_t W, float lambda_dssim, const float* render_hwc,
+                                             const float* gt_chw, const float* dm_dmu1, const float* dm_dsigma1_sq,
+                                             const float* dm_dsigma12, float* v_render_hwc, void* stream) {
+    return photometric_backward(H, W, lambda_dssim, render_hwc, gt_chw, dm_dmu1, dm_dsigma1_sq, dm_dsigma12,
+                                v_render_hwc, nullptr, nullptr, nullptr, stream);
+}
+
+extern "C" int gsx_photometric_loss_backward_finish(uint32_t H, uint32_t W, float lambda_dssim,
+                                                    const float* render_hwc, const float* gt_chw,
+                                                    const float* dm_dmu1, const float* dm_dsigma1_sq,
+                                                    const float* dm_dsigma12, const float* l1_partials,
+                                                    const float* ssim_partials, float* loss_out,
+                                                    float* v_render_hwc, void* stream) {
+    GSX_REQUIRE(loss_out != nullptr, GSX_ERR_INVALID_ARGUMENT, "photometric_loss_backward_finish: loss_out is null");
+    return photometric_backward(H, W, lambda_dssim, render_hwc, gt_chw, dm_dmu1, dm_dsigma1_sq, dm_dsigma12,
+                                v_render_hwc, l1_partials, ssim_partials, loss_out, stream);
 }

@@ -419,26 +419,32 @@ class TrainStep:
         return (tiles << 32) | (depth.to(torch.int64) & 0xFFFFFFFF)
 
     # -- loss ---------------------------------------------------------------------------------------
-    def loss_forward(self, gt_chw):
-        """image = clamp(render, 0, 1) CHW; loss = (1-l) L1 + l (1 - SSIM_valid); result stays on the device."""
+    def loss_forward(self, gt_chw, finish=True):
+        """image = clamp(render, 0, 1) CHW; loss = (1-l) L1 + l (1 - SSIM_valid); result stays on the device.
+        finish = False (fused loss only): the loss value is left to backward(), whose loss kernel adds the partial
+        sums up on the way."""
         lb, s, H, W = self.lib, self._stream(), self.H, self.W
         self.gt = gt_chw
+        self._loss_due = False
         if self.fused_loss:
             self._run("photometric_loss_forward", lb.gsx_photometric_loss_forward, c_u32(H), c_u32(W),
                       c_f(0.01 ** 2), c_f(0.03 ** 2), _p(self.render), _p(gt_chw), _p(self.dm1), _p(self.dm2),
                       _p(self.dm3), _p(self.l1_partials), _p(self.ssim_partials), s)
             fin = (c_u32(3), c_u32(H), c_u32(W), c_f(self.lambda_dssim), _p(self.l1_partials), _p(self.ssim_partials),
                    c_u32(self.n_partials_fused), _p(self.loss_out))
+            self._loss_due = not finish
             if self.side is None:
-                self._run("photometric_loss_finish", lb.gsx_photometric_loss_finish, *fin, s)
+                if finish:
+                    self._run("photometric_loss_finish", lb.gsx_photometric_loss_finish, *fin, s)
             else:  # the value is only reported: its reduction runs beside the backward pass
                 self.ev_loss_fork.record(torch.cuda.current_stream(self.dev))
                 self.side.wait_event(self.ev_loss_fork)
                 with torch.cuda.stream(self.side):
                     self._order_on_side_stream()  # the backward pass waits for this one, not for the reduction
-                    self._run("photometric_loss_finish", lb.gsx_photometric_loss_finish, *fin, self._stream())
-                    self.ev_loss_join.record(self.side)
-                self.loss_pending = True
+                    if finish:
+                        self._run("photometric_loss_finish", lb.gsx_photometric_loss_finish, *fin, self._stream())
+                        self.ev_loss_join.record(self.side)
+                self.loss_pending = finish
             return self.loss_out
         self._run("image_from_render", lb.gsx_image_from_render, c_u32(H), c_u32(W), _p(self.render), _p(gt_chw), _p(self.image),
                                        _p(self.l1_partials), s)
@@ -459,7 +465,12 @@ class TrainStep:
         lb, s, N, H, W = self.lib, self._stream(), self.N, self.H, self.W
         P, A, J, G, V = self.params, self.act, self.proj, self.grads, self.v_act
         dimg = None
-        if self.fused_loss:
+        if self.fused_loss and getattr(self, "_loss_due", False):
+            self._run("photometric_loss_backward", lb.gsx_photometric_loss_backward_finish, c_u32(H), c_u32(W),
+                      c_f(self.lambda_dssim), _p(self.render), _p(self.gt), _p(self.dm1), _p(self.dm2), _p(self.dm3),
+                      _p(self.l1_partials), _p(self.ssim_partials), _p(self.loss_out), _p(self.v_render), s)
+            self._loss_due = False
+        elif self.fused_loss:
             self._run("photometric_loss_backward", lb.gsx_photometric_loss_backward, c_u32(H), c_u32(W),
                       c_f(self.lambda_dssim), _p(self.render), _p(self.gt), _p(self.dm1), _p(self.dm2), _p(self.dm3),
                       _p(self.v_render), s)
@@ -610,7 +621,7 @@ class TrainStep:
         self._check_capacity()
         self.iteration += 1
         self.forward(viewmat, K, W, H)
-        self.loss_forward(gt_chw)
+        self.loss_forward(gt_chw, finish=not self.fused_loss)
         self.backward()
         self.adam()
         if self.loss_pending:  # the next step's loss pass overwrites the partial sums: rejoin the side stream

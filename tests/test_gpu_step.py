@@ -278,6 +278,45 @@ def test_pair_count_on_the_device_changes_nothing(gsx, cuda):
     assert b.lists_error() == (0, 0)
 
 
+def test_loss_value_from_the_backward_loss_kernel(gsx, cuda):
+    """a whole step leaves the loss reduction to the backward loss kernel (its first workgroup adds up the partial
+    sums): loss, L1 and SSIM terms, d loss / d render and the parameters equal, bit for bit, those of the path with
+    the separate reduction launch"""
+    from lichtfeld_studio_amd.trainer import TrainStep
+    sc = gsx.scenes.config(3, 20_000)
+    sc.scaling_raw += 1.2
+    cam = gsx.scenes.orbit_camera(0.7, 4.0, 309, 205, 287.0)
+    W, H = cam.width, cam.height
+    vm = torch.from_numpy(cam.viewmat[None].copy()).to(cuda)
+    Km = torch.from_numpy(cam.K[None].copy()).to(cuda)
+    gt = torch.rand((1, 3, H, W), generator=torch.Generator().manual_seed(5)).to(cuda)
+    for overlap in (False, True):
+        a = TrainStep(sc, cuda, fused_update=True, fused_loss=True, overlap=overlap)
+        b = TrainStep(sc, cuda, fused_update=True, fused_loss=True, overlap=overlap)
+        for it in range(2):
+            a.iteration += 1
+            a.forward(vm, Km, W, H)
+            a.loss_forward(gt)  # with its own reduction launch
+            a.backward()
+            b.iteration += 1
+            b.forward(vm, Km, W, H)
+            b.loss_out.fill_(-1.0)
+            b.loss_forward(gt, finish=False)
+            b.backward()
+            torch.cuda.synchronize()
+            assert torch.equal(a.loss_out, b.loss_out) and float(b.loss_out[0]) > 0, (overlap, it)
+            assert torch.equal(a.v_render, b.v_render)
+            b.ws_bwd.copy_(a.ws_bwd)
+            for ts in (a, b):
+                ts.adam()
+                if ts.loss_pending:
+                    torch.cuda.current_stream(cuda).wait_event(ts.ev_loss_join)
+                    ts.loss_pending = False
+        torch.cuda.synchronize()
+        for k in a.params:
+            assert torch.equal(a.params[k], b.params[k]), k
+
+
 def test_pairs_outgrowing_the_buffers_hold_the_step_back(gsx, cuda):
     """count on the device, and a camera that suddenly sees several times the pairs the buffers hold: that step
     renders nothing, the optimiser leaves parameters and moments untouched, and the next step starts with larger
