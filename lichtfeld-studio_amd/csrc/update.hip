@@ -56,7 +56,8 @@ __device__ __forceinline__ void adam_row(float* __restrict__ P, float* __restric
 
 template <bool LDS16>
 __global__ void __launch_bounds__(256) backward_update_kernel(const UpdateArgs a_in) {
-    __shared__ float4 lds[LDS16 ? 4 * 32 * kShLdsF4 : 1];
+    constexpr uint32_t kGradF4 = 5; // what a lane leaves for the coefficient update: 16 basis values, 3 colour gradients, nb
+    __shared__ float4 lds[LDS16 ? 4 * 64 * kGradF4 : 1];
     const uint32_t e = blockIdx.x * 256u + threadIdx.x;
     UpdateArgs a = a_in;
     if (a.step_scalars != nullptr) { // a replayed launch takes the step's scalars from memory
@@ -77,7 +78,7 @@ __global__ void __launch_bounds__(256) backward_update_kernel(const UpdateArgs a
         return;
     }
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    float4* wave_lds = lds + (LDS16 ? wave * 32 * kShLdsF4 : 0);
+    float4* wave_lds = lds + (LDS16 ? wave * 64 * kGradF4 : 0);
     const bool in = e < a.N;
 
     float B[25];
@@ -137,79 +138,102 @@ __global__ void __launch_bounds__(256) backward_update_kernel(const UpdateArgs a
 
     // ---- Adam on the SH tensor; gradient of coefficient (k, c) = B[k] * vc[c] for k < nb, else 0 ----
     // The update is elementwise, so the parameter and both moments are processed where they lie, with coalesced
-    // 16-byte accesses; only the gradient rows (one per lane) are turned into that layout through LDS, 32 rows at a
-    // time.  Position q of a half = float4 (q % 12) of row (q / 12).
+    // 16-byte accesses: position q of a wave's 64 rows = float4 (q % 12) of row (q / 12).  The gradient is an outer
+    // product, so a lane leaves only its 16 basis values, its three colour gradients and nb in LDS (5 float4) and
+    // the lane that owns position q rebuilds the four gradient elements there - the same products B[k] * vc[c].
+    // The bytes are streamed in four batches of 3 x 3 float4 per lane; the requests of a batch leave before the
+    // batch in front of it is worked on, so that every wave keeps 18 KiB of reads in flight.
     if (LDS16) {
         const uint32_t row0 = blockIdx.x * 256u + wave * 64u;
         if (row0 >= a.N)
             return; // whole wave out of range
-        const bool skip = a.skip_shN != 0;
-        const uint32_t n_f4 = min(64u, a.N - row0) * kShRowF4;
+        const uint32_t rows = min(64u, a.N - row0), n_f4 = rows * kShRowF4;
+        float4* __restrict__ P4 = reinterpret_cast<float4*>(a.shs) + (size_t)row0 * kShRowF4;
+        float4* __restrict__ M4 = reinterpret_cast<float4*>(a.m_shs) + (size_t)row0 * kShRowF4;
+        float4* __restrict__ V4 = reinterpret_cast<float4*>(a.v_shs) + (size_t)row0 * kShRowF4;
+        if (a.skip_shN != 0) {
+            // the higher bands are frozen: only the DC coefficient (elements 0..2 of a row) moves; lane = row
+            if (lane < rows) {
+                const uint32_t q = lane * kShRowF4;
+                float4 p = load_streaming(P4 + q), m = load_streaming(M4 + q), v = load_streaming(V4 + q);
+                float* pv = reinterpret_cast<float*>(&p);
+                float* mv = reinterpret_cast<float*>(&m);
+                float* vv = reinterpret_cast<float*>(&v);
 #pragma unroll
-        for (uint32_t half = 0; half < 2; ++half) {
-            if ((lane >> 5) == half) {
-#pragma unroll
-                for (uint32_t j = 0; j < kShRowF4; ++j) {
-                    float t[4];
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const int i = 4 * (int)j + q, k = i / 3, c = i - 3 * k;
-                        t[q] = k < nb ? B[k] * vc[c] : 0.f;
-                    }
-                    wave_lds[(lane & 31u) * kShLdsF4 + j] = make_float4(t[0], t[1], t[2], t[3]);
+                for (int t = 0; t < 3; ++t) {
+                    const float g = nb > 0 ? B[0] * vc[t] : 0.f;
+                    const float m1 = adam_m(mv[t], g, a.beta1);
+                    const float v1 = adam_v(vv[t], g, a.beta2);
+                    pv[t] = adam_p(pv[t], m1, v1, a.lr_sh0, a.eps, a.bc1_rcp, a.bc2_sqrt_rcp);
+                    mv[t] = m1;
+                    vv[t] = v1;
                 }
+                store_streaming(P4 + q, p);
+                store_streaming(M4 + q, m);
+                store_streaming(V4 + q, v);
             }
-            __builtin_amdgcn_wave_barrier();
-            const uint32_t base = half * 32u * kShRowF4; // first float4 of this half inside the wave's rows
-            const size_t g0 = (size_t)row0 * kShRowF4 + base;
-            float4* __restrict__ P4 = reinterpret_cast<float4*>(a.shs) + g0;
-            float4* __restrict__ M4 = reinterpret_cast<float4*>(a.m_shs) + g0;
-            float4* __restrict__ V4 = reinterpret_cast<float4*>(a.v_shs) + g0;
-            constexpr uint32_t kPer = 3; // float4 per lane and batch (two batches per half)
-#pragma unroll 1
-            for (uint32_t batch = 0; batch < 2; ++batch) {
-            float4 p4[kPer], m4[kPer], v4[kPer];
-            bool act[kPer];
+            return;
+        }
+        constexpr uint32_t kPer = 3, kBatches = kShRowF4 / kPer; // float4 per lane, array and batch
+        float4 p4[2][kPer], m4[2][kPer], v4[2][kPer];
+        // requests of a batch: unconditional, from addresses clamped into the wave's rows
+        auto request = [&](uint32_t batch, uint32_t buf) {
 #pragma unroll
-            for (uint32_t i = 0; i < kPer; ++i) { // the batch's requests leave before the first result is used
-                const uint32_t q = (batch * kPer + i) * 64u + lane;
-                const uint32_t col = q - ((q * 43691u) >> 19) * kShRowF4;
-                // with the higher bands frozen only the first float4 of a row (DC + one more element) is touched
-                act[i] = base + q < n_f4 && !(skip && col != 0);
-                if (act[i]) { // read once, written once: streamed past the caches
-                    p4[i] = load_streaming(P4 + q);
-                    m4[i] = load_streaming(M4 + q);
-                    v4[i] = load_streaming(V4 + q);
-                }
+            for (uint32_t i = 0; i < kPer; ++i) {
+                const uint32_t q = min((batch * kPer + i) * 64u + lane, n_f4 - 1u);
+                p4[buf][i] = load_streaming(P4 + q);
+                m4[buf][i] = load_streaming(M4 + q);
+                v4[buf][i] = load_streaming(V4 + q);
             }
+        };
+        request(0, 0);
+        {
+            float4* mine = wave_lds + lane * kGradF4;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                mine[j] = make_float4(4 * j + 0 < nb ? B[4 * j + 0] : 0.f, 4 * j + 1 < nb ? B[4 * j + 1] : 0.f,
+                                      4 * j + 2 < nb ? B[4 * j + 2] : 0.f, 4 * j + 3 < nb ? B[4 * j + 3] : 0.f);
+            mine[4] = make_float4(vc[0], vc[1], vc[2], __int_as_float(nb));
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (uint32_t batch = 0; batch < kBatches; ++batch) {
+            const uint32_t cur = batch & 1u;
+            if (batch + 1 < kBatches)
+                request(batch + 1, cur ^ 1u);
 #pragma unroll
             for (uint32_t i = 0; i < kPer; ++i) {
                 const uint32_t q = (batch * kPer + i) * 64u + lane;
-                const uint32_t r = (q * 43691u) >> 19, col = q - r * kShRowF4;
-                if (!act[i])
-                    continue;
-                const float4 g4 = wave_lds[r * kShLdsF4 + col];
-                const float* gv = reinterpret_cast<const float*>(&g4);
-                float* pv = reinterpret_cast<float*>(&p4[i]);
-                float* mv = reinterpret_cast<float*>(&m4[i]);
-                float* vv = reinterpret_cast<float*>(&v4[i]);
+                const uint32_t r = (q * 43691u) >> 19, col = q - r * kShRowF4; // q / 12 for q < 768
+                // elements 4 col .. 4 col + 3 of the row: coefficient k0 from colour c0 on, then coefficient k0 + 1
+                const uint32_t i0 = 4u * col, k0 = (i0 * 43u) >> 7 /* i0 / 3 for i0 <= 44 */, c0 = i0 - 3u * k0;
+                const float* gf = reinterpret_cast<const float*>(wave_lds + r * kGradF4);
+                const float b0 = gf[k0], b1 = gf[k0 + 1u];
+                const float4 cv = wave_lds[r * kGradF4 + 4u];
+                const int row_nb = __float_as_int(cv.w);
+                float* pv = reinterpret_cast<float*>(&p4[cur][i]);
+                float* mv = reinterpret_cast<float*>(&m4[cur][i]);
+                float* vv = reinterpret_cast<float*>(&v4[cur][i]);
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    const bool dc = col == 0 && t < 3; // elements 0..2 of a row: the DC coefficient
-                    if (!dc && skip)
-                        continue;
-                    const float m1 = adam_m(mv[t], gv[t], a.beta1);
-                    const float v1 = adam_v(vv[t], gv[t], a.beta2);
+                for (uint32_t t = 0; t < 4; ++t) {
+                    const uint32_t idx = c0 + t; // 0..5
+                    const bool next = idx >= 3u;
+                    const uint32_t c = next ? idx - 3u : idx;
+                    const float colour = c == 0u ? cv.x : (c == 1u ? cv.y : cv.z);
+                    const float gv = (int)(k0 + (next ? 1u : 0u)) < row_nb ? (next ? b1 : b0) * colour : 0.f;
+                    const bool dc = col == 0u && t < 3u; // elements 0..2 of a row: the DC coefficient
+                    const float m1 = adam_m(mv[t], gv, a.beta1);
+                    const float v1 = adam_v(vv[t], gv, a.beta2);
                     pv[t] = adam_p(pv[t], m1, v1, dc ? a.lr_sh0 : a.lr_shN, a.eps, a.bc1_rcp, a.bc2_sqrt_rcp);
                     mv[t] = m1;
                     vv[t] = v1;
                 }
-                store_streaming(P4 + q, p4[i]);
-                store_streaming(M4 + q, m4[i]);
-                store_streaming(V4 + q, v4[i]);
+                if (q < n_f4) {
+                    store_streaming(P4 + q, p4[cur][i]);
+                    store_streaming(M4 + q, m4[cur][i]);
+                    store_streaming(V4 + q, v4[cur][i]);
+                }
             }
-            }
-            __builtin_amdgcn_wave_barrier();
         }
         return;
     }
