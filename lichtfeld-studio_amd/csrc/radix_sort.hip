@@ -122,8 +122,8 @@ struct RadixChain {
     uint32_t total_replicas, total_stride; // digit_total = sum of this many tables, total_stride words apart
 };
 
-// NW waves per workgroup (a tile of 64 NW ITEMS pairs): chained passes take eight, which halves the number of places a
-// look-back walks; threads 0..255 double as the digits.
+// NW waves per workgroup (a tile of 64 NW ITEMS pairs): chained passes take eight or sixteen, for tiles of 8192 pairs -
+// half as many places for a look-back to walk; threads 0..255 double as the digits.
 template <typename KeyT, uint32_t ITEMS, bool CHAINED, bool WRITE_KEYS, uint32_t NW = 4>
 __global__ void __launch_bounds__(64 * NW) radix_scatter_kernel(uint32_t n, const KeyT* __restrict__ keys_in,
                                                              const int32_t* __restrict__ vals_in,
@@ -420,10 +420,16 @@ int radix_sort_pairs_32_bits(int64_t n, int64_t* keys0, int32_t* vals0, int64_t*
 
 namespace gsx {
 // ---- one launch per pass (declared in gsx_common.h) ------------------------------------------------
-// chained passes always take the large tiles: the look-back walks as many places as there are workgroups with work.
-// The status table is sized for tiles of 4096 pairs; the passes take tiles of 64 kChainedWaves 16 pairs and use its
-// first rows.
-static constexpr uint32_t kChainedWaves = 8;
+// chained passes always take tiles of kChainedTile pairs: the look-back walks as many places as there are workgroups
+// with work.  (The status table is sized for tiles of 4096 pairs; the passes use its first rows.)  A pass is bound by
+// the latency of what one wave does one thing after the other - ranking, reordering and writing its share of the
+// tile - so the 64-bit passes (one workgroup per CU either way) split the tile over sixteen waves of 8 pairs per lane;
+// the 16-bit passes keep eight waves of 16, of which two workgroups fit a CU.
+static constexpr uint32_t kChainedTile = 8192;
+template <typename KeyT>
+struct ChainedShape {
+    static constexpr uint32_t kWaves = sizeof(KeyT) == 8 ? 16 : 8, kItems = kChainedTile / (64 * kWaves);
+};
 uint32_t radix_chained_rows(int64_t n_max) { return n_max <= 0 ? 1u : cdiv((uint64_t)n_max, 256u * kItemsLarge); }
 
 namespace {
@@ -435,7 +441,7 @@ int chained_pass(uint32_t n_max, const KeyT* kin, const int32_t* vin, KeyT* kout
     GSX_REQUIRE(bits >= 1 && bits <= kRadixBits && kin && vin && vout && (kout || !write_keys) && digit_total &&
                     a.status && a.error,
                 GSX_ERR_INVALID_ARGUMENT, "chained radix pass: bad argument");
-    const uint32_t items = kItemsLarge, rows = cdiv((uint64_t)n_max, 64u * kChainedWaves * kItemsLarge);
+    const uint32_t rows = cdiv((uint64_t)n_max, kChainedTile);
     const uint32_t mask = (1u << bits) - 1u;
     RadixChain c;
     c.n_dev = a.n_dev, c.status = a.status, c.clear_status = a.clear_status;
@@ -443,20 +449,15 @@ int chained_pass(uint32_t n_max, const KeyT* kin, const int32_t* vin, KeyT* kout
     GSX_REQUIRE(a.total_replicas <= 4, GSX_ERR_INVALID_ARGUMENT, "chained radix pass: at most 4 total tables");
     c.total_replicas = a.total_replicas ? a.total_replicas : 1u, c.total_stride = a.total_stride;
     hipStream_t s = (hipStream_t)stream;
-#define GSX_CHAINED(IT, WK)                                                                                       \
-    hipLaunchKernelGGL((radix_scatter_kernel<KeyT, IT, true, WK, kChainedWaves>), dim3(rows), dim3(64 * kChainedWaves), \
-                       0, s, n_max, kin, vin, kout, vout, shift, mask, rows, (const uint32_t*)nullptr, digit_total, c)
-    if (items == kItemsSmall) {
-        if (write_keys)
-            GSX_CHAINED(kItemsSmall, true);
-        else
-            GSX_CHAINED(kItemsSmall, false);
-    } else {
-        if (write_keys)
-            GSX_CHAINED(kItemsLarge, true);
-        else
-            GSX_CHAINED(kItemsLarge, false);
-    }
+    using Shape = ChainedShape<KeyT>;
+#define GSX_CHAINED(WK)                                                                                        \
+    hipLaunchKernelGGL((radix_scatter_kernel<KeyT, Shape::kItems, true, WK, Shape::kWaves>), dim3(rows),      \
+                       dim3(64 * Shape::kWaves), 0, s, n_max, kin, vin, kout, vout, shift, mask, rows,        \
+                       (const uint32_t*)nullptr, digit_total, c)
+    if (write_keys)
+        GSX_CHAINED(true);
+    else
+        GSX_CHAINED(false);
 #undef GSX_CHAINED
     GSX_LAUNCH_CHECK();
     return GSX_OK;
