@@ -60,12 +60,13 @@ def test_train_step_matches_oracle(gsx, orc, cuda, cfg, n, use_ssim, reg):
 
 
 @pytest.mark.parametrize("cfg,n,freeze,reg", [(1, 10_000, False, 0.0), (3, 30_000, False, 0.0),
-                                              (3, 30_001, True, 0.0), (3, 20_003, False, 0.01)])
+                                              (3, 30_001, True, 0.0), (3, 20_003, False, 0.01),
+                                              (3, 37, True, 0.0), (3, 130, False, 0.01)])
 def test_fused_update_equals_separate_kernels(gsx, cuda, cfg, n, freeze, reg):
     """epilogue + SH backward + activation VJPs + Adam in one pass (gsx_backward_update_fused) leaves parameters and
     both moments bit-identical to the separate kernels, over three iterations (K = 1 and K = 16 paths, with and
-    without the frozen shN group, a Gaussian count that is not a multiple of the block size, with the scale / opacity
-    regularisation gradients folded in)"""
+    without the frozen shN group, Gaussian counts that are not a multiple of the block size or of a wave - down to
+    less than one wave -, with the scale / opacity regularisation gradients folded in)"""
     from lichtfeld_studio_amd.trainer import TrainStep
     sc = gsx.scenes.config(cfg, n)
     if cfg == 3:
