@@ -74,8 +74,10 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     __shared__ float acc_extra[XLDS ? kBatch * NX : 1];
     __shared__ float cuts[kBatch];
     __shared__ uint8_t lists[4][kBatch];
-    __shared__ int32_t id_batch[kBatch];
-    __shared__ __align__(16) float acc[kBatch * kAcc];
+    __shared__ int32_t id_batch[NX > 0 ? kBatch : 1]; // ids of the batch: only the extra channels' paths read them
+    // LDS sums of a batch: the 13 numbers in use of a row (slot 12 holds the opacity sum, the row's element 15)
+    constexpr uint32_t kAccLds = 13;
+    __shared__ __align__(16) float acc[kBatch * kAccLds];
     // the region tests of a batch are over before its first sum is formed: their operands lie in the accumulators'
     // bytes (8 KB less per workgroup: four workgroups per CU instead of three)
     float4* const region = reinterpret_cast<float4*>(acc);
@@ -162,10 +164,9 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
         const uint32_t t_start = (uint32_t)max(0, batch_end - wave_bin_final);
         const uint32_t n_sel = (uint32_t)__builtin_amdgcn_readfirstlane((int)stage_and_select(
             records, flatten_ids, batch_end, -1, (uint32_t)batch_size, tr, px, t_start,
-            t_start < (uint32_t)batch_size, stage, region, cuts, id_batch, wave_list));
-#pragma unroll
-        for (uint32_t k = 0; k < kAcc / 4; ++k)
-            reinterpret_cast<float4*>(acc)[tr * (kAcc / 4) + k] = make_float4(0.f, 0.f, 0.f, 0.f);
+            t_start < (uint32_t)batch_size, stage, region, cuts, NX > 0 ? id_batch : nullptr, wave_list));
+        for (uint32_t k = tr; k < kBatch * kAccLds / 4; k += 256u)
+            reinterpret_cast<float4*>(acc)[k] = make_float4(0.f, 0.f, 0.f, 0.f);
         __syncthreads();
         if (XLDS) {
             if ((int32_t)tr < batch_size) {
@@ -303,7 +304,8 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             if ((lane & 3u) == 0) {
                 const uint32_t comp = ((lane >> 5) & 1u) * 8u + ((lane >> 4) & 1u) * 4u + ((lane >> 3) & 1u) * 2u +
                                       ((lane >> 2) & 1u);
-                atomicAdd(&acc[(uint32_t)t * kAcc + comp], total); // LDS: ds_add_f32
+                if (comp < 12u || comp == 15u)
+                    atomicAdd(&acc[(uint32_t)t * kAccLds + min(comp, 12u)], total); // LDS: ds_add_f32
             }
         }
         __syncthreads();
@@ -315,9 +317,9 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             const uint32_t gi = s * 16u + (tr >> 4);
             const uint32_t k = tr & 15u;
             if ((int32_t)gi < batch_size) {
-                const float val = acc[gi * kAcc + k];
+                const float val = (k < 12u || k == 15u) ? acc[gi * kAccLds + min(k, 12u)] : 0.f;
                 if (val != 0.f)
-                    unsafeAtomicAdd(&gacc[(size_t)id_batch[gi] * kAcc + k], val);
+                    unsafeAtomicAdd(&gacc[(size_t)flatten_ids[batch_end - (int32_t)gi] * kAcc + k], val);
             }
         }
         if (XLDS && (int32_t)tr < batch_size) {
