@@ -357,6 +357,7 @@ __device__ __forceinline__ void store_record(float4* __restrict__ r, vec3 gro, f
 // registers of the staging lane's wave via `region`.  Then build, per wave, the ordered list of batch slots whose
 // region meets the wave's 8x8 block and whose slot index is >= t_start.  Returns the length of the wave's list.
 // Contains two barriers.
+template <uint32_t BATCH = kBatch>
 __device__ __forceinline__ uint32_t stage_and_select(const float4* __restrict__ records,
                                                      const int32_t* __restrict__ flatten_ids, int32_t first,
                                                      int32_t step, uint32_t count, uint32_t tr, const TilePixel& px,
@@ -381,7 +382,7 @@ __device__ __forceinline__ uint32_t stage_and_select(const float4* __restrict__ 
     if (wave_active) {
         const uint32_t lane = tr & 63u;
 #pragma unroll
-        for (uint32_t r = 0; r < kBatch / 64; ++r) {
+        for (uint32_t r = 0; r < BATCH / 64; ++r) {
             const uint32_t t = r * 64u + lane;
             bool hit = false;
             if (t < count && t >= t_start) {

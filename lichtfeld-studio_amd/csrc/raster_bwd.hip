@@ -23,6 +23,8 @@
 
 namespace gsx {
 
+static constexpr uint32_t kBwdBatch = 256; // list entries staged at a time (128 and 192 measured the same)
+
 static constexpr uint32_t kAcc = 16; // floats per Gaussian: rgb 3, k q 3, k q (x) q 6 (symmetric), 3 unused, opacity 1
 
 __global__ void __launch_bounds__(256) fill_f32_kernel(size_t n, float v, float* __restrict__ out) {
@@ -65,19 +67,19 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     float* __restrict__ gacc /*[N,16]*/, float* __restrict__ gextra /*[N, CDIM - 3]*/,
     unsigned long long* __restrict__ stats = nullptr) {
     constexpr uint32_t NC = CDIM < 3 ? CDIM : 3; // channels carried by the record
-    __shared__ float4 stage[kBatch * 4];
+    __shared__ float4 stage[kBwdBatch * 4];
     constexpr uint32_t NX = CDIM > 3 ? CDIM - 3 : 0; // channels beyond the record's three
     // up to six of them are staged and accumulated in LDS; beyond that (16 channels and more: not a training path)
     // their colours are read from memory in the loop and every wave adds its sums to memory itself
     constexpr bool XLDS = NX > 0 && NX <= 6;
-    __shared__ float extra[XLDS ? kBatch * NX : 1];
-    __shared__ float acc_extra[XLDS ? kBatch * NX : 1];
-    __shared__ float cuts[kBatch];
-    __shared__ uint8_t lists[4][kBatch];
-    __shared__ int32_t id_batch[NX > 0 ? kBatch : 1]; // ids of the batch: only the extra channels' paths read them
+    __shared__ float extra[XLDS ? kBwdBatch * NX : 1];
+    __shared__ float acc_extra[XLDS ? kBwdBatch * NX : 1];
+    __shared__ float cuts[kBwdBatch];
+    __shared__ uint8_t lists[4][kBwdBatch];
+    __shared__ int32_t id_batch[NX > 0 ? kBwdBatch : 1]; // ids of the batch: only the extra channels' paths read them
     // LDS sums of a batch: the 13 numbers in use of a row (slot 12 holds the opacity sum, the row's element 15)
     constexpr uint32_t kAccLds = 13;
-    __shared__ __align__(16) float acc[kBatch * kAccLds];
+    __shared__ __align__(16) float acc[kBwdBatch * kAccLds];
     // the region tests of a batch are over before its first sum is formed: their operands lie in the accumulators'
     // bytes (8 KB less per workgroup: four workgroups per CU instead of three)
     float4* const region = reinterpret_cast<float4*>(acc);
@@ -152,20 +154,20 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     range_end = min(range_end, block_max + 1);
     if (range_end <= range_start)
         return;
-    const uint32_t num_batches = (uint32_t)(range_end - range_start + (int32_t)kBatch - 1) / kBatch;
+    const uint32_t num_batches = (uint32_t)(range_end - range_start + (int32_t)kBwdBatch - 1) / kBwdBatch;
     uint32_t n_eval = 0, n_valid = 0, n_iter = 0;
     const uint64_t inside_mask = __builtin_amdgcn_ballot_w64(inside);
 
     for (uint32_t b = 0; b < num_batches; ++b) {
         // back to front: slot 0 of the batch is the farthest Gaussian (:211-216)
-        const int32_t batch_end = range_end - 1 - (int32_t)(kBatch * b);
-        const int32_t batch_size = min((int32_t)kBatch, batch_end + 1 - range_start);
+        const int32_t batch_end = range_end - 1 - (int32_t)(kBwdBatch * b);
+        const int32_t batch_size = min((int32_t)kBwdBatch, batch_end + 1 - range_start);
         // slots in front of t_start lie behind every last contributor of this wave
         const uint32_t t_start = (uint32_t)max(0, batch_end - wave_bin_final);
-        const uint32_t n_sel = (uint32_t)__builtin_amdgcn_readfirstlane((int)stage_and_select(
+        const uint32_t n_sel = (uint32_t)__builtin_amdgcn_readfirstlane((int)stage_and_select<kBwdBatch>(
             records, flatten_ids, batch_end, -1, (uint32_t)batch_size, tr, px, t_start,
             t_start < (uint32_t)batch_size, stage, region, cuts, NX > 0 ? id_batch : nullptr, wave_list));
-        for (uint32_t k = tr; k < kBatch * kAccLds / 4; k += 256u)
+        for (uint32_t k = tr; k < kBwdBatch * kAccLds / 4; k += 256u)
             reinterpret_cast<float4*>(acc)[k] = make_float4(0.f, 0.f, 0.f, 0.f);
         __syncthreads();
         if (XLDS) {
@@ -313,7 +315,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             continue;
         // flush: 16 lanes per Gaussian, one 64-byte row each
 #pragma unroll 4
-        for (uint32_t s = 0; s < kBatch / 16; ++s) {
+        for (uint32_t s = 0; s < kBwdBatch / 16; ++s) {
             const uint32_t gi = s * 16u + (tr >> 4);
             const uint32_t k = tr & 15u;
             if ((int32_t)gi < batch_size) {

@@ -14,6 +14,8 @@
 
 namespace gsx {
 
+static constexpr uint32_t kFwdBatch = 192; // list entries staged at a time: 20 KB of LDS, seven workgroups per CU (256: 27 KB, six, and a launch 12 % longer)
+
 // One record per Gaussian (all N: rows of Gaussians that no tile lists are never read).
 __global__ void __launch_bounds__(256) pack_records_kernel(uint32_t N, uint32_t CDIM,
                                                             const float* __restrict__ means,
@@ -63,12 +65,12 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
     uint32_t* __restrict__ tile_walk /*nullable*/, float* __restrict__ render_colors,
     float* __restrict__ render_alphas,
     int32_t* __restrict__ last_ids, unsigned long long* __restrict__ stats) {
-    __shared__ float4 stage[kBatch * 4];
-    __shared__ float4 region[kBatch * 2];
-    __shared__ float cuts[kBatch];
-    __shared__ uint8_t lists[4][kBatch];
-    __shared__ int32_t ids[CDIM > 3 ? kBatch : 1];
-    __shared__ float extra[CDIM > 3 ? kBatch * (CDIM - 3) : 1]; // channels beyond the third
+    __shared__ float4 stage[kFwdBatch * 4];
+    __shared__ float4 region[kFwdBatch * 2];
+    __shared__ float cuts[kFwdBatch];
+    __shared__ uint8_t lists[4][kFwdBatch];
+    __shared__ int32_t ids[CDIM > 3 ? kFwdBatch : 1];
+    __shared__ float extra[CDIM > 3 ? kFwdBatch * (CDIM - 3) : 1]; // channels beyond the third
 
     const uint32_t tile_id = tile_order != nullptr ? tile_order[blockIdx.x] : blockIdx.x;
     const uint32_t tr = threadIdx.x;
@@ -107,7 +109,7 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
     const int32_t range_end = (tile_id == tile_width * tile_height - 1 && n_isects != kCountInOffsets)
                                   ? (int32_t)n_isects
                                   : tile_offsets[tile_id + 1];
-    const uint32_t num_batches = (uint32_t)(range_end - range_start + (int32_t)kBatch - 1) / kBatch;
+    const uint32_t num_batches = (uint32_t)(range_end - range_start + (int32_t)kFwdBatch - 1) / kFwdBatch;
 
     bool done = !inside || !ray_ok;
     float T = 1.0f;
@@ -122,10 +124,10 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
         // all four waves saturated: nothing left to stage (:190-194)
         if (__syncthreads_and(done))
             break;
-        const uint32_t batch_start = (uint32_t)range_start + kBatch * b;
-        const uint32_t batch_size = min(kBatch, (uint32_t)range_end - batch_start);
+        const uint32_t batch_start = (uint32_t)range_start + kFwdBatch * b;
+        const uint32_t batch_size = min(kFwdBatch, (uint32_t)range_end - batch_start);
         const bool wave_active = __builtin_amdgcn_ballot_w64(!done) != 0;
-        const uint32_t n_sel = stage_and_select(records, flatten_ids, (int32_t)batch_start, 1, batch_size, tr, px, 0u,
+        const uint32_t n_sel = stage_and_select<kFwdBatch>(records, flatten_ids, (int32_t)batch_start, 1, batch_size, tr, px, 0u,
                                                 wave_active, stage, region, cuts, CDIM > 3 ? ids : nullptr,
                                                 wave_list);
         if (CDIM > 3) {
