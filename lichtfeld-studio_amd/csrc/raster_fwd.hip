@@ -4,7 +4,7 @@
 // block.  What a (pixel, Gaussian) pair needs from the Gaussian - M = diag(1/scale) R(quat)^T, gro = M (ray_o -
 // mean), opacity, colour - does not depend on the tile, so it is built once per Gaussian as a 96-byte record
 // (gsx_record.h) by pack_records_kernel (or by the fused per-Gaussian pass of a training step) instead of once per
-// tile the Gaussian touches.  The tile's depth-sorted records are staged through LDS 256 at a time; every wave
+// tile the Gaussian touches.  The tile's depth-sorted records are staged through LDS 192 at a time; every wave
 // then keeps the slots whose exact pixel bounds meet its 8x8 block (ballot + prefix count, order preserved) and
 // walks only those, reading each record with wave-uniform addresses (LDS broadcast), evaluating the ray / Gaussian
 // response with explicit FMAs and compositing front to back.  Pairs outside the bounds have alpha < 1/255 and are
