@@ -200,11 +200,10 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             const vec3 grd = mk3(fma(m0.z, ray_d.z, fma(m0.y, ray_d.y, m0.x * ray_d.x)),
                                  fma(m1.y, ray_d.z, fma(m1.x, ray_d.y, m0.w * ray_d.x)),
                                  fma(m2.x, ray_d.z, fma(m1.w, ray_d.y, m1.z * ray_d.x)));
-            // safe_normalize without a branch: the reciprocal length is reused by the VJP below
+            // safe_normalize (Utils.cuh:181-184) without its test: a zero vector times the finite rsqrt(0) of the
+            // written-out sequence is the zero vector the test would have left
             const float l2 = dot(grd, grd);
-            const float il_any = gsx::rsqrt(l2);
-            const float il = l2 > 0.0f ? il_any : 1.0f;
-            const vec3 grd_n = scale(grd, il);
+            const vec3 grd_n = scale(grd, gsx::rsqrt(l2));
             const vec3 gcrod = cross(grd_n, gro);
             const float grayDist = dot(gcrod, gcrod);
             const float power = -0.5f * grayDist;

@@ -165,10 +165,10 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
             const vec3 gd = mk3(fma(m0.z, ray_d.z, fma(m0.y, ray_d.y, m0.x * ray_d.x)),
                                 fma(m1.y, ray_d.z, fma(m1.x, ray_d.y, m0.w * ray_d.x)),
                                 fma(m2.x, ray_d.z, fma(m1.w, ray_d.y, m1.z * ray_d.x)));
-            // safe_normalize (Utils.cuh:181-184) as a select instead of a branch
+            // safe_normalize (Utils.cuh:181-184) without its test: a zero vector times the finite rsqrt(0) of the
+            // written-out sequence is the zero vector the test would have left
             const float l2 = dot(gd, gd);
-            const float il_any = gsx::rsqrt(l2);
-            const vec3 grd = scale(gd, l2 > 0.0f ? il_any : 1.0f);
+            const vec3 grd = scale(gd, gsx::rsqrt(l2));
             const vec3 gcrod = cross(grd, gro);
             const float grayDist = dot(gcrod, gcrod);
             const float power = -0.5f * grayDist;
