@@ -19,9 +19,9 @@
 //   |g^ x v|^2 <= (k/|g|^2) |v - gro/z|^2,   v = b1 dx + b2 dy,   g^ = gro/|gro|
 // a 2x2 quadratic form: an ellipse with closed-form centre, extent and axis-aligned bounding box.  k is inflated
 // for the rounding of the in-kernel evaluation of d^2 (whose absolute error grows with |gro|), the ellipse by
-// 0.4 % and the tested rectangles by one pixel, so the region is a superset of the contributing pixels; anything
-// that is not a proper ellipse (camera inside the k-ellipsoid, hyperbolic silhouette, non-finite numbers) falls
-// back to "everywhere".
+// 0.4 %, the bounding box by one pixel and the tested rectangles by a quarter, so the region is a superset of the
+// contributing pixels; anything that is not a proper, well-conditioned ellipse (camera inside the k-ellipsoid,
+// hyperbolic or nearly parabolic silhouette, non-finite numbers) falls back to "everywhere".
 #pragma once
 
 #include "gsx_math.h"
@@ -31,6 +31,7 @@ namespace gsx {
 static constexpr uint32_t kRecordFloats = 24; // 96 bytes
 static constexpr uint32_t kRecordF4 = 6;
 static constexpr float kLogAlphaInv = 5.5412635f; // ln 255
+static constexpr float kBlockMargin = 0.25f;        // pixels added around a block's pixel centres in the region test
 static constexpr float kPowerFloor = -80.0f;      // no cut-off is below this: exp_nonpos stays in its domain
 
 struct RecordRegion {
@@ -87,6 +88,12 @@ GSX_HD RecordRegion record_region(vec3 gro, const mat3& M, float opacity, vec3 m
     const float det = a00 * a11 - a01 * a01;
     if (!(det > 0.f) || !(a00 > 0.f) || !(a11 > 0.f))
         return full;
+    // A silhouette that is nearly a parabola (a needle reaching towards the camera plane: an ellipse hundreds of
+    // image widths long whose centre lies as far outside) leaves det as the small difference of two products:
+    // centre and extent then carry its relative error a00 a11 / det times over, and the block test adds terms of
+    // that size to get a value near 1.  Past a ratio of 256 (an axis ratio of 32 at 45 degrees) no region is claimed.
+    if (!(det * 256.0f > a00 * a11))
+        return full;
     const float inv_det = 1.0f / det;
     const float dcx = -(a11 * be0 - a01 * be1) * inv_det;
     const float dcy = -(a00 * be1 - a01 * be0) * inv_det;
@@ -119,14 +126,15 @@ GSX_HD RecordRegion record_region(vec3 gro, const mat3& M, float opacity, vec3 m
 }
 
 // Can a pixel of the 8x8 block whose first pixel is (wi0, wj0) contribute?  Bounding box first, then the
-// minimum of the ellipse's quadratic form over the block's rectangle of pixel centres grown by one pixel.
+// minimum of the ellipse's quadratic form over the block's rectangle of pixel centres grown by a quarter pixel
+// (the brute-force comparison with every pixel finds no miss with no growth at all).
 GSX_HD bool record_region_hits_block(int32_t jmin, int32_t imin, int32_t jmax, int32_t imax, float a00, float a01,
                                      float a11, float pcx, float pcy, int32_t wi0, int32_t wj0) {
     if (!(jmin <= wj0 + 7 && jmax >= wj0 && imin <= wi0 + 7 && imax >= wi0))
         return false;
     // rectangle relative to the ellipse centre
-    const float x0 = ((float)wj0 - 0.5f) - pcx, x1 = ((float)wj0 + 8.5f) - pcx;
-    const float y0 = ((float)wi0 - 0.5f) - pcy, y1 = ((float)wi0 + 8.5f) - pcy;
+    const float x0 = ((float)wj0 + 0.5f - kBlockMargin) - pcx, x1 = ((float)wj0 + 7.5f + kBlockMargin) - pcx;
+    const float y0 = ((float)wi0 + 0.5f - kBlockMargin) - pcy, y1 = ((float)wi0 + 7.5f + kBlockMargin) - pcy;
     if (x0 <= 0.f && x1 >= 0.f && y0 <= 0.f && y1 >= 0.f)
         return true; // centre inside
     // minimum of q over the four edges (q is convex, its unconstrained minimum lies outside the rectangle).  Where

@@ -470,6 +470,37 @@ def test_fused_forward_bit_exact(gsx, orc, cuda, n, bg):
         assert torch.equal(a, b), name
 
 
+@pytest.mark.parametrize("seed", [2005, 3105])
+def test_needle_gaussians_forward_bit_exact(gsx, orc, cuda, seed):
+    """Gaussians with axis ratios up to 10^3 and more, among them needles that reach towards the camera plane: their
+    silhouette is an ellipse hundreds of image widths long, for which the rasterizers' pixel region must claim
+    nothing (the draws are those of the region's own conservativeness test).  Image, alpha and last contributors
+    bit-identical to the checker, which evaluates every pair."""
+    ops = gsx.ops
+    rng = np.random.default_rng(seed)
+    n, W, H = 6000, 160, 120
+    cam = gsx.scenes.orbit_camera(5.3, 4.0, W, H, 150.0)
+    means = rng.normal(0, 0.6, (n, 3)).astype(np.float32)
+    log_s = rng.uniform(np.log(1e-4), np.log(0.5), (n, 1)) + rng.normal(0, 2.0, (n, 3))
+    scales = np.exp(log_s).astype(np.float32)
+    quats = rng.normal(0, 1, (n, 4)).astype(np.float32)
+    quats /= np.linalg.norm(quats, axis=1, keepdims=True)
+    op = np.exp(rng.uniform(np.log(1 / 300), 0, n)).astype(np.float32)
+    shs = rng.normal(0, 0.4, (n, 16, 3)).astype(np.float32)
+    h = dict(means=means, quats=quats, scales=scales, op=op, shs=shs, vm=cam.viewmat[None], K=cam.K[None])
+    d = {k: T(v, cuda) for k, v in h.items()}
+    ref = orc.rasterize_from_world_with_sh_fwd(h["means"], h["quats"], h["scales"], h["op"], h["shs"], 3, None, W, H, 16,
+                                               h["vm"], h["K"])
+    got = ops.rasterize_from_world_with_sh_fwd(d["means"], d["quats"], d["scales"], d["op"], d["shs"], 3, None, None, W,
+                                               H, 16, d["vm"], None, d["K"], 0, 0.3, 0.01, 1e4, 0.0, 1.0, False, 0,
+                                               ops.UnscentedTransformParameters(), 4)
+    assert (ref[2][0, :, 0] > 0).sum() > 500 and ref[1].mean() > 0.05  # the case is not vacuous
+    bits_equal(N(got[7]), ref[7], "sort order")
+    bits_equal(N(got[8]), ref[8], "last contributors")
+    bits_equal(N(got[0]), ref[0], "image")
+    bits_equal(N(got[1]), ref[1], "alpha")
+
+
 def check_raster_gradients(got5, o32_5, g64, tag="", bound=None):
     """Gradient bar of the rasterizer backward (oracle/checks.py: measured miss fractions against the fp32
     reference-order checker and against float64, then the element and whole-tensor bars with the fp32 checker's own

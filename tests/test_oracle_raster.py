@@ -204,14 +204,20 @@ def test_backward_matches_finite_differences_of_the_model(orc):
     assert np.all(np.abs(g64[:, 10:13]).sum(1)[np.bincount(flat, minlength=24) == 0] == 0)
 
 
-@pytest.mark.parametrize("trial", range(7))
+@pytest.mark.parametrize("trial", range(9))
 def test_record_pixel_bounds_are_conservative(gsx, orc, trial):
     """The per-Gaussian pixel bounds the GPU rasterizers skip by (csrc/gsx_record.h, compiled here for the host) must
     contain every pixel that reaches alpha >= 1/255 in the checker's per-pair arithmetic: brute force over all pixels
     for Gaussians from sub-pixel to screen-filling, anisotropy up to ~1e3, opacities from below the threshold to 1,
-    cameras inside the cloud, long focal lengths and an off-centre crop of a large image."""
-    rng = np.random.default_rng(100 + trial)
-    n, W, H = 1200, 160, 120
+    cameras inside the cloud, long focal lengths and an off-centre crop of a large image.  Trials 7 and 8: larger
+    draws of the most anisotropic case - among them needles that reach towards the camera plane, whose silhouette is
+    an ellipse hundreds of image widths long (nearly a parabola: the region must give up on those)."""
+    seed, base = 100 + trial, trial
+    if trial >= 7:
+        seed, base = [2005, 3105][trial - 7], 5
+    rng = np.random.default_rng(seed)
+    n, W, H = (1200 if trial < 7 else 6000), 160, 120
+    trial = base
     f = [150.0, 400.0, 80.0, 1000.0, 150.0, 150.0, 3200.0][trial]
     radius = [4.0, 4.0, 2.0, 6.0, 1.0, 4.0, 4.0][trial]
     cam = gsx.scenes.orbit_camera(0.3 + trial, radius, W, H, f)
