@@ -157,8 +157,11 @@ def main():
         gt = tgt.render[0].clamp(0, 1).permute(2, 0, 1).contiguous()[None].clone()
         del tgt
         torch.cuda.empty_cache()
-    else:
+    elif hasattr(sc, "target"):
         gt = torch.from_numpy(sc.target[None].copy()).to(dev)
+    else:
+        sys.exit(f"bench.py: configuration {args.config} has no training target (a forward-only parity case); "
+                 "the training step is timed on configurations 1, 3, 4 and 5")
     use_ssim = args.config != 1  # configuration 1 is L1 only
     ts = TrainStep(sc, dev, use_ssim=use_ssim, fused_update=not args.separate_update,
                    fused_loss=not args.separate_update, overlap=not args.no_overlap,

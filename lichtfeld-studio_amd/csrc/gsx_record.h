@@ -88,11 +88,12 @@ GSX_HD RecordRegion record_region(vec3 gro, const mat3& M, float opacity, vec3 m
     const float det = a00 * a11 - a01 * a01;
     if (!(det > 0.f) || !(a00 > 0.f) || !(a11 > 0.f))
         return full;
-    // A silhouette that is nearly a parabola (a needle reaching towards the camera plane: an ellipse hundreds of
-    // image widths long whose centre lies as far outside) leaves det as the small difference of two products:
-    // centre and extent then carry its relative error a00 a11 / det times over, and the block test adds terms of
-    // that size to get a value near 1.  Past a ratio of 256 (an axis ratio of 32 at 45 degrees) no region is claimed.
-    if (!(det * 256.0f > a00 * a11))
+    // A thin ellipse lying diagonally, or a silhouette that is nearly a parabola (a needle reaching towards the
+    // camera plane), leaves det as the small difference of two products, and the quadratic form of the block test as
+    // a small sum of large terms: both carry the rounding of a00, a01, a11 multiplied by a00 a11 / det.  Drawn needles
+    // show the form at contributing pixels growing by ~ratio x 2^-22: it uses up the 0.8 % margin at a ratio of 2^15.
+    // Past 2^11 (an axis ratio of 90 at 45 degrees) no region is claimed.
+    if (!(det * 2048.0f > a00 * a11))
         return full;
     const float inv_det = 1.0f / det;
     const float dcx = -(a11 * be0 - a01 * be1) * inv_det;
