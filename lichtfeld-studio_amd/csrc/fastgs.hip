@@ -566,7 +566,7 @@ __global__ void __launch_bounds__(256) fgs_blend_bwd_kernel(
             if (__builtin_amdgcn_ballot_w64(valid) == 0)
                 continue;
             // branch-free from here: a lane that is not valid carries ra = 1 and zero weights
-            const float ra = valid ? __builtin_amdgcn_rcpf(1.0f - alpha) : 1.0f;
+            const float ra = valid ? gsx::rcp_refined(1.0f - alpha) : 1.0f;
             T *= ra; // transmittance in front of this Gaussian
             const float w = valid ? T * alpha : 0.f;
             const float col0 = q1.z > 0.0f ? q1.z : 0.0f, col1 = q1.w > 0.0f ? q1.w : 0.0f,

@@ -230,9 +230,9 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
 
             // From here on without branches: a lane that is not valid carries ra = 1 and fac = v_alpha = 0, which
             // leaves its T and colour buffer unchanged and makes all 16 of its partials zero.  The decisions above
-            // use the forward pass's exact arithmetic; the derivative chain may use the hardware reciprocal.
+            // use the forward pass's exact arithmetic; the derivative chain may use the (refined) hardware reciprocal.
             float v[kAcc];
-            const float ra = valid ? __builtin_amdgcn_rcpf(1.0f - alpha) : 1.0f;
+            const float ra = valid ? gsx::rcp_refined(1.0f - alpha) : 1.0f;
             T *= ra;
             const float fac = valid ? alpha * T : 0.f;
             const float col[3] = {m2.y, m2.z, m2.w};

@@ -501,6 +501,55 @@ def test_needle_gaussians_forward_bit_exact(gsx, orc, cuda, seed):
     bits_equal(N(got[1]), ref[1], "alpha")
 
 
+@pytest.mark.parametrize("K", [127, 128, 129, 191, 192, 193, 256, 257, 384, 385])
+def test_tile_lists_at_the_staging_batch_boundaries(gsx, orc, cuda, K):
+    """Every tile's list has exactly K entries, K around the multiples of the numbers of entries the two rasterizers
+    stage at a time (192 forward, 128 backward): K faint, screen-filling Gaussians, so no pixel saturates and every
+    entry of every batch composites.  Forward bit-identical to the checker, gradients to the bar of the backward
+    test."""
+    ops = gsx.ops
+    rng = np.random.default_rng(K)
+    W, H = 48, 32
+    cam = gsx.scenes.orbit_camera(0.3, 4.0, W, H, 40.0)
+    means = rng.normal(0, 0.1, (K, 3)).astype(np.float32)
+    scales = np.exp(rng.normal(np.log(2.0), 0.1, (K, 3))).astype(np.float32)
+    quats = rng.normal(0, 1, (K, 4)).astype(np.float32)
+    quats /= np.linalg.norm(quats, axis=1, keepdims=True)
+    op = rng.uniform(0.008, 0.012, K).astype(np.float32)
+    shs = rng.normal(0, 0.4, (K, 16, 3)).astype(np.float32)
+    h = dict(means=means, quats=quats, scales=scales, op=op, shs=shs, vm=cam.viewmat[None], K=cam.K[None],
+             bg=np.array([[0.1, 0.2, 0.3]], np.float32))
+    d = {k: T(v, cuda) for k, v in h.items()}
+    ut = ops.UnscentedTransformParameters()
+    ref = orc.rasterize_from_world_with_sh_fwd(h["means"], h["quats"], h["scales"], h["op"], h["shs"], 3, h["bg"], W, H,
+                                               16, h["vm"], h["K"])
+    fwd = ops.rasterize_from_world_with_sh_fwd(d["means"], d["quats"], d["scales"], d["op"], d["shs"], 3, d["bg"], None,
+                                               W, H, 16, d["vm"], None, d["K"], 0, 0.3, 0.01, 1e4, 0.0, 1.0, False, 0,
+                                               ut, 4)
+    renders, alphas, radii, means2d, depths, colors, offsets, flat, last_ids, comp = fwd
+    lengths = np.diff(np.append(N(offsets).reshape(-1), N(flat).shape[0]))
+    assert (lengths == K).all(), lengths  # the case is what it says
+    bits_equal(N(flat), ref[7], "sort order")
+    bits_equal(N(last_ids), ref[8], "last contributors")
+    bits_equal(N(renders), ref[0], "image")
+    bits_equal(N(alphas), ref[1], "alpha")
+    assert N(alphas).max() < 0.99 and N(last_ids).max() == N(flat).shape[0] - 1  # no pixel ends early
+    # cotangents of one sign: every Gaussian sums over all 1 536 pixels, and this test is about the lists, not about
+    # how an fp32 sum of that length cancels
+    v_r = rng.uniform(0.5, 1.5, tuple(renders.shape)).astype(np.float32)
+    v_a = rng.uniform(0.5, 1.5, tuple(alphas.shape)).astype(np.float32)
+    got5 = ops.rasterize_to_pixels_from_world_3dgs_bwd(d["means"], d["quats"], d["scales"], colors, d["op"][None].contiguous(),
+                                                       d["bg"], None, W, H, 16, d["vm"], None, d["K"], 0, ut, 4, None,
+                                                       None, None, offsets, flat, alphas, last_ids, T(v_r, cuda),
+                                                       T(v_a, cuda))
+    args = (h["means"], h["quats"], h["scales"], N(colors), h["op"][None], h["bg"])
+    o32 = orc.rasterize_to_pixels_from_world_3dgs_bwd(*args, None, W, H, 16, h["vm"], h["K"], N(offsets), N(flat),
+                                                      N(alphas), N(last_ids), v_r, v_a)
+    g64, b64 = orc.rasterize_bwd_f64(*args, W, H, 16, h["vm"], h["K"], N(offsets), N(flat), N(alphas), N(last_ids), v_r,
+                                     v_a)
+    check_raster_gradients([N(x) for x in got5], o32, g64, tag=f"K={K}", bound=b64)
+
+
 def check_raster_gradients(got5, o32_5, g64, tag="", bound=None):
     """Gradient bar of the rasterizer backward (oracle/checks.py: measured miss fractions against the fp32
     reference-order checker and against float64, then the element and whole-tensor bars with the fp32 checker's own

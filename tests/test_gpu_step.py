@@ -353,8 +353,11 @@ def test_pairs_outgrowing_the_buffers_hold_the_step_back(gsx, cuda):
     torch.cuda.synchronize()
     assert a.steps_held == 1 and a.step_count == b.step_count == 2 and a.iteration == b.iteration == 2
     assert a.cap >= a.n_isects == b.n_isects and a.lists_error() == (0, 0)
-    assert torch.equal(a.render, b.render)
-    for k in a.params:  # the two runs add up their gradients in different (atomic) orders
+    # the two runs add up the first step's gradients in different (atomic) orders: the parameters the second step
+    # renders agree to rounding, not to the bit
+    diff = (a.render - b.render).abs()
+    assert float(diff.max()) <= 2e-3 and float((diff > 2e-6).float().mean()) < 1e-2, float(diff.max())
+    for k in a.params:
         assert torch.allclose(a.params[k], b.params[k], rtol=0, atol=2.2 * a.lrs["opacity"]), k
         close = (a.params[k] - b.params[k]).abs() <= 1e-6 + 1e-3 * a.lrs["opacity"]
         assert close.float().mean() > 0.999, k
