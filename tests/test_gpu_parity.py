@@ -78,6 +78,31 @@ def test_math_primitives_bit_exact(gsx, orc, cuda):
         bits_equal(got, ref, name)
 
 
+def test_refined_reciprocal_has_no_one_sided_error(gsx, cuda):
+    """The backward rasterizers rebuild a pixel's transmittance by multiplying with 1 / (1 - alpha) entry by entry, so
+    an error of one sign in that reciprocal adds up along the list.  On the range of 1 - alpha the refined hardware
+    reciprocal stays within one unit in the last place of the exact quotient and its mean signed error is a small
+    fraction of a unit; the bare instruction's mean error is printed beside it."""
+    import ctypes
+    L = gsx._lib
+    rng = np.random.default_rng(5)
+    x = rng.uniform(0.001, 1.0, 400_000).astype(np.float32)
+    xd, out = T(x, cuda), {}
+    for which in (12, 13):
+        y = torch.empty_like(xd)
+        L.check(L.lib().gsx_debug_math(ctypes.c_int(which), ctypes.c_uint32(x.size), ctypes.c_void_p(xd.data_ptr()),
+                                       ctypes.c_void_p(None), ctypes.c_void_p(y.data_ptr()), ctypes.c_void_p(None)))
+        torch.cuda.synchronize()
+        exact = 1.0 / x.astype(np.float64)
+        ulp = np.spacing(exact.astype(np.float32)).astype(np.float64)
+        out[which] = (N(y).astype(np.float64) - exact) / ulp
+    refined, bare = out[12], out[13]
+    print(f"reciprocal error in units of the last place: refined max {np.abs(refined).max():.3f} mean {refined.mean():+.4f}"
+          f" | bare max {np.abs(bare).max():.3f} mean {bare.mean():+.4f}")
+    assert np.abs(refined).max() <= 1.0
+    assert abs(refined.mean()) <= 0.02
+
+
 # ---------------------------------------------------------------------------------------------
 # projection / SH / intersect / sort / offsets: bit-exact
 # ---------------------------------------------------------------------------------------------
