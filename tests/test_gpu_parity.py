@@ -575,6 +575,44 @@ def test_tile_lists_at_the_staging_batch_boundaries(gsx, orc, cuda, K):
     check_raster_gradients([N(x) for x in got5], o32, g64, tag=f"K={K}", bound=b64)
 
 
+def test_equal_depths_keep_index_order(gsx, orc, cuda):
+    """3 000 faint Gaussians on one plane in front of an axis-aligned camera: every depth is the same float, so the
+    order inside a tile's list is the order of the indices (the reference's sort is stable and so is this one), lists
+    are 2 000 and more entries long and every pixel walks them to the end.  Sort order, last contributors, image and
+    alpha bit-identical to the checker."""
+    ops = gsx.ops
+    rng = np.random.default_rng(77)
+    n, W, H = 3000, 64, 48
+    vm = np.eye(4, dtype=np.float32)
+    vm[2, 3] = 4.0
+    K = gsx.scenes.intrinsics(W, H, 60.0)
+    means = np.concatenate([rng.normal(0, 0.6, (n, 2)), np.zeros((n, 1))], 1).astype(np.float32)
+    scales = np.exp(rng.normal(np.log(0.8), 0.3, (n, 3))).astype(np.float32)
+    quats = rng.normal(0, 1, (n, 4)).astype(np.float32)
+    quats /= np.linalg.norm(quats, axis=1, keepdims=True)
+    op = rng.uniform(0.0045, 0.006, n).astype(np.float32)
+    shs = rng.normal(0, 0.4, (n, 16, 3)).astype(np.float32)
+    h = dict(means=means, quats=quats, scales=scales, op=op, shs=shs, vm=vm[None], K=K[None])
+    d = {k: T(v, cuda) for k, v in h.items()}
+    ref = orc.rasterize_from_world_with_sh_fwd(h["means"], h["quats"], h["scales"], h["op"], h["shs"], 3, None, W, H, 16,
+                                               h["vm"], h["K"])
+    got = ops.rasterize_from_world_with_sh_fwd(d["means"], d["quats"], d["scales"], d["op"], d["shs"], 3, None, None, W,
+                                               H, 16, d["vm"], None, d["K"], 0, 0.3, 0.01, 1e4, 0.0, 1.0, False, 0,
+                                               ops.UnscentedTransformParameters(), 4)
+    depths = ref[4][0][ref[2][0, :, 0] > 0]
+    assert depths.size > 2500 and (depths == depths[0]).all()  # the case is what it says
+    offsets, flat = ref[6].reshape(-1), ref[7]
+    bounds = np.append(offsets, flat.shape[0])
+    assert np.diff(bounds).max() >= 2000
+    for a, b in zip(bounds[:-1], bounds[1:]):
+        assert (np.diff(flat[a:b]) > 0).all()  # ties in depth: index order
+    bits_equal(N(got[7]), flat, "sort order")
+    bits_equal(N(got[8]), ref[8], "last contributors")
+    bits_equal(N(got[0]), ref[0], "image")
+    bits_equal(N(got[1]), ref[1], "alpha")
+    assert ref[1].max() < 0.9999  # nobody saturates: the lists are walked to their ends
+
+
 def check_raster_gradients(got5, o32_5, g64, tag="", bound=None):
     """Gradient bar of the rasterizer backward (oracle/checks.py: measured miss fractions against the fp32
     reference-order checker and against float64, then the element and whole-tensor bars with the fp32 checker's own
