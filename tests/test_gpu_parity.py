@@ -611,6 +611,20 @@ def test_equal_depths_keep_index_order(gsx, orc, cuda):
     bits_equal(N(got[0]), ref[0], "image")
     bits_equal(N(got[1]), ref[1], "alpha")
     assert ref[1].max() < 0.9999  # nobody saturates: the lists are walked to their ends
+    # backward over the same lists: the transmittance is rebuilt through up to 2 000 entries per pixel
+    renders, alphas, colors, offs, flt, last_ids = got[0], got[1], got[5], got[6], got[7], got[8]
+    v_r = rng.normal(0, 1, tuple(renders.shape)).astype(np.float32)
+    v_a = rng.normal(0, 1, tuple(alphas.shape)).astype(np.float32)
+    ut = ops.UnscentedTransformParameters()
+    got5 = ops.rasterize_to_pixels_from_world_3dgs_bwd(d["means"], d["quats"], d["scales"], colors,
+                                                       d["op"][None].contiguous(), None, None, W, H, 16, d["vm"], None,
+                                                       d["K"], 0, ut, 4, None, None, None, offs, flt, alphas, last_ids,
+                                                       T(v_r, cuda), T(v_a, cuda))
+    args = (h["means"], h["quats"], h["scales"], N(colors), h["op"][None], None)
+    o32 = orc.rasterize_to_pixels_from_world_3dgs_bwd(*args, None, W, H, 16, h["vm"], h["K"], N(offs), N(flt), N(alphas),
+                                                      N(last_ids), v_r, v_a)
+    g64, b64 = orc.rasterize_bwd_f64(*args, W, H, 16, h["vm"], h["K"], N(offs), N(flt), N(alphas), N(last_ids), v_r, v_a)
+    check_raster_gradients([N(x) for x in got5], o32, g64, tag="plane ", bound=b64)
 
 
 def check_raster_gradients(got5, o32_5, g64, tag="", bound=None):
