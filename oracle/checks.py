@@ -27,15 +27,17 @@ of one rounding applied to every term, the textbook scale of what an fp32 evalua
 Where no BOUND exists for a tensor, step 3 uses the fp32 checker's own error as the yardstick:
 max(FLOOR_MULT * E999, MAX_MULT * EMAX), its 99.9th percentile and maximum |error| against float64 on that tensor.
 
-Measured over every test of the suite (operator tests of all camera models, configurations 1, 3 and 5 at full size,
-two iterations of the benchmarked path), largest figure of each kind:
-  miss fraction   GPU 1.01 x the fp32 checker's (means, opacities, colours 0.98 - 1.01; quaternions and scales 0.2 - 0.5:
-                  the kernel sums k q (x) q per Gaussian and never forms the two large terms, the checker follows the
-                  reference and cancels them in fp32 for every pair)
-  L2              GPU 1.00 x the fp32 checker's (quaternions 0.5 - 0.9, scales 0.7 - 0.9), SH coefficients up to 4.4 x on
-                  tensors whose whole error is 2.4e-7, i.e. two roundings: what L2_EPS is for
+Measured over every test of the suite (operator tests of all camera models, list lengths around the staging batches,
+2 000-entry lists, configurations 1, 3, 4 and 5 at full size, two iterations of the benchmarked path), largest figure of
+each kind:
+  miss fraction   GPU 1.05 x the fp32 checker's on the step's tensors, 1.21 x on one operator test where both are below
+                  1e-3 (quaternions and scales 0.2 - 0.5: the kernel sums k q (x) q per Gaussian and never forms the
+                  two large terms, the checker follows the reference and cancels them in fp32 for every pair)
+  L2              GPU at most 1.35 x the fp32 checker's on means, quaternions, scales and opacities; colour gradients of
+                  stacked faint Gaussians 2.1 x and SH coefficients up to 12 x on tensors whose whole error is 5e-8 and
+                  2.6e-7, i.e. two roundings: what L2_EPS is for
   per element     c needed by the GPU within 1.05 x of what the fp32 checker needs (opacity gradients of long lists:
-                  215 against 214), and below 2.0 where the checker needs less than 2
+                  710 against 709), and below 1.8 where the checker needs less than 2
 The multipliers leave head-room for the order of the atomic additions, which changes from run to run:
 MISS_RATIO 1.5, L2_MULT 2, COND_RATIO 1.5 with COND_MULT 4 as the least bar.
 """
