@@ -19,8 +19,9 @@ GSX_API int gsx_debug_math(int which, uint32_t n, const float* x, const float* x
 /* Measurement hook (no counterpart in the reference): a plain device-to-device copy kernel of `bytes` bytes (a
  * multiple of 16), the known-size yardstick for HBM byte counters and achieved-bandwidth figures. */
 GSX_API int gsx_debug_copy(const void* src, void* dst, size_t bytes, void* stream);
-/* Test hook: the 64-lane, 16-value wave reduction of the rasterizer backward.  in [n_waves,64,16] -> out [n_waves,16]. */
-GSX_API int gsx_debug_wave_reduce16(uint32_t n_waves, const float* in, float* out, void* stream);
+/* Test hook: the 64-lane wave reductions of the backward rasterizers, for `values` = 16, 13 (the 3DGUT backward) or 9
+ * (the fastgs backward) sums at a time.  in [n_waves,64,values] -> out [n_waves,values]. */
+GSX_API int gsx_debug_wave_reduce(uint32_t values, uint32_t n_waves, const float* in, float* out, void* stream);
 
 /* Pair counts of one forward pass, for turning kernel times into rates (no counterpart in the reference).
  * stats_out: device uint64[8] = {(pixel, Gaussian) pairs the forward evaluates, pairs composited, pairs the backward

@@ -505,6 +505,8 @@ __global__ void __launch_bounds__(256) fgs_blend_bwd_kernel(
     __shared__ int32_t block_max;
     const uint32_t tile_id = tile_order[blockIdx.x]; // dearest tiles first
     const uint32_t tr = threadIdx.x, lane = tr & 63u;
+    // which of the 9 per-Gaussian sums this lane ends up with after the wave reduction (15: none)
+    const uint32_t sum_index = (lane & 3u) == 0 ? wave_reduce9_index(lane) : 15u;
     const TilePixel px = tile_pixel(tile_id, grid_w, tr);
     const bool inside = px.i < height && px.j < width;
     const float pxf = (float)px.j + 0.5f, pyf = (float)px.i + 0.5f;
@@ -578,7 +580,7 @@ __global__ void __launch_bounds__(256) fgs_blend_bwd_kernel(
             adot = fma(w, cdot, adot);
             const float ad = valid ? alpha * dL_dalpha : 0.f;
             const float helper = -ad;
-            float v[16];
+            float v[9];
             v[0] = helper * (q0.z * dx + q0.w * dy);
             v[1] = helper * (q0.w * dx + q1.x * dy);
             v[2] = 0.5f * helper * dx * dx;
@@ -588,16 +590,9 @@ __global__ void __launch_bounds__(256) fgs_blend_bwd_kernel(
             v[6] = q1.z >= 0.0f ? w * g0 : 0.f; // zero where the colour was clamped (:286-291)
             v[7] = q1.w >= 0.0f ? w * g1 : 0.f;
             v[8] = q2.x >= 0.0f ? w * g2 : 0.f;
-#pragma unroll
-            for (int k = 9; k < 16; ++k)
-                v[k] = 0.f;
-            const float total = wave_reduce16(v, lane);
-            if ((lane & 3u) == 0) {
-                const uint32_t comp = ((lane >> 5) & 1u) * 8u + ((lane >> 4) & 1u) * 4u + ((lane >> 3) & 1u) * 2u +
-                                      ((lane >> 2) & 1u);
-                if (comp < 9u)
-                    atomicAdd(&acc[(uint32_t)t * kFgsAcc + comp], total); // LDS: ds_add_f32
-            }
+            const float total = wave_reduce9(v, lane);
+            if (sum_index < 9u)
+                atomicAdd(&acc[(uint32_t)t * kFgsAcc + sum_index], total); // LDS: ds_add_f32
         }
         __syncthreads();
 #pragma unroll 4

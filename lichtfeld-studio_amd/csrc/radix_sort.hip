@@ -2,13 +2,17 @@
 // (gsplat/IntersectTile.cu:290-328 calls cub::DeviceRadixSort::SortPairs with a DoubleBuffer), and the same sort
 // for (uint16 tile index, int32 value) pairs.
 //
-// 8-bit digits.  Per pass three launches: block histograms -> one scan block per digit turns its row of the
+// 8-bit digits.  A large sort is one launch per pass behind two small ones: a fill of the bookkeeping words, one
+// read of the keys that counts the digits of every pass, then the chained passes below (2 + P launches; the 45-bit
+// keys of the reference's sort: 8 instead of 18).  Smaller sorts, the entry point that brings no workspace and more
+// than 2^30 pairs take three launches per pass: block histograms -> one scan block per digit turns its row of the
 // digit-major table into running counts and leaves the digit's total -> stable scatter (every block adds the
 // exclusive scan of the 256 totals itself; no atomics between blocks, nothing to zero).  A
 // block owns a tile of 256 x ITEMS consecutive pairs; inside the block each 64-lane wave owns a quarter of them
 // and ranks them 64 at a time with wave-wide match masks (one 64-bit mask per digit in LDS, set by atomic OR), so
 // the order (wave, round, lane) equals the input order and the sort is stable.  The ranked pairs are first placed in LDS in digit order and then
 // written out by consecutive lanes, so that every (tile, digit) run leaves the block as whole cache lines.
+#include <algorithm>
 #include <mutex>
 
 #include "gsx_common.h"
@@ -106,6 +110,69 @@ __global__ void __launch_bounds__(256) radix_scan_kernel(uint32_t nblocks, uint3
     }
     if (t == 0)
         digit_total[d] = carry;
+}
+
+// ---- digit counts of all passes in one read of the keys ---------------------------------------------
+struct RadixDigits {
+    uint32_t passes;
+    uint32_t shift[8], mask[8];
+};
+static constexpr uint32_t kTotalReplicas = 4;
+
+// totals[pass][replica][256] += the number of keys whose digit of that pass is d; a workgroup counts in LDS (a wave
+// whose keys share a digit - the upper bytes of sorted or narrow keys - adds once) and adds its counts to one of the
+// replicas.  Grid-stride over chunks of 256 x 16 keys.
+template <typename KeyT>
+__global__ void __launch_bounds__(256) radix_totals_kernel(uint32_t n, const KeyT* __restrict__ keys, RadixDigits dg,
+                                                            uint32_t* __restrict__ totals) {
+    __shared__ uint32_t lh[8][kRadix];
+    const uint32_t t = threadIdx.x, lane = t & 63u;
+    for (uint32_t p = 0; p < dg.passes; ++p)
+        lh[p][t] = 0;
+    __syncthreads();
+    for (uint64_t chunk = (uint64_t)blockIdx.x * 4096u; chunk < n; chunk += (uint64_t)gridDim.x * 4096u) {
+        KeyT key[16];
+#pragma unroll
+        for (uint32_t r = 0; r < 16; ++r) {
+            const uint64_t idx = chunk + r * 256u + t;
+            key[r] = idx < n ? keys[idx] : (KeyT)0;
+        }
+#pragma unroll
+        for (uint32_t r = 0; r < 16; ++r) {
+            const bool valid = chunk + r * 256u + t < n;
+            const uint64_t active = __ballot(valid);
+            if (active == 0)
+                continue;
+            const uint32_t first = (uint32_t)__builtin_ctzll(active);
+            for (uint32_t p = 0; p < dg.passes; ++p) {
+                const uint32_t d = digit_of(key[r], dg.shift[p], dg.mask[p]);
+                const uint32_t d_first = (uint32_t)__builtin_amdgcn_readlane((int)d, first);
+                if (__ballot(valid && d != d_first) == 0) {
+                    if (lane == first)
+                        atomicAdd(&lh[p][d], (uint32_t)__builtin_popcountll(active));
+                } else if (valid) {
+                    atomicAdd(&lh[p][d], 1u);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    uint32_t* mine = totals + (size_t)(blockIdx.x % kTotalReplicas) * kRadix;
+    for (uint32_t p = 0; p < dg.passes; ++p) {
+        const uint32_t c = lh[p][t];
+        if (c != 0)
+            atomicAdd(mine + (size_t)p * kTotalReplicas * kRadix + t, c);
+    }
+}
+
+// zeroes the bookkeeping words of a chained sort (digit counts, error word, the first pass's status rows) and leaves
+// the number of pairs where the passes read it
+// (words n_word and n_word + 1: every word has one writer)
+__global__ void __launch_bounds__(256) radix_prepare_kernel(size_t n_words, uint32_t* __restrict__ words,
+                                                             size_t n_word, int64_t n) {
+    const size_t i = (size_t)blockIdx.x * 256u + threadIdx.x;
+    if (i < n_words)
+        words[i] = i == n_word ? (uint32_t)(uint64_t)n : i == n_word + 1 ? (uint32_t)((uint64_t)n >> 32) : 0u;
 }
 
 // ---- stable scatter -------------------------------------------------------------------------------
@@ -302,21 +369,41 @@ __global__ void __launch_bounds__(64 * NW) radix_scatter_kernel(uint32_t n, cons
 
 } // namespace gsx
 
+namespace gsx {
+namespace {
+template <typename KeyT>
+int chained_pass(uint32_t n_max, const KeyT* kin, const int32_t* vin, KeyT* kout, int32_t* vout, uint32_t shift,
+                 uint32_t bits, const uint32_t* digit_total, const RadixChainArgs& a, bool write_keys, void* stream);
+} // namespace
+} // namespace gsx
+
 using namespace gsx;
 
 namespace {
 static constexpr uint32_t kMaxPasses = 8;
 struct SortLayout {
+    // the three-launch pass: histogram table [256][nblocks] and the digit totals
     uint32_t nblocks;
-    size_t hist_off, totals_off, total;
+    size_t hist_off, totals_off, tabled_total;
+    // the chained sort, behind it: digit counts of every pass [8][kTotalReplicas][256], a line with the error word
+    // and the number of pairs, two status tables of `rows` x 256 words used in turn
+    uint32_t rows;
+    size_t digits_off, misc_off, status_off[2], total;
 };
+static constexpr size_t kDigitsBytes = (size_t)kMaxPasses * kTotalReplicas * kRadix * 4;
 uint32_t sort_items(int64_t n) { return n <= kSmallSortLimit ? kItemsSmall : kItemsLarge; }
 SortLayout sort_layout(int64_t n) {
     SortLayout L;
     L.nblocks = cdiv((uint64_t)n, 256u * sort_items(n));
     L.hist_off = 0;
     L.totals_off = align_up((size_t)L.nblocks * kRadix * 4, 256);
-    L.total = L.totals_off + (size_t)kRadix * 4;
+    L.tabled_total = L.totals_off + (size_t)kRadix * 4;
+    L.rows = radix_chained_rows(n);
+    L.digits_off = align_up(L.tabled_total, 256);
+    L.misc_off = L.digits_off + kDigitsBytes;
+    L.status_off[0] = L.misc_off + 256;
+    L.status_off[1] = L.status_off[0] + (size_t)L.rows * kRadix * 4;
+    L.total = L.status_off[1] + (size_t)L.rows * kRadix * 4;
     return L;
 }
 } // namespace
@@ -339,10 +426,11 @@ extern "C" int gsx_radix_sort_pairs_selector(int64_t n, uint32_t begin_bit, uint
 namespace {
 // first_hist_done: the caller's own kernel has already left the first pass's histogram table in the workspace
 // (gsx::radix_first_pass_table)
+// chained: the workspace holds gsx_radix_sort_pairs_workspace_bytes(n) (false: only the three-launch pass's part)
 template <typename KeyT>
 int sort_pairs(const char* what, int64_t n, KeyT* keys0, int32_t* vals0, KeyT* keys1, int32_t* vals1,
                uint32_t begin_bit, uint32_t end_bit, void* workspace, size_t workspace_bytes, int* selector_host,
-               void* stream, bool first_hist_done = false) {
+               void* stream, bool first_hist_done = false, bool chained = true) {
     if (selector_host)
         *selector_host = 0;
     if (n <= 0)
@@ -352,8 +440,13 @@ int sort_pairs(const char* what, int64_t n, KeyT* keys0, int32_t* vals0, KeyT* k
     GSX_REQUIRE(end_bit >= 1 && end_bit <= 8 * sizeof(KeyT) && begin_bit < end_bit, GSX_ERR_INVALID_ARGUMENT,
                 "%s: bits [%u, %u)", what, begin_bit, end_bit);
     const SortLayout L = sort_layout(n);
-    GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 && workspace_bytes >= L.total,
-                GSX_ERR_WORKSPACE, "%s: workspace needs %zu bytes, 256-byte aligned", what, L.total);
+    // measured: the chained sort is ahead from ~2 M pairs with 64-bit keys (310 against 339 us at 5.67 M pairs and 45
+    // bits, 834 against 973 us at 16 M) and from ~30 M pairs with 16-bit keys (706 against 812 us at 64 M); below, its
+    // few large workgroups and the extra read of the keys cost more than the launches they save
+    chained = chained && n < (1ll << kLbValueBits) && n > (sizeof(KeyT) == 8 ? kSmallSortLimit : (1ll << 25));
+    const size_t need = chained ? L.total : L.tabled_total;
+    GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 && workspace_bytes >= need,
+                GSX_ERR_WORKSPACE, "%s: workspace needs %zu bytes, 256-byte aligned", what, need);
     uint32_t* hist = (uint32_t*)((char*)workspace + L.hist_off);
     uint32_t* totals = (uint32_t*)((char*)workspace + L.totals_off);
     hipStream_t s = (hipStream_t)stream;
@@ -365,6 +458,45 @@ int sort_pairs(const char* what, int64_t n, KeyT* keys0, int32_t* vals0, KeyT* k
     const uint32_t width_lo = n_bits / passes, n_wide = n_bits % passes;
     int sel = 0;
     uint32_t shift = begin_bit;
+    if (chained) {
+        char* ws = (char*)workspace;
+        uint32_t* digits = (uint32_t*)(ws + L.digits_off);
+        uint32_t* error = (uint32_t*)(ws + L.misc_off);
+        int64_t* n_slot = (int64_t*)(ws + L.misc_off + 8);
+        uint32_t* status[2] = {(uint32_t*)(ws + L.status_off[0]), (uint32_t*)(ws + L.status_off[1])};
+        // digit counts, the line with the error word and the first status table are one run of words
+        const size_t n_words = (L.status_off[1] - L.digits_off) / 4;
+        hipLaunchKernelGGL(radix_prepare_kernel, dim3((uint32_t)cdiv((uint64_t)n_words, 256u)), dim3(256), 0, s, n_words,
+                           digits, (size_t)((uint32_t*)n_slot - digits), n);
+        GSX_LAUNCH_CHECK();
+        RadixDigits dg;
+        dg.passes = passes;
+        for (uint32_t pass = 0, at = begin_bit; pass < kMaxPasses; ++pass) {
+            const uint32_t bits = pass < passes ? width_lo + (pass < n_wide ? 1u : 0u) : 0u;
+            dg.shift[pass] = at, dg.mask[pass] = (1u << bits) - 1u;
+            at += bits;
+        }
+        const uint32_t blocks = (uint32_t)std::min<uint64_t>(cdiv((uint64_t)n, 4096u), 1024u);
+        hipLaunchKernelGGL(radix_totals_kernel<KeyT>, dim3(blocks), dim3(256), 0, s, (uint32_t)n, keys0, dg, digits);
+        GSX_LAUNCH_CHECK();
+        for (uint32_t pass = 0; pass < passes; ++pass) {
+            const uint32_t bits = width_lo + (pass < n_wide ? 1u : 0u);
+            RadixChainArgs a;
+            a.n_dev = n_slot, a.status = status[pass & 1u], a.error = error;
+            a.clear_status = pass + 1 < passes ? status[(pass + 1) & 1u] : nullptr, a.clear_rows = L.rows;
+            a.total_replicas = kTotalReplicas, a.total_stride = kRadix;
+            const int rc = chained_pass<KeyT>((uint32_t)n, sel ? keys1 : keys0, sel ? vals1 : vals0, sel ? keys0 : keys1,
+                                              sel ? vals0 : vals1, shift, bits,
+                                              digits + (size_t)pass * kTotalReplicas * kRadix, a, true, stream);
+            if (rc != GSX_OK)
+                return rc;
+            sel ^= 1;
+            shift += bits;
+        }
+        if (selector_host)
+            *selector_host = sel;
+        return GSX_OK;
+    }
     const uint32_t items = sort_items(n);
     for (uint32_t pass = 0; pass < passes; ++pass) {
         const uint32_t bits = width_lo + (pass < n_wide ? 1u : 0u);
@@ -532,13 +664,13 @@ extern "C" int gsx_radix_sort_pairs_static(int64_t n, int64_t* keys0, int32_t* v
                 "radix_sort_pairs_static: n = %lld exceeds the built-in scratch's limit of %lld pairs "
                 "(use gsx_radix_sort_pairs with a workspace)",
                 (long long)n, (long long)GSX_RADIX_SORT_STATIC_MAX_PAIRS);
-    GSX_REQUIRE(gsx_radix_sort_pairs_workspace_bytes(n) <= kStaticScratchBytes, GSX_ERR_WORKSPACE,
-                "radix_sort_pairs_static: %zu bytes of scratch needed, %zu built in",
-                gsx_radix_sort_pairs_workspace_bytes(n), kStaticScratchBytes);
+    GSX_REQUIRE(sort_layout(n).tabled_total <= kStaticScratchBytes, GSX_ERR_WORKSPACE,
+                "radix_sort_pairs_static: %zu bytes of scratch needed, %zu built in", sort_layout(n).tabled_total,
+                kStaticScratchBytes);
     void* ws = nullptr;
     const int st = static_scratch(&ws);
     if (st != GSX_OK)
         return st;
     return sort_pairs<int64_t>("radix_sort_pairs_static", n, keys0, vals0, keys1, vals1, begin_bit, end_bit, ws,
-                               kStaticScratchBytes, selector_host, stream);
+                               kStaticScratchBytes, selector_host, stream, false, false);
 }

@@ -33,18 +33,28 @@ __global__ void __launch_bounds__(256) fill_f32_kernel(size_t n, float v, float*
         out[i] = v;
 }
 
-// probe of wave_reduce16 for tests: in [n_waves][64 lanes][16], out [n_waves][16]
-__global__ void __launch_bounds__(64) wave_reduce16_probe_kernel(const float* __restrict__ in, float* __restrict__ out) {
-    float v[16];
+// probe of the wave reductions for tests: in [n_waves][64 lanes][V], out [n_waves][V], V = 16, 13 or 9
+template <uint32_t V>
+__global__ void __launch_bounds__(64) wave_reduce_probe_kernel(const float* __restrict__ in, float* __restrict__ out) {
+    float v[V];
     const uint32_t lane = threadIdx.x;
 #pragma unroll
-    for (uint32_t k = 0; k < 16; ++k)
-        v[k] = in[((size_t)blockIdx.x * 64 + lane) * 16 + k];
-    const float total = wave_reduce16(v, lane);
-    if ((lane & 3u) == 0) {
-        const uint32_t comp = ((lane >> 5) & 1u) * 8u + ((lane >> 4) & 1u) * 4u + ((lane >> 3) & 1u) * 2u + ((lane >> 2) & 1u);
-        out[(size_t)blockIdx.x * 16 + comp] = total;
+    for (uint32_t k = 0; k < V; ++k)
+        v[k] = in[((size_t)blockIdx.x * 64 + lane) * V + k];
+    float total;
+    uint32_t index;
+    if constexpr (V == 16) {
+        total = wave_reduce16(v, lane);
+        index = wave_component(lane);
+    } else if constexpr (V == 13) {
+        total = wave_reduce13(v, lane);
+        index = wave_reduce13_index(lane);
+    } else {
+        total = wave_reduce9(v, lane);
+        index = wave_reduce9_index(lane);
     }
+    if ((lane & 3u) == 0 && index < V)
+        out[(size_t)blockIdx.x * V + index] = total;
 }
 
 // CDIM = 3: the RGB training path.  CDIM = 1 / 4: the depth render modes (Rasterization.cpp:374-393).  Channels
@@ -90,6 +100,8 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
         return;
     const uint32_t tr = threadIdx.x;
     const uint32_t lane = tr & 63u;
+    // which of the 13 per-Gaussian sums this lane ends up with after the wave reduction (15: none)
+    const uint32_t sum_index = (lane & 3u) == 0 ? wave_reduce13_index(lane) : 15u;
     const TilePixel px = tile_pixel(tile_id, tile_width, tr);
     const uint32_t i = px.i, j = px.j;
     bool inside = (i < image_height && j < image_width);
@@ -229,9 +241,9 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             }
 
             // From here on without branches: a lane that is not valid carries ra = 1 and fac = v_alpha = 0, which
-            // leaves its T and colour buffer unchanged and makes all 16 of its partials zero.  The decisions above
+            // leaves its T and colour buffer unchanged and makes all 13 of its partials zero.  The decisions above
             // use the forward pass's exact arithmetic; the derivative chain may use the (refined) hardware reciprocal.
-            float v[kAcc];
+            float v[13]; // colours 0-2, k q 3-5, k q (x) q 6-11, opacity 12
             const float ra = valid ? gsx::rcp_refined(1.0f - alpha) : 1.0f;
             T *= ra;
             const float fac = valid ? alpha * T : 0.f;
@@ -283,10 +295,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             v[9] = v_gro.y * q.y;
             v[10] = v_gro.y * q.z;
             v[11] = v_gro.z * q.z;
-            v[12] = 0.f;
-            v[13] = 0.f;
-            v[14] = 0.f;
-            v[15] = v_opac;
+            v[12] = v_opac;
             behind = fma(-cdot, fac, behind);
 #pragma unroll
             for (uint32_t k = 0; k < NX; ++k) { // the gradients of the channels beyond the third: their own wave sums
@@ -301,13 +310,9 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
                         unsafeAtomicAdd(&gextra[(size_t)id_batch[t] * (NX ? NX : 1) + k], e);
                 }
             }
-            const float total = wave_reduce16(v, lane);
-            if ((lane & 3u) == 0) {
-                const uint32_t comp = ((lane >> 5) & 1u) * 8u + ((lane >> 4) & 1u) * 4u + ((lane >> 3) & 1u) * 2u +
-                                      ((lane >> 2) & 1u);
-                if (comp < 12u || comp == 15u)
-                    atomicAdd(&acc[(uint32_t)t * kAccLds + min(comp, 12u)], total); // LDS: ds_add_f32
-            }
+            const float total = wave_reduce13(v, lane);
+            if (sum_index < 13u)
+                atomicAdd(&acc[(uint32_t)t * kAccLds + sum_index], total); // LDS: ds_add_f32
         }
         __syncthreads();
         if (STATS)
@@ -390,11 +395,18 @@ __global__ void __launch_bounds__(256) rasterize_bwd_epilogue_kernel(
 
 using namespace gsx;
 
-extern "C" int gsx_debug_wave_reduce16(uint32_t n_waves, const float* in, float* out, void* stream) {
+extern "C" int gsx_debug_wave_reduce(uint32_t values, uint32_t n_waves, const float* in, float* out, void* stream) {
+    GSX_REQUIRE(values == 16 || values == 13 || values == 9, GSX_ERR_INVALID_ARGUMENT,
+                "debug_wave_reduce: %u values (16, 13 or 9)", values);
     if (n_waves == 0)
         return GSX_OK;
-    GSX_REQUIRE(in && out, GSX_ERR_INVALID_ARGUMENT, "debug_wave_reduce16: null tensor");
-    hipLaunchKernelGGL(wave_reduce16_probe_kernel, dim3(n_waves), dim3(64), 0, (hipStream_t)stream, in, out);
+    GSX_REQUIRE(in && out, GSX_ERR_INVALID_ARGUMENT, "debug_wave_reduce: null tensor");
+    if (values == 16)
+        hipLaunchKernelGGL(wave_reduce_probe_kernel<16>, dim3(n_waves), dim3(64), 0, (hipStream_t)stream, in, out);
+    else if (values == 13)
+        hipLaunchKernelGGL(wave_reduce_probe_kernel<13>, dim3(n_waves), dim3(64), 0, (hipStream_t)stream, in, out);
+    else
+        hipLaunchKernelGGL(wave_reduce_probe_kernel<9>, dim3(n_waves), dim3(64), 0, (hipStream_t)stream, in, out);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

@@ -268,7 +268,8 @@ def test_tile_count_prefix_sums(gsx, cuda, n):
     assert np.array_equal(cum.cpu().numpy(), want)
 
 
-@pytest.mark.parametrize("n,bits", [(1, 12), (65, 1), (4097, 8), (100_003, 12), (3_000_000, 13), (2_500_000, 16)])
+@pytest.mark.parametrize("n,bits", [(1, 12), (65, 1), (4097, 8), (100_003, 12), (3_000_000, 13), (2_500_000, 16),
+                                    (40_000_000, 15)])  # the last one: above the size where the passes are chained
 def test_tile_pair_sort_stable(gsx, cuda, n, bits):
     """the 16-bit-key sort is the stable sort on bits [0, bits): numpy's stable argsort of the masked keys (bits above
     the range do not take part and travel with their pair)"""
@@ -401,7 +402,7 @@ def test_tile_pairs_need_a_small_grid(gsx, cuda):
                                               c_p(x.data_ptr()), c_p(0)))
 
 
-@pytest.mark.parametrize("n", [1, 63, 64, 65, 4095, 4096, 4097, 100_003, 3_000_000])
+@pytest.mark.parametrize("n", [1, 63, 64, 65, 4095, 4096, 4097, 100_003, 2_097_152, 2_097_153, 3_000_000])
 def test_radix_sort_stable(gsx, orc, cuda, n):
     ops = gsx.ops
     rng = np.random.default_rng(n)
@@ -838,18 +839,20 @@ def test_add_noise_and_quats(gsx, orc, cuda):
     bits_equal(N(R), orc.quats_to_rotmats(rq), '')
 
 
-def test_wave_reduce16_probe(gsx, cuda):
-    """the 64-lane x 16-value halving reduction of the backward rasterizer (permlane swaps + DPP mirrors)"""
+@pytest.mark.parametrize("values", [16, 13, 9])
+def test_wave_reduce_probe(gsx, cuda, values):
+    """the 64-lane halving reductions of the backward rasterizers (permlane swaps + DPP mirrors) for 16, 13 and 9
+    sums at a time: every sum lands in the lane that is said to own it"""
     import ctypes
     L = gsx._lib
-    rng = np.random.default_rng(0)
+    rng = np.random.default_rng(values)
     nw = 37
-    x = rng.normal(0, 1, (nw, 64, 16)).astype(np.float32)
-    x[3] = np.arange(64 * 16, dtype=np.float32).reshape(64, 16)  # exact integers: any mis-routed lane shows
+    x = rng.normal(0, 1, (nw, 64, values)).astype(np.float32)
+    x[3] = np.arange(64 * values, dtype=np.float32).reshape(64, values)  # exact integers: any mis-routed lane shows
     xd = T(x, cuda)
-    out = torch.zeros((nw, 16), dtype=torch.float32, device=cuda)
-    L.check(L.lib().gsx_debug_wave_reduce16(ctypes.c_uint32(nw), ctypes.c_void_p(xd.data_ptr()),
-                                            ctypes.c_void_p(out.data_ptr()), ctypes.c_void_p(None)))
+    out = torch.full((nw, values), float("nan"), dtype=torch.float32, device=cuda)
+    L.check(L.lib().gsx_debug_wave_reduce(ctypes.c_uint32(values), ctypes.c_uint32(nw), ctypes.c_void_p(xd.data_ptr()),
+                                          ctypes.c_void_p(out.data_ptr()), ctypes.c_void_p(None)))
     torch.cuda.synchronize()
     got = N(out)
     assert np.array_equal(got[3], x[3].sum(0))
