@@ -30,6 +30,7 @@ static constexpr float kFgsMinT = 1e-4f;             // :21
 // 32-lane warp (:32).  A cooperative round on 64 lanes costs a wave-wide pass per Gaussian however few tiles are left:
 // 12 measured best at 1 M Gaussians (preprocess 105 -> 78 us, instances 98 -> 65 us; 4, 8, 16, 32, 64 tried)
 static constexpr uint32_t kFgsSequential = 12;
+static constexpr uint32_t kFgsMaxRestFloats = 45; // 15 higher-band coefficients x 3 channels (degree 3)
 static constexpr uint32_t kFgsPrimF4 = 3;            // per-primitive record: 12 floats
 static constexpr uint32_t kFgsAcc = 12;              // backward accumulator row (9 used)
 
@@ -625,6 +626,14 @@ __global__ void __launch_bounds__(256) fgs_preprocess_bwd_kernel(
     const bool in = i < N;
     const bool live = in && n_touched[i] != 0;
     const uint32_t B = c.total_rest;
+    // The gradient rows of the higher SH bands (180 bytes a Gaussian at degree 3) leave through LDS: a lane fills its
+    // own row there and the workgroup then writes its 256 rows, which are one contiguous piece of grad_shN, with
+    // 16-byte stores by consecutive lanes (a lane storing its row itself touches 64 cache lines per instruction:
+    // 202 us against 121 us at 1 M Gaussians).  Reading the coefficient rows the same way gains nothing here, and in
+    // the forward kernel the 46 KB of LDS cost more occupancy than the loads save (78 -> 122 us): not done.
+    __shared__ __align__(16) float g_stage[256 * kFgsMaxRestFloats];
+    const bool staged = 3u * B <= kFgsMaxRestFloats; // more stored bands than degree 3 has: every lane stores its own row
+    float* const gco = staged ? g_stage + threadIdx.x * 3u * B : grad_shN + (size_t)(in ? i : 0u) * 3u * B;
     float dcam[3] = {0.f, 0.f, 0.f}, mean[3] = {0.f, 0.f, 0.f};
     if (in && !live) {
 #pragma unroll
@@ -633,7 +642,7 @@ __global__ void __launch_bounds__(256) fgs_preprocess_bwd_kernel(
         reinterpret_cast<float4*>(grad_rotations_raw)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         grad_opacities_raw[i] = 0.f;
         for (uint32_t k = 0; k < 3 * B; ++k)
-            grad_shN[(size_t)i * 3 * B + k] = 0.f;
+            gco[k] = 0.f;
     }
     if (live) {
         float4* row = reinterpret_cast<float4*>(gacc + (size_t)i * kFgsAcc);
@@ -651,7 +660,6 @@ __global__ void __launch_bounds__(256) fgs_preprocess_bwd_kernel(
         for (int ch = 0; ch < 3; ++ch)
             grad_sh0[3 * (size_t)i + ch] = 0.28209479177387814f * gcol[ch];
         float dpos[3] = {0.f, 0.f, 0.f};
-        float* gco = grad_shN + (size_t)i * B * 3;
         const uint32_t active = c.active_bases;
         const uint32_t written = active > 9 ? 15u : (active > 4 ? 8u : (active > 1 ? 3u : 0u));
         for (uint32_t k = 3 * written; k < 3 * B; ++k)
@@ -805,6 +813,16 @@ __global__ void __launch_bounds__(256) fgs_preprocess_bwd_kernel(
             const float sx = gm2[0] * (0.5f * c.w), sy = gm2[1] * (0.5f * c.h);
             densification_info[(size_t)N + i] += gsx::sqrt(sx * sx + sy * sy);
         }
+    }
+    if (staged && B != 0) {
+        __syncthreads();
+        const size_t first_row = (size_t)blockIdx.x * 256u;
+        const uint32_t floats = (uint32_t)min((size_t)256, (size_t)N - first_row) * 3u * B;
+        float* const dst = grad_shN + first_row * 3u * B; // 16-byte aligned: 256 rows are a multiple of four floats
+        for (uint32_t k = threadIdx.x; k < floats / 4u; k += 256u)
+            reinterpret_cast<float4*>(dst)[k] = reinterpret_cast<const float4*>(g_stage)[k];
+        for (uint32_t k = (floats & ~3u) + threadIdx.x; k < floats; k += 256u)
+            dst[k] = g_stage[k];
     }
     if (grad_w2c_partial != nullptr) { // kernels_backward.cuh:177-190; uniform branch, every lane takes part
         const uint32_t lane = threadIdx.x & 63u;
