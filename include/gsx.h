@@ -142,7 +142,9 @@ GSX_API uint32_t gsx_n_bits(uint32_t n);
 /* ---- a5: gsplat::radix_sort_double_buffer (Intersect.h:39-46; IntersectTile.cu:290-328) ----
  * Stable ascending LSD radix sort of (i64 key, i32 value) pairs on key bits [begin_bit, end_bit) (the reference
  * passes begin_bit = 0).  Buffers 0 (keys0/vals0, the input) and 1 (keys1/vals1) are ping-ponged; *selector_host
- * (host int) says which pair holds the result (like cub::DoubleBuffer::selector). */
+ * (host int) says which pair holds the result (like cub::DoubleBuffer::selector).  The workspace needs no particular
+ * contents on entry; from 2 M pairs on, the sort is a fill of its bookkeeping words, one count of the digits of
+ * every pass and one launch per 8-bit pass, below that three launches per pass (same result either way). */
 GSX_API size_t gsx_radix_sort_pairs_workspace_bytes(int64_t n);
 /* the selector gsx_radix_sort_pairs will report for this size and bit range (known before the sort runs) */
 GSX_API int gsx_radix_sort_pairs_selector(int64_t n, uint32_t begin_bit, uint32_t end_bit);
