@@ -227,7 +227,9 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
                 valid = false;
             if ((reach_mask & near_mask) == 0)
                 continue;
-            const float vis = gsx::exp_nonpos(gsx::fmax(power, kPowerFloor)); // lanes that are not valid may be far
+            // (a lane below its cut-off may be far outside exp_nonpos's range: what it gets back is meaningless and
+            // stays in that lane - it is not valid, and everything it feeds below goes through a select on `valid`)
+            const float vis = gsx::exp_nonpos(power);
             const float alpha = gsx::fmin(0.999f, a.w * vis);
             const uint64_t alpha_mask =
                 __builtin_amdgcn_ballot_w64(!(power > 0.f)) & __builtin_amdgcn_ballot_w64(!(alpha < 1.f / 255.f));
@@ -267,10 +269,9 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
                 cdot = fma(XLDS ? extra[(uint32_t)t * (NX ? NX : 1) + k]
                                 : colors[(size_t)id_batch[t] * CDIM + 3 + k],
                            v_render_c[CDIM > 3 ? 3 + k : 0], cdot);
-            float v_alpha = fma(T, cdot, ra * behind);
+            const float v_alpha = fma(T, cdot, ra * behind);
             // the clamp at 0.999 has zero derivative (:322)
-            v_alpha = (valid && a.w * vis <= 0.999f) ? v_alpha : 0.f;
-            const float v_opac = vis * v_alpha;
+            const float v_opac = (valid && a.w * vis <= 0.999f) ? vis * v_alpha : 0.f;
             // Geometry (:325-345).  With n = grd / |grd|, g = gro and q = g - (g . n) n (the point of the pixel's ray
             // nearest the Gaussian's centre, in the Gaussian's frame) the reference's chain is, exactly,
             //   v_gro = k q,   v_grd = t v_gro,   k = -opacity v_opacity,   t = -(g . n) / |grd|,
