@@ -443,9 +443,11 @@ __global__ void __launch_bounds__(256) fgs_blend_fwd_kernel(
             const float4 q0 = stage[t * 3 + 0], q1 = stage[t * 3 + 1];
             const float dx = q0.x - pxf, dy = q0.y - pyf;
             const float sigma_over_2 = 0.5f * (q0.z * dx * dx + q1.x * dy * dy) + q0.w * dx * dy;
-            if (done || sigma_over_2 < 0.0f)
+            // beyond 87 the exponential is zero (gsx::exp) and alpha with it; up to there its restricted variant has
+            // the same bits
+            if (done || sigma_over_2 < 0.0f || sigma_over_2 > 87.0f)
                 continue;
-            const float gaussian = gsx::exp(-sigma_over_2);
+            const float gaussian = gsx::exp_nonpos(-sigma_over_2);
             const float og = q1.y * gaussian;
             const float alpha = og < kFgsMaxAlpha ? og : kFgsMaxAlpha;
             if (alpha < kFgsMinAlpha)
@@ -560,11 +562,11 @@ __global__ void __launch_bounds__(256) fgs_blend_bwd_kernel(
             const float4 q0 = stage[t * 3 + 0], q1 = stage[t * 3 + 1], q2 = stage[t * 3 + 2];
             const float dx = q0.x - pxf, dy = q0.y - pyf;
             const float sigma_over_2 = 0.5f * (q0.z * dx * dx + q1.x * dy * dy) + q0.w * dx * dy;
-            if (sigma_over_2 < 0.0f)
+            if (sigma_over_2 < 0.0f || sigma_over_2 > 87.0f) // beyond 87: exp = 0 and alpha below the threshold
                 valid = false;
             if (__builtin_amdgcn_ballot_w64(valid) == 0)
                 continue;
-            const float gaussian = gsx::exp(-(valid ? sigma_over_2 : 0.0f));
+            const float gaussian = gsx::exp_nonpos(-(valid ? sigma_over_2 : 0.0f)); // gsx::exp's bits on [-87, 0]
             const float og = q1.y * gaussian;
             const float alpha = og < kFgsMaxAlpha ? og : kFgsMaxAlpha;
             if (alpha < kFgsMinAlpha)
