@@ -231,9 +231,9 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             // stays in that lane - it is not valid, and everything it feeds below goes through a select on `valid`)
             const float vis = gsx::exp_nonpos(power);
             const float alpha = gsx::fmin(0.999f, a.w * vis);
-            const uint64_t alpha_mask =
-                __builtin_amdgcn_ballot_w64(!(power > 0.f)) & __builtin_amdgcn_ballot_w64(!(alpha < 1.f / 255.f));
-            if (power > 0.f || alpha < 1.f / 255.f)
+            // (the reference's `power > 0` never fires: the power is -0.5 times a sum of squares)
+            const uint64_t alpha_mask = __builtin_amdgcn_ballot_w64(!(alpha < 1.f / 255.f));
+            if (alpha < 1.f / 255.f)
                 valid = false;
             if ((reach_mask & near_mask & alpha_mask) == 0)
                 continue; // no lane of this wave sees the Gaussian (:286-289)
