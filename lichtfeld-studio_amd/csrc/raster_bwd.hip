@@ -222,9 +222,9 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             // below the record's cut-off alpha < 1/255 whatever the rounding: decided without the exp
             // (the wave-wide tests combine the comparisons' own lane masks: a ballot of the combined flag would first
             // turn it into a register and compare that again)
-            const uint64_t near_mask = __builtin_amdgcn_ballot_w64(!(power < cuts[t]));
-            if (power < cuts[t])
-                valid = false;
+            const bool near = !(power < cuts[t]);
+            const uint64_t near_mask = __builtin_amdgcn_ballot_w64(near);
+            valid = valid && near;
             if ((reach_mask & near_mask) == 0)
                 continue;
             // (a lane below its cut-off may be far outside exp_nonpos's range: what it gets back is meaningless and
@@ -232,9 +232,9 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             const float vis = gsx::exp_nonpos(power);
             const float alpha = gsx::fmin(0.999f, a.w * vis);
             // (the reference's `power > 0` never fires: the power is -0.5 times a sum of squares)
-            const uint64_t alpha_mask = __builtin_amdgcn_ballot_w64(!(alpha < 1.f / 255.f));
-            if (alpha < 1.f / 255.f)
-                valid = false;
+            const bool opaque_enough = !(alpha < 1.f / 255.f);
+            const uint64_t alpha_mask = __builtin_amdgcn_ballot_w64(opaque_enough);
+            valid = valid && opaque_enough;
             if ((reach_mask & near_mask & alpha_mask) == 0)
                 continue; // no lane of this wave sees the Gaussian (:286-289)
             if (STATS) {
