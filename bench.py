@@ -126,9 +126,13 @@ def main():
     ap.add_argument("--host-count", action="store_true",
                     help="fetch the pair count to the host in every step (default: it stays on the device)")
     ap.add_argument("--cpu-threads", type=int, default=0, help="threads for the CPU baseline (0 = all)")
-    ap.add_argument("--workload", choices=["gut", "fastgs"], default="gut",
-                    help="gut: the training step of the metric (default); fastgs: forward + backward of the "
-                         "reference's default rasterizer on the same scene (a secondary line, not the metric)")
+    ap.add_argument("--workload", choices=["gut", "ops_path", "fastgs"], default="gut",
+                    help="gut: the training step of the metric (default); ops_path: the same step issued operator by "
+                         "operator through the C++ mirror of gsplat/Ops.h, with autograd and ATen glue, as "
+                         "LichtFeld's trainer issues it; fastgs: forward + backward of the reference's default "
+                         "rasterizer on the same scene (a secondary line, not the metric)")
+    ap.add_argument("--no-boundary-path", action="store_true",
+                    help="leave the operator-by-operator step (boundary_path) out of the default line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the path has no multi-GPU part); use --gpus 1", file=sys.stderr)
@@ -163,6 +167,18 @@ def main():
         sys.exit(f"bench.py: configuration {args.config} has no training target (a forward-only parity case); "
                  "the training step is timed on configurations 1, 3, 4 and 5")
     use_ssim = args.config != 1  # configuration 1 is L1 only
+    if args.workload == "ops_path":
+        res = run_ops_path(args, gsx, sc, viewmat, Kmat, W, H, gt, dev)
+        print(json.dumps({
+            "metric": "train it/s issued operator by operator through the gsplat/Ops.h mirror (secondary; the "
+                      "BASELINE metric is the default workload)",
+            "value": res["it_per_s"], "unit": "it/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "f32", "data": "synthetic",
+            "config": {"workload": f"BASELINE configs[{args.config - 1}] through OpsPathTrainer "
+                                   "(csrc/host/ops_path.cpp)", "n_gaussians": int(sc.means.shape[0]),
+                       "image": [W, H]}, "boundary_path": res}))
+        return
     ts = TrainStep(sc, dev, use_ssim=use_ssim, fused_update=not args.separate_update,
                    fused_loss=not args.separate_update, overlap=not args.no_overlap,
                    one_front_pass=args.one_front_pass, device_count=not args.host_count)
@@ -277,6 +293,16 @@ def main():
                 "(rocprofv3 FETCH_SIZE + WRITE_SIZE, copy-kernel calibrated) from profiles/",
     }
 
+    # the same step through the C++ layers a LichtFeld build links: operator by operator as its trainer issues them
+    # (ops_path), and the C++ step driver over the fused entry points (cpp_train_step)
+    boundary = None
+    if default_workload and not args.no_boundary_path and not args.separate_update:
+        boundary = {"ops_path": run_ops_path(args, gsx, sc, viewmat, Kmat, W, H, gt, dev),
+                    "cpp_train_step": run_cpp_step(args, gsx, sc, viewmat, Kmat, W, H, gt, dev)}
+        headline = args.steps / elapsed
+        boundary["ops_path_vs_headline"] = round(boundary["ops_path"]["it_per_s"] / headline, 3)
+        boundary["cpp_train_step_vs_headline"] = round(boundary["cpp_train_step"]["it_per_s"] / headline, 3)
+
     cpu_baseline, parity = None, None
     if not args.no_cpu_baseline:
         cpu_baseline = run_cpu_baseline(gsx, sc, cam, gt.cpu().numpy()[0], use_ssim, args.cpu_threads)
@@ -306,12 +332,84 @@ def main():
                    "contributing_half_blocks_8x4": half_rows, "contributing_half_blocks_4x8": half_cols, "loss": loss, "setup_s": round(setup_s, 1)},
         "raster_fwd_ms": kernels.get("rasterize_to_pixels_from_world_3dgs_fwd", {}).get("ms"),
         "raster_bwd_ms": round(dom_ms, 4),
-        "roofline": roofline, "cpu_baseline": cpu_baseline, "parity_in_bench": parity,
+        "roofline": roofline, "cpu_baseline": cpu_baseline, "parity_in_bench": parity, "boundary_path": boundary,
         "copy_probe": {"bytes_moved": 2 * copy_bytes, "GBps": round(copy_gbs, 1),
                        "note": "gsx_debug_copy, 1 GiB read + 1 GiB written: measured streaming bandwidth"},
         "kernels": kernels,
     }
     print(json.dumps(out))
+
+
+def run_ops_path(args, gsx, sc, viewmat, Kmat, W, H, gt, dev, steps=None, warmup=None):
+    """The step of the metric issued the way Trainer::train_step issues it (trainer.cpp:599-875): ATen activations and
+    concatenation, the autograd Function around rasterize_from_world_with_sh_fwd / _bwd, clamp / permute, l1_loss +
+    fused_ssim, loss.backward(), one adam_step_wrapper launch per group - all in C++ (csrc/host/ops_path.cpp)."""
+    import numpy as np
+    import torch
+    from lichtfeld_studio_amd import _lib
+    from lichtfeld_studio_amd.trainer import DEFAULT_LRS
+    ext = _lib.torch_ext()
+    steps = args.steps if steps is None else steps
+    warmup = args.warmup if warmup is None else warmup
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(dev)
+    lrs = [DEFAULT_LRS[k] for k in ("means", "sh0", "shN", "scaling", "rotation", "opacity")]
+    tr = ext.OpsPathTrainer(t(sc.means), t(sc.sh0), t(sc.shN), t(sc.scaling_raw), t(sc.rotation_raw),
+                            t(sc.opacity_raw.reshape(-1, 1)), int(sc.sh_degree), lrs, 0.2, False)
+    gt3 = gt[0].contiguous()
+    views = [viewmat, viewmat.clone()]
+    first = None
+    for i in range(warmup):
+        loss = tr.train_step(i + 1, views[i % 2], Kmat, W, H, gt3)
+        if i == 0:
+            first = float(loss)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for i in range(steps):
+        loss = tr.train_step(warmup + i + 1, views[i % 2], Kmat, W, H, gt3)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t1
+    # the same with the reference's loss.item() after backward (trainer.cpp:708): the host waits for the device once
+    # per step
+    t2 = time.perf_counter()
+    for i in range(steps):
+        loss = tr.train_step(warmup + steps + i + 1, views[i % 2], Kmat, W, H, gt3)
+        last = float(loss)
+    torch.cuda.synchronize()
+    elapsed_item = time.perf_counter() - t2
+    return {"it_per_s": round(steps / elapsed, 3), "ms_per_step": round(1e3 * elapsed / steps, 4),
+            "it_per_s_with_loss_item": round(steps / elapsed_item, 3), "first_loss": first, "last_loss": last,
+            "what": "OpsPathTrainer.train_step: rasterize_from_world_with_sh_fwd/_bwd under autograd, ATen "
+                    "activations / cat / clamp / permute / l1_loss, fused_ssim, six adam_step_wrapper launches"}
+
+
+def run_cpp_step(args, gsx, sc, viewmat, Kmat, W, H, gt, dev, steps=None, warmup=None):
+    """gsx::TrainStep (csrc/host/train_step.cpp): the step of the metric over the fused entry points, driven from
+    C++ - the launches of the default workload without the interpreter between them."""
+    import numpy as np
+    import torch
+    from lichtfeld_studio_amd import _lib
+    from lichtfeld_studio_amd.trainer import DEFAULT_LRS
+    ext = _lib.torch_ext()
+    steps = args.steps if steps is None else steps
+    warmup = args.warmup if warmup is None else warmup
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(dev)
+    lrs = [DEFAULT_LRS[k] for k in ("means", "sh0", "shN", "scaling", "rotation", "opacity")]
+    cs = ext.TrainStep(t(sc.means), t(np.concatenate([sc.sh0, sc.shN], 1)), t(sc.scaling_raw), t(sc.rotation_raw),
+                       t(sc.opacity_raw.reshape(-1)), lrs, sh_degree=int(sc.sh_degree))
+    views = [viewmat, viewmat.clone()]
+    cs.steps(views, Kmat, W, H, gt, 1)
+    first = [float(x) for x in cs.loss_out.cpu()]
+    if warmup > 1:
+        cs.steps(views, Kmat, W, H, gt, warmup - 1)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    cs.steps(views, Kmat, W, H, gt, steps)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t1
+    assert cs.lists_error() == (0, 0) and cs.steps_held == 0
+    return {"it_per_s": round(steps / elapsed, 3), "ms_per_step": round(1e3 * elapsed / steps, 4),
+            "first_loss": first, "n_isects": int(cs.n_isects()),
+            "what": "gsx::TrainStep::step called from a C++ loop: the 18 launches of the default workload"}
 
 
 def run_fastgs(args, gsx, sc, cam, dev):

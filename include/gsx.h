@@ -475,6 +475,10 @@ typedef struct gsx_update_args {
      * kernel runs, in place of the three fields above (a launch replayed from a HIP graph keeps its by-value
      * arguments; the step's scalars change every iteration) */
     const float* step_scalars;
+    /* nullable, PINNED HOST memory (hipHostMalloc), one u64: with `hold` given, every launch stores
+     * hold[1] << 32 | hold[0] there as they stand after the launch (one 8-byte store at system scope) - the host sees
+     * the sticky error bits and the number of calls held back so far without a synchronisation */
+    uint64_t* hold_report;
 } gsx_update_args;
 GSX_API int gsx_backward_update_fused(const gsx_update_args* args_host, void* stream);
 

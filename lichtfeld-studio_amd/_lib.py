@@ -69,7 +69,7 @@ class UpdateArgs(ctypes.Structure):
                                     "beta1", "beta2", "eps", "bias_correction1_rcp",
                                     "bias_correction2_sqrt_rcp")] +
                 [("skip_shN", ctypes.c_int32), ("reg_scaling", c_f), ("reg_opacity", c_f), ("hold", c_p),
-                 ("step_scalars", c_p)])
+                 ("step_scalars", c_p), ("hold_report", c_p)])
 
 
 class GsxError(RuntimeError):
@@ -114,3 +114,14 @@ def lib():
 def check(status):
     if status != GSX_OK:
         raise GsxError(status, lib().gsx_last_error().decode())
+
+
+def torch_ext():
+    """gsx_torch_ext: the pybind11 module over the C++ host layer (csrc/host/*.cpp), built in-tree by build_ext.py.
+    Fails loudly when it has not been built."""
+    import importlib
+    import sys
+    import torch  # noqa: F401  (LibTorch must be loaded first)
+    if _HERE not in sys.path:
+        sys.path.insert(0, _HERE)
+    return importlib.import_module("gsx_torch_ext")

@@ -53,8 +53,10 @@ def build():
         raise RuntimeError("libgsx.so is missing: run build.py first")
     os.makedirs(OBJ, exist_ok=True)
     cflags, ldflags = _flags()
-    srcs = [os.path.join(HOST, "gsplat_ops.cpp"), os.path.join(HOST, "fastgs_api.cpp"), os.path.join(HOST, "bindings.cpp")]
-    with ThreadPoolExecutor(max_workers=3) as ex:
+    srcs = [os.path.join(HOST, "gsplat_ops.cpp"), os.path.join(HOST, "fastgs_api.cpp"), os.path.join(HOST, "ops_path.cpp"),
+            os.path.join(HOST, "train_step.cpp"),
+            os.path.join(HOST, "bindings.cpp")]
+    with ThreadPoolExecutor(max_workers=5) as ex:
         objs = list(ex.map(_compile, [(s, cflags) for s in srcs]))
     subprocess.run([CXX, *objs, *ldflags, "-o", OUT], check=True)
     return OUT

@@ -9,6 +9,14 @@
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
 #include <c10/util/Exception.h>
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
+#include <deque>
+#include <memory>
+#include <mutex>
+#include <optional>
+#include <vector>
 
 #include "gsx.h"
 
@@ -502,6 +510,110 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> rasterize
     return std::make_tuple(v_means, v_quats, v_scales, v_colors, v_opacities);
 }
 
+
+namespace {
+
+// ---------------------------------------------------------------------------------------------------------------
+// The training camera's path through the two fused operators (one perfect pinhole, global shutter, RGB, no
+// compensations): the sequence gs::training::rasterize reaches every iteration (rasterizer.cpp:138-166).  Same
+// results as the general composition below, with what the reference allocates, recomputes and waits for per call
+// kept between calls instead:
+//  - scratch (tile-list workspace, backward accumulators, the pinned count slot, a second stream) lives in a
+//    StepScratch per (device, stream);
+//  - the pair count stays on the device until everything up to the rasterizer is queued (Intersect.cpp:76 blocks on
+//    it before the emission can even be sized);
+//  - the raster records and the per-tile costs of the forward pass ride in the storage of the `colors` output, so the
+//    backward pass that gets `colors` back finds them there (weak reference to the storage: no stale hits).
+// ---------------------------------------------------------------------------------------------------------------
+struct StepScratch {
+    int device = -1;
+    void* stream = nullptr;
+    std::mutex busy;  // one call at a time per (device, stream); other streams have their own scratch
+    uint32_t N = 0, tw = 0, th = 0;
+    int64_t cap = 0;
+    at::Tensor lists_ws, pinned, accum, order;
+    uint32_t accum_N = 0;
+    hipStream_t side = nullptr;
+    hipEvent_t fork = nullptr, join = nullptr;
+};
+
+std::mutex g_scratch_mutex;
+std::vector<std::unique_ptr<StepScratch>> g_scratch;
+
+StepScratch& scratch_for(const at::Tensor& like, void* stream) {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    const int dev = like.device().index();
+    for (auto& s : g_scratch)
+        if (s->device == dev && s->stream == stream)
+            return *s;
+    auto s = std::make_unique<StepScratch>();
+    s->device = dev;
+    s->stream = stream;
+    s->side = c10::hip::getStreamFromPool(/*isHighPriority=*/false, (c10::DeviceIndex)dev).stream();
+    TORCH_CHECK(hipEventCreateWithFlags(&s->fork, hipEventDisableTiming) == hipSuccess &&
+                    hipEventCreateWithFlags(&s->join, hipEventDisableTiming) == hipSuccess,
+                "gsx: hipEventCreate failed");
+    s->pinned = at::empty({1}, at::TensorOptions().dtype(at::kLong).pinned_memory(true));
+    g_scratch.push_back(std::move(s));
+    return *g_scratch.back();
+}
+
+// what a forward pass left in the storage behind its `colors` output
+struct ForwardExtras {
+    c10::weak_intrusive_ptr<c10::StorageImpl> storage;
+    uint32_t N, W, H, tw, th;
+    int64_t records_at, walk_at;  // float offsets into the storage
+    const void *means, *viewmat, *K;
+};
+std::mutex g_extras_mutex;
+std::deque<ForwardExtras> g_extras;
+
+void remember_extras(ForwardExtras e) {
+    std::lock_guard<std::mutex> lock(g_extras_mutex);
+    g_extras.erase(std::remove_if(g_extras.begin(), g_extras.end(), [](const ForwardExtras& x) { return x.storage.expired(); }),
+                   g_extras.end());
+    if (g_extras.size() >= 16)
+        g_extras.pop_front();
+    g_extras.push_back(std::move(e));
+}
+
+std::optional<ForwardExtras> find_extras(const at::Tensor& colors) {
+    if (!colors.defined() || !colors.has_storage())
+        return std::nullopt;
+    const c10::StorageImpl* impl = colors.storage().unsafeGetStorageImpl();
+    std::lock_guard<std::mutex> lock(g_extras_mutex);
+    for (auto it = g_extras.rbegin(); it != g_extras.rend(); ++it)
+        if (it->storage._unsafe_get_target() == impl && !it->storage.expired())
+            return *it;
+    return std::nullopt;
+}
+
+inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+
+// the pair count of gsx_tile_lists, once it has landed in the pinned slot
+int64_t await_count(const at::Tensor& pinned, void* stream) {
+    volatile int64_t* slot = pinned.data_ptr<int64_t>();
+    for (int i = 0; i < 4000000; ++i) {
+        const int64_t n = *slot;
+        if (n >= 0)
+            return n;
+    }
+    TORCH_CHECK(hipStreamSynchronize((hipStream_t)stream) == hipSuccess, "gsx: hipStreamSynchronize failed");
+    return *slot;
+}
+
+bool training_camera(const at::Tensor& viewmats0, const gsplat::OptT& viewmats1, const gsplat::OptT& masks,
+                     gsplat::CameraModelType camera_model, ShutterType rs_type, const gsplat::OptT& radial,
+                     const gsplat::OptT& tangential, const gsplat::OptT& thin_prism, bool calc_compensations,
+                     int render_mode, uint32_t tile_size, uint32_t tile_width, uint32_t tile_height) {
+    (void)masks;
+    return viewmats0.size(0) == 1 && !has(viewmats1) && camera_model == gsplat::PINHOLE && rs_type == ShutterType::GLOBAL &&
+           !has(radial) && !has(tangential) && !has(thin_prism) && !calc_compensations && render_mode == 0 &&
+           tile_size == 16 && gsx_intersect_tile_pairs_fit(tile_width, tile_height);
+}
+
+} // namespace
+
 // The fused operators hand the caller's background ([C,3] from gs::training::rasterize, rasterizer.cpp:84-87, 147)
 // to a kernel that blends `channels` values per pixel (Rasterization.cpp:401-407): with RGB + depth it would read one
 // float past each row.  Here the missing channels' background is 0 and surplus ones are dropped (for one camera the
@@ -551,6 +663,96 @@ rasterize_from_world_with_sh_fwd(const at::Tensor means, const at::Tensor quats,
                                          thin_prism_coeffs);
     at::Tensor radii = std::get<0>(proj), means2d = std::get<1>(proj), depths = std::get<2>(proj);
     at::Tensor compensations = std::get<4>(proj);
+    const uint32_t tile_width = (image_width + tile_size - 1) / tile_size;
+    const uint32_t tile_height = (image_height + tile_size - 1) / tile_size;
+    if (N > 0 && image_width > 0 && image_height > 0 &&
+        training_camera(viewmats0, viewmats1, masks, camera_model, rs_type, radial_coeffs, tangential_coeffs,
+                        thin_prism_coeffs, calc_compensations, render_mode, tile_size, tile_width, tile_height)) {
+        sized(sh_coeffs, "sh_coeffs", {N, -1, 3});
+        const OptT bg = fit_backgrounds(backgrounds, 3);
+        TORCH_CHECK(!has(bg) || (bg->dim() == 2 && bg->size(0) == 1), "backgrounds must be [C, channels], got ",
+                    bg->sizes());
+        sized(masks, "masks", {1, tile_height, tile_width});
+        void* stream = cur_stream(means);
+        StepScratch& sc = scratch_for(means, stream);
+        std::lock_guard<std::mutex> busy(sc.busy);
+        const uint32_t tiles = tile_width * tile_height;
+        // colours | raster records | per-tile walk lengths in one storage: the backward pass finds the last two
+        // behind the colours it is handed back
+        const int64_t records_at = round_up(3 * (int64_t)N, 64);
+        const int64_t walk_at = records_at + (int64_t)(gsx_raster_records_bytes(N) / 4);
+        at::Tensor pack = at::empty({walk_at + tiles}, means.options());
+        at::Tensor colors = pack.narrow(0, 0, 3 * (int64_t)N).view({1, (int64_t)N, 3});
+        float* records = pack.data_ptr<float>() + records_at;
+        uint32_t* walk = reinterpret_cast<uint32_t*>(pack.data_ptr<float>() + walk_at);
+        auto hip_ok = [](hipError_t e) { TORCH_CHECK(e == hipSuccess, "gsx: ", hipGetErrorString(e)); };
+        hip_ok(hipEventRecord(sc.fork, (hipStream_t)stream));
+        hip_ok(hipStreamWaitEvent(sc.side, sc.fork, 0));
+        // SH colours + records beside the (latency-bound) tile lists
+        gsx_check(gsx_sh_colors_records_from_world(N, (uint32_t)sh_coeffs.size(1), sh_degree, means.data_ptr<float>(),
+                                                   quats.data_ptr<float>(), scaled_scales.data_ptr<float>(),
+                                                   op_flat.data_ptr<float>(), sh_coeffs.data_ptr<float>(),
+                                                   radii.data_ptr<int32_t>(), viewmats0.data_ptr<float>(),
+                                                   Ks.data_ptr<float>(), image_width, image_height,
+                                                   colors.data_ptr<float>(), records, sc.side));
+        hip_ok(hipEventRecord(sc.join, sc.side));
+        auto opt = means.options();
+        at::Tensor renders = at::empty({1, image_height, image_width, 3}, opt);
+        at::Tensor alphas = at::empty({1, image_height, image_width, 1}, opt);
+        at::Tensor last_ids = at::empty({1, image_height, image_width}, opt.dtype(at::kInt));
+        at::Tensor flat, offsets_full;
+        int64_t n = 0;
+        for (int attempt = 0;; ++attempt) {
+            if (sc.cap == 0)
+                sc.cap = 1 << 20;
+            if (sc.N != N || sc.tw != tile_width || sc.th != tile_height || !sc.lists_ws.defined()) {
+                const size_t bytes = gsx_tile_lists_workspace_bytes(N, sc.cap, tile_width, tile_height);
+                sc.lists_ws = workspace(bytes, means);
+                gsx_check(gsx_tile_lists_init(N, sc.cap, tile_width, tile_height, sc.lists_ws.data_ptr(),
+                                              (size_t)sc.lists_ws.numel(), stream));
+                sc.order = at::empty({(int64_t)tiles}, opt.dtype(at::kInt));
+                sc.N = N, sc.tw = tile_width, sc.th = tile_height;
+            }
+            flat = at::empty({sc.cap}, opt.dtype(at::kInt));
+            offsets_full = at::empty({(int64_t)tiles + 1}, opt.dtype(at::kInt));
+            *sc.pinned.data_ptr<int64_t>() = -1;
+            gsx_check(gsx_tile_lists(N, means2d.data_ptr<float>(), radii.data_ptr<int32_t>(), depths.data_ptr<float>(),
+                                     tile_size, tile_width, tile_height, sc.cap, sc.lists_ws.data_ptr(),
+                                     (size_t)sc.lists_ws.numel(), flat.data_ptr<int32_t>(),
+                                     offsets_full.data_ptr<int32_t>(), sc.pinned.data_ptr<int64_t>(), stream, sc.side));
+            gsx_check(gsx_tile_order(GSX_COUNT_IN_OFFSETS, offsets_full.data_ptr<int32_t>(), nullptr, tile_width,
+                                     tile_height, (uint32_t*)sc.order.data_ptr<int32_t>(), stream));
+            if (attempt == 0)
+                hip_ok(hipStreamWaitEvent((hipStream_t)stream, sc.join, 0));
+            gsx_check(gsx_rasterize_records_fwd(GSX_COUNT_IN_OFFSETS, records, nullptr, 3, fptr(bg), bptr(masks),
+                                                image_width, image_height, viewmats0.data_ptr<float>(),
+                                                Ks.data_ptr<float>(), offsets_full.data_ptr<int32_t>(),
+                                                flat.data_ptr<int32_t>(), (const uint32_t*)sc.order.data_ptr<int32_t>(),
+                                                walk, renders.data_ptr<float>(), alphas.data_ptr<float>(),
+                                                last_ids.data_ptr<int32_t>(), stream));
+            // everything up to the rasterizer is queued: only now does the host look at the count
+            n = await_count(sc.pinned, stream);
+            TORCH_CHECK(n < (1ll << 31), "gsx: ", n, " intersections do not fit int32 indices (Intersect.cpp:84-85)");
+            if (n <= sc.cap) {
+                if (n > sc.cap - sc.cap / 10) {  // room for the next call
+                    sc.cap = n + n / 4 + 1024;
+                    sc.lists_ws = at::Tensor();
+                }
+                break;
+            }
+            TORCH_CHECK(attempt == 0, "gsx: tile lists did not fit their buffers twice");
+            // the lists did not fit and were left empty: larger buffers (a fresh workspace, whose error word is
+            // clear), and the lists and the render once more
+            sc.cap = n + n / 4 + 1024;
+            sc.lists_ws = at::Tensor();
+        }
+        ForwardExtras ex{pack.storage().getWeakStorageImpl(), N, image_width, image_height, tile_width, tile_height, records_at, walk_at, means.data_ptr(),
+                         viewmats0.data_ptr(), Ks.data_ptr()};
+        remember_extras(std::move(ex));
+        at::Tensor offsets = offsets_full.narrow(0, 0, tiles).view({1, (int64_t)tile_height, (int64_t)tile_width});
+        return std::make_tuple(renders, alphas, radii, means2d, depths, colors, offsets, flat.narrow(0, 0, n), last_ids,
+                               compensations);
+    }
     at::Tensor colors;
     if (render_mode == 0 || render_mode == 3 || render_mode == 4) {
         // Rasterization.cpp:356-378 in one pass: dirs, radii mask, SH, + 0.5, clamp
@@ -566,8 +768,6 @@ rasterize_from_world_with_sh_fwd(const at::Tensor means, const at::Tensor quats,
     at::Tensor final_opacities = op_flat.unsqueeze(0);
     if (calc_compensations && compensations.defined() && compensations.numel() > 0)
         final_opacities = at::mul(final_opacities, compensations).contiguous();
-    const uint32_t tile_width = (image_width + tile_size - 1) / tile_size;
-    const uint32_t tile_height = (image_height + tile_size - 1) / tile_size;
     at::Tensor flatten_ids, offsets;
     if (!tile_lists(means2d, radii, depths, tile_size, tile_width, tile_height, &flatten_ids, &offsets)) {
         auto isect = intersect_tile(means2d, radii, depths, at::nullopt, at::nullopt, C, tile_size, tile_width,
@@ -610,6 +810,77 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> rasterize
     if (calc_compensations && compensations.defined() && compensations.numel() > 0)
         final_opacities = at::mul(final_opacities, compensations).contiguous();
     at::Tensor scaled_scales = scaling_modifier == 1.0f ? scales : at::mul(scales, scaling_modifier);
+    const uint32_t N = (uint32_t)means.size(0);
+    const uint32_t tile_width = tile_size ? (image_width + tile_size - 1) / tile_size : 0;
+    const uint32_t tile_height = tile_size ? (image_height + tile_size - 1) / tile_size : 0;
+    const std::optional<ForwardExtras> found = find_extras(colors);
+    if (N > 0 && tile_size == 16 && found && found->N == N && found->W == image_width &&
+        found->H == image_height && found->means == means.data_ptr() && found->viewmat == viewmats0.data_ptr() &&
+        found->K == Ks.data_ptr() &&
+        training_camera(viewmats0, viewmats1, masks, camera_model, rs_type, radial_coeffs, tangential_coeffs,
+                        thin_prism_coeffs, calc_compensations, render_mode, tile_size, tile_width, tile_height)) {
+        // the forward pass of the same inputs left its records and per-tile costs behind `colors`
+        const ForwardExtras& ex = *found;
+        CHECK_INPUT(colors);
+        CHECK_INPUT(tile_offsets);
+        CHECK_INPUT(flatten_ids);
+        CHECK_INPUT(render_alphas);
+        CHECK_INPUT(last_ids);
+        CHECK_INPUT(radii);
+        CHECK_INPUT(viewmats0);
+        sized(means, "means", {N, 3});
+        sized(quats, "quats", {N, 4});
+        sized(scales, "scales", {N, 3});
+        TORCH_CHECK(opacities.numel() == N, "opacities must hold ", N, " values, got ", opacities.sizes());
+        sized(sh_coeffs, "sh_coeffs", {N, -1, 3});
+        sized(colors, "colors", {1, N, 3});
+        sized(radii, "radii", {1, N, 2});
+        sized(tile_offsets, "tile_offsets", {1, tile_height, tile_width});
+        sized(masks, "masks", {1, tile_height, tile_width});
+        sized(render_alphas, "render_alphas", {1, image_height, image_width, 1});
+        sized(last_ids, "last_ids", {1, image_height, image_width});
+        sized(v_render_colors, "v_render_colors", {1, image_height, image_width, 3});
+        sized(v_render_alphas, "v_render_alphas", {1, image_height, image_width, 1});
+        const OptT bg = fit_backgrounds(backgrounds, 3);
+        void* stream = cur_stream(means);
+        StepScratch& sc = scratch_for(means, stream);
+        std::lock_guard<std::mutex> busy(sc.busy);
+        const size_t accum_bytes = gsx_rasterize_bwd_accum_bytes(N);
+        if (sc.accum_N != N || !sc.accum.defined()) {  // zeroed once: the epilogue leaves the rows it read zeroed
+            sc.accum = at::zeros({(int64_t)accum_bytes}, means.options().dtype(at::kByte));
+            sc.accum_N = N;
+        }
+        const uint32_t tiles = tile_width * tile_height;
+        if (!sc.order.defined() || sc.order.numel() != tiles)
+            sc.order = at::empty({(int64_t)tiles}, means.options().dtype(at::kInt));
+        const float* base = static_cast<const float*>(colors.storage().data());
+        const float* records = base + ex.records_at;
+        const uint32_t* walk = reinterpret_cast<const uint32_t*>(base + ex.walk_at);
+        const int64_t n = flatten_ids.size(0);
+        gsx_check(gsx_tile_order(n, nullptr, walk, tile_width, tile_height, (uint32_t*)sc.order.data_ptr<int32_t>(),
+                                 stream));
+        gsx_check(gsx_rasterize_bwd_accumulate(
+            1, N, n, records, nullptr, 3, fptr(bg), bptr(masks), image_width, image_height, tile_size,
+            viewmats0.data_ptr<float>(), Ks.data_ptr<float>(), tile_offsets.data_ptr<int32_t>(),
+            flatten_ids.data_ptr<int32_t>(), (const uint32_t*)sc.order.data_ptr<int32_t>(),
+            render_alphas.data_ptr<float>(), last_ids.data_ptr<int32_t>(), v_render_colors.data_ptr<float>(),
+            v_render_alphas.data_ptr<float>(), sc.accum.data_ptr(), accum_bytes, stream));
+        at::Tensor v_means = at::empty_like(means), v_quats = at::empty_like(quats), v_scales = at::empty_like(scales);
+        at::Tensor v_colors = at::empty_like(colors), v_opacities = at::empty_like(opacities);
+        gsx_check(gsx_rasterize_bwd_finish(N, means.data_ptr<float>(), quats.data_ptr<float>(),
+                                           scaled_scales.data_ptr<float>(), viewmats0.data_ptr<float>(),
+                                           sc.accum.data_ptr(), accum_bytes, 1, 3, v_means.data_ptr<float>(),
+                                           v_quats.data_ptr<float>(), v_scales.data_ptr<float>(),
+                                           v_colors.data_ptr<float>(), v_opacities.data_ptr<float>(), stream));
+        at::Tensor v_sh = at::empty_like(sh_coeffs);
+        gsx_check(gsx_sh_colors_from_world_bwd(N, (uint32_t)sh_coeffs.size(1), sh_degree, means.data_ptr<float>(),
+                                               radii.data_ptr<int32_t>(), viewmats0.data_ptr<float>(),
+                                               colors.data_ptr<float>(), v_colors.data_ptr<float>(),
+                                               v_sh.data_ptr<float>(), stream));
+        if (scaling_modifier != 1.0f)
+            v_scales = at::mul(v_scales, scaling_modifier);  // Rasterization.cpp:633
+        return std::make_tuple(v_means, v_quats, v_scales, v_opacities, v_sh);
+    }
     auto g = rasterize_to_pixels_from_world_3dgs_bwd(means, quats, scaled_scales, colors, final_opacities.contiguous(),
                                                      fit_backgrounds(backgrounds, colors.size(-1)), masks, image_width, image_height, tile_size,
                                                      viewmats0, viewmats1, Ks, camera_model, ut_params, rs_type,

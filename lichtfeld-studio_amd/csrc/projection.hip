@@ -223,6 +223,8 @@ __device__ __forceinline__ bool project_ut(const ProjCfg& cfg, const CamPose& cp
     return true;
 }
 
+// GENERAL = false: every camera a perfect pinhole with a global shutter (no coefficient rows, no end-of-frame pose)
+template <bool GENERAL>
 __global__ void __launch_bounds__(256) projection_ut_kernel(
     uint32_t C, uint32_t N, const float* __restrict__ means, const float* __restrict__ quats,
     const float* __restrict__ scales, const float* __restrict__ opacities, const float* __restrict__ viewmats0,
@@ -239,18 +241,22 @@ __global__ void __launch_bounds__(256) projection_ut_kernel(
     cfg.fy = Ks[cid * 9 + 4];
     cfg.cx = Ks[cid * 9 + 2];
     cfg.cy = Ks[cid * 9 + 5];
-    const uint32_t n_radial = camera_model == GSX_FISHEYE ? 4u : 6u; // ProjectionUT3DGSFused.cu:103, 124
-    cfg.cam = load_camera_model(camera_model, radial != nullptr ? radial + cid * n_radial : nullptr,
-                                tangential != nullptr ? tangential + cid * 2 : nullptr,
-                                thin_prism != nullptr ? thin_prism + cid * 4 : nullptr, cfg.fx, cfg.fy, cfg.cx, cfg.cy,
-                                cfg.W, cfg.H);
-    const CamPose cp = load_cam_pose(viewmats0 + cid * 16, viewmats1 != nullptr ? viewmats1 + cid * 16 : nullptr,
-                                     rs_type, cfg.W, cfg.H);
+    if (GENERAL) {
+        const uint32_t n_radial = camera_model == GSX_FISHEYE ? 4u : 6u; // ProjectionUT3DGSFused.cu:103, 124
+        cfg.cam = load_camera_model(camera_model, radial != nullptr ? radial + cid * n_radial : nullptr,
+                                    tangential != nullptr ? tangential + cid * 2 : nullptr,
+                                    thin_prism != nullptr ? thin_prism + cid * 4 : nullptr, cfg.fx, cfg.fy, cfg.cx,
+                                    cfg.cy, cfg.W, cfg.H);
+    }
+    const CamPose cp = GENERAL ? load_cam_pose(viewmats0 + cid * 16,
+                                               viewmats1 != nullptr ? viewmats1 + cid * 16 : nullptr, rs_type, cfg.W,
+                                               cfg.H)
+                               : load_cam_pose(viewmats0 + cid * 16);
     ProjOut o;
     quat qc;
     vec3 tc;
     shutter_pose(cp, 0.5f, &qc, &tc);
-    const bool ok = project_ut<true>(cfg, cp, qc, tc, ld3(means, gid), ld4q(quats, gid), ld3(scales, gid), opacities != nullptr,
+    const bool ok = project_ut<GENERAL>(cfg, cp, qc, tc, ld3(means, gid), ld4q(quats, gid), ld3(scales, gid), opacities != nullptr,
                                opacities != nullptr ? opacities[gid] : 0.f, &o);
     int2* r2 = reinterpret_cast<int2*>(radii);
     if (!ok) {
@@ -925,10 +931,14 @@ extern "C" int gsx_projection_ut_3dgs_fused(
     set_ut_constants(cfg, ut);
     cfg.fx = cfg.fy = cfg.cx = cfg.cy = 0.f;
     memset(&cfg.cam, 0, sizeof(cfg.cam));
-    hipLaunchKernelGGL(projection_ut_kernel, dim3(cdiv((uint64_t)C * N, 256)), dim3(256), 0, (hipStream_t)stream, C,
-                       N, means, quats, scales, opacities, viewmats0, viewmats1, rs_type, Ks, camera_model,
-                       radial_coeffs, tangential_coeffs, thin_prism_coeffs, cfg, radii, means2d, depths, conics,
-                       compensations);
+    // the trainer's camera (rasterizer.cpp:33-35, rasterizer_autograd.cpp:59-60) takes the instance without the
+    // other models' branches: same arithmetic, same results
+    const bool plain = camera_model == GSX_PINHOLE && !radial_coeffs && !tangential_coeffs && !thin_prism_coeffs &&
+                       viewmats1 == nullptr && rs_type == GSX_GLOBAL;
+    hipLaunchKernelGGL(plain ? projection_ut_kernel<false> : projection_ut_kernel<true>,
+                       dim3(cdiv((uint64_t)C * N, 256)), dim3(256), 0, (hipStream_t)stream, C, N, means, quats, scales,
+                       opacities, viewmats0, viewmats1, rs_type, Ks, camera_model, radial_coeffs, tangential_coeffs,
+                       thin_prism_coeffs, cfg, radii, means2d, depths, conics, compensations);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

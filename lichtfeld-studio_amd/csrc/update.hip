@@ -30,6 +30,7 @@ struct UpdateArgs {
     float reg_scaling, reg_opacity;
     uint32_t* hold;             // nullable: [0] != 0 -> change nothing and count the call in [1]
     const float* step_scalars;  // nullable: device [3] = bc1_rcp, bc2_sqrt_rcp, skip_shN (0 / 1), read at run time
+    uint64_t* hold_report;      // nullable, pinned host memory: receives hold[1] << 32 | hold[0]
 };
 
 // new first / second moment of one element (the first two lines of adam_one)
@@ -68,8 +69,12 @@ __global__ void __launch_bounds__(256) backward_update_kernel(const UpdateArgs a
     if (a.hold != nullptr && a.hold[0] != 0u) {
         // the step's render is not valid (its tile lists did not fit): parameters and moments stay as they are; the
         // accumulator rows are cleared all the same
-        if (e == 0)
-            atomicAdd(&a.hold[1], 1u);
+        if (e == 0) {
+            const uint32_t held = atomicAdd(&a.hold[1], 1u) + 1u;
+            if (a.hold_report != nullptr)
+                __hip_atomic_store(a.hold_report, ((uint64_t)held << 32) | a.hold[0], __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_SYSTEM);
+        }
         if (e < a.N) {
             float4* row = reinterpret_cast<float4*>(a.acc + (size_t)e * 16);
             const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -77,6 +82,8 @@ __global__ void __launch_bounds__(256) backward_update_kernel(const UpdateArgs a
         }
         return;
     }
+    if (e == 0 && a.hold != nullptr && a.hold_report != nullptr)
+        __hip_atomic_store(a.hold_report, (uint64_t)a.hold[1] << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     float4* wave_lds = lds + (LDS16 ? wave * 64 * kGradF4 : 0);
     const bool in = e < a.N;
@@ -292,7 +299,17 @@ extern "C" int gsx_backward_update_fused(const gsx_update_args* args, void* stre
     a.bc1_rcp = args->bias_correction1_rcp, a.bc2_sqrt_rcp = args->bias_correction2_sqrt_rcp;
     a.skip_shN = args->skip_shN;
     a.reg_scaling = args->reg_scaling, a.reg_opacity = args->reg_opacity;
-    a.hold = args->hold, a.step_scalars = args->step_scalars;
+    a.hold = args->hold, a.step_scalars = args->step_scalars, a.hold_report = args->hold_report;
+    if (a.hold_report != nullptr) {
+        hipPointerAttribute_t attr;
+        const bool known = hipPointerGetAttributes(&attr, a.hold_report) == hipSuccess;
+        if (!known)
+            (void)hipGetLastError();
+        GSX_REQUIRE(known && attr.type == hipMemoryTypeHost && attr.devicePointer != nullptr, GSX_ERR_INVALID_ARGUMENT,
+                    "backward_update_fused: hold_report must be pinned host memory (hipHostMalloc)");
+        GSX_REQUIRE(a.hold != nullptr, GSX_ERR_INVALID_ARGUMENT, "backward_update_fused: hold_report without hold");
+        a.hold_report = (uint64_t*)attr.devicePointer;
+    }
     const bool lds16 = a.K == 16 && ((((uintptr_t)a.shs) | ((uintptr_t)a.m_shs) | ((uintptr_t)a.v_shs)) & 15u) == 0;
     const dim3 grid(cdiv(a.N, 256)), block(256);
     if (lds16)

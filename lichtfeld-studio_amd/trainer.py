@@ -41,6 +41,9 @@ class TrainStep:
         self.device_count = bool(device_count and fused_update)
         self.lists_ws, self._lists_dims, self._lists_active = None, None, False
         self.steps_held = 0
+        # the fused update stores (calls held back << 32 | sticky error bits of the tile lists) here after every launch
+        self.hold_report = torch.zeros(1, dtype=torch.int64, pin_memory=True)
+        self._hold_slot = ctypes.c_uint64.from_address(self.hold_report.data_ptr())
         f = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(self.dev)
         self.N = scene.means.shape[0]
         self.K = 1 + scene.shN.shape[1]
@@ -151,12 +154,29 @@ class TrainStep:
         w = self.lists_ws[self._lists_error_at:self._lists_error_at + 8].cpu().numpy().view(np.uint32)
         return int(w[0]), int(w[1])
 
+    def clear_lists_error(self):
+        """after a raised look-back error: zero the sticky error word and the held-call counter"""
+        torch.cuda.synchronize(self.dev)
+        _, held = self.lists_error()
+        self.steps_held += held
+        self.step_count -= held
+        self.iteration -= held
+        self.lists_ws[self._lists_error_at:self._lists_error_at + 8].zero_()
+        torch.cuda.synchronize(self.dev)
+        self._hold_slot.value = 0
+
     def _check_capacity(self):
         """Start of a step with the count on the device: the last count that reached the host decides whether the
         buffers grow.  More pairs than the buffers held means that step (and every step queued behind it) rendered
         nothing and was held back from the optimiser: they are counted back out of the iteration counters."""
         if not self._lists_active:
             return
+        if self._hold_slot.value & 2:
+            # a chained pass gave up waiting for its predecessor: the lists of that step (and the renders since) are
+            # invalid and the optimiser has been held since - not a condition to train through
+            bits, held = self.lists_error()
+            raise L.GsxError(-4, f"tile lists: a look-back's bounded wait ran out (error bits {bits}); {held} "
+                                 "optimiser call(s) were held back.  clear_lists_error() re-arms the lists")
         n = self._n_slot.value
         if n <= int(self.cap * 0.9):
             return
@@ -543,7 +563,8 @@ class TrainStep:
                 # weight / element count in float32, as the separate regularisation kernels form it
                 float(np.float32(self.scale_reg) / np.float32(3 * self.N)) if self.scale_reg > 0.0 else 0.0,
                 float(np.float32(self.opacity_reg) / np.float32(self.N)) if self.opacity_reg > 0.0 else 0.0,
-                self._lists_error if self._lists_active else None, None)
+                self._lists_error if self._lists_active else None, None,
+                self.hold_report.data_ptr() if self._lists_active else None)
             self._run("backward_update_fused", self.lib.gsx_backward_update_fused, ctypes.byref(a), self._stream())
             return
         names = ["means", "shs", "scaling", "rotation", "opacity"]
