@@ -12,9 +12,16 @@
 //  3. tile_table_kernel      +1 / -1 at every rectangle's corners in a (Th + 1) x (Tw + 1) grid and a 2-D prefix
 //                            sum over it give every tile's list length, hence tile_offsets, the pair count, and the
 //                            digit histograms of the pair sort - before a single pair exists;
-//  4. tile_emit_chained_kernel  writes (16-bit tile index, id) pairs in depth order; a workgroup's position in the
-//                            output comes from a chained look-back over the workgroups' pair counts;
-//  5. two chained radix passes over the tile bits (the second one writes flatten_ids only).
+//  4. super_emit_kernel      The tile grid is cut into at most 256 SUPER-TILES of 4 x 4 ... 16 x 16 tiles.  Every
+//                            Gaussian, in depth order, leaves one entry (super-tile << 32 | rectangle, id) per
+//                            super-tile its rectangle meets - 1.2 - 2 entries a Gaussian, against 7 - 30 (tile,
+//                            Gaussian) pairs; a workgroup's position in the output comes from a chained look-back over
+//                            the workgroups' entry counts;
+//  5. one chained radix pass over the super-tile byte groups the entries by super-tile, depth order kept;
+//  6. tile_gather_kernel     one wave per tile walks its super-tile's entries (staged through LDS, shared by the 16
+//                            waves of the workgroup) and writes the ids whose rectangle covers the tile, in order, to
+//                            the tile's place in flatten_ids: every list is written once, front to back, and no
+//                            (tile, id) pair is ever sorted.
 //
 // Everything downstream sizes its work by `capacity` and reads the actual count from device memory.  If the count
 // exceeds the capacity, every tile's list is left EMPTY (tile_offsets all zero), bit 0 of the error word is set and
@@ -38,6 +45,7 @@ static constexpr uint32_t kKeysPerBlock = 4 * kKeysThreads; // 4 consecutive Gau
 static constexpr uint32_t kEmitThreads = 1024;  // tile_emit_chained_kernel: likewise
 static constexpr uint32_t kTableBlocks = 32;    // tile_table_kernel: workgroups that share the corner counting
 static constexpr uint32_t kMaxLdsCells = 36 * 1024; // corner grids up to this many cells are counted in LDS
+static constexpr uint32_t kSliceEntries = 2048; // tile_gather_kernel: entries of one super-tile a workgroup takes
 static constexpr uint32_t kHistReplicas = 4;    // copies of the depth-byte histograms (fewer additions per address)
 
 // adds 1 to hist[digit] for every live lane; one LDS atomic per wave when all its live lanes share the digit
@@ -62,7 +70,8 @@ __global__ void __launch_bounds__(kKeysThreads) depth_keys_kernel(
     int64_t* __restrict__ keys, int32_t* __restrict__ vals, uint32_t* __restrict__ rects,
     uint32_t* __restrict__ status /*[blocks]*/, int64_t* __restrict__ counts, uint32_t* __restrict__ error,
     uint32_t* __restrict__ clear_status, uint32_t clear_rows, uint32_t* __restrict__ clear_emit_status,
-    uint32_t clear_emit_words, uint32_t* __restrict__ depth_hist) {
+    uint32_t clear_emit_words, uint32_t* __restrict__ clear_super_hist, uint32_t* __restrict__ clear_gather_status,
+    uint32_t gather_rows_max, uint32_t n_super, uint32_t* __restrict__ depth_hist) {
     constexpr uint32_t kWaves = kKeysThreads / 64u;
     __shared__ uint32_t wave_total[kWaves];
     __shared__ uint32_t base_s;
@@ -75,6 +84,14 @@ __global__ void __launch_bounds__(kKeysThreads) depth_keys_kernel(
         clear_status[wd] = 0u;
     for (uint32_t wd = blockIdx.x * kKeysThreads + t; wd < clear_emit_words; wd += gridDim.x * kKeysThreads)
         clear_emit_status[wd] = 0u;
+    if (blockIdx.x == 0) // the entry counts per super-tile of the call before (kHistReplicas x 256 words)
+        clear_super_hist[t] = 0u;
+    {
+        // the status rows the gather of the call before used: its entry count is still in counts[3]
+        const uint32_t rows = min(gather_rows_max, (uint32_t)counts[3] / kSliceEntries + n_super);
+        for (uint32_t wd = blockIdx.x * kKeysThreads + t; wd < rows * 256u; wd += gridDim.x * kKeysThreads)
+            clear_gather_status[wd] = 0u;
+    }
     uint32_t lo[4], hi[4];
     uint32_t mine = 0;
     // the lane's four Gaussians: every load leaves before the first result is used (indices clamped, results
@@ -166,17 +183,15 @@ __global__ void __launch_bounds__(kKeysThreads) depth_keys_kernel(
 // it in `replicas`; the last one to finish adds the replicas up and turns the corner counts into per-tile counts
 // (2-D inclusive prefix sum), tile_offsets [n_tiles + 1] (exclusive prefix in row-major tile order, the count in the
 // last entry), counts[0] = the count the launches behind this one use (0 when it exceeds the capacity), counts[1] =
-// the true count, and the two digit histograms of the pair sort.
+// the true count.
 template <bool in_lds>
 __global__ void __launch_bounds__(1024) tile_table_kernel(
     const uint32_t* __restrict__ rects, uint32_t tile_width, uint32_t tile_height,
     int32_t* __restrict__ replicas /*[kTableBlocks][cells], or [cells] zeroed when !in_lds*/,
-    uint32_t* __restrict__ done_counter, int64_t capacity,
-    uint32_t bits0, uint32_t bits1, int32_t* __restrict__ tile_offsets, uint32_t* __restrict__ pair_hist /*[2][256]*/,
+    uint32_t* __restrict__ done_counter, int64_t capacity, int32_t* __restrict__ tile_offsets,
     int64_t* __restrict__ counts, int64_t* host_slot, uint32_t* __restrict__ error) {
     extern __shared__ int32_t lds_grid[];
     __shared__ unsigned long long wave_tot[16];
-    __shared__ uint32_t h0[256], h1[256];
     __shared__ uint32_t last_s;
     const uint32_t t = threadIdx.x, lane = t & 63u, wv = t >> 6;
     const uint32_t gw = tile_width + 1u, gh = tile_height + 1u, n_tiles = tile_width * tile_height;
@@ -282,10 +297,6 @@ __global__ void __launch_bounds__(1024) tile_table_kernel(
     }
     __syncthreads();
     auto tile_count = [&](uint32_t i) { return (uint32_t)GSX_GRID((i / tile_width) * gw + i % tile_width); };
-    if (t < 256) {
-        h0[t] = 0;
-        h1[t] = 0;
-    }
     // exclusive prefix over the tiles: a contiguous chunk per lane
     const uint32_t chunk = (n_tiles + 1023u) / 1024u;
     const uint32_t first = min(t * chunk, n_tiles), last = min(first + chunk, n_tiles);
@@ -309,25 +320,15 @@ __global__ void __launch_bounds__(1024) tile_table_kernel(
         total += wave_tot[k];
     }
     const bool fits = total <= (unsigned long long)capacity && total <= (unsigned long long)kLbValueMask;
-    const uint32_t mask0 = (1u << bits0) - 1u, mask1 = bits1 ? (1u << bits1) - 1u : 0u;
     unsigned long long run = before + incl - mine;
     for (uint32_t i = first; i < last; ++i) {
-        const uint32_t c = tile_count(i);
         tile_offsets[i] = fits ? (int32_t)run : 0;
-        run += c;
-        if (fits && c) {
-            atomicAdd(&h0[i & mask0], c);
-            atomicAdd(&h1[(i >> bits0) & mask1], c);
-        }
+        run += tile_count(i);
     }
     __syncthreads();
     if (!in_lds) // the shared grid in global memory is left zeroed for the next call
         for (uint32_t i = t; i < cells; i += 1024u)
             GSX_GRID(i) = 0;
-    if (t < 256) {
-        pair_hist[t] = h0[t];
-        pair_hist[256u + t] = h1[t];
-    }
     if (t == 0) {
         tile_offsets[n_tiles] = fits ? (int32_t)total : 0;
         counts[0] = fits ? (int64_t)total : 0;
@@ -340,20 +341,22 @@ __global__ void __launch_bounds__(1024) tile_table_kernel(
 }
 #undef GSX_GRID
 
-// (16-bit tile index, id) pairs in depth order from the sorted keys.  Workgroup p covers sorted positions
-// [1024 p, 1024 p + 1024); its first output position is the pair count of all positions in front of it, obtained by a
-// chained look-back over the workgroups' counts.  Inside the workgroup a wave flattens the runs of its 64 positions so
-// that consecutive lanes write consecutive pairs.
-__global__ void __launch_bounds__(kEmitThreads) tile_emit_chained_kernel(
-    const int64_t* __restrict__ sorted_keys, const int32_t* __restrict__ order, uint32_t tile_width,
-    const int64_t* __restrict__ counts, uint32_t* __restrict__ status, uint16_t* __restrict__ tile_keys,
-    int32_t* __restrict__ ids, uint32_t* __restrict__ clear_status, uint32_t clear_rows,
-    uint32_t* __restrict__ clear_key_status, uint32_t clear_key_words, uint32_t* __restrict__ clear_depth_hist,
-    uint32_t* __restrict__ error) {
+// Entries (super-tile << 32 | rectangle, id) in depth order from the sorted keys: one per super-tile a Gaussian's
+// rectangle meets.  Workgroup p covers sorted positions [1024 p, 1024 p + 1024); its first output position is the
+// entry count of all positions in front of it, obtained by a chained look-back over the workgroups' counts.  Inside
+// the workgroup a wave flattens the runs of its 64 positions so that consecutive lanes write consecutive entries.
+// The launch also counts the entries per super-tile (the digit totals of the pass behind it).
+__global__ void __launch_bounds__(kEmitThreads) super_emit_kernel(
+    const int64_t* __restrict__ sorted_keys, const int32_t* __restrict__ order, uint32_t sx_shift, uint32_t sy_shift,
+    uint32_t super_width, int64_t* __restrict__ counts, uint32_t* __restrict__ status,
+    int64_t* __restrict__ entry_keys, int32_t* __restrict__ entry_ids, uint32_t* __restrict__ super_hist,
+    uint32_t* __restrict__ clear_status, uint32_t clear_rows, uint32_t* __restrict__ clear_key_status,
+    uint32_t clear_key_words, uint32_t* __restrict__ clear_depth_hist, uint32_t* __restrict__ error) {
     constexpr uint32_t kWaves = kEmitThreads / 64u;
-    __shared__ uint32_t s_incl[kWaves][64], s_xy[kWaves][64], s_w[kWaves][64], s_idx[kWaves][64];
+    __shared__ uint32_t s_incl[kWaves][64], s_hi[kWaves][64], s_idx[kWaves][64];
     __shared__ uint32_t wave_total[kWaves];
     __shared__ uint32_t base_s;
+    __shared__ uint32_t sh[256];
     const uint32_t t = threadIdx.x, lane = t & 63u, wv = t >> 6;
     const uint32_t place = blockIdx.x;
     for (uint32_t wd = place * kEmitThreads + t; wd < clear_rows * 256u; wd += gridDim.x * kEmitThreads)
@@ -365,15 +368,20 @@ __global__ void __launch_bounds__(kEmitThreads) tile_emit_chained_kernel(
         clear_depth_hist[r * 1024u + t] = 0u;
     const uint32_t limit = (uint32_t)counts[0]; // 0 when the pairs do not fit: nothing is written
     const uint32_t n = (uint32_t)counts[2];     // Gaussians that touch a tile
-    if (place * kEmitThreads >= n || limit == 0)
+    if (place * kEmitThreads >= n || limit == 0) {
+        if (place == 0 && t == 0)
+            counts[3] = 0; // no entries (every later workgroup returns as well)
         return; // nobody behind this workgroup needs its (empty) contribution
+    }
+    if (t < 256)
+        sh[t] = 0u;
     const uint32_t i = place * kEmitThreads + t;
-    uint32_t x0 = 0, y0 = 0, w = 0, cnt = 0, idx = 0;
+    uint32_t hi = 0, cnt = 0, idx = 0;
     if (i < n) {
-        const uint32_t hi = (uint32_t)((uint64_t)sorted_keys[i] >> 32);
-        x0 = hi & 255u, y0 = (hi >> 8) & 255u;
-        w = ((hi >> 16) & 255u) - x0;
-        cnt = ((hi >> 24) - y0) * w;
+        hi = (uint32_t)((uint64_t)sorted_keys[i] >> 32);
+        const uint32_t X0 = (hi & 255u) >> sx_shift, X1 = ((((hi >> 16) & 255u) - 1u) >> sx_shift) + 1u;
+        const uint32_t Y0 = ((hi >> 8) & 255u) >> sy_shift, Y1 = (((hi >> 24) - 1u) >> sy_shift) + 1u;
+        cnt = (X1 - X0) * (Y1 - Y0);
         idx = (uint32_t)order[i];
     }
     uint32_t incl = cnt;
@@ -384,8 +392,7 @@ __global__ void __launch_bounds__(kEmitThreads) tile_emit_chained_kernel(
             incl += up;
     }
     s_incl[wv][lane] = incl;
-    s_xy[wv][lane] = x0 | (y0 << 16);
-    s_w[wv][lane] = w;
+    s_hi[wv][lane] = hi;
     s_idx[wv][lane] = idx;
     if (lane == 63)
         wave_total[wv] = incl;
@@ -401,6 +408,8 @@ __global__ void __launch_bounds__(kEmitThreads) tile_emit_chained_kernel(
         if (lane == 0) {
             if (place != 0)
                 lb_publish(status + place, kLbPrefix, before + block_total);
+            if ((place + 1u) * kEmitThreads >= n)
+                counts[3] = (int64_t)(before + block_total); // entries there are (<= pairs: they fit)
             base_s = before;
         }
     }
@@ -411,24 +420,204 @@ __global__ void __launch_bounds__(kEmitThreads) tile_emit_chained_kernel(
         wave_base += k < wv ? wave_total[k] : 0u;
     const uint32_t total = wave_total[wv];
     for (uint32_t k = lane; k < total; k += 64u) {
-        uint32_t lo = 0, hi = 63; // smallest l with incl[l] > k
+        uint32_t lo = 0, up = 63; // smallest l with incl[l] > k
 #pragma unroll
         for (uint32_t step = 0; step < 6; ++step) {
-            const uint32_t mid = (lo + hi) >> 1;
+            const uint32_t mid = (lo + up) >> 1;
             if (s_incl[wv][mid] > k)
-                hi = mid;
+                up = mid;
             else
                 lo = mid + 1;
         }
         const uint32_t l = lo;
         const uint32_t local = k - (l ? s_incl[wv][l - 1] : 0u);
-        const uint32_t gw = s_w[wv][l], xy = s_xy[wv][l];
+        const uint32_t h = s_hi[wv][l];
+        const uint32_t X0 = (h & 255u) >> sx_shift, X1 = ((((h >> 16) & 255u) - 1u) >> sx_shift) + 1u;
+        const uint32_t Y0 = ((h >> 8) & 255u) >> sy_shift;
+        const uint32_t gw = X1 - X0;
         const uint32_t row = local / gw;
-        const uint32_t tile_id = ((xy >> 16) + row) * tile_width + ((xy & 0xffffu) + (local - row * gw));
+        const uint32_t super_id = (Y0 + row) * super_width + X0 + (local - row * gw);
         const uint32_t pos = wave_base + k;
         if (pos < limit) {
-            tile_keys[pos] = (uint16_t)tile_id;
-            ids[pos] = (int32_t)s_idx[wv][l];
+            entry_keys[pos] = (int64_t)(((uint64_t)super_id << 32) | h);
+            entry_ids[pos] = (int32_t)s_idx[wv][l];
+            atomicAdd(&sh[super_id & 255u], 1u);
+        }
+    }
+    __syncthreads();
+    if (t < 256 && sh[t] != 0u)
+        atomicAdd(&super_hist[(place % kHistReplicas) * 256u + t], sh[t]);
+}
+
+// flatten_ids from the entries grouped by super-tile.  A workgroup takes one SLICE: up to kSliceEntries consecutive
+// entries of one super-tile.  Staging a slice in LDS turns every entry's rectangle into a bit mask over the tiles of
+// the super-tile (bit l = tile l, row-major inside the super-tile; WORDS x 32 bits); whether an entry belongs to a
+// tile is then one bit test, and 64 entries are tested with two vector instructions.  The 16 waves share the
+// super-tile's tiles; for a tile a wave walks the slice 64 entries at a time - once to count the entries of the tile,
+// once to write them.  Between the two, the slice's per-tile counts are chained to those of the slices in front of
+// it within the super-tile by a look-back over one status row per slice (a column per tile; the first slice of a
+// super-tile publishes a complete prefix, which ends the walk): the k-th entry of tile T in this slice goes to
+// flatten_ids[tile_offsets[T] + entries of T in earlier slices + k].  Every list is written front to back in depth
+// order; no (tile, id) pair is formed or sorted.
+template <uint32_t WORDS>
+__global__ void __launch_bounds__(1024) tile_gather_kernel(
+    const int64_t* __restrict__ entry_keys, const int32_t* __restrict__ entry_ids,
+    const uint32_t* __restrict__ super_hist, const int64_t* __restrict__ counts,
+    const int32_t* __restrict__ tile_offsets, uint32_t tile_width, uint32_t tile_height, uint32_t sx_shift,
+    uint32_t sy_shift, uint32_t super_width, uint32_t n_super, uint32_t* __restrict__ status,
+    uint32_t* __restrict__ error, int32_t* __restrict__ flatten_ids) {
+    constexpr uint32_t kTilesPerWave = WORDS * 2u;       // 32 WORDS tiles over 16 waves
+    __shared__ uint32_t s_mask[WORDS][kSliceEntries];
+    __shared__ int32_t s_id[kSliceEntries];
+    __shared__ uint32_t seg_start[256], seg_len[256], slice_start[256];
+    __shared__ uint32_t wave_a[4], wave_b[4];
+    __shared__ uint32_t cnt[WORDS * 32u], base[WORDS * 32u];
+    const uint32_t t = threadIdx.x, lane = t & 63u, wv = t >> 6;
+    const uint32_t limit = (uint32_t)counts[0];
+    const uint32_t place = blockIdx.x;
+    // beyond the last slice there can be (entries / slice + one partial slice per super-tile): nothing to do
+    if (limit == 0 || place >= (uint32_t)counts[3] / kSliceEntries + n_super)
+        return;
+    // entries and slices in front of every super-tile (exclusive prefix sums over at most 256 counts)
+    uint32_t len = 0, nsl = 0, in_len = 0, in_nsl = 0;
+    if (t < 256) {
+        if (t < n_super)
+#pragma unroll
+            for (uint32_t r = 0; r < kHistReplicas; ++r)
+                len += super_hist[r * 256u + t];
+        nsl = (len + kSliceEntries - 1u) / kSliceEntries;
+        in_len = len, in_nsl = nsl;
+#pragma unroll
+        for (uint32_t off = 1; off < 64; off <<= 1) {
+            const uint32_t ua = (uint32_t)__shfl_up((int)in_len, off, 64), ub = (uint32_t)__shfl_up((int)in_nsl, off, 64);
+            if (lane >= off) {
+                in_len += ua;
+                in_nsl += ub;
+            }
+        }
+        if (lane == 63) {
+            wave_a[wv] = in_len;
+            wave_b[wv] = in_nsl;
+        }
+    }
+    __syncthreads();
+    if (t < 256) {
+        uint32_t ba = 0, bb = 0;
+#pragma unroll
+        for (uint32_t k = 0; k < 4; ++k) {
+            ba += k < wv ? wave_a[k] : 0u;
+            bb += k < wv ? wave_b[k] : 0u;
+        }
+        seg_start[t] = ba + in_len - len;
+        seg_len[t] = len;
+        slice_start[t] = bb + in_nsl - nsl;
+    }
+    __syncthreads();
+    if (place >= wave_b[0] + wave_b[1] + wave_b[2] + wave_b[3])
+        return;
+    // the super-tile of this slice: the last one whose first slice is not behind `place`
+    uint32_t lo = 0, hi = 255;
+#pragma unroll
+    for (uint32_t step = 0; step < 8; ++step) {
+        const uint32_t mid = (lo + hi + 1u) >> 1;
+        if (slice_start[mid] <= place)
+            lo = mid;
+        else
+            hi = mid - 1u;
+    }
+    const uint32_t sup = lo, k_slice = place - slice_start[sup];
+    const uint32_t a = seg_start[sup] + k_slice * kSliceEntries;
+    const uint32_t n_here = min(kSliceEntries, seg_start[sup] + seg_len[sup] - a);
+    const uint32_t tx0 = (sup % super_width) << sx_shift, ty0 = (sup / super_width) << sy_shift;
+    const uint32_t sx = 1u << sx_shift, sy = 1u << sy_shift;
+    const uint32_t rows_per_word = 32u >> sx_shift;
+#pragma unroll
+    for (uint32_t k = 0; k < kSliceEntries / 1024u; ++k) {
+        const uint32_t j = k * 1024u + t;
+        uint32_t m[WORDS];
+#pragma unroll
+        for (uint32_t w = 0; w < WORDS; ++w)
+            m[w] = 0u;
+        int32_t id = 0;
+        if (j < n_here) {
+            const uint32_t r = (uint32_t)(uint64_t)entry_keys[a + j];
+            id = entry_ids[a + j];
+            // the rectangle inside this super-tile, in its own tile coordinates
+            const uint32_t x0 = max(r & 255u, tx0) - tx0, x1 = min((r >> 16) & 255u, tx0 + sx) - tx0;
+            const uint32_t y0 = max((r >> 8) & 255u, ty0) - ty0, y1 = min(r >> 24, ty0 + sy) - ty0;
+            const uint32_t row_bits = (1u << x1) - (1u << x0);
+#pragma unroll
+            for (uint32_t w = 0; w < WORDS; ++w)
+                for (uint32_t q = 0; q < rows_per_word; ++q) {
+                    const uint32_t row = w * rows_per_word + q;
+                    if (row >= y0 && row < y1)
+                        m[w] |= row_bits << (q << sx_shift);
+                }
+        }
+#pragma unroll
+        for (uint32_t w = 0; w < WORDS; ++w)
+            s_mask[w][j] = m[w]; // zero beyond the slice's end: no entry
+        s_id[j] = id;
+    }
+    const uint64_t below = (1ull << lane) - 1ull;
+    __syncthreads();
+    // tiles wv, wv + 16, ... of the super-tile: tile wv + 16 i is bit (wv + 16 (i & 1)) of word i / 2
+    uint32_t c[kTilesPerWave];
+#pragma unroll
+    for (uint32_t i = 0; i < kTilesPerWave; ++i)
+        c[i] = 0u;
+    const uint32_t bit0 = 1u << wv, bit1 = 1u << (wv + 16u);
+    const uint32_t groups = (n_here + 63u) / 64u;
+    for (uint32_t g = 0; g < groups; ++g) {
+        uint32_t m[WORDS];
+#pragma unroll
+        for (uint32_t w = 0; w < WORDS; ++w)
+            m[w] = s_mask[w][g * 64u + lane];
+#pragma unroll
+        for (uint32_t i = 0; i < kTilesPerWave; ++i)
+            c[i] += (uint32_t)__popcll(__ballot((m[i >> 1] & ((i & 1u) ? bit1 : bit0)) != 0u));
+    }
+    if (lane == 0)
+#pragma unroll
+        for (uint32_t i = 0; i < kTilesPerWave; ++i)
+            cnt[wv + 16u * i] = c[i];
+    __syncthreads();
+    if (t < WORDS * 32u) {
+        const uint32_t mine = cnt[t];
+        uint32_t before = 0;
+        const uint32_t tx = tx0 + (t & (sx - 1u)), ty = ty0 + (t >> sx_shift);
+        const bool on_grid = (t >> sx_shift) < sy && tx < tile_width && ty < tile_height;
+        const uint32_t offset = on_grid ? (uint32_t)tile_offsets[ty * tile_width + tx] : 0u;
+        if (k_slice == 0) {
+            lb_publish(status + (size_t)place * 256u + t, kLbPrefix, mine);
+        } else {
+            lb_publish(status + (size_t)place * 256u + t, kLbAggregate, mine);
+            before = lb_exclusive(status, place, 256u, t, error);
+            lb_publish(status + (size_t)place * 256u + t, kLbPrefix, before + mine);
+        }
+        base[t] = before + offset;
+    }
+    __syncthreads();
+    uint32_t at[kTilesPerWave];
+#pragma unroll
+    for (uint32_t i = 0; i < kTilesPerWave; ++i)
+        at[i] = base[wv + 16u * i];
+    for (uint32_t g = 0; g < groups; ++g) {
+        uint32_t m[WORDS];
+#pragma unroll
+        for (uint32_t w = 0; w < WORDS; ++w)
+            m[w] = s_mask[w][g * 64u + lane];
+        const int32_t id = s_id[g * 64u + lane];
+#pragma unroll
+        for (uint32_t i = 0; i < kTilesPerWave; ++i) {
+            const bool in = (m[i >> 1] & ((i & 1u) ? bit1 : bit0)) != 0u;
+            const uint64_t mask = __ballot(in);
+            if (in) {
+                const uint32_t pos = at[i] + (uint32_t)__popcll(mask & below);
+                if (pos < limit)
+                    flatten_ids[pos] = id;
+            }
+            at[i] += (uint32_t)__popcll(mask);
         }
     }
 }
@@ -446,13 +635,15 @@ using namespace gsx;
 namespace {
 struct ListsLayout {
     // zeroed by gsx_tile_lists_init and left zero by every call: the head of the workspace
-    size_t depth_hist, counts, error, done_counter, kstatus, shared_grid, head_end;
+    size_t depth_hist, super_hist, counts, error, done_counter, kstatus, shared_grid, head_end;
     size_t keys0, keys1, vals0, vals1, rects; // depth sort: i64 [N] x 2, i32 [N] x 2; u32 [N]
-    size_t replicas, pair_hist;
-    size_t dstatus0, dstatus1, estatus, pstatus0, pstatus1;
-    size_t tkeys0, tkeys1, ids0, ids1; // pairs: u16 [capacity] x 2, i32 [capacity] x 2
+    size_t replicas;
+    size_t dstatus0, dstatus1, estatus, pstatus, gstatus;
+    uint32_t grows; // status rows of the gather: one per slice there can be
+    size_t ekeys0, ekeys1, eids0, eids1; // entries: i64 [capacity] x 2, i32 [capacity] x 2
     size_t total;
     uint32_t kblocks, drows, prows, ewords, cells, table_blocks;
+    uint32_t sx_shift, sy_shift, super_width, n_super, parts; // super-tiles of (1 << sx_shift) x (1 << sy_shift) tiles
     bool grid_in_lds;
 };
 ListsLayout lists_layout(uint32_t N, int64_t capacity, uint32_t tw, uint32_t th) {
@@ -470,15 +661,25 @@ ListsLayout lists_layout(uint32_t N, int64_t capacity, uint32_t tw, uint32_t th)
     L.cells = (tw + 1) * (th + 1);
     L.grid_in_lds = L.cells <= kMaxLdsCells;
     L.table_blocks = std::min(kTableBlocks, std::max(1u, N / (128u * 1024u)));
+    // the smallest super-tiles of which the grid holds at most 256 (one byte of the entry keys names them)
+    static const uint32_t shapes[5][2] = {{2, 2}, {3, 2}, {3, 3}, {4, 3}, {4, 4}};
+    for (const auto& sh : shapes) {
+        L.sx_shift = sh[0], L.sy_shift = sh[1];
+        L.super_width = cdiv(tw, 1u << L.sx_shift);
+        L.n_super = L.super_width * cdiv(th, 1u << L.sy_shift);
+        if (L.n_super <= 256u)
+            break;
+    }
+    L.parts = (1u << (L.sx_shift + L.sy_shift)) / 16u;
     L.depth_hist = take((size_t)kHistReplicas * 4 * 256 * 4);
-    L.counts = take(3 * 8);
+    L.super_hist = take((size_t)kHistReplicas * 256 * 4);
+    L.counts = take(4 * 8);
     L.error = take(2 * 4);
     L.done_counter = take(4);
     L.kstatus = take((size_t)L.kblocks * 4);
     L.shared_grid = take(L.grid_in_lds ? 0 : (size_t)L.cells * 4);
     L.head_end = o;
     L.replicas = take(L.grid_in_lds ? (size_t)kTableBlocks * L.cells * 4 : 0);
-    L.pair_hist = take(2 * 256 * 4);
     L.keys0 = take((size_t)N * 8);
     L.keys1 = take((size_t)N * 8);
     L.vals0 = take((size_t)N * 4);
@@ -487,12 +688,15 @@ ListsLayout lists_layout(uint32_t N, int64_t capacity, uint32_t tw, uint32_t th)
     L.dstatus0 = take((size_t)L.drows * 1024);
     L.dstatus1 = take((size_t)L.drows * 1024);
     L.estatus = take((size_t)L.ewords * 4);
-    L.pstatus0 = take((size_t)L.prows * 1024);
-    L.pstatus1 = take((size_t)L.prows * 1024);
-    L.tkeys0 = take((size_t)capacity * 2);
-    L.tkeys1 = take((size_t)capacity * 2);
-    L.ids0 = take((size_t)capacity * 4);
-    L.ids1 = take((size_t)capacity * 4);
+    L.pstatus = take((size_t)L.prows * 1024);
+    L.grows = (uint32_t)cdiv((uint64_t)capacity, kSliceEntries) + L.n_super;
+    L.gstatus = take((size_t)L.grows * 1024);
+    // an entry stands for at least one (tile, Gaussian) pair: entries that exceed the pair capacity cannot occur
+    // once the pairs fit
+    L.ekeys0 = take((size_t)capacity * 8);
+    L.ekeys1 = take((size_t)capacity * 8);
+    L.eids0 = take((size_t)capacity * 4);
+    L.eids1 = take((size_t)capacity * 4);
     L.total = o;
     return L;
 }
@@ -548,6 +752,11 @@ extern "C" int gsx_tile_lists_init(uint32_t N, int64_t capacity, uint32_t tile_w
     hipLaunchKernelGGL(zero_words_kernel, dim3(cdiv(words, 256)), dim3(256), 0, (hipStream_t)stream, words,
                        (uint32_t*)workspace);
     GSX_LAUNCH_CHECK();
+    // the gather's status rows: a call clears the rows the call before it used, so all of them start out zero
+    const size_t gwords = (size_t)L.grows * 256;
+    hipLaunchKernelGGL(zero_words_kernel, dim3(cdiv(gwords, 256)), dim3(256), 0, (hipStream_t)stream, gwords,
+                       (uint32_t*)((char*)workspace + L.gstatus));
+    GSX_LAUNCH_CHECK();
     return GSX_OK;
 }
 
@@ -590,21 +799,17 @@ extern "C" int gsx_tile_lists(uint32_t N, const float* means2d, const int32_t* r
     int64_t* keys[2] = {(int64_t*)(ws + L.keys0), (int64_t*)(ws + L.keys1)};
     int32_t* vals[2] = {(int32_t*)(ws + L.vals0), (int32_t*)(ws + L.vals1)};
     uint32_t* dstatus[2] = {u32p(L.dstatus0), u32p(L.dstatus1)};
-    uint32_t* pstatus[2] = {u32p(L.pstatus0), u32p(L.pstatus1)};
     uint32_t* error = u32p(L.error);
     int64_t* counts = (int64_t*)(ws + L.counts);
     hipStream_t s = (hipStream_t)stream;
 
     hipLaunchKernelGGL(depth_keys_kernel, dim3(L.kblocks), dim3(kKeysThreads), 0, s, N, means2d, radii, depths,
                        (float)tile_size, tile_width, tile_height, keys[0], vals[0], u32p(L.rects), u32p(L.kstatus),
-                       counts, error, dstatus[0], L.drows, u32p(L.estatus), L.ewords, u32p(L.depth_hist));
+                       counts, error, dstatus[0], L.drows, u32p(L.estatus), L.ewords, u32p(L.super_hist),
+                       u32p(L.gstatus), L.grows, L.n_super, u32p(L.depth_hist));
     GSX_LAUNCH_CHECK();
     // The tile table needs the rectangles only, not their depth order: with a second stream it is formed while the
     // sort runs.
-    const uint32_t tile_bits = gsx_n_bits(tile_width * tile_height);
-    const uint32_t passes = tile_bits > 8 ? 2u : 1u;
-    const uint32_t bits0 = passes == 2 ? (tile_bits + 1) / 2 : (tile_bits ? tile_bits : 1u);
-    const uint32_t bits1 = passes == 2 ? tile_bits - bits0 : 0u;
     hipStream_t ts = side_stream != nullptr && side_stream != stream ? (hipStream_t)side_stream : s;
     SideEvents* ev = nullptr;
     if (ts != s) {
@@ -615,12 +820,12 @@ extern "C" int gsx_tile_lists(uint32_t N, const float* means2d, const int32_t* r
     }
     if (L.grid_in_lds)
         hipLaunchKernelGGL(tile_table_kernel<true>, dim3(L.table_blocks), dim3(1024), table_lds, ts, u32p(L.rects),
-                           tile_width, tile_height, (int32_t*)(ws + L.replicas), u32p(L.done_counter), capacity, bits0,
-                           bits1, tile_offsets, u32p(L.pair_hist), counts, slot, error);
+                           tile_width, tile_height, (int32_t*)(ws + L.replicas), u32p(L.done_counter), capacity,
+                           tile_offsets, counts, slot, error);
     else
         hipLaunchKernelGGL(tile_table_kernel<false>, dim3(L.table_blocks), dim3(1024), 0, ts, u32p(L.rects),
                            tile_width, tile_height, (int32_t*)(ws + L.shared_grid), u32p(L.done_counter), capacity,
-                           bits0, bits1, tile_offsets, u32p(L.pair_hist), counts, slot, error);
+                           tile_offsets, counts, slot, error);
     GSX_LAUNCH_CHECK();
     if (ts != s)
         GSX_HIP_CHECK(hipEventRecord(ev->table_done, ts));
@@ -636,28 +841,37 @@ extern "C" int gsx_tile_lists(uint32_t N, const float* means2d, const int32_t* r
     }
     if (ts != s)
         GSX_HIP_CHECK(hipStreamWaitEvent(s, ev->table_done, 0));
-    uint16_t* tkeys[2] = {(uint16_t*)(ws + L.tkeys0), (uint16_t*)(ws + L.tkeys1)};
-    int32_t* ids[2] = {(int32_t*)(ws + L.ids0), (int32_t*)(ws + L.ids1)};
-    hipLaunchKernelGGL(tile_emit_chained_kernel, dim3(L.ewords), dim3(kEmitThreads), 0, s, keys[0], vals[0], tile_width,
-                       counts, u32p(L.estatus), tkeys[0], ids[0], pstatus[0], L.prows, u32p(L.kstatus), L.kblocks,
-                       u32p(L.depth_hist), error);
+    int64_t* ekeys[2] = {(int64_t*)(ws + L.ekeys0), (int64_t*)(ws + L.ekeys1)};
+    int32_t* eids[2] = {(int32_t*)(ws + L.eids0), (int32_t*)(ws + L.eids1)};
+    hipLaunchKernelGGL(super_emit_kernel, dim3(L.ewords), dim3(kEmitThreads), 0, s, keys[0], vals[0], L.sx_shift,
+                       L.sy_shift, L.super_width, counts, u32p(L.estatus), ekeys[0], eids[0], u32p(L.super_hist),
+                       u32p(L.pstatus), L.prows, u32p(L.kstatus), L.kblocks, u32p(L.depth_hist), error);
     GSX_LAUNCH_CHECK();
-    for (uint32_t pass = 0; pass < passes; ++pass) {
-        const bool last = pass + 1 == passes;
+    {
         RadixChainArgs a;
-        a.n_dev = counts, a.status = pstatus[pass], a.error = error;
-        a.total_replicas = 1, a.total_stride = 0;
-        a.clear_status = last ? nullptr : pstatus[1], a.clear_rows = L.prows;
-        if ((rc = radix_chained_pass_u16((uint32_t)capacity, tkeys[pass], ids[pass], tkeys[pass ^ 1u],
-                                         last ? flatten_ids : ids[pass ^ 1u], pass ? bits0 : 0u, pass ? bits1 : bits0,
-                                         u32p(L.pair_hist) + 256u * pass, a, !last, s)) != GSX_OK)
+        a.n_dev = counts + 3, a.status = u32p(L.pstatus), a.error = error;
+        a.total_replicas = kHistReplicas, a.total_stride = 256;
+        a.clear_status = nullptr, a.clear_rows = 0;
+        if ((rc = radix_chained_pass_i64((uint32_t)capacity, ekeys[0], eids[0], ekeys[1], eids[1], 32u, 8u,
+                                         u32p(L.super_hist), a, s)) != GSX_OK)
             return rc;
     }
+    // the coverage masks have one bit per tile of a super-tile: 1, 2, 4 or 8 words of 32
+    const uint32_t mask_words = std::max(1u, (1u << (L.sx_shift + L.sy_shift)) / 32u);
+    auto gather = mask_words == 1   ? tile_gather_kernel<1>
+                  : mask_words == 2 ? tile_gather_kernel<2>
+                  : mask_words == 4 ? tile_gather_kernel<4>
+                                    : tile_gather_kernel<8>;
+    hipLaunchKernelGGL(gather, dim3(L.grows), dim3(1024), 0, s, ekeys[1], eids[1], u32p(L.super_hist), counts,
+                       tile_offsets, tile_width, tile_height, L.sx_shift, L.sy_shift, L.super_width, L.n_super,
+                       u32p(L.gstatus), error, flatten_ids);
+    GSX_LAUNCH_CHECK();
     return GSX_OK;
 }
 
 // where a caller can read the outcome of the last call on the device: counts[0] = pairs in the lists (0 if they did
-// not fit), counts[1] = pairs there are, counts[2] = Gaussians that touch a tile; error[0]: bit 0 = capacity
+// not fit), counts[1] = pairs there are, counts[2] = Gaussians that touch a tile, counts[3] = (super-tile, Gaussian)
+// entries; error[0]: bit 0 = capacity
 // exceeded, bit 1 = a look-back gave up; error[1]: free for the caller (gsx_update_args.hold counts there)
 extern "C" const int64_t* gsx_tile_lists_counts(uint32_t N, int64_t capacity, uint32_t tile_width,
                                                 uint32_t tile_height, const void* workspace) {
