@@ -20,7 +20,7 @@ namespace gsx {
 
 static constexpr uint32_t kLbEmpty = 0u, kLbAggregate = 1u, kLbPrefix = 2u;
 static constexpr uint32_t kLbValueBits = 30u, kLbValueMask = (1u << kLbValueBits) - 1u;
-static constexpr uint32_t kLbSpinLimit = 1u << 20;
+static constexpr uint32_t kLbSpinLimit = 1u << 16; // about a tenth of a second: far beyond any wait that ends
 
 __device__ __forceinline__ void lb_publish(uint32_t* slot, uint32_t state, uint32_t value) {
     __hip_atomic_store(slot, (state << kLbValueBits) | value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -14,6 +14,7 @@
 // written out by consecutive lanes, so that every (tile, digit) run leaves the block as whole cache lines.
 #include <algorithm>
 #include <mutex>
+#include <vector>
 
 #include "gsx_common.h"
 #include "gsx_lookback.h"
@@ -192,7 +193,7 @@ struct RadixChain {
 // NW waves per workgroup (a tile of 64 NW ITEMS pairs): chained passes take eight or sixteen, for tiles of 8192 pairs -
 // half as many places for a look-back to walk; threads 0..255 double as the digits.
 template <typename KeyT, uint32_t ITEMS, bool CHAINED, bool WRITE_KEYS, uint32_t NW = 4>
-__global__ void __launch_bounds__(64 * NW) radix_scatter_kernel(uint32_t n, const KeyT* __restrict__ keys_in,
+__global__ void __launch_bounds__(64 * NW, NW == 8 ? 4 : 1) radix_scatter_kernel(uint32_t n, const KeyT* __restrict__ keys_in,
                                                              const int32_t* __restrict__ vals_in,
                                                              KeyT* __restrict__ keys_out,
                                                              int32_t* __restrict__ vals_out, uint32_t shift,
@@ -210,12 +211,24 @@ __global__ void __launch_bounds__(64 * NW) radix_scatter_kernel(uint32_t n, cons
     unsigned long long(*match)[kRadix] = reinterpret_cast<unsigned long long(*)[kRadix]>(overlay);
     int32_t* s_vals = reinterpret_cast<int32_t*>(overlay);
     KeyT* s_keys = reinterpret_cast<KeyT*>(overlay + kTileN * 4);
-    const uint32_t t = threadIdx.x;
+    const uint32_t t_in = threadIdx.x;
+    // the 64-bit chained passes (one workgroup per CU) loop over places; the 16-bit ones (two per CU, half the LDS)
+    // keep one place per workgroup: the loop costs them registers they do not have
+    constexpr bool kLoop = CHAINED && sizeof(KeyT) == 8;
+    // A chained launch has no more workgroups than the GPU holds at once; workgroup b takes the places b,
+    // b + gridDim.x, ... in turn, so a launch sized for a buffer's capacity does not queue hundreds of empty
+    // workgroups behind the few that have work, each waiting for a whole CU's LDS.  (All of them resident matters:
+    // place gridDim.x waits for place gridDim.x - 1, whose workgroup must have been started.)
+#pragma clang loop unroll(disable)
+    for (uint32_t place = blockIdx.x;; place += gridDim.x) {
+    // (the lane's index is made opaque once per place: otherwise every address of the body is kept in registers
+    // across the loop, and the kernel no longer fits the registers its occupancy allows)
+    uint32_t t = t_in;
+    asm volatile("" : "+v"(t));
     const uint32_t w = t >> 6, lane = t & 63u;
-    const uint32_t place = blockIdx.x;
+    const uint64_t lt_mask = (1ull << lane) - 1ull;
     const uint32_t tile_base = place * kTileN;
     const uint32_t wave_base = tile_base + w * kWaveN;
-    const uint64_t lt_mask = (1ull << lane) - 1ull;
     KeyT key[ITEMS];
     int32_t val[ITEMS];
     uint32_t rank[ITEMS]; // rank among the wave's pairs with the same digit
@@ -243,7 +256,7 @@ __global__ void __launch_bounds__(64 * NW) radix_scatter_kernel(uint32_t n, cons
             n = nd < (int64_t)n ? (uint32_t)(nd < 0 ? 0 : nd) : n;
         }
         // housekeeping for the pass after this one (its launch starts after this one has ended)
-        if (chain.clear_status != nullptr)
+        if (chain.clear_status != nullptr && place == blockIdx.x)
             for (size_t wd = (size_t)place * kThreads + t; wd < (size_t)chain.clear_rows * kRadix;
                  wd += (size_t)gridDim.x * kThreads)
                 chain.clear_status[wd] = 0u;
@@ -364,6 +377,10 @@ __global__ void __launch_bounds__(64 * NW) radix_scatter_kernel(uint32_t n, cons
                 vals_out[pos] = s_vals[slot];
             }
         }
+    }
+    if (!kLoop)
+        break;
+    __syncthreads(); // the tile in LDS has been written out
     }
 }
 
@@ -562,6 +579,33 @@ template <typename KeyT>
 struct ChainedShape {
     static constexpr uint32_t kWaves = sizeof(KeyT) == 8 ? 16 : 8, kItems = kChainedTile / (64 * kWaves);
 };
+// How many workgroups of `kernel` (no dynamic LDS) one device runs at the same time: what the runtime's occupancy
+// calculation gives per CU, times the CUs.  Remembered per (device, kernel).
+int resident_workgroups(const void* kernel, int threads, uint32_t* out) {
+    struct Entry {
+        int device;
+        const void* kernel;
+        uint32_t value;
+    };
+    static std::mutex mutex;
+    static std::vector<Entry> known;
+    int dev = -1;
+    GSX_HIP_CHECK(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(mutex);
+    for (const Entry& e : known)
+        if (e.device == dev && e.kernel == kernel) {
+            *out = e.value;
+            return GSX_OK;
+        }
+    int per_cu = 0, cus = 0;
+    GSX_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0));
+    GSX_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    GSX_REQUIRE(per_cu >= 1 && cus >= 1, GSX_ERR_HIP, "chained radix pass: %d workgroups per CU on %d CUs", per_cu, cus);
+    known.push_back({dev, kernel, (uint32_t)per_cu * (uint32_t)cus});
+    *out = known.back().value;
+    return GSX_OK;
+}
+
 uint32_t radix_chained_rows(int64_t n_max) { return n_max <= 0 ? 1u : cdiv((uint64_t)n_max, 256u * kItemsLarge); }
 
 namespace {
@@ -582,8 +626,23 @@ int chained_pass(uint32_t n_max, const KeyT* kin, const int32_t* vin, KeyT* kout
     c.total_replicas = a.total_replicas ? a.total_replicas : 1u, c.total_stride = a.total_stride;
     hipStream_t s = (hipStream_t)stream;
     using Shape = ChainedShape<KeyT>;
+    // as many workgroups as the device holds at once - asked of the runtime for this very kernel, whose registers
+    // and LDS decide it; each takes the places blockIdx.x, blockIdx.x + groups, ... in turn
+    uint32_t resident = 0;
+    if (write_keys) {
+        const int rc = resident_workgroups((const void*)radix_scatter_kernel<KeyT, Shape::kItems, true, true, Shape::kWaves>,
+                                           64 * Shape::kWaves, &resident);
+        if (rc != GSX_OK)
+            return rc;
+    } else {
+        const int rc = resident_workgroups((const void*)radix_scatter_kernel<KeyT, Shape::kItems, true, false, Shape::kWaves>,
+                                           64 * Shape::kWaves, &resident);
+        if (rc != GSX_OK)
+            return rc;
+    }
+    const uint32_t groups = sizeof(KeyT) == 8 ? std::min(rows, resident) : rows;
 #define GSX_CHAINED(WK)                                                                                        \
-    hipLaunchKernelGGL((radix_scatter_kernel<KeyT, Shape::kItems, true, WK, Shape::kWaves>), dim3(rows),      \
+    hipLaunchKernelGGL((radix_scatter_kernel<KeyT, Shape::kItems, true, WK, Shape::kWaves>), dim3(groups),    \
                        dim3(64 * Shape::kWaves), 0, s, n_max, kin, vin, kout, vout, shift, mask, rows,        \
                        (const uint32_t*)nullptr, digit_total, c)
     if (write_keys)

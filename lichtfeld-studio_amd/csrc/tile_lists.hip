@@ -348,7 +348,7 @@ __global__ void __launch_bounds__(1024) tile_table_kernel(
 // The launch also counts the entries per super-tile (the digit totals of the pass behind it).
 __global__ void __launch_bounds__(kEmitThreads) super_emit_kernel(
     const int64_t* __restrict__ sorted_keys, const int32_t* __restrict__ order, uint32_t sx_shift, uint32_t sy_shift,
-    uint32_t super_width, int64_t* __restrict__ counts, uint32_t* __restrict__ status,
+    uint32_t super_width, uint32_t capacity, int64_t* __restrict__ counts, uint32_t* __restrict__ status,
     int64_t* __restrict__ entry_keys, int32_t* __restrict__ entry_ids, uint32_t* __restrict__ super_hist,
     uint32_t* __restrict__ clear_status, uint32_t clear_rows, uint32_t* __restrict__ clear_key_status,
     uint32_t clear_key_words, uint32_t* __restrict__ clear_depth_hist, uint32_t* __restrict__ error) {
@@ -366,9 +366,11 @@ __global__ void __launch_bounds__(kEmitThreads) super_emit_kernel(
     static_assert(kEmitThreads == 1024, "one histogram word per lane");
     for (uint32_t r = place; r < kHistReplicas; r += gridDim.x)
         clear_depth_hist[r * 1024u + t] = 0u;
-    const uint32_t limit = (uint32_t)counts[0]; // 0 when the pairs do not fit: nothing is written
-    const uint32_t n = (uint32_t)counts[2];     // Gaussians that touch a tile
-    if (place * kEmitThreads >= n || limit == 0) {
+    // Nothing here waits for the tile table: entries are written while they fit the buffers (an entry stands for at
+    // least one pair, so they all do when the pairs do; when the pairs do not, the gather leaves every list empty).
+    const uint32_t limit = capacity;
+    const uint32_t n = (uint32_t)counts[2]; // Gaussians that touch a tile
+    if (place * kEmitThreads >= n) {
         if (place == 0 && t == 0)
             counts[3] = 0; // no entries (every later workgroup returns as well)
         return; // nobody behind this workgroup needs its (empty) contribution
@@ -406,10 +408,11 @@ __global__ void __launch_bounds__(kEmitThreads) super_emit_kernel(
             lb_publish(status + place, place == 0 ? kLbPrefix : kLbAggregate, block_total);
         const uint32_t before = lb_exclusive_wave(status, place, error);
         if (lane == 0) {
+            // (saturating: counts beyond 2^30 - 1 cannot fit any buffer, and must not reach the state bits)
             if (place != 0)
-                lb_publish(status + place, kLbPrefix, before + block_total);
+                lb_publish(status + place, kLbPrefix, min(before + block_total, kLbValueMask));
             if ((place + 1u) * kEmitThreads >= n)
-                counts[3] = (int64_t)(before + block_total); // entries there are (<= pairs: they fit)
+                counts[3] = (int64_t)(before + block_total); // entries there are
             base_s = before;
         }
     }
@@ -441,8 +444,8 @@ __global__ void __launch_bounds__(kEmitThreads) super_emit_kernel(
         if (pos < limit) {
             entry_keys[pos] = (int64_t)(((uint64_t)super_id << 32) | h);
             entry_ids[pos] = (int32_t)s_idx[wv][l];
-            atomicAdd(&sh[super_id & 255u], 1u);
         }
+        atomicAdd(&sh[super_id & 255u], 1u);
     }
     __syncthreads();
     if (t < 256 && sh[t] != 0u)
@@ -467,16 +470,17 @@ __global__ void __launch_bounds__(1024) tile_gather_kernel(
     uint32_t sy_shift, uint32_t super_width, uint32_t n_super, uint32_t* __restrict__ status,
     uint32_t* __restrict__ error, int32_t* __restrict__ flatten_ids) {
     constexpr uint32_t kTilesPerWave = WORDS * 2u;       // 32 WORDS tiles over 16 waves
-    __shared__ uint32_t s_mask[WORDS][kSliceEntries];
-    __shared__ int32_t s_id[kSliceEntries];
+    constexpr uint32_t kSlice = kSliceEntries;
+    __shared__ uint32_t s_mask[WORDS][kSlice];
+    __shared__ int32_t s_id[kSlice];
     __shared__ uint32_t seg_start[256], seg_len[256], slice_start[256];
     __shared__ uint32_t wave_a[4], wave_b[4];
     __shared__ uint32_t cnt[WORDS * 32u], base[WORDS * 32u];
     const uint32_t t = threadIdx.x, lane = t & 63u, wv = t >> 6;
-    const uint32_t limit = (uint32_t)counts[0];
     const uint32_t place = blockIdx.x;
-    // beyond the last slice there can be (entries / slice + one partial slice per super-tile): nothing to do
-    if (limit == 0 || place >= (uint32_t)counts[3] / kSliceEntries + n_super)
+    // counts[0] == 0: the pairs do not fit their buffer and every list stays empty.  Beyond the last slice there can
+    // be (entries / slice + one partial slice per super-tile): nothing to do
+    if (counts[0] == 0 || place >= (uint32_t)counts[3] / kSlice + n_super)
         return;
     // entries and slices in front of every super-tile (exclusive prefix sums over at most 256 counts)
     uint32_t len = 0, nsl = 0, in_len = 0, in_nsl = 0;
@@ -485,7 +489,7 @@ __global__ void __launch_bounds__(1024) tile_gather_kernel(
 #pragma unroll
             for (uint32_t r = 0; r < kHistReplicas; ++r)
                 len += super_hist[r * 256u + t];
-        nsl = (len + kSliceEntries - 1u) / kSliceEntries;
+        nsl = (len + kSlice - 1u) / kSlice;
         in_len = len, in_nsl = nsl;
 #pragma unroll
         for (uint32_t off = 1; off < 64; off <<= 1) {
@@ -526,13 +530,13 @@ __global__ void __launch_bounds__(1024) tile_gather_kernel(
             hi = mid - 1u;
     }
     const uint32_t sup = lo, k_slice = place - slice_start[sup];
-    const uint32_t a = seg_start[sup] + k_slice * kSliceEntries;
-    const uint32_t n_here = min(kSliceEntries, seg_start[sup] + seg_len[sup] - a);
+    const uint32_t a = seg_start[sup] + k_slice * kSlice;
+    const uint32_t n_here = min(kSlice, seg_start[sup] + seg_len[sup] - a);
     const uint32_t tx0 = (sup % super_width) << sx_shift, ty0 = (sup / super_width) << sy_shift;
     const uint32_t sx = 1u << sx_shift, sy = 1u << sy_shift;
     const uint32_t rows_per_word = 32u >> sx_shift;
 #pragma unroll
-    for (uint32_t k = 0; k < kSliceEntries / 1024u; ++k) {
+    for (uint32_t k = 0; k < kSlice / 1024u; ++k) {
         const uint32_t j = k * 1024u + t;
         uint32_t m[WORDS];
 #pragma unroll
@@ -612,11 +616,9 @@ __global__ void __launch_bounds__(1024) tile_gather_kernel(
         for (uint32_t i = 0; i < kTilesPerWave; ++i) {
             const bool in = (m[i >> 1] & ((i & 1u) ? bit1 : bit0)) != 0u;
             const uint64_t mask = __ballot(in);
-            if (in) {
-                const uint32_t pos = at[i] + (uint32_t)__popcll(mask & below);
-                if (pos < limit)
-                    flatten_ids[pos] = id;
-            }
+            // (a position is the tile's offset + entries in front: below the pair count, which fits the buffer)
+            if (in)
+                flatten_ids[at[i] + (uint32_t)__popcll(mask & below)] = id;
             at[i] += (uint32_t)__popcll(mask);
         }
     }
@@ -839,12 +841,11 @@ extern "C" int gsx_tile_lists(uint32_t N, const float* means2d, const int32_t* r
                                          u32p(L.depth_hist) + 256u * pass, a, s)) != GSX_OK)
             return rc;
     }
-    if (ts != s)
-        GSX_HIP_CHECK(hipStreamWaitEvent(s, ev->table_done, 0));
     int64_t* ekeys[2] = {(int64_t*)(ws + L.ekeys0), (int64_t*)(ws + L.ekeys1)};
     int32_t* eids[2] = {(int32_t*)(ws + L.eids0), (int32_t*)(ws + L.eids1)};
     hipLaunchKernelGGL(super_emit_kernel, dim3(L.ewords), dim3(kEmitThreads), 0, s, keys[0], vals[0], L.sx_shift,
-                       L.sy_shift, L.super_width, counts, u32p(L.estatus), ekeys[0], eids[0], u32p(L.super_hist),
+                       L.sy_shift, L.super_width, (uint32_t)capacity, counts, u32p(L.estatus), ekeys[0], eids[0],
+                       u32p(L.super_hist),
                        u32p(L.pstatus), L.prows, u32p(L.kstatus), L.kblocks, u32p(L.depth_hist), error);
     GSX_LAUNCH_CHECK();
     {
@@ -856,6 +857,8 @@ extern "C" int gsx_tile_lists(uint32_t N, const float* means2d, const int32_t* r
                                          u32p(L.super_hist), a, s)) != GSX_OK)
             return rc;
     }
+    if (ts != s) // the gather is the first launch that needs the tile table (tile_offsets, the fit decision)
+        GSX_HIP_CHECK(hipStreamWaitEvent(s, ev->table_done, 0));
     // the coverage masks have one bit per tile of a super-tile: 1, 2, 4 or 8 words of 32
     const uint32_t mask_words = std::max(1u, (1u << (L.sx_shift + L.sy_shift)) / 32u);
     auto gather = mask_words == 1   ? tile_gather_kernel<1>
