@@ -253,6 +253,13 @@ def main():
     tile_bits = int(L.lib().gsx_n_bits(ctypes.c_uint32(ts.tw * ts.th)))
     abytes = (algorithmic_bytes(ts.N, ts.K, H, W, ts.n_isects, tile_bits, 2) if ts.compact else
               algorithmic_bytes(ts.N, ts.K, H, W, ts.n_isects, 32 + tile_bits + 1))
+    if ts._lists_active:
+        # gsx_tile_lists by what it has to move: the projection's outputs in; per Gaussian that touches a tile a key,
+        # an id and a rectangle written and four radix passes over key + id (read + write); per (super-tile, Gaussian)
+        # entry a key + id written, one radix pass over them and their read by the gather; the lists and offsets out
+        _, pairs, visible, entries = ts.lists_counts()
+        abytes["tile_lists"] = (ts.N * 20 + visible * (16 + 4 * 24) + entries * (12 + 24 + 12) + pairs * 4 +
+                                (ts.tw * ts.th + 1) * 4)
     kernels = {}
     for k, ms in stage_ms.items():
         e = {"ms": round(ms, 4)}
@@ -324,7 +331,9 @@ def main():
         "config": {"workload": f"BASELINE configs[{args.config - 1}]: {ts.N} Gaussians SH degree {ts.sh_degree}, "
                                f"{W}x{H}, fwd + " + ("0.8 L1 + 0.2 (1-SSIM)" if use_ssim else "L1") +
                                " + bwd + fused Adam", "n_gaussians": ts.N, "image": [W, H], "n_isects": ts.n_isects,
-                   "tiles": ts.tw * ts.th, "pairs_fwd": pairs_fwd, "pairs_composited": pairs_comp,
+                   "tiles": ts.tw * ts.th, "tile_list_counts": dict(zip(("pairs_in_lists", "pairs", "gaussians_on_tiles",
+                                                                         "super_tile_entries"), ts.lists_counts())),
+                   "pairs_fwd": pairs_fwd, "pairs_composited": pairs_comp,
                    "pairs_bwd": pairs_bwd, "camera_tensor": "same every step" if args.same_camera else "changes every step",
                    "pair_count": "fetched by the host" if args.host_count else "stays on the device",
                    "bwd_wave_iterations": bwd_wave_iters, "wave_iterations": wave_iters,

@@ -144,8 +144,16 @@ GSX_API uint32_t gsx_n_bits(uint32_t n);
  * passes begin_bit = 0).  Buffers 0 (keys0/vals0, the input) and 1 (keys1/vals1) are ping-ponged; *selector_host
  * (host int) says which pair holds the result (like cub::DoubleBuffer::selector).  The workspace needs no particular
  * contents on entry; from 2 M pairs on, the sort is a fill of its bookkeeping words, one count of the digits of
- * every pass and one launch per 8-bit pass, below that three launches per pass (same result either way). */
+ * every pass and one launch per 8-bit pass, below that three launches per pass (same result either way).
+ * The one-launch passes chain their workgroups by a look-back whose every wait is bounded (about a tenth of a second):
+ * should a wait run out - a GPU so over-subscribed that a workgroup's predecessor does not get to run - the pass ends
+ * normally, every position it writes stays inside the buffers, bit 1 of an error word inside the workspace is set and
+ * the result is NOT sorted.  gsx_radix_sort_pairs_error gives that word's device address (NULL for sizes that take the
+ * three-launch passes, which cannot fail this way); each call clears it first.  A caller that cannot rule the
+ * condition out reads the word (4 bytes) after the sort and sorts again if it is not zero. */
 GSX_API size_t gsx_radix_sort_pairs_workspace_bytes(int64_t n);
+/* key_bytes: 8 (gsx_radix_sort_pairs) or 2 (gsx_radix_sort_tile_pairs) */
+GSX_API uint32_t* gsx_radix_sort_pairs_error(int64_t n, uint32_t key_bytes, void* workspace);
 /* the selector gsx_radix_sort_pairs will report for this size and bit range (known before the sort runs) */
 GSX_API int gsx_radix_sort_pairs_selector(int64_t n, uint32_t begin_bit, uint32_t end_bit);
 GSX_API int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, int64_t* keys1, int32_t* vals1,

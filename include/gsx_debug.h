@@ -23,6 +23,12 @@ GSX_API int gsx_debug_copy(const void* src, void* dst, size_t bytes, void* strea
  * (the fastgs backward) sums at a time.  in [n_waves,64,values] -> out [n_waves,values]. */
 GSX_API int gsx_debug_wave_reduce(uint32_t values, uint32_t n_waves, const float* in, float* out, void* stream);
 
+/* Test hook: how many empty reads a chained look-back (the one-launch radix passes, gsx_tile_lists) waits for a
+ * predecessor before it gives up; limit < 0 restores the default (65 536, about a tenth of a second).  With 0 every
+ * look-back that meets an empty word gives up at once: the give-up path (bit 1 of the error word, positions that stay
+ * inside the buffers, every kernel ending normally) can be exercised without making anything wait.  Process-wide. */
+GSX_API int gsx_debug_set_lookback_spin_limit(int64_t limit);
+
 /* Pair counts of one forward pass, for turning kernel times into rates (no counterpart in the reference).
  * stats_out: device uint64[8] = {(pixel, Gaussian) pairs the forward evaluates, pairs composited, pairs the backward
  * walks, (wave, Gaussian) iterations executed, (wave, Gaussian) iterations removed by the pixel bounds, executed

@@ -14,8 +14,8 @@ __all__ = ["_lib", "ops", "scenes", "build"]
 
 
 def __getattr__(name):
-    # ops / fused_* / trainer import torch; load them on first use
-    if name in ("ops", "build", "fused_ssim", "fused_adam", "trainer", "mcmc"):
+    # these import torch (or drive a compiler): loaded on first use
+    if name in ("ops", "build", "build_ext", "trainer", "rasterizer", "fastgs", "ply"):
         import importlib
         return importlib.import_module(f"{__name__}.{name}")
     raise AttributeError(name)

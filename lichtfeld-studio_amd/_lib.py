@@ -106,6 +106,7 @@ def lib():
                      "gsx_rasterize_bwd_workspace_bytes_for", "gsx_rasterize_bwd_accum_bytes_for"):
             getattr(L, name).restype = c_sz
         L.gsx_tile_lists_counts.restype = c_p
+        L.gsx_radix_sort_pairs_error.restype = c_p
         L.gsx_tile_lists_error.restype = c_p
         _lib = L
     return _lib

@@ -1,7 +1,11 @@
 // core.hip - error reporting, version, argument checks shared by the entry points.
 #include <stdarg.h>
 
+#include <algorithm>
+#include <atomic>
+
 #include "gsx_common.h"
+#include "gsx_lookback.h"
 
 namespace gsx {
 
@@ -69,6 +73,19 @@ __global__ void __launch_bounds__(256) copy_probe_kernel(const float4* __restric
 }
 
 } // namespace gsx
+
+namespace gsx {
+static std::atomic<int64_t> g_spin_limit{-1};
+uint32_t lookback_spin_limit() {
+    const int64_t v = g_spin_limit.load(std::memory_order_relaxed);
+    return v < 0 ? kLbSpinLimit : (uint32_t)v;
+}
+} // namespace gsx
+
+extern "C" int gsx_debug_set_lookback_spin_limit(int64_t limit) {
+    gsx::g_spin_limit.store(limit < 0 ? -1 : std::min<int64_t>(limit, gsx::kLbSpinLimit), std::memory_order_relaxed);
+    return GSX_OK;
+}
 
 extern "C" int gsx_debug_copy(const void* src, void* dst, size_t bytes, void* stream) {
     if (bytes == 0)

@@ -1064,6 +1064,9 @@ extern "C" int gsx_fastgs_backward(uint32_t N, const float* means, const float* 
                     grad_scales_raw && grad_rotations_raw && grad_opacities_raw && grad_sh_coefficients_0 &&
                     (grad_sh_coefficients_rest || settings->total_bases_sh_rest == 0),
                 GSX_ERR_INVALID_ARGUMENT, "fastgs_backward: null tensor");
+    // rows of up to 45 floats leave the workgroups as 16-byte stores
+    GSX_REQUIRE(((uintptr_t)grad_sh_coefficients_rest & 15) == 0, GSX_ERR_INVALID_ARGUMENT,
+                "fastgs_backward: grad_sh_coefficients_rest needs 16-byte alignment");
     GSX_REQUIRE(accum && ((uintptr_t)accum & 255) == 0 && accum_bytes >= gsx_fastgs_accum_bytes(N), GSX_ERR_WORKSPACE,
                 "fastgs_backward: accumulator needs %zu bytes, 256-byte aligned, zeroed", gsx_fastgs_accum_bytes(N));
     GSX_REQUIRE(n_instances >= 0 && n_instances < (1ll << 31), GSX_ERR_OVERFLOW, "fastgs_backward: %lld instances",

@@ -67,6 +67,8 @@ int radix_sort_pairs_32_bits(int64_t n, int64_t* keys0, int32_t* vals0, int64_t*
 // caller provides digit_total[256] = how many of the pairs carry each digit, a status table of
 // radix_chained_rows(n_max) x 256 empty (zero) words; the launch can clear the table of the pass that follows it.  n_dev (nullable): the number of pairs is min(*n_dev, n_max), read on the device.
 // Limit: n_max < 2^30.  error: device word, bit 1 is set if a look-back's bounded wait ran out.
+// how many empty reads a look-back waits before it gives up (gsx_lookback.h): the default, or what a test set
+uint32_t lookback_spin_limit();
 struct RadixChainArgs {
     const int64_t* n_dev;
     uint32_t *status, *clear_status;

@@ -28,8 +28,9 @@ __device__ __forceinline__ void lb_publish(uint32_t* slot, uint32_t state, uint3
 
 // Whether a waiting lane should give up: the bounded wait ran out here, or somewhere else already (then every lane
 // still waiting ends too, so a launch that cannot make progress ends after about one wait, not one per workgroup).
-__device__ __forceinline__ bool lb_give_up(uint32_t spins, uint32_t* error) {
-    if (spins > kLbSpinLimit ||
+// (`limit`: kLbSpinLimit, or what a test set through gsx_debug_set_lookback_spin_limit to see the give-up path)
+__device__ __forceinline__ bool lb_give_up(uint32_t spins, uint32_t* error, uint32_t limit) {
+    if (spins > limit ||
         ((spins & 255u) == 0 && (__hip_atomic_load(error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & 2u) != 0)) {
         atomicOr(error, 2u);
         return true;
@@ -43,7 +44,8 @@ __device__ __forceinline__ bool lb_give_up(uint32_t spins, uint32_t* error) {
 // from this XCD's L2, and the walk is as long as the prefixes have not caught up with the aggregates.
 // When the bounded wait runs out, bit 1 of *error is set and the partial sum returned.
 __device__ __forceinline__ uint32_t lb_exclusive(const uint32_t* status, uint32_t p, uint32_t stride,
-                                                 uint32_t column, uint32_t* error) {
+                                                 uint32_t column, uint32_t* error,
+                                                 uint32_t limit = kLbSpinLimit) {
     constexpr int kWindow = 8;
     uint32_t sum = 0, spins = 0;
     int64_t q = (int64_t)p - 1;
@@ -69,7 +71,7 @@ __device__ __forceinline__ uint32_t lb_exclusive(const uint32_t* status, uint32_
             break;
         q -= used;
         if (used == 0) {
-            if (lb_give_up(++spins, error))
+            if (lb_give_up(++spins, error, limit))
                 break;
             __builtin_amdgcn_s_sleep(1);
         }
@@ -79,7 +81,8 @@ __device__ __forceinline__ uint32_t lb_exclusive(const uint32_t* status, uint32_
 
 // The same sum for a table with one word per place, formed by a whole wave (all 64 lanes must call; all receive the
 // sum): lane l looks at place p - 1 - l, so 64 predecessors are inspected per round.
-__device__ __forceinline__ uint32_t lb_exclusive_wave(const uint32_t* status, uint32_t p, uint32_t* error) {
+__device__ __forceinline__ uint32_t lb_exclusive_wave(const uint32_t* status, uint32_t p, uint32_t* error,
+                                                      uint32_t limit = kLbSpinLimit) {
     const uint32_t lane = threadIdx.x & 63u;
     uint32_t sum = 0, spins = 0;
     int64_t top = (int64_t)p - 1; // the nearest place not yet added
@@ -104,7 +107,7 @@ __device__ __forceinline__ uint32_t lb_exclusive_wave(const uint32_t* status, ui
         if (usable == 0) {
             bool stop = false;
             if (lane == 0)
-                stop = lb_give_up(++spins, error);
+                stop = lb_give_up(++spins, error, limit);
             if (__ballot(stop))
                 break;
             __builtin_amdgcn_s_sleep(1);

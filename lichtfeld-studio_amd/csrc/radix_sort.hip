@@ -188,6 +188,7 @@ struct RadixChain {
     uint32_t clear_rows;
     uint32_t* error;        // bit 1 is set when a look-back gave up
     uint32_t total_replicas, total_stride; // digit_total = sum of this many tables, total_stride words apart
+    uint32_t spin_limit;    // empty reads after which a look-back gives up
 };
 
 // NW waves per workgroup (a tile of 64 NW ITEMS pairs): chained passes take eight or sixteen, for tiles of 8192 pairs -
@@ -343,7 +344,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 4 : 1) radix_scatter_kernel
             }
             uint32_t earlier; // pairs with digit t in the workgroups in front of this one
             if (CHAINED) {
-                earlier = lb_exclusive(chain.status, place, kRadix, t, chain.error);
+                earlier = lb_exclusive(chain.status, place, kRadix, t, chain.error, chain.spin_limit);
                 if (place != 0)
                     lb_publish(chain.status + (size_t)place * kRadix + t, kLbPrefix, earlier + tot);
             } else {
@@ -408,6 +409,10 @@ struct SortLayout {
     size_t digits_off, misc_off, status_off[2], total;
 };
 static constexpr size_t kDigitsBytes = (size_t)kMaxPasses * kTotalReplicas * kRadix * 4;
+// whether sort_pairs takes the chained passes for this size
+bool sort_is_chained(int64_t n, uint32_t key_bytes) {
+    return n < (1ll << kLbValueBits) && n > (key_bytes == 8 ? kSmallSortLimit : (1ll << 25));
+}
 uint32_t sort_items(int64_t n) { return n <= kSmallSortLimit ? kItemsSmall : kItemsLarge; }
 SortLayout sort_layout(int64_t n) {
     SortLayout L;
@@ -460,7 +465,7 @@ int sort_pairs(const char* what, int64_t n, KeyT* keys0, int32_t* vals0, KeyT* k
     // measured: the chained sort is ahead from ~2 M pairs with 64-bit keys (310 against 339 us at 5.67 M pairs and 45
     // bits, 834 against 973 us at 16 M) and from ~30 M pairs with 16-bit keys (706 against 812 us at 64 M); below, its
     // few large workgroups and the extra read of the keys cost more than the launches they save
-    chained = chained && n < (1ll << kLbValueBits) && n > (sizeof(KeyT) == 8 ? kSmallSortLimit : (1ll << 25));
+    chained = chained && sort_is_chained(n, (uint32_t)sizeof(KeyT));
     const size_t need = chained ? L.total : L.tabled_total;
     GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 && workspace_bytes >= need,
                 GSX_ERR_WORKSPACE, "%s: workspace needs %zu bytes, 256-byte aligned", what, need);
@@ -624,6 +629,7 @@ int chained_pass(uint32_t n_max, const KeyT* kin, const int32_t* vin, KeyT* kout
     c.clear_rows = a.clear_rows, c.error = a.error;
     GSX_REQUIRE(a.total_replicas <= 4, GSX_ERR_INVALID_ARGUMENT, "chained radix pass: at most 4 total tables");
     c.total_replicas = a.total_replicas ? a.total_replicas : 1u, c.total_stride = a.total_stride;
+    c.spin_limit = lookback_spin_limit();
     hipStream_t s = (hipStream_t)stream;
     using Shape = ChainedShape<KeyT>;
     // as many workgroups as the device holds at once - asked of the runtime for this very kernel, whose registers
@@ -666,6 +672,12 @@ int radix_chained_pass_u16(uint32_t n_max, const uint16_t* kin, const int32_t* v
     return chained_pass<uint16_t>(n_max, kin, vin, kout, vout, shift, bits, digit_total, a, write_keys, stream);
 }
 } // namespace gsx
+
+extern "C" uint32_t* gsx_radix_sort_pairs_error(int64_t n, uint32_t key_bytes, void* workspace) {
+    if (workspace == nullptr || n <= 0 || (key_bytes != 8 && key_bytes != 2) || !sort_is_chained(n, key_bytes))
+        return nullptr;
+    return (uint32_t*)((char*)workspace + sort_layout(n).misc_off);
+}
 
 extern "C" int gsx_radix_sort_pairs(int64_t n, int64_t* keys0, int32_t* vals0, int64_t* keys1, int32_t* vals1,
                                     uint32_t begin_bit, uint32_t end_bit, void* workspace, size_t workspace_bytes,

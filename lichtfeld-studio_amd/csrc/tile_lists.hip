@@ -33,6 +33,7 @@
 // on a single word 20 ns each, serialised).  Counts meet through per-workgroup rows and replicas instead.
 #include <algorithm>
 #include <mutex>
+#include <vector>
 
 #include "gsx_common.h"
 #include "gsx_lookback.h"
@@ -71,7 +72,7 @@ __global__ void __launch_bounds__(kKeysThreads) depth_keys_kernel(
     uint32_t* __restrict__ status /*[blocks]*/, int64_t* __restrict__ counts, uint32_t* __restrict__ error,
     uint32_t* __restrict__ clear_status, uint32_t clear_rows, uint32_t* __restrict__ clear_emit_status,
     uint32_t clear_emit_words, uint32_t* __restrict__ clear_super_hist, uint32_t* __restrict__ clear_gather_status,
-    uint32_t gather_rows_max, uint32_t n_super, uint32_t* __restrict__ depth_hist) {
+    uint32_t gather_rows_max, uint32_t n_super, uint32_t* __restrict__ depth_hist, uint32_t spin_limit) {
     constexpr uint32_t kWaves = kKeysThreads / 64u;
     __shared__ uint32_t wave_total[kWaves];
     __shared__ uint32_t base_s;
@@ -150,7 +151,7 @@ __global__ void __launch_bounds__(kKeysThreads) depth_keys_kernel(
         for (uint32_t b = 0; b < 4; ++b)
             wave_hist_add(lh[b], (lo[k] >> (8u * b)) & 255u, hi[k] != 0u);
     if (wv == 0) {
-        const uint32_t before = lb_exclusive_wave(status, blockIdx.x, error);
+        const uint32_t before = lb_exclusive_wave(status, blockIdx.x, error, spin_limit);
         if (lane == 0) {
             if (blockIdx.x != 0)
                 lb_publish(status + blockIdx.x, kLbPrefix, before + block_total);
@@ -239,7 +240,11 @@ __global__ void __launch_bounds__(1024) tile_table_kernel(
         for (uint32_t i = t; i < cells; i += 1024u)
             __hip_atomic_store(&replicas[(size_t)blockIdx.x * cells + i], GSX_GRID(i), __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads(); // every lane's stores have been acknowledged
+    // The election below must not overtake the replicas: every lane waits for its own stores to be acknowledged
+    // (vmcnt(0): they are device-scope stores, acknowledged by the level the other XCDs read) before the barrier
+    // lets thread 0 add to the counter.  The workgroup that finds the counter complete therefore sees every replica.
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+    __syncthreads();
     if (t == 0)
         last_s = atomicAdd(done_counter, 1u) == gridDim.x - 1u ? 1u : 0u;
     __syncthreads();
@@ -351,7 +356,8 @@ __global__ void __launch_bounds__(kEmitThreads) super_emit_kernel(
     uint32_t super_width, uint32_t capacity, int64_t* __restrict__ counts, uint32_t* __restrict__ status,
     int64_t* __restrict__ entry_keys, int32_t* __restrict__ entry_ids, uint32_t* __restrict__ super_hist,
     uint32_t* __restrict__ clear_status, uint32_t clear_rows, uint32_t* __restrict__ clear_key_status,
-    uint32_t clear_key_words, uint32_t* __restrict__ clear_depth_hist, uint32_t* __restrict__ error) {
+    uint32_t clear_key_words, uint32_t* __restrict__ clear_depth_hist, uint32_t* __restrict__ error,
+    uint32_t spin_limit) {
     constexpr uint32_t kWaves = kEmitThreads / 64u;
     __shared__ uint32_t s_incl[kWaves][64], s_hi[kWaves][64], s_idx[kWaves][64];
     __shared__ uint32_t wave_total[kWaves];
@@ -406,7 +412,7 @@ __global__ void __launch_bounds__(kEmitThreads) super_emit_kernel(
     if (wv == 0) {
         if (lane == 0)
             lb_publish(status + place, place == 0 ? kLbPrefix : kLbAggregate, block_total);
-        const uint32_t before = lb_exclusive_wave(status, place, error);
+        const uint32_t before = lb_exclusive_wave(status, place, error, spin_limit);
         if (lane == 0) {
             // (saturating: counts beyond 2^30 - 1 cannot fit any buffer, and must not reach the state bits)
             if (place != 0)
@@ -468,7 +474,7 @@ __global__ void __launch_bounds__(1024) tile_gather_kernel(
     const uint32_t* __restrict__ super_hist, const int64_t* __restrict__ counts,
     const int32_t* __restrict__ tile_offsets, uint32_t tile_width, uint32_t tile_height, uint32_t sx_shift,
     uint32_t sy_shift, uint32_t super_width, uint32_t n_super, uint32_t* __restrict__ status,
-    uint32_t* __restrict__ error, int32_t* __restrict__ flatten_ids) {
+    uint32_t* __restrict__ error, uint32_t spin_limit, int32_t* __restrict__ flatten_ids) {
     constexpr uint32_t kTilesPerWave = WORDS * 2u;       // 32 WORDS tiles over 16 waves
     constexpr uint32_t kSlice = kSliceEntries;
     __shared__ uint32_t s_mask[WORDS][kSlice];
@@ -596,7 +602,7 @@ __global__ void __launch_bounds__(1024) tile_gather_kernel(
             lb_publish(status + (size_t)place * 256u + t, kLbPrefix, mine);
         } else {
             lb_publish(status + (size_t)place * 256u + t, kLbAggregate, mine);
-            before = lb_exclusive(status, place, 256u, t, error);
+            before = lb_exclusive(status, place, 256u, t, error, spin_limit);
             lb_publish(status + (size_t)place * 256u + t, kLbPrefix, before + mine);
         }
         base[t] = before + offset;
@@ -702,24 +708,29 @@ ListsLayout lists_layout(uint32_t N, int64_t capacity, uint32_t tw, uint32_t th)
     L.total = o;
     return L;
 }
-// two events per device for the fork / join with a caller's second stream (created once, never destroyed)
+// two events per (device, stream) for the fork / join with a caller's second stream (created once, never destroyed):
+// calls on different streams - other workspaces, other host threads - do not share them
 struct SideEvents {
+    int device;
+    void* stream;
     hipEvent_t keys_done, table_done;
 };
-int side_events(SideEvents** out) {
+int side_events(void* stream, SideEvents** out) {
     static std::mutex mutex;
-    static SideEvents events[64];
-    static bool made[64] = {};
+    static std::vector<SideEvents*> known;
     int dev = -1;
     GSX_HIP_CHECK(hipGetDevice(&dev));
-    GSX_REQUIRE(dev >= 0 && dev < 64, GSX_ERR_UNSUPPORTED, "tile_lists: device ordinal %d", dev);
     std::lock_guard<std::mutex> lock(mutex);
-    if (!made[dev]) {
-        GSX_HIP_CHECK(hipEventCreateWithFlags(&events[dev].keys_done, hipEventDisableTiming));
-        GSX_HIP_CHECK(hipEventCreateWithFlags(&events[dev].table_done, hipEventDisableTiming));
-        made[dev] = true;
-    }
-    *out = &events[dev];
+    for (SideEvents* e : known)
+        if (e->device == dev && e->stream == stream) {
+            *out = e;
+            return GSX_OK;
+        }
+    SideEvents* e = new SideEvents{dev, stream, nullptr, nullptr};
+    GSX_HIP_CHECK(hipEventCreateWithFlags(&e->keys_done, hipEventDisableTiming));
+    GSX_HIP_CHECK(hipEventCreateWithFlags(&e->table_done, hipEventDisableTiming));
+    known.push_back(e);
+    *out = e;
     return GSX_OK;
 }
 int check_lists_args(const char* who, uint32_t N, int64_t capacity, uint32_t tw, uint32_t th) {
@@ -804,18 +815,19 @@ extern "C" int gsx_tile_lists(uint32_t N, const float* means2d, const int32_t* r
     uint32_t* error = u32p(L.error);
     int64_t* counts = (int64_t*)(ws + L.counts);
     hipStream_t s = (hipStream_t)stream;
+    const uint32_t spin_limit = lookback_spin_limit();
 
     hipLaunchKernelGGL(depth_keys_kernel, dim3(L.kblocks), dim3(kKeysThreads), 0, s, N, means2d, radii, depths,
                        (float)tile_size, tile_width, tile_height, keys[0], vals[0], u32p(L.rects), u32p(L.kstatus),
                        counts, error, dstatus[0], L.drows, u32p(L.estatus), L.ewords, u32p(L.super_hist),
-                       u32p(L.gstatus), L.grows, L.n_super, u32p(L.depth_hist));
+                       u32p(L.gstatus), L.grows, L.n_super, u32p(L.depth_hist), spin_limit);
     GSX_LAUNCH_CHECK();
     // The tile table needs the rectangles only, not their depth order: with a second stream it is formed while the
     // sort runs.
     hipStream_t ts = side_stream != nullptr && side_stream != stream ? (hipStream_t)side_stream : s;
     SideEvents* ev = nullptr;
     if (ts != s) {
-        if ((rc = side_events(&ev)) != GSX_OK)
+        if ((rc = side_events(stream, &ev)) != GSX_OK)
             return rc;
         GSX_HIP_CHECK(hipEventRecord(ev->keys_done, s));
         GSX_HIP_CHECK(hipStreamWaitEvent(ts, ev->keys_done, 0));
@@ -846,7 +858,7 @@ extern "C" int gsx_tile_lists(uint32_t N, const float* means2d, const int32_t* r
     hipLaunchKernelGGL(super_emit_kernel, dim3(L.ewords), dim3(kEmitThreads), 0, s, keys[0], vals[0], L.sx_shift,
                        L.sy_shift, L.super_width, (uint32_t)capacity, counts, u32p(L.estatus), ekeys[0], eids[0],
                        u32p(L.super_hist),
-                       u32p(L.pstatus), L.prows, u32p(L.kstatus), L.kblocks, u32p(L.depth_hist), error);
+                       u32p(L.pstatus), L.prows, u32p(L.kstatus), L.kblocks, u32p(L.depth_hist), error, spin_limit);
     GSX_LAUNCH_CHECK();
     {
         RadixChainArgs a;
@@ -867,7 +879,7 @@ extern "C" int gsx_tile_lists(uint32_t N, const float* means2d, const int32_t* r
                                     : tile_gather_kernel<8>;
     hipLaunchKernelGGL(gather, dim3(L.grows), dim3(1024), 0, s, ekeys[1], eids[1], u32p(L.super_hist), counts,
                        tile_offsets, tile_width, tile_height, L.sx_shift, L.sy_shift, L.super_width, L.n_super,
-                       u32p(L.gstatus), error, flatten_ids);
+                       u32p(L.gstatus), error, spin_limit, flatten_ids);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

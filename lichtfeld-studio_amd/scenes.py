@@ -115,9 +115,10 @@ def plumbing_scene(n=10_000, seed=0, width=256, height=256, f=280.0):
 
 
 def cluster_scene(n, seed, name, sh_degree=3, n_clusters=32, cluster_sigma=0.3, logscale_mu=-4.5, logscale_sigma=0.7,
-                  opacity_sigma=1.5, ball_fraction=0.0, ball_radius=0.5):
+                  opacity_sigma=1.5, ball_fraction=0.0, ball_radius=0.5, geometry_only=False):
     """BASELINE configurations 2-5: mixture of isotropic clusters inside [-2,2]^3 (optionally with a
-    fraction of the means concentrated in a ball at the origin), SH degree 3."""
+    fraction of the means concentrated in a ball at the origin), SH degree 3.  geometry_only: the SH coefficients
+    (drawn last, most of the generator's time) are left out - means, scales, rotations, opacities are the same."""
     rng = np.random.default_rng(seed)
     centres = rng.uniform(-2.0, 2.0, (n_clusters, 3))
     cid = rng.integers(0, n_clusters, n)
@@ -132,6 +133,9 @@ def cluster_scene(n, seed, name, sh_degree=3, n_clusters=32, cluster_sigma=0.3, 
     scaling_raw = rng.normal(logscale_mu, logscale_sigma, (n, 3)).astype(np.float32)
     rotation_raw = _normalize(rng.normal(0.0, 1.0, (n, 4)))
     opacity_raw = rng.normal(0.0, opacity_sigma, (n, 1)).astype(np.float32)
+    if geometry_only:
+        sh0, shN = np.zeros((n, 1, 3), np.float32), np.zeros((n, 0, 3), np.float32)
+        return Scene(name, means, sh0, shN, scaling_raw, rotation_raw, opacity_raw, 0, [])
     sh0, shN = _sh(rng, n, sh_degree, dc_is_colour=False)
     return Scene(name, means, sh0, shN, scaling_raw, rotation_raw, opacity_raw, sh_degree, [])
 
@@ -139,9 +143,10 @@ def cluster_scene(n, seed, name, sh_degree=3, n_clusters=32, cluster_sigma=0.3, 
 CFG5_LOGSCALE_MU = -5.0
 
 
-def config5_literal(n=6_000_000):
+def config5_literal(n=6_000_000, geometry_only=False):
     """Configuration 5 with the log-scale mean exactly as stated (-3.5): more intersections than int32 can index."""
-    sc = cluster_scene(n, 5, "cfg5-literal", logscale_mu=-3.5, logscale_sigma=1.0, ball_fraction=0.7)
+    sc = cluster_scene(n, 5, "cfg5-literal", logscale_mu=-3.5, logscale_sigma=1.0, ball_fraction=0.7,
+                       geometry_only=geometry_only)
     sc.cameras = [orbit_camera(2.6, 4.0, 3840, 2160, 3200.0)]
     return sc
 

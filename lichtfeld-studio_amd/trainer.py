@@ -146,6 +146,17 @@ class TrainStep:
         self.flat_out = torch.empty(self.cap, dtype=torch.int32, device=self.dev)
         self._lists_dims = dims
 
+    def lists_counts(self):
+        """(pairs in the lists, pairs there are, Gaussians that touch a tile, (super-tile, Gaussian) entries) of the
+        last gsx_tile_lists call; synchronises"""
+        if self.lists_ws is None:
+            return 0, 0, 0, 0
+        a = (c_u32(self.N), c_i64(self.cap), c_u32(self.tw), c_u32(self.th))
+        at = self.lib.gsx_tile_lists_counts(*a, c_p(self.lists_ws.data_ptr())) - self.lists_ws.data_ptr()
+        torch.cuda.synchronize(self.dev)
+        w = self.lists_ws[at:at + 32].cpu().numpy().view(np.int64)
+        return tuple(int(x) for x in w)
+
     def lists_error(self):
         """(error bits, optimiser calls held back) of the tile lists so far; synchronises"""
         if self.lists_ws is None:

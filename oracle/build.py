@@ -31,5 +31,25 @@ def build(force=True):
     return OUT
 
 
+def sanitize():
+    """The checker's sources and oracle/sanitize_driver.cpp as one executable under AddressSanitizer and
+    UndefinedBehaviorSanitizer (host code only), run once: a small training iteration through the C entry points with
+    exactly sized heap buffers.  Returns the driver's output; raises when the build or the run fails."""
+    exe = os.path.join(HERE, "sanitize_check")
+    flags = ["-O1", "-g", "-march=x86-64-v3", "-ffp-contract=off", "-fno-fast-math", "-fopenmp", "-std=c++17",
+             "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer",
+             "-Wno-unknown-pragmas"]
+    subprocess.run(["g++", *flags, "-I", MATH_INC, *SRCS, os.path.join(HERE, "sanitize_driver.cpp"), "-o", exe],
+                   check=True)
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:abort_on_error=1", OMP_NUM_THREADS="4")
+    r = subprocess.run([exe], capture_output=True, text=True, env=env)
+    if r.returncode != 0:
+        raise RuntimeError(f"sanitize_check failed (exit {r.returncode}):\n{r.stdout}\n{r.stderr}")
+    return r.stdout.strip()
+
+
 if __name__ == "__main__":
-    print(build(force="--if-stale" not in sys.argv))
+    if "--sanitize" in sys.argv:
+        print(sanitize())
+    else:
+        print(build(force="--if-stale" not in sys.argv))

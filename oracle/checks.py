@@ -55,6 +55,13 @@ L2_MULT = 2.0
 L2_EPS = 4 * 1.1920929e-07
 MISS_RATIO = 1.5
 MISS_SLACK = 2e-4
+# The same comparison in its plain form, against the fp32 reference-order checker itself:
+#   |gpu - fp32| <= PLAIN_RTOL |fp32| + PLAIN_ATOL_RMS * rms(fp32 tensor over the Gaussians that carry a gradient).
+# The absolute term is what the cancellation in the reference's own order costs the CHECKER on the elements that are
+# small sums of large terms (the float64 columns of the report show on which side the error lies).
+PLAIN_RTOL = 1e-3
+PLAIN_ATOL_RMS = 1e-3
+PLAIN = []  # (tag + name, needed atol / rms) of every call, for the summary
 
 REPORT = []  # lines for the end-of-session summary (tests/conftest.py prints them)
 
@@ -92,6 +99,15 @@ def gradient_bar(tag, name, gpu, o32, f64, bound=None, rel=REL):
     ex_o = np.abs(o - t) - rel * np.abs(t)
     nt = np.linalg.norm(t)
     l2g, l2o = float(np.linalg.norm(g - t) / nt), float(np.linalg.norm(o - t) / nt)
+    # plain rtol + atol form against the fp32 checker
+    live_rows = np.abs(o.reshape(rows.shape)).sum(1) > 0
+    rms = float(np.sqrt(np.mean(np.square(o.reshape(rows.shape)[live_rows])))) if live_rows.any() else 0.0
+    plain_need = float((np.abs(g - o) - PLAIN_RTOL * np.abs(o)).max()) / max(rms, 1e-300)
+    PLAIN.append((f"{tag}{name}", plain_need))
+    report(f"{tag}{name:12s} plain form: |gpu - fp32| <= {PLAIN_RTOL:g} |fp32| + atol needs atol = "
+           f"{max(plain_need, 0.0):.2e} x rms(fp32) (bar {PLAIN_ATOL_RMS:g}; rms {rms:.3e})")
+    assert plain_need <= PLAIN_ATOL_RMS, (f"{tag}{name}: |gpu - fp32 checker| exceeds {PLAIN_RTOL:g} |fp32| + "
+                                          f"{PLAIN_ATOL_RMS:g} rms by needing {plain_need:.3e} rms")
     head = (f"{tag}{name:12s} n={m['n']:9d} miss>1e-3: gpu|fp32 {m['gpu_vs_fp32']:.2e} gpu|f64 {m['gpu_vs_f64']:.2e} "
             f"fp32|f64 {m['fp32_vs_f64']:.2e}  need: ")
     tail = f", L2 {l2g / max(l2o, 1e-300):.2f} x fp32's ({l2g:.1e} vs {l2o:.1e})"

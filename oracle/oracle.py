@@ -233,6 +233,21 @@ def spherical_harmonics_bwd(K, degrees_to_use, dirs, coeffs, masks, v_colors, co
     return v_coeffs, v_dirs
 
 
+def intersect_tile_count(means2d, radii, C, tile_size, tile_width, tile_height):
+    """The first launch of intersect_tile alone (IntersectTile.cu:46-114 with null outputs, Intersect.cpp:58-76):
+    -> tiles_per_gauss [C,N] i32 and the number of intersections (an int64: it may exceed what int32 indexes)."""
+    means2d = _f32(means2d)
+    radii = np.ascontiguousarray(radii, dtype=np.int32)
+    N = means2d.shape[1]
+    tpg = np.zeros((C, N), np.int32)
+    cum = np.zeros((C, N), np.int64)
+    n_isects = c_i64(0)
+    _chk(lib().orc_intersect_tile_count(c_u32(C), c_u32(N), _p(means2d), _p(radii), c_u32(tile_size),
+                                        c_u32(tile_width), c_u32(tile_height), _p(tpg), _p(cum),
+                                        ctypes.byref(n_isects)), "intersect_tile_count")
+    return tpg, int(n_isects.value)
+
+
 def intersect_tile(means2d, radii, depths, C, tile_size, tile_width, tile_height, sort=True):
     """gsplat/Ops.h:28-38 (unpacked).  -> tiles_per_gauss [C,N] i32, isect_ids [I] i64, flatten_ids [I] i32."""
     means2d, depths = _f32(means2d), _f32(depths)

@@ -70,3 +70,9 @@ def pytest_terminal_summary(terminalreporter):
         terminalreporter.write_sep("-", "measured parity: fraction of elements outside 1e-3 relative, needed multipliers")
         for line in checks.REPORT:
             terminalreporter.write_line(line)
+        if checks.PLAIN:
+            worst = max(checks.PLAIN, key=lambda x: x[1])
+            terminalreporter.write_line(
+                f"plain form over {len(checks.PLAIN)} tensors: |gpu - fp32 checker| <= {checks.PLAIN_RTOL:g} |fp32| + "
+                f"{checks.PLAIN_ATOL_RMS:g} rms(fp32) holds everywhere; largest atol needed {max(worst[1], 0.0):.2e} rms "
+                f"({worst[0].strip()})")

@@ -162,3 +162,30 @@ def test_bench_finds_its_kernel_in_the_committed_traffic_summary():
     prefix = re.search(r'measured_traffic_bytes\("([^"]+)"\)', src).group(1)
     nbytes = bench.measured_traffic_bytes(prefix)
     assert nbytes is not None and 5e7 < nbytes < 2e9, (prefix, nbytes)
+
+
+def test_config5_as_stated_exceeds_int32_pairs(gsx, orc):
+    """BASELINE configs[4] with its literal parameters (log-scales ~N(-3.5, 1) at 3840x2160, f = 3200): the count
+    pass of intersect_tile alone (no pair is formed) gives more (tile, Gaussian) pairs than the int32 flatten_ids /
+    uint32 n_isects of the reference can index (Intersect.cpp:84-85, IntersectTile.cu:45,207) - which is why the
+    suite's configuration 5 uses log-scale mean -5.0, and why the library answers GSX_ERR_OVERFLOW to the literal one."""
+    sc = gsx.scenes.config5_literal(geometry_only=True)
+    cam = sc.cameras[0]
+    means, quats, scales, op, _ = gsx.scenes.activate(sc)
+    assert means.shape[0] == 6_000_000 and (cam.width, cam.height) == (3840, 2160)
+    radii, means2d = orc.projection_ut_3dgs_fused(means, quats, scales, op, cam.viewmat[None], cam.K[None], cam.width,
+                                                  cam.height)[:2]
+    tiles_per_gauss, n = orc.intersect_tile_count(means2d, radii, 1, 16, (cam.width + 15) // 16,
+                                                  (cam.height + 15) // 16)
+    assert n == int(tiles_per_gauss.astype(np.int64).sum())
+    assert n > 2 ** 31, n
+    # the re-scaled configuration the suite runs has the same geometry generator and differs in that one parameter
+    assert gsx.scenes.CFG5_LOGSCALE_MU == -5.0
+
+
+def test_checker_under_address_and_undefined_behaviour_sanitizers():
+    """oracle/build.py --sanitize: the checker's sources under -fsanitize=address,undefined run one small training
+    iteration with exactly sized heap buffers (any overrun or undefined operation aborts it)"""
+    from oracle import build as obuild
+    out = obuild.sanitize()
+    assert "sanitize_driver ok" in out, out

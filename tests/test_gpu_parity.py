@@ -418,6 +418,51 @@ def test_radix_sort_stable(gsx, orc, cuda, n):
     bits_equal(N(v), ref_v, '')
 
 
+def test_chained_sort_reports_a_look_back_that_gave_up(gsx, cuda):
+    """The one-launch radix passes bound every wait of their look-back.  With the bound set to zero from the host
+    (gsx_debug_set_lookback_spin_limit; nothing is made to wait) the first look-back that meets a predecessor's empty
+    word gives up: every kernel still ends normally, nothing is written out of bounds, and the error word that
+    gsx_radix_sort_pairs_error points to reads 2.  With the bound restored the same buffers sort correctly and the
+    word reads 0."""
+    import ctypes
+    L = gsx._lib
+    lb = L.lib()
+    n = 4_000_000
+    g = torch.Generator(device=cuda).manual_seed(3)
+    keys = torch.randint(0, 1 << 44, (n,), generator=g, device=cuda, dtype=torch.int64)
+    vals = torch.arange(n, device=cuda, dtype=torch.int32)
+    nbytes = lb.gsx_radix_sort_pairs_workspace_bytes(ctypes.c_int64(n))
+    ws = torch.empty((nbytes,), dtype=torch.uint8, device=cuda)
+    assert lb.gsx_radix_sort_pairs_error(ctypes.c_int64(100_000), ctypes.c_uint32(8), ctypes.c_void_p(ws.data_ptr())) is None
+    err_at = lb.gsx_radix_sort_pairs_error(ctypes.c_int64(n), ctypes.c_uint32(8), ctypes.c_void_p(ws.data_ptr()))
+    assert err_at is not None and 0 <= err_at - ws.data_ptr() < nbytes
+    word = lambda: int(ws[err_at - ws.data_ptr():err_at - ws.data_ptr() + 4].cpu().numpy().view(np.uint32)[0])
+
+    def sort():
+        k0, v0 = keys.clone(), vals.clone()
+        k1, v1 = torch.full_like(k0, -1), torch.full_like(v0, -1)
+        sel = ctypes.c_int(0)
+        L.check(lb.gsx_radix_sort_pairs(ctypes.c_int64(n), ctypes.c_void_p(k0.data_ptr()), ctypes.c_void_p(v0.data_ptr()),
+                                        ctypes.c_void_p(k1.data_ptr()), ctypes.c_void_p(v1.data_ptr()),
+                                        ctypes.c_uint32(0), ctypes.c_uint32(44), ctypes.c_void_p(ws.data_ptr()),
+                                        ctypes.c_size_t(nbytes), ctypes.byref(sel),
+                                        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        torch.cuda.synchronize()
+        return (k1, v1) if sel.value else (k0, v0)
+
+    try:
+        L.check(lb.gsx_debug_set_lookback_spin_limit(ctypes.c_int64(0)))
+        k, v = sort()
+        assert word() == 2, "no look-back met an empty word: the give-up path did not run"
+        assert int(v.min()) >= -1 and int(v.max()) < n  # whatever landed came from the input
+    finally:
+        L.check(lb.gsx_debug_set_lookback_spin_limit(ctypes.c_int64(-1)))
+    k, v = sort()
+    assert word() == 0
+    ref_k, order = torch.sort(keys, stable=True)
+    assert torch.equal(k, ref_k) and torch.equal(v.long(), order)
+
+
 def test_radix_sort_bit_range(gsx, orc, cuda):
     """only bits [0, end_bit) take part: keys that differ above end_bit keep their input order"""
     import ctypes
