@@ -260,6 +260,9 @@ def main():
         _, pairs, visible, entries = ts.lists_counts()
         abytes["tile_lists"] = (ts.N * 20 + visible * (16 + 4 * 24) + entries * (12 + 24 + 12) + pairs * 4 +
                                 (ts.tw * ts.th + 1) * 4)
+        # the SH / record pass reads every row's radii and skips the rows the projection culled: it is priced by
+        # the rows it moves (mean, coefficients, activated parameters in; colour and record out)
+        abytes["sh_colors_records_from_world"] = ts.N * 8 + visible * (12 + 12 * ts.K + 32 + 12 + 96)
     kernels = {}
     for k, ms in stage_ms.items():
         e = {"ms": round(ms, 4)}

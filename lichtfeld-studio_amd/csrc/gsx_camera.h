@@ -248,4 +248,42 @@ GSX_HD void equirect_unproject(float W, float H, float px, float py, vec3* ray) 
     ray->x = dx / len, ray->y = dy / len, ray->z = dz / len;
 }
 
+// ---- unscented transform through a perfect pinhole under one rigid pose (the training camera) ----
+// The reference rotates each of the seven world-space sigma points by the pose's quaternion and divides twice per
+// point (Cameras.cuh:1070-1119, 362-369, 431-455).  The same points, formed where they are used: the mean goes
+// through the pose once, each of the three scaled axes through its rotation matrix once, and the points are
+// mean_c +- axis_c; the perspective division is one reciprocal per point.  Mathematically the same map (rotation is
+// linear), ~40 % of the instructions; pinned by the float64 unscented-transform model of
+// tests/test_oracle_geometry.py, shared by the kernels and the CPU checker.
+//   Rc, t : rotation matrix and translation of the pose;  Rg : rotation matrix of the Gaussian (mat3_cast);
+//   sq    : sqrt(3 + lambda);  out[0] = mean, out[1..3] = mean + axis, out[4..6] = mean - axis (camera coordinates)
+GSX_HD void ut_sigma_points_camera(const mat3& Rc, vec3 t, vec3 mean, const mat3& Rg, vec3 scl, float sq,
+                                   vec3 (&out)[7]) {
+    out[0] = add(mul(Rc, mean), t);
+    const float sc[3] = {scl.x, scl.y, scl.z};
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+#endif
+    for (int a = 0; a < 3; ++a) {
+        const float s = sq * sc[a];
+        const vec3 axis_c = mul(Rc, mk3(s * Rg.m[0][a], s * Rg.m[1][a], s * Rg.m[2][a]));
+        out[a + 1] = add(out[0], axis_c);
+        out[a + 4] = sub(out[0], axis_c);
+    }
+}
+
+// camera_ray_to_image_point of the perfect pinhole (Cameras.cuh:431-455) with one reciprocal: invalid behind the
+// camera, valid inside the image grown by margin_factor on every side
+GSX_HD bool pinhole_project_point(vec3 pc, float fx, float fy, float cx, float cy, float W, float H,
+                                  float margin_factor, vec2* out) {
+    out->x = 0.f;
+    out->y = 0.f;
+    if (pc.z <= 0.f)
+        return false;
+    const float iz = 1.0f / pc.z;
+    out->x = fma(pc.x * iz, fx, cx);
+    out->y = fma(pc.y * iz, fy, cy);
+    return in_image_margin(out->x, out->y, W, H, margin_factor);
+}
+
 } // namespace gsx

@@ -130,12 +130,17 @@ __device__ __forceinline__ bool project_world_point(const ProjCfg& cfg, const Ca
 }
 
 // GENERAL = false: the perfect pinhole with a global shutter (the training step's camera), decided at compile time
+// Rc: mat3_cast(cp.q_start), read by the GENERAL = false instance only (its sigma points go through the pose as a
+// matrix, gsx_camera.h ut_sigma_points_camera)
 template <bool GENERAL>
-__device__ __forceinline__ bool project_ut(const ProjCfg& cfg, const CamPose& cp, quat qc, vec3 tc, vec3 mean,
-                                           quat q_in, vec3 scl, bool has_opacity, float opacity_in, ProjOut* o) {
+__device__ __forceinline__ bool project_ut(const ProjCfg& cfg, const CamPose& cp, quat qc, vec3 tc, const mat3& Rc,
+                                           vec3 mean, quat q_in, vec3 scl, bool has_opacity, float opacity_in,
+                                           ProjOut* o) {
     // qc, tc: the centre-of-shutter pose shutter_pose(cp, 0.5) (ProjectionUT3DGSFused.cu:76-77)
     const quat q = quat_normalize(q_in);
-    const vec3 mean_c = add(quat_rotate(qc, mean), tc);
+    // one pose for the whole frame: the centre-of-shutter pose is the start pose, and the mean in camera coordinates
+    // is the first sigma point
+    const vec3 mean_c = GENERAL ? add(quat_rotate(qc, mean), tc) : add(mul(Rc, mean), cp.t_start);
     // the equirectangular model sees behind the camera (ProjectionUT3DGSFused.cu:78)
     if ((mean_c.z < cfg.near_plane && !(GENERAL && cfg.cam.type == 3)) || mean_c.z > cfg.far_plane)
         return false;
@@ -147,19 +152,28 @@ __device__ __forceinline__ bool project_ut(const ProjCfg& cfg, const CamPose& cp
     vec2 ip[7];
     vec2 m2 = {0.f, 0.f};
     bool valid = cfg.ut_require_all != 0;
+    vec3 pc[7]; // the sigma points in camera coordinates (perfect pinhole, one pose)
+    if (!GENERAL)
+        ut_sigma_points_camera(Rc, cp.t_start, mean, Rg, scl, sq, pc);
 #pragma unroll
     for (int i = 0; i < 7; ++i) {
-        vec3 p;
-        if (i == 0) {
-            p = mean;
-        } else {
-            const int a = (i - 1) % 3;
-            const float s = sq * sc[a];
-            const vec3 delta = mk3(s * Rg.m[0][a], s * Rg.m[1][a], s * Rg.m[2][a]);
-            p = (i <= 3) ? add(mean, delta) : sub(mean, delta);
-        }
         vec2 uv;
-        const bool pv = project_world_point<GENERAL>(cfg, cp, p, &uv);
+        bool pv;
+        if (GENERAL) {
+            vec3 p;
+            if (i == 0) {
+                p = mean;
+            } else {
+                const int a = (i - 1) % 3;
+                const float s = sq * sc[a];
+                const vec3 delta = mk3(s * Rg.m[0][a], s * Rg.m[1][a], s * Rg.m[2][a]);
+                p = (i <= 3) ? add(mean, delta) : sub(mean, delta);
+            }
+            pv = project_world_point<GENERAL>(cfg, cp, p, &uv);
+        } else {
+            pv = pinhole_project_point(pc[i], cfg.fx, cfg.fy, cfg.cx, cfg.cy, (float)cfg.W, (float)cfg.H,
+                                       cfg.ut_margin, &uv);
+        }
         if (cfg.ut_require_all) {
             valid &= pv;
             if (!pv)
@@ -223,6 +237,48 @@ __device__ __forceinline__ bool project_ut(const ProjCfg& cfg, const CamPose& cp
     return true;
 }
 
+// The pose of the one perfect-pinhole, global-shutter camera for a whole workgroup: the first wave derives it from
+// the view matrix (quaternion of its rotation, rotation matrix of that quaternion - a few hundred instructions whose
+// results are the same for every lane of the launch) and every lane reads it back from LDS.  Every thread of the
+// workgroup must call it.  Of `cp` only the start translation is set, and qc / tc are the identity: the plain
+// instance of project_ut reads nothing else.
+struct WorkgroupPose {
+    CamPose cp;
+    quat qc;
+    vec3 tc;
+    mat3 Rc;
+};
+__device__ __forceinline__ WorkgroupPose workgroup_pose(const float* __restrict__ viewmat) {
+    __shared__ float s[12];
+    if (threadIdx.x < 64u) {
+        const CamPose cp = load_cam_pose(viewmat);
+        const mat3 Rc = mat3_cast(cp.q_start);
+        if (threadIdx.x == 0) {
+            s[0] = cp.t_start.x, s[1] = cp.t_start.y, s[2] = cp.t_start.z;
+#pragma unroll
+            for (int r = 0; r < 3; ++r)
+#pragma unroll
+                for (int c = 0; c < 3; ++c)
+                    s[3 + 3 * r + c] = Rc.m[r][c];
+        }
+    }
+    __syncthreads();
+    WorkgroupPose p;
+    p.qc.w = 1.f, p.qc.x = 0.f, p.qc.y = 0.f, p.qc.z = 0.f;
+    p.tc = mk3(0.f, 0.f, 0.f);
+    p.cp.q_start = p.qc, p.cp.q_end = p.qc;
+    p.cp.t_start = mk3(s[0], s[1], s[2]);
+    p.cp.t_end = p.cp.t_start;
+    p.cp.rs_type = GSX_GLOBAL;
+    p.cp.W = 0, p.cp.H = 0;
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int c = 0; c < 3; ++c)
+            p.Rc.m[r][c] = s[3 + 3 * r + c];
+    return p;
+}
+
 // GENERAL = false: every camera a perfect pinhole with a global shutter (no coefficient rows, no end-of-frame pose)
 template <bool GENERAL>
 __global__ void __launch_bounds__(256) projection_ut_kernel(
@@ -234,6 +290,9 @@ __global__ void __launch_bounds__(256) projection_ut_kernel(
     int32_t* __restrict__ radii, float* __restrict__ means2d,
     float* __restrict__ depths, float* __restrict__ conics, float* __restrict__ compensations) {
     const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    WorkgroupPose wp;
+    if (!GENERAL)
+        wp = workgroup_pose(viewmats0); // one camera (check_camera_args)
     if (idx >= C * N)
         return;
     const uint32_t cid = idx / N, gid = idx % N;
@@ -248,15 +307,13 @@ __global__ void __launch_bounds__(256) projection_ut_kernel(
                                     thin_prism != nullptr ? thin_prism + cid * 4 : nullptr, cfg.fx, cfg.fy, cfg.cx,
                                     cfg.cy, cfg.W, cfg.H);
     }
-    const CamPose cp = GENERAL ? load_cam_pose(viewmats0 + cid * 16,
-                                               viewmats1 != nullptr ? viewmats1 + cid * 16 : nullptr, rs_type, cfg.W,
-                                               cfg.H)
-                               : load_cam_pose(viewmats0 + cid * 16);
     ProjOut o;
-    quat qc;
-    vec3 tc;
-    shutter_pose(cp, 0.5f, &qc, &tc);
-    const bool ok = project_ut<GENERAL>(cfg, cp, qc, tc, ld3(means, gid), ld4q(quats, gid), ld3(scales, gid), opacities != nullptr,
+    if (GENERAL) {
+        wp.cp = load_cam_pose(viewmats0 + cid * 16, viewmats1 != nullptr ? viewmats1 + cid * 16 : nullptr, rs_type,
+                              cfg.W, cfg.H);
+        shutter_pose(wp.cp, 0.5f, &wp.qc, &wp.tc);
+    }
+    const bool ok = project_ut<GENERAL>(cfg, wp.cp, wp.qc, wp.tc, wp.Rc, ld3(means, gid), ld4q(quats, gid), ld3(scales, gid), opacities != nullptr,
                                opacities != nullptr ? opacities[gid] : 0.f, &o);
     int2* r2 = reinterpret_cast<int2*>(radii);
     if (!ok) {
@@ -275,13 +332,15 @@ __global__ void __launch_bounds__(256) projection_ut_kernel(
 
 // activate_params + projection in one pass (C == 1): raw parameters in, activated parameters and the projection
 // outputs out - the same values as the two separate kernels.
-__global__ void __launch_bounds__(256) projection_ut_raw_kernel(
+// 512 lanes a workgroup: the pose costs one wave in eight its few hundred instructions
+__global__ void __launch_bounds__(512) projection_ut_raw_kernel(
     uint32_t N, const float* __restrict__ means, const float* __restrict__ opacity_raw,
     const float* __restrict__ scaling_raw, const float* __restrict__ rotation_raw,
     const float* __restrict__ viewmat, const float* __restrict__ Ks, ProjCfg cfg, float* __restrict__ opacities,
     float* __restrict__ scales, float* __restrict__ quats, int32_t* __restrict__ radii, float* __restrict__ means2d,
     float* __restrict__ depths, float* __restrict__ conics) {
-    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t idx = blockIdx.x * 512u + threadIdx.x;
+    const WorkgroupPose wp = workgroup_pose(viewmat);
     if (idx >= N)
         return;
     const Activated a = activate(opacity_raw[idx], ld3(scaling_raw, idx), ld4q(rotation_raw, idx));
@@ -294,12 +353,9 @@ __global__ void __launch_bounds__(256) projection_ut_raw_kernel(
     cfg.fy = Ks[4];
     cfg.cx = Ks[2];
     cfg.cy = Ks[5];
-    const CamPose cp = load_cam_pose(viewmat);
-    quat qc;
-    vec3 tc;
-    shutter_pose(cp, 0.5f, &qc, &tc);
     ProjOut o;
-    const bool ok = project_ut<false>(cfg, cp, qc, tc, ld3(means, idx), a.quat, a.scales, true, a.opacity, &o);
+    const bool ok = project_ut<false>(cfg, wp.cp, wp.qc, wp.tc, wp.Rc, ld3(means, idx), a.quat, a.scales, true,
+                                      a.opacity, &o);
     int2* r2 = reinterpret_cast<int2*>(radii);
     if (!ok) {
         r2[idx] = make_int2(0, 0);
@@ -817,6 +873,7 @@ __global__ void __launch_bounds__(256) project_sh_records_kernel(
     const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t ic = min(idx, N - 1);
+    const WorkgroupPose wp = workgroup_pose(viewmat);
     const vec3 mean = ld3(means, ic);
     const Activated a = activate(opacity_raw[ic], ld3(scaling_raw, ic), ld4q(rotation_raw, ic));
     bool live = false;
@@ -830,12 +887,8 @@ __global__ void __launch_bounds__(256) project_sh_records_kernel(
         cfg.fy = Ks[4];
         cfg.cx = Ks[2];
         cfg.cy = Ks[5];
-        const CamPose cp = load_cam_pose(viewmat);
-        quat qc;
-        vec3 tc;
-        shutter_pose(cp, 0.5f, &qc, &tc);
         ProjOut o;
-        live = project_ut<false>(cfg, cp, qc, tc, mean, a.quat, a.scales, true, a.opacity, &o);
+        live = project_ut<false>(cfg, wp.cp, wp.qc, wp.tc, wp.Rc, mean, a.quat, a.scales, true, a.opacity, &o);
         int2* r2 = reinterpret_cast<int2*>(radii);
         if (!live) {
             r2[idx] = make_int2(0, 0);
@@ -961,7 +1014,7 @@ extern "C" int gsx_activate_project_ut(uint32_t N, const float* means, const flo
     cfg.W = image_width, cfg.H = image_height;
     cfg.eps2d = eps2d, cfg.near_plane = near_plane, cfg.far_plane = far_plane, cfg.radius_clip = radius_clip;
     set_ut_constants(cfg, ut);
-    hipLaunchKernelGGL(projection_ut_raw_kernel, dim3(cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream, N, means,
+    hipLaunchKernelGGL(projection_ut_raw_kernel, dim3(cdiv(N, 512)), dim3(512), 0, (hipStream_t)stream, N, means,
                        opacity_raw, scaling_raw, rotation_raw, viewmat, K, cfg, opacities, scales, quats, radii,
                        means2d, depths, conics);
     GSX_LAUNCH_CHECK();

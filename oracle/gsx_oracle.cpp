@@ -350,9 +350,12 @@ ORC_API int orc_projection_ut_3dgs_fused(
         const float cx = Ks[cid * 9 + 2], cy = Ks[cid * 9 + 5];
         const RollingShutter rs = make_rolling_shutter(viewmats0 + cid * 16, nullptr);
 
-        // :76-82 centre-of-shutter pose, near/far cull
+        // :76-82 centre-of-shutter pose, near/far cull.  The trainer's camera (see `plain` below) has one pose for
+        // the whole frame: its mean in camera coordinates is the first sigma point, taken through the pose's matrix.
+        const bool plain = g_model == 0 && !g_dist.on && g_rs_type == 4 && !g_has_end_pose;
         const ShutterPose pose = interpolate_shutter_pose(0.5f, rs);
-        const vec3 mean_c = gsx::add(gsx::quat_rotate(pose.q, mean), pose.t);
+        const vec3 mean_c = plain ? gsx::add(gsx::mul(gsx::mat3_cast(rs.q_start), mean), rs.t_start)
+                                  : gsx::add(gsx::quat_rotate(pose.q, mean), pose.t);
         if ((mean_c.z < near_plane && g_model != 3) || mean_c.z > far_plane) { // :78
             radii[idx * 2] = 0;
             radii[idx * 2 + 1] = 0;
@@ -386,10 +389,20 @@ ORC_API int orc_projection_ut_3dgs_fused(
         bool culled = false;
         vec2 ip[7];
         vec2 m2 = {0.f, 0.f};
+        // The perfect pinhole under a global shutter (the trainer's camera) takes the sigma points through the start
+        // pose as a 3x3 matrix - R (mean +- s r_a) = R mean +- R (s r_a), so one product per axis serves two points -
+        // and projects with one reciprocal of z per point: the same real-valued function as the general route
+        // below, rounded differently (each image point within a few ulp).  The kernels take the same two helpers
+        // under the same condition.
+        vec3 pts_c[7];
+        if (plain)
+            gsx::ut_sigma_points_camera(gsx::mat3_cast(rs.q_start), rs.t_start, mean, Rg, scale, sq, pts_c);
         for (int i = 0; i < 7; ++i) {
             vec2 p;
-            const bool pv = project_world_point_shutter(pts[i], rs, fx, fy, cx, cy, image_width, image_height,
-                                                        ut_margin, &p);
+            const bool pv = plain ? gsx::pinhole_project_point(pts_c[i], fx, fy, cx, cy, (float)image_width,
+                                                               (float)image_height, ut_margin, &p)
+                                  : project_world_point_shutter(pts[i], rs, fx, fy, cx, cy, image_width,
+                                                                image_height, ut_margin, &p);
             if (ut_require_all) {
                 valid &= pv;
                 if (!pv) {

@@ -1081,7 +1081,7 @@ def test_opencv_distortion_fused_forward_backward(gsx, orc, cuda, which):
 
 def test_opencv_distortion_projection_and_errors(gsx, orc, cuda):
     """gsx_projection_ut_3dgs_fused with coefficients: radii / means2d / depths / conics bit-identical to the checker;
-    zero coefficients give the perfect pinhole's results; other camera models and rolling shutter stay unsupported"""
+    zero coefficients give the perfect pinhole's results up to rounding; other camera models and rolling shutter stay unsupported"""
     ops = gsx.ops
     sc, cam, h, d = _fused_inputs(gsx, cuda, 30000)
     ut = ops.UnscentedTransformParameters()
@@ -1099,10 +1099,22 @@ def test_opencv_distortion_projection_and_errors(gsx, orc, cuda):
     for k, name in ((1, "means2d"), (2, "depths"), (3, "conics")):
         bits_equal(N(got[k])[0][vis], ref[k][0][vis], name)
     zero = [torch.zeros_like(dev[k]) for k in ("radial", "tangential", "thin_prism")]
+    # All-zero coefficients describe the perfect pinhole, but take the general route (a quaternion rotation and a
+    # division per sigma point) where "no coefficients" takes the matrix route with one reciprocal: the same function,
+    # rounded differently.  The unscented weights (-99 for the centre, +16.7 for the six others at alpha = 0.1)
+    # amplify an ulp of an image point (4e-6 px at 60 px) a few hundred times in the mean and the covariance.
     a, b = call(*zero), call(None, None, None)
-    assert torch.equal(a[0], b[0])
-    vis = (b[0][0, :, 0] > 0)
-    assert torch.equal(a[1][0][vis], b[1][0][vis]) and torch.equal(a[3][0][vis], b[3][0][vis])
+    ra, rb = a[0][0].cpu().numpy().astype(np.int64), b[0][0].cpu().numpy().astype(np.int64)
+    assert np.abs(ra - rb).max() <= 1 and (ra != rb).any(axis=1).mean() < 2e-3
+    vis = (ra[:, 0] > 0) & (rb[:, 0] > 0)
+    ma, mb = N(a[1])[0][vis], N(b[1])[0][vis]
+    err = np.abs(ma - mb)  # pixels; an ulp of a sigma point's image is 1.5e-5 px at this image's width
+    assert err.max() < 0.03 and np.median(err) < 1e-3, (err.max(), np.median(err))
+    ca, cb = N(a[3])[0][vis].astype(np.float64), N(b[3])[0][vis].astype(np.float64)
+    scale = np.sqrt(np.abs(cb[:, [0]] * cb[:, [2]]))  # size of the conic (the off-diagonal may be near zero)
+    assert (np.abs(ca - cb) / scale).max() < 5e-3, (np.abs(ca - cb) / scale).max()
+    da, db = N(a[2])[0][vis], N(b[2])[0][vis]  # depths: a quaternion rotation against a matrix row
+    assert (np.abs(da - db) <= 4 * np.spacing(np.abs(db))).all()
     with pytest.raises(RuntimeError, match="PINHOLE, FISHEYE and EQUIRECTANGULAR are supported"):
         call(None, None, None, model=1)  # ORTHO
     with pytest.raises(RuntimeError, match="shutter type 7"):
