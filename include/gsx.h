@@ -235,8 +235,9 @@ GSX_API uint32_t* gsx_tile_lists_error(uint32_t N, int64_t capacity, uint32_t ti
                                        void* workspace);
 
 /* ---- a7: gsplat::rasterize_to_pixels_from_world_3dgs_fwd (Ops.h:100-129; ...3DGSFwd.cu:19-285) ----
- * colors [C,N,channels] (channels in {1,2,3,4,5,8,9,16,17,32}: Rasterization.cpp:106-128 up to 32; beyond that
- * GSX_ERR_UNSUPPORTED), opacities [C,N], backgrounds [C,channels] nullable,
+ * colors [C,N,channels] (channels in {1,2,3,4,5,8,9,16,17,32,33,64,65,128,129,256,257,512,513}, the counts of
+ * Rasterization.cpp:106-128; any other GSX_ERR_UNSUPPORTED; beyond 32 the rasterizers run once per 32 channels),
+ * opacities [C,N], backgrounds [C,channels] nullable,
  * masks u8 [C,Th,Tw] nullable, tile_offsets i32 [C,Th,Tw], flatten_ids i32 [n_isects]
  * -> render_colors [C,H,W,channels], render_alphas [C,H,W,1], last_ids i32 [C,H,W]. tile_size must be 16.
  *

@@ -304,10 +304,14 @@ __device__ __forceinline__ vec3 camera_ray_origin(const CamPose& cp) {
 // ---- tile geometry shared by the forward and backward rasterizers ----------------------------
 // One 256-lane workgroup per 16x16 tile; wave w owns the 8x8 pixel block (w & 1, w >> 1), lane l the pixel
 // (l >> 3, l & 7) of it: compact blocks keep a wave's pixels coherent (saturation, bounds rejection).
-// colour channel counts the rasterizers are instantiated for (gsplat/Rasterization.cpp:106-128 up to 32)
+// colour channel counts the rasterizers take (gsplat/Rasterization.cpp:106-128): up to 32 an instance each, beyond
+// that one instance that takes 32 channels per launch, counted at run time
 static inline bool raster_channels_built(uint32_t c) {
-    return c == 1 || c == 2 || c == 3 || c == 4 || c == 5 || c == 8 || c == 9 || c == 16 || c == 17 || c == 32;
+    return c == 1 || c == 2 || c == 3 || c == 4 || c == 5 || c == 8 || c == 9 || c == 16 || c == 17 || c == 32 ||
+           c == 33 || c == 64 || c == 65 || c == 128 || c == 129 || c == 256 || c == 257 || c == 512 || c == 513;
 }
+static constexpr const char* kRasterChannelsText =
+    "supported: 1, 2, 3, 4, 5, 8, 9, 16, 17, 32, 33, 64, 65, 128, 129, 256, 257, 512, 513";
 static constexpr uint32_t kTile = 16;
 // what (uint32_t)GSX_COUNT_IN_OFFSETS is inside the kernels
 static constexpr uint32_t kCountInOffsets = 0xFFFFFFFFu;

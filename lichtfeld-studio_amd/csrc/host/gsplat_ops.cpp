@@ -34,9 +34,10 @@ using gsplat::OptT;
 
 inline void* cur_stream(const at::Tensor& t) { return (void*)c10::hip::getCurrentHIPStream(t.device().index()).stream(); }
 
-// the channel counts the rasterizers are built for (Rasterization.cpp:106-128 lists up to 513)
+// the channel counts the rasterizers take (Rasterization.cpp:106-128)
 inline bool channels_built(uint32_t c) {
-    return c == 1 || c == 2 || c == 3 || c == 4 || c == 5 || c == 8 || c == 9 || c == 16 || c == 17 || c == 32;
+    return c == 1 || c == 2 || c == 3 || c == 4 || c == 5 || c == 8 || c == 9 || c == 16 || c == 17 || c == 32 ||
+           c == 33 || c == 64 || c == 65 || c == 128 || c == 129 || c == 256 || c == 257 || c == 512 || c == 513;
 }
 inline void gsx_check(int status) { TORCH_CHECK(status == GSX_OK, "gsx (", gsx_status_string(status), "): ", gsx_last_error()); }
 

@@ -62,7 +62,10 @@ __global__ void __launch_bounds__(64) wave_reduce_probe_kernel(const float* __re
 // [N, CDIM - 3].
 // STATS: count instead of differentiating (for roofline accounting): stats[0] += pairs whose alpha is evaluated,
 // [1] += valid pairs, [2] += (wave, Gaussian) iterations executed.
-template <uint32_t CDIM, bool DIST, bool STATS = false>
+// WIDE: more than 32 channels, CDIM (= 32) of them per launch: channels [c0, c0 + nc) of rows `stride` floats long,
+// every one read from `colors`.  Every sum of a row is linear in the image gradient, so each launch adds the share
+// of its own channels (the launch with c0 = 0 also that of the alpha gradient) to the same accumulators.
+template <uint32_t CDIM, bool DIST, bool STATS = false, bool WIDE = false>
 __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     uint32_t n_isects, const float4* __restrict__ records, const float* __restrict__ colors,
     const float* __restrict__ backgrounds,
@@ -75,10 +78,13 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     const float* __restrict__ render_alphas, const int32_t* __restrict__ last_ids,
     const float* __restrict__ v_render_colors, const float* __restrict__ v_render_alphas,
     float* __restrict__ gacc /*[N,16]*/, float* __restrict__ gextra /*[N, CDIM - 3]*/,
-    unsigned long long* __restrict__ stats = nullptr) {
-    constexpr uint32_t NC = CDIM < 3 ? CDIM : 3; // channels carried by the record
+    unsigned long long* __restrict__ stats = nullptr, uint32_t stride = CDIM, uint32_t c0 = 0, uint32_t nc = CDIM) {
+    static_assert(!WIDE || (CDIM == 32 && !STATS), "the wide instance takes 32 channels a launch");
+    if (!WIDE)
+        stride = CDIM, c0 = 0, nc = CDIM;
+    constexpr uint32_t NC = WIDE ? 0 : (CDIM < 3 ? CDIM : 3); // channels carried by the record
     __shared__ float4 stage[kBwdBatch * 4];
-    constexpr uint32_t NX = CDIM > 3 ? CDIM - 3 : 0; // channels beyond the record's three
+    constexpr uint32_t NX = CDIM - NC; // channels read from `colors`: those beyond the record's three (WIDE: all)
     // up to six of them are staged and accumulated in LDS; beyond that (16 channels and more: not a training path)
     // their colours are read from memory in the loop and every wave adds its sums to memory itself
     constexpr bool XLDS = NX > 0 && NX <= 6;
@@ -133,13 +139,14 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     float v_render_c[CDIM];
 #pragma unroll
     for (uint32_t k = 0; k < CDIM; ++k)
-        v_render_c[k] = STATS ? 0.f : v_render_colors[(size_t)pix_id * CDIM + k];
-    const float v_render_a = STATS ? 0.f : v_render_alphas[pix_id];
+        v_render_c[k] = (STATS || k >= nc) ? 0.f : v_render_colors[(size_t)pix_id * stride + c0 + k];
+    const float v_render_a = (STATS || c0 != 0) ? 0.f : v_render_alphas[pix_id];
     float bg_dot = 0.f;
     if (backgrounds != nullptr) {
 #pragma unroll
         for (uint32_t k = 0; k < CDIM; ++k)
-            bg_dot += backgrounds[k] * v_render_c[k];
+            if (k < nc)
+                bg_dot += backgrounds[c0 + k] * v_render_c[k];
     }
     // what ra multiplies in v_alpha: T_final (v_render_a - bg . v_render) (:313-321) minus sum_k buffer_k v_render_k
     // (:186, :309), which starts at zero and is updated in the loop
@@ -186,7 +193,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             if ((int32_t)tr < batch_size) {
 #pragma unroll
                 for (uint32_t k = 0; k < NX; ++k)
-                    extra[tr * (NX ? NX : 1) + k] = colors[(size_t)id_batch[tr] * CDIM + 3 + k];
+                    extra[tr * (NX ? NX : 1) + k] = colors[(size_t)id_batch[tr] * stride + NC + k];
             }
             __syncthreads();
         }
@@ -250,7 +257,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             T *= ra;
             const float fac = valid ? alpha * T : 0.f;
             const float col[3] = {m2.y, m2.z, m2.w};
-            v[0] = fac * v_render_c[0];
+            v[0] = NC > 0 ? fac * v_render_c[0] : 0.f;
             v[1] = NC > 1 ? fac * v_render_c[NC > 1 ? 1 : 0] : 0.f;
             v[2] = NC > 2 ? fac * v_render_c[NC > 2 ? 2 : 0] : 0.f;
             // The derivative chain is written with fused multiply-adds (the compiler does not contract on its own
@@ -260,15 +267,17 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             // v_render_k and bdot = sum_k buffer_k v_render_k; buffer_k grows by c_k fac per Gaussian (:343), so bdot
             // grows by cdot fac.  `behind` = T_final (v_render_a - bg . v_render) - bdot collects everything ra
             // multiplies (:313-321): one running scalar per pixel instead of one per channel.
-            float cdot = col[0] * v_render_c[0];
+            float cdot = NC > 0 ? col[0] * v_render_c[0] : 0.f;
 #pragma unroll
             for (uint32_t k = 1; k < NC; ++k)
                 cdot = fma(col[k], v_render_c[k], cdot);
+            // (a row of `colors` is the same for the whole wave: the compiler reads it through the scalar path)
+            const float* const crow = NX > 0 && !XLDS ? colors + (size_t)id_batch[t] * stride + c0 + NC : nullptr;
 #pragma unroll
             for (uint32_t k = 0; k < NX; ++k)
-                cdot = fma(XLDS ? extra[(uint32_t)t * (NX ? NX : 1) + k]
-                                : colors[(size_t)id_batch[t] * CDIM + 3 + k],
-                           v_render_c[CDIM > 3 ? 3 + k : 0], cdot);
+                if (NC + k < nc)
+                    cdot = fma(XLDS ? extra[(uint32_t)t * (NX ? NX : 1) + k] : crow[k], v_render_c[NX ? NC + k : 0],
+                               cdot);
             const float v_alpha = fma(T, cdot, ra * behind);
             // the clamp at 0.999 has zero derivative (:322)
             const float v_opac = (valid && a.w * vis <= 0.999f) ? vis * v_alpha : 0.f;
@@ -300,15 +309,23 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             behind = fma(-cdot, fac, behind);
 #pragma unroll
             for (uint32_t k = 0; k < NX; ++k) { // the gradients of the channels beyond the third: their own wave sums
-                float e = fac * v_render_c[CDIM > 3 ? 3 + k : 0];
+                if (!(NC + k < nc))
+                    continue;
+                float e = fac * v_render_c[NX ? NC + k : 0];
 #pragma unroll
                 for (int m = 32; m >= 1; m >>= 1)
                     e += __shfl_xor(e, m, 64);
                 if (lane == 0) {
-                    if (XLDS)
+                    if (XLDS) {
                         atomicAdd(&acc_extra[(uint32_t)t * (NX ? NX : 1) + k], e);
-                    else if (e != 0.f)
-                        unsafeAtomicAdd(&gextra[(size_t)id_batch[t] * (NX ? NX : 1) + k], e);
+                    } else if (e != 0.f) {
+                        // channel c of the whole row: the first three live in the 16-float rows, the others in
+                        // gextra [N, stride - 3]
+                        const uint32_t c = c0 + NC + k;
+                        float* const at = (WIDE && c < 3u) ? &gacc[(size_t)id_batch[t] * kAcc + c]
+                                                           : &gextra[(size_t)id_batch[t] * (stride - 3u) + (c - 3u)];
+                        unsafeAtomicAdd(at, e);
+                    }
                 }
             }
             const float total = wave_reduce13(v, lane);
@@ -467,7 +484,7 @@ static int rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isects, co
                 GSX_ERR_INVALID_ARGUMENT, "rasterize bwd: null tensor");
     GSX_REQUIRE(((uintptr_t)records & 15) == 0, GSX_ERR_WORKSPACE, "rasterize bwd: records need 16-byte alignment");
     GSX_REQUIRE(raster_channels_built(channels), GSX_ERR_UNSUPPORTED,
-                "rasterize bwd: %u channels (built: 1, 2, 3, 4, 5, 8, 9, 16, 17, 32)", channels);
+                "rasterize bwd: %u channels (%s)", channels, kRasterChannelsText);
     GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 &&
                     workspace_bytes >= gsx_rasterize_bwd_accum_bytes_for(N, channels),
                 GSX_ERR_WORKSPACE, "rasterize bwd: accumulators need %zu bytes, 256-byte aligned",
@@ -498,7 +515,27 @@ static int rasterize_bwd_accumulate(uint32_t C, uint32_t N, int64_t n_isects, co
     case 9: GSX_LAUNCH_BWD2(9); break;
     case 16: GSX_LAUNCH_BWD2(16); break;
     case 17: GSX_LAUNCH_BWD2(17); break;
-    default: GSX_LAUNCH_BWD2(32); break;
+    case 32: GSX_LAUNCH_BWD2(32); break;
+    default:
+        // 33 ... 513 channels: 32 of them per launch, counted at run time
+        for (uint32_t c0 = 0; c0 < channels; c0 += 32) {
+            const uint32_t nc = channels - c0 < 32u ? channels - c0 : 32u;
+            if (distorted)
+                hipLaunchKernelGGL((rasterize_bwd_kernel<32, true, false, true>), dim3(tw * th), dim3(256), 0,
+                                   (hipStream_t)stream, (uint32_t)n_isects, (const float4*)records, colors, backgrounds,
+                                   masks, image_width, image_height, tw, th, viewmats0, Ks, camera_model, radial,
+                                   tangential, thin_prism, viewmats1, rs_type, tile_offsets, tile_order, flatten_ids,
+                                   render_alphas, last_ids, v_render_colors, v_render_alphas, (float*)workspace, gextra,
+                                   (unsigned long long*)nullptr, channels, c0, nc);
+            else
+                hipLaunchKernelGGL((rasterize_bwd_kernel<32, false, false, true>), dim3(tw * th), dim3(256), 0,
+                                   (hipStream_t)stream, (uint32_t)n_isects, (const float4*)records, colors, backgrounds,
+                                   masks, image_width, image_height, tw, th, viewmats0, Ks, camera_model, radial,
+                                   tangential, thin_prism, viewmats1, rs_type, tile_offsets, tile_order, flatten_ids,
+                                   render_alphas, last_ids, v_render_colors, v_render_alphas, (float*)workspace, gextra,
+                                   (unsigned long long*)nullptr, channels, c0, nc);
+        }
+        break;
     }
 #undef GSX_LAUNCH_BWD2
 #undef GSX_LAUNCH_BWD
@@ -559,7 +596,7 @@ extern "C" int gsx_rasterize_bwd_finish(uint32_t N, const float* means, const fl
     GSX_REQUIRE(means && quats && scales && viewmats0 && v_means && v_quats && v_scales && v_colors && v_opacities,
                 GSX_ERR_INVALID_ARGUMENT, "rasterize bwd: null tensor");
     GSX_REQUIRE(raster_channels_built(channels), GSX_ERR_UNSUPPORTED,
-                "rasterize bwd: %u channels (built: 1, 2, 3, 4, 5, 8, 9, 16, 17, 32)", channels);
+                "rasterize bwd: %u channels (%s)", channels, kRasterChannelsText);
     GSX_REQUIRE(workspace != nullptr && workspace_bytes >= gsx_rasterize_bwd_accum_bytes_for(N, channels),
                 GSX_ERR_WORKSPACE, "rasterize bwd: accumulators need %zu bytes",
                 gsx_rasterize_bwd_accum_bytes_for(N, channels));
@@ -587,7 +624,7 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
     if (N == 0)
         return GSX_OK;
     GSX_REQUIRE(raster_channels_built(channels), GSX_ERR_UNSUPPORTED,
-                "rasterize bwd: %u channels (built: 1, 2, 3, 4, 5, 8, 9, 16, 17, 32)", channels);
+                "rasterize bwd: %u channels (%s)", channels, kRasterChannelsText);
     GSX_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0 &&
                     workspace_bytes >= gsx_rasterize_bwd_workspace_bytes_for(N, channels),
                 GSX_ERR_WORKSPACE, "rasterize bwd: workspace needs %zu bytes, 256-byte aligned",

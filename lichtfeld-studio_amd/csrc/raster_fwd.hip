@@ -53,7 +53,11 @@ __global__ void __launch_bounds__(256) pack_records_kernel(uint32_t N, uint32_t 
 // DIST: any camera but the perfect pinhole with a global shutter - OpenCV distortion, fisheye, equirectangular,
 // rolling shutter (each pixel's ray comes from the model's unprojection under the pose of its exposure time; a pixel
 // without a valid ray is done from the start, RasterizeToPixelsFromWorld3DGSFwd.cu:145).
-template <uint32_t CDIM, bool STATS, bool DIST>
+// WIDE: more than 32 channels, CDIM (= 32) of them per launch: channels [c0, c0 + nc) of rows `stride` floats long,
+// every one of them read from `colors` (the records' three colours are channels 0-2 of the whole row and are not
+// used).  Each launch walks the lists again with the same arithmetic, so a pixel's weights, and with them every
+// channel's sum, do not depend on the split; the launch with c0 = 0 writes alphas and last ids.
+template <uint32_t CDIM, bool STATS, bool DIST, bool WIDE = false>
 __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
     uint32_t n_isects, const float4* __restrict__ records, const float* __restrict__ colors,
     const float* __restrict__ backgrounds, const uint8_t* __restrict__ masks, uint32_t image_width,
@@ -64,13 +68,18 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
     const int32_t* __restrict__ flatten_ids, const uint32_t* __restrict__ tile_order /*nullable*/,
     uint32_t* __restrict__ tile_walk /*nullable*/, float* __restrict__ render_colors,
     float* __restrict__ render_alphas,
-    int32_t* __restrict__ last_ids, unsigned long long* __restrict__ stats) {
+    int32_t* __restrict__ last_ids, unsigned long long* __restrict__ stats, uint32_t stride = CDIM, uint32_t c0 = 0,
+    uint32_t nc = CDIM) {
+    static_assert(!WIDE || (CDIM == 32 && !STATS), "the wide instance takes 32 channels a launch");
+    constexpr uint32_t NX = WIDE ? CDIM : (CDIM > 3 ? CDIM - 3 : 0); // channels staged from `colors`
+    if (!WIDE)
+        stride = CDIM, c0 = 0, nc = CDIM;
     __shared__ float4 stage[kFwdBatch * 4];
     __shared__ float4 region[kFwdBatch * 2];
     __shared__ float cuts[kFwdBatch];
     __shared__ uint8_t lists[4][kFwdBatch];
-    __shared__ int32_t ids[CDIM > 3 ? kFwdBatch : 1];
-    __shared__ float extra[CDIM > 3 ? kFwdBatch * (CDIM - 3) : 1]; // channels beyond the third
+    __shared__ int32_t ids[NX ? kFwdBatch : 1];
+    __shared__ float extra[NX ? kFwdBatch * NX : 1]; // channels beyond the third (WIDE: all of the launch's)
 
     const uint32_t tile_id = tile_order != nullptr ? tile_order[blockIdx.x] : blockIdx.x;
     const uint32_t tr = threadIdx.x;
@@ -85,7 +94,8 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
         if (inside && !STATS) {
 #pragma unroll
             for (uint32_t k = 0; k < CDIM; ++k)
-                render_colors[(size_t)pix_id * CDIM + k] = backgrounds == nullptr ? 0.0f : backgrounds[k];
+                if (k < nc)
+                    render_colors[(size_t)pix_id * stride + c0 + k] = backgrounds == nullptr ? 0.0f : backgrounds[c0 + k];
         }
         if (tile_walk != nullptr && tr == 0 && !STATS)
             tile_walk[tile_id] = 0u; // a masked tile costs nothing
@@ -128,13 +138,14 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
         const uint32_t batch_size = min(kFwdBatch, (uint32_t)range_end - batch_start);
         const bool wave_active = __builtin_amdgcn_ballot_w64(!done) != 0;
         const uint32_t n_sel = stage_and_select<kFwdBatch>(records, flatten_ids, (int32_t)batch_start, 1, batch_size, tr, px, 0u,
-                                                wave_active, stage, region, cuts, CDIM > 3 ? ids : nullptr,
+                                                wave_active, stage, region, cuts, NX > 0 ? ids : nullptr,
                                                 wave_list);
-        if (CDIM > 3) {
+        if (NX > 0) {
             if (tr < batch_size) {
+                const float* row = colors + (size_t)ids[tr] * stride + c0;
 #pragma unroll
-                for (uint32_t k = 3; k < CDIM; ++k)
-                    extra[tr * (CDIM > 3 ? CDIM - 3 : 1) + (k - 3)] = colors[(size_t)ids[tr] * CDIM + k];
+                for (uint32_t k = CDIM - NX; k < CDIM; ++k)
+                    extra[tr * (NX ? NX : 1) + (k - (CDIM - NX))] = k < nc ? row[k] : 0.f;
             }
             __syncthreads();
         }
@@ -196,14 +207,16 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
                 continue;
             }
             const float vis = alpha * T;
-            pix_out[0] = fma(m2.y, vis, pix_out[0]);
-            if (CDIM > 1)
-                pix_out[1] = fma(m2.z, vis, pix_out[1]);
-            if (CDIM > 2)
-                pix_out[2] = fma(m2.w, vis, pix_out[2]);
+            if (!WIDE) {
+                pix_out[0] = fma(m2.y, vis, pix_out[0]);
+                if (CDIM > 1)
+                    pix_out[1] = fma(m2.z, vis, pix_out[1]);
+                if (CDIM > 2)
+                    pix_out[2] = fma(m2.w, vis, pix_out[2]);
+            }
 #pragma unroll
-            for (uint32_t k = 3; k < CDIM; ++k)
-                pix_out[k] = fma(extra[t * (CDIM > 3 ? CDIM - 3 : 1) + (k - 3)], vis, pix_out[k]);
+            for (uint32_t k = CDIM - NX; k < CDIM; ++k)
+                pix_out[k] = fma(extra[t * (NX ? NX : 1) + (k - (CDIM - NX))], vis, pix_out[k]);
             cur_idx = batch_start + t;
             T = next_T;
             if (STATS)
@@ -228,12 +241,15 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
     }
 
     if (inside) {
-        render_alphas[pix_id] = 1.0f - T;
+        if (c0 == 0) {
+            render_alphas[pix_id] = 1.0f - T;
+            last_ids[pix_id] = (int32_t)cur_idx;
+        }
 #pragma unroll
         for (uint32_t k = 0; k < CDIM; ++k)
-            render_colors[(size_t)pix_id * CDIM + k] =
-                backgrounds == nullptr ? pix_out[k] : fma(T, backgrounds[k], pix_out[k]);
-        last_ids[pix_id] = (int32_t)cur_idx;
+            if (k < nc)
+                render_colors[(size_t)pix_id * stride + c0 + k] =
+                    backgrounds == nullptr ? pix_out[k] : fma(T, backgrounds[c0 + k], pix_out[k]);
     }
     if (tile_walk != nullptr) {
         // how far into its list this tile's pixels went (entries up to the last contributor): what the tile costs
@@ -274,7 +290,7 @@ int pack_raster_records(uint32_t N, const float* means, const float* quats, cons
     const dim3 grid(cdiv(N, 256)), block(256);
     hipStream_t s = (hipStream_t)stream;
     GSX_REQUIRE(raster_channels_built(channels), GSX_ERR_UNSUPPORTED,
-                "pack_raster_records: %u channels (built: 1, 2, 3, 4, 5, 8, 9, 16, 17, 32)", channels);
+                "pack_raster_records: %u channels (%s)", channels, kRasterChannelsText);
     hipLaunchKernelGGL(pack_records_kernel, grid, block, 0, s, N, channels, means, quats, scales, opacities, colors,
                        viewmat, K, image_width, image_height, pinhole, rolling, (float4*)records);
     GSX_LAUNCH_CHECK();
@@ -324,8 +340,28 @@ int rasterize_records_fwd(int64_t n_isects, const void* records, const float* co
     case 17: GSX_LAUNCH_FWD2(17); break;
     case 32: GSX_LAUNCH_FWD2(32); break;
     default:
-        set_error("rasterize fwd: %u channels (built: 1, 2, 3, 4, 5, 8, 9, 16, 17, 32)", channels);
-        return GSX_ERR_UNSUPPORTED;
+        if (!raster_channels_built(channels)) {
+            set_error("rasterize fwd: %u channels (%s)", channels, kRasterChannelsText);
+            return GSX_ERR_UNSUPPORTED;
+        }
+        // 33 ... 513 channels: 32 of them per launch, counted at run time
+        for (uint32_t c0 = 0; c0 < channels; c0 += 32) {
+            const uint32_t nc = channels - c0 < 32u ? channels - c0 : 32u;
+            uint32_t* const walk = c0 == 0 ? tile_walk : nullptr;
+            if (distorted)
+                hipLaunchKernelGGL((rasterize_fwd_kernel<32, false, true, true>), grid, block, 0, s, (uint32_t)n_isects,
+                                   (const float4*)records, colors, backgrounds, masks, image_width, image_height, tw,
+                                   th, viewmat, K, camera_model, radial, tangential, thin_prism, viewmat1, rs_type,
+                                   tile_offsets, flatten_ids, tile_order, walk, render_colors, render_alphas, last_ids,
+                                   (unsigned long long*)nullptr, channels, c0, nc);
+            else
+                hipLaunchKernelGGL((rasterize_fwd_kernel<32, false, false, true>), grid, block, 0, s,
+                                   (uint32_t)n_isects, (const float4*)records, colors, backgrounds, masks, image_width,
+                                   image_height, tw, th, viewmat, K, camera_model, radial, tangential, thin_prism,
+                                   viewmat1, rs_type, tile_offsets, flatten_ids, tile_order, walk, render_colors,
+                                   render_alphas, last_ids, (unsigned long long*)nullptr, channels, c0, nc);
+        }
+        break;
     }
 #undef GSX_LAUNCH_FWD2
 #undef GSX_LAUNCH_FWD
@@ -370,7 +406,7 @@ extern "C" int gsx_rasterize_to_pixels_from_world_3dgs_fwd(
         return GSX_OK;
     GSX_REQUIRE(tile_size == kTile, GSX_ERR_UNSUPPORTED, "rasterize fwd: tile_size %u (only 16 is built)", tile_size);
     GSX_REQUIRE(raster_channels_built(channels), GSX_ERR_UNSUPPORTED,
-                "rasterize fwd: %u channels (built: 1, 2, 3, 4, 5, 8, 9, 16, 17, 32)", channels);
+                "rasterize fwd: %u channels (%s)", channels, kRasterChannelsText);
     GSX_REQUIRE(viewmats0 && Ks, GSX_ERR_INVALID_ARGUMENT, "rasterize fwd: null tensor");
     GSX_REQUIRE(n_isects == 0 || (means && quats && scales && colors && opacities && flatten_ids),
                 GSX_ERR_INVALID_ARGUMENT, "rasterize fwd: null Gaussian tensor");

@@ -317,7 +317,7 @@ def projection_ut_3dgs_fused(means, quats, scales, opacities, viewmats0, viewmat
 
 
 # colour channel counts the rasterizers are built for (gsplat/Rasterization.cpp:106-128 lists up to 513)
-RASTER_CHANNELS = (1, 2, 3, 4, 5, 8, 9, 16, 17, 32)
+RASTER_CHANNELS = (1, 2, 3, 4, 5, 8, 9, 16, 17, 32, 33, 64, 65, 128, 129, 256, 257, 512, 513)
 
 
 def _fit_backgrounds(backgrounds, channels):

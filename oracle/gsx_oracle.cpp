@@ -867,7 +867,7 @@ ORC_API int orc_rasterize_to_pixels_from_world_3dgs_fwd(
     const uint8_t* masks /*nullable*/, uint32_t image_width, uint32_t image_height, uint32_t tile_size,
     const float* viewmats0, const float* Ks, const int32_t* tile_offsets, const int32_t* flatten_ids,
     float* render_colors, float* render_alphas, int32_t* last_ids, int64_t* pairs_evaluated) {
-    if (C != 1 || CDIM > 64)
+    if (C != 1 || CDIM > 513)
         return -2;
     (void)N;
     const uint32_t tile_width = (image_width + tile_size - 1) / tile_size;
@@ -904,7 +904,7 @@ ORC_API int orc_rasterize_to_pixels_from_world_3dgs_fwd(
                     pixel_world_ray((float)j + 0.5f, (float)i + 0.5f, fx, fy, cx, cy, rs, &ray_o, &ray_d);
                 float T = 1.0f;
                 uint32_t cur_idx = 0;
-                float pix_out[64] = {};
+                float pix_out[513] = {};
                 // a pixel without a valid ray is done from the start (RasterizeToPixelsFromWorld3DGSFwd.cu:145)
                 for (int32_t t = 0; t < (ray_ok ? cnt : 0); ++t) {
                     ++pairs;
@@ -956,7 +956,7 @@ ORC_API int orc_rasterize_to_pixels_from_world_3dgs_bwd(
     const float* render_alphas, const int32_t* last_ids, const float* v_render_colors,
     const float* v_render_alphas, float* v_means, float* v_quats, float* v_scales, float* v_colors,
     float* v_opacities) {
-    constexpr uint32_t kMaxC = 64;
+    constexpr uint32_t kMaxC = 513; // Rasterization.cpp:106-128
     if (C != 1 || CDIM < 1 || CDIM > kMaxC)
         return -2;
     const size_t kRow = 11 + CDIM; // mean 3, quat 4, scale 3, opacity 1, then the colour channels

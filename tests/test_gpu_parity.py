@@ -963,10 +963,11 @@ def test_depth_render_modes(gsx, orc, cuda, render_mode):
     assert np.abs(oc[..., -1]).max() > 0
 
 
-@pytest.mark.parametrize("channels", [2, 5, 8, 9, 16, 17, 32])
+@pytest.mark.parametrize("channels", [2, 5, 8, 9, 16, 17, 32, 33, 64, 65, 129, 513])
 def test_rasterizer_channel_counts(gsx, orc, cuda, channels):
-    """the colour-channel counts of Rasterization.cpp:106-128 beyond LichtFeld's own 1 / 3 / 4 (up to 32): forward
-    bit-identical to the checker, the gradient of every channel and of the geometry within the bars"""
+    """the colour-channel counts of Rasterization.cpp:106-128 beyond LichtFeld's own 1 / 3 / 4 (beyond 32 channels
+    the rasterizers take 32 per launch, counted at run time): forward bit-identical to the checker, the gradient of
+    every channel and of the geometry within the bars"""
     ops = gsx.ops
     sc, cam, h, d = _fused_inputs(gsx, cuda, 3000)
     ut = ops.UnscentedTransformParameters()
