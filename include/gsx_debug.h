@@ -29,6 +29,10 @@ GSX_API int gsx_debug_wave_reduce(uint32_t values, uint32_t n_waves, const float
  * inside the buffers, every kernel ending normally) can be exercised without making anything wait.  Process-wide. */
 GSX_API int gsx_debug_set_lookback_spin_limit(int64_t limit);
 
+/* Tuning hook: output rows per strip of the SSIM / photometric-loss kernels (0 = chosen per image size).  The buffer
+ * sizes gsx_photometric_partials reports follow it: set it before anything is sized.  Process-wide. */
+GSX_API void gsx_debug_set_ssim_strip_rows(int rows);
+
 /* Pair counts of one forward pass, for turning kernel times into rates (no counterpart in the reference).
  * stats_out: device uint64[8] = {(pixel, Gaussian) pairs the forward evaluates, pairs composited, pairs the backward
  * walks, (wave, Gaussian) iterations executed, (wave, Gaussian) iterations removed by the pixel bounds, executed

@@ -3,18 +3,20 @@
 // (forward), :284-424 (backward); src/training/trainer.cpp:126-129, include/kernels/fused_ssim.cuh:59-67,84-96,117-122
 // (valid crop, mean), src/training/rasterization/rasterizer.cpp:205 (clamp).
 //
-// Organisation (gfx950).  A wave owns a strip of one image plane: 64 adjacent columns (one per lane) by 12 output
-// rows, and walks it top to bottom, one INPUT row per step (12 + 10 steps):
+// Organisation (gfx950).  A wave owns a strip of one image plane: 64 adjacent columns (one per lane) by r output
+// rows, and walks it top to bottom, one INPUT row per step (r + 10 steps; r is chosen per image so that the launch
+// fills the CUs evenly, see strip_rows - 17 at 1237 x 822, three workgroups on every CU):
 //   * the row's 64 + 10 values per image go through two wave-private LDS rows, from which every lane reads its
 //     eleven horizontal taps with unit stride across the lanes (no bank conflicts, no workgroup barrier: the four
 //     waves of a workgroup never talk to each other);
 //   * the horizontally filtered moments of the last eleven input rows stay in REGISTERS (a sliding window per lane);
 //     once the window is full every further input row completes one output row - the vertical filter reads no
 //     memory at all.  The row loop is unrolled eleven times, after which every window slot is back in the register
-//     it started in: the window slides without a single move (22 steps = two passes through the unrolled body);
+//     it started in: the window slides without a single move (the steps left over after the last full block of
+//     eleven run as a nest of conditions that the walk leaves where it ends);
 //   * input rows are requested from memory two steps before they are used, by unconditional loads whose results
 //     nothing touches until then.
-// A strip re-reads 10 halo rows per 12 and 10 halo columns per 64; the three colour planes of the interleaved render
+// A strip re-reads 10 halo rows per r and 10 halo columns per 64; the three colour planes of the interleaved render
 // are three waves of one workgroup, and the workgroups of one XCD cover one contiguous eighth of the image, so these
 // re-reads are served by that XCD's L2.
 // Each output applies the taps in the reference's order (symmetric pairs from the centre outwards, then the centre;
@@ -28,8 +30,10 @@ namespace gsx {
 
 static constexpr int HALO = 5;
 static constexpr int kStripCols = 64;  // one per lane
-static constexpr int kFwdRows = 12;    // output rows per strip: 12 + 10 input rows = 2 x 11 steps (23 rows per strip
-static constexpr int kBwdRows = 12;    // leave too few waves: measured 34 / 41 us against 33 / 32 us at 1237 x 822)
+// Output rows per strip are chosen per launch (strip_rows): a strip of r rows costs r + 10 steps, so taller strips
+// waste less on the halo, while the launch should fill every CU evenly and still leave each SIMD a few waves to hide
+// latencies behind.
+static constexpr int kMinRows = 12, kMaxRows = 56;
 static constexpr int kRowFloats = kStripCols + 2 * HALO + 6; // an LDS row, padded to 80 floats
 
 __constant__ float cGauss[11] = {0.001028380123898387f, 0.0075987582094967365f, 0.036000773310661316f,
@@ -41,6 +45,7 @@ __constant__ float cGauss[11] = {0.001028380123898387f, 0.0075987582094967365f, 
 struct Strip {
     int col0, row0; // first output column / row
     int H, W;
+    int rows;       // output rows of the strip
 };
 
 // The 74 columns an input row contributes to a strip: one value per lane for the columns col0 - 5 + lane and, in the
@@ -105,18 +110,42 @@ __device__ __forceinline__ void push_window(float (&win)[N][11], const float (&r
     }
 }
 
+// The row walk of a strip: `steps` calls of step(0), step(1), ...  Eleven at a time as straight-line code, after which
+// the window is back in the registers it started in (a step's shift of the window is a renaming there).  What is left
+// over (fewer than eleven steps) runs as a nest of conditions, each step inside the one before: the walk leaves from
+// wherever it ends and never rejoins, so no path has to move the window into place for another.
+template <int J, class Step>
+__device__ __forceinline__ void walk_tail(int it0, int left, const Step& step) {
+    if constexpr (J < 10) {
+        if (J < left) {
+            step(it0 + J);
+            walk_tail<J + 1>(it0, left, step);
+        }
+    }
+}
+template <class Step>
+__device__ __forceinline__ void walk_rows(int steps, const Step& step) {
+    int it0 = 0;
+    for (; it0 + 11 <= steps; it0 += 11) {
+#pragma unroll
+        for (int j = 0; j < 11; ++j)
+            step(it0 + j);
+    }
+    walk_tail<0>(it0, steps - it0, step);
+}
+
 // ---- forward -----------------------------------------------------------------------------------------------------
 // loadx / loady: loaders of the two images for this plane, (row, column) -> the value in memory; prepx: what turns a
 // loaded X value into the image value (the clamp of the training path).  Per output pixel `emit(row, col, ssim,
 // dmu1, dsigma1_sq, dsigma12)` is called (image pixels only); returns the lane's sum of |X - Y| over its output pixels.
 // lds: two rows of kRowFloats (X and Y of the current input row).
-template <int ROWS, class LoadX, class PrepX, class LoadY, class Emit>
+template <class LoadX, class PrepX, class LoadY, class Emit>
 __device__ __forceinline__ float ssim_forward_strip(const Strip& st, float C1, float C2, float* lds,
                                                     const LoadX& loadx, const PrepX& prepx, const LoadY& loady,
                                                     const Emit& emit) {
     const int lane = threadIdx.x & 63;
     const int col = st.col0 + lane;
-    const int row_end = min(st.row0 + ROWS, st.H); // one past the last output row
+    const int row_end = min(st.row0 + st.rows, st.H); // one past the last output row
     float* lds_x = lds;
     float* lds_y = lds + kRowFloats;
     float win[5][11];
@@ -133,9 +162,8 @@ __device__ __forceinline__ float ssim_forward_strip(const Strip& st, float C1, f
         xm[k] = loadx(q.row_c, q.col_m), xh[k] = loadx(q.row_c, q.col_h);
         ym[k] = loady(q.row_c, q.col_m), yh[k] = loady(q.row_c, q.col_h);
     }
-    static_assert((ROWS + 2 * HALO) % 11 == 0, "the window returns to its registers every eleven rows");
-#pragma unroll 11
-    for (int it = 0; it < ROWS + 2 * HALO; ++it) {
+    const int steps = st.rows + 2 * HALO;
+    auto step = [&](int it) __attribute__((always_inline)) {
         const int row = st.row0 - HALO + it;
         bool main_ok, halo_ok;
         row_valid(st, row, lane, &main_ok, &halo_ok);
@@ -192,7 +220,8 @@ __device__ __forceinline__ float ssim_forward_strip(const Strip& st, float C1, f
             emit(out_row, col, CD * r, fma(two_mu1 * CD, rrB - r * rA, ((mu2 + mu2) * (D_ - C_)) * r), -(CD * rrB),
                  (C_ + C_) * r);
         }
-    }
+    };
+    walk_rows(steps, step);
     return l1;
 }
 
@@ -200,12 +229,12 @@ __device__ __forceinline__ float ssim_forward_strip(const Strip& st, float C1, f
 // load4(row, col, v[4]): the three derivative maps at an image pixel as they lie in memory, and a fourth word for
 // the factor; factor(row, col, v[3]): d loss / d map there (ssim.cu:305-337 multiplies the two); emit(row, col, s0,
 // s1, s2): the three filtered sums of an output pixel (:385-421).
-template <int ROWS, class Load4, class Factor, class Emit>
+template <class Load4, class Factor, class Emit>
 __device__ __forceinline__ void ssim_backward_strip(const Strip& st, float* lds0, float* lds1, float* lds2,
                                                     const Load4& load4, const Factor& factor, const Emit& emit) {
     const int lane = threadIdx.x & 63;
     const int col = st.col0 + lane;
-    const int row_end = min(st.row0 + ROWS, st.H);
+    const int row_end = min(st.row0 + st.rows, st.H);
     float win[3][11];
 #pragma unroll
     for (int k = 0; k < 3; ++k)
@@ -222,9 +251,8 @@ __device__ __forceinline__ void ssim_backward_strip(const Strip& st, float* lds0
     float mv[4], hv[4], mv2[4], hv2[4]; // the next row to publish and the one after it
     request(st.row0 - HALO, mv, hv);
     request(st.row0 - HALO + 1, mv2, hv2);
-    static_assert((ROWS + 2 * HALO) % 11 == 0, "the window returns to its registers every eleven rows");
-#pragma unroll 11
-    for (int it = 0; it < ROWS + 2 * HALO; ++it) {
+    const int steps = st.rows + 2 * HALO;
+    auto step = [&](int it) __attribute__((always_inline)) {
         const int row = st.row0 - HALO + it;
         bool main_ok, halo_ok;
         row_valid(st, row, lane, &main_ok, &halo_ok);
@@ -258,7 +286,8 @@ __device__ __forceinline__ void ssim_backward_strip(const Strip& st, float* lds0
             filter_window(win, f);
             emit(out_row, col, f[0], f[1], f[2]);
         }
-    }
+    };
+    walk_rows(steps, step);
 }
 
 // the strip of wave `w` (over all waves of the launch): plane-major so that the planes of one strip are neighbours
@@ -270,6 +299,7 @@ __device__ __forceinline__ Strip strip_of(uint32_t w, int planes, int H, int W, 
     st.col0 = (int)(s % (uint32_t)strips_x) * kStripCols;
     st.row0 = (int)(s / (uint32_t)strips_x) * rows;
     st.H = H, st.W = W;
+    st.rows = rows;
     return st;
 }
 __host__ __device__ static inline uint32_t strip_count(uint32_t H, uint32_t W, uint32_t rows) {
@@ -284,21 +314,21 @@ __host__ __device__ static inline uint32_t xcd_grid(uint32_t n) { return 8u * ((
 __device__ __forceinline__ uint32_t xcd_block(uint32_t b, uint32_t n) { return (b & 7u) * ((n + 7u) / 8u) + (b >> 3); }
 
 // gsplat-style operator (include/kernels/ssim.cuh:11-19): img1 / img2 [planes,H,W] -> map and the derivative maps
-__global__ void __launch_bounds__(256) fusedssim_kernel(int planes, int H, int W, float C1, float C2,
+__global__ void __launch_bounds__(256) fusedssim_kernel(int rows_per_strip, int planes, int H, int W, float C1, float C2,
                                                          const float* __restrict__ img1,
                                                          const float* __restrict__ img2, float* __restrict__ ssim_map,
                                                          float* __restrict__ dm_dmu1,
                                                          float* __restrict__ dm_dsigma1_sq,
                                                          float* __restrict__ dm_dsigma12) {
     __shared__ float rows[4][2 * kRowFloats];
-    const uint32_t n_waves = strip_count(H, W, kFwdRows) * (uint32_t)planes;
+    const uint32_t n_waves = strip_count(H, W, rows_per_strip) * (uint32_t)planes;
     const uint32_t wave = threadIdx.x >> 6, w = xcd_block(blockIdx.x, (n_waves + 3u) / 4u) * 4u + wave;
     if (w >= n_waves)
         return;
     int plane;
-    const Strip st = strip_of(w, planes, H, W, kFwdRows, &plane);
+    const Strip st = strip_of(w, planes, H, W, rows_per_strip, &plane);
     const size_t base = (size_t)plane * H * W;
-    ssim_forward_strip<kFwdRows>(
+    ssim_forward_strip(
         st, C1, C2, rows[wave], [&](int y, int x) { return img1[base + (size_t)y * W + x]; },
         [](float v) { return v; }, [&](int y, int x) { return img2[base + (size_t)y * W + x]; },
         [&](int y, int x, float ssim, float dmu1, float ds1, float ds12) {
@@ -314,18 +344,18 @@ __global__ void __launch_bounds__(256) fusedssim_kernel(int planes, int H, int W
 
 // include/kernels/ssim.cuh:21-28 -> d loss / d img1
 __global__ void __launch_bounds__(256) fusedssim_backward_kernel(
-    int planes, int H, int W, const float* __restrict__ img1, const float* __restrict__ img2,
+    int rows_per_strip, int planes, int H, int W, const float* __restrict__ img1, const float* __restrict__ img2,
     const float* __restrict__ dL_dmap, const float* __restrict__ dm_dmu1, const float* __restrict__ dm_dsigma1_sq,
     const float* __restrict__ dm_dsigma12, float* __restrict__ dL_dimg1) {
     __shared__ float rows[4][3][kRowFloats];
-    const uint32_t n_waves = strip_count(H, W, kBwdRows) * (uint32_t)planes;
+    const uint32_t n_waves = strip_count(H, W, rows_per_strip) * (uint32_t)planes;
     const uint32_t wave = threadIdx.x >> 6, w = xcd_block(blockIdx.x, (n_waves + 3u) / 4u) * 4u + wave;
     if (w >= n_waves)
         return;
     int plane;
-    const Strip st = strip_of(w, planes, H, W, kBwdRows, &plane);
+    const Strip st = strip_of(w, planes, H, W, rows_per_strip, &plane);
     const size_t base = (size_t)plane * H * W;
-    ssim_backward_strip<kBwdRows>(
+    ssim_backward_strip(
         st, rows[wave][0], rows[wave][1], rows[wave][2],
         [&](int y, int x, float (&v)[4]) {
             const size_t gi = base + (size_t)y * W + x;
@@ -492,7 +522,7 @@ __global__ void __launch_bounds__(256) render_grad_from_loss_kernel(uint32_t HW,
 // forward: clamp + HWC -> CHW on load, SSIM moments and derivative maps, and per wave the sums of |image - gt| and of
 // the SSIM map over the valid crop (what image_from_render + fusedssim + ssim_valid_partials do in three passes; the
 // clamped image and the SSIM map themselves are never written).
-__global__ void __launch_bounds__(256) photometric_fwd_kernel(int H, int W, float C1, float C2,
+__global__ void __launch_bounds__(256) photometric_fwd_kernel(int rows_per_strip, int H, int W, float C1, float C2,
                                                                const float* __restrict__ render_hwc,
                                                                const float* __restrict__ gt_chw,
                                                                float* __restrict__ dm_dmu1,
@@ -501,16 +531,16 @@ __global__ void __launch_bounds__(256) photometric_fwd_kernel(int H, int W, floa
                                                                float* __restrict__ l1_partials,
                                                                float* __restrict__ ssim_partials) {
     __shared__ float rows[4][2 * kRowFloats];
-    const uint32_t n_waves = strip_count(H, W, kFwdRows) * 3u;
+    const uint32_t n_waves = strip_count(H, W, rows_per_strip) * 3u;
     const uint32_t wave = threadIdx.x >> 6, w = xcd_block(blockIdx.x, (n_waves + 3u) / 4u) * 4u + wave;
     if (w >= n_waves)
         return;
     int c;
-    const Strip st = strip_of(w, 3, H, W, kFwdRows, &c);
+    const Strip st = strip_of(w, 3, H, W, rows_per_strip, &c);
     const size_t base = (size_t)c * H * W;
     const bool crop = H > 10 && W > 10;
     float ss = 0.f;
-    float l1 = ssim_forward_strip<kFwdRows>(
+    float l1 = ssim_forward_strip(
         st, C1, C2, rows[wave],
         [&](int y, int x) { return render_hwc[((size_t)y * W + x) * 3 + c]; },
         [](float v) { return gsx::fmin(gsx::fmax(v, 0.0f), 1.0f); }, // rasterizer.cpp:205
@@ -537,7 +567,8 @@ __global__ void __launch_bounds__(256) photometric_fwd_kernel(int H, int W, floa
 // backward: d loss / d render in one pass - the SSIM chain with d loss / d map = -lambda / count inside the valid crop
 // formed on the fly (fused_ssim.cuh:84-96), the L1 sign term, the clamp VJP and the CHW -> HWC permute (what
 // fusedssim_backward + render_grad_from_loss do in two passes with two intermediate images).
-__global__ void __launch_bounds__(256) photometric_bwd_kernel(int H, int W, float ssim_scale, float l1_scale,
+__global__ void __launch_bounds__(256) photometric_bwd_kernel(int rows_per_strip, int H, int W, float ssim_scale,
+                                                               float l1_scale,
                                                                const float* __restrict__ render_hwc,
                                                                const float* __restrict__ gt_chw,
                                                                const float* __restrict__ dm_dmu1,
@@ -556,15 +587,15 @@ __global__ void __launch_bounds__(256) photometric_bwd_kernel(int H, int W, floa
         loss_from_partials(3u, (uint32_t)H, (uint32_t)W, lambda_dssim, l1_partials, ssim_partials, n_partials,
                            loss_out, lds);
     }
-    const uint32_t n_waves = strip_count(H, W, kBwdRows) * 3u;
+    const uint32_t n_waves = strip_count(H, W, rows_per_strip) * 3u;
     const uint32_t wave = threadIdx.x >> 6, w = xcd_block(blockIdx.x, (n_waves + 3u) / 4u) * 4u + wave;
     if (w >= n_waves)
         return;
     int c;
-    const Strip st = strip_of(w, 3, H, W, kBwdRows, &c);
+    const Strip st = strip_of(w, 3, H, W, rows_per_strip, &c);
     const size_t base = (size_t)c * H * W;
     const bool crop = H > 10 && W > 10;
-    ssim_backward_strip<kBwdRows>(
+    ssim_backward_strip(
         st, rows[wave][0], rows[wave][1], rows[wave][2],
         [&](int y, int x, float (&v)[4]) {
             const size_t gi = base + (size_t)y * W + x;
@@ -590,6 +621,37 @@ __global__ void __launch_bounds__(256) photometric_bwd_kernel(int H, int W, floa
 
 using namespace gsx;
 
+// Output rows per strip for an image of `planes` planes: the launch takes ceil(workgroups / CUs) rounds of r + 10
+// steps each on its fullest CU; among the heights that leave every CU at least three workgroups (three waves per
+// SIMD to hide latencies behind - below that the walk runs at the speed of its LDS and memory round trips) the
+// cheapest wins, the lowest on a tie.  Small images take the lowest strips.
+static int g_strip_rows = 0;
+extern "C" void gsx_debug_set_ssim_strip_rows(int rows) { g_strip_rows = rows; }
+static int strip_rows(uint32_t H, uint32_t W, uint32_t planes) {
+    if (g_strip_rows >= 1)
+        return g_strip_rows;
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        cus = n;
+    }
+    int best = kMinRows;
+    uint64_t best_cost = ~0ull;
+    for (int r = kMinRows; r <= kMaxRows; ++r) {
+        const uint64_t wgs = ((uint64_t)strip_count(H, W, (uint32_t)r) * planes + 3) / 4;
+        const uint64_t per_cu = (wgs + (uint64_t)cus - 1) / (uint64_t)cus;
+        if (per_cu < 3 && r > kMinRows)
+            break; // taller strips only thin the launch further
+        const uint64_t cost = per_cu * (uint64_t)(r + 2 * HALO);
+        if (cost < best_cost)
+            best_cost = cost, best = r;
+    }
+    return best;
+}
+
 extern "C" int gsx_fusedssim(int B, int CH, int H, int W, float C1, float C2, const float* img1, const float* img2,
                              float* ssim_map, float* dm_dmu1, float* dm_dsigma1_sq, float* dm_dsigma12,
                              void* stream) {
@@ -599,10 +661,11 @@ extern "C" int gsx_fusedssim(int B, int CH, int H, int W, float C1, float C2, co
     const bool train = dm_dmu1 != nullptr;
     GSX_REQUIRE(train == (dm_dsigma1_sq != nullptr) && train == (dm_dsigma12 != nullptr), GSX_ERR_INVALID_ARGUMENT,
                 "fusedssim: the three derivative maps must be given together");
-    GSX_REQUIRE((int64_t)B * CH * strip_count((uint32_t)H, (uint32_t)W, kBwdRows) < (1ll << 31),
+    GSX_REQUIRE((int64_t)B * CH * strip_count((uint32_t)H, (uint32_t)W, kMinRows) < (1ll << 31),
                 GSX_ERR_INVALID_ARGUMENT, "fusedssim: B*CH*H*W too large");
-    const uint32_t waves = strip_count((uint32_t)H, (uint32_t)W, kFwdRows) * (uint32_t)(B * CH);
-    hipLaunchKernelGGL(fusedssim_kernel, dim3(xcd_grid(cdiv(waves, 4))), dim3(256), 0, (hipStream_t)stream, B * CH, H, W, C1, C2,
+    const int rows = strip_rows((uint32_t)H, (uint32_t)W, (uint32_t)(B * CH));
+    const uint32_t waves = strip_count((uint32_t)H, (uint32_t)W, (uint32_t)rows) * (uint32_t)(B * CH);
+    hipLaunchKernelGGL(fusedssim_kernel, dim3(xcd_grid(cdiv(waves, 4))), dim3(256), 0, (hipStream_t)stream, rows, B * CH, H, W, C1, C2,
                        img1, img2, ssim_map, dm_dmu1, dm_dsigma1_sq, dm_dsigma12);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
@@ -618,10 +681,11 @@ extern "C" int gsx_fusedssim_backward(int B, int CH, int H, int W, float C1, flo
         return GSX_OK;
     GSX_REQUIRE(img1 && img2 && dL_dmap && dm_dmu1 && dm_dsigma1_sq && dm_dsigma12 && dL_dimg1,
                 GSX_ERR_INVALID_ARGUMENT, "fusedssim_backward: null tensor");
-    GSX_REQUIRE((int64_t)B * CH * strip_count((uint32_t)H, (uint32_t)W, kBwdRows) < (1ll << 31),
+    GSX_REQUIRE((int64_t)B * CH * strip_count((uint32_t)H, (uint32_t)W, kMinRows) < (1ll << 31),
                 GSX_ERR_INVALID_ARGUMENT, "fusedssim_backward: B*CH*H*W too large");
-    const uint32_t waves = strip_count((uint32_t)H, (uint32_t)W, kBwdRows) * (uint32_t)(B * CH);
-    hipLaunchKernelGGL(fusedssim_backward_kernel, dim3(xcd_grid(cdiv(waves, 4))), dim3(256), 0, (hipStream_t)stream, B * CH, H,
+    const int rows = strip_rows((uint32_t)H, (uint32_t)W, (uint32_t)(B * CH));
+    const uint32_t waves = strip_count((uint32_t)H, (uint32_t)W, (uint32_t)rows) * (uint32_t)(B * CH);
+    hipLaunchKernelGGL(fusedssim_backward_kernel, dim3(xcd_grid(cdiv(waves, 4))), dim3(256), 0, (hipStream_t)stream, rows, B * CH, H,
                        W, img1, img2, dL_dmap, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, dL_dimg1);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
@@ -692,7 +756,7 @@ extern "C" int gsx_render_grad_from_loss(uint32_t H, uint32_t W, float lambda_ds
 }
 
 extern "C" uint32_t gsx_photometric_partials(uint32_t H, uint32_t W) {
-    return 3u * strip_count(H, W, kFwdRows); // one pair of sums per wave
+    return 3u * strip_count(H, W, (uint32_t)strip_rows(H, W, 3)); // one pair of sums per wave
 }
 
 extern "C" int gsx_photometric_loss_forward(uint32_t H, uint32_t W, float C1, float C2, const float* render_hwc,
@@ -704,8 +768,9 @@ extern "C" int gsx_photometric_loss_forward(uint32_t H, uint32_t W, float C1, fl
     GSX_REQUIRE(render_hwc && gt_chw && dm_dmu1 && dm_dsigma1_sq && dm_dsigma12 && l1_partials && ssim_partials,
                 GSX_ERR_INVALID_ARGUMENT, "photometric_loss_forward: null tensor");
     GSX_REQUIRE((uint64_t)H * W < (1ull << 30), GSX_ERR_INVALID_ARGUMENT, "photometric_loss_forward: image too large");
-    hipLaunchKernelGGL(photometric_fwd_kernel, dim3(xcd_grid(cdiv(3u * strip_count(H, W, kFwdRows), 4))), dim3(256),
-                       0, (hipStream_t)stream, (int)H, (int)W, C1, C2,
+    const int rows = strip_rows(H, W, 3);
+    hipLaunchKernelGGL(photometric_fwd_kernel, dim3(xcd_grid(cdiv(3u * strip_count(H, W, (uint32_t)rows), 4))),
+                       dim3(256), 0, (hipStream_t)stream, rows, (int)H, (int)W, C1, C2,
                        render_hwc, gt_chw, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, l1_partials, ssim_partials);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
@@ -725,8 +790,9 @@ static int photometric_backward(uint32_t H, uint32_t W, float lambda_dssim, cons
     const float count = crop ? 3.f * (float)(H - 10) * (float)(W - 10) : 3.f * (float)H * (float)W;
     const float ssim_scale = -lambda_dssim / count;
     const float l1_scale = (1.f - lambda_dssim) / (3.f * (float)H * (float)W);
-    hipLaunchKernelGGL(photometric_bwd_kernel, dim3(xcd_grid(cdiv(3u * strip_count(H, W, kBwdRows), 4))), dim3(256),
-                       0, (hipStream_t)stream, (int)H, (int)W, ssim_scale,
+    const int rows = strip_rows(H, W, 3);
+    hipLaunchKernelGGL(photometric_bwd_kernel, dim3(xcd_grid(cdiv(3u * strip_count(H, W, (uint32_t)rows), 4))),
+                       dim3(256), 0, (hipStream_t)stream, rows, (int)H, (int)W, ssim_scale,
                        l1_scale, render_hwc, gt_chw, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, v_render_hwc, lambda_dssim,
                        l1_partials, ssim_partials, gsx_photometric_partials(H, W), loss_out);
     GSX_LAUNCH_CHECK();
