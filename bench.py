@@ -289,7 +289,7 @@ def main():
     roofline = {
         "kernel": "rasterize_bwd_kernel", "bound": "fp32_valu", "achieved": round(dom_tf, 3),
         "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s", "frac": round(dom_tf / PEAK_FP32_TFLOPS, 4),
-        "traffic": measured_traffic_bytes("gsx::rasterize_bwd_kernel<3u, false, false>") if default_workload else None,
+        "traffic": measured_traffic_bytes("gsx::rasterize_bwd_kernel<3u, false, false, false>") if default_workload else None,
         "avg_launch_ms": round(dom_ms, 4), "launches": len(in_loop[dominant]),
         "frac_nonpacked": round(dom_tf / (PEAK_FP32_TFLOPS / 2), 4),
         "frac_pairs_evaluated": round(tflops(flops_bwd_evaluated) / PEAK_FP32_TFLOPS, 4),

@@ -198,11 +198,13 @@ GSX_API int gsx_intersect_tile_pairs_offset(int64_t n_isects, const uint16_t* ti
 /* ---- a4-a6 as one call whose pair count never crosses to the host (one camera, grids up to 255 x 255) ----
  * No single counterpart in the reference: this is intersect_tile + radix_sort_double_buffer + intersect_offset
  * (Intersect.cpp:41-137, IntersectTile.cu:23-114, 206-252, 290-328) for the caller that only feeds the rasterizers,
- * without the `.item()` of Intersect.cpp:76.  Nine launches: depth keys (+ byte histograms + tile-rectangle corners),
- * tile table (a 2-D prefix sum over the corners gives every list's length, hence tile_offsets and the count, before a
- * pair exists), four one-launch radix passes over the N depth keys, the emission of (u16 tile, id) pairs in depth
- * order, two one-launch radix passes over the tile bits.  The one-launch passes chain their workgroups by a bounded
- * look-back over per-workgroup counts.
+ * without the `.item()` of Intersect.cpp:76.  Nine launches: depth keys (+ byte histograms), four one-launch radix
+ * passes over the depth keys of the Gaussians that touch a tile, the tile table (+1 / -1 at every rectangle's corners
+ * and a 2-D prefix sum give every list's length, hence tile_offsets and the count, before a pair exists), the
+ * emission of one (super-tile, rectangle, id) entry per super-tile a Gaussian meets (the grid is cut into at most 256
+ * super-tiles), one one-launch radix pass that groups the entries by super-tile, and a gather that writes every
+ * tile's list front to back from its super-tile's entries - no (tile, id) pair is sorted.  The one-launch passes and
+ * the gather chain their workgroups by a bounded look-back over per-workgroup counts.
  *   means2d [N,2], radii [N,2], depths [N] as the projection leaves them; 16-byte aligned
  *   flatten_ids  i32 [capacity]            out: element for element the flatten_ids of the separate operators
  *   tile_offsets i32 [Th * Tw + 1]         out: the operators' tile_offsets, and the pair count in the last entry

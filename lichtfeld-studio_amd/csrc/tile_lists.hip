@@ -18,10 +18,11 @@
 //                            Gaussian) pairs; a workgroup's position in the output comes from a chained look-back over
 //                            the workgroups' entry counts;
 //  5. one chained radix pass over the super-tile byte groups the entries by super-tile, depth order kept;
-//  6. tile_gather_kernel     one wave per tile walks its super-tile's entries (staged through LDS, shared by the 16
-//                            waves of the workgroup) and writes the ids whose rectangle covers the tile, in order, to
-//                            the tile's place in flatten_ids: every list is written once, front to back, and no
-//                            (tile, id) pair is ever sorted.
+//  6. tile_gather_kernel     a workgroup takes a slice of up to 2 048 entries of one super-tile, turns every
+//                            entry's rectangle into a bit mask over the super-tile's tiles, counts and then writes,
+//                            per tile, the ids whose bit is set - in order, to the tile's place in flatten_ids;
+//                            slices of one super-tile meet through a chained look-back over per-tile counts.  Every
+//                            list is written once, front to back, and no (tile, id) pair is ever sorted.
 //
 // Everything downstream sizes its work by `capacity` and reads the actual count from device memory.  If the count
 // exceeds the capacity, every tile's list is left EMPTY (tile_offsets all zero), bit 0 of the error word is set and
