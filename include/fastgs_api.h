@@ -1,5 +1,5 @@
 // fastgs_api.h - the C++ host interface of the fastgs backend with the names, namespace, argument order and return
-// tuples of LichtFeld-Studio's src/training/fastgs/rasterization/include/rasterization_api.h:25-75, implemented in
+// tuples of LichtFeld-Studio's src/training/fastgs/rasterization/include/rasterization_api.h:12-75, implemented in
 // lichtfeld-studio_amd/csrc/host/fastgs_api.cpp on top of the C ABI of gsx_fastgs.h.  A LichtFeld build keeps its own
 // header; this one exists so that the implementation can be compiled and tested without the reference tree.
 #pragma once
@@ -9,6 +9,21 @@
 #include <tuple>
 
 namespace fast_gs::rasterization {
+
+    // rasterization_api.h:12-23: the camera and image parameters of one view, as LichtFeld's fast_rasterize gathers
+    // them before it spreads them over the wrappers' arguments (fast_rasterizer.cpp:35-45, fast_rasterizer_autograd.cpp:19)
+    struct FastGSSettings {
+        at::Tensor cam_position;
+        int active_sh_bases;
+        int width;
+        int height;
+        float focal_x;
+        float focal_y;
+        float center_x;
+        float center_y;
+        float near_plane;
+        float far_plane;
+    };
 
     // (image [3,H,W], alpha [1,H,W], per_primitive_buffers, per_tile_buffers, per_instance_buffers,
     //  per_bucket_buffers, n_visible_primitives, n_instances, n_buckets, primitive selector, instance selector).

@@ -120,6 +120,15 @@ GSX_API int gsx_intersect_tile_emit(uint32_t C, uint32_t N, const float* means2d
                                     const float* depths, const int64_t* cum_tiles_per_gauss, const int32_t* order,
                                     uint32_t tile_size, uint32_t tile_width, uint32_t tile_height, int64_t* isect_ids,
                                     int32_t* flatten_ids, void* stream);
+/* Packed rows (means2d [nnz,2], radii [nnz,2], depths [nnz], camera_ids i64 [nnz] with values in [0, C);
+ * Intersect.cpp:32-39, IntersectTile.cu:50, 86-94): count with gsx_intersect_tile_count(1, nnz, ...) - a row's tile
+ * count does not depend on its camera -, then emit with this call; flatten_ids index the packed rows.  gaussian_ids
+ * are not needed here (the reference's kernel does not read them either). */
+GSX_API int gsx_intersect_tile_emit_packed(uint32_t C, uint32_t nnz, const float* means2d, const int32_t* radii,
+                                           const float* depths, const int64_t* camera_ids,
+                                           const int64_t* cum_tiles_per_gauss, uint32_t tile_size,
+                                           uint32_t tile_width, uint32_t tile_height, int64_t* isect_ids,
+                                           int32_t* flatten_ids, void* stream);
 /* The same with the writes bounded to the first `capacity` entries: lets a caller that reuses its buffers emit
  * while the total is still on its way to the host, and repeat the call only if the total exceeded the buffers. */
 GSX_API int gsx_intersect_tile_emit_capped(uint32_t C, uint32_t N, const float* means2d, const int32_t* radii,

@@ -174,15 +174,47 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> intersect_tile(const at::Tensor m
     CHECK_INPUT(radii);
     CHECK_INPUT(depths);
     const bool packed = means2d.dim() == 2;
-    if (packed) {
-        TORCH_CHECK(camera_ids.has_value() && gaussian_ids.has_value(),
-                    "When packed is set, camera_ids and gaussian_ids must be provided.");
-        TORCH_CHECK(false, "packed intersect_tile is not built (LichtFeld never uses it: rasterizer.cpp:25)");
-    }
-    const uint32_t N = (uint32_t)means2d.size(1);
     const uint32_t tile_n_bits = gsx_n_bits(tile_width * tile_height);
     const uint32_t cam_n_bits = gsx_n_bits(C);
     at::Tensor tiles_per_gauss = at::empty_like(depths, depths.options().dtype(at::kInt));
+    if (packed) { // rows [nnz], each naming its camera (Intersect.cpp:32-39, IntersectTile.cu:50, 86-94)
+        TORCH_CHECK(camera_ids.has_value() && gaussian_ids.has_value(),
+                    "When packed is set, camera_ids and gaussian_ids must be provided.");
+        CHECK_INPUT(camera_ids.value());
+        CHECK_INPUT(gaussian_ids.value());
+        const int64_t nnz = means2d.size(0);
+        TORCH_CHECK(camera_ids->scalar_type() == at::kLong && gaussian_ids->scalar_type() == at::kLong,
+                    "camera_ids and gaussian_ids must be int64");
+        TORCH_CHECK(means2d.size(1) == 2 && radii.dim() == 2 && radii.size(0) == nnz && radii.size(1) == 2 &&
+                        depths.numel() == nnz && camera_ids->numel() == nnz && gaussian_ids->numel() == nnz,
+                    "packed intersect_tile: means2d [nnz,2], radii [nnz,2], depths / camera_ids / gaussian_ids [nnz]");
+        void* stream = cur_stream(means2d);
+        at::Tensor cum = at::empty({nnz}, depths.options().dtype(at::kLong));
+        int64_t n_isects = 0;
+        at::Tensor ws = workspace(gsx_intersect_tile_count_workspace_bytes(1, (uint32_t)nnz), depths);
+        gsx_check(gsx_intersect_tile_count(1, (uint32_t)nnz, means2d.data_ptr<float>(), radii.data_ptr<int32_t>(),
+                                           tile_size, tile_width, tile_height, tiles_per_gauss.data_ptr<int32_t>(),
+                                           cum.data_ptr<int64_t>(), ws.data_ptr(), (size_t)ws.numel(), &n_isects,
+                                           stream));
+        at::Tensor isect_ids = at::empty({n_isects}, depths.options().dtype(at::kLong));
+        at::Tensor flatten_ids = at::empty({n_isects}, depths.options().dtype(at::kInt));
+        if (n_isects)
+            gsx_check(gsx_intersect_tile_emit_packed(C, (uint32_t)nnz, means2d.data_ptr<float>(),
+                                                     radii.data_ptr<int32_t>(), depths.data_ptr<float>(),
+                                                     camera_ids->data_ptr<int64_t>(), cum.data_ptr<int64_t>(),
+                                                     tile_size, tile_width, tile_height,
+                                                     isect_ids.data_ptr<int64_t>(), flatten_ids.data_ptr<int32_t>(),
+                                                     stream));
+        if (n_isects && sort) {
+            at::Tensor isect_ids_sorted = at::empty_like(isect_ids);
+            at::Tensor flatten_ids_sorted = at::empty_like(flatten_ids);
+            sort_pairs(n_isects, 0u, 32 + tile_n_bits + cam_n_bits, isect_ids, flatten_ids, isect_ids_sorted,
+                       flatten_ids_sorted);
+            return std::make_tuple(tiles_per_gauss, isect_ids_sorted, flatten_ids_sorted);
+        }
+        return std::make_tuple(tiles_per_gauss, isect_ids, flatten_ids);
+    }
+    const uint32_t N = (uint32_t)means2d.size(1);
     // one camera, sorted output: visit the Gaussians in depth order and sort on the tile bits only (same array as
     // one sort on every bit, Intersect.cpp:104-113, because the sort is stable)
     const bool two_level = sort && C == 1;

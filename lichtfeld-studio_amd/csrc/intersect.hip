@@ -180,7 +180,8 @@ __global__ void __launch_bounds__(256) tile_emit_kernel(uint32_t n, uint32_t N, 
                                                          uint32_t tile_n_bits, int64_t capacity,
                                                          int64_t* __restrict__ isect_ids,
                                                          uint16_t* __restrict__ tile_keys /*COMPACT*/,
-                                                         int32_t* __restrict__ flatten_ids) {
+                                                         int32_t* __restrict__ flatten_ids,
+                                                         const int64_t* __restrict__ camera_ids = nullptr) {
     __shared__ uint32_t s_incl[4][64], s_xy[4][64], s_w[4][64], s_idx[4][64], s_lo[COMPACT ? 1 : 4][64],
         s_hi[COMPACT ? 1 : 4][64];
     const uint32_t i = blockIdx.x * 256u + threadIdx.x;
@@ -205,7 +206,8 @@ __global__ void __launch_bounds__(256) tile_emit_kernel(uint32_t n, uint32_t N, 
     const uint32_t cnt = live ? (r.y1 - r.y0) * w : 0u;
     int64_t key_base = 0;
     if (cnt) {
-        const int64_t cid = idx / N;
+        // packed rows name their camera themselves (IntersectTile.cu:86-94)
+        const int64_t cid = camera_ids != nullptr ? camera_ids[idx] : (int64_t)(idx / N);
         if (!FROM_KEYS)
             depth_bits = f2u(depths[idx]);
         key_base = (cid << (32 + tile_n_bits)) | (int64_t)(uint64_t)depth_bits; // zero-extended bits (:96-98)
@@ -642,6 +644,30 @@ extern "C" int gsx_intersect_tile_emit_capped(uint32_t C, uint32_t N, const floa
                        radii, depths, (const int64_t*)nullptr, cum_tiles_per_gauss, order, (float)tile_size, tile_width,
                        tile_height, gsx_n_bits(tile_width * tile_height), capacity, isect_ids, (uint16_t*)nullptr,
                        flatten_ids);
+    GSX_LAUNCH_CHECK();
+    return GSX_OK;
+}
+
+// Packed rows ([nnz] instead of [C, N]; Intersect.cpp:32-39, IntersectTile.cu:50, 86-94): the count is that of one
+// camera with nnz rows (a row's tile count does not depend on its camera), the emission takes each row's camera
+// from camera_ids; flatten_ids index the packed rows.
+extern "C" int gsx_intersect_tile_emit_packed(uint32_t C, uint32_t nnz, const float* means2d, const int32_t* radii,
+                                              const float* depths, const int64_t* camera_ids,
+                                              const int64_t* cum_tiles_per_gauss, uint32_t tile_size,
+                                              uint32_t tile_width, uint32_t tile_height, int64_t* isect_ids,
+                                              int32_t* flatten_ids, void* stream) {
+    if (nnz == 0)
+        return GSX_OK;
+    GSX_REQUIRE(means2d && radii && depths && camera_ids && cum_tiles_per_gauss && isect_ids && flatten_ids,
+                GSX_ERR_INVALID_ARGUMENT, "intersect_tile_emit_packed: null tensor");
+    GSX_REQUIRE(nnz < (1u << 31), GSX_ERR_INVALID_ARGUMENT, "intersect_tile_emit_packed: nnz >= 2^31");
+    const int rc = check_tile_grid("intersect_tile_emit_packed", C, tile_size, tile_width, tile_height);
+    if (rc != GSX_OK)
+        return rc;
+    hipLaunchKernelGGL(tile_emit_kernel<false>, dim3(cdiv(nnz, 256)), dim3(256), 0, (hipStream_t)stream, nnz, nnz,
+                       means2d, radii, depths, (const int64_t*)nullptr, cum_tiles_per_gauss, (const int32_t*)nullptr,
+                       (float)tile_size, tile_width, tile_height, gsx_n_bits(tile_width * tile_height), INT64_MAX,
+                       isect_ids, (uint16_t*)nullptr, flatten_ids, camera_ids);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }

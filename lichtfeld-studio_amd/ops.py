@@ -114,12 +114,13 @@ def intersect_tile(means2d, radii, depths, camera_ids, gaussian_ids, C, tile_siz
                    sort=True):
     """Ops.h:28-38 -> (tiles_per_gauss [C,N] i32, isect_ids [I] i64, flatten_ids [I] i32)"""
     _f32(means2d, "means2d"), _check_input(radii, "radii"), _f32(depths, "depths")
+    if radii.dtype != torch.int32:
+        raise RuntimeError("radii must be int32")
     if means2d.dim() == 2:
         if camera_ids is None or gaussian_ids is None:  # Intersect.cpp:34-36
             raise RuntimeError("When packed is set, camera_ids and gaussian_ids must be provided.")
-        raise NotImplementedError("packed intersect_tile is not built (LichtFeld never uses it: rasterizer.cpp:25)")
-    if radii.dtype != torch.int32:
-        raise RuntimeError("radii must be int32")
+        return _intersect_tile_packed(means2d, radii, depths, camera_ids, gaussian_ids, C, tile_size, tile_width,
+                                      tile_height, sort)
     dev = means2d.device
     N = means2d.size(1)
     _sized(means2d, "means2d", C, N, 2), _sized(radii, "radii", C, N, 2), _sized(depths, "depths", C, N)
@@ -162,6 +163,40 @@ def intersect_tile(means2d, radii, depths, camera_ids, gaussian_ids, C, tile_siz
             cam_n_bits = lib().gsx_n_bits(c_u32(C))
             isect_ids, flatten_ids = radix_sort_double_buffer(n, tile_n_bits, cam_n_bits, isect_ids, flatten_ids,
                                                               begin_bit=32 if two_level else 0)
+    return tiles_per_gauss, isect_ids, flatten_ids
+
+
+def _intersect_tile_packed(means2d, radii, depths, camera_ids, gaussian_ids, C, tile_size, tile_width, tile_height,
+                           sort):
+    """packed rows [nnz] (Intersect.cpp:32-39): the count of one camera with nnz rows, the emission with each row's
+    camera from camera_ids (IntersectTile.cu:86-94), the reference's one sort over all bits"""
+    _check_input(camera_ids, "camera_ids"), _check_input(gaussian_ids, "gaussian_ids")
+    if camera_ids.dtype != torch.int64 or gaussian_ids.dtype != torch.int64:
+        raise RuntimeError("camera_ids and gaussian_ids must be int64")
+    dev = means2d.device
+    nnz = means2d.size(0)
+    _sized(means2d, "means2d", nnz, 2), _sized(radii, "radii", nnz, 2), _sized(depths, "depths", nnz)
+    _sized(camera_ids, "camera_ids", nnz), _sized(gaussian_ids, "gaussian_ids", nnz)
+    tiles_per_gauss = torch.empty_like(depths, dtype=torch.int32)
+    n_isects = c_i64(0)
+    with torch.cuda.device(dev):
+        cum = torch.empty((nnz,), dtype=torch.int64, device=dev)
+        ws = _workspace(lib().gsx_intersect_tile_count_workspace_bytes(c_u32(1), c_u32(nnz)), dev)
+        check(lib().gsx_intersect_tile_count(c_u32(1), c_u32(nnz), _ptr(means2d), _ptr(radii), c_u32(tile_size),
+                                             c_u32(tile_width), c_u32(tile_height), _ptr(tiles_per_gauss), _ptr(cum),
+                                             _ptr(ws), c_sz(ws.numel()), ctypes.byref(n_isects), _stream(dev)))
+        n = n_isects.value
+        isect_ids = torch.empty((n,), dtype=torch.int64, device=dev)
+        flatten_ids = torch.empty((n,), dtype=torch.int32, device=dev)
+        if n:
+            check(lib().gsx_intersect_tile_emit_packed(
+                c_u32(C), c_u32(nnz), _ptr(means2d), _ptr(radii), _ptr(depths), _ptr(camera_ids), _ptr(cum),
+                c_u32(tile_size), c_u32(tile_width), c_u32(tile_height), _ptr(isect_ids), _ptr(flatten_ids),
+                _stream(dev)))
+        if n and sort:
+            tile_n_bits = lib().gsx_n_bits(c_u32(tile_width * tile_height))
+            cam_n_bits = lib().gsx_n_bits(c_u32(C))
+            isect_ids, flatten_ids = radix_sort_double_buffer(n, tile_n_bits, cam_n_bits, isect_ids, flatten_ids)
     return tiles_per_gauss, isect_ids, flatten_ids
 
 

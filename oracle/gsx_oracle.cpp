@@ -767,10 +767,12 @@ ORC_API int orc_intersect_tile_count(uint32_t C, uint32_t N, const float* means2
     return 0;
 }
 
-ORC_API int orc_intersect_tile_emit(uint32_t C, uint32_t N, const float* means2d, const int32_t* radii,
-                                    const float* depths, const int64_t* cum_tiles_per_gauss, uint32_t tile_size,
-                                    uint32_t tile_width, uint32_t tile_height, int64_t* isect_ids,
-                                    int32_t* flatten_ids) {
+// camera_ids: null for [C, N] rows (camera = idx / N); else packed rows [nnz = C * N as passed], each naming its
+// camera (IntersectTile.cu:86-94)
+static int intersect_tile_emit(uint32_t C, uint32_t N, const float* means2d, const int32_t* radii,
+                               const float* depths, const int64_t* camera_ids, const int64_t* cum_tiles_per_gauss,
+                               uint32_t tile_size, uint32_t tile_width, uint32_t tile_height, int64_t* isect_ids,
+                               int32_t* flatten_ids) {
     const int64_t n = (int64_t)C * N;
     const uint32_t tile_n_bits = orc_tile_n_bits(tile_width * tile_height);
 #pragma omp parallel for schedule(static)
@@ -780,7 +782,7 @@ ORC_API int orc_intersect_tile_emit(uint32_t C, uint32_t N, const float* means2d
         tile_bounds(means2d, radii, idx, tile_size, tile_width, tile_height, &x0, &y0, &x1, &y1, &skip);
         if (skip)
             continue;
-        const int64_t cid = idx / N;
+        const int64_t cid = camera_ids != nullptr ? camera_ids[idx] : idx / N;
         const int64_t cid_enc = cid << (32 + tile_n_bits);
         uint32_t dbits;
         std::memcpy(&dbits, depths + idx, 4);
@@ -795,6 +797,23 @@ ORC_API int orc_intersect_tile_emit(uint32_t C, uint32_t N, const float* means2d
             }
     }
     return 0;
+}
+
+ORC_API int orc_intersect_tile_emit(uint32_t C, uint32_t N, const float* means2d, const int32_t* radii,
+                                    const float* depths, const int64_t* cum_tiles_per_gauss, uint32_t tile_size,
+                                    uint32_t tile_width, uint32_t tile_height, int64_t* isect_ids,
+                                    int32_t* flatten_ids) {
+    return intersect_tile_emit(C, N, means2d, radii, depths, nullptr, cum_tiles_per_gauss, tile_size, tile_width,
+                               tile_height, isect_ids, flatten_ids);
+}
+
+ORC_API int orc_intersect_tile_emit_packed(uint32_t nnz, const float* means2d, const int32_t* radii,
+                                           const float* depths, const int64_t* camera_ids,
+                                           const int64_t* cum_tiles_per_gauss, uint32_t tile_size,
+                                           uint32_t tile_width, uint32_t tile_height, int64_t* isect_ids,
+                                           int32_t* flatten_ids) {
+    return intersect_tile_emit(1, nnz, means2d, radii, depths, camera_ids, cum_tiles_per_gauss, tile_size,
+                               tile_width, tile_height, isect_ids, flatten_ids);
 }
 
 // =============================================================================================

@@ -272,6 +272,33 @@ def intersect_tile(means2d, radii, depths, C, tile_size, tile_width, tile_height
     return tpg, ids, flat
 
 
+def intersect_tile_packed(means2d, radii, depths, camera_ids, C, tile_size, tile_width, tile_height, sort=True):
+    """gsplat/Ops.h:28-38 with packed rows (means2d [nnz,2], camera_ids [nnz]; Intersect.cpp:32-39,
+    IntersectTile.cu:50, 86-94).  -> tiles_per_gauss [nnz] i32, isect_ids [I] i64, flatten_ids [I] i32 (packed row
+    indices)."""
+    means2d, depths = _f32(means2d), _f32(depths)
+    radii = np.ascontiguousarray(radii, dtype=np.int32)
+    camera_ids = np.ascontiguousarray(camera_ids, dtype=np.int64)
+    nnz = means2d.shape[0]
+    tpg = np.zeros((nnz,), np.int32)
+    cum = np.zeros((nnz,), np.int64)
+    n_isects = c_i64(0)
+    _chk(lib().orc_intersect_tile_count(c_u32(1), c_u32(nnz), _p(means2d), _p(radii), c_u32(tile_size),
+                                        c_u32(tile_width), c_u32(tile_height), _p(tpg), _p(cum),
+                                        ctypes.byref(n_isects)), "intersect_tile_count")
+    n = n_isects.value
+    ids = np.zeros((n,), np.int64)
+    flat = np.zeros((n,), np.int32)
+    if n:
+        _chk(lib().orc_intersect_tile_emit_packed(c_u32(nnz), _p(means2d), _p(radii), _p(depths), _p(camera_ids),
+                                                  _p(cum), c_u32(tile_size), c_u32(tile_width), c_u32(tile_height),
+                                                  _p(ids), _p(flat)), "intersect_tile_emit_packed")
+    if n and sort:
+        end_bit = 32 + tile_n_bits(tile_width * tile_height) + tile_n_bits(C)
+        ids, flat = radix_sort_pairs(ids, flat, end_bit)
+    return tpg, ids, flat
+
+
 def radix_sort_pairs(keys, vals, end_bit):
     """gsplat/Intersect.h:39-46: stable ascending sort on bits [0, end_bit)."""
     keys = np.ascontiguousarray(keys, dtype=np.int64)

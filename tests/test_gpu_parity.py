@@ -214,6 +214,39 @@ def test_intersect_sort_offsets_bit_exact(gsx, orc, cuda):
     assert ids.numel() == 0 and flat.numel() == 0 and int(tpg.sum()) == 0
 
 
+def test_intersect_packed_rows(gsx, orc, cpp, cuda):
+    """packed [nnz] rows with camera_ids / gaussian_ids (Intersect.cpp:32-39): counts, keys and values bit-identical to
+    the checker, sorted and not, through the ctypes and the C++ mirrors; the ranges of every camera from the sorted
+    keys; packed without ids is refused as in the reference"""
+    ops = gsx.ops
+    rng = np.random.default_rng(11)
+    C, n, tw, th = 3, 20000, 78, 52
+    means2d = np.stack([rng.uniform(-20, tw * 16 + 20, (C, n)), rng.uniform(-20, th * 16 + 20, (C, n))], -1)
+    means2d = means2d.astype(np.float32)
+    radii = rng.integers(0, 40, (C, n, 2)).astype(np.int32)
+    radii[:, ::5] = 0
+    depths = rng.uniform(0.1, 50.0, (C, n)).astype(np.float32)
+    depths[:, 100:200] = depths[0, 100]  # ties
+    keep = np.argwhere((radii > 0).all(-1))
+    keep = keep[rng.permutation(len(keep))]
+    cam_ids, gauss_ids = keep[:, 0].astype(np.int64), keep[:, 1].astype(np.int64)
+    pm, pr, pd = means2d[cam_ids, gauss_ids], radii[cam_ids, gauss_ids], depths[cam_ids, gauss_ids]
+    dev = [T(x, cuda) for x in (pm, pr, pd, cam_ids, gauss_ids)]
+    for sort in (False, True):
+        ref_tpg, ref_ids, ref_flat = orc.intersect_tile_packed(pm, pr, pd, cam_ids, C, 16, tw, th, sort)
+        assert ref_ids.shape[0] > 300000
+        for name, fn in (("ctypes", ops.intersect_tile), ("c++", cpp.intersect_tile)):
+            tpg, ids, flat = fn(*dev, C, 16, tw, th, sort)
+            bits_equal(N(tpg), ref_tpg, f"{name} tiles_per_gauss")
+            bits_equal(N(ids), ref_ids, f"{name} keys (sort={sort})")
+            bits_equal(N(flat), ref_flat, f"{name} values (sort={sort})")
+    bits_equal(N(ops.intersect_offset(ids, C, tw, th)), orc.intersect_offset(ref_ids, C, tw, th), "per-tile ranges")
+    with pytest.raises(RuntimeError, match="camera_ids and gaussian_ids must be provided"):
+        ops.intersect_tile(dev[0], dev[1], dev[2], None, None, C, 16, tw, th, True)
+    with pytest.raises(RuntimeError, match="camera_ids and gaussian_ids must be provided"):
+        cpp.intersect_tile(dev[0], dev[1], dev[2], None, None, C, 16, tw, th, True)
+
+
 @pytest.mark.parametrize("grid", [(255, 40), (256, 40), (40, 300), (255, 255)])
 def test_intersect_wide_tile_grids(gsx, orc, cuda, grid):
     """tile grids at and beyond 255 tiles per side: up to 255 x 255 the depth keys carry each Gaussian's tile rectangle

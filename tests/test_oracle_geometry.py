@@ -337,6 +337,39 @@ def test_intersect_brute_force_and_invariants(orc):
     assert np.all(orc.intersect_offset(np.zeros(0, np.int64), 1, tw, th) == 0)
 
 
+def test_intersect_packed_rows_brute_force(orc):
+    """packed rows (Intersect.cpp:32-39): the rows of a [C, N] problem that have a footprint, in any order, each naming
+    its camera - keys are (camera << (32 + tile bits)) | tile << 32 | depth bits by brute force, values the packed row
+    index; sorted, the camera / tile / depth part of the keys equals that of the unpacked problem"""
+    rng = np.random.default_rng(5)
+    C, n, W, H, tile = 3, 300, 200, 120, 16
+    tw, th = (W + 15) // 16, (H + 15) // 16
+    means2d = rng.uniform(-60, 260, (C, n, 2)).astype(np.float32)
+    radii = rng.integers(0, 40, (C, n, 2)).astype(np.int32)
+    radii[:, ::7] = 0
+    depths = np.exp(rng.normal(1, 0.5, (C, n))).astype(np.float32)
+    keep = np.argwhere((radii > 0).all(-1))
+    keep = keep[rng.permutation(len(keep))]  # packed rows come in no particular order
+    cam_ids, gauss_ids = keep[:, 0].astype(np.int64), keep[:, 1].astype(np.int64)
+    pm, pr, pd = means2d[cam_ids, gauss_ids], radii[cam_ids, gauss_ids], depths[cam_ids, gauss_ids]
+    tpg, ids, flat = orc.intersect_tile_packed(pm, pr, pd, cam_ids, C, tile, tw, th, sort=False)
+    want = brute_force_tiles(pm, pr, tile, tw, th)
+    assert [len(t) for t in want] == list(tpg) and tpg.sum() == ids.shape[0] > 1000
+    tile_bits = orc.tile_n_bits(tw * th)
+    exp_ids = np.array([(int(cam_ids[r]) << (32 + tile_bits)) | (t << 32) | int(pd[r].view(np.uint32))
+                        for r, ts in enumerate(want) for t in ts], np.int64)
+    exp_flat = np.array([r for r, ts in enumerate(want) for _ in ts], np.int32)
+    assert np.array_equal(ids, exp_ids) and np.array_equal(flat, exp_flat)
+    _, sid, sflat = orc.intersect_tile_packed(pm, pr, pd, cam_ids, C, tile, tw, th, sort=True)
+    order = np.argsort(exp_ids, kind="stable")
+    assert np.array_equal(sid, exp_ids[order]) and np.array_equal(sflat, exp_flat[order])
+    # against the unpacked problem: same multiset of keys; per key the same (camera, Gaussian) set
+    _, uid, uflat = orc.intersect_tile(means2d, radii, depths, C, tile, tw, th, sort=True)
+    assert np.array_equal(sid, uid)
+    packed_pairs = sorted(zip(sid.tolist(), (cam_ids[sflat] * n + gauss_ids[sflat]).tolist()))
+    assert packed_pairs == sorted(zip(uid.tolist(), uflat.tolist()))
+
+
 def test_intersect_key_layout_and_bits(orc):
     assert [orc.tile_n_bits(t) for t in (1, 2, 255, 256, 4056, 8160, 32400)] == [1, 2, 8, 9, 12, 13, 15]
     # one Gaussian covering a 2x3 block of tiles: row-major emission, depth bits in the low word
