@@ -228,7 +228,8 @@ GSX_API int gsx_intersect_tile_pairs_offset(int64_t n_isects, const uint16_t* ti
  * while the depth sort runs on `stream` (forked and joined with events inside the call; all results are ordered on
  * `stream` when the call returns).
  * The workspace's head must be zeroed once by gsx_tile_lists_init; every call leaves it ready for the next one.  Calls
- * that share a workspace must not overlap. */
+ * that share a workspace must not overlap, and host threads that call with the same `stream` must take turns: the
+ * events that fork and join the two streams are kept per device and `stream`. */
 #define GSX_COUNT_IN_OFFSETS (-1ll)
 GSX_API size_t gsx_tile_lists_workspace_bytes(uint32_t N, int64_t capacity, uint32_t tile_width,
                                               uint32_t tile_height);
