@@ -1041,6 +1041,60 @@ def test_rasterizer_channel_counts(gsx, orc, cuda, channels):
     assert per_channel.max() <= 1e-3, per_channel
 
 
+def test_wide_channel_counts_with_masks_distortion_and_no_background(gsx, orc, cuda):
+    """33 channels (two launches of the run-time channel count instance: 32 + 1) in the cases the plain test leaves
+    out: per-tile masks with and without a background (a masked tile shows the background in every channel), and the
+    distorted camera's instance - forward bit-identical to the checker, gradients within 1e-3 of each tensor's scale"""
+    ops = gsx.ops
+    sc, cam, h, d = _fused_inputs(gsx, cuda, 3000)
+    ut = ops.UnscentedTransformParameters()
+    ch = 33
+    rng = np.random.default_rng(33)
+    n = h["means"].shape[0]
+    colors_h = rng.uniform(0, 1, (1, n, ch)).astype(np.float32)
+    bg_h = rng.uniform(0, 1, (1, ch)).astype(np.float32)
+    colors_d, op1 = T(colors_h, cuda), d["op"][None].contiguous()
+    tw, th = (cam.width + 15) // 16, (cam.height + 15) // 16
+    masks_h = rng.uniform(0, 1, (1, th, tw)) > 0.3
+    dist = {k: T(np.asarray(v, np.float32)[None], cuda) for k, v in _DIST.items()}
+    for name, coeffs, masks, bg in (("masks + background", None, masks_h, bg_h), ("masks, no background", None, masks_h, None),
+                                    ("distorted", dist, None, bg_h)):
+        co = (None, None, None) if coeffs is None else (coeffs["radial"], coeffs["tangential"], coeffs["thin_prism"])
+        got = ops.rasterize_from_world_with_sh_fwd(d["means"], d["quats"], d["scales"], d["op"], d["shs"], 3, d["bg"],
+                                                   None, cam.width, cam.height, 16, d["vm"], None, d["K"], 0, 0.3, 0.01,
+                                                   1e4, 0.0, 1.0, False, 0, ut, 4, *co)
+        offsets, flat = got[6], got[7]
+        m_d = None if masks is None else T(masks, cuda)
+        bg_d = None if bg is None else T(bg, cuda)
+        renders, alphas, last_ids = ops.rasterize_to_pixels_from_world_3dgs_fwd(
+            d["means"], d["quats"], d["scales"], colors_d, op1, bg_d, m_d, cam.width, cam.height, 16, d["vm"], None,
+            d["K"], 0, ut, 4, *co, offsets, flat)
+        args = (h["means"], h["quats"], h["scales"], colors_h, h["op"][None], bg)
+        from contextlib import nullcontext
+        with (orc.distortion(**_DIST) if coeffs is not None else nullcontext()):
+            ref = orc.rasterize_to_pixels_from_world_3dgs_fwd(*args, masks, cam.width, cam.height, 16, h["vm"], h["K"],
+                                                              N(offsets), N(flat))
+            v_r = rng.normal(0, 1, tuple(renders.shape)).astype(np.float32)
+            v_a = rng.normal(0, 1, tuple(alphas.shape)).astype(np.float32)
+            o5 = orc.rasterize_to_pixels_from_world_3dgs_bwd(*args, masks, cam.width, cam.height, 16, h["vm"], h["K"],
+                                                             N(offsets), N(flat), N(alphas), N(last_ids), v_r, v_a)
+        # alpha and last ids of a masked tile are left unwritten (Rasterization.cpp allocates them with at::empty)
+        pm = (np.ones((cam.height, cam.width), bool) if masks is None
+              else np.repeat(np.repeat(masks[0], 16, 0), 16, 1)[:cam.height, :cam.width])
+        bits_equal(N(renders), ref[0], f"{name}: image")
+        bits_equal(N(alphas)[0, pm], ref[1][0, pm], f"{name}: alpha")
+        bits_equal(N(last_ids)[0, pm], ref[2][0, pm], f"{name}: last ids")
+        assert np.abs(ref[0][..., -1]).max() > 0
+        got5 = ops.rasterize_to_pixels_from_world_3dgs_bwd(d["means"], d["quats"], d["scales"], colors_d, op1, bg_d, m_d,
+                                                           cam.width, cam.height, 16, d["vm"], None, d["K"], 0, ut, 4,
+                                                           *co, offsets, flat, alphas, last_ids, T(v_r, cuda),
+                                                           T(v_a, cuda))
+        for tn, a, b in zip(("v_means", "v_quats", "v_scales", "v_colors", "v_opacities"), got5, o5):
+            a, b = N(a).reshape(np.asarray(b).shape), np.asarray(b)
+            assert np.abs(a - b).max() <= 1e-3 * np.abs(b).max(), f"{name} {tn}: {np.abs(a - b).max()} vs {np.abs(b).max()}"
+            assert np.abs(b).max() > 0
+
+
 def test_rasterizer_rejects_unbuilt_channel_counts(gsx, cuda):
     ops = gsx.ops
     sc, cam, h, d = _fused_inputs(gsx, cuda, 300)
