@@ -114,6 +114,40 @@ def test_projection_matches_float64_unscented_transform_and_ewa_limit(orc):
                                    atol=1e-9)
 
 
+def test_projection_plain_route_equals_the_general_route_to_rounding(orc):
+    """the trainer's camera takes the sigma points through the pose as a matrix and projects with one reciprocal per
+    point; with all-zero distortion coefficients the same camera takes the general route (quaternion rotation, a
+    division per coordinate).  Same function, other rounding: radii within one unit on a handful of Gaussians, image
+    points within what the unscented weights (-99, +16.7) make of a few ulp, depths within 4 ulp - and the plain
+    route is no further from the float64 model than the general one"""
+    rng = np.random.default_rng(3)
+    V = np.eye(4, dtype=np.float32)
+    V[:3, :3] = Rotation.from_euler("xyz", [0.2, -0.3, 0.1]).as_matrix()
+    V[:3, 3] = [0.1, -0.2, 5.0]
+    K = np.array([[600, 0, 330], [0, 580, 250], [0, 0, 1]], np.float32)
+    W, H = 640, 480
+    n = 4000
+    means = rng.uniform(-1.5, 1.5, (n, 3)).astype(np.float32)
+    quats = rng.normal(0, 1, (n, 4)).astype(np.float32)
+    scales = np.exp(rng.uniform(np.log(0.01), np.log(0.3), (n, 3))).astype(np.float32)
+    plain = orc.projection_ut_3dgs_fused(means, quats, scales, None, V[None], K[None], W, H)
+    with orc.distortion(radial=[0.0] * 6, tangential=[0.0] * 2, thin_prism=[0.0] * 4):
+        general = orc.projection_ut_3dgs_fused(means, quats, scales, None, V[None], K[None], W, H)
+    ra, rb = plain[0][0].astype(np.int64), general[0][0].astype(np.int64)
+    assert np.abs(ra - rb).max() <= 1 and (ra != rb).any(axis=1).mean() < 2e-3
+    vis = (ra[:, 0] > 0) & (rb[:, 0] > 0)
+    assert vis.sum() > 3000
+    assert np.abs(plain[1][0][vis] - general[1][0][vis]).max() < 0.03
+    assert (np.abs(plain[2][0][vis] - general[2][0][vis]) <= 4 * np.spacing(np.abs(general[2][0][vis]))).all()
+    assert not np.array_equal(plain[1][0][vis], general[1][0][vis])  # they ARE two evaluations
+    err_p, err_g = [], []
+    for i in np.flatnonzero(vis)[:200]:
+        m, _, _, _ = ut_project_f64(means[i].astype(np.float64), quats[i], scales[i].astype(np.float64), V, K)
+        err_p.append(np.abs(plain[1][0, i] - m).max())
+        err_g.append(np.abs(general[1][0, i] - m).max())
+    assert np.mean(err_p) <= 1.5 * np.mean(err_g) + 1e-5, (np.mean(err_p), np.mean(err_g))
+
+
 def test_projection_culling_cases(orc):
     V, K, W, H = look_cam()
     one = lambda mean, s=0.05, o=0.9, **kw: orc.projection_ut_3dgs_fused(
