@@ -164,6 +164,15 @@ def test_bench_finds_its_kernel_in_the_committed_traffic_summary():
     assert nbytes is not None and 5e7 < nbytes < 2e9, (prefix, nbytes)
 
 
+def test_bench_refuses_more_than_one_gpu():
+    """the path has no multi-GPU part: bench.py --gpus 2 exits with a message that says so, before touching a GPU"""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode == 2 and "ONE GPU" in r.stderr and r.stdout.strip() == ""
+
+
 def test_config5_as_stated_exceeds_int32_pairs(gsx, orc):
     """BASELINE configs[4] with its literal parameters (log-scales ~N(-3.5, 1) at 3840x2160, f = 3200): the count
     pass of intersect_tile alone (no pair is formed) gives more (tile, Gaussian) pairs than the int32 flatten_ids /
