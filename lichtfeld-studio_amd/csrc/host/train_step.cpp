@@ -102,6 +102,10 @@ namespace gsx {
     TrainStep::~TrainStep() {
         if (!impl_)
             return;
+        // the buffers were allocated for the current stream: what the second stream still has queued on them must be
+        // over before the allocator hands them to somebody else
+        if (impl_->side != nullptr)
+            (void)hipStreamSynchronize(impl_->side);
         for (hipEvent_t e : {impl_->ev_fork, impl_->ev_join, impl_->ev_loss_fork, impl_->ev_order_join})
             if (e != nullptr)
                 (void)hipEventDestroy(e);
