@@ -90,6 +90,16 @@ class TrainStep:
         self.order_pending, self._order_due = False, None
         self.loss_out = torch.empty(3, dtype=torch.float32, device=self.dev)
 
+    def __del__(self):
+        # the buffers were allocated for the current stream: what the second stream still has queued on them must be
+        # over before the allocator hands them to somebody else
+        side = getattr(self, "side", None)
+        if side is not None:
+            try:
+                side.synchronize()
+            except Exception:
+                pass
+
     def _allocate_per_gaussian(self, N):
         """every buffer whose size follows the number of Gaussians"""
         self.N = N
