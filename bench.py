@@ -103,6 +103,48 @@ def algorithmic_bytes(N, K, H, W, n_isects, sort_bits, key_bytes=8):
     }
 
 
+def run_mcmc_part(ts, dev, reps=5):
+    """What configuration 4 runs behind the step (mcmc.cpp:112-190, 349-367): relocation of the 5 % of the Gaussians
+    with the lowest opacity onto Gaussians drawn from a multinomial over the others' opacities (Eq. 9 rebalancing,
+    n_max = 51), and noise on the means.  The draw is the caller's (torch, outside the timed calls); the two library
+    calls are timed with HIP events.  Not part of `value`: the metric is the step."""
+    import numpy as np
+    import torch
+    n_dead = ts.N // 20
+    op = torch.sigmoid(ts.params["opacity"].reshape(-1))
+    order = torch.argsort(op, stable=True)
+    dead = torch.sort(order[:n_dead]).values.contiguous()
+    alive = torch.sort(order[n_dead:]).values
+    g = torch.Generator(device=dev).manual_seed(44)
+    # torch.multinomial takes at most 2^24 categories: draw by inverting the cumulative distribution
+    cdf = torch.cumsum(op[alive].double(), 0)
+    u = torch.rand(n_dead, generator=g, device=dev, dtype=torch.float64) * cdf[-1]
+    sampled = alive[torch.searchsorted(cdf, u).clamp_(max=alive.numel() - 1)].contiguous()
+    b = np.zeros((51, 51), np.float32)
+    for n in range(51):
+        for k in range(n + 1):
+            x = np.float32(1.0)
+            for i in range(k):
+                x = np.float32(x * (np.float32(n - i) / np.float32(i + 1)))
+            b[n, k] = x
+    binoms = torch.from_numpy(b).to(dev)
+    t_rel, t_noise = [], []
+    for r in range(reps):
+        e = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+        e[0].record()
+        ts.relocate(sampled, dead, binoms)
+        e[1].record()
+        ts.inject_noise(None, seed=r)
+        e[2].record()
+        torch.cuda.synchronize()
+        t_rel.append(e[0].elapsed_time(e[1]))
+        t_noise.append(e[1].elapsed_time(e[2]))
+    return {"relocated": int(n_dead), "relocate_ms": round(float(np.median(t_rel)), 4),
+            "noise_ms": round(float(np.median(t_noise)), 4),
+            "what": "gsx_mcmc_relocate (5 % of the Gaussians, caller-drawn index sets) and gsx_add_noise_philox after "
+                    "the timed steps; not part of value"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -233,6 +275,10 @@ def main():
         ts.step(views[i % len(views)], Kmat, W, H, gt)
     stage_ms = {k: float(np.mean(v)) for k, v in ts.stop_timing().items()}
 
+    mcmc = None
+    if args.config == 4:
+        mcmc = run_mcmc_part(ts, dev)
+
     # known-size copy: the yardstick for byte counters and the measured streaming bandwidth of this GPU
     copy_bytes = 1 << 30  # well beyond the 256 MB last-level cache
     cp_src = torch.empty(copy_bytes, dtype=torch.uint8, device=dev)
@@ -345,6 +391,7 @@ def main():
         "raster_fwd_ms": kernels.get("rasterize_to_pixels_from_world_3dgs_fwd", {}).get("ms"),
         "raster_bwd_ms": round(dom_ms, 4),
         "roofline": roofline, "cpu_baseline": cpu_baseline, "parity_in_bench": parity, "boundary_path": boundary,
+        "mcmc": mcmc,
         "copy_probe": {"bytes_moved": 2 * copy_bytes, "GBps": round(copy_gbs, 1),
                        "note": "gsx_debug_copy, 1 GiB read + 1 GiB written: measured streaming bandwidth"},
         "kernels": kernels,
