@@ -22,6 +22,9 @@ int orc_intersect_tile_count(uint32_t C, uint32_t N, const float* means2d, const
 int orc_intersect_tile_emit(uint32_t C, uint32_t N, const float* means2d, const int32_t* radii, const float* depths,
                             const int64_t* cum_tiles_per_gauss, uint32_t tile_size, uint32_t tile_width,
                             uint32_t tile_height, int64_t* isect_ids, int32_t* flatten_ids);
+int orc_intersect_tile_emit_packed(uint32_t nnz, const float* means2d, const int32_t* radii, const float* depths,
+                                   const int64_t* camera_ids, const int64_t* cum_tiles_per_gauss, uint32_t tile_size,
+                                   uint32_t tile_width, uint32_t tile_height, int64_t* isect_ids, int32_t* flatten_ids);
 uint32_t orc_tile_n_bits(uint32_t n_tiles);
 int orc_radix_sort_pairs(int64_t n, const int64_t* keys_in, const int32_t* vals_in, uint32_t end_bit,
                          int64_t* keys_out, int32_t* vals_out);
@@ -113,6 +116,18 @@ int main() {
     std::vector<int32_t> flat(n_isects), flat_sorted(n_isects), offsets(tw * th);
     CHECK(orc_intersect_tile_emit(1, N, means2d.data(), radii.data(), depths.data(), cum.data(), tile, tw, th,
                                   ids.data(), flat.data()) == 0);
+    {
+        // the same rows as packed rows of two cameras: the same keys up to the camera bits
+        std::vector<int64_t> cams(N), pids(n_isects);
+        std::vector<int32_t> pflat(n_isects);
+        for (uint32_t i = 0; i < N; ++i)
+            cams[i] = i & 1;
+        CHECK(orc_intersect_tile_emit_packed(N, means2d.data(), radii.data(), depths.data(), cams.data(), cum.data(),
+                                             tile, tw, th, pids.data(), pflat.data()) == 0);
+        const int64_t low = (1ll << (32 + orc_tile_n_bits(tw * th))) - 1;
+        for (int64_t i = 0; i < n_isects; ++i)
+            CHECK((pids[i] & low) == ids[i] && pflat[i] == flat[i] && (pids[i] >> (32 + orc_tile_n_bits(tw * th))) == (flat[i] & 1));
+    }
     CHECK(orc_radix_sort_pairs(n_isects, ids.data(), flat.data(), 32 + orc_tile_n_bits(tw * th) + 1, ids_sorted.data(),
                                flat_sorted.data()) == 0);
     CHECK(orc_intersect_offset(n_isects, ids_sorted.data(), 1, tw, th, offsets.data()) == 0);
