@@ -75,48 +75,42 @@ GSX_HD float rsqrt(float x) {
     return y;
 }
 
-// e^x.  Cody-Waite reduction, degree-5 Horner core, exponent applied through the bit pattern.
-// x < -87 returns 0 (the true value is below 1.7e-38), x > 88.7 returns +inf.
+// e^x.  n = round(x log2 e) through the 1.5 * 2^23 addition (the integer is then also the low mantissa bits of t),
+// Cody-Waite reduction r = x - n ln 2 in two exact-product steps, a degree-6 polynomial in Horner form (minimax on
+// |r| <= ln 2 / 2 with the constant and linear coefficients fixed at 1: 3.4e-9 relative), scaling by 2^n.
+// Below 1 unit in the last place on the whole range (all 2.1e9 arguments compared with the double-precision
+// exponential).  x < -87 returns 0 (the true value is below 1.7e-38), x > 88.7 returns +inf.
+GSX_HD float exp_core(float x, float* t_out) {
+    const float t = fma(x, 1.44269504088896341f, 12582912.0f);
+    const float n = t - 12582912.0f;
+    float r = fma(n, -0.693359375f, x);
+    r = fma(n, 2.12194440e-4f, r);
+    float p = 1.3855284778e-3f;
+    p = fma(p, r, 8.3686923608e-3f);
+    p = fma(p, r, 4.1667662561e-2f);
+    p = fma(p, r, 1.6666521132e-1f);
+    p = fma(p, r, 4.9999997020e-1f);
+    p = fma(p, r, 1.0f);
+    *t_out = t;
+    return fma(p, r, 1.0f); // in (0.70, 1.42)
+}
 GSX_HD float exp(float x) {
     if (x < -87.0f)
         return 0.0f;
     if (x > 88.7f)
         return u2f(0x7f800000u);
-    const float n = __builtin_rintf(x * 1.44269504088896341f);
-    float r = fma(n, -0.693359375f, x);
-    r = fma(n, 2.12194440e-4f, r);
-    float p = 1.9875691500e-4f;
-    p = fma(p, r, 1.3981999507e-3f);
-    p = fma(p, r, 8.3334519073e-3f);
-    p = fma(p, r, 4.1665795894e-2f);
-    p = fma(p, r, 1.6666665459e-1f);
-    p = fma(p, r, 5.0000001201e-1f);
-    const float z = r * r;
-    float y = fma(p, z, r) + 1.0f;
-    // y in (0.70, 1.42); scale by 2^n in two exact steps so that n = 128 does not overflow early.
-    const int ni = (int)n;
-    const int n1 = ni >> 1;
-    const int n2 = ni - n1;
-    y = y * u2f((uint32_t)(n1 + 127) << 23);
-    y = y * u2f((uint32_t)(n2 + 127) << 23);
-    return y;
+    float t;
+    const float y = exp_core(x, &t);
+    return __builtin_ldexpf(y, (int)(f2u(t) - 0x4B400000u)); // exact scaling by 2^n, n in [-126, 128]
 }
 
-// gsx::exp restricted to -87 <= x <= 0, where its two range tests never fire and its two-step scaling is a single
-// exact multiplication by 2^n (n in [-126, 0]): the same bits for fewer instructions.
+// gsx::exp restricted to -87 <= x <= 0, where its two range tests never fire and the result is a normal number, so
+// that the scaling is an addition of n to the exponent field (t's low bits, shifted): the same bits for fewer
+// instructions.
 GSX_HD float exp_nonpos(float x) {
-    const float n = __builtin_rintf(x * 1.44269504088896341f);
-    float r = fma(n, -0.693359375f, x);
-    r = fma(n, 2.12194440e-4f, r);
-    float p = 1.9875691500e-4f;
-    p = fma(p, r, 1.3981999507e-3f);
-    p = fma(p, r, 8.3334519073e-3f);
-    p = fma(p, r, 4.1665795894e-2f);
-    p = fma(p, r, 1.6666665459e-1f);
-    p = fma(p, r, 5.0000001201e-1f);
-    const float z = r * r;
-    const float y = fma(p, z, r) + 1.0f;
-    return y * u2f((uint32_t)((int)n + 127) << 23);
+    float t;
+    const float y = exp_core(x, &t);
+    return u2f((f2u(t) << 23) + f2u(y));
 }
 
 // natural log of a positive normal float (Cephes logf scheme).
