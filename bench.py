@@ -468,7 +468,7 @@ def run_cpp_step(args, gsx, sc, viewmat, Kmat, W, H, gt, dev, steps=None, warmup
     assert cs.lists_error() == (0, 0) and cs.steps_held == 0
     return {"it_per_s": round(steps / elapsed, 3), "ms_per_step": round(1e3 * elapsed / steps, 4),
             "first_loss": first, "n_isects": int(cs.n_isects()),
-            "what": "gsx::TrainStep::step called from a C++ loop: the 18 launches of the default workload"}
+            "what": "gsx::TrainStep::step called from a C++ loop: the 17 launches of the default workload"}
 
 
 def run_fastgs(args, gsx, sc, cam, dev):

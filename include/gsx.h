@@ -536,6 +536,18 @@ GSX_API int gsx_photometric_loss_backward_finish(uint32_t H, uint32_t W, float l
                                                  const float* dm_dsigma1_sq, const float* dm_dsigma12,
                                                  const float* l1_partials, const float* ssim_partials,
                                                  float* loss_out, float* v_render_hwc, void* stream);
+/* gsx_photometric_loss_backward(_finish, with loss_out != NULL) and gsx_tile_order by tile_cost in one launch (no
+ * counterpart in the reference): one workgroup more than the image needs sorts the tiles for the backward rasterizer
+ * that follows, so that the order costs neither a launch nor a second stream with its events.  tile_cost: u32
+ * [tile_width * tile_height] (the tile_walk of gsx_rasterize_records_fwd), tile_order: as gsx_tile_order writes it.
+ * loss_out, l1_partials, ssim_partials: nullable together (no loss value then). */
+GSX_API int gsx_photometric_loss_backward_order(uint32_t H, uint32_t W, float lambda_dssim, const float* render_hwc,
+                                                const float* gt_chw, const float* dm_dmu1,
+                                                const float* dm_dsigma1_sq, const float* dm_dsigma12,
+                                                const float* l1_partials, const float* ssim_partials,
+                                                float* loss_out, float* v_render_hwc, uint32_t tile_width,
+                                                uint32_t tile_height, const uint32_t* tile_cost,
+                                                uint32_t* tile_order, void* stream);
 /* v_render [H,W,3] = d loss / d render: L1 sign term + lambda * SSIM term (dL_dimg_ssim is
  * gsx_fusedssim_backward's output for dL_dmap = -lambda / count on the valid crop, 0 elsewhere), passed through
  * the clamp VJP (zero where render < 0 or > 1) and the CHW -> HWC permute. */

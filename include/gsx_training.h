@@ -123,7 +123,7 @@ namespace gsx {
             float scale_reg = 0.f, opacity_reg = 0.f;  // trainer.cpp:136-174; 0 = off
             int sh_degree = 3;                     // active degree
             bool freeze_shN_early = false;         // fused_adam.cpp:69-70 (true: the product's schedule)
-            bool overlap = true;                   // SH / record pass and tile orders on a second stream
+            bool overlap = true;                   // SH / record pass, tile table and list-length tile order on a second stream
             bool order_tiles = true;               // rasterize the dearest tiles first
             int64_t initial_pair_capacity = 0;     // room for (Gaussian, tile) pairs before the first count; 0 = auto
         };

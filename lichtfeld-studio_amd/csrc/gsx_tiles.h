@@ -42,4 +42,72 @@ __device__ __forceinline__ uint32_t packed_rect_count(uint32_t hi) {
     return (((hi >> 24) & 255u) - ((hi >> 8) & 255u)) * (((hi >> 16) & 255u) - (hi & 255u));
 }
 
+// ---- visiting order of the tiles for the rasterizers: longest lists first -----------------------------------------
+// The rasterizers' workgroups are handed out in launch order as slots free up; with the long lists first the short
+// ones fill the end of the launch instead of a few long ones running on alone.  Counting sort on a logarithmic
+// length class (16 classes per octave), descending; the order inside a class is whatever the atomics give (no
+// result depends on the order tiles are visited in).
+static constexpr uint32_t kLenClasses = 512;
+__device__ __forceinline__ uint32_t tile_len_class(uint32_t len) {
+    if (len == 0)
+        return 0;
+    const uint32_t e = 31u - (uint32_t)__clz((int)len);
+    const uint32_t m = e >= 4 ? (len >> (e - 4)) & 15u : (len << (4 - e)) & 15u; // four bits below the leading one
+    return min(e * 16u + m + 1u, kLenClasses - 1u);
+}
+
+// The whole sort by one workgroup of THREADS lanes (a multiple of 64, at most 1024); every lane of the workgroup
+// calls it.  A tile's cost is tile_cost[tile], or with tile_cost == nullptr the length of its list in tile_offsets.
+// cursor: LDS [kLenClasses], wave_total: LDS [16].
+template <uint32_t THREADS>
+__device__ __forceinline__ void tile_order_block(uint32_t n_tiles, uint32_t n_isects,
+                                                 const int32_t* __restrict__ tile_offsets,
+                                                 const uint32_t* __restrict__ tile_cost,
+                                                 uint32_t* __restrict__ tile_order, uint32_t* cursor,
+                                                 uint32_t* wave_total) {
+    static_assert(THREADS % 64 == 0 && THREADS <= 1024 && kLenClasses % 64 == 0, "whole waves");
+    const uint32_t t = threadIdx.x, lane = t & 63u, w = t >> 6;
+    for (uint32_t c = t; c < kLenClasses; c += THREADS)
+        cursor[c] = 0;
+    __syncthreads();
+    auto length = [&](uint32_t tile) {
+        if (tile_cost != nullptr)
+            return tile_cost[tile];
+        const uint32_t end =
+            (tile + 1 < n_tiles || n_isects == kCountInOffsets) ? (uint32_t)tile_offsets[tile + 1] : n_isects;
+        return end - (uint32_t)tile_offsets[tile];
+    };
+    for (uint32_t tile = t; tile < n_tiles; tile += THREADS)
+        atomicAdd(&cursor[tile_len_class(length(tile))], 1u);
+    __syncthreads();
+    // first position of every class, dearest class first: an exclusive scan over the classes in descending order,
+    // THREADS classes at a time (virtual index v owns class kLenClasses - 1 - v)
+    uint32_t carry = 0;
+    for (uint32_t base = 0; base < kLenClasses; base += THREADS) {
+        const uint32_t v = base + t;
+        const uint32_t c = kLenClasses - 1u - v;
+        const uint32_t n = v < kLenClasses ? cursor[c] : 0u;
+        uint32_t incl = n;
+#pragma unroll
+        for (uint32_t off = 1; off < 64; off <<= 1) {
+            const uint32_t up = (uint32_t)__shfl_up((int)incl, off, 64);
+            if (lane >= off)
+                incl += up;
+        }
+        if (lane == 63)
+            wave_total[w] = incl;
+        __syncthreads();
+        uint32_t before = carry;
+        for (uint32_t k = 0; k < w; ++k)
+            before += wave_total[k];
+        if (v < kLenClasses)
+            cursor[c] = before + incl - n;
+        for (uint32_t k = 0; k < THREADS / 64; ++k)
+            carry += wave_total[k];
+        __syncthreads();
+    }
+    for (uint32_t tile = t; tile < n_tiles; tile += THREADS)
+        tile_order[atomicAdd(&cursor[tile_len_class(length(tile))], 1u)] = tile;
+}
+
 } // namespace gsx

@@ -3,8 +3,9 @@
 // optimizers/fused_adam.cpp:22-95) driven from C++ over the fused entry points of gsx.h.  LibTorch provides the
 // tensors, the current stream and a second stream; every kernel is this library's.  Launch order per step:
 //   activations + UT projection | SH colours + raster records (second stream) | tile lists (9 launches) |
-//   tile order | rasterize forward | photometric loss forward | tile order by cost (second stream) |
-//   photometric loss backward (+ loss value) | rasterize backward | epilogue + SH backward + activation VJPs + Adam
+//   tile order | rasterize forward | photometric loss forward |
+//   photometric loss backward (+ loss value, + tile order by cost) | rasterize backward |
+//   epilogue + SH backward + activation VJPs + Adam
 #include "gsx_training.h"
 
 #include <c10/core/DeviceGuard.h>
@@ -33,7 +34,7 @@ namespace gsx {
         int W = 0, H = 0;
         uint32_t tw = 0, th = 0;
         hipStream_t side = nullptr;
-        hipEvent_t ev_fork = nullptr, ev_join = nullptr, ev_loss_fork = nullptr, ev_order_join = nullptr;
+        hipEvent_t ev_fork = nullptr, ev_join = nullptr;
         // per Gaussian
         torch::Tensor opacities, scales, quats, radii, means2d, depths, colors, records, accum;
         // per image
@@ -41,7 +42,7 @@ namespace gsx {
         // tile lists
         torch::Tensor lists_ws, flat_out, n_pinned, hold_pinned;
         uint32_t* lists_error = nullptr;  // device u32 [2] inside lists_ws
-        bool cap_confirmed = false, have_walk = false, order_due = false, order_pending = false;
+        bool cap_confirmed = false, have_walk = false, order_due = false;
         const void *walk_viewmat = nullptr, *walk_K = nullptr;
         int walk_W = 0, walk_H = 0;
         const float* gt = nullptr;
@@ -95,7 +96,7 @@ namespace gsx {
         m.n_pinned = torch::zeros({1}, torch::TensorOptions().dtype(torch::kLong).pinned_memory(true));
         m.hold_pinned = torch::zeros({1}, torch::TensorOptions().dtype(torch::kLong).pinned_memory(true));
         m.side = c10::hip::getStreamFromPool(/*isHighPriority=*/false, m.device.index()).stream();
-        for (hipEvent_t* e : {&m.ev_fork, &m.ev_join, &m.ev_loss_fork, &m.ev_order_join})
+        for (hipEvent_t* e : {&m.ev_fork, &m.ev_join})
             hip_ok(hipEventCreateWithFlags(e, hipEventDisableTiming));
     }
 
@@ -106,7 +107,7 @@ namespace gsx {
         // over before the allocator hands them to somebody else
         if (impl_->side != nullptr)
             (void)hipStreamSynchronize(impl_->side);
-        for (hipEvent_t e : {impl_->ev_fork, impl_->ev_join, impl_->ev_loss_fork, impl_->ev_order_join})
+        for (hipEvent_t e : {impl_->ev_fork, impl_->ev_join})
             if (e != nullptr)
                 (void)hipEventDestroy(e);
     }
@@ -124,7 +125,7 @@ namespace gsx {
         const int64_t tiles = (int64_t)m.tw * m.th;
         m.offsets_full = torch::empty({tiles + 1}, io);  // the last entry: the pair count
         m.tile_order = torch::empty({tiles}, io), m.tile_walk = torch::empty({tiles}, io);
-        m.have_walk = false, m.order_due = false, m.order_pending = false;
+        m.have_walk = false, m.order_due = false;
         render = torch::empty({1, H, W, 3}, fo), alpha = torch::empty({1, H, W, 1}, fo);
         last_ids = torch::empty({1, H, W}, io);
         m.v_render = torch::empty({1, H, W, 3}, fo), m.v_alpha = torch::zeros({1, H, W, 1}, fo);
@@ -219,10 +220,6 @@ namespace gsx {
         Impl& m = *impl_;
         hipStream_t s = m.main();
         const bool two = opt_.overlap;
-        if (m.order_pending) {
-            hip_ok(hipStreamWaitEvent(s, m.ev_order_join, 0));
-            m.order_pending = false;
-        }
         ensure_image(H, W);
         ensure_lists();
         m.viewmat = f(viewmat), m.Kmat = f(Kmat);
@@ -316,23 +313,17 @@ namespace gsx {
         // loss = (1 - lambda) L1 + lambda (1 - SSIM_valid) on clamp(render) (rasterizer.cpp:205, trainer.cpp:107-134)
         ok(gsx_photometric_loss_forward(Hu, Wu, 0.01f * 0.01f, 0.03f * 0.03f, f(render), f(gt_chw), f(m.dm1), f(m.dm2),
                                         f(m.dm3), f(m.l1_partials), f(m.ssim_partials), s));
-        if (opt_.overlap && m.order_due) {  // the order for the backward pass, beside the loss kernels
-            hip_ok(hipEventRecord(m.ev_loss_fork, s));
-            hip_ok(hipStreamWaitEvent(m.side, m.ev_loss_fork, 0));
-            ok(gsx_tile_order(GSX_COUNT_IN_OFFSETS, nullptr, u32(m.tile_walk), m.tw, m.th, u32(m.tile_order), m.side));
-            hip_ok(hipEventRecord(m.ev_order_join, m.side));
-            m.order_due = false, m.order_pending = true;
-        }
-        ok(gsx_photometric_loss_backward_finish(Hu, Wu, opt_.lambda_dssim, f(render), f(gt_chw), f(m.dm1), f(m.dm2),
-                                                f(m.dm3), f(m.l1_partials), f(m.ssim_partials), f(loss_out),
-                                                f(m.v_render), s));
         if (m.order_due) {
-            ok(gsx_tile_order(GSX_COUNT_IN_OFFSETS, nullptr, u32(m.tile_walk), m.tw, m.th, u32(m.tile_order), s));
+            // the order for the backward pass rides on the loss kernel (one workgroup more): a fork and a join of the
+            // second stream would cost this one ~14 us of idle time
+            ok(gsx_photometric_loss_backward_order(Hu, Wu, opt_.lambda_dssim, f(render), f(gt_chw), f(m.dm1), f(m.dm2),
+                                                   f(m.dm3), f(m.l1_partials), f(m.ssim_partials), f(loss_out),
+                                                   f(m.v_render), m.tw, m.th, u32(m.tile_walk), u32(m.tile_order), s));
             m.order_due = false;
-        }
-        if (m.order_pending) {
-            hip_ok(hipStreamWaitEvent(s, m.ev_order_join, 0));
-            m.order_pending = false;
+        } else {
+            ok(gsx_photometric_loss_backward_finish(Hu, Wu, opt_.lambda_dssim, f(render), f(gt_chw), f(m.dm1),
+                                                    f(m.dm2), f(m.dm3), f(m.l1_partials), f(m.ssim_partials),
+                                                    f(loss_out), f(m.v_render), s));
         }
         ok(gsx_rasterize_bwd_accumulate(1, m.N, GSX_COUNT_IN_OFFSETS, m.records.data_ptr(), nullptr, 3, f(m.bg),
                                         nullptr, Wu, Hu, 16, m.viewmat, m.Kmat, i32(m.offsets_full), i32(m.flat_out),

@@ -264,62 +264,14 @@ __global__ void __launch_bounds__(256) tile_emit_kernel(uint32_t n, uint32_t N, 
     }
 }
 
-// ---- visiting order of the tiles for the rasterizers: longest lists first -----------------------------------------
-// The rasterizers' workgroups are handed out in launch order as slots free up; with the long lists first the short
-// ones fill the end of the launch instead of a few long ones running on alone.  Counting sort on a logarithmic
-// length class (16 classes per octave), descending; the order inside a class is whatever the atomics give (no
-// result depends on the order tiles are visited in).
-static constexpr uint32_t kLenClasses = 512;
-__device__ __forceinline__ uint32_t tile_len_class(uint32_t len) {
-    if (len == 0)
-        return 0;
-    const uint32_t e = 31u - (uint32_t)__clz((int)len);
-    const uint32_t m = e >= 4 ? (len >> (e - 4)) & 15u : (len << (4 - e)) & 15u; // four bits below the leading one
-    return min(e * 16u + m + 1u, kLenClasses - 1u);
-}
-
+// ---- visiting order of the tiles for the rasterizers: longest lists first (tile_order_block, gsx_tiles.h) ---------
 __global__ void __launch_bounds__(1024) tile_order_kernel(uint32_t n_tiles, uint32_t n_isects,
                                                            const int32_t* __restrict__ tile_offsets,
                                                            const uint32_t* __restrict__ tile_cost /*nullable*/,
                                                            uint32_t* __restrict__ tile_order) {
     __shared__ uint32_t cursor[kLenClasses];
-    for (uint32_t c = threadIdx.x; c < kLenClasses; c += 1024)
-        cursor[c] = 0;
-    __syncthreads();
-    auto length = [&](uint32_t t) {
-        if (tile_cost != nullptr)
-            return tile_cost[t];
-        const uint32_t end = (t + 1 < n_tiles || n_isects == kCountInOffsets) ? (uint32_t)tile_offsets[t + 1] : n_isects;
-        return end - (uint32_t)tile_offsets[t];
-    };
-    for (uint32_t t = threadIdx.x; t < n_tiles; t += 1024)
-        atomicAdd(&cursor[tile_len_class(length(t))], 1u);
-    __syncthreads();
-    { // first position of every class, dearest class first: an exclusive scan over the classes in descending order
-        __shared__ uint32_t wave_total[kLenClasses / 64];
-        const uint32_t t = threadIdx.x, lane = t & 63u, w = t >> 6;
-        const uint32_t c = kLenClasses - 1u - t; // thread t owns class c (t < kLenClasses)
-        const uint32_t n = t < kLenClasses ? cursor[c] : 0u;
-        uint32_t incl = n;
-#pragma unroll
-        for (uint32_t off = 1; off < 64; off <<= 1) {
-            const uint32_t up = (uint32_t)__shfl_up((int)incl, off, 64);
-            if (lane >= off)
-                incl += up;
-        }
-        if (lane == 63 && w < kLenClasses / 64)
-            wave_total[w] = incl;
-        __syncthreads();
-        if (t < kLenClasses) {
-            uint32_t before = 0;
-            for (uint32_t k = 0; k < w; ++k)
-                before += wave_total[k];
-            cursor[c] = before + incl - n;
-        }
-    }
-    __syncthreads();
-    for (uint32_t t = threadIdx.x; t < n_tiles; t += 1024)
-        tile_order[atomicAdd(&cursor[tile_len_class(length(t))], 1u)] = t;
+    __shared__ uint32_t wave_total[16];
+    tile_order_block<1024>(n_tiles, n_isects, tile_offsets, tile_cost, tile_order, cursor, wave_total);
 }
 
 // What a forward pass leaves per pixel (alpha, position of the last contributor) gives the tile cost too: how far

@@ -25,6 +25,7 @@
 // reciprocal products and its sums contracted).  Results do not depend on the strip geometry and equal the CPU
 // checker's, which fixes the same evaluation, to the last bit.
 #include "gsx_common.h"
+#include "gsx_tiles.h"
 
 namespace gsx {
 
@@ -578,7 +579,18 @@ __global__ void __launch_bounds__(256) photometric_bwd_kernel(int rows_per_strip
                                                                float lambda_dssim,
                                                                const float* __restrict__ l1_partials,
                                                                const float* __restrict__ ssim_partials,
-                                                               uint32_t n_partials, float* __restrict__ loss_out) {
+                                                               uint32_t n_partials, float* __restrict__ loss_out,
+                                                               uint32_t n_tiles,
+                                                               const uint32_t* __restrict__ tile_cost,
+                                                               uint32_t* __restrict__ tile_order) {
+    if (tile_order != nullptr && blockIdx.x == gridDim.x - 1u) {
+        // one workgroup more than the image needs: it sorts the tiles by what they cost the forward rasterizer, for
+        // the backward rasterizer that follows this launch (no launch, stream or event of its own)
+        __shared__ uint32_t cursor[kLenClasses];
+        __shared__ uint32_t wave_total[16];
+        tile_order_block<256>(n_tiles, kCountInOffsets, nullptr, tile_cost, tile_order, cursor, wave_total);
+        return;
+    }
     __shared__ float rows[4][3][kRowFloats];
     if (loss_out != nullptr && blockIdx.x == 0) {
         // the loss value itself, which only gets reported: the forward kernel's partial sums are complete when this
@@ -779,7 +791,8 @@ extern "C" int gsx_photometric_loss_forward(uint32_t H, uint32_t W, float C1, fl
 static int photometric_backward(uint32_t H, uint32_t W, float lambda_dssim, const float* render_hwc,
                                 const float* gt_chw, const float* dm_dmu1, const float* dm_dsigma1_sq,
                                 const float* dm_dsigma12, float* v_render_hwc, const float* l1_partials,
-                                const float* ssim_partials, float* loss_out, void* stream) {
+                                const float* ssim_partials, float* loss_out, uint32_t n_tiles,
+                                const uint32_t* tile_cost, uint32_t* tile_order, void* stream) {
     if ((uint64_t)H * W == 0)
         return GSX_OK;
     GSX_REQUIRE(render_hwc && gt_chw && dm_dmu1 && dm_dsigma1_sq && dm_dsigma12 && v_render_hwc,
@@ -791,10 +804,12 @@ static int photometric_backward(uint32_t H, uint32_t W, float lambda_dssim, cons
     const float ssim_scale = -lambda_dssim / count;
     const float l1_scale = (1.f - lambda_dssim) / (3.f * (float)H * (float)W);
     const int rows = strip_rows(H, W, 3);
-    hipLaunchKernelGGL(photometric_bwd_kernel, dim3(xcd_grid(cdiv(3u * strip_count(H, W, (uint32_t)rows), 4))),
-                       dim3(256), 0, (hipStream_t)stream, rows, (int)H, (int)W, ssim_scale,
-                       l1_scale, render_hwc, gt_chw, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, v_render_hwc, lambda_dssim,
-                       l1_partials, ssim_partials, gsx_photometric_partials(H, W), loss_out);
+    // (the strips' workgroups find their place from their own index and the strip count, not from the grid size)
+    const uint32_t blocks = xcd_grid(cdiv(3u * strip_count(H, W, (uint32_t)rows), 4)) + (tile_order ? 1u : 0u);
+    hipLaunchKernelGGL(photometric_bwd_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, rows, (int)H, (int)W,
+                       ssim_scale, l1_scale, render_hwc, gt_chw, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, v_render_hwc,
+                       lambda_dssim, l1_partials, ssim_partials, gsx_photometric_partials(H, W), loss_out, n_tiles,
+                       tile_cost, tile_order);
     GSX_LAUNCH_CHECK();
     return GSX_OK;
 }
@@ -803,7 +818,7 @@ extern "C" int gsx_photometric_loss_backward(uint32_t H, uint32_t W, float lambd
                                              const float* gt_chw, const float* dm_dmu1, const float* dm_dsigma1_sq,
                                              const float* dm_dsigma12, float* v_render_hwc, void* stream) {
     return photometric_backward(H, W, lambda_dssim, render_hwc, gt_chw, dm_dmu1, dm_dsigma1_sq, dm_dsigma12,
-                                v_render_hwc, nullptr, nullptr, nullptr, stream);
+                                v_render_hwc, nullptr, nullptr, nullptr, 0, nullptr, nullptr, stream);
 }
 
 extern "C" int gsx_photometric_loss_backward_finish(uint32_t H, uint32_t W, float lambda_dssim,
@@ -814,5 +829,23 @@ extern "C" int gsx_photometric_loss_backward_finish(uint32_t H, uint32_t W, floa
                                                     float* v_render_hwc, void* stream) {
     GSX_REQUIRE(loss_out != nullptr, GSX_ERR_INVALID_ARGUMENT, "photometric_loss_backward_finish: loss_out is null");
     return photometric_backward(H, W, lambda_dssim, render_hwc, gt_chw, dm_dmu1, dm_dsigma1_sq, dm_dsigma12,
-                                v_render_hwc, l1_partials, ssim_partials, loss_out, stream);
+                                v_render_hwc, l1_partials, ssim_partials, loss_out, 0, nullptr, nullptr, stream);
+}
+
+extern "C" int gsx_photometric_loss_backward_order(uint32_t H, uint32_t W, float lambda_dssim,
+                                                   const float* render_hwc, const float* gt_chw,
+                                                   const float* dm_dmu1, const float* dm_dsigma1_sq,
+                                                   const float* dm_dsigma12, const float* l1_partials,
+                                                   const float* ssim_partials, float* loss_out,
+                                                   float* v_render_hwc, uint32_t tile_width, uint32_t tile_height,
+                                                   const uint32_t* tile_cost, uint32_t* tile_order, void* stream) {
+    const uint64_t n_tiles = (uint64_t)tile_width * tile_height;
+    GSX_REQUIRE(n_tiles > 0 && n_tiles < (1ull << 31), GSX_ERR_INVALID_ARGUMENT,
+                "photometric_loss_backward_order: %u x %u tiles", tile_width, tile_height);
+    GSX_REQUIRE(tile_cost && tile_order, GSX_ERR_INVALID_ARGUMENT, "photometric_loss_backward_order: null tile tensor");
+    if ((uint64_t)H * W == 0) // no image, no launch to ride on
+        return gsx_tile_order(GSX_COUNT_IN_OFFSETS, nullptr, tile_cost, tile_width, tile_height, tile_order, stream);
+    return photometric_backward(H, W, lambda_dssim, render_hwc, gt_chw, dm_dmu1, dm_dsigma1_sq, dm_dsigma12,
+                                v_render_hwc, l1_partials, ssim_partials, loss_out, (uint32_t)n_tiles, tile_cost,
+                                tile_order, stream);
 }

@@ -477,15 +477,16 @@ class TrainStep:
             if self.side is None:
                 if finish:
                     self._run("photometric_loss_finish", lb.gsx_photometric_loss_finish, *fin, s)
-            else:  # the value is only reported: its reduction runs beside the backward pass
+            elif finish:  # the value is only reported: its reduction runs beside the backward pass
                 self.ev_loss_fork.record(torch.cuda.current_stream(self.dev))
                 self.side.wait_event(self.ev_loss_fork)
                 with torch.cuda.stream(self.side):
                     self._order_on_side_stream()  # the backward pass waits for this one, not for the reduction
-                    if finish:
-                        self._run("photometric_loss_finish", lb.gsx_photometric_loss_finish, *fin, self._stream())
-                        self.ev_loss_join.record(self.side)
-                self.loss_pending = finish
+                    self._run("photometric_loss_finish", lb.gsx_photometric_loss_finish, *fin, self._stream())
+                    self.ev_loss_join.record(self.side)
+                self.loss_pending = True
+            # (finish = False: the loss kernel of backward() forms the value and the tile order on its way - a fork
+            # and a join of the second stream cost the current one ~14 us of idle time, more than either is worth)
             return self.loss_out
         self._run("image_from_render", lb.gsx_image_from_render, c_u32(H), c_u32(W), _p(self.render), _p(gt_chw), _p(self.image),
                                        _p(self.l1_partials), s)
@@ -507,9 +508,15 @@ class TrainStep:
         P, A, J, G, V = self.params, self.act, self.proj, self.grads, self.v_act
         dimg = None
         if self.fused_loss and getattr(self, "_loss_due", False):
-            self._run("photometric_loss_backward", lb.gsx_photometric_loss_backward_finish, c_u32(H), c_u32(W),
-                      c_f(self.lambda_dssim), _p(self.render), _p(self.gt), _p(self.dm1), _p(self.dm2), _p(self.dm3),
-                      _p(self.l1_partials), _p(self.ssim_partials), _p(self.loss_out), _p(self.v_render), s)
+            loss_args = (c_u32(H), c_u32(W), c_f(self.lambda_dssim), _p(self.render), _p(self.gt), _p(self.dm1),
+                         _p(self.dm2), _p(self.dm3), _p(self.l1_partials), _p(self.ssim_partials), _p(self.loss_out),
+                         _p(self.v_render))
+            if self._order_due is not None:  # one workgroup more sorts the tiles for the backward rasterizer
+                self._run("photometric_loss_backward", lb.gsx_photometric_loss_backward_order, *loss_args,
+                          c_u32(self.tw), c_u32(self.th), _p(self.tile_walk), _p(self.tile_order), s)
+                self._order_due = None
+            else:
+                self._run("photometric_loss_backward", lb.gsx_photometric_loss_backward_finish, *loss_args, s)
             self._loss_due = False
         elif self.fused_loss:
             self._run("photometric_loss_backward", lb.gsx_photometric_loss_backward, c_u32(H), c_u32(W),

@@ -161,6 +161,67 @@ def test_fused_loss_equals_separate_kernels(gsx, cuda, W, H):
     assert np.array_equal(va == 0, vb == 0)  # the clamp mask
 
 
+@pytest.mark.parametrize("W,H,tw,th", [(309, 205, 401, 10), (64, 48, 4, 3), (9, 7, 1, 1), (1237, 822, 78, 52)])
+def test_loss_backward_that_also_orders_the_tiles(gsx, cuda, W, H, tw, th):
+    """gsx_photometric_loss_backward_order = gsx_photometric_loss_backward_finish (d loss / d render and the loss
+    value bit for bit) + gsx_tile_order by cost (a permutation of the tiles, cost classes falling), in one launch;
+    tile grids of every size beside images of every size (the extra workgroup does not depend on the image)"""
+    from lichtfeld_studio_amd._lib import c_f, c_p, c_u32, check, lib
+    L = lib()
+    g = torch.Generator().manual_seed(W * 7 + tw)
+    render = (torch.rand((H, W, 3), generator=g) * 1.6 - 0.3).to(cuda)
+    gt = torch.rand((3, H, W), generator=g).to(cuda)
+    dm = [torch.empty((3, H, W), dtype=torch.float32, device=cuda) for _ in range(3)]
+    n_part = L.gsx_photometric_partials(c_u32(H), c_u32(W))
+    l1p, ssp = (torch.empty(n_part, dtype=torch.float32, device=cuda) for _ in range(2))
+    s = c_p(torch.cuda.current_stream(cuda).cuda_stream)
+    P = lambda t: c_p(t.data_ptr())
+    check(L.gsx_photometric_loss_forward(c_u32(H), c_u32(W), c_f(1e-4), c_f(9e-4), P(render), P(gt), P(dm[0]),
+                                         P(dm[1]), P(dm[2]), P(l1p), P(ssp), s))
+    rng = np.random.default_rng(tw * 31 + th)
+    T = tw * th
+    cost = np.concatenate([np.zeros(T // 10, np.int64), rng.integers(0, 40, T - T // 10 - T // 5),
+                           rng.integers(0, 1 << 21, T // 5)])[:T]
+    cost = np.resize(cost, T)
+    rng.shuffle(cost)
+    cost_d = torch.from_numpy(cost.astype(np.int32)).to(cuda)
+    out = {}
+    for name in ("finish", "order"):
+        v = torch.full((H, W, 3), 7.0, dtype=torch.float32, device=cuda)
+        loss = torch.full((3,), -1.0, dtype=torch.float32, device=cuda)
+        order = torch.full((T,), -1, dtype=torch.int32, device=cuda)
+        common = (c_u32(H), c_u32(W), c_f(0.2), P(render), P(gt), P(dm[0]), P(dm[1]), P(dm[2]), P(l1p), P(ssp),
+                  P(loss), P(v))
+        if name == "finish":
+            check(L.gsx_photometric_loss_backward_finish(*common, s))
+        else:
+            check(L.gsx_photometric_loss_backward_order(*common, c_u32(tw), c_u32(th), P(cost_d), P(order), s))
+        torch.cuda.synchronize()
+        out[name] = (v.cpu().numpy(), loss.cpu().numpy(), order.cpu().numpy().astype(np.int64))
+    assert np.array_equal(out["finish"][0].view(np.int32), out["order"][0].view(np.int32))
+    assert np.array_equal(out["finish"][1].view(np.int32), out["order"][1].view(np.int32))
+    assert (out["finish"][0] != 0).any() and np.all(out["finish"][2] == -1)
+    o = out["order"][2]
+    assert np.array_equal(np.sort(o), np.arange(T))
+
+    def klass(n):  # 16 classes per octave
+        if n == 0:
+            return 0
+        e = int(n).bit_length() - 1
+        m = (n >> (e - 4)) & 15 if e >= 4 else (n << (4 - e)) & 15
+        return e * 16 + m + 1
+    assert np.all(np.diff(np.array([klass(int(n)) for n in cost[o]])) <= 0)
+    # the same order (up to the order inside a class) as the kernel of its own
+    ref = torch.full((T,), -1, dtype=torch.int32, device=cuda)
+    from lichtfeld_studio_amd._lib import c_i64
+    check(L.gsx_tile_order(c_i64(-1), c_p(None), P(cost_d), c_u32(tw), c_u32(th), P(ref), s))
+    r = ref.cpu().numpy().astype(np.int64)
+    assert np.array_equal(np.array([klass(int(n)) for n in cost[o]]), np.array([klass(int(n)) for n in cost[r]]))
+    # null tile tensors are refused
+    with pytest.raises(gsx._lib.GsxError):
+        check(L.gsx_photometric_loss_backward_order(*common, c_u32(tw), c_u32(th), c_p(None), P(order), s))
+
+
 @pytest.mark.parametrize("n", [1, 255, 300_001, 3_000_000])
 def test_l1_regularization_kernels(gsx, orc, cuda, n):
     """gsx_exp_l1_regularization / gsx_sigmoid_l1_regularization: gradients added onto existing ones bit for bit as
