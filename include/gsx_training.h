@@ -109,7 +109,7 @@ namespace gsx::training {
 namespace gsx {
 
     // One training iteration over the fused entry points of gsx.h - what Trainer::train_step (trainer.cpp:599-875)
-    // + MCMC::step (mcmc.cpp:410-417) + FusedAdam::step (fused_adam.cpp:22-95) do for the --gut backend, as 18 kernel
+    // + MCMC::step (mcmc.cpp:410-417) + FusedAdam::step (fused_adam.cpp:22-95) do for the --gut backend, as 17 kernel
     // launches on two streams with every buffer allocated once and no host wait inside a step.  The caller keeps
     // the tensors (they are updated in place); `shs` holds sh0 | shN as one [N,K,3] tensor - sh0() / shN() are the
     // views a SplatData keeps instead of its two tensors.
