@@ -152,13 +152,15 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
         if (STATS && wave_active)
             n_skip += batch_size - n_sel;
 
-        for (uint32_t s = 0; s < n_sel; ++s) {
-            if (__builtin_amdgcn_ballot_w64(!done) == 0)
+        // A pixel leaves the loop when it is saturated, the wave when its last pixel has (the loop's own divergence:
+        // the lane mask shrinks with scalar instructions only; the counting instance keeps the wave-wide form)
+        for (uint32_t s = 0; s < n_sel && (STATS || !done); ++s) {
+            if (STATS && __builtin_amdgcn_ballot_w64(!done) == 0)
                 break; // this wave's 64 pixels are all saturated
             const uint32_t t = wave_list[s];
             if (STATS)
                 ++n_iter;
-            if (done)
+            if (STATS && done)
                 continue;
             if (STATS)
                 ++n_eval;
