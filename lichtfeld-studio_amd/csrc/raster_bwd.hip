@@ -92,7 +92,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
     __shared__ float acc_extra[XLDS ? kBwdBatch * NX : 1];
     __shared__ float cuts[kBwdBatch];
     __shared__ uint8_t lists[4][kBwdBatch];
-    __shared__ int32_t id_batch[NX > 0 ? kBwdBatch : 1]; // ids of the batch: only the extra channels' paths read them
+    __shared__ int32_t id_batch[kBwdBatch]; // ids of the batch: for the flush and the extra channels' paths
     // LDS sums of a batch: the 13 numbers in use of a row (slot 12 holds the opacity sum, the row's element 15)
     constexpr uint32_t kAccLds = 13;
     __shared__ __align__(16) float acc[kBwdBatch * kAccLds];
@@ -185,7 +185,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
         const uint32_t t_start = (uint32_t)max(0, batch_end - wave_bin_final);
         const uint32_t n_sel = (uint32_t)__builtin_amdgcn_readfirstlane((int)stage_and_select<kBwdBatch>(
             records, flatten_ids, batch_end, -1, (uint32_t)batch_size, tr, px, t_start,
-            t_start < (uint32_t)batch_size, stage, region, cuts, NX > 0 ? id_batch : nullptr, wave_list));
+            t_start < (uint32_t)batch_size, stage, region, cuts, id_batch, wave_list));
         for (uint32_t k = tr; k < kBwdBatch * kAccLds / 4; k += 256u)
             reinterpret_cast<float4*>(acc)[k] = make_float4(0.f, 0.f, 0.f, 0.f);
         __syncthreads();
@@ -343,7 +343,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             if ((int32_t)gi < batch_size) {
                 const float val = (k < 12u || k == 15u) ? acc[gi * kAccLds + min(k, 12u)] : 0.f;
                 if (val != 0.f)
-                    unsafeAtomicAdd(&gacc[(size_t)flatten_ids[batch_end - (int32_t)gi] * kAcc + k], val);
+                    unsafeAtomicAdd(&gacc[(size_t)id_batch[gi] * kAcc + k], val); // (slot gi = entry batch_end - gi)
             }
         }
         if (XLDS && (int32_t)tr < batch_size) {
