@@ -58,6 +58,7 @@ __global__ void __launch_bounds__(256) math_unary_kernel(int which, uint32_t n, 
     case 11: r = gsx::exp_nonpos(a); break;
     case 12: r = gsx::rcp_refined(a); break;
     case 13: r = gsx::rcp_approx(a); break;
+    case 15: r = gsx::min_limit(x2[i], a); break;
     default: break;
     }
     y[i] = r;
@@ -105,7 +106,8 @@ extern "C" int gsx_debug_math(int which, uint32_t n, const float* x, const float
     if (n == 0)
         return GSX_OK;
     GSX_REQUIRE(x && y, GSX_ERR_INVALID_ARGUMENT, "debug_math: null tensor");
-    GSX_REQUIRE(which < 7 || which >= 11 || x2 != nullptr, GSX_ERR_INVALID_ARGUMENT, "debug_math: second operand is null");
+    GSX_REQUIRE(which < 7 || (which >= 11 && which != 15) || x2 != nullptr, GSX_ERR_INVALID_ARGUMENT,
+                "debug_math: second operand is null");
     hipLaunchKernelGGL(gsx::math_unary_kernel, dim3(gsx::cdiv(n, 256)), dim3(256), 0, (hipStream_t)stream, which, n, x,
                        x2, y);
     GSX_LAUNCH_CHECK();

@@ -32,6 +32,15 @@ namespace gsx {
 GSX_HD float fma(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 GSX_HD float fmin(float a, float b) { return a < b ? a : b; } // operand order matters for NaN only
 GSX_HD float fmax(float a, float b) { return a > b ? a : b; }
+// min(limit, x) for a limit that is a number: the other operand if that is a number too and smaller, else the limit
+// (what CUDA's min / fminf gives: a NaN x yields the limit).  One v_min_f32 on the device; the same values on the host.
+GSX_HD float min_limit(float limit, float x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_fminf(limit, x);
+#else
+    return x < limit ? x : limit;
+#endif
+}
 GSX_HD float fabs(float a) { return __builtin_fabsf(a); }
 GSX_HD float floor(float a) { return __builtin_floorf(a); }
 GSX_HD float ceil(float a) { return __builtin_ceilf(a); }

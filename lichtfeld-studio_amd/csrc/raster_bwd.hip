@@ -237,7 +237,7 @@ __global__ void __launch_bounds__(256) rasterize_bwd_kernel(
             // (a lane below its cut-off may be far outside exp_nonpos's range: what it gets back is meaningless and
             // stays in that lane - it is not valid, and everything it feeds below goes through a select on `valid`)
             const float vis = gsx::exp_nonpos(power);
-            const float alpha = gsx::fmin(0.999f, a.w * vis);
+            const float alpha = gsx::min_limit(0.999f, a.w * vis);
             // (the reference's `power > 0` never fires: the power is -0.5 times a sum of squares)
             const bool opaque_enough = !(alpha < 1.f / 255.f);
             const uint64_t alpha_mask = __builtin_amdgcn_ballot_w64(opaque_enough);

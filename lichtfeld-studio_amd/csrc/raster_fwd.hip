@@ -188,7 +188,7 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
             // below the record's cut-off alpha < 1/255 whatever the rounding: decided without the exp
             const bool far_away = power < cuts[t];
             if (STATS) {
-                const bool contributes = !far_away && gsx::fmin(0.999f, a.w * gsx::exp_nonpos(power)) >= 1.f / 255.f;
+                const bool contributes = !far_away && gsx::min_limit(0.999f, a.w * gsx::exp_nonpos(power)) >= 1.f / 255.f;
                 const uint64_t act = __builtin_amdgcn_ballot_w64(true);
                 const uint64_t cm = __builtin_amdgcn_ballot_w64(contributes);
                 if (cm != 0 && (act & ((1ull << (tr & 63u)) - 1ull)) == 0) { // first active lane counts for the wave
@@ -200,7 +200,7 @@ __global__ void __launch_bounds__(256) rasterize_fwd_kernel(
             }
             if (__builtin_amdgcn_ballot_w64(!far_away) == 0 || far_away)
                 continue;
-            const float alpha = gsx::fmin(0.999f, a.w * gsx::exp_nonpos(power)); // cut <= power <= 0
+            const float alpha = gsx::min_limit(0.999f, a.w * gsx::exp_nonpos(power)); // cut <= power <= 0
             if (alpha < 1.f / 255.f)
                 continue;
             const float next_T = T * (1.0f - alpha);

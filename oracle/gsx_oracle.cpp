@@ -936,7 +936,7 @@ ORC_API int orc_rasterize_to_pixels_from_world_3dgs_fwd(
                     const vec3 gcrod = gsx::cross(grd, gro);
                     const float grayDist = gsx::dot(gcrod, gcrod);
                     const float power = -0.5f * grayDist;
-                    const float alpha = gsx::fmin(0.999f, opac * gsx::exp(power));
+                    const float alpha = gsx::min_limit(0.999f, opac * gsx::exp(power));
                     if (alpha < 1.f / 255.f)
                         continue;
                     const float next_T = T * (1.0f - alpha);
@@ -1036,7 +1036,7 @@ ORC_API int orc_rasterize_to_pixels_from_world_3dgs_bwd(
                     const float grayDist = gsx::dot(gcrod, gcrod);
                     const float power = -0.5f * grayDist;
                     const float vis = gsx::exp(power);
-                    const float alpha = gsx::fmin(0.999f, opac * vis);
+                    const float alpha = gsx::min_limit(0.999f, opac * vis);
                     if (power > 0.f || alpha < 1.f / 255.f)
                         continue;
 
@@ -1232,7 +1232,7 @@ ORC_API int orc_rasterize_bwd_f64(
                         const vec3 grdf = gsx::safe_normalize(gsx::mul(Mf, ray_df));
                         const vec3 cf = gsx::cross(grdf, grof);
                         const float powerf = -0.5f * gsx::dot(cf, cf);
-                        alphaf = gsx::fmin(0.999f, opacities[g] * gsx::exp(powerf));
+                        alphaf = gsx::min_limit(0.999f, opacities[g] * gsx::exp(powerf));
                         if (powerf > 0.f || alphaf < 1.f / 255.f)
                             continue;
                     }
@@ -1857,7 +1857,7 @@ ORC_API void orc_math_pow(int64_t n, const float* x, const float* e, float* y) {
     for (int64_t i = 0; i < n; ++i)
         y[i] = gsx::pow(x[i], e[i]);
 }
-// which: 7 pow, 8 x / x2, 9 sqrt(x), 10 fma(x, x2, x)  (same numbering as the device probe)
+// which: 7 pow, 8 x / x2, 9 sqrt(x), 10 fma(x, x2, x), 15 min_limit(x2, x)  (same numbering as the device probe)
 // probes of the camera-model primitives of gsx_camera.h: 0 atan2(x, x2), 1 cbrt(x), 2 asin(x), 3 cos(x),
 // 4 fisheye_max_angle_sq(x, x2, x3)
 ORC_API void orc_math_camera(int which, int64_t n, const float* x, const float* x2, const float* x3, float* y) {
@@ -1879,6 +1879,7 @@ ORC_API void orc_math_binary(int which, int64_t n, const float* x, const float* 
         case 8: y[i] = x[i] / x2[i]; break;
         case 9: y[i] = gsx::sqrt(x[i]); break;
         case 10: y[i] = gsx::fma(x[i], x2[i], x[i]); break;
+        case 15: y[i] = gsx::min_limit(x2[i], x[i]); break;
         default: y[i] = 0.f;
         }
     }
@@ -1951,7 +1952,7 @@ ORC_API int orc_record_bounds_check(uint32_t N, const float* means, const float*
                 const vec3 grd = gsx::safe_normalize(gsx::mul(M, ray_d));
                 const vec3 gcrod = gsx::cross(grd, gro);
                 const float power = -0.5f * gsx::dot(gcrod, gcrod);
-                const float alpha = gsx::fmin(0.999f, opacities[g] * gsx::exp(power));
+                const float alpha = gsx::min_limit(0.999f, opacities[g] * gsx::exp(power));
                 if (alpha < 1.f / 255.f)
                     continue;
                 ++cnt;

@@ -610,7 +610,7 @@ def math_pow(x, e):
 
 
 def math_binary(which, x, x2):
-    names = {"pow": 7, "div": 8, "sqrt": 9, "fma": 10}
+    names = {"pow": 7, "div": 8, "sqrt": 9, "fma": 10, "min_limit": 15}
     x, x2 = _f32(x), _f32(x2)
     y = np.empty_like(x)
     lib().orc_math_binary(c_i(names[which]), c_i64(x.size), _p(x), _p(x2), _p(y))

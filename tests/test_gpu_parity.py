@@ -63,6 +63,8 @@ def test_math_primitives_bit_exact(gsx, orc, cuda):
         9: (np.exp(rng.uniform(-80, 80, n)), np.ones(n), "sqrt"),
         10: (rng.normal(0, 1, n), rng.normal(0, 1, n), "fma"),
         11: (np.concatenate([rng.uniform(-87, 0, n - 3), [0.0, -87.0, -1e-30]]), None, "exp"),  # restricted variant
+        15: (np.concatenate([rng.normal(0.999, 0.5, n - 4), [np.nan, np.inf, -np.inf, 0.999]]),
+             np.full(n, 0.999), "min_limit"),
     }
     for which, (x, x2, name) in cases.items():
         x = x.astype(np.float32)

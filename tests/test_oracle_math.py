@@ -30,6 +30,15 @@ def test_exp_log_rsqrt_accuracy(orc):
                                atol=1e-37)
 
 
+def test_min_limit_is_cudas_min(orc):
+    """min_limit(limit, x): the smaller of two numbers, and the limit when x is NaN (CUDA's min / fminf, which the
+    reference's `min(0.999f, opac * vis)` is, RasterizeToPixelsFromWorld3DGSFwd.cu:239)"""
+    x = np.array([0.5, 0.999, 1.5, -2.0, np.inf, -np.inf, np.nan, 0.0], np.float32)
+    got = orc.math_binary("min_limit", x, np.full(x.size, 0.999, np.float32))
+    want = np.fmin(np.float32(0.999), x)  # fmin ignores a NaN operand
+    assert np.array_equal(got, want) and got[6] == np.float32(0.999)
+
+
 def test_sin_acos(orc):
     rng = np.random.default_rng(1)
     x = rng.uniform(-np.pi, np.pi, 200_000).astype(np.float32)
