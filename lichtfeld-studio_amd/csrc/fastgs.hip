@@ -436,16 +436,16 @@ __global__ void __launch_bounds__(256) fgs_blend_fwd_kernel(
         const bool wave_active = __builtin_amdgcn_ballot_w64(!done) != 0;
         const uint32_t n_sel = (uint32_t)__builtin_amdgcn_readfirstlane(
             (int)fgs_stage_and_select(prims, inst, first, 1, count, tr, px, 0, wave_active, stage, nullptr, wave_list));
-        for (uint32_t s = 0; s < n_sel; ++s) {
-            if (__builtin_amdgcn_ballot_w64(!done) == 0)
-                break;
+        // a pixel leaves the loop when it is saturated, the wave when its last pixel has (the loop's own divergence:
+        // the lane mask shrinks with scalar instructions only)
+        for (uint32_t s = 0; s < n_sel && !done; ++s) {
             const uint32_t t = wave_list[s];
             const float4 q0 = stage[t * 3 + 0], q1 = stage[t * 3 + 1];
             const float dx = q0.x - pxf, dy = q0.y - pyf;
             const float sigma_over_2 = 0.5f * (q0.z * dx * dx + q1.x * dy * dy) + q0.w * dx * dy;
             // beyond 87 the exponential is zero (gsx::exp) and alpha with it; up to there its restricted variant has
             // the same bits
-            if (done || sigma_over_2 < 0.0f || sigma_over_2 > 87.0f)
+            if (sigma_over_2 < 0.0f || sigma_over_2 > 87.0f)
                 continue;
             const float gaussian = gsx::exp_nonpos(-sigma_over_2);
             const float og = q1.y * gaussian;
