@@ -337,7 +337,9 @@ GSX_API int gsx_rasterize_to_pixels_from_world_3dgs_bwd(
 
 /* ---- g1 glue of a9 (Rasterization.cpp:356-378 and :608-624), fused into one pass each ----
  * fwd: colors [N,3] = max(SH(means - campos(viewmat)) + 0.5, 0) where radii > 0, else 0.
- * bwd: v_sh_coeffs [N,K,3] fully written from v_colors with the clamp mask applied. */
+ * bwd: v_sh_coeffs [N,K,3] fully written from v_colors with the clamp mask applied.
+ * radii [N,2] on an 8-byte boundary (a Gaussian's two radii are read with one load), here and in the fused passes
+ * below that take them. */
 GSX_API int gsx_sh_colors_from_world(uint32_t N, uint32_t K, uint32_t sh_degree, const float* means,
                                      const float* sh_coeffs, const int32_t* radii, const float* viewmat,
                                      float* colors, void* stream);
@@ -478,7 +480,7 @@ typedef struct gsx_update_args {
     float *means, *opacity_raw, *scaling_raw, *rotation_raw, *shs;                        /* parameters (in / out) */
     float *m_means, *m_opacity, *m_scaling, *m_rotation, *m_shs;                          /* exp_avg (in / out) */
     float *v_means, *v_opacity, *v_scaling, *v_rotation, *v_shs;                          /* exp_avg_sq (in / out) */
-    const int32_t* radii;  /* [N,2] of the forward pass */
+    const int32_t* radii;  /* [N,2] of the forward pass; 8-byte aligned */
     const float* colors;   /* [N,3] of the forward pass (clamp mask) */
     const float* viewmat;  /* [4,4] */
     void* accumulators;    /* gsx_rasterize_bwd_accumulate's workspace; consumed rows are zeroed */

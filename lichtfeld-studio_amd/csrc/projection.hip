@@ -589,10 +589,12 @@ __global__ void __launch_bounds__(256) sh_fwd_generic_kernel(uint32_t N, uint32_
     if (e >= N)
         return;
     bool live;
-    if (WORLD)
-        live = radii[e * 2] > 0 && radii[e * 2 + 1] > 0;
-    else
+    if (WORLD) { // both radii with one 8-byte load (two loads behind `&&` are two round trips in a row)
+        const int2 rad = reinterpret_cast<const int2*>(radii)[e];
+        live = rad.x > 0 && rad.y > 0;
+    } else {
         live = masks == nullptr || masks[e];
+    }
     if (!live) {
         if (WORLD) {
             colors[e * 3 + 0] = 0.f;
@@ -648,10 +650,12 @@ __global__ void __launch_bounds__(256) sh_bwd_generic_kernel(uint32_t N, uint32_
     float v[3] = {0.f, 0.f, 0.f};
     if (e < N) {
         bool live;
-        if (WORLD)
-            live = radii[e * 2] > 0 && radii[e * 2 + 1] > 0;
-        else
+        if (WORLD) {
+            const int2 rad = reinterpret_cast<const int2*>(radii)[e];
+            live = rad.x > 0 && rad.y > 0;
+        } else {
             live = masks == nullptr || masks[e];
+        }
         if (live) {
             vec3 dir = ld3(dirs_or_means, e);
             if (WORLD)
@@ -834,7 +838,9 @@ __global__ void __launch_bounds__(256) sh_records_kernel(uint32_t N, uint32_t K,
     __shared__ float4 lds[LDS16 ? 4 * kShWaveLdsF4 : 1];
     const uint32_t e = blockIdx.x * 256u + threadIdx.x;
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const bool live = e < N && radii[e * 2] > 0 && radii[e * 2 + 1] > 0;
+    // (both radii with one unconditional 8-byte load: `a > 0 && b > 0` on two loads is two round trips in a row)
+    const int2 rad = reinterpret_cast<const int2*>(radii)[min(e, N - 1)];
+    const bool live = e < N && rad.x > 0 && rad.y > 0;
     // everything the record needs is requested now, together with the coefficient rows below: one memory round
     // trip instead of one per phase (the 44 bytes are read for Gaussians without a tile too)
     const uint32_t ec = min(e, N - 1);
@@ -1063,6 +1069,7 @@ extern "C" int gsx_sh_colors_from_world(uint32_t N, uint32_t K, uint32_t sh_degr
         return GSX_OK;
     GSX_REQUIRE(means && sh_coeffs && radii && viewmat && colors, GSX_ERR_INVALID_ARGUMENT,
                 "sh_colors_from_world: null tensor");
+    GSX_REQUIRE(((uintptr_t)radii & 7) == 0, GSX_ERR_INVALID_ARGUMENT, "sh_colors_from_world: radii need 8-byte alignment");
     GSX_REQUIRE(sh_degree <= 4 && K >= (sh_degree + 1) * (sh_degree + 1), GSX_ERR_INVALID_ARGUMENT,
                 "sh_colors_from_world: degree %u needs K >= %u (got %u)", sh_degree, (sh_degree + 1) * (sh_degree + 1),
                 K);
@@ -1083,8 +1090,9 @@ extern "C" int gsx_sh_colors_records_from_world(uint32_t N, uint32_t K, uint32_t
     GSX_REQUIRE(sh_degree <= 4 && K >= (sh_degree + 1) * (sh_degree + 1), GSX_ERR_INVALID_ARGUMENT,
                 "sh_colors_records_from_world: degree %u needs K >= %u (got %u)", sh_degree,
                 (sh_degree + 1) * (sh_degree + 1), K);
-    GSX_REQUIRE(((uintptr_t)records & 15) == 0 && ((uintptr_t)quats & 15) == 0, GSX_ERR_INVALID_ARGUMENT,
-                "sh_colors_records_from_world: records / quats need 16-byte alignment");
+    GSX_REQUIRE(((uintptr_t)records & 15) == 0 && ((uintptr_t)quats & 15) == 0 && ((uintptr_t)radii & 7) == 0,
+                GSX_ERR_INVALID_ARGUMENT,
+                "sh_colors_records_from_world: records / quats need 16-byte alignment, radii 8-byte");
     const bool lds16 = K == 16 && (((uintptr_t)sh_coeffs) & 15u) == 0;
     const dim3 grid(cdiv(N, 256)), block(256);
     if (lds16)
@@ -1148,6 +1156,8 @@ extern "C" int gsx_sh_colors_from_world_bwd(uint32_t N, uint32_t K, uint32_t sh_
         return GSX_OK;
     GSX_REQUIRE(means && radii && viewmat && colors && v_colors && v_sh_coeffs, GSX_ERR_INVALID_ARGUMENT,
                 "sh_colors_from_world_bwd: null tensor");
+    GSX_REQUIRE(((uintptr_t)radii & 7) == 0, GSX_ERR_INVALID_ARGUMENT,
+                "sh_colors_from_world_bwd: radii need 8-byte alignment");
     GSX_REQUIRE(sh_degree <= 4 && K >= (sh_degree + 1) * (sh_degree + 1), GSX_ERR_INVALID_ARGUMENT,
                 "sh_colors_from_world_bwd: degree %u needs K >= %u (got %u)", sh_degree,
                 (sh_degree + 1) * (sh_degree + 1), K);

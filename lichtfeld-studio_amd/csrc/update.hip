@@ -103,6 +103,9 @@ __global__ void __launch_bounds__(256) backward_update_kernel(const UpdateArgs a
             row[0] = z, row[1] = z, row[2] = z, row[3] = z; // ready for the next backward pass
         }
         const vec3 mean = ld3(a.means, e);
+        // requested here with everything else (behind `live` and `&&` they were three round trips of their own)
+        const int2 rad = reinterpret_cast<const int2*>(a.radii)[e];
+        const float col_in[3] = {a.colors[e * 3 + 0], a.colors[e * 3 + 1], a.colors[e * 3 + 2]};
         const float o_raw = a.opacity_raw[e];
         const vec3 s_raw = ld3(a.scaling_raw, e);
         const quat q_raw = ld4q(a.rotation_raw, e);
@@ -116,13 +119,13 @@ __global__ void __launch_bounds__(256) backward_update_kernel(const UpdateArgs a
         gq.w = vq[0], gq.x = vq[1], gq.y = vq[2], gq.z = vq[3];
         const ActivationVjp av = activation_vjp(o_raw, s_raw, q_raw, r3.w, mk3(vs[0], vs[1], vs[2]), gq);
         // ---- SH backward inputs (sh_colors_from_world_bwd) ----
-        const bool live = a.radii[e * 2] > 0 && a.radii[e * 2 + 1] > 0;
+        const bool live = rad.x > 0 && rad.y > 0;
         if (live) {
             nb = sh_basis(a.sh_degree, sub(mean, campos_from_viewmat(a.viewmat)), B);
             const float v_col[3] = {r0.x, r0.y, r0.z};
 #pragma unroll
             for (int c = 0; c < 3; ++c)
-                vc[c] = a.colors[e * 3 + c] <= 0.0f ? 0.f : v_col[c]; // clamp VJP (Rasterization.cpp:609-610)
+                vc[c] = col_in[c] <= 0.0f ? 0.f : v_col[c]; // clamp VJP (Rasterization.cpp:609-610)
         }
         // ---- Adam on the small tensors ----
         adam_row<3>(a.means, a.m_means, a.v_means, e, vm, a.lr_means, a);
@@ -281,8 +284,10 @@ extern "C" int gsx_backward_update_fused(const gsx_update_args* args, void* stre
     const uint32_t need = (args->sh_degree + 1) * (args->sh_degree + 1);
     GSX_REQUIRE(args->sh_degree <= 4 && args->K >= need, GSX_ERR_INVALID_ARGUMENT,
                 "backward_update_fused: degree %u needs K >= %u (K = %u)", args->sh_degree, need, args->K);
-    GSX_REQUIRE((((uintptr_t)args->accumulators) & 15) == 0 && (((uintptr_t)args->rotation_raw) & 15) == 0,
-                GSX_ERR_INVALID_ARGUMENT, "backward_update_fused: accumulators / rotation need 16-byte alignment");
+    GSX_REQUIRE((((uintptr_t)args->accumulators) & 15) == 0 && (((uintptr_t)args->rotation_raw) & 15) == 0 &&
+                    (((uintptr_t)args->radii) & 7) == 0,
+                GSX_ERR_INVALID_ARGUMENT,
+                "backward_update_fused: accumulators / rotation need 16-byte alignment, radii 8-byte");
     UpdateArgs a;
     memset(&a, 0, sizeof(a));
     a.N = args->N, a.K = args->K, a.sh_degree = args->sh_degree;
