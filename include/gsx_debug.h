@@ -14,8 +14,8 @@ extern "C" {
  * device so that a test can compare it bit for bit with a host build.  which: 0 exp, 1 log, 2 rsqrt, 3 sin, 4 acos,
  * 5 sigmoid, 6 saturating float->u32, 7 pow(x, x2), 8 x / x2, 9 sqrt, 10 fma(x, x2, x), 11 exp restricted to
  * -87 <= x <= 0 (the rasterizers' variant; must equal 0 on that range), 12 the hardware reciprocal with one Newton
- * step (the gradient chains' 1 / (1 - alpha)), 13 the bare hardware reciprocal, 15 min_limit(x2, x) (the rasterizers' clamp
- * of alpha: x2 a number, x anything including NaN). */
+ * step (the gradient chains' 1 / (1 - alpha)), 13 the bare hardware reciprocal, 15 min_limit(x2, x) (the
+ * rasterizers' clamp of alpha: x2 a number, x anything including NaN). */
 GSX_API int gsx_debug_math(int which, uint32_t n, const float* x, const float* x2, float* y, void* stream);
 /* Measurement hook (no counterpart in the reference): a plain device-to-device copy kernel of `bytes` bytes (a
  * multiple of 16), the known-size yardstick for HBM byte counters and achieved-bandwidth figures. */
